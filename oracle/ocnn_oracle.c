@@ -1,0 +1,1008 @@
+/* TEST INFRASTRUCTURE -- CPU restatement ("oracle") of the O-CNN octree hot
+ * path in plain C99.  See ocnn_oracle.h for the pinning status of each entry
+ * point.  This file is the checker: the shipped HIP library never links,
+ * loads or calls it.
+ *
+ * Paths in comments are relative to the reference checkout root. */
+#include "ocnn_oracle.h"
+
+#include <math.h>
+#include <stddef.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ------------------------------------------------------------------------ */
+/* Wire format: OctreeInfo (octree/octree/octree_info.h:96-118), 716 bytes,
+ * payload starts at 720 (octree_info.cpp:254-268). */
+typedef struct {
+  char magic[16];
+  int batch_size, depth, full_layer, adp_layer;
+  unsigned char is_adaptive; /* +3 pad */
+  float th_dist, th_norm;
+  unsigned char key2xyz, has_node_dis; /* +2 pad */
+  int nnum[16], nnum_cum[16], nnum_nempty[16];
+  int content_flags;
+  int channels[16], locations[16];
+  float bbmin[3], bbmax[3];
+  unsigned char extrapolate, save_pts;
+  char reserved[254];
+  int ptr_dis[16];
+} OInfo;
+
+#define SA(c, n) typedef char static_assert_##n[(c) ? 1 : -1]
+SA(sizeof(OInfo) == 716, size);
+SA(offsetof(OInfo, th_dist) == 36, thd);
+SA(offsetof(OInfo, key2xyz) == 44, k2x);
+SA(offsetof(OInfo, nnum) == 48, nnum);
+SA(offsetof(OInfo, content_flags) == 240, cf);
+SA(offsetof(OInfo, bbmin) == 372, bb);
+SA(offsetof(OInfo, extrapolate) == 396, ex);
+SA(offsetof(OInfo, ptr_dis) == 652, pd);
+
+enum { kKey = 1, kChild = 2, kNeigh = 4, kFeature = 8, kLabel = 16, kSplit = 32 };
+#define KPTYPE 6
+static const char kMagic[] = "_OCTREE_2.0_"; /* 64-bit keys: octree_info.cpp:7-11 */
+
+/* PointsInfo (octree/octree/points_info.h:35-39), 88 bytes. */
+typedef struct {
+  char magic[16];
+  int pt_num, content_flags;
+  int channels[8], ptr_dis[8];
+} PInfo;
+SA(sizeof(PInfo) == 88, psize);
+enum { pPoint = 1, pNormal = 2, pFeature = 4, pLabel = 8 };
+
+static int prop_index(int ptype) { /* octree_info.cpp:283-291 */
+  for (int i = 0; i < KPTYPE; ++i) if (ptype & (1 << i)) return i;
+  return 0;
+}
+static int has_prop(const OInfo* o, int p) { return (o->content_flags & p) != 0; }
+static int channel_of(const OInfo* o, int p) {
+  return has_prop(o, p) ? o->channels[prop_index(p)] : 0;
+}
+static int location_of(const OInfo* o, int p) {
+  return has_prop(o, p) ? o->locations[prop_index(p)] : 0;
+}
+static int size_of(int p) { /* octree_info.cpp:143-155 */
+  if (p == kChild || p == kNeigh) return 4;
+  if (p == kFeature || p == kLabel || p == kSplit) return 4;
+  if (p == kKey) return 8;
+  return 0;
+}
+static void info_reset(OInfo* o) { /* octree_info.cpp:75-78 */
+  memset(o, 0, sizeof(*o));
+  strcpy(o->magic, kMagic);
+}
+static void set_channel(OInfo* o, int p, int ch) { /* octree_info.cpp:231-243 */
+  int i = prop_index(p);
+  if (ch > 0) { o->channels[i] = ch; o->content_flags |= p; }
+  else { o->channels[i] = 0; o->content_flags &= ~p; }
+}
+static void set_location(OInfo* o, int p, int lc) { o->locations[prop_index(p)] = lc; }
+static void set_property(OInfo* o, int p, int ch, int lc) { set_channel(o, p, ch); set_location(o, p, lc); }
+static void set_batch_size(OInfo* o, int b) { o->batch_size = b < 1 ? 1 : b; }
+static void set_depth(OInfo* o, int d) { o->depth = o->full_layer < d ? d : o->full_layer; }
+static void set_full_layer(OInfo* o, int fd) { o->full_layer = fd < 1 ? 1 : fd; }
+static void set_nnum_cum(OInfo* o, int capacity) { /* octree_info.cpp:215-222 */
+  o->nnum_cum[0] = 0;
+  for (int d = 1; d < o->depth + 2; ++d) o->nnum_cum[d] = o->nnum_cum[d - 1] + o->nnum[d - 1];
+  o->nnum_cum[o->depth + 2] = capacity > o->nnum_cum[o->depth + 1] ? capacity : o->nnum_cum[o->depth + 1];
+}
+static int total_nnum(const OInfo* o) { return o->nnum_cum[o->depth + 1]; }
+static int total_capacity(const OInfo* o) { return o->nnum_cum[o->depth + 2]; }
+static void set_ptr_dis(OInfo* o) { /* octree_info.cpp:254-268 */
+  o->ptr_dis[0] = (int)((sizeof(OInfo) + 7) / 8 * 8);
+  for (int i = 1; i <= KPTYPE; ++i) {
+    int p = 1 << (i - 1);
+    int lc = location_of(o, p);
+    int num = lc == -1 ? total_capacity(o) : o->nnum[lc];
+    o->ptr_dis[i] = o->ptr_dis[i - 1] + size_of(p) * num * o->channels[i - 1];
+  }
+}
+static int ptr_dis(const OInfo* o, int p, int depth) { /* octree_info.cpp:157-167 */
+  if (!has_prop(o, p)) return -1;
+  int dis = o->ptr_dis[prop_index(p)];
+  if (location_of(o, p) == -1) dis += o->nnum_cum[depth] * channel_of(o, p) * size_of(p);
+  return dis;
+}
+static int sizeof_octree(const OInfo* o) { return o->ptr_dis[KPTYPE]; }
+static float bbox_max_width(const OInfo* o) { /* octree_info.cpp:169-178 */
+  float w = o->bbmax[0] - o->bbmin[0];
+  for (int i = 1; i < 3; ++i) { float d = o->bbmax[i] - o->bbmin[i]; if (d > w) w = d; }
+  if (w == 0.0f) w = 1.0e-10f;
+  return w;
+}
+static void* prop_ptr(const void* blob, int p, int depth) {
+  int dis = ptr_dis((const OInfo*)blob, p, depth);
+  return dis < 0 ? NULL : (char*)blob + dis;
+}
+
+/* result of the last blob-producing call */
+static char* g_last = NULL;
+static int64_t g_last_sz = 0;
+static char* result_alloc(int64_t sz) {
+  free(g_last);
+  g_last = (char*)calloc(sz > 0 ? (size_t)sz : 1, 1);
+  g_last_sz = g_last ? sz : 0;
+  return g_last;
+}
+int64_t orc_fetch(void* out, int64_t cap) {
+  if (!g_last || g_last_sz > cap) return ORC_E_BADARG;
+  memcpy(out, g_last, (size_t)g_last_sz);
+  return g_last_sz;
+}
+
+/* ------------------------------------------------------------------------ */
+/* Key math: octree/octree/octree_nn.cpp:551-575 */
+static uint64_t compute_key(const uint64_t* pt, int depth) {
+  uint64_t key = 0;
+  for (int i = 0; i < depth; i++) {
+    uint64_t mask = 1u << i;
+    for (int j = 0; j < 3; j++) key |= (pt[j] & mask) << (2 * i + 2 - j);
+  }
+  return key;
+}
+static void compute_pt(uint64_t* pt, uint64_t key, int depth) {
+  pt[0] = pt[1] = pt[2] = 0;
+  for (int i = 0; i < depth; i++)
+    for (int j = 0; j < 3; j++) {
+      uint64_t mask = (uint64_t)1 << (3 * i + 2 - j);
+      pt[j] |= (key & mask) >> (2 * i + 2 - j);
+    }
+}
+/* octree_nn.cpp:578-619: packed xyz = four uint16 sub-fields (x,y,z,id) */
+void orc_xyz2key(uint64_t* key, const uint64_t* xyz, int num, int depth) {
+  for (int i = 0; i < num; ++i) {
+    uint16_t f[4]; memcpy(f, xyz + i, 8);
+    uint64_t pt[3] = { f[0], f[1], f[2] };
+    uint64_t k = compute_key(pt, depth);
+    uint16_t g[4]; memcpy(g, &k, 8);
+    g[3] = f[3];
+    memcpy(key + i, g, 8);
+  }
+}
+void orc_key2xyz(uint64_t* xyz, const uint64_t* key, int num, int depth) {
+  for (int i = 0; i < num; ++i) {
+    uint64_t pt[3]; compute_pt(pt, key[i], depth);
+    uint16_t f[4]; memcpy(f, key + i, 8);
+    for (int j = 0; j < 3; ++j) f[j] = (uint16_t)pt[j];
+    memcpy(xyz + i, f, 8);
+  }
+}
+void orc_key2idx(int* idx, const uint64_t* key, int num) {
+  for (int i = 0; i < num; ++i) idx[i] = (int)(key[i] >> 48);
+}
+/* octree_nn.cpp:541-548 */
+void orc_search_key(int* idx, const uint64_t* key, int n_key, const uint64_t* query, int n_query) {
+  for (int i = 0; i < n_query; ++i) {
+    int lo = 0, hi = n_key; /* lower_bound */
+    while (lo < hi) { int mid = lo + (hi - lo) / 2; if (key[mid] < query[i]) lo = mid + 1; else hi = mid; }
+    idx[i] = (lo >= n_key || key[lo] != query[i]) ? -1 : lo;
+  }
+}
+
+/* ------------------------------------------------------------------------ */
+/* NeighHelper tables: octree/octree/octree_nn.cpp:6-81 */
+static int g_ni3[216], g_parent[512], g_dis[64], g_tables_ready = 0;
+static const int kSub111[] = { 13 };
+static const int kSub222[] = { 13, 14, 16, 17, 22, 23, 25, 26 };
+static const int kSub311[] = { 4, 13, 22 };
+static const int kSub131[] = { 10, 13, 16 };
+static const int kSub113[] = { 12, 13, 14 };
+static const int kSub331[] = { 1, 4, 7, 10, 13, 16, 19, 22, 25 };
+static const int kSub313[] = { 3, 4, 5, 12, 13, 14, 21, 22, 23 };
+static const int kSub133[] = { 9, 10, 11, 12, 13, 14, 15, 16, 17 };
+static void init_tables(void) {
+  if (g_tables_ready) return;
+  int id = 0;
+  for (int ijk = 0; ijk < 8; ++ijk)
+    for (int xyz = 0; xyz < 27; ++xyz) {
+      int k = ijk % 2, p = ijk / 2, j = p % 2, i = p / 2;
+      int z = xyz % 3, q = xyz / 3, y = q % 3, x = q / 3;
+      g_ni3[id++] = ((x + i) << 4) | ((y + j) << 2) | (z + k);
+    }
+  int tmp[64]; id = 0;
+  for (int x = 1; x < 5; ++x)
+    for (int y = 1; y < 5; ++y)
+      for (int z = 1; z < 5; ++z) {
+        tmp[id] = (x / 2) * 9 + (y / 2) * 3 + (z / 2);
+        g_dis[id] = ((x % 2) << 2) | ((y % 2) << 1) | (z % 2);
+        id++;
+      }
+  for (int i = 0; i < 8; ++i)
+    for (int j = 0; j < 64; ++j) g_parent[i * 64 + j] = g_ni3[i * 27 + tmp[j]];
+  g_tables_ready = 1;
+}
+int orc_get_ni(const int* ks, int* out) { /* octree_nn.cpp:111-119 */
+  init_tables();
+  int code = ks[0] * 100 + ks[1] * 10 + ks[2];
+  const int* sub = NULL; int sz = 0;
+  switch (code) {
+    case 333: memcpy(out, g_ni3, sizeof(g_ni3)); return 216;
+    case 111: sub = kSub111; sz = 1; break;
+    case 222: sub = kSub222; sz = 8; break;
+    case 311: sub = kSub311; sz = 3; break;
+    case 131: sub = kSub131; sz = 3; break;
+    case 113: sub = kSub113; sz = 3; break;
+    case 331: sub = kSub331; sz = 9; break;
+    case 313: sub = kSub313; sz = 9; break;
+    case 133: sub = kSub133; sz = 9; break;
+    default: return ORC_E_UNSUPPORTED;
+  }
+  for (int i = 0; i < 8; ++i)
+    for (int j = 0; j < sz; ++j) out[i * sz + j] = g_ni3[i * 27 + sub[j]];
+  return 8 * sz;
+}
+void orc_get_parent(int* out) { init_tables(); memcpy(out, g_parent, sizeof(g_parent)); }
+void orc_get_dis(int* out) { init_tables(); memcpy(out, g_dis, sizeof(g_dis)); }
+
+/* octree_nn.cpp:357-380 */
+void orc_calc_neigh_sparse(int* neigh_child, const int* neigh, const int* children, int node_num) {
+  init_tables();
+  for (int i = 0; i < node_num; ++i) {
+    int l0 = children[i];
+    if (l0 == -1) continue;
+    const int* ngh0 = neigh + (i >> 3 << 6);
+    const int* pi0 = g_parent + (i % 8) * 64;
+    int* ngh1 = neigh_child + ((int64_t)l0 << 6);
+    for (int j = 0; j < 64; ++j) {
+      ngh1[j] = -1;
+      int k = ngh0[pi0[j]];
+      if (k != -1) { int l1 = children[k]; if (l1 != -1) ngh1[j] = (l1 << 3) + g_dis[j]; }
+    }
+  }
+}
+/* octree_nn.cpp:382-424 */
+void orc_calc_neigh_full(int* neigh, int depth, int batch) {
+  const uint64_t node_num = (uint64_t)1 << (3 * depth), bound = (uint64_t)1 << depth;
+  for (uint64_t n = 0; n < (uint64_t)batch; ++n)
+    for (uint64_t i = 0; i < node_num; i += 8) {
+      uint64_t p0[3]; compute_pt(p0, i, depth);
+      for (uint64_t x = 0; x < 4; ++x)
+        for (uint64_t y = 0; y < 4; ++y)
+          for (uint64_t z = 0; z < 4; ++z) {
+            uint64_t p1[3] = { p0[0] + x - 1, p0[1] + y - 1, p0[2] + z - 1 };
+            int v = -1;
+            if ((p1[0] & bound) == 0 && (p1[1] & bound) == 0 && (p1[2] & bound) == 0)
+              v = (int)(compute_key(p1, depth) + n * node_num);
+            neigh[((x << 4) | (y << 2) | z) + i * 8 + n * node_num * 8] = v;
+          }
+    }
+}
+
+/* ------------------------------------------------------------------------ */
+/* octree_nn.cpp:427-473 */
+void orc_generate_key_child(uint64_t* key_child, const uint64_t* key, const int* child, int node_num) {
+  for (int i = 0; i < node_num; ++i) {
+    int label = child[i];
+    if (label < 0) continue;
+    uint16_t k0[4]; memcpy(k0, key + i, 8);
+    for (int j = 0; j < 8; ++j) {
+      uint16_t k1[4];
+      k1[0] = (uint16_t)((k0[0] << 1) | ((j & 4) >> 2));
+      k1[1] = (uint16_t)((k0[1] << 1) | ((j & 2) >> 1));
+      k1[2] = (uint16_t)((k0[2] << 1) | (j & 1));
+      k1[3] = k0[3];
+      memcpy(key_child + 8 * (int64_t)label + j, k1, 8);
+    }
+  }
+}
+void orc_generate_key_full(uint64_t* key, int depth, int batch) {
+  int node_num = 1 << (3 * depth);
+  for (int n = 0; n < batch; ++n)
+    for (int k = 0; k < node_num; ++k) {
+      uint64_t pt[3]; compute_pt(pt, (uint64_t)k, depth);
+      uint16_t f[4] = { (uint16_t)pt[0], (uint16_t)pt[1], (uint16_t)pt[2], (uint16_t)n };
+      memcpy(key + (int64_t)n * node_num + k, f, 8);
+    }
+}
+int orc_generate_label(int* label, const int* btm, int btm_h, int mask) {
+  int top_h = 0;
+  for (int i = 0; i < btm_h; ++i) label[i] = (mask == btm[i]) ? top_h++ : -1;
+  return top_h;
+}
+
+/* ------------------------------------------------------------------------ */
+/* octree_nn.cpp:163-185 */
+void orc_pad_forward(float* Y, int Hy, int C, const float* X, int Hx, const int* label, float dval) {
+  for (int c = 0; c < C; ++c)
+    for (int h = 0; h < Hy; ++h)
+      Y[(int64_t)c * Hy + h] = label[h] == -1 ? dval : X[(int64_t)c * Hx + label[h]];
+}
+void orc_pad_backward(float* X, int Hx, int C, const float* Y, int Hy, const int* label) {
+  for (int c = 0; c < C; ++c)
+    for (int h = 0; h < Hy; ++h)
+      if (label[h] != -1) X[(int64_t)c * Hx + label[h]] = Y[(int64_t)c * Hy + h];
+}
+static void pad_backward_int(int* X, const int* Y, int Hy, const int* label) {
+  for (int h = 0; h < Hy; ++h) if (label[h] != -1) X[label[h]] = Y[h];
+}
+
+/* octree_nn.cpp:188-241 */
+void orc_octree2col(float* col, const float* data, int channel, int height,
+    int kernel_sdim, int stride, const int* neigh, const int* ni, int height_col, int n) {
+  const int64_t octree_h = (int64_t)height << (3 * (stride - 1));
+  for (int c = 0; c < channel; ++c)
+    for (int k = 0; k < kernel_sdim; ++k) {
+      int64_t h_start = (int64_t)n * height_col;
+      int64_t i_start = ((int64_t)c * kernel_sdim + k) * height_col - h_start;
+      for (int64_t h = h_start; h < h_start + height_col; ++h) {
+        if (h >= height) { col[i_start + h] = 0.0f; continue; }
+        int64_t index = stride == 2 ? (h << 6) + ni[k] : (h >> 3 << 6) + ni[(h % 8) * kernel_sdim + k];
+        int p = neigh[index];
+        col[i_start + h] = p == -1 ? 0.0f : data[c * octree_h + p];
+      }
+    }
+}
+void orc_col2octree(const float* col, float* data, int channel, int height,
+    int kernel_sdim, int stride, const int* neigh, const int* ni, int height_col, int n) {
+  const int64_t octree_h = (int64_t)height << (3 * (stride - 1));
+  if (n == 0) memset(data, 0, sizeof(float) * (size_t)(channel * octree_h));
+  for (int c = 0; c < channel; ++c)
+    for (int k = 0; k < kernel_sdim; ++k) {
+      int64_t h_start = (int64_t)n * height_col;
+      int64_t i_start = ((int64_t)c * kernel_sdim + k) * height_col - h_start;
+      for (int64_t h = h_start; h < h_start + height_col; ++h) {
+        if (h >= height) continue;
+        int64_t index = stride == 2 ? (h << 6) + ni[k] : (h >> 3 << 6) + ni[(h % 8) * kernel_sdim + k];
+        int p = neigh[index];
+        if (p != -1) data[c * octree_h + p] += col[i_start + h];
+      }
+    }
+}
+/* octree_nn.cpp:244-298 */
+void orc_octree2colP(float* col, const float* data, int channel, int height,
+    int octree_h, int kernel_sdim, int stride, const int* neigh, const int* ni,
+    const int* child, const int* ichild, int height_col, int n) {
+  for (int c = 0; c < channel; ++c)
+    for (int k = 0; k < kernel_sdim; ++k) {
+      int64_t h_start = (int64_t)n * height_col;
+      int64_t i_start = ((int64_t)c * kernel_sdim + k) * height_col - h_start;
+      for (int64_t h = h_start; h < h_start + height_col; ++h) {
+        if (h >= height) { col[i_start + h] = 0.0f; continue; }
+        int64_t index;
+        if (stride == 2) index = (h << 6) + ni[k];
+        else { int hp = ichild[h]; index = ((int64_t)hp >> 3 << 6) + ni[(hp % 8) * kernel_sdim + k]; }
+        int p = neigh[index];
+        if (p >= 0) p = child[p];
+        col[i_start + h] = p < 0 ? 0.0f : data[(int64_t)c * octree_h + p];
+      }
+    }
+}
+void orc_col2octreeP(const float* col, float* data, int channel, int height,
+    int octree_h, int kernel_sdim, int stride, const int* neigh, const int* ni,
+    const int* child, const int* ichild, int height_col, int n) {
+  if (n == 0) memset(data, 0, sizeof(float) * (size_t)channel * (size_t)octree_h);
+  for (int c = 0; c < channel; ++c)
+    for (int k = 0; k < kernel_sdim; ++k) {
+      int64_t h_start = (int64_t)n * height_col;
+      int64_t i_start = ((int64_t)c * kernel_sdim + k) * height_col - h_start;
+      for (int64_t h = h_start; h < h_start + height_col; ++h) {
+        if (h >= height) continue;
+        int64_t index;
+        if (stride == 2) index = (h << 6) + ni[k];
+        else { int hp = ichild[h]; index = ((int64_t)hp >> 3 << 6) + ni[(hp % 8) * kernel_sdim + k]; }
+        int p = neigh[index];
+        if (p >= 0) p = child[p];
+        if (p >= 0) data[(int64_t)c * octree_h + p] += col[i_start + h];
+      }
+    }
+}
+
+/* octree_nn.cpp:301-354 */
+void orc_max_pool(float* top, int top_h, int* mask, const float* btm, int btm_h, int channel) {
+  for (int c = 0; c < channel; ++c) {
+    for (int h = 0; h < top_h; ++h) {
+      int hb = 8 * h;
+      top[h] = btm[hb]; mask[h] = hb;
+      for (int idx = hb + 1; idx < hb + 8; ++idx)
+        if (btm[idx] > top[h]) { top[h] = btm[idx]; mask[h] = idx; }
+    }
+    mask += top_h; top += top_h; btm += btm_h;
+  }
+}
+void orc_max_unpool(const float* top, int top_h, const int* mask, float* btm, int btm_h, int channel) {
+  memset(btm, 0, sizeof(float) * (size_t)btm_h * (size_t)channel);
+  for (int c = 0; c < channel; ++c) {
+    for (int h = 0; h < top_h; ++h) btm[mask[h]] = top[h];
+    mask += top_h; top += top_h; btm += btm_h;
+  }
+}
+void orc_mask_pool(float* top, int top_h, const int* mask, const float* btm, int btm_h, int channel) {
+  for (int c = 0; c < channel; ++c) {
+    for (int h = 0; h < top_h; ++h) top[h] = btm[mask[h]];
+    mask += top_h; top += top_h; btm += btm_h;
+  }
+}
+
+/* ------------------------------------------------------------------------ */
+/* Textbook SGEMM, row-major, k ascending per output element.  The reference
+ * ships no CPU GEMMEngine (octree/octree/octree_conv.h:86 is only a pointer);
+ * its data flow is octree/octree/octree_conv.cpp:157-207. */
+void orc_sgemm(int transA, int transB, int M, int N, int K, const float* A,
+    const float* B, float beta, float* C) {
+  for (int m = 0; m < M; ++m) {
+    float* c = C + (int64_t)m * N;
+    if (beta == 0.0f) memset(c, 0, sizeof(float) * (size_t)N);
+    else if (beta != 1.0f) for (int n = 0; n < N; ++n) c[n] *= beta;
+    for (int k = 0; k < K; ++k) {
+      float a = transA ? A[(int64_t)k * M + m] : A[(int64_t)m * K + k];
+      if (!transB) {
+        const float* b = B + (int64_t)k * N;
+        for (int n = 0; n < N; ++n) c[n] += a * b[n];
+      } else {
+        for (int n = 0; n < N; ++n) c[n] += a * B[(int64_t)n * K + k];
+      }
+    }
+  }
+}
+
+/* Shape rules of OctreeBaseConv::reshape (octree/octree/octree_conv.cpp:48-104). */
+typedef struct {
+  int top_depth, workspace_depth, top_h, workspace_h, child_h, ichild_h, octree_h;
+} ConvShape;
+static int conv_shape(const OInfo* o, int depth, int stride, int nempty, int deconv, ConvShape* s) {
+  s->top_depth = s->workspace_depth = depth;
+  if (stride == 2) {
+    if (deconv) s->top_depth = s->workspace_depth = depth + 1;
+    else s->top_depth = depth - 1;
+    if (!(0 <= s->top_depth && s->top_depth <= o->depth)) return ORC_E_BADARG;
+  }
+  int top_h;
+  if (!nempty) {
+    top_h = o->nnum[s->top_depth];
+    if (stride == 2 && !deconv) top_h = o->nnum_nempty[s->top_depth];
+  } else top_h = o->nnum_nempty[s->top_depth];
+  if (top_h == 0) top_h = 1;
+  s->top_h = top_h;
+  s->workspace_h = top_h;
+  if (stride == 2) s->workspace_h = deconv ? o->nnum[s->top_depth] / 8 : o->nnum[depth] / 8;
+  s->child_h = s->ichild_h = s->octree_h = 0;
+  if (nempty) {
+    s->child_h = o->nnum[s->workspace_depth];
+    s->ichild_h = o->nnum_nempty[s->workspace_depth];
+    s->octree_h = o->nnum_nempty[depth];
+    if (stride == 2 && deconv) s->octree_h = o->nnum_nempty[s->top_depth];
+  }
+  return 0;
+}
+int orc_conv_top_h(const void* blob, int depth, int stride, int nempty, int is_deconv) {
+  ConvShape s;
+  int e = conv_shape((const OInfo*)blob, depth, stride, nempty, is_deconv, &s);
+  return e < 0 ? e : s.top_h;
+}
+static int check_btm_h(const OInfo* o, int depth, int stride, int nempty, int deconv, int btm_h) {
+  /* pytorch/cpp/octree_conv.cpp:72-78 */
+  if ((stride == 2 && deconv) || nempty) return btm_h == o->nnum_nempty[depth];
+  return btm_h == o->nnum[depth];
+}
+static int* make_ichild(const OInfo* o, const int* child, const ConvShape* s) {
+  /* pytorch/cpp/octree_conv.cpp:108-117 */
+  (void)o;
+  int* seq = (int*)malloc(sizeof(int) * (size_t)(s->child_h + 1));
+  int* ichild = (int*)calloc((size_t)(s->ichild_h + 1), sizeof(int));
+  for (int i = 0; i < s->child_h; ++i) seq[i] = i;
+  pad_backward_int(ichild, seq, s->child_h, child);
+  free(seq);
+  return ichild;
+}
+int orc_octree_conv(float* top, const float* btm, int channel_in, int btm_h,
+    const float* weights, const void* blob, int depth, int num_output,
+    const int* ks, int stride, int nempty) {
+  const OInfo* o = (const OInfo*)blob;
+  ConvShape s; int ni[216];
+  if (depth <= 0 || num_output <= 0 || (stride != 1 && stride != 2)) return ORC_E_BADARG;
+  int e = conv_shape(o, depth, stride, nempty, 0, &s); if (e < 0) return e;
+  int nni = orc_get_ni(ks, ni); if (nni < 0) return nni;
+  if (!check_btm_h(o, depth, stride, nempty, 0, btm_h)) return ORC_E_BADARG;
+  int ksdim = ks[0] * ks[1] * ks[2], kdim = ksdim * channel_in;
+  const int* neigh = (const int*)prop_ptr(blob, kNeigh, s.workspace_depth);
+  float* col = (float*)malloc(sizeof(float) * (size_t)kdim * (size_t)s.workspace_h + 4);
+  if (!col) return ORC_E_NOMEM;
+  if (!nempty) {
+    orc_octree2col(col, btm, channel_in, s.workspace_h, ksdim, stride, neigh, ni, s.workspace_h, 0);
+  } else {
+    const int* child = (const int*)prop_ptr(blob, kChild, s.workspace_depth);
+    int* ichild = make_ichild(o, child, &s);
+    orc_octree2colP(col, btm, channel_in, s.workspace_h, s.octree_h, ksdim, stride, neigh, ni,
+        child, ichild, s.workspace_h, 0);
+    free(ichild);
+  }
+  orc_sgemm(0, 0, num_output, s.workspace_h, kdim, weights, col, 0.0f, top);
+  free(col);
+  return s.top_h;
+}
+int orc_octree_deconv(float* top, const float* btm, int channel_in, int btm_h,
+    const float* weights, const void* blob, int depth, int num_output,
+    const int* ks, int stride, int nempty) {
+  const OInfo* o = (const OInfo*)blob;
+  ConvShape s; int ni[216];
+  if (depth <= 0 || num_output <= 0 || (stride != 1 && stride != 2)) return ORC_E_BADARG;
+  int e = conv_shape(o, depth, stride, nempty, 1, &s); if (e < 0) return e;
+  int nni = orc_get_ni(ks, ni); if (nni < 0) return nni;
+  if (!check_btm_h(o, depth, stride, nempty, 1, btm_h)) return ORC_E_BADARG;
+  /* deconv: conv_out_channels = channel_in, conv_in_channels = num_output
+   * (octree_conv.cpp:31-35); forward is backward_cpu_gemm
+   * (pytorch/cpp/octree_conv.cpp:212). */
+  int ksdim = ks[0] * ks[1] * ks[2], kdim = ksdim * num_output;
+  const int* neigh = (const int*)prop_ptr(blob, kNeigh, s.workspace_depth);
+  float* col = (float*)malloc(sizeof(float) * (size_t)kdim * (size_t)s.workspace_h + 4);
+  if (!col) return ORC_E_NOMEM;
+  orc_sgemm(1, 0, kdim, s.workspace_h, channel_in, weights, btm, 0.0f, col);
+  if (!nempty) {
+    orc_col2octree(col, top, num_output, s.workspace_h, ksdim, stride, neigh, ni, s.workspace_h, 0);
+  } else {
+    const int* child = (const int*)prop_ptr(blob, kChild, s.workspace_depth);
+    int* ichild = make_ichild(o, child, &s);
+    orc_col2octreeP(col, top, num_output, s.workspace_h, s.octree_h, ksdim, stride, neigh, ni,
+        child, ichild, s.workspace_h, 0);
+    free(ichild);
+  }
+  free(col);
+  return s.top_h;
+}
+
+/* ------------------------------------------------------------------------ */
+/* points2octree: pytorch/cpp/point2octree.cpp:5-34,
+ * OctreeInfo::initialize octree/octree/octree_info.cpp:13-73,
+ * Octree::build octree/octree/octree.cpp:74-121. */
+typedef struct { uint64_t key, idx; } Code;
+static int code_cmp(const void* a, const void* b) { /* std::sort of pair<key,idx>: octree.cpp:193 */
+  const Code* x = (const Code*)a; const Code* y = (const Code*)b;
+  if (x->key != y->key) return x->key < y->key ? -1 : 1;
+  if (x->idx != y->idx) return x->idx < y->idx ? -1 : 1;
+  return 0;
+}
+/* octree.cpp:890-904: in-place unique, returns new size, idx gets n_unique+1 entries */
+static int unique_key(uint64_t* keys, int n, uint64_t* idx) {
+  int ni = 0, j = 1;
+  idx[ni++] = 0;
+  for (int i = 1; i < n; i++)
+    if (keys[i] != keys[i - 1]) { idx[ni++] = (uint64_t)i; keys[j++] = keys[i]; }
+  idx[ni] = (uint64_t)n;
+  return n > 0 ? j : 0;
+}
+
+int64_t orc_points2octree(const void* points_blob, int depth, int full_depth,
+    int node_dis, int node_feature, int split_label, int adaptive,
+    int adp_depth, float th_normal, float th_distance, int extrapolate,
+    int save_pts, int key2xyz, const float* bbmin_in, const float* bbmax_in) {
+  const PInfo* pi = (const PInfo*)points_blob;
+  if (strcmp(pi->magic, "_POINTS_1.0_") != 0 || pi->pt_num <= 0) return ORC_E_BADARG;
+  if (node_feature || adaptive) return ORC_E_UNSUPPORTED; /* octree.cpp:454-806, 958-1135 not restated */
+  const int npt = pi->pt_num;
+  const char* base = (const char*)points_blob;
+  const float* pts = (pi->content_flags & pPoint) ? (const float*)(base + pi->ptr_dis[0]) : NULL;
+  const float* normals = (pi->content_flags & pNormal) ? (const float*)(base + pi->ptr_dis[1]) : NULL;
+  const float* features = (pi->content_flags & pFeature) ? (const float*)(base + pi->ptr_dis[2]) : NULL;
+  const float* labels = (pi->content_flags & pLabel) ? (const float*)(base + pi->ptr_dis[3]) : NULL;
+  const int ch_normal = normals ? pi->channels[1] : 0;
+  const int ch_feature = features ? pi->channels[2] : 0;
+  const int ch_label = labels ? pi->channels[3] : 0;
+  if (!pts) return ORC_E_BADARG;
+
+  /* OctreeInfo::initialize, octree_info.cpp:13-73 */
+  OInfo o; info_reset(&o);
+  set_batch_size(&o, 1);
+  set_depth(&o, depth);
+  set_full_layer(&o, full_depth);
+  o.adp_layer = adp_depth;
+  o.is_adaptive = adaptive ? 1 : 0;
+  o.has_node_dis = node_dis ? 1 : 0;
+  o.key2xyz = key2xyz ? 1 : 0;
+  o.extrapolate = extrapolate ? 1 : 0;
+  o.save_pts = save_pts ? 1 : 0;
+  o.th_norm = th_normal;
+  o.th_dist = th_distance;
+  set_property(&o, kKey, (key2xyz && depth > 8) ? 2 : 1, -1);
+  set_property(&o, kChild, 1, -1);
+  if (split_label) set_property(&o, kSplit, 1, -1);
+  int channel = ch_normal + ch_feature;
+  if (node_dis) { channel += 1; if (ch_normal == 0) channel += 3; }
+  if (save_pts) channel += 3;
+  set_channel(&o, kFeature, channel);
+  set_location(&o, kFeature, (node_feature || adaptive) ? -1 : depth);
+  if (ch_label == 1) {
+    set_channel(&o, kLabel, 1);
+    set_location(&o, kLabel, (node_feature || adaptive) ? -1 : depth);
+  }
+  for (int i = 0; i < 3; ++i) { o.bbmin[i] = -1.0f; o.bbmax[i] = 1.0f; }
+  if (bbmin_in && bbmax_in)
+    for (int i = 0; i < 3; ++i) { o.bbmin[i] = bbmin_in[i]; o.bbmax[i] = bbmax_in[i]; }
+  depth = o.depth;
+  const int full_layer = o.full_layer;
+  if (depth < 1 || depth > 16 || full_layer > depth) return ORC_E_BADARG;
+
+  /* normalize_pts, octree.cpp:155-170 */
+  const float mul = (float)(1 << depth) / bbox_max_width(&o);
+  float* pts_scaled = (float*)malloc(sizeof(float) * 3 * (size_t)npt);
+  for (int i = 0; i < npt; i++)
+    for (int j = 0; j < 3; j++) pts_scaled[3 * i + j] = (pts[3 * i + j] - o.bbmin[j]) * mul;
+
+  /* sort_keys, octree.cpp:172-203 */
+  Code* code = (Code*)malloc(sizeof(Code) * (size_t)npt);
+  for (int i = 0; i < npt; i++) {
+    uint64_t pt[3];
+    for (int j = 0; j < 3; ++j) pt[j] = (uint64_t)pts_scaled[3 * i + j];
+    code[i].key = compute_key(pt, depth);
+    code[i].idx = (uint64_t)i;
+  }
+  qsort(code, (size_t)npt, sizeof(Code), code_cmp);
+  uint64_t* node_keys = (uint64_t*)malloc(sizeof(uint64_t) * (size_t)npt);
+  uint64_t* sorted_idx = (uint64_t*)malloc(sizeof(uint64_t) * (size_t)npt);
+  for (int i = 0; i < npt; i++) { node_keys[i] = code[i].key; sorted_idx[i] = code[i].idx; }
+  free(code);
+  uint64_t* unique_idx = (uint64_t*)malloc(sizeof(uint64_t) * ((size_t)npt + 1));
+  int n_keys = unique_key(node_keys, npt, unique_idx);
+
+  /* build_structure, octree.cpp:205-283 */
+  uint64_t* keys[17]; int* children[17]; int nnum[17] = { 0 };
+  for (int d = 0; d <= 16; ++d) { keys[d] = NULL; children[d] = NULL; }
+  for (int d = 0; d <= full_layer; d++) {
+    int n = 1 << (3 * d);
+    nnum[d] = n;
+    keys[d] = (uint64_t*)malloc(sizeof(uint64_t) * (size_t)n);
+    children[d] = (int*)malloc(sizeof(int) * (size_t)n);
+    for (int i = 0; i < n; i++) { keys[d][i] = (uint64_t)i; children[d][i] = d != full_layer ? i : -1; }
+  }
+  uint64_t* parent_keys = (uint64_t*)malloc(sizeof(uint64_t) * ((size_t)n_keys + 1));
+  uint64_t* parent_pidx = (uint64_t*)malloc(sizeof(uint64_t) * ((size_t)n_keys + 2));
+  for (int d = depth; d > full_layer; --d) {
+    int n = n_keys;
+    for (int i = 0; i < n; i++) parent_keys[i] = node_keys[i] >> 3;
+    int np = unique_key(parent_keys, n, parent_pidx);
+    int nch = np << 3;
+    nnum[d] = nch;
+    keys[d] = (uint64_t*)malloc(sizeof(uint64_t) * ((size_t)nch + 1));
+    children[d] = (int*)malloc(sizeof(int) * ((size_t)nch + 1));
+    for (int i = 0; i < nch; i++) { keys[d][i] = (parent_keys[i >> 3] << 3) | (uint64_t)(i % 8); children[d][i] = -1; }
+    for (int i = 0; i < np; i++)
+      for (uint64_t j = parent_pidx[i]; j < parent_pidx[i + 1]; j++)
+        children[d][(node_keys[j] & 7u) | ((uint64_t)i << 3)] = (int)j;
+    memcpy(node_keys, parent_keys, sizeof(uint64_t) * (size_t)np);
+    n_keys = np;
+  }
+  if (depth > full_layer)
+    for (int i = 0; i < n_keys; i++) children[full_layer][node_keys[i]] = i;
+  free(parent_keys); free(parent_pidx);
+
+  /* calc_node_num, octree.cpp:285-309 */
+  for (int d = 0; d <= depth; ++d) {
+    o.nnum[d] = nnum[d];
+    o.nnum_nempty[d] = 0;
+    for (int i = nnum[d] - 1; i >= 0; i--)
+      if (children[d][i] != -1) { o.nnum_nempty[d] = children[d][i] + 1; break; }
+  }
+  set_nnum_cum(&o, 0);
+  set_ptr_dis(&o);
+
+  /* calc_signal (finest level), octree.cpp:312-452 */
+  const int nn = nnum[depth];
+  const int* child_d = children[depth];
+  float* avg_normals = NULL; float* avg_features = NULL; float* avg_labels = NULL;
+  float* avg_pts = NULL; float* displacement = NULL;
+  int ch_dis = 0;
+  if (normals) {
+    avg_normals = (float*)calloc((size_t)ch_normal * (size_t)nn + 1, sizeof(float));
+    float* acc = (float*)malloc(sizeof(float) * (size_t)(ch_normal + 1));
+    for (int i = 0; i < nn; i++) {
+      int t = child_d[i];
+      if (t == -1) continue;
+      for (int c = 0; c < ch_normal; ++c) acc[c] = 0.0f;
+      for (uint64_t j = unique_idx[t]; j < unique_idx[t + 1]; j++) {
+        uint64_t h = sorted_idx[j];
+        for (int c = 0; c < ch_normal; ++c) acc[c] += normals[ch_normal * h + c];
+      }
+      float len = 0.0f;
+      for (int c = 0; c < ch_normal; ++c) len += acc[c] * acc[c];
+      float factor = sqrtf(len);
+      if (factor < 1.0e-6f) {
+        uint64_t h = sorted_idx[unique_idx[t]];
+        for (int c = 0; c < ch_normal; ++c) acc[c] = normals[ch_normal * h + c];
+        len = 0.0f;
+        for (int c = 0; c < ch_normal; ++c) len += acc[c] * acc[c];
+        factor = sqrtf(len) + 1.0e-30f;
+      }
+      for (int c = 0; c < ch_normal; ++c) avg_normals[(int64_t)c * nn + i] = acc[c] / factor;
+    }
+    free(acc);
+  }
+  if (features) {
+    avg_features = (float*)calloc((size_t)ch_feature * (size_t)nn + 1, sizeof(float));
+    float* acc = (float*)malloc(sizeof(float) * (size_t)(ch_feature + 1));
+    for (int i = 0; i < nn; i++) {
+      int t = child_d[i];
+      if (t == -1) continue;
+      for (int c = 0; c < ch_feature; ++c) acc[c] = 0.0f;
+      for (uint64_t j = unique_idx[t]; j < unique_idx[t + 1]; j++) {
+        uint64_t h = sorted_idx[j];
+        for (int c = 0; c < ch_feature; ++c) acc[c] += features[ch_feature * h + c];
+      }
+      float factor = (float)(unique_idx[t + 1] - unique_idx[t]) + 1.0e-30f;
+      for (int c = 0; c < ch_feature; ++c) avg_features[(int64_t)c * nn + i] = acc[c] / factor;
+    }
+    free(acc);
+  }
+  if (labels) {
+    avg_labels = (float*)malloc(sizeof(float) * ((size_t)nn + 1));
+    for (int i = 0; i < nn; ++i) avg_labels[i] = -1.0f;
+    float mx = labels[0];
+    for (int i = 1; i < npt; ++i) if (labels[i] > mx) mx = labels[i];
+    int max_label = (int)mx + 1;
+    int* cnt = (int*)malloc(sizeof(int) * (size_t)(max_label > 0 ? max_label : 1));
+    for (int i = 0; i < nn; i++) {
+      int t = child_d[i];
+      if (t == -1) continue;
+      int valid = 0;
+      for (int l = 0; l < max_label; ++l) cnt[l] = 0;
+      for (uint64_t j = unique_idx[t]; j < unique_idx[t + 1]; j++) {
+        int l = (int)labels[sorted_idx[j]];
+        if (l < 0) continue;
+        cnt[l] += 1; valid += 1;
+      }
+      if (valid > 0) {
+        int best = 0;
+        for (int l = 1; l < max_label; ++l) if (cnt[l] > cnt[best]) best = l;
+        avg_labels[i] = (float)best;
+      }
+    }
+    free(cnt);
+  }
+  if (o.has_node_dis || o.save_pts) {
+    const float mulD = 1.1547f;
+    avg_pts = (float*)calloc(3 * (size_t)nn + 1, sizeof(float));
+    ch_dis = normals ? 1 : 4;
+    displacement = (float*)calloc((size_t)ch_dis * (size_t)nn + 1, sizeof(float));
+    for (int i = 0; i < nn; i++) {
+      int t = child_d[i];
+      if (t == -1) continue;
+      float avg_pt[3] = { 0.0f, 0.0f, 0.0f };
+      for (uint64_t j = unique_idx[t]; j < unique_idx[t + 1]; j++) {
+        uint64_t h = sorted_idx[j];
+        for (int c = 0; c < 3; ++c) avg_pt[c] += pts_scaled[3 * h + c];
+      }
+      float dis[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
+      float factor = (float)(unique_idx[t + 1] - unique_idx[t]) + 1.0e-30f;
+      for (int c = 0; c < 3; ++c) {
+        avg_pt[c] /= factor;
+        float ip = 0.0f;
+        float fp = modff(avg_pt[c], &ip);
+        dis[c] = fp - 0.5f;
+        if (normals) dis[3] += dis[c] * avg_normals[(int64_t)c * nn + i];
+        else dis[3] = 1.0f;
+        avg_pts[(int64_t)c * nn + i] = avg_pt[c];
+      }
+      if (normals) displacement[i] = dis[3] * mulD;
+      else {
+        for (int c = 0; c < 3; ++c) displacement[(int64_t)c * nn + i] = dis[c];
+        displacement[3 * (int64_t)nn + i] = dis[3] * mulD;
+      }
+    }
+  }
+
+  /* serialize, octree.cpp:907-956 */
+  const int sz = sizeof_octree(&o);
+  char* buf = result_alloc(sz);
+  if (!buf) return ORC_E_NOMEM;
+  memcpy(buf, &o, sizeof(o));
+  {
+    const int kch = channel_of(&o, kKey);
+    uint64_t* kdst = (uint64_t*)prop_ptr(buf, kKey, 0);
+    for (int d = 0; d <= depth; ++d) {
+      if (o.key2xyz) { /* key_to_xyz, octree.cpp:1137-1156: nnum*channel entries, first nnum written */
+        for (int i = 0; i < nnum[d]; ++i) {
+          uint64_t pt[3]; compute_pt(pt, keys[d][i], d);
+          uint16_t f[4] = { (uint16_t)pt[0], (uint16_t)pt[1], (uint16_t)pt[2], 0 };
+          memcpy(kdst + i, f, 8);
+        }
+      } else memcpy(kdst, keys[d], sizeof(uint64_t) * (size_t)nnum[d]);
+      kdst += (o.key2xyz ? (int64_t)nnum[d] * kch : nnum[d]);
+    }
+    int* cdst = (int*)prop_ptr(buf, kChild, 0);
+    for (int d = 0; d <= depth; ++d) { memcpy(cdst, children[d], sizeof(int) * (size_t)nnum[d]); cdst += nnum[d]; }
+    /* features = normals | displacement | point features | average points; location == depth here */
+    float* fdst = (float*)prop_ptr(buf, kFeature, depth);
+    if (fdst) {
+      if (avg_normals) { memcpy(fdst, avg_normals, sizeof(float) * (size_t)ch_normal * nn); fdst += (int64_t)ch_normal * nn; }
+      if (o.has_node_dis) { memcpy(fdst, displacement, sizeof(float) * (size_t)ch_dis * nn); fdst += (int64_t)ch_dis * nn; }
+      if (avg_features) { memcpy(fdst, avg_features, sizeof(float) * (size_t)ch_feature * nn); fdst += (int64_t)ch_feature * nn; }
+      if (o.save_pts) { memcpy(fdst, avg_pts, sizeof(float) * 3 * (size_t)nn); fdst += 3 * (int64_t)nn; }
+    }
+    float* ldst = (float*)prop_ptr(buf, kLabel, depth);
+    if (ldst && avg_labels) memcpy(ldst, avg_labels, sizeof(float) * (size_t)nn);
+    /* calc_split_label (non-adaptive), octree.cpp:1158-1178 */
+    float* sdst = (float*)prop_ptr(buf, kSplit, 0);
+    if (sdst)
+      for (int d = 0; d <= depth; ++d) {
+        for (int i = 0; i < nnum[d]; ++i) sdst[i] = children[d][i] == -1 ? 0.0f : 1.0f;
+        sdst += nnum[d];
+      }
+  }
+  for (int d = 0; d <= 16; ++d) { free(keys[d]); free(children[d]); }
+  free(avg_normals); free(avg_features); free(avg_labels); free(avg_pts); free(displacement);
+  free(pts_scaled); free(node_keys); free(sorted_idx); free(unique_idx);
+  return sz;
+}
+
+/* ------------------------------------------------------------------------ */
+/* merge_octrees: octree/octree/merge_octrees.cpp:7-198,
+ * consistency rule octree_info.cpp:118-130. */
+static int is_consistent(const OInfo* a, const OInfo* b) {
+  return strcmp(a->magic, b->magic) == 0 &&
+      memcmp(a->channels, b->channels, sizeof(a->channels)) == 0 &&
+      memcmp(a->locations, b->locations, sizeof(a->locations)) == 0 &&
+      a->batch_size == b->batch_size && a->depth == b->depth &&
+      a->full_layer == b->full_layer && a->adp_layer == b->adp_layer &&
+      a->is_adaptive == b->is_adaptive && a->key2xyz == b->key2xyz &&
+      a->has_node_dis == b->has_node_dis && a->content_flags == b->content_flags;
+}
+int64_t orc_octree_batch(const void* const* blobs, int B) {
+  if (B < 1) return ORC_E_BADARG;
+  const OInfo* first = (const OInfo*)blobs[0];
+  const int depth = first->depth, full_layer = first->full_layer;
+  if (depth < 1 || depth > 16) return ORC_E_BADARG;
+  for (int i = 0; i < B; ++i) {
+    const OInfo* oi = (const OInfo*)blobs[i];
+    if (strcmp(oi->magic, kMagic) != 0 || !is_consistent(first, oi)) return ORC_E_BADARG;
+  }
+  const int D1 = depth + 1;
+  int* cum = (int*)calloc((size_t)D1 * (size_t)(B + 1), sizeof(int));     /* nnum_cum_layer_ */
+  int* cum_ne = (int*)calloc((size_t)D1 * (size_t)(B + 1), sizeof(int));  /* nnum_cum_nempty_layer_ */
+  for (int d = 0; d < D1; ++d)
+    for (int i = 0; i < B; ++i) {
+      const OInfo* oi = (const OInfo*)blobs[i];
+      cum[(i + 1) * D1 + d] = cum[i * D1 + d] + oi->nnum[d];
+      cum_ne[(i + 1) * D1 + d] = cum_ne[i * D1 + d] + oi->nnum_nempty[d];
+    }
+  OInfo ob = *first; /* set_batch_info, merge_octrees.cpp:92-107 */
+  set_batch_size(&ob, B);
+  set_property(&ob, kNeigh, 8, -1);
+  for (int d = 0; d < D1; ++d) { ob.nnum[d] = cum[B * D1 + d]; ob.nnum_nempty[d] = cum_ne[B * D1 + d]; }
+  set_nnum_cum(&ob, 0);
+  set_ptr_dis(&ob);
+  const int sz = sizeof_octree(&ob);
+  char* out = result_alloc(sz);
+  if (!out) { free(cum); free(cum_ne); return ORC_E_NOMEM; }
+  memcpy(out, &ob, sizeof(ob));
+
+  for (int i = 0; i < B; ++i) {
+    const void* in = blobs[i];
+    const OInfo* oi = (const OInfo*)in;
+    for (int d = 0; d < D1 && has_prop(&ob, kKey); ++d) { /* keys: batch id into sub-field 3 */
+      uint64_t* des = (uint64_t*)prop_ptr(out, kKey, d) + cum[i * D1 + d];
+      const uint64_t* src = (const uint64_t*)prop_ptr(in, kKey, d);
+      for (int j = 0; j < oi->nnum[d]; ++j)
+        des[j] = (src[j] & 0x0000FFFFFFFFFFFFull) | ((uint64_t)(uint16_t)i << 48);
+    }
+    for (int d = 0; d < D1 && has_prop(&ob, kChild); ++d) { /* children: offset by non-empty count */
+      int* des = (int*)prop_ptr(out, kChild, d) + cum[i * D1 + d];
+      const int* src = (const int*)prop_ptr(in, kChild, d);
+      for (int j = 0; j < oi->nnum[d]; ++j) des[j] = src[j] == -1 ? -1 : src[j] + cum_ne[i * D1 + d];
+    }
+    if (has_prop(&ob, kFeature)) { /* features: interleave per channel */
+      int fc = channel_of(&ob, kFeature);
+      int d0 = location_of(&ob, kFeature) == depth ? depth : 0;
+      for (int d = d0; d < D1; ++d)
+        for (int c = 0; c < fc; ++c) {
+          float* des = (float*)prop_ptr(out, kFeature, d) + (int64_t)c * ob.nnum[d] + cum[i * D1 + d];
+          const float* src = (const float*)prop_ptr(in, kFeature, d) + (int64_t)c * oi->nnum[d];
+          memcpy(des, src, sizeof(float) * (size_t)oi->nnum[d]);
+        }
+    }
+    if (has_prop(&ob, kLabel)) {
+      int d0 = location_of(&ob, kLabel) == depth ? depth : 0;
+      for (int d = d0; d < D1; ++d)
+        memcpy((float*)prop_ptr(out, kLabel, d) + cum[i * D1 + d], prop_ptr(in, kLabel, d),
+            sizeof(float) * (size_t)oi->nnum[d]);
+    }
+    if (has_prop(&ob, kSplit)) {
+      int d0 = location_of(&ob, kSplit) == depth ? depth : 0;
+      for (int d = d0; d < D1; ++d)
+        memcpy((float*)prop_ptr(out, kSplit, d) + cum[i * D1 + d], prop_ptr(in, kSplit, d),
+            sizeof(float) * (size_t)oi->nnum[d]);
+    }
+  }
+  for (int d = 1; d < D1; ++d) { /* merge_octrees.cpp:185-197 */
+    if (d <= full_layer) orc_calc_neigh_full((int*)prop_ptr(out, kNeigh, d), d, B);
+    else orc_calc_neigh_sparse((int*)prop_ptr(out, kNeigh, d), (const int*)prop_ptr(out, kNeigh, d - 1),
+        (const int*)prop_ptr(out, kChild, d - 1), ob.nnum[d - 1]);
+  }
+  free(cum); free(cum_ne);
+  return sz;
+}
+
+/* ------------------------------------------------------------------------ */
+/* octree_new / octree_grow / octree_update / octree_set_property:
+ * pytorch/cpp/octree_grow.cpp:13-190, pytorch/cpp/octree_property.cpp:308-325 */
+int64_t orc_octree_new(int batch_size, int channel, int node_dis, int adaptive_layer) {
+  if (batch_size < 1) return ORC_E_BADARG;
+  OInfo o; info_reset(&o);
+  set_batch_size(&o, batch_size);
+  set_depth(&o, 0);
+  set_full_layer(&o, 0);
+  o.has_node_dis = node_dis ? 1 : 0;
+  if (adaptive_layer > 1) { o.is_adaptive = 1; o.adp_layer = adaptive_layer; }
+  o.key2xyz = 1;
+  set_property(&o, kKey, 1, -1);
+  set_property(&o, kChild, 1, -1);
+  set_property(&o, kNeigh, 8, -1);
+  set_property(&o, kFeature, channel, -1);
+  for (int i = 0; i < 3; ++i) { o.bbmin[i] = 0.0f; o.bbmax[i] = 2.0f; }
+  o.nnum[0] = batch_size;
+  set_nnum_cum(&o, 0);
+  o.nnum_nempty[0] = batch_size;
+  set_ptr_dis(&o);
+  int sz = sizeof_octree(&o);
+  char* out = result_alloc(sz);
+  if (!out) return ORC_E_NOMEM;
+  memcpy(out, &o, sizeof(o));
+  uint64_t* key = (uint64_t*)prop_ptr(out, kKey, 0);
+  int* child = (int*)prop_ptr(out, kChild, 0);
+  for (int i = 0; i < batch_size; ++i) { key[i] = (uint64_t)i; child[i] = i; }
+  return sz;
+}
+int64_t orc_octree_grow(const void* in, int target_depth, int full_octree) {
+  const OInfo* oi = (const OInfo*)in;
+  if (target_depth < 1 || target_depth > 15) return ORC_E_BADARG;
+  const int batch = oi->batch_size;
+  const int node_num = oi->nnum_nempty[target_depth - 1] << 3;
+  OInfo o = *oi; /* update_octreeinfo, octree_grow.cpp:57-73 */
+  set_depth(&o, target_depth);
+  if (full_octree) set_full_layer(&o, target_depth);
+  float width = (float)(1 << target_depth);
+  for (int i = 0; i < 3; ++i) { o.bbmin[i] = 0.0f; o.bbmax[i] = width; }
+  o.nnum[target_depth] = node_num;
+  o.nnum_nempty[target_depth] = node_num;
+  set_nnum_cum(&o, 0);
+  set_ptr_dis(&o);
+  int sz = sizeof_octree(&o);
+  char* out = result_alloc(sz);
+  if (!out) return ORC_E_NOMEM;
+  memcpy(out, &o, sizeof(o));
+  /* copy_octree_gpu, octree_grow.cpp:75-87 */
+  int64_t ncum = oi->nnum_cum[target_depth];
+  memcpy(prop_ptr(out, kKey, 0), prop_ptr(in, kKey, 0), 8 * (size_t)(ncum * channel_of(oi, kKey)));
+  memcpy(prop_ptr(out, kChild, 0), prop_ptr(in, kChild, 0), 4 * (size_t)(ncum * channel_of(oi, kChild)));
+  memcpy(prop_ptr(out, kNeigh, 0), prop_ptr(in, kNeigh, 0), 4 * (size_t)(ncum * channel_of(oi, kNeigh)));
+  if (has_prop(oi, kFeature))
+    memcpy(prop_ptr(out, kFeature, 0), prop_ptr(in, kFeature, 0), 4 * (size_t)(ncum * channel_of(oi, kFeature)));
+  int* neigh = (int*)prop_ptr(out, kNeigh, target_depth);
+  uint64_t* key = (uint64_t*)prop_ptr(out, kKey, target_depth);
+  int* child = (int*)prop_ptr(out, kChild, target_depth);
+  if (full_octree) {
+    orc_calc_neigh_full(neigh, target_depth, batch);
+    orc_generate_key_full(key, target_depth, batch);
+  } else {
+    const int* label = (const int*)prop_ptr(out, kChild, target_depth - 1);
+    orc_calc_neigh_sparse(neigh, (const int*)prop_ptr(out, kNeigh, target_depth - 1), label,
+        o.nnum[target_depth - 1]);
+    orc_generate_key_child(key, (const uint64_t*)prop_ptr(out, kKey, target_depth - 1), label,
+        o.nnum[target_depth - 1]);
+  }
+  for (int i = 0; i < node_num; ++i) child[i] = i;
+  return sz;
+}
+int64_t orc_octree_update(const void* in, const int* label, int n_label, int depth, int split) {
+  const OInfo* oi = (const OInfo*)in;
+  if (n_label != oi->nnum[depth]) return ORC_E_BADARG;
+  int sz = sizeof_octree(oi);
+  char* out = result_alloc(sz);
+  if (!out) return ORC_E_NOMEM;
+  memcpy(out, in, (size_t)sz);
+  int* children = (int*)prop_ptr(out, kChild, depth);
+  int split_num = orc_generate_label(children, label, n_label, split);
+  if (split_num == 0) { split_num = 1; children[0] = 0; }
+  ((OInfo*)out)->nnum_nempty[depth] = split_num;
+  return sz;
+}
+int64_t orc_octree_set_property(const void* in, const float* data, int64_t count, int depth) {
+  const OInfo* oi = (const OInfo*)in;
+  if (count != (int64_t)oi->nnum[depth] * channel_of(oi, kFeature)) return ORC_E_BADARG;
+  int sz = sizeof_octree(oi);
+  char* out = result_alloc(sz);
+  if (!out) return ORC_E_NOMEM;
+  memcpy(out, in, (size_t)sz);
+  memcpy(prop_ptr(out, kFeature, depth), data, sizeof(float) * (size_t)count);
+  return sz;
+}
