@@ -1,0 +1,226 @@
+/* C-ABI of libocnn_hip.so: the O-CNN octree hot path as hand-written HIP
+ * kernels for gfx950 (MI355X).
+ *
+ * Conventions
+ *  - Every entry point returns 0 on success or a negative OCNN_E_* code; the
+ *    message of the last failure on the calling thread is ocnn_last_error().
+ *    Nothing aborts the process (the reference CHECK()s abort:
+ *    octree/octree/logs.h:23-29).
+ *  - Pointers named *_dev / data / top / btm / col / neigh / key ... are DEVICE
+ *    pointers; `info` is always a HOST pointer to the 716-byte OctreeInfo
+ *    header of the blob (octree/octree/octree_info.h:96-118).  The reference
+ *    re-reads that header from the device with a blocking copy on every call
+ *    (octree/octree/octree_parser.cu:4-27); here the caller keeps a host copy.
+ *  - The caller owns every buffer; the library allocates nothing and never
+ *    synchronises unless the function says so.  `stream` is a hipStream_t
+ *    (NULL = default stream); all work of a call is enqueued on it.
+ *  - Feature tensors are channel-major [C, H] as in the reference
+ *    (pytorch/cpp/octree2col.cpp:59-62).  `dtype` selects the element type of
+ *    feature/weight buffers: OCNN_F32 (reference precision) or OCNN_BF16
+ *    (bf16 storage, fp32 accumulate; no counterpart in the reference, whose
+ *    ops are float/double only: octree/octree/octree_conv.cpp:360-361).
+ *  - Keys are 64-bit (the reference's KEY64 build, mandatory for its PyTorch
+ *    frontend: pytorch/setup.py:29,58); child/neigh/mask/label are int32.
+ *  - Neighbour index tables (`ni`, `parent`, `dis` of NeighHelper,
+ *    octree/octree/octree_nn.cpp:6-81) live inside the library; where the
+ *    reference takes a device `ni` pointer these functions take the host
+ *    `kernel_size[3]` instead.
+ */
+#ifndef OCNN_HIP_H_
+#define OCNN_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* ocnn_stream_t; /* hipStream_t */
+
+enum { OCNN_F32 = 0, OCNN_BF16 = 1 };
+
+enum {
+  OCNN_OK = 0,
+  OCNN_E_BADARG = -1,      /* null pointer, negative size, bad enum */
+  OCNN_E_UNSUPPORTED = -2, /* valid request this build does not implement */
+  OCNN_E_SHAPE = -3,       /* tensor height/channel disagrees with the octree */
+  OCNN_E_WORKSPACE = -4,   /* workspace missing or too small */
+  OCNN_E_HIP = -5,         /* a HIP runtime call failed */
+  OCNN_E_FORMAT = -6       /* malformed OctreeInfo / PointsInfo header */
+};
+
+/* property selectors = OctreeInfo::PropType (octree/octree/octree_info.h:12-14) */
+enum { OCNN_KEY = 1, OCNN_CHILD = 2, OCNN_NEIGH = 4, OCNN_FEATURE = 8, OCNN_LABEL = 16, OCNN_SPLIT = 32 };
+
+#define OCNN_INFO_BYTES 716   /* sizeof(OctreeInfo) */
+#define OCNN_HEADER_BYTES 720 /* payload offset, octree_info.cpp:258 */
+#define OCNN_POINTS_INFO_BYTES 88 /* sizeof(PointsInfo), points_info.h:35-39 */
+
+const char* ocnn_last_error(void);
+int ocnn_version(void);
+/* 0 when device `dev` exists and is a gfx950 part. */
+int ocnn_device_check(int dev);
+
+/* ---- OctreeInfo accessors (host only).  Replace OctreeInfo::node_num() etc.,
+ * octree/octree/octree_info.h:34-61 and check_format octree_info.cpp:80-116. */
+int ocnn_info_check(const void* info);
+int ocnn_info_batch_size(const void* info);
+int ocnn_info_depth(const void* info);
+int ocnn_info_full_depth(const void* info);
+int ocnn_info_is_key2xyz(const void* info);
+int ocnn_info_node_num(const void* info, int depth);
+int ocnn_info_node_num_nempty(const void* info, int depth);
+int ocnn_info_node_num_cum(const void* info, int depth);
+int ocnn_info_total_nnum(const void* info);
+int ocnn_info_channel(const void* info, int ptype);
+int ocnn_info_location(const void* info, int ptype);
+/* byte offset of a property at a depth inside the blob, -1 if absent
+ * (OctreeInfo::ptr_dis, octree_info.cpp:157-167) */
+int64_t ocnn_info_ptr_dis(const void* info, int ptype, int depth);
+int64_t ocnn_info_sizeof_octree(const void* info);
+
+/* ---- padding: pad_forward_gpu / pad_backward_gpu, octree/octree/octree_nn.h:69-77,
+ * octree_nn.cu:65-106.  pad_backward writes only the rows label[] names. */
+int ocnn_pad_forward(void* Y, int Hy, int C, const void* X, int Hx, const int* label,
+    float dval, int dtype, ocnn_stream_t stream);
+int ocnn_pad_backward(void* X, int Hx, int C, const void* Y, int Hy, const int* label,
+    int dtype, ocnn_stream_t stream);
+/* int32 variant used to invert `children` into `ichild`
+ * (pytorch/cpp/octree2col.cpp:10-20): ichild[child[h]] = h. */
+int ocnn_make_ichild(int* ichild, int n_nempty, const int* child, int n_node, ocnn_stream_t stream);
+
+/* ---- octree2col / col2octree: octree/octree/octree_nn.h:80-120, octree_nn.cu:110-253.
+ * Same argument meaning as the reference; `kernel_size` (host) replaces `ni`. */
+int ocnn_octree2col(void* col, const void* data, int channel, int height, const int* kernel_size,
+    int stride, const int* neigh, int height_col, int n, int dtype, ocnn_stream_t stream);
+int ocnn_col2octree(const void* col, void* data, int channel, int height, const int* kernel_size,
+    int stride, const int* neigh, int height_col, int n, int dtype, ocnn_stream_t stream);
+int ocnn_octree2colP(void* col, const void* data, int channel, int height, int octree_h,
+    const int* kernel_size, int stride, const int* neigh, const int* child, const int* ichild,
+    int height_col, int n, int dtype, ocnn_stream_t stream);
+int ocnn_col2octreeP(const void* col, void* data, int channel, int height, int octree_h,
+    const int* kernel_size, int stride, const int* neigh, const int* child, const int* ichild,
+    int height_col, int n, int dtype, ocnn_stream_t stream);
+
+/* ---- pooling: octree/octree/octree_nn.h:122-139, octree_nn.cu:258-327.
+ * mask holds absolute row indices; the first maximum wins. */
+int ocnn_octree_max_pool(void* top, int top_h, int* mask, const void* btm, int btm_h,
+    int channel, int dtype, ocnn_stream_t stream);
+int ocnn_octree_max_unpool(const void* top, int top_h, const int* mask, void* btm, int btm_h,
+    int channel, int dtype, ocnn_stream_t stream);
+int ocnn_octree_mask_pool(void* top, int top_h, const int* mask, const void* btm, int btm_h,
+    int channel, int dtype, ocnn_stream_t stream);
+
+/* ---- neighbour tables: calc_neigh_gpu (both overloads),
+ * octree/octree/octree_nn.h:142-147, octree_nn.cu:331-413. */
+int ocnn_calc_neigh_sparse(int* neigh_child, const int* neigh, const int* children,
+    int node_num, ocnn_stream_t stream);
+int ocnn_calc_neigh_full(int* neigh, int depth, int batch_size, ocnn_stream_t stream);
+
+/* ---- keys / labels: octree/octree/octree_nn.h:150-192, 229-240,
+ * octree_nn.cu:417-488, 575-665. */
+int ocnn_generate_key_child(uint64_t* key_child, const uint64_t* key, const int* child,
+    int node_num, ocnn_stream_t stream);
+int ocnn_generate_key_full(uint64_t* key, int depth, int batch_size, ocnn_stream_t stream);
+/* label[i] = (btm[i]==mask) ? running count : -1; the count goes to *count_dev
+ * (device int).  scratch_dev: at least ocnn_generate_label_scratch_bytes(btm_h). */
+size_t ocnn_generate_label_scratch_bytes(int btm_h);
+int ocnn_generate_label(int* label, int* count_dev, const int* btm, int btm_h, int mask,
+    void* scratch_dev, size_t scratch_bytes, ocnn_stream_t stream);
+int ocnn_sequence(int* ptr, int num, ocnn_stream_t stream);
+int ocnn_search_key(int* idx, const uint64_t* key, int n_key, const uint64_t* query,
+    int n_query, ocnn_stream_t stream);
+int ocnn_xyz2key(uint64_t* key, const uint64_t* xyz, int num, int depth, ocnn_stream_t stream);
+int ocnn_key2xyz(uint64_t* xyz, const uint64_t* key, int num, int depth, ocnn_stream_t stream);
+int ocnn_key2idx(int* idx, const uint64_t* key, int num, ocnn_stream_t stream);
+
+/* ---- octree convolution / deconvolution: OctreeConvOp / OctreeDeconvOp,
+ * pytorch/cpp/octree_conv.cpp:131-213, shape rules octree/octree/octree_conv.cpp:10-122.
+ * Implemented as an implicit GEMM on the matrix cores: the neighbour gather
+ * feeds MFMA directly, no [Cin*K, H] column buffer is materialised.
+ *   weights: [conv_out, conv_in*K] row-major with column index c*K + k
+ *            (conv: [num_output, channel_in*K]; deconv: [channel_in, num_output*K])
+ *   btm:     [channel_in, btm_h]     top: [num_output, top_h]
+ * ocnn_conv_shape fills the output height, the input height the octree
+ * demands (pytorch/cpp/octree_conv.cpp:72-78) and the workspace the call needs. */
+int ocnn_conv_shape(const void* info, int depth, int channel_in, int num_output,
+    const int* kernel_size, int stride, int nempty, int is_deconv, int dtype,
+    int* top_h, int* btm_h, size_t* workspace_bytes);
+int ocnn_octree_conv(void* top, const void* btm, int channel_in, int btm_h, const void* weights,
+    const void* octree_dev, const void* info, int depth, int num_output, const int* kernel_size,
+    int stride, int nempty, int dtype, void* workspace_dev, size_t workspace_bytes,
+    ocnn_stream_t stream);
+int ocnn_octree_deconv(void* top, const void* btm, int channel_in, int btm_h, const void* weights,
+    const void* octree_dev, const void* info, int depth, int num_output, const int* kernel_size,
+    int stride, int nempty, int dtype, void* workspace_dev, size_t workspace_bytes,
+    ocnn_stream_t stream);
+
+/* ---- octree construction on the device: points2octree + octree_batch fused.
+ * Replaces Octree::build (octree/octree/octree.cpp:74-121) driven as in
+ * pytorch/cpp/point2octree.cpp:5-34, and merge_octrees
+ * (octree/octree/merge_octrees.cpp:7-198) driven as in pytorch/cpp/octree_batch.cpp:5-22.
+ *
+ * One call builds n_clouds point clouds; the result is bit-identical to what
+ * the reference produces for points2octree on each cloud (n_clouds == 1 and
+ * merged == 0) or for octree_batch over those octrees (merged == 1, which
+ * also fills the neighbour tables).
+ *
+ *   points_dev[i]   device pointer to the i-th serialized point cloud
+ *   points_info[i]  host pointer to its 88-byte PointsInfo header
+ * Step 1 (ocnn_points2octree_plan) sorts the points and counts the nodes; it
+ * ends with ONE device-to-host copy of the node counts, waits for it, and
+ * writes the finished OctreeInfo header to `info_out` (host).  The caller then
+ * allocates ocnn_info_sizeof_octree(info_out) bytes and step 2
+ * (ocnn_points2octree_emit) writes the blob.  The workspace must stay
+ * untouched between the two steps.
+ * The adaptive / node_feature / extrapolate options of the reference
+ * (octree.cpp:454-806, 958-1135) are not implemented: OCNN_E_UNSUPPORTED. */
+typedef struct {
+  int depth, full_depth;
+  int node_dis, node_feature, split_label, adaptive, adp_depth;
+  float th_normal, th_distance;
+  int extrapolate, save_pts, key2xyz;
+  int merged;          /* 0: single-octree blob (n_clouds must be 1); 1: octree_batch blob */
+  int has_bbox;        /* 0: [-1,1]^3 as pytorch/cpp does (octree_info.cpp:68-69) */
+  float bbmin[3], bbmax[3];
+} ocnn_build_params;
+size_t ocnn_points2octree_workspace_bytes(int64_t total_points, int n_clouds, int depth);
+int ocnn_points2octree_plan(const void* const* points_dev, const void* const* points_info,
+    int n_clouds, const ocnn_build_params* params, void* workspace_dev, size_t workspace_bytes,
+    void* info_out, ocnn_stream_t stream);
+int ocnn_points2octree_emit(void* octree_out_dev, const void* info, void* workspace_dev,
+    size_t workspace_bytes, ocnn_stream_t stream);
+
+/* ---- octree_batch of already serialized octrees that live on the device
+ * (merge_octrees, octree/octree/merge_octrees.cpp:7-198).  `out_info` (host)
+ * is filled by ocnn_octree_batch_info from the n host headers; the caller
+ * allocates ocnn_info_sizeof_octree(out_info) bytes for `out_dev`. */
+int ocnn_octree_batch_info(const void* const* infos, int n, void* out_info);
+size_t ocnn_octree_batch_workspace_bytes(int n, int depth);
+/* waits once for its (small) host-to-device table upload before returning */
+int ocnn_octree_batch(void* out_dev, const void* out_info, const void* const* octrees_dev,
+    const void* const* infos, int n, void* workspace_dev, size_t workspace_bytes,
+    ocnn_stream_t stream);
+
+/* ---- decoder-side growth: octree_new / octree_grow / octree_update,
+ * pytorch/cpp/octree_grow.cpp:13-190.  The *_info functions compute the
+ * header of the result on the host; the caller allocates and the second
+ * function fills the blob on the device (the header is written too). */
+int ocnn_octree_new_info(int batch_size, int channel, int node_dis, int adaptive_layer, void* out_info);
+int ocnn_octree_new(void* out_dev, const void* out_info, ocnn_stream_t stream);
+int ocnn_octree_grow_info(const void* in_info, int target_depth, int full_octree, void* out_info);
+int ocnn_octree_grow(void* out_dev, const void* out_info, const void* in_dev, const void* in_info,
+    int target_depth, int full_octree, ocnn_stream_t stream);
+/* octree_update rewrites children[depth] of `octree_dev` IN PLACE from
+ * `label` (the caller clones first, as pytorch/cpp/octree_grow.cpp:165 does),
+ * copies the split count back (one device-to-host copy, waited for), patches
+ * nnum_nempty[depth] in `info` (host) and in the device header. */
+size_t ocnn_octree_update_scratch_bytes(int n_label);
+int ocnn_octree_update(void* octree_dev, void* info, const int* label, int n_label, int depth,
+    int split, void* scratch_dev, size_t scratch_bytes, ocnn_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OCNN_HIP_H_ */

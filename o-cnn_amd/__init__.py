@@ -1,0 +1,15 @@
+"""MI355X-native octree hot path of O-CNN.
+
+The directory name is not a Python identifier; load the package with
+`importlib.import_module("o-cnn_amd")` (the repository root on sys.path).
+
+  nn        -- mirror of the reference's `ocnn.nn` extension functions
+               (pytorch/cpp/pybind.cpp:3-49) over libocnn_hip.so
+  layers    -- mirror of the thin Python modules of pytorch/ocnn
+               (octree_conv.py, octree_pool.py, octree_pad.py)
+  synthetic -- seeded synthetic point clouds of the benchmark configurations
+"""
+from . import lib, nn, layers, synthetic  # noqa: F401
+from .nn import *  # noqa: F401,F403
+from .layers import (OctreeConv, OctreeDeconv, OctreeConvFast, OctreeDeconvFast,  # noqa: F401
+                     OctreeMaxPool, OctreeMaxUnpool, OctreeAvgPool, OctreePad, OctreeDepad)

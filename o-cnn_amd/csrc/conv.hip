@@ -1,0 +1,406 @@
+// Octree convolution / deconvolution as an implicit GEMM on the CDNA4 matrix
+// cores.  The reference computes  top = W[Co, Ci*K] x octree2col(btm)[Ci*K, H]
+// through a column buffer in HBM (octree/octree/octree_conv.cpp:276-325); here
+// the gather through the neighbour table feeds MFMA operands directly:
+//
+//   out[m, n] = sum_{tap k} sum_{c}  A[k][m][c] * in[c, src(n, k)]
+//
+// One wavefront owns 64 output columns (two 32-wide MFMA column tiles) and all
+// output channels (MT row tiles of 32 per pass).  For every tap it looks up the
+// source row of its columns once, then walks the input channels feeding
+// v_mfma_f32_32x32x2_f32 (fp32) or v_mfma_f32_32x32x16_bf16 (bf16 storage, fp32
+// accumulate).  Weights are re-laid out once per call into MFMA A-fragment
+// order so that each fragment is one coalesced 256-byte (fp32) or 1-KiB (bf16)
+// load shared by all wavefronts through the vector L1.
+#include "ocnn_common.h"
+
+namespace ocnn {
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+enum { kModeS1 = 0, kModeS2Conv = 1, kModeS2Deconv = 2 };
+
+struct ConvArgs {
+  int M, Cin, N, K;     // output channels, input channels, output columns, taps
+  int Hin, Hout;        // row lengths of the input / output tensors
+  int mode, nempty;
+  int mtiles;           // ceil(M / 32)
+  int csteps;           // channel steps per tap: ceil(Cin/2) fp32, ceil(Cin/16) bf16
+  int slot[27];         // neighbour slot of tap k for sibling 0
+  const int* neigh;
+  const int* child;
+  const int* ichild;
+};
+
+constexpr int kWaveCols = 64;                 // output columns per wavefront
+constexpr int kConvWaves = 4;                 // wavefronts per workgroup
+constexpr int kTileCols = kWaveCols * kConvWaves;
+
+// source row of output column n for tap k (-1: contributes zero)
+__device__ inline int conv_src(const ConvArgs& a, int n, int k) {
+  if (n >= a.N) return -1;
+  int p;
+  if (a.mode == kModeS1) {
+    int node = a.nempty ? a.ichild[n] : n;
+    p = a.neigh[((int64_t)(node >> 3) << 6) + sibling_slot(node & 7) + a.slot[k]];
+    if (a.nempty && p >= 0) p = a.child[p];
+  } else if (a.mode == kModeS2Conv) {
+    p = a.neigh[((int64_t)n << 6) + a.slot[k]];
+    if (a.nempty && p >= 0) p = a.child[p];
+  } else {
+    int node = a.nempty ? a.ichild[n] : n;
+    p = (k == (node & 7)) ? (node >> 3) : -1;
+  }
+  return (p >= 0 && p < a.Hin) ? p : -1;
+}
+
+// XCD-aware tile order: consecutive workgroup ids land on different XCDs, so give
+// each XCD one contiguous range of column tiles (neighbouring tiles share
+// neighbour rows, which then stay in that XCD's L2).
+__device__ inline int xcd_tile(int bid, int n_tiles) {
+  constexpr int kXcd = 8;
+  int per = (n_tiles + kXcd - 1) / kXcd;
+  return (bid % kXcd) * per + bid / kXcd;
+}
+
+// ---- weight re-layout ----------------------------------------------------------
+// W'(m, c, k) = W[m*sm + c*sc + k]; conv: sm = Cin*K, sc = K; deconv: sm = K, sc = M*K.
+// fp32 fragment (tap, cstep, mtile): lane l holds A[m = 32*mtile + (l&31)][c = 2*cstep + (l>>5)].
+__global__ void pack_weights_f32(float* __restrict__ Wt, const float* __restrict__ W, int M, int Cin, int K,
+    int mtiles, int csteps, int64_t sm, int64_t sc) {
+  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t total = (int64_t)K * csteps * mtiles * 64;
+  if (id >= total) return;
+  int l = (int)(id & 63);
+  int64_t f = id >> 6;
+  int mt = (int)(f % mtiles);
+  f /= mtiles;
+  int cs = (int)(f % csteps);
+  int k = (int)(f / csteps);
+  int m = mt * 32 + (l & 31), c = 2 * cs + (l >> 5);
+  Wt[id] = (m < M && c < Cin) ? W[m * sm + c * sc + k] : 0.0f;
+}
+// bf16 fragment: lane l holds A[m = 32*mtile + (l&31)][c = 16*cstep + 8*(l>>5) + j], j = 0..7
+__global__ void pack_weights_bf16(uint16_t* __restrict__ Wt, const uint16_t* __restrict__ W, int M, int Cin,
+    int K, int mtiles, int csteps, int64_t sm, int64_t sc) {
+  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t total = (int64_t)K * csteps * mtiles * 64 * 8;
+  if (id >= total) return;
+  int j = (int)(id & 7);
+  int l = (int)((id >> 3) & 63);
+  int64_t f = id >> 9;
+  int mt = (int)(f % mtiles);
+  f /= mtiles;
+  int cs = (int)(f % csteps);
+  int k = (int)(f / csteps);
+  int m = mt * 32 + (l & 31), c = 16 * cs + 8 * (l >> 5) + j;
+  Wt[id] = (m < M && c < Cin) ? W[m * sm + c * sc + k] : (uint16_t)0;
+}
+
+// ---- main kernels ----------------------------------------------------------------
+// Accumulator layout of the 32x32 MFMA: lane l, register i holds
+// D[row = 8*(i/4) + 4*(l>>5) + (i%4)][col = l&31].
+template <typename OutT, int MT>
+__device__ inline void store_tiles(const ConvArgs& a, OutT* __restrict__ out, floatx16 (&acc)[MT][2],
+    int mt0, int n0, int lane) {
+  const int r = lane & 31, kh = lane >> 5;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      int n = n0 + nt * 32 + r;
+      if (n >= a.N) continue;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        int m = (mt0 + mt) * 32 + 8 * (i / 4) + 4 * kh + (i % 4);
+        if (m < a.M) {
+          if (sizeof(OutT) == 4) reinterpret_cast<float*>(out)[(int64_t)m * a.Hout + n] = acc[mt][nt][i];
+          else reinterpret_cast<uint16_t*>(out)[(int64_t)m * a.Hout + n] = f32_to_bf16(acc[mt][nt][i]);
+        }
+      }
+    }
+}
+
+template <int MT>
+__global__ __launch_bounds__(kConvWaves * 64) void conv_f32_kernel(ConvArgs a, float* __restrict__ out,
+    const float* __restrict__ in, const float* __restrict__ Wt, int n_tiles) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = xcd_tile(blockIdx.x, n_tiles);
+  if (tile >= n_tiles) return;
+  const int n0 = tile * kTileCols + wave * kWaveCols;
+  if (n0 >= a.N) return;
+  const int r = lane & 31, kh = lane >> 5;
+
+  for (int mt0 = 0; mt0 < a.mtiles; mt0 += MT) {
+    floatx16 acc[MT][2];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
+
+    for (int k = 0; k < a.K; ++k) {
+      const int s0 = conv_src(a, n0 + r, k), s1 = conv_src(a, n0 + 32 + r, k);
+      const float* wk = Wt + ((int64_t)k * a.csteps * a.mtiles + mt0) * 64 + lane;
+#pragma unroll 4
+      for (int cs = 0; cs < a.csteps; ++cs) {
+        const int c = 2 * cs + kh;
+        const bool cv = c < a.Cin;
+        float b0 = (cv && s0 >= 0) ? in[(int64_t)c * a.Hin + s0] : 0.0f;
+        float b1 = (cv && s1 >= 0) ? in[(int64_t)c * a.Hin + s1] : 0.0f;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          float av = (mt0 + mt < a.mtiles) ? wk[((int64_t)cs * a.mtiles + mt) * 64] : 0.0f;
+          acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b0, acc[mt][0], 0, 0, 0);
+          acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b1, acc[mt][1], 0, 0, 0);
+        }
+      }
+    }
+    store_tiles<float, MT>(a, out, acc, mt0, n0, lane);
+  }
+}
+
+template <int MT>
+__global__ __launch_bounds__(kConvWaves * 64) void conv_bf16_kernel(ConvArgs a, uint16_t* __restrict__ out,
+    const uint16_t* __restrict__ in, const uint16_t* __restrict__ Wt, int n_tiles) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = xcd_tile(blockIdx.x, n_tiles);
+  if (tile >= n_tiles) return;
+  const int n0 = tile * kTileCols + wave * kWaveCols;
+  if (n0 >= a.N) return;
+  const int r = lane & 31, kh = lane >> 5;
+
+  for (int mt0 = 0; mt0 < a.mtiles; mt0 += MT) {
+    floatx16 acc[MT][2];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
+
+    for (int k = 0; k < a.K; ++k) {
+      const int s0 = conv_src(a, n0 + r, k), s1 = conv_src(a, n0 + 32 + r, k);
+      const uint4* wk = reinterpret_cast<const uint4*>(Wt) + ((int64_t)k * a.csteps * a.mtiles + mt0) * 64 + lane;
+      for (int cs = 0; cs < a.csteps; ++cs) {
+        const int cb = 16 * cs + 8 * kh;
+        union { uint16_t u[8]; bf16x8 v; } b0, b1;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int c = cb + j;
+          const bool cv = c < a.Cin;
+          b0.u[j] = (cv && s0 >= 0) ? in[(int64_t)c * a.Hin + s0] : (uint16_t)0;
+          b1.u[j] = (cv && s1 >= 0) ? in[(int64_t)c * a.Hin + s1] : (uint16_t)0;
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          union { uint4 q; bf16x8 v; } av;
+          av.q = (mt0 + mt < a.mtiles) ? wk[((int64_t)cs * a.mtiles + mt) * 64] : make_uint4(0, 0, 0, 0);
+          acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b0.v, acc[mt][0], 0, 0, 0);
+          acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b1.v, acc[mt][1], 0, 0, 0);
+        }
+      }
+    }
+    store_tiles<uint16_t, MT>(a, out, acc, mt0, n0, lane);
+  }
+}
+
+template <typename T>
+__global__ void zero_rows_kernel(T* p, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += step) p[i] = (T)0;
+}
+
+__global__ void ichild_kernel(int* __restrict__ ichild, int n_nempty, const int* __restrict__ child, int n) {
+  int h = blockIdx.x * blockDim.x + threadIdx.x;
+  if (h >= n) return;
+  int l = child[h];
+  if (l >= 0 && l < n_nempty) ichild[l] = h;
+}
+
+// Shape rules of OctreeBaseConv::reshape (octree/octree/octree_conv.cpp:48-104)
+// and the input-height check of pytorch/cpp/octree_conv.cpp:72-78.
+struct ConvPlan {
+  int top_depth, workspace_depth, top_h, btm_h, workspace_h;
+  int child_h, ichild_h;
+  int mode;
+  KernelTaps taps;
+  int mtiles, csteps;
+  size_t wt_bytes, ichild_bytes, total_bytes;
+};
+
+inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+int make_plan(const Info* o, int depth, int channel_in, int num_output, const int* ks, int stride,
+    int nempty, int deconv, int dtype, ConvPlan* p) {
+  OCNN_REQUIRE(o && ks, OCNN_E_BADARG, "null pointer");
+  int e = ocnn_info_check(o);
+  if (e) return e;
+  OCNN_REQUIRE(depth > 0 && depth <= o->depth, OCNN_E_BADARG, "depth %d not in [1,%d]", depth, o->depth);
+  OCNN_REQUIRE(num_output > 0 && channel_in > 0, OCNN_E_BADARG, "channels %d -> %d", channel_in, num_output);
+  OCNN_REQUIRE(stride == 1 || stride == 2, OCNN_E_BADARG, "stride %d", stride);
+  OCNN_REQUIRE(dtype == OCNN_F32 || dtype == OCNN_BF16, OCNN_E_BADARG, "dtype %d", dtype);
+  OCNN_REQUIRE(kernel_taps(ks, &p->taps), OCNN_E_UNSUPPORTED, "kernel size %d%d%d", ks[0], ks[1], ks[2]);
+  OCNN_REQUIRE(o->has(OCNN_NEIGH) && o->has(OCNN_CHILD), OCNN_E_FORMAT,
+      "the octree holds no neighbour table (not an octree_batch result)");
+  p->top_depth = p->workspace_depth = depth;
+  if (stride == 2) {
+    if (deconv) p->top_depth = p->workspace_depth = depth + 1;
+    else p->top_depth = depth - 1;
+    OCNN_REQUIRE(p->top_depth >= 0 && p->top_depth <= o->depth, OCNN_E_BADARG,
+        "output depth %d outside the octree", p->top_depth);
+  }
+  int top_h;
+  if (!nempty) {
+    top_h = o->nnum[p->top_depth];
+    if (stride == 2 && !deconv) top_h = o->nnum_nempty[p->top_depth];
+  } else {
+    top_h = o->nnum_nempty[p->top_depth];
+  }
+  if (top_h == 0) top_h = 1;
+  p->top_h = top_h;
+  p->workspace_h = top_h;
+  if (stride == 2) p->workspace_h = deconv ? o->nnum[p->top_depth] / 8 : o->nnum[depth] / 8;
+  p->btm_h = ((stride == 2 && deconv) || nempty) ? o->nnum_nempty[depth] : o->nnum[depth];
+  p->child_h = o->nnum[p->workspace_depth];
+  p->ichild_h = o->nnum_nempty[p->workspace_depth];
+  if (stride == 1) p->mode = kModeS1;
+  else if (!deconv) p->mode = kModeS2Conv;
+  else {
+    OCNN_REQUIRE(ks[0] == 2 && ks[1] == 2 && ks[2] == 2, OCNN_E_UNSUPPORTED,
+        "stride-2 deconvolution is implemented for the 2x2x2 kernel only");
+    p->mode = kModeS2Deconv;
+  }
+  p->mtiles = (num_output + 31) / 32;
+  p->csteps = dtype == OCNN_F32 ? (channel_in + 1) / 2 : (channel_in + 15) / 16;
+  size_t frag = dtype == OCNN_F32 ? 64 * sizeof(float) : 64 * 8 * sizeof(uint16_t);
+  p->wt_bytes = align256((size_t)p->taps.count * p->csteps * p->mtiles * frag);
+  p->ichild_bytes = nempty ? align256(sizeof(int) * (size_t)(p->ichild_h + 1)) : 0;
+  p->total_bytes = p->wt_bytes + p->ichild_bytes;
+  return OCNN_OK;
+}
+
+int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, const void* weights,
+    const void* octree_dev, const void* info, int depth, int num_output, const int* ks, int stride,
+    int nempty, int dtype, void* ws, size_t ws_bytes, hipStream_t s) {
+  OCNN_REQUIRE(top && btm && weights && octree_dev && info, OCNN_E_BADARG, "null pointer");
+  const Info* o = as_info(info);
+  ConvPlan p;
+  int e = make_plan(o, depth, channel_in, num_output, ks, stride, nempty, deconv, dtype, &p);
+  if (e) return e;
+  OCNN_REQUIRE(btm_h == p.btm_h, OCNN_E_SHAPE, "input height %d, the octree has %d rows at depth %d",
+      btm_h, p.btm_h, depth);
+  OCNN_REQUIRE(ws && ws_bytes >= p.total_bytes, OCNN_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes,
+      p.total_bytes);
+  OCNN_REQUIRE((reinterpret_cast<uintptr_t>(ws) & 15) == 0, OCNN_E_WORKSPACE, "workspace not 16-byte aligned");
+
+  const char* blob = static_cast<const char*>(octree_dev);
+  ConvArgs a;
+  a.M = num_output;
+  a.Cin = channel_in;
+  a.N = p.top_h;
+  a.K = p.taps.count;
+  a.Hin = btm_h;
+  a.Hout = p.top_h;
+  a.mode = p.mode;
+  a.nempty = nempty ? 1 : 0;
+  a.mtiles = p.mtiles;
+  a.csteps = p.csteps;
+  for (int k = 0; k < 27; ++k) {
+    int tap = k < p.taps.count ? p.taps.tap[k] : 13;
+    // deconvolution gathers through the mirrored offset: the rows h that scatter
+    // to p through tap k are exactly the neighbours of p at the opposite offset
+    a.slot[k] = tap_slot(deconv ? 26 - tap : tap);
+  }
+  a.neigh = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_NEIGH, p.workspace_depth));
+  a.child = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_CHILD, p.workspace_depth));
+  a.ichild = nullptr;
+  // degenerate layer without nodes: the reference emits one zero column
+  // (octree_conv.cpp:82) -- nothing to gather
+  bool empty_layer = (nempty ? o->nnum_nempty[p.top_depth] : (stride == 2 && !deconv
+      ? o->nnum_nempty[p.top_depth] : o->nnum[p.top_depth])) == 0;
+  if (empty_layer) {
+    int64_t cnt = (int64_t)num_output * p.top_h;
+    if (dtype == OCNN_F32) zero_rows_kernel<float><<<blocks_for(cnt), kBlock, 0, s>>>((float*)top, cnt);
+    else zero_rows_kernel<uint16_t><<<blocks_for(cnt), kBlock, 0, s>>>((uint16_t*)top, cnt);
+    OCNN_LAUNCH_OK("zero_rows");
+    return OCNN_OK;
+  }
+
+  char* wsb = static_cast<char*>(ws);
+  if (nempty) {
+    int* ichild = reinterpret_cast<int*>(wsb + p.wt_bytes);
+    ichild_kernel<<<blocks_for(p.child_h), kBlock, 0, s>>>(ichild, p.ichild_h, a.child, p.child_h);
+    OCNN_LAUNCH_OK("ichild");
+    a.ichild = ichild;
+  }
+  // conv: W[num_output, channel_in*K]; deconv: W[channel_in, num_output*K]
+  int64_t sm = deconv ? a.K : (int64_t)channel_in * a.K;
+  int64_t sc = deconv ? (int64_t)num_output * a.K : a.K;
+  int n_tiles = (a.N + kTileCols - 1) / kTileCols;
+  int grid = ((n_tiles + 7) / 8) * 8;
+  if (dtype == OCNN_F32) {
+    int64_t total = (int64_t)a.K * a.csteps * a.mtiles * 64;
+    pack_weights_f32<<<blocks_for(total), kBlock, 0, s>>>((float*)wsb, (const float*)weights, a.M, a.Cin, a.K,
+        a.mtiles, a.csteps, sm, sc);
+    OCNN_LAUNCH_OK("pack_weights");
+    if (a.mtiles == 1)
+      conv_f32_kernel<1><<<grid, kConvWaves * 64, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
+    else if (a.mtiles <= 2 || a.mtiles % 4 != 0)
+      conv_f32_kernel<2><<<grid, kConvWaves * 64, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
+    else
+      conv_f32_kernel<4><<<grid, kConvWaves * 64, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
+  } else {
+    int64_t total = (int64_t)a.K * a.csteps * a.mtiles * 64 * 8;
+    pack_weights_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)wsb, (const uint16_t*)weights, a.M, a.Cin,
+        a.K, a.mtiles, a.csteps, sm, sc);
+    OCNN_LAUNCH_OK("pack_weights");
+    if (a.mtiles == 1)
+      conv_bf16_kernel<1><<<grid, kConvWaves * 64, 0, s>>>(a, (uint16_t*)top, (const uint16_t*)btm, (const uint16_t*)wsb, n_tiles);
+    else if (a.mtiles <= 2 || a.mtiles % 4 != 0)
+      conv_bf16_kernel<2><<<grid, kConvWaves * 64, 0, s>>>(a, (uint16_t*)top, (const uint16_t*)btm, (const uint16_t*)wsb, n_tiles);
+    else
+      conv_bf16_kernel<4><<<grid, kConvWaves * 64, 0, s>>>(a, (uint16_t*)top, (const uint16_t*)btm, (const uint16_t*)wsb, n_tiles);
+  }
+  OCNN_LAUNCH_OK("octree_conv");
+  return OCNN_OK;
+}
+
+}  // namespace
+}  // namespace ocnn
+
+using namespace ocnn;
+
+extern "C" {
+
+int ocnn_conv_shape(const void* info, int depth, int channel_in, int num_output, const int* kernel_size,
+    int stride, int nempty, int is_deconv, int dtype, int* top_h, int* btm_h, size_t* workspace_bytes) {
+  ConvPlan p;
+  int e = make_plan(as_info(info), depth, channel_in, num_output, kernel_size, stride, nempty, is_deconv,
+      dtype, &p);
+  if (e) return e;
+  if (top_h) *top_h = p.top_h;
+  if (btm_h) *btm_h = p.btm_h;
+  if (workspace_bytes) *workspace_bytes = p.total_bytes;
+  return OCNN_OK;
+}
+
+int ocnn_octree_conv(void* top, const void* btm, int channel_in, int btm_h, const void* weights,
+    const void* octree_dev, const void* info, int depth, int num_output, const int* kernel_size, int stride,
+    int nempty, int dtype, void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream) {
+  return run_conv(0, top, btm, channel_in, btm_h, weights, octree_dev, info, depth, num_output, kernel_size,
+      stride, nempty, dtype, workspace_dev, workspace_bytes, as_stream(stream));
+}
+
+int ocnn_octree_deconv(void* top, const void* btm, int channel_in, int btm_h, const void* weights,
+    const void* octree_dev, const void* info, int depth, int num_output, const int* kernel_size, int stride,
+    int nempty, int dtype, void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream) {
+  return run_conv(1, top, btm, channel_in, btm_h, weights, octree_dev, info, depth, num_output, kernel_size,
+      stride, nempty, dtype, workspace_dev, workspace_bytes, as_stream(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,401 @@
+// Blob-level operations on serialized octrees that live on the device:
+//   octree_batch  (merge_octrees, octree/octree/merge_octrees.cpp:7-198)
+//   octree_new / octree_grow / octree_update (pytorch/cpp/octree_grow.cpp:13-190)
+// Header arithmetic runs on the host from the caller's host copies of the
+// headers; the payload never leaves the device.
+#include "ocnn_common.h"
+#include "scan.h"
+
+#include <vector>
+
+namespace ocnn {
+namespace {
+
+struct HeaderArg { uint32_t w[OCNN_HEADER_BYTES / 4]; };
+__global__ void g_write_header_kernel(uint32_t* __restrict__ dst, HeaderArg h) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < OCNN_HEADER_BYTES / 4) dst[i] = h.w[i];
+}
+int write_header(void* blob, const Info& o, hipStream_t s) {
+  HeaderArg h;
+  memset(&h, 0, sizeof(h));
+  memcpy(&h, &o, sizeof(Info));
+  g_write_header_kernel<<<1, kBlock, 0, s>>>(reinterpret_cast<uint32_t*>(blob), h);
+  OCNN_LAUNCH_OK("write_header");
+  return OCNN_OK;
+}
+
+__global__ void g_zero_kernel(uint32_t* p, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += step) p[i] = 0u;
+}
+int zero_payload(void* blob, const Info& o, hipStream_t s) {
+  int64_t words = (o.sizeof_octree() - OCNN_HEADER_BYTES) / 4;
+  if (words <= 0) return OCNN_OK;
+  unsigned grid = blocks_for(words, kBlock * 8);
+  if (grid > 65535u * 16) grid = 65535u * 16;
+  g_zero_kernel<<<grid, kBlock, 0, s>>>(reinterpret_cast<uint32_t*>(static_cast<char*>(blob) + OCNN_HEADER_BYTES), words);
+  OCNN_LAUNCH_OK("zero_payload");
+  return OCNN_OK;
+}
+
+template <typename T>
+__global__ void g_copy_kernel(T* __restrict__ dst, const T* __restrict__ src, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += step) dst[i] = src[i];
+}
+template <typename T>
+int copy_dev(T* dst, const T* src, int64_t n, hipStream_t s) {
+  if (n <= 0) return OCNN_OK;
+  unsigned grid = blocks_for(n, kBlock * 4);
+  if (grid > 65535u * 16) grid = 65535u * 16;
+  g_copy_kernel<T><<<grid, kBlock, 0, s>>>(dst, src, n);
+  OCNN_LAUNCH_OK("copy");
+  return OCNN_OK;
+}
+
+__global__ void g_seq_key_child_kernel(uint64_t* __restrict__ key, int* __restrict__ child, int n) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  if (key) key[i] = (uint64_t)i;
+  child[i] = i;
+}
+
+// ---- merge ---------------------------------------------------------------------
+// Per depth one launch per property over the merged node range; the source octree
+// of a node is found by binary search in the per-depth cumulative node counts.
+struct MergeTable {       // device layout: arrays indexed [d * (B+1) + b] / [(prop*B + b) * 17 + d]
+  const int* cum;         // node offset of octree b at depth d
+  const int* cum_ne;      // non-empty offset
+  const int64_t* src_off; // byte offset of (prop, octree, depth) inside its blob, -1 if absent
+  const char* const* src; // blob pointers
+  int B;
+};
+__device__ inline int find_src(const int* __restrict__ cum, int B, int t) {
+  int lo = 0, hi = B - 1;
+  while (lo < hi) {
+    int mid = (lo + hi + 1) >> 1;
+    if (cum[mid] <= t) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+enum { kPKey = 0, kPChild = 1, kPFeature = 2, kPLabel = 3, kPSplit = 4, kPCount = 5 };
+
+__global__ void merge_key_child_kernel(uint64_t* __restrict__ key, int* __restrict__ child, int d, int n,
+    MergeTable m) {
+  int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n) return;
+  const int* cum = m.cum + d * (m.B + 1);
+  int b = find_src(cum, m.B, t);
+  int j = t - cum[b];
+  const char* src = m.src[b];
+  if (key) {
+    uint64_t k = reinterpret_cast<const uint64_t*>(src + m.src_off[(kPKey * m.B + b) * 17 + d])[j];
+    key[t] = (k & 0x0000ffffffffffffull) | ((uint64_t)(b & 0xffff) << 48);
+  }
+  if (child) {
+    int c = reinterpret_cast<const int*>(src + m.src_off[(kPChild * m.B + b) * 17 + d])[j];
+    child[t] = c == -1 ? -1 : c + m.cum_ne[d * (m.B + 1) + b];
+  }
+}
+// float property with `channel` channels: dst[c, t] = src_b[c, j]
+__global__ void merge_float_kernel(float* __restrict__ dst, int prop, int channel, int d, int n, MergeTable m) {
+  int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n) return;
+  const int* cum = m.cum + d * (m.B + 1);
+  int b = find_src(cum, m.B, t);
+  int j = t - cum[b];
+  int nb = cum[b + 1] - cum[b];
+  const float* src = reinterpret_cast<const float*>(m.src[b] + m.src_off[(prop * m.B + b) * 17 + d]);
+  for (int c = 0; c < channel; ++c) dst[(int64_t)c * n + t] = src[(int64_t)c * nb + j];
+}
+
+inline size_t al(size_t v) { return (v + 255) & ~(size_t)255; }
+struct MergeLayout { size_t cum, cum_ne, src_off, src, total; };
+MergeLayout merge_layout(int B, int depth) {
+  MergeLayout L;
+  size_t off = 0;
+  auto take = [&](size_t b) { size_t o = off; off += al(b); return o; };
+  L.cum = take(sizeof(int) * (size_t)(depth + 1) * (B + 1));
+  L.cum_ne = take(sizeof(int) * (size_t)(depth + 1) * (B + 1));
+  L.src_off = take(sizeof(int64_t) * (size_t)kPCount * B * 17);
+  L.src = take(sizeof(char*) * (size_t)B);
+  L.total = off;
+  return L;
+}
+
+}  // namespace
+}  // namespace ocnn
+
+using namespace ocnn;
+
+extern "C" {
+
+// ---- octree_batch ------------------------------------------------------------------
+int ocnn_octree_batch_info(const void* const* infos, int n, void* out_info) {
+  OCNN_REQUIRE(infos && out_info && n >= 1 && n <= 65535, OCNN_E_BADARG, "bad argument");
+  const Info* first = as_info(infos[0]);
+  for (int i = 0; i < n; ++i) {
+    OCNN_REQUIRE(infos[i], OCNN_E_BADARG, "null info %d", i);
+    int e = ocnn_info_check(infos[i]);
+    if (e) return e;
+    OCNN_REQUIRE(first->consistent_with(*as_info(infos[i])), OCNN_E_FORMAT,
+        "The formats of input octrees are not consistent (octree %d)", i);
+  }
+  OCNN_REQUIRE(first->depth >= 1, OCNN_E_FORMAT, "depth %d", first->depth);
+  OCNN_REQUIRE(first->channel(OCNN_KEY) <= 1, OCNN_E_UNSUPPORTED, "two-channel keys cannot be merged");
+  Info o = *first;  // set_batch_info, merge_octrees.cpp:92-107
+  o.set_batch_size(n);
+  o.set_property(OCNN_NEIGH, 8, -1);
+  for (int d = 0; d <= o.depth; ++d) {
+    int64_t a = 0, b = 0;
+    for (int i = 0; i < n; ++i) { a += as_info(infos[i])->nnum[d]; b += as_info(infos[i])->nnum_nempty[d]; }
+    OCNN_REQUIRE(a < (1ll << 28), OCNN_E_BADARG, "merged level %d too large", d);
+    o.nnum[d] = (int)a;
+    o.nnum_nempty[d] = (int)b;
+  }
+  o.set_nnum_cum();
+  o.set_ptr_dis();
+  memcpy(out_info, &o, sizeof(Info));
+  return OCNN_OK;
+}
+
+size_t ocnn_octree_batch_workspace_bytes(int n, int depth) {
+  if (n < 1 || depth < 0 || depth > 16) return 0;
+  return merge_layout(n, depth).total;
+}
+
+int ocnn_octree_batch(void* out_dev, const void* out_info, const void* const* octrees_dev,
+    const void* const* infos, int n, void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream) {
+  OCNN_REQUIRE(out_dev && out_info && octrees_dev && infos && n >= 1, OCNN_E_BADARG, "bad argument");
+  const Info& o = *as_info(out_info);
+  const int B = n, depth = o.depth, fl = o.full_layer;
+  OCNN_REQUIRE(o.batch_size == B && o.has(OCNN_NEIGH), OCNN_E_BADARG, "out_info is not the batch header");
+  MergeLayout L = merge_layout(B, depth);
+  OCNN_REQUIRE(workspace_dev && workspace_bytes >= L.total, OCNN_E_WORKSPACE, "workspace %zu < %zu bytes",
+      workspace_bytes, L.total);
+  hipStream_t s = as_stream(stream);
+
+  // host tables
+  std::vector<int> cum((size_t)(depth + 1) * (B + 1), 0), cum_ne((size_t)(depth + 1) * (B + 1), 0);
+  std::vector<int64_t> src_off((size_t)kPCount * B * 17, -1);
+  std::vector<const char*> src(B);
+  const int props[kPCount] = {OCNN_KEY, OCNN_CHILD, OCNN_FEATURE, OCNN_LABEL, OCNN_SPLIT};
+  for (int b = 0; b < B; ++b) {
+    const Info* oi = as_info(infos[b]);
+    OCNN_REQUIRE(octrees_dev[b], OCNN_E_BADARG, "null octree %d", b);
+    src[b] = static_cast<const char*>(octrees_dev[b]);
+    for (int d = 0; d <= depth; ++d) {
+      cum[d * (B + 1) + b + 1] = cum[d * (B + 1) + b] + oi->nnum[d];
+      cum_ne[d * (B + 1) + b + 1] = cum_ne[d * (B + 1) + b] + oi->nnum_nempty[d];
+      for (int p = 0; p < kPCount; ++p) src_off[((size_t)p * B + b) * 17 + d] = oi->ptr_dis(props[p], d);
+    }
+  }
+  for (int d = 0; d <= depth; ++d)
+    OCNN_REQUIRE(cum[d * (B + 1) + B] == o.nnum[d], OCNN_E_BADARG, "out_info disagrees with the inputs at depth %d", d);
+  char* ws = static_cast<char*>(workspace_dev);
+  OCNN_HIP_OK(hipMemcpyAsync(ws + L.cum, cum.data(), cum.size() * sizeof(int), hipMemcpyHostToDevice, s));
+  OCNN_HIP_OK(hipMemcpyAsync(ws + L.cum_ne, cum_ne.data(), cum_ne.size() * sizeof(int), hipMemcpyHostToDevice, s));
+  OCNN_HIP_OK(hipMemcpyAsync(ws + L.src_off, src_off.data(), src_off.size() * sizeof(int64_t), hipMemcpyHostToDevice, s));
+  OCNN_HIP_OK(hipMemcpyAsync(ws + L.src, src.data(), src.size() * sizeof(char*), hipMemcpyHostToDevice, s));
+  OCNN_HIP_OK(hipStreamSynchronize(s));  // the tables above are host memory of this call
+  MergeTable m;
+  m.cum = reinterpret_cast<const int*>(ws + L.cum);
+  m.cum_ne = reinterpret_cast<const int*>(ws + L.cum_ne);
+  m.src_off = reinterpret_cast<const int64_t*>(ws + L.src_off);
+  m.src = reinterpret_cast<const char* const*>(ws + L.src);
+  m.B = B;
+
+  char* blob = static_cast<char*>(out_dev);
+  int e = zero_payload(blob, o, s);
+  if (e) return e;
+  e = write_header(blob, o, s);
+  if (e) return e;
+  for (int d = 0; d <= depth; ++d) {
+    int n_d = o.nnum[d];
+    if (n_d == 0) continue;
+    uint64_t* key = o.has(OCNN_KEY) ? reinterpret_cast<uint64_t*>(blob + o.ptr_dis(OCNN_KEY, d)) : nullptr;
+    int* child = o.has(OCNN_CHILD) ? reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_CHILD, d)) : nullptr;
+    merge_key_child_kernel<<<blocks_for(n_d), kBlock, 0, s>>>(key, child, d, n_d, m);
+    const int fprops[3] = {OCNN_FEATURE, OCNN_LABEL, OCNN_SPLIT};
+    const int findex[3] = {kPFeature, kPLabel, kPSplit};
+    for (int q = 0; q < 3; ++q) {
+      if (!o.has(fprops[q])) continue;
+      if (o.location(fprops[q]) == depth && d != depth) continue;
+      merge_float_kernel<<<blocks_for(n_d), kBlock, 0, s>>>(
+          reinterpret_cast<float*>(blob + o.ptr_dis(fprops[q], d)), findex[q], o.channel(fprops[q]), d, n_d, m);
+    }
+    OCNN_LAUNCH_OK("merge");
+  }
+  OCNN_REQUIRE(o.has(OCNN_CHILD), OCNN_E_FORMAT, "octrees without child links cannot get neighbour tables");
+  for (int d = 1; d <= depth; ++d) {
+    int* neigh = reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_NEIGH, d));
+    if (d <= fl) e = ocnn_calc_neigh_full(neigh, d, B, stream);
+    else e = ocnn_calc_neigh_sparse(neigh, reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_NEIGH, d - 1)),
+        reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_CHILD, d - 1)), o.nnum[d - 1], stream);
+    if (e) return e;
+  }
+  return OCNN_OK;
+}
+
+// ---- octree_new / octree_grow / octree_update -------------------------------------------
+int ocnn_octree_new_info(int batch_size, int channel, int node_dis, int adaptive_layer, void* out_info) {
+  OCNN_REQUIRE(out_info && batch_size >= 1 && channel >= 0, OCNN_E_BADARG, "bad argument");
+  Info o;  // pytorch/cpp/octree_grow.cpp:110-140
+  o.reset();
+  o.set_batch_size(batch_size);
+  o.set_depth(0);
+  o.set_full_layer(0);
+  o.has_node_dis = node_dis ? 1 : 0;
+  if (adaptive_layer > 1) { o.is_adaptive = 1; o.adp_layer = adaptive_layer; }
+  o.key2xyz = 1;
+  o.set_property(OCNN_KEY, 1, -1);
+  o.set_property(OCNN_CHILD, 1, -1);
+  o.set_property(OCNN_NEIGH, 8, -1);
+  o.set_property(OCNN_FEATURE, channel, -1);
+  for (int i = 0; i < 3; ++i) { o.bbmin[i] = 0.0f; o.bbmax[i] = 2.0f; }
+  o.nnum[0] = batch_size;
+  o.set_nnum_cum();
+  o.nnum_nempty[0] = batch_size;
+  o.set_ptr_dis();
+  memcpy(out_info, &o, sizeof(Info));
+  return OCNN_OK;
+}
+
+int ocnn_octree_new(void* out_dev, const void* out_info, ocnn_stream_t stream) {
+  OCNN_REQUIRE(out_dev && out_info, OCNN_E_BADARG, "null pointer");
+  const Info& o = *as_info(out_info);
+  hipStream_t s = as_stream(stream);
+  char* blob = static_cast<char*>(out_dev);
+  int e = zero_payload(blob, o, s);
+  if (e) return e;
+  e = write_header(blob, o, s);
+  if (e) return e;
+  int n = o.nnum[0];
+  g_seq_key_child_kernel<<<blocks_for(n), kBlock, 0, s>>>(reinterpret_cast<uint64_t*>(blob + o.ptr_dis(OCNN_KEY, 0)),
+      reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_CHILD, 0)), n);
+  OCNN_LAUNCH_OK("octree_new");
+  return OCNN_OK;
+}
+
+int ocnn_octree_grow_info(const void* in_info, int target_depth, int full_octree, void* out_info) {
+  OCNN_REQUIRE(in_info && out_info, OCNN_E_BADARG, "null pointer");
+  const Info* oi = as_info(in_info);
+  OCNN_REQUIRE(target_depth >= 1 && target_depth <= 13, OCNN_E_BADARG, "target_depth %d", target_depth);
+  OCNN_REQUIRE(target_depth == oi->depth + 1 || (oi->depth == 0 && oi->full_layer == 1 && target_depth == 1),
+      OCNN_E_BADARG, "octree_grow adds depth %d to an octree of depth %d", target_depth, oi->depth);
+  OCNN_REQUIRE(oi->has(OCNN_KEY) && oi->has(OCNN_CHILD) && oi->has(OCNN_NEIGH), OCNN_E_FORMAT,
+      "octree_grow needs key, child and neigh properties");
+  int64_t node_num = (int64_t)oi->nnum_nempty[target_depth - 1] << 3;
+  OCNN_REQUIRE(node_num < (1ll << 28), OCNN_E_BADARG, "grown level too large");
+  Info o = *oi;  // update_octreeinfo, octree_grow.cpp:57-73
+  o.set_depth(target_depth);
+  if (full_octree) o.set_full_layer(target_depth);
+  float width = (float)(1 << target_depth);
+  for (int i = 0; i < 3; ++i) { o.bbmin[i] = 0.0f; o.bbmax[i] = width; }
+  o.nnum[target_depth] = (int)node_num;
+  o.nnum_nempty[target_depth] = (int)node_num;
+  o.set_nnum_cum();
+  o.set_ptr_dis();
+  memcpy(out_info, &o, sizeof(Info));
+  return OCNN_OK;
+}
+
+int ocnn_octree_grow(void* out_dev, const void* out_info, const void* in_dev, const void* in_info,
+    int target_depth, int full_octree, ocnn_stream_t stream) {
+  OCNN_REQUIRE(out_dev && out_info && in_dev && in_info, OCNN_E_BADARG, "null pointer");
+  Info check;
+  int e = ocnn_octree_grow_info(in_info, target_depth, full_octree, &check);
+  if (e) return e;
+  OCNN_REQUIRE(memcmp(&check, out_info, sizeof(Info)) == 0, OCNN_E_BADARG, "out_info is not the grown header");
+  const Info& o = *as_info(out_info);
+  const Info& oi = *as_info(in_info);
+  hipStream_t s = as_stream(stream);
+  char* blob = static_cast<char*>(out_dev);
+  const char* in = static_cast<const char*>(in_dev);
+  e = zero_payload(blob, o, s);
+  if (e) return e;
+  e = write_header(blob, o, s);
+  if (e) return e;
+  // copy_octree_gpu, octree_grow.cpp:75-87: everything below the new depth
+  int64_t ncum = oi.nnum_cum[target_depth];
+  e = copy_dev(reinterpret_cast<uint64_t*>(blob + o.ptr_dis(OCNN_KEY, 0)),
+      reinterpret_cast<const uint64_t*>(in + oi.ptr_dis(OCNN_KEY, 0)), ncum * oi.channel(OCNN_KEY), s);
+  if (e) return e;
+  e = copy_dev(reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_CHILD, 0)),
+      reinterpret_cast<const int*>(in + oi.ptr_dis(OCNN_CHILD, 0)), ncum * oi.channel(OCNN_CHILD), s);
+  if (e) return e;
+  e = copy_dev(reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_NEIGH, 0)),
+      reinterpret_cast<const int*>(in + oi.ptr_dis(OCNN_NEIGH, 0)), ncum * oi.channel(OCNN_NEIGH), s);
+  if (e) return e;
+  if (oi.has(OCNN_FEATURE)) {
+    e = copy_dev(reinterpret_cast<float*>(blob + o.ptr_dis(OCNN_FEATURE, 0)),
+        reinterpret_cast<const float*>(in + oi.ptr_dis(OCNN_FEATURE, 0)), ncum * oi.channel(OCNN_FEATURE), s);
+    if (e) return e;
+  }
+  int* neigh = reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_NEIGH, target_depth));
+  uint64_t* key = reinterpret_cast<uint64_t*>(blob + o.ptr_dis(OCNN_KEY, target_depth));
+  int* child = reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_CHILD, target_depth));
+  const int node_num = o.nnum[target_depth];
+  if (full_octree) {
+    e = ocnn_calc_neigh_full(neigh, target_depth, o.batch_size, stream);
+    if (e) return e;
+    e = ocnn_generate_key_full(key, target_depth, o.batch_size, stream);
+    if (e) return e;
+  } else {
+    const int* label = reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_CHILD, target_depth - 1));
+    e = ocnn_calc_neigh_sparse(neigh, reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_NEIGH, target_depth - 1)),
+        label, o.nnum[target_depth - 1], stream);
+    if (e) return e;
+    e = ocnn_generate_key_child(key, reinterpret_cast<const uint64_t*>(blob + o.ptr_dis(OCNN_KEY, target_depth - 1)),
+        label, o.nnum[target_depth - 1], stream);
+    if (e) return e;
+  }
+  if (node_num > 0) {
+    g_seq_key_child_kernel<<<blocks_for(node_num), kBlock, 0, s>>>(nullptr, child, node_num);
+    OCNN_LAUNCH_OK("sequence");
+  }
+  return OCNN_OK;
+}
+
+__global__ void g_fix_empty_split_kernel(int* children, int* count) {
+  if (threadIdx.x == 0 && blockIdx.x == 0 && *count == 0) { children[0] = 0; *count = 1; }
+}
+__global__ void g_patch_nempty_kernel(int* header_nempty_d, const int* count) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) *header_nempty_d = *count;
+}
+
+int ocnn_octree_update(void* octree_dev, void* info, const int* label, int n_label, int depth, int split,
+    void* scratch_dev, size_t scratch_bytes, ocnn_stream_t stream) {
+  OCNN_REQUIRE(octree_dev && info && label, OCNN_E_BADARG, "null pointer");
+  Info* o = static_cast<Info*>(info);
+  OCNN_REQUIRE(depth >= 0 && depth <= o->depth, OCNN_E_BADARG, "depth %d", depth);
+  OCNN_REQUIRE(n_label == o->nnum[depth], OCNN_E_SHAPE, "label has %d entries, depth %d has %d nodes", n_label,
+      depth, o->nnum[depth]);
+  size_t need = scan_scratch_bytes(n_label) + 256;
+  OCNN_REQUIRE(scratch_dev && scratch_bytes >= need, OCNN_E_WORKSPACE, "scratch %zu < %zu bytes", scratch_bytes, need);
+  hipStream_t s = as_stream(stream);
+  char* blob = static_cast<char*>(octree_dev);
+  int* children = reinterpret_cast<int*>(blob + o->ptr_dis(OCNN_CHILD, depth));
+  int* count_dev = reinterpret_cast<int*>(scratch_dev);
+  void* scan_scratch = static_cast<char*>(scratch_dev) + 256;
+  int e = ocnn_generate_label(children, count_dev, label, n_label, split, scan_scratch, scratch_bytes - 256, stream);
+  if (e) return e;
+  // degenerate case: nothing splits -> keep one node (octree_grow.cpp:180-185)
+  g_fix_empty_split_kernel<<<1, 64, 0, s>>>(children, count_dev);
+  g_patch_nempty_kernel<<<1, 64, 0, s>>>(reinterpret_cast<int*>(blob + offsetof(Info, nnum_nempty)) + depth, count_dev);
+  OCNN_LAUNCH_OK("octree_update");
+  int split_num = 0;
+  OCNN_HIP_OK(hipMemcpyAsync(&split_num, count_dev, sizeof(int), hipMemcpyDeviceToHost, s));
+  OCNN_HIP_OK(hipStreamSynchronize(s));
+  o->nnum_nempty[depth] = split_num;
+  return OCNN_OK;
+}
+
+size_t ocnn_octree_update_scratch_bytes(int n_label) {
+  return scan_scratch_bytes(n_label < 0 ? 0 : n_label) + 256;
+}
+
+}  // extern "C"

@@ -1,0 +1,143 @@
+// Host-side pieces: error reporting, the OctreeInfo header arithmetic and the
+// kernel-shape tables.  Layout rules follow octree/octree/octree_info.cpp:143-268.
+#include "ocnn_common.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+
+namespace ocnn {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+void Info::reset() {
+  memset(this, 0, sizeof(Info));
+  strcpy(magic, "_OCTREE_2.0_");
+}
+
+void Info::set_channel(int ptype, int ch) {
+  int i = index_of(ptype);
+  if (ch > 0) {
+    channels[i] = ch;
+    content_flags |= ptype;
+  } else {
+    channels[i] = 0;
+    content_flags &= ~ptype;
+  }
+}
+
+void Info::set_nnum_cum(int capacity) {
+  nnum_cum[0] = 0;
+  for (int d = 1; d < depth + 2; ++d) nnum_cum[d] = nnum_cum[d - 1] + nnum[d - 1];
+  nnum_cum[depth + 2] = capacity > nnum_cum[depth + 1] ? capacity : nnum_cum[depth + 1];
+}
+
+void Info::set_ptr_dis() {
+  ptr_dis_[0] = OCNN_HEADER_BYTES;
+  for (int i = 1; i <= 6; ++i) {
+    int ptype = 1 << (i - 1);
+    int lc = location(ptype);
+    int num = lc == -1 ? total_capacity() : nnum[lc];
+    ptr_dis_[i] = ptr_dis_[i - 1] + size_of(ptype) * num * channels[i - 1];
+  }
+}
+
+float Info::bbox_max_width() const {
+  float w = bbmax[0] - bbmin[0];
+  for (int i = 1; i < 3; ++i) {
+    float d = bbmax[i] - bbmin[i];
+    if (d > w) w = d;
+  }
+  if (w == 0.0f) w = 1.0e-10f;
+  return w;
+}
+
+bool Info::consistent_with(const Info& o) const {  // octree_info.cpp:118-130
+  return strcmp(magic, o.magic) == 0 && memcmp(channels, o.channels, sizeof(channels)) == 0 &&
+      memcmp(locations, o.locations, sizeof(locations)) == 0 && batch_size == o.batch_size &&
+      depth == o.depth && full_layer == o.full_layer && adp_layer == o.adp_layer &&
+      is_adaptive == o.is_adaptive && key2xyz == o.key2xyz && has_node_dis == o.has_node_dis &&
+      content_flags == o.content_flags;
+}
+
+bool kernel_taps(const int* ks, KernelTaps* out) {
+  if (!ks) return false;
+  for (int a = 0; a < 3; ++a) if (ks[a] < 1 || ks[a] > 3) return false;
+  // Per axis: size 3 -> offsets {0,1,2}; size 1 -> {1}; size 2 -> {1,2}
+  // (the "222" kernel is the 8 octants on the positive side, octree_nn.cpp:13).
+  // Mixed shapes containing a 2 (other than 222) are not in the reference's table.
+  int code = ks[0] * 100 + ks[1] * 10 + ks[2];
+  bool has2 = ks[0] == 2 || ks[1] == 2 || ks[2] == 2;
+  if (has2 && code != 222) return false;
+  int lo[3], hi[3];
+  for (int a = 0; a < 3; ++a) {
+    lo[a] = ks[a] == 3 ? 0 : 1;
+    hi[a] = ks[a] == 1 ? 1 : 2;
+  }
+  int n = 0;
+  for (int x = lo[0]; x <= hi[0]; ++x)
+    for (int y = lo[1]; y <= hi[1]; ++y)
+      for (int z = lo[2]; z <= hi[2]; ++z) out->tap[n++] = x * 9 + y * 3 + z;
+  out->count = n;
+  return true;
+}
+
+}  // namespace ocnn
+
+using ocnn::Info;
+using ocnn::as_info;
+
+extern "C" {
+
+const char* ocnn_last_error(void) { return ocnn::g_err; }
+int ocnn_version(void) { return 100; }
+
+int ocnn_device_check(int dev) {
+  int n = 0;
+  OCNN_HIP_OK(hipGetDeviceCount(&n));
+  OCNN_REQUIRE(dev >= 0 && dev < n, OCNN_E_BADARG, "device %d of %d", dev, n);
+  hipDeviceProp_t p;
+  OCNN_HIP_OK(hipGetDeviceProperties(&p, dev));
+  OCNN_REQUIRE(strncmp(p.gcnArchName, "gfx950", 6) == 0, OCNN_E_UNSUPPORTED,
+      "device %d is %s, this library holds gfx950 code only", dev, p.gcnArchName);
+  return OCNN_OK;
+}
+
+int ocnn_info_check(const void* info) {  // octree_info.cpp:80-116
+  OCNN_REQUIRE(info, OCNN_E_BADARG, "null info");
+  const Info* o = as_info(info);
+  OCNN_REQUIRE(memcmp(o->magic, "_OCTREE_2.0_", 13) == 0, OCNN_E_FORMAT,
+      "octree magic is not _OCTREE_2.0_ (64-bit keys)");
+  OCNN_REQUIRE(o->batch_size >= 0, OCNN_E_FORMAT, "batch_size %d", o->batch_size);
+  OCNN_REQUIRE(o->depth >= 0 && o->depth <= 16, OCNN_E_FORMAT, "depth %d not in [0,16]", o->depth);
+  OCNN_REQUIRE(o->full_layer >= 0 && o->full_layer <= (o->depth < 1 ? 1 : o->depth), OCNN_E_FORMAT,
+      "full_layer %d not in [0,depth]", o->full_layer);
+  for (int i = 0; i < 6; ++i) {
+    OCNN_REQUIRE((o->channels[i] == 0) == ((o->content_flags & (1 << i)) == 0), OCNN_E_FORMAT,
+        "content_flags inconsistent with channels[%d]", i);
+    OCNN_REQUIRE(o->channels[i] == 0 || o->locations[i] == -1 || o->locations[i] == o->depth,
+        OCNN_E_FORMAT, "locations[%d] = %d", i, o->locations[i]);
+  }
+  return OCNN_OK;
+}
+int ocnn_info_batch_size(const void* info) { return as_info(info)->batch_size; }
+int ocnn_info_depth(const void* info) { return as_info(info)->depth; }
+int ocnn_info_full_depth(const void* info) { return as_info(info)->full_layer; }
+int ocnn_info_is_key2xyz(const void* info) { return as_info(info)->key2xyz; }
+int ocnn_info_node_num(const void* info, int d) { return (d < 0 || d > 15) ? -1 : as_info(info)->nnum[d]; }
+int ocnn_info_node_num_nempty(const void* info, int d) { return (d < 0 || d > 15) ? -1 : as_info(info)->nnum_nempty[d]; }
+int ocnn_info_node_num_cum(const void* info, int d) { return (d < 0 || d > 15) ? -1 : as_info(info)->nnum_cum[d]; }
+int ocnn_info_total_nnum(const void* info) { return as_info(info)->total_nnum(); }
+int ocnn_info_channel(const void* info, int ptype) { return as_info(info)->channel(ptype); }
+int ocnn_info_location(const void* info, int ptype) { return as_info(info)->location(ptype); }
+int64_t ocnn_info_ptr_dis(const void* info, int ptype, int d) { return as_info(info)->ptr_dis(ptype, d); }
+int64_t ocnn_info_sizeof_octree(const void* info) { return as_info(info)->sizeof_octree(); }
+
+}  // extern "C"

@@ -1,0 +1,266 @@
+// Integer kernels on the octree structure: neighbour tables, key generation,
+// Morton <-> packed-xyz conversion, sorted-key search, label compaction.
+// Everything here is bit-exact integer work bound by HBM bandwidth.
+#include "ocnn_common.h"
+#include "scan.h"
+
+namespace ocnn {
+
+// Morton helpers: bit i of axis j lands at bit 3*i + 2 - j (x highest), the
+// convention of compute_key / compute_pt (octree/octree/octree_nn.cpp:551-575).
+__host__ __device__ inline uint64_t spread3(uint64_t v) {  // 16 bits -> every third bit
+  v &= 0xffffull;
+  v = (v | (v << 32)) & 0x00ff00000000ffffull;
+  v = (v | (v << 16)) & 0x00ff0000ff0000ffull;
+  v = (v | (v << 8)) & 0xf00f00f00f00f00full;
+  v = (v | (v << 4)) & 0x30c30c30c30c30c3ull;
+  v = (v | (v << 2)) & 0x9249249249249249ull;
+  return v;
+}
+__host__ __device__ inline uint64_t compact3(uint64_t v) {  // inverse of spread3
+  v &= 0x9249249249249249ull;
+  v = (v | (v >> 2)) & 0x30c30c30c30c30c3ull;
+  v = (v | (v >> 4)) & 0xf00f00f00f00f00full;
+  v = (v | (v >> 8)) & 0x00ff0000ff0000ffull;
+  v = (v | (v >> 16)) & 0x00ff00000000ffffull;
+  v = (v | (v >> 32)) & 0xffffull;
+  return v;
+}
+__host__ __device__ inline uint64_t morton_encode(uint32_t x, uint32_t y, uint32_t z, int depth) {
+  uint64_t m = depth >= 16 ? 0xffffull : ((1ull << depth) - 1);
+  return (spread3(x & m) << 2) | (spread3(y & m) << 1) | spread3(z & m);
+}
+__host__ __device__ inline void morton_decode(uint64_t key, int depth, uint32_t* x, uint32_t* y, uint32_t* z) {
+  uint64_t m = depth >= 16 ? 0xffffull : ((1ull << depth) - 1);
+  *x = (uint32_t)(compact3(key >> 2) & m);
+  *y = (uint32_t)(compact3(key >> 1) & m);
+  *z = (uint32_t)(compact3(key) & m);
+}
+
+namespace {
+
+// ---- neighbour tables --------------------------------------------------------
+// Sparse layer: one wavefront per parent-level node, one lane per slot of the
+// 4x4x4 block of its child group.  Slot (x,y,z) of the child block lies at
+// child-level offset (x-1,y-1,z-1) from child 0, i.e. in the parent-level node at
+// offset ((x+1)>>1)-1 per axis, as its octant ((x+1)&1, ...).
+__global__ void calc_neigh_sparse_kernel(int* __restrict__ neigh_child, const int* __restrict__ neigh,
+    const int* __restrict__ children, int node_num) {
+  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int i = (int)(id >> 6), j = (int)(id & 63);
+  if (i >= node_num) return;
+  int l0 = children[i];
+  if (l0 < 0) return;
+  int x = j >> 4, y = (j >> 2) & 3, z = j & 3;
+  int sib = i & 7;
+  int px = ((x + 1) >> 1) + (sib >> 2), py = ((y + 1) >> 1) + ((sib >> 1) & 1), pz = ((z + 1) >> 1) + (sib & 1);
+  int octant = (((x + 1) & 1) << 2) | (((y + 1) & 1) << 1) | ((z + 1) & 1);
+  int k = neigh[((int64_t)(i >> 3) << 6) + ((px << 4) | (py << 2) | pz)];
+  int t = -1;
+  if (k >= 0) {
+    int l1 = children[k];
+    if (l1 >= 0) t = (l1 << 3) + octant;
+  }
+  neigh_child[((int64_t)l0 << 6) + j] = t;
+}
+
+// Full layer: closed form through Morton decode / encode.
+__global__ void calc_neigh_full_kernel(int* __restrict__ neigh, int depth, int64_t total) {
+  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= total) return;
+  const int64_t node_num = (int64_t)1 << (3 * depth);
+  const int64_t groups = node_num >> 3;
+  int slot = (int)(id & 63);
+  int64_t g = id >> 6;
+  int64_t n = g / groups;
+  uint64_t i = (uint64_t)(g % groups) << 3;
+  uint32_t x0, y0, z0;
+  morton_decode(i, depth, &x0, &y0, &z0);
+  uint32_t x1 = x0 + (slot >> 4) - 1, y1 = y0 + ((slot >> 2) & 3) - 1, z1 = z0 + (slot & 3) - 1;
+  const uint32_t bound = 1u << depth;
+  int v = -1;
+  // a coordinate of -1 or 2^depth has the bound bit set (two's complement / carry)
+  if (((x1 | y1 | z1) & bound) == 0) v = (int)(morton_encode(x1, y1, z1, depth) + (uint64_t)n * node_num);
+  neigh[id] = v;
+}
+
+// ---- keys -----------------------------------------------------------------------
+__global__ void gen_key_child_kernel(uint64_t* __restrict__ key_child, const uint64_t* __restrict__ key,
+    const int* __restrict__ child, int64_t total) {
+  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= total) return;
+  int i = (int)(id >> 3), j = (int)(id & 7);
+  int label = child[i];
+  if (label < 0) return;
+  uint64_t k0 = key[i];
+  uint64_t x = (((k0 & 0xffffu) << 1) | ((j >> 2) & 1)) & 0xffffu;
+  uint64_t y = ((((k0 >> 16) & 0xffffu) << 1) | ((j >> 1) & 1)) & 0xffffu;
+  uint64_t z = ((((k0 >> 32) & 0xffffu) << 1) | (j & 1)) & 0xffffu;
+  key_child[8 * (int64_t)label + j] = x | (y << 16) | (z << 32) | (k0 & 0xffff000000000000ull);
+}
+
+__global__ void gen_key_full_kernel(uint64_t* __restrict__ key, int depth, int64_t total) {
+  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= total) return;
+  const int64_t node_num = (int64_t)1 << (3 * depth);
+  uint32_t x, y, z;
+  morton_decode((uint64_t)(id % node_num), depth, &x, &y, &z);
+  key[id] = (uint64_t)x | ((uint64_t)y << 16) | ((uint64_t)z << 32) | ((uint64_t)((id / node_num) & 0xffff) << 48);
+}
+
+__global__ void xyz2key_kernel(uint64_t* __restrict__ key, const uint64_t* __restrict__ xyz, int num, int depth) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= num) return;
+  uint64_t v = xyz[i];
+  uint64_t k = morton_encode((uint32_t)(v & 0xffff), (uint32_t)((v >> 16) & 0xffff),
+      (uint32_t)((v >> 32) & 0xffff), depth);
+  key[i] = (k & 0x0000ffffffffffffull) | (v & 0xffff000000000000ull);
+}
+
+__global__ void key2xyz_kernel(uint64_t* __restrict__ xyz, const uint64_t* __restrict__ key, int num, int depth) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= num) return;
+  uint64_t k = key[i];
+  uint32_t x, y, z;
+  morton_decode(k, depth, &x, &y, &z);
+  xyz[i] = (uint64_t)x | ((uint64_t)y << 16) | ((uint64_t)z << 32) | (k & 0xffff000000000000ull);
+}
+
+__global__ void key2idx_kernel(int* __restrict__ idx, const uint64_t* __restrict__ key, int num) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < num) idx[i] = (int)(key[i] >> 48);
+}
+
+__global__ void sequence_kernel(int* __restrict__ p, int num) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < num) p[i] = i;
+}
+
+// lower_bound over the sorted key array, -1 on a miss (octree_nn.cpp:541-548)
+__global__ void search_key_kernel(int* __restrict__ idx, const uint64_t* __restrict__ key, int n_key,
+    const uint64_t* __restrict__ query, int n_query) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_query) return;
+  uint64_t q = query[i];
+  int lo = 0, hi = n_key;
+  while (lo < hi) {
+    int mid = lo + ((hi - lo) >> 1);
+    if (key[mid] < q) lo = mid + 1; else hi = mid;
+  }
+  idx[i] = (lo < n_key && key[lo] == q) ? lo : -1;
+}
+
+struct LabelPred {
+  const int* btm;
+  int mask;
+  __device__ bool operator()(int64_t i) const { return btm[i] == mask; }
+};
+struct LabelOut {
+  int* label;
+  __device__ void operator()(int64_t i, bool f, int rank) const { label[i] = f ? rank : -1; }
+};
+
+}  // namespace
+}  // namespace ocnn
+
+using namespace ocnn;
+
+extern "C" {
+
+int ocnn_calc_neigh_sparse(int* neigh_child, const int* neigh, const int* children, int node_num,
+    ocnn_stream_t stream) {
+  OCNN_REQUIRE(neigh_child && neigh && children, OCNN_E_BADARG, "null pointer");
+  OCNN_REQUIRE(node_num >= 0, OCNN_E_BADARG, "node_num %d", node_num);
+  if (node_num == 0) return OCNN_OK;
+  int64_t threads = (int64_t)node_num << 6;
+  calc_neigh_sparse_kernel<<<blocks_for(threads), kBlock, 0, as_stream(stream)>>>(neigh_child, neigh,
+      children, node_num);
+  OCNN_LAUNCH_OK("calc_neigh_sparse");
+  return OCNN_OK;
+}
+
+int ocnn_calc_neigh_full(int* neigh, int depth, int batch_size, ocnn_stream_t stream) {
+  OCNN_REQUIRE(neigh, OCNN_E_BADARG, "null pointer");
+  OCNN_REQUIRE(depth >= 1 && depth <= 9 && batch_size >= 1, OCNN_E_BADARG,
+      "depth %d batch %d (a full layer deeper than 9 does not fit int32 indices)", depth, batch_size);
+  int64_t total = (int64_t)batch_size << (3 * depth + 3);
+  OCNN_REQUIRE(total < (1ll << 34), OCNN_E_BADARG, "full layer too large");
+  calc_neigh_full_kernel<<<blocks_for(total), kBlock, 0, as_stream(stream)>>>(neigh, depth, total);
+  OCNN_LAUNCH_OK("calc_neigh_full");
+  return OCNN_OK;
+}
+
+int ocnn_generate_key_child(uint64_t* key_child, const uint64_t* key, const int* child, int node_num,
+    ocnn_stream_t stream) {
+  OCNN_REQUIRE(key_child && key && child && node_num >= 0, OCNN_E_BADARG, "bad argument");
+  if (node_num == 0) return OCNN_OK;
+  int64_t total = (int64_t)node_num << 3;
+  gen_key_child_kernel<<<blocks_for(total), kBlock, 0, as_stream(stream)>>>(key_child, key, child, total);
+  OCNN_LAUNCH_OK("generate_key_child");
+  return OCNN_OK;
+}
+
+int ocnn_generate_key_full(uint64_t* key, int depth, int batch_size, ocnn_stream_t stream) {
+  OCNN_REQUIRE(key && depth >= 0 && depth <= 10 && batch_size >= 1, OCNN_E_BADARG, "bad argument");
+  int64_t total = (int64_t)batch_size << (3 * depth);
+  gen_key_full_kernel<<<blocks_for(total), kBlock, 0, as_stream(stream)>>>(key, depth, total);
+  OCNN_LAUNCH_OK("generate_key_full");
+  return OCNN_OK;
+}
+
+size_t ocnn_generate_label_scratch_bytes(int btm_h) { return scan_scratch_bytes(btm_h < 0 ? 0 : btm_h); }
+
+int ocnn_generate_label(int* label, int* count_dev, const int* btm, int btm_h, int mask,
+    void* scratch_dev, size_t scratch_bytes, ocnn_stream_t stream) {
+  OCNN_REQUIRE(label && count_dev && btm && btm_h >= 0, OCNN_E_BADARG, "bad argument");
+  OCNN_REQUIRE(scratch_dev && scratch_bytes >= scan_scratch_bytes(btm_h), OCNN_E_WORKSPACE,
+      "scratch %zu < %zu bytes", scratch_bytes, scan_scratch_bytes(btm_h));
+  LabelPred pred{btm, mask};
+  LabelOut out{label};
+  hipError_t e = flag_scan(pred, out, (int64_t)btm_h, (int*)scratch_dev, count_dev, as_stream(stream));
+  OCNN_REQUIRE(e == hipSuccess, OCNN_E_HIP, "generate_label: %s", hipGetErrorString(e));
+  return OCNN_OK;
+}
+
+int ocnn_sequence(int* ptr, int num, ocnn_stream_t stream) {
+  OCNN_REQUIRE(ptr && num >= 0, OCNN_E_BADARG, "bad argument");
+  if (num == 0) return OCNN_OK;
+  sequence_kernel<<<blocks_for(num), kBlock, 0, as_stream(stream)>>>(ptr, num);
+  OCNN_LAUNCH_OK("sequence");
+  return OCNN_OK;
+}
+
+int ocnn_search_key(int* idx, const uint64_t* key, int n_key, const uint64_t* query, int n_query,
+    ocnn_stream_t stream) {
+  OCNN_REQUIRE(idx && query && (key || n_key == 0) && n_key >= 0 && n_query >= 0, OCNN_E_BADARG, "bad argument");
+  if (n_query == 0) return OCNN_OK;
+  search_key_kernel<<<blocks_for(n_query), kBlock, 0, as_stream(stream)>>>(idx, key, n_key, query, n_query);
+  OCNN_LAUNCH_OK("search_key");
+  return OCNN_OK;
+}
+
+int ocnn_xyz2key(uint64_t* key, const uint64_t* xyz, int num, int depth, ocnn_stream_t stream) {
+  OCNN_REQUIRE(key && xyz && num >= 0 && depth >= 0 && depth <= 16, OCNN_E_BADARG, "bad argument");
+  if (num == 0) return OCNN_OK;
+  xyz2key_kernel<<<blocks_for(num), kBlock, 0, as_stream(stream)>>>(key, xyz, num, depth);
+  OCNN_LAUNCH_OK("xyz2key");
+  return OCNN_OK;
+}
+
+int ocnn_key2xyz(uint64_t* xyz, const uint64_t* key, int num, int depth, ocnn_stream_t stream) {
+  OCNN_REQUIRE(key && xyz && num >= 0 && depth >= 0 && depth <= 16, OCNN_E_BADARG, "bad argument");
+  if (num == 0) return OCNN_OK;
+  key2xyz_kernel<<<blocks_for(num), kBlock, 0, as_stream(stream)>>>(xyz, key, num, depth);
+  OCNN_LAUNCH_OK("key2xyz");
+  return OCNN_OK;
+}
+
+int ocnn_key2idx(int* idx, const uint64_t* key, int num, ocnn_stream_t stream) {
+  OCNN_REQUIRE(idx && key && num >= 0, OCNN_E_BADARG, "bad argument");
+  if (num == 0) return OCNN_OK;
+  key2idx_kernel<<<blocks_for(num), kBlock, 0, as_stream(stream)>>>(idx, key, num);
+  OCNN_LAUNCH_OK("key2idx");
+  return OCNN_OK;
+}
+
+}  // extern "C"

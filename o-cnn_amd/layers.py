@@ -1,0 +1,148 @@
+"""Forward-only mirrors of the thin Python modules of the reference
+(pytorch/ocnn/octree_conv.py:75-158, octree_pool.py:69-103, octree_pad.py:47-72).
+They add exactly the compositions the reference adds around the extension calls:
+`octree_pad` after a stride-2 convolution, `octree_depad` before a stride-2
+deconvolution, pad / depad around pooling.  Gradients are not implemented."""
+import torch
+from torch import nn
+
+from . import nn as F
+
+
+def resize_with_last_val(list_in, num=3):
+  out = list(list_in)
+  while len(out) < num:
+    out.append(out[-1])
+  return out
+
+
+class OctreeConvBase(nn.Module):
+  def __init__(self, depth, channel_in, channel_out, kernel_size=[3], stride=1, nempty=False):
+    super().__init__()
+    self.depth = depth
+    self.channel_in = channel_in
+    self.channel_out = channel_out
+    self.kernel_size = resize_with_last_val(kernel_size)
+    self.stride = stride
+    self.nempty = nempty
+    self.kdim = self.kernel_size[0] * self.kernel_size[1] * self.kernel_size[2]
+    conv_in = channel_in if self.is_conv_layer() else channel_out
+    conv_out = channel_out if self.is_conv_layer() else channel_in
+    self.cdim = conv_in * self.kdim
+    self.weights = nn.Parameter(torch.empty(conv_out, self.cdim))
+    nn.init.xavier_uniform_(self.weights)
+
+  def is_conv_layer(self):
+    raise NotImplementedError
+
+  def extra_repr(self):
+    return ('depth={}, channel_in={}, channel_out={}, kernel_size={}, stride={}, nempty={}'
+            .format(self.depth, self.channel_in, self.channel_out, self.kernel_size,
+                    self.stride, self.nempty))
+
+
+class OctreeConv(OctreeConvBase):
+  def is_conv_layer(self):
+    return True
+
+  def forward(self, data, octree):
+    assert data.size(1) == self.channel_in
+    conv = F.octree_conv(data, self.weights.detach(), octree, self.depth, self.channel_out,
+                         self.kernel_size, self.stride, self.nempty)
+    if self.stride == 2 and not self.nempty:
+      conv = F.octree_pad(conv, octree, self.depth - 1)
+    return conv
+
+
+class OctreeDeconv(OctreeConvBase):
+  def is_conv_layer(self):
+    return False
+
+  def forward(self, data, octree):
+    assert data.size(1) == self.channel_in
+    if self.stride == 2 and not self.nempty:
+      data = F.octree_depad(data, octree, self.depth)
+    return F.octree_deconv(data, self.weights.detach(), octree, self.depth, self.channel_out,
+                           self.kernel_size, self.stride, self.nempty)
+
+
+class OctreeConvFast(OctreeConvBase):
+  """octree2col + matrix product: the explicit form the implicit-GEMM kernel replaces."""
+
+  def is_conv_layer(self):
+    return True
+
+  def forward(self, data, octree):
+    col = F.octree2col(data, octree, self.depth, self.kernel_size, self.stride, False)
+    col = col.view([self.cdim, -1])
+    conv = torch.mm(self.weights.detach(), col)
+    conv = torch.unsqueeze(torch.unsqueeze(conv, 0), -1)
+    if self.stride == 2:
+      conv = F.octree_pad(conv, octree, self.depth - 1)
+    return conv
+
+
+class OctreeDeconvFast(OctreeConvBase):
+  def is_conv_layer(self):
+    return False
+
+  def forward(self, data, octree):
+    depth = self.depth
+    if self.stride == 2:
+      data = F.octree_depad(data, octree, depth)
+      depth = depth + 1
+    data = torch.squeeze(torch.squeeze(data, dim=0), dim=-1)
+    col = torch.mm(self.weights.detach().t(), data)
+    col = col.view(self.channel_out, self.kdim, -1)
+    return F.col2octree(col, octree, depth, self.kernel_size, self.stride, False)
+
+
+class OctreePoolBase(nn.Module):
+  def __init__(self, depth):
+    super().__init__()
+    self.depth = depth
+
+  def extra_repr(self):
+    return 'depth={}'.format(self.depth)
+
+
+class OctreeMaxPool(OctreePoolBase):
+  def __init__(self, depth, return_indices=False):
+    super().__init__(depth)
+    self.return_indices = return_indices
+
+  def forward(self, data, octree):
+    pool, mask = F.octree_max_pool(data, octree, self.depth)
+    output = F.octree_pad(pool, octree, self.depth - 1)
+    return output if not self.return_indices else (output, mask)
+
+
+class OctreeMaxUnpool(OctreePoolBase):
+  def forward(self, data, mask, octree):
+    pool = F.octree_depad(data, octree, self.depth)
+    return F.octree_max_unpool(pool, mask, octree, self.depth + 1)
+
+
+class OctreeAvgPool(OctreePoolBase):
+  def forward(self, data, octree):
+    channel = data.shape[1]
+    pool = data.view(1, channel, -1, 8).mean(dim=3, keepdims=True)
+    return F.octree_pad(pool, octree, self.depth - 1)
+
+
+class OctreePad(nn.Module):
+  def __init__(self, depth, val=0.0):
+    super().__init__()
+    self.depth, self.val = depth, val
+
+  def forward(self, data_in, octree):
+    return F.octree_pad(data_in, octree, self.depth, self.val)
+
+
+class OctreeDepad(nn.Module):
+  def __init__(self, depth):
+    super().__init__()
+    self.depth = depth
+
+  def forward(self, data_in, octree):
+    return F.octree_depad(data_in, octree, self.depth)

@@ -1,0 +1,639 @@
+"""Host-side mirror of the reference's `ocnn.nn` extension (pytorch/cpp/pybind.cpp:3-49,
+signatures pytorch/cpp/ocnn.h:11-72) over the C-ABI of libocnn_hip.so.
+
+Same function names, argument order, tensor shapes and depth conventions as the
+reference.  PyTorch only provides device memory and the current stream; every
+computation happens in the HIP library.  Differences a caller can see:
+  * octrees and point clouds live on the GPU (a CPU tensor is moved there); the
+    results of `points2octree` and `octree_batch` are CUDA tensors;
+  * the 716-byte octree header is read back from the device once per blob tensor
+    and cached on the tensor object, not once per operator call;
+  * failures raise `OcnnError` instead of aborting the process;
+  * `points2octree_batch` (build + octree_batch fused in one pass) and bfloat16
+    feature tensors are additions.
+"""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import lib as _lib
+from .lib import BF16, F32, OcnnError, BuildParams  # noqa: F401
+from .lib import CHILD, FEATURE, KEY, LABEL, NEIGH, SPLIT, HEADER_BYTES, INFO_BYTES
+
+__all__ = [
+    "points2octree", "points2octree_batch", "octree_batch", "octree_property",
+    "octree_set_property", "octree2col", "col2octree", "octree_conv", "octree_deconv",
+    "octree_pad", "octree_depad", "octree_max_pool", "octree_max_unpool", "octree_mask_pool",
+    "octree_encode_key", "octree_decode_key", "octree_xyz2key", "octree_key2xyz",
+    "octree_search_key", "octree_new", "octree_grow", "octree_update", "points_new",
+    "octree_info",
+]
+
+
+# ---- plumbing ---------------------------------------------------------------------
+def _ptr(t):
+  return C.c_void_p(t.data_ptr() if t is not None else 0)
+
+
+def _stream():
+  return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev():
+  if not torch.cuda.is_available():
+    raise RuntimeError("o-cnn_amd needs a GPU: there is no CPU path")
+  return torch.device("cuda", torch.cuda.current_device())
+
+
+def _dtype_code(t):
+  if t.dtype == torch.float32:
+    return F32
+  if t.dtype == torch.bfloat16:
+    return BF16
+  raise TypeError("feature tensors must be float32 or bfloat16, got %s" % t.dtype)
+
+
+def _ks(kernel_size):
+  ks = list(kernel_size)
+  while len(ks) < 3:           # resize_with_last_val, pytorch/ocnn/octree_conv.py:8-12
+    ks.append(ks[-1])
+  return (C.c_int * 3)(*ks[:3]), ks[:3]
+
+
+_workspaces = {}
+
+
+def _workspace(nbytes, tag="main"):
+  """A cached, growing device scratch buffer per (device, tag)."""
+  key = (torch.cuda.current_device(), tag)
+  buf = _workspaces.get(key)
+  if buf is None or buf.numel() < nbytes:
+    buf = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=_dev())
+    _workspaces[key] = buf
+  return buf
+
+
+class _Info:
+  """Host copy of an octree header plus typed accessors (through the C-ABI)."""
+
+  def __init__(self, raw):
+    self.raw = np.ascontiguousarray(raw[:INFO_BYTES], dtype=np.uint8).copy()
+    self.p = C.c_void_p(self.raw.ctypes.data)
+    L = _lib.get()
+    self._L = L
+    self.depth = L.ocnn_info_depth(self.p)
+    self.full_depth = L.ocnn_info_full_depth(self.p)
+    self.batch_size = L.ocnn_info_batch_size(self.p)
+    self.key2xyz = bool(L.ocnn_info_is_key2xyz(self.p))
+
+  def nnum(self, d):
+    return self._L.ocnn_info_node_num(self.p, d)
+
+  def nnum_nempty(self, d):
+    return self._L.ocnn_info_node_num_nempty(self.p, d)
+
+  def nnum_cum(self, d):
+    return self._L.ocnn_info_node_num_cum(self.p, d)
+
+  def total_nnum(self):
+    return self._L.ocnn_info_total_nnum(self.p)
+
+  def channel(self, ptype):
+    return self._L.ocnn_info_channel(self.p, ptype)
+
+  def location(self, ptype):
+    return self._L.ocnn_info_location(self.p, ptype)
+
+  def ptr_dis(self, ptype, d):
+    return self._L.ocnn_info_ptr_dis(self.p, ptype, d)
+
+  def size(self):
+    return self._L.ocnn_info_sizeof_octree(self.p)
+
+
+def octree_info(octree):
+  """Header of an octree blob tensor; read from the device at most once per tensor."""
+  info = getattr(octree, "_ocnn_info", None)
+  if info is None:
+    if octree.dtype != torch.uint8 or octree.dim() != 1 or octree.numel() < HEADER_BYTES:
+      raise ValueError("an octree is a 1-D uint8 tensor of at least %d bytes" % HEADER_BYTES)
+    info = _Info(octree[:INFO_BYTES].cpu().numpy())
+    _lib.call("ocnn_info_check", info.p)
+    octree._ocnn_info = info
+  return info
+
+
+def _attach(octree, raw_info):
+  octree._ocnn_info = _Info(raw_info)
+  return octree
+
+
+def _to_dev(t):
+  if t.is_cuda:
+    return t.contiguous()
+  info = getattr(t, "_ocnn_info", None)
+  out = t.contiguous().to(_dev())
+  if info is not None:
+    out._ocnn_info = info
+  return out
+
+
+def _prop_view(octree, info, ptype, depth, count, dtype):
+  """1-D view of `count` elements of a property at a depth inside the blob."""
+  off = info.ptr_dis(ptype, depth)
+  if off < 0:
+    return None
+  itemsize = torch.empty((), dtype=dtype).element_size()
+  return octree[off:off + count * itemsize].view(dtype)
+
+
+# ---- octree construction -------------------------------------------------------------
+def _points_header(points):
+  hdr = points[:_lib.POINTS_INFO_BYTES].cpu().numpy().copy()
+  return hdr
+
+
+def _build(points_list, merged, depth, full_depth, node_dis, node_feature, split_label, adaptive,
+           adp_depth, th_normal, th_distance, extrapolate, save_pts, key2xyz, bbox=None):
+  pts = [_to_dev(p) for p in points_list]
+  hdrs = [getattr(p, "_ocnn_points_info", None) for p in points_list]
+  for i, h in enumerate(hdrs):
+    if h is None:
+      hdrs[i] = _points_header(pts[i])
+  n = len(pts)
+  total = int(sum(int(h[16:20].view(np.int32)[0]) for h in hdrs))
+  L = _lib.get()
+  bp = BuildParams(depth=depth, full_depth=full_depth, node_dis=int(node_dis),
+                   node_feature=int(node_feature), split_label=int(split_label),
+                   adaptive=int(adaptive), adp_depth=adp_depth, th_normal=th_normal,
+                   th_distance=th_distance, extrapolate=int(extrapolate), save_pts=int(save_pts),
+                   key2xyz=int(key2xyz), merged=int(merged), has_bbox=int(bbox is not None))
+  if bbox is not None:
+    bp.bbmin = (C.c_float * 3)(*bbox[0])
+    bp.bbmax = (C.c_float * 3)(*bbox[1])
+  eff_depth = max(depth, max(full_depth, 1))
+  ws_bytes = L.ocnn_points2octree_workspace_bytes(total, n, eff_depth)
+  if ws_bytes == 0:
+    raise OcnnError(-1, "bad build arguments (points %d, clouds %d, depth %d)" % (total, n, depth))
+  ws = _workspace(ws_bytes + 256, "build")
+  base = (ws.data_ptr() + 255) & ~255
+  dev_ptrs = (C.c_void_p * n)(*[p.data_ptr() for p in pts])
+  hdr_ptrs = (C.c_void_p * n)(*[h.ctypes.data for h in hdrs])
+  info_raw = np.zeros(INFO_BYTES, np.uint8)
+  _lib.call("ocnn_points2octree_plan", dev_ptrs, hdr_ptrs, n, C.byref(bp), C.c_void_p(base),
+            C.c_size_t(ws_bytes), C.c_void_p(info_raw.ctypes.data), _stream())
+  info = _Info(info_raw)
+  out = torch.empty(info.size(), dtype=torch.uint8, device=_dev())
+  _lib.call("ocnn_points2octree_emit", _ptr(out), info.p, C.c_void_p(base), C.c_size_t(ws_bytes),
+            _stream())
+  out._ocnn_info = info
+  return out
+
+
+def points2octree(points, depth, full_depth=2, node_dis=False, node_feature=False,
+                  split_label=False, adaptive=False, adp_depth=4, th_normal=0.1,
+                  th_distance=2.0, extrapolate=False, save_pts=False, key2xyz=False):
+  """pytorch/cpp/point2octree.cpp:5-34 -- one serialized octree from one point cloud."""
+  return _build([points], False, depth, full_depth, node_dis, node_feature, split_label,
+                adaptive, adp_depth, th_normal, th_distance, extrapolate, save_pts, key2xyz)
+
+
+def points2octree_batch(points_list, depth, full_depth=2, node_dis=False, node_feature=False,
+                        split_label=False, adaptive=False, adp_depth=4, th_normal=0.1,
+                        th_distance=2.0, extrapolate=False, save_pts=False, key2xyz=False):
+  """`octree_batch([points2octree(p, ...) for p in points_list])` in one device pass
+  (the composition `collate_octrees` performs, pytorch/ocnn/transforms.py:127-148)."""
+  return _build(list(points_list), True, depth, full_depth, node_dis, node_feature, split_label,
+                adaptive, adp_depth, th_normal, th_distance, extrapolate, save_pts, key2xyz)
+
+
+def octree_batch(octrees):
+  """pytorch/cpp/octree_batch.cpp:5-22 -- merge serialized octrees, add neighbour tables."""
+  octs = [_to_dev(o) for o in octrees]
+  infos = [octree_info(o) for o in octs]
+  n = len(octs)
+  L = _lib.get()
+  info_ptrs = (C.c_void_p * n)(*[i.raw.ctypes.data for i in infos])
+  out_raw = np.zeros(INFO_BYTES, np.uint8)
+  _lib.call("ocnn_octree_batch_info", info_ptrs, n, C.c_void_p(out_raw.ctypes.data))
+  out_info = _Info(out_raw)
+  out = torch.empty(out_info.size(), dtype=torch.uint8, device=_dev())
+  ws_bytes = L.ocnn_octree_batch_workspace_bytes(n, out_info.depth)
+  ws = _workspace(ws_bytes, "batch")
+  dev_ptrs = (C.c_void_p * n)(*[o.data_ptr() for o in octs])
+  _lib.call("ocnn_octree_batch", _ptr(out), out_info.p, dev_ptrs, info_ptrs, n, _ptr(ws),
+            C.c_size_t(ws_bytes), _stream())
+  out._ocnn_info = out_info
+  return out
+
+
+def points_new(pts, normals=None, features=None, labels=None):
+  """pytorch/cpp/points_property.cpp `points_new`: serialized point cloud (88-byte header,
+  then xyz, normal, feature, label arrays point-major: octree/octree/points.cpp:96-148)."""
+  dev = pts.device
+  pts = pts.reshape(-1, 3).to(torch.float32).contiguous()
+  n = pts.shape[0]
+  if n == 0:
+    raise ValueError("empty point cloud")
+  arrs, chans, flags = [pts], [3, 0, 0, 0], 1
+  for i, a in enumerate((normals, features, labels), start=1):
+    if a is None or a.numel() == 0:
+      continue
+    a = a.reshape(n, -1).to(torch.float32).contiguous()
+    if (i == 1 and a.shape[1] != 3) or (i == 3 and a.shape[1] != 1):
+      raise ValueError("normals need 3 channels and labels 1")
+    chans[i] = a.shape[1]
+    flags |= 1 << i
+    arrs.append(a)
+  hdr = np.zeros(_lib.POINTS_INFO_BYTES, np.uint8)
+  hdr[:12] = np.frombuffer(b"_POINTS_1.0_", np.uint8)
+  ints = hdr[16:].view(np.int32)
+  ints[0], ints[1] = n, flags
+  ints[2:6] = chans
+  dis = [_lib.POINTS_INFO_BYTES]
+  for c in chans:
+    dis.append(dis[-1] + 4 * n * c)
+  ints[10:15] = dis
+  parts = [torch.from_numpy(hdr).to(dev)] + [a.reshape(-1).view(torch.uint8) for a in arrs]
+  out = torch.cat(parts)
+  out._ocnn_points_info = hdr
+  return out
+
+
+# ---- properties ------------------------------------------------------------------------
+def octree_property(octree, property, depth=0):
+  """pytorch/cpp/octree_property.cpp:11-344."""
+  info = octree_info(octree)
+  name = property
+  nnum = info.nnum(depth) if depth > 0 else info.total_nnum()
+  dev = octree.device
+  if name in ("key", "xyz"):
+    ch = info.channel(KEY)
+    src = _prop_view(octree, info, KEY, depth, ch * nnum, torch.int64)
+    convert = info.key2xyz if name == "key" else not info.key2xyz
+    if not convert:
+      return src.clone()
+    fn = "ocnn_xyz2key" if name == "key" else "ocnn_key2xyz"
+    src_d = _to_dev(src)
+    out = torch.zeros_like(src_d)
+    if depth > 0:
+      _lib.call(fn, _ptr(out), _ptr(src_d), ch * nnum, depth, _stream())
+    else:   # depth 0 is left as zero, as in the reference loop (d = 1 .. depth)
+      for d in range(1, info.depth + 1):
+        n_d, c_d = info.nnum(d), info.nnum_cum(d)
+        if n_d:
+          _lib.call(fn, _ptr(out[c_d:c_d + n_d]), _ptr(src_d[c_d:c_d + n_d]), n_d, d, _stream())
+    return out.to(dev)
+  if name == "index":
+    ch = info.channel(KEY)
+    src = _to_dev(_prop_view(octree, info, KEY, depth, ch * nnum, torch.int64))
+    out = torch.zeros(ch * nnum, dtype=torch.int32, device=src.device)
+    _lib.call("ocnn_key2idx", _ptr(out), _ptr(src), ch * nnum, _stream())
+    return out.to(dev)
+  if name == "child":
+    return _prop_view(octree, info, CHILD, depth, nnum * info.channel(CHILD), torch.int32).clone()
+  if name == "neigh":
+    ch = info.channel(NEIGH)
+    return _prop_view(octree, info, NEIGH, depth, nnum * ch, torch.int32).clone().view(nnum, ch)
+  if name == "feature":
+    ch = info.channel(FEATURE)
+    v = _prop_view(octree, info, FEATURE, depth, nnum * ch, torch.float32)
+    if v is None:
+      raise OcnnError(-6, "The features do not exist: d = %d" % depth)
+    return v.clone().view(1, ch, nnum, 1)
+  if name == "label":
+    return _prop_view(octree, info, LABEL, depth, nnum * info.channel(LABEL), torch.float32).clone()
+  if name == "split":
+    return _prop_view(octree, info, SPLIT, depth, nnum * info.channel(SPLIT), torch.float32).clone()
+  ints = None
+  if name == "node_num":
+    ints = [info.nnum(depth)] if depth > 0 else [info.nnum(d) for d in range(info.depth + 1)]
+  elif name in ("node_num_ne", "node_num_nempty"):
+    ints = [info.nnum_nempty(depth)] if depth > 0 else \
+        [info.nnum_nempty(d) for d in range(info.depth + 1)]
+  elif name == "node_num_cum":
+    ints = [info.nnum_cum(depth)] if depth > 0 else [info.nnum_cum(d) for d in range(info.depth + 2)]
+  elif name == "batch_size":
+    ints = [info.batch_size]
+  elif name == "depth":
+    ints = [info.depth]
+  elif name == "full_depth":
+    ints = [info.full_depth]
+  if ints is None:
+    raise OcnnError(-1, "Unsupport octree property: %s" % name)
+  return torch.tensor(ints, dtype=torch.int32, device=dev)
+
+
+def octree_set_property(octree, data, depth):
+  """pytorch/cpp/octree_property.cpp:308-325 -- returns a copy with the features of one depth replaced."""
+  info = octree_info(octree)
+  count = info.nnum(depth) * info.channel(FEATURE)
+  if data.numel() != count:
+    raise OcnnError(-3, "Wrong Property Size")
+  out = octree.clone()
+  out._ocnn_info = info
+  _prop_view(out, info, FEATURE, depth, count, torch.float32).copy_(
+      data.to(torch.float32).reshape(-1))
+  return out
+
+
+# ---- octree2col / col2octree ---------------------------------------------------------------
+def _ichild(octree, info, depth):
+  n, ne = info.nnum(depth), info.nnum_nempty(depth)
+  child = _prop_view(octree, info, CHILD, depth, n, torch.int32)
+  ichild = torch.zeros(max(ne, 1), dtype=torch.int32, device=octree.device)
+  _lib.call("ocnn_make_ichild", _ptr(ichild), ne, _ptr(child), n, _stream())
+  return child, ichild
+
+
+def octree2col(data_in, octree, depth, kernel_size, stride, nempty):
+  """pytorch/cpp/octree2col.cpp:47-237: [1,C,H,1] -> [C, K, H_out]."""
+  octree = _to_dev(octree)
+  info = octree_info(octree)
+  ksc, ks = _ks(kernel_size)
+  data_in = data_in.contiguous()
+  dt = _dtype_code(data_in)
+  channel, btm_h = data_in.size(1), data_in.size(2)
+  K = ks[0] * ks[1] * ks[2]
+  neigh = _prop_view(octree, info, NEIGH, depth, info.nnum(depth) * 8, torch.int32)
+  if not nempty:
+    if btm_h != info.nnum(depth):
+      raise OcnnError(-3, "octree2col: height %d != node_num(%d) = %d" % (btm_h, depth, info.nnum(depth)))
+    top_h = btm_h
+    if stride == 2:
+      top_h = btm_h // 8
+      if top_h != info.nnum_nempty(depth - 1):
+        raise OcnnError(-3, "octree2col: stride-2 height mismatch")
+    out = torch.zeros(channel, K, top_h, dtype=data_in.dtype, device=data_in.device)
+    _lib.call("ocnn_octree2col", _ptr(out), _ptr(data_in), channel, top_h, ksc, stride, _ptr(neigh),
+              max(top_h, 1), 0, dt, _stream())
+    return out
+  if btm_h != info.nnum_nempty(depth):
+    raise OcnnError(-3, "octree2col: height %d != node_num_nempty(%d)" % (btm_h, depth))
+  child, ichild = _ichild(octree, info, depth)
+  top_h = btm_h if stride == 1 else info.nnum_nempty(depth - 1)
+  out = torch.zeros(channel, K, top_h, dtype=data_in.dtype, device=data_in.device)
+  _lib.call("ocnn_octree2colP", _ptr(out), _ptr(data_in), channel, top_h, btm_h, ksc, stride,
+            _ptr(neigh), _ptr(child), _ptr(ichild), max(top_h, 1), 0, dt, _stream())
+  return out
+
+
+def col2octree(grad_in, octree, depth, kernel_size, stride, nempty):
+  """pytorch/cpp/octree2col.cpp:95-237: [C, K, H_out] -> [1,C,H,1] (scatter-add)."""
+  octree = _to_dev(octree)
+  info = octree_info(octree)
+  ksc, ks = _ks(kernel_size)
+  grad_in = grad_in.contiguous()
+  dt = _dtype_code(grad_in)
+  channel, top_h = grad_in.size(0), grad_in.size(2)
+  neigh = _prop_view(octree, info, NEIGH, depth, info.nnum(depth) * 8, torch.int32)
+  if stride == 2 and top_h != info.nnum_nempty(depth - 1):
+    raise OcnnError(-3, "col2octree: stride-2 height mismatch")
+  if not nempty:
+    btm_h = info.nnum(depth)
+    out = torch.zeros(1, channel, btm_h, 1, dtype=grad_in.dtype, device=grad_in.device)
+    _lib.call("ocnn_col2octree", _ptr(grad_in), _ptr(out), channel, top_h, ksc, stride, _ptr(neigh),
+              max(top_h, 1), 0, dt, _stream())
+    return out
+  btm_h = info.nnum_nempty(depth)
+  if stride == 1 and top_h != btm_h:
+    raise OcnnError(-3, "col2octree: height mismatch")
+  child, ichild = _ichild(octree, info, depth)
+  out = torch.zeros(1, channel, btm_h, 1, dtype=grad_in.dtype, device=grad_in.device)
+  _lib.call("ocnn_col2octreeP", _ptr(grad_in), _ptr(out), channel, top_h, btm_h, ksc, stride,
+            _ptr(neigh), _ptr(child), _ptr(ichild), max(top_h, 1), 0, dt, _stream())
+  return out
+
+
+# ---- convolution -------------------------------------------------------------------------------
+def _conv(fn, is_deconv, data_in, weights, octree, depth, num_output, kernel_size, stride, nempty):
+  octree = _to_dev(octree)
+  info = octree_info(octree)
+  ksc, _ = _ks(kernel_size)
+  data_in = data_in.contiguous()
+  weights = weights.contiguous()
+  dt = _dtype_code(data_in)
+  if weights.dtype != data_in.dtype:
+    raise TypeError("weights and data must have the same dtype")
+  channel_in, btm_h = data_in.size(1), data_in.size(2)
+  top_h, need_h, ws_bytes = C.c_int(), C.c_int(), C.c_size_t()
+  _lib.call("ocnn_conv_shape", info.p, depth, channel_in, num_output, ksc, stride, int(nempty),
+            int(is_deconv), dt, C.byref(top_h), C.byref(need_h), C.byref(ws_bytes))
+  ws = _workspace(ws_bytes.value + 256, "conv")
+  base = (ws.data_ptr() + 255) & ~255
+  out = torch.empty(1, num_output, top_h.value, 1, dtype=data_in.dtype, device=data_in.device)
+  _lib.call(fn, _ptr(out), _ptr(data_in), channel_in, btm_h, _ptr(weights), _ptr(octree), info.p,
+            depth, num_output, ksc, stride, int(nempty), dt, C.c_void_p(base),
+            C.c_size_t(ws_bytes.value), _stream())
+  return out
+
+
+def octree_conv(data_in, weights, octree, depth, num_output, kernel_size, stride, nempty):
+  """pytorch/cpp/octree_conv.cpp:131-157: [1,Ci,H,1] x [Co, Ci*K] -> [1,Co,top_h,1]."""
+  return _conv("ocnn_octree_conv", False, data_in, weights, octree, depth, num_output,
+               kernel_size, stride, nempty)
+
+
+def octree_deconv(data_in, weights, octree, depth, num_output, kernel_size, stride, nempty):
+  """pytorch/cpp/octree_conv.cpp:189-216: weights are [Ci, Co*K]."""
+  return _conv("ocnn_octree_deconv", True, data_in, weights, octree, depth, num_output,
+               kernel_size, stride, nempty)
+
+
+# ---- pad / pool ------------------------------------------------------------------------------------
+def octree_pad(data_in, octree, depth, val=0.0):
+  """pytorch/cpp/octree_pad.cpp:6-32."""
+  octree = _to_dev(octree)
+  info = octree_info(octree)
+  if depth < 1:
+    raise OcnnError(-1, "Depth should be larger than 1")
+  data_in = data_in.contiguous()
+  channel, btm_h = data_in.size(1), data_in.size(2)
+  if btm_h != info.nnum_nempty(depth):
+    raise OcnnError(-3, "pad, d = %d, channel = %d: height %d != %d" %
+                    (depth, channel, btm_h, info.nnum_nempty(depth)))
+  top_h = info.nnum(depth)
+  child = _prop_view(octree, info, CHILD, depth, top_h, torch.int32)
+  out = torch.empty(1, channel, top_h, 1, dtype=data_in.dtype, device=data_in.device)
+  _lib.call("ocnn_pad_forward", _ptr(out), top_h, channel, _ptr(data_in), btm_h, _ptr(child),
+            C.c_float(val), _dtype_code(data_in), _stream())
+  return out
+
+
+def octree_depad(data_in, octree, depth):
+  """pytorch/cpp/octree_pad.cpp:34-60."""
+  octree = _to_dev(octree)
+  info = octree_info(octree)
+  if depth < 1:
+    raise OcnnError(-1, "Depth should be larger than 1")
+  data_in = data_in.contiguous()
+  channel, top_h = data_in.size(1), data_in.size(2)
+  if top_h != info.nnum(depth):
+    raise OcnnError(-3, "depad, d = %d, channel = %d: height %d != %d" %
+                    (depth, channel, top_h, info.nnum(depth)))
+  btm_h = info.nnum_nempty(depth)
+  child = _prop_view(octree, info, CHILD, depth, top_h, torch.int32)
+  out = torch.zeros(1, channel, btm_h, 1, dtype=data_in.dtype, device=data_in.device)
+  _lib.call("ocnn_pad_backward", _ptr(out), btm_h, channel, _ptr(data_in), top_h, _ptr(child),
+            _dtype_code(data_in), _stream())
+  return out
+
+
+def octree_max_pool(data_in, octree, depth):
+  """pytorch/cpp/octree_pool.cpp:6-34: `depth` is the input depth; returns (pooled, mask)."""
+  info = octree_info(octree)
+  data_in = data_in.contiguous()
+  channel, btm_h = data_in.size(1), data_in.size(2)
+  if info.nnum(depth) != btm_h:
+    raise OcnnError(-3, "max_pool: height %d != node_num(%d) = %d" % (btm_h, depth, info.nnum(depth)))
+  if depth <= 1:
+    raise OcnnError(-1, "Depth should be larger than 1")
+  top_h = btm_h >> 3
+  top = torch.empty(1, channel, top_h, 1, dtype=data_in.dtype, device=data_in.device)
+  mask = torch.empty(1, channel, top_h, 1, dtype=torch.int32, device=data_in.device)
+  _lib.call("ocnn_octree_max_pool", _ptr(top), top_h, _ptr(mask), _ptr(data_in), btm_h, channel,
+            _dtype_code(data_in), _stream())
+  return top, mask
+
+
+def octree_max_unpool(data_in, mask, octree, depth):
+  """pytorch/cpp/octree_pool.cpp:36-62: `depth` is the output depth."""
+  info = octree_info(octree)
+  data_in = data_in.contiguous()
+  mask = mask.contiguous()
+  channel, top_h = data_in.size(1), data_in.size(2)
+  if top_h != info.nnum_nempty(depth - 1):
+    raise OcnnError(-3, "max_unpool: height %d != node_num_nempty(%d)" % (top_h, depth - 1))
+  if mask.size(1) != channel or mask.size(2) != top_h:
+    raise OcnnError(-3, "max_unpool: mask shape")
+  btm_h = top_h << 3
+  btm = torch.empty(1, channel, btm_h, 1, dtype=data_in.dtype, device=data_in.device)
+  _lib.call("ocnn_octree_max_unpool", _ptr(data_in), top_h, _ptr(mask), _ptr(btm), btm_h, channel,
+            _dtype_code(data_in), _stream())
+  return btm
+
+
+def octree_mask_pool(data_in, mask, octree, depth):
+  """pytorch/cpp/octree_pool.cpp:64-90."""
+  info = octree_info(octree)
+  data_in = data_in.contiguous()
+  mask = mask.contiguous()
+  channel, btm_h = data_in.size(1), data_in.size(2)
+  top_h = mask.size(2)
+  if info.nnum(depth) != btm_h or top_h != btm_h >> 3:
+    raise OcnnError(-3, "mask_pool: height mismatch")
+  top = torch.empty(1, channel, top_h, 1, dtype=data_in.dtype, device=data_in.device)
+  _lib.call("ocnn_octree_mask_pool", _ptr(top), top_h, _ptr(mask), _ptr(data_in), btm_h, channel,
+            _dtype_code(data_in), _stream())
+  return top
+
+
+# ---- keys ----------------------------------------------------------------------------------------------
+def octree_encode_key(xyz):
+  """pytorch/cpp/octree_key.cpp:11-29: int16 [N,4] (x,y,z,id) -> int64 [N] (bit copy)."""
+  if xyz.dim() != 2 or xyz.size(1) != 4:
+    raise OcnnError(-1, "The input must be [N, 4]")
+  return xyz.contiguous().to(torch.int16).view(torch.int64).reshape(-1).clone()
+
+
+def octree_decode_key(key):
+  """pytorch/cpp/octree_key.cpp:31-47."""
+  if key.dim() != 1:
+    raise OcnnError(-1, "The dim of input tensor must be 1.")
+  return key.contiguous().view(torch.int16).reshape(-1, 4).clone()
+
+
+def _key_op(fn, t, depth):
+  t = t.contiguous()
+  if t.numel() < 1:
+    raise OcnnError(-1, "The numel of the input tensor must be larger than 1.")
+  src = _to_dev(t)
+  out = torch.empty_like(src)
+  _lib.call(fn, _ptr(out), _ptr(src), src.numel(), depth, _stream())
+  return out.to(t.device)
+
+
+def octree_xyz2key(xyz, depth):
+  """pytorch/cpp/octree_key.cpp:49-64."""
+  return _key_op("ocnn_xyz2key", xyz, depth)
+
+
+def octree_key2xyz(key, depth):
+  """pytorch/cpp/octree_key.cpp:66-81."""
+  return _key_op("ocnn_key2xyz", key, depth)
+
+
+def octree_search_key(key, octree, depth, key_is_xyz, nempty):
+  """pytorch/cpp/octree_key.cpp:83-132: index of each query key at `depth`, -1 on a miss."""
+  octree = _to_dev(octree)
+  info = octree_info(octree)
+  key = _to_dev(key.contiguous())
+  n_query = key.numel()
+  if n_query < 1:
+    raise OcnnError(-1, "The numel of the input tensor must be larger than 1.")
+  if key_is_xyz:
+    tmp = torch.empty_like(key)
+    _lib.call("ocnn_xyz2key", _ptr(tmp), _ptr(key), n_query, depth, _stream())
+    key = tmp
+  des_h = info.nnum(depth)
+  des = _prop_view(octree, info, KEY, depth, des_h, torch.int64)
+  if nempty:
+    ne = info.nnum_nempty(depth)
+    child = _prop_view(octree, info, CHILD, depth, des_h, torch.int32)
+    # keys of the non-empty nodes, in node order (the reference depads the key array)
+    tmp = torch.zeros(max(ne, 1), dtype=torch.int64, device=octree.device)
+    tmp[:ne] = des[child >= 0]
+    des, des_h = tmp, ne
+  if info.key2xyz:
+    tmp = torch.empty_like(des)
+    if des_h:
+      _lib.call("ocnn_xyz2key", _ptr(tmp), _ptr(des), des_h, depth, _stream())
+    des = tmp
+  out = torch.empty(n_query, dtype=torch.int32, device=octree.device)
+  _lib.call("ocnn_search_key", _ptr(out), _ptr(des), des_h, _ptr(key), n_query, _stream())
+  return out
+
+
+# ---- growth ----------------------------------------------------------------------------------------------
+def octree_new(batch_size, channel, node_dis, adaptive_layer=0):
+  """pytorch/cpp/octree_grow.cpp:110-153."""
+  raw = np.zeros(INFO_BYTES, np.uint8)
+  _lib.call("ocnn_octree_new_info", batch_size, channel, int(node_dis), adaptive_layer,
+            C.c_void_p(raw.ctypes.data))
+  info = _Info(raw)
+  out = torch.empty(info.size(), dtype=torch.uint8, device=_dev())
+  _lib.call("ocnn_octree_new", _ptr(out), info.p, _stream())
+  out._ocnn_info = info
+  return out
+
+
+def octree_grow(octree_in, target_depth, full_octree):
+  """pytorch/cpp/octree_grow.cpp:13-54."""
+  octree_in = _to_dev(octree_in)
+  iin = octree_info(octree_in)
+  raw = np.zeros(INFO_BYTES, np.uint8)
+  _lib.call("ocnn_octree_grow_info", iin.p, target_depth, int(full_octree), C.c_void_p(raw.ctypes.data))
+  info = _Info(raw)
+  out = torch.empty(info.size(), dtype=torch.uint8, device=octree_in.device)
+  _lib.call("ocnn_octree_grow", _ptr(out), info.p, _ptr(octree_in), iin.p, target_depth,
+            int(full_octree), _stream())
+  out._ocnn_info = info
+  return out
+
+
+def octree_update(octree_in, label_in, depth, split):
+  """pytorch/cpp/octree_grow.cpp:164-190: children[depth] from the split labels."""
+  octree_in = _to_dev(octree_in)
+  iin = octree_info(octree_in)
+  out = octree_in.clone()
+  info = _Info(iin.raw)
+  label = _to_dev(label_in.contiguous().to(torch.int32))
+  n = label.numel()
+  sb = _lib.get().ocnn_octree_update_scratch_bytes(n)
+  ws = _workspace(sb + 256, "update")
+  base = (ws.data_ptr() + 255) & ~255
+  _lib.call("ocnn_octree_update", _ptr(out), info.p, _ptr(label), n, depth, split,
+            C.c_void_p(base), C.c_size_t(sb), _stream())
+  out._ocnn_info = _Info(info.raw)
+  return out
