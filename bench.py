@@ -1,0 +1,249 @@
+"""Benchmark of the octree hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
+
+Workload (BASELINE.json configs[3], the configuration the metric is quoted on): a
+synthetic 5 m x 5 m x 3 m room sampled to 250 000 points, built on the GPU into an
+octree of depth 9 (full_depth 2).  One step = one 3x3x3 stride-1 octree convolution
+with Cin = Cout = 64 in fp32 over all depth-9 octants, inputs resident in HBM.
+`value` = octants/s of that step.  Sub-measurements of the other kernels of the path
+(bf16 conv, stride-2 conv, depth-7 batch, octree build, neighbour table, pooling) go
+to `extra`, each timed with HIP events on the stream the kernels run on.
+Prints ONE JSON line.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0
+PEAK_MFMA_TFLOPS = {"f32": 157.3, "bf16": 2500.0}
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--gpus", type=int, default=1)
+  ap.add_argument("--steps", type=int, default=20)
+  ap.add_argument("--warmup", type=int, default=3)
+  ap.add_argument("--quick", action="store_true", help="skip the sub-measurements and the CPU baseline")
+  ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+  args = ap.parse_args()
+  if args.gpus != 1:
+    print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
+          file=sys.stderr)
+    sys.exit(2)
+
+  import torch
+  oc = importlib.import_module("o-cnn_amd")
+  F = oc.nn
+  oc.lib.call("ocnn_device_check", 0)
+  torch.cuda.set_device(0)
+  dev = torch.device("cuda", 0)
+
+  def timed(fn, steps, warmup):
+    """average milliseconds per call, HIP events on the current stream"""
+    for _ in range(warmup):
+      fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+      fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+  def points_tensor(p, n, f):
+    return F.points_new(torch.from_numpy(p), torch.from_numpy(n),
+                        torch.from_numpy(f) if f is not None else None).to(dev)
+
+  # ---- scene octree, depth 9 (built on the GPU) ------------------------------------------
+  pts, nrm, rgb = oc.synthetic.room_cloud(250000, 3)
+  scene_pts = points_tensor(pts, nrm, rgb)
+  scene_pts._ocnn_points_info = scene_pts[:88].cpu().numpy().copy()
+  octree = F.points2octree_batch([scene_pts], 9, 2)
+  info = F.octree_info(octree)
+  depth = 9
+  H9, H8, Hne9, Hne8 = info.nnum(9), info.nnum(8), info.nnum_nempty(9), info.nnum_nempty(8)
+
+  C = 64
+  g = torch.Generator(device="cpu").manual_seed(2)
+  x32 = torch.randn(1, C, H9, 1, generator=g).to(dev)
+  w32 = (torch.randn(C, C * 27, generator=g) * 0.02).to(dev)
+
+  def conv_step():
+    return F.octree_conv(x32, w32, octree, depth, C, [3, 3, 3], 1, False)
+
+  # ---- timed region of the headline metric -------------------------------------------------
+  for _ in range(args.warmup):
+    conv_step()
+  torch.cuda.synchronize()
+  e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+  t0 = time.perf_counter()
+  e0.record()
+  for _ in range(args.steps):
+    conv_step()
+  e1.record()
+  torch.cuda.synchronize()
+  wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+  ms = e0.elapsed_time(e1) / args.steps
+  flops = 2.0 * H9 * 27 * C * C
+  value = H9 / (ms * 1e-3)
+  achieved_tflops = flops / (ms * 1e-3) / 1e12
+
+  out = {
+      "metric": "octree-conv octants/s (3x3x3 stride 1, Cin=Cout=64, depth 9)",
+      "value": value,
+      "unit": "octants/s",
+      "n_gpus": 1,
+      "steps": args.steps,
+      "warmup": args.warmup,
+      "ms_per_step": ms,
+      "higher_is_better": True,
+      "scaling": "weak",
+      "vs_baseline": None,
+      "dtype": "f32",
+      "data": "synthetic",
+      "config": {"workload": "cfg4 scene: 250000-point room, octree depth 9 full_depth 2, "
+                             "conv 3x3x3 s1 64->64 over %d octants" % H9,
+                 "octants_d9": H9, "octants_d8": H8, "nonempty_d9": Hne9, "points": 250000},
+      "roofline": {"bound": "mfma", "achieved": achieved_tflops, "peak": PEAK_MFMA_TFLOPS["f32"],
+                   "unit": "TFLOP/s", "frac": achieved_tflops / PEAK_MFMA_TFLOPS["f32"],
+                   "traffic": None, "kernel": "conv_f32_kernel",
+                   "algorithmic_flops_per_launch": flops},
+      "wall_ms_per_step": wall_ms,
+  }
+
+  extra = {}
+  if not args.quick:
+    reps, wu = max(3, args.steps // 4), 1
+
+    def conv_case(name, oct_, d, x, w, ks, stride, nempty=False, deconv=False, n_out=C):
+      fn = F.octree_deconv if deconv else F.octree_conv
+      t = timed(lambda: fn(x, w, oct_, d, n_out, ks, stride, nempty), reps, wu)
+      K = ks[0] * ks[1] * ks[2]
+      cols = x.shape[2] if stride == 1 else (x.shape[2] // 8 if not deconv else x.shape[2])
+      fl = 2.0 * cols * K * x.shape[1] * n_out
+      dt = "bf16" if x.dtype == torch.bfloat16 else "f32"
+      extra[name] = {"ms": t, "octants_per_s": x.shape[2] / (t * 1e-3),
+                     "tflops": fl / (t * 1e-3) / 1e12,
+                     "frac_mfma_peak": fl / (t * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS[dt]}
+
+    x16, w16 = x32.bfloat16(), w32.bfloat16()
+    conv_case("conv333_s1_d9_bf16", octree, 9, x16, w16, [3, 3, 3], 1)
+    w2 = (torch.randn(C, C * 8, generator=g) * 0.02).to(dev)
+    conv_case("conv222_s2_d9_f32", octree, 9, x32, w2, [2, 2, 2], 2)
+    conv_case("conv222_s2_d9_bf16", octree, 9, x16, w2.bfloat16(), [2, 2, 2], 2)
+    xne = torch.randn(1, C, Hne9, 1, generator=g).to(dev)
+    conv_case("conv333_s1_d9_f32_nempty", octree, 9, xne, w32, [3, 3, 3], 1, nempty=True)
+    x8 = torch.randn(1, C, Hne8, 1, generator=g).to(dev)
+    conv_case("deconv222_s2_d8to9_f32", octree, 8, x8, w2, [2, 2, 2], 2, deconv=True)
+
+    # bandwidth-bound kernels on the depth-9 scene (algorithmic bytes / time)
+    s = 4
+    t = timed(lambda: F.octree_max_pool(x32, octree, 9), reps, wu)
+    by = C * H9 * s + C * (H9 // 8) * (s + 4)
+    extra["max_pool_d9_f32"] = {"ms": t, "GBs": by / t / 1e6, "frac_hbm_peak": by / t / 1e6 / PEAK_HBM_GBS}
+    top, mask = F.octree_max_pool(x32, octree, 9)
+    t = timed(lambda: F.octree_max_unpool(top, mask, octree, 9), reps, wu)
+    extra["max_unpool_d9_f32"] = {"ms": t, "GBs": by / t / 1e6, "frac_hbm_peak": by / t / 1e6 / PEAK_HBM_GBS}
+    t = timed(lambda: F.octree_pad(top, octree, 8), reps, wu)
+    by = C * (Hne8 + H8) * s + H8 * 4
+    extra["pad_d8_f32"] = {"ms": t, "GBs": by / t / 1e6, "frac_hbm_peak": by / t / 1e6 / PEAK_HBM_GBS}
+    # neighbour table of depth 9 from depth 8 (the kernel octree_batch / octree_grow run)
+    neigh8 = F.octree_property(octree, "neigh", 8).reshape(-1)
+    child8 = F.octree_property(octree, "child", 8)
+    neigh9 = torch.empty(H9 * 8, dtype=torch.int32, device=dev)
+    import ctypes as Ct
+    st = lambda: Ct.c_void_p(torch.cuda.current_stream().cuda_stream)
+    t = timed(lambda: oc.lib.call("ocnn_calc_neigh_sparse", Ct.c_void_p(neigh9.data_ptr()),
+                                  Ct.c_void_p(neigh8.data_ptr()), Ct.c_void_p(child8.data_ptr()),
+                                  H8, st()), reps, wu)
+    by = H9 * 8 * 4 + H8 * (4 + 8 * 4)
+    extra["calc_neigh_d9"] = {"ms": t, "GBs": by / t / 1e6, "frac_hbm_peak": by / t / 1e6 / PEAK_HBM_GBS}
+
+    # octree construction: wall time including its one device-to-host copy
+    def build_scene():
+      return F.points2octree_batch([scene_pts], 9, 2)
+    build_scene()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+      build_scene()
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / reps
+    by = 250000 * (12 + 12 + 12) + sum(info.nnum(d) * (12 + 32) for d in range(10)) + H9 * 4 * 6 + 720
+    extra["points2octree_scene_d9"] = {"ms": t * 1e3, "Mpts_per_s": 0.25 / t,
+                                       "GBs": by / t / 1e9, "frac_hbm_peak": by / t / 1e9 / PEAK_HBM_GBS}
+
+    # depth-7 batch (configs[2]): 16 clouds of 50 000 points
+    clouds = [oc.synthetic.shape_cloud(50000, 200 + i) for i in range(16)]
+    cl = [points_tensor(*c) for c in clouds]
+    for c in cl:
+      c._ocnn_points_info = c[:88].cpu().numpy().copy()
+    oct7 = F.points2octree_batch(cl, 7, 2)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+      F.points2octree_batch(cl, 7, 2)
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / reps
+    extra["points2octree_batch16_d7"] = {"ms": t * 1e3, "Mpts_per_s": 0.8 / t}
+    i7 = F.octree_info(oct7)
+    H7 = i7.nnum(7)
+    x7 = torch.randn(1, C, H7, 1, generator=g).to(dev)
+    extra["octants_d7"] = H7
+    conv_case("conv333_s1_d7_f32", oct7, 7, x7, w32, [3, 3, 3], 1)
+    conv_case("conv333_s1_d7_bf16", oct7, 7, x7.bfloat16(), w16, [3, 3, 3], 1)
+    conv_case("conv222_s2_d7_f32", oct7, 7, x7, w2, [2, 2, 2], 2)
+  out["extra"] = extra
+
+  # ---- CPU baseline (reported, not the target) -----------------------------------------------
+  if not (args.quick or args.no_cpu):
+    from oracle.checker import Checker, OctreeBlob
+    orc = Checker("orc")
+    blob_host = octree.cpu().numpy()
+    ob = OctreeBlob(blob_host)
+    sample = 32768
+    neigh = ob.prop("neigh", 9).reshape(-1)
+    xh = x32.cpu().numpy().reshape(C, H9)
+    wh = w32.cpu().numpy()
+    ni = orc.get_ni([3, 3, 3])
+    col = np.empty((C * 27, sample), np.float32)
+    import ctypes as Ct
+    P = lambda a: a.ctypes.data_as(Ct.c_void_p)
+    t0 = time.perf_counter()
+    # first chunk of `sample` columns: octree2col_cpu chunk + single-thread SGEMM
+    orc.fn("octree2col")(P(col), P(xh), C, H9, 27, 1, P(neigh), P(ni), sample, 0)
+    y = orc.sgemm(wh, col)
+    t = time.perf_counter() - t0
+    out["cpu_baseline"] = {"value": sample / t, "unit": "octants/s", "cores": 1, "kind": "port",
+                           "sample": "first %d of %d depth-9 octants: octree2col_cpu chunk + "
+                                     "single-thread textbook SGEMM (64 x 1728 x %d), %.1f s"
+                                     % (sample, H9, sample, t)}
+    # the sample also checks the GPU result
+    yg = conv_step().cpu().numpy().reshape(C, H9)[:, :sample]
+    out["cpu_baseline"]["gpu_vs_cpu_max_rel_err"] = float(np.abs(yg - y).max() / np.abs(y).max())
+    ref_ok = os.path.exists(os.path.join(ROOT, "oracle", "_ref", "libocnn_ref.so"))
+    chk = Checker("ref") if ref_ok else orc
+    pb = scene_pts.cpu().numpy()
+    t0 = time.perf_counter()
+    single = chk.points2octree(pb, 9, 2)
+    merged = chk.octree_batch([single])
+    t = time.perf_counter() - t0
+    out["cpu_baseline"]["points2octree_plus_batch"] = {
+        "Mpts_per_s": 0.25 / t, "seconds": t, "cores": 1, "kind": "reference" if ref_ok else "port",
+        "bit_exact_vs_gpu": bool(np.array_equal(merged, blob_host))}
+
+  print(json.dumps(out))
+
+
+if __name__ == "__main__":
+  main()

@@ -1,0 +1,72 @@
+"""Writes the golden fixtures of tests/golden/ from the REAL reference, compiled from
+its own sources into oracle/_ref/libocnn_ref.so by oracle/Makefile.  Run in the build
+container (the reference checkout must be present):
+
+    python tests/golden/make_golden.py
+
+Outputs (data only -- inputs and expected outputs):
+  octree_samples.npz   the six octree blobs embedded in the reference's
+                       octree/octree/octree_samples.cpp (octree_1 .. octree_6), as
+                       `octree::get_one_octree` returns them in a 64-bit-key build;
+                       these are the shared fixtures of the reference's own tests
+  cfg1_octree.npz      expected points2octree blob of BASELINE config 1
+                       (3000 points on the unit sphere, depth 5, full_depth 2)
+  config_hashes.json   SHA-256 of the expected blobs of BASELINE configs 1-4 at full size
+                       (inputs are regenerated from the seeded generators; the hash of
+                       the input blob is stored too, to detect generator drift)
+"""
+import hashlib
+import importlib
+import json
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+
+from oracle.checker import Checker, make_points_blob  # noqa: E402
+
+synthetic = importlib.import_module("o-cnn_amd.synthetic")
+
+
+def sha(a):
+  return hashlib.sha256(np.ascontiguousarray(a).tobytes()).hexdigest()
+
+
+def main():
+  ref = Checker("ref")
+  np.savez_compressed(os.path.join(HERE, "octree_samples.npz"),
+                      **{"octree_%d" % i: ref.octree_sample("octree_%d" % i) for i in range(1, 7)})
+
+  pts, nrm, _ = synthetic.sphere_cloud(3000, 0)
+  pb = make_points_blob(pts, nrm)
+  single = ref.points2octree(pb, 5, 2)
+  np.savez_compressed(os.path.join(HERE, "cfg1_octree.npz"), octree=single)
+
+  hashes = {"cfg1": {"input": sha(pb), "single": sha(single),
+                     "batch": sha(ref.octree_batch([single]))}}
+  # config 2: 32 shapes x 10000 points, depth 6
+  blobs = [make_points_blob(*synthetic.shape_cloud(10000, 100 + i)[:2]) for i in range(32)]
+  singles = [ref.points2octree(b, 6, 2) for b in blobs]
+  hashes["cfg2"] = {"input": sha(np.concatenate(blobs)), "batch": sha(ref.octree_batch(singles)),
+                    "first_single": sha(singles[0])}
+  # config 3: 16 shapes x 50000 points, depth 7
+  blobs = [make_points_blob(*synthetic.shape_cloud(50000, 200 + i)[:2]) for i in range(16)]
+  singles = [ref.points2octree(b, 7, 2) for b in blobs]
+  hashes["cfg3"] = {"input": sha(np.concatenate(blobs)), "batch": sha(ref.octree_batch(singles)),
+                    "first_single": sha(singles[0])}
+  # config 4: room, 250000 points with RGB features, depth 9
+  p, n, f = synthetic.room_cloud(250000, 3)
+  pb = make_points_blob(p, n, f)
+  single = ref.points2octree(pb, 9, 2)
+  hashes["cfg4"] = {"input": sha(pb), "single": sha(single), "batch": sha(ref.octree_batch([single]))}
+  with open(os.path.join(HERE, "config_hashes.json"), "w") as fh:
+    json.dump(hashes, fh, indent=1, sort_keys=True)
+  print(json.dumps(hashes, indent=1))
+
+
+if __name__ == "__main__":
+  main()

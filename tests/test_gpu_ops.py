@@ -1,0 +1,316 @@
+"""GPU parity of the feature operators: octree2col / col2octree, conv / deconv (fp32 within
+1e-4 relative, bf16 within 2e-2 relative of the CPU oracle), pooling and padding (bit exact)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle.checker import OctreeBlob, make_points_blob
+
+pytestmark = pytest.mark.gpu
+
+TOL_F32 = 1e-4   # relative to the largest magnitude of the expected tensor
+TOL_BF16 = 2e-2
+
+KERNELS = [[3, 3, 3], [2, 2, 2], [3, 1, 1], [1, 3, 1], [1, 1, 3], [3, 3, 1], [3, 1, 3], [1, 3, 3], [1, 1, 1]]
+
+
+def T(a):
+  return torch.from_numpy(np.ascontiguousarray(a))
+
+
+def relerr(got, exp):
+  return float(np.abs(got.astype(np.float64) - exp).max() / (np.abs(exp).max() + 1e-30))
+
+
+@pytest.fixture(scope="module")
+def tree(oc, orc, samples, synthetic):
+  """A batch of three built octrees (depth 6) plus the sample batch of the reference tests."""
+  pbs = [make_points_blob(*synthetic.shape_cloud(4000, 31 + i)[:2]) for i in range(3)]
+  host = orc.octree_batch([orc.points2octree(p, 6, 2) for p in pbs])
+  shost = orc.octree_batch([samples[n] for n in ("octree_1", "octree_2", "octree_2", "octree_1")])
+  return {"host": host, "dev": T(host).cuda(), "blob": OctreeBlob(host),
+          "shost": shost, "sdev": T(shost).cuda(), "sblob": OctreeBlob(shost)}
+
+
+def closed_form_col(data, idx_map, stride):
+  K, C = len(idx_map), data.shape[0]
+  top_h = 8 if stride == 1 else 1
+  out = np.zeros((C, K, top_h), np.float32)
+  for c in range(C):
+    for k in range(K):
+      for h in range(top_h):
+        z, y, x = h & 1, (h & 2) >> 1, h >> 2
+        t = idx_map[k]
+        z, y, x = z + t % 3 - 1, y + (t // 3) % 3 - 1, x + t // 9 - 1
+        if -1 < x < 2 and -1 < y < 2 and -1 < z < 2:
+          out[c, k, h] = data[c, x * 4 + y * 2 + z]
+  return out
+
+
+def test_octree2col_closed_form(oc, samples):
+  """pytorch/test/test_octree2col.py:23-67 incl. the nempty variant on the all-non-empty depth 1."""
+  maps = {(3, 3, 3): list(range(27)), (2, 2, 2): [13, 14, 16, 17, 22, 23, 25, 26], (3, 1, 1): [4, 13, 22],
+          (3, 3, 1): [1, 4, 7, 10, 13, 16, 19, 22, 25], (1, 1, 1): [13]}
+  octree = oc.nn.octree_batch([T(samples["octree_1"])])
+  data = np.random.default_rng(0).uniform(-1, 1, (1, 3, 8, 1)).astype(np.float32)
+  for stride in (1, 2):
+    for ks, m in maps.items():
+      exp = closed_form_col(data.reshape(3, 8), m, stride)
+      for nempty in (False, True):
+        got = oc.nn.octree2col(T(data).cuda(), octree, 1, list(ks), stride, nempty)
+        assert np.array_equal(got.cpu().numpy(), exp), (ks, stride, nempty)
+
+
+@pytest.mark.parametrize("stride", [1, 2])
+def test_col_ops_vs_oracle(oc, orc, tree, stride):
+  b, dev = tree["blob"], tree["dev"]
+  d = 5
+  H, Hne = int(b.nnum[d]), int(b.nnum_nempty[d])
+  neigh, child = b.prop("neigh", d).reshape(-1), b.prop("child", d)
+  ichild = np.zeros(Hne, np.int32)
+  ichild[child[child >= 0]] = np.nonzero(child >= 0)[0]
+  rng = np.random.default_rng(1)
+  x = rng.standard_normal((5, H)).astype(np.float32)
+  xn = rng.standard_normal((5, Hne)).astype(np.float32)
+  for ks in KERNELS:
+    h = H if stride == 1 else H // 8
+    col = oc.nn.octree2col(T(x).cuda().view(1, 5, H, 1), dev, d, ks, stride, False)
+    exp = orc.octree2col(x, ks, stride, neigh, h)
+    assert np.array_equal(col.cpu().numpy(), exp), ks
+    colb = oc.nn.octree2col(T(x).cuda().view(1, 5, H, 1).bfloat16(), dev, d, ks, stride, False)
+    assert torch.equal(colb, T(exp).cuda().bfloat16())
+    back = oc.nn.col2octree(col, dev, d, ks, stride, False)
+    assert relerr(back.cpu().numpy().reshape(5, H), orc.col2octree(exp, ks, stride, neigh, h)) < TOL_F32
+    hp = Hne if stride == 1 else H // 8
+    colp = oc.nn.octree2col(T(xn).cuda().view(1, 5, Hne, 1), dev, d, ks, stride, True)
+    expp = orc.octree2colP(xn, ks, stride, neigh, child, ichild, hp)
+    assert np.array_equal(colp.cpu().numpy(), expp), ks
+    backp = oc.nn.col2octree(colp, dev, d, ks, stride, True)
+    assert relerr(backp.cpu().numpy().reshape(5, Hne),
+                  orc.col2octreeP(expp, ks, stride, neigh, child, ichild, hp, Hne)) < TOL_F32
+
+
+CONV_CASES = [(ks, s, ne) for ks in KERNELS for s in (1, 2) for ne in (False, True)]
+
+
+@pytest.mark.parametrize("ks,stride,nempty", CONV_CASES)
+def test_conv_vs_oracle(oc, orc, tree, ks, stride, nempty):
+  b, dev, host = tree["blob"], tree["dev"], tree["host"]
+  d = 5
+  K = ks[0] * ks[1] * ks[2]
+  rng = np.random.default_rng(2)
+  for ci, co in ((3, 32), (20, 70)):
+    hin = int(b.nnum_nempty[d] if nempty else b.nnum[d])
+    x = rng.standard_normal((ci, hin)).astype(np.float32)
+    w = (rng.standard_normal((co, ci * K)) * 0.1).astype(np.float32)
+    exp = orc.octree_conv(x, w, host, d, co, ks, stride, nempty)
+    xt, wt = T(x).cuda().view(1, ci, hin, 1), T(w).cuda()
+    got = oc.nn.octree_conv(xt, wt, dev, d, co, ks, stride, nempty)
+    assert tuple(got.shape) == (1, co, exp.shape[1], 1)
+    assert relerr(got.cpu().numpy().reshape(exp.shape), exp) < TOL_F32
+    got16 = oc.nn.octree_conv(xt.bfloat16(), wt.bfloat16(), dev, d, co, ks, stride, nempty)
+    assert got16.dtype == torch.bfloat16
+    assert relerr(got16.float().cpu().numpy().reshape(exp.shape), exp) < TOL_BF16
+
+
+DECONV_CASES = [(ks, 1, ne) for ks in KERNELS for ne in (False, True)] + [([2, 2, 2], 2, False), ([2, 2, 2], 2, True)]
+
+
+@pytest.mark.parametrize("ks,stride,nempty", DECONV_CASES)
+def test_deconv_vs_oracle(oc, orc, tree, ks, stride, nempty):
+  b, dev, host = tree["blob"], tree["dev"], tree["host"]
+  d = 5 if stride == 1 else 4
+  K = ks[0] * ks[1] * ks[2]
+  rng = np.random.default_rng(3)
+  for ci, co in ((8, 5), (33, 40)):
+    hin = int(b.nnum_nempty[d] if (nempty or stride == 2) else b.nnum[d])
+    x = rng.standard_normal((ci, hin)).astype(np.float32)
+    w = (rng.standard_normal((ci, co * K)) * 0.1).astype(np.float32)
+    exp = orc.octree_deconv(x, w, host, d, co, ks, stride, nempty)
+    xt, wt = T(x).cuda().view(1, ci, hin, 1), T(w).cuda()
+    got = oc.nn.octree_deconv(xt, wt, dev, d, co, ks, stride, nempty)
+    assert relerr(got.cpu().numpy().reshape(exp.shape), exp) < TOL_F32
+    got16 = oc.nn.octree_deconv(xt.bfloat16(), wt.bfloat16(), dev, d, co, ks, stride, nempty)
+    assert relerr(got16.float().cpu().numpy().reshape(exp.shape), exp) < TOL_BF16
+
+
+def test_conv_wide_channels(oc, orc, tree):
+  """Channel counts of the benchmark stacks, incl. more than one pass over the output tiles."""
+  b, dev, host = tree["blob"], tree["dev"], tree["host"]
+  rng = np.random.default_rng(4)
+  for d, ci, co in ((4, 64, 64), (4, 128, 256), (3, 256, 32), (4, 64, 100), (4, 1, 1)):
+    H = int(b.nnum[d])
+    x = rng.standard_normal((ci, H)).astype(np.float32)
+    w = (rng.standard_normal((co, ci * 27)) * 0.02).astype(np.float32)
+    exp = orc.octree_conv(x, w, host, d, co, [3, 3, 3], 1)
+    got = oc.nn.octree_conv(T(x).cuda().view(1, ci, H, 1), T(w).cuda(), dev, d, co, [3, 3, 3], 1, False)
+    assert relerr(got.cpu().numpy().reshape(exp.shape), exp) < TOL_F32, (d, ci, co)
+    got16 = oc.nn.octree_conv(T(x).cuda().view(1, ci, H, 1).bfloat16(), T(w).cuda().bfloat16(), dev, d, co,
+                              [3, 3, 3], 1, False)
+    assert relerr(got16.float().cpu().numpy().reshape(exp.shape), exp) < TOL_BF16, (d, ci, co)
+
+
+def test_conv_on_reference_sample_batch(oc, orc, tree):
+  """The shapes of pytorch/test/test_octree_conv.py: depth 4, 3 -> 5 channels."""
+  sb, sdev, shost = tree["sblob"], tree["sdev"], tree["shost"]
+  rng = np.random.default_rng(5)
+  d = 4
+  H = int(sb.nnum[d])
+  x = rng.uniform(-1, 1, (3, H)).astype(np.float32)
+  for ks in ([3, 3, 3], [2, 2, 2], [3, 1, 1], [3, 3, 1], [1, 1, 1]):
+    for stride in (1, 2):
+      K = ks[0] * ks[1] * ks[2]
+      w = rng.uniform(-0.5, 0.5, (5, 3 * K)).astype(np.float32)
+      conv = oc.OctreeConv(d, 3, 5, ks, stride).cuda()
+      fast = oc.OctreeConvFast(d, 3, 5, ks, stride).cuda()
+      with torch.no_grad():
+        conv.weights.copy_(T(w))
+        fast.weights.copy_(T(w))
+      xt = T(x).cuda().view(1, 3, H, 1)
+      y1, y2 = conv(xt, sdev), fast(xt, sdev)
+      assert y1.shape == y2.shape
+      assert torch.allclose(y1, y2, atol=1e-5)
+      exp = orc.octree_conv(x, w, shost, d, 5, ks, stride)
+      if stride == 2:
+        exp = orc.pad(exp, sb.prop("child", d - 1))
+      assert relerr(y1.cpu().numpy().reshape(exp.shape), exp) < TOL_F32
+      # nempty identity of the reference test: mask -> conv -> select
+      mask3 = T(sb.prop("child", d) >= 0).cuda()
+      d_out = d if stride == 1 else d - 1
+      mask4 = T(sb.prop("child", d_out) >= 0).cuda()
+      conv_ne = oc.OctreeConv(d, 3, 5, ks, stride, True).cuda()
+      with torch.no_grad():
+        conv_ne.weights.copy_(T(w))
+      y3 = conv_ne(xt[:, :, mask3], sdev)
+      y4 = conv(xt * mask3.view(1, 1, -1, 1).float(), sdev)[:, :, mask4]
+      assert torch.allclose(y3, y4, atol=1e-5)
+
+
+def test_deconv_layers(oc, orc, tree):
+  sb, sdev, shost = tree["sblob"], tree["sdev"], tree["shost"]
+  rng = np.random.default_rng(6)
+  for ks, stride in (([3, 3, 3], 1), ([2, 2, 2], 2), ([3, 1, 1], 1)):
+    d = 4 if stride == 1 else 3
+    H = int(sb.nnum[d])
+    K = ks[0] * ks[1] * ks[2]
+    x = rng.uniform(-1, 1, (3, H)).astype(np.float32)
+    w = rng.uniform(-0.5, 0.5, (3, 5 * K)).astype(np.float32)
+    dec = oc.OctreeDeconv(d, 3, 5, ks, stride).cuda()
+    fast = oc.OctreeDeconvFast(d, 3, 5, ks, stride).cuda()
+    with torch.no_grad():
+      dec.weights.copy_(T(w))
+      fast.weights.copy_(T(w))
+    xt = T(x).cuda().view(1, 3, H, 1)
+    y1, y2 = dec(xt, sdev), fast(xt, sdev)
+    assert y1.shape == y2.shape and torch.allclose(y1, y2, atol=1e-5)
+
+
+def test_conv_shape_errors(oc, tree):
+  dev, b = tree["dev"], tree["blob"]
+  x = torch.zeros(1, 4, int(b.nnum[5]) + 1, 1, device="cuda")
+  w = torch.zeros(8, 4 * 27, device="cuda")
+  with pytest.raises(oc.lib.OcnnError) as e:
+    oc.nn.octree_conv(x, w, dev, 5, 8, [3, 3, 3], 1, False)
+  assert e.value.code == -3
+  with pytest.raises(oc.lib.OcnnError) as e:
+    oc.nn.octree_conv(x, w, dev, 5, 8, [2, 3, 3], 1, False)
+  assert e.value.code == -2
+  with pytest.raises(oc.lib.OcnnError) as e:
+    oc.nn.octree_conv(x, w, dev, 9, 8, [3, 3, 3], 1, False)
+  assert e.value.code == -1
+  single = oc.nn.points2octree(T(make_points_blob([[0, 0, 0]], [[1, 0, 0]])), 5, 2)
+  with pytest.raises(oc.lib.OcnnError) as e:   # no neighbour table without octree_batch
+    oc.nn.octree_conv(torch.zeros(1, 4, 8, 1, device="cuda"), w, single, 5, 8, [3, 3, 3], 1, False)
+  assert e.value.code == -6
+
+
+def test_pool_literals(oc, samples):
+  """pytorch/test/test_octree_pool.py:10-101 (forward values and masks)."""
+  octree = oc.nn.octree_batch([T(samples["octree_1"])] * 2)
+  data = np.array([[1.1, 2.2, 3.3, 4.4, 5.5, 6.6, 7.7, 8.8], [8.1, 7.2, 6.3, 5.4, 4.5, 3.6, 2.7, 1.8]], np.float32)
+  data = np.concatenate([data, data], axis=1).reshape(1, 2, 16, 1)
+  out_gt = np.zeros((2, 16), np.float32)
+  out_gt[0, [0, 8]], out_gt[1, [0, 8]] = 8.8, 8.1
+  out, mask = oc.OctreeMaxPool(5, return_indices=True)(T(data).cuda(), octree)
+  assert np.array_equal(mask.cpu().numpy(), np.array([[[[7], [15]], [[0], [8]]]], np.int32))
+  assert np.array_equal(out.cpu().numpy().reshape(2, 16), out_gt)
+  # unpool: depth 4 -> 5 with a hand-written mask
+  m = T(np.array([[[[1], [9]], [[2], [10]]]], np.int32)).cuda()
+  un = oc.OctreeMaxUnpool(4)(T(data).cuda(), m, octree)
+  un_gt = np.zeros((2, 16), np.float32)
+  un_gt[0, [1, 9]], un_gt[1, [2, 10]] = 1.1, 8.1
+  assert np.array_equal(un.cpu().numpy().reshape(2, 16), un_gt)
+  avg_in = np.array([[8.0, 2.2, 3.3, 4.4, 5.5, 6.6, 7.6, 0.8], [12.0, 7.0, 6.0, 5.0, 4.0, 3.0, 3.0, 8.0]], np.float32)
+  avg_in = np.concatenate([avg_in, avg_in], axis=1).reshape(1, 2, 16, 1)
+  avg = oc.OctreeAvgPool(5)(T(avg_in).cuda(), octree).cpu().numpy().reshape(2, 16)
+  avg_gt = np.zeros((2, 16), np.float32)
+  avg_gt[0, [0, 8]], avg_gt[1, [0, 8]] = 4.8, 6.0
+  assert np.allclose(avg, avg_gt)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_pool_pad_vs_oracle(oc, orc, tree, dtype):
+  b, dev = tree["blob"], tree["dev"]
+  d = 6
+  H = int(b.nnum[d])
+  rng = np.random.default_rng(7)
+  x = rng.integers(-4, 4, (9, H)).astype(np.float32) / 2   # many ties, exactly representable in bf16
+  xt = T(x).cuda().view(1, 9, H, 1).to(dtype)
+  top, mask = oc.nn.octree_max_pool(xt, dev, d)
+  et, em = orc.max_pool(x)
+  assert np.array_equal(top.float().cpu().numpy().reshape(et.shape), et)
+  assert np.array_equal(mask.cpu().numpy().reshape(em.shape), em)
+  un = oc.nn.octree_max_unpool(top, mask, dev, d)
+  assert np.array_equal(un.float().cpu().numpy().reshape(9, H), orc.max_unpool(et, em))
+  mp = oc.nn.octree_mask_pool(xt, mask, dev, d)
+  assert np.array_equal(mp.float().cpu().numpy().reshape(et.shape), orc.mask_pool(x, em))
+  # a mask that points outside its own sibling group (never produced by max_pool)
+  foreign = em.copy()
+  foreign[:, ::5] = (foreign[:, ::5] + 8 * 3) % H
+  un2 = oc.nn.octree_max_unpool(top, T(foreign).cuda().view(1, 9, -1, 1), dev, d)
+  got, exp = un2.float().cpu().numpy().reshape(9, H), orc.max_unpool(et, foreign)
+  clash = np.zeros((9, H), bool)   # positions hit twice have no defined winner in the reference either
+  for c in range(9):
+    idx, cnt = np.unique(foreign[c], return_counts=True)
+    clash[c, idx[cnt > 1]] = True
+  assert np.array_equal(got[~clash], exp[~clash])
+  child = b.prop("child", d - 1)
+  pd = oc.nn.octree_pad(top, dev, d - 1, 1.5)
+  assert np.array_equal(pd.float().cpu().numpy().reshape(9, -1), orc.pad(et, child, 1.5))
+  dp = oc.nn.octree_depad(pd, dev, d - 1)
+  assert np.array_equal(dp.float().cpu().numpy().reshape(et.shape), et)
+  with pytest.raises(oc.lib.OcnnError) as e:
+    oc.nn.octree_pad(xt, dev, d - 1)
+  assert e.value.code == -3
+
+
+def test_full_size_properties(oc, synthetic):
+  """Size-independent properties on the depth-9 scene of BASELINE config 4: linearity of
+  the convolution, unpool/mask-pool round trip, depad(pad(x)) == x."""
+  p, n, f = synthetic.room_cloud(250000, 3)
+  octree = oc.nn.points2octree_batch([T(make_points_blob(p, n, f)).cuda()], 9, 2)
+  info = oc.nn.octree_info(octree)
+  H = info.nnum(9)
+  g = torch.Generator().manual_seed(0)
+  C = 64
+  x = torch.randn(1, C, H, 1, generator=g).cuda()
+  y = torch.randn(1, C, H, 1, generator=g).cuda()
+  w = (torch.randn(C, C * 27, generator=g) * 0.02).cuda()
+  conv = lambda t: oc.nn.octree_conv(t, w, octree, 9, C, [3, 3, 3], 1, False)
+  lhs = conv(2.0 * x - 3.0 * y)
+  rhs = 2.0 * conv(x) - 3.0 * conv(y)
+  assert float((lhs - rhs).abs().max() / rhs.abs().max()) < 1e-4
+  top, mask = oc.nn.octree_max_pool(x, octree, 9)
+  un = oc.nn.octree_max_unpool(top, mask, octree, 9)
+  assert torch.equal(oc.nn.octree_mask_pool(un, mask, octree, 9), top)
+  assert int((un != 0).sum()) <= top.numel()
+  assert torch.equal(un.view(C, -1, 8).amax(2), torch.clamp(top.view(C, -1), min=0) * (top.view(C, -1) > 0)
+                     + torch.clamp(top.view(C, -1), max=0) * 0)
+  pd = oc.nn.octree_pad(top, octree, 8)
+  assert torch.equal(oc.nn.octree_depad(pd, octree, 8), top)
+  # stride-2 conv then deconv keep the documented heights
+  w2 = (torch.randn(C, C * 8, generator=g) * 0.02).cuda()
+  down = oc.nn.octree_conv(x, w2, octree, 9, C, [2, 2, 2], 2, False)
+  assert down.shape[2] == info.nnum_nempty(8)
+  up = oc.nn.octree_deconv(down, w2, octree, 8, C, [2, 2, 2], 2, False)
+  assert up.shape[2] == H

@@ -1,0 +1,273 @@
+"""GPU parity: octree construction, batching, neighbour tables, keys, growth.
+Everything integer/byte valued is compared bit for bit with the CPU oracle."""
+import hashlib
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import GOLDEN, sha
+from oracle.checker import OctreeBlob, make_points_blob
+
+pytestmark = pytest.mark.gpu
+
+
+def T(a):
+  return torch.from_numpy(np.ascontiguousarray(a))
+
+
+def three_point_cloud():
+  return make_points_blob([0, 0, 0, 1, 1, 0, 1.0625, 1.0625, 0], [1, 0, 0, -1, 0, 0, 0, 1, 0],
+                          [1, -1, 2, -2, 3, -3], [0, 2, 2])
+
+
+def test_build_known_answer_on_gpu(oc, orc):
+  """The known-answer cloud of octree/test/test_octree.cpp:92-190 (custom bounding box,
+  normals + features + labels, displacement, split labels)."""
+  pb = three_point_cloud()
+  got = oc.nn._build([T(pb)], False, 5, 1, True, False, True, False, 4, 0.1, 2.0, False, False, False,
+                     bbox=([0, 0, 0], [2, 2, 2]))
+  exp = orc.points2octree(pb, 5, 1, node_dis=True, split_label=True, bbmin=[0, 0, 0], bbmax=[2, 2, 2])
+  assert np.array_equal(got.cpu().numpy(), exp)
+  b = OctreeBlob(got.cpu().numpy())
+  assert list(b.nnum_nempty[:6]) == [1, 2, 2, 2, 2, 3]
+  assert np.array_equal(b.prop("label", 5)[[0, 8, 14]], [0, 2, 2])
+
+
+def test_build_golden_config1(oc, synthetic, hashes):
+  pts, nrm, _ = synthetic.sphere_cloud(3000, 0)
+  pb = make_points_blob(pts, nrm)
+  assert sha(pb) == hashes["cfg1"]["input"]
+  z = np.load(GOLDEN + "/cfg1_octree.npz")
+  single = oc.nn.points2octree(T(pb), 5, 2)
+  assert np.array_equal(single.cpu().numpy(), z["octree"])
+  assert sha(oc.nn.points2octree_batch([T(pb)], 5, 2).cpu().numpy()) == hashes["cfg1"]["batch"]
+  assert sha(oc.nn.octree_batch([single]).cpu().numpy()) == hashes["cfg1"]["batch"]
+
+
+FLAG_CASES = [dict(), dict(node_dis=True), dict(split_label=True), dict(save_pts=True), dict(key2xyz=True),
+              dict(node_dis=True, split_label=True, save_pts=True, key2xyz=True)]
+
+
+@pytest.mark.parametrize("case", range(len(FLAG_CASES)))
+def test_build_random_vs_oracle(oc, orc, case):
+  kw = FLAG_CASES[case]
+  rng = np.random.default_rng(100 + case)
+  for trial in range(5):
+    n = int(rng.integers(1, 5000))
+    pts = rng.uniform(-0.999, 0.999, (n, 3)).astype(np.float32)
+    nrm = rng.standard_normal((n, 3)).astype(np.float32) if trial != 1 else None
+    feat = rng.uniform(0, 1, (n, 1 + trial % 3)).astype(np.float32) if trial >= 1 else None
+    lab = rng.integers(-1, 6, n).astype(np.float32) if trial in (2, 4) else None
+    pb = make_points_blob(pts, nrm, feat, lab)
+    depth = int(rng.integers(2, 10))
+    fd = int(rng.integers(1, min(depth, 3) + 1))
+    got = oc.nn.points2octree(T(pb), depth, fd, **kw).cpu().numpy()
+    assert np.array_equal(got, orc.points2octree(pb, depth, fd, **kw)), (trial, n, depth, fd, kw)
+
+
+def test_build_edge_cases(oc, orc):
+  rng = np.random.default_rng(7)
+  one = make_points_blob([[0.3, -0.2, 0.7]], [[0, 0, 1]])
+  same_voxel = make_points_blob(np.full((500, 3), 0.123, np.float32) + rng.uniform(0, 1e-4, (500, 3)).astype(np.float32),
+                                rng.standard_normal((500, 3)).astype(np.float32))
+  cancelling = make_points_blob([[0.5, 0.5, 0.5], [0.5, 0.5, 0.5]], [[1, 0, 0], [-1, 0, 0]])  # |sum of normals| < 1e-6
+  corner = make_points_blob([[-1, -1, -1], [0.9999, 0.9999, 0.9999], [0, 0, 0]], [[1, 0, 0]] * 3)
+  for pb in (one, same_voxel, cancelling, corner):
+    for depth, fd in ((5, 2), (3, 3), (9, 1), (1, 1), (2, 1)):
+      got = oc.nn.points2octree(T(pb), depth, fd, node_dis=True).cpu().numpy()
+      assert np.array_equal(got, orc.points2octree(pb, depth, fd, node_dis=True)), (depth, fd)
+
+
+def test_build_rejects_what_it_cannot_do(oc):
+  pb = make_points_blob([[0, 0, 0]], [[1, 0, 0]])
+  with pytest.raises(oc.lib.OcnnError) as e:
+    oc.nn.points2octree(T(pb), 5, 2, adaptive=True)
+  assert e.value.code == -2
+  bad = pb.copy()
+  bad[0] = 0
+  with pytest.raises(oc.lib.OcnnError) as e:
+    oc.nn.points2octree(T(bad), 5, 2)
+  assert e.value.code == -6
+
+
+@pytest.mark.parametrize("cfg,n_clouds,n_pts,depth,seed0", [("cfg2", 32, 10000, 6, 100), ("cfg3", 16, 50000, 7, 200)])
+def test_full_size_batches_hash(oc, synthetic, hashes, cfg, n_clouds, n_pts, depth, seed0):
+  """BASELINE configs 2 and 3 at full size: the fused build+batch blob and the blob of
+  batching separately built octrees both hash to what the compiled reference produced."""
+  blobs = [make_points_blob(*synthetic.shape_cloud(n_pts, seed0 + i)[:2]) for i in range(n_clouds)]
+  assert sha(np.concatenate(blobs)) == hashes[cfg]["input"]
+  clouds = [T(b).cuda() for b in blobs]
+  fused = oc.nn.points2octree_batch(clouds, depth, 2)
+  assert sha(fused.cpu().numpy()) == hashes[cfg]["batch"]
+  singles = [oc.nn.points2octree(c, depth, 2) for c in clouds]
+  assert sha(singles[0].cpu().numpy()) == hashes[cfg]["first_single"]
+  assert sha(oc.nn.octree_batch(singles).cpu().numpy()) == hashes[cfg]["batch"]
+
+
+def test_full_size_scene_hash(oc, synthetic, hashes):
+  p, n, f = synthetic.room_cloud(250000, 3)
+  pb = make_points_blob(p, n, f)
+  assert sha(pb) == hashes["cfg4"]["input"]
+  cloud = T(pb).cuda()
+  assert sha(oc.nn.points2octree(cloud, 9, 2).cpu().numpy()) == hashes["cfg4"]["single"]
+  merged = oc.nn.points2octree_batch([cloud], 9, 2)
+  assert sha(merged.cpu().numpy()) == hashes["cfg4"]["batch"]
+  # size-independent invariants of the structure at full size
+  b = OctreeBlob(merged.cpu().numpy())
+  for d in range(3, 10):
+    assert b.nnum[d] == 8 * b.nnum_nempty[d - 1]
+    k = b.prop("key", d).astype(np.int64)
+    assert np.all(np.diff(k) > 0)
+    c = b.prop("child", d)
+    assert np.array_equal(c[c >= 0], np.arange(b.nnum_nempty[d]))
+
+
+def test_octree_batch_samples(oc, orc, samples):
+  for names in (["octree_1"] * 2, ["octree_1", "octree_2"], ["octree_2", "octree_2", "octree_1"],
+                ["octree_1", "octree_2", "octree_2", "octree_1"], ["octree_3", "octree_4"],
+                ["octree_5", "octree_5"], ["octree_6"] * 3):
+    got = oc.nn.octree_batch([T(samples[n]) for n in names]).cpu().numpy()
+    assert np.array_equal(got, orc.octree_batch([samples[n] for n in names])), names
+  with pytest.raises(oc.lib.OcnnError) as e:
+    oc.nn.octree_batch([T(samples["octree_1"]), T(samples["octree_3"])])
+  assert e.value.code == -6 and "not consistent" in str(e.value)
+
+
+def test_property_literals(oc, samples):
+  """pytorch/test/test_octree_property.py:9-54."""
+  octree = oc.nn.octree_batch([T(samples["octree_1"])] * 2)
+  P = oc.nn.octree_property
+  assert np.array_equal(P(octree, "index", 5).cpu().numpy(), [0] * 8 + [1] * 8)
+  f = np.zeros((3, 16), np.float32)
+  f[:, 0] = f[:, 8] = 3.0 ** 0.5 / 3.0
+  assert np.allclose(P(octree, "feature", 5).cpu().numpy(), f[None, :, :, None])
+  c = -np.ones(16)
+  c[0], c[8] = 0, 1
+  assert np.array_equal(P(octree, "child", 5).cpu().numpy(), c)
+  parts = torch.cat([P(octree, "child", d) for d in range(1, 6)])
+  assert np.array_equal(P(octree, "child").cpu().numpy()[2:], parts.cpu().numpy())
+  assert P(octree, "node_num", 5).item() == 16 and P(octree, "node_num_cum", 5).item() == 178
+  assert np.array_equal(P(octree, "node_num").cpu().numpy(), [2, 16, 128, 16, 16, 16])
+  assert np.array_equal(P(octree, "node_num_cum").cpu().numpy(), [0, 2, 18, 146, 162, 178, 194])
+  assert (P(octree, "batch_size").item(), P(octree, "depth").item(), P(octree, "full_depth").item()) == (2, 5, 2)
+  assert tuple(P(octree, "neigh", 5).shape) == (16, 8)
+  with pytest.raises(oc.lib.OcnnError):
+    P(octree, "nonsense")
+
+
+def test_neighbour_kernels(oc, orc, samples, synthetic):
+  import ctypes as C
+  st = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)
+  for depth, batch in ((1, 1), (2, 3), (3, 2), (5, 2)):
+    out = torch.empty(batch * 8 ** depth * 8, dtype=torch.int32, device="cuda")
+    oc.lib.call("ocnn_calc_neigh_full", C.c_void_p(out.data_ptr()), depth, batch, st())
+    assert np.array_equal(out.cpu().numpy(), orc.calc_neigh_full(depth, batch))
+  pbs = [make_points_blob(*synthetic.shape_cloud(3000, 11 + i)[:2]) for i in range(3)]
+  b = OctreeBlob(orc.octree_batch([orc.points2octree(p, 7, 2) for p in pbs]))
+  for d in range(3, 8):
+    neigh, child = b.prop("neigh", d - 1).reshape(-1), b.prop("child", d - 1)
+    out = torch.full((int(b.nnum[d]) * 8,), -7, dtype=torch.int32, device="cuda")
+    neigh_d, child_d = T(neigh).cuda(), T(child).cuda()
+    oc.lib.call("ocnn_calc_neigh_sparse", C.c_void_p(out.data_ptr()), C.c_void_p(neigh_d.data_ptr()),
+                C.c_void_p(child_d.data_ptr()), child.size, st())
+    assert np.array_equal(out.cpu().numpy(), b.prop("neigh", d).reshape(-1)), d
+
+
+def pack(x, y, z, i):
+  return (x | (y << 16) | (z << 32) | (i << 48))
+
+
+def test_key_ops(oc, orc, samples):
+  """pytorch/test/test_octree_key.py."""
+  F = oc.nn
+  octree = F.octree_batch([T(samples["octree_1"])] * 2)
+  xyz = F.octree_property(octree, "xyz", 5)
+  pts = F.octree_decode_key(xyz)
+  gt = [[16, 16, 16], [16, 16, 17], [16, 17, 16], [16, 17, 17], [17, 16, 16], [17, 16, 17], [17, 17, 16], [17, 17, 17]]
+  exp = np.array([g + [i] for i in (0, 1) for g in gt], np.int16)
+  assert np.array_equal(pts.cpu().numpy(), exp)
+  assert torch.equal(F.octree_encode_key(pts), xyz)
+  key = F.octree_xyz2key(xyz, 5)
+  assert torch.equal(F.octree_key2xyz(key, 5), xyz)
+  assert torch.equal(F.octree_property(octree, "key", 5), key)
+  q = torch.tensor([28673, 281474976739335, 10], dtype=torch.int64, device="cuda")
+  assert F.octree_search_key(q, octree, 5, False, False).cpu().tolist() == [1, 15, -1]
+  q = torch.tensor([28672, 28673, 281474976739328, 10], dtype=torch.int64, device="cuda")
+  assert F.octree_search_key(q, octree, 5, False, True).cpu().tolist() == [0, -1, 1, -1]
+  assert F.octree_search_key(xyz[[3, 12]], octree, 5, True, False).cpu().tolist() == [3, 12]
+  x64 = torch.tensor([[2049, 4095, 8011, 1], [511, 4095, 8011, 0]], dtype=torch.int16, device="cuda")
+  enc = F.octree_encode_key(x64)
+  assert torch.equal(F.octree_decode_key(F.octree_key2xyz(F.octree_xyz2key(enc, 13), 13)), x64)
+  rng = np.random.default_rng(5)
+  for depth in (1, 4, 9, 16):
+    v = rng.integers(0, 1 << 62, 4000).astype(np.uint64)
+    vt = T(v.view(np.int64)).cuda()
+    assert np.array_equal(F.octree_xyz2key(vt, depth).cpu().numpy().view(np.uint64), orc.xyz2key(v, depth))
+    assert np.array_equal(F.octree_key2xyz(vt, depth).cpu().numpy().view(np.uint64), orc.key2xyz(v, depth))
+
+
+def test_generate_key_label_search(oc, orc):
+  import ctypes as C
+  st = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)
+  P = lambda t: C.c_void_p(t.data_ptr())
+  for depth, batch in ((1, 2), (3, 3)):
+    out = torch.empty(batch * 8 ** depth, dtype=torch.int64, device="cuda")
+    oc.lib.call("ocnn_generate_key_full", P(out), depth, batch, st())
+    assert np.array_equal(out.cpu().numpy().view(np.uint64), orc.generate_key_full(depth, batch))
+  rng = np.random.default_rng(6)
+  key = orc.generate_key_full(3, 2)
+  child = np.full(key.size, -1, np.int32)
+  sel = np.sort(rng.choice(key.size, 300, replace=False))
+  child[sel] = np.arange(300)
+  out = torch.zeros(2400, dtype=torch.int64, device="cuda")
+  key_d, child_d = T(key.view(np.int64)).cuda(), T(child).cuda()
+  oc.lib.call("ocnn_generate_key_child", P(out), P(key_d), P(child_d), key.size, st())
+  assert np.array_equal(out.cpu().numpy().view(np.uint64), orc.generate_key_child(key, child, 2400))
+  for n in (1, 5, 1023, 1024, 1025, 300000):
+    btm = rng.integers(0, 3, n).astype(np.int32)
+    lab = torch.empty(n, dtype=torch.int32, device="cuda")
+    cnt = torch.zeros(1, dtype=torch.int32, device="cuda")
+    sb = oc.lib.get().ocnn_generate_label_scratch_bytes(n)
+    scratch = torch.empty(sb, dtype=torch.uint8, device="cuda")
+    btm_d = T(btm).cuda()
+    oc.lib.call("ocnn_generate_label", P(lab), P(cnt), P(btm_d), n, 1, P(scratch), C.c_size_t(sb), st())
+    exp, total = orc.generate_label(btm, 1)
+    assert np.array_equal(lab.cpu().numpy(), exp) and cnt.item() == total
+  keys = np.unique(rng.integers(0, 1 << 50, 100000).astype(np.uint64))
+  q = np.concatenate([keys[::13], rng.integers(0, 1 << 50, 5000).astype(np.uint64)])
+  idx = torch.empty(q.size, dtype=torch.int32, device="cuda")
+  keys_d, q_d = T(keys.view(np.int64)).cuda(), T(q.view(np.int64)).cuda()
+  oc.lib.call("ocnn_search_key", P(idx), P(keys_d), keys.size, P(q_d), q.size, st())
+  assert np.array_equal(idx.cpu().numpy(), orc.search_key(keys, q))
+
+
+def test_grow_md5_on_gpu(oc, samples):
+  """pytorch/test/test_octree_grow.py: rebuild octree_2 with new/grow/update/set_property."""
+  F = oc.nn
+  gt = T(samples["octree_2"]).cuda()
+  depth, channel = 5, 3
+  o = F.octree_new(1, channel, False)
+  o = F.octree_grow(o, 1, True)
+  o = F.octree_grow(o, 2, True)
+  for d in range(2, depth + 1):
+    label = (F.octree_property(gt, "child", d) > -1).to(torch.int32)
+    o = F.octree_update(o, label, d, 1)
+    if d < depth:
+      o = F.octree_grow(o, d + 1, False)
+  o = F.octree_set_property(o, F.octree_property(gt, "feature", depth), depth)
+  assert hashlib.md5(o.cpu().numpy().tobytes()).hexdigest().upper() == "D569D5BB23D34795C5FD81397F56275B"
+
+
+def test_update_degenerate_and_errors(oc, orc):
+  F = oc.nn
+  o = F.octree_grow(F.octree_new(2, 1, False), 1, True)
+  u = F.octree_update(o, torch.zeros(16, dtype=torch.int32), 1, 1)
+  exp = orc.octree_update(orc.octree_grow(orc.octree_new(2, 1, False, 0), 1, True), np.zeros(16, np.int32), 1, 1)
+  assert np.array_equal(u.cpu().numpy(), exp)
+  assert F.octree_info(u).nnum_nempty(1) == 1
+  with pytest.raises(oc.lib.OcnnError) as e:
+    F.octree_update(o, torch.zeros(15, dtype=torch.int32), 1, 1)
+  assert e.value.code == -3
+  with pytest.raises(oc.lib.OcnnError):
+    F.octree_grow(o, 3, False)
