@@ -208,6 +208,147 @@ __global__ __launch_bounds__(kConvWaves * 64) void conv_bf16_kernel(ConvArgs a, 
   }
 }
 
+
+// ---- LDS-staged kernel for stride-1 convolutions over all nodes -----------------------
+// The eight siblings of a group read their taps from ONE 4x4x4 block of neighbour slots,
+// so the block is gathered once per group and channel (64 values) and then serves all
+// 8 x K (sibling, tap) pairs from LDS: 3.4x fewer global gathers than per-tap gathering
+// for the 27-tap kernel, and every operand of the MFMA loop comes out of LDS.
+//
+// Workgroup = 4 wavefronts = 256 columns = 32 sibling groups; wavefront w owns groups
+// 8w .. 8w+7 (its own 64 columns), stages only those, and computes all output channels of
+// a pass (MT row tiles).  The channel loop runs in slabs of kSlab = 4 input channels:
+//   LDS X [kSlab][32 groups][80]  fp32: the neighbour blocks (wavefront-private parts)
+//   LDS W [K][2][MT][64]          fp32: the slab's weights in A-fragment order (shared)
+// Group g sits at word 80*g + {0,2,8,10}[g&3]: with that skew the 32 lanes of a half
+// wavefront (4 groups x 8 siblings, sibling offsets {0,1,4,5,16,17,20,21}) hit 32
+// different banks for every tap.
+// The next slab's gathers and weights are issued before the MFMA loop of the current
+// slab and land in LDS after it, so their latency hides behind ~14k cycles of MFMA.
+constexpr int kSlab = 4;
+constexpr int kGroupStride = 80;
+constexpr int kPlane = 32 * kGroupStride;   // words per channel plane
+
+__device__ inline int group_base(int g) {
+  return g * kGroupStride + ((g & 1) << 1) + ((g & 2) << 2);
+}
+
+template <int MT, int K>
+__global__ __launch_bounds__(256, 2) void conv_s1_f32_lds_kernel(ConvArgs a, float* __restrict__ out,
+    const float* __restrict__ in, const float* __restrict__ Wt, int n_tiles) {
+  constexpr int kWWords = K * 2 * MT * 64;          // weight words per (pass, slab)
+  constexpr int kWVec = (kWWords / 4 + 255) / 256;  // float4 loads per thread
+  __shared__ float sX[kSlab * kPlane];
+  __shared__ __attribute__((aligned(16))) float sW[kWWords];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = xcd_tile(blockIdx.x, n_tiles);
+  if (tile >= n_tiles) return;
+  const int n0 = tile * kTileCols + wave * kWaveCols;
+  const int r = lane & 31, kh = lane >> 5;
+  const int nslab = (a.Cin + kSlab - 1) / kSlab;
+  const int npass = (a.mtiles + MT - 1) / MT;
+
+  // neighbour rows of slot `lane` of my eight groups (kept for all slabs and passes)
+  int nb[8];
+  const int group0 = (tile * kTileCols) / 8 + wave * 8;
+  const int n_groups = a.N >> 3;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    int g = group0 + j;
+    int v = g < n_groups ? a.neigh[((int64_t)g << 6) + lane] : -1;
+    nb[j] = (v >= 0 && v < a.Hin) ? v : -1;
+  }
+  // LDS word offsets of my two B columns (channel plane and tap slot are added per read)
+  int boff[2];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt)
+    boff[nt] = group_base(wave * 8 + nt * 4 + (r >> 3)) + sibling_slot(r & 7) + kh * kPlane;
+
+  for (int pass = 0; pass < npass; ++pass) {
+    floatx16 acc[MT][2];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
+
+    float xr[8][kSlab];
+    float4 wr[kWVec];
+    auto fetch = [&](int slab) {
+      const float4* wsrc = reinterpret_cast<const float4*>(Wt + ((int64_t)pass * nslab + slab) * kWWords);
+#pragma unroll
+      for (int v = 0; v < kWVec; ++v) {
+        int idx = v * 256 + threadIdx.x;
+        wr[v] = idx < kWWords / 4 ? wsrc[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int cc = 0; cc < kSlab; ++cc) {
+        const int c = slab * kSlab + cc;
+        if (c < a.Cin) {
+          const float* pc = in + (int64_t)c * a.Hin;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            float v = pc[(uint32_t)max(nb[j], 0)];
+            xr[j][cc] = nb[j] >= 0 ? v : 0.0f;
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) xr[j][cc] = 0.0f;
+        }
+      }
+    };
+    fetch(0);
+    for (int slab = 0; slab < nslab; ++slab) {
+      __syncthreads();  // everyone is done reading the previous slab
+#pragma unroll
+      for (int v = 0; v < kWVec; ++v) {
+        int idx = v * 256 + threadIdx.x;
+        if (idx < kWWords / 4) reinterpret_cast<float4*>(sW)[idx] = wr[v];
+      }
+#pragma unroll
+      for (int cc = 0; cc < kSlab; ++cc)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) sX[cc * kPlane + group_base(wave * 8 + j) + lane] = xr[j][cc];
+      __syncthreads();
+      if (slab + 1 < nslab) fetch(slab + 1);
+#pragma unroll 3
+      for (int k = 0; k < K; ++k) {
+        const int slot = a.slot[k];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          float b0 = sX[boff[0] + ks * 2 * kPlane + slot];
+          float b1 = sX[boff[1] + ks * 2 * kPlane + slot];
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            float av = sW[((k * 2 + ks) * MT + mt) * 64 + lane];
+            acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b0, acc[mt][0], 0, 0, 0);
+            acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b1, acc[mt][1], 0, 0, 0);
+          }
+        }
+      }
+    }
+    if (n0 < a.N) store_tiles<float, MT>(a, out, acc, pass * MT, n0, lane);
+  }
+}
+
+// weights in the order the LDS kernel copies them: [pass][slab][tap][kstep][mt][lane]
+__global__ void pack_weights_lds_f32(float* __restrict__ Wt, const float* __restrict__ W, int M, int Cin, int K,
+    int MT, int npass, int nslab, int64_t sm, int64_t sc) {
+  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t total = (int64_t)npass * nslab * K * 2 * MT * 64;
+  if (id >= total) return;
+  int l = (int)(id & 63);
+  int64_t f = id >> 6;
+  int mt = (int)(f % MT); f /= MT;
+  int ks = (int)(f % 2); f /= 2;
+  int k = (int)(f % K); f /= K;
+  int slab = (int)(f % nslab);
+  int pass = (int)(f / nslab);
+  int m = (pass * MT + mt) * 32 + (l & 31), c = slab * kSlab + 2 * ks + (l >> 5);
+  Wt[id] = (m < M && c < Cin) ? W[m * sm + c * sc + k] : 0.0f;
+}
+
 template <typename T>
 __global__ void zero_rows_kernel(T* p, int64_t n) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -279,6 +420,10 @@ int make_plan(const Info* o, int depth, int channel_in, int num_output, const in
   p->csteps = dtype == OCNN_F32 ? (channel_in + 1) / 2 : (channel_in + 15) / 16;
   size_t frag = dtype == OCNN_F32 ? 64 * sizeof(float) : 64 * 8 * sizeof(uint16_t);
   p->wt_bytes = align256((size_t)p->taps.count * p->csteps * p->mtiles * frag);
+  if (dtype == OCNN_F32) {  // the LDS kernel pads channels to slabs of 4 and row tiles to passes
+    size_t lds_words = (size_t)((p->mtiles + 1) / 2) * ((channel_in + kSlab - 1) / kSlab) * p->taps.count * 2 * 2 * 64;
+    p->wt_bytes = align256(lds_words * sizeof(float) > p->wt_bytes ? lds_words * sizeof(float) : p->wt_bytes);
+  }
   p->ichild_bytes = nempty ? align256(sizeof(int) * (size_t)(p->ichild_h + 1)) : 0;
   p->total_bytes = p->wt_bytes + p->ichild_bytes;
   return OCNN_OK;
@@ -343,7 +488,18 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
   int64_t sc = deconv ? (int64_t)num_output * a.K : a.K;
   int n_tiles = (a.N + kTileCols - 1) / kTileCols;
   int grid = ((n_tiles + 7) / 8) * 8;
-  if (dtype == OCNN_F32) {
+  if (dtype == OCNN_F32 && a.mode == kModeS1 && !a.nempty && a.K == 27) {
+    const int MT = a.mtiles == 1 ? 1 : 2;
+    const int npass = (a.mtiles + MT - 1) / MT, nslab = (a.Cin + kSlab - 1) / kSlab;
+    int64_t total = (int64_t)npass * nslab * a.K * 2 * MT * 64;
+    pack_weights_lds_f32<<<blocks_for(total), kBlock, 0, s>>>((float*)wsb, (const float*)weights, a.M, a.Cin, a.K,
+        MT, npass, nslab, sm, sc);
+    OCNN_LAUNCH_OK("pack_weights_lds");
+    if (MT == 1)
+      conv_s1_f32_lds_kernel<1, 27><<<grid, 256, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
+    else
+      conv_s1_f32_lds_kernel<2, 27><<<grid, 256, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
+  } else if (dtype == OCNN_F32) {
     int64_t total = (int64_t)a.K * a.csteps * a.mtiles * 64;
     pack_weights_f32<<<blocks_for(total), kBlock, 0, s>>>((float*)wsb, (const float*)weights, a.M, a.Cin, a.K,
         a.mtiles, a.csteps, sm, sc);
