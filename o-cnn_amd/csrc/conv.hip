@@ -349,6 +349,173 @@ __global__ void pack_weights_lds_f32(float* __restrict__ Wt, const float* __rest
   Wt[id] = (m < M && c < Cin) ? W[m * sm + c * sc + k] : 0.0f;
 }
 
+
+// ---- LDS-staged bf16 kernel (3x3x3, stride 1, all nodes) ----------------------------------
+// v_mfma_f32_32x32x16_bf16 wants 8 consecutive input channels of one column per lane, which
+// the channel-major [C, H] tensor cannot deliver without eight 2-byte gathers.  So the input
+// is first transposed to row-major [H + 1, Cpad] bf16 (row H is all zero and stands for a
+// missing neighbour, Cpad = Cin rounded up to 16): a neighbour is then one contiguous row
+// and every staged element moves as a 16-byte vector.
+//
+// Slab = 16 channels (one MFMA k-step per tap).  Per sibling group only two x-layers of the
+// 4x4x4 block are resident (taps with offset dx read layers dx and dx+1): layer x lives in
+// the units with bit0 == x&1 and layer x+2 overwrites layer x, so every slot is still
+// gathered exactly once per slab.  The weights of the 9 taps of one dx sit next to it.
+//   LDS X [2 halves of 8 channels][32 groups][32 units] x 16 B = 32 KiB
+//   LDS W [9 taps][MT][64 lanes] x 16 B                        = 18 KiB (MT = 2)
+// 50 KiB per workgroup: three workgroups per CU.  Unit index of slot (x,y,z):
+//   (x&1) | (y&1)<<1 | (z&1)<<2 | (y>>1)<<3 | (z>>1)<<4
+// so the 8 siblings of a group (consecutive lanes) always read 8 different 16-byte units.
+constexpr int kB16Half = 32 * 32;  // 16-byte units per 8-channel half
+
+__device__ inline int b16_unit(int x, int y, int z) {
+  return (x & 1) | ((y & 1) << 1) | ((z & 1) << 2) | ((y >> 1) << 3) | ((z >> 1) << 4);
+}
+
+template <typename T>
+__global__ void transpose_rows_kernel(T* __restrict__ dst, const T* __restrict__ src, int C, int H, int Cpad) {
+  // src [C, H] -> dst [H + 1, Cpad]; 64 x 64 tiles through LDS, both sides coalesced
+  __shared__ T tile[64][65];
+  const int h0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 256 threads: 4 rows per step
+  for (int i = ty; i < 64; i += 4) {
+    int c = c0 + i, h = h0 + tx;
+    tile[i][tx] = (c < C && h < H) ? src[(int64_t)c * H + h] : (T)0;
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    int h = h0 + i, c = c0 + tx;
+    if (h <= H && c < Cpad) dst[(int64_t)h * Cpad + c] = h < H ? tile[tx][i] : (T)0;
+  }
+}
+
+template <int MT>
+__global__ __launch_bounds__(256, 2) void conv_s1_bf16_lds_kernel(ConvArgs a, uint16_t* __restrict__ out,
+    const uint4* __restrict__ xt, const uint4* __restrict__ Wt, int n_tiles, int cpad8) {
+  constexpr int kWUnits = 9 * MT * 64;               // 16-byte units per weight chunk
+  constexpr int kWVec = (kWUnits + 255) / 256;
+  __shared__ uint4 sX[2 * kB16Half];
+  __shared__ uint4 sW[kWUnits];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = xcd_tile(blockIdx.x, n_tiles);
+  if (tile >= n_tiles) return;
+  const int n0 = tile * kTileCols + wave * kWaveCols;
+  const int r = lane & 31, kh = lane >> 5;
+  const int nslab = cpad8 >> 1;                       // 16-channel slabs
+  const int npass = (a.mtiles + MT - 1) / MT;
+
+  // staging role of this lane: half s_kh, (y,z) = s_yz, groups 8*wave + 2*j + s_g (j = 0..3)
+  const int s_kh = lane & 1, s_yz = (lane >> 1) & 15, s_g = lane >> 5;
+  const int s_y = s_yz >> 2, s_z = s_yz & 3;
+  int nb[4][4];  // [j][x-layer] neighbour row (H = the zero row)
+  const int group0 = (tile * kTileCols) / 8 + wave * 8;
+  const int n_groups = a.N >> 3;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    int g = group0 + 2 * j + s_g;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      int v = g < n_groups ? a.neigh[((int64_t)g << 6) + (x << 4) + s_yz] : -1;
+      nb[j][x] = (v >= 0 && v < a.Hin) ? v : a.Hin;
+    }
+  }
+  // compute role: column r of each of the two column tiles, channel half kh
+  const int sib = r & 7, si = sib >> 2, sj = (sib >> 1) & 1, sk = sib & 1;
+  int cbase[2];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) cbase[nt] = kh * kB16Half + (wave * 8 + nt * 4 + (r >> 3)) * 32;
+
+  for (int pass = 0; pass < npass; ++pass) {
+    floatx16 acc[MT][2];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
+
+    uint4 xr[2][4];
+    uint4 wr[kWVec];
+    // fetch(slab, dx): the weights of the 9 taps with offset dx and the x-layer(s) they add:
+    // dx = 0 brings layers 0 and 1, dx = 1 layer 2, dx = 2 layer 3
+#define OCNN_FETCH(SLAB, DX)                                                                   \
+    do {                                                                                       \
+      const uint4* wsrc = Wt + (((int64_t)pass * nslab + (SLAB)) * 3 + (DX)) * kWUnits;        \
+      _Pragma("unroll") for (int v = 0; v < kWVec; ++v) {                                      \
+        int idx = v * 256 + threadIdx.x;                                                       \
+        wr[v] = idx < kWUnits ? wsrc[idx] : make_uint4(0, 0, 0, 0);                            \
+      }                                                                                        \
+      const int col = (SLAB) * 2 + s_kh;                                                       \
+      _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                          \
+        xr[0][j] = xt[(int64_t)nb[j][(DX) + 1] * cpad8 + col];                                 \
+        if ((DX) == 0) xr[1][j] = xt[(int64_t)nb[j][0] * cpad8 + col];                         \
+      }                                                                                        \
+    } while (0)
+    OCNN_FETCH(0, 0);
+    for (int slab = 0; slab < nslab; ++slab) {
+#pragma unroll
+      for (int dx = 0; dx < 3; ++dx) {
+        __syncthreads();
+#pragma unroll
+        for (int v = 0; v < kWVec; ++v) {
+          int idx = v * 256 + threadIdx.x;
+          if (idx < kWUnits) sW[idx] = wr[v];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int g = wave * 8 + 2 * j + s_g;
+          sX[s_kh * kB16Half + g * 32 + b16_unit(dx + 1, s_y, s_z)] = xr[0][j];
+          if (dx == 0) sX[s_kh * kB16Half + g * 32 + b16_unit(0, s_y, s_z)] = xr[1][j];
+        }
+        __syncthreads();
+        if (dx == 0) OCNN_FETCH(slab, 1);
+        else if (dx == 1) OCNN_FETCH(slab, 2);
+        else if (slab + 1 < nslab) OCNN_FETCH(slab + 1, 0);
+        const int ux = (dx + si) & 1;
+#pragma unroll
+        for (int dy = 0; dy < 3; ++dy)
+#pragma unroll
+          for (int dz = 0; dz < 3; ++dz) {
+            const int y = dy + sj, z = dz + sk;
+            const int unit = ux | ((y & 1) << 1) | ((z & 1) << 2) | ((y >> 1) << 3) | ((z >> 1) << 4);
+            union { uint4 q; bf16x8 v; } b0, b1;
+            b0.q = sX[cbase[0] + unit];
+            b1.q = sX[cbase[1] + unit];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+              union { uint4 q; bf16x8 v; } av;
+              av.q = sW[((dy * 3 + dz) * MT + mt) * 64 + lane];
+              acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b0.v, acc[mt][0], 0, 0, 0);
+              acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b1.v, acc[mt][1], 0, 0, 0);
+            }
+          }
+      }
+    }
+#undef OCNN_FETCH
+    if (n0 < a.N) store_tiles<uint16_t, MT>(a, out, acc, pass * MT, n0, lane);
+  }
+}
+
+// weights for the bf16 LDS kernel: [pass][slab][dx][dy*3+dz][mt][lane][8 channels]; the tap
+// index counts geometric offsets, so a deconvolution (which gathers through the mirrored
+// offset) reads weight tap 26 - k
+__global__ void pack_weights_lds_bf16(uint16_t* __restrict__ Wt, const uint16_t* __restrict__ W, int M, int Cin,
+    int MT, int npass, int nslab, int64_t sm, int64_t sc, int mirror) {
+  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t total = (int64_t)npass * nslab * 27 * MT * 64 * 8;
+  if (id >= total) return;
+  int j = (int)(id & 7);
+  int l = (int)((id >> 3) & 63);
+  int64_t f = id >> 9;
+  int mt = (int)(f % MT); f /= MT;
+  int k = (int)(f % 27); f /= 27;
+  int slab = (int)(f % nslab);
+  int pass = (int)(f / nslab);
+  int m = (pass * MT + mt) * 32 + (l & 31), c = slab * 16 + 8 * (l >> 5) + j;
+  int kw = mirror ? 26 - k : k;
+  Wt[id] = (m < M && c < Cin) ? W[m * sm + c * sc + kw] : (uint16_t)0;
+}
+
 template <typename T>
 __global__ void zero_rows_kernel(T* p, int64_t n) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -371,7 +538,7 @@ struct ConvPlan {
   int mode;
   KernelTaps taps;
   int mtiles, csteps;
-  size_t wt_bytes, ichild_bytes, total_bytes;
+  size_t wt_bytes, ichild_bytes, xt_bytes, total_bytes;
 };
 
 inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -425,7 +592,16 @@ int make_plan(const Info* o, int depth, int channel_in, int num_output, const in
     p->wt_bytes = align256(lds_words * sizeof(float) > p->wt_bytes ? lds_words * sizeof(float) : p->wt_bytes);
   }
   p->ichild_bytes = nempty ? align256(sizeof(int) * (size_t)(p->ichild_h + 1)) : 0;
-  p->total_bytes = p->wt_bytes + p->ichild_bytes;
+  p->xt_bytes = 0;
+  if (dtype == OCNN_BF16 && stride == 1 && !nempty && p->taps.count == 27) {
+    // LDS kernel: weights padded to passes of 2 row tiles and slabs of 16 channels, plus the
+    // row-major copy of the input ([H + 1, Cpad] bf16)
+    size_t cpad = (size_t)(channel_in + 15) / 16 * 16;
+    size_t w = (size_t)((p->mtiles + 1) / 2) * (cpad / 16) * 27 * 2 * 64 * 8 * sizeof(uint16_t);
+    if (w > p->wt_bytes) p->wt_bytes = align256(w);
+    p->xt_bytes = align256(((size_t)p->btm_h + 1) * cpad * sizeof(uint16_t));
+  }
+  p->total_bytes = p->wt_bytes + p->ichild_bytes + p->xt_bytes;
   return OCNN_OK;
 }
 
@@ -510,6 +686,22 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
       conv_f32_kernel<2><<<grid, kConvWaves * 64, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
     else
       conv_f32_kernel<4><<<grid, kConvWaves * 64, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
+  } else if (a.mode == kModeS1 && !a.nempty && a.K == 27) {
+    const int MT = a.mtiles == 1 ? 1 : 2;
+    const int cpad = (a.Cin + 15) / 16 * 16;
+    const int npass = (a.mtiles + MT - 1) / MT, nslab = cpad / 16;
+    int64_t total = (int64_t)npass * nslab * 27 * MT * 64 * 8;
+    pack_weights_lds_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)wsb, (const uint16_t*)weights, a.M, a.Cin,
+        MT, npass, nslab, sm, sc, deconv);
+    uint16_t* xt = reinterpret_cast<uint16_t*>(wsb + p.wt_bytes + p.ichild_bytes);
+    dim3 tgrid((a.Hin + 1 + 63) / 64, (cpad + 63) / 64);
+    transpose_rows_kernel<uint16_t><<<tgrid, 256, 0, s>>>(xt, (const uint16_t*)btm, a.Cin, a.Hin, cpad);
+    OCNN_LAUNCH_OK("pack/transpose");
+    // the kernel walks geometric offsets in natural order (the packer mirrored the weights)
+    if (MT == 1)
+      conv_s1_bf16_lds_kernel<1><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, n_tiles, cpad / 8);
+    else
+      conv_s1_bf16_lds_kernel<2><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, n_tiles, cpad / 8);
   } else {
     int64_t total = (int64_t)a.K * a.csteps * a.mtiles * 64 * 8;
     pack_weights_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)wsb, (const uint16_t*)weights, a.M, a.Cin,
