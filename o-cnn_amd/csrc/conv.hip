@@ -516,6 +516,312 @@ __global__ void pack_weights_lds_bf16(uint16_t* __restrict__ Wt, const uint16_t*
   Wt[id] = (m < M && c < Cin) ? W[m * sm + c * sc + kw] : (uint16_t)0;
 }
 
+
+// ---- 2x2x2 stride-2 convolution over all nodes ----------------------------------------------
+//   out[co, h] = sum_ci sum_s W[co, ci*8 + s] * x[ci, 8h + s]
+// The 8 taps of column h are the 8 children of parent h: 32 contiguous bytes (fp32) per
+// channel.  Lane (n, kh) of a column tile loads ONE float4 = taps 4kh .. 4kh+3 of column n, so
+// a wavefront load is a fully coalesced 1-KiB read and every input element is read exactly
+// once; the four values feed four MFMA k-steps whose k-pairs are (tap j, tap 4+j) -- the
+// weights are packed in that order.  HBM-bound at Cin = Cout = 64 (28 flop/byte).
+constexpr int kS2Slab = 4;  // input channels per weight slab (fp32)
+
+template <int MT>
+__global__ __launch_bounds__(256) void conv_s2_f32_kernel(ConvArgs a, float* __restrict__ out,
+    const float* __restrict__ in, const float* __restrict__ Wt, int n_tiles) {
+  constexpr int kWWords = kS2Slab * 4 * MT * 64;
+  constexpr int kWVec = (kWWords / 4 + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float sW[kWWords];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = xcd_tile(blockIdx.x, n_tiles);
+  if (tile >= n_tiles) return;
+  const int n0 = tile * kTileCols + wave * kWaveCols;
+  const int r = lane & 31, kh = lane >> 5;
+  const int nslab = (a.Cin + kS2Slab - 1) / kS2Slab;
+  const int npass = (a.mtiles + MT - 1) / MT;
+  // element offset of my float4 inside a channel row, per column tile (-1: column out of range)
+  int64_t xoff[2];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+    int n = n0 + nt * 32 + r;
+    xoff[nt] = n < a.N ? (int64_t)n * 8 + 4 * kh : -1;
+  }
+  for (int pass = 0; pass < npass; ++pass) {
+    floatx16 acc[MT][2];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
+    float4 wr[kWVec];
+    auto fetch_w = [&](int slab) {
+      const float4* wsrc = reinterpret_cast<const float4*>(Wt + ((int64_t)pass * nslab + slab) * kWWords);
+#pragma unroll
+      for (int v = 0; v < kWVec; ++v) {
+        int idx = v * 256 + threadIdx.x;
+        wr[v] = idx < kWWords / 4 ? wsrc[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    };
+    fetch_w(0);
+    for (int slab = 0; slab < nslab; ++slab) {
+      __syncthreads();
+#pragma unroll
+      for (int v = 0; v < kWVec; ++v) {
+        int idx = v * 256 + threadIdx.x;
+        if (idx < kWWords / 4) reinterpret_cast<float4*>(sW)[idx] = wr[v];
+      }
+      __syncthreads();
+      if (slab + 1 < nslab) fetch_w(slab + 1);
+      float4 b[kS2Slab][2];
+#pragma unroll
+      for (int cc = 0; cc < kS2Slab; ++cc) {
+        const int c = slab * kS2Slab + cc;
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+          b[cc][nt] = (c < a.Cin && xoff[nt] >= 0)
+              ? *reinterpret_cast<const float4*>(in + (int64_t)c * a.Hin + xoff[nt])
+              : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int cc = 0; cc < kS2Slab; ++cc)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float b0 = j == 0 ? b[cc][0].x : j == 1 ? b[cc][0].y : j == 2 ? b[cc][0].z : b[cc][0].w;
+          const float b1 = j == 0 ? b[cc][1].x : j == 1 ? b[cc][1].y : j == 2 ? b[cc][1].z : b[cc][1].w;
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            float av = sW[((cc * 4 + j) * MT + mt) * 64 + lane];
+            acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b0, acc[mt][0], 0, 0, 0);
+            acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b1, acc[mt][1], 0, 0, 0);
+          }
+        }
+    }
+    if (n0 < a.N) store_tiles<float, MT>(a, out, acc, pass * MT, n0, lane);
+  }
+}
+// [pass][slab][cc][j][mt][lane]: lane (m, kh) <- W[m][(slab*4+cc)*8 + 4kh + j]
+__global__ void pack_weights_s2_f32(float* __restrict__ Wt, const float* __restrict__ W, int M, int Cin, int MT,
+    int npass, int nslab) {
+  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t total = (int64_t)npass * nslab * kS2Slab * 4 * MT * 64;
+  if (id >= total) return;
+  int l = (int)(id & 63);
+  int64_t f = id >> 6;
+  int mt = (int)(f % MT); f /= MT;
+  int j = (int)(f % 4); f /= 4;
+  int cc = (int)(f % kS2Slab); f /= kS2Slab;
+  int slab = (int)(f % nslab);
+  int pass = (int)(f / nslab);
+  int m = (pass * MT + mt) * 32 + (l & 31), c = slab * kS2Slab + cc;
+  Wt[id] = (m < M && c < Cin) ? W[(int64_t)m * Cin * 8 + c * 8 + 4 * (l >> 5) + j] : 0.0f;
+}
+
+// bf16: one 16-byte load = all 8 taps of (channel ci0 + kh, column n); an MFMA k-step of 16
+// covers two input channels.  Slab = 8 channels = 4 k-steps.
+template <int MT>
+__global__ __launch_bounds__(256) void conv_s2_bf16_kernel(ConvArgs a, uint16_t* __restrict__ out,
+    const uint16_t* __restrict__ in, const uint4* __restrict__ Wt, int n_tiles) {
+  constexpr int kWUnits = 4 * MT * 64;
+  __shared__ uint4 sW[kWUnits];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = xcd_tile(blockIdx.x, n_tiles);
+  if (tile >= n_tiles) return;
+  const int n0 = tile * kTileCols + wave * kWaveCols;
+  const int r = lane & 31, kh = lane >> 5;
+  const int nslab = (a.Cin + 7) / 8;
+  const int npass = (a.mtiles + MT - 1) / MT;
+  int64_t xoff[2];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+    int n = n0 + nt * 32 + r;
+    xoff[nt] = n < a.N ? (int64_t)n * 8 : -1;
+  }
+  for (int pass = 0; pass < npass; ++pass) {
+    floatx16 acc[MT][2];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
+    for (int slab = 0; slab < nslab; ++slab) {
+      __syncthreads();
+      for (int idx = threadIdx.x; idx < kWUnits; idx += 256)
+        sW[idx] = Wt[((int64_t)pass * nslab + slab) * kWUnits + idx];
+      __syncthreads();
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int c = slab * 8 + 2 * q + kh;
+        union { uint4 v4; bf16x8 v; } b0, b1;
+        b0.v4 = (c < a.Cin && xoff[0] >= 0) ? *reinterpret_cast<const uint4*>(in + (int64_t)c * a.Hin + xoff[0])
+                                            : make_uint4(0, 0, 0, 0);
+        b1.v4 = (c < a.Cin && xoff[1] >= 0) ? *reinterpret_cast<const uint4*>(in + (int64_t)c * a.Hin + xoff[1])
+                                            : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          union { uint4 v4; bf16x8 v; } av;
+          av.v4 = sW[(q * MT + mt) * 64 + lane];
+          acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b0.v, acc[mt][0], 0, 0, 0);
+          acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b1.v, acc[mt][1], 0, 0, 0);
+        }
+      }
+    }
+    if (n0 < a.N) store_tiles<uint16_t, MT>(a, out, acc, pass * MT, n0, lane);
+  }
+}
+// [pass][slab][q][mt][lane][j]: lane (m, kh), tap j <- W[m][(slab*8 + 2q + kh)*8 + j]
+__global__ void pack_weights_s2_bf16(uint16_t* __restrict__ Wt, const uint16_t* __restrict__ W, int M, int Cin,
+    int MT, int npass, int nslab) {
+  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t total = (int64_t)npass * nslab * 4 * MT * 64 * 8;
+  if (id >= total) return;
+  int j = (int)(id & 7);
+  int l = (int)((id >> 3) & 63);
+  int64_t f = id >> 9;
+  int mt = (int)(f % MT); f /= MT;
+  int q = (int)(f % 4); f /= 4;
+  int slab = (int)(f % nslab);
+  int pass = (int)(f / nslab);
+  int m = (pass * MT + mt) * 32 + (l & 31), c = slab * 8 + 2 * q + (l >> 5);
+  Wt[id] = (m < M && c < Cin) ? W[(int64_t)m * Cin * 8 + c * 8 + j] : (uint16_t)0;
+}
+
+// ---- 2x2x2 stride-2 deconvolution over all nodes ----------------------------------------------
+//   out[co, 8h + s] = sum_ci W[ci, co*8 + s] * in[ci, h]
+// A GEMM with rows m' = co*8 + s (the weight matrix transposed, no re-layout needed for fp32:
+// row ci of W is contiguous over m'), K = Cin, columns = parents h.  In the 32x32 accumulator
+// a lane holds 4 consecutive rows = 4 consecutive children of one (co, h): one 16-byte store;
+// the two half wavefronts complete the 32-byte sibling group, consecutive lanes are consecutive
+// parents, so stores are coalesced and every child is written exactly once (no atomics, no
+// zero fill -- the reference scatters with atomicAdd, octree/octree/octree_nn.cu:130-174).
+template <typename OutT>
+__device__ inline void store_children(const ConvArgs& a, OutT* __restrict__ out, const floatx16& acc,
+    int row0, int n, int kh) {
+  // rows row0 + 8q + 4kh + (0..3), q = 0..3  ->  co = (row0 >> 3) + q, children 4kh .. 4kh+3
+  if (n >= a.N) return;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    int co = (row0 >> 3) + q;
+    if (co >= a.M) continue;
+    int64_t o = (int64_t)co * a.Hout + (int64_t)n * 8 + 4 * kh;
+    if (sizeof(OutT) == 4) {
+      *reinterpret_cast<float4*>(reinterpret_cast<float*>(out) + o) =
+          make_float4(acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
+    } else {
+      uint2 v;
+      v.x = (uint32_t)f32_to_bf16(acc[4 * q]) | ((uint32_t)f32_to_bf16(acc[4 * q + 1]) << 16);
+      v.y = (uint32_t)f32_to_bf16(acc[4 * q + 2]) | ((uint32_t)f32_to_bf16(acc[4 * q + 3]) << 16);
+      *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(out) + o) = v;
+    }
+  }
+}
+
+constexpr int kD2MT = 4;  // row tiles per pass: 128 rows = 16 output channels x 8 children
+
+__global__ __launch_bounds__(256) void deconv_s2_f32_kernel(ConvArgs a, float* __restrict__ out,
+    const float* __restrict__ in, const float* __restrict__ W, int n_tiles) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = xcd_tile(blockIdx.x, n_tiles);
+  if (tile >= n_tiles) return;
+  const int n0 = tile * kTileCols + wave * kWaveCols;
+  if (n0 >= a.N) return;
+  const int r = lane & 31, kh = lane >> 5;
+  const int rows = a.M * 8;
+  const int npass = (rows + 32 * kD2MT - 1) / (32 * kD2MT);
+  const int ksteps = (a.Cin + 1) / 2;
+  int ncol[2];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) ncol[nt] = n0 + nt * 32 + r;
+  for (int pass = 0; pass < npass; ++pass) {
+    floatx16 acc[kD2MT][2];
+#pragma unroll
+    for (int mt = 0; mt < kD2MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
+    const int row_base = pass * 32 * kD2MT;
+#pragma unroll 2
+    for (int ks = 0; ks < ksteps; ++ks) {
+      const int c = 2 * ks + kh;
+      const bool cv = c < a.Cin;
+      float b0 = (cv && ncol[0] < a.N) ? in[(int64_t)c * a.Hin + ncol[0]] : 0.0f;
+      float b1 = (cv && ncol[1] < a.N) ? in[(int64_t)c * a.Hin + ncol[1]] : 0.0f;
+#pragma unroll
+      for (int mt = 0; mt < kD2MT; ++mt) {
+        int m = row_base + mt * 32 + r;
+        float av = (cv && m < rows) ? W[(int64_t)c * rows + m] : 0.0f;
+        acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b0, acc[mt][0], 0, 0, 0);
+        acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b1, acc[mt][1], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int mt = 0; mt < kD2MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) store_children<float>(a, out, acc[mt][nt], row_base + mt * 32, ncol[nt], kh);
+  }
+}
+
+// bf16: activations come from the row-major copy [H + 1, Cpad] (16-byte operand loads); weights
+// packed [pass][kstep][mt][lane][8]: lane (m', kh), j <- W[16*kstep + 8kh + j][m']
+__global__ __launch_bounds__(256) void deconv_s2_bf16_kernel(ConvArgs a, uint16_t* __restrict__ out,
+    const uint4* __restrict__ xt, const uint4* __restrict__ Wt, int n_tiles, int cpad8) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = xcd_tile(blockIdx.x, n_tiles);
+  if (tile >= n_tiles) return;
+  const int n0 = tile * kTileCols + wave * kWaveCols;
+  if (n0 >= a.N) return;
+  const int r = lane & 31, kh = lane >> 5;
+  const int rows = a.M * 8;
+  const int npass = (rows + 32 * kD2MT - 1) / (32 * kD2MT);
+  const int ksteps = cpad8 >> 1;
+  int ncol[2];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) ncol[nt] = n0 + nt * 32 + r;
+  for (int pass = 0; pass < npass; ++pass) {
+    floatx16 acc[kD2MT][2];
+#pragma unroll
+    for (int mt = 0; mt < kD2MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
+    const int row_base = pass * 32 * kD2MT;
+#pragma unroll 2
+    for (int ks = 0; ks < ksteps; ++ks) {
+      union { uint4 v4; bf16x8 v; } b0, b1;
+      b0.v4 = xt[(int64_t)min(ncol[0], a.Hin) * cpad8 + 2 * ks + kh];
+      b1.v4 = xt[(int64_t)min(ncol[1], a.Hin) * cpad8 + 2 * ks + kh];
+#pragma unroll
+      for (int mt = 0; mt < kD2MT; ++mt) {
+        union { uint4 v4; bf16x8 v; } av;
+        av.v4 = Wt[(((int64_t)pass * ksteps + ks) * kD2MT + mt) * 64 + lane];
+        acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b0.v, acc[mt][0], 0, 0, 0);
+        acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b1.v, acc[mt][1], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int mt = 0; mt < kD2MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) store_children<uint16_t>(a, out, acc[mt][nt], row_base + mt * 32, ncol[nt], kh);
+  }
+}
+__global__ void pack_weights_d2_bf16(uint16_t* __restrict__ Wt, const uint16_t* __restrict__ W, int rows, int Cin,
+    int npass, int ksteps) {
+  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t total = (int64_t)npass * ksteps * kD2MT * 64 * 8;
+  if (id >= total) return;
+  int j = (int)(id & 7);
+  int l = (int)((id >> 3) & 63);
+  int64_t f = id >> 9;
+  int mt = (int)(f % kD2MT); f /= kD2MT;
+  int ks = (int)(f % ksteps);
+  int pass = (int)(f / ksteps);
+  int m = (pass * kD2MT + mt) * 32 + (l & 31), c = 16 * ks + 8 * (l >> 5) + j;
+  Wt[id] = (m < rows && c < Cin) ? W[(int64_t)c * rows + m] : (uint16_t)0;
+}
+
 template <typename T>
 __global__ void zero_rows_kernel(T* p, int64_t n) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -601,6 +907,20 @@ int make_plan(const Info* o, int depth, int channel_in, int num_output, const in
     if (w > p->wt_bytes) p->wt_bytes = align256(w);
     p->xt_bytes = align256(((size_t)p->btm_h + 1) * cpad * sizeof(uint16_t));
   }
+  const bool is222 = ks[0] == 2 && ks[1] == 2 && ks[2] == 2;
+  if (stride == 2 && !nempty && is222 && !deconv) {  // dedicated stride-2 kernels: padded packing
+    size_t npass = (size_t)(p->mtiles + 1) / 2;
+    size_t w = dtype == OCNN_F32 ? npass * ((channel_in + 3) / 4) * kS2Slab * 4 * 2 * 64 * sizeof(float)
+                                 : npass * ((channel_in + 7) / 8) * 4 * 2 * 64 * 8 * sizeof(uint16_t);
+    if (w > p->wt_bytes) p->wt_bytes = align256(w);
+  }
+  if (stride == 2 && !nempty && is222 && deconv && dtype == OCNN_BF16) {
+    size_t cpad = (size_t)(channel_in + 15) / 16 * 16;
+    size_t npass = ((size_t)num_output * 8 + 32 * kD2MT - 1) / (32 * kD2MT);
+    size_t w = npass * (cpad / 16) * kD2MT * 64 * 8 * sizeof(uint16_t);
+    if (w > p->wt_bytes) p->wt_bytes = align256(w);
+    p->xt_bytes = align256(((size_t)p->btm_h + 1) * cpad * sizeof(uint16_t));
+  }
   p->total_bytes = p->wt_bytes + p->ichild_bytes + p->xt_bytes;
   return OCNN_OK;
 }
@@ -664,7 +984,43 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
   int64_t sc = deconv ? (int64_t)num_output * a.K : a.K;
   int n_tiles = (a.N + kTileCols - 1) / kTileCols;
   int grid = ((n_tiles + 7) / 8) * 8;
-  if (dtype == OCNN_F32 && a.mode == kModeS1 && !a.nempty && a.K == 27) {
+  const bool k222 = ks[0] == 2 && ks[1] == 2 && ks[2] == 2;
+  if (a.mode == kModeS2Conv && !a.nempty && k222 && (a.Hin & 7) == 0 &&
+      (reinterpret_cast<uintptr_t>(btm) & 15) == 0) {
+    const int MT = a.mtiles == 1 ? 1 : 2;
+    const int npass = (a.mtiles + MT - 1) / MT;
+    if (dtype == OCNN_F32) {
+      const int nslab = (a.Cin + kS2Slab - 1) / kS2Slab;
+      int64_t total = (int64_t)npass * nslab * kS2Slab * 4 * MT * 64;
+      pack_weights_s2_f32<<<blocks_for(total), kBlock, 0, s>>>((float*)wsb, (const float*)weights, a.M, a.Cin, MT, npass, nslab);
+      if (MT == 1) conv_s2_f32_kernel<1><<<grid, 256, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
+      else conv_s2_f32_kernel<2><<<grid, 256, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
+    } else {
+      const int nslab = (a.Cin + 7) / 8;
+      int64_t total = (int64_t)npass * nslab * 4 * MT * 64 * 8;
+      pack_weights_s2_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)wsb, (const uint16_t*)weights, a.M, a.Cin, MT, npass, nslab);
+      if (MT == 1) conv_s2_bf16_kernel<1><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const uint16_t*)btm, (const uint4*)wsb, n_tiles);
+      else conv_s2_bf16_kernel<2><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const uint16_t*)btm, (const uint4*)wsb, n_tiles);
+    }
+  } else if (a.mode == kModeS2Deconv && !a.nempty && (reinterpret_cast<uintptr_t>(top) & 15) == 0) {
+    // columns are the parents here: one column tile writes the 8 children of 256 parents
+    ConvArgs d = a;
+    d.N = a.Hin;
+    int d_tiles = (d.N + kTileCols - 1) / kTileCols;
+    int d_grid = ((d_tiles + 7) / 8) * 8;
+    if (dtype == OCNN_F32) {
+      deconv_s2_f32_kernel<<<d_grid, 256, 0, s>>>(d, (float*)top, (const float*)btm, (const float*)weights, d_tiles);
+    } else {
+      const int cpad = (a.Cin + 15) / 16 * 16;
+      const int rows = a.M * 8, npass = (rows + 32 * kD2MT - 1) / (32 * kD2MT), ksteps = cpad / 16;
+      int64_t total = (int64_t)npass * ksteps * kD2MT * 64 * 8;
+      pack_weights_d2_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)wsb, (const uint16_t*)weights, rows, a.Cin, npass, ksteps);
+      uint16_t* xt = reinterpret_cast<uint16_t*>(wsb + p.wt_bytes + p.ichild_bytes);
+      dim3 tgrid((a.Hin + 1 + 63) / 64, (cpad + 63) / 64);
+      transpose_rows_kernel<uint16_t><<<tgrid, 256, 0, s>>>(xt, (const uint16_t*)btm, a.Cin, a.Hin, cpad);
+      deconv_s2_bf16_kernel<<<d_grid, 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles, cpad / 8);
+    }
+  } else if (dtype == OCNN_F32 && a.mode == kModeS1 && !a.nempty && a.K == 27) {
     const int MT = a.mtiles == 1 ? 1 : 2;
     const int npass = (a.mtiles + MT - 1) / MT, nslab = (a.Cin + kSlab - 1) / kSlab;
     int64_t total = (int64_t)npass * nslab * a.K * 2 * MT * 64;
