@@ -127,25 +127,26 @@ __global__ void radix_hist_kernel(const uint64_t* __restrict__ key, int64_t n, i
   hist[(int64_t)threadIdx.x * n_blocks + blockIdx.x] = h[threadIdx.x];  // digit-major
 }
 
-// exclusive scan of the digit-major histogram (single workgroup)
-__global__ void radix_scan_kernel(int* __restrict__ hist, int64_t n) {
+// Scan of the digit-major histogram in two levels: workgroup d turns row d (the counts of
+// digit d in every tile) into exclusive offsets within the digit and records the digit
+// total; the scatter kernel adds the exclusive scan of the 256 totals itself.
+__global__ void radix_scan_kernel(int* __restrict__ hist, int n_blocks, int* __restrict__ digit_total) {
   __shared__ int carry;
+  int* row = hist + (int64_t)blockIdx.x * n_blocks;
   if (threadIdx.x == 0) carry = 0;
   __syncthreads();
-  for (int64_t start = 0; start < n; start += kBlock * 4) {
-    int64_t i0 = start + (int64_t)threadIdx.x * 4;
-    int v[4], s = 0;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) { v[j] = i0 + j < n ? hist[i0 + j] : 0; s += v[j]; }
+  for (int start = 0; start < n_blocks; start += kBlock) {
+    int i = start + threadIdx.x;
+    int v = i < n_blocks ? row[i] : 0;
     int total;
-    int ex = block_exclusive_scan(s, &total);
-    int c = carry + ex;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) { if (i0 + j < n) hist[i0 + j] = c; c += v[j]; }
+    int ex = block_exclusive_scan(v, &total);
+    int c = carry;
+    if (i < n_blocks) row[i] = c + ex;
     __syncthreads();
-    if (threadIdx.x == 0) carry += total;
+    if (threadIdx.x == 0) carry = c + total;
     __syncthreads();
   }
+  if (threadIdx.x == 0) digit_total[blockIdx.x] = carry;
 }
 
 // Each round places 256 consecutive elements; inside a wavefront the rank among
@@ -154,11 +155,15 @@ __global__ void radix_scan_kernel(int* __restrict__ hist, int64_t n) {
 // lane) equals the input order, which keeps the sort stable.
 __global__ void radix_scatter_kernel(const uint64_t* __restrict__ key_in, const uint32_t* __restrict__ val_in,
     uint64_t* __restrict__ key_out, uint32_t* __restrict__ val_out, int64_t n, int shift,
-    const int* __restrict__ hist, int n_blocks) {
+    const int* __restrict__ hist, int n_blocks, const int* __restrict__ digit_total) {
   __shared__ int running[256];
   __shared__ int wave_cnt[kWaves][256];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  running[threadIdx.x] = hist[(int64_t)threadIdx.x * n_blocks + blockIdx.x];
+  {
+    int total;
+    int digit_base = block_exclusive_scan(digit_total[threadIdx.x], &total);
+    running[threadIdx.x] = digit_base + hist[(int64_t)threadIdx.x * n_blocks + blockIdx.x];
+  }
 #pragma unroll
   for (int w = 0; w < kWaves; ++w) wave_cnt[w][threadIdx.x] = 0;
   __syncthreads();
@@ -396,24 +401,49 @@ __global__ void leaf_signal_kernel(float* __restrict__ feature, float* __restric
 
 // ---- neighbour kernels (same arithmetic as octree_index.hip; private copies keep this
 // translation unit self-contained) ----------------------------------------------------------
+// Sparse-layer neighbour table.  A workgroup takes 256 consecutive parent-level nodes,
+// compacts the non-empty ones into LDS (most nodes of a deep level are empty) and then
+// every wavefront writes the 64-slot blocks of the compacted nodes, two nodes per
+// iteration so that two dependent load chains (neigh -> children) are in flight.
 __global__ void b_neigh_sparse_kernel(int* __restrict__ neigh_child, const int* __restrict__ neigh,
     const int* __restrict__ children, int node_num) {
-  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  int i = (int)(id >> 6), j = (int)(id & 63);
-  if (i >= node_num) return;
-  int l0 = children[i];
-  if (l0 < 0) return;
-  int x = j >> 4, y = (j >> 2) & 3, z = j & 3;
-  int sib = i & 7;
-  int px = ((x + 1) >> 1) + (sib >> 2), py = ((y + 1) >> 1) + ((sib >> 1) & 1), pz = ((z + 1) >> 1) + (sib & 1);
-  int octant = (((x + 1) & 1) << 2) | (((y + 1) & 1) << 1) | ((z + 1) & 1);
-  int k = neigh[((int64_t)(i >> 3) << 6) + ((px << 4) | (py << 2) | pz)];
-  int t = -1;
-  if (k >= 0) {
-    int l1 = children[k];
-    if (l1 >= 0) t = (l1 << 3) + octant;
+  __shared__ int s_node[kBlock], s_rank[kBlock], s_count;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int i = blockIdx.x * kBlock + threadIdx.x;
+  const int l0 = i < node_num ? children[i] : -1;
+  int total;
+  const int pos = block_exclusive_scan(l0 >= 0 ? 1 : 0, &total);
+  if (l0 >= 0) { s_node[pos] = i; s_rank[pos] = l0; }
+  if (threadIdx.x == 0) s_count = total;
+  __syncthreads();
+  const int count = s_count;
+  const int x = lane >> 4, y = (lane >> 2) & 3, z = lane & 3;
+  const int hx = (x + 1) >> 1, hy = (y + 1) >> 1, hz = (z + 1) >> 1;
+  const int octant = (((x + 1) & 1) << 2) | (((y + 1) & 1) << 1) | ((z + 1) & 1);
+  for (int e = wave * 2; e < count; e += 2 * (kBlock / 64)) {
+    int t[2], rank[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      t[u] = -1;
+      rank[u] = -1;
+      if (e + u < count) {
+        const int node = s_node[e + u];
+        rank[u] = s_rank[e + u];
+        const int sib = node & 7;
+        const int slot = ((hx + (sib >> 2)) << 4) | ((hy + ((sib >> 1) & 1)) << 2) | (hz + (sib & 1));
+        t[u] = neigh[((int64_t)(node >> 3) << 6) + slot];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      int v = -1;
+      if (t[u] >= 0) {
+        const int l1 = children[t[u]];
+        if (l1 >= 0) v = (l1 << 3) + octant;
+      }
+      if (rank[u] >= 0) neigh_child[((int64_t)rank[u] << 6) + lane] = v;
+    }
   }
-  neigh_child[((int64_t)l0 << 6) + j] = t;
 }
 __global__ void b_neigh_full_kernel(int* __restrict__ neigh, int depth, int64_t total) {
   int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -454,7 +484,7 @@ Layout make_layout(int64_t N, int B, int depth) {
   size_t n = (size_t)(N > 0 ? N : 1);
   for (int i = 0; i < 2; ++i) { L.key[i] = take(8 * n); L.val[i] = take(4 * n); }
   L.hist_blocks = (int)((n + kSortTile - 1) / kSortTile);
-  L.hist = take(sizeof(int) * 256 * (size_t)L.hist_blocks);
+  L.hist = take(sizeof(int) * 256 * ((size_t)L.hist_blocks + 1));  // + 256 digit totals
   L.scan = take(scan_scratch_bytes((int64_t)n));
   L.ustart = take(4 * (n + 1));
   L.leaf_node = take(4 * n);
@@ -572,6 +602,7 @@ int ocnn_points2octree_plan(const void* const* points_dev, const void* const* po
   uint64_t* d_key[2] = {reinterpret_cast<uint64_t*>(ws + L.key[0]), reinterpret_cast<uint64_t*>(ws + L.key[1])};
   uint32_t* d_val[2] = {reinterpret_cast<uint32_t*>(ws + L.val[0]), reinterpret_cast<uint32_t*>(ws + L.val[1])};
   int* d_hist = reinterpret_cast<int*>(ws + L.hist);
+  int* d_digit_total = d_hist + (int64_t)256 * L.hist_blocks;
   int* d_scan = reinterpret_cast<int*>(ws + L.scan);
   int* d_ustart = reinterpret_cast<int*>(ws + L.ustart);
 
@@ -596,9 +627,9 @@ int ocnn_points2octree_plan(const void* const* points_dev, const void* const* po
     int nbits = 3 * depth + cloud_bits;
     for (int shift = 0; shift < nbits; shift += 8) {
       radix_hist_kernel<<<L.hist_blocks, kBlock, 0, s>>>(d_key[cur], N, shift, d_hist, L.hist_blocks);
-      radix_scan_kernel<<<1, kBlock, 0, s>>>(d_hist, (int64_t)256 * L.hist_blocks);
+      radix_scan_kernel<<<256, kBlock, 0, s>>>(d_hist, L.hist_blocks, d_digit_total);
       radix_scatter_kernel<<<L.hist_blocks, kBlock, 0, s>>>(d_key[cur], d_val[cur], d_key[cur ^ 1], d_val[cur ^ 1],
-          N, shift, d_hist, L.hist_blocks);
+          N, shift, d_hist, L.hist_blocks, d_digit_total);
       OCNN_LAUNCH_OK("radix pass");
       cur ^= 1;
     }
@@ -748,8 +779,7 @@ int ocnn_points2octree_emit(void* octree_out_dev, const void* info, void* worksp
         int64_t total = (int64_t)B << (3 * d + 3);
         b_neigh_full_kernel<<<blocks_for(total), kBlock, 0, s>>>(neigh, d, total);
       } else if (o.nnum[d - 1] > 0) {
-        int64_t threads = (int64_t)o.nnum[d - 1] << 6;
-        b_neigh_sparse_kernel<<<blocks_for(threads), kBlock, 0, s>>>(neigh,
+        b_neigh_sparse_kernel<<<blocks_for(o.nnum[d - 1]), kBlock, 0, s>>>(neigh,
             reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_NEIGH, d - 1)),
             reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_CHILD, d - 1)), o.nnum[d - 1]);
       }

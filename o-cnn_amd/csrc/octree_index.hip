@@ -40,28 +40,49 @@ __host__ __device__ inline void morton_decode(uint64_t key, int depth, uint32_t*
 namespace {
 
 // ---- neighbour tables --------------------------------------------------------
-// Sparse layer: one wavefront per parent-level node, one lane per slot of the
-// 4x4x4 block of its child group.  Slot (x,y,z) of the child block lies at
-// child-level offset (x-1,y-1,z-1) from child 0, i.e. in the parent-level node at
-// offset ((x+1)>>1)-1 per axis, as its octant ((x+1)&1, ...).
+// Sparse-layer neighbour table.  A workgroup takes 256 consecutive parent-level nodes,
+// compacts the non-empty ones into LDS (most nodes of a deep level are empty) and then
+// every wavefront writes the 64-slot blocks of the compacted nodes, two nodes per
+// iteration so that two dependent load chains (neigh -> children) are in flight.
 __global__ void calc_neigh_sparse_kernel(int* __restrict__ neigh_child, const int* __restrict__ neigh,
     const int* __restrict__ children, int node_num) {
-  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  int i = (int)(id >> 6), j = (int)(id & 63);
-  if (i >= node_num) return;
-  int l0 = children[i];
-  if (l0 < 0) return;
-  int x = j >> 4, y = (j >> 2) & 3, z = j & 3;
-  int sib = i & 7;
-  int px = ((x + 1) >> 1) + (sib >> 2), py = ((y + 1) >> 1) + ((sib >> 1) & 1), pz = ((z + 1) >> 1) + (sib & 1);
-  int octant = (((x + 1) & 1) << 2) | (((y + 1) & 1) << 1) | ((z + 1) & 1);
-  int k = neigh[((int64_t)(i >> 3) << 6) + ((px << 4) | (py << 2) | pz)];
-  int t = -1;
-  if (k >= 0) {
-    int l1 = children[k];
-    if (l1 >= 0) t = (l1 << 3) + octant;
+  __shared__ int s_node[kBlock], s_rank[kBlock], s_count;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int i = blockIdx.x * kBlock + threadIdx.x;
+  const int l0 = i < node_num ? children[i] : -1;
+  int total;
+  const int pos = block_exclusive_scan(l0 >= 0 ? 1 : 0, &total);
+  if (l0 >= 0) { s_node[pos] = i; s_rank[pos] = l0; }
+  if (threadIdx.x == 0) s_count = total;
+  __syncthreads();
+  const int count = s_count;
+  const int x = lane >> 4, y = (lane >> 2) & 3, z = lane & 3;
+  const int hx = (x + 1) >> 1, hy = (y + 1) >> 1, hz = (z + 1) >> 1;
+  const int octant = (((x + 1) & 1) << 2) | (((y + 1) & 1) << 1) | ((z + 1) & 1);
+  for (int e = wave * 2; e < count; e += 2 * (kBlock / 64)) {
+    int t[2], rank[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      t[u] = -1;
+      rank[u] = -1;
+      if (e + u < count) {
+        const int node = s_node[e + u];
+        rank[u] = s_rank[e + u];
+        const int sib = node & 7;
+        const int slot = ((hx + (sib >> 2)) << 4) | ((hy + ((sib >> 1) & 1)) << 2) | (hz + (sib & 1));
+        t[u] = neigh[((int64_t)(node >> 3) << 6) + slot];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      int v = -1;
+      if (t[u] >= 0) {
+        const int l1 = children[t[u]];
+        if (l1 >= 0) v = (l1 << 3) + octant;
+      }
+      if (rank[u] >= 0) neigh_child[((int64_t)rank[u] << 6) + lane] = v;
+    }
   }
-  neigh_child[((int64_t)l0 << 6) + j] = t;
 }
 
 // Full layer: closed form through Morton decode / encode.
@@ -172,8 +193,7 @@ int ocnn_calc_neigh_sparse(int* neigh_child, const int* neigh, const int* childr
   OCNN_REQUIRE(neigh_child && neigh && children, OCNN_E_BADARG, "null pointer");
   OCNN_REQUIRE(node_num >= 0, OCNN_E_BADARG, "node_num %d", node_num);
   if (node_num == 0) return OCNN_OK;
-  int64_t threads = (int64_t)node_num << 6;
-  calc_neigh_sparse_kernel<<<blocks_for(threads), kBlock, 0, as_stream(stream)>>>(neigh_child, neigh,
+  calc_neigh_sparse_kernel<<<blocks_for(node_num), kBlock, 0, as_stream(stream)>>>(neigh_child, neigh,
       children, node_num);
   OCNN_LAUNCH_OK("calc_neigh_sparse");
   return OCNN_OK;
