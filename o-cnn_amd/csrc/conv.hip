@@ -19,6 +19,7 @@ namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));  // one 16-byte LDS / global unit
 
 enum { kModeS1 = 0, kModeS2Conv = 1, kModeS2Deconv = 2 };
 
@@ -391,11 +392,11 @@ __global__ void transpose_rows_kernel(T* __restrict__ dst, const T* __restrict__
 
 template <int MT>
 __global__ __launch_bounds__(256, 2) void conv_s1_bf16_lds_kernel(ConvArgs a, uint16_t* __restrict__ out,
-    const uint4* __restrict__ xt, const uint4* __restrict__ Wt, int n_tiles, int cpad8) {
+    const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles, int cpad8) {
   constexpr int kWUnits = 9 * MT * 64;               // 16-byte units per weight chunk
   constexpr int kWVec = (kWUnits + 255) / 256;
-  __shared__ uint4 sX[2 * kB16Half];
-  __shared__ uint4 sW[kWUnits];
+  __shared__ u32x4 sX[2 * kB16Half];
+  __shared__ u32x4 sW[kWUnits];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int tile = xcd_tile(blockIdx.x, n_tiles);
   if (tile >= n_tiles) return;
@@ -434,64 +435,73 @@ __global__ __launch_bounds__(256, 2) void conv_s1_bf16_lds_kernel(ConvArgs a, ui
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
 
-    uint4 xr[2][4];
-    uint4 wr[kWVec];
-    // fetch(slab, dx): the weights of the 9 taps with offset dx and the x-layer(s) they add:
-    // dx = 0 brings layers 0 and 1, dx = 1 layer 2, dx = 2 layer 3
-#define OCNN_FETCH(SLAB, DX)                                                                   \
+    // Phases: a slab has four, phase L stages x-layer L (into the units with bit0 == L&1;
+    // layer L overwrites layer L-2, whose last readers finished before the phase's first
+    // barrier) and, for L >= 1, the weights of the 9 taps with dx = L-1, then computes them.
+    // Layer L of a later phase is requested two phases ahead into register set L&1, the
+    // weights one phase ahead, so the requests have one or two compute phases to land.
+    u32x4 xr[2][4];
+    u32x4 wr[kWVec];
+#define OCNN_FETCH_W(SLAB, DX)                                                                 \
     do {                                                                                       \
-      const uint4* wsrc = Wt + (((int64_t)pass * nslab + (SLAB)) * 3 + (DX)) * kWUnits;        \
+      const u32x4* wsrc = Wt + (((int64_t)pass * nslab + (SLAB)) * 3 + (DX)) * kWUnits;        \
       _Pragma("unroll") for (int v = 0; v < kWVec; ++v) {                                      \
         int idx = v * 256 + threadIdx.x;                                                       \
-        wr[v] = idx < kWUnits ? wsrc[idx] : make_uint4(0, 0, 0, 0);                            \
-      }                                                                                        \
-      const int col = (SLAB) * 2 + s_kh;                                                       \
-      _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                          \
-        xr[0][j] = xt[(int64_t)nb[j][(DX) + 1] * cpad8 + col];                                 \
-        if ((DX) == 0) xr[1][j] = xt[(int64_t)nb[j][0] * cpad8 + col];                         \
+        wr[v] = idx < kWUnits ? wsrc[idx] : (u32x4)(0u);                                       \
       }                                                                                        \
     } while (0)
-    OCNN_FETCH(0, 0);
+#define OCNN_FETCH_X(SLAB, L)                                                                  \
+    do {                                                                                       \
+      const int col = (SLAB) * 2 + s_kh;                                                       \
+      _Pragma("unroll") for (int j = 0; j < 4; ++j)                                            \
+        xr[(L) & 1][j] = xt[(int64_t)nb[j][L] * cpad8 + col];                                  \
+    } while (0)
+#define OCNN_PHASE(SLAB, L)                                                                    \
+    do {                                                                                       \
+      __syncthreads();                                                                         \
+      if ((L) >= 1) {                                                                          \
+        _Pragma("unroll") for (int v = 0; v < kWVec; ++v) {                                    \
+          int idx = v * 256 + threadIdx.x;                                                     \
+          if (idx < kWUnits) sW[idx] = wr[v];                                                  \
+        }                                                                                      \
+      }                                                                                        \
+      _Pragma("unroll") for (int j = 0; j < 4; ++j)                                            \
+        sX[s_kh * kB16Half + (wave * 8 + 2 * j + s_g) * 32 + b16_unit(L, s_y, s_z)] = xr[(L) & 1][j]; \
+      __syncthreads();                                                                         \
+      /* weights of the next computing phase: phase L requests those of dx = L */            \
+      if ((L) <= 2) OCNN_FETCH_W(SLAB, L);                                                     \
+      /* x-layer two phases ahead */                                                           \
+      if ((L) <= 1) OCNN_FETCH_X(SLAB, (L) + 2);                                               \
+      else if ((SLAB) + 1 < nslab) OCNN_FETCH_X((SLAB) + 1, (L) - 2);                          \
+      if ((L) >= 1) {                                                                          \
+        const int ux = ((L) - 1 + si) & 1;                                                     \
+        _Pragma("unroll") for (int dy = 0; dy < 3; ++dy)                                       \
+        _Pragma("unroll") for (int dz = 0; dz < 3; ++dz) {                                     \
+          const int y = dy + sj, z = dz + sk;                                                  \
+          const int unit = ux | ((y & 1) << 1) | ((z & 1) << 2) | ((y >> 1) << 3) | ((z >> 1) << 4); \
+          union { u32x4 q; bf16x8 v; } b0, b1;                                                 \
+          b0.q = sX[cbase[0] + unit];                                                          \
+          b1.q = sX[cbase[1] + unit];                                                          \
+          _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                  \
+            union { u32x4 q; bf16x8 v; } av;                                                   \
+            av.q = sW[((dy * 3 + dz) * MT + mt) * 64 + lane];                                  \
+            acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b0.v, acc[mt][0], 0, 0, 0); \
+            acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b1.v, acc[mt][1], 0, 0, 0); \
+          }                                                                                    \
+        }                                                                                      \
+      }                                                                                        \
+    } while (0)
+    OCNN_FETCH_X(0, 0);
+    OCNN_FETCH_X(0, 1);
     for (int slab = 0; slab < nslab; ++slab) {
-#pragma unroll
-      for (int dx = 0; dx < 3; ++dx) {
-        __syncthreads();
-#pragma unroll
-        for (int v = 0; v < kWVec; ++v) {
-          int idx = v * 256 + threadIdx.x;
-          if (idx < kWUnits) sW[idx] = wr[v];
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int g = wave * 8 + 2 * j + s_g;
-          sX[s_kh * kB16Half + g * 32 + b16_unit(dx + 1, s_y, s_z)] = xr[0][j];
-          if (dx == 0) sX[s_kh * kB16Half + g * 32 + b16_unit(0, s_y, s_z)] = xr[1][j];
-        }
-        __syncthreads();
-        if (dx == 0) OCNN_FETCH(slab, 1);
-        else if (dx == 1) OCNN_FETCH(slab, 2);
-        else if (slab + 1 < nslab) OCNN_FETCH(slab + 1, 0);
-        const int ux = (dx + si) & 1;
-#pragma unroll
-        for (int dy = 0; dy < 3; ++dy)
-#pragma unroll
-          for (int dz = 0; dz < 3; ++dz) {
-            const int y = dy + sj, z = dz + sk;
-            const int unit = ux | ((y & 1) << 1) | ((z & 1) << 2) | ((y >> 1) << 3) | ((z >> 1) << 4);
-            union { uint4 q; bf16x8 v; } b0, b1;
-            b0.q = sX[cbase[0] + unit];
-            b1.q = sX[cbase[1] + unit];
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-              union { uint4 q; bf16x8 v; } av;
-              av.q = sW[((dy * 3 + dz) * MT + mt) * 64 + lane];
-              acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b0.v, acc[mt][0], 0, 0, 0);
-              acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b1.v, acc[mt][1], 0, 0, 0);
-            }
-          }
-      }
+      OCNN_PHASE(slab, 0);
+      OCNN_PHASE(slab, 1);
+      OCNN_PHASE(slab, 2);
+      OCNN_PHASE(slab, 3);
     }
-#undef OCNN_FETCH
+#undef OCNN_FETCH_W
+#undef OCNN_FETCH_X
+#undef OCNN_PHASE
     if (n0 < a.N) store_tiles<uint16_t, MT>(a, out, acc, pass * MT, n0, lane);
   }
 }
@@ -1055,9 +1065,9 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     OCNN_LAUNCH_OK("pack/transpose");
     // the kernel walks geometric offsets in natural order (the packer mirrored the weights)
     if (MT == 1)
-      conv_s1_bf16_lds_kernel<1><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, n_tiles, cpad / 8);
+      conv_s1_bf16_lds_kernel<1><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad / 8);
     else
-      conv_s1_bf16_lds_kernel<2><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, n_tiles, cpad / 8);
+      conv_s1_bf16_lds_kernel<2><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad / 8);
   } else {
     int64_t total = (int64_t)a.K * a.csteps * a.mtiles * 64 * 8;
     pack_weights_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)wsb, (const uint16_t*)weights, a.M, a.Cin,
