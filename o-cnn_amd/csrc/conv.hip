@@ -373,20 +373,44 @@ __device__ inline int b16_unit(int x, int y, int z) {
   return (x & 1) | ((y & 1) << 1) | ((z & 1) << 2) | ((y >> 1) << 3) | ((z >> 1) << 4);
 }
 
-template <typename T>
-__global__ void transpose_rows_kernel(T* __restrict__ dst, const T* __restrict__ src, int C, int H, int Cpad) {
-  // src [C, H] -> dst [H + 1, Cpad]; 64 x 64 tiles through LDS, both sides coalesced
-  __shared__ T tile[64][65];
-  const int h0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 256 threads: 4 rows per step
-  for (int i = ty; i < 64; i += 4) {
-    int c = c0 + i, h = h0 + tx;
-    tile[i][tx] = (c < C && h < H) ? src[(int64_t)c * H + h] : (T)0;
+// Row-major copy of a channel-major bf16 tensor: src [C, H] -> dst [H + 1, Cpad], row H zero.
+// 64 channels x 128 rows per workgroup; reads are 4-byte (two rows of one
+// channel) and coalesced per channel row, writes are 16-byte (8 channels of one row) and,
+// for Cpad = 64, contiguous over the whole tile.
+__global__ __launch_bounds__(256) void transpose_rows_bf16_kernel(uint16_t* __restrict__ dst,
+    const uint16_t* __restrict__ src, int C, int H, int Cpad) {
+  constexpr int kPitch = 130;  // halfwords; 8 channel rows apart = 8 banks apart
+  __shared__ __attribute__((aligned(16))) uint16_t tile[64 * kPitch];
+  const int h0 = blockIdx.x * 128, c0 = blockIdx.y * 64;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const bool even = (H & 1) == 0;
+#pragma unroll 4
+  for (int pass = 0; pass < 16; ++pass) {
+    const int cl = pass * 4 + wave, c = c0 + cl, h = h0 + 2 * lane;
+    uint32_t v = 0;
+    if (c < C) {
+      const uint16_t* p = src + (int64_t)c * H + h;
+      if (even && h + 1 < H) v = *reinterpret_cast<const uint32_t*>(p);
+      else {
+        if (h < H) v = p[0];
+        if (h + 1 < H) v |= (uint32_t)p[1] << 16;
+      }
+    }
+    *reinterpret_cast<uint32_t*>(&tile[cl * kPitch + 2 * lane]) = v;
   }
   __syncthreads();
-  for (int i = ty; i < 64; i += 4) {
-    int h = h0 + i, c = c0 + tx;
-    if (h <= H && c < Cpad) dst[(int64_t)h * Cpad + c] = h < H ? tile[tx][i] : (T)0;
+  const int cg = threadIdx.x & 7, hh = threadIdx.x >> 3;
+  if (c0 + cg * 8 >= Cpad) return;
+#pragma unroll
+  for (int pass = 0; pass < 4; ++pass) {
+    const int hl = pass * 32 + hh, h = h0 + hl;
+    if (h > H) continue;
+    uint32_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      w[j] = (uint32_t)tile[(cg * 8 + 2 * j) * kPitch + hl] | ((uint32_t)tile[(cg * 8 + 2 * j + 1) * kPitch + hl] << 16);
+    uint4 o = h < H ? make_uint4(w[0], w[1], w[2], w[3]) : make_uint4(0, 0, 0, 0);
+    *reinterpret_cast<uint4*>(dst + (int64_t)h * Cpad + c0 + cg * 8) = o;
   }
 }
 
@@ -1026,8 +1050,8 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
       int64_t total = (int64_t)npass * ksteps * kD2MT * 64 * 8;
       pack_weights_d2_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)wsb, (const uint16_t*)weights, rows, a.Cin, npass, ksteps);
       uint16_t* xt = reinterpret_cast<uint16_t*>(wsb + p.wt_bytes + p.ichild_bytes);
-      dim3 tgrid((a.Hin + 1 + 63) / 64, (cpad + 63) / 64);
-      transpose_rows_kernel<uint16_t><<<tgrid, 256, 0, s>>>(xt, (const uint16_t*)btm, a.Cin, a.Hin, cpad);
+      dim3 tgrid((a.Hin + 1 + 127) / 128, (cpad + 63) / 64);
+      transpose_rows_bf16_kernel<<<tgrid, 256, 0, s>>>(xt, (const uint16_t*)btm, a.Cin, a.Hin, cpad);
       deconv_s2_bf16_kernel<<<d_grid, 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles, cpad / 8);
     }
   } else if (dtype == OCNN_F32 && a.mode == kModeS1 && !a.nempty && a.K == 27) {
@@ -1060,8 +1084,8 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     pack_weights_lds_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)wsb, (const uint16_t*)weights, a.M, a.Cin,
         MT, npass, nslab, sm, sc, deconv);
     uint16_t* xt = reinterpret_cast<uint16_t*>(wsb + p.wt_bytes + p.ichild_bytes);
-    dim3 tgrid((a.Hin + 1 + 63) / 64, (cpad + 63) / 64);
-    transpose_rows_kernel<uint16_t><<<tgrid, 256, 0, s>>>(xt, (const uint16_t*)btm, a.Cin, a.Hin, cpad);
+    dim3 tgrid((a.Hin + 1 + 127) / 128, (cpad + 63) / 64);
+    transpose_rows_bf16_kernel<<<tgrid, 256, 0, s>>>(xt, (const uint16_t*)btm, a.Cin, a.Hin, cpad);
     OCNN_LAUNCH_OK("pack/transpose");
     // the kernel walks geometric offsets in natural order (the packer mirrored the weights)
     if (MT == 1)
