@@ -156,6 +156,15 @@ int ocnn_octree_deconv(void* top, const void* btm, int channel_in, int btm_h, co
     int stride, int nempty, int dtype, void* workspace_dev, size_t workspace_bytes,
     ocnn_stream_t stream);
 
+/* Convolution or deconvolution with the epilogue of the reference's conv -> BatchNorm -> ReLU
+ * modules (pytorch/ocnn/modules.py:23-36) folded in: `weights` already carry the BatchNorm
+ * scale, `bias` (device, fp32 [num_output], may be NULL) its shift; relu != 0 clamps at zero.
+ * Bias and ReLU act on the fp32 accumulator before the store. */
+int ocnn_octree_conv_fused(void* top, const void* btm, int channel_in, int btm_h, const void* weights,
+    const float* bias, int relu, int is_deconv, const void* octree_dev, const void* info, int depth,
+    int num_output, const int* kernel_size, int stride, int nempty, int dtype, void* workspace_dev,
+    size_t workspace_bytes, ocnn_stream_t stream);
+
 /* ---- octree construction on the device: points2octree + octree_batch fused.
  * Replaces Octree::build (octree/octree/octree.cpp:74-121) driven as in
  * pytorch/cpp/point2octree.cpp:5-34, and merge_octrees

@@ -7,9 +7,11 @@ The directory name is not a Python identifier; load the package with
                (pytorch/cpp/pybind.cpp:3-49) over libocnn_hip.so
   layers    -- mirror of the thin Python modules of pytorch/ocnn
                (octree_conv.py, octree_pool.py, octree_pad.py)
+  stacks    -- conv -> BatchNorm -> ReLU (folded) operator sequences of the benchmark
+               configurations (LeNet trunk, U-Net encoder / decoder)
   synthetic -- seeded synthetic point clouds of the benchmark configurations
 """
-from . import lib, nn, layers, synthetic  # noqa: F401
+from . import lib, nn, layers, stacks, synthetic  # noqa: F401
 from .nn import *  # noqa: F401,F403
 from .layers import (OctreeConv, OctreeDeconv, OctreeConvFast, OctreeDeconvFast,  # noqa: F401
                      OctreeMaxPool, OctreeMaxUnpool, OctreeAvgPool, OctreePad, OctreeDepad)

@@ -33,7 +33,16 @@ struct ConvArgs {
   const int* neigh;
   const int* child;
   const int* ichild;
+  const float* bias;    // optional per-output-channel bias (fp32), added before the store
+  int relu;             // optional max(., 0) before the store
 };
+
+// epilogue shared by every kernel: bias and ReLU are applied to the fp32 accumulator
+__device__ inline float finish(const ConvArgs& a, float v, int m) {
+  if (a.bias) v += a.bias[m];
+  if (a.relu) v = fmaxf(v, 0.0f);
+  return v;
+}
 
 constexpr int kWaveCols = 64;                 // output columns per wavefront
 constexpr int kConvWaves = 4;                 // wavefronts per workgroup
@@ -117,8 +126,9 @@ __device__ inline void store_tiles(const ConvArgs& a, OutT* __restrict__ out, fl
       for (int i = 0; i < 16; ++i) {
         int m = (mt0 + mt) * 32 + 8 * (i / 4) + 4 * kh + (i % 4);
         if (m < a.M) {
-          if (sizeof(OutT) == 4) reinterpret_cast<float*>(out)[(int64_t)m * a.Hout + n] = acc[mt][nt][i];
-          else reinterpret_cast<uint16_t*>(out)[(int64_t)m * a.Hout + n] = f32_to_bf16(acc[mt][nt][i]);
+          const float v = finish(a, acc[mt][nt][i], m);
+          if (sizeof(OutT) == 4) reinterpret_cast<float*>(out)[(int64_t)m * a.Hout + n] = v;
+          else reinterpret_cast<uint16_t*>(out)[(int64_t)m * a.Hout + n] = f32_to_bf16(v);
         }
       }
     }
@@ -739,13 +749,14 @@ __device__ inline void store_children(const ConvArgs& a, OutT* __restrict__ out,
     int co = (row0 >> 3) + q;
     if (co >= a.M) continue;
     int64_t o = (int64_t)co * a.Hout + (int64_t)n * 8 + 4 * kh;
+    const float v0 = finish(a, acc[4 * q], co), v1 = finish(a, acc[4 * q + 1], co);
+    const float v2 = finish(a, acc[4 * q + 2], co), v3 = finish(a, acc[4 * q + 3], co);
     if (sizeof(OutT) == 4) {
-      *reinterpret_cast<float4*>(reinterpret_cast<float*>(out) + o) =
-          make_float4(acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
+      *reinterpret_cast<float4*>(reinterpret_cast<float*>(out) + o) = make_float4(v0, v1, v2, v3);
     } else {
       uint2 v;
-      v.x = (uint32_t)f32_to_bf16(acc[4 * q]) | ((uint32_t)f32_to_bf16(acc[4 * q + 1]) << 16);
-      v.y = (uint32_t)f32_to_bf16(acc[4 * q + 2]) | ((uint32_t)f32_to_bf16(acc[4 * q + 3]) << 16);
+      v.x = (uint32_t)f32_to_bf16(v0) | ((uint32_t)f32_to_bf16(v1) << 16);
+      v.y = (uint32_t)f32_to_bf16(v2) | ((uint32_t)f32_to_bf16(v3) << 16);
       *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(out) + o) = v;
     }
   }
@@ -961,7 +972,8 @@ int make_plan(const Info* o, int depth, int channel_in, int num_output, const in
 
 int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, const void* weights,
     const void* octree_dev, const void* info, int depth, int num_output, const int* ks, int stride,
-    int nempty, int dtype, void* ws, size_t ws_bytes, hipStream_t s) {
+    int nempty, int dtype, void* ws, size_t ws_bytes, hipStream_t s, const float* bias = nullptr,
+    int relu = 0) {
   OCNN_REQUIRE(top && btm && weights && octree_dev && info, OCNN_E_BADARG, "null pointer");
   const Info* o = as_info(info);
   ConvPlan p;
@@ -994,6 +1006,8 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
   a.neigh = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_NEIGH, p.workspace_depth));
   a.child = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_CHILD, p.workspace_depth));
   a.ichild = nullptr;
+  a.bias = bias;
+  a.relu = relu ? 1 : 0;
   // degenerate layer without nodes: the reference emits one zero column
   // (octree_conv.cpp:82) -- nothing to gather
   bool empty_layer = (nempty ? o->nnum_nempty[p.top_depth] : (stride == 2 && !deconv
@@ -1139,6 +1153,14 @@ int ocnn_octree_deconv(void* top, const void* btm, int channel_in, int btm_h, co
     int nempty, int dtype, void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream) {
   return run_conv(1, top, btm, channel_in, btm_h, weights, octree_dev, info, depth, num_output, kernel_size,
       stride, nempty, dtype, workspace_dev, workspace_bytes, as_stream(stream));
+}
+
+int ocnn_octree_conv_fused(void* top, const void* btm, int channel_in, int btm_h, const void* weights,
+    const float* bias, int relu, int is_deconv, const void* octree_dev, const void* info, int depth,
+    int num_output, const int* kernel_size, int stride, int nempty, int dtype, void* workspace_dev,
+    size_t workspace_bytes, ocnn_stream_t stream) {
+  return run_conv(is_deconv ? 1 : 0, top, btm, channel_in, btm_h, weights, octree_dev, info, depth, num_output,
+      kernel_size, stride, nempty, dtype, workspace_dev, workspace_bytes, as_stream(stream), bias, relu);
 }
 
 }  // extern "C"

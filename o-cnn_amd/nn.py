@@ -24,6 +24,7 @@ from .lib import CHILD, FEATURE, KEY, LABEL, NEIGH, SPLIT, HEADER_BYTES, INFO_BY
 __all__ = [
     "points2octree", "points2octree_batch", "octree_batch", "octree_property",
     "octree_set_property", "octree2col", "col2octree", "octree_conv", "octree_deconv",
+    "octree_conv_fused",
     "octree_pad", "octree_depad", "octree_max_pool", "octree_max_unpool", "octree_mask_pool",
     "octree_encode_key", "octree_decode_key", "octree_xyz2key", "octree_key2xyz",
     "octree_search_key", "octree_new", "octree_grow", "octree_update", "points_new",
@@ -407,7 +408,8 @@ def col2octree(grad_in, octree, depth, kernel_size, stride, nempty):
 
 
 # ---- convolution -------------------------------------------------------------------------------
-def _conv(fn, is_deconv, data_in, weights, octree, depth, num_output, kernel_size, stride, nempty):
+def _conv(fn, is_deconv, data_in, weights, octree, depth, num_output, kernel_size, stride, nempty,
+          bias=None, relu=False):
   octree = _to_dev(octree)
   info = octree_info(octree)
   ksc, _ = _ks(kernel_size)
@@ -423,9 +425,18 @@ def _conv(fn, is_deconv, data_in, weights, octree, depth, num_output, kernel_siz
   ws = _workspace(ws_bytes.value + 256, "conv")
   base = (ws.data_ptr() + 255) & ~255
   out = torch.empty(1, num_output, top_h.value, 1, dtype=data_in.dtype, device=data_in.device)
-  _lib.call(fn, _ptr(out), _ptr(data_in), channel_in, btm_h, _ptr(weights), _ptr(octree), info.p,
-            depth, num_output, ksc, stride, int(nempty), dt, C.c_void_p(base),
-            C.c_size_t(ws_bytes.value), _stream())
+  if fn == "ocnn_octree_conv_fused":
+    if bias is not None:
+      bias = bias.to(torch.float32).contiguous()
+      if bias.numel() != num_output:
+        raise OcnnError(-3, "bias needs num_output entries")
+    _lib.call(fn, _ptr(out), _ptr(data_in), channel_in, btm_h, _ptr(weights), _ptr(bias), int(relu),
+              int(is_deconv), _ptr(octree), info.p, depth, num_output, ksc, stride, int(nempty), dt,
+              C.c_void_p(base), C.c_size_t(ws_bytes.value), _stream())
+  else:
+    _lib.call(fn, _ptr(out), _ptr(data_in), channel_in, btm_h, _ptr(weights), _ptr(octree), info.p,
+              depth, num_output, ksc, stride, int(nempty), dt, C.c_void_p(base),
+              C.c_size_t(ws_bytes.value), _stream())
   return out
 
 
@@ -439,6 +450,15 @@ def octree_deconv(data_in, weights, octree, depth, num_output, kernel_size, stri
   """pytorch/cpp/octree_conv.cpp:189-216: weights are [Ci, Co*K]."""
   return _conv("ocnn_octree_deconv", True, data_in, weights, octree, depth, num_output,
                kernel_size, stride, nempty)
+
+
+def octree_conv_fused(data_in, weights, bias, relu, octree, depth, num_output, kernel_size, stride,
+                      nempty, deconv=False):
+  """conv (or deconv) + per-channel bias + optional ReLU in one kernel: the inference form of
+  the reference's conv -> BatchNorm -> ReLU modules (pytorch/ocnn/modules.py:23-36) once the
+  BatchNorm statistics are folded into `weights` and `bias`."""
+  return _conv("ocnn_octree_conv_fused", deconv, data_in, weights, octree, depth, num_output,
+               kernel_size, stride, nempty, bias=bias, relu=relu)
 
 
 # ---- pad / pool ------------------------------------------------------------------------------------

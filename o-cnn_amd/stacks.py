@@ -1,0 +1,94 @@
+"""Operator sequences of the benchmark configurations, issued in the reference's order.
+
+The reference wraps every convolution as conv -> BatchNorm2d(eps = 1e-3) -> ReLU
+(`OctreeConvBnRelu`, pytorch/ocnn/modules.py:23-36).  At inference the BatchNorm is an
+affine map per output channel, so it folds into the weights and a bias; the fused kernel
+applies bias and ReLU to the accumulator before the store.
+
+  lenet_trunk  conv -> BN -> ReLU -> max_pool (+pad) per depth, as pytorch/ocnn/lenet.py:24-32
+  unet_trunk   encoder / decoder with 2x2x2 stride-2 down-convolutions and deconvolutions and
+               skip concatenations, the op order of pytorch/ocnn/unet.py:61-92 with one
+               convolution per stage
+"""
+import torch
+
+from . import nn as F
+
+BN_EPS = 1e-3  # pytorch/ocnn/modules.py:5
+
+
+def fold_bn(weights, gamma, beta, mean, var, eps=BN_EPS, deconv=False, kdim=None):
+  """(W', b') with  BN(conv(x, W)) == conv(x, W') + b'.
+  conv weights are [Cout, Cin*K]; deconv weights are [Cin, Cout*K] (column co*K + k)."""
+  scale = gamma / torch.sqrt(var + eps)
+  if not deconv:
+    w = weights * scale[:, None]
+  else:
+    cout = scale.numel()
+    w = (weights.view(weights.shape[0], cout, kdim) * scale[None, :, None]).reshape(weights.shape)
+  return w.contiguous(), (beta - mean * scale).contiguous()
+
+
+def conv_bn_relu(data, w, b, octree, depth, cout, kernel_size=(3, 3, 3), stride=1, nempty=False,
+                 deconv=False, relu=True):
+  """OctreeConvBnRelu / OctreeDeConvBnRelu with folded BatchNorm, including the pad / depad the
+  reference modules add around stride-2 layers (pytorch/ocnn/octree_conv.py:102-127)."""
+  ks = list(kernel_size)
+  if deconv and stride == 2 and not nempty:
+    data = F.octree_depad(data, octree, depth)
+  out = F.octree_conv_fused(data, w.to(data.dtype), b, relu, octree, depth, cout, ks, stride, nempty,
+                            deconv=deconv)
+  if (not deconv) and stride == 2 and not nempty:
+    # a padded (empty) node holds 0 in the reference because the pad comes after conv but
+    # before BatchNorm; after folding the empty nodes must receive relu(b) instead of 0:
+    # the reference order is conv -> pad -> BN -> ReLU.
+    padded = F.octree_pad(out, octree, depth - 1, 0.0)
+    child = F.octree_property(octree, "child", depth - 1)
+    fill = torch.relu(b) if relu else b
+    empty = (child < 0).view(1, 1, -1, 1)
+    out = torch.where(empty, fill.to(out.dtype).view(1, -1, 1, 1), padded)
+  return out
+
+
+def lenet_trunk(octree, depth, params, data=None, to_depth=2):
+  """params[d] = (w, b) for the conv at depth d (3x3x3, stride 1); returns the features at
+  `to_depth` after the last pool."""
+  if data is None:
+    data = F.octree_property(octree, "feature", depth)
+  for d in range(depth, to_depth, -1):
+    w, b = params[d]
+    data = conv_bn_relu(data, w, b, octree, d, w.shape[0])
+    pool, _ = F.octree_max_pool(data, octree, d)
+    data = F.octree_pad(pool, octree, d - 1)
+  return data
+
+
+def unet_trunk(octree, depth, params, data=None, stages=3, nempty=False):
+  """params: dict with keys ('conv', d), ('down', d), ('up', d), ('dec', d) -> (w, b).
+  Encoder: conv at `depth`, then per stage a 2x2x2 stride-2 conv to depth-1 and a 3x3x3 conv;
+  decoder: per stage a 2x2x2 stride-2 deconv to depth+1, concatenation with the encoder
+  feature of that depth, and a 3x3x3 conv."""
+  if data is None:
+    data = F.octree_property(octree, "feature", depth)
+    if nempty:
+      data = F.octree_depad(data, octree, depth)
+  feats = {}
+  w, b = params[("conv", depth)]
+  feats[depth] = conv_bn_relu(data, w, b, octree, depth, w.shape[0], nempty=nempty)
+  d = depth
+  for _ in range(stages):
+    w, b = params[("down", d)]
+    x = conv_bn_relu(feats[d], w, b, octree, d, w.shape[0], (2, 2, 2), 2, nempty)
+    d -= 1
+    w, b = params[("conv", d)]
+    feats[d] = conv_bn_relu(x, w, b, octree, d, w.shape[0], nempty=nempty)
+  x = feats[d]
+  for _ in range(stages):
+    w, b = params[("up", d)]
+    cout = w.shape[1] // 8
+    x = conv_bn_relu(x, w, b, octree, d, cout, (2, 2, 2), 2, nempty, deconv=True)
+    d += 1
+    x = torch.cat([feats[d], x], dim=1)
+    w, b = params[("dec", d)]
+    x = conv_bn_relu(x, w, b, octree, d, w.shape[0], nempty=nempty)
+  return x
