@@ -26,6 +26,12 @@ sys.path.insert(0, ROOT)
 PEAK_HBM_GBS = 8000.0
 PEAK_MFMA_TFLOPS = {"f32": 157.3, "bf16": 2500.0}
 
+# HBM bytes per launch of the headline kernel, from two `rocprofv3 --pmc` runs (FETCH_SIZE,
+# WRITE_SIZE) scaled by a 1-GiB device copy: see
+# profiles/conv_s1_f32_lds_kernel__scene_depth9__hbm_traffic.md.  Counters cannot be read from
+# inside this process, so the recorded figure is reported for the workload it was taken on.
+RECORDED_TRAFFIC = {("conv_s1_f32_lds_kernel", 1494168, 64, 64): 1.018e9}
+
 
 def main():
   ap = argparse.ArgumentParser()
@@ -34,6 +40,9 @@ def main():
   ap.add_argument("--warmup", type=int, default=3)
   ap.add_argument("--quick", action="store_true", help="skip the sub-measurements and the CPU baseline")
   ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+  ap.add_argument("--calib", action="store_true",
+                  help="also run a plain device copy of 1 GiB three times (the known-size kernel "
+                       "that scales the FETCH_SIZE / WRITE_SIZE counters of a --pmc run)")
   args = ap.parse_args()
   if args.gpus != 1:
     print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -81,6 +90,14 @@ def main():
   def conv_step():
     return F.octree_conv(x32, w32, octree, depth, C, [3, 3, 3], 1, False)
 
+  if args.calib:
+    src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+      dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+
   # ---- timed region of the headline metric -------------------------------------------------
   for _ in range(args.warmup):
     conv_step()
@@ -116,7 +133,8 @@ def main():
                  "octants_d9": H9, "octants_d8": H8, "nonempty_d9": Hne9, "points": 250000},
       "roofline": {"bound": "mfma", "achieved": achieved_tflops, "peak": PEAK_MFMA_TFLOPS["f32"],
                    "unit": "TFLOP/s", "frac": achieved_tflops / PEAK_MFMA_TFLOPS["f32"],
-                   "traffic": None, "kernel": "conv_f32_kernel",
+                   "traffic": RECORDED_TRAFFIC.get(("conv_s1_f32_lds_kernel", H9, C, C)),
+                   "kernel": "conv_s1_f32_lds_kernel<2,27>",
                    "algorithmic_flops_per_launch": flops},
       "wall_ms_per_step": wall_ms,
   }
@@ -203,6 +221,102 @@ def main():
     conv_case("conv333_s1_d7_f32", oct7, 7, x7, w32, [3, 3, 3], 1)
     conv_case("conv333_s1_d7_bf16", oct7, 7, x7.bfloat16(), w16, [3, 3, 3], 1)
     conv_case("conv222_s2_d7_f32", oct7, 7, x7, w2, [2, 2, 2], 2)
+    conv_case("conv222_s2_d7_bf16", oct7, 7, x7.bfloat16(), w2.bfloat16(), [2, 2, 2], 2)
+    conv_case("deconv222_s2_d8to9_bf16", octree, 8, x8.bfloat16(), w2.bfloat16(), [2, 2, 2], 2, deconv=True)
+    conv_case("deconv333_s1_d9_f32", octree, 9, x32, w32, [3, 3, 3], 1, deconv=True)
+
+    def hbm(name, t, by):
+      extra[name] = {"ms": t, "GBs": by / t / 1e6, "frac_hbm_peak": by / t / 1e6 / PEAK_HBM_GBS}
+
+    # remaining streaming ops of the path on the depth-9 scene
+    pd8 = F.octree_pad(top, octree, 8)
+    hbm("depad_d8_f32", timed(lambda: F.octree_depad(pd8, octree, 8), reps, wu), C * (Hne8 + H8) * s + H8 * 4)
+    hbm("mask_pool_d9_f32", timed(lambda: F.octree_mask_pool(x32, mask, octree, 9), reps, wu),
+        C * (H9 // 8) * (2 * s + 4))
+    hbm("max_pool_d9_bf16", timed(lambda: F.octree_max_pool(x16, octree, 9), reps, wu),
+        C * H9 * 2 + C * (H9 // 8) * (2 + 4))
+    c8 = 8
+    xc = x32[:, :c8].contiguous()
+    col = F.octree2col(xc, octree, 9, [3, 3, 3], 1, False)
+    by = c8 * H9 * s + H9 * 8 * 4 + c8 * 27 * H9 * s
+    hbm("octree2col_333_d9_c8_f32", timed(lambda: F.octree2col(xc, octree, 9, [3, 3, 3], 1, False), reps, wu), by)
+    hbm("col2octree_333_d9_c8_f32", timed(lambda: F.col2octree(col, octree, 9, [3, 3, 3], 1, False), reps, wu), by)
+    del col
+    # integer kernels
+    key9 = F.octree_property(octree, "key", 9)
+    hbm("xyz2key_d9", timed(lambda: F.octree_xyz2key(key9, 9), reps, wu), H9 * 16)
+    q = key9[torch.randint(0, H9, (1 << 20,), generator=g).to(dev)]
+    hbm("search_key_d9_1Mq", timed(lambda: F.octree_search_key(q, octree, 9, False, False), reps, wu),
+        (1 << 20) * 12)
+    lab = (child8 >= 0).to(torch.int32)
+    P = lambda t_: Ct.c_void_p(t_.data_ptr())
+    lab_out = torch.empty_like(lab)
+    cnt = torch.zeros(1, dtype=torch.int32, device=dev)
+    sb = oc.lib.get().ocnn_generate_label_scratch_bytes(H8)
+    scratch = torch.empty(sb, dtype=torch.uint8, device=dev)
+    hbm("generate_label_d8", timed(lambda: oc.lib.call("ocnn_generate_label", P(lab_out), P(cnt), P(lab), H8, 1,
+                                                          P(scratch), Ct.c_size_t(sb), st()), reps, wu), H8 * 8)
+    # decoder-side growth: octree_update(depth 8) + octree_grow(to depth 9) of the depth-8 prefix
+    oct8 = F.octree_new(1, 4, False)
+    for d in range(1, 3):
+      oct8 = F.octree_grow(oct8, d, True)
+    for d in range(2, 9):
+      labd = (F.octree_property(octree, "child", d) >= 0).to(torch.int32)
+      oct8 = F.octree_update(oct8, labd, d, 1)
+      if d < 8:
+        oct8 = F.octree_grow(oct8, d + 1, False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+      grown = F.octree_grow(F.octree_update(oct8, lab, 8, 1), 9, False)
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / reps
+    extra["octree_update_d8_plus_grow_d9"] = {
+        "ms": t * 1e3, "new_nodes": F.octree_info(grown).nnum(9),
+        "GBs": (H9 * (8 + 4 + 32) + H8 * (4 + 4 + 32 + 8)) / t / 1e9}
+    # merge of 16 separately built, serialized octrees (octree_batch on device blobs)
+    singles = [F.points2octree(c, 7, 2) for c in cl]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+      F.octree_batch(singles)
+    torch.cuda.synchronize()
+    extra["octree_batch_16_blobs_d7"] = {"ms": (time.perf_counter() - t0) / reps * 1e3,
+                                         "nodes": int(sum(i7.nnum(d) for d in range(8)))}
+
+    # operator sequences with folded BatchNorm (conv + bias + ReLU fused)
+    def rand_params(spec):
+      prm = {}
+      for key, shape in spec.items():
+        cout = shape[1] // 8 if key[0] == "up" else shape[0]
+        fan = shape[0] if key[0] == "up" else shape[1]
+        prm[key] = ((torch.randn(*shape, generator=g) / fan ** 0.5).to(dev),
+                    (torch.randn(cout, generator=g) * 0.1).to(dev))
+      return prm
+
+    ch = {9: 32, 8: 64, 7: 128, 6: 256}
+    spec = {("conv", 9): (32, 6 * 27)}
+    for d in (9, 8, 7):
+      spec[("down", d)] = (ch[d - 1], ch[d] * 8)
+      spec[("conv", d - 1)] = (ch[d - 1], ch[d - 1] * 27)
+    for d in (6, 7, 8):
+      spec[("up", d)] = (ch[d], ch[d + 1] * 8)
+      spec[("dec", d + 1)] = (ch[d + 1], 2 * ch[d + 1] * 27)
+    up = rand_params(spec)
+    feat9 = F.octree_property(octree, "feature", 9)
+    t = timed(lambda: oc.stacks.unet_trunk(octree, 9, up, data=feat9), max(2, reps // 2), 1)
+    extra["unet_trunk_scene_d9_f32"] = {"ms": t, "points_per_s": 250000 / (t * 1e-3)}
+    up16 = {k: (w.bfloat16(), b) for k, (w, b) in up.items()}
+    f16 = feat9.bfloat16()
+    t = timed(lambda: oc.stacks.unet_trunk(octree, 9, up16, data=f16), max(2, reps // 2), 1)
+    extra["unet_trunk_scene_d9_bf16"] = {"ms": t, "points_per_s": 250000 / (t * 1e-3)}
+    clouds2 = [points_tensor(*oc.synthetic.shape_cloud(10000, 100 + i)) for i in range(32)]
+    oct6 = F.points2octree_batch(clouds2, 6, 2)
+    lch = {6: (3, 32), 5: (32, 64), 4: (64, 128), 3: (128, 256)}
+    lp = {d: ((torch.randn(co, ci * 27, generator=g) / (ci * 27) ** 0.5).to(dev),
+              (torch.randn(co, generator=g) * 0.1).to(dev)) for d, (ci, co) in lch.items()}
+    t = timed(lambda: oc.stacks.lenet_trunk(oct6, 6, lp), reps, wu)
+    extra["lenet_trunk_batch32_d6_f32"] = {"ms": t, "shapes_per_s": 32 / (t * 1e-3)}
   out["extra"] = extra
 
   # ---- CPU baseline (reported, not the target) -----------------------------------------------
