@@ -75,40 +75,6 @@ __device__ inline int xcd_tile(int bid, int n_tiles) {
   return (bid % kXcd) * per + bid / kXcd;
 }
 
-// ---- weight re-layout ----------------------------------------------------------
-// W'(m, c, k) = W[m*sm + c*sc + k]; conv: sm = Cin*K, sc = K; deconv: sm = K, sc = M*K.
-// fp32 fragment (tap, cstep, mtile): lane l holds A[m = 32*mtile + (l&31)][c = 2*cstep + (l>>5)].
-__global__ void pack_weights_f32(float* __restrict__ Wt, const float* __restrict__ W, int M, int Cin, int K,
-    int mtiles, int csteps, int64_t sm, int64_t sc) {
-  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  int64_t total = (int64_t)K * csteps * mtiles * 64;
-  if (id >= total) return;
-  int l = (int)(id & 63);
-  int64_t f = id >> 6;
-  int mt = (int)(f % mtiles);
-  f /= mtiles;
-  int cs = (int)(f % csteps);
-  int k = (int)(f / csteps);
-  int m = mt * 32 + (l & 31), c = 2 * cs + (l >> 5);
-  Wt[id] = (m < M && c < Cin) ? W[m * sm + c * sc + k] : 0.0f;
-}
-// bf16 fragment: lane l holds A[m = 32*mtile + (l&31)][c = 16*cstep + 8*(l>>5) + j], j = 0..7
-__global__ void pack_weights_bf16(uint16_t* __restrict__ Wt, const uint16_t* __restrict__ W, int M, int Cin,
-    int K, int mtiles, int csteps, int64_t sm, int64_t sc) {
-  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  int64_t total = (int64_t)K * csteps * mtiles * 64 * 8;
-  if (id >= total) return;
-  int j = (int)(id & 7);
-  int l = (int)((id >> 3) & 63);
-  int64_t f = id >> 9;
-  int mt = (int)(f % mtiles);
-  f /= mtiles;
-  int cs = (int)(f % csteps);
-  int k = (int)(f / csteps);
-  int m = mt * 32 + (l & 31), c = 16 * cs + 8 * (l >> 5) + j;
-  Wt[id] = (m < M && c < Cin) ? W[m * sm + c * sc + k] : (uint16_t)0;
-}
-
 // ---- main kernels ----------------------------------------------------------------
 // Accumulator layout of the 32x32 MFMA: lane l, register i holds
 // D[row = 8*(i/4) + 4*(l>>5) + (i%4)][col = l&31].
@@ -134,17 +100,55 @@ __device__ inline void store_tiles(const ConvArgs& a, OutT* __restrict__ out, fl
     }
 }
 
+// ---- general gather kernel over a row-major copy of the input -------------------------------
+// Every case without a dedicated kernel (non-empty-node convolutions, the small kernel shapes,
+// stride-2 cases other than 2x2x2 over all nodes) runs here.  The input is first copied
+// row-major ([H + 1, Cpad], row H zero = missing neighbour), so that the source row of a column
+// is contiguous over channels and one 16-byte load per lane brings 4 (fp32) or 8 (bf16) input
+// channels: 4x / 8x fewer gather instructions than per-channel gathers from the channel-major
+// tensor, which is what bounds this kernel.  Lane (n, kh) loads channels 4kh..4kh+3 of an
+// 8-channel group and the four values feed four MFMA k-steps with k-pairs (j, 4+j).
+// Loop nest: pass over 32*MT output rows -> tap -> 64-channel slab (its weights staged in LDS
+// in A-fragment order, next slab prefetched) -> 8-channel group.
+constexpr int kRowSlab = 64;
+
+__global__ __launch_bounds__(256) void transpose_rows_f32_kernel(float* __restrict__ dst,
+    const float* __restrict__ src, int C, int H, int Cpad) {
+  __shared__ float tile[64][65];
+  const int h0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    int c = c0 + i, h = h0 + tx;
+    tile[i][tx] = (c < C && h < H) ? src[(int64_t)c * H + h] : 0.0f;
+  }
+  __syncthreads();
+  const int cq = threadIdx.x & 15, hh = threadIdx.x >> 4;  // 16 lanes x float4 = one 64-channel row
+  if (c0 + cq * 4 >= Cpad) return;
+  for (int i = hh; i < 64; i += 16) {
+    int h = h0 + i;
+    if (h > H) continue;
+    float4 v = h < H ? make_float4(tile[cq * 4][i], tile[cq * 4 + 1][i], tile[cq * 4 + 2][i], tile[cq * 4 + 3][i])
+                     : make_float4(0.f, 0.f, 0.f, 0.f);
+    *reinterpret_cast<float4*>(dst + (int64_t)h * Cpad + c0 + cq * 4) = v;
+  }
+}
+
 template <int MT>
-__global__ __launch_bounds__(kConvWaves * 64) void conv_f32_kernel(ConvArgs a, float* __restrict__ out,
-    const float* __restrict__ in, const float* __restrict__ Wt, int n_tiles) {
+__global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* __restrict__ out,
+    const float4* __restrict__ xt, const float* __restrict__ Wt, int n_tiles, int cpad) {
+  constexpr int kWWords = (kRowSlab / 8) * 4 * MT * 64;  // weights of one (tap, slab)
+  constexpr int kWVec = kWWords / 4 / 256;               // float4 per thread (4 for MT = 2)
+  __shared__ __attribute__((aligned(16))) float sW[kWWords];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int tile = xcd_tile(blockIdx.x, n_tiles);
   if (tile >= n_tiles) return;
   const int n0 = tile * kTileCols + wave * kWaveCols;
-  if (n0 >= a.N) return;
   const int r = lane & 31, kh = lane >> 5;
-
-  for (int mt0 = 0; mt0 < a.mtiles; mt0 += MT) {
+  const int nslab = (cpad + kRowSlab - 1) / kRowSlab;
+  const int npass = (a.mtiles + MT - 1) / MT;
+  const int cpad4 = cpad >> 2;
+  const int nstage = a.K * nslab;
+  for (int pass = 0; pass < npass; ++pass) {
     floatx16 acc[MT][2];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -152,39 +156,80 @@ __global__ __launch_bounds__(kConvWaves * 64) void conv_f32_kernel(ConvArgs a, f
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
-
-    for (int k = 0; k < a.K; ++k) {
-      const int s0 = conv_src(a, n0 + r, k), s1 = conv_src(a, n0 + 32 + r, k);
-      const float* wk = Wt + ((int64_t)k * a.csteps * a.mtiles + mt0) * 64 + lane;
-#pragma unroll 4
-      for (int cs = 0; cs < a.csteps; ++cs) {
-        const int c = 2 * cs + kh;
-        const bool cv = c < a.Cin;
-        float b0 = (cv && s0 >= 0) ? in[(int64_t)c * a.Hin + s0] : 0.0f;
-        float b1 = (cv && s1 >= 0) ? in[(int64_t)c * a.Hin + s1] : 0.0f;
+    float4 wr[kWVec > 0 ? kWVec : 1];
+    auto fetch_w = [&](int stage) {
+      const float4* wsrc = reinterpret_cast<const float4*>(Wt + ((int64_t)pass * nstage + stage) * kWWords);
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          float av = (mt0 + mt < a.mtiles) ? wk[((int64_t)cs * a.mtiles + mt) * 64] : 0.0f;
-          acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b0, acc[mt][0], 0, 0, 0);
-          acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b1, acc[mt][1], 0, 0, 0);
+      for (int v = 0; v < kWVec; ++v) wr[v] = wsrc[v * 256 + threadIdx.x];
+    };
+    fetch_w(0);
+    int stage = 0;
+    for (int k = 0; k < a.K; ++k) {
+      int s0 = conv_src(a, n0 + r, k), s1 = conv_src(a, n0 + 32 + r, k);
+      if (s0 < 0) s0 = a.Hin;
+      if (s1 < 0) s1 = a.Hin;
+      const float4* row0 = xt + (int64_t)s0 * cpad4 + kh;
+      const float4* row1 = xt + (int64_t)s1 * cpad4 + kh;
+      for (int slab = 0; slab < nslab; ++slab, ++stage) {
+        __syncthreads();
+#pragma unroll
+        for (int v = 0; v < kWVec; ++v) reinterpret_cast<float4*>(sW)[v * 256 + threadIdx.x] = wr[v];
+        __syncthreads();
+        if (stage + 1 < nstage) fetch_w(stage + 1);
+        const int ngroup = min(kRowSlab, cpad - slab * kRowSlab) >> 3;
+        for (int c8 = 0; c8 < ngroup; ++c8) {
+          const float4 b0 = row0[(slab * kRowSlab + c8 * 8) >> 2];
+          const float4 b1 = row1[(slab * kRowSlab + c8 * 8) >> 2];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float v0 = j == 0 ? b0.x : j == 1 ? b0.y : j == 2 ? b0.z : b0.w;
+            const float v1 = j == 0 ? b1.x : j == 1 ? b1.y : j == 2 ? b1.z : b1.w;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+              const float av = sW[((c8 * 4 + j) * MT + mt) * 64 + lane];
+              acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, v0, acc[mt][0], 0, 0, 0);
+              acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, v1, acc[mt][1], 0, 0, 0);
+            }
+          }
         }
       }
     }
-    store_tiles<float, MT>(a, out, acc, mt0, n0, lane);
+    if (n0 < a.N) store_tiles<float, MT>(a, out, acc, pass * MT, n0, lane);
   }
+}
+// [pass][tap][slab][c8][j][mt][lane]: lane (m, kh) <- W'(m, slab*64 + c8*8 + 4kh + j, tap)
+__global__ void pack_weights_rows_f32(float* __restrict__ Wt, const float* __restrict__ W, int M, int Cin, int K,
+    int MT, int npass, int nslab, int64_t sm, int64_t sc) {
+  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t total = (int64_t)npass * K * nslab * (kRowSlab / 8) * 4 * MT * 64;
+  if (id >= total) return;
+  int l = (int)(id & 63);
+  int64_t f = id >> 6;
+  int mt = (int)(f % MT); f /= MT;
+  int j = (int)(f % 4); f /= 4;
+  int c8 = (int)(f % (kRowSlab / 8)); f /= (kRowSlab / 8);
+  int slab = (int)(f % nslab); f /= nslab;
+  int k = (int)(f % K);
+  int pass = (int)(f / K);
+  int m = (pass * MT + mt) * 32 + (l & 31), c = slab * kRowSlab + c8 * 8 + 4 * (l >> 5) + j;
+  Wt[id] = (m < M && c < Cin) ? W[m * sm + c * sc + k] : 0.0f;
 }
 
 template <int MT>
-__global__ __launch_bounds__(kConvWaves * 64) void conv_bf16_kernel(ConvArgs a, uint16_t* __restrict__ out,
-    const uint16_t* __restrict__ in, const uint16_t* __restrict__ Wt, int n_tiles) {
+__global__ __launch_bounds__(256) void conv_rows_bf16_kernel(ConvArgs a, uint16_t* __restrict__ out,
+    const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles, int cpad) {
+  constexpr int kWUnits = (kRowSlab / 16) * MT * 64;  // 16-byte units of one (tap, slab)
+  __shared__ u32x4 sW[kWUnits];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int tile = xcd_tile(blockIdx.x, n_tiles);
   if (tile >= n_tiles) return;
   const int n0 = tile * kTileCols + wave * kWaveCols;
-  if (n0 >= a.N) return;
   const int r = lane & 31, kh = lane >> 5;
-
-  for (int mt0 = 0; mt0 < a.mtiles; mt0 += MT) {
+  const int nslab = (cpad + kRowSlab - 1) / kRowSlab;
+  const int npass = (a.mtiles + MT - 1) / MT;
+  const int cpad8 = cpad >> 3;
+  const int nstage = a.K * nslab;
+  for (int pass = 0; pass < npass; ++pass) {
     floatx16 acc[MT][2];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -192,33 +237,67 @@ __global__ __launch_bounds__(kConvWaves * 64) void conv_bf16_kernel(ConvArgs a, 
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
-
+    u32x4 wr[2];
+    auto fetch_w = [&](int stage) {
+      const u32x4* wsrc = Wt + ((int64_t)pass * nstage + stage) * kWUnits;
+#pragma unroll
+      for (int v = 0; v < 2; ++v) {
+        int idx = v * 256 + threadIdx.x;
+        wr[v] = idx < kWUnits ? wsrc[idx] : (u32x4)(0u);
+      }
+    };
+    fetch_w(0);
+    int stage = 0;
     for (int k = 0; k < a.K; ++k) {
-      const int s0 = conv_src(a, n0 + r, k), s1 = conv_src(a, n0 + 32 + r, k);
-      const uint4* wk = reinterpret_cast<const uint4*>(Wt) + ((int64_t)k * a.csteps * a.mtiles + mt0) * 64 + lane;
-      for (int cs = 0; cs < a.csteps; ++cs) {
-        const int cb = 16 * cs + 8 * kh;
-        union { uint16_t u[8]; bf16x8 v; } b0, b1;
+      int s0 = conv_src(a, n0 + r, k), s1 = conv_src(a, n0 + 32 + r, k);
+      if (s0 < 0) s0 = a.Hin;
+      if (s1 < 0) s1 = a.Hin;
+      const u32x4* row0 = xt + (int64_t)s0 * cpad8 + kh;
+      const u32x4* row1 = xt + (int64_t)s1 * cpad8 + kh;
+      for (int slab = 0; slab < nslab; ++slab, ++stage) {
+        __syncthreads();
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int c = cb + j;
-          const bool cv = c < a.Cin;
-          b0.u[j] = (cv && s0 >= 0) ? in[(int64_t)c * a.Hin + s0] : (uint16_t)0;
-          b1.u[j] = (cv && s1 >= 0) ? in[(int64_t)c * a.Hin + s1] : (uint16_t)0;
+        for (int v = 0; v < 2; ++v) {
+          int idx = v * 256 + threadIdx.x;
+          if (idx < kWUnits) sW[idx] = wr[v];
         }
+        __syncthreads();
+        if (stage + 1 < nstage) fetch_w(stage + 1);
+        const int ngroup = min(kRowSlab, cpad - slab * kRowSlab) >> 4;
+        for (int c16 = 0; c16 < ngroup; ++c16) {
+          union { u32x4 q; bf16x8 v; } b0, b1;
+          b0.q = row0[(slab * kRowSlab + c16 * 16) >> 3];
+          b1.q = row1[(slab * kRowSlab + c16 * 16) >> 3];
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          union { uint4 q; bf16x8 v; } av;
-          av.q = (mt0 + mt < a.mtiles) ? wk[((int64_t)cs * a.mtiles + mt) * 64] : make_uint4(0, 0, 0, 0);
-          acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b0.v, acc[mt][0], 0, 0, 0);
-          acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b1.v, acc[mt][1], 0, 0, 0);
+          for (int mt = 0; mt < MT; ++mt) {
+            union { u32x4 q; bf16x8 v; } av;
+            av.q = sW[(c16 * MT + mt) * 64 + lane];
+            acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b0.v, acc[mt][0], 0, 0, 0);
+            acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b1.v, acc[mt][1], 0, 0, 0);
+          }
         }
       }
     }
-    store_tiles<uint16_t, MT>(a, out, acc, mt0, n0, lane);
+    if (n0 < a.N) store_tiles<uint16_t, MT>(a, out, acc, pass * MT, n0, lane);
   }
 }
-
+// [pass][tap][slab][c16][mt][lane][j]: lane (m, kh), j <- W'(m, slab*64 + c16*16 + 8kh + j, tap)
+__global__ void pack_weights_rows_bf16(uint16_t* __restrict__ Wt, const uint16_t* __restrict__ W, int M, int Cin,
+    int K, int MT, int npass, int nslab, int64_t sm, int64_t sc) {
+  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t total = (int64_t)npass * K * nslab * (kRowSlab / 16) * MT * 64 * 8;
+  if (id >= total) return;
+  int j = (int)(id & 7);
+  int l = (int)((id >> 3) & 63);
+  int64_t f = id >> 9;
+  int mt = (int)(f % MT); f /= MT;
+  int c16 = (int)(f % (kRowSlab / 16)); f /= (kRowSlab / 16);
+  int slab = (int)(f % nslab); f /= nslab;
+  int k = (int)(f % K);
+  int pass = (int)(f / K);
+  int m = (pass * MT + mt) * 32 + (l & 31), c = slab * kRowSlab + c16 * 16 + 8 * (l >> 5) + j;
+  Wt[id] = (m < M && c < Cin) ? W[m * sm + c * sc + k] : (uint16_t)0;
+}
 
 // ---- LDS-staged kernel for stride-1 convolutions over all nodes -----------------------
 // The eight siblings of a group read their taps from ONE 4x4x4 block of neighbour slots,
@@ -889,7 +968,7 @@ struct ConvPlan {
   int mode;
   KernelTaps taps;
   int mtiles, csteps;
-  size_t wt_bytes, ichild_bytes, xt_bytes, total_bytes;
+  size_t wt_bytes, ichild_bytes, xt_bytes, xt_general, total_bytes;
 };
 
 inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -935,9 +1014,15 @@ int make_plan(const Info* o, int depth, int channel_in, int num_output, const in
     p->mode = kModeS2Deconv;
   }
   p->mtiles = (num_output + 31) / 32;
-  p->csteps = dtype == OCNN_F32 ? (channel_in + 1) / 2 : (channel_in + 15) / 16;
-  size_t frag = dtype == OCNN_F32 ? 64 * sizeof(float) : 64 * 8 * sizeof(uint16_t);
-  p->wt_bytes = align256((size_t)p->taps.count * p->csteps * p->mtiles * frag);
+  p->csteps = 0;
+  {  // general row-major gather path: padded weights + the row-major copy of the input
+    size_t cpad = dtype == OCNN_F32 ? ((size_t)channel_in + 7) / 8 * 8 : ((size_t)channel_in + 15) / 16 * 16;
+    size_t nslab = (cpad + kRowSlab - 1) / kRowSlab, npass = (size_t)(p->mtiles + 1) / 2;
+    size_t per_stage = dtype == OCNN_F32 ? (kRowSlab / 8) * 4 * 2 * 64 * sizeof(float)
+                                         : (kRowSlab / 16) * 2 * 64 * 8 * sizeof(uint16_t);
+    p->wt_bytes = align256(npass * p->taps.count * nslab * per_stage);
+    p->xt_general = align256(((size_t)p->btm_h + 1) * cpad * (dtype == OCNN_F32 ? 4 : 2));
+  }
   if (dtype == OCNN_F32) {  // the LDS kernel pads channels to slabs of 4 and row tiles to passes
     size_t lds_words = (size_t)((p->mtiles + 1) / 2) * ((channel_in + kSlab - 1) / kSlab) * p->taps.count * 2 * 2 * 64;
     p->wt_bytes = align256(lds_words * sizeof(float) > p->wt_bytes ? lds_words * sizeof(float) : p->wt_bytes);
@@ -966,6 +1051,7 @@ int make_plan(const Info* o, int depth, int channel_in, int num_output, const in
     if (w > p->wt_bytes) p->wt_bytes = align256(w);
     p->xt_bytes = align256(((size_t)p->btm_h + 1) * cpad * sizeof(uint16_t));
   }
+  if (p->xt_general > p->xt_bytes) p->xt_bytes = p->xt_general;  // one buffer serves whichever path runs
   p->total_bytes = p->wt_bytes + p->ichild_bytes + p->xt_bytes;
   return OCNN_OK;
 }
@@ -1080,16 +1166,21 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     else
       conv_s1_f32_lds_kernel<2, 27><<<grid, 256, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
   } else if (dtype == OCNN_F32) {
-    int64_t total = (int64_t)a.K * a.csteps * a.mtiles * 64;
-    pack_weights_f32<<<blocks_for(total), kBlock, 0, s>>>((float*)wsb, (const float*)weights, a.M, a.Cin, a.K,
-        a.mtiles, a.csteps, sm, sc);
-    OCNN_LAUNCH_OK("pack_weights");
-    if (a.mtiles == 1)
-      conv_f32_kernel<1><<<grid, kConvWaves * 64, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
-    else if (a.mtiles <= 2 || a.mtiles % 4 != 0)
-      conv_f32_kernel<2><<<grid, kConvWaves * 64, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
+    const int MT = a.mtiles == 1 ? 1 : 2;
+    const int cpad = (a.Cin + 7) / 8 * 8;
+    const int npass = (a.mtiles + MT - 1) / MT, nslab = (cpad + kRowSlab - 1) / kRowSlab;
+    int64_t total = (int64_t)npass * a.K * nslab * (kRowSlab / 8) * 4 * MT * 64;
+    pack_weights_rows_f32<<<blocks_for(total), kBlock, 0, s>>>((float*)wsb, (const float*)weights, a.M, a.Cin, a.K,
+        MT, npass, nslab, sm, sc);
+    OCNN_LAUNCH_OK("pack_weights_rows");
+    float* xt = (float*)(wsb + p.wt_bytes + p.ichild_bytes);
+    dim3 tg((a.Hin + 64) / 64, (cpad + 63) / 64);
+    transpose_rows_f32_kernel<<<tg, 256, 0, s>>>(xt, (const float*)btm, a.Cin, a.Hin, cpad);
+    OCNN_LAUNCH_OK("transpose_rows");
+    if (MT == 1)
+      conv_rows_f32_kernel<1><<<grid, 256, 0, s>>>(a, (float*)top, (const float4*)xt, (const float*)wsb, n_tiles, cpad);
     else
-      conv_f32_kernel<4><<<grid, kConvWaves * 64, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
+      conv_rows_f32_kernel<2><<<grid, 256, 0, s>>>(a, (float*)top, (const float4*)xt, (const float*)wsb, n_tiles, cpad);
   } else if (a.mode == kModeS1 && !a.nempty && a.K == 27) {
     const int MT = a.mtiles == 1 ? 1 : 2;
     const int cpad = (a.Cin + 15) / 16 * 16;
@@ -1107,16 +1198,21 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     else
       conv_s1_bf16_lds_kernel<2><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad / 8);
   } else {
-    int64_t total = (int64_t)a.K * a.csteps * a.mtiles * 64 * 8;
-    pack_weights_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)wsb, (const uint16_t*)weights, a.M, a.Cin,
-        a.K, a.mtiles, a.csteps, sm, sc);
-    OCNN_LAUNCH_OK("pack_weights");
-    if (a.mtiles == 1)
-      conv_bf16_kernel<1><<<grid, kConvWaves * 64, 0, s>>>(a, (uint16_t*)top, (const uint16_t*)btm, (const uint16_t*)wsb, n_tiles);
-    else if (a.mtiles <= 2 || a.mtiles % 4 != 0)
-      conv_bf16_kernel<2><<<grid, kConvWaves * 64, 0, s>>>(a, (uint16_t*)top, (const uint16_t*)btm, (const uint16_t*)wsb, n_tiles);
+    const int MT = a.mtiles == 1 ? 1 : 2;
+    const int cpad = (a.Cin + 15) / 16 * 16;
+    const int npass = (a.mtiles + MT - 1) / MT, nslab = (cpad + kRowSlab - 1) / kRowSlab;
+    int64_t total = (int64_t)npass * a.K * nslab * (kRowSlab / 16) * MT * 64 * 8;
+    pack_weights_rows_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)wsb, (const uint16_t*)weights, a.M,
+        a.Cin, a.K, MT, npass, nslab, sm, sc);
+    OCNN_LAUNCH_OK("pack_weights_rows");
+    uint16_t* xt = (uint16_t*)(wsb + p.wt_bytes + p.ichild_bytes);
+    dim3 tg((a.Hin + 1 + 127) / 128, (cpad + 63) / 64);
+    transpose_rows_bf16_kernel<<<tg, 256, 0, s>>>(xt, (const uint16_t*)btm, a.Cin, a.Hin, cpad);
+    OCNN_LAUNCH_OK("transpose_rows");
+    if (MT == 1)
+      conv_rows_bf16_kernel<1><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
     else
-      conv_bf16_kernel<4><<<grid, kConvWaves * 64, 0, s>>>(a, (uint16_t*)top, (const uint16_t*)btm, (const uint16_t*)wsb, n_tiles);
+      conv_rows_bf16_kernel<2><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
   }
   OCNN_LAUNCH_OK("octree_conv");
   return OCNN_OK;

@@ -42,8 +42,8 @@ namespace {
 // ---- neighbour tables --------------------------------------------------------
 // Sparse-layer neighbour table.  A workgroup takes 256 consecutive parent-level nodes,
 // compacts the non-empty ones into LDS (most nodes of a deep level are empty) and then
-// every wavefront writes the 64-slot blocks of the compacted nodes, two nodes per
-// iteration so that two dependent load chains (neigh -> children) are in flight.
+// every wavefront writes the 64-slot blocks of the compacted nodes, four nodes per
+// iteration so that four dependent load chains (neigh -> children) are in flight.
 __global__ void calc_neigh_sparse_kernel(int* __restrict__ neigh_child, const int* __restrict__ neigh,
     const int* __restrict__ children, int node_num) {
   __shared__ int s_node[kBlock], s_rank[kBlock], s_count;
@@ -59,10 +59,10 @@ __global__ void calc_neigh_sparse_kernel(int* __restrict__ neigh_child, const in
   const int x = lane >> 4, y = (lane >> 2) & 3, z = lane & 3;
   const int hx = (x + 1) >> 1, hy = (y + 1) >> 1, hz = (z + 1) >> 1;
   const int octant = (((x + 1) & 1) << 2) | (((y + 1) & 1) << 1) | ((z + 1) & 1);
-  for (int e = wave * 2; e < count; e += 2 * (kBlock / 64)) {
-    int t[2], rank[2];
+  for (int e = wave * 4; e < count; e += 4 * (kBlock / 64)) {
+    int t[4], rank[4];
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int u = 0; u < 4; ++u) {
       t[u] = -1;
       rank[u] = -1;
       if (e + u < count) {
@@ -74,7 +74,7 @@ __global__ void calc_neigh_sparse_kernel(int* __restrict__ neigh_child, const in
       }
     }
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int u = 0; u < 4; ++u) {
       int v = -1;
       if (t[u] >= 0) {
         const int l1 = children[t[u]];
