@@ -92,3 +92,43 @@ def unet_trunk(octree, depth, params, data=None, stages=3, nempty=False):
     w, b = params[("dec", d)]
     x = conv_bn_relu(x, w, b, octree, d, w.shape[0], nempty=nempty)
   return x
+
+
+def create_full_octree(depth, channel, batch_size=1, node_dis=True):
+  """pytorch/ocnn/modules.py:325-330."""
+  octree = F.octree_new(batch_size, channel, node_dis)
+  for target_depth in range(1, depth + 1):
+    octree = F.octree_grow(octree, target_depth, True)
+  return octree
+
+
+def completion_decoder(code, params, split_labels, depth, full_depth, batch_size=1, channel_out=4,
+                       signal=None):
+  """The shape-decoding loop of pytorch/ocnn/ounet.py:103-131 (`decode_shape`) without the skip
+  connections: starting from a full octree at `full_depth`, per depth a 2x2x2 stride-2
+  deconvolution up, a 3x3x3 convolution, the split decision, `octree_update` (child links from
+  the labels) and `octree_grow` (keys / children / neighbours of the next depth).
+
+  code          features at full_depth, [1, C, batch*8^full_depth, 1]
+  params        {('up', d): (w, b), ('conv', d): (w, b)} for d in full_depth+1 .. depth
+  split_labels  {d: int32[H_d]}; label 1 = split.  A callable `f(d, features) -> labels` stands
+                for the reference's prediction head.
+  signal        optional callable `f(features) -> [1, channel_out, H_depth, 1]` written as the
+                finest-level feature of the result
+  Returns (octree, {d: features}).
+  """
+  octree = create_full_octree(full_depth, channel_out, batch_size)
+  feats = {full_depth: code}
+  for d in range(full_depth, depth + 1):
+    if d > full_depth:
+      w, b = params[("up", d)]
+      x = conv_bn_relu(feats[d - 1], w, b, octree, d - 1, w.shape[1] // 8, (2, 2, 2), 2, deconv=True)
+      w, b = params[("conv", d)]
+      feats[d] = conv_bn_relu(x, w, b, octree, d, w.shape[0])
+    label = split_labels(d, feats[d]) if callable(split_labels) else split_labels[d]
+    octree = F.octree_update(octree, label.to(torch.int32), d, 1)
+    if d < depth:
+      octree = F.octree_grow(octree, d + 1, False)
+    elif signal is not None:
+      octree = F.octree_set_property(octree, signal(feats[d]), d)
+  return octree, feats

@@ -564,13 +564,415 @@ static int unique_key(uint64_t* keys, int n, uint64_t* idx) {
   return n > 0 ? j : 0;
 }
 
+
+/* ---- all-depth signals, extrapolation and trimming of Octree::build -------- */
+/* MarchingCube::corner_ / edge_vert_ conventions, marching_cube_table.cpp:312-321.
+ * The edge mask of a cube case (edge_table_) is the set of edges whose two end
+ * corners lie on different sides, so it is derived instead of tabulated. */
+static const float kCorner[8][3] = {
+  { 0, 0, 0 }, { 0, 0, 1 }, { 0, 1, 1 }, { 0, 1, 0 }, { 1, 0, 0 }, { 1, 0, 1 }, { 1, 1, 1 }, { 1, 1, 0 } };
+static const int kEdgeVert[12][2] = {
+  { 0, 1 }, { 1, 2 }, { 2, 3 }, { 3, 0 }, { 4, 5 }, { 5, 6 }, { 6, 7 }, { 7, 4 }, { 0, 4 }, { 1, 5 }, { 2, 6 }, { 3, 7 } };
+/* intersect_cube, marching_cube.cpp:83-98 with MarchingCube::contouring :40-65 (vertices only) */
+static int intersect_cube(float* V, const float* pt, const float* pt_base, const float* normal) {
+  float fval[8];
+  for (int k = 0; k < 8; ++k) {
+    fval[k] = 0.0f;
+    for (int j = 0; j < 3; ++j) fval[k] += (kCorner[k][j] + pt_base[j] - pt[j]) * normal[j];
+  }
+  unsigned cube_case = 0;
+  for (int i = 0; i < 8; ++i) if (fval[i] < 0.0f) cube_case |= 1u << i;
+  int nv = 0;
+  for (int e = 0; e < 12; ++e) {
+    int v1 = kEdgeVert[e][0], v2 = kEdgeVert[e][1];
+    if ((((cube_case >> v1) ^ (cube_case >> v2)) & 1u) == 0) continue;
+    float df = fval[v2] - fval[v1];
+    if (df == 0) df += 1.0e-10f;
+    float t = -fval[v1] / df;
+    for (int j = 0; j < 3; ++j) {
+      float pj = kCorner[v1][j] + t * (kCorner[v2][j] - kCorner[v1][j]);
+      V[3 * nv + j] = pj + pt_base[j];
+    }
+    nv++;
+  }
+  return nv;
+}
+static float norm2f(const float* v, int n) { /* math_functions.cpp:257-263 */
+  float len = 0.0f;
+  for (int i = 0; i < n; ++i) len += v[i] * v[i];
+  return sqrtf(len);
+}
+/* OctreeParser::key2xyz<float>, octree_parser.cpp:151-165: with the key2xyz flag the
+ * (still Morton) key is read as packed 16-bit fields, exactly as the reference does. */
+static void key2xyz_f(float* xyz, uint64_t key, int depth, int flag) {
+  if (flag) {
+    uint16_t f[4]; memcpy(f, &key, 8);
+    for (int c = 0; c < 3; ++c) xyz[c] = (float)f[c];
+  } else {
+    uint64_t pt[3]; compute_pt(pt, key, depth);
+    for (int c = 0; c < 3; ++c) xyz[c] = (float)pt[c];
+  }
+}
+typedef struct {
+  int depth, full_layer, adp_layer, key2xyz;
+  int ch_normal, ch_pt, ch_feature, ch_label, ch_dis, max_label;
+  int has_dis;
+  int nnum[17];
+  uint64_t* keys[17]; int* children[17];
+  float* normals[17]; float* pts[17]; float* features[17]; float* labels[17]; float* dis[17];
+  float* nerr[17]; float* derr[17]; float* split[17];
+  int* dnum[17]; int* didx[17];
+} Tree;
+
+/* covered_depth_nodes, octree.cpp:958-1002 */
+static void covered_depth_nodes(Tree* t) {
+  const int D = t->depth;
+  for (int d = 0; d <= D; ++d) {
+    t->dnum[d] = (int*)calloc((size_t)t->nnum[d] + 1, sizeof(int));
+    t->didx[d] = (int*)malloc(sizeof(int) * ((size_t)t->nnum[d] + 1));
+    for (int i = 0; i < t->nnum[d]; ++i) t->didx[d][i] = -1;
+  }
+  for (int i = 0; i < t->nnum[D]; ++i) { t->dnum[D][i] = 1; t->didx[D][i] = i; }
+  for (int i = 0; i < t->nnum[D - 1]; ++i) {
+    int c = t->children[D - 1][i];
+    if (c == -1) continue;
+    t->dnum[D - 1][i] = 8; t->didx[D - 1][i] = c * 8;
+  }
+  for (int d = D - 2; d >= 0; --d)
+    for (int i = 0; i < t->nnum[d]; ++i) {
+      int c = t->children[d][i];
+      if (c == -1) continue;
+      c *= 8;
+      for (int j = 0; j < 8; ++j) t->dnum[d][i] += t->dnum[d + 1][c + j];
+      for (int j = 0; j < 8; ++j)
+        if (t->didx[d + 1][c + j] != -1) { t->didx[d][i] = t->didx[d + 1][c + j]; break; }
+    }
+}
+
+/* calc_signal(calc_normal_err, calc_dist_err), octree.cpp:454-664 */
+static void calc_signal_all(Tree* t, int calc_normal_err, int calc_dist_err) {
+  const int D = t->depth, nD = t->nnum[D];
+  const float imul = 2.0f / sqrtf(3.0f);
+  const int* child_D = t->children[D];
+  const float* nrm_D = t->normals[D]; const float* pt_D = t->pts[D];
+  const float* feat_D = t->features[D]; const float* lab_D = t->labels[D];
+  const int cn = t->ch_normal, cp = t->ch_pt, cf = t->ch_feature;
+  const int has_normal = nrm_D != NULL, has_pt = pt_D != NULL, has_feature = feat_D != NULL,
+      has_label = lab_D != NULL, has_dis = t->dis[D] != NULL;
+  if (calc_normal_err) { t->nerr[D] = (float*)malloc(sizeof(float) * ((size_t)nD + 1)); for (int i = 0; i < nD; ++i) t->nerr[D][i] = 1.0e20f; }
+  if (calc_dist_err) { t->derr[D] = (float*)malloc(sizeof(float) * ((size_t)nD + 1)); for (int i = 0; i < nD; ++i) t->derr[D][i] = 1.0e20f; }
+  float* n_avg = (float*)calloc((size_t)(cn > 3 ? cn : 3) + 1, sizeof(float));
+  float* f_avg = (float*)calloc((size_t)cf + 1, sizeof(float));
+  int* l_avg = (int*)calloc((size_t)(t->max_label > 0 ? t->max_label : 1), sizeof(int));
+  for (int d = D - 1; d >= 0; --d) {
+    const int n = t->nnum[d];
+    const int* dnum = t->dnum[d]; const int* didx = t->didx[d]; const int* child = t->children[d];
+    const float scale = (float)(1 << (D - d));
+    const int ch_dis = has_normal ? 1 : 4;
+    if (has_normal) t->normals[d] = (float*)calloc((size_t)n * cn + 1, sizeof(float));
+    if (has_pt) t->pts[d] = (float*)calloc((size_t)n * cp + 1, sizeof(float));
+    if (has_feature) t->features[d] = (float*)calloc((size_t)n * cf + 1, sizeof(float));
+    if (has_label) { t->labels[d] = (float*)malloc(sizeof(float) * ((size_t)n + 1)); for (int i = 0; i < n; ++i) t->labels[d][i] = -1.0f; }
+    if (has_dis) t->dis[d] = (float*)calloc((size_t)n * ch_dis + 1, sizeof(float));
+    if (calc_normal_err) { t->nerr[d] = (float*)malloc(sizeof(float) * ((size_t)n + 1)); for (int i = 0; i < n; ++i) t->nerr[d][i] = 1.0e20f; }
+    if (calc_dist_err) { t->derr[d] = (float*)malloc(sizeof(float) * ((size_t)n + 1)); for (int i = 0; i < n; ++i) t->derr[d][i] = 1.0e20f; }
+    for (int i = 0; i < n; ++i) {
+      if (child[i] == -1) continue;
+      const int j0 = didx[i], j1 = didx[i] + dnum[i];
+      for (int c = 0; c < cn; ++c) n_avg[c] = 0.0f;
+      if (has_normal) {
+        for (int j = j0; j < j1; ++j) {
+          if (child_D[j] == -1) continue;
+          for (int c = 0; c < cn; ++c) n_avg[c] += nrm_D[(int64_t)c * nD + j];
+        }
+        float len = norm2f(n_avg, cn);
+        if (len < 1.0e-6f) {
+          for (int j = j0; j < j1; ++j) {
+            if (child_D[j] == -1) continue;
+            for (int c = 0; c < cn; ++c) n_avg[c] = nrm_D[(int64_t)c * nD + j];
+          }
+          len = norm2f(n_avg, cn) + 1.0e-30f;
+        }
+        for (int c = 0; c < cn; ++c) { n_avg[c] /= len; t->normals[d][(int64_t)c * n + i] = n_avg[c]; }
+      }
+      float count = 1.0e-30f;
+      for (int j = j0; j < j1; ++j) if (child_D[j] != -1) count += 1.0f;
+      float pt_avg[3] = { 0.0f, 0.0f, 0.0f };
+      if (has_pt) {
+        for (int j = j0; j < j1; ++j) {
+          if (child_D[j] == -1) continue;
+          for (int c = 0; c < cp; ++c) pt_avg[c] += pt_D[(int64_t)c * nD + j];
+        }
+        for (int c = 0; c < cp; ++c) { pt_avg[c] /= count * scale; t->pts[d][(int64_t)c * n + i] = pt_avg[c]; }
+      }
+      if (has_feature) {
+        for (int c = 0; c < cf; ++c) f_avg[c] = 0.0f;
+        for (int j = j0; j < j1; ++j) {
+          if (child_D[j] == -1) continue;
+          for (int c = 0; c < cf; ++c) f_avg[c] += feat_D[(int64_t)c * nD + j];
+        }
+        for (int c = 0; c < cf; ++c) { f_avg[c] /= count; t->features[d][(int64_t)c * n + i] = f_avg[c]; }
+      }
+      if (has_label) {
+        int valid = 0;
+        for (int l = 0; l < t->max_label; ++l) l_avg[l] = 0;
+        for (int j = j0; j < j1; ++j) {
+          int l = (int)lab_D[j];
+          if (l < 0) continue;
+          l_avg[l] += 1; valid += 1;
+        }
+        if (valid > 0) {
+          int best = 0;
+          for (int l = 1; l < t->max_label; ++l) if (l_avg[l] > l_avg[best]) best = l;
+          t->labels[d][i] = (float)best;
+        }
+      }
+      uint64_t ptu[3]; compute_pt(ptu, t->keys[d][i], d);
+      float pt_base[3] = { (float)ptu[0], (float)ptu[1], (float)ptu[2] };
+      if (has_dis) {
+        float dis_avg[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
+        for (int c = 0; c < 3; ++c) {
+          float fract = pt_avg[c] - pt_base[c];
+          dis_avg[c] = fract - 0.5f;
+          if (has_normal) dis_avg[3] += dis_avg[c] * n_avg[c]; else dis_avg[3] = 1.0f;
+        }
+        if (!has_normal) {
+          for (int c = 0; c < 3; ++c) t->dis[d][(int64_t)c * n + i] = dis_avg[c];
+          t->dis[d][3 * (int64_t)n + i] = dis_avg[3] * imul;
+        } else t->dis[d][i] = dis_avg[3] * imul;
+      }
+      if (calc_normal_err && has_normal && d >= t->adp_layer) {
+        float nm_err = 0.0f;
+        for (int j = j0; j < j1; ++j) {
+          if (child_D[j] == -1) continue;
+          for (int c = 0; c < 3; ++c) { float tmp = nrm_D[(int64_t)c * nD + j] - n_avg[c]; nm_err += tmp * tmp; }
+        }
+        nm_err /= count;
+        t->nerr[d][i] = nm_err;
+      }
+      if (calc_dist_err && has_pt && d >= t->adp_layer) {
+        float distance_max1 = -1.0f;
+        float pt_avg1[3] = { pt_avg[0] * scale, pt_avg[1] * scale, pt_avg[2] * scale };
+        for (int j = j0; j < j1; ++j) {
+          if (child_D[j] == -1) continue;
+          float dis = 0.0f;
+          for (int c = 0; c < 3; ++c) dis += (pt_D[(int64_t)c * nD + j] - pt_avg1[c]) * n_avg[c];
+          dis = fabsf(dis);
+          if (dis > distance_max1) distance_max1 = dis;
+        }
+        float distance_max2 = -1.0f;
+        float vtx[36];
+        int nv = intersect_cube(vtx, pt_avg, pt_base, n_avg);
+        if (nv == 0) distance_max2 = 5.0e10f;
+        for (int k = 0; k < 3 * nv; ++k) vtx[k] *= scale;
+        for (int k = 0; k < nv; ++k) {
+          float distance_min = 1.0e30f;
+          for (int j = j0; j < j1; ++j) {
+            if (child_D[j] == -1) continue;
+            float dis = 0.0f;
+            for (int c = 0; c < 3; ++c) { float ptc = pt_D[(int64_t)c * nD + j] - vtx[3 * k + c]; dis += ptc * ptc; }
+            dis = sqrtf(dis);
+            if (dis < distance_min) distance_min = dis;
+          }
+          if (distance_min > distance_max2) distance_max2 = distance_min;
+        }
+        t->derr[d][i] = distance_max2 > distance_max1 ? distance_max2 : distance_max1;
+      }
+    }
+  }
+  free(n_avg); free(f_avg); free(l_avg);
+}
+
+/* calc_split_label, octree.cpp:1158-1178 */
+static void calc_split_label(Tree* t, int adaptive) {
+  for (int d = 0; d <= t->depth; ++d) {
+    const int n = t->nnum[d];
+    free(t->split[d]);
+    t->split[d] = (float*)malloc(sizeof(float) * ((size_t)n + 1));
+    for (int i = 0; i < n; ++i) {
+      t->split[d][i] = 1.0f;
+      if (t->children[d][i] == -1) {
+        t->split[d][i] = 0.0f;
+        if (adaptive) {
+          float a = fabsf(t->normals[d][i]) + fabsf(t->normals[d][n + i]) + fabsf(t->normals[d][2 * (int64_t)n + i]);
+          if (a != 0) t->split[d][i] = 2.0f;
+        }
+      }
+    }
+  }
+}
+
+/* extrapolate_signal, octree.cpp:666-806 */
+static void extrapolate_signal(Tree* t) {
+  const int D = t->depth;
+  const float imul = 2.0f / sqrtf(3.0f);
+  const int cn = t->ch_normal, cf = t->ch_feature;
+  const int has_dis = t->dis[D] != NULL, has_normal = t->normals[D] != NULL,
+      has_feature = t->features[D] != NULL, has_label = t->labels[D] != NULL;
+  static const float xyzs[8][3] = { { 0, 0, 0 }, { 0, 0, 1 }, { 0, 1, 0 }, { 0, 1, 1 }, { 1, 0, 0 }, { 1, 0, 1 }, { 1, 1, 0 }, { 1, 1, 1 } };
+  float* n_avg = (float*)calloc((size_t)(cn > 3 ? cn : 3) + 1, sizeof(float));
+  float* f_avg = (float*)calloc((size_t)cf + 1, sizeof(float));
+  int* l_avg = (int*)calloc((size_t)(t->max_label > 0 ? t->max_label : 1), sizeof(int));
+  for (int d = D; d >= t->full_layer; --d) {
+    const int n = t->nnum[d];
+    const int* child = t->children[d];
+    float* normal_d = t->normals[d]; float* label_d = t->labels[d];
+    float* feature_d = t->features[d]; float* dis_d = t->dis[d];
+    for (int i = 0; i < n; ++i) {
+      if (child[i] != -1) continue;
+      const int id = i % 8, i_base = i - id;
+      float count = 1.0e-30f;
+      for (int j = i_base; j < i_base + 8; ++j) if (child[j] != -1) count += 1.0f;
+      for (int c = 0; c < (cn > 3 ? cn : 3); ++c) n_avg[c] = 0.0f;
+      if (has_normal) {
+        for (int j = i_base; j < i_base + 8; ++j) {
+          if (child[j] == -1) continue;
+          for (int c = 0; c < cn; ++c) n_avg[c] += normal_d[(int64_t)c * n + j];
+        }
+        float ilen = 1.0f / (norm2f(n_avg, cn) + 1.0e-30f);
+        for (int c = 0; c < cn; ++c) { n_avg[c] *= ilen; normal_d[(int64_t)c * n + i] = n_avg[c]; }
+      }
+      if (has_feature) {
+        for (int c = 0; c < cf; ++c) f_avg[c] = 0.0f;
+        for (int j = i_base; j < i_base + 8; ++j) {
+          if (child[j] == -1) continue;
+          for (int c = 0; c < cf; ++c) f_avg[c] += feature_d[(int64_t)c * n + j];
+        }
+        for (int c = 0; c < cf; ++c) { f_avg[c] /= count; feature_d[(int64_t)c * n + i] = f_avg[c]; }
+      }
+      if (has_label) {
+        int valid = 0;
+        for (int l = 0; l < t->max_label; ++l) l_avg[l] = 0;
+        for (int j = i_base; j < i_base + 8; ++j) {
+          int l = (int)label_d[j];
+          if (l < 0) continue;
+          l_avg[l] += 1; valid += 1;
+        }
+        if (valid > 0) {
+          int best = 0;
+          for (int l = 1; l < t->max_label; ++l) if (l_avg[l] > l_avg[best]) best = l;
+          label_d[i] = (float)best;
+        }
+      }
+      if (has_dis && count > 0.5f) {
+        float dis = 0;
+        for (int j = i_base; j < i_base + 8; ++j) {
+          if (child[j] == -1) continue;
+          dis += dis_d[j];
+          for (int c = 0; c < cn; ++c) dis += normal_d[(int64_t)c * n + j] * (xyzs[j % 8][c] - xyzs[id][c]) * imul;
+        }
+        dis /= count;
+        if (dis > 3.0f) dis = 3.0f;
+        if (dis < -3.0f) dis = -3.0f;
+        if (fabsf(dis) < 1.0f) {
+          unsigned cube_cases = 0;
+          for (int k = 0; k < 8; ++k) {
+            float fval = dis;
+            for (int j = 0; j < 3; ++j) fval += (0.5f - kCorner[k][j]) * n_avg[j] * imul;
+            if (fval < 0) cube_cases |= 1u << k;
+          }
+          if (cube_cases != 255 && cube_cases != 0) dis = dis < 0 ? -1.0f : 1.0f;
+        }
+        dis_d[i] = dis;
+      }
+      if (has_dis && count < 0.5f) {
+        int j_min = -1;
+        float pti[3], ptj[3], dis_min = 1.0e30f;
+        key2xyz_f(pti, t->keys[d][i], d, t->key2xyz);
+        for (int j = 0; j < n; ++j) {
+          if (child[j] == -1) continue;
+          key2xyz_f(ptj, t->keys[d][j], d, t->key2xyz);
+          float dd = fabsf(pti[0] - ptj[0]) + fabsf(pti[1] - ptj[1]) + fabsf(pti[2] - ptj[2]);
+          if (dd < dis_min) { dis_min = dd; j_min = j; }
+        }
+        if (j_min < 0) continue; /* the reference indexes with -1 here (undefined); no such layer is ever built */
+        float dis = dis_d[j_min];
+        key2xyz_f(ptj, t->keys[d][j_min], d, t->key2xyz);
+        for (int c = 0; c < cn; ++c) dis += normal_d[(int64_t)c * n + j_min] * (ptj[c] - pti[c]) * imul;
+        if (dis > 0.0f) dis = 2.0f;
+        if (dis < 0.0f) dis = -2.0f;
+        dis_d[i] = dis;
+      }
+    }
+  }
+  free(n_avg); free(f_avg); free(l_avg);
+}
+
+/* trim_octree (structure and signals), octree.cpp:1004-1135 */
+static void trim_signal(float** sig, int channel, int n_old, const unsigned char* drop, int n_new) {
+  if (!*sig || channel == 0) return;
+  float* out = (float*)malloc(sizeof(float) * ((size_t)n_new * channel + 1));
+  int k = 0;
+  for (int i = 0; i < n_old; ++i) {
+    if (drop[i] == 0) continue;
+    for (int c = 0; c < channel; ++c) out[(int64_t)c * n_new + k] = (*sig)[(int64_t)c * n_old + i];
+    k++;
+  }
+  free(*sig); *sig = out;
+}
+static void trim_octree(Tree* t, float th_dist, float th_norm) {
+  enum { kDrop = 0, kDropChildren = 1, kKeep = 2 };
+  const int D = t->depth, A = t->adp_layer;
+  unsigned char* drop[17];
+  for (int d = 0; d <= D; ++d) { drop[d] = (unsigned char*)malloc((size_t)t->nnum[d] + 1); memset(drop[d], kKeep, (size_t)t->nnum[d] + 1); }
+  for (int d = A; d <= D; ++d) {
+    const int n_dp = t->nnum[d - 1];
+    const int* child_d = t->children[d]; const int* child_dp = t->children[d - 1];
+    int all_drop = 1;
+    for (int i = 0; i < n_dp; ++i) {
+      int c = child_dp[i];
+      if (c == -1) continue;
+      for (int j = 0; j < 8; ++j) {
+        int idx = c * 8 + j;
+        if (drop[d - 1][i] == kKeep) {
+          if ((!t->has_dis || t->derr[d][idx] < th_dist) && t->nerr[d][idx] < th_norm) drop[d][idx] = kDropChildren;
+        } else drop[d][idx] = kDrop;
+        if (all_drop) all_drop = !(drop[d][idx] == kKeep && child_d[idx] != -1);
+      }
+    }
+    if (all_drop) {
+      int max_idx = 0; float max_err = -1.0f;
+      for (int i = 0; i < n_dp; ++i) {
+        int c = child_dp[i];
+        if (c == -1 || drop[d - 1][i] != kKeep) continue;
+        for (int j = 0; j < 8; ++j) {
+          int idx = c * 8 + j;
+          if (child_d[idx] != -1 && t->nerr[d][idx] > max_err) { max_err = t->nerr[d][idx]; max_idx = idx; }
+        }
+      }
+      drop[d][max_idx] = kKeep;
+    }
+  }
+  for (int d = A; d <= D; ++d) {
+    const int n = t->nnum[d];
+    int n_new = 0;
+    for (int i = 0; i < n; ++i) if (drop[d][i] != kDrop) n_new++;
+    uint64_t* key = (uint64_t*)malloc(sizeof(uint64_t) * ((size_t)n_new + 1));
+    int* ch = (int*)malloc(sizeof(int) * ((size_t)n_new + 1));
+    int k = 0, id = 0;
+    for (int i = 0; i < n; ++i) {
+      if (drop[d][i] == kDrop) continue;
+      key[k] = t->keys[d][i];
+      ch[k] = (drop[d][i] == kKeep && t->children[d][i] != -1) ? id++ : -1;
+      k++;
+    }
+    free(t->keys[d]); t->keys[d] = key;
+    free(t->children[d]); t->children[d] = ch;
+    trim_signal(&t->dis[d], t->ch_dis, n, drop[d], n_new);
+    trim_signal(&t->normals[d], t->ch_normal, n, drop[d], n_new);
+    trim_signal(&t->features[d], t->ch_feature, n, drop[d], n_new);
+    trim_signal(&t->labels[d], 1, n, drop[d], n_new);
+    t->nnum[d] = n_new;
+  }
+  for (int d = 0; d <= D; ++d) free(drop[d]);
+}
+
 int64_t orc_points2octree(const void* points_blob, int depth, int full_depth,
     int node_dis, int node_feature, int split_label, int adaptive,
     int adp_depth, float th_normal, float th_distance, int extrapolate,
     int save_pts, int key2xyz, const float* bbmin_in, const float* bbmax_in) {
   const PInfo* pi = (const PInfo*)points_blob;
   if (strcmp(pi->magic, "_POINTS_1.0_") != 0 || pi->pt_num <= 0) return ORC_E_BADARG;
-  if (node_feature || adaptive) return ORC_E_UNSUPPORTED; /* octree.cpp:454-806, 958-1135 not restated */
   const int npt = pi->pt_num;
   const char* base = (const char*)points_blob;
   const float* pts = (pi->content_flags & pPoint) ? (const float*)(base + pi->ptr_dis[0]) : NULL;
@@ -581,6 +983,8 @@ int64_t orc_points2octree(const void* points_blob, int depth, int full_depth,
   const int ch_feature = features ? pi->channels[2] : 0;
   const int ch_label = labels ? pi->channels[3] : 0;
   if (!pts) return ORC_E_BADARG;
+  /* trim_octree reads normal_err_ (exists only with normals) and leaves avg_pts_ untrimmed */
+  if (adaptive && (!normals || save_pts || adp_depth < 1)) return ORC_E_UNSUPPORTED;
 
   /* OctreeInfo::initialize, octree_info.cpp:13-73 */
   OInfo o; info_reset(&o);
@@ -682,7 +1086,7 @@ int64_t orc_points2octree(const void* points_blob, int depth, int full_depth,
   const int* child_d = children[depth];
   float* avg_normals = NULL; float* avg_features = NULL; float* avg_labels = NULL;
   float* avg_pts = NULL; float* displacement = NULL;
-  int ch_dis = 0;
+  int ch_dis = 0, max_label_all = 0;
   if (normals) {
     avg_normals = (float*)calloc((size_t)ch_normal * (size_t)nn + 1, sizeof(float));
     float* acc = (float*)malloc(sizeof(float) * (size_t)(ch_normal + 1));
@@ -730,6 +1134,7 @@ int64_t orc_points2octree(const void* points_blob, int depth, int full_depth,
     float mx = labels[0];
     for (int i = 1; i < npt; ++i) if (labels[i] > mx) mx = labels[i];
     int max_label = (int)mx + 1;
+    max_label_all = max_label;
     int* cnt = (int*)malloc(sizeof(int) * (size_t)(max_label > 0 ? max_label : 1));
     for (int i = 0; i < nn; i++) {
       int t = child_d[i];
@@ -781,6 +1186,34 @@ int64_t orc_points2octree(const void* points_blob, int depth, int full_depth,
     }
   }
 
+  /* all-depth signals, split labels, extrapolation, trimming: Octree::build, octree.cpp:96-120 */
+  Tree t; memset(&t, 0, sizeof(t));
+  t.depth = depth; t.full_layer = full_layer; t.adp_layer = o.adp_layer; t.key2xyz = o.key2xyz;
+  t.ch_normal = ch_normal; t.ch_pt = avg_pts ? 3 : 0; t.ch_feature = ch_feature; t.ch_label = avg_labels ? 1 : 0;
+  t.ch_dis = ch_dis; t.has_dis = o.has_node_dis; t.max_label = max_label_all;
+  for (int d = 0; d <= depth; ++d) { t.nnum[d] = nnum[d]; t.keys[d] = keys[d]; t.children[d] = children[d]; }
+  t.normals[depth] = avg_normals; t.features[depth] = avg_features; t.labels[depth] = avg_labels;
+  t.pts[depth] = avg_pts; t.dis[depth] = displacement;
+  const int all_depths = location_of(&o, kFeature) == -1;
+  if (all_depths) {
+    covered_depth_nodes(&t);
+    calc_signal_all(&t, o.is_adaptive && normals, o.is_adaptive && o.has_node_dis && normals);
+  }
+  if (split_label) calc_split_label(&t, o.is_adaptive);
+  if (o.extrapolate && all_depths) extrapolate_signal(&t);
+  if (o.is_adaptive) {
+    trim_octree(&t, o.th_dist, o.th_norm);
+    for (int d = 0; d <= depth; ++d) { /* calc_node_num, octree.cpp:285-309 */
+      o.nnum[d] = t.nnum[d];
+      o.nnum_nempty[d] = 0;
+      for (int i = t.nnum[d] - 1; i >= 0; i--)
+        if (t.children[d][i] != -1) { o.nnum_nempty[d] = t.children[d][i] + 1; break; }
+    }
+    set_nnum_cum(&o, 0);
+    set_ptr_dis(&o);
+    if (split_label) calc_split_label(&t, 1);
+  }
+
   /* serialize, octree.cpp:907-956 */
   const int sz = sizeof_octree(&o);
   char* buf = result_alloc(sz);
@@ -790,37 +1223,40 @@ int64_t orc_points2octree(const void* points_blob, int depth, int full_depth,
     const int kch = channel_of(&o, kKey);
     uint64_t* kdst = (uint64_t*)prop_ptr(buf, kKey, 0);
     for (int d = 0; d <= depth; ++d) {
+      const int n = t.nnum[d];
       if (o.key2xyz) { /* key_to_xyz, octree.cpp:1137-1156: nnum*channel entries, first nnum written */
-        for (int i = 0; i < nnum[d]; ++i) {
-          uint64_t pt[3]; compute_pt(pt, keys[d][i], d);
+        memset(kdst, 0, sizeof(uint64_t) * (size_t)n * kch);
+        for (int i = 0; i < n; ++i) {
+          uint64_t pt[3]; compute_pt(pt, t.keys[d][i], d);
           uint16_t f[4] = { (uint16_t)pt[0], (uint16_t)pt[1], (uint16_t)pt[2], 0 };
           memcpy(kdst + i, f, 8);
         }
-      } else memcpy(kdst, keys[d], sizeof(uint64_t) * (size_t)nnum[d]);
-      kdst += (o.key2xyz ? (int64_t)nnum[d] * kch : nnum[d]);
+      } else memcpy(kdst, t.keys[d], sizeof(uint64_t) * (size_t)n);
+      kdst += (o.key2xyz ? (int64_t)n * kch : n);
     }
     int* cdst = (int*)prop_ptr(buf, kChild, 0);
-    for (int d = 0; d <= depth; ++d) { memcpy(cdst, children[d], sizeof(int) * (size_t)nnum[d]); cdst += nnum[d]; }
-    /* features = normals | displacement | point features | average points; location == depth here */
-    float* fdst = (float*)prop_ptr(buf, kFeature, depth);
-    if (fdst) {
-      if (avg_normals) { memcpy(fdst, avg_normals, sizeof(float) * (size_t)ch_normal * nn); fdst += (int64_t)ch_normal * nn; }
-      if (o.has_node_dis) { memcpy(fdst, displacement, sizeof(float) * (size_t)ch_dis * nn); fdst += (int64_t)ch_dis * nn; }
-      if (avg_features) { memcpy(fdst, avg_features, sizeof(float) * (size_t)ch_feature * nn); fdst += (int64_t)ch_feature * nn; }
-      if (o.save_pts) { memcpy(fdst, avg_pts, sizeof(float) * 3 * (size_t)nn); fdst += 3 * (int64_t)nn; }
-    }
-    float* ldst = (float*)prop_ptr(buf, kLabel, depth);
-    if (ldst && avg_labels) memcpy(ldst, avg_labels, sizeof(float) * (size_t)nn);
-    /* calc_split_label (non-adaptive), octree.cpp:1158-1178 */
+    for (int d = 0; d <= depth; ++d) { memcpy(cdst, t.children[d], sizeof(int) * (size_t)t.nnum[d]); cdst += t.nnum[d]; }
+    /* features = normals | displacement | point features | average points, per stored depth */
+    float* fdst = (float*)prop_ptr(buf, kFeature, all_depths ? 0 : depth);
+    if (fdst)
+      for (int d = all_depths ? 0 : depth; d <= depth; ++d) {
+        const int64_t n = t.nnum[d];
+        if (t.normals[d]) { memcpy(fdst, t.normals[d], sizeof(float) * (size_t)(ch_normal * n)); fdst += ch_normal * n; }
+        if (o.has_node_dis && t.dis[d]) { memcpy(fdst, t.dis[d], sizeof(float) * (size_t)(ch_dis * n)); fdst += ch_dis * n; }
+        if (t.features[d]) { memcpy(fdst, t.features[d], sizeof(float) * (size_t)(ch_feature * n)); fdst += ch_feature * n; }
+        if (o.save_pts && t.pts[d]) { memcpy(fdst, t.pts[d], sizeof(float) * (size_t)(3 * n)); fdst += 3 * n; }
+      }
+    float* ldst = (float*)prop_ptr(buf, kLabel, all_depths ? 0 : depth);
+    if (ldst && avg_labels)
+      for (int d = all_depths ? 0 : depth; d <= depth; ++d) { memcpy(ldst, t.labels[d], sizeof(float) * (size_t)t.nnum[d]); ldst += t.nnum[d]; }
     float* sdst = (float*)prop_ptr(buf, kSplit, 0);
     if (sdst)
-      for (int d = 0; d <= depth; ++d) {
-        for (int i = 0; i < nnum[d]; ++i) sdst[i] = children[d][i] == -1 ? 0.0f : 1.0f;
-        sdst += nnum[d];
-      }
+      for (int d = 0; d <= depth; ++d) { memcpy(sdst, t.split[d], sizeof(float) * (size_t)t.nnum[d]); sdst += t.nnum[d]; }
   }
-  for (int d = 0; d <= 16; ++d) { free(keys[d]); free(children[d]); }
-  free(avg_normals); free(avg_features); free(avg_labels); free(avg_pts); free(displacement);
+  for (int d = 0; d <= 16; ++d) {
+    free(t.keys[d]); free(t.children[d]); free(t.normals[d]); free(t.features[d]); free(t.labels[d]);
+    free(t.pts[d]); free(t.dis[d]); free(t.nerr[d]); free(t.derr[d]); free(t.split[d]); free(t.dnum[d]); free(t.didx[d]);
+  }
   free(pts_scaled); free(node_keys); free(sorted_idx); free(unique_idx);
   return sz;
 }

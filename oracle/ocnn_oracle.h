@@ -21,9 +21,12 @@
  *   new/grow/update ..... MD5 of the rebuilt octree_2 quoted in
  *                         pytorch/test/test_octree_grow.py
  *   search_key .......... literal vectors of pytorch/test/test_octree_key.py
- * NOT restated (parity unpinned, calls return ORC_E_UNSUPPORTED): the
- * adaptive / node_feature / extrapolate branches of Octree::build
- * (octree/octree/octree.cpp:454-806, 958-1135).
+ *   adaptive build ...... (all-depth signals, error metrics, extrapolation, trimming:
+ *                         octree/octree/octree.cpp:454-806, 958-1178) every literal of
+ *                         octree/test/test_octree.cpp:196-331 (TestOctreeTrim), compiled
+ *                         reference byte for byte on seeded smooth surfaces
+ * Returns ORC_E_UNSUPPORTED only where the reference itself reads out of bounds: an adaptive
+ * build without normals or with save_pts.
  */
 #ifndef OCNN_ORACLE_H_
 #define OCNN_ORACLE_H_

@@ -63,6 +63,22 @@ def main():
   pb = make_points_blob(p, n, f)
   single = ref.points2octree(pb, 9, 2)
   hashes["cfg4"] = {"input": sha(pb), "single": sha(single), "batch": sha(ref.octree_batch([single]))}
+  # adaptive build (config 5 builds its inputs this way): one ellipsoid, depth 6
+  rng = np.random.default_rng(77)
+  u = rng.standard_normal((4000, 3))
+  u /= np.linalg.norm(u, axis=1, keepdims=True)
+  ax = np.array([1, 0.6, 0.4])
+  nrm = u / ax
+  nrm = nrm / np.linalg.norm(nrm, axis=1, keepdims=True)
+  pb = make_points_blob((u * 0.8 * ax).astype(np.float32), nrm.astype(np.float32))
+  hashes["adaptive"] = {"input": sha(pb), "octree": sha(ref.points2octree(
+      pb, 6, 2, node_dis=True, split_label=True, adaptive=True, adp_depth=4, th_normal=0.1, th_distance=2.0))}
+  # config 5: 16 adaptive octrees at depth 7 from 50000-point shape clouds
+  blobs = [make_points_blob(*synthetic.shape_cloud(50000, 300 + i)[:2]) for i in range(16)]
+  singles = [ref.points2octree(b, 7, 2, node_dis=True, split_label=True, adaptive=True, adp_depth=4,
+                               th_normal=0.1, th_distance=2.0) for b in blobs]
+  hashes["cfg5"] = {"input": sha(np.concatenate(blobs)), "batch": sha(ref.octree_batch(singles)),
+                    "first_single": sha(singles[0])}
   with open(os.path.join(HERE, "config_hashes.json"), "w") as fh:
     json.dump(hashes, fh, indent=1, sort_keys=True)
   print(json.dumps(hashes, indent=1))

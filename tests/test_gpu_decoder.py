@@ -1,0 +1,100 @@
+"""BASELINE config 5 at test size: a batch of ADAPTIVE octrees (built by the CPU oracle, whose
+adaptive build is pinned against the compiled reference) is merged on the GPU, and the
+shape-completion decoder loop (2x2x2 stride-2 deconv up, 3x3x3 conv, split labels from the
+ground truth, octree_update, octree_grow) rebuilds the ground-truth structure level by level.
+Structure is compared bit-exactly, features within 1e-4 (fp32)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle.checker import OctreeBlob, make_points_blob
+
+pytestmark = pytest.mark.gpu
+
+ADAPTIVE = dict(node_dis=True, split_label=True, adaptive=True, adp_depth=3, th_normal=0.1, th_distance=2.0)
+
+
+def T(a):
+  return torch.from_numpy(np.ascontiguousarray(a))
+
+
+def relerr(got, exp):
+  return float(np.abs(got.astype(np.float64) - exp).max() / (np.abs(exp).max() + 1e-30))
+
+
+@pytest.fixture(scope="module")
+def adaptive_batch(orc, synthetic):
+  singles = [orc.points2octree(make_points_blob(*synthetic.shape_cloud(4000, 300 + i)[:2]), 5, 2, **ADAPTIVE)
+             for i in range(3)]
+  return singles, orc.octree_batch(singles)
+
+
+def test_adaptive_octrees_merge_on_gpu(oc, orc, adaptive_batch):
+  """octree_batch over octrees whose features / labels live at every depth (location -1) and
+  that carry split labels (merge_octrees.cpp:144-177)."""
+  singles, host = adaptive_batch
+  b = OctreeBlob(host)
+  assert b.is_adaptive and b.location("feature") == -1 and b.has("split") and b.channel("feature") == 4
+  assert any((b.prop("split", d) == 2).any() for d in range(3, 6)), "nothing was trimmed"
+  got = oc.nn.octree_batch([T(s) for s in singles]).cpu().numpy()
+  assert np.array_equal(got, host)
+  # the merged adaptive octree is a valid operand of the operators: neighbour-table conv at depth 4
+  rng = np.random.default_rng(0)
+  x = rng.standard_normal((4, int(b.nnum[4]))).astype(np.float32)
+  w = (rng.standard_normal((8, 4 * 27)) * 0.1).astype(np.float32)
+  exp = orc.octree_conv(x, w, host, 4, 8, [3, 3, 3], 1)
+  out = oc.nn.octree_conv(T(x).cuda().view(1, 4, -1, 1), T(w).cuda(), T(host).cuda(), 4, 8, [3, 3, 3], 1, False)
+  assert relerr(out.cpu().numpy().reshape(exp.shape), exp) < 1e-4
+
+
+def oracle_decoder(orc, code, params, labels, depth, full_depth, batch):
+  o = orc.octree_new(batch, 4, True, 0)
+  for d in range(1, full_depth + 1):
+    o = orc.octree_grow(o, d, True)
+  feats = {full_depth: code}
+  for d in range(full_depth, depth + 1):
+    if d > full_depth:
+      child = OctreeBlob(o).prop("child", d - 1)
+      w, bias = params[("up", d)]
+      x = orc.octree_deconv(feats[d - 1][:, child >= 0], w, o, d - 1, w.shape[1] // 8, [2, 2, 2], 2)
+      x = np.maximum(x + bias[:, None], 0)
+      w, bias = params[("conv", d)]
+      feats[d] = np.maximum(orc.octree_conv(x, w, o, d, w.shape[0], [3, 3, 3], 1) + bias[:, None], 0)
+    o = orc.octree_update(o, labels[d], d, 1)
+    if d < depth:
+      o = orc.octree_grow(o, d + 1, False)
+  return o, feats
+
+
+def test_completion_decoder_rebuilds_ground_truth(oc, orc, adaptive_batch):
+  singles, host = adaptive_batch
+  gt = OctreeBlob(host)
+  depth, fd, batch = 5, 2, 3
+  labels = {d: (gt.prop("split", d) == 1).astype(np.int32) for d in range(fd, depth + 1)}
+  rng = np.random.default_rng(5)
+  chans = {2: 32, 3: 24, 4: 16, 5: 8}
+  params = {}
+  for d in range(fd + 1, depth + 1):
+    params[("up", d)] = ((rng.standard_normal((chans[d - 1], chans[d] * 8)) * 0.2).astype(np.float32),
+                         (rng.standard_normal(chans[d]) * 0.1).astype(np.float32))
+    params[("conv", d)] = ((rng.standard_normal((chans[d], chans[d] * 27)) * 0.1).astype(np.float32),
+                           (rng.standard_normal(chans[d]) * 0.1).astype(np.float32))
+  code = rng.standard_normal((chans[fd], batch * 8 ** fd)).astype(np.float32)
+
+  exp_o, exp_f = oracle_decoder(orc, code, params, labels, depth, fd, batch)
+  dev_params = {k: (T(w).cuda(), T(b).cuda()) for k, (w, b) in params.items()}
+  got_o, got_f = oc.stacks.completion_decoder(
+      T(code).cuda().view(1, chans[fd], -1, 1), dev_params, {d: T(l).cuda() for d, l in labels.items()},
+      depth, fd, batch_size=batch, channel_out=4)
+  assert np.array_equal(got_o.cpu().numpy(), exp_o)            # keys, children, neighbours, header
+  for d in range(fd + 1, depth + 1):
+    assert relerr(got_f[d].cpu().numpy().reshape(exp_f[d].shape), exp_f[d]) < 1e-4, d
+
+  # the grown structure IS the ground truth's: same node counts, same voxels, same child links
+  g = OctreeBlob(got_o.cpu().numpy())
+  F = oc.nn
+  gt_dev = T(host).cuda()
+  for d in range(fd, depth + 1):
+    assert g.nnum[d] == gt.nnum[d] and g.nnum_nempty[d] == gt.nnum_nempty[d]
+    assert torch.equal(F.octree_property(got_o, "xyz", d), F.octree_property(gt_dev, "xyz", d))
+    assert np.array_equal(g.prop("child", d), gt.prop("child", d))

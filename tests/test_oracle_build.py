@@ -186,6 +186,111 @@ def test_golden_config1(orc, synthetic, hashes):
 
 
 def test_unsupported_is_reported(orc):
-  pb = make_points_blob([[0, 0, 0]], [[1, 0, 0]])
+  # trimming reads the per-node normal error, which exists only for clouds with normals
+  pb = make_points_blob([[0, 0, 0]])
   with pytest.raises(RuntimeError):
     orc.points2octree(pb, 5, 2, adaptive=True)
+
+
+def test_adaptive_known_answer(orc):
+  """octree/test/test_octree.cpp:196-331 (TestOctreeTrim), every literal of it."""
+  blob = orc.points2octree(three_point_cloud(), 5, 1, node_dis=True, split_label=True, adaptive=True,
+                           adp_depth=3, th_normal=5.0, th_distance=3.0, bbmin=[0, 0, 0], bbmax=[2, 2, 2])
+  b = OctreeBlob(blob)
+  assert (b.depth, b.full_layer, b.adp_layer) == (5, 1, 3)
+  assert list(b.nnum[:6]) == [1, 8, 16, 16, 16, 8]
+  assert list(b.nnum_cum[:7]) == [0, 1, 9, 25, 41, 57, 65]
+  assert list(b.nnum_nempty[:6]) == [1, 2, 2, 2, 1, 1]
+  g8 = list(range(8))
+  keys = [0] + g8 + g8 + list(range(48, 56)) + g8 + list(range(384, 392)) + g8 + list(range(3072, 3080)) + g8
+  assert np.concatenate([b.prop("key", d) for d in range(6)]).tolist() == keys
+  m7 = [-1] * 7
+  children = ([0, 0, -1, -1, -1, -1, -1, 1, -1] + [0] + m7 + [1] + m7 + [0] + m7 + [1] + m7 +
+              [0] + m7 + [-1] + m7 + [0] + m7)
+  assert np.concatenate([b.prop("child", d) for d in range(6)]).tolist() == children
+  assert b.channel("feature") == 6
+  z7, z15 = [0.0] * 7, [0.0] * 15
+  s = 0.707107
+  f0 = [0, 1.0, 0, -0.180422, 2.0, -2.0]
+  f1 = ([1.0, 0, 0, 0, 0, 0, -s, 0] + [0, 0, 0, 0, 0, 0, s, 0] + [0.0] * 8 + [-0.57735] + z7 +
+        [1.0, 0, 0, 0, 0, 0, 2.5, 0] + [-1.0, 0, 0, 0, 0, 0, -2.5, 0])
+  f2 = ([1.0] + z7 + [-s] + z7 + [0.0] * 8 + [s] + z7 + [0.0] * 16 + [-0.57735] + z15 +
+        [1.0] + z7 + [2.5] + z7 + [-1.0] + z7 + [-2.5] + z7)
+  f5 = [1.0] + z7 + [0.0] * 16 + [-0.57735] + z7 + [1.0] + z7 + [-1.0] + z7
+  for d, want in enumerate([f0, f1, f2, f2, f2, f5]):
+    np.testing.assert_allclose(b.prop("feature", d).reshape(-1), np.float32(want), rtol=1e-5, atol=1e-6)
+  l7 = [-1.0] * 7
+  labels = ([2.0, 0, -1, -1, -1, -1, -1, 2.0, -1] + ([0.0] + l7 + [2.0] + l7) * 3 + [0.0] + l7)
+  assert np.concatenate([b.prop("label", d) for d in range(6)]).tolist() == labels
+  s7 = [0.0] * 7
+  split = ([1.0, 1.0, 0, 0, 0, 0, 0, 1.0, 0] + ([1.0] + s7 + [1.0] + s7) * 2 + [1.0] + s7 + [2.0] + s7 +
+           [1.0] + s7)
+  assert np.concatenate([b.prop("split", d) for d in range(6)]).tolist() == split
+
+
+ADAPTIVE_CASES = [
+    dict(adaptive=True, node_dis=True, split_label=True),
+    dict(adaptive=True, node_dis=True, split_label=True, extrapolate=True),
+    dict(adaptive=True),
+    dict(node_feature=True),
+    dict(node_feature=True, node_dis=True, extrapolate=True, split_label=True),
+    dict(node_feature=True, save_pts=True, node_dis=True),
+    dict(adaptive=True, node_dis=True, key2xyz=True, extrapolate=True, split_label=True),
+]
+
+
+def smooth_cloud(rng, n, kind):
+  """Points on an ellipsoid or on a tilted plane: smooth enough for the trimming to act."""
+  if kind == 0:
+    u = rng.standard_normal((n, 3))
+    u /= np.linalg.norm(u, axis=1, keepdims=True)
+    ax = np.array([1, 0.6, 0.4])
+    pts, nrm = u * 0.8 * ax, u / ax
+  else:
+    pts = rng.uniform(-0.9, 0.9, (n, 3))
+    pts[:, 2] = 0.3 * pts[:, 0] + 0.1
+    nrm = np.tile(np.array([[-0.3, 0, 1.0]]), (n, 1))
+  nrm = nrm / np.linalg.norm(nrm, axis=1, keepdims=True)
+  return pts.astype(np.float32), nrm.astype(np.float32)
+
+
+@pytest.mark.parametrize("case", range(len(ADAPTIVE_CASES)))
+def test_adaptive_build_vs_compiled_reference(orc, ref, case):
+  """All-depth signals, error metrics, extrapolation and trimming (octree.cpp:454-806, 958-1178)
+  byte for byte against the compiled reference."""
+  kw = ADAPTIVE_CASES[case]
+  rng = np.random.default_rng(50 + case)
+  for trial in range(5):
+    n = int(rng.integers(200, 5000))
+    pts, nrm = smooth_cloud(rng, n, trial % 2)
+    feat = rng.uniform(0, 1, (n, 2)).astype(np.float32) if trial >= 2 else None
+    lab = rng.integers(-1, 4, n).astype(np.float32) if trial >= 3 else None
+    pb = make_points_blob(pts, nrm, feat, lab)
+    depth = int(rng.integers(4, 8))
+    fd = int(rng.integers(1, 3))
+    extra = dict(adp_depth=int(rng.integers(fd + 1, depth + 1)), th_normal=float(rng.choice([0.1, 0.3, 5.0])),
+                 th_distance=float(rng.choice([0.5, 2.0, 3.0])))
+    a = orc.points2octree(pb, depth, fd, **extra, **kw)
+    b = ref.points2octree(pb, depth, fd, **extra, **kw)
+    assert np.array_equal(a, b)
+
+
+def test_adaptive_golden(orc, hashes):
+  """The committed hash was written from the compiled reference (tests/golden/make_golden.py)."""
+  rng = np.random.default_rng(77)
+  pts, nrm = smooth_cloud(rng, 4000, 0)
+  pb = make_points_blob(pts, nrm)
+  assert sha(pb) == hashes["adaptive"]["input"], "the seeded generator drifted"
+  blob = orc.points2octree(pb, 6, 2, node_dis=True, split_label=True, adaptive=True, adp_depth=4,
+                           th_normal=0.1, th_distance=2.0)
+  assert sha(blob) == hashes["adaptive"]["octree"]
+
+
+def test_golden_config5(orc, synthetic, hashes):
+  """BASELINE config 5 inputs at full size: 16 adaptive octrees at depth 7, merged."""
+  blobs = [make_points_blob(*synthetic.shape_cloud(50000, 300 + i)[:2]) for i in range(16)]
+  assert sha(np.concatenate(blobs)) == hashes["cfg5"]["input"], "the seeded generator drifted"
+  singles = [orc.points2octree(b, 7, 2, node_dis=True, split_label=True, adaptive=True, adp_depth=4,
+                               th_normal=0.1, th_distance=2.0) for b in blobs]
+  assert sha(singles[0]) == hashes["cfg5"]["first_single"]
+  assert sha(orc.octree_batch(singles)) == hashes["cfg5"]["batch"]
