@@ -224,6 +224,13 @@ def main():
     conv_case("conv222_s2_d7_bf16", oct7, 7, x7.bfloat16(), w2.bfloat16(), [2, 2, 2], 2)
     conv_case("deconv222_s2_d8to9_bf16", octree, 8, x8.bfloat16(), w2.bfloat16(), [2, 2, 2], 2, deconv=True)
     conv_case("deconv333_s1_d9_f32", octree, 9, x32, w32, [3, 3, 3], 1, deconv=True)
+    # gradients of the headline conv: weight gradient (contraction over the octants) + data
+    # gradient (the transposed operator); 2 x the forward flops in total
+    gy = torch.randn(1, C, H9, 1, generator=g).to(dev)
+    t = timed(lambda: F.octree_conv_grad(x32, w32, octree, gy, 9, C, [3, 3, 3], 1, False), max(2, reps // 2), 1)
+    fl = 2 * 2.0 * H9 * 27 * C * C
+    extra["conv333_s1_d9_f32_grad"] = {"ms": t, "octants_per_s": H9 / (t * 1e-3), "tflops": fl / (t * 1e-3) / 1e12,
+                                       "frac_mfma_peak": fl / (t * 1e-3) / 1e12 / PEAK_F32}
 
     def hbm(name, t, by):
       extra[name] = {"ms": t, "GBs": by / t / 1e6, "frac_hbm_peak": by / t / 1e6 / PEAK_HBM_GBS}
@@ -317,6 +324,18 @@ def main():
               (torch.randn(co, generator=g) * 0.1).to(dev)) for d, (ci, co) in lch.items()}
     t = timed(lambda: oc.stacks.lenet_trunk(oct6, 6, lp), reps, wu)
     extra["lenet_trunk_batch32_d6_f32"] = {"ms": t, "shapes_per_s": 32 / (t * 1e-3)}
+    # completion decoder loop (configs[4] shape): 16 octrees at depth 7 regrown from depth 2 with
+    # the split labels of the built batch, deconv up + 3x3x3 conv per depth, channels 256 -> 32
+    dch = {2: 256, 3: 128, 4: 64, 5: 32, 6: 32, 7: 32}
+    dspec = {}
+    for d in range(3, 8):
+      dspec[("up", d)] = (dch[d - 1], dch[d] * 8)
+      dspec[("conv", d)] = (dch[d], dch[d] * 27)
+    dp = rand_params(dspec)
+    dlabels = {d: (F.octree_property(oct7, "child", d) >= 0).to(torch.int32) for d in range(2, 8)}
+    code = torch.randn(1, 256, 16 * 64, 1, generator=g).to(dev)
+    t = timed(lambda: oc.stacks.completion_decoder(code, dp, dlabels, 7, 2, batch_size=16), max(2, reps // 2), 1)
+    extra["completion_decoder_batch16_d7_f32"] = {"ms": t, "octants_d7": H7, "octrees_per_s": 16 / (t * 1e-3)}
   out["extra"] = extra
 
   # ---- CPU baseline (reported, not the target) -----------------------------------------------

@@ -165,6 +165,25 @@ int ocnn_octree_conv_fused(void* top, const void* btm, int channel_in, int btm_h
     int num_output, const int* kernel_size, int stride, int nempty, int dtype, void* workspace_dev,
     size_t workspace_bytes, ocnn_stream_t stream);
 
+/* ---- gradients: OctreeConvGradOp / OctreeDeconvGradOp, pytorch/cpp/octree_conv.cpp:159-250
+ * (weight_gpu_gemm / backward_gpu_gemm / forward_gpu_gemm, octree/octree/octree_conv.cpp:276-356).
+ * Arguments are those of the forward call plus `grad_out` [num_output, top_h]; the results have
+ * the shapes of `data_in` and `weights`.  Either result pointer may be NULL to skip it.
+ * The weight gradient contracts over the octree nodes on the matrix cores without a column
+ * buffer and adds its partial sums in a fixed order (reproducible); the data gradient is the
+ * transposed operator with the same weight buffer.  fp32 only (OCNN_E_UNSUPPORTED otherwise);
+ * a stride-2 convolution's data gradient exists for the 2x2x2 kernel only. */
+int ocnn_conv_grad_workspace_bytes(const void* info, int depth, int channel_in, int num_output,
+    const int* kernel_size, int stride, int nempty, int is_deconv, int dtype, size_t* workspace_bytes);
+int ocnn_octree_conv_grad(void* grad_data, void* grad_weights, const void* data_in, int channel_in,
+    int btm_h, const void* weights, const void* grad_out, const void* octree_dev, const void* info,
+    int depth, int num_output, const int* kernel_size, int stride, int nempty, int dtype,
+    void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream);
+int ocnn_octree_deconv_grad(void* grad_data, void* grad_weights, const void* data_in, int channel_in,
+    int btm_h, const void* weights, const void* grad_out, const void* octree_dev, const void* info,
+    int depth, int num_output, const int* kernel_size, int stride, int nempty, int dtype,
+    void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream);
+
 /* ---- octree construction on the device: points2octree + octree_batch fused.
  * Replaces Octree::build (octree/octree/octree.cpp:74-121) driven as in
  * pytorch/cpp/point2octree.cpp:5-34, and merge_octrees

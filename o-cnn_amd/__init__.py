@@ -5,13 +5,15 @@ The directory name is not a Python identifier; load the package with
 
   nn        -- mirror of the reference's `ocnn.nn` extension functions
                (pytorch/cpp/pybind.cpp:3-49) over libocnn_hip.so
+  autograd  -- torch.autograd functions pairing every operator with its adjoint, as the
+               Function classes of pytorch/ocnn do
   layers    -- mirror of the thin Python modules of pytorch/ocnn
                (octree_conv.py, octree_pool.py, octree_pad.py)
   stacks    -- conv -> BatchNorm -> ReLU (folded) operator sequences of the benchmark
                configurations (LeNet trunk, U-Net encoder / decoder)
   synthetic -- seeded synthetic point clouds of the benchmark configurations
 """
-from . import lib, nn, layers, stacks, synthetic  # noqa: F401
+from . import lib, nn, autograd, layers, stacks, synthetic  # noqa: F401
 from .nn import *  # noqa: F401,F403
 from .layers import (OctreeConv, OctreeDeconv, OctreeConvFast, OctreeDeconvFast,  # noqa: F401
                      OctreeMaxPool, OctreeMaxUnpool, OctreeAvgPool, OctreePad, OctreeDepad)

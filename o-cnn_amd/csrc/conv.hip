@@ -1218,6 +1218,249 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
   return OCNN_OK;
 }
 
+
+// ---- weight gradient ----------------------------------------------------------------------
+// G[m, c*K + k] = sum_n A[m, n] * X[c, src(n, k)]   (weight_gpu_gemm, octree_conv.cpp:327-356,
+// without the column buffer).  A is the operand on the column side of the convolution geometry
+// ([M, N]), X the gathered side, read from its row-major copy xt[Hin + 1][cpad] (row Hin zero).
+// The reduction runs over the columns, so the MFMA k dimension is n: lane (m, kh) loads one
+// float4 of A = columns n0 + 4kh .. + 3, and step j multiplies the column pair (n0 + j,
+// n0 + 4 + j); lane (c, kh) gathers xt[src(n0 + 4kh + j, tap)][c], 128 contiguous bytes per half
+// wavefront.  A wavefront is one slice: it walks every n_slices-th block of 8 columns with its
+// own accumulators for 3 taps x (MT x NT) 32x32 tiles and writes them to partial[slice]; a second
+// kernel adds the slices in a fixed order, so the result is reproducible (no atomics).
+constexpr int kWgTaps = 3;
+
+template <int MT, int NT>
+__global__ __launch_bounds__(256, 2) void conv_wgrad_f32_kernel(ConvArgs a, const float* __restrict__ A,
+    const float* __restrict__ xt, float* __restrict__ partial, int cpad, int mpad, int n_slices, int cpasses) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int slice = blockIdx.x * 4 + wave;
+  const int tap0 = blockIdx.y * kWgTaps;
+  const int mpass = blockIdx.z / cpasses, cpass = blockIdx.z % cpasses;
+  const int r = lane & 31, kh = lane >> 5;
+  floatx16 acc[kWgTaps][MT][NT];
+#pragma unroll
+  for (int t = 0; t < kWgTaps; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[t][mt][nt][i] = 0.0f;
+  const int nblocks = (a.N + 7) >> 3;
+  const bool vec_ok = (a.N & 3) == 0 && (reinterpret_cast<uintptr_t>(A) & 15) == 0;
+  for (int b = slice; b < nblocks; b += n_slices) {
+    const int n0 = b * 8 + 4 * kh;
+    float av[MT][4];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = (mpass * MT + mt) * 32 + r;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) av[mt][j] = 0.0f;
+      if (m < a.M) {
+        const float* ap = A + (int64_t)m * a.N + n0;
+        if (vec_ok && n0 + 4 <= a.N) {
+          const float4 v = *reinterpret_cast<const float4*>(ap);
+          av[mt][0] = v.x; av[mt][1] = v.y; av[mt][2] = v.z; av[mt][3] = v.w;
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) if (n0 + j < a.N) av[mt][j] = ap[j];
+        }
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < kWgTaps; ++t) {
+      const int tap = tap0 + t;
+      int src[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        int sidx = tap < a.K ? conv_src(a, n0 + j, tap) : -1;
+        src[j] = sidx < 0 ? a.Hin : sidx;
+      }
+      float bv[4][NT];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          bv[j][nt] = xt[(int64_t)src[j] * cpad + (cpass * NT + nt) * 32 + r];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+            acc[t][mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[mt][j], bv[j][nt], acc[t][mt][nt], 0, 0, 0);
+    }
+  }
+  // partial[slice][tap][m][c]: lanes of a half wavefront write 128 contiguous bytes
+#pragma unroll
+  for (int t = 0; t < kWgTaps; ++t) {
+    const int tap = tap0 + t;
+    if (tap >= a.K) continue;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int m = (mpass * MT + mt) * 32 + 8 * (i / 4) + 4 * kh + (i % 4);
+          const int c = (cpass * NT + nt) * 32 + r;
+          partial[(((int64_t)slice * a.K + tap) * mpad + m) * cpad + c] = acc[t][mt][nt][i];
+        }
+  }
+}
+__global__ void conv_wgrad_reduce_kernel(float* __restrict__ G, const float* __restrict__ partial, int n_slices,
+    int M, int Cin, int K, int mpad, int cpad) {
+  const int64_t per = (int64_t)K * mpad * cpad;
+  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= per) return;
+  const int c = (int)(id % cpad), m = (int)((id / cpad) % mpad), k = (int)(id / ((int64_t)cpad * mpad));
+  if (m >= M || c >= Cin) return;
+  float sum = 0.0f;
+  for (int sl = 0; sl < n_slices; ++sl) sum += partial[sl * per + id];
+  G[((int64_t)m * Cin + c) * K + k] = sum;
+}
+
+struct WgradPlan {
+  int MT, NT, mpasses, cpasses, mpad, cpad, n_slices, tapgroups;
+  size_t xt_bytes, partial_bytes, ichild_bytes, total_bytes;
+};
+// `p` is the plan of the underlying convolution geometry (deconv = 0): M rows on the column side,
+// channel_in channels on the gathered side.
+void make_wgrad_plan(const ConvPlan& p, int M, int channel_in, int nempty, WgradPlan* w) {
+  const int mtiles = (M + 31) / 32, ctiles = (channel_in + 31) / 32;
+  w->MT = mtiles == 1 ? 1 : 2;
+  w->NT = ctiles == 1 ? 1 : 2;
+  w->mpasses = (mtiles + w->MT - 1) / w->MT;
+  w->cpasses = (ctiles + w->NT - 1) / w->NT;
+  w->mpad = w->mpasses * w->MT * 32;
+  w->cpad = w->cpasses * w->NT * 32;
+  w->tapgroups = (p.taps.count + kWgTaps - 1) / kWgTaps;
+  // about three workgroups per compute unit in total, never more slices than column blocks
+  const int nblocks = (p.top_h + 7) / 8;
+  int per_launch = w->tapgroups * w->mpasses * w->cpasses;
+  int groups = (768 + per_launch - 1) / per_launch;
+  int max_groups = (nblocks + 3) / 4;
+  if (groups > max_groups) groups = max_groups;
+  if (groups < 1) groups = 1;
+  w->n_slices = groups * 4;
+  w->xt_bytes = align256(((size_t)p.btm_h + 1) * w->cpad * sizeof(float));
+  w->partial_bytes = align256((size_t)w->n_slices * p.taps.count * w->mpad * w->cpad * sizeof(float));
+  w->ichild_bytes = nempty ? align256(sizeof(int) * (size_t)(p.ichild_h + 1)) : 0;
+  w->total_bytes = w->xt_bytes + w->partial_bytes + w->ichild_bytes;
+}
+
+// grad_w[M, channel_in * K] from A [M, top_h] (column side) and X [channel_in, btm_h] (gathered side)
+int run_wgrad(float* grad_w, const float* A, int M, const float* X, int channel_in, const Info* o,
+    const void* octree_dev, const ConvPlan& p, int nempty, void* ws, size_t ws_bytes, hipStream_t s) {
+  WgradPlan w;
+  make_wgrad_plan(p, M, channel_in, nempty, &w);
+  OCNN_REQUIRE(ws && ws_bytes >= w.total_bytes, OCNN_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes, w.total_bytes);
+  const char* blob = static_cast<const char*>(octree_dev);
+  char* wsb = static_cast<char*>(ws);
+  ConvArgs a;
+  a.M = M; a.Cin = channel_in; a.N = p.top_h; a.K = p.taps.count; a.Hin = p.btm_h; a.Hout = p.top_h;
+  a.mode = p.mode; a.nempty = nempty ? 1 : 0; a.mtiles = (M + 31) / 32; a.csteps = 0;
+  for (int k = 0; k < 27; ++k) a.slot[k] = tap_slot(k < p.taps.count ? p.taps.tap[k] : 13);
+  a.neigh = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_NEIGH, p.workspace_depth));
+  a.child = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_CHILD, p.workspace_depth));
+  a.ichild = nullptr; a.bias = nullptr; a.relu = 0;
+  float* xt = reinterpret_cast<float*>(wsb);
+  float* partial = reinterpret_cast<float*>(wsb + w.xt_bytes);
+  if (nempty) {
+    int* ichild = reinterpret_cast<int*>(wsb + w.xt_bytes + w.partial_bytes);
+    ichild_kernel<<<blocks_for(p.child_h), kBlock, 0, s>>>(ichild, p.ichild_h, a.child, p.child_h);
+    OCNN_LAUNCH_OK("ichild");
+    a.ichild = ichild;
+  }
+  dim3 tg((a.Hin + 64) / 64, (w.cpad + 63) / 64);
+  transpose_rows_f32_kernel<<<tg, 256, 0, s>>>(xt, X, channel_in, a.Hin, w.cpad);
+  OCNN_LAUNCH_OK("transpose_rows");
+  dim3 grid(w.n_slices / 4, w.tapgroups, w.mpasses * w.cpasses);
+  if (w.MT == 1 && w.NT == 1)
+    conv_wgrad_f32_kernel<1, 1><<<grid, 256, 0, s>>>(a, A, xt, partial, w.cpad, w.mpad, w.n_slices, w.cpasses);
+  else if (w.MT == 1)
+    conv_wgrad_f32_kernel<1, 2><<<grid, 256, 0, s>>>(a, A, xt, partial, w.cpad, w.mpad, w.n_slices, w.cpasses);
+  else if (w.NT == 1)
+    conv_wgrad_f32_kernel<2, 1><<<grid, 256, 0, s>>>(a, A, xt, partial, w.cpad, w.mpad, w.n_slices, w.cpasses);
+  else
+    conv_wgrad_f32_kernel<2, 2><<<grid, 256, 0, s>>>(a, A, xt, partial, w.cpad, w.mpad, w.n_slices, w.cpasses);
+  OCNN_LAUNCH_OK("conv_wgrad");
+  int64_t per = (int64_t)a.K * w.mpad * w.cpad;
+  conv_wgrad_reduce_kernel<<<blocks_for(per), kBlock, 0, s>>>(grad_w, partial, w.n_slices, M, channel_in, a.K,
+      w.mpad, w.cpad);
+  OCNN_LAUNCH_OK("conv_wgrad_reduce");
+  return OCNN_OK;
+}
+
+// Plans of the three pieces of a gradient call: the weight-gradient geometry (always a
+// convolution), and the operator that computes the data gradient (the transposed operator).
+struct GradPlan {
+  ConvPlan geom, data;
+  WgradPlan w;
+  int geom_depth, data_depth, data_cin, data_cout, wg_M, wg_C;
+  size_t total_bytes;
+};
+int make_grad_plan(const Info* o, int is_deconv, int depth, int channel_in, int num_output, const int* ks,
+    int stride, int nempty, int dtype, GradPlan* g) {
+  OCNN_REQUIRE(dtype == OCNN_F32, OCNN_E_UNSUPPORTED, "gradients are computed in fp32 only");
+  int e;
+  if (!is_deconv) {
+    // forward conv: X[Cin] at depth -> Y[Cout].  grad_w = dY * col(X)^T; grad_X = deconv(dY; W).
+    g->geom_depth = depth;
+    g->wg_M = num_output; g->wg_C = channel_in;
+    e = make_plan(o, depth, channel_in, num_output, ks, stride, nempty, 0, dtype, &g->geom);
+    if (e) return e;
+    g->data_depth = stride == 2 ? depth - 1 : depth;
+    g->data_cin = num_output; g->data_cout = channel_in;
+    e = make_plan(o, g->data_depth, num_output, channel_in, ks, stride, nempty, 1, dtype, &g->data);
+  } else {
+    // forward deconv: X[Cin] at depth -> Y[Cout] at depth (+1).  grad_w = X * col(dY)^T;
+    // grad_X = conv(dY; W).
+    g->geom_depth = stride == 2 ? depth + 1 : depth;
+    g->wg_M = channel_in; g->wg_C = num_output;
+    e = make_plan(o, g->geom_depth, num_output, channel_in, ks, stride, nempty, 0, dtype, &g->geom);
+    if (e) return e;
+    g->data_depth = g->geom_depth;
+    g->data_cin = num_output; g->data_cout = channel_in;
+    g->data = g->geom;
+  }
+  if (e) return e;
+  make_wgrad_plan(g->geom, g->wg_M, g->wg_C, nempty, &g->w);
+  g->total_bytes = g->w.total_bytes > g->data.total_bytes ? g->w.total_bytes : g->data.total_bytes;
+  return OCNN_OK;
+}
+
+int run_grad(int is_deconv, void* grad_data, void* grad_w, const void* data_in, int channel_in, int btm_h,
+    const void* weights, const void* grad_out, const void* octree_dev, const void* info, int depth,
+    int num_output, const int* ks, int stride, int nempty, int dtype, void* ws, size_t ws_bytes, hipStream_t s) {
+  OCNN_REQUIRE(data_in && weights && grad_out && octree_dev && info, OCNN_E_BADARG, "null pointer");
+  OCNN_REQUIRE(grad_data || grad_w, OCNN_E_BADARG, "nothing to compute");
+  const Info* o = as_info(info);
+  GradPlan g;
+  int e = make_grad_plan(o, is_deconv, depth, channel_in, num_output, ks, stride, nempty, dtype, &g);
+  if (e) return e;
+  const int in_h = is_deconv ? g.geom.top_h : g.geom.btm_h;    // rows of data_in
+  const int out_h = is_deconv ? g.geom.btm_h : g.geom.top_h;   // rows of grad_out
+  OCNN_REQUIRE(btm_h == in_h, OCNN_E_SHAPE, "input height %d, the octree has %d rows at depth %d", btm_h, in_h, depth);
+  OCNN_REQUIRE(ws && ws_bytes >= g.total_bytes, OCNN_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes, g.total_bytes);
+  if (grad_w) {
+    const float* A = static_cast<const float*>(is_deconv ? data_in : grad_out);
+    const float* X = static_cast<const float*>(is_deconv ? grad_out : data_in);
+    e = run_wgrad(static_cast<float*>(grad_w), A, g.wg_M, X, g.wg_C, o, octree_dev, g.geom, nempty, ws, ws_bytes, s);
+    if (e) return e;
+  }
+  if (grad_data) {
+    // the transposed operator with the same weight buffer; its workspace use starts after the
+    // weight-gradient kernels on the same stream have finished
+    e = run_conv(is_deconv ? 0 : 1, grad_data, grad_out, g.data_cin, out_h, weights, octree_dev, info, g.data_depth,
+        g.data_cout, ks, stride, nempty, dtype, ws, ws_bytes, s);
+    if (e) return e;
+  }
+  return OCNN_OK;
+}
+
 }  // namespace
 }  // namespace ocnn
 
@@ -1258,5 +1501,32 @@ int ocnn_octree_conv_fused(void* top, const void* btm, int channel_in, int btm_h
   return run_conv(is_deconv ? 1 : 0, top, btm, channel_in, btm_h, weights, octree_dev, info, depth, num_output,
       kernel_size, stride, nempty, dtype, workspace_dev, workspace_bytes, as_stream(stream), bias, relu);
 }
+
+int ocnn_conv_grad_workspace_bytes(const void* info, int depth, int channel_in, int num_output,
+    const int* kernel_size, int stride, int nempty, int is_deconv, int dtype, size_t* workspace_bytes) {
+  GradPlan g;
+  int e = make_grad_plan(as_info(info), is_deconv, depth, channel_in, num_output, kernel_size, stride, nempty,
+      dtype, &g);
+  if (e) return e;
+  if (workspace_bytes) *workspace_bytes = g.total_bytes;
+  return OCNN_OK;
+}
+
+int ocnn_octree_conv_grad(void* grad_data, void* grad_weights, const void* data_in, int channel_in, int btm_h,
+    const void* weights, const void* grad_out, const void* octree_dev, const void* info, int depth,
+    int num_output, const int* kernel_size, int stride, int nempty, int dtype, void* workspace_dev,
+    size_t workspace_bytes, ocnn_stream_t stream) {
+  return run_grad(0, grad_data, grad_weights, data_in, channel_in, btm_h, weights, grad_out, octree_dev, info,
+      depth, num_output, kernel_size, stride, nempty, dtype, workspace_dev, workspace_bytes, as_stream(stream));
+}
+
+int ocnn_octree_deconv_grad(void* grad_data, void* grad_weights, const void* data_in, int channel_in, int btm_h,
+    const void* weights, const void* grad_out, const void* octree_dev, const void* info, int depth,
+    int num_output, const int* kernel_size, int stride, int nempty, int dtype, void* workspace_dev,
+    size_t workspace_bytes, ocnn_stream_t stream) {
+  return run_grad(1, grad_data, grad_weights, data_in, channel_in, btm_h, weights, grad_out, octree_dev, info,
+      depth, num_output, kernel_size, stride, nempty, dtype, workspace_dev, workspace_bytes, as_stream(stream));
+}
+
 
 }  // extern "C"

@@ -1,12 +1,13 @@
-"""Forward-only mirrors of the thin Python modules of the reference
+"""Mirrors of the thin Python modules of the reference
 (pytorch/ocnn/octree_conv.py:75-158, octree_pool.py:69-103, octree_pad.py:47-72).
 They add exactly the compositions the reference adds around the extension calls:
 `octree_pad` after a stride-2 convolution, `octree_depad` before a stride-2
-deconvolution, pad / depad around pooling.  Gradients are not implemented."""
+deconvolution, pad / depad around pooling.  Every call goes through the autograd
+functions, so the modules train (fp32) as well as infer."""
 import torch
 from torch import nn
 
-from . import nn as F
+from . import autograd as F
 
 
 def resize_with_last_val(list_in, num=3):
@@ -47,7 +48,7 @@ class OctreeConv(OctreeConvBase):
 
   def forward(self, data, octree):
     assert data.size(1) == self.channel_in
-    conv = F.octree_conv(data, self.weights.detach(), octree, self.depth, self.channel_out,
+    conv = F.octree_conv(data, self.weights, octree, self.depth, self.channel_out,
                          self.kernel_size, self.stride, self.nempty)
     if self.stride == 2 and not self.nempty:
       conv = F.octree_pad(conv, octree, self.depth - 1)
@@ -62,7 +63,7 @@ class OctreeDeconv(OctreeConvBase):
     assert data.size(1) == self.channel_in
     if self.stride == 2 and not self.nempty:
       data = F.octree_depad(data, octree, self.depth)
-    return F.octree_deconv(data, self.weights.detach(), octree, self.depth, self.channel_out,
+    return F.octree_deconv(data, self.weights, octree, self.depth, self.channel_out,
                            self.kernel_size, self.stride, self.nempty)
 
 
@@ -75,7 +76,7 @@ class OctreeConvFast(OctreeConvBase):
   def forward(self, data, octree):
     col = F.octree2col(data, octree, self.depth, self.kernel_size, self.stride, False)
     col = col.view([self.cdim, -1])
-    conv = torch.mm(self.weights.detach(), col)
+    conv = torch.mm(self.weights, col)
     conv = torch.unsqueeze(torch.unsqueeze(conv, 0), -1)
     if self.stride == 2:
       conv = F.octree_pad(conv, octree, self.depth - 1)
@@ -92,7 +93,7 @@ class OctreeDeconvFast(OctreeConvBase):
       data = F.octree_depad(data, octree, depth)
       depth = depth + 1
     data = torch.squeeze(torch.squeeze(data, dim=0), dim=-1)
-    col = torch.mm(self.weights.detach().t(), data)
+    col = torch.mm(self.weights.t(), data)
     col = col.view(self.channel_out, self.kdim, -1)
     return F.col2octree(col, octree, depth, self.kernel_size, self.stride, False)
 

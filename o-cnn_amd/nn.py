@@ -461,6 +461,46 @@ def octree_conv_fused(data_in, weights, bias, relu, octree, depth, num_output, k
                kernel_size, stride, nempty, bias=bias, relu=relu)
 
 
+def _conv_grad(fn, is_deconv, data_in, weights, octree, grad_in, depth, num_output, kernel_size, stride,
+               nempty):
+  octree = _to_dev(octree)
+  info = octree_info(octree)
+  ksc, _ = _ks(kernel_size)
+  data_in, weights, grad_in = data_in.contiguous(), weights.contiguous(), grad_in.contiguous()
+  dt = _dtype_code(data_in)
+  if weights.dtype != data_in.dtype or grad_in.dtype != data_in.dtype:
+    raise TypeError("data, weights and gradient must have the same dtype")
+  channel_in, btm_h = data_in.size(1), data_in.size(2)
+  top_h, need_h, ws_bytes = C.c_int(), C.c_int(), C.c_size_t()
+  _lib.call("ocnn_conv_shape", info.p, depth, channel_in, num_output, ksc, stride, int(nempty),
+            int(is_deconv), dt, C.byref(top_h), C.byref(need_h), None)
+  if grad_in.size(1) != num_output or grad_in.size(2) != top_h.value:
+    raise OcnnError(-3, "gradient shape %s, the operator's output is [1, %d, %d, 1]" %
+                    (tuple(grad_in.shape), num_output, top_h.value))
+  _lib.call("ocnn_conv_grad_workspace_bytes", info.p, depth, channel_in, num_output, ksc, stride,
+            int(nempty), int(is_deconv), dt, C.byref(ws_bytes))
+  ws = _workspace(ws_bytes.value + 256, "conv")
+  base = (ws.data_ptr() + 255) & ~255
+  grad_data = torch.empty_like(data_in)
+  grad_w = torch.empty_like(weights)
+  _lib.call(fn, _ptr(grad_data), _ptr(grad_w), _ptr(data_in), channel_in, btm_h, _ptr(weights),
+            _ptr(grad_in), _ptr(octree), info.p, depth, num_output, ksc, stride, int(nempty), dt,
+            C.c_void_p(base), C.c_size_t(ws_bytes.value), _stream())
+  return [grad_data, grad_w]
+
+
+def octree_conv_grad(data_in, weights, octree, grad_in, depth, num_output, kernel_size, stride, nempty):
+  """pytorch/cpp/octree_conv.cpp:159-189 -> [grad_data, grad_weights] (fp32)."""
+  return _conv_grad("ocnn_octree_conv_grad", False, data_in, weights, octree, grad_in, depth, num_output,
+                    kernel_size, stride, nempty)
+
+
+def octree_deconv_grad(data_in, weights, octree, grad_in, depth, num_output, kernel_size, stride, nempty):
+  """pytorch/cpp/octree_conv.cpp:218-250 -> [grad_data, grad_weights] (fp32)."""
+  return _conv_grad("ocnn_octree_deconv_grad", True, data_in, weights, octree, grad_in, depth, num_output,
+                    kernel_size, stride, nempty)
+
+
 # ---- pad / pool ------------------------------------------------------------------------------------
 def octree_pad(data_in, octree, depth, val=0.0):
   """pytorch/cpp/octree_pad.cpp:6-32."""

@@ -368,6 +368,28 @@ class Checker:
     return self._conv("octree_deconv", True, data, weights, blob, depth, num_output,
                       kernel_size, stride, nempty)
 
+  def _grad(self, name, data, weights, grad_out, blob, depth, num_output, kernel_size, stride, nempty):
+    data, weights, grad_out = _f32(data), _f32(weights), _f32(grad_out)
+    blob = np.ascontiguousarray(blob, dtype=np.uint8)
+    ks = _i32(kernel_size)
+    gd, gw = np.zeros_like(data), np.zeros_like(weights)
+    r = self.fn(name)(_p(gd), _p(gw), _p(data), data.shape[0], data.shape[1], _p(weights), _p(grad_out),
+                      _p(blob), depth, num_output, _p(ks), stride, int(nempty))
+    if r < 0:
+      raise RuntimeError("%s failed: %d" % (name, r))
+    return gd, gw
+
+  def octree_conv_grad(self, data, weights, grad_out, blob, depth, num_output, kernel_size, stride,
+                       nempty=False):
+    """-> (grad_data, grad_weights), pytorch/cpp/octree_conv.cpp:159-189."""
+    return self._grad("octree_conv_grad", data, weights, grad_out, blob, depth, num_output, kernel_size,
+                      stride, nempty)
+
+  def octree_deconv_grad(self, data, weights, grad_out, blob, depth, num_output, kernel_size, stride,
+                         nempty=False):
+    return self._grad("octree_deconv_grad", data, weights, grad_out, blob, depth, num_output, kernel_size,
+                      stride, nempty)
+
 
 def make_points_blob(pts, normals=None, features=None, labels=None):
   """Serialized point cloud (octree/octree/points_info.h:35-39, points.cpp:96-148):

@@ -543,6 +543,77 @@ int orc_octree_deconv(float* top, const float* btm, int channel_in, int btm_h,
   return s.top_h;
 }
 
+
+/* Gradients: OctreeConvGradOp / OctreeDeconvGradOp (pytorch/cpp/octree_conv.cpp:159-250) over
+ * weight_cpu_gemm / backward_cpu_gemm / forward_cpu_gemm (octree_conv.cpp:190-268).
+ *   conv:   grad_w[Co, Ci*K]  = grad_out[Co, H'] * octree2col(data_in)^T
+ *           grad_data         = col2octree(W^T * grad_out)          (== deconv of grad_out)
+ *   deconv: grad_w[Ci, Co*K]  = data_in[Ci, H'] * octree2col(grad_out)^T
+ *           grad_data         = W * octree2col(grad_out)             (== conv of grad_out) */
+static int conv_col(float* col, const float* x, int channel, const void* blob, const ConvShape* s,
+    int ksdim, int stride, int nempty, const int* ni) {
+  const OInfo* o = (const OInfo*)blob;
+  const int* neigh = (const int*)prop_ptr(blob, kNeigh, s->workspace_depth);
+  if (!nempty) {
+    orc_octree2col(col, x, channel, s->workspace_h, ksdim, stride, neigh, ni, s->workspace_h, 0);
+  } else {
+    const int* child = (const int*)prop_ptr(blob, kChild, s->workspace_depth);
+    int* ichild = make_ichild(o, child, s);
+    orc_octree2colP(col, x, channel, s->workspace_h, s->octree_h, ksdim, stride, neigh, ni,
+        child, ichild, s->workspace_h, 0);
+    free(ichild);
+  }
+  return 0;
+}
+int orc_octree_conv_grad(float* grad_data, float* grad_w, const float* data_in, int channel_in, int btm_h,
+    const float* weights, const float* grad_out, const void* blob, int depth, int num_output,
+    const int* ks, int stride, int nempty) {
+  const OInfo* o = (const OInfo*)blob;
+  ConvShape s; int ni[216];
+  if (depth <= 0 || num_output <= 0 || (stride != 1 && stride != 2)) return ORC_E_BADARG;
+  int e = conv_shape(o, depth, stride, nempty, 0, &s); if (e < 0) return e;
+  int nni = orc_get_ni(ks, ni); if (nni < 0) return nni;
+  if (!check_btm_h(o, depth, stride, nempty, 0, btm_h)) return ORC_E_BADARG;
+  int ksdim = ks[0] * ks[1] * ks[2], kdim = ksdim * channel_in;
+  float* col = (float*)malloc(sizeof(float) * (size_t)kdim * (size_t)s.workspace_h + 4);
+  if (!col) return ORC_E_NOMEM;
+  conv_col(col, data_in, channel_in, blob, &s, ksdim, stride, nempty, ni);
+  /* weight_cpu_gemm: weights_diff (zeroed) += top_diff * col^T */
+  orc_sgemm(0, 1, num_output, kdim, s.workspace_h, grad_out, col, 0.0f, grad_w);
+  /* backward_cpu_gemm: col_diff = W^T * top_diff, then col2octree */
+  orc_sgemm(1, 0, kdim, s.workspace_h, num_output, weights, grad_out, 0.0f, col);
+  const int* neigh = (const int*)prop_ptr(blob, kNeigh, s.workspace_depth);
+  if (!nempty) {
+    orc_col2octree(col, grad_data, channel_in, s.workspace_h, ksdim, stride, neigh, ni, s.workspace_h, 0);
+  } else {
+    const int* child = (const int*)prop_ptr(blob, kChild, s.workspace_depth);
+    int* ichild = make_ichild(o, child, &s);
+    orc_col2octreeP(col, grad_data, channel_in, s.workspace_h, s.octree_h, ksdim, stride, neigh, ni,
+        child, ichild, s.workspace_h, 0);
+    free(ichild);
+  }
+  free(col);
+  return btm_h;
+}
+int orc_octree_deconv_grad(float* grad_data, float* grad_w, const float* data_in, int channel_in, int btm_h,
+    const float* weights, const float* grad_out, const void* blob, int depth, int num_output,
+    const int* ks, int stride, int nempty) {
+  const OInfo* o = (const OInfo*)blob;
+  ConvShape s; int ni[216];
+  if (depth <= 0 || num_output <= 0 || (stride != 1 && stride != 2)) return ORC_E_BADARG;
+  int e = conv_shape(o, depth, stride, nempty, 1, &s); if (e < 0) return e;
+  int nni = orc_get_ni(ks, ni); if (nni < 0) return nni;
+  if (!check_btm_h(o, depth, stride, nempty, 1, btm_h)) return ORC_E_BADARG;
+  int ksdim = ks[0] * ks[1] * ks[2], kdim = ksdim * num_output;
+  float* col = (float*)malloc(sizeof(float) * (size_t)kdim * (size_t)s.workspace_h + 4);
+  if (!col) return ORC_E_NOMEM;
+  conv_col(col, grad_out, num_output, blob, &s, ksdim, stride, nempty, ni);
+  orc_sgemm(0, 1, channel_in, kdim, s.workspace_h, data_in, col, 0.0f, grad_w);
+  orc_sgemm(0, 0, channel_in, s.workspace_h, kdim, weights, col, 0.0f, grad_data);
+  free(col);
+  return btm_h;
+}
+
 /* ------------------------------------------------------------------------ */
 /* points2octree: pytorch/cpp/point2octree.cpp:5-34,
  * OctreeInfo::initialize octree/octree/octree_info.cpp:13-73,

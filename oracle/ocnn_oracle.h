@@ -17,6 +17,8 @@
  *   octree2col/col2octree closed form on the full depth-1 layer, adjointness,
  *                         P == pad o col o depad identity, compiled reference
  *   conv / deconv ....... dense zero-padded conv3d on a full layer, adjointness
+ *   conv / deconv grads . <grad_w, W'> == <grad_out, conv(x; W')> for random W' (the op is linear
+ *                         in W), <grad_data, x'> == <grad_out, conv(x'; W)>, dense conv3d autograd
  *   pool / unpool / pad . literal vectors of pytorch/test/test_octree_pool.py
  *   new/grow/update ..... MD5 of the rebuilt octree_2 quoted in
  *                         pytorch/test/test_octree_grow.py
@@ -101,6 +103,15 @@ int orc_octree_conv(float* top, const float* btm, int channel_in, int btm_h,
     const int* kernel_size, int stride, int nempty);
 int orc_octree_deconv(float* top, const float* btm, int channel_in, int btm_h,
     const float* weights, const void* blob, int depth, int num_output,
+    const int* kernel_size, int stride, int nempty);
+
+/* OctreeConvGradOp / OctreeDeconvGradOp, pytorch/cpp/octree_conv.cpp:159-250:
+ * grad_data has the shape of data_in, grad_w the shape of weights. */
+int orc_octree_conv_grad(float* grad_data, float* grad_w, const float* data_in, int channel_in, int btm_h,
+    const float* weights, const float* grad_out, const void* blob, int depth, int num_output,
+    const int* kernel_size, int stride, int nempty);
+int orc_octree_deconv_grad(float* grad_data, float* grad_w, const float* data_in, int channel_in, int btm_h,
+    const float* weights, const float* grad_out, const void* blob, int depth, int num_output,
     const int* kernel_size, int stride, int nempty);
 
 #ifdef __cplusplus

@@ -276,3 +276,71 @@ def test_kernels_vs_compiled_reference(orc, ref, batch4):
   assert np.array_equal(orc.xyz2key(keys, 9), ref.xyz2key(keys, 9))
   assert np.array_equal(orc.key2xyz(keys, 9), ref.key2xyz(keys, 9))
   assert np.array_equal(orc.key2idx(keys), ref.key2idx(keys))
+
+
+@pytest.mark.parametrize("stride", [1, 2])
+@pytest.mark.parametrize("ks", [[3, 3, 3], [2, 2, 2], [3, 1, 1], [1, 1, 1]])
+def test_conv_grads_are_the_adjoints(orc, samples, ks, stride):
+  """The op is bilinear: <grad_w, W'> == <grad_out, conv(x; W')> for every W' and
+  <grad_data, x'> == <grad_out, conv(x'; W)> for every x' (OctreeConvGradOp,
+  pytorch/cpp/octree_conv.cpp:159-189); the same for the deconvolution."""
+  blob = orc.octree_batch([samples["octree_2"], samples["octree_1"]])
+  b = OctreeBlob(blob)
+  Ci, Co, K = 3, 4, ks[0] * ks[1] * ks[2]
+  rng = np.random.default_rng(8)
+  dot = lambda a, c: float(np.vdot(a.astype(np.float64), c.astype(np.float64)))
+  for nempty in (False, True):
+    dc = 4
+    hx = int(b.nnum_nempty[dc] if nempty else b.nnum[dc])
+    x = rng.standard_normal((Ci, hx)).astype(np.float32)
+    w = rng.standard_normal((Co, Ci * K)).astype(np.float32)
+    y = orc.octree_conv(x, w, blob, dc, Co, ks, stride, nempty)
+    g = rng.standard_normal(y.shape).astype(np.float32)
+    gd, gw = orc.octree_conv_grad(x, w, g, blob, dc, Co, ks, stride, nempty)
+    assert gd.shape == x.shape and gw.shape == w.shape
+    for _ in range(3):
+      w2 = rng.standard_normal(w.shape).astype(np.float32)
+      x2 = rng.standard_normal(x.shape).astype(np.float32)
+      assert np.isclose(dot(gw, w2), dot(g, orc.octree_conv(x, w2, blob, dc, Co, ks, stride, nempty)), rtol=1e-4)
+      assert np.isclose(dot(gd, x2), dot(g, orc.octree_conv(x2, w, blob, dc, Co, ks, stride, nempty)), rtol=1e-4)
+    # a single weight entry: grad_w[m, j] == <grad_out, conv(x; e_mj)>
+    m, j = 2, (Ci * K) // 2
+    e = np.zeros_like(w); e[m, j] = 1.0
+    assert np.isclose(gw[m, j], dot(g, orc.octree_conv(x, e, blob, dc, Co, ks, stride, nempty)), rtol=1e-4, atol=1e-5)
+    # deconvolution: input at dd, weights [Cin_d, Cout_d * K]
+    dd = dc if stride == 1 else dc - 1
+    hd = int(b.nnum_nempty[dd] if (nempty or stride == 2) else b.nnum[dd])
+    xd = rng.standard_normal((Co, hd)).astype(np.float32)
+    wd = rng.standard_normal((Co, Ci * K)).astype(np.float32)
+    yd = orc.octree_deconv(xd, wd, blob, dd, Ci, ks, stride, nempty)
+    gy = rng.standard_normal(yd.shape).astype(np.float32)
+    gd, gw = orc.octree_deconv_grad(xd, wd, gy, blob, dd, Ci, ks, stride, nempty)
+    assert gd.shape == xd.shape and gw.shape == wd.shape
+    for _ in range(3):
+      w2 = rng.standard_normal(wd.shape).astype(np.float32)
+      x2 = rng.standard_normal(xd.shape).astype(np.float32)
+      assert np.isclose(dot(gw, w2), dot(gy, orc.octree_deconv(xd, w2, blob, dd, Ci, ks, stride, nempty)), rtol=1e-4)
+      assert np.isclose(dot(gd, x2), dot(gy, orc.octree_deconv(x2, wd, blob, dd, Ci, ks, stride, nempty)), rtol=1e-4)
+
+
+def test_conv_grads_full_layer_match_dense_autograd(orc, samples):
+  """On a full layer the gradients are those of torch's dense conv3d."""
+  depth = 2
+  blob = orc.octree_batch([samples["octree_1"]])
+  n, S = 8 ** depth, 2 ** depth
+  rng = np.random.default_rng(9)
+  Ci, Co = 3, 4
+  x = rng.standard_normal((Ci, n)).astype(np.float32)
+  w = rng.standard_normal((Co, Ci * 27)).astype(np.float32)
+  g = rng.standard_normal((Co, n)).astype(np.float32)
+  gd, gw = orc.octree_conv_grad(x, w, g, blob, depth, Co, [3, 3, 3], 1)
+  xs, ys, zs = morton_to_grid(x, depth)
+  grid = np.zeros((1, Ci, S, S, S), np.float32)
+  grid[0][:, xs, ys, zs] = x
+  gg = np.zeros((1, Co, S, S, S), np.float32)
+  gg[0][:, xs, ys, zs] = g
+  xt = torch.from_numpy(grid).requires_grad_(True)
+  wt = torch.from_numpy(w.reshape(Co, Ci, 3, 3, 3).copy()).requires_grad_(True)
+  torch.nn.functional.conv3d(xt, wt, padding=1).backward(torch.from_numpy(gg))
+  assert np.allclose(gw, wt.grad.numpy().reshape(Co, Ci * 27), atol=1e-4)
+  assert np.allclose(gd, xt.grad.numpy()[0][:, xs, ys, zs], atol=1e-4)
