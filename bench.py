@@ -230,7 +230,7 @@ def main():
     t = timed(lambda: F.octree_conv_grad(x32, w32, octree, gy, 9, C, [3, 3, 3], 1, False), max(2, reps // 2), 1)
     fl = 2 * 2.0 * H9 * 27 * C * C
     extra["conv333_s1_d9_f32_grad"] = {"ms": t, "octants_per_s": H9 / (t * 1e-3), "tflops": fl / (t * 1e-3) / 1e12,
-                                       "frac_mfma_peak": fl / (t * 1e-3) / 1e12 / PEAK_F32}
+                                       "frac_mfma_peak": fl / (t * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS["f32"]}
 
     def hbm(name, t, by):
       extra[name] = {"ms": t, "GBs": by / t / 1e6, "frac_hbm_peak": by / t / 1e6 / PEAK_HBM_GBS}

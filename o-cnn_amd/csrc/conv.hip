@@ -1226,9 +1226,36 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
 // The reduction runs over the columns, so the MFMA k dimension is n: lane (m, kh) loads one
 // float4 of A = columns n0 + 4kh .. + 3, and step j multiplies the column pair (n0 + j,
 // n0 + 4 + j); lane (c, kh) gathers xt[src(n0 + 4kh + j, tap)][c], 128 contiguous bytes per half
-// wavefront.  A wavefront is one slice: it walks every n_slices-th block of 8 columns with its
+// wavefront.  A wavefront is one slice: it walks a contiguous range of blocks of 8 columns with its
 // own accumulators for 3 taps x (MT x NT) 32x32 tiles and writes them to partial[slice]; a second
 // kernel adds the slices in a fixed order, so the result is reproducible (no atomics).
+// Source row for the weight gradient, without branches so that the index loads of all
+// (tap, column) pairs of a block are in flight together; a missing neighbour, a column or a
+// tap out of range all map to row Hin of the row-major copy, which is zero.
+__device__ inline int wgrad_src(const ConvArgs& a, int n, int k) {
+  const bool live = n < a.N && k < a.K;
+  const int nn = min(n, a.N - 1), kk = min(k, a.K - 1);
+  int p;
+  if (a.mode == kModeS2Deconv) {
+    const int node = a.nempty ? a.ichild[nn] : nn;
+    p = (kk == (node & 7)) ? (node >> 3) : -1;
+  } else {
+    int64_t at;
+    if (a.mode == kModeS1) {
+      const int node = a.nempty ? a.ichild[nn] : nn;
+      at = ((int64_t)(node >> 3) << 6) + sibling_slot(node & 7) + a.slot[kk];
+    } else {
+      at = ((int64_t)nn << 6) + a.slot[kk];
+    }
+    p = a.neigh[at];
+    if (a.nempty) {
+      const int c = a.child[max(p, 0)];
+      p = p >= 0 ? c : -1;
+    }
+  }
+  return (live && p >= 0 && p < a.Hin) ? p : a.Hin;
+}
+
 constexpr int kWgTaps = 3;
 
 template <int MT, int NT>
@@ -1250,7 +1277,16 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_f32_kernel(ConvArgs a, cons
         for (int i = 0; i < 16; ++i) acc[t][mt][nt][i] = 0.0f;
   const int nblocks = (a.N + 7) >> 3;
   const bool vec_ok = (a.N & 3) == 0 && (reinterpret_cast<uintptr_t>(A) & 15) == 0;
-  for (int b = slice; b < nblocks; b += n_slices) {
+  // a slice is a contiguous range of column blocks: the 128-byte lines of A a wavefront touches
+  // (one per row, 16 bytes used per block) and the neighbour rows of xt are reused from L1
+  const int per_slice = (nblocks + n_slices - 1) / n_slices;
+  const int b_end = min(nblocks, (slice + 1) * per_slice);
+  // with two column tiles, tile nt holds the channels 2n + nt, so that one 8-byte load per lane
+  // feeds both tiles and a half wavefront reads 256 contiguous bytes of a row
+  const float* xcol = xt + (NT == 2 ? cpass * 64 + 2 * r : cpass * 32 + r);
+  for (int b = slice * per_slice; b < b_end; ++b) {
+    // all source rows of the block with one load: lane (t, column) = (lane >> 3, lane & 7)
+    const int srcv = wgrad_src(a, b * 8 + (lane & 7), tap0 + min(lane >> 3, kWgTaps - 1));
     const int n0 = b * 8 + 4 * kh;
     float av[MT][4];
 #pragma unroll
@@ -1271,19 +1307,19 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_f32_kernel(ConvArgs a, cons
     }
 #pragma unroll
     for (int t = 0; t < kWgTaps; ++t) {
-      const int tap = tap0 + t;
-      int src[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        int sidx = tap < a.K ? conv_src(a, n0 + j, tap) : -1;
-        src[j] = sidx < 0 ? a.Hin : sidx;
-      }
       float bv[4][NT];
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          bv[j][nt] = xt[(int64_t)src[j] * cpad + (cpass * NT + nt) * 32 + r];
+      for (int j = 0; j < 4; ++j) {
+        const int lo = __builtin_amdgcn_readlane(srcv, t * 8 + j);
+        const int hi = __builtin_amdgcn_readlane(srcv, t * 8 + 4 + j);
+        const float* row = xcol + (int64_t)(kh ? hi : lo) * cpad;
+        if (NT == 2) {
+          const float2 v = *reinterpret_cast<const float2*>(row);
+          bv[j][0] = v.x; bv[j][NT - 1] = v.y;
+        } else {
+          bv[j][0] = *row;
+        }
+      }
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -1293,7 +1329,7 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_f32_kernel(ConvArgs a, cons
             acc[t][mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[mt][j], bv[j][nt], acc[t][mt][nt], 0, 0, 0);
     }
   }
-  // partial[slice][tap][m][c]: lanes of a half wavefront write 128 contiguous bytes
+  // partial[slice][tap][m][c]: a half wavefront writes 128 (256) contiguous bytes
 #pragma unroll
   for (int t = 0; t < kWgTaps; ++t) {
     const int tap = tap0 + t;
@@ -1301,13 +1337,15 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_f32_kernel(ConvArgs a, cons
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int m = (mpass * MT + mt) * 32 + 8 * (i / 4) + 4 * kh + (i % 4);
-          const int c = (cpass * NT + nt) * 32 + r;
-          partial[(((int64_t)slice * a.K + tap) * mpad + m) * cpad + c] = acc[t][mt][nt][i];
+      for (int i = 0; i < 16; ++i) {
+        const int m = (mpass * MT + mt) * 32 + 8 * (i / 4) + 4 * kh + (i % 4);
+        float* dst = partial + (((int64_t)slice * a.K + tap) * mpad + m) * cpad;
+        if (NT == 2) {
+          *reinterpret_cast<float2*>(dst + cpass * 64 + 2 * r) = make_float2(acc[t][mt][0][i], acc[t][mt][NT - 1][i]);
+        } else {
+          dst[cpass * 32 + r] = acc[t][mt][0][i];
         }
+      }
   }
 }
 __global__ void conv_wgrad_reduce_kernel(float* __restrict__ G, const float* __restrict__ partial, int n_slices,
@@ -1337,10 +1375,11 @@ void make_wgrad_plan(const ConvPlan& p, int M, int channel_in, int nempty, Wgrad
   w->mpad = w->mpasses * w->MT * 32;
   w->cpad = w->cpasses * w->NT * 32;
   w->tapgroups = (p.taps.count + kWgTaps - 1) / kWgTaps;
-  // about three workgroups per compute unit in total, never more slices than column blocks
+  // one round of resident workgroups (two per compute unit at this register budget), so that
+  // no second, half-empty round trails; never more slices than column blocks
   const int nblocks = (p.top_h + 7) / 8;
   int per_launch = w->tapgroups * w->mpasses * w->cpasses;
-  int groups = (768 + per_launch - 1) / per_launch;
+  int groups = 512 / per_launch;
   int max_groups = (nblocks + 3) / 4;
   if (groups > max_groups) groups = max_groups;
   if (groups < 1) groups = 1;
