@@ -161,6 +161,7 @@ def main():
     conv_case("conv222_s2_d9_bf16", octree, 9, x16, w2.bfloat16(), [2, 2, 2], 2)
     xne = torch.randn(1, C, Hne9, 1, generator=g).to(dev)
     conv_case("conv333_s1_d9_f32_nempty", octree, 9, xne, w32, [3, 3, 3], 1, nempty=True)
+    conv_case("conv333_s1_d9_bf16_nempty", octree, 9, xne.bfloat16(), w16, [3, 3, 3], 1, nempty=True)
     x8 = torch.randn(1, C, Hne8, 1, generator=g).to(dev)
     conv_case("deconv222_s2_d8to9_f32", octree, 8, x8, w2, [2, 2, 2], 2, deconv=True)
 

@@ -27,7 +27,8 @@ class OctreeConvFunction(Function):
   @staticmethod
   def backward(ctx, grad_in):
     data_in, weights, octree = ctx.saved_tensors
-    grad_data, grad_w = F.octree_conv_grad(data_in, weights, octree, grad_in.contiguous(), *ctx.cfg)
+    grad_data, grad_w = F.octree_conv_grad(data_in, weights, octree, grad_in.contiguous(), *ctx.cfg,
+                                           need_data=ctx.needs_input_grad[0], need_weights=ctx.needs_input_grad[1])
     return (grad_data, grad_w) + (None,) * 6
 
 
@@ -42,7 +43,8 @@ class OctreeDeconvFunction(Function):
   @staticmethod
   def backward(ctx, grad_in):
     data_in, weights, octree = ctx.saved_tensors
-    grad_data, grad_w = F.octree_deconv_grad(data_in, weights, octree, grad_in.contiguous(), *ctx.cfg)
+    grad_data, grad_w = F.octree_deconv_grad(data_in, weights, octree, grad_in.contiguous(), *ctx.cfg,
+                                             need_data=ctx.needs_input_grad[0], need_weights=ctx.needs_input_grad[1])
     return (grad_data, grad_w) + (None,) * 6
 
 

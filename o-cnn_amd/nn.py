@@ -462,7 +462,7 @@ def octree_conv_fused(data_in, weights, bias, relu, octree, depth, num_output, k
 
 
 def _conv_grad(fn, is_deconv, data_in, weights, octree, grad_in, depth, num_output, kernel_size, stride,
-               nempty):
+               nempty, need_data=True, need_weights=True):
   octree = _to_dev(octree)
   info = octree_info(octree)
   ksc, _ = _ks(kernel_size)
@@ -481,24 +481,29 @@ def _conv_grad(fn, is_deconv, data_in, weights, octree, grad_in, depth, num_outp
             int(nempty), int(is_deconv), dt, C.byref(ws_bytes))
   ws = _workspace(ws_bytes.value + 256, "conv")
   base = (ws.data_ptr() + 255) & ~255
-  grad_data = torch.empty_like(data_in)
-  grad_w = torch.empty_like(weights)
+  grad_data = torch.empty_like(data_in) if need_data else None
+  grad_w = torch.empty_like(weights) if need_weights else None
+  if grad_data is None and grad_w is None:
+    return [None, None]
   _lib.call(fn, _ptr(grad_data), _ptr(grad_w), _ptr(data_in), channel_in, btm_h, _ptr(weights),
             _ptr(grad_in), _ptr(octree), info.p, depth, num_output, ksc, stride, int(nempty), dt,
             C.c_void_p(base), C.c_size_t(ws_bytes.value), _stream())
   return [grad_data, grad_w]
 
 
-def octree_conv_grad(data_in, weights, octree, grad_in, depth, num_output, kernel_size, stride, nempty):
-  """pytorch/cpp/octree_conv.cpp:159-189 -> [grad_data, grad_weights] (fp32)."""
+def octree_conv_grad(data_in, weights, octree, grad_in, depth, num_output, kernel_size, stride, nempty,
+                     need_data=True, need_weights=True):
+  """pytorch/cpp/octree_conv.cpp:159-189 -> [grad_data, grad_weights] (fp32); a gradient that is
+  not needed is skipped and returned as None."""
   return _conv_grad("ocnn_octree_conv_grad", False, data_in, weights, octree, grad_in, depth, num_output,
-                    kernel_size, stride, nempty)
+                    kernel_size, stride, nempty, need_data, need_weights)
 
 
-def octree_deconv_grad(data_in, weights, octree, grad_in, depth, num_output, kernel_size, stride, nempty):
+def octree_deconv_grad(data_in, weights, octree, grad_in, depth, num_output, kernel_size, stride, nempty,
+                       need_data=True, need_weights=True):
   """pytorch/cpp/octree_conv.cpp:218-250 -> [grad_data, grad_weights] (fp32)."""
   return _conv_grad("ocnn_octree_deconv_grad", True, data_in, weights, octree, grad_in, depth, num_output,
-                    kernel_size, stride, nempty)
+                    kernel_size, stride, nempty, need_data, need_weights)
 
 
 # ---- pad / pool ------------------------------------------------------------------------------------

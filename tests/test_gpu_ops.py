@@ -173,7 +173,19 @@ def test_conv_on_reference_sample_batch(oc, orc, tree):
       exp = orc.octree_conv(x, w, shost, d, 5, ks, stride)
       if stride == 2:
         exp = orc.pad(exp, sb.prop("child", d - 1))
-      assert relerr(y1.cpu().numpy().reshape(exp.shape), exp) < TOL_F32
+      assert relerr(y1.detach().cpu().numpy().reshape(exp.shape), exp) < TOL_F32
+      # gradients of the fused operator == gradients of octree2col + mm (the reference's own
+      # comparison, pytorch/test/test_octree_conv.py:55-72)
+      # (the data gradient of a stride-2 convolution exists for the 2x2x2 kernel only)
+      want_x = stride == 1 or ks == [2, 2, 2]
+      xg1 = xt.clone().requires_grad_(want_x)
+      xg2 = xt.clone().requires_grad_(want_x)
+      gy = torch.randn_like(y1)
+      conv(xg1, sdev).backward(gy)
+      fast(xg2, sdev).backward(gy)
+      if want_x:
+        assert torch.allclose(xg1.grad, xg2.grad, atol=1e-5)
+      assert torch.allclose(conv.weights.grad, fast.weights.grad, atol=1e-4)
       # nempty identity of the reference test: mask -> conv -> select
       mask3 = T(sb.prop("child", d) >= 0).cuda()
       d_out = d if stride == 1 else d - 1
@@ -203,6 +215,13 @@ def test_deconv_layers(oc, orc, tree):
     xt = T(x).cuda().view(1, 3, H, 1)
     y1, y2 = dec(xt, sdev), fast(xt, sdev)
     assert y1.shape == y2.shape and torch.allclose(y1, y2, atol=1e-5)
+    xg1 = xt.clone().requires_grad_(True)
+    xg2 = xt.clone().requires_grad_(True)
+    gy = torch.randn_like(y1)
+    dec(xg1, sdev).backward(gy)
+    fast(xg2, sdev).backward(gy)
+    assert torch.allclose(xg1.grad, xg2.grad, atol=1e-5)
+    assert torch.allclose(dec.weights.grad, fast.weights.grad, atol=1e-4)
 
 
 def test_conv_shape_errors(oc, tree):
