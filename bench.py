@@ -375,6 +375,29 @@ def main():
     out["cpu_baseline"]["points2octree_plus_batch"] = {
         "Mpts_per_s": 0.25 / t, "seconds": t, "cores": 1, "kind": "reference" if ref_ok else "port",
         "bit_exact_vs_gpu": bool(np.array_equal(merged, blob_host))}
+    # the other rows of the path on one host core, same scene (bounded: a few seconds in total)
+    rows = {}
+
+    def cpu_row(name, fn, units, unit):
+      t0 = time.perf_counter()
+      r = fn()
+      dt = time.perf_counter() - t0
+      rows[name] = {"seconds": dt, unit: units / dt, "cores": 1, "kind": "port"}
+      return r
+
+    Cs = 16  # channels of the streaming samples
+    xs = xh[:Cs]
+    pooled, maskh = cpu_row("max_pool_d9", lambda: orc.max_pool(xs), H9, "octants_per_s")
+    cpu_row("max_unpool_d9", lambda: orc.max_unpool(pooled, maskh), H9, "octants_per_s")
+    cpu_row("mask_pool_d9", lambda: orc.mask_pool(xs, maskh), H9, "octants_per_s")
+    child8 = ob.prop("child", 8)
+    padded = cpu_row("pad_d8", lambda: orc.pad(pooled, child8), H8, "octants_per_s")
+    cpu_row("depad_d8", lambda: orc.depad(padded, child8, pooled.shape[1]), H8, "octants_per_s")
+    cpu_row("octree_batch_with_calc_neigh", lambda: orc.octree_batch([single]), sum(ob.nnum[:10]), "nodes_per_s")
+    lab8 = (child8 >= 0).astype(np.int32)
+    upd = cpu_row("octree_update_d8", lambda: orc.octree_update(merged, lab8, 8, 1), H8, "nodes_per_s")
+    del upd
+    out["cpu_baseline"]["rows"] = rows
 
   print(json.dumps(out))
 
