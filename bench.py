@@ -202,6 +202,26 @@ def main():
     extra["points2octree_scene_d9"] = {"ms": t * 1e3, "Mpts_per_s": 0.25 / t,
                                        "GBs": by / t / 1e9, "frac_hbm_peak": by / t / 1e9 / PEAK_HBM_GBS}
 
+    # point-cloud transforms in front of the build (normalise -> rotate/scale/jitter -> clip)
+    def transform_scene():
+      q = F.normalize_points(scene_pts, 1.05, [0.01, 0.0, -0.01])
+      q = F.transform_points(q, [0.05, 0.1, -0.05], [1.1, 0.9, 1.0], [0.05, -0.05, 0.02], 0.0, "")
+      return F.clip_points(q, [-1.0] * 3, [1.0] * 3)
+    transform_scene()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+      transform_scene()
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / reps
+    pbytes = scene_pts.numel()
+    extra["normalize_transform_clip_scene"] = {"ms": t * 1e3, "Mpts_per_s": 0.25 / t,
+                                               "GBs": 6 * pbytes / t / 1e9}
+    t0 = time.perf_counter()
+    for _ in range(reps):
+      F.bounding_sphere(scene_pts, "sphere")
+    extra["bounding_sphere_scene"] = {"ms": (time.perf_counter() - t0) / reps * 1e3}
+
     # depth-7 batch (configs[2]): 16 clouds of 50 000 points
     clouds = [oc.synthetic.shape_cloud(50000, 200 + i) for i in range(16)]
     cl = [points_tensor(*c) for c in clouds]

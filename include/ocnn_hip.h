@@ -184,6 +184,39 @@ int ocnn_octree_deconv_grad(void* grad_data, void* grad_weights, const void* dat
     int depth, int num_output, const int* kernel_size, int stride, int nempty, int dtype,
     void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream);
 
+/* ---- file formats.  A `.octree` / `.points` file is the serialized blob itself
+ * (Octree::read_octree / write_octree, octree/octree/octree.cpp:41-68; Points::read_points /
+ * write_points, points.cpp:9-37).  Files written by a 32-bit-key build carry "_OCTREE_1.0_" and
+ * 4-byte keys: ocnn_upgrade_key64 (upgrade_key64, octree/octree/transform_octree.cpp:433-497)
+ * converts one to the 64-bit layout on the HOST (both buffers are host memory).  With out == NULL
+ * only *out_bytes is filled. */
+int ocnn_upgrade_key64(const void* octree32, size_t bytes, void* out, size_t out_capacity, size_t* out_bytes);
+
+/* ---- point-cloud transforms on the device: pytorch/cpp/transform_points.cpp:7-125 over
+ * PointsParser (octree/octree/points_parser.cpp:42-260).  `points_info` is a HOST copy of the
+ * cloud's 88-byte header.  Results are bit-identical to the host loops.
+ *   ocnn_bounding_sphere   method_box = 0: the sphere of math_functions.cpp:49-108 (the build
+ *                          without Miniball); 1: the bounding-box sphere (:22-30).  out4 (host) =
+ *                          radius, centre; blocks until it has arrived.
+ *   ocnn_normalize_points  translate by -center, scale by 1/radius (:51-71)
+ *   ocnn_transform_points  displace along normals, rotate (angle[3], radians), jitter, scale,
+ *                          orient normals ("", "x", "y", "z", "xyz") (:73-109); out may equal in
+ *   ocnn_clip_points       keeps the points strictly inside the box (:111-125): the kept points
+ *                          are compacted to the front of every array of `out_dev` (a copy of the
+ *                          input otherwise, as the host's in-place compaction leaves it),
+ *                          inbox_mask_dev[pt_num] gets 0/1, out_info (host, 88 bytes) the new
+ *                          header; blocks once for the count. */
+size_t ocnn_points_workspace_bytes(int pt_num);
+int ocnn_bounding_sphere(const void* points_dev, const void* points_info, int method_box, float* out4,
+    void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream);
+int ocnn_normalize_points(void* out_dev, const void* in_dev, const void* points_info, float radius,
+    const float* center, ocnn_stream_t stream);
+int ocnn_transform_points(void* out_dev, const void* in_dev, const void* points_info, const float* angle,
+    const float* scale, const float* jitter, float offset, const char* normal_axis, ocnn_stream_t stream);
+int ocnn_clip_points(void* out_dev, void* out_info, int* inbox_mask_dev, const void* in_dev,
+    const void* points_info, const float* bbmin, const float* bbmax, void* workspace_dev,
+    size_t workspace_bytes, ocnn_stream_t stream);
+
 /* ---- octree construction on the device: points2octree + octree_batch fused.
  * Replaces Octree::build (octree/octree/octree.cpp:74-121) driven as in
  * pytorch/cpp/point2octree.cpp:5-34, and merge_octrees

@@ -140,4 +140,54 @@ int ocnn_info_location(const void* info, int ptype) { return as_info(info)->loca
 int64_t ocnn_info_ptr_dis(const void* info, int ptype, int d) { return as_info(info)->ptr_dis(ptype, d); }
 int64_t ocnn_info_sizeof_octree(const void* info) { return as_info(info)->sizeof_octree(); }
 
+// upgrade_key64, octree/octree/transform_octree.cpp:433-497: a file written by a 32-bit-key build
+// ("_OCTREE_1.0_": 4-byte keys) converted to the 64-bit-key layout every operator expects.
+// A host-side format conversion done once when a file is loaded; both buffers are host memory.
+int ocnn_upgrade_key64(const void* octree32, size_t bytes, void* out, size_t out_capacity, size_t* out_bytes) {
+  OCNN_REQUIRE(octree32 && out_bytes, OCNN_E_BADARG, "null pointer");
+  OCNN_REQUIRE(bytes >= sizeof(Info), OCNN_E_FORMAT, "blob shorter than its header");
+  const Info* in = as_info(octree32);
+  OCNN_REQUIRE(memcmp(in->magic, "_OCTREE_1.0_", 13) == 0, OCNN_E_FORMAT, "octree magic is not _OCTREE_1.0_");
+  OCNN_REQUIRE(in->depth >= 0 && in->depth <= 16, OCNN_E_FORMAT, "depth %d not in [0,16]", in->depth);
+  OCNN_REQUIRE((size_t)in->ptr_dis_[6] <= bytes, OCNN_E_FORMAT, "blob shorter than its header says");
+  Info o = *in;
+  memcpy(o.magic, "_OCTREE_2.0_", 13);
+  o.set_ptr_dis();
+  *out_bytes = (size_t)o.sizeof_octree();
+  if (!out) return OCNN_OK;  // size query
+  OCNN_REQUIRE(out_capacity >= *out_bytes, OCNN_E_WORKSPACE, "output %zu < %zu bytes", out_capacity, *out_bytes);
+  memset(out, 0, *out_bytes);
+  memcpy(out, &o, sizeof(o));
+  const char* src = static_cast<const char*>(octree32);
+  char* dst = static_cast<char*>(out);
+  const int num = o.total_nnum(), depth = o.depth;
+  const uint32_t* key_in = reinterpret_cast<const uint32_t*>(src + in->ptr_dis_[0]);
+  uint64_t* key_out = reinterpret_cast<uint64_t*>(dst + o.ptr_dis(OCNN_KEY, 0));
+  for (int i = 0; i < num; ++i) {
+    if (o.key2xyz) {  // four 8-bit fields widen to four 16-bit fields
+      uint8_t f8[4];
+      uint16_t f16[4];
+      memcpy(f8, key_in + i, 4);
+      for (int j = 0; j < 4; ++j) f16[j] = f8[j];
+      memcpy(key_out + i, f16, 8);
+    } else {
+      key_out[i] = key_in[i];
+    }
+  }
+  memcpy(dst + o.ptr_dis(OCNN_CHILD, 0), src + in->ptr_dis_[1], sizeof(int) * (size_t)num);
+  const int props[3] = {OCNN_FEATURE, OCNN_LABEL, OCNN_SPLIT};
+  for (int q = 0; q < 3; ++q) {
+    const int p = props[q];
+    if (!o.has(p)) continue;
+    const int ch = p == OCNN_FEATURE ? o.channel(p) : 1;
+    const int d0 = o.location(p) == depth ? depth : 0;
+    for (int d = d0; d <= depth; ++d) {
+      int64_t dis_in = in->ptr_dis_[Info::index_of(p)];
+      if (o.location(p) == -1) dis_in += (int64_t)in->nnum_cum[d] * o.channel(p) * 4;
+      memcpy(dst + o.ptr_dis(p, d), src + dis_in, sizeof(float) * (size_t)o.nnum[d] * ch);
+    }
+  }
+  return OCNN_OK;
+}
+
 }  // extern "C"

@@ -262,6 +262,124 @@ def points_new(pts, normals=None, features=None, labels=None):
   return out
 
 
+# ---- point-cloud transforms (pytorch/cpp/transform_points.cpp) ---------------------------------
+def _points_hdr(points):
+  hdr = getattr(points, "_ocnn_points_info", None)
+  if hdr is None:
+    hdr = _points_header(points)
+    points._ocnn_points_info = hdr
+  return hdr
+
+
+def _f3(v):
+  v = [float(x) for x in v]
+  while len(v) < 3:
+    v.append(v[-1])
+  return (C.c_float * 3)(*v[:3])
+
+
+def _points_ws(hdr):
+  nbytes = _lib.get().ocnn_points_workspace_bytes(int(hdr[16:20].view(np.int32)[0]))
+  ws = _workspace(nbytes + 256, "points")
+  return C.c_void_p((ws.data_ptr() + 255) & ~255), C.c_size_t(nbytes)
+
+
+def bounding_sphere(points, method="sphere"):
+  """-> [radius, cx, cy, cz] (pytorch/cpp/transform_points.cpp:7-35).  'sphere' is the reference
+  build without Miniball (octree/octree/math_functions.cpp:49-108), anything else the sphere
+  around the bounding box."""
+  points = _to_dev(points)
+  hdr = _points_hdr(points)
+  out = (C.c_float * 4)()
+  base, nbytes = _points_ws(hdr)
+  _lib.call("ocnn_bounding_sphere", _ptr(points), C.c_void_p(hdr.ctypes.data), int(method != "sphere"), out,
+            base, nbytes, _stream())
+  return [float(x) for x in out]
+
+
+def normalize_points(points, radius, center):
+  """pytorch/cpp/transform_points.cpp:51-71."""
+  points = _to_dev(points)
+  hdr = _points_hdr(points)
+  out = torch.empty_like(points)
+  _lib.call("ocnn_normalize_points", _ptr(out), _ptr(points), C.c_void_p(hdr.ctypes.data), C.c_float(radius),
+            _f3(center), _stream())
+  out._ocnn_points_info = hdr
+  return out
+
+
+def transform_points(points, angle, scale, jitter, offset=0.0, normal_axis=""):
+  """pytorch/cpp/transform_points.cpp:73-109 (angles in radians)."""
+  points = _to_dev(points)
+  hdr = _points_hdr(points)
+  out = torch.empty_like(points)
+  _lib.call("ocnn_transform_points", _ptr(out), _ptr(points), C.c_void_p(hdr.ctypes.data), _f3(angle), _f3(scale),
+            _f3(jitter), C.c_float(offset), normal_axis.encode(), _stream())
+  out._ocnn_points_info = hdr
+  return out
+
+
+def clip_points(points, bbmin, bbmax):
+  """-> [points, inbox_mask int32] (pytorch/cpp/transform_points.cpp:111-125); the mask stays on
+  the device."""
+  points = _to_dev(points)
+  hdr = _points_hdr(points)
+  npt = int(hdr[16:20].view(np.int32)[0])
+  out = torch.empty_like(points)
+  mask = torch.empty(npt, dtype=torch.int32, device=points.device)
+  new_hdr = np.zeros(_lib.POINTS_INFO_BYTES, np.uint8)
+  base, nbytes = _points_ws(hdr)
+  _lib.call("ocnn_clip_points", _ptr(out), C.c_void_p(new_hdr.ctypes.data), _ptr(mask), _ptr(points),
+            C.c_void_p(hdr.ctypes.data), _f3(bbmin), _f3(bbmax), base, nbytes, _stream())
+  out._ocnn_points_info = new_hdr
+  return [out, mask]
+
+
+# ---- files ------------------------------------------------------------------------------------
+def upgrade_key64(octree32):
+  """upgrade_key64 (octree/octree/transform_octree.cpp:433-497) on a host uint8 tensor / array."""
+  raw = np.ascontiguousarray(octree32.cpu().numpy() if torch.is_tensor(octree32) else octree32, dtype=np.uint8)
+  nbytes = C.c_size_t()
+  _lib.call("ocnn_upgrade_key64", C.c_void_p(raw.ctypes.data), C.c_size_t(raw.size), None, C.c_size_t(0),
+            C.byref(nbytes))
+  out = np.empty(nbytes.value, np.uint8)
+  _lib.call("ocnn_upgrade_key64", C.c_void_p(raw.ctypes.data), C.c_size_t(raw.size), C.c_void_p(out.ctypes.data),
+            C.c_size_t(out.size), C.byref(nbytes))
+  return torch.from_numpy(out)
+
+
+def read_octree(path):
+  """A `.octree` file is the serialized blob (Octree::read_octree, octree/octree/octree.cpp:41-55);
+  a file from a 32-bit-key build is upgraded on the way in.  Returns a host uint8 tensor."""
+  raw = np.fromfile(path, dtype=np.uint8)
+  if raw.size < INFO_BYTES:
+    raise OcnnError(-6, "%s: shorter than an octree header" % path)
+  if bytes(raw[:12]) == b"_OCTREE_1.0_":
+    return upgrade_key64(raw)
+  _Info(raw)  # validates the header
+  return torch.from_numpy(raw)
+
+
+def write_octree(octree, path):
+  """Octree::write_octree, octree/octree/octree.cpp:57-68."""
+  octree.cpu().numpy().tofile(path)
+
+
+def read_points(path):
+  """Points::read_points, octree/octree/points.cpp:9-27 -> host uint8 tensor."""
+  raw = np.fromfile(path, dtype=np.uint8)
+  if raw.size < _lib.POINTS_INFO_BYTES or bytes(raw[:12]) != b"_POINTS_1.0_":
+    raise OcnnError(-6, "%s: not a _POINTS_1.0_ file" % path)
+  out = torch.from_numpy(raw)
+  out._ocnn_points_info = raw[:_lib.POINTS_INFO_BYTES].copy()
+  return out
+
+
+def write_points(points, path):
+  """Points::write_points, octree/octree/points.cpp:29-37."""
+  points.cpu().numpy().tofile(path)
+
+
 # ---- properties ------------------------------------------------------------------------
 def octree_property(octree, property, depth=0):
   """pytorch/cpp/octree_property.cpp:11-344."""

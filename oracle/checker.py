@@ -125,7 +125,8 @@ class Checker:
     else:
       raise ValueError(prefix)
     for n in ("fetch", "points2octree", "octree_batch", "octree_sample",
-              "octree_new", "octree_grow", "octree_update", "octree_set_property"):
+              "octree_new", "octree_grow", "octree_update", "octree_set_property",
+              "normalize_points", "transform_points", "clip_points", "upgrade_key64"):
       f = getattr(self.lib, prefix + "_" + n, None)
       if f is not None:
         f.restype = C.c_int64
@@ -158,10 +159,41 @@ class Checker:
         _p(bmax) if bmax is not None else None)
     return self._fetch(sz)
 
+  # ---- point-cloud transforms (pytorch/cpp/transform_points.cpp) --------------------------
+  def bounding_sphere(self, points_blob, method="sphere"):
+    pb = np.ascontiguousarray(points_blob, dtype=np.uint8)
+    out = np.zeros(4, np.float32)
+    if self.fn("bounding_sphere")(_p(pb), int(method != "sphere"), _p(out)) < 0:
+      raise RuntimeError("bounding_sphere failed")
+    return out
+
+  def normalize_points(self, points_blob, radius, center):
+    pb = np.ascontiguousarray(points_blob, dtype=np.uint8)
+    return self._fetch(self.fn("normalize_points")(_p(pb), C.c_int64(pb.size), C.c_float(radius),
+                                                   _p(_f32(center))))
+
+  def transform_points(self, points_blob, angle, scale, jitter, offset=0.0, normal_axis=""):
+    pb = np.ascontiguousarray(points_blob, dtype=np.uint8)
+    return self._fetch(self.fn("transform_points")(
+        _p(pb), C.c_int64(pb.size), _p(_f32(angle)), _p(_f32(scale)), _p(_f32(jitter)),
+        C.c_float(offset), normal_axis.encode()))
+
+  def clip_points(self, points_blob, bbmin, bbmax):
+    pb = np.ascontiguousarray(points_blob, dtype=np.uint8)
+    npt = int(pb[16:20].view(np.int32)[0])
+    mask = np.zeros(npt, np.int32)
+    out = self._fetch(self.fn("clip_points")(_p(pb), C.c_int64(pb.size), _p(_f32(bbmin)), _p(_f32(bbmax)),
+                                             _p(mask)))
+    return out, mask
+
   def octree_batch(self, blobs):
     blobs = [np.ascontiguousarray(b, dtype=np.uint8) for b in blobs]
     arr = (C.c_void_p * len(blobs))(*[b.ctypes.data for b in blobs])
     return self._fetch(self.fn("octree_batch")(arr, len(blobs)))
+
+  def upgrade_key64(self, blob32):
+    b = np.ascontiguousarray(blob32, dtype=np.uint8)
+    return self._fetch(self.fn("upgrade_key64")(_p(b), C.c_int64(b.size)))
 
   def octree_sample(self, name):
     return self._fetch(self.fn("octree_sample")(name.encode()))

@@ -7,6 +7,9 @@
 #include "ocnn_oracle.h"
 
 #include <math.h>
+#include <float.h>
+#define ORC_COS(x) ((float)cos((double)(x)))
+#define ORC_SIN(x) ((float)sin((double)(x)))
 #include <stddef.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -1329,6 +1332,241 @@ int64_t orc_points2octree(const void* points_blob, int depth, int full_depth,
     free(t.pts[d]); free(t.dis[d]); free(t.nerr[d]); free(t.derr[d]); free(t.split[d]); free(t.dnum[d]); free(t.didx[d]);
   }
   free(pts_scaled); free(node_keys); free(sorted_idx); free(unique_idx);
+  return sz;
+}
+
+
+/* ------------------------------------------------------------------------ */
+/* Point-cloud transforms: pytorch/cpp/transform_points.cpp:7-125 over
+ * PointsParser (octree/octree/points_parser.cpp:42-260) and
+ * math_functions.cpp:49-251.  Each works on a copy of the blob. */
+static float* pprop(char* blob, int bit) { /* points_parser.cpp:22-36 */
+  PInfo* pi = (PInfo*)blob;
+  int idx = 0; while ((1 << idx) != bit) ++idx;
+  if (!(pi->content_flags & bit)) return NULL;
+  return (float*)(blob + pi->ptr_dis[idx]);
+}
+static void bounding_box(float* bbmin, float* bbmax, const float* pt, int npt) { /* math_functions.cpp:113-128 */
+  if (npt < 1) return;
+  for (int i = 0; i < 3; ++i) bbmin[i] = bbmax[i] = pt[i];
+  for (int i = 1; i < npt; ++i)
+    for (int j = 0; j < 3; ++j) {
+      float tmp = pt[3 * i + j];
+      if (tmp < bbmin[j]) bbmin[j] = tmp;
+      if (tmp > bbmax[j]) bbmax[j] = tmp;
+    }
+}
+/* the build without Miniball, math_functions.cpp:49-108 */
+static void bounding_sphere(float* radius_out, float* center, const float* pt, int npt) {
+  float bb[3][2] = { { FLT_MAX, -FLT_MAX }, { FLT_MAX, -FLT_MAX }, { FLT_MAX, -FLT_MAX } };
+  int id[6] = { 0, 0, 0, 0, 0, 0 };
+  for (int i = 0; i < 3 * npt; i += 3)
+    for (int a = 0; a < 3; ++a) {
+      if (pt[i + a] < bb[a][0]) { id[2 * a] = i; bb[a][0] = pt[i + a]; }
+      if (pt[i + a] > bb[a][1]) { id[2 * a + 1] = i; bb[a][1] = pt[i + a]; }
+    }
+  float radius = 0; int choose = -1;
+  for (int i = 0; i < 3; i++) {
+    float dx = pt[id[2 * i]] - pt[id[2 * i + 1]];
+    float dy = pt[id[2 * i] + 1] - pt[id[2 * i + 1] + 1];
+    float dz = pt[id[2 * i] + 2] - pt[id[2 * i + 1] + 2];
+    float r2 = dx * dx + dy * dy + dz * dz;
+    if (r2 > radius) { radius = r2; choose = 2 * i; }
+  }
+  if (choose < 0) choose = 0; /* all points coincide: the reference reads id[-1] (undefined) */
+  for (int c = 0; c < 3; ++c) center[c] = 0.5f * (pt[id[choose] + c] + pt[id[choose + 1] + c]);
+  float radius2 = radius * 0.25f;
+  radius = sqrtf(radius2);
+  for (int i = 0; i < 3 * npt; i += 3) {
+    float dx = pt[i] - center[0], dy = pt[i + 1] - center[1], dz = pt[i + 2] - center[2];
+    float dis2 = dx * dx + dy * dy + dz * dz;
+    if (dis2 > radius2) {
+      float old_to_p = (float)sqrt((double)dis2);
+      radius = (radius + old_to_p) * 0.5f;
+      radius2 = radius * radius;
+      float old_to_new = old_to_p - radius;
+      for (int c = 0; c < 3; ++c) center[c] = (radius * center[c] + old_to_new * pt[i + c]) / old_to_p;
+    }
+  }
+  *radius_out = radius;
+}
+int orc_bounding_sphere(const void* blob, int method_box, float* out4) {
+  const PInfo* pi = (const PInfo*)blob;
+  if (strcmp(pi->magic, "_POINTS_1.0_") != 0 || pi->pt_num <= 0) return ORC_E_BADARG;
+  const float* pt = (const float*)((const char*)blob + pi->ptr_dis[0]);
+  float radius = 0.0f, center[3] = { 0.0f, 0.0f, 0.0f };
+  if (!method_box) bounding_sphere(&radius, center, pt, pi->pt_num);
+  else {
+    float bbmin[3] = { 0, 0, 0 }, bbmax[3] = { 0, 0, 0 };
+    bounding_box(bbmin, bbmax, pt, pi->pt_num);
+    for (int j = 0; j < 3; ++j) {
+      center[j] = (bbmax[j] + bbmin[j]) / 2.0f;
+      float width = (bbmax[j] - bbmin[j]) / 2.0f;
+      radius += width * width;
+    }
+    radius = sqrtf(radius + 1.0e-20f);
+  }
+  out4[0] = radius; out4[1] = center[0]; out4[2] = center[1]; out4[3] = center[2];
+  return 0;
+}
+static char* points_copy(const void* blob, int64_t bytes) {
+  const PInfo* pi = (const PInfo*)blob;
+  if (strcmp(pi->magic, "_POINTS_1.0_") != 0 || pi->pt_num <= 0) return NULL;
+  char* out = result_alloc(bytes);
+  if (out) memcpy(out, blob, (size_t)bytes);
+  return out;
+}
+static void pts_translate(char* b, const float* t) { /* points_parser.cpp:42-51 */
+  float* pt = pprop(b, pPoint); int npt = ((PInfo*)b)->pt_num;
+  for (int i = 0; i < npt; ++i) for (int m = 0; m < 3; ++m) pt[3 * i + m] += t[m];
+}
+static void normalize_nx3(float* p, int npt) { /* math_functions.cpp:242-251 */
+  for (int i = 0; i < npt; ++i) {
+    float inv = 1.0f / (norm2f(p + 3 * i, 3) + 1.0e-15f);
+    for (int m = 0; m < 3; ++m) p[3 * i + m] = p[3 * i + m] * inv;
+  }
+}
+static void pts_scale(char* b, const float* s) { /* points_parser.cpp:75-101 */
+  if ((s[0] == 1.0f && s[1] == 1.0f && s[2] == 1.0f) || s[0] == 0.0f || s[1] == 0.0f || s[2] == 0.0f) return;
+  float* pt = pprop(b, pPoint); int npt = ((PInfo*)b)->pt_num;
+  for (int i = 0; i < npt; ++i) for (int j = 0; j < 3; ++j) pt[3 * i + j] *= s[j];
+  if (s[0] == s[1] && s[0] == s[2]) return;
+  const float t[3] = { 1.0f / s[0], 1.0f / s[1], 1.0f / s[2] };
+  float* nm = pprop(b, pNormal);
+  if (nm) {
+    for (int i = 0; i < npt; ++i) for (int j = 0; j < 3; ++j) nm[3 * i + j] *= t[j];
+    normalize_nx3(nm, npt);
+  }
+}
+static void matrix_prod(float* Cm, const float* A, const float* B, int M, int N, int K) { /* math_functions.cpp:185-196 */
+  for (int n = 0; n < N; ++n)
+    for (int m = 0; m < M; ++m) {
+      Cm[n * M + m] = 0;
+      for (int k = 0; k < K; ++k) Cm[n * M + m] += A[k * M + m] * B[n * K + k];
+    }
+}
+void orc_rotation_matrix(float* rot, const float* angle) { /* math_functions.cpp:148-158 */
+  float cosx = ORC_COS(angle[0]), sinx = ORC_SIN(angle[0]);
+  float cosy = ORC_COS(angle[1]), siny = ORC_SIN(angle[1]);
+  float cosz = ORC_COS(angle[2]), sinz = ORC_SIN(angle[2]);
+  const float rotx[9] = { 1.0f, 0, 0, 0, cosx, sinx, 0, -sinx, cosx };
+  const float roty[9] = { cosy, 0, -siny, 0, 1.0f, 0, siny, 0, cosy };
+  const float rotz[9] = { cosz, sinz, 0, -sinz, cosz, 0, 0, 0, 1.0f };
+  float tmp[9];
+  matrix_prod(tmp, rotx, roty, 3, 3, 3);
+  matrix_prod(rot, tmp, rotz, 3, 3, 3);
+}
+static void pts_rotate(char* b, const float* angles) { /* points_parser.cpp:118-131 */
+  float rot[9];
+  orc_rotation_matrix(rot, angles);
+  int npt = ((PInfo*)b)->pt_num;
+  float* tmp = (float*)malloc(sizeof(float) * 3 * (size_t)npt);
+  float* pt = pprop(b, pPoint);
+  matrix_prod(tmp, rot, pt, 3, npt, 3);
+  memcpy(pt, tmp, sizeof(float) * 3 * (size_t)npt);
+  float* nm = pprop(b, pNormal);
+  if (nm) { matrix_prod(tmp, rot, nm, 3, npt, 3); memcpy(nm, tmp, sizeof(float) * 3 * (size_t)npt); }
+  free(tmp);
+}
+int64_t orc_normalize_points(const void* blob, int64_t bytes, float radius, const float* center) {
+  char* b = points_copy(blob, bytes); if (!b) return ORC_E_BADARG;
+  const float dis[3] = { -center[0], -center[1], -center[2] };
+  if (dis[0] != 0.0f || dis[1] != 0.0f || dis[2] != 0.0f) pts_translate(b, dis);
+  const float inv = 1.0f / radius;
+  const float scale[3] = { inv, inv, inv };
+  if (scale[0] != 1.0f || scale[1] != 1.0f || scale[2] != 1.0f) pts_scale(b, scale);
+  return bytes;
+}
+int64_t orc_transform_points(const void* blob, int64_t bytes, const float* angle, const float* scale,
+    const float* jitter, float offset, const char* normal_axis) {
+  char* b = points_copy(blob, bytes); if (!b) return ORC_E_BADARG;
+  const float kEPS = 1.0e-10f;
+  const int npt = ((PInfo*)b)->pt_num;
+  float* pt = pprop(b, pPoint); float* nm = pprop(b, pNormal);
+  if (offset > kEPS && nm) /* displace, points_parser.cpp:53-65 */
+    for (int i = 0; i < npt; ++i) for (int m = 0; m < 3; ++m) pt[3 * i + m] += nm[3 * i + m] * offset;
+  if (fabs(angle[0]) > kEPS || fabs(angle[1]) > kEPS || fabs(angle[2]) > kEPS) pts_rotate(b, angle);
+  if (fabs(jitter[0]) > kEPS || fabs(jitter[1]) > kEPS || fabs(jitter[2]) > kEPS) pts_translate(b, jitter);
+  if (scale[0] != 1.0f || scale[1] != 1.0f || scale[2] != 1.0f) pts_scale(b, scale);
+  if (normal_axis && normal_axis[0] && nm) { /* orient_normal, points_parser.cpp:228-260 */
+    if (!strcmp(normal_axis, "x") || !strcmp(normal_axis, "y") || !strcmp(normal_axis, "z")) {
+      int j = normal_axis[0] - 'x';
+      for (int i = 0; i < npt; ++i)
+        if (nm[3 * i + j] < 0) for (int c = 0; c < 3; ++c) nm[3 * i + c] = -nm[3 * i + c];
+    } else if (!strcmp(normal_axis, "xyz")) {
+      for (int i = 0; i < 3 * npt; ++i) if (nm[i] < 0) nm[i] = -nm[i];
+    }
+  }
+  return bytes;
+}
+int64_t orc_clip_points(const void* blob, int64_t bytes, const float* bbmin, const float* bbmax, int* in_bbox) {
+  char* b = points_copy(blob, bytes); if (!b) return ORC_E_BADARG; /* points_parser.cpp:153-194 */
+  PInfo* pi = (PInfo*)b;
+  int npt = pi->pt_num, inside = 0;
+  float* pts = pprop(b, pPoint);
+  for (int i = 0; i < npt; ++i) {
+    in_bbox[i] = bbmin[0] < pts[3 * i] && pts[3 * i] < bbmax[0] && bbmin[1] < pts[3 * i + 1] && pts[3 * i + 1] < bbmax[1] &&
+        bbmin[2] < pts[3 * i + 2] && pts[3 * i + 2] < bbmax[2];
+    inside += in_bbox[i];
+  }
+  if (inside == npt) return bytes;
+  if (inside == 0) { inside = 1; in_bbox[0] = 1; for (int i = 0; i < 3; ++i) pts[i] = bbmin[i]; }
+  for (int t = 0; t < 4; ++t) {
+    if (!(pi->content_flags & (1 << t)) || pi->channels[t] == 0) continue;
+    int ch = pi->channels[t];
+    float* p = (float*)(b + pi->ptr_dis[t]);
+    for (int i = 0, j = 0; i < npt; ++i) {
+      if (!in_bbox[i]) continue;
+      for (int c = 0; c < ch; ++c) p[j * ch + c] = p[i * ch + c];
+      j++;
+    }
+  }
+  pi->pt_num = inside;
+  return bytes;
+}
+
+
+/* ------------------------------------------------------------------------ */
+/* upgrade_key64, octree/octree/transform_octree.cpp:433-497: a blob written by a
+ * 32-bit-key build ("_OCTREE_1.0_", 4-byte keys) -> the 64-bit-key layout. */
+int64_t orc_upgrade_key64(const void* blob32, int64_t bytes) {
+  const OInfo* in = (const OInfo*)blob32;
+  if (bytes < (int64_t)sizeof(OInfo) || strcmp(in->magic, "_OCTREE_1.0_") != 0) return ORC_E_BADARG;
+  OInfo o = *in;
+  strcpy(o.magic, kMagic);
+  set_ptr_dis(&o);
+  const int sz = sizeof_octree(&o);
+  char* out = result_alloc(sz);
+  if (!out) return ORC_E_NOMEM;
+  memcpy(out, &o, sizeof(o));
+  const char* src = (const char*)blob32;
+  const int num = total_nnum(&o), depth = o.depth;
+  /* keys: widened one by one; packed xyz keys widen each of their four fields */
+  const uint32_t* key_in = (const uint32_t*)(src + in->ptr_dis[0]);
+  uint64_t* key_out = (uint64_t*)prop_ptr(out, kKey, 0);
+  for (int i = 0; i < num; ++i) {
+    if (o.key2xyz) {
+      uint8_t f8[4]; uint16_t f16[4];
+      memcpy(f8, key_in + i, 4);
+      for (int j = 0; j < 4; ++j) f16[j] = (uint16_t)f8[j];
+      memcpy(key_out + i, f16, 8);
+    } else key_out[i] = (uint64_t)key_in[i];
+  }
+  memcpy(prop_ptr(out, kChild, 0), src + in->ptr_dis[1], sizeof(int) * (size_t)num);
+  const int props[3] = { kFeature, kLabel, kSplit };
+  for (int q = 0; q < 3; ++q) {
+    const int p = props[q];
+    if (!has_prop(&o, p)) continue;
+    const int idx = prop_index(p);
+    const int ch = p == kFeature ? channel_of(&o, p) : 1;
+    const int d0 = location_of(&o, p) == depth ? depth : 0;
+    for (int d = d0; d <= depth; ++d) {
+      /* the input's per-depth offset follows octree_info.cpp:157-167 with ITS ptr_dis */
+      int dis_in = in->ptr_dis[idx];
+      if (location_of(&o, p) == -1) dis_in += in->nnum_cum[d] * channel_of(&o, p) * 4;
+      memcpy(prop_ptr(out, p, d), src + dis_in, sizeof(float) * (size_t)o.nnum[d] * ch);
+    }
+  }
   return sz;
 }
 

@@ -19,6 +19,10 @@
  *   conv / deconv ....... dense zero-padded conv3d on a full layer, adjointness
  *   conv / deconv grads . <grad_w, W'> == <grad_out, conv(x; W')> for random W' (the op is linear
  *                         in W), <grad_data, x'> == <grad_out, conv(x'; W)>, dense conv3d autograd
+ *   upgrade_key64 ....... the reference's six embedded 32-bit sample blobs -> their 64-bit
+ *                         forms (golden fixture), compiled reference on downgraded blobs
+ *   point transforms .... compiled reference byte for byte; rotation = product of the three axis
+ *                         rotations (closed form), clip = boolean mask + compaction (numpy)
  *   pool / unpool / pad . literal vectors of pytorch/test/test_octree_pool.py
  *   new/grow/update ..... MD5 of the rebuilt octree_2 quoted in
  *                         pytorch/test/test_octree_grow.py
@@ -104,6 +108,19 @@ int orc_octree_conv(float* top, const float* btm, int channel_in, int btm_h,
 int orc_octree_deconv(float* top, const float* btm, int channel_in, int btm_h,
     const float* weights, const void* blob, int depth, int num_output,
     const int* kernel_size, int stride, int nempty);
+
+/* upgrade_key64, octree/octree/transform_octree.cpp:433-497 (result through orc_fetch) */
+int64_t orc_upgrade_key64(const void* blob32, int64_t bytes);
+
+/* Point-cloud transforms, pytorch/cpp/transform_points.cpp:7-125.  The blob-producing calls
+ * return the size of the transformed copy (orc_fetch). */
+int orc_bounding_sphere(const void* points_blob, int method_box, float* out4);
+int64_t orc_normalize_points(const void* points_blob, int64_t bytes, float radius, const float* center);
+int64_t orc_transform_points(const void* points_blob, int64_t bytes, const float* angle, const float* scale,
+    const float* jitter, float offset, const char* normal_axis);
+int64_t orc_clip_points(const void* points_blob, int64_t bytes, const float* bbmin, const float* bbmax,
+    int* inbox_mask);
+void orc_rotation_matrix(float* rot, const float* angle);
 
 /* OctreeConvGradOp / OctreeDeconvGradOp, pytorch/cpp/octree_conv.cpp:159-250:
  * grad_data has the shape of data_in, grad_w the shape of weights. */

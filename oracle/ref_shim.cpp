@@ -15,6 +15,11 @@
 #include <octree_nn.h>
 #include <octree_samples.h>
 #include <points.h>
+#include <math_functions.h>
+#include <transform_octree.h>
+
+#include <cmath>
+#include <string>
 
 #include <cstdint>
 #include <cstring>
@@ -70,6 +75,13 @@ int64_t ref_octree_sample(const char* name) {
   if (!p || sz == 0) return -1;
   g_last.assign((const char*)p, (const char*)p + sz);
   return (int64_t)sz;
+}
+
+// octree/octree/transform_octree.cpp:433-497: 32-bit-key blob ("_OCTREE_1.0_") -> 64-bit keys
+int64_t ref_upgrade_key64(const void* blob32, int64_t bytes) {
+  std::vector<char> in((const char*)blob32, (const char*)blob32 + bytes), out;
+  upgrade_key64(out, in);
+  return keep(out);
 }
 
 int ref_get_ni(const int* ks, int* out) {
@@ -164,6 +176,66 @@ void ref_key2xyz(uint64_t* xyz, const uint64_t* key, int num, int depth) {
 }
 void ref_key2idx(int* idx, const uint64_t* key, int num) {
   key2idx_cpu<uintk>(idx, (const uintk*)key, num);
+}
+
+
+// pytorch/cpp/transform_points.cpp:7-125, on a copy of the blob (setup_transform).
+int ref_bounding_sphere(const void* points_blob, int method_box, float* out4) {
+  Points pts;
+  pts.set(points_blob);
+  std::string msg;
+  if (!pts.info().check_format(msg)) return -1;
+  float radius = 0.0f, center[3] = {0.0f};
+  if (!method_box) {
+    bounding_sphere(radius, center, pts.points(), pts.info().pt_num());
+  } else {
+    float bbmin[3] = {0.0f}, bbmax[3] = {0.0f};
+    bounding_box(bbmin, bbmax, pts.points(), pts.info().pt_num());
+    for (int j = 0; j < 3; ++j) {
+      center[j] = (bbmax[j] + bbmin[j]) / 2.0f;
+      float width = (bbmax[j] - bbmin[j]) / 2.0f;
+      radius += width * width;
+    }
+    radius = sqrtf(radius + 1.0e-20f);
+  }
+  out4[0] = radius; out4[1] = center[0]; out4[2] = center[1]; out4[3] = center[2];
+  return 0;
+}
+static bool open_copy(const void* blob, int64_t bytes, Points& pts) {
+  g_last.assign((const char*)blob, (const char*)blob + bytes);
+  pts.set(g_last.data());
+  std::string msg;
+  return pts.info().check_format(msg);
+}
+int64_t ref_normalize_points(const void* blob, int64_t bytes, float radius, const float* center) {
+  Points pts;
+  if (!open_copy(blob, bytes, pts)) return -1;
+  const float dis[3] = {-center[0], -center[1], -center[2]};
+  if (dis[0] != 0.0f || dis[1] != 0.0f || dis[2] != 0.0f) pts.translate(dis);
+  const float inv_radius = 1.0f / radius;
+  const float scale[3] = {inv_radius, inv_radius, inv_radius};
+  if (scale[0] != 1.0f || scale[1] != 1.0f || scale[2] != 1.0f) pts.scale(scale);
+  return (int64_t)g_last.size();
+}
+int64_t ref_transform_points(const void* blob, int64_t bytes, const float* angle, const float* scale,
+    const float* jitter, float offset, const char* normal_axis) {
+  Points pts;
+  if (!open_copy(blob, bytes, pts)) return -1;
+  const float kEPS = 1.0e-10f;
+  if (offset > kEPS) pts.displace(offset);
+  if (fabs(angle[0]) > kEPS || fabs(angle[1]) > kEPS || fabs(angle[2]) > kEPS) pts.rotate(angle);
+  if (fabs(jitter[0]) > kEPS || fabs(jitter[1]) > kEPS || fabs(jitter[2]) > kEPS) pts.translate(jitter);
+  if (scale[0] != 1.0f || scale[1] != 1.0f || scale[2] != 1.0f) pts.scale(scale);
+  std::string axis(normal_axis ? normal_axis : "");
+  if (!axis.empty()) pts.orient_normal(axis);
+  return (int64_t)g_last.size();
+}
+int64_t ref_clip_points(const void* blob, int64_t bytes, const float* bbmin, const float* bbmax, int* inbox_mask) {
+  Points pts;
+  if (!open_copy(blob, bytes, pts)) return -1;
+  std::vector<int> mask = pts.clip(bbmin, bbmax);
+  memcpy(inbox_mask, mask.data(), mask.size() * sizeof(int));
+  return (int64_t)g_last.size();
 }
 
 }  // extern "C"

@@ -41,6 +41,21 @@ def main():
   np.savez_compressed(os.path.join(HERE, "octree_samples.npz"),
                       **{"octree_%d" % i: ref.octree_sample("octree_%d" % i) for i in range(1, 7)})
 
+  # the same six samples as the reference stores them: 32-bit keys ("_OCTREE_1.0_"), read from the
+  # sample translation unit compiled without KEY64 (oracle/Makefile)
+  import ctypes as C
+  import subprocess
+  so32 = os.path.join(ROOT, "oracle", "_ref", "libocnn_samples32.so")
+  sym = subprocess.check_output("nm -D %s | grep get_one_octree" % so32, shell=True).decode().split()[-1]
+  get = getattr(C.CDLL(so32), sym)
+  get.restype, get.argtypes = C.c_void_p, [C.c_char_p, C.POINTER(C.c_size_t)]
+  raw32 = {}
+  for i in range(1, 7):
+    sz = C.c_size_t()
+    ptr = get(("octree_%d" % i).encode(), C.byref(sz))
+    raw32["octree_%d" % i] = np.ctypeslib.as_array((C.c_ubyte * sz.value).from_address(ptr)).copy()
+  np.savez_compressed(os.path.join(HERE, "octree_samples_key32.npz"), **raw32)
+
   pts, nrm, _ = synthetic.sphere_cloud(3000, 0)
   pb = make_points_blob(pts, nrm)
   single = ref.points2octree(pb, 5, 2)
