@@ -184,6 +184,26 @@ int ocnn_octree_deconv_grad(void* grad_data, void* grad_weights, const void* dat
     int depth, int num_output, const int* kernel_size, int stride, int nempty, int dtype,
     void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream);
 
+/* ---- feature transfer between octrees and to free points.
+ * ocnn_align_forward / backward: align_forward_gpu / align_backward_gpu
+ * (octree/octree/octree_nn.h:196-201, octree_nn.cu:710-752): top[c, idx[h]] = btm[c, h] for
+ * idx[h] != -1 (top is zero-filled first); backward gathers.  `octree_align`
+ * (pytorch/cpp/octree_align.cpp:9-83) = key arrays of both octrees -> ocnn_search_key -> this.
+ * ocnn_octree_interp: octree_nearest_pts (method 0) / octree_trilinear_pts (method 1) of
+ * pytorch/ocnn/modules.py:209-275 in two kernels.  key[n_key]: the sorted Morton keys of the
+ * searched depth (de-padded by the caller for nempty, as octree_search_key does,
+ * pytorch/cpp/octree_key.cpp:83-132); pts [n_pts, 4] = (x, y, z in [0, 2^depth], batch id);
+ * out [channel, n_pts].  idx / weight [n_pts * K] (K = 1 nearest, 8 linear) are filled for the
+ * backward call, which zero-fills grad_data [channel, H] and scatters with fp32 atomics. */
+int ocnn_align_forward(float* top, int top_h, int channel, const float* btm, int btm_h, const int* idx,
+    ocnn_stream_t stream);
+int ocnn_align_backward(const float* top, int top_h, int channel, float* btm, int btm_h, const int* idx,
+    ocnn_stream_t stream);
+int ocnn_octree_interp(float* out, const float* data, int channel, int H, const uint64_t* key, int n_key,
+    const float* pts, int n_pts, int depth, int method, int* idx, float* weight, ocnn_stream_t stream);
+int ocnn_octree_interp_backward(float* grad_data, const float* grad_out, int channel, int H, int n_pts,
+    int method, const int* idx, const float* weight, ocnn_stream_t stream);
+
 /* ---- file formats.  A `.octree` / `.points` file is the serialized blob itself
  * (Octree::read_octree / write_octree, octree/octree/octree.cpp:41-68; Points::read_points /
  * write_points, points.cpp:9-37).  Files written by a 32-bit-key build carry "_OCTREE_1.0_" and

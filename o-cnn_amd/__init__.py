@@ -16,4 +16,6 @@ The directory name is not a Python identifier; load the package with
 from . import lib, nn, autograd, layers, stacks, synthetic  # noqa: F401
 from .nn import *  # noqa: F401,F403
 from .layers import (OctreeConv, OctreeDeconv, OctreeConvFast, OctreeDeconvFast,  # noqa: F401
-                     OctreeMaxPool, OctreeMaxUnpool, OctreeAvgPool, OctreePad, OctreeDepad)
+                     OctreeMaxPool, OctreeMaxUnpool, OctreeAvgPool, OctreePad, OctreeDepad,
+                     OctreeTrilinear, OctreeInterp, OctreeAlign, octree_nearest_pts,
+                     octree_trilinear_pts, octree_trilinear)

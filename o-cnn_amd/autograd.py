@@ -143,6 +143,40 @@ class Col2OctreeFunction(Function):
     return (F.octree2col(grad_in.contiguous(), octree, *ctx.cfg),) + (None,) * 5
 
 
+class OctreeAlignFunction(Function):
+  """pytorch/ocnn/octree_align.py: (data, src_octree, des_octree, depth) -> (aligned, idx)."""
+
+  @staticmethod
+  def forward(ctx, src_data, src_octree, des_octree, depth):
+    out, idx = F.octree_align(src_data.contiguous(), src_octree, des_octree, depth)
+    ctx.save_for_backward(idx)
+    ctx.mark_non_differentiable(idx)
+    return out, idx
+
+  @staticmethod
+  def backward(ctx, grad_out, _idx_grad):
+    idx, = ctx.saved_tensors
+    return F.octree_align_grad(grad_out.contiguous(), idx), None, None, None
+
+
+class OctreeInterpFunction(Function):
+  """Nearest / trilinear interpolation of node features at free points
+  (pytorch/ocnn/modules.py:209-275); differentiable in the features."""
+
+  @staticmethod
+  def forward(ctx, data, octree, depth, pts, method, nempty):
+    out, idx, weight = F.octree_interp_pts(data, octree, depth, pts, method, nempty)
+    ctx.save_for_backward(idx, weight)
+    ctx.cfg = (data.size(2), method)
+    return out
+
+  @staticmethod
+  def backward(ctx, grad_out):
+    idx, weight = ctx.saved_tensors
+    H, method = ctx.cfg
+    return (F.octree_interp_pts_grad(grad_out.contiguous(), idx, weight, H, method),) + (None,) * 5
+
+
 octree_conv = OctreeConvFunction.apply
 octree_deconv = OctreeDeconvFunction.apply
 octree_max_pool = OctreeMaxPoolFunction.apply
@@ -152,3 +186,5 @@ octree_pad = OctreePadFunction.apply
 octree_depad = OctreeDepadFunction.apply
 octree2col = Octree2ColFunction.apply
 col2octree = Col2OctreeFunction.apply
+octree_align = OctreeAlignFunction.apply
+octree_interp_pts = OctreeInterpFunction.apply

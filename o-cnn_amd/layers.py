@@ -147,3 +147,60 @@ class OctreeDepad(nn.Module):
 
   def forward(self, data_in, octree):
     return F.octree_depad(data_in, octree, self.depth)
+
+
+def octree_nearest_pts(data, octree, depth, pts, nempty=False):
+  """pytorch/ocnn/modules.py:209-221."""
+  return F.octree_interp_pts(data, octree, depth, pts, "nearest", nempty)
+
+
+def octree_trilinear_pts(data, octree, depth, pts, nempty=False):
+  """pytorch/ocnn/modules.py:224-268; pts must be scaled into [0, 2^depth]."""
+  return F.octree_interp_pts(data, octree, depth, pts, "linear", nempty)
+
+
+def octree_trilinear(data, octree, depth, target_depth):
+  """Interpolate from `depth` to the node centres of `target_depth` (modules.py:271-281)."""
+  from . import nn as ops
+  xyz = ops.octree_property(octree, "xyz", target_depth)
+  xyz = ops.octree_decode_key(xyz).float()
+  scale = 2.0 ** (depth - target_depth)
+  xyz = (xyz + torch.tensor([0.5, 0.5, 0.5, 0.0], device=xyz.device)) * \
+      torch.tensor([scale, scale, scale, 1.0], device=xyz.device)
+  return octree_trilinear_pts(data, octree, depth, xyz)
+
+
+class OctreeTrilinear(nn.Module):
+  def __init__(self, depth):
+    super().__init__()
+    self.depth = depth
+
+  def forward(self, data, octree):
+    return octree_trilinear(data, octree, self.depth, self.depth + 1)
+
+
+class OctreeInterp(nn.Module):
+  """pytorch/ocnn/modules.py:294-318: points in [-1, 1] (+ batch id) -> [0, 2^depth]."""
+
+  def __init__(self, depth, method='linear', nempty=False):
+    super().__init__()
+    self.depth, self.method, self.nempty = depth, method, nempty
+
+  def forward(self, data, octree, pts):
+    xyz = (pts[:, :3] + 1.0) * (2 ** (self.depth - 1))
+    pts = torch.cat([xyz, pts[:, 3:]], dim=1)
+    if self.method not in ('nearest', 'linear'):
+      raise ValueError
+    return F.octree_interp_pts(data, octree, self.depth, pts, self.method, self.nempty)
+
+  def extra_repr(self):
+    return 'depth={}, method={}, nempty={}'.format(self.depth, self.method, self.nempty)
+
+
+class OctreeAlign(nn.Module):
+  def __init__(self, depth):
+    super().__init__()
+    self.depth = depth
+
+  def forward(self, data, src_octree, des_octree):
+    return F.octree_align(data, src_octree, des_octree, self.depth)

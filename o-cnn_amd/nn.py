@@ -747,18 +747,9 @@ def octree_key2xyz(key, depth):
   return _key_op("ocnn_key2xyz", key, depth)
 
 
-def octree_search_key(key, octree, depth, key_is_xyz, nempty):
-  """pytorch/cpp/octree_key.cpp:83-132: index of each query key at `depth`, -1 on a miss."""
-  octree = _to_dev(octree)
-  info = octree_info(octree)
-  key = _to_dev(key.contiguous())
-  n_query = key.numel()
-  if n_query < 1:
-    raise OcnnError(-1, "The numel of the input tensor must be larger than 1.")
-  if key_is_xyz:
-    tmp = torch.empty_like(key)
-    _lib.call("ocnn_xyz2key", _ptr(tmp), _ptr(key), n_query, depth, _stream())
-    key = tmp
+def _morton_keys(octree, info, depth, nempty=False):
+  """(sorted Morton keys of a depth as int64 tensor, their number); de-padded for nempty and
+  converted from packed xyz where the octree stores those (pytorch/cpp/octree_key.cpp:95-124)."""
   des_h = info.nnum(depth)
   des = _prop_view(octree, info, KEY, depth, des_h, torch.int64)
   if nempty:
@@ -773,8 +764,138 @@ def octree_search_key(key, octree, depth, key_is_xyz, nempty):
     if des_h:
       _lib.call("ocnn_xyz2key", _ptr(tmp), _ptr(des), des_h, depth, _stream())
     des = tmp
+  return des, des_h
+
+
+def octree_search_key(key, octree, depth, key_is_xyz, nempty):
+  """pytorch/cpp/octree_key.cpp:83-132: index of each query key at `depth`, -1 on a miss."""
+  octree = _to_dev(octree)
+  info = octree_info(octree)
+  key = _to_dev(key.contiguous())
+  n_query = key.numel()
+  if n_query < 1:
+    raise OcnnError(-1, "The numel of the input tensor must be larger than 1.")
+  if key_is_xyz:
+    tmp = torch.empty_like(key)
+    _lib.call("ocnn_xyz2key", _ptr(tmp), _ptr(key), n_query, depth, _stream())
+    key = tmp
+  des, des_h = _morton_keys(octree, info, depth, nempty)
   out = torch.empty(n_query, dtype=torch.int32, device=octree.device)
   _lib.call("ocnn_search_key", _ptr(out), _ptr(des), des_h, _ptr(key), n_query, _stream())
+  return out
+
+
+# ---- feature transfer ---------------------------------------------------------------------------
+def octree_align(src_data, src_octree, des_octree, depth):
+  """pytorch/cpp/octree_align.cpp:9-61 -> [des_data [1,C,des_h,1], idx int32 [src_h]]: the
+  features of `src_octree`'s nodes moved to the nodes of `des_octree` with the same key."""
+  src_octree, des_octree = _to_dev(src_octree), _to_dev(des_octree)
+  sinfo, dinfo = octree_info(src_octree), octree_info(des_octree)
+  src_data = src_data.contiguous()
+  if src_data.dtype != torch.float32:
+    raise TypeError("octree_align is fp32")
+  channel, src_h = src_data.size(1), src_data.size(2)
+  if sinfo.nnum(depth) != src_h:
+    raise OcnnError(-3, "octree_align: %d rows, the source octree has %d nodes at depth %d"
+                    % (src_h, sinfo.nnum(depth), depth))
+  src_key, _ = _morton_keys(src_octree, sinfo, depth)
+  des_key, des_h = _morton_keys(des_octree, dinfo, depth)
+  idx = torch.empty(src_h, dtype=torch.int32, device=src_data.device)
+  _lib.call("ocnn_search_key", _ptr(idx), _ptr(des_key), des_h, _ptr(src_key), src_h, _stream())
+  out = torch.empty(1, channel, des_h, 1, dtype=torch.float32, device=src_data.device)
+  _lib.call("ocnn_align_forward", _ptr(out), des_h, channel, _ptr(src_data), src_h, _ptr(idx), _stream())
+  return [out, idx]
+
+
+def octree_align_grad(des_grad, idx):
+  """pytorch/cpp/octree_align.cpp:63-83."""
+  des_grad = des_grad.contiguous()
+  channel, des_h, src_h = des_grad.size(1), des_grad.size(2), idx.numel()
+  out = torch.empty(1, channel, src_h, 1, dtype=torch.float32, device=des_grad.device)
+  _lib.call("ocnn_align_backward", _ptr(des_grad), des_h, channel, _ptr(out), src_h, _ptr(idx.contiguous()),
+            _stream())
+  return out
+
+
+def octree_interp_pts(data, octree, depth, pts, method="linear", nempty=False):
+  """octree_nearest_pts / octree_trilinear_pts (pytorch/ocnn/modules.py:209-275) fused:
+  data [1,C,H,1] at `depth`, pts [N,4] = (x, y, z in [0, 2^depth], batch id)
+  -> ([1,C,N,1], idx int32 [N,K], weight fp32 [N,K]) with K = 1 (nearest) or 8 (linear)."""
+  if method not in ("nearest", "linear"):
+    raise ValueError(method)
+  octree = _to_dev(octree)
+  info = octree_info(octree)
+  data = data.contiguous()
+  pts = _to_dev(pts).to(torch.float32).contiguous()
+  if data.dtype != torch.float32 or pts.dim() != 2 or pts.size(1) != 4:
+    raise TypeError("fp32 data [1,C,H,1] and points [N,4] expected")
+  channel, H, n = data.size(1), data.size(2), pts.size(0)
+  key, n_key = _morton_keys(octree, info, depth, nempty)
+  if H != n_key:
+    raise OcnnError(-3, "interpolation: %d rows, the octree has %d %snodes at depth %d"
+                    % (H, n_key, "non-empty " if nempty else "", depth))
+  K = 1 if method == "nearest" else 8
+  out = torch.empty(1, channel, n, 1, dtype=torch.float32, device=data.device)
+  idx = torch.empty(n, K, dtype=torch.int32, device=data.device)
+  weight = torch.empty(n, K, dtype=torch.float32, device=data.device)
+  _lib.call("ocnn_octree_interp", _ptr(out), _ptr(data), channel, H, _ptr(key), n_key, _ptr(pts), n, depth,
+            int(method == "linear"), _ptr(idx), _ptr(weight), _stream())
+  return out, idx, weight
+
+
+def octree_interp_pts_grad(grad_out, idx, weight, H, method="linear"):
+  grad_out = grad_out.contiguous()
+  channel, n = grad_out.size(1), grad_out.size(2)
+  out = torch.empty(1, channel, H, 1, dtype=torch.float32, device=grad_out.device)
+  _lib.call("ocnn_octree_interp_backward", _ptr(out), _ptr(grad_out), channel, H, n, int(method == "linear"),
+            _ptr(idx), _ptr(weight), _stream())
+  return out
+
+
+# ---- point-cloud properties (pytorch/cpp/points_property.cpp) ----------------------------------
+_PT_PROPS = {"xyz": 0, "xyzi": 0, "normal": 1, "feature": 2, "label": 3}
+
+
+def _points_array(points, prop):
+  hdr = _points_hdr(points)
+  ints = hdr[16:].view(np.int32)
+  t = _PT_PROPS[prop]
+  npt, flags, ch, off = int(ints[0]), int(ints[1]), int(ints[2 + t]), int(ints[10 + t])
+  if not (flags & (1 << t)) or ch == 0:
+    return None, npt, 0, off
+  return points[off:off + 4 * npt * ch].view(torch.float32).view(npt, ch), npt, ch, off
+
+
+def points_property(points, property):
+  """pytorch/cpp/points_property.cpp:92-109 -> float32 [pt_num, channel] (None if absent)."""
+  arr, _, _, _ = _points_array(points, property)
+  return None if arr is None else arr.clone()
+
+
+def points_batch_property(points_list, property):
+  """pytorch/cpp/points_property.cpp:111-160: the property of several clouds stacked; 'xyzi'
+  appends the index of the cloud as a fourth column."""
+  parts = []
+  for i, p in enumerate(points_list):
+    arr, npt, _, _ = _points_array(p, property)
+    if arr is None:
+      raise OcnnError(-1, "The specified property does not exist.")
+    if property == "xyzi":
+      arr = torch.cat([arr, torch.full((npt, 1), float(i), dtype=torch.float32, device=arr.device)], dim=1)
+    parts.append(arr)
+  return torch.cat(parts, dim=0)
+
+
+def points_set_property(points, data, property):
+  """pytorch/cpp/points_property.cpp:58-90: a copy of the cloud with one property replaced."""
+  arr, npt, ch, off = _points_array(points, property)
+  if arr is None:
+    raise OcnnError(-1, "The property does not exist.")
+  if data.dim() != 2 or data.size(0) != npt or data.size(1) != ch:
+    raise OcnnError(-3, "points_set_property: [%d, %d] expected" % (npt, ch))
+  out = points.clone()
+  out[off:off + 4 * npt * ch] = data.to(torch.float32).contiguous().view(-1).view(torch.uint8).to(points.device)
+  out._ocnn_points_info = _points_hdr(points)
   return out
 
 
