@@ -222,6 +222,16 @@ def main():
       F.bounding_sphere(scene_pts, "sphere")
     extra["bounding_sphere_scene"] = {"ms": (time.perf_counter() - t0) / reps * 1e3}
 
+    # trilinear interpolation of 64 channels at 1 M free points (segmentation head), and
+    # octree_align of the depth-9 features onto the same octree
+    ipts = torch.cat([torch.rand(1 << 20, 3, generator=g) * 512.0, torch.zeros(1 << 20, 1)], dim=1).to(dev)
+    t = timed(lambda: F.octree_interp_pts(x32, octree, 9, ipts, "linear"), reps, wu)
+    extra["trilinear_1Mpts_c64_d9"] = {"ms": t, "Mpts_per_s": (1 << 20) / t / 1e3,
+                                       "GBs": (1 << 20) * (64 * 4 * 9 + 16) / t / 1e6}
+    t = timed(lambda: F.octree_align(x32, octree, octree, 9), reps, wu)
+    by = 2 * C * H9 * 4 + H9 * 20
+    extra["octree_align_d9_c64"] = {"ms": t, "GBs": by / t / 1e6, "frac_hbm_peak": by / t / 1e6 / PEAK_HBM_GBS}
+
     # depth-7 batch (configs[2]): 16 clouds of 50 000 points
     clouds = [oc.synthetic.shape_cloud(50000, 200 + i) for i in range(16)]
     cl = [points_tensor(*c) for c in clouds]
