@@ -384,10 +384,7 @@ __global__ __launch_bounds__(256, 2) void conv_s1_f32_lds_kernel(ConvArgs a, flo
         if (c < a.Cin) {
           const float* pc = in + (int64_t)c * a.Hin;
 #pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            float v = pc[(uint32_t)max(nb[j], 0)];
-            xr[j][cc] = nb[j] >= 0 ? v : 0.0f;
-          }
+          for (int j = 0; j < 8; ++j) xr[j][cc] = pc[(uint32_t)max(nb[j], 0)];  // masked when staged
         } else {
 #pragma unroll
           for (int j = 0; j < 8; ++j) xr[j][cc] = 0.0f;
@@ -405,7 +402,8 @@ __global__ __launch_bounds__(256, 2) void conv_s1_f32_lds_kernel(ConvArgs a, flo
 #pragma unroll
       for (int cc = 0; cc < kSlab; ++cc)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) sX[cc * kPlane + group_base(wave * 8 + j) + lane] = xr[j][cc];
+        for (int j = 0; j < 8; ++j)  // the mask is applied here so that nothing waits for the gathers earlier
+          sX[cc * kPlane + group_base(wave * 8 + j) + lane] = nb[j] >= 0 ? xr[j][cc] : 0.0f;
       __syncthreads();
       if (slab + 1 < nslab) fetch(slab + 1);
 #pragma unroll 3
@@ -1262,9 +1260,31 @@ __device__ inline int wgrad_src(const ConvArgs& a, int n, int k) {
   return (live && p >= 0 && p < a.Hin) ? p : a.Hin;
 }
 
+// aq[n / 4][mpad][4] <- A[M][N]: four consecutive columns of a row become one 16-byte unit, rows
+// are contiguous within a column quad; zero beyond M and N (N is padded to whole 8-column blocks).
+__global__ __launch_bounds__(256) void interleave_quads_kernel(float* __restrict__ aq, const float* __restrict__ A,
+    int M, int N, int mpad, int n_quads) {
+  __shared__ float tile[64][65];
+  const int n0 = blockIdx.x * 64, m0 = blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    const int m = m0 + i, n = n0 + tx;
+    tile[i][tx] = (m < M && n < N) ? A[(int64_t)m * N + n] : 0.0f;
+  }
+  __syncthreads();
+  // 16 column quads x 64 rows: consecutive threads take consecutive rows of one quad
+  for (int u = threadIdx.x; u < 16 * 64; u += 256) {
+    const int q = u >> 6, i = u & 63;
+    const int quad = (n0 >> 2) + q, m = m0 + i;
+    if (quad < n_quads && m < mpad)
+      *reinterpret_cast<float4*>(aq + ((int64_t)quad * mpad + m) * 4) =
+          make_float4(tile[i][4 * q], tile[i][4 * q + 1], tile[i][4 * q + 2], tile[i][4 * q + 3]);
+  }
+}
+
 constexpr int kWgTaps = 3;
 
-template <int MT, int NT>
+template <int MT, int NT, bool FAST>
 __global__ __launch_bounds__(256, 2) void conv_wgrad_f32_kernel(ConvArgs a, const float* __restrict__ A,
     const float* __restrict__ xt, float* __restrict__ partial, int cpad, int mpad, int n_slices, int cpasses) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -1282,7 +1302,6 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_f32_kernel(ConvArgs a, cons
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[t][mt][nt][i] = 0.0f;
   const int nblocks = (a.N + 7) >> 3;
-  const bool vec_ok = (a.N & 3) == 0 && (reinterpret_cast<uintptr_t>(A) & 15) == 0;
   // a slice is a contiguous range of column blocks: the 128-byte lines of A a wavefront touches
   // (one per row, 16 bytes used per block) and the neighbour rows of xt are reused from L1
   const int per_slice = (nblocks + n_slices - 1) / n_slices;
@@ -1290,49 +1309,93 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_f32_kernel(ConvArgs a, cons
   // with two column tiles, tile nt holds the channels 2n + nt, so that one 8-byte load per lane
   // feeds both tiles and a half wavefront reads 256 contiguous bytes of a row
   const float* xcol = xt + (NT == 2 ? cpass * 64 + 2 * r : cpass * 32 + r);
-  for (int b = slice * per_slice; b < b_end; ++b) {
-    // all source rows of the block with one load: lane (t, column) = (lane >> 3, lane & 7)
-    const int srcv = wgrad_src(a, b * 8 + (lane & 7), tap0 + min(lane >> 3, kWgTaps - 1));
-    const int n0 = b * 8 + 4 * kh;
-    float av[MT][4];
+  // software pipeline: the source rows and the A values of block b + 1 are requested before the
+  // MFMAs of block b, and all gathers of a block are in flight together
+  // FAST = stride 1 over all nodes with whole sibling groups: the index load then carries no
+  // branches, so the compiler keeps it in flight across the MFMAs
+  const int my_tap = min(tap0 + min(lane >> 3, kWgTaps - 1), a.K - 1);
+  const bool tap_live = tap0 + min(lane >> 3, kWgTaps - 1) < a.K;
+  const int my_slot = sibling_slot(lane & 7) + a.slot[my_tap];
+  auto load_src = [&](int b) {
+    // all source rows of a block with one load: lane (t, column) = (lane >> 3, lane & 7)
+    if (FAST) return a.neigh[((int64_t)b << 6) + my_slot];  // range-checked when it is used
+    return wgrad_src(a, b * 8 + (lane & 7), tap0 + min(lane >> 3, kWgTaps - 1));
+  };
+  // A comes from its quad-interleaved copy aq[n / 4][mpad][4] (zero beyond M and N): the 32 lanes of
+  // a half wavefront read 512 contiguous bytes, every byte of a cache line is used, and the load
+  // needs no bounds check.  (Read in place, [M, N] row-major, a wavefront touches one 128-byte line
+  // per row and block and uses 16 bytes of it; eight wavefronts then overflow the L1 and A is
+  // fetched eight times.)
+  auto load_a = [&](int b, float (&av)[MT][4]) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       const int m = (mpass * MT + mt) * 32 + r;
+      const float4 v = *reinterpret_cast<const float4*>(A + (((int64_t)b * 2 + kh) * mpad + m) * 4);
+      av[mt][0] = v.x; av[mt][1] = v.y; av[mt][2] = v.z; av[mt][3] = v.w;
+    }
+  };
+  // gathers of one tap of a block: 4 column pairs x NT tiles
+  auto load_b = [&](int srcv, int t, float (&bv)[4][NT]) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) av[mt][j] = 0.0f;
-      if (m < a.M) {
-        const float* ap = A + (int64_t)m * a.N + n0;
-        if (vec_ok && n0 + 4 <= a.N) {
-          const float4 v = *reinterpret_cast<const float4*>(ap);
-          av[mt][0] = v.x; av[mt][1] = v.y; av[mt][2] = v.z; av[mt][3] = v.w;
-        } else {
-#pragma unroll
-          for (int j = 0; j < 4; ++j) if (n0 + j < a.N) av[mt][j] = ap[j];
-        }
+    for (int j = 0; j < 4; ++j) {
+      const int lo = __builtin_amdgcn_readlane(srcv, t * 8 + j);
+      const int hi = __builtin_amdgcn_readlane(srcv, t * 8 + 4 + j);
+      const float* row = xcol + (int64_t)(kh ? hi : lo) * cpad;
+      if (NT == 2) {
+        const float2 v = *reinterpret_cast<const float2*>(row);
+        bv[j][0] = v.x; bv[j][NT - 1] = v.y;
+      } else {
+        bv[j][0] = *row;
       }
     }
+  };
+  auto mfma_tap = [&](int t, const float (&av)[MT][4], const float (&bv)[4][NT]) {
 #pragma unroll
-    for (int t = 0; t < kWgTaps; ++t) {
-      float bv[4][NT];
+    for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int lo = __builtin_amdgcn_readlane(srcv, t * 8 + j);
-        const int hi = __builtin_amdgcn_readlane(srcv, t * 8 + 4 + j);
-        const float* row = xcol + (int64_t)(kh ? hi : lo) * cpad;
-        if (NT == 2) {
-          const float2 v = *reinterpret_cast<const float2*>(row);
-          bv[j][0] = v.x; bv[j][NT - 1] = v.y;
-        } else {
-          bv[j][0] = *row;
-        }
-      }
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          acc[t][mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[mt][j], bv[j][nt], acc[t][mt][nt], 0, 0, 0);
+  };
+  auto checked = [&](int v) { return FAST ? ((tap_live && v >= 0 && v < a.Hin) ? v : a.Hin) : v; };
+  // Software pipeline at tap granularity: while the 4 * MT * NT MFMAs of one tap run, the gathers
+  // of the next tap are in flight, and the source rows and A values of the NEXT block are
+  // requested a whole block ahead.
+  static_assert(kWgTaps == 3, "the pipeline below is written for three taps per wavefront");
+  const int b_begin = slice * per_slice;
+  if (b_begin < b_end) {
+    int srcv = checked(load_src(b_begin));
+    float av[MT][4], bv0[4][NT], bv1[4][NT];
+    load_a(b_begin, av);
+    load_b(srcv, 0, bv0);
+    for (int b = b_begin; b < b_end; ++b) {
+      const int bn = min(b + 1, b_end - 1);  // the last block is requested twice: no branch
+      float av_cur[MT][4];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          av_cur[mt][j] = av[mt][j];
+      int srcv_next = load_src(bn);
+      load_a(bn, av);
+      load_b(srcv, 1, bv1);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_tap(0, av_cur, bv0);
+      __builtin_amdgcn_sched_barrier(0);
+      load_b(srcv, 2, bv0);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_tap(1, av_cur, bv1);
+      __builtin_amdgcn_sched_barrier(0);
+      srcv = checked(srcv_next);
+      load_b(srcv, 0, bv1);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_tap(2, av_cur, bv0);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int nt = 0; nt < NT; ++nt)
-            acc[t][mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[mt][j], bv[j][nt], acc[t][mt][nt], 0, 0, 0);
+        for (int nt = 0; nt < NT; ++nt) bv0[j][nt] = bv1[j][nt];
     }
   }
   // partial[slice][tap][m][c]: a half wavefront writes 128 (256) contiguous bytes
@@ -1368,7 +1431,7 @@ __global__ void conv_wgrad_reduce_kernel(float* __restrict__ G, const float* __r
 
 struct WgradPlan {
   int MT, NT, mpasses, cpasses, mpad, cpad, n_slices, tapgroups;
-  size_t xt_bytes, partial_bytes, ichild_bytes, total_bytes;
+  size_t xt_bytes, partial_bytes, ichild_bytes, aq_bytes, total_bytes;
 };
 // `p` is the plan of the underlying convolution geometry (deconv = 0): M rows on the column side,
 // channel_in channels on the gathered side.
@@ -1393,7 +1456,8 @@ void make_wgrad_plan(const ConvPlan& p, int M, int channel_in, int nempty, Wgrad
   w->xt_bytes = align256(((size_t)p.btm_h + 1) * w->cpad * sizeof(float));
   w->partial_bytes = align256((size_t)w->n_slices * p.taps.count * w->mpad * w->cpad * sizeof(float));
   w->ichild_bytes = nempty ? align256(sizeof(int) * (size_t)(p.ichild_h + 1)) : 0;
-  w->total_bytes = w->xt_bytes + w->partial_bytes + w->ichild_bytes;
+  w->aq_bytes = align256((size_t)nblocks * 2 * w->mpad * 4 * sizeof(float));
+  w->total_bytes = w->xt_bytes + w->partial_bytes + w->ichild_bytes + w->aq_bytes;
 }
 
 // grad_w[M, channel_in * K] from A [M, top_h] (column side) and X [channel_in, btm_h] (gathered side)
@@ -1422,15 +1486,26 @@ int run_wgrad(float* grad_w, const float* A, int M, const float* X, int channel_
   dim3 tg((a.Hin + 64) / 64, (w.cpad + 63) / 64);
   transpose_rows_f32_kernel<<<tg, 256, 0, s>>>(xt, X, channel_in, a.Hin, w.cpad);
   OCNN_LAUNCH_OK("transpose_rows");
+  float* aq = reinterpret_cast<float*>(wsb + w.xt_bytes + w.partial_bytes + w.ichild_bytes);
+  const int n_quads = ((a.N + 7) / 8) * 2;
+  dim3 qg((n_quads * 4 + 63) / 64, (w.mpad + 63) / 64);
+  interleave_quads_kernel<<<qg, 256, 0, s>>>(aq, A, M, a.N, w.mpad, n_quads);
+  OCNN_LAUNCH_OK("interleave_quads");
   dim3 grid(w.n_slices / 4, w.tapgroups, w.mpasses * w.cpasses);
-  if (w.MT == 1 && w.NT == 1)
-    conv_wgrad_f32_kernel<1, 1><<<grid, 256, 0, s>>>(a, A, xt, partial, w.cpad, w.mpad, w.n_slices, w.cpasses);
-  else if (w.MT == 1)
-    conv_wgrad_f32_kernel<1, 2><<<grid, 256, 0, s>>>(a, A, xt, partial, w.cpad, w.mpad, w.n_slices, w.cpasses);
-  else if (w.NT == 1)
-    conv_wgrad_f32_kernel<2, 1><<<grid, 256, 0, s>>>(a, A, xt, partial, w.cpad, w.mpad, w.n_slices, w.cpasses);
-  else
-    conv_wgrad_f32_kernel<2, 2><<<grid, 256, 0, s>>>(a, A, xt, partial, w.cpad, w.mpad, w.n_slices, w.cpasses);
+  // whole sibling groups (N % 8 == 0), every column a node
+  const bool fast = a.mode == kModeS1 && !a.nempty && (a.N & 7) == 0;
+#define OCNN_WGRAD(MT_, NT_)                                                                                     \
+  do {                                                                                                           \
+    if (fast) conv_wgrad_f32_kernel<MT_, NT_, true><<<grid, 256, 0, s>>>(a, aq, xt, partial, w.cpad, w.mpad,     \
+        w.n_slices, w.cpasses);                                                                                  \
+    else conv_wgrad_f32_kernel<MT_, NT_, false><<<grid, 256, 0, s>>>(a, aq, xt, partial, w.cpad, w.mpad,         \
+        w.n_slices, w.cpasses);                                                                                  \
+  } while (0)
+  if (w.MT == 1 && w.NT == 1) OCNN_WGRAD(1, 1);
+  else if (w.MT == 1) OCNN_WGRAD(1, 2);
+  else if (w.NT == 1) OCNN_WGRAD(2, 1);
+  else OCNN_WGRAD(2, 2);
+#undef OCNN_WGRAD
   OCNN_LAUNCH_OK("conv_wgrad");
   int64_t per = (int64_t)a.K * w.mpad * w.cpad;
   conv_wgrad_reduce_kernel<<<blocks_for(per), kBlock, 0, s>>>(grad_w, partial, w.n_slices, M, channel_in, a.K,
