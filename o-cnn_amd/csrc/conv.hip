@@ -343,6 +343,7 @@ __global__ __launch_bounds__(256, 2) void conv_s1_f32_lds_kernel(ConvArgs a, flo
   const int r = lane & 31, kh = lane >> 5;
   const int nslab = (a.Cin + kSlab - 1) / kSlab;
   const int npass = (a.mtiles + MT - 1) / MT;
+  const bool mirrored = a.slot[0] != 0;  // deconvolution walks the taps through the opposite offsets
 
   // neighbour rows of slot `lane` of my eight groups (kept for all slabs and passes)
   int nb[8];
@@ -406,18 +407,27 @@ __global__ __launch_bounds__(256, 2) void conv_s1_f32_lds_kernel(ConvArgs a, flo
           sX[cc * kPlane + group_base(wave * 8 + j) + lane] = nb[j] >= 0 ? xr[j][cc] : 0.0f;
       __syncthreads();
       if (slab + 1 < nslab) fetch(slab + 1);
-#pragma unroll 3
-      for (int k = 0; k < K; ++k) {
-        const int slot = a.slot[k];
+      // taps in (dx, dy) pairs of three dz each: the slot of tap (dx, dy, dz) is dx<<4 | dy<<2 | dz
+      // (mirrored: 42 minus that), computed instead of read from the argument block, so the loop
+      // holds no scalar load to wait for
+      static_assert(K == 27, "slot arithmetic below is the 3x3x3 kernel's");
+#pragma unroll 1
+      for (int kxy = 0; kxy < 9; ++kxy) {
+        const int s3 = ((kxy / 3) << 4) | ((kxy % 3) << 2);
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-          float b0 = sX[boff[0] + ks * 2 * kPlane + slot];
-          float b1 = sX[boff[1] + ks * 2 * kPlane + slot];
+        for (int kz = 0; kz < 3; ++kz) {
+          const int k = kxy * 3 + kz;
+          const int slot = mirrored ? 42 - (s3 | kz) : (s3 | kz);
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            float av = sW[((k * 2 + ks) * MT + mt) * 64 + lane];
-            acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b0, acc[mt][0], 0, 0, 0);
-            acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b1, acc[mt][1], 0, 0, 0);
+          for (int ks = 0; ks < 2; ++ks) {
+            float b0 = sX[boff[0] + ks * 2 * kPlane + slot];
+            float b1 = sX[boff[1] + ks * 2 * kPlane + slot];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+              float av = sW[((k * 2 + ks) * MT + mt) * 64 + lane];
+              acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b0, acc[mt][0], 0, 0, 0);
+              acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b1, acc[mt][1], 0, 0, 0);
+            }
           }
         }
       }
