@@ -162,27 +162,53 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
 #pragma unroll
       for (int v = 0; v < kWVec; ++v) wr[v] = wsrc[v * 256 + threadIdx.x];
     };
+    // Software pipeline over the stages (tap, 64-channel slab): while the MFMAs of one stage run,
+    // the weights AND all gathers of the next stage (8 channel groups x 2 columns, 16 bytes each)
+    // are in flight; the source rows of a tap are looked up two taps ahead.
+    float4 nx0[kRowSlab / 8], nx1[kRowSlab / 8];
+    auto src_of = [&](int k, int half) { return k < a.K ? conv_src(a, n0 + half * 32 + r, k) : -1; };
+    auto fetch_x = [&](int s0, int s1, int slab) {
+      const float4* row0 = xt + (int64_t)(s0 < 0 ? a.Hin : s0) * cpad4 + kh;
+      const float4* row1 = xt + (int64_t)(s1 < 0 ? a.Hin : s1) * cpad4 + kh;
+      const int ngroup = min(kRowSlab, cpad - slab * kRowSlab) >> 3;
+#pragma unroll
+      for (int c8 = 0; c8 < kRowSlab / 8; ++c8)
+        if (c8 < ngroup) {
+          nx0[c8] = row0[(slab * kRowSlab + c8 * 8) >> 2];
+          nx1[c8] = row1[(slab * kRowSlab + c8 * 8) >> 2];
+        }
+    };
+    int s0c = src_of(0, 0), s1c = src_of(0, 1);      // rows of the current tap
+    int s0n = src_of(1, 0), s1n = src_of(1, 1);      // ... of the next one
     fetch_w(0);
+    fetch_x(s0c, s1c, 0);
     int stage = 0;
-    int s0n = conv_src(a, n0 + r, 0), s1n = conv_src(a, n0 + 32 + r, 0);
     for (int k = 0; k < a.K; ++k) {
-      const int s0 = s0n < 0 ? a.Hin : s0n, s1 = s1n < 0 ? a.Hin : s1n;
-      if (k + 1 < a.K) {  // the next tap's source rows arrive while this tap is multiplied
-        s0n = conv_src(a, n0 + r, k + 1);
-        s1n = conv_src(a, n0 + 32 + r, k + 1);
-      }
-      const float4* row0 = xt + (int64_t)s0 * cpad4 + kh;
-      const float4* row1 = xt + (int64_t)s1 * cpad4 + kh;
+      const int s0n2 = src_of(k + 2, 0), s1n2 = src_of(k + 2, 1);
       for (int slab = 0; slab < nslab; ++slab, ++stage) {
         __syncthreads();
 #pragma unroll
         for (int v = 0; v < kWVec; ++v) reinterpret_cast<float4*>(sW)[v * 256 + threadIdx.x] = wr[v];
         __syncthreads();
-        if (stage + 1 < nstage) fetch_w(stage + 1);
+        // group c8 of the NEXT stage is requested right after group c8 of this one has been read
+        // out of its registers, so every gather has seven eighths of a stage to arrive
+        const bool more = stage + 1 < nstage;
+        const bool same_tap = slab + 1 < nslab;
+        const int nslab_next = same_tap ? slab + 1 : 0;
+        const int s0x = same_tap ? s0c : s0n, s1x = same_tap ? s1c : s1n;
+        const float4* nrow0 = xt + (int64_t)(s0x < 0 ? a.Hin : s0x) * cpad4 + kh + ((nslab_next * kRowSlab) >> 2);
+        const float4* nrow1 = xt + (int64_t)(s1x < 0 ? a.Hin : s1x) * cpad4 + kh + ((nslab_next * kRowSlab) >> 2);
+        const int ngroup_next = more ? (min(kRowSlab, cpad - nslab_next * kRowSlab) >> 3) : 0;
+        if (more) fetch_w(stage + 1);
         const int ngroup = min(kRowSlab, cpad - slab * kRowSlab) >> 3;
-        for (int c8 = 0; c8 < ngroup; ++c8) {
-          const float4 b0 = row0[(slab * kRowSlab + c8 * 8) >> 2];
-          const float4 b1 = row1[(slab * kRowSlab + c8 * 8) >> 2];
+#pragma unroll
+        for (int c8 = 0; c8 < kRowSlab / 8; ++c8) {
+          const float4 b0 = nx0[c8], b1 = nx1[c8];
+          if (c8 < ngroup_next) {
+            nx0[c8] = nrow0[c8 * 2];
+            nx1[c8] = nrow1[c8 * 2];
+          }
+          if (c8 >= ngroup) continue;  // uniform
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const float v0 = j == 0 ? b0.x : j == 1 ? b0.y : j == 2 ? b0.z : b0.w;
@@ -196,6 +222,7 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
           }
         }
       }
+      s0c = s0n; s1c = s1n; s0n = s0n2; s1n = s1n2;
     }
     if (n0 < a.N) store_tiles<float, MT>(a, out, acc, pass * MT, n0, lane);
   }
@@ -249,17 +276,28 @@ __global__ __launch_bounds__(256) void conv_rows_bf16_kernel(ConvArgs a, uint16_
         wr[v] = idx < kWUnits ? wsrc[idx] : (u32x4)(0u);
       }
     };
+    // same pipeline as the fp32 kernel: weights and all gathers of the next stage (4 groups of 16
+    // channels x 2 columns) are requested before the MFMAs of the current one
+    u32x4 nx0[kRowSlab / 16], nx1[kRowSlab / 16];
+    auto src_of = [&](int k, int half) { return k < a.K ? conv_src(a, n0 + half * 32 + r, k) : -1; };
+    auto fetch_x = [&](int s0, int s1, int slab) {
+      const u32x4* row0 = xt + (int64_t)(s0 < 0 ? a.Hin : s0) * cpad8 + kh;
+      const u32x4* row1 = xt + (int64_t)(s1 < 0 ? a.Hin : s1) * cpad8 + kh;
+      const int ngroup = min(kRowSlab, cpad - slab * kRowSlab) >> 4;
+#pragma unroll
+      for (int c16 = 0; c16 < kRowSlab / 16; ++c16)
+        if (c16 < ngroup) {
+          nx0[c16] = row0[(slab * kRowSlab + c16 * 16) >> 3];
+          nx1[c16] = row1[(slab * kRowSlab + c16 * 16) >> 3];
+        }
+    };
+    int s0c = src_of(0, 0), s1c = src_of(0, 1);
+    int s0n = src_of(1, 0), s1n = src_of(1, 1);
     fetch_w(0);
+    fetch_x(s0c, s1c, 0);
     int stage = 0;
-    int s0n = conv_src(a, n0 + r, 0), s1n = conv_src(a, n0 + 32 + r, 0);
     for (int k = 0; k < a.K; ++k) {
-      const int s0 = s0n < 0 ? a.Hin : s0n, s1 = s1n < 0 ? a.Hin : s1n;
-      if (k + 1 < a.K) {
-        s0n = conv_src(a, n0 + r, k + 1);
-        s1n = conv_src(a, n0 + 32 + r, k + 1);
-      }
-      const u32x4* row0 = xt + (int64_t)s0 * cpad8 + kh;
-      const u32x4* row1 = xt + (int64_t)s1 * cpad8 + kh;
+      const int s0n2 = src_of(k + 2, 0), s1n2 = src_of(k + 2, 1);
       for (int slab = 0; slab < nslab; ++slab, ++stage) {
         __syncthreads();
 #pragma unroll
@@ -268,12 +306,25 @@ __global__ __launch_bounds__(256) void conv_rows_bf16_kernel(ConvArgs a, uint16_
           if (idx < kWUnits) sW[idx] = wr[v];
         }
         __syncthreads();
-        if (stage + 1 < nstage) fetch_w(stage + 1);
+        const bool more = stage + 1 < nstage;
+        const bool same_tap = slab + 1 < nslab;
+        const int nslab_next = same_tap ? slab + 1 : 0;
+        const int s0x = same_tap ? s0c : s0n, s1x = same_tap ? s1c : s1n;
+        const u32x4* nrow0 = xt + (int64_t)(s0x < 0 ? a.Hin : s0x) * cpad8 + kh + ((nslab_next * kRowSlab) >> 3);
+        const u32x4* nrow1 = xt + (int64_t)(s1x < 0 ? a.Hin : s1x) * cpad8 + kh + ((nslab_next * kRowSlab) >> 3);
+        const int ngroup_next = more ? (min(kRowSlab, cpad - nslab_next * kRowSlab) >> 4) : 0;
+        if (more) fetch_w(stage + 1);
         const int ngroup = min(kRowSlab, cpad - slab * kRowSlab) >> 4;
-        for (int c16 = 0; c16 < ngroup; ++c16) {
+#pragma unroll
+        for (int c16 = 0; c16 < kRowSlab / 16; ++c16) {
           union { u32x4 q; bf16x8 v; } b0, b1;
-          b0.q = row0[(slab * kRowSlab + c16 * 16) >> 3];
-          b1.q = row1[(slab * kRowSlab + c16 * 16) >> 3];
+          b0.q = nx0[c16];
+          b1.q = nx1[c16];
+          if (c16 < ngroup_next) {
+            nx0[c16] = nrow0[c16 * 2];
+            nx1[c16] = nrow1[c16 * 2];
+          }
+          if (c16 >= ngroup) continue;  // uniform
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
             union { u32x4 q; bf16x8 v; } av;
@@ -283,6 +334,7 @@ __global__ __launch_bounds__(256) void conv_rows_bf16_kernel(ConvArgs a, uint16_
           }
         }
       }
+      s0c = s0n; s1c = s1n; s0n = s0n2; s1n = s1n2;
     }
     if (n0 < a.N) store_tiles<uint16_t, MT>(a, out, acc, pass * MT, n0, lane);
   }
