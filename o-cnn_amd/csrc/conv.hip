@@ -909,47 +909,92 @@ __device__ inline void store_children(const ConvArgs& a, OutT* __restrict__ out,
 
 constexpr int kD2MT = 4;  // row tiles per pass: 128 rows = 16 output channels x 8 children
 
-__global__ __launch_bounds__(256) void deconv_s2_f32_kernel(ConvArgs a, float* __restrict__ out,
+// fp32: a wavefront keeps its 64 columns x 64 input channels in registers (read once, coalesced,
+// reused by every pass), a pass is 64 rows = 8 output channels x 8 children whose weights
+// [64 channels][64 rows] are staged in LDS (the next pass's are in flight meanwhile), and the MFMA
+// loop reads A from LDS and B from registers.  With more than 64 input channels the register
+// block is refilled for the next chunk right after each k-step has consumed its pair.
+constexpr int kD2fMT = 2;
+constexpr int kD2fChunk = 64;
+
+__global__ __launch_bounds__(256, 2) void deconv_s2_f32_kernel(ConvArgs a, float* __restrict__ out,
     const float* __restrict__ in, const float* __restrict__ W, int n_tiles) {
+  __shared__ __attribute__((aligned(16))) float sW[kD2fChunk * 32 * kD2fMT];
+  constexpr int kWVec = kD2fChunk * 32 * kD2fMT / 4 / 256;  // float4 per thread and stage
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int tile = xcd_tile(blockIdx.x, n_tiles);
   if (tile >= n_tiles) return;
   const int n0 = tile * kTileCols + wave * kWaveCols;
-  if (n0 >= a.N) return;
   const int r = lane & 31, kh = lane >> 5;
   const int rows = a.M * 8;
-  const int npass = (rows + 32 * kD2MT - 1) / (32 * kD2MT);
-  const int ksteps = (a.Cin + 1) / 2;
+  const int npass = (rows + 32 * kD2fMT - 1) / (32 * kD2fMT);
+  const int nchunk = (a.Cin + kD2fChunk - 1) / kD2fChunk;
+  const int nstage = npass * nchunk;
   int ncol[2];
+  const float* xcol[2];
 #pragma unroll
-  for (int nt = 0; nt < 2; ++nt) ncol[nt] = n0 + nt * 32 + r;
-  for (int pass = 0; pass < npass; ++pass) {
-    floatx16 acc[kD2MT][2];
+  for (int nt = 0; nt < 2; ++nt) {
+    ncol[nt] = n0 + nt * 32 + r;
+    xcol[nt] = in + min(ncol[nt], a.N - 1);  // columns beyond N are computed but never stored
+  }
+  // channel 2ks + kh of a chunk; channels beyond Cin read channel Cin - 1 and meet zero weights
+  float xb[kD2fChunk / 2][2];
+  auto load_x = [&](int chunk, int ks) {
+    const int c = min(chunk * kD2fChunk + 2 * ks + kh, a.Cin - 1);
 #pragma unroll
-    for (int mt = 0; mt < kD2MT; ++mt)
+    for (int nt = 0; nt < 2; ++nt) xb[ks][nt] = xcol[nt][(int64_t)c * a.Hin];
+  };
+  float4 wr[kWVec];
+  auto fetch_w = [&](int stage) {
+    const int pass = stage / nchunk, chunk = stage % nchunk;
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
+    for (int v = 0; v < kWVec; ++v) {
+      const int idx = v * 256 + threadIdx.x;              // [channel][16 row quads]
+      const int c = chunk * kD2fChunk + idx / (8 * kD2fMT);
+      const int row = pass * 32 * kD2fMT + 4 * (idx % (8 * kD2fMT));
+      wr[v] = (c < a.Cin && row < rows) ? *reinterpret_cast<const float4*>(W + (int64_t)c * rows + row)
+                                        : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  };
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
-    const int row_base = pass * 32 * kD2MT;
-#pragma unroll 2
-    for (int ks = 0; ks < ksteps; ++ks) {
-      const int c = 2 * ks + kh;
-      const bool cv = c < a.Cin;
-      float b0 = (cv && ncol[0] < a.N) ? in[(int64_t)c * a.Hin + ncol[0]] : 0.0f;
-      float b1 = (cv && ncol[1] < a.N) ? in[(int64_t)c * a.Hin + ncol[1]] : 0.0f;
+  for (int ks = 0; ks < kD2fChunk / 2; ++ks) load_x(0, ks);
+  fetch_w(0);
+  floatx16 acc[kD2fMT][2];
+  for (int stage = 0; stage < nstage; ++stage) {
+    const int pass = stage / nchunk, chunk = stage % nchunk;
+    if (chunk == 0) {
 #pragma unroll
-      for (int mt = 0; mt < kD2MT; ++mt) {
-        int m = row_base + mt * 32 + r;
-        float av = (cv && m < rows) ? W[(int64_t)c * rows + m] : 0.0f;
+      for (int mt = 0; mt < kD2fMT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int v = 0; v < kWVec; ++v) reinterpret_cast<float4*>(sW)[v * 256 + threadIdx.x] = wr[v];
+    __syncthreads();
+    if (stage + 1 < nstage) fetch_w(stage + 1);
+    const int next_chunk = (chunk + 1) % nchunk;
+    const bool refill = nchunk > 1 && stage + 1 < nstage;
+#pragma unroll
+    for (int ks = 0; ks < kD2fChunk / 2; ++ks) {
+      const float b0 = xb[ks][0], b1 = xb[ks][1];
+      if (refill) load_x(next_chunk, ks);
+#pragma unroll
+      for (int mt = 0; mt < kD2fMT; ++mt) {
+        const float av = sW[(2 * ks + kh) * 32 * kD2fMT + mt * 32 + r];
         acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b0, acc[mt][0], 0, 0, 0);
         acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b1, acc[mt][1], 0, 0, 0);
       }
     }
+    if (chunk == nchunk - 1) {
+      const int row_base = pass * 32 * kD2fMT;
 #pragma unroll
-    for (int mt = 0; mt < kD2MT; ++mt)
+      for (int mt = 0; mt < kD2fMT; ++mt)
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt) store_children<float>(a, out, acc[mt][nt], row_base + mt * 32, ncol[nt], kh);
+        for (int nt = 0; nt < 2; ++nt) store_children<float>(a, out, acc[mt][nt], row_base + mt * 32, ncol[nt], kh);
+    }
   }
 }
 
@@ -1202,7 +1247,8 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
       if (MT == 1) conv_s2_bf16_kernel<1><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const uint16_t*)btm, (const uint4*)wsb, n_tiles);
       else conv_s2_bf16_kernel<2><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const uint16_t*)btm, (const uint4*)wsb, n_tiles);
     }
-  } else if (a.mode == kModeS2Deconv && !a.nempty && (reinterpret_cast<uintptr_t>(top) & 15) == 0) {
+  } else if (a.mode == kModeS2Deconv && !a.nempty && (reinterpret_cast<uintptr_t>(top) & 15) == 0 &&
+             (dtype != OCNN_F32 || (reinterpret_cast<uintptr_t>(weights) & 15) == 0)) {
     // columns are the parents here: one column tile writes the 8 children of 256 parents
     ConvArgs d = a;
     d.N = a.Hin;
