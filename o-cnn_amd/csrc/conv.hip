@@ -713,7 +713,7 @@ __global__ void pack_weights_lds_bf16(uint16_t* __restrict__ Wt, const uint16_t*
 // a wavefront load is a fully coalesced 1-KiB read and every input element is read exactly
 // once; the four values feed four MFMA k-steps whose k-pairs are (tap j, tap 4+j) -- the
 // weights are packed in that order.  HBM-bound at Cin = Cout = 64 (28 flop/byte).
-constexpr int kS2Slab = 4;  // input channels per weight slab (fp32)
+constexpr int kS2Slab = 8;  // input channels per weight slab (fp32)
 
 template <int MT>
 __global__ __launch_bounds__(256) void conv_s2_f32_kernel(ConvArgs a, float* __restrict__ out,
@@ -728,13 +728,31 @@ __global__ __launch_bounds__(256) void conv_s2_f32_kernel(ConvArgs a, float* __r
   const int r = lane & 31, kh = lane >> 5;
   const int nslab = (a.Cin + kS2Slab - 1) / kS2Slab;
   const int npass = (a.mtiles + MT - 1) / MT;
-  // element offset of my float4 inside a channel row, per column tile (-1: column out of range)
-  int64_t xoff[2];
+  // my float4 inside a channel row, per column tile.  Columns beyond N are clamped (computed, never
+  // stored) and channels beyond Cin read channel Cin - 1 (their weights are zero), so the loads
+  // carry no branch and stay in flight across the MFMAs.
+  const float* xbase[2];
 #pragma unroll
-  for (int nt = 0; nt < 2; ++nt) {
-    int n = n0 + nt * 32 + r;
-    xoff[nt] = n < a.N ? (int64_t)n * 8 + 4 * kh : -1;
-  }
+  for (int nt = 0; nt < 2; ++nt) xbase[nt] = in + (int64_t)min(n0 + nt * 32 + r, a.N - 1) * 8 + 4 * kh;
+  float4 b[kS2Slab][2];
+  auto load_x = [&](int slab, int cc) {
+    const int c = min(slab * kS2Slab + cc, a.Cin - 1);
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) b[cc][nt] = *reinterpret_cast<const float4*>(xbase[nt] + (int64_t)c * a.Hin);
+  };
+  const int nstage = npass * nslab;
+  float4 wr[kWVec];
+  auto fetch_w = [&](int stage) {
+    const float4* wsrc = reinterpret_cast<const float4*>(Wt + (int64_t)stage * kWWords);
+#pragma unroll
+    for (int v = 0; v < kWVec; ++v) {
+      int idx = v * 256 + threadIdx.x;
+      wr[v] = idx < kWWords / 4 ? wsrc[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  };
+  fetch_w(0);
+#pragma unroll
+  for (int cc = 0; cc < kS2Slab; ++cc) load_x(0, cc);
   for (int pass = 0; pass < npass; ++pass) {
     floatx16 acc[MT][2];
 #pragma unroll
@@ -743,17 +761,8 @@ __global__ __launch_bounds__(256) void conv_s2_f32_kernel(ConvArgs a, float* __r
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
-    float4 wr[kWVec];
-    auto fetch_w = [&](int slab) {
-      const float4* wsrc = reinterpret_cast<const float4*>(Wt + ((int64_t)pass * nslab + slab) * kWWords);
-#pragma unroll
-      for (int v = 0; v < kWVec; ++v) {
-        int idx = v * 256 + threadIdx.x;
-        wr[v] = idx < kWWords / 4 ? wsrc[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
-      }
-    };
-    fetch_w(0);
     for (int slab = 0; slab < nslab; ++slab) {
+      const int stage = pass * nslab + slab;
       __syncthreads();
 #pragma unroll
       for (int v = 0; v < kWVec; ++v) {
@@ -761,23 +770,17 @@ __global__ __launch_bounds__(256) void conv_s2_f32_kernel(ConvArgs a, float* __r
         if (idx < kWWords / 4) reinterpret_cast<float4*>(sW)[idx] = wr[v];
       }
       __syncthreads();
-      if (slab + 1 < nslab) fetch_w(slab + 1);
-      float4 b[kS2Slab][2];
+      const bool more = stage + 1 < nstage;
+      if (more) fetch_w(stage + 1);
+      const int next_slab = slab + 1 < nslab ? slab + 1 : 0;
 #pragma unroll
       for (int cc = 0; cc < kS2Slab; ++cc) {
-        const int c = slab * kS2Slab + cc;
-#pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
-          b[cc][nt] = (c < a.Cin && xoff[nt] >= 0)
-              ? *reinterpret_cast<const float4*>(in + (int64_t)c * a.Hin + xoff[nt])
-              : make_float4(0.f, 0.f, 0.f, 0.f);
-      }
-#pragma unroll
-      for (int cc = 0; cc < kS2Slab; ++cc)
+        const float4 c0 = b[cc][0], c1 = b[cc][1];
+        if (more) load_x(next_slab, cc);  // the next slab's channel takes the registers just read
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float b0 = j == 0 ? b[cc][0].x : j == 1 ? b[cc][0].y : j == 2 ? b[cc][0].z : b[cc][0].w;
-          const float b1 = j == 0 ? b[cc][1].x : j == 1 ? b[cc][1].y : j == 2 ? b[cc][1].z : b[cc][1].w;
+          const float b0 = j == 0 ? c0.x : j == 1 ? c0.y : j == 2 ? c0.z : c0.w;
+          const float b1 = j == 0 ? c1.x : j == 1 ? c1.y : j == 2 ? c1.z : c1.w;
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
             float av = sW[((cc * 4 + j) * MT + mt) * 64 + lane];
@@ -785,11 +788,12 @@ __global__ __launch_bounds__(256) void conv_s2_f32_kernel(ConvArgs a, float* __r
             acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b1, acc[mt][1], 0, 0, 0);
           }
         }
+      }
     }
     if (n0 < a.N) store_tiles<float, MT>(a, out, acc, pass * MT, n0, lane);
   }
 }
-// [pass][slab][cc][j][mt][lane]: lane (m, kh) <- W[m][(slab*4+cc)*8 + 4kh + j]
+// [pass][slab][cc][j][mt][lane]: lane (m, kh) <- W[m][(slab*kS2Slab+cc)*8 + 4kh + j]
 __global__ void pack_weights_s2_f32(float* __restrict__ Wt, const float* __restrict__ W, int M, int Cin, int MT,
     int npass, int nslab) {
   int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -1151,7 +1155,7 @@ int make_plan(const Info* o, int depth, int channel_in, int num_output, const in
   const bool is222 = ks[0] == 2 && ks[1] == 2 && ks[2] == 2;
   if (stride == 2 && !nempty && is222 && !deconv) {  // dedicated stride-2 kernels: padded packing
     size_t npass = (size_t)(p->mtiles + 1) / 2;
-    size_t w = dtype == OCNN_F32 ? npass * ((channel_in + 3) / 4) * kS2Slab * 4 * 2 * 64 * sizeof(float)
+    size_t w = dtype == OCNN_F32 ? npass * ((channel_in + kS2Slab - 1) / kS2Slab) * kS2Slab * 4 * 2 * 64 * sizeof(float)
                                  : npass * ((channel_in + 7) / 8) * 4 * 2 * 64 * 8 * sizeof(uint16_t);
     if (w > p->wt_bytes) p->wt_bytes = align256(w);
   }
