@@ -202,6 +202,26 @@ def main():
     extra["points2octree_scene_d9"] = {"ms": t * 1e3, "Mpts_per_s": 0.25 / t,
                                        "GBs": by / t / 1e9, "frac_hbm_peak": by / t / 1e9 / PEAK_HBM_GBS}
 
+    # the same build at a size where launches no longer dominate: 8 scenes merged, 2 M points
+    big = []
+    for i in range(8):
+      q = points_tensor(pts + np.float32(1e-4 * i), nrm, rgb)
+      q._ocnn_points_info = q[:88].cpu().numpy().copy()
+      big.append(q)
+    ob = F.points2octree_batch(big, 9, 2)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+      ob = F.points2octree_batch(big, 9, 2)
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / reps
+    ib = F.octree_info(ob)
+    nodes = sum(ib.nnum(d) for d in range(10))
+    by = 2.0e6 * 48 + nodes * 44 + ib.nnum(9) * 4 * 6 + 720
+    extra["points2octree_8scenes_d9"] = {"ms": t * 1e3, "Mpts_per_s": 2.0 / t, "nodes": nodes,
+                                         "GBs": by / t / 1e9, "frac_hbm_peak": by / t / 1e9 / PEAK_HBM_GBS}
+    del big, ob
+
     # point-cloud transforms in front of the build (normalise -> rotate/scale/jitter -> clip)
     def transform_scene():
       q = F.normalize_points(scene_pts, 1.05, [0.01, 0.0, -0.01])

@@ -669,7 +669,8 @@ int ocnn_points2octree_plan(const void* const* points_dev, const void* const* po
     o.set_property(OCNN_NEIGH, 8, -1);
   }
   o.set_nnum_cum();
-  o.set_ptr_dis();
+  OCNN_REQUIRE(o.set_ptr_dis(), OCNN_E_SHAPE,
+      "the octree would exceed the 2 GiB that the 32-bit offsets of the serialized format can address");
   memcpy(info_out, &o, sizeof(Info));
 
   st.params = *params;

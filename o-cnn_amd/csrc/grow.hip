@@ -157,7 +157,8 @@ int ocnn_octree_batch_info(const void* const* infos, int n, void* out_info) {
     o.nnum_nempty[d] = (int)b;
   }
   o.set_nnum_cum();
-  o.set_ptr_dis();
+  OCNN_REQUIRE(o.set_ptr_dis(), OCNN_E_SHAPE,
+      "the octree would exceed the 2 GiB that the 32-bit offsets of the serialized format can address");
   memcpy(out_info, &o, sizeof(Info));
   return OCNN_OK;
 }
@@ -259,7 +260,8 @@ int ocnn_octree_new_info(int batch_size, int channel, int node_dis, int adaptive
   o.nnum[0] = batch_size;
   o.set_nnum_cum();
   o.nnum_nempty[0] = batch_size;
-  o.set_ptr_dis();
+  OCNN_REQUIRE(o.set_ptr_dis(), OCNN_E_SHAPE,
+      "the octree would exceed the 2 GiB that the 32-bit offsets of the serialized format can address");
   memcpy(out_info, &o, sizeof(Info));
   return OCNN_OK;
 }
@@ -298,7 +300,8 @@ int ocnn_octree_grow_info(const void* in_info, int target_depth, int full_octree
   o.nnum[target_depth] = (int)node_num;
   o.nnum_nempty[target_depth] = (int)node_num;
   o.set_nnum_cum();
-  o.set_ptr_dis();
+  OCNN_REQUIRE(o.set_ptr_dis(), OCNN_E_SHAPE,
+      "the octree would exceed the 2 GiB that the 32-bit offsets of the serialized format can address");
   memcpy(out_info, &o, sizeof(Info));
   return OCNN_OK;
 }

@@ -2,6 +2,8 @@
 // kernel-shape tables.  Layout rules follow octree/octree/octree_info.cpp:143-268.
 #include "ocnn_common.h"
 
+#include <cstdint>
+
 #include <stdarg.h>
 #include <stdio.h>
 
@@ -39,14 +41,19 @@ void Info::set_nnum_cum(int capacity) {
   nnum_cum[depth + 2] = capacity > nnum_cum[depth + 1] ? capacity : nnum_cum[depth + 1];
 }
 
-void Info::set_ptr_dis() {
-  ptr_dis_[0] = OCNN_HEADER_BYTES;
+bool Info::set_ptr_dis() {
+  int64_t dis = OCNN_HEADER_BYTES;
+  ptr_dis_[0] = (int)dis;
+  bool fits = true;
   for (int i = 1; i <= 6; ++i) {
     int ptype = 1 << (i - 1);
     int lc = location(ptype);
     int num = lc == -1 ? total_capacity() : nnum[lc];
-    ptr_dis_[i] = ptr_dis_[i - 1] + size_of(ptype) * num * channels[i - 1];
+    dis += (int64_t)size_of(ptype) * num * channels[i - 1];
+    if (dis > INT32_MAX || num < 0) fits = false;
+    ptr_dis_[i] = fits ? (int)dis : INT32_MAX;
   }
+  return fits;
 }
 
 float Info::bbox_max_width() const {
@@ -152,7 +159,7 @@ int ocnn_upgrade_key64(const void* octree32, size_t bytes, void* out, size_t out
   OCNN_REQUIRE((size_t)in->ptr_dis_[6] <= bytes, OCNN_E_FORMAT, "blob shorter than its header says");
   Info o = *in;
   memcpy(o.magic, "_OCTREE_2.0_", 13);
-  o.set_ptr_dis();
+  OCNN_REQUIRE(o.set_ptr_dis(), OCNN_E_SHAPE, "the upgraded octree exceeds the 2 GiB the format can address");
   *out_bytes = (size_t)o.sizeof_octree();
   if (!out) return OCNN_OK;  // size query
   OCNN_REQUIRE(out_capacity >= *out_bytes, OCNN_E_WORKSPACE, "output %zu < %zu bytes", out_capacity, *out_bytes);

@@ -55,7 +55,8 @@ struct Info {
   void set_depth(int d) { depth = full_layer < d ? d : full_layer; }
   void set_full_layer(int fd) { full_layer = fd < 1 ? 1 : fd; }
   void set_nnum_cum(int capacity = 0);
-  void set_ptr_dis();
+  // false: the blob would exceed what the 32-bit offsets of the serialized format can address
+  bool set_ptr_dis();
   float bbox_max_width() const;
   bool consistent_with(const Info& o) const;
 };

@@ -271,3 +271,22 @@ def test_update_degenerate_and_errors(oc, orc):
   assert e.value.code == -3
   with pytest.raises(oc.lib.OcnnError):
     F.octree_grow(o, 3, False)
+
+
+def test_octree_beyond_the_format_limit_is_refused(oc, synthetic):
+  """The serialized format addresses its payload with 32-bit offsets (octree_info.h: ptr_dis_),
+  so an octree above 2 GiB cannot be represented: an error code, never a wrapped size."""
+  F = oc.nn
+  p, n, f = synthetic.room_cloud(250000, 3)
+  clouds = []
+  for i in range(24):
+    blob = make_points_blob(p + np.float32(1e-4 * i), n, f)
+    t = T(blob).cuda()
+    t._ocnn_points_info = blob[:88].copy()
+    clouds.append(t)
+  with pytest.raises(oc.lib.OcnnError) as e:
+    F.points2octree_batch(clouds, 9, 2)
+  assert e.value.code == -3 and "2 GiB" in str(e.value)
+  # the workspace is reusable after the refusal
+  o = F.points2octree_batch(clouds[:2], 9, 2)
+  assert F.octree_info(o).batch_size == 2
