@@ -272,6 +272,26 @@ int ocnn_points2octree_plan(const void* const* points_dev, const void* const* po
     void* info_out, ocnn_stream_t stream);
 int ocnn_points2octree_emit(void* octree_out_dev, const void* info, void* workspace_dev,
     size_t workspace_bytes, ocnn_stream_t stream);
+/* Both steps in one call: after step 1 the blob is obtained from `alloc(bytes, alloc_ctx)`
+ * (device memory, 8-byte aligned, owned by the caller; a null return fails the call) and
+ * returned in *octree_out_dev.  Same result as the two steps; it spares the host work
+ * between them, which is a sizeable part of a small build
+ * (pytorch/cpp/point2octree.cpp:5-34 allocates its output tensor the same way, after
+ * the build knows its size). */
+/* The sort and the level scan chain their tiles through bounded waits.  The first attempt
+ * of a plan orders tiles by workgroup index; if a wait of `polls` polls runs out, the plan is
+ * repeated once with ticket order (slower, cannot starve).  ocnn_points2octree_wait_limit sets
+ * `polls` (0 restores the default, a negative value fails every first attempt: used by the
+ * tests to exercise the repeat) and returns the previous value;
+ * ocnn_points2octree_ticket_reruns counts the repeats so far.  No counterpart in the
+ * reference, whose build is sequential. */
+int ocnn_points2octree_wait_limit(int polls);
+int ocnn_points2octree_ticket_reruns(void);
+typedef void* (*ocnn_alloc_fn)(size_t bytes, void* alloc_ctx);
+int ocnn_points2octree(const void* const* points_dev, const void* const* points_info,
+    int n_clouds, const ocnn_build_params* params, void* workspace_dev, size_t workspace_bytes,
+    ocnn_alloc_fn alloc, void* alloc_ctx, void* info_out, void** octree_out_dev,
+    ocnn_stream_t stream);
 
 /* ---- octree_batch of already serialized octrees that live on the device
  * (merge_octrees, octree/octree/merge_octrees.cpp:7-198).  `out_info` (host)

@@ -7,42 +7,35 @@
 // Here ONE sort handles every cloud of the batch: the sort key is
 // (cloud << 3*depth | morton), so the sorted order is already the node order of
 // the merged batch octree, and child links are global ranks -- exactly what
-// merge_octrees produces by offsetting per-cloud links.  Steps:
-//   keygen -> stable LSD radix sort (8-bit digits, wavefront-ballot ranking)
-//   -> unique leaves (flag scan) -> per level: parents = unique(key >> 3)
-//   -> [one copy of the level sizes to the host: the caller must size the blob]
-//   -> per level keys / children written straight into the blob, leaf signal
-//      averaged per leaf in ascending point order (same float summation order as
-//      the reference), neighbour tables level by level.
-#include "ocnn_common.h"
-#include "scan.h"
+// merge_octrees produces by offsetting per-cloud links.  A small octree is bound
+// by the number of dependent launches and memory round trips, so the work is
+// packed into few launches with short dependency chains:
+//
+//   plan:  init (control words, cloud table)
+//          keys + the digit histograms of every sort pass
+//          one launch per sort pass: stable LSD radix sort; each tile publishes
+//            its digit counts and looks back over the tiles before it for its
+//            global offsets (no separate scan launches)
+//          ONE scan for every level at once: element i starts a new node at level
+//            d iff it differs from element i-1 above bit 3*(depth-d); the
+//            per-level counts travel as 16-bit fields of four 64-bit words
+//          [one copy of the level sizes to the host: the caller must size the blob]
+//   emit:  one launch writes header, keys, children, split labels and full-layer
+//            neighbour tables of every level (the children of a sibling group
+//            are found by position, nothing is scattered);
+//          one launch writes the signal of the finest level, a full row per
+//            wavefront (zeros for empty nodes);
+//          one launch per sparse level for the neighbour tables (each needs the
+//            level above).
+#include "octree_kernels.h"
 
+#include <atomic>
+#include <type_traits>
 #include <map>
 #include <mutex>
 #include <vector>
 
 namespace ocnn {
-
-// from octree_index.hip
-__host__ __device__ inline uint64_t b_spread3(uint64_t v) {
-  v &= 0xffffull;
-  v = (v | (v << 32)) & 0x00ff00000000ffffull;
-  v = (v | (v << 16)) & 0x00ff0000ff0000ffull;
-  v = (v | (v << 8)) & 0xf00f00f00f00f00full;
-  v = (v | (v << 4)) & 0x30c30c30c30c30c3ull;
-  v = (v | (v << 2)) & 0x9249249249249249ull;
-  return v;
-}
-__host__ __device__ inline uint64_t b_compact3(uint64_t v) {
-  v &= 0x9249249249249249ull;
-  v = (v | (v >> 2)) & 0x30c30c30c30c30c3ull;
-  v = (v | (v >> 4)) & 0xf00f00f00f00f00full;
-  v = (v | (v >> 8)) & 0x00ff0000ff0000ffull;
-  v = (v | (v >> 16)) & 0x00ff00000000ffffull;
-  v = (v | (v >> 32)) & 0xffffull;
-  return v;
-}
-
 namespace {
 
 struct CloudDesc {
@@ -54,17 +47,37 @@ struct CloudDesc {
 };
 
 constexpr int kMaxLevels = 17;
-struct Counts {            // device-resident, copied to the host once
-  int nne[kMaxLevels];     // non-empty nodes per depth (valid for depth >= full_layer)
-  int pad[15];
+constexpr int kMaxPasses = 8;
+constexpr uint32_t kFlagSum = 1u << 30;    // status word: published (the count is in the low bits)
+constexpr uint32_t kCountMask = (1u << 30) - 1;
+
+struct Control {                 // device-resident, zeroed by init_kernel
+  int nne[kMaxLevels];           // non-empty nodes per depth (valid for depth >= full_layer)
+  int error;                     // a bounded wait ran out (never expected)
+  unsigned ticket[kMaxPasses + 1];  // tile tickets: one per sort pass, the last for the level scan
+  int pad[5];
 };
+static_assert(sizeof(Control) == 128, "Control layout");
 
 struct BuildGeom {
   int depth, full_layer, n_clouds;
+  int passes, bits;            // sort: `passes` digits of `bits` bits each
   int64_t n_points;
   float bbmin[3];
-  float mul;               // 2^depth / bbox width, computed on the host in fp32
+  float mul;                   // 2^depth / bbox width, computed on the host in fp32
 };
+
+// ---- 0. control words and the cloud table ---------------------------------------------
+constexpr int kArgClouds = 48;
+struct CloudChunk { CloudDesc c[kArgClouds]; };
+
+__global__ void init_kernel(uint32_t* __restrict__ zero, int64_t zero_words, CloudDesc* __restrict__ clouds,
+    CloudChunk chunk, int first, int count) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) clouds[first + i] = chunk.c[i];
+  const int64_t step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < zero_words; i += step) zero[i] = 0;
+}
 
 // ---- 1. keys -----------------------------------------------------------------------
 __device__ inline int find_cloud(const CloudDesc* __restrict__ clouds, int n_clouds, int64_t i) {
@@ -88,247 +101,461 @@ __device__ inline float scale_coord(float p, float bbmin, float mul) {
   return __fmul_rn(__fsub_rn(p, bbmin), mul);
 }
 
-__global__ void keygen_kernel(uint64_t* __restrict__ key, uint32_t* __restrict__ val,
-    const CloudDesc* __restrict__ clouds, BuildGeom g) {
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= g.n_points) return;
-  int b = find_cloud(clouds, g.n_clouds, i);
-  const float* p = clouds[b].xyz + 3 * (i - clouds[b].offset);
-  uint64_t m = (1ull << g.depth) - 1;
-  uint64_t k = 0;
-#pragma unroll
-  for (int j = 0; j < 3; ++j) {
-    // float -> unsigned truncation as static_cast<uintk> (octree.cpp:184); only the low
-    // `depth` bits are interleaved (octree_nn.cpp:551-560)
-    uint32_t q = (uint32_t)scale_coord(p[j], g.bbmin[j], g.mul);
-    k |= b_spread3(q & m) << (2 - j);
-  }
-  key[i] = ((uint64_t)b << (3 * g.depth)) | k;
-  val[i] = (uint32_t)i;
-}
-
-// ---- 2. radix sort (LSD, 8-bit digits, stable) ----------------------------------------
-constexpr int kSortItems = 8;
-constexpr int kSortTile = kBlock * kSortItems;   // 2048 elements per workgroup
-constexpr int kWaves = kBlock / 64;
-
-__global__ void radix_hist_kernel(const uint64_t* __restrict__ key, int64_t n, int shift,
-    int* __restrict__ hist, int n_blocks) {
-  __shared__ int h[256];
-  h[threadIdx.x] = 0;
-  __syncthreads();
-  int64_t base = (int64_t)blockIdx.x * kSortTile;
-#pragma unroll
-  for (int q = 0; q < kSortItems; ++q) {
-    int64_t i = base + q * kBlock + threadIdx.x;
-    if (i < n) atomicAdd(&h[(int)((key[i] >> shift) & 255)], 1);
-  }
-  __syncthreads();
-  hist[(int64_t)threadIdx.x * n_blocks + blockIdx.x] = h[threadIdx.x];  // digit-major
-}
-
-// Scan of the digit-major histogram in two levels: workgroup d turns row d (the counts of
-// digit d in every tile) into exclusive offsets within the digit and records the digit
-// total; the scatter kernel adds the exclusive scan of the 256 totals itself.
-__global__ void radix_scan_kernel(int* __restrict__ hist, int n_blocks, int* __restrict__ digit_total) {
-  __shared__ int carry;
-  int* row = hist + (int64_t)blockIdx.x * n_blocks;
-  if (threadIdx.x == 0) carry = 0;
-  __syncthreads();
-  for (int start = 0; start < n_blocks; start += kBlock) {
-    int i = start + threadIdx.x;
-    int v = i < n_blocks ? row[i] : 0;
-    int total;
-    int ex = block_exclusive_scan(v, &total);
-    int c = carry;
-    if (i < n_blocks) row[i] = c + ex;
+// Sort keys and, on the way, the digit histogram of every sort pass (the passes
+// themselves then need no counting launch).  Neighbouring points mostly share their high
+// digits: a wavefront whose lanes all hold the same digit adds its count once instead of
+// serialising 64 LDS atomics on one address.
+constexpr int kKeyItems = 8;
+constexpr int kKeyGrid = 512;   // workgroups at most: each adds its histograms to the global ones once
+constexpr int kHistCopies = 16; // global histogram copies: atomics on one address are served one by one
+__global__ __launch_bounds__(kBlock) void keygen_kernel(uint64_t* __restrict__ key, uint32_t* __restrict__ val,
+    const CloudDesc* __restrict__ clouds, int* __restrict__ hist, BuildGeom g) {
+  __shared__ int h[kMaxPasses][256];
+  __shared__ int s_off[kBlock + 1];     // offsets of the clouds a chunk touches
+  for (int p = 0; p < g.passes; ++p) h[p][threadIdx.x] = 0;
+  const uint64_t m = (1ull << g.depth) - 1;
+  const uint32_t dmask = (1u << g.bits) - 1;
+  const int lane = threadIdx.x & 63;
+  const int64_t chunks = (g.n_points + kBlock * kKeyItems - 1) / (kBlock * kKeyItems);
+  for (int64_t chunk = blockIdx.x; chunk < chunks; chunk += gridDim.x) {
+    const int64_t base = chunk * (kBlock * kKeyItems);
+    const int64_t last = min(base + kBlock * kKeyItems, g.n_points) - 1;
+    // clouds of the first and last point of the chunk; the table between them goes to LDS
+    const int b_lo = find_cloud(clouds, g.n_clouds, base);
+    const int b_hi = find_cloud(clouds, g.n_clouds, last);
+    const int span = min(b_hi - b_lo + 1, kBlock);
     __syncthreads();
-    if (threadIdx.x == 0) carry = c + total;
+    if ((int)threadIdx.x < span) s_off[threadIdx.x] = clouds[b_lo + threadIdx.x].offset;
     __syncthreads();
+    int cloud[kKeyItems];
+    float xyz[kKeyItems][3];
+#pragma unroll
+    for (int q = 0; q < kKeyItems; ++q) {
+      const int64_t i = base + q * kBlock + threadIdx.x;
+      cloud[q] = 0;
+      xyz[q][0] = xyz[q][1] = xyz[q][2] = 0.0f;
+      if (i < g.n_points) {
+        int b = b_lo;
+        if (b_hi - b_lo < kBlock) {  // last cloud of the span with offset <= i
+          int lo = 0, hi = span - 1;
+          while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (s_off[mid] <= i) lo = mid; else hi = mid - 1;
+          }
+          b += lo;
+        } else {
+          b = find_cloud(clouds, g.n_clouds, i);
+        }
+        cloud[q] = b;
+        const float* p = clouds[b].xyz + 3 * (i - clouds[b].offset);
+        xyz[q][0] = p[0]; xyz[q][1] = p[1]; xyz[q][2] = p[2];
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < kKeyItems; ++q) {
+      const int64_t i = base + q * kBlock + threadIdx.x;
+      const bool valid = i < g.n_points;
+      uint64_t k = 0;
+#pragma unroll
+      for (int j = 0; j < 3; ++j) {
+        // float -> unsigned truncation as static_cast<uintk> (octree.cpp:184); only the low
+        // `depth` bits are interleaved (octree_nn.cpp:551-560)
+        uint32_t c = (uint32_t)scale_coord(xyz[q][j], g.bbmin[j], g.mul);
+        k |= spread3(c & m) << (2 - j);
+      }
+      k |= (uint64_t)cloud[q] << (3 * g.depth);
+      if (valid) {
+        key[i] = k;
+        val[i] = (uint32_t)i;
+      }
+      const uint64_t active = __ballot(valid);
+      if (active != 0) {
+        const int leader = __ffsll((long long)active) - 1;
+        for (int ps = 0; ps < g.passes; ++ps) {
+          const int d = (int)((uint32_t)(k >> (ps * g.bits)) & dmask);
+          const int d0 = __shfl(d, leader, 64);
+          if (__ballot(valid && d != d0) == 0) {
+            if (lane == leader) atomicAdd(&h[ps][d0], __popcll(active));
+          } else if (valid) {
+            atomicAdd(&h[ps][d], 1);
+          }
+        }
+      }
+    }
   }
-  if (threadIdx.x == 0) digit_total[blockIdx.x] = carry;
+  __syncthreads();
+  for (int p = 0; p < g.passes; ++p) {
+    const int c = h[p][threadIdx.x];
+    if (c) atomicAdd(&hist[((blockIdx.x % kHistCopies) * kMaxPasses + p) * 256 + threadIdx.x], c);
+  }
 }
 
-// Each round places 256 consecutive elements; inside a wavefront the rank among
-// equal digits comes from eight ballots (one per digit bit), across wavefronts and
-// rounds from per-digit running counters in LDS.  Element order (round, wavefront,
-// lane) equals the input order, which keeps the sort stable.
-__global__ void radix_scatter_kernel(const uint64_t* __restrict__ key_in, const uint32_t* __restrict__ val_in,
-    uint64_t* __restrict__ key_out, uint32_t* __restrict__ val_out, int64_t n, int shift,
-    const int* __restrict__ hist, int n_blocks, const int* __restrict__ digit_total) {
-  __shared__ int running[256];
-  __shared__ int wave_cnt[kWaves][256];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  {
-    int total;
-    int digit_base = block_exclusive_scan(digit_total[threadIdx.x], &total);
-    running[threadIdx.x] = digit_base + hist[(int64_t)threadIdx.x * n_blocks + blockIdx.x];
-  }
+// ---- 2. radix sort (LSD, stable), one launch per digit ------------------------------------
+__device__ inline uint32_t status_load(const uint32_t* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ inline void status_store(uint32_t* p, uint32_t v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Sum of the counts of tiles 0 .. tile-1 for one scan lane (a digit / a level), in two levels:
+// tiles form groups of 32.  Every tile publishes its count; the last tile of a group adds the
+// group up and publishes the group's count; a tile then needs the counts of the groups before
+// its own and of the tiles before it inside its group.  All tiles start together, so a chain
+// that walks back tile by tile would take as many round trips as there are tiles; here it is
+// two hand-offs whatever the number of tiles.
+//
+// A tile only ever waits for tiles before it.  First try: tile = workgroup index, which ends
+// as long as the device starts workgroups in index order (a thousand same-address ticket
+// atomics cost more than the pass itself).  Every wait is bounded; if one ever runs out, the
+// host repeats the plan with tile ids drawn from a ticket counter, where every earlier tile
+// is running by construction.
+constexpr int kGroupTiles = 32;
+
+// sum of `count` (<= 32) status words of one scan lane from tile / group `first` on, waiting
+// until all of them are published; `stride` = scan lanes per tile (the words of one tile are
+// contiguous, so a workgroup reads and writes whole rows).  All words are requested together.
+__device__ inline int wait_sum(const uint32_t* __restrict__ status, int stride, int lane_id, int first, int count,
+    int spin_limit, int* __restrict__ error) {
+  const uint32_t* p = status + (int64_t)first * stride + lane_id;
+  int spins = 0;
+  for (;;) {
+    uint32_t s[kGroupTiles];
 #pragma unroll
-  for (int w = 0; w < kWaves; ++w) wave_cnt[w][threadIdx.x] = 0;
-  __syncthreads();
-  int64_t base = (int64_t)blockIdx.x * kSortTile;
-  for (int q = 0; q < kSortItems; ++q) {
-    int64_t i = base + q * kBlock + threadIdx.x;
-    bool valid = i < n;
-    uint64_t k = valid ? key_in[i] : 0;
-    uint32_t v = valid ? val_in[i] : 0;
-    int d = (int)((k >> shift) & 255);
+    for (int j = 0; j < kGroupTiles; ++j) s[j] = j < count ? status_load(p + (int64_t)j * stride) : kFlagSum;
+    uint32_t all = kFlagSum;
+    int sum = 0;
+#pragma unroll
+    for (int j = 0; j < kGroupTiles; ++j) { all &= s[j]; sum += (int)(s[j] & kCountMask); }
+    if (all & kFlagSum) return sum;
+    if (++spins > spin_limit) { *error = 1; return sum; }
+    __builtin_amdgcn_s_sleep(1);
+  }
+}
+
+// publish the count of (tile, lane)
+__device__ inline void tile_publish(uint32_t* __restrict__ tile_status, int stride, int lane_id, int tile, int cnt) {
+  status_store(&tile_status[(int64_t)tile * stride + lane_id], (uint32_t)cnt | kFlagSum);
+}
+// counts of all tiles before `tile` (after tile_publish)
+__device__ inline int tile_prefix(const uint32_t* __restrict__ tile_status, uint32_t* __restrict__ group_status,
+    int stride, int lane_id, int tile, int cnt, int spin_limit, int* __restrict__ error) {
+  const int g = tile / kGroupTiles, j = tile % kGroupTiles;
+  const int within = j > 0 ? wait_sum(tile_status, stride, lane_id, g * kGroupTiles, j, spin_limit, error) : 0;
+  if (j == kGroupTiles - 1) status_store(&group_status[(int64_t)g * stride + lane_id], (uint32_t)(within + cnt) | kFlagSum);
+  int before = within;
+  for (int g0 = 0; g0 < g; g0 += kGroupTiles)
+    before += wait_sum(group_status, stride, lane_id, g0, min(kGroupTiles, g - g0), spin_limit, error);
+  return before;
+}
+
+// A tile is 256 * ITEMS consecutive elements; wavefront w owns the w-th quarter and ranks it
+// 64 elements at a time: the rank among equal digits inside a round comes from ballots (one
+// per digit bit), across rounds from the wavefront's own running counters in LDS, so the
+// order (wavefront, round, lane) equals the input order and the sort is stable.  The tile is
+// then reordered in LDS so that equal digits leave as contiguous runs.
+template <int ITEMS, bool TICKETS>
+__global__ __launch_bounds__(kBlock) void sort_pass_kernel(const uint64_t* __restrict__ key_in,
+    const uint32_t* __restrict__ val_in, uint64_t* __restrict__ key_out, uint32_t* __restrict__ val_out, int n,
+    int shift, int bits, const int* __restrict__ hist, uint32_t* __restrict__ status,
+    uint32_t* __restrict__ group_status, Control* __restrict__ ctl, int pass, int spin_limit) {
+  constexpr int kTile = kBlock * ITEMS;
+  __shared__ int s_tile;
+  __shared__ int wave_cnt[kBlock / 64][256];
+  __shared__ int s_gbase[256];
+  __shared__ uint64_t s_key[kTile];
+  __shared__ uint32_t s_val[kTile];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (TICKETS) {
+    if (tid == 0) s_tile = (int)atomicAdd(&ctl->ticket[pass], 1u);
+    __syncthreads();
+  }
+  if (spin_limit < 0 && tid == 0 && blockIdx.x == 0) ctl->error = 1;  // a forced failure (tests)
+  const int tile = TICKETS ? s_tile : (int)blockIdx.x;
+  const int tile_n = min(kTile, n - tile * kTile);
+  const int wbase = tile * kTile + wave * 64 * ITEMS;
+  const uint32_t dmask = (1u << bits) - 1;
+
+  uint64_t k[ITEMS];
+  uint32_t v[ITEMS];
+  int loc[ITEMS];
+#pragma unroll
+  for (int q = 0; q < ITEMS; ++q) {
+    const int i = wbase + q * 64 + lane;
+    k[q] = i < n ? key_in[i] : 0;
+    v[q] = i < n ? val_in[i] : 0;
+  }
+  int digit_total = 0;
+#pragma unroll
+  for (int c = 0; c < kHistCopies; ++c) digit_total += hist[c * kMaxPasses * 256 + tid];
+#pragma unroll
+  for (int w = 0; w < kBlock / 64; ++w) wave_cnt[w][tid] = 0;
+  int unused;
+  const int digit_base = block_exclusive_scan(digit_total, &unused);  // elements with a smaller digit
+  // Rank of an element among the lanes of its round with the same digit: from ballots.  The
+  // first lane of each digit group then adds the group to the wavefront's counter; the LDS
+  // unit applies the atomics of a wavefront in program order, so the returned values are the
+  // counts of the earlier rounds and the rounds need not wait for one another.
+  int leader[ITEMS], earlier[ITEMS];
+#pragma unroll
+  for (int q = 0; q < ITEMS; ++q) {
+    const bool valid = wbase + q * 64 + lane < n;
+    const int d = (int)((uint32_t)(k[q] >> shift) & dmask);
     uint64_t peers = __ballot(valid);
-#pragma unroll
-    for (int b = 0; b < 8; ++b) {
-      uint64_t m = __ballot((d >> b) & 1);
+    for (int b = 0; b < bits; ++b) {
+      const uint64_t m = __ballot((d >> b) & 1);
       peers &= ((d >> b) & 1) ? m : ~m;
     }
-    int rank = __popcll(peers & ((1ull << lane) - 1));
-    if (valid && rank == 0) wave_cnt[wave][d] = __popcll(peers);
-    __syncthreads();
-    if (valid) {
-      int pos = running[d] + rank;
-      for (int w = 0; w < wave; ++w) pos += wave_cnt[w][d];
-      key_out[pos] = k;
-      val_out[pos] = v;
-    }
-    __syncthreads();
-    {
-      int t = 0;
+    loc[q] = __popcll(peers & ((1ull << lane) - 1));
+    leader[q] = valid ? __ffsll((long long)peers) - 1 : lane;
+    earlier[q] = 0;
+    if (valid && leader[q] == lane) earlier[q] = atomicAdd(&wave_cnt[wave][d], __popcll(peers));
+  }
 #pragma unroll
-      for (int w = 0; w < kWaves; ++w) { t += wave_cnt[w][threadIdx.x]; wave_cnt[w][threadIdx.x] = 0; }
-      running[threadIdx.x] += t;
+  for (int q = 0; q < ITEMS; ++q) loc[q] += __shfl(earlier[q], leader[q], 64);
+  __syncthreads();
+  // thread = digit: count of the tile (published at once: later tiles wait for it), position of
+  // the digit's run inside the tile, offsets of the wavefronts inside the run
+  int cnt = 0, local;
+  {
+    int c[kBlock / 64];
+#pragma unroll
+    for (int w = 0; w < kBlock / 64; ++w) { c[w] = wave_cnt[w][tid]; cnt += c[w]; }
+    tile_publish(status, 256, tid, tile, cnt);
+    local = block_exclusive_scan(cnt, &unused);
+    int run = local;
+#pragma unroll
+    for (int w = 0; w < kBlock / 64; ++w) { wave_cnt[w][tid] = run; run += c[w]; }
+  }
+  __syncthreads();
+  // reorder the tile in LDS (this needs nothing from other tiles and frees the registers)
+#pragma unroll
+  for (int q = 0; q < ITEMS; ++q) {
+    if (wbase + q * 64 + lane < n) {
+      const int d = (int)((uint32_t)(k[q] >> shift) & dmask);
+      const int p = wave_cnt[wave][d] + loc[q];
+      s_key[p] = k[q];
+      s_val[p] = v[q];
     }
-    __syncthreads();
+  }
+  s_gbase[tid] = digit_base - local + tile_prefix(status, group_status, 256, tid, tile, cnt, spin_limit, &ctl->error);
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < ITEMS; ++q) {
+    const int t = q * kBlock + tid;
+    if (t < tile_n) {
+      const uint64_t kk = s_key[t];
+      const int pos = s_gbase[(uint32_t)(kk >> shift) & dmask] + t;
+      key_out[pos] = kk;
+      val_out[pos] = s_val[t];
+    }
   }
 }
 
-// ---- 3. unique leaves and parent levels ------------------------------------------------
-struct LeafPred {
-  const uint64_t* key; int64_t n;
-  __device__ bool operator()(int64_t i) const { return i == 0 || key[i] != key[i - 1]; }
+// ---- 3. all levels in one scan -------------------------------------------------------------
+// Element i of the sorted keys is the first point of a new node at level d iff it differs
+// from element i-1 in a bit at or above 3*(depth-d).  Its `first level` a (relative to the
+// full layer) says it heads a node at every level >= a.  The number of heads at level
+// full_layer + f up to an element is carried in field f (16 bits) of four 64-bit words, so
+// one scan serves every level.
+// (named members, not an array: a run-time choice between array elements would be turned into
+// indexed addressing and move the whole struct out of the registers)
+struct Packed4 {
+  uint64_t w0, w1, w2, w3;
 };
-struct LeafOut {
-  const uint64_t* key; uint64_t* ukey; int* ustart; int64_t n;
-  __device__ void operator()(int64_t i, bool f, int rank) const {
-    if (f) { ukey[rank] = key[i]; ustart[rank] = (int)i; }
-    if (i == n - 1) ustart[rank + (f ? 1 : 0)] = (int)n;
+template <int N, class F>
+__device__ inline void static_for(F&& f) {
+  if constexpr (N > 0) {
+    static_for<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
   }
-};
-// list_d (size *n_dev) -> list_{d-1}: heads of runs of equal key >> 3
-struct ParentPred {
-  const uint64_t* list; const int* n_dev;
-  __device__ bool operator()(int64_t j) const {
-    return j < *n_dev && (j == 0 || (list[j] >> 3) != (list[j - 1] >> 3));
+}
+__device__ inline uint64_t heads_word(int s) {  // fields >= s of one word set to 1
+  constexpr uint64_t kOnes = 0x0001000100010001ull;
+  return s <= 0 ? kOnes : (s >= 4 ? 0ull : kOnes << (16 * s));
+}
+__device__ inline Packed4 heads_from(int a) {  // one count in every field f >= a
+  return Packed4{heads_word(a), heads_word(a - 4), heads_word(a - 8), heads_word(a - 12)};
+}
+__device__ inline void add_to(Packed4& a, const Packed4& b) {
+  a.w0 += b.w0; a.w1 += b.w1; a.w2 += b.w2; a.w3 += b.w3;
+}
+__device__ inline int field_of(const Packed4& p, int f) {
+  const uint64_t lo = f < 4 ? p.w0 : p.w1, hi = f < 12 ? p.w2 : p.w3;
+  const uint64_t w = f < 8 ? lo : hi;
+  return (int)((w >> (16 * (f & 3))) & 0xffff);
+}
+__device__ inline uint64_t wave_inclusive_scan_u64(uint64_t v) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const uint64_t t = __shfl_up((unsigned long long)v, d, 64);
+    if (lane >= d) v += t;
   }
-};
-struct ParentOut {
-  const uint64_t* list; const int* n_dev; uint64_t* parent_list; int* prank;
-  __device__ void operator()(int64_t j, bool f, int rank) const {
-    if (j >= *n_dev) return;
-    int r = rank + (f ? 1 : 0) - 1;  // rank of this element's parent
-    prank[j] = r;
-    if (f) parent_list[r] = list[j] >> 3;
+  return v;
+}
+__device__ inline Packed4 block_exclusive_scan_p4(Packed4 v, Packed4* block_total) {
+  __shared__ uint64_t wave_sum[kBlock / 64][4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const Packed4 inc = {wave_inclusive_scan_u64(v.w0), wave_inclusive_scan_u64(v.w1), wave_inclusive_scan_u64(v.w2),
+      wave_inclusive_scan_u64(v.w3)};
+  if (lane == 63) {
+    wave_sum[wave][0] = inc.w0; wave_sum[wave][1] = inc.w1; wave_sum[wave][2] = inc.w2; wave_sum[wave][3] = inc.w3;
   }
+  __syncthreads();
+  uint64_t base[4] = {0, 0, 0, 0}, tot[4] = {0, 0, 0, 0};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+#pragma unroll
+    for (int w = 0; w < kBlock / 64; ++w) {
+      const uint64_t s = wave_sum[w][j];
+      if (w < wave) base[j] += s;
+      tot[j] += s;
+    }
+  }
+  __syncthreads();
+  *block_total = Packed4{tot[0], tot[1], tot[2], tot[3]};
+  return Packed4{base[0] + inc.w0 - v.w0, base[1] + inc.w1 - v.w1, base[2] + inc.w2 - v.w2, base[3] + inc.w3 - v.w3};
+}
+
+struct LevelOut {
+  uint64_t* list[kMaxLevels];   // list[d][r]: key (cloud << 3d | morton) of the r-th non-empty node of level d
+  int* first[kMaxLevels];       // first[d][r]: rank at level d+1 of that node's first child; [nne_d] = nne_{d+1}
+  int* ustart;                  // first sorted point of each leaf; [n_leaf] = n_points
 };
 
-// ---- 4. emit: structure -------------------------------------------------------------------
-struct EmitGeom {
-  int depth, full_layer, n_clouds, key2xyz, key_channel;
-};
+constexpr int kLevelItems = 8;
+constexpr int kLevelTile = kBlock * kLevelItems;
 
+template <bool TICKETS>
+__global__ __launch_bounds__(kBlock) void levels_kernel(const uint64_t* __restrict__ key, int n, int depth,
+    int full_layer, LevelOut out, uint32_t* __restrict__ status, uint32_t* __restrict__ group_status,
+    Control* __restrict__ ctl, int spin_limit) {
+  __shared__ int s_tile;
+  __shared__ int s_before[16];
+  const int tid = threadIdx.x;
+  if (TICKETS) {
+    if (tid == 0) s_tile = (int)atomicAdd(&ctl->ticket[kMaxPasses], 1u);
+    __syncthreads();
+  }
+  const int tile = TICKETS ? s_tile : (int)blockIdx.x;
+  const int L = depth - full_layer + 1;  // levels full_layer .. depth
+  const int i0 = tile * kLevelTile + tid * kLevelItems;
+
+  uint64_t k[kLevelItems];
+  int a[kLevelItems];
+  const uint64_t before_first = i0 > 0 && i0 - 1 < n ? key[i0 - 1] : 0;
+  static_for<kLevelItems>([&](auto J) {   // compile-time indices keep k[] and a[] in registers
+    constexpr int j = decltype(J)::value;
+    k[j] = i0 + j < n ? key[i0 + j] : 0;
+  });
+  Packed4 mine = {0, 0, 0, 0};
+  static_for<kLevelItems>([&](auto J) {
+    constexpr int j = decltype(J)::value;
+    const int i = i0 + j;
+    a[j] = 64;  // heads nothing (also: beyond the end)
+    if (i < n) {
+      if (i == 0) a[j] = 0;
+      else {
+        uint64_t prev = before_first;
+        if constexpr (j > 0) prev = k[j - 1];
+        const uint64_t x = k[j] ^ prev;
+        if (x != 0) {
+          const int t = (63 - __clzll((long long)x)) / 3;   // differs at level depth - t
+          a[j] = max(0, depth - t - full_layer);
+        }
+      }
+      if (a[j] < L) add_to(mine, heads_from(a[j]));
+    }
+  });
+  Packed4 total;
+  const Packed4 run = block_exclusive_scan_p4(mine, &total);  // heads of this tile before this thread
+  if (tid < 16) {
+    tile_publish(status, 16, tid, tile, field_of(total, tid));
+    s_before[tid] = tile_prefix(status, group_status, 16, tid, tile, field_of(total, tid), spin_limit, &ctl->error);
+  }
+  __syncthreads();
+  // level by level (uniform over the workgroup, so the output pointers are scalars): b_* =
+  // heads before this thread at level f / f+1, c_* = the same among its own elements
+  const bool has_last = i0 <= n - 1 && n - 1 < i0 + kLevelItems;
+  for (int f = 0; f < L; ++f) {
+    const int d = full_layer + f;
+    const int shift = 3 * (depth - d);
+    const int b0 = s_before[f] + field_of(run, f);
+    const int b1 = f + 1 < L ? s_before[f + 1] + field_of(run, f + 1) : 0;
+    uint64_t* __restrict__ list = out.list[d];
+    int* __restrict__ first = out.first[d];
+    int c0 = 0, c1 = 0;
+    static_for<kLevelItems>([&](auto J) {   // compile-time indices keep k[] and a[] in registers
+      constexpr int j = decltype(J)::value;
+      c1 += a[j] <= f + 1 ? 1 : 0;
+      if (a[j] <= f) {
+        const int r = b0 + c0;
+        ++c0;
+        list[r] = k[j] >> shift;
+        if (f + 1 < L) first[r] = b1 + c1 - 1;
+        else out.ustart[r] = i0 + j;
+      }
+    });
+    if (has_last) {
+      ctl->nne[d] = b0 + c0;
+      if (f + 1 < L) first[b0 + c0] = b1 + c1;
+      else out.ustart[b0 + c0] = n;
+    }
+  }
+}
+
+// ---- 4. emit -------------------------------------------------------------------------------
 __device__ inline uint64_t out_key(uint64_t morton, int d, int cloud, int key2xyz) {
   // raw Morton key, or packed (x, y, z) 16-bit fields (Octree::key_to_xyz, octree.cpp:1137-1156);
   // the cloud index goes to the top 16 bits as merge_octrees does (merge_octrees.cpp:126-131)
   uint64_t k = morton;
   if (key2xyz) {
     uint64_t m = d >= 16 ? 0xffffull : ((1ull << d) - 1);
-    k = (b_compact3(morton >> 2) & m) | ((b_compact3(morton >> 1) & m) << 16) | ((b_compact3(morton) & m) << 32);
+    k = (compact3(morton >> 2) & m) | ((compact3(morton >> 1) & m) << 16) | ((compact3(morton) & m) << 32);
   }
   return (k & 0x0000ffffffffffffull) | ((uint64_t)(cloud & 0xffff) << 48);
 }
 
-// full layers: node t = cloud * 8^d + i, key i, child t (or -1 on the last full layer)
-__global__ void emit_full_kernel(uint64_t* __restrict__ key, int* __restrict__ child, int d, int64_t total,
-    EmitGeom g) {
-  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= total) return;
-  int64_t per = (int64_t)1 << (3 * d);
-  int cloud = (int)(t / per);
-  uint64_t i = (uint64_t)(t % per);
-  key[t] = out_key(i, d, cloud, g.key2xyz);
-  child[t] = d < g.full_layer ? (int)t : -1;
-}
-// sparse layers: node t = 8 * parent_rank + octant; key from the parent's key
-__global__ void emit_sparse_kernel(uint64_t* __restrict__ key, int* __restrict__ child, int d, int64_t total,
-    const uint64_t* __restrict__ parent_list, EmitGeom g) {
-  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= total) return;
-  uint64_t pk = parent_list[t >> 3];               // cloud << 3(d-1) | morton_{d-1}
-  int cloud = (int)(pk >> (3 * (d - 1)));
-  uint64_t pm = pk & ((1ull << (3 * (d - 1))) - 1);
-  key[t] = out_key((pm << 3) | (uint64_t)(t & 7), d, cloud, g.key2xyz);
-  child[t] = -1;
-}
-// child links: the j-th non-empty node of depth d points to rank j
-__global__ void emit_links_kernel(int* __restrict__ child, int d, int nne, const uint64_t* __restrict__ list,
-    const int* __restrict__ prank, int* __restrict__ leaf_node, EmitGeom g) {
-  int j = blockIdx.x * blockDim.x + threadIdx.x;
-  if (j >= nne) return;
-  uint64_t k = list[j];
-  int64_t node;
-  if (d == g.full_layer) {
-    int cloud = (int)(k >> (3 * d));
-    node = ((int64_t)cloud << (3 * d)) + (int64_t)(k & ((1ull << (3 * d)) - 1));
-  } else {
-    node = ((int64_t)prank[j] << 3) + (int64_t)(k & 7);
-  }
-  child[node] = j;
-  if (leaf_node) leaf_node[j] = (int)node;
-}
-
-struct HeaderArg { uint32_t w[OCNN_HEADER_BYTES / 4]; };
-__global__ void write_header_kernel(uint32_t* __restrict__ dst, HeaderArg h) {
-  int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < OCNN_HEADER_BYTES / 4) dst[i] = h.w[i];
-}
-
-__global__ void fill_f32_kernel(float* p, int64_t n, float v) {
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  int64_t step = (int64_t)gridDim.x * blockDim.x;
-  for (; i < n; i += step) p[i] = v;
-}
-__global__ void split_kernel(float* __restrict__ split, const int* __restrict__ child, int64_t n) {
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) split[i] = child[i] < 0 ? 0.0f : 1.0f;  // calc_split_label, octree.cpp:1158-1178
-}
-
-// ---- 5. emit: leaf signal -----------------------------------------------------------------
 struct SignalGeom {
-  int depth, n_clouds, nnum_d;      // nnum_d = node count of the finest level (row length)
-  int ch_normal, ch_feature, has_label, has_dis, save_pts;
+  int depth, nnum_d;      // nnum_d = node count of the finest level (row length)
+  int ch_feature, channels, has_label, has_dis, save_pts;
   float bbmin[3], mul;
 };
 
-// One thread per non-empty leaf; its points are visited in ascending original index
-// (the sort is stable), so every sum is taken in the reference's order
-// (octree.cpp:312-452).  All float operations are individually rounded.
-__global__ void leaf_signal_kernel(float* __restrict__ feature, float* __restrict__ label_out, int n_leaf,
-    const uint64_t* __restrict__ ukey, const int* __restrict__ ustart, const uint32_t* __restrict__ sorted_idx,
-    const int* __restrict__ leaf_node, const CloudDesc* __restrict__ clouds, SignalGeom g) {
-  int j = blockIdx.x * blockDim.x + threadIdx.x;
-  if (j >= n_leaf) return;
-  const int cloud = (int)(ukey[j] >> (3 * g.depth));
+// Signal of one non-empty leaf: its points are visited in ascending original index (the
+// sort is stable), so every sum is taken in the reference's order (octree.cpp:312-452).
+// All float operations are individually rounded.
+__device__ inline void leaf_signal(float* __restrict__ feature, float* __restrict__ label_out, int node,
+    int cloud, int s0, int s1, const uint32_t* __restrict__ sorted_idx, const CloudDesc* __restrict__ clouds,
+    const SignalGeom& g) {
   const CloudDesc cd = clouds[cloud];
-  const int s0 = ustart[j], s1 = ustart[j + 1];
-  const int node = leaf_node[j];
   const int64_t H = g.nnum_d;
   float* out = feature + node;  // channel c lives at out[c * H]
+  // one pass over the points: every attribute of a point is requested together
+  constexpr int kRegFeatures = 8;
+  const int F = cd.feature ? g.ch_feature : 0;
+  const bool need_pt = g.has_dis || g.save_pts;
+  float acc[3] = {0.0f, 0.0f, 0.0f}, avg_pt[3] = {0.0f, 0.0f, 0.0f}, facc[kRegFeatures];
+#pragma unroll
+  for (int c = 0; c < kRegFeatures; ++c) facc[c] = 0.0f;
+  for (int i = s0; i < s1; ++i) {
+    const int64_t idx = (int64_t)(sorted_idx[i] - cd.offset);
+    if (cd.normal) {
+      const float* q = cd.normal + 3 * idx;
+      for (int c = 0; c < 3; ++c) acc[c] = __fadd_rn(acc[c], q[c]);
+    }
+    if (need_pt) {
+      const float* q = cd.xyz + 3 * idx;
+      for (int c = 0; c < 3; ++c) avg_pt[c] = __fadd_rn(avg_pt[c], scale_coord(q[c], g.bbmin[c], g.mul));
+    }
+    const float* q = cd.feature + F * idx;
+#pragma unroll
+    for (int c = 0; c < kRegFeatures; ++c)
+      if (c < F) facc[c] = __fadd_rn(facc[c], q[c]);
+  }
   int ch = 0;
   float nrm[3] = {0.0f, 0.0f, 0.0f};
   if (cd.normal) {
-    float acc[3] = {0.0f, 0.0f, 0.0f};
-    for (int i = s0; i < s1; ++i) {
-      const float* q = cd.normal + 3 * (int64_t)(sorted_idx[i] - cd.offset);
-      for (int c = 0; c < 3; ++c) acc[c] = __fadd_rn(acc[c], q[c]);
-    }
     float len = 0.0f;
     for (int c = 0; c < 3; ++c) len = __fadd_rn(len, __fmul_rn(acc[c], acc[c]));
     float factor = sqrt_rn(len);
@@ -342,12 +569,7 @@ __global__ void leaf_signal_kernel(float* __restrict__ feature, float* __restric
     ch += 3;
   }
   const float count = __fadd_rn((float)(s1 - s0), 1.0e-30f);
-  float avg_pt[3] = {0.0f, 0.0f, 0.0f};
-  if (g.has_dis || g.save_pts) {
-    for (int i = s0; i < s1; ++i) {
-      const float* q = cd.xyz + 3 * (int64_t)(sorted_idx[i] - cd.offset);
-      for (int c = 0; c < 3; ++c) avg_pt[c] = __fadd_rn(avg_pt[c], scale_coord(q[c], g.bbmin[c], g.mul));
-    }
+  if (need_pt) {
     float dis[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     for (int c = 0; c < 3; ++c) {
       avg_pt[c] = div_rn(avg_pt[c], count);
@@ -366,14 +588,17 @@ __global__ void leaf_signal_kernel(float* __restrict__ feature, float* __restric
       }
     }
   }
-  if (cd.feature) {
-    for (int c = 0; c < g.ch_feature; ++c) {
-      float acc = 0.0f;
+  if (F > 0) {
+#pragma unroll
+    for (int c = 0; c < kRegFeatures; ++c)
+      if (c < F) out[(ch + c) * H] = div_rn(facc[c], count);
+    for (int c = kRegFeatures; c < F; ++c) {   // channels beyond the register budget: one more pass each
+      float sum = 0.0f;
       for (int i = s0; i < s1; ++i)
-        acc = __fadd_rn(acc, cd.feature[(int64_t)g.ch_feature * (sorted_idx[i] - cd.offset) + c]);
-      out[(ch + c) * H] = div_rn(acc, count);
+        sum = __fadd_rn(sum, cd.feature[(int64_t)F * (sorted_idx[i] - cd.offset) + c]);
+      out[(ch + c) * H] = div_rn(sum, count);
     }
-    ch += g.ch_feature;
+    ch += F;
   }
   if (g.save_pts) {
     for (int c = 0; c < 3; ++c) out[(ch + c) * H] = avg_pt[c];
@@ -399,98 +624,243 @@ __global__ void leaf_signal_kernel(float* __restrict__ feature, float* __restric
   }
 }
 
-// ---- neighbour kernels (same arithmetic as octree_index.hip; private copies keep this
-// translation unit self-contained) ----------------------------------------------------------
-// Sparse-layer neighbour table.  A workgroup takes 256 consecutive parent-level nodes,
-// compacts the non-empty ones into LDS (most nodes of a deep level are empty) and then
-// every wavefront writes the 64-slot blocks of the compacted nodes, four nodes per
-// iteration so that four dependent load chains (neigh -> children) are in flight.
-__global__ void b_neigh_sparse_kernel(int* __restrict__ neigh_child, const int* __restrict__ neigh,
-    const int* __restrict__ children, int node_num) {
-  __shared__ int s_node[kBlock], s_rank[kBlock], s_count;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int i = blockIdx.x * kBlock + threadIdx.x;
-  const int l0 = i < node_num ? children[i] : -1;
-  int total;
-  const int pos = block_exclusive_scan(l0 >= 0 ? 1 : 0, &total);
-  if (l0 >= 0) { s_node[pos] = i; s_rank[pos] = l0; }
-  if (threadIdx.x == 0) s_count = total;
-  __syncthreads();
-  const int count = s_count;
-  const int x = lane >> 4, y = (lane >> 2) & 3, z = lane & 3;
-  const int hx = (x + 1) >> 1, hy = (y + 1) >> 1, hz = (z + 1) >> 1;
-  const int octant = (((x + 1) & 1) << 2) | (((y + 1) & 1) << 1) | ((z + 1) & 1);
-  for (int e = wave * 4; e < count; e += 4 * (kBlock / 64)) {
-    int t[4], rank[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      t[u] = -1;
-      rank[u] = -1;
-      if (e + u < count) {
-        const int node = s_node[e + u];
-        rank[u] = s_rank[e + u];
-        const int sib = node & 7;
-        const int slot = ((hx + (sib >> 2)) << 4) | ((hy + ((sib >> 1) & 1)) << 2) | (hz + (sib & 1));
-        t[u] = neigh[((int64_t)(node >> 3) << 6) + slot];
+// The emit launch is cut into segments of whole workgroups; each segment is one kind of
+// work on one level.
+enum SegKind { kSegHeader = 0, kSegFull = 1, kSegFullNeigh = 2, kSegSparse = 3 };
+constexpr int kMaxSeg = 56;
+struct HeaderArg { uint32_t w[OCNN_HEADER_BYTES / 4]; };
+
+struct EmitArgs {
+  HeaderArg hdr;
+  int depth, full_layer, n_clouds, key2xyz, key_channel;
+  int n_seg;
+  int seg_begin[kMaxSeg + 1];          // first workgroup of each segment
+  unsigned char seg_kind[kMaxSeg], seg_level[kMaxSeg];
+  int nnum[kMaxLevels], nne[kMaxLevels];
+  int64_t off_key[kMaxLevels], off_child[kMaxLevels], off_split[kMaxLevels], off_neigh[kMaxLevels];
+  int64_t off_feature, off_label;      // of the finest level; -1: absent
+  const uint64_t* list[kMaxLevels];
+  const int* first[kMaxLevels];
+  const int* ustart;
+  const uint32_t* sorted_idx;
+  const CloudDesc* clouds;
+  SignalGeom sg;
+};
+static_assert(sizeof(EmitArgs) <= 3800, "kernel arguments must stay below 4 KiB");
+
+__global__ __launch_bounds__(kBlock) void emit_kernel(char* __restrict__ blob, const EmitArgs a) {
+  __shared__ uint64_t s_key[kBlock * 8];
+  __shared__ int s_child[kBlock * 8];
+  int seg = 0;
+  while (seg + 1 < a.n_seg && (int)blockIdx.x >= a.seg_begin[seg + 1]) ++seg;
+  const int kind = a.seg_kind[seg], d = a.seg_level[seg];
+  const int block = blockIdx.x - a.seg_begin[seg];
+  const int tid = threadIdx.x;
+
+  if (kind == kSegHeader) {
+    // header (the tail of the 720-byte block is padding, zero); depth 0 holds no neighbour table
+    uint32_t* dst = reinterpret_cast<uint32_t*>(blob);
+    for (int i = tid; i < OCNN_HEADER_BYTES / 4; i += kBlock) dst[i] = a.hdr.w[i];
+    if (a.off_neigh[0] >= 0) {
+      int* n0 = reinterpret_cast<int*>(blob + a.off_neigh[0]);
+      for (int i = tid; i < a.nnum[0] * 8; i += kBlock) n0[i] = 0;
+    }
+    return;
+  }
+  if (kind == kSegFullNeigh) {  // closed form (octree_nn.cpp:382-424)
+    const int64_t id = (int64_t)block * kBlock + tid;
+    const int64_t node_num = (int64_t)1 << (3 * d);
+    if (id >= ((int64_t)a.n_clouds * node_num) << 3) return;
+    const int64_t groups = node_num >> 3;
+    const int slot = (int)(id & 63);
+    const int64_t g = id >> 6;
+    const int64_t cloud = g / groups;
+    uint32_t x0, y0, z0;
+    morton_decode((uint64_t)(g % groups) << 3, d, &x0, &y0, &z0);
+    const uint32_t x1 = x0 + (slot >> 4) - 1, y1 = y0 + ((slot >> 2) & 3) - 1, z1 = z0 + (slot & 3) - 1;
+    int v = -1;
+    if (((x1 | y1 | z1) & (1u << d)) == 0) v = (int)(morton_encode(x1, y1, z1, d) + (uint64_t)cloud * node_num);
+    reinterpret_cast<int*>(blob + a.off_neigh[d])[id] = v;
+    return;
+  }
+  uint64_t* key = reinterpret_cast<uint64_t*>(blob + a.off_key[d]);
+  int* child = reinterpret_cast<int*>(blob + a.off_child[d]);
+  float* split = a.off_split[d] >= 0 ? reinterpret_cast<float*>(blob + a.off_split[d]) : nullptr;
+  const int n_d = a.nnum[d];
+  if (kind == kSegFull) {
+    // full layers: node t = cloud * 8^d + i, key i; child t, or on the last full layer the
+    // rank among the non-empty nodes
+    const int64_t t = (int64_t)block * kBlock + tid;
+    if (t >= n_d) return;
+    const int64_t per = (int64_t)1 << (3 * d);
+    const int cloud = (int)(t / per);
+    const uint64_t i = (uint64_t)(t % per);
+    key[t] = out_key(i, d, cloud, a.key2xyz);
+    if (a.key_channel == 2) key[n_d + t] = 0;
+    int c = (int)t;
+    if (d == a.full_layer) {
+      c = -1;
+      if (a.depth > a.full_layer) {
+        const uint64_t want = ((uint64_t)cloud << (3 * d)) | i;
+        const uint64_t* __restrict__ list = a.list[d];
+        int lo = 0, hi = a.nne[d];
+        while (lo < hi) {
+          const int mid = (lo + hi) >> 1;
+          if (list[mid] < want) lo = mid + 1; else hi = mid;
+        }
+        if (lo < a.nne[d] && list[lo] == want) c = lo;
       }
     }
+    child[t] = c;
+    if (split) split[t] = c < 0 ? 0.0f : 1.0f;  // calc_split_label, octree.cpp:1158-1178
+    return;
+  }
+  // sparse layers: thread = sibling group p (the children of the p-th non-empty node of level
+  // d-1): node 8p + octant, key from the parent's key; the non-empty ones are consecutive in
+  // list[d] from first[d-1][p]
+  const int groups = a.nne[d - 1];
+  const int p = block * kBlock + tid;
+  if (p < groups) {
+    const uint64_t pk = a.list[d - 1][p];     // cloud << 3(d-1) | morton_{d-1}
+    const int cloud = (int)(pk >> (3 * (d - 1)));
+    const uint64_t pm = pk & ((1ull << (3 * (d - 1))) - 1);
+    const int c0 = a.first[d - 1][p], c1 = a.first[d - 1][p + 1];
+    int oct[8];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      int v = -1;
-      if (t[u] >= 0) {
-        const int l1 = children[t[u]];
-        if (l1 >= 0) v = (l1 << 3) + octant;
-      }
-      if (rank[u] >= 0) neigh_child[((int64_t)rank[u] << 6) + lane] = v;
+    for (int u = 0; u < 8; ++u) oct[u] = c0 + u < c1 ? (int)(a.list[d][c0 + u] & 7) : 8;
+#pragma unroll
+    for (int o = 0; o < 8; ++o) {
+      int c = -1;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) c = oct[u] == o ? c0 + u : c;
+      s_child[tid * 8 + o] = c;
+      s_key[tid * 8 + o] = out_key((pm << 3) | (uint64_t)o, d, cloud, a.key2xyz);
     }
   }
+  __syncthreads();
+  const int64_t node0 = (int64_t)block * kBlock * 8;
+  const int rows = min(kBlock * 8, n_d - (int)node0);  // nodes of this workgroup
+  for (int r = tid; r < rows; r += kBlock) {
+    key[node0 + r] = s_key[r];
+    if (a.key_channel == 2) key[n_d + node0 + r] = 0;
+    const int c = s_child[r];
+    child[node0 + r] = c;
+    if (split) split[node0 + r] = c < 0 ? 0.0f : 1.0f;
+  }
 }
-__global__ void b_neigh_full_kernel(int* __restrict__ neigh, int depth, int64_t total) {
-  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (id >= total) return;
-  const int64_t node_num = (int64_t)1 << (3 * depth);
-  const int64_t groups = node_num >> 3;
-  int slot = (int)(id & 63);
-  int64_t grp = id >> 6;
-  int64_t n = grp / groups;
-  uint64_t i = (uint64_t)(grp % groups) << 3;
-  uint64_t m = (1ull << depth) - 1;
-  uint32_t x0 = (uint32_t)(b_compact3(i >> 2) & m), y0 = (uint32_t)(b_compact3(i >> 1) & m),
-           z0 = (uint32_t)(b_compact3(i) & m);
-  uint32_t x1 = x0 + (slot >> 4) - 1, y1 = y0 + ((slot >> 2) & 3) - 1, z1 = z0 + (slot & 3) - 1;
-  const uint32_t bound = 1u << depth;
-  int v = -1;
-  if (((x1 | y1 | z1) & bound) == 0)
-    v = (int)(((b_spread3(x1 & m) << 2) | (b_spread3(y1 & m) << 1) | b_spread3(z1 & m)) + (uint64_t)n * node_num);
-  neigh[id] = v;
+
+// Signal of the finest level, one thread per node: empty nodes get zeros (label -1), so every
+// row of the feature block is written exactly once, in full wavefront-wide rows.
+__global__ __launch_bounds__(kBlock) void leaf_signal_kernel(float* __restrict__ feature,
+    float* __restrict__ label, const int* __restrict__ child, const uint64_t* __restrict__ leaf_key,
+    const int* __restrict__ ustart, const uint32_t* __restrict__ sorted_idx, const CloudDesc* __restrict__ clouds,
+    SignalGeom g) {
+  const int node = blockIdx.x * blockDim.x + threadIdx.x;
+  if (node >= g.nnum_d) return;
+  const int j = child[node];
+  if (label) label[node] = -1.0f;
+  if (j < 0) {
+    for (int c = 0; c < g.channels; ++c) feature[(int64_t)c * g.nnum_d + node] = 0.0f;
+    return;
+  }
+  leaf_signal(feature, label, node, (int)(leaf_key[j] >> (3 * g.depth)), ustart[j], ustart[j + 1], sorted_idx,
+      clouds, g);
+}
+
+// The same through LDS: a workgroup takes kSignalTile consecutive nodes.  Their non-empty
+// ones are consecutive leaves (ranks grow with the node index), so threads 0 .. count-1 take
+// one leaf each -- dense wavefronts for the point gathers, where the kernel above keeps one
+// lane in seven busy at depth 9 -- and put the result into an LDS image of the tile's rows,
+// which is then written out in full rows.  Needs channels <= kSignalStage.
+constexpr int kSignalTile = 1024, kSignalStage = 8;
+__global__ __launch_bounds__(kBlock) void leaf_signal_staged_kernel(float* __restrict__ feature,
+    float* __restrict__ label, const int* __restrict__ child, const uint64_t* __restrict__ leaf_key,
+    const int* __restrict__ ustart, const uint32_t* __restrict__ sorted_idx, const CloudDesc* __restrict__ clouds,
+    SignalGeom g) {
+  extern __shared__ float s_dyn[];           // [channels][kSignalTile] rows, then labels
+  __shared__ unsigned short s_node[kSignalTile];
+  __shared__ int s_first, s_last;
+  float* s_out = s_dyn;
+  float* s_label = s_dyn + (size_t)g.channels * kSignalTile;
+  const int tid = threadIdx.x;
+  const int node0 = blockIdx.x * kSignalTile;
+  const int rows = min(kSignalTile, g.nnum_d - node0);
+  if (tid == 0) { s_first = 0x7fffffff; s_last = -1; }
+  int c[kSignalTile / kBlock];
+#pragma unroll
+  for (int q = 0; q < kSignalTile / kBlock; ++q) {
+    const int r = q * kBlock + tid;
+    c[q] = r < rows ? child[node0 + r] : -1;
+  }
+  for (int i = tid; i < g.channels * kSignalTile; i += kBlock) s_out[i] = 0.0f;
+  if (label)
+    for (int i = tid; i < kSignalTile; i += kBlock) s_label[i] = -1.0f;
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < kSignalTile / kBlock; ++q)
+    if (c[q] >= 0) { atomicMin(&s_first, c[q]); atomicMax(&s_last, c[q]); }
+  __syncthreads();
+  const int j0 = s_first, count = s_last - s_first + 1;   // count <= 0: no leaf here
+#pragma unroll
+  for (int q = 0; q < kSignalTile / kBlock; ++q)
+    if (c[q] >= 0) s_node[c[q] - j0] = (unsigned short)(q * kBlock + tid);
+  __syncthreads();
+  SignalGeom lg = g;
+  lg.nnum_d = kSignalTile;   // row length of the LDS image
+  for (int t = tid; t < count; t += kBlock) {
+    const int j = j0 + t;
+    leaf_signal(s_out, label ? s_label : nullptr, (int)s_node[t], (int)(leaf_key[j] >> (3 * g.depth)), ustart[j],
+        ustart[j + 1], sorted_idx, clouds, lg);
+  }
+  __syncthreads();
+  for (int ch = 0; ch < g.channels; ++ch)
+    for (int r = tid; r < rows; r += kBlock) feature[(int64_t)ch * g.nnum_d + node0 + r] = s_out[ch * kSignalTile + r];
+  if (label)
+    for (int r = tid; r < rows; r += kBlock) label[node0 + r] = s_label[r];
+}
+
+__global__ void fill_f32_kernel(float* p, int64_t n, float v) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t step = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += step) p[i] = v;
 }
 
 // ---- host side -------------------------------------------------------------------------------
 inline size_t al(size_t v) { return (v + 255) & ~(size_t)255; }
+inline int sort_items(int64_t n) { return n <= (1 << 19) ? 4 : 8; }
+// status rows (one per tile / per group of tiles) of a pass
+inline size_t status_words(int tiles) { return (size_t)tiles; }
+inline size_t group_words(int tiles) { return (size_t)(tiles / kGroupTiles + 1); }
 
 struct Layout {          // byte offsets inside the workspace
-  size_t clouds, counts, key[2], val[2], hist, scan, ustart, leaf_node;
-  size_t list[kMaxLevels], prank[kMaxLevels];
+  size_t clouds, control, hist, sort_status, sort_groups, level_status, level_groups, zero_end;
+  size_t key[2], val[2], ustart;
+  size_t list[kMaxLevels], first[kMaxLevels];
   size_t total;
-  int hist_blocks;
+  int sort_tiles, level_tiles;
 };
 
 Layout make_layout(int64_t N, int B, int depth) {
   Layout L;
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off += al(bytes); return o; };
-  L.clouds = take(sizeof(CloudDesc) * (size_t)(B > 0 ? B : 1));
-  L.counts = take(sizeof(Counts));
   size_t n = (size_t)(N > 0 ? N : 1);
+  L.clouds = take(sizeof(CloudDesc) * (size_t)(B > 0 ? B : 1));
+  L.sort_tiles = (int)((n + kBlock * sort_items(N) - 1) / (kBlock * sort_items(N)));
+  L.level_tiles = (int)((n + kLevelTile - 1) / kLevelTile);
+  // one zeroed region: control words, histograms, look-back status of every pass
+  L.control = take(sizeof(Control));
+  L.hist = take(sizeof(int) * 256 * kMaxPasses * kHistCopies);
+  L.sort_status = take(sizeof(uint32_t) * 256 * status_words(L.sort_tiles) * kMaxPasses);
+  L.sort_groups = take(sizeof(uint32_t) * 256 * group_words(L.sort_tiles) * kMaxPasses);
+  L.level_status = take(sizeof(uint32_t) * 16 * status_words(L.level_tiles));
+  L.level_groups = take(sizeof(uint32_t) * 16 * group_words(L.level_tiles));
+  L.zero_end = off;
   for (int i = 0; i < 2; ++i) { L.key[i] = take(8 * n); L.val[i] = take(4 * n); }
-  L.hist_blocks = (int)((n + kSortTile - 1) / kSortTile);
-  L.hist = take(sizeof(int) * 256 * ((size_t)L.hist_blocks + 1));  // + 256 digit totals
-  L.scan = take(scan_scratch_bytes((int64_t)n));
   L.ustart = take(4 * (n + 1));
-  L.leaf_node = take(4 * n);
   for (int d = 0; d < kMaxLevels; ++d) {
-    if (d <= depth) { L.list[d] = take(8 * n); L.prank[d] = take(4 * n); }
-    else { L.list[d] = L.prank[d] = 0; }
+    if (d <= depth) { L.list[d] = take(8 * n); L.first[d] = take(4 * (n + 1)); }
+    else { L.list[d] = L.first[d] = 0; }
   }
   L.total = off;
   return L;
@@ -508,6 +878,29 @@ struct PlanState {
 };
 std::mutex g_plans_mutex;
 std::map<void*, PlanState> g_plans;
+
+// bounded waits of the look-back (polls of one status window, each followed by a short sleep)
+constexpr int kFirstWaitLimit = 1 << 16, kTicketWaitLimit = 1 << 22;
+std::atomic<int> g_first_wait_limit{kFirstWaitLimit};
+std::atomic<int> g_ticket_reruns{0};
+
+// Pinned host slots for the one device-to-host copy of a plan (a pageable destination
+// would be staged and cost a second wait).
+std::mutex g_slots_mutex;
+std::vector<Control*> g_free_slots;
+Control* take_slot() {
+  {
+    std::lock_guard<std::mutex> lock(g_slots_mutex);
+    if (!g_free_slots.empty()) { Control* s = g_free_slots.back(); g_free_slots.pop_back(); return s; }
+  }
+  void* p = nullptr;
+  if (hipHostMalloc(&p, sizeof(Control), hipHostMallocDefault) != hipSuccess) return nullptr;
+  return static_cast<Control*>(p);
+}
+void give_slot(Control* s) {
+  std::lock_guard<std::mutex> lock(g_slots_mutex);
+  g_free_slots.push_back(s);
+}
 
 }  // namespace
 }  // namespace ocnn
@@ -553,7 +946,7 @@ int ocnn_points2octree_plan(const void* const* points_dev, const void* const* po
     c.offset = (int)N;
     c.count = pi->pt_num;
     N += pi->pt_num;
-    OCNN_REQUIRE(N < (1ll << 31), OCNN_E_BADARG, "more than 2^31 points");
+    OCNN_REQUIRE(N < (1ll << 30), OCNN_E_BADARG, "more than 2^30 points");
   }
   const int ch_normal = (p0->content_flags & 2) ? p0->channels[1] : 0;
   const int ch_feature = (p0->content_flags & 4) ? p0->channels[2] : 0;
@@ -598,15 +991,11 @@ int ocnn_points2octree_plan(const void* const* points_dev, const void* const* po
   OCNN_REQUIRE((reinterpret_cast<uintptr_t>(workspace_dev) & 255) == 0, OCNN_E_WORKSPACE, "workspace not 256-byte aligned");
   char* ws = static_cast<char*>(workspace_dev);
   CloudDesc* d_clouds = reinterpret_cast<CloudDesc*>(ws + L.clouds);
-  Counts* d_counts = reinterpret_cast<Counts*>(ws + L.counts);
+  Control* d_ctl = reinterpret_cast<Control*>(ws + L.control);
   uint64_t* d_key[2] = {reinterpret_cast<uint64_t*>(ws + L.key[0]), reinterpret_cast<uint64_t*>(ws + L.key[1])};
   uint32_t* d_val[2] = {reinterpret_cast<uint32_t*>(ws + L.val[0]), reinterpret_cast<uint32_t*>(ws + L.val[1])};
   int* d_hist = reinterpret_cast<int*>(ws + L.hist);
-  int* d_digit_total = d_hist + (int64_t)256 * L.hist_blocks;
-  int* d_scan = reinterpret_cast<int*>(ws + L.scan);
-  int* d_ustart = reinterpret_cast<int*>(ws + L.ustart);
-
-  OCNN_HIP_OK(hipMemcpyAsync(d_clouds, clouds.data(), sizeof(CloudDesc) * n_clouds, hipMemcpyHostToDevice, s));
+  uint32_t* d_sort_status = reinterpret_cast<uint32_t*>(ws + L.sort_status);
 
   BuildGeom g;
   g.depth = depth;
@@ -615,46 +1004,89 @@ int ocnn_points2octree_plan(const void* const* points_dev, const void* const* po
   g.n_points = N;
   for (int i = 0; i < 3; ++i) g.bbmin[i] = o.bbmin[i];
   g.mul = float(1 << depth) / o.bbox_max_width();  // octree.cpp:159
+  int cloud_bits = 0;
+  while ((1 << cloud_bits) < n_clouds) ++cloud_bits;
+  const int nbits = 3 * depth + cloud_bits;
+  g.passes = (nbits + 7) / 8;
+  g.bits = (nbits + g.passes - 1) / g.passes;
+
+  // control words + the cloud table (passed as kernel arguments, 48 clouds a launch: no
+  // staged host-to-device copy)
+  auto init = [&]() -> int {
+    const int64_t zero_words = depth > fl ? (int64_t)((L.zero_end - L.control) / 4) : (int64_t)(sizeof(Control) / 4);
+    for (int first = 0; first < n_clouds; first += kArgClouds) {
+      CloudChunk chunk;
+      memset(&chunk, 0, sizeof(chunk));
+      const int count = n_clouds - first < kArgClouds ? n_clouds - first : kArgClouds;
+      memcpy(chunk.c, clouds.data() + first, sizeof(CloudDesc) * count);
+      const int64_t zw = first == 0 ? zero_words : 0;
+      int64_t blocks = (zw + kBlock * 4 - 1) / (kBlock * 4);
+      if (blocks < 1) blocks = 1;
+      if (blocks > 1024) blocks = 1024;
+      init_kernel<<<(unsigned)blocks, kBlock, 0, s>>>(reinterpret_cast<uint32_t*>(ws + L.control), zw, d_clouds,
+          chunk, first, count);
+    }
+    OCNN_LAUNCH_OK("init");
+    return OCNN_OK;
+  };
 
   PlanState st;
   memset(&st, 0, sizeof(st));
   int cur = 0;
-  if (depth > fl) {
-    keygen_kernel<<<blocks_for(N), kBlock, 0, s>>>(d_key[0], d_val[0], d_clouds, g);
+  // keys, sort, level scan, counts to the host; *wait_error: a bounded wait ran out
+  auto sort_and_scan = [&](bool tickets, int spin_limit, int* wait_error) -> int {
+    cur = 0;
+    keygen_kernel<<<min(blocks_for(N, kBlock * kKeyItems), (unsigned)kKeyGrid), kBlock, 0, s>>>(d_key[0], d_val[0],
+        d_clouds, d_hist, g);
     OCNN_LAUNCH_OK("keygen");
-    int cloud_bits = 0;
-    while ((1 << cloud_bits) < n_clouds) ++cloud_bits;
-    int nbits = 3 * depth + cloud_bits;
-    for (int shift = 0; shift < nbits; shift += 8) {
-      radix_hist_kernel<<<L.hist_blocks, kBlock, 0, s>>>(d_key[cur], N, shift, d_hist, L.hist_blocks);
-      radix_scan_kernel<<<256, kBlock, 0, s>>>(d_hist, L.hist_blocks, d_digit_total);
-      radix_scatter_kernel<<<L.hist_blocks, kBlock, 0, s>>>(d_key[cur], d_val[cur], d_key[cur ^ 1], d_val[cur ^ 1],
-          N, shift, d_hist, L.hist_blocks, d_digit_total);
-      OCNN_LAUNCH_OK("radix pass");
+    for (int p = 0; p < g.passes; ++p) {
+      uint32_t* status = d_sort_status + (size_t)p * 256 * status_words(L.sort_tiles);
+      uint32_t* groups = reinterpret_cast<uint32_t*>(ws + L.sort_groups) + (size_t)p * 256 * group_words(L.sort_tiles);
+      auto launch = [&](auto kernel) {
+        kernel<<<L.sort_tiles, kBlock, 0, s>>>(d_key[cur], d_val[cur], d_key[cur ^ 1], d_val[cur ^ 1], (int)N,
+            p * g.bits, g.bits, d_hist + p * 256, status, groups, d_ctl, p, spin_limit);
+      };
+      if (sort_items(N) == 4) { if (tickets) launch(sort_pass_kernel<4, true>); else launch(sort_pass_kernel<4, false>); }
+      else { if (tickets) launch(sort_pass_kernel<8, true>); else launch(sort_pass_kernel<8, false>); }
+      OCNN_LAUNCH_OK("sort pass");
       cur ^= 1;
     }
-    // unique leaves
-    uint64_t* list_D = reinterpret_cast<uint64_t*>(ws + L.list[depth]);
-    LeafPred lp{d_key[cur], N};
-    LeafOut lo{d_key[cur], list_D, d_ustart, N};
-    hipError_t e = flag_scan(lp, lo, N, d_scan, &d_counts->nne[depth], s);
-    OCNN_REQUIRE(e == hipSuccess, OCNN_E_HIP, "leaf scan: %s", hipGetErrorString(e));
-    // parents, level by level (sizes stay on the device: grids cover the upper bound N)
-    for (int d = depth; d > fl; --d) {
-      const uint64_t* list = reinterpret_cast<const uint64_t*>(ws + L.list[d]);
-      uint64_t* plist = reinterpret_cast<uint64_t*>(ws + L.list[d - 1]);
-      int* prank = reinterpret_cast<int*>(ws + L.prank[d]);
-      ParentPred pp{list, &d_counts->nne[d]};
-      ParentOut po{list, &d_counts->nne[d], plist, prank};
-      e = flag_scan(pp, po, N, d_scan, &d_counts->nne[d - 1], s);
-      OCNN_REQUIRE(e == hipSuccess, OCNN_E_HIP, "parent scan: %s", hipGetErrorString(e));
+    LevelOut lo;
+    memset(&lo, 0, sizeof(lo));
+    for (int d = fl; d <= depth; ++d) {
+      lo.list[d] = reinterpret_cast<uint64_t*>(ws + L.list[d]);
+      lo.first[d] = reinterpret_cast<int*>(ws + L.first[d]);
     }
-    Counts h;
-    OCNN_HIP_OK(hipMemcpyAsync(&h, d_counts, sizeof(Counts), hipMemcpyDeviceToHost, s));
-    OCNN_HIP_OK(hipStreamSynchronize(s));
-    for (int d = fl; d <= depth; ++d) st.nne[d] = h.nne[d];
-  } else {
-    OCNN_HIP_OK(hipStreamSynchronize(s));  // the cloud table came from host memory of this call
+    lo.ustart = reinterpret_cast<int*>(ws + L.ustart);
+    uint32_t* level_status = reinterpret_cast<uint32_t*>(ws + L.level_status);
+    uint32_t* level_groups = reinterpret_cast<uint32_t*>(ws + L.level_groups);
+    if (tickets) levels_kernel<true><<<L.level_tiles, kBlock, 0, s>>>(d_key[cur], (int)N, depth, fl, lo, level_status, level_groups, d_ctl, spin_limit);
+    else levels_kernel<false><<<L.level_tiles, kBlock, 0, s>>>(d_key[cur], (int)N, depth, fl, lo, level_status, level_groups, d_ctl, spin_limit);
+    OCNN_LAUNCH_OK("levels");
+    Control* h = take_slot();
+    OCNN_REQUIRE(h, OCNN_E_HIP, "no pinned host memory for the node counts");
+    hipError_t e = hipMemcpyAsync(h, d_ctl, sizeof(Control), hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    for (int d = fl; d <= depth; ++d) st.nne[d] = h->nne[d];
+    *wait_error = h->error;
+    give_slot(h);
+    OCNN_REQUIRE(e == hipSuccess, OCNN_E_HIP, "node counts: %s", hipGetErrorString(e));
+    return OCNN_OK;
+  };
+
+  int rc = init();
+  if (rc != OCNN_OK) return rc;
+  if (depth > fl) {
+    int wait_error = 0;
+    rc = sort_and_scan(false, g_first_wait_limit.load(), &wait_error);
+    if (rc != OCNN_OK) return rc;
+    if (wait_error) {  // tiles did not start in index order: once more, with ticket order
+      g_ticket_reruns.fetch_add(1);
+      rc = init();
+      if (rc == OCNN_OK) rc = sort_and_scan(true, kTicketWaitLimit, &wait_error);
+      if (rc != OCNN_OK) return rc;
+      OCNN_REQUIRE(wait_error == 0, OCNN_E_HIP, "a tile waited too long for the tiles before it");
+    }
   }
 
   // ---- node counts (calc_node_num, octree.cpp:285-309; batch sums merge_octrees.cpp:39-90)
@@ -710,84 +1142,120 @@ int ocnn_points2octree_emit(void* octree_out_dev, const void* info, void* worksp
   const int depth = o.depth, fl = o.full_layer, B = st.n_clouds;
   char* ws = static_cast<char*>(workspace_dev);
   char* blob = static_cast<char*>(octree_out_dev);
-  const CloudDesc* d_clouds = reinterpret_cast<const CloudDesc*>(ws + L.clouds);
-  const uint32_t* d_sorted_idx = reinterpret_cast<const uint32_t*>(ws + L.val[st.sorted_buf]);
-  const int* d_ustart = reinterpret_cast<const int*>(ws + L.ustart);
-  int* d_leaf_node = reinterpret_cast<int*>(ws + L.leaf_node);
 
-  // header (the tail of the 720-byte header block is padding and must be zero)
-  HeaderArg hdr;
-  memset(&hdr, 0, sizeof(hdr));
-  memcpy(&hdr, &o, sizeof(Info));
-  write_header_kernel<<<1, kBlock, 0, s>>>(reinterpret_cast<uint32_t*>(blob), hdr);
-  OCNN_LAUNCH_OK("write_header");
-
-  EmitGeom eg{depth, fl, B, o.key2xyz, o.channel(OCNN_KEY)};
-  const int kch = o.channel(OCNN_KEY);
-  if (kch == 2) {  // two-channel keys: the second half of each level stays zero (octree.cpp:1145)
-    int64_t cnt = (int64_t)o.total_nnum() * 2 * 2;  // as 4-byte words
-    fill_f32_kernel<<<blocks_for(cnt, kBlock * 4), kBlock, 0, s>>>(reinterpret_cast<float*>(blob + o.ptr_dis(OCNN_KEY, 0)), cnt, 0.0f);
+  EmitArgs a;
+  memset(&a, 0, sizeof(a));
+  memcpy(&a.hdr, &o, sizeof(Info));
+  a.depth = depth;
+  a.full_layer = fl;
+  a.n_clouds = B;
+  a.key2xyz = o.key2xyz;
+  a.key_channel = o.channel(OCNN_KEY);
+  for (int d = 0; d < kMaxLevels; ++d) {
+    a.off_key[d] = a.off_child[d] = a.off_split[d] = a.off_neigh[d] = -1;
+    if (d > depth) continue;
+    a.nnum[d] = o.nnum[d];
+    a.nne[d] = st.nne[d];
+    a.off_key[d] = o.ptr_dis(OCNN_KEY, d);
+    a.off_child[d] = o.ptr_dis(OCNN_CHILD, d);
+    a.off_split[d] = o.ptr_dis(OCNN_SPLIT, d);
+    a.off_neigh[d] = o.ptr_dis(OCNN_NEIGH, d);
+    a.list[d] = reinterpret_cast<const uint64_t*>(ws + L.list[d]);
+    a.first[d] = reinterpret_cast<const int*>(ws + L.first[d]);
   }
-  for (int d = 0; d <= depth; ++d) {
-    uint64_t* key = reinterpret_cast<uint64_t*>(blob + o.ptr_dis(OCNN_KEY, d));
-    int* child = reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_CHILD, d));
-    int64_t n = o.nnum[d];
-    if (n == 0) continue;
-    if (d <= fl) emit_full_kernel<<<blocks_for(n), kBlock, 0, s>>>(key, child, d, n, eg);
-    else emit_sparse_kernel<<<blocks_for(n), kBlock, 0, s>>>(key, child, d, n,
-        reinterpret_cast<const uint64_t*>(ws + L.list[d - 1]), eg);
-    if (d >= fl && depth > fl && st.nne[d] > 0)
-      emit_links_kernel<<<blocks_for(st.nne[d]), kBlock, 0, s>>>(child, d, st.nne[d],
-          reinterpret_cast<const uint64_t*>(ws + L.list[d]), reinterpret_cast<const int*>(ws + L.prank[d]),
-          d == depth ? d_leaf_node : nullptr, eg);
-    OCNN_LAUNCH_OK("emit structure");
-  }
-  // features / labels of the finest level
   const int64_t HD = o.nnum[depth];
   const int fch = o.channel(OCNN_FEATURE);
-  float* feature = fch > 0 ? reinterpret_cast<float*>(blob + o.ptr_dis(OCNN_FEATURE, depth)) : nullptr;
-  float* label = o.has(OCNN_LABEL) ? reinterpret_cast<float*>(blob + o.ptr_dis(OCNN_LABEL, depth)) : nullptr;
-  if (feature && HD > 0) fill_f32_kernel<<<blocks_for(fch * HD, kBlock * 4), kBlock, 0, s>>>(feature, fch * HD, 0.0f);
-  if (label && HD > 0) fill_f32_kernel<<<blocks_for(HD, kBlock * 4), kBlock, 0, s>>>(label, HD, -1.0f);
-  if (depth > fl && st.nne[depth] > 0 && (feature || label)) {
-    SignalGeom sg;
-    sg.depth = depth;
-    sg.n_clouds = B;
-    sg.nnum_d = (int)HD;
-    sg.ch_normal = st.ch_normal;
-    sg.ch_feature = st.ch_feature;
-    sg.has_label = label != nullptr;
-    sg.has_dis = o.has_node_dis;
-    sg.save_pts = o.save_pts;
-    for (int i = 0; i < 3; ++i) sg.bbmin[i] = o.bbmin[i];
-    sg.mul = st.mul;
-    leaf_signal_kernel<<<blocks_for(st.nne[depth], 64), 64, 0, s>>>(feature, label, st.nne[depth],
-        reinterpret_cast<const uint64_t*>(ws + L.list[depth]), d_ustart, d_sorted_idx, d_leaf_node, d_clouds, sg);
+  a.off_feature = fch > 0 ? o.ptr_dis(OCNN_FEATURE, depth) : -1;
+  a.off_label = o.has(OCNN_LABEL) ? o.ptr_dis(OCNN_LABEL, depth) : -1;
+  a.ustart = reinterpret_cast<const int*>(ws + L.ustart);
+  a.sorted_idx = reinterpret_cast<const uint32_t*>(ws + L.val[st.sorted_buf]);
+  a.clouds = reinterpret_cast<const CloudDesc*>(ws + L.clouds);
+  a.sg.depth = depth;
+  a.sg.nnum_d = (int)HD;
+  a.sg.ch_feature = st.ch_feature;
+  a.sg.channels = fch;
+  a.sg.has_label = a.off_label >= 0;
+  a.sg.has_dis = o.has_node_dis;
+  a.sg.save_pts = o.save_pts;
+  for (int i = 0; i < 3; ++i) a.sg.bbmin[i] = o.bbmin[i];
+  a.sg.mul = st.mul;
+
+  int n_seg = 0, blocks = 0;
+  auto add_seg = [&](int kind, int level, int64_t nblocks) {
+    if (nblocks <= 0) return;
+    a.seg_begin[n_seg] = blocks;
+    a.seg_kind[n_seg] = (unsigned char)kind;
+    a.seg_level[n_seg] = (unsigned char)level;
+    ++n_seg;
+    blocks += (int)nblocks;
+  };
+  add_seg(kSegHeader, 0, 1);
+  for (int d = depth; d > fl; --d) add_seg(kSegSparse, d, blocks_for(st.nne[d - 1]) * (st.nne[d - 1] > 0 ? 1 : 0));
+  for (int d = 0; d <= fl; ++d) {
+    add_seg(kSegFull, d, blocks_for(o.nnum[d]));
+    if (o.has(OCNN_NEIGH) && d >= 1) add_seg(kSegFullNeigh, d, blocks_for((int64_t)B << (3 * d + 3)));
+  }
+  a.seg_begin[n_seg] = blocks;
+  a.n_seg = n_seg;
+  emit_kernel<<<blocks, kBlock, 0, s>>>(blob, a);
+  OCNN_LAUNCH_OK("emit");
+
+  if (depth > fl && HD > 0 && (a.off_feature >= 0 || a.off_label >= 0)) {
+    float* f_ptr = a.off_feature >= 0 ? reinterpret_cast<float*>(blob + a.off_feature) : nullptr;
+    float* l_ptr = a.off_label >= 0 ? reinterpret_cast<float*>(blob + a.off_label) : nullptr;
+    const int* c_ptr = reinterpret_cast<const int*>(blob + a.off_child[depth]);
+    if (fch <= kSignalStage) {
+      const size_t lds = sizeof(float) * kSignalTile * (size_t)(fch + (l_ptr ? 1 : 0));
+      leaf_signal_staged_kernel<<<blocks_for(HD, kSignalTile), kBlock, lds, s>>>(f_ptr, l_ptr, c_ptr, a.list[depth],
+          a.ustart, a.sorted_idx, a.clouds, a.sg);
+    } else {
+      leaf_signal_kernel<<<blocks_for(HD), kBlock, 0, s>>>(f_ptr, l_ptr, c_ptr, a.list[depth], a.ustart,
+          a.sorted_idx, a.clouds, a.sg);
+    }
     OCNN_LAUNCH_OK("leaf_signal");
   }
-  if (o.has(OCNN_SPLIT)) {
-    int64_t n = o.total_nnum();
-    split_kernel<<<blocks_for(n), kBlock, 0, s>>>(reinterpret_cast<float*>(blob + o.ptr_dis(OCNN_SPLIT, 0)),
-        reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_CHILD, 0)), n);
-    OCNN_LAUNCH_OK("split");
+  if (depth == fl && HD > 0) {  // no sparse level: the finest level carries no signal
+    if (a.off_feature >= 0)
+      fill_f32_kernel<<<blocks_for(fch * HD, kBlock * 4), kBlock, 0, s>>>(reinterpret_cast<float*>(blob + a.off_feature), fch * HD, 0.0f);
+    if (a.off_label >= 0)
+      fill_f32_kernel<<<blocks_for(HD, kBlock * 4), kBlock, 0, s>>>(reinterpret_cast<float*>(blob + a.off_label), HD, -1.0f);
+    OCNN_LAUNCH_OK("fill");
   }
-  if (o.has(OCNN_NEIGH)) {  // merge_octrees.cpp:185-197; depth 0 holds no table (left zero)
-    int64_t n0 = (int64_t)o.nnum[0] * 8;
-    fill_f32_kernel<<<blocks_for(n0), kBlock, 0, s>>>(reinterpret_cast<float*>(blob + o.ptr_dis(OCNN_NEIGH, 0)), n0, 0.0f);
-    for (int d = 1; d <= depth; ++d) {
-      int* neigh = reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_NEIGH, d));
-      if (d <= fl) {
-        int64_t total = (int64_t)B << (3 * d + 3);
-        b_neigh_full_kernel<<<blocks_for(total), kBlock, 0, s>>>(neigh, d, total);
-      } else if (o.nnum[d - 1] > 0) {
-        b_neigh_sparse_kernel<<<blocks_for(o.nnum[d - 1]), kBlock, 0, s>>>(neigh,
-            reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_NEIGH, d - 1)),
-            reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_CHILD, d - 1)), o.nnum[d - 1]);
-      }
+  if (o.has(OCNN_NEIGH)) {  // merge_octrees.cpp:185-197: sparse levels, each from the level above
+    for (int d = fl + 1; d <= depth; ++d) {
+      if (o.nnum[d - 1] <= 0) continue;
+      launch_neigh_sparse(reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_NEIGH, d)),
+          reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_NEIGH, d - 1)),
+          reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_CHILD, d - 1)), o.nnum[d - 1], s);
       OCNN_LAUNCH_OK("neigh");
     }
   }
   return OCNN_OK;
+}
+
+int ocnn_points2octree_wait_limit(int polls) {
+  const int before = g_first_wait_limit.load();
+  g_first_wait_limit.store(polls == 0 ? kFirstWaitLimit : polls);
+  return before;
+}
+int ocnn_points2octree_ticket_reruns(void) { return g_ticket_reruns.load(); }
+
+int ocnn_points2octree(const void* const* points_dev, const void* const* points_info, int n_clouds,
+    const ocnn_build_params* params, void* workspace_dev, size_t workspace_bytes, ocnn_alloc_fn alloc,
+    void* alloc_ctx, void* info_out, void** octree_out_dev, ocnn_stream_t stream) {
+  OCNN_REQUIRE(alloc && octree_out_dev, OCNN_E_BADARG, "null pointer");
+  int e = ocnn_points2octree_plan(points_dev, points_info, n_clouds, params, workspace_dev, workspace_bytes,
+      info_out, stream);
+  if (e != OCNN_OK) return e;
+  void* blob = alloc((size_t)static_cast<const Info*>(info_out)->sizeof_octree(), alloc_ctx);
+  if (!blob) {
+    std::lock_guard<std::mutex> lock(g_plans_mutex);
+    g_plans.erase(workspace_dev);
+    return fail(OCNN_E_BADARG, "the allocator returned no memory for %lld bytes",
+        (long long)static_cast<const Info*>(info_out)->sizeof_octree());
+  }
+  *octree_out_dev = blob;
+  return ocnn_points2octree_emit(blob, info_out, workspace_dev, workspace_bytes, stream);
 }
 
 }  // extern "C"

@@ -1,109 +1,10 @@
 // Integer kernels on the octree structure: neighbour tables, key generation,
 // Morton <-> packed-xyz conversion, sorted-key search, label compaction.
 // Everything here is bit-exact integer work bound by HBM bandwidth.
-#include "ocnn_common.h"
-#include "scan.h"
+#include "octree_kernels.h"
 
 namespace ocnn {
-
-// Morton helpers: bit i of axis j lands at bit 3*i + 2 - j (x highest), the
-// convention of compute_key / compute_pt (octree/octree/octree_nn.cpp:551-575).
-__host__ __device__ inline uint64_t spread3(uint64_t v) {  // 16 bits -> every third bit
-  v &= 0xffffull;
-  v = (v | (v << 32)) & 0x00ff00000000ffffull;
-  v = (v | (v << 16)) & 0x00ff0000ff0000ffull;
-  v = (v | (v << 8)) & 0xf00f00f00f00f00full;
-  v = (v | (v << 4)) & 0x30c30c30c30c30c3ull;
-  v = (v | (v << 2)) & 0x9249249249249249ull;
-  return v;
-}
-__host__ __device__ inline uint64_t compact3(uint64_t v) {  // inverse of spread3
-  v &= 0x9249249249249249ull;
-  v = (v | (v >> 2)) & 0x30c30c30c30c30c3ull;
-  v = (v | (v >> 4)) & 0xf00f00f00f00f00full;
-  v = (v | (v >> 8)) & 0x00ff0000ff0000ffull;
-  v = (v | (v >> 16)) & 0x00ff00000000ffffull;
-  v = (v | (v >> 32)) & 0xffffull;
-  return v;
-}
-__host__ __device__ inline uint64_t morton_encode(uint32_t x, uint32_t y, uint32_t z, int depth) {
-  uint64_t m = depth >= 16 ? 0xffffull : ((1ull << depth) - 1);
-  return (spread3(x & m) << 2) | (spread3(y & m) << 1) | spread3(z & m);
-}
-__host__ __device__ inline void morton_decode(uint64_t key, int depth, uint32_t* x, uint32_t* y, uint32_t* z) {
-  uint64_t m = depth >= 16 ? 0xffffull : ((1ull << depth) - 1);
-  *x = (uint32_t)(compact3(key >> 2) & m);
-  *y = (uint32_t)(compact3(key >> 1) & m);
-  *z = (uint32_t)(compact3(key) & m);
-}
-
 namespace {
-
-// ---- neighbour tables --------------------------------------------------------
-// Sparse-layer neighbour table.  A workgroup takes 256 consecutive parent-level nodes,
-// compacts the non-empty ones into LDS (most nodes of a deep level are empty) and then
-// every wavefront writes the 64-slot blocks of the compacted nodes, four nodes per
-// iteration so that four dependent load chains (neigh -> children) are in flight.
-__global__ void calc_neigh_sparse_kernel(int* __restrict__ neigh_child, const int* __restrict__ neigh,
-    const int* __restrict__ children, int node_num) {
-  __shared__ int s_node[kBlock], s_rank[kBlock], s_count;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int i = blockIdx.x * kBlock + threadIdx.x;
-  const int l0 = i < node_num ? children[i] : -1;
-  int total;
-  const int pos = block_exclusive_scan(l0 >= 0 ? 1 : 0, &total);
-  if (l0 >= 0) { s_node[pos] = i; s_rank[pos] = l0; }
-  if (threadIdx.x == 0) s_count = total;
-  __syncthreads();
-  const int count = s_count;
-  const int x = lane >> 4, y = (lane >> 2) & 3, z = lane & 3;
-  const int hx = (x + 1) >> 1, hy = (y + 1) >> 1, hz = (z + 1) >> 1;
-  const int octant = (((x + 1) & 1) << 2) | (((y + 1) & 1) << 1) | ((z + 1) & 1);
-  for (int e = wave * 4; e < count; e += 4 * (kBlock / 64)) {
-    int t[4], rank[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      t[u] = -1;
-      rank[u] = -1;
-      if (e + u < count) {
-        const int node = s_node[e + u];
-        rank[u] = s_rank[e + u];
-        const int sib = node & 7;
-        const int slot = ((hx + (sib >> 2)) << 4) | ((hy + ((sib >> 1) & 1)) << 2) | (hz + (sib & 1));
-        t[u] = neigh[((int64_t)(node >> 3) << 6) + slot];
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      int v = -1;
-      if (t[u] >= 0) {
-        const int l1 = children[t[u]];
-        if (l1 >= 0) v = (l1 << 3) + octant;
-      }
-      if (rank[u] >= 0) neigh_child[((int64_t)rank[u] << 6) + lane] = v;
-    }
-  }
-}
-
-// Full layer: closed form through Morton decode / encode.
-__global__ void calc_neigh_full_kernel(int* __restrict__ neigh, int depth, int64_t total) {
-  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (id >= total) return;
-  const int64_t node_num = (int64_t)1 << (3 * depth);
-  const int64_t groups = node_num >> 3;
-  int slot = (int)(id & 63);
-  int64_t g = id >> 6;
-  int64_t n = g / groups;
-  uint64_t i = (uint64_t)(g % groups) << 3;
-  uint32_t x0, y0, z0;
-  morton_decode(i, depth, &x0, &y0, &z0);
-  uint32_t x1 = x0 + (slot >> 4) - 1, y1 = y0 + ((slot >> 2) & 3) - 1, z1 = z0 + (slot & 3) - 1;
-  const uint32_t bound = 1u << depth;
-  int v = -1;
-  // a coordinate of -1 or 2^depth has the bound bit set (two's complement / carry)
-  if (((x1 | y1 | z1) & bound) == 0) v = (int)(morton_encode(x1, y1, z1, depth) + (uint64_t)n * node_num);
-  neigh[id] = v;
-}
 
 // ---- keys -----------------------------------------------------------------------
 __global__ void gen_key_child_kernel(uint64_t* __restrict__ key_child, const uint64_t* __restrict__ key,
@@ -193,8 +94,7 @@ int ocnn_calc_neigh_sparse(int* neigh_child, const int* neigh, const int* childr
   OCNN_REQUIRE(neigh_child && neigh && children, OCNN_E_BADARG, "null pointer");
   OCNN_REQUIRE(node_num >= 0, OCNN_E_BADARG, "node_num %d", node_num);
   if (node_num == 0) return OCNN_OK;
-  calc_neigh_sparse_kernel<<<blocks_for(node_num), kBlock, 0, as_stream(stream)>>>(neigh_child, neigh,
-      children, node_num);
+  launch_neigh_sparse(neigh_child, neigh, children, node_num, as_stream(stream));
   OCNN_LAUNCH_OK("calc_neigh_sparse");
   return OCNN_OK;
 }
@@ -205,7 +105,7 @@ int ocnn_calc_neigh_full(int* neigh, int depth, int batch_size, ocnn_stream_t st
       "depth %d batch %d (a full layer deeper than 9 does not fit int32 indices)", depth, batch_size);
   int64_t total = (int64_t)batch_size << (3 * depth + 3);
   OCNN_REQUIRE(total < (1ll << 34), OCNN_E_BADARG, "full layer too large");
-  calc_neigh_full_kernel<<<blocks_for(total), kBlock, 0, as_stream(stream)>>>(neigh, depth, total);
+  neigh_full_kernel<<<blocks_for(total), kBlock, 0, as_stream(stream)>>>(neigh, depth, total);
   OCNN_LAUNCH_OK("calc_neigh_full");
   return OCNN_OK;
 }

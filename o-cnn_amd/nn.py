@@ -155,6 +155,9 @@ def _points_header(points):
   return hdr
 
 
+_ALLOC_FN = C.CFUNCTYPE(C.c_void_p, C.c_size_t, C.c_void_p)
+
+
 def _build(points_list, merged, depth, full_depth, node_dis, node_feature, split_label, adaptive,
            adp_depth, th_normal, th_distance, extrapolate, save_pts, key2xyz, bbox=None):
   pts = [_to_dev(p) for p in points_list]
@@ -182,13 +185,19 @@ def _build(points_list, merged, depth, full_depth, node_dis, node_feature, split
   dev_ptrs = (C.c_void_p * n)(*[p.data_ptr() for p in pts])
   hdr_ptrs = (C.c_void_p * n)(*[h.ctypes.data for h in hdrs])
   info_raw = np.zeros(INFO_BYTES, np.uint8)
-  _lib.call("ocnn_points2octree_plan", dev_ptrs, hdr_ptrs, n, C.byref(bp), C.c_void_p(base),
-            C.c_size_t(ws_bytes), C.c_void_p(info_raw.ctypes.data), _stream())
-  info = _Info(info_raw)
-  out = torch.empty(info.size(), dtype=torch.uint8, device=_dev())
-  _lib.call("ocnn_points2octree_emit", _ptr(out), info.p, C.c_void_p(base), C.c_size_t(ws_bytes),
-            _stream())
-  out._ocnn_info = info
+  holder = []
+
+  def alloc(nbytes, _ctx):
+    t = torch.empty(int(nbytes), dtype=torch.uint8, device=_dev())
+    holder.append(t)
+    return t.data_ptr()
+
+  out_ptr = C.c_void_p()
+  _lib.call("ocnn_points2octree", dev_ptrs, hdr_ptrs, n, C.byref(bp), C.c_void_p(base),
+            C.c_size_t(ws_bytes), _ALLOC_FN(alloc), None, C.c_void_p(info_raw.ctypes.data),
+            C.byref(out_ptr), _stream())
+  out = holder[0]
+  out._ocnn_info = _Info(info_raw)
   return out
 
 

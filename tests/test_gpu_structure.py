@@ -79,6 +79,87 @@ def test_build_edge_cases(oc, orc):
       assert np.array_equal(got, orc.points2octree(pb, depth, fd, node_dis=True)), (depth, fd)
 
 
+def test_build_wide_features_and_many_clouds(oc, orc):
+  """More feature channels than the leaf kernel stages in LDS, more clouds than one launch
+  of the cloud table carries, labels and displacement together."""
+  rng = np.random.default_rng(21)
+  n = 3000
+  pts = rng.uniform(-0.999, 0.999, (n, 3)).astype(np.float32)
+  nrm = rng.standard_normal((n, 3)).astype(np.float32)
+  feat = rng.uniform(0, 1, (n, 11)).astype(np.float32)
+  lab = rng.integers(0, 4, n).astype(np.float32)
+  pb = make_points_blob(pts, nrm, feat, lab)
+  for kw in (dict(), dict(node_dis=True, save_pts=True)):
+    got = oc.nn.points2octree(T(pb), 6, 2, **kw).cpu().numpy()
+    assert np.array_equal(got, orc.points2octree(pb, 6, 2, **kw)), kw
+  blobs = []
+  for i in range(70):
+    m = int(rng.integers(1, 400))
+    blobs.append(make_points_blob(rng.uniform(-0.999, 0.999, (m, 3)).astype(np.float32),
+                                  rng.standard_normal((m, 3)).astype(np.float32)))
+  got = oc.nn.points2octree_batch([T(b) for b in blobs], 5, 2).cpu().numpy()
+  assert np.array_equal(got, orc.octree_batch([orc.points2octree(b, 5, 2) for b in blobs]))
+
+
+def test_build_two_steps_and_ticket_repeat(oc, orc, synthetic):
+  """The plan / emit pair gives the blob of the one-call entry point; a first attempt that is
+  made to fail from the host is repeated with ticket order and gives the same blob."""
+  import ctypes as C
+  p, nrm, f = synthetic.room_cloud(60000, 5)
+  pb = make_points_blob(p, nrm, f)
+  exp = orc.octree_batch([orc.points2octree(pb, 8, 2)])
+  cloud = T(pb).cuda()
+  L = oc.lib.get()
+  hdr = pb[:88].copy()
+  bp = oc.lib.BuildParams(depth=8, full_depth=2, adp_depth=4, th_normal=0.1, th_distance=2.0, merged=1)
+  ws_bytes = L.ocnn_points2octree_workspace_bytes(60000, 1, 8)
+  ws = torch.empty(ws_bytes + 256, dtype=torch.uint8, device="cuda")
+  base = (ws.data_ptr() + 255) & ~255
+  dev = (C.c_void_p * 1)(cloud.data_ptr())
+  hp = (C.c_void_p * 1)(hdr.ctypes.data)
+  info = np.zeros(716, np.uint8)
+  stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+  oc.lib.call("ocnn_points2octree_plan", dev, hp, 1, C.byref(bp), C.c_void_p(base), C.c_size_t(ws_bytes),
+              C.c_void_p(info.ctypes.data), stream)
+  size = L.ocnn_info_sizeof_octree(C.c_void_p(info.ctypes.data))
+  assert size == exp.size
+  out = torch.empty(size, dtype=torch.uint8, device="cuda")
+  oc.lib.call("ocnn_points2octree_emit", C.c_void_p(out.data_ptr()), C.c_void_p(info.ctypes.data),
+              C.c_void_p(base), C.c_size_t(ws_bytes), stream)
+  assert np.array_equal(out.cpu().numpy(), exp)
+  # emit without a plan on this workspace is an error, not a crash
+  assert L.ocnn_points2octree_emit(C.c_void_p(out.data_ptr()), C.c_void_p(info.ctypes.data), C.c_void_p(base),
+                                   C.c_size_t(ws_bytes), stream) != 0
+
+  before = L.ocnn_points2octree_ticket_reruns()
+  old = L.ocnn_points2octree_wait_limit(-1)
+  try:
+    got = oc.nn.points2octree_batch([cloud], 8, 2)
+  finally:
+    L.ocnn_points2octree_wait_limit(old)
+  assert L.ocnn_points2octree_ticket_reruns() == before + 1
+  assert np.array_equal(got.cpu().numpy(), exp)
+  assert np.array_equal(oc.nn.points2octree_batch([cloud], 8, 2).cpu().numpy(), exp)
+  assert L.ocnn_points2octree_ticket_reruns() == before + 1
+
+
+def test_build_large_tiles(oc, synthetic):
+  """More than 2^19 points (the larger sort tile): the structure invariants hold and the blob
+  equals the blob of batching the separately built octrees."""
+  clouds = []
+  for i in range(3):
+    p, nrm, f = synthetic.room_cloud(200000, 11 + i)
+    clouds.append(T(make_points_blob(p, nrm, f)).cuda())
+  fused = oc.nn.points2octree_batch(clouds, 8, 2)
+  singles = [oc.nn.points2octree(c, 8, 2) for c in clouds]
+  assert torch.equal(fused, oc.nn.octree_batch(singles))
+  b = OctreeBlob(fused.cpu().numpy())
+  for d in range(3, 9):
+    assert b.nnum[d] == 8 * b.nnum_nempty[d - 1]
+    c = b.prop("child", d)
+    assert np.array_equal(c[c >= 0], np.arange(b.nnum_nempty[d]))
+
+
 def test_build_rejects_what_it_cannot_do(oc):
   pb = make_points_blob([[0, 0, 0]], [[1, 0, 0]])
   with pytest.raises(oc.lib.OcnnError) as e:
