@@ -33,6 +33,11 @@ PEAK_MFMA_TFLOPS = {"f32": 157.3, "bf16": 2500.0}
 RECORDED_TRAFFIC = {("conv_s1_f32_lds_kernel", 1494168, 64, 64): 1.018e9}
 
 
+def oc_points_blob(cloud):
+  from oracle.checker import make_points_blob
+  return make_points_blob(cloud[0], cloud[1])
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--gpus", type=int, default=1)
@@ -265,6 +270,17 @@ def main():
     torch.cuda.synchronize()
     t = (time.perf_counter() - t0) / reps
     extra["points2octree_batch16_d7"] = {"ms": t * 1e3, "Mpts_per_s": 0.8 / t}
+    # the adaptive build of configs[4]'s input: all-depth signals, plane-fit errors, trimming,
+    # one cloud at a time, then octree_batch (summation order of the reference kept: bit-exact)
+    adp = dict(node_dis=True, split_label=True, adaptive=True, adp_depth=4, th_normal=0.1, th_distance=2.0)
+    F.points2octree_batch(cl, 7, 2, **adp)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(max(2, reps // 4)):
+      F.points2octree_batch(cl, 7, 2, **adp)
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / max(2, reps // 4)
+    extra["points2octree_adaptive_batch16_d7"] = {"ms": t * 1e3, "Mpts_per_s": 0.8 / t}
     i7 = F.octree_info(oct7)
     H7 = i7.nnum(7)
     x7 = torch.randn(1, C, H7, 1, generator=g).to(dev)
@@ -447,6 +463,11 @@ def main():
     lab8 = (child8 >= 0).astype(np.int32)
     upd = cpu_row("octree_update_d8", lambda: orc.octree_update(merged, lab8, 8, 1), H8, "nodes_per_s")
     del upd
+    pb5 = oc_points_blob(oc.synthetic.shape_cloud(50000, 200))
+    cpu_row("points2octree_adaptive_one_cloud_d7", lambda: chk.points2octree(
+        pb5, 7, 2, node_dis=True, split_label=True, adaptive=True, adp_depth=4, th_normal=0.1, th_distance=2.0),
+        50000, "points_per_s")
+    rows["points2octree_adaptive_one_cloud_d7"]["kind"] = "reference" if ref_ok else "port"
     out["cpu_baseline"]["rows"] = rows
 
   print(json.dumps(out))

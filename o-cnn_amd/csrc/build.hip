@@ -27,6 +27,7 @@
 //            wavefront (zeros for empty nodes);
 //          one launch per sparse level for the neighbour tables (each needs the
 //            level above).
+#include "build_adaptive.h"
 #include "octree_kernels.h"
 
 #include <atomic>
@@ -538,20 +539,41 @@ __device__ inline void leaf_signal(float* __restrict__ feature, float* __restric
   float acc[3] = {0.0f, 0.0f, 0.0f}, avg_pt[3] = {0.0f, 0.0f, 0.0f}, facc[kRegFeatures];
 #pragma unroll
   for (int c = 0; c < kRegFeatures; ++c) facc[c] = 0.0f;
-  for (int i = s0; i < s1; ++i) {
-    const int64_t idx = (int64_t)(sorted_idx[i] - cd.offset);
-    if (cd.normal) {
-      const float* q = cd.normal + 3 * idx;
-      for (int c = 0; c < 3; ++c) acc[c] = __fadd_rn(acc[c], q[c]);
-    }
-    if (need_pt) {
-      const float* q = cd.xyz + 3 * idx;
-      for (int c = 0; c < 3; ++c) avg_pt[c] = __fadd_rn(avg_pt[c], scale_coord(q[c], g.bbmin[c], g.mul));
-    }
-    const float* q = cd.feature + F * idx;
+  // two points at a time: all their loads are requested before the first sum, the sums
+  // themselves stay in ascending point order
+  constexpr int kChunk = 2;
+  for (int i0 = s0; i0 < s1; i0 += kChunk) {
+    int64_t idx[kChunk];
+    float nv[kChunk][3], pv[kChunk][3], fv[kChunk][kRegFeatures];
 #pragma unroll
-    for (int c = 0; c < kRegFeatures; ++c)
-      if (c < F) facc[c] = __fadd_rn(facc[c], q[c]);
+    for (int u = 0; u < kChunk; ++u) idx[u] = i0 + u < s1 ? (int64_t)(sorted_idx[i0 + u] - cd.offset) : -1;
+#pragma unroll
+    for (int u = 0; u < kChunk; ++u) {
+      if (idx[u] < 0) continue;
+      if (cd.normal) {
+        const float* q = cd.normal + 3 * idx[u];
+        for (int c = 0; c < 3; ++c) nv[u][c] = q[c];
+      }
+      if (need_pt) {
+        const float* q = cd.xyz + 3 * idx[u];
+        for (int c = 0; c < 3; ++c) pv[u][c] = q[c];
+      }
+      const float* q = cd.feature + F * idx[u];
+#pragma unroll
+      for (int c = 0; c < kRegFeatures; ++c)
+        if (c < F) fv[u][c] = q[c];
+    }
+#pragma unroll
+    for (int u = 0; u < kChunk; ++u) {
+      if (idx[u] < 0) continue;
+      if (cd.normal)
+        for (int c = 0; c < 3; ++c) acc[c] = __fadd_rn(acc[c], nv[u][c]);
+      if (need_pt)
+        for (int c = 0; c < 3; ++c) avg_pt[c] = __fadd_rn(avg_pt[c], scale_coord(pv[u][c], g.bbmin[c], g.mul));
+#pragma unroll
+      for (int c = 0; c < kRegFeatures; ++c)
+        if (c < F) facc[c] = __fadd_rn(facc[c], fv[u][c]);
+    }
   }
   int ch = 0;
   float nrm[3] = {0.0f, 0.0f, 0.0f};
@@ -921,7 +943,7 @@ int ocnn_points2octree_plan(const void* const* points_dev, const void* const* po
   OCNN_REQUIRE(n_clouds >= 1 && n_clouds <= 65535, OCNN_E_BADARG, "n_clouds %d", n_clouds);
   OCNN_REQUIRE(params->merged || n_clouds == 1, OCNN_E_BADARG, "a single-octree blob holds one cloud");
   OCNN_REQUIRE(!params->node_feature && !params->adaptive, OCNN_E_UNSUPPORTED,
-      "node_feature / adaptive octrees are not built on the device");
+      "node_feature / adaptive octrees take two rounds of allocation: use ocnn_points2octree");
   hipStream_t s = as_stream(stream);
 
   // ---- headers: every cloud must carry the same properties (OctreeInfo::is_consistent)
@@ -1243,7 +1265,41 @@ int ocnn_points2octree_ticket_reruns(void) { return g_ticket_reruns.load(); }
 int ocnn_points2octree(const void* const* points_dev, const void* const* points_info, int n_clouds,
     const ocnn_build_params* params, void* workspace_dev, size_t workspace_bytes, ocnn_alloc_fn alloc,
     void* alloc_ctx, void* info_out, void** octree_out_dev, ocnn_stream_t stream) {
-  OCNN_REQUIRE(alloc && octree_out_dev, OCNN_E_BADARG, "null pointer");
+  OCNN_REQUIRE(alloc && octree_out_dev && params && points_info && points_dev, OCNN_E_BADARG, "null pointer");
+  if (params->node_feature || params->adaptive) {
+    // Signals at every depth / trimming: a plain single octree first (raw Morton keys, average
+    // points kept whenever the displacement is), then the second stage on top of it.
+    OCNN_REQUIRE(n_clouds == 1 && !params->merged, OCNN_E_UNSUPPORTED,
+        "node_feature / adaptive octrees are built one cloud at a time (batch them with ocnn_octree_batch)");
+    const PointsInfo* pi = static_cast<const PointsInfo*>(points_info[0]);
+    OCNN_REQUIRE(pi, OCNN_E_BADARG, "null cloud header");
+    const bool has_normal = (pi->content_flags & 2) != 0;
+    // trim_octree reads the normal error (exists only with normals) and leaves the average
+    // points untrimmed (octree.cpp:1004-1135): the reference cannot build these either
+    OCNN_REQUIRE(!params->adaptive || (has_normal && !params->save_pts && params->adp_depth >= 1),
+        OCNN_E_UNSUPPORTED, "adaptive octrees need normals, no save_pts and adp_depth >= 1");
+    ocnn_build_params p0 = *params;
+    p0.node_feature = p0.adaptive = p0.key2xyz = p0.split_label = p0.extrapolate = 0;
+    p0.save_pts = (params->node_dis || params->save_pts) ? 1 : 0;
+    AdaptiveInput in;
+    int e = ocnn_points2octree_plan(points_dev, points_info, 1, &p0, workspace_dev, workspace_bytes, &in.info0, stream);
+    if (e != OCNN_OK) return e;
+    in.blob0 = static_cast<char*>(alloc((size_t)in.info0.sizeof_octree(), alloc_ctx));
+    if (!in.blob0) {
+      std::lock_guard<std::mutex> lock(g_plans_mutex);
+      g_plans.erase(workspace_dev);
+      return fail(OCNN_E_BADARG, "the allocator returned no memory for the first-stage octree");
+    }
+    e = ocnn_points2octree_emit(in.blob0, &in.info0, workspace_dev, workspace_bytes, stream);
+    if (e != OCNN_OK) return e;
+    in.ch_normal = has_normal ? pi->channels[1] : 0;
+    in.ch_feature = (pi->content_flags & 4) ? pi->channels[2] : 0;
+    in.ch_dis = params->node_dis ? (has_normal ? 1 : 4) : 0;
+    in.has_pt = p0.save_pts;
+    in.has_label = (pi->content_flags & 8) && pi->channels[3] == 1;
+    in.params = *params;
+    return adaptive_finish(in, alloc, alloc_ctx, info_out, octree_out_dev, as_stream(stream));
+  }
   int e = ocnn_points2octree_plan(points_dev, points_info, n_clouds, params, workspace_dev, workspace_bytes,
       info_out, stream);
   if (e != OCNN_OK) return e;

@@ -160,6 +160,12 @@ _ALLOC_FN = C.CFUNCTYPE(C.c_void_p, C.c_size_t, C.c_void_p)
 
 def _build(points_list, merged, depth, full_depth, node_dis, node_feature, split_label, adaptive,
            adp_depth, th_normal, th_distance, extrapolate, save_pts, key2xyz, bbox=None):
+  if merged and (node_feature or adaptive):
+    # octrees with a signal at every depth are built one cloud at a time and merged afterwards,
+    # as collate_octrees does (pytorch/ocnn/transforms.py:127-148)
+    return octree_batch([_build([p], False, depth, full_depth, node_dis, node_feature, split_label, adaptive,
+                                adp_depth, th_normal, th_distance, extrapolate, save_pts, key2xyz, bbox)
+                         for p in points_list])
   pts = [_to_dev(p) for p in points_list]
   hdrs = [getattr(p, "_ocnn_points_info", None) for p in points_list]
   for i, h in enumerate(hdrs):
@@ -196,7 +202,7 @@ def _build(points_list, merged, depth, full_depth, node_dis, node_feature, split
   _lib.call("ocnn_points2octree", dev_ptrs, hdr_ptrs, n, C.byref(bp), C.c_void_p(base),
             C.c_size_t(ws_bytes), _ALLOC_FN(alloc), None, C.c_void_p(info_raw.ctypes.data),
             C.byref(out_ptr), _stream())
-  out = holder[0]
+  out = [t for t in holder if t.data_ptr() == out_ptr.value][-1]   # (scratch blocks come first)
   out._ocnn_info = _Info(info_raw)
   return out
 

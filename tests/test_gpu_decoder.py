@@ -23,10 +23,24 @@ def relerr(got, exp):
 
 
 @pytest.fixture(scope="module")
-def adaptive_batch(orc, synthetic):
-  singles = [orc.points2octree(make_points_blob(*synthetic.shape_cloud(4000, 300 + i)[:2]), 5, 2, **ADAPTIVE)
-             for i in range(3)]
+def adaptive_clouds(synthetic):
+  return [make_points_blob(*synthetic.shape_cloud(4000, 300 + i)[:2]) for i in range(3)]
+
+
+@pytest.fixture(scope="module")
+def adaptive_batch(orc, adaptive_clouds):
+  singles = [orc.points2octree(pb, 5, 2, **ADAPTIVE) for pb in adaptive_clouds]
   return singles, orc.octree_batch(singles)
+
+
+def test_adaptive_octrees_built_on_gpu(oc, adaptive_clouds, adaptive_batch):
+  """The decoder's input is built on the device too: adaptive points2octree per cloud, then
+  octree_batch, byte for byte the oracle's batch."""
+  singles, host = adaptive_batch
+  built = [oc.nn.points2octree(T(pb), 5, 2, **ADAPTIVE) for pb in adaptive_clouds]
+  for got, exp in zip(built, singles):
+    assert np.array_equal(got.cpu().numpy(), exp)
+  assert np.array_equal(oc.nn.points2octree_batch([T(pb) for pb in adaptive_clouds], 5, 2, **ADAPTIVE).cpu().numpy(), host)
 
 
 def test_adaptive_octrees_merge_on_gpu(oc, orc, adaptive_batch):

@@ -161,15 +161,95 @@ def test_build_large_tiles(oc, synthetic):
 
 
 def test_build_rejects_what_it_cannot_do(oc):
-  pb = make_points_blob([[0, 0, 0]], [[1, 0, 0]])
+  pb = make_points_blob([[0, 0, 0]])          # no normals: trimming has no normal error to read
   with pytest.raises(oc.lib.OcnnError) as e:
     oc.nn.points2octree(T(pb), 5, 2, adaptive=True)
+  assert e.value.code == -2
+  pb = make_points_blob([[0, 0, 0]], [[1, 0, 0]])
+  with pytest.raises(oc.lib.OcnnError) as e:
+    oc.nn.points2octree(T(pb), 5, 2, adaptive=True, save_pts=True)
   assert e.value.code == -2
   bad = pb.copy()
   bad[0] = 0
   with pytest.raises(oc.lib.OcnnError) as e:
     oc.nn.points2octree(T(bad), 5, 2)
   assert e.value.code == -6
+
+
+def test_adaptive_known_answer_on_gpu(oc, orc):
+  """octree/test/test_octree.cpp:196-331 (TestOctreeTrim) built on the device."""
+  pb = three_point_cloud()
+  kw = dict(node_dis=True, split_label=True, adaptive=True, adp_depth=3, th_normal=5.0, th_distance=3.0)
+  got = oc.nn._build([T(pb)], False, 5, 1, True, False, True, True, 3, 5.0, 3.0, False, False, False,
+                     bbox=([0, 0, 0], [2, 2, 2])).cpu().numpy()
+  assert np.array_equal(got, orc.points2octree(pb, 5, 1, bbmin=[0, 0, 0], bbmax=[2, 2, 2], **kw))
+  b = OctreeBlob(got)
+  assert list(b.nnum[:6]) == [1, 8, 16, 16, 16, 8] and list(b.nnum_nempty[:6]) == [1, 2, 2, 2, 1, 1]
+  assert b.prop("split", 4).tolist() == [1.0] + [0.0] * 7 + [2.0] + [0.0] * 7
+
+
+ADAPTIVE_CASES = [
+    dict(adaptive=True, node_dis=True, split_label=True),
+    dict(adaptive=True, node_dis=True, split_label=True, extrapolate=True),
+    dict(adaptive=True),
+    dict(node_feature=True),
+    dict(node_feature=True, node_dis=True, extrapolate=True, split_label=True),
+    dict(node_feature=True, save_pts=True, node_dis=True),
+    dict(adaptive=True, node_dis=True, key2xyz=True, extrapolate=True, split_label=True),
+]
+
+
+def smooth_cloud(rng, n, kind):
+  """Points on an ellipsoid or on a tilted plane: smooth enough for the trimming to act."""
+  if kind == 0:
+    u = rng.standard_normal((n, 3))
+    u /= np.linalg.norm(u, axis=1, keepdims=True)
+    ax = np.array([1, 0.6, 0.4])
+    pts, nrm = u * 0.8 * ax, u / ax
+  else:
+    pts = rng.uniform(-0.9, 0.9, (n, 3))
+    pts[:, 2] = 0.3 * pts[:, 0] + 0.1
+    nrm = np.tile(np.array([[-0.3, 0, 1.0]]), (n, 1))
+  nrm = nrm / np.linalg.norm(nrm, axis=1, keepdims=True)
+  return pts.astype(np.float32), nrm.astype(np.float32)
+
+
+@pytest.mark.parametrize("case", range(len(ADAPTIVE_CASES)))
+def test_adaptive_build_vs_oracle(oc, orc, case):
+  """All-depth signals, error metrics, extrapolation and trimming (octree.cpp:454-806,
+  958-1178) on the device: the blob equals the oracle's byte for byte (the oracle equals the
+  compiled reference on these very cases)."""
+  kw = ADAPTIVE_CASES[case]
+  rng = np.random.default_rng(50 + case)
+  for trial in range(5):
+    n = int(rng.integers(200, 5000))
+    pts, nrm = smooth_cloud(rng, n, trial % 2)
+    feat = rng.uniform(0, 1, (n, 2)).astype(np.float32) if trial >= 2 else None
+    lab = rng.integers(-1, 4, n).astype(np.float32) if trial >= 3 else None
+    pb = make_points_blob(pts, nrm, feat, lab)
+    depth = int(rng.integers(4, 8))
+    fd = int(rng.integers(1, 3))
+    extra = dict(adp_depth=int(rng.integers(fd + 1, depth + 1)), th_normal=float(rng.choice([0.1, 0.3, 5.0])),
+                 th_distance=float(rng.choice([0.5, 2.0, 3.0])))
+    got = oc.nn.points2octree(T(pb), depth, fd, **extra, **kw).cpu().numpy()
+    exp = orc.points2octree(pb, depth, fd, **extra, **kw)
+    assert got.size == exp.size and np.array_equal(got, exp), (trial, n, depth, fd, extra, kw)
+
+
+def test_adaptive_golden_and_config5_on_gpu(oc, synthetic, hashes):
+  """The committed hashes were written from the compiled reference: one small adaptive octree
+  and BASELINE config 5's input (16 adaptive octrees at depth 7, merged), built on the device."""
+  rng = np.random.default_rng(77)
+  pts, nrm = smooth_cloud(rng, 4000, 0)
+  pb = make_points_blob(pts, nrm)
+  assert sha(pb) == hashes["adaptive"]["input"]
+  kw = dict(node_dis=True, split_label=True, adaptive=True, adp_depth=4, th_normal=0.1, th_distance=2.0)
+  assert sha(oc.nn.points2octree(T(pb), 6, 2, **kw).cpu().numpy()) == hashes["adaptive"]["octree"]
+  blobs = [make_points_blob(*synthetic.shape_cloud(50000, 300 + i)[:2]) for i in range(16)]
+  assert sha(np.concatenate(blobs)) == hashes["cfg5"]["input"]
+  clouds = [T(b).cuda() for b in blobs]
+  assert sha(oc.nn.points2octree(clouds[0], 7, 2, **kw).cpu().numpy()) == hashes["cfg5"]["first_single"]
+  assert sha(oc.nn.points2octree_batch(clouds, 7, 2, **kw).cpu().numpy()) == hashes["cfg5"]["batch"]
 
 
 @pytest.mark.parametrize("cfg,n_clouds,n_pts,depth,seed0", [("cfg2", 32, 10000, 6, 100), ("cfg3", 16, 50000, 7, 200)])
