@@ -115,6 +115,102 @@ __device__ inline int intersect_cube(float* V, const float* pt, const float* pt_
   return nv;
 }
 
+// Ordered sums over the non-empty leaves j0 <= j < j1.  `load(j, vals)` fetches the NV values
+// of leaf j into this lane's registers.  256 leaves at a time are requested together (the
+// chain of a node high up in the tree covers the whole finest level: memory latency must not
+// be paid per leaf), the non-empty ones are packed into the wavefront's LDS block in leaf
+// order, and then lane c adds up value c leaf after leaf: the channels run side by side, each
+// in the reference's order.  Returns the number of non-empty leaves; sum[c] / last[c] get the
+// sum and the last value of channel c on every lane.
+constexpr int kPassRounds = 4, kPassValues = 8;
+template <int NV, class Load>
+__device__ inline int ordered_sums(int j0, int j1, int lane, const int* __restrict__ child_D, float* __restrict__ lds,
+    Load load, float* sum, float* last) {
+  static_assert(NV <= kPassValues, "LDS block too small");
+  int leaves = 0;
+  float acc = 0.0f, lastv = 0.0f;
+  for (int base = j0; base < j1; base += 64 * kPassRounds) {
+    float vals[kPassRounds][NV];
+    bool ok[kPassRounds];
+#pragma unroll
+    for (int u = 0; u < kPassRounds; ++u) {
+      const int j = base + u * 64 + lane;
+      ok[u] = j < j1 && child_D[j] != -1;
+    }
+#pragma unroll
+    for (int u = 0; u < kPassRounds; ++u) {
+#pragma unroll
+      for (int c = 0; c < NV; ++c) vals[u][c] = 0.0f;
+      if (ok[u]) load(base + u * 64 + lane, vals[u]);
+    }
+    int total = 0;
+#pragma unroll
+    for (int u = 0; u < kPassRounds; ++u) {
+      const uint64_t mask = __ballot(ok[u]);
+      if (ok[u]) {
+        const int p = total + __popcll(mask & ((1ull << lane) - 1));
+#pragma unroll
+        for (int c = 0; c < NV; ++c) lds[p * NV + c] = vals[u][c];
+      }
+      total += __popcll(mask);
+    }
+    __builtin_amdgcn_wave_barrier();   // same wavefront: the LDS unit keeps its accesses in order
+    if (lane < NV) {
+#pragma unroll 8
+      for (int t = 0; t < total; ++t) {
+        lastv = lds[t * NV + lane];
+        acc = __fadd_rn(acc, lastv);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+    leaves += total;
+  }
+#pragma unroll
+  for (int c = 0; c < NV; ++c) { sum[c] = read_lane(acc, c); last[c] = read_lane(lastv, c); }
+  return leaves;
+}
+// The same packing for a sum whose terms interleave the channels (the normal error): every lane
+// takes the same walk over the packed leaves, `term(vals)` gives the leaf's terms in order.
+template <int NV, class Load, class Terms>
+__device__ inline void ordered_terms(int j0, int j1, int lane, const int* __restrict__ child_D, float* __restrict__ lds,
+    Load load, Terms terms) {
+  for (int base = j0; base < j1; base += 64 * kPassRounds) {
+    float vals[kPassRounds][NV];
+    bool ok[kPassRounds];
+#pragma unroll
+    for (int u = 0; u < kPassRounds; ++u) {
+      const int j = base + u * 64 + lane;
+      ok[u] = j < j1 && child_D[j] != -1;
+    }
+#pragma unroll
+    for (int u = 0; u < kPassRounds; ++u) {
+#pragma unroll
+      for (int c = 0; c < NV; ++c) vals[u][c] = 0.0f;
+      if (ok[u]) load(base + u * 64 + lane, vals[u]);
+    }
+    int total = 0;
+#pragma unroll
+    for (int u = 0; u < kPassRounds; ++u) {
+      const uint64_t mask = __ballot(ok[u]);
+      if (ok[u]) {
+        const int p = total + __popcll(mask & ((1ull << lane) - 1));
+#pragma unroll
+        for (int c = 0; c < NV; ++c) lds[p * NV + c] = vals[u][c];
+      }
+      total += __popcll(mask);
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll 4
+    for (int t = 0; t < total; ++t) {
+      float one[NV];
+#pragma unroll
+      for (int c = 0; c < NV; ++c) one[c] = lds[t * NV + c];
+      terms(one);
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
 struct SignalArgs {
   int d, depth, n, nD, cf, ch_dis, adp_layer, calc_nerr, calc_derr;
   float imul;
@@ -126,11 +222,22 @@ struct SignalArgs {
   float *normal, *pt, *feature, *label, *dis, *nerr, *derr;   // level d (null: absent)
 };
 
-// one wavefront per node of level d
-__global__ __launch_bounds__(kBlock) void signal_kernel(SignalArgs a) {
+// One wavefront per node; every level above the finest in one launch, the root first (its
+// chain is the longest, the others run beside it).
+struct SignalLevels {
+  int first_wave[kMaxD + 1];     // of level d; [depth] = total
+  SignalArgs level[kMaxD - 1];
+};
+__global__ __launch_bounds__(kBlock) void signal_kernel(const SignalLevels* __restrict__ levels, int depth) {
   const int lane = threadIdx.x & 63;
-  const int i = (int)((blockIdx.x * (unsigned)kBlock + threadIdx.x) >> 6);
-  if (i >= a.n) return;
+  const int w = (int)((blockIdx.x * (unsigned)kBlock + threadIdx.x) >> 6);
+  if (w >= levels->first_wave[depth]) return;
+  int d = 0;
+  while (w >= levels->first_wave[d + 1]) ++d;
+  const SignalArgs& a = levels->level[d];
+  const int i = w - levels->first_wave[d];
+  __shared__ float s_pass[kBlock / 64][kPassRounds * 64 * kPassValues];
+  float* lds = s_pass[threadIdx.x >> 6];
   const int64_t n = a.n, nD = a.nD;
   const bool has_normal = a.nrm_D != nullptr, has_pt = a.pt_D != nullptr;
   if (a.child[i] == -1) {   // empty: zero signal, no label, errors "infinite"
@@ -150,25 +257,12 @@ __global__ __launch_bounds__(kBlock) void signal_kernel(SignalArgs a) {
 
   // sums of normals and points over the non-empty leaves, in leaf order
   float n_avg[3] = {0.0f, 0.0f, 0.0f}, last_n[3] = {0.0f, 0.0f, 0.0f}, pt_avg[3] = {0.0f, 0.0f, 0.0f};
-  int leaves = 0;
-  for (int base = j0; base < j1; base += 64) {
-    const int j = base + lane;
-    const bool ok = j < j1 && a.child_D[j] != -1;
-    float v[3] = {0.0f, 0.0f, 0.0f}, p[3] = {0.0f, 0.0f, 0.0f};
-    if (ok && has_normal) for (int c = 0; c < 3; ++c) v[c] = a.nrm_D[c * nD + j];
-    if (ok && has_pt) for (int c = 0; c < 3; ++c) p[c] = a.pt_D[c * nD + j];
-    uint64_t mask = __ballot(ok);
-    leaves += __popcll(mask);
-    while (mask) {
-      const int src = __ffsll((long long)mask) - 1;
-      mask &= mask - 1;
-      for (int c = 0; c < 3; ++c) {
-        last_n[c] = read_lane(v[c], src);
-        n_avg[c] = __fadd_rn(n_avg[c], last_n[c]);
-        pt_avg[c] = __fadd_rn(pt_avg[c], read_lane(p[c], src));
-      }
-    }
-  }
+  float sum6[6], last6[6];
+  const int leaves = ordered_sums<6>(j0, j1, lane, a.child_D, lds, [&](int j, float* v) {
+    if (has_normal) for (int c = 0; c < 3; ++c) v[c] = a.nrm_D[c * nD + j];
+    if (has_pt) for (int c = 0; c < 3; ++c) v[3 + c] = a.pt_D[c * nD + j];
+  }, sum6, last6);
+  for (int c = 0; c < 3; ++c) { n_avg[c] = sum6[c]; last_n[c] = last6[c]; pt_avg[c] = sum6[3 + c]; }
   if (has_normal) {
     float len = norm3(n_avg);
     if (len < 1.0e-6f) {
@@ -184,20 +278,14 @@ __global__ __launch_bounds__(kBlock) void signal_kernel(SignalArgs a) {
     for (int c = 0; c < 3; ++c) pt_avg[c] = div_rn(pt_avg[c], div);
     if (lane == 0) for (int c = 0; c < 3; ++c) a.pt[c * n + i] = pt_avg[c];
   }
-  for (int c = 0; c < a.cf; ++c) {   // features: one ordered pass per channel
-    float f_avg = 0.0f;
-    for (int base = j0; base < j1; base += 64) {
-      const int j = base + lane;
-      const bool ok = j < j1 && a.child_D[j] != -1;
-      const float v = ok ? a.feat_D[c * nD + j] : 0.0f;
-      uint64_t mask = __ballot(ok);
-      while (mask) {
-        const int src = __ffsll((long long)mask) - 1;
-        mask &= mask - 1;
-        f_avg = __fadd_rn(f_avg, read_lane(v, src));
-      }
-    }
-    if (lane == 0) a.feature[c * n + i] = div_rn(f_avg, count);
+  for (int c0 = 0; c0 < a.cf; c0 += kPassValues) {   // features: eight channels per ordered pass
+    float fsum[kPassValues], flast[kPassValues];
+    const int nc = min(kPassValues, a.cf - c0);
+    ordered_sums<kPassValues>(j0, j1, lane, a.child_D, lds, [&](int j, float* v) {
+      for (int c = 0; c < kPassValues; ++c) if (c < nc) v[c] = a.feat_D[(c0 + c) * nD + j];
+    }, fsum, flast);
+    if (lane == 0)
+      for (int c = 0; c < kPassValues; ++c) if (c < nc) a.feature[(c0 + c) * n + i] = div_rn(fsum[c], count);
   }
   if (a.label) {
     // most frequent label of the range, the smallest one on a tie: walk the distinct labels upwards
@@ -242,21 +330,14 @@ __global__ __launch_bounds__(kBlock) void signal_kernel(SignalArgs a) {
     float nm_err = 1.0e20f;
     if (a.calc_nerr && has_normal && a.d >= a.adp_layer) {
       nm_err = 0.0f;
-      for (int base = j0; base < j1; base += 64) {
-        const int j = base + lane;
-        const bool ok = j < j1 && a.child_D[j] != -1;
-        float v[3] = {0.0f, 0.0f, 0.0f};
-        if (ok) for (int c = 0; c < 3; ++c) v[c] = a.nrm_D[c * nD + j];
-        uint64_t mask = __ballot(ok);
-        while (mask) {
-          const int src = __ffsll((long long)mask) - 1;
-          mask &= mask - 1;
-          for (int c = 0; c < 3; ++c) {
-            const float tmp = __fsub_rn(read_lane(v[c], src), n_avg[c]);
-            nm_err = __fadd_rn(nm_err, __fmul_rn(tmp, tmp));
-          }
-        }
-      }
+      ordered_terms<3>(j0, j1, lane, a.child_D, lds,
+          [&](int j, float* v) { for (int c = 0; c < 3; ++c) v[c] = a.nrm_D[c * nD + j]; },
+          [&](const float* v) {
+            for (int c = 0; c < 3; ++c) {
+              const float tmp = __fsub_rn(v[c], n_avg[c]);
+              nm_err = __fadd_rn(nm_err, __fmul_rn(tmp, tmp));
+            }
+          });
       nm_err = div_rn(nm_err, count);
     }
     if (lane == 0) a.nerr[i] = nm_err;
@@ -580,6 +661,7 @@ int adaptive_finish(const AdaptiveInput& in, ocnn_alloc_fn alloc, void* alloc_ct
   const size_t o_counts = take(sizeof(int) * 64);      // [0..16] kept nodes, [17..33] kept links, [34..50] any_kept
   const size_t o_best = take(sizeof(unsigned long long) * kMaxD);
   const size_t o_hdr = take(OCNN_HEADER_BYTES);
+  const size_t o_levels = take(sizeof(SignalLevels));
   char* ws = static_cast<char*>(alloc(off, alloc_ctx));
   OCNN_REQUIRE(ws, OCNN_E_BADARG, "the allocator returned no memory for %zu bytes of scratch", off);
   OCNN_REQUIRE((reinterpret_cast<uintptr_t>(ws) & 7) == 0, OCNN_E_BADARG, "scratch not 8-byte aligned");
@@ -627,17 +709,29 @@ int adaptive_finish(const AdaptiveInput& in, ocnn_alloc_fn alloc, void* alloc_ct
   OCNN_LAUNCH_OK("cover");
   fill_kernel<<<blocks_for(o0.nnum[D]), kBlock, 0, s>>>(nerr[D], o0.nnum[D], 1.0e20f);
   fill_kernel<<<blocks_for(o0.nnum[D]), kBlock, 0, s>>>(derr[D], o0.nnum[D], 1.0e20f);
-  for (int d = D - 1; d >= 0; --d) {
-    SignalArgs a;
-    memset(&a, 0, sizeof(a));
-    a.d = d; a.depth = D; a.n = o0.nnum[d]; a.nD = o0.nnum[D]; a.cf = cf; a.ch_dis = ch_dis;
-    a.adp_layer = o0.adp_layer; a.calc_nerr = adaptive && cn; a.calc_derr = adaptive && P.node_dis && cn;
-    a.imul = imul;
-    a.key = key[d]; a.child = child[d]; a.dnum = dnum[d]; a.didx = didx[d];
-    a.child_D = child[D]; a.nrm_D = normal[D]; a.pt_D = pt[D]; a.feat_D = feature[D]; a.lab_D = label[D];
-    a.normal = normal[d]; a.pt = pt[d]; a.feature = feature[d]; a.label = label[d]; a.dis = dis[d];
-    a.nerr = nerr[d]; a.derr = derr[d];
-    signal_kernel<<<blocks_for((int64_t)a.n * 64), kBlock, 0, s>>>(a);
+  {
+    SignalLevels* L = new SignalLevels;
+    memset(L, 0, sizeof(SignalLevels));
+    int waves = 0;
+    for (int d = 0; d < D; ++d) {
+      SignalArgs& a = L->level[d];
+      a.d = d; a.depth = D; a.n = o0.nnum[d]; a.nD = o0.nnum[D]; a.cf = cf; a.ch_dis = ch_dis;
+      a.adp_layer = o0.adp_layer; a.calc_nerr = adaptive && cn; a.calc_derr = adaptive && P.node_dis && cn;
+      a.imul = imul;
+      a.key = key[d]; a.child = child[d]; a.dnum = dnum[d]; a.didx = didx[d];
+      a.child_D = child[D]; a.nrm_D = normal[D]; a.pt_D = pt[D]; a.feat_D = feature[D]; a.lab_D = label[D];
+      a.normal = normal[d]; a.pt = pt[d]; a.feature = feature[d]; a.label = label[d]; a.dis = dis[d];
+      a.nerr = nerr[d]; a.derr = derr[d];
+      L->first_wave[d] = waves;
+      waves += a.n;
+    }
+    for (int d = D; d <= kMaxD; ++d) L->first_wave[d] = waves;
+    hipError_t e = hipMemcpyAsync(ws + o_levels, L, sizeof(SignalLevels), hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);   // the table is host memory of this call
+    delete L;
+    OCNN_REQUIRE(e == hipSuccess, OCNN_E_HIP, "level table: %s", hipGetErrorString(e));
+    if (waves > 0)
+      signal_kernel<<<blocks_for((int64_t)waves * 64), kBlock, 0, s>>>(reinterpret_cast<const SignalLevels*>(ws + o_levels), D);
   }
   OCNN_LAUNCH_OK("signal");
 
