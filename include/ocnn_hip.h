@@ -293,6 +293,16 @@ int ocnn_points2octree(const void* const* points_dev, const void* const* points_
     ocnn_alloc_fn alloc, void* alloc_ctx, void* info_out, void** octree_out_dev,
     ocnn_stream_t stream);
 
+/* ---- octree_scan, pytorch/cpp/transform_octree.cpp:5-22 over ScanOctree
+ * (octree/octree/transform_octree.cpp:11-297): the part of a single octree that is visible
+ * from `n_axis` directions (`axis`: 3 floats each, host), z-buffered at `scale` pixels per
+ * finest-level cell.  Scratch memory and the result come from `alloc` (see
+ * ocnn_points2octree); one device-to-host copy (the surviving node counts) is waited for.
+ * Bit-identical to the reference's result. */
+int ocnn_octree_scan(const void* octree_dev, const void* info, const float* axis, int n_axis,
+    float scale, ocnn_alloc_fn alloc, void* alloc_ctx, void* info_out, void** octree_out_dev,
+    ocnn_stream_t stream);
+
 /* ---- octree_batch of already serialized octrees that live on the device
  * (merge_octrees, octree/octree/merge_octrees.cpp:7-198).  `out_info` (host)
  * is filled by ocnn_octree_batch_info from the n host headers; the caller

@@ -28,7 +28,7 @@ __all__ = [
     "octree_pad", "octree_depad", "octree_max_pool", "octree_max_unpool", "octree_mask_pool",
     "octree_encode_key", "octree_decode_key", "octree_xyz2key", "octree_key2xyz",
     "octree_search_key", "octree_new", "octree_grow", "octree_update", "points_new",
-    "octree_info",
+    "octree_info", "octree_scan",
 ]
 
 
@@ -222,6 +222,32 @@ def points2octree_batch(points_list, depth, full_depth=2, node_dis=False, node_f
   (the composition `collate_octrees` performs, pytorch/ocnn/transforms.py:127-148)."""
   return _build(list(points_list), True, depth, full_depth, node_dis, node_feature, split_label,
                 adaptive, adp_depth, th_normal, th_distance, extrapolate, save_pts, key2xyz)
+
+
+def octree_scan(octree, axis, scale=1.0):
+  """pytorch/cpp/transform_octree.cpp:5-22 -- the part of a single octree seen from the view
+  directions `axis` (3 floats per direction), as the completion data set makes its partial
+  scans (pytorch/projects/datasets/completion.py:9-36)."""
+  octree = _to_dev(octree)
+  info = octree_info(octree)
+  ax = np.ascontiguousarray(np.asarray(axis, dtype=np.float32).reshape(-1))
+  if ax.size == 0 or ax.size % 3:
+    raise ValueError("axis needs 3 floats per direction")
+  holder = []
+
+  def alloc(nbytes, _ctx):
+    t = torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=_dev())
+    holder.append(t)
+    return t.data_ptr()
+
+  info_raw = np.zeros(INFO_BYTES, np.uint8)
+  out_ptr = C.c_void_p()
+  _lib.call("ocnn_octree_scan", _ptr(octree), info.p, C.c_void_p(ax.ctypes.data), ax.size // 3,
+            C.c_float(scale), _ALLOC_FN(alloc), None, C.c_void_p(info_raw.ctypes.data), C.byref(out_ptr),
+            _stream())
+  out = [t for t in holder if t.data_ptr() == out_ptr.value][-1]
+  out._ocnn_info = _Info(info_raw)
+  return out
 
 
 def octree_batch(octrees):

@@ -126,7 +126,7 @@ class Checker:
       raise ValueError(prefix)
     for n in ("fetch", "points2octree", "octree_batch", "octree_sample",
               "octree_new", "octree_grow", "octree_update", "octree_set_property",
-              "normalize_points", "transform_points", "clip_points", "upgrade_key64"):
+              "normalize_points", "transform_points", "clip_points", "upgrade_key64", "octree_scan"):
       f = getattr(self.lib, prefix + "_" + n, None)
       if f is not None:
         f.restype = C.c_int64
@@ -190,6 +190,12 @@ class Checker:
     blobs = [np.ascontiguousarray(b, dtype=np.uint8) for b in blobs]
     arr = (C.c_void_p * len(blobs))(*[b.ctypes.data for b in blobs])
     return self._fetch(self.fn("octree_batch")(arr, len(blobs)))
+
+  def octree_scan(self, blob, axis, scale=1.0):
+    b = np.ascontiguousarray(blob, dtype=np.uint8)
+    ax = np.ascontiguousarray(axis, dtype=np.float32).reshape(-1)
+    assert ax.size % 3 == 0
+    return self._fetch(self.fn("octree_scan")(_p(b), _p(ax), ax.size // 3, C.c_float(scale)))
 
   def upgrade_key64(self, blob32):
     b = np.ascontiguousarray(blob32, dtype=np.uint8)

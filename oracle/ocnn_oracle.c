@@ -1751,3 +1751,161 @@ int64_t orc_octree_set_property(const void* in, const float* data, int64_t count
   memcpy(prop_ptr(out, kFeature, depth), data, sizeof(float) * (size_t)count);
   return sz;
 }
+
+
+/* ------------------------------------------------------------------------ */
+/* octree_scan: ScanOctree, octree/octree/transform_octree.cpp:11-297, driven as
+ * pytorch/cpp/transform_octree.cpp:5-22 does.  `axis` holds n_axis view directions
+ * (3 floats each); a finest-level node is kept iff it is non-empty, faces one of the
+ * views and is the nearest node of its pixel in that view's z-buffer.  Pinned against
+ * the compiled reference (tests/test_oracle_scan.py). */
+static float dot3(const float* a, const float* b) { return a[0] * b[0] + a[1] * b[1] + a[2] * b[2]; }
+static void rotation_from_axes(float* rot, const float* axis0, const float* axis1) { /* math_functions.cpp:130-173 */
+  float angle = dot3(axis0, axis1);
+  if (angle < -1) angle = -1;
+  if (angle > 1) angle = 1;
+  angle = (float)acos((double)angle);
+  float axis[3];
+  axis[0] = axis0[1] * axis1[2] - axis0[2] * axis1[1];
+  axis[1] = axis0[2] * axis1[0] - axis0[0] * axis1[2];
+  axis[2] = axis0[0] * axis1[1] - axis0[1] * axis1[0];
+  float ilen = (float)(1.0 / ((double)norm2f(axis, 3) + 1.0e-10));
+  for (int i = 0; i < 3; ++i) axis[i] *= ilen;
+  float cosa = ORC_COS(angle), cosa1 = 1 - cosa, sina = ORC_SIN(angle);
+  rot[0] = cosa + axis[0] * axis[0] * cosa1;
+  rot[1] = axis[0] * axis[1] * cosa1 + axis[2] * sina;
+  rot[2] = axis[0] * axis[2] * cosa1 - axis[1] * sina;
+  rot[3] = axis[0] * axis[1] * cosa1 - axis[2] * sina;
+  rot[4] = cosa + axis[1] * axis[1] * cosa1;
+  rot[5] = axis[1] * axis[2] * cosa1 + axis[0] * sina;
+  rot[6] = axis[0] * axis[2] * cosa1 + axis[1] * sina;
+  rot[7] = axis[1] * axis[2] * cosa1 - axis[0] * sina;
+  rot[8] = cosa + axis[2] * axis[2] * cosa1;
+}
+/* the view frame and the pixel grid of one direction: set_axis + bbox_xy, transform_octree.cpp:13-92 */
+void orc_scan_frame(float* frame /* x[3] y[3] z[3] bbmin[3] */, int* width, const float* z, int depth, float scale_) {
+  float rot[9], z0[3] = { 0, 0, 1 };
+  rotation_from_axes(rot, z0, z);
+  float* x_ = frame; float* y_ = frame + 3; float* z_ = frame + 6; float* bbmin = frame + 9;
+  for (int i = 0; i < 3; ++i) { x_[i] = rot[i]; y_[i] = rot[3 + i]; z_[i] = z[i]; }
+  float bbmax[3];
+  for (int i = 0; i < 3; ++i) { bbmin[i] = FLT_MAX; bbmax[i] = -FLT_MAX; }
+  for (int i = 0; i < 8; ++i) {
+    float pt[3] = { (float)(i / 4), (float)((i / 2) % 2), (float)(i % 2) };
+    float x = dot3(pt, x_), y = dot3(pt, y_), zz = dot3(pt, z_);
+    if (x < bbmin[0]) bbmin[0] = x;
+    if (x > bbmax[0]) bbmax[0] = x;
+    if (y < bbmin[1]) bbmin[1] = y;
+    if (y > bbmax[1]) bbmax[1] = y;
+    if (zz < bbmin[2]) bbmin[2] = zz;
+    if (zz > bbmax[2]) bbmax[2] = zz;
+  }
+  float wmax = -1, scale = (float)(1 << depth);
+  for (int i = 0; i < 3; ++i) {
+    bbmax[i] *= scale; bbmin[i] *= scale;
+    float dis = bbmax[i] - bbmin[i];
+    if (dis > wmax) wmax = dis;
+  }
+  *width = (int)(wmax * scale_) + 2;
+}
+int64_t orc_octree_scan(const void* blob, const float* axis, int n_axis, float scale_) {
+  const OInfo* oi = (const OInfo*)blob;
+  const int depth = oi->depth, full = oi->full_layer;
+  if (oi->batch_size != 1 || channel_of(oi, kKey) != 1) return ORC_E_UNSUPPORTED;
+  const int num = oi->nnum[depth];
+  unsigned char* drop[17];
+  for (int d = 0; d <= depth; ++d) { drop[d] = (unsigned char*)malloc((size_t)oi->nnum[d] + 1); memset(drop[d], 1, (size_t)oi->nnum[d] + 1); }
+  const uint64_t* key_D = (const uint64_t*)prop_ptr(blob, kKey, depth);
+  const int* child_D = (const int*)prop_ptr(blob, kChild, depth);
+  const int fch = channel_of(oi, kFeature), floc = location_of(oi, kFeature);
+  const float* feat_D = has_prop(oi, kFeature) ? (const float*)prop_ptr(blob, kFeature, depth) : NULL;
+  const int normal_ok = feat_D && (floc == -1 || floc == depth) && fch >= 3;
+  for (int a = 0; a < n_axis; ++a) {
+    float frame[12]; int width;
+    orc_scan_frame(frame, &width, axis + 3 * a, depth, scale_);
+    const float* x_ = frame; const float* y_ = frame + 3; const float* z_ = frame + 6; const float* bbmin = frame + 9;
+    int* id_buffer = (int*)malloc(sizeof(int) * (size_t)width * width);
+    float* z_buffer = (float*)malloc(sizeof(float) * (size_t)width * width);
+    unsigned char* flags = (unsigned char*)malloc((size_t)num + 1);
+    memset(flags, 1, (size_t)num + 1);
+    for (int i = 0; i < width * width; ++i) { id_buffer[i] = -1; z_buffer[i] = FLT_MAX; }
+    for (int i = 0; i < num; ++i) { /* z_buffer, transform_octree.cpp:99-138 */
+      if (child_D[i] < 0) continue;
+      float normal[3] = { 0, 0, 0 };
+      if (normal_ok) for (int c = 0; c < 3; ++c) normal[c] = feat_D[(int64_t)c * num + i];
+      if (dot3(normal, z_) >= 0) continue;
+      float pt[3];
+      key2xyz_f(pt, key_D[i], depth, oi->key2xyz);
+      float x = (dot3(x_, pt) - bbmin[0]) * scale_;
+      float y = (dot3(y_, pt) - bbmin[1]) * scale_;
+      float z = dot3(z_, pt);
+      int k = (int)(x + 0.5f) * width + (int)(y + 0.5f);
+      if (z_buffer[k] > z) {
+        z_buffer[k] = z;
+        if (id_buffer[k] >= 0) flags[id_buffer[k]] = 1;
+        id_buffer[k] = i;
+        flags[i] = 0;
+      }
+    }
+    for (int j = 0; j < num; ++j) if (flags[j] == 0) drop[depth][j] = 0;
+    free(id_buffer); free(z_buffer); free(flags);
+  }
+  /* generate_flags, transform_octree.cpp:140-170 */
+  for (int d = 0; d < full; ++d) memset(drop[d], 0, (size_t)oi->nnum[d]);
+  for (int d = depth - 1; d >= full; --d) {
+    const int* child_d = (const int*)prop_ptr(blob, kChild, d);
+    for (int i = 0; i < oi->nnum[d]; ++i) {
+      int j = child_d[i], dr = 1;
+      if (j < 0) continue;
+      for (int k = j * 8; k < j * 8 + 8; ++k) if (drop[d + 1][k] == 0) { dr = 0; break; }
+      drop[d][i] = (unsigned char)dr;
+    }
+  }
+  /* trim_octree, transform_octree.cpp:172-297 */
+  OInfo o = *oi;
+  int nne[17] = { 0 }, nn[17] = { 0 };
+  for (int d = 0; d < full; ++d) nne[d] = 1 << (3 * d);
+  for (int d = full; d <= depth; ++d) { int c = 0; for (int i = 0; i < oi->nnum[d]; ++i) if (drop[d][i] == 0) c++; nne[d] = c; }
+  nn[0] = 1;
+  for (int d = 1; d <= depth; ++d) nn[d] = 8 * nne[d - 1];
+  for (int d = 0; d <= depth; ++d) { o.nnum[d] = nn[d]; o.nnum_nempty[d] = nne[d]; }
+  set_nnum_cum(&o, 0);
+  set_ptr_dis(&o);
+  const int sz = sizeof_octree(&o);
+  char* out = result_alloc(sz);
+  if (!out) return ORC_E_NOMEM;
+  memset(out, 0, (size_t)sz);
+  memcpy(out, &o, sizeof(o));
+  const int lloc = location_of(oi, kLabel), lch = channel_of(oi, kLabel);
+  const int sloc = location_of(oi, kSplit), sch = channel_of(oi, kSplit);
+  for (int d = 1; d <= depth; ++d) {
+    const int num_p = oi->nnum[d - 1];
+    const unsigned char* drop_p = drop[d - 1]; const unsigned char* drop_d = drop[d];
+    const int* child_in = (const int*)prop_ptr(blob, kChild, d - 1);
+    const uint64_t* key_in = (const uint64_t*)prop_ptr(blob, kKey, d);
+    int* child_out = (int*)prop_ptr(out, kChild, d);
+    uint64_t* key_out = (uint64_t*)prop_ptr(out, kKey, d);
+    const int nnum_in = oi->nnum[d], nnum_out = o.nnum[d];
+    const float* f_in = (fch && (floc == -1 || d == depth)) ? (const float*)prop_ptr(blob, kFeature, d) : NULL;
+    float* f_out = f_in ? (float*)prop_ptr(out, kFeature, d) : NULL;
+    const float* l_in = (lch && (lloc == -1 || d == depth)) ? (const float*)prop_ptr(blob, kLabel, d) : NULL;
+    float* l_out = l_in ? (float*)prop_ptr(out, kLabel, d) : NULL;
+    const float* s_in = (sch && (sloc == -1 || d == depth)) ? (const float*)prop_ptr(blob, kSplit, d) : NULL;
+    float* s_out = s_in ? (float*)prop_ptr(out, kSplit, d) : NULL;
+    int j = 0, id = 0;
+    for (int i = 0; i < num_p; ++i) {
+      if (drop_p[i] == 1) continue;
+      const int t = child_in[i];
+      for (int k = 8 * t; k < 8 * t + 8; ++k) {
+        key_out[j] = key_in[k];
+        child_out[j] = drop_d[k] == 0 ? id++ : -1;
+        if (f_out) for (int c = 0; c < fch; ++c) f_out[(int64_t)c * nnum_out + j] = drop_d[k] == 0 ? f_in[(int64_t)c * nnum_in + k] : 0;
+        if (l_out) l_out[j] = drop_d[k] == 0 ? l_in[k] : -1;
+        if (s_out) s_out[j] = drop_d[k] == 0 ? s_in[k] : 0;
+        j++;
+      }
+    }
+  }
+  for (int d = 0; d <= depth; ++d) free(drop[d]);
+  return sz;
+}

@@ -78,6 +78,17 @@ int64_t ref_octree_sample(const char* name) {
 }
 
 // octree/octree/transform_octree.cpp:433-497: 32-bit-key blob ("_OCTREE_1.0_") -> 64-bit keys
+// pytorch/cpp/transform_octree.cpp:5-22
+int64_t ref_octree_scan(const void* blob, const float* axis, int n_axis, float scale) {
+  OctreeParser parser;
+  parser.set_cpu(blob);
+  ScanOctree scan_octree(scale);
+  std::vector<float> ax(axis, axis + 3 * n_axis);
+  std::vector<char> out;
+  scan_octree.scan(out, parser, ax);
+  return keep(out);
+}
+
 int64_t ref_upgrade_key64(const void* blob32, int64_t bytes) {
   std::vector<char> in((const char*)blob32, (const char*)blob32 + bytes), out;
   upgrade_key64(out, in);
