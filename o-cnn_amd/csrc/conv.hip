@@ -521,7 +521,8 @@ __global__ void pack_weights_lds_f32(float* __restrict__ Wt, const float* __rest
 //   LDS W [9 taps][MT][64 lanes] x 16 B                        = 18 KiB (MT = 2)
 // 50 KiB per workgroup: three workgroups per CU.  Unit index of slot (x,y,z):
 //   (x&1) | (y&1)<<1 | (z&1)<<2 | (y>>1)<<3 | (z>>1)<<4
-// so the 8 siblings of a group (consecutive lanes) always read 8 different 16-byte units.
+// so the 8 siblings of a group (consecutive lanes) always read 8 different 16-byte units;
+// odd groups store unit u at u ^ 8 (see the kernel).
 constexpr int kB16Half = 32 * 32;  // 16-byte units per 8-channel half
 
 __device__ inline int b16_unit(int x, int y, int z) {
@@ -604,6 +605,10 @@ __global__ __launch_bounds__(256, 2) void conv_s1_bf16_lds_kernel(ConvArgs a, ui
   int cbase[2];
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) cbase[nt] = kh * kB16Half + (wave * 8 + nt * 4 + (r >> 3)) * 32;
+  // Odd groups keep their units with bit 3 flipped: a 16-byte LDS read is served sixteen lanes
+  // (two sibling groups) at a time, and the blocks of two groups, 512 bytes apart, would meet in
+  // the same banks.
+  const int gswz = ((r >> 3) & 1) << 3;
 
   for (int pass = 0; pass < npass; ++pass) {
     floatx16 acc[MT][2];
@@ -645,7 +650,7 @@ __global__ __launch_bounds__(256, 2) void conv_s1_bf16_lds_kernel(ConvArgs a, ui
         }                                                                                      \
       }                                                                                        \
       _Pragma("unroll") for (int j = 0; j < 4; ++j)                                            \
-        sX[s_kh * kB16Half + (wave * 8 + 2 * j + s_g) * 32 + b16_unit(L, s_y, s_z)] = xr[(L) & 1][j]; \
+        sX[s_kh * kB16Half + (wave * 8 + 2 * j + s_g) * 32 + (b16_unit(L, s_y, s_z) ^ (s_g << 3))] = xr[(L) & 1][j]; \
       __syncthreads();                                                                         \
       /* weights of the next computing phase: phase L requests those of dx = L */            \
       if ((L) <= 2) OCNN_FETCH_W(SLAB, L);                                                     \
@@ -657,7 +662,7 @@ __global__ __launch_bounds__(256, 2) void conv_s1_bf16_lds_kernel(ConvArgs a, ui
         _Pragma("unroll") for (int dy = 0; dy < 3; ++dy)                                       \
         _Pragma("unroll") for (int dz = 0; dz < 3; ++dz) {                                     \
           const int y = dy + sj, z = dz + sk;                                                  \
-          const int unit = ux | ((y & 1) << 1) | ((z & 1) << 2) | ((y >> 1) << 3) | ((z >> 1) << 4); \
+          const int unit = (ux | ((y & 1) << 1) | ((z & 1) << 2) | ((y >> 1) << 3) | ((z >> 1) << 4)) ^ gswz; \
           union { u32x4 q; bf16x8 v; } b0, b1;                                                 \
           b0.q = sX[cbase[0] + unit];                                                          \
           b1.q = sX[cbase[1] + unit];                                                          \
