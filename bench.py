@@ -45,6 +45,9 @@ def main():
   ap.add_argument("--warmup", type=int, default=3)
   ap.add_argument("--quick", action="store_true", help="skip the sub-measurements and the CPU baseline")
   ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+  ap.add_argument("--build-only", action="store_true",
+                  help="run only the octree construction of the scene (12 builds) and print its time: "
+                       "the workload of the per-kernel rocprof summary of the build")
   ap.add_argument("--calib", action="store_true",
                   help="also run a plain device copy of 1 GiB three times (the known-size kernel "
                        "that scales the FETCH_SIZE / WRITE_SIZE counters of a --pmc run)")
@@ -86,6 +89,17 @@ def main():
   info = F.octree_info(octree)
   depth = 9
   H9, H8, Hne9, Hne8 = info.nnum(9), info.nnum(8), info.nnum_nempty(9), info.nnum_nempty(8)
+
+  if args.build_only:
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(12):
+      F.points2octree_batch([scene_pts], 9, 2)
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / 12
+    print(json.dumps({"metric": "points2octree + octree_batch, depth-9 scene", "ms": t * 1e3,
+                      "Mpts_per_s": 0.25 / t, "octants_d9": H9}))
+    return
 
   C = 64
   g = torch.Generator(device="cpu").manual_seed(2)

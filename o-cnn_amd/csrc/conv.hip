@@ -75,6 +75,15 @@ __device__ inline int xcd_tile(int bid, int n_tiles) {
   return (bid % kXcd) * per + bid / kXcd;
 }
 
+// A level with few column tiles cannot fill the device by tiles alone: the passes over the
+// output channels (independent of one another) are then dealt out over blockIdx.y.
+inline int pass_split(int n_tiles, int npass) {
+  constexpr int kWanted = 768;   // workgroups that keep 256 CUs busy with two or three each
+  if (n_tiles >= kWanted || npass <= 1) return 1;
+  const int p = (kWanted + n_tiles - 1) / n_tiles;
+  return p < npass ? p : npass;
+}
+
 // ---- main kernels ----------------------------------------------------------------
 // Accumulator layout of the 32x32 MFMA: lane l, register i holds
 // D[row = 8*(i/4) + 4*(l>>5) + (i%4)][col = l&31].
@@ -148,7 +157,7 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
   const int npass = (a.mtiles + MT - 1) / MT;
   const int cpad4 = cpad >> 2;
   const int nstage = a.K * nslab;
-  for (int pass = 0; pass < npass; ++pass) {
+  for (int pass = blockIdx.y; pass < npass; pass += gridDim.y) {  // passes may be dealt out over workgroups
     floatx16 acc[MT][2];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -259,7 +268,7 @@ __global__ __launch_bounds__(256) void conv_rows_bf16_kernel(ConvArgs a, uint16_
   const int npass = (a.mtiles + MT - 1) / MT;
   const int cpad8 = cpad >> 3;
   const int nstage = a.K * nslab;
-  for (int pass = 0; pass < npass; ++pass) {
+  for (int pass = blockIdx.y; pass < npass; pass += gridDim.y) {  // passes may be dealt out over workgroups
     floatx16 acc[MT][2];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -413,7 +422,7 @@ __global__ __launch_bounds__(256, 2) void conv_s1_f32_lds_kernel(ConvArgs a, flo
   for (int nt = 0; nt < 2; ++nt)
     boff[nt] = group_base(wave * 8 + nt * 4 + (r >> 3)) + sibling_slot(r & 7) + kh * kPlane;
 
-  for (int pass = 0; pass < npass; ++pass) {
+  for (int pass = blockIdx.y; pass < npass; pass += gridDim.y) {  // passes may be dealt out over workgroups
     floatx16 acc[MT][2];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -610,7 +619,7 @@ __global__ __launch_bounds__(256, 2) void conv_s1_bf16_lds_kernel(ConvArgs a, ui
   // the same banks.
   const int gswz = ((r >> 3) & 1) << 3;
 
-  for (int pass = 0; pass < npass; ++pass) {
+  for (int pass = blockIdx.y; pass < npass; pass += gridDim.y) {  // passes may be dealt out over workgroups
     floatx16 acc[MT][2];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -1023,7 +1032,7 @@ __global__ __launch_bounds__(256) void deconv_s2_bf16_kernel(ConvArgs a, uint16_
   int ncol[2];
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) ncol[nt] = n0 + nt * 32 + r;
-  for (int pass = 0; pass < npass; ++pass) {
+  for (int pass = blockIdx.y; pass < npass; pass += gridDim.y) {  // passes may be dealt out over workgroups
     floatx16 acc[kD2MT][2];
 #pragma unroll
     for (int mt = 0; mt < kD2MT; ++mt)
@@ -1273,7 +1282,7 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
       uint16_t* xt = reinterpret_cast<uint16_t*>(wsb + p.wt_bytes + p.ichild_bytes);
       dim3 tgrid((a.Hin + 1 + 127) / 128, (cpad + 63) / 64);
       transpose_rows_bf16_kernel<<<tgrid, 256, 0, s>>>(xt, (const uint16_t*)btm, a.Cin, a.Hin, cpad);
-      deconv_s2_bf16_kernel<<<d_grid, 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles, cpad / 8);
+      deconv_s2_bf16_kernel<<<dim3(d_grid, pass_split(d_tiles, (d.M * 8 + 32 * kD2MT - 1) / (32 * kD2MT))), 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles, cpad / 8);
     }
   } else if (dtype == OCNN_F32 && a.mode == kModeS1 && !a.nempty && a.K == 27) {
     const int MT = a.mtiles == 1 ? 1 : 2;
@@ -1283,9 +1292,9 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
         MT, npass, nslab, sm, sc);
     OCNN_LAUNCH_OK("pack_weights_lds");
     if (MT == 1)
-      conv_s1_f32_lds_kernel<1, 27><<<grid, 256, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
+      conv_s1_f32_lds_kernel<1, 27><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
     else
-      conv_s1_f32_lds_kernel<2, 27><<<grid, 256, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
+      conv_s1_f32_lds_kernel<2, 27><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
   } else if (dtype == OCNN_F32) {
     const int MT = a.mtiles == 1 ? 1 : 2;
     const int cpad = (a.Cin + 7) / 8 * 8;
@@ -1299,9 +1308,9 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     transpose_rows_f32_kernel<<<tg, 256, 0, s>>>(xt, (const float*)btm, a.Cin, a.Hin, cpad);
     OCNN_LAUNCH_OK("transpose_rows");
     if (MT == 1)
-      conv_rows_f32_kernel<1><<<grid, 256, 0, s>>>(a, (float*)top, (const float4*)xt, (const float*)wsb, n_tiles, cpad);
+      conv_rows_f32_kernel<1><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (float*)top, (const float4*)xt, (const float*)wsb, n_tiles, cpad);
     else
-      conv_rows_f32_kernel<2><<<grid, 256, 0, s>>>(a, (float*)top, (const float4*)xt, (const float*)wsb, n_tiles, cpad);
+      conv_rows_f32_kernel<2><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (float*)top, (const float4*)xt, (const float*)wsb, n_tiles, cpad);
   } else if (a.mode == kModeS1 && !a.nempty && a.K == 27) {
     const int MT = a.mtiles == 1 ? 1 : 2;
     const int cpad = (a.Cin + 15) / 16 * 16;
@@ -1315,9 +1324,9 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     OCNN_LAUNCH_OK("pack/transpose");
     // the kernel walks geometric offsets in natural order (the packer mirrored the weights)
     if (MT == 1)
-      conv_s1_bf16_lds_kernel<1><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad / 8);
+      conv_s1_bf16_lds_kernel<1><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad / 8);
     else
-      conv_s1_bf16_lds_kernel<2><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad / 8);
+      conv_s1_bf16_lds_kernel<2><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad / 8);
   } else {
     const int MT = a.mtiles == 1 ? 1 : 2;
     const int cpad = (a.Cin + 15) / 16 * 16;
@@ -1331,9 +1340,9 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     transpose_rows_bf16_kernel<<<tg, 256, 0, s>>>(xt, (const uint16_t*)btm, a.Cin, a.Hin, cpad);
     OCNN_LAUNCH_OK("transpose_rows");
     if (MT == 1)
-      conv_rows_bf16_kernel<1><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
+      conv_rows_bf16_kernel<1><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
     else
-      conv_rows_bf16_kernel<2><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
+      conv_rows_bf16_kernel<2><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
   }
   OCNN_LAUNCH_OK("octree_conv");
   return OCNN_OK;
