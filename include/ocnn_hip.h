@@ -91,7 +91,13 @@ int ocnn_pad_backward(void* X, int Hx, int C, const void* Y, int Hy, const int* 
 int ocnn_make_ichild(int* ichild, int n_nempty, const int* child, int n_node, ocnn_stream_t stream);
 
 /* ---- octree2col / col2octree: octree/octree/octree_nn.h:80-120, octree_nn.cu:110-253.
- * Same argument meaning as the reference; `kernel_size` (host) replaces `ni`. */
+ * Same argument meaning as the reference; `kernel_size` (host) replaces `ni`.
+ * col2octree sets the rows of `data` on chunk n == 0 and adds to them on later chunks.
+ * For the neighbour table of an octree it sums each row's taps in ascending tap order
+ * (no atomics, same result on every run); the call first checks on the device that the
+ * table maps back and forth consistently and otherwise scatter-adds as the reference
+ * does, so any table gives the reference's result.  col2octreeP with stride 2 and a null
+ * `ichild` always scatter-adds. */
 int ocnn_octree2col(void* col, const void* data, int channel, int height, const int* kernel_size,
     int stride, const int* neigh, int height_col, int n, int dtype, ocnn_stream_t stream);
 int ocnn_col2octree(const void* col, void* data, int channel, int height, const int* kernel_size,

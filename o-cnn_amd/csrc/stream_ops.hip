@@ -8,6 +8,9 @@
 // of channels.
 #include "ocnn_common.h"
 
+#include <algorithm>
+#include <atomic>
+
 namespace ocnn {
 namespace {
 
@@ -64,53 +67,272 @@ __global__ void make_ichild_kernel(int* __restrict__ ichild, int n_nempty,
 // ---- octree2col / col2octree -------------------------------------------------
 struct ColArgs {
   int channel, height, octree_h, K, stride, height_col, n;
-  int slot[27];  // neighbour slot of each tap for sibling 0
+  int slot[27];   // neighbour slot of each tap for sibling 0
+  int rslot[27];  // slot of the opposite offset (the tap seen from the neighbour's side)
 };
 
 // neighbour row of column h for tap k, -1 when absent.  P = non-empty variant.
 template <bool P>
-__device__ inline int col_source(const ColArgs& a, int h, int k, const int* __restrict__ neigh,
-    const int* __restrict__ child, const int* __restrict__ ichild) {
-  int64_t index;
-  if (a.stride == 2) {
-    index = ((int64_t)h << 6) + a.slot[k];
-  } else {
-    int hp = P ? ichild[h] : h;
-    index = ((int64_t)(hp >> 3) << 6) + sibling_slot(hp & 7) + a.slot[k];
-  }
-  int p = neigh[index];
-  if (P && p >= 0) p = child[p];
-  return p;
+__device__ inline int64_t col_base(const ColArgs& a, int h, const int* __restrict__ ichild) {
+  if (a.stride == 2) return (int64_t)h << 6;
+  int hp = P ? ichild[h] : h;
+  return ((int64_t)(hp >> 3) << 6) + sibling_slot(hp & 7);
 }
+template <bool P>
+__device__ inline int col_source(const ColArgs& a, int64_t base, int k, const int* __restrict__ neigh,
+    const int* __restrict__ child) {
+  int p = neigh[base + a.slot[k]];
+  if (P && p >= 0) p = child[p];
+  return (p >= 0 && p < a.octree_h) ? p : -1;
+}
+
+// column whose tap k reads row p, -1 when there is none: the neighbour of p at the
+// opposite offset (a stride-2 column is a sibling group, named by its first node).
+// Equal to the inverse of col_source whenever the table is a neighbour table of an
+// octree, which col_check_kernel verifies.
+template <bool P>
+__device__ inline int col_target(const ColArgs& a, int p, int k, const int* __restrict__ neigh,
+    const int* __restrict__ child, const int* __restrict__ ichild) {
+  int pp = P ? ichild[p] : p;
+  int q = neigh[((int64_t)(pp >> 3) << 6) + sibling_slot(pp & 7) + a.rslot[k]];
+  if (q < 0) return -1;
+  int h;
+  if (a.stride == 2) {
+    if (q & 7) return -1;
+    h = q >> 3;
+  } else {
+    h = P ? child[q] : q;
+  }
+  return (h >= 0 && h < a.height) ? h : -1;
+}
+
+// A workgroup covers kColTile columns.  The rows of col are height_col elements apart,
+// so a row starts anywhere inside a 256-byte line, and a wavefront storing 64
+// consecutive elements that straddle a line boundary costs almost twice one that
+// does not.  Each row (channel, tap) is therefore shifted by its own 0..63 columns so
+// that its stores are aligned; the neighbour rows of the tile plus a 64-column apron
+// are staged in LDS per tap, where every row finds them under its own shift.
+constexpr int kColTile = 256, kColApron = 64;
 
 template <typename T, bool P>
-__global__ void octree2col_kernel(T* __restrict__ col, const T* __restrict__ data, ColArgs a,
-    const int* __restrict__ neigh, const int* __restrict__ child, const int* __restrict__ ichild) {
-  int hl = blockIdx.x * blockDim.x + threadIdx.x;  // column inside the chunk
-  if (hl >= a.height_col) return;
-  int k = blockIdx.y;
-  int h = a.n * a.height_col + hl;
-  int p = h < a.height ? col_source<P>(a, h, k, neigh, child, ichild) : -1;
-  int c0 = blockIdx.z * kChanChunk, c1 = min(a.channel, c0 + kChanChunk);
-  for (int c = c0; c < c1; ++c)
-    col[((int64_t)c * a.K + k) * a.height_col + hl] =
-        (p < 0 || p >= a.octree_h) ? zero_of<T>() : data[(int64_t)c * a.octree_h + p];
+__global__ void __launch_bounds__(kColTile) octree2col_kernel(T* __restrict__ col,
+    const T* __restrict__ data, ColArgs a, const int* __restrict__ neigh,
+    const int* __restrict__ child, const int* __restrict__ ichild) {
+  __shared__ int s_src[2][kColTile + kColApron];
+  const int tid = threadIdx.x;
+  const int first = blockIdx.x * kColTile - kColApron;  // column staged at s_src[.][0]
+  const int lo = a.n * a.height_col;
+  // staged columns of this thread: first + tid, and first + kColTile + tid for tid < kColApron
+  int hl0 = first + tid, hl1 = first + kColTile + tid;
+  bool live0 = hl0 >= 0 && hl0 < a.height_col && lo + hl0 < a.height;
+  bool live1 = tid < kColApron && hl1 < a.height_col && lo + hl1 < a.height;
+  int64_t base0 = live0 ? col_base<P>(a, lo + hl0, ichild) : 0;
+  int64_t base1 = live1 ? col_base<P>(a, lo + hl1, ichild) : 0;
+  const int c0 = blockIdx.y * kChanChunk, c1 = min(a.channel, c0 + kChanChunk);
+  const uint64_t col_elem = reinterpret_cast<uintptr_t>(col) / sizeof(T);
+  // Tap k + 1 is looked up and its values are loaded before tap k is stored, so the
+  // loads of one tap fly while the stores of the previous one drain.
+  T v[kChanChunk], vn[kChanChunk];
+  int64_t at[kChanChunk], atn[kChanChunk];
+  auto stage = [&](int k) {
+    int* src = s_src[k & 1];
+    src[tid] = live0 ? col_source<P>(a, base0, k, neigh, child) : -1;
+    if (tid < kColApron) src[kColTile + tid] = live1 ? col_source<P>(a, base1, k, neigh, child) : -1;
+  };
+  auto load = [&](int k, T* val, int64_t* where) {
+    const int* src = s_src[k & 1];
+#pragma unroll
+    for (int j = 0; j < kChanChunk; ++j) {
+      int c = c0 + j;
+      int64_t row = ((int64_t)c * a.K + k) * a.height_col;
+      int shift = (int)((col_elem + (uint64_t)row) & (kColApron - 1));
+      int hl = first + kColApron + tid - shift;
+      bool ok = c < c1 && hl >= 0 && hl < a.height_col;
+      where[j] = ok ? row + hl : -1;
+      int p = ok ? src[kColApron + tid - shift] : -1;
+      val[j] = p < 0 ? zero_of<T>() : data[(int64_t)c * a.octree_h + p];
+    }
+  };
+  stage(0);
+  __syncthreads();
+  load(0, v, at);
+  for (int k = 0; k < a.K; ++k) {
+    if (k + 1 < a.K) stage(k + 1);
+    __syncthreads();  // one barrier per tap: the buffer written here was last read two taps ago
+    if (k + 1 < a.K) load(k + 1, vn, atn);
+#pragma unroll
+    for (int j = 0; j < kChanChunk; ++j)
+      if (at[j] >= 0) col[at[j]] = v[j];
+#pragma unroll
+    for (int j = 0; j < kChanChunk; ++j) { v[j] = vn[j]; at[j] = atn[j]; }
+  }
 }
 
+// Stride 1 over all nodes: the 27 taps of the 8 columns of a sibling group all lie in
+// the group's 64-entry block, so a workgroup gathers each block of its tile once per
+// channel (64 reads per group instead of 8 x 27) into LDS and serves every tap from
+// there, with the same per-row shift for aligned stores.  Entry s of staged group g
+// sits at g * 64 + (s ^ spread(g)), spread() moving the low bits of g to bits 1, 3, 5:
+// the 8 columns of a group differ in bits 0, 2, 4 of s, so a wavefront's 64 reads hit
+// 64 different banks.
+constexpr int kStageGroups = (kColTile + kColApron) / 8 + 1;  // + 1: a chunk may start inside a group
+constexpr int kStageSlots = kStageGroups * 64;
+constexpr int kStagePerThread = (kStageSlots + kColTile - 1) / kColTile;
+
+__device__ inline int stage_index(int g, int s) {
+  return g * 64 + (s ^ (((g & 1) << 1) | ((g & 2) << 2) | ((g & 4) << 3)));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kColTile) octree2col_block_kernel(T* __restrict__ col,
+    const T* __restrict__ data, ColArgs a, const int* __restrict__ neigh) {
+  __shared__ T s_val[2][kStageSlots];
+  const int tid = threadIdx.x;
+  const int lo = a.n * a.height_col;
+  const int first = blockIdx.x * kColTile - kColApron;  // first column the tile may store
+  const int g0 = (lo + first) >> 3;                      // first staged group (may be negative)
+  int src[kStagePerThread];  // rows behind this thread's staged entries, the same for every channel
+#pragma unroll
+  for (int j = 0; j < kStagePerThread; ++j) {
+    int i = tid + j * kColTile, g = g0 + (i >> 6);
+    int p = -1;
+    if (i < kStageSlots && g >= 0 && (int64_t)g * 8 < a.height) p = neigh[((int64_t)g << 6) + (i & 63)];
+    src[j] = (p >= 0 && p < a.octree_h) ? p : -1;
+  }
+  const uint64_t col_elem = reinterpret_cast<uintptr_t>(col) / sizeof(T);
+  // The rows of the next channel are gathered into registers while the taps of this
+  // one are stored.
+  T next[kStagePerThread];
+  auto gather = [&](int c) {
+    const T* row_in = data + (int64_t)c * a.octree_h;
+#pragma unroll
+    for (int j = 0; j < kStagePerThread; ++j) next[j] = src[j] < 0 ? zero_of<T>() : row_in[src[j]];
+  };
+  if ((int)blockIdx.y < a.channel) gather(blockIdx.y);
+  int turn = 0;
+  for (int c = blockIdx.y; c < a.channel; c += gridDim.y, turn ^= 1) {  // few tiles: channels dealt out
+    T* val = s_val[turn];
+#pragma unroll
+    for (int j = 0; j < kStagePerThread; ++j) {
+      int i = tid + j * kColTile;
+      if (i < kStageSlots) val[stage_index(i >> 6, i & 63)] = next[j];
+    }
+    __syncthreads();  // one barrier per channel: the other buffer is still being read
+    if (c + (int)gridDim.y < a.channel) gather(c + gridDim.y);
+#pragma unroll 9
+    for (int k = 0; k < a.K; ++k) {
+      int64_t row = ((int64_t)c * a.K + k) * a.height_col;
+      int shift = (int)((col_elem + (uint64_t)row) & (kColApron - 1));
+      int hl = first + kColApron + tid - shift;
+      if (hl < 0 || hl >= a.height_col) continue;
+      int h = lo + hl;
+      T v = zero_of<T>();
+      if (h < a.height) v = val[stage_index((h >> 3) - g0, sibling_slot(h & 7) + a.slot[k])];
+      col[row + hl] = v;
+    }
+  }
+}
+
+// Slots that record, per call, that a table is not symmetric.  A call owns slot
+// id % kColSlots and the value id, which no other call ever writes, so slots need no
+// clearing; calls overlapping on other streams only collide kColSlots calls apart.
+constexpr int kColSlots = 1024;
+__device__ unsigned long long g_col_asymmetric[kColSlots];
+std::atomic<unsigned long long> g_col_calls{0};
+
+// The gather form of col2octree below is exact when (column h, tap k) -> row p and
+// (row p, tap k) -> column h are inverse maps.  y = 0 walks the columns of the chunk,
+// y = 1 the rows; any pair that does not map back marks the call.
+template <bool P>
+__global__ void col_check_kernel(ColArgs a, const int* __restrict__ neigh,
+    const int* __restrict__ child, const int* __restrict__ ichild, unsigned long long id,
+    bool no_inverse) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (no_inverse) {  // the caller gave no inverse child table: always scatter
+    if (i == 0 && blockIdx.y == 0) g_col_asymmetric[id % kColSlots] = id;
+    return;
+  }
+  int lo = a.n * a.height_col, hi = min(a.height, lo + a.height_col);
+  bool bad = false;
+  if (blockIdx.y == 0) {
+    int h = lo + i;
+    if (h >= hi) return;
+    int64_t base = col_base<P>(a, h, ichild);
+    for (int k = 0; k < a.K; ++k) {
+      int p = col_source<P>(a, base, k, neigh, child);
+      if (p >= 0 && col_target<P>(a, p, k, neigh, child, ichild) != h) bad = true;
+    }
+  } else {
+    int p = i;
+    if (p >= a.octree_h) return;
+    for (int k = 0; k < a.K; ++k) {
+      int h = col_target<P>(a, p, k, neigh, child, ichild);
+      if (h >= lo && h < hi &&
+          col_source<P>(a, col_base<P>(a, h, ichild), k, neigh, child) != p) bad = true;
+    }
+  }
+  if (bad) g_col_asymmetric[id % kColSlots] = id;
+}
+
+// Gather form: one thread per row sums its taps in ascending order, no atomics.
+// Leaves the work to col2octree_atomic_kernel when the call is marked (and then only
+// clears the rows if this is the first chunk).
 template <bool P>
 __global__ void col2octree_kernel(const float* __restrict__ col, float* __restrict__ data, ColArgs a,
-    const int* __restrict__ neigh, const int* __restrict__ child, const int* __restrict__ ichild) {
+    const int* __restrict__ neigh, const int* __restrict__ child, const int* __restrict__ ichild,
+    unsigned long long id) {
+  int p = blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= a.octree_h) return;
+  bool marked = g_col_asymmetric[id % kColSlots] == id;
+  int c0 = blockIdx.y * kChanChunk, c1 = min(a.channel, c0 + kChanChunk);
+  float acc[kChanChunk];
+#pragma unroll
+  for (int j = 0; j < kChanChunk; ++j) acc[j] = 0.0f;
+  if (!marked) {
+    int lo = a.n * a.height_col, hi = min(a.height, lo + a.height_col);
+    int hl[27];  // column of every tap inside the chunk, -1 when there is none
+#pragma unroll
+    for (int k = 0; k < 27; ++k) {
+      int h = k < a.K ? col_target<P>(a, p, k, neigh, child, ichild) : -1;
+      hl[k] = (h >= lo && h < hi) ? h - lo : -1;
+    }
+#pragma unroll
+    for (int k = 0; k < 27; ++k) {
+      if (hl[k] < 0) continue;
+#pragma unroll
+      for (int j = 0; j < kChanChunk; ++j)
+        if (c0 + j < c1) acc[j] += col[((int64_t)(c0 + j) * a.K + k) * a.height_col + hl[k]];
+    }
+  } else if (a.n != 0) {
+    return;
+  }
+#pragma unroll
+  for (int j = 0; j < kChanChunk; ++j)
+    if (c0 + j < c1) {
+      float* dst = &data[(int64_t)(c0 + j) * a.octree_h + p];
+      *dst = a.n == 0 ? acc[j] : *dst + acc[j];
+    }
+}
+
+// Scatter form, for any table (octree_nn.cu:130-174); runs only for a marked call.
+template <bool P>
+__global__ void col2octree_atomic_kernel(const float* __restrict__ col, float* __restrict__ data,
+    ColArgs a, const int* __restrict__ neigh, const int* __restrict__ child,
+    const int* __restrict__ ichild, unsigned long long id) {
+  if (g_col_asymmetric[id % kColSlots] != id) return;
   int hl = blockIdx.x * blockDim.x + threadIdx.x;
   if (hl >= a.height_col) return;
-  int k = blockIdx.y;
   int h = a.n * a.height_col + hl;
   if (h >= a.height) return;
-  int p = col_source<P>(a, h, k, neigh, child, ichild);
-  if (p < 0 || p >= a.octree_h) return;
-  int c0 = blockIdx.z * kChanChunk, c1 = min(a.channel, c0 + kChanChunk);
-  for (int c = c0; c < c1; ++c)
-    unsafeAtomicAdd(&data[(int64_t)c * a.octree_h + p],
-        col[((int64_t)c * a.K + k) * a.height_col + hl]);
+  int64_t base = col_base<P>(a, h, ichild);
+  int c0 = blockIdx.y * kChanChunk, c1 = min(a.channel, c0 + kChanChunk);
+  for (int k = 0; k < a.K; ++k) {
+    int p = col_source<P>(a, base, k, neigh, child);
+    if (p < 0) continue;
+    for (int c = c0; c < c1; ++c)
+      unsafeAtomicAdd(&data[(int64_t)c * a.octree_h + p],
+          col[((int64_t)c * a.K + k) * a.height_col + hl]);
+  }
 }
 
 // ---- pooling -------------------------------------------------------------------
@@ -213,7 +435,10 @@ bool fill_col_args(ColArgs* a, int channel, int height, int octree_h, const int*
   a->stride = stride;
   a->height_col = height_col;
   a->n = n;
-  for (int k = 0; k < 27; ++k) a->slot[k] = k < t.count ? tap_slot(t.tap[k]) : 0;
+  for (int k = 0; k < 27; ++k) {
+    a->slot[k] = k < t.count ? tap_slot(t.tap[k]) : 0;
+    a->rslot[k] = k < t.count ? tap_slot(26 - t.tap[k]) : 0;
+  }
   return true;
 }
 
@@ -222,6 +447,8 @@ int check_col(const void* col, const void* data, int channel, int height, const 
   OCNN_REQUIRE(col && data && neigh && ks, OCNN_E_BADARG, "null pointer");
   OCNN_REQUIRE(channel > 0 && height >= 0 && height_col > 0 && n >= 0, OCNN_E_BADARG,
       "channel %d height %d height_col %d n %d", channel, height, height_col, n);
+  OCNN_REQUIRE(((int64_t)n + 1) * height_col <= INT32_MAX, OCNN_E_BADARG,
+      "chunk %d of %d columns is out of range", n, height_col);
   OCNN_REQUIRE(stride == 1 || stride == 2, OCNN_E_BADARG, "stride %d", stride);
   OCNN_REQUIRE(dtype == OCNN_F32 || dtype == OCNN_BF16, OCNN_E_BADARG, "dtype %d", dtype);
   return OCNN_OK;
@@ -236,11 +463,21 @@ int run_octree2col(void* col, const void* data, int channel, int height, int oct
   ColArgs a;
   OCNN_REQUIRE(fill_col_args(&a, channel, height, octree_h, ks, stride, height_col, n),
       OCNN_E_UNSUPPORTED, "kernel size %d%d%d", ks[0], ks[1], ks[2]);
-  dim3 grid(blocks_for(height_col), a.K, (channel + kChanChunk - 1) / kChanChunk);
+  unsigned tiles = blocks_for((int64_t)height_col + kColApron - 1, kColTile);
+  if (!P && stride == 1) {
+    dim3 grid(tiles, std::min<unsigned>(channel, std::max(1u, 2048u / tiles)));
+    if (dtype == OCNN_F32)
+      octree2col_block_kernel<float><<<grid, kColTile, 0, s>>>((float*)col, (const float*)data, a, neigh);
+    else
+      octree2col_block_kernel<uint16_t><<<grid, kColTile, 0, s>>>((uint16_t*)col, (const uint16_t*)data, a, neigh);
+    OCNN_LAUNCH_OK("octree2col");
+    return OCNN_OK;
+  }
+  dim3 grid(tiles, (channel + kChanChunk - 1) / kChanChunk);
   if (dtype == OCNN_F32)
-    octree2col_kernel<float, P><<<grid, kBlock, 0, s>>>((float*)col, (const float*)data, a, neigh, child, ichild);
+    octree2col_kernel<float, P><<<grid, kColTile, 0, s>>>((float*)col, (const float*)data, a, neigh, child, ichild);
   else
-    octree2col_kernel<uint16_t, P><<<grid, kBlock, 0, s>>>((uint16_t*)col, (const uint16_t*)data, a, neigh, child, ichild);
+    octree2col_kernel<uint16_t, P><<<grid, kColTile, 0, s>>>((uint16_t*)col, (const uint16_t*)data, a, neigh, child, ichild);
   OCNN_LAUNCH_OK("octree2col");
   return OCNN_OK;
 }
@@ -255,15 +492,29 @@ int run_col2octree(const void* col, void* data, int channel, int height, int oct
   ColArgs a;
   OCNN_REQUIRE(fill_col_args(&a, channel, height, octree_h, ks, stride, height_col, n),
       OCNN_E_UNSUPPORTED, "kernel size %d%d%d", ks[0], ks[1], ks[2]);
-  if (n == 0) {  // the output is cleared once, by the first chunk (octree_nn.cpp:226)
-    int64_t cnt = (int64_t)channel * octree_h;
-    fill_kernel<float><<<blocks_for(cnt, kBlock * 4), kBlock, 0, s>>>((float*)data, cnt, 0.0f);
-    OCNN_LAUNCH_OK("fill");
-  }
-  if (height == 0) return OCNN_OK;
-  dim3 grid(blocks_for(height_col), a.K, (channel + kChanChunk - 1) / kChanChunk);
-  col2octree_kernel<P><<<grid, kBlock, 0, s>>>((const float*)col, (float*)data, a, neigh, child, ichild);
+  if (octree_h == 0) return OCNN_OK;
+  // The first chunk (n == 0) overwrites the rows, later ones add to them
+  // (octree_nn.cpp:226 clears the output before the first chunk).
+  unsigned long long id = ++g_col_calls;
+  bool can_invert = !P || ichild != nullptr;
+  int chunk_cols = (int)std::max<int64_t>(0,
+      std::min<int64_t>(height, ((int64_t)n + 1) * height_col) - (int64_t)n * height_col);
+  int chans = (channel + kChanChunk - 1) / kChanChunk;
+  // At stride 1 with a tap set that holds the opposite of each of its taps, a row's
+  // columns are found the way a column's rows are (tap k one way is the opposite tap
+  // the other way), so over the whole range one direction of the check says it all.
+  bool one_way = stride == 1 && ks[0] != 2 && n == 0 && chunk_cols == height && height == octree_h;
+  dim3 check_grid(blocks_for(std::max(std::max(chunk_cols, octree_h), 1)), one_way ? 1 : 2);
+  col_check_kernel<P><<<check_grid, kBlock, 0, s>>>(a, neigh, child, ichild, id, !can_invert);
+  OCNN_LAUNCH_OK("col_check");
+  col2octree_kernel<P><<<dim3(blocks_for(octree_h), chans), kBlock, 0, s>>>((const float*)col,
+      (float*)data, a, neigh, child, ichild, id);
   OCNN_LAUNCH_OK("col2octree");
+  if (chunk_cols > 0) {
+    col2octree_atomic_kernel<P><<<dim3(blocks_for(height_col), chans), kBlock, 0, s>>>(
+        (const float*)col, (float*)data, a, neigh, child, ichild, id);
+    OCNN_LAUNCH_OK("col2octree_atomic");
+  }
   return OCNN_OK;
 }
 

@@ -525,7 +525,7 @@ def octree2col(data_in, octree, depth, kernel_size, stride, nempty):
       top_h = btm_h // 8
       if top_h != info.nnum_nempty(depth - 1):
         raise OcnnError(-3, "octree2col: stride-2 height mismatch")
-    out = torch.zeros(channel, K, top_h, dtype=data_in.dtype, device=data_in.device)
+    out = torch.empty(channel, K, top_h, dtype=data_in.dtype, device=data_in.device)
     _lib.call("ocnn_octree2col", _ptr(out), _ptr(data_in), channel, top_h, ksc, stride, _ptr(neigh),
               max(top_h, 1), 0, dt, _stream())
     return out
@@ -533,7 +533,7 @@ def octree2col(data_in, octree, depth, kernel_size, stride, nempty):
     raise OcnnError(-3, "octree2col: height %d != node_num_nempty(%d)" % (btm_h, depth))
   child, ichild = _ichild(octree, info, depth)
   top_h = btm_h if stride == 1 else info.nnum_nempty(depth - 1)
-  out = torch.zeros(channel, K, top_h, dtype=data_in.dtype, device=data_in.device)
+  out = torch.empty(channel, K, top_h, dtype=data_in.dtype, device=data_in.device)
   _lib.call("ocnn_octree2colP", _ptr(out), _ptr(data_in), channel, top_h, btm_h, ksc, stride,
             _ptr(neigh), _ptr(child), _ptr(ichild), max(top_h, 1), 0, dt, _stream())
   return out
@@ -552,7 +552,7 @@ def col2octree(grad_in, octree, depth, kernel_size, stride, nempty):
     raise OcnnError(-3, "col2octree: stride-2 height mismatch")
   if not nempty:
     btm_h = info.nnum(depth)
-    out = torch.zeros(1, channel, btm_h, 1, dtype=grad_in.dtype, device=grad_in.device)
+    out = torch.empty(1, channel, btm_h, 1, dtype=grad_in.dtype, device=grad_in.device)
     _lib.call("ocnn_col2octree", _ptr(grad_in), _ptr(out), channel, top_h, ksc, stride, _ptr(neigh),
               max(top_h, 1), 0, dt, _stream())
     return out
@@ -560,7 +560,7 @@ def col2octree(grad_in, octree, depth, kernel_size, stride, nempty):
   if stride == 1 and top_h != btm_h:
     raise OcnnError(-3, "col2octree: height mismatch")
   child, ichild = _ichild(octree, info, depth)
-  out = torch.zeros(1, channel, btm_h, 1, dtype=grad_in.dtype, device=grad_in.device)
+  out = torch.empty(1, channel, btm_h, 1, dtype=grad_in.dtype, device=grad_in.device)
   _lib.call("ocnn_col2octreeP", _ptr(grad_in), _ptr(out), channel, top_h, btm_h, ksc, stride,
             _ptr(neigh), _ptr(child), _ptr(ichild), max(top_h, 1), 0, dt, _stream())
   return out

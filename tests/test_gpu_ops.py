@@ -90,6 +90,58 @@ def test_col_ops_vs_oracle(oc, orc, tree, stride):
                   orc.col2octreeP(expp, ks, stride, neigh, child, ichild, hp, Hne)) < TOL_F32
 
 
+def test_col2octree_any_table_and_chunks(oc, orc, tree):
+  """col2octree through the C-ABI in column chunks (octree_nn.cpp:216-241 adds chunk n to the
+  rows the earlier chunks left), on the octree's own table and on tables that are not
+  neighbour tables of any octree: entries shuffled inside each sibling block, and all
+  entries naming one row, where the sum must still be the scatter-add of the reference."""
+  import ctypes as C
+  b = tree["blob"]
+  d = 5
+  H, Hne = int(b.nnum[d]), int(b.nnum_nempty[d])
+  own, child = b.prop("neigh", d).reshape(-1).copy(), b.prop("child", d)
+  ichild = np.zeros(Hne, np.int32)
+  ichild[child[child >= 0]] = np.nonzero(child >= 0)[0]
+  rng = np.random.default_rng(7)
+  shuffled = own.reshape(-1, 64).copy()
+  for row in shuffled[::3]:
+    rng.shuffle(row)
+  same = np.where(own >= 0, 5, -1).astype(np.int32)
+  P = lambda t: C.c_void_p(t.data_ptr())
+  st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+  child_d, ichild_d = T(child).cuda(), T(ichild).cuda()
+  for name, table in (("own", own), ("shuffled", shuffled.reshape(-1)), ("same", same)):
+    table_d = T(table.astype(np.int32)).cuda()
+    for ks, stride in (([3, 3, 3], 1), ([2, 2, 2], 2), ([3, 1, 3], 1), ([3, 3, 3], 2)):
+      K = int(np.prod(ks))
+      ksc = (C.c_int * 3)(*ks)
+      h = H if stride == 1 else H // 8
+      col = rng.standard_normal((5, K, h)).astype(np.float32)
+      exp = orc.col2octree(col, ks, stride, table, h)
+      hc = (h + 2) // 3                                  # three chunks, the last one ragged
+      out = torch.full((5, H), 7.0, device="cuda")       # stale values the first chunk must replace
+      for n in range(3):
+        piece = np.zeros((5, K, hc), np.float32)
+        w = max(0, min(h, (n + 1) * hc) - n * hc)
+        piece[:, :, :w] = col[:, :, n * hc:n * hc + w]
+        piece_d = T(piece).cuda()
+        oc.lib.call("ocnn_col2octree", P(piece_d), P(out), 5, h, ksc, stride, P(table_d), hc, n, 0, st)
+      assert relerr(out.cpu().numpy(), exp) < TOL_F32, (name, ks, stride)
+      hp = Hne if stride == 1 else H // 8
+      colp = rng.standard_normal((5, K, hp)).astype(np.float32)
+      expp = orc.col2octreeP(colp, ks, stride, table, child, ichild, hp, Hne)
+      outp = torch.full((5, Hne), 7.0, device="cuda")
+      colp_d = T(colp).cuda()
+      oc.lib.call("ocnn_col2octreeP", P(colp_d), P(outp), 5, hp, Hne, ksc, stride, P(table_d), P(child_d),
+                  P(ichild_d), hp, 0, 0, st)
+      assert relerr(outp.cpu().numpy(), expp) < TOL_F32, (name, "P", ks, stride)
+      if stride == 2:   # without the inverse child table only the scatter form can run
+        outq = torch.full((5, Hne), 7.0, device="cuda")
+        oc.lib.call("ocnn_col2octreeP", P(colp_d), P(outq), 5, hp, Hne, ksc, stride, P(table_d),
+                    P(child_d), C.c_void_p(0), hp, 0, 0, st)
+        assert relerr(outq.cpu().numpy(), expp) < TOL_F32, (name, "P, no ichild", ks, stride)
+
+
 CONV_CASES = [(ks, s, ne) for ks in KERNELS for s in (1, 2) for ne in (False, True)]
 
 
