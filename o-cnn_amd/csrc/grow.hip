@@ -6,6 +6,8 @@
 #include "ocnn_common.h"
 #include "scan.h"
 
+#include <algorithm>
+#include <mutex>
 #include <vector>
 
 namespace ocnn {
@@ -62,6 +64,85 @@ __global__ void g_seq_key_child_kernel(uint64_t* __restrict__ key, int* __restri
   if (key) key[i] = (uint64_t)i;
   child[i] = i;
 }
+
+// ---- octree_grow in one launch -------------------------------------------------------
+// The grown blob is a list of byte ranges, each produced by one rule: the header, copies
+// of the old properties, zeros, and the new depth's child indices 0..n-1; the new depth's
+// keys are written from the side of their parents (the old deepest level), one item per
+// (parent, child).  Ranges are dealt out over the workgroups of ONE launch.  A range is
+// walked in 4-byte words counted from the 256-byte line its destination starts in, so
+// that every wavefront stores one whole aligned line.
+constexpr int kGrowRanges = 20;
+constexpr int kGrowWordsPerBlock = kBlock * 16;
+enum { kGrowHeader = 0, kGrowCopy, kGrowZero, kGrowSequence, kGrowKeyChild };
+struct GrowPlan {
+  int n;
+  int kind[kGrowRanges];
+  unsigned first_block[kGrowRanges + 1];
+  int64_t dst[kGrowRanges], src[kGrowRanges], words[kGrowRanges];  // byte offsets; words or items
+  int64_t parent_key, parent_child;                                   // byte offsets in the old blob
+};
+
+__global__ void __launch_bounds__(kBlock) g_grow_kernel(char* __restrict__ out,
+    const char* __restrict__ in, GrowPlan p, HeaderArg h) {
+  int r = 0;
+  while (r + 1 < p.n && blockIdx.x >= p.first_block[r + 1]) ++r;
+  const int kind = p.kind[r];
+  const int64_t begin = (int64_t)(blockIdx.x - p.first_block[r]) * kGrowWordsPerBlock;
+  if (kind == kGrowKeyChild) {  // generate_key, octree_nn.cpp:427-463, for the children of the old level
+    const uint64_t* pkey = reinterpret_cast<const uint64_t*>(in + p.parent_key);
+    const int* pchild = reinterpret_cast<const int*>(in + p.parent_child);
+    uint64_t* key = reinterpret_cast<uint64_t*>(out + p.dst[r]);
+    const int64_t stop = min(p.words[r], begin + kGrowWordsPerBlock);
+    for (int64_t id = begin + threadIdx.x; id < stop; id += kBlock) {
+      int i = (int)(id >> 3), j = (int)(id & 7);
+      int label = pchild[i];
+      if (label < 0) continue;
+      uint64_t k0 = pkey[i];
+      uint64_t x = (((k0 & 0xffffu) << 1) | ((j >> 2) & 1)) & 0xffffu;
+      uint64_t y = ((((k0 >> 16) & 0xffffu) << 1) | ((j >> 1) & 1)) & 0xffffu;
+      uint64_t z = ((((k0 >> 32) & 0xffffu) << 1) | (j & 1)) & 0xffffu;
+      key[8 * (int64_t)label + j] = x | (y << 16) | (z << 32) | (k0 & 0xffff000000000000ull);
+    }
+    return;
+  }
+  const uintptr_t dst_addr = reinterpret_cast<uintptr_t>(out) + p.dst[r];
+  const int64_t lead = (int64_t)((dst_addr & 255) >> 2);  // words between the line start and the range
+  uint32_t* dst = reinterpret_cast<uint32_t*>(dst_addr) - lead;
+  const uint32_t* src = reinterpret_cast<const uint32_t*>(in + p.src[r]) - lead;
+  const int64_t stop = min(p.words[r] + lead, begin + kGrowWordsPerBlock);
+  for (int64_t v = begin + threadIdx.x; v < stop; v += kBlock) {
+    if (v < lead) continue;
+    uint32_t val = 0;
+    if (kind == kGrowCopy) val = src[v];
+    else if (kind == kGrowSequence) val = (uint32_t)(v - lead);
+    else if (kind == kGrowHeader) val = h.w[v - lead];
+    dst[v] = val;
+  }
+}
+
+struct GrowRanges {
+  GrowPlan plan;
+  void add(int kind, int64_t dst, int64_t src, int64_t count) {
+    if (count <= 0) return;
+    plan.kind[plan.n] = kind;
+    plan.dst[plan.n] = dst;
+    plan.src[plan.n] = src;
+    plan.words[plan.n] = count;
+    ++plan.n;
+  }
+  // blocks per range; a range that is walked from its line start has up to 63 extra words
+  unsigned finish() {
+    unsigned total = 0;
+    for (int r = 0; r < plan.n; ++r) {
+      plan.first_block[r] = total;
+      int64_t span = plan.words[r] + (plan.kind[r] == kGrowKeyChild ? 0 : 63);
+      total += (unsigned)((span + kGrowWordsPerBlock - 1) / kGrowWordsPerBlock);
+    }
+    plan.first_block[plan.n] = total;
+    return total;
+  }
+};
 
 // ---- merge ---------------------------------------------------------------------
 // Per depth one launch per property over the merged node range; the source octree
@@ -318,49 +399,79 @@ int ocnn_octree_grow(void* out_dev, const void* out_info, const void* in_dev, co
   hipStream_t s = as_stream(stream);
   char* blob = static_cast<char*>(out_dev);
   const char* in = static_cast<const char*>(in_dev);
-  e = zero_payload(blob, o, s);
-  if (e) return e;
-  e = write_header(blob, o, s);
-  if (e) return e;
-  // copy_octree_gpu, octree_grow.cpp:75-87: everything below the new depth
-  int64_t ncum = oi.nnum_cum[target_depth];
-  e = copy_dev(reinterpret_cast<uint64_t*>(blob + o.ptr_dis(OCNN_KEY, 0)),
-      reinterpret_cast<const uint64_t*>(in + oi.ptr_dis(OCNN_KEY, 0)), ncum * oi.channel(OCNN_KEY), s);
-  if (e) return e;
-  e = copy_dev(reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_CHILD, 0)),
-      reinterpret_cast<const int*>(in + oi.ptr_dis(OCNN_CHILD, 0)), ncum * oi.channel(OCNN_CHILD), s);
-  if (e) return e;
-  e = copy_dev(reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_NEIGH, 0)),
-      reinterpret_cast<const int*>(in + oi.ptr_dis(OCNN_NEIGH, 0)), ncum * oi.channel(OCNN_NEIGH), s);
-  if (e) return e;
-  if (oi.has(OCNN_FEATURE)) {
-    e = copy_dev(reinterpret_cast<float*>(blob + o.ptr_dis(OCNN_FEATURE, 0)),
-        reinterpret_cast<const float*>(in + oi.ptr_dis(OCNN_FEATURE, 0)), ncum * oi.channel(OCNN_FEATURE), s);
-    if (e) return e;
-  }
-  int* neigh = reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_NEIGH, target_depth));
-  uint64_t* key = reinterpret_cast<uint64_t*>(blob + o.ptr_dis(OCNN_KEY, target_depth));
-  int* child = reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_CHILD, target_depth));
+  // copy_octree_gpu, octree_grow.cpp:75-87: everything below the new depth is copied, the
+  // rest of the payload starts as zeros (the reference allocates the blob with torch::zeros)
+  const int64_t ncum = oi.nnum_cum[target_depth];
   const int node_num = o.nnum[target_depth];
+  const int64_t key_new = o.ptr_dis(OCNN_KEY, target_depth);
+  const int64_t child_new = o.ptr_dis(OCNN_CHILD, target_depth);
+  const int64_t neigh_new = o.ptr_dis(OCNN_NEIGH, target_depth);
+  struct Span { int64_t at, bytes; };
+  std::vector<Span> written;  // payload bytes that some rule or a later kernel writes
+  GrowRanges g;
+  memset(&g.plan, 0, sizeof(g.plan));
+  g.add(kGrowHeader, 0, 0, OCNN_HEADER_BYTES / 4);
+  const int props[4] = {OCNN_KEY, OCNN_CHILD, OCNN_NEIGH, OCNN_FEATURE};
+  const int elem[4] = {8, 4, 4, 4};
+  for (int i = 0; i < 4; ++i) {
+    if (!oi.has(props[i])) continue;
+    int64_t bytes = ncum * oi.channel(props[i]) * elem[i];
+    g.add(kGrowCopy, o.ptr_dis(props[i], 0), oi.ptr_dis(props[i], 0), bytes / 4);
+    written.push_back({o.ptr_dis(props[i], 0), bytes});
+  }
+  written.push_back({key_new, (int64_t)node_num * 8});
+  written.push_back({child_new, (int64_t)node_num * 4});
+  written.push_back({neigh_new, (int64_t)node_num * 32});
+  std::sort(written.begin(), written.end(), [](const Span& x, const Span& y) { return x.at < y.at; });
+  int64_t at = OCNN_HEADER_BYTES;
+  const int64_t blob_end = o.sizeof_octree();
+  for (size_t i = 0; i <= written.size(); ++i) {
+    int64_t next = i < written.size() ? written[i].at : blob_end;
+    if (next > at) g.add(kGrowZero, at, 0, (next - at) / 4);
+    if (i < written.size()) at = std::max(at, written[i].at + written[i].bytes);
+  }
+  g.add(kGrowSequence, child_new, 0, node_num);
+  if (!full_octree) {
+    g.add(kGrowKeyChild, key_new, 0, (int64_t)o.nnum[target_depth - 1] << 3);
+    g.plan.parent_key = oi.ptr_dis(OCNN_KEY, target_depth - 1);
+    g.plan.parent_child = oi.ptr_dis(OCNN_CHILD, target_depth - 1);
+  }
+  HeaderArg h;
+  memset(&h, 0, sizeof(h));
+  memcpy(&h, &o, sizeof(Info));
+  unsigned blocks = g.finish();
+  g_grow_kernel<<<blocks, kBlock, 0, s>>>(blob, in, g.plan, h);
+  OCNN_LAUNCH_OK("octree_grow");
+  // the new level's neighbours (and, for a full level, its keys) come from the old blob's tables
+  int* neigh = reinterpret_cast<int*>(blob + neigh_new);
   if (full_octree) {
     e = ocnn_calc_neigh_full(neigh, target_depth, o.batch_size, stream);
     if (e) return e;
-    e = ocnn_generate_key_full(key, target_depth, o.batch_size, stream);
+    e = ocnn_generate_key_full(reinterpret_cast<uint64_t*>(blob + key_new), target_depth, o.batch_size, stream);
     if (e) return e;
   } else {
-    const int* label = reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_CHILD, target_depth - 1));
-    e = ocnn_calc_neigh_sparse(neigh, reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_NEIGH, target_depth - 1)),
-        label, o.nnum[target_depth - 1], stream);
+    e = ocnn_calc_neigh_sparse(neigh, reinterpret_cast<const int*>(in + oi.ptr_dis(OCNN_NEIGH, target_depth - 1)),
+        reinterpret_cast<const int*>(in + oi.ptr_dis(OCNN_CHILD, target_depth - 1)), o.nnum[target_depth - 1], stream);
     if (e) return e;
-    e = ocnn_generate_key_child(key, reinterpret_cast<const uint64_t*>(blob + o.ptr_dis(OCNN_KEY, target_depth - 1)),
-        label, o.nnum[target_depth - 1], stream);
-    if (e) return e;
-  }
-  if (node_num > 0) {
-    g_seq_key_child_kernel<<<blocks_for(node_num), kBlock, 0, s>>>(nullptr, child, node_num);
-    OCNN_LAUNCH_OK("sequence");
   }
   return OCNN_OK;
+}
+
+// pinned words for counts that a call waits for; kept for the life of the process
+static std::mutex g_pinned_mutex;
+static std::vector<int*> g_pinned_free;
+static int* take_pinned_int() {
+  {
+    std::lock_guard<std::mutex> lock(g_pinned_mutex);
+    if (!g_pinned_free.empty()) { int* p = g_pinned_free.back(); g_pinned_free.pop_back(); return p; }
+  }
+  void* p = nullptr;
+  if (hipHostMalloc(&p, 64, hipHostMallocDefault) != hipSuccess) return nullptr;
+  return static_cast<int*>(p);
+}
+static void give_pinned_int(int* p) {
+  std::lock_guard<std::mutex> lock(g_pinned_mutex);
+  g_pinned_free.push_back(p);
 }
 
 __global__ void g_fix_empty_split_kernel(int* children, int* count) {
@@ -390,9 +501,14 @@ int ocnn_octree_update(void* octree_dev, void* info, const int* label, int n_lab
   g_fix_empty_split_kernel<<<1, 64, 0, s>>>(children, count_dev);
   g_patch_nempty_kernel<<<1, 64, 0, s>>>(reinterpret_cast<int*>(blob + offsetof(Info, nnum_nempty)) + depth, count_dev);
   OCNN_LAUNCH_OK("octree_update");
-  int split_num = 0;
-  OCNN_HIP_OK(hipMemcpyAsync(&split_num, count_dev, sizeof(int), hipMemcpyDeviceToHost, s));
-  OCNN_HIP_OK(hipStreamSynchronize(s));
+  // the count comes back through pinned memory: a copy into pageable memory is staged
+  int* pinned = take_pinned_int();
+  OCNN_REQUIRE(pinned, OCNN_E_HIP, "no pinned host memory for the split count");
+  hipError_t err = hipMemcpyAsync(pinned, count_dev, sizeof(int), hipMemcpyDeviceToHost, s);
+  if (err == hipSuccess) err = hipStreamSynchronize(s);
+  int split_num = *pinned;
+  give_pinned_int(pinned);
+  OCNN_REQUIRE(err == hipSuccess, OCNN_E_HIP, "split count: %s", hipGetErrorString(err));
   o->nnum_nempty[depth] = split_num;
   return OCNN_OK;
 }
