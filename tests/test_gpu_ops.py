@@ -90,6 +90,59 @@ def test_col_ops_vs_oracle(oc, orc, tree, stride):
                   orc.col2octreeP(expp, ks, stride, neigh, child, ichild, hp, Hne)) < TOL_F32
 
 
+def test_octree2col_chunks_and_unaligned_rows(oc, orc, tree):
+  """octree2col through the C-ABI in column chunks (chunk n holds columns n*height_col ..., the
+  columns past the last node are zero, octree_nn.cpp:188-214), written into a buffer that does
+  not start on a 256-byte line, for all nodes and for the non-empty ones, fp32 and bf16."""
+  import ctypes as C
+  b = tree["blob"]
+  d = 5
+  H, Hne = int(b.nnum[d]), int(b.nnum_nempty[d])
+  neigh, child = b.prop("neigh", d).reshape(-1), b.prop("child", d)
+  ichild = np.zeros(Hne, np.int32)
+  ichild[child[child >= 0]] = np.nonzero(child >= 0)[0]
+  rng = np.random.default_rng(11)
+  P = lambda t, off=0: C.c_void_p(t.data_ptr() + off)
+  st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+  neigh_d, child_d, ichild_d = T(neigh).cuda(), T(child).cuda(), T(ichild).cuda()
+  Cc = 11   # more than one channel chunk, the last one ragged
+  x = rng.standard_normal((Cc, H)).astype(np.float32)
+  xn = rng.standard_normal((Cc, Hne)).astype(np.float32)
+  for dt, tt in ((0, torch.float32), (1, torch.bfloat16)):
+    x_d, xn_d = T(x).cuda().to(tt), T(xn).cuda().to(tt)
+    xr, xnr = x_d.float().cpu().numpy(), xn_d.float().cpu().numpy()
+    for ks, stride in (([3, 3, 3], 1), ([2, 2, 2], 2), ([1, 3, 3], 1), ([3, 3, 3], 2)):
+      K = int(np.prod(ks))
+      ksc = (C.c_int * 3)(*ks)
+      h = H if stride == 1 else H // 8
+      full = orc.octree2col(xr, ks, stride, neigh, h)
+      hc = (h + 2) // 3 + 5
+      for n in range(3):
+        exp = np.zeros((Cc, K, hc), np.float32)
+        w = max(0, min(h, (n + 1) * hc) - n * hc)
+        exp[:, :, :w] = full[:, :, n * hc:n * hc + w]
+        buf = torch.full((Cc * K * hc + 64,), 9.0, device="cuda", dtype=tt)
+        skew = 3 * buf.element_size()   # the output starts three elements into the buffer
+        oc.lib.call("ocnn_octree2col", P(buf, skew), P(x_d), Cc, h, ksc, stride, P(neigh_d), hc, n, dt, st)
+        got = buf.float().cpu().numpy()
+        assert np.array_equal(got[3:3 + Cc * K * hc].reshape(Cc, K, hc), exp), (dt, ks, stride, n)
+        assert np.all(got[:3] == 9.0) and np.all(got[3 + Cc * K * hc:] == 9.0), "wrote outside the chunk"
+      hp = Hne if stride == 1 else H // 8
+      fullp = orc.octree2colP(xnr, ks, stride, neigh, child, ichild, hp)
+      hc = (hp + 1) // 2 + 3
+      for n in range(2):
+        exp = np.zeros((Cc, K, hc), np.float32)
+        w = max(0, min(hp, (n + 1) * hc) - n * hc)
+        exp[:, :, :w] = fullp[:, :, n * hc:n * hc + w]
+        buf = torch.full((Cc * K * hc + 64,), 9.0, device="cuda", dtype=tt)
+        skew = 5 * buf.element_size()
+        oc.lib.call("ocnn_octree2colP", P(buf, skew), P(xn_d), Cc, hp, Hne, ksc, stride, P(neigh_d), P(child_d),
+                    P(ichild_d), hc, n, dt, st)
+        got = buf.float().cpu().numpy()
+        assert np.array_equal(got[5:5 + Cc * K * hc].reshape(Cc, K, hc), exp), ("P", dt, ks, stride, n)
+        assert np.all(got[:5] == 9.0) and np.all(got[5 + Cc * K * hc:] == 9.0), "wrote outside the chunk"
+
+
 def test_col2octree_any_table_and_chunks(oc, orc, tree):
   """col2octree through the C-ABI in column chunks (octree_nn.cpp:216-241 adds chunk n to the
   rows the earlier chunks left), on the octree's own table and on tables that are not
