@@ -648,7 +648,10 @@ __device__ inline void leaf_signal(float* __restrict__ feature, float* __restric
 
 // The emit launch is cut into segments of whole workgroups; each segment is one kind of
 // work on one level.
-enum SegKind { kSegHeader = 0, kSegFull = 1, kSegFullNeigh = 2, kSegSparse = 3 };
+enum SegKind { kSegHeader = 0, kSegFull = 1, kSegFullNeigh = 2, kSegSparse = 3, kSegNeighSearch = 4 };
+// sparse levels with at most this many sibling groups get their neighbour table inside the emit
+// launch (by key search); larger ones from the table of the level above, one launch each
+constexpr int kSearchGroups = 8192;
 constexpr int kMaxSeg = 56;
 struct HeaderArg { uint32_t w[OCNN_HEADER_BYTES / 4]; };
 
@@ -703,6 +706,37 @@ __global__ __launch_bounds__(kBlock) void emit_kernel(char* __restrict__ blob, c
     int v = -1;
     if (((x1 | y1 | z1) & (1u << d)) == 0) v = (int)(morton_encode(x1, y1, z1, d) + (uint64_t)cloud * node_num);
     reinterpret_cast<int*>(blob + a.off_neigh[d])[id] = v;
+    return;
+  }
+  if (kind == kSegNeighSearch) {
+    // Neighbour table of a small sparse level straight from the geometry, so that it waits for
+    // no other level: wavefront = sibling group g (children of the g-th non-empty node of level
+    // d-1), lane = slot (x<<4 | y<<2 | z) = the node at offset (x-1, y-1, z-1) from sibling 0.
+    // That node exists iff it lies inside the cube and its parent is a non-empty node of the
+    // same cloud: the parent's rank r in the sorted list gives the index 8r + octant.  Equal to
+    // what calc_neigh derives level by level (octree_nn.cpp:357-380).
+    const int g = block * (kBlock / 64) + (tid >> 6);
+    if (g >= a.nne[d - 1]) return;
+    const int lane = tid & 63;
+    const int bits = 3 * (d - 1);
+    const uint64_t* __restrict__ list = a.list[d - 1];
+    const uint64_t pk = list[g];
+    const uint64_t cloud_bits = (pk >> bits) << bits;
+    uint32_t px, py, pz;
+    morton_decode(pk - cloud_bits, d - 1, &px, &py, &pz);
+    const int nx = 2 * (int)px + (lane >> 4) - 1, ny = 2 * (int)py + ((lane >> 2) & 3) - 1,
+              nz = 2 * (int)pz + (lane & 3) - 1;
+    int v = -1;
+    if (nx >= 0 && ny >= 0 && nz >= 0 && ((nx | ny | nz) >> d) == 0) {
+      const uint64_t want = cloud_bits | morton_encode((uint32_t)nx >> 1, (uint32_t)ny >> 1, (uint32_t)nz >> 1, d - 1);
+      int lo = 0, hi = a.nne[d - 1];
+      while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (list[mid] < want) lo = mid + 1; else hi = mid;
+      }
+      if (lo < a.nne[d - 1] && list[lo] == want) v = 8 * lo + (((nx & 1) << 2) | ((ny & 1) << 1) | (nz & 1));
+    }
+    reinterpret_cast<int*>(blob + a.off_neigh[d])[((int64_t)g << 6) + lane] = v;
     return;
   }
   uint64_t* key = reinterpret_cast<uint64_t*>(blob + a.off_key[d]);
@@ -1217,6 +1251,12 @@ int ocnn_points2octree_emit(void* octree_out_dev, const void* info, void* worksp
     add_seg(kSegFull, d, blocks_for(o.nnum[d]));
     if (o.has(OCNN_NEIGH) && d >= 1) add_seg(kSegFullNeigh, d, blocks_for((int64_t)B << (3 * d + 3)));
   }
+  int searched_to = fl;  // sparse levels up to here have their neighbour table after this launch
+  if (o.has(OCNN_NEIGH))
+    for (int d = fl + 1; d <= depth && st.nne[d - 1] > 0 && st.nne[d - 1] <= kSearchGroups; ++d) {
+      add_seg(kSegNeighSearch, d, blocks_for(st.nne[d - 1], kBlock / 64));
+      searched_to = d;
+    }
   a.seg_begin[n_seg] = blocks;
   a.n_seg = n_seg;
   emit_kernel<<<blocks, kBlock, 0, s>>>(blob, a);
@@ -1244,7 +1284,7 @@ int ocnn_points2octree_emit(void* octree_out_dev, const void* info, void* worksp
     OCNN_LAUNCH_OK("fill");
   }
   if (o.has(OCNN_NEIGH)) {  // merge_octrees.cpp:185-197: sparse levels, each from the level above
-    for (int d = fl + 1; d <= depth; ++d) {
+    for (int d = searched_to + 1; d <= depth; ++d) {
       if (o.nnum[d - 1] <= 0) continue;
       launch_neigh_sparse(reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_NEIGH, d)),
           reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_NEIGH, d - 1)),
