@@ -164,37 +164,114 @@ __device__ inline int find_src(const int* __restrict__ cum, int B, int t) {
 }
 enum { kPKey = 0, kPChild = 1, kPFeature = 2, kPLabel = 3, kPSplit = 4, kPCount = 5 };
 
-__global__ void merge_key_child_kernel(uint64_t* __restrict__ key, int* __restrict__ child, int d, int n,
-    MergeTable m) {
-  int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= n) return;
-  const int* cum = m.cum + d * (m.B + 1);
-  int b = find_src(cum, m.B, t);
-  int j = t - cum[b];
-  const char* src = m.src[b];
-  if (key) {
-    uint64_t k = reinterpret_cast<const uint64_t*>(src + m.src_off[(kPKey * m.B + b) * 17 + d])[j];
-    key[t] = (k & 0x0000ffffffffffffull) | ((uint64_t)(b & 0xffff) << 48);
+// One launch merges every property of every depth: the launch is cut into segments of whole
+// workgroups (header, zero ranges, key + child of a depth, one float property of a depth).
+enum { kMergeHeader = 0, kMergeZero, kMergeKeyChild, kMergeFloat };
+constexpr int kMergeSegMax = 96;
+struct MergeSeg {
+  int kind, depth, prop, channel;
+  unsigned first_block, pad;
+  int64_t dst_key, dst_child;   // byte offsets in the merged blob (dst_key also: zero / float target)
+  int64_t count;                // nodes of the depth, or 4-byte words to clear
+};
+
+// source octree of the workgroup's nodes: one search per workgroup when all its nodes come
+// from one octree (the rule on large levels), a short search per thread otherwise
+__device__ inline int block_src(const int* __restrict__ cum, int B, int t_first, int t_last, int t,
+    int* s_range) {
+  if (threadIdx.x == 0) {
+    s_range[0] = find_src(cum, B, t_first);
+    s_range[1] = find_src(cum, B, t_last);
   }
-  if (child) {
-    int c = reinterpret_cast<const int*>(src + m.src_off[(kPChild * m.B + b) * 17 + d])[j];
-    child[t] = c == -1 ? -1 : c + m.cum_ne[d * (m.B + 1) + b];
+  __syncthreads();
+  int lo = s_range[0], hi = s_range[1];
+  while (lo < hi) {
+    int mid = (lo + hi + 1) >> 1;
+    if (cum[mid] <= t) lo = mid; else hi = mid - 1;
   }
+  return lo;
 }
-// float property with `channel` channels: dst[c, t] = src_b[c, j]
-__global__ void merge_float_kernel(float* __restrict__ dst, int prop, int channel, int d, int n, MergeTable m) {
-  int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= n) return;
+
+__global__ void __launch_bounds__(kBlock) merge_kernel(char* __restrict__ blob, MergeTable m,
+    const MergeSeg* __restrict__ segs, int n_seg, HeaderArg h) {
+  __shared__ int s_range[2];
+  int lo = 0, hi = n_seg - 1;
+  while (lo < hi) {
+    int mid = (lo + hi + 1) >> 1;
+    if (segs[mid].first_block <= blockIdx.x) lo = mid; else hi = mid - 1;
+  }
+  const MergeSeg sg = segs[lo];
+  const int64_t i = (int64_t)(blockIdx.x - sg.first_block) * kBlock + threadIdx.x;
+  if (sg.kind == kMergeHeader) {
+    if (i < OCNN_HEADER_BYTES / 4) reinterpret_cast<uint32_t*>(blob)[i] = h.w[i];
+    return;
+  }
+  if (sg.kind == kMergeZero) {
+    uint32_t* dst = reinterpret_cast<uint32_t*>(blob + sg.dst_key);
+    for (int64_t w = i * 4; w < min(sg.count, i * 4 + 4); ++w) dst[w] = 0u;
+    return;
+  }
+  const int d = sg.depth, n = (int)sg.count;
+  const int t_first = (int)((int64_t)(blockIdx.x - sg.first_block) * kBlock);
+  const int t = (int)i;
   const int* cum = m.cum + d * (m.B + 1);
-  int b = find_src(cum, m.B, t);
-  int j = t - cum[b];
-  int nb = cum[b + 1] - cum[b];
-  const float* src = reinterpret_cast<const float*>(m.src[b] + m.src_off[(prop * m.B + b) * 17 + d]);
-  for (int c = 0; c < channel; ++c) dst[(int64_t)c * n + t] = src[(int64_t)c * nb + j];
+  const int b = block_src(cum, m.B, t_first, min(t_first + kBlock, n) - 1, min(t, n - 1), s_range);
+  if (t >= n) return;
+  const int j = t - cum[b];
+  const char* src = m.src[b];
+  if (sg.kind == kMergeKeyChild) {
+    // keys get the octree's index in their top 16 bits, child links move up by the non-empty
+    // nodes of the octrees before (merge_octrees.cpp:126-145)
+    if (sg.dst_key >= 0) {
+      uint64_t k = reinterpret_cast<const uint64_t*>(src + m.src_off[(kPKey * m.B + b) * 17 + d])[j];
+      reinterpret_cast<uint64_t*>(blob + sg.dst_key)[t] = (k & 0x0000ffffffffffffull) | ((uint64_t)(b & 0xffff) << 48);
+    }
+    if (sg.dst_child >= 0) {
+      int c = reinterpret_cast<const int*>(src + m.src_off[(kPChild * m.B + b) * 17 + d])[j];
+      reinterpret_cast<int*>(blob + sg.dst_child)[t] = c == -1 ? -1 : c + m.cum_ne[d * (m.B + 1) + b];
+    }
+    return;
+  }
+  // float property with `channel` channels: dst[c, t] = src_b[c, j] (merge_octrees.cpp:147-183)
+  const int nb = cum[b + 1] - cum[b];
+  const float* fsrc = reinterpret_cast<const float*>(src + m.src_off[(sg.prop * m.B + b) * 17 + d]);
+  float* dst = reinterpret_cast<float*>(blob + sg.dst_key);
+  for (int c = 0; c < sg.channel; ++c) dst[(int64_t)c * n + t] = fsrc[(int64_t)c * nb + j];
+}
+
+// Pinned staging buffers for host tables that a stream copies asynchronously.  A buffer is
+// busy until the event recorded behind its copy has completed; buffers live as long as the
+// process.
+struct Staging {
+  void* host = nullptr;
+  size_t bytes = 0;
+  hipEvent_t done = nullptr;
+  bool busy = false;
+};
+std::mutex g_staging_mutex;
+std::vector<Staging*> g_staging;
+Staging* take_staging(size_t bytes) {
+  std::lock_guard<std::mutex> lock(g_staging_mutex);
+  for (Staging* st : g_staging) {
+    if (st->busy && hipEventQuery(st->done) == hipSuccess) st->busy = false;
+    if (!st->busy && st->bytes >= bytes) { st->busy = true; return st; }
+  }
+  Staging* st = new Staging();
+  size_t cap = bytes < 65536 ? 65536 : bytes;
+  if (hipHostMalloc(&st->host, cap, hipHostMallocDefault) != hipSuccess ||
+      hipEventCreateWithFlags(&st->done, hipEventDisableTiming) != hipSuccess) {
+    if (st->host) (void)hipHostFree(st->host);
+    delete st;
+    return nullptr;
+  }
+  st->bytes = cap;
+  st->busy = true;
+  g_staging.push_back(st);
+  return st;
 }
 
 inline size_t al(size_t v) { return (v + 255) & ~(size_t)255; }
-struct MergeLayout { size_t cum, cum_ne, src_off, src, total; };
+struct MergeLayout { size_t cum, cum_ne, src_off, src, segs, total; };
 MergeLayout merge_layout(int B, int depth) {
   MergeLayout L;
   size_t off = 0;
@@ -203,6 +280,7 @@ MergeLayout merge_layout(int B, int depth) {
   L.cum_ne = take(sizeof(int) * (size_t)(depth + 1) * (B + 1));
   L.src_off = take(sizeof(int64_t) * (size_t)kPCount * B * 17);
   L.src = take(sizeof(char*) * (size_t)B);
+  L.segs = take(sizeof(MergeSeg) * (size_t)kMergeSegMax);
   L.total = off;
   return L;
 }
@@ -260,10 +338,13 @@ int ocnn_octree_batch(void* out_dev, const void* out_info, const void* const* oc
       workspace_bytes, L.total);
   hipStream_t s = as_stream(stream);
 
-  // host tables
-  std::vector<int> cum((size_t)(depth + 1) * (B + 1), 0), cum_ne((size_t)(depth + 1) * (B + 1), 0);
-  std::vector<int64_t> src_off((size_t)kPCount * B * 17, -1);
-  std::vector<const char*> src(B);
+  // host tables, laid out as in the workspace so that one copy carries them all
+  std::vector<char> tables(L.total, 0);
+  int* cum = reinterpret_cast<int*>(tables.data() + L.cum);
+  int* cum_ne = reinterpret_cast<int*>(tables.data() + L.cum_ne);
+  int64_t* src_off = reinterpret_cast<int64_t*>(tables.data() + L.src_off);
+  const char** src = reinterpret_cast<const char**>(tables.data() + L.src);
+  MergeSeg* segs = reinterpret_cast<MergeSeg*>(tables.data() + L.segs);
   const int props[kPCount] = {OCNN_KEY, OCNN_CHILD, OCNN_FEATURE, OCNN_LABEL, OCNN_SPLIT};
   for (int b = 0; b < B; ++b) {
     const Info* oi = as_info(infos[b]);
@@ -277,12 +358,65 @@ int ocnn_octree_batch(void* out_dev, const void* out_info, const void* const* oc
   }
   for (int d = 0; d <= depth; ++d)
     OCNN_REQUIRE(cum[d * (B + 1) + B] == o.nnum[d], OCNN_E_BADARG, "out_info disagrees with the inputs at depth %d", d);
+
+  // segments of the merge launch; what no segment and no neighbour kernel writes is cleared
+  // (the reference starts from a zeroed buffer, merge_octrees.cpp:109-113)
+  struct Span { int64_t at, bytes; };
+  std::vector<Span> written;
+  int n_seg = 0;
+  unsigned blocks = 0;
+  auto add_seg = [&](int kind, int d, int prop, int channel, int64_t dst_key, int64_t dst_child, int64_t count,
+                     int64_t items) {
+    if (items <= 0 || n_seg >= kMergeSegMax) return;
+    MergeSeg& g = segs[n_seg++];
+    g.kind = kind; g.depth = d; g.prop = prop; g.channel = channel;
+    g.first_block = blocks; g.dst_key = dst_key; g.dst_child = dst_child; g.count = count;
+    blocks += blocks_for(items);
+  };
+  add_seg(kMergeHeader, 0, 0, 0, 0, 0, 0, OCNN_HEADER_BYTES / 4);
+  const int fprops[3] = {OCNN_FEATURE, OCNN_LABEL, OCNN_SPLIT};
+  const int findex[3] = {kPFeature, kPLabel, kPSplit};
+  for (int d = depth; d >= 0; --d) {  // the large levels first
+    const int n_d = o.nnum[d];
+    if (n_d == 0) continue;
+    const int64_t k_off = o.has(OCNN_KEY) ? o.ptr_dis(OCNN_KEY, d) : -1;
+    const int64_t c_off = o.has(OCNN_CHILD) ? o.ptr_dis(OCNN_CHILD, d) : -1;
+    add_seg(kMergeKeyChild, d, 0, 0, k_off, c_off, n_d, n_d);
+    if (k_off >= 0) written.push_back({k_off, (int64_t)n_d * 8});
+    if (c_off >= 0) written.push_back({c_off, (int64_t)n_d * 4});
+    for (int q = 0; q < 3; ++q) {
+      if (!o.has(fprops[q])) continue;
+      if (o.location(fprops[q]) == depth && d != depth) continue;
+      const int ch = o.channel(fprops[q]);
+      add_seg(kMergeFloat, d, findex[q], ch, o.ptr_dis(fprops[q], d), -1, n_d, n_d);
+      written.push_back({o.ptr_dis(fprops[q], d), (int64_t)n_d * ch * 4});
+    }
+    if (d >= 1) written.push_back({o.ptr_dis(OCNN_NEIGH, d), (int64_t)n_d * 32});
+  }
+  std::sort(written.begin(), written.end(), [](const Span& x, const Span& y) { return x.at < y.at; });
+  {
+    int64_t at = OCNN_HEADER_BYTES;
+    const int64_t blob_end = o.sizeof_octree();
+    for (size_t i = 0; i <= written.size(); ++i) {
+      const int64_t next = i < written.size() ? written[i].at : blob_end;
+      if (next > at) add_seg(kMergeZero, 0, 0, 0, at, -1, (next - at) / 4, (next - at + 15) / 16);
+      if (i < written.size()) at = std::max(at, written[i].at + written[i].bytes);
+    }
+  }
+  OCNN_REQUIRE(n_seg < kMergeSegMax, OCNN_E_UNSUPPORTED, "too many segments to merge");
   char* ws = static_cast<char*>(workspace_dev);
-  OCNN_HIP_OK(hipMemcpyAsync(ws + L.cum, cum.data(), cum.size() * sizeof(int), hipMemcpyHostToDevice, s));
-  OCNN_HIP_OK(hipMemcpyAsync(ws + L.cum_ne, cum_ne.data(), cum_ne.size() * sizeof(int), hipMemcpyHostToDevice, s));
-  OCNN_HIP_OK(hipMemcpyAsync(ws + L.src_off, src_off.data(), src_off.size() * sizeof(int64_t), hipMemcpyHostToDevice, s));
-  OCNN_HIP_OK(hipMemcpyAsync(ws + L.src, src.data(), src.size() * sizeof(char*), hipMemcpyHostToDevice, s));
-  OCNN_HIP_OK(hipStreamSynchronize(s));  // the tables above are host memory of this call
+  // The tables travel through a pinned staging buffer that is handed back when the stream has
+  // passed the copy, so the call does not wait for the device.
+  Staging* stage = take_staging(L.total);
+  OCNN_REQUIRE(stage, OCNN_E_HIP, "no pinned host memory for the merge tables");
+  memcpy(stage->host, tables.data(), L.total);
+  hipError_t ce = hipMemcpyAsync(ws, stage->host, L.total, hipMemcpyHostToDevice, s);
+  if (ce == hipSuccess) ce = hipEventRecord(stage->done, s);
+  if (ce != hipSuccess) {
+    (void)hipStreamSynchronize(s);
+    stage->busy = false;
+    return fail(OCNN_E_HIP, "merge tables: %s", hipGetErrorString(ce));
+  }
   MergeTable m;
   m.cum = reinterpret_cast<const int*>(ws + L.cum);
   m.cum_ne = reinterpret_cast<const int*>(ws + L.cum_ne);
@@ -291,26 +425,12 @@ int ocnn_octree_batch(void* out_dev, const void* out_info, const void* const* oc
   m.B = B;
 
   char* blob = static_cast<char*>(out_dev);
-  int e = zero_payload(blob, o, s);
-  if (e) return e;
-  e = write_header(blob, o, s);
-  if (e) return e;
-  for (int d = 0; d <= depth; ++d) {
-    int n_d = o.nnum[d];
-    if (n_d == 0) continue;
-    uint64_t* key = o.has(OCNN_KEY) ? reinterpret_cast<uint64_t*>(blob + o.ptr_dis(OCNN_KEY, d)) : nullptr;
-    int* child = o.has(OCNN_CHILD) ? reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_CHILD, d)) : nullptr;
-    merge_key_child_kernel<<<blocks_for(n_d), kBlock, 0, s>>>(key, child, d, n_d, m);
-    const int fprops[3] = {OCNN_FEATURE, OCNN_LABEL, OCNN_SPLIT};
-    const int findex[3] = {kPFeature, kPLabel, kPSplit};
-    for (int q = 0; q < 3; ++q) {
-      if (!o.has(fprops[q])) continue;
-      if (o.location(fprops[q]) == depth && d != depth) continue;
-      merge_float_kernel<<<blocks_for(n_d), kBlock, 0, s>>>(
-          reinterpret_cast<float*>(blob + o.ptr_dis(fprops[q], d)), findex[q], o.channel(fprops[q]), d, n_d, m);
-    }
-    OCNN_LAUNCH_OK("merge");
-  }
+  HeaderArg h;
+  memset(&h, 0, sizeof(h));
+  memcpy(&h, &o, sizeof(Info));
+  merge_kernel<<<blocks, kBlock, 0, s>>>(blob, m, reinterpret_cast<const MergeSeg*>(ws + L.segs), n_seg, h);
+  OCNN_LAUNCH_OK("merge");
+  int e = OCNN_OK;
   OCNN_REQUIRE(o.has(OCNN_CHILD), OCNN_E_FORMAT, "octrees without child links cannot get neighbour tables");
   for (int d = 1; d <= depth; ++d) {
     int* neigh = reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_NEIGH, d));
