@@ -34,26 +34,135 @@ __global__ void fill_kernel(T* p, int64_t n, T v) {
 }
 
 // ---- pad / depad -----------------------------------------------------------
+// A workgroup takes kPadTile rows of the padded side and kChanChunk channels; the labels of
+// the tile sit in LDS.  A feature row starts anywhere inside a 256-byte line, and a
+// wavefront store that straddles a line boundary costs almost twice an aligned one, so
+// every channel walks the tile rotated by its own amount: wavefronts store whole lines and
+// only the two ends of the tile are partial.
+constexpr int kPadTile = 1024;
+
 template <typename T>
-__global__ void pad_forward_kernel(T* __restrict__ Y, int Hy, int C, const T* __restrict__ X,
-    int Hx, const int* __restrict__ label, T dval) {
-  int h = blockIdx.x * blockDim.x + threadIdx.x;
-  if (h >= Hy) return;
-  int l = label[h];
-  int c0 = blockIdx.y * kChanChunk, c1 = min(C, c0 + kChanChunk);
-  for (int c = c0; c < c1; ++c)
-    Y[(int64_t)c * Hy + h] = (l < 0 || l >= Hx) ? dval : X[(int64_t)c * Hx + l];
+__device__ inline int line_rotation(const T* row) {  // elements up to the next 64-element boundary
+  return (int)((0 - (reinterpret_cast<uintptr_t>(row) / sizeof(T))) & 63);
 }
 
 template <typename T>
-__global__ void pad_backward_kernel(T* __restrict__ X, int Hx, int C, const T* __restrict__ Y,
-    int Hy, const int* __restrict__ label) {
-  int h = blockIdx.x * blockDim.x + threadIdx.x;
-  if (h >= Hy) return;
-  int l = label[h];
-  if (l < 0 || l >= Hx) return;  // rows outside X are ignored rather than written
-  int c0 = blockIdx.y * kChanChunk, c1 = min(C, c0 + kChanChunk);
-  for (int c = c0; c < c1; ++c) X[(int64_t)c * Hx + l] = Y[(int64_t)c * Hy + h];
+__global__ void __launch_bounds__(kBlock) pad_forward_kernel(T* __restrict__ Y, int Hy, int C,
+    const T* __restrict__ X, int Hx, const int* __restrict__ label, T dval) {
+  __shared__ int s_l[kPadTile];
+  const int tid = threadIdx.x;
+  const int tile0 = blockIdx.x * kPadTile;
+  const int rows = min(kPadTile, Hy - tile0);
+#pragma unroll
+  for (int q = 0; q < kPadTile / kBlock; ++q) {
+    const int r = q * kBlock + tid;
+    const int l = r < rows ? label[tile0 + r] : -1;
+    s_l[r] = (l < 0 || l >= Hx) ? -1 : l;
+  }
+  __syncthreads();
+  for (int c = blockIdx.y; c < C; c += gridDim.y) {  // channels dealt out over blockIdx.y
+    T* row = Y + (int64_t)c * Hy + tile0;
+    const T* xin = X + (int64_t)c * Hx;
+    const int rot = line_rotation(row);
+    T v[kPadTile / kBlock];
+    int at[kPadTile / kBlock];
+#pragma unroll
+    for (int q = 0; q < kPadTile / kBlock; ++q) {
+      const int r = (q * kBlock + tid + rot) & (kPadTile - 1);
+      at[q] = r < rows ? r : -1;
+      const int l = r < rows ? s_l[r] : -1;
+      v[q] = l < 0 ? dval : xin[l];
+    }
+#pragma unroll
+    for (int q = 0; q < kPadTile / kBlock; ++q)
+      if (at[q] >= 0) row[at[q]] = v[q];
+  }
+}
+
+// X[c, label[h]] = Y[c, h].  The labels of a tile normally are consecutive numbers in
+// ascending order (they are ranks of non-empty nodes), so the tile owns one contiguous piece
+// of X: the workgroup inverts the labels in LDS and stores that piece densely.  A tile whose
+// labels are anything else (gaps, repeats, a wide spread) is scattered row by row instead.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) pad_backward_kernel(T* __restrict__ X, int Hx, int C,
+    const T* __restrict__ Y, int Hy, const int* __restrict__ label) {
+  __shared__ int s_l[kPadTile];
+  __shared__ int s_h[kPadTile];
+  __shared__ int s_lo[kBlock / 64], s_hi[kBlock / 64];
+  const int tid = threadIdx.x;
+  const int tile0 = blockIdx.x * kPadTile;
+  const int rows = min(kPadTile, Hy - tile0);
+  int lo = 0x7fffffff, hi = -1;
+#pragma unroll
+  for (int q = 0; q < kPadTile / kBlock; ++q) {
+    const int r = q * kBlock + tid;
+    int l = r < rows ? label[tile0 + r] : -1;
+    if (l < 0 || l >= Hx) l = -1;  // rows outside X are ignored rather than written
+    s_l[r] = l;
+    s_h[r] = -1;
+    if (l >= 0) { lo = min(lo, l); hi = max(hi, l); }
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    lo = min(lo, __shfl_xor(lo, off));
+    hi = max(hi, __shfl_xor(hi, off));
+  }
+  if ((tid & 63) == 0) { s_lo[tid >> 6] = lo; s_hi[tid >> 6] = hi; }
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < kBlock / 64; ++w) { lo = min(lo, s_lo[w]); hi = max(hi, s_hi[w]); }
+  if (hi < 0) return;  // nothing of this tile lands in X
+  const int span = hi - lo + 1;
+  bool dense = span <= kPadTile;
+  if (dense) {
+#pragma unroll
+    for (int q = 0; q < kPadTile / kBlock; ++q) {
+      const int r = q * kBlock + tid;
+      if (s_l[r] >= 0) s_h[s_l[r] - lo] = r;
+    }
+    __syncthreads();
+    bool all_set = true;
+#pragma unroll
+    for (int q = 0; q < kPadTile / kBlock; ++q) {
+      const int i = q * kBlock + tid;
+      if (i < span && s_h[i] < 0) all_set = false;
+    }
+    dense = __syncthreads_and(all_set) != 0;
+    // a label named twice leaves a gap elsewhere, so `dense` also means: no repeats
+  }
+  for (int c0 = blockIdx.y * kChanChunk; c0 < C; c0 += gridDim.y * kChanChunk) {  // chunks dealt out
+  const int c1 = min(C, c0 + kChanChunk);
+  if (dense) {
+    // the piece of X is a quarter of the tile or less on a sparse level, so the loads that
+    // can be in flight are the channels' rather than the rows': all channels of a row first
+    const T* yin = Y + (int64_t)c0 * Hy + tile0;
+    T* row0 = X + (int64_t)c0 * Hx + lo;
+    for (int q = 0; q * kBlock < span + 64; ++q) {
+      T v[kChanChunk];
+      int at[kChanChunk];
+#pragma unroll
+      for (int j = 0; j < kChanChunk; ++j) {
+        const int rot = line_rotation(row0 + (int64_t)j * Hx);
+        const int i = q * kBlock + tid - ((64 - rot) & 63);  // wavefronts start on line boundaries
+        at[j] = (c0 + j < c1 && i >= 0 && i < span) ? i : -1;
+        if (at[j] >= 0) v[j] = yin[(int64_t)j * Hy + s_h[i]];
+      }
+#pragma unroll
+      for (int j = 0; j < kChanChunk; ++j)
+        if (at[j] >= 0) row0[(int64_t)j * Hx + at[j]] = v[j];
+    }
+  } else {
+    for (int c = c0; c < c1; ++c) {
+      const T* yin = Y + (int64_t)c * Hy + tile0;
+      T* xout = X + (int64_t)c * Hx;
+#pragma unroll
+      for (int q = 0; q < kPadTile / kBlock; ++q) {
+        const int r = q * kBlock + tid;
+        if (s_l[r] >= 0) xout[s_l[r]] = yin[r];
+      }
+    }
+  }
+  }
 }
 
 __global__ void make_ichild_kernel(int* __restrict__ ichild, int n_nempty,
@@ -539,7 +648,10 @@ int ocnn_pad_forward(void* Y, int Hy, int C, const void* X, int Hx, const int* l
   OCNN_REQUIRE(Y && label && (X || Hx == 0), OCNN_E_BADARG, "null pointer");
   OCNN_REQUIRE(Hy >= 0 && Hx >= 0 && C > 0, OCNN_E_BADARG, "Hy %d Hx %d C %d", Hy, Hx, C);
   if (Hy == 0) return OCNN_OK;
-  dim3 grid(blocks_for(Hy), (C + kChanChunk - 1) / kChanChunk);
+  // the labels of a tile are staged once per workgroup: few workgroups per tile when there
+  // are many tiles
+  const unsigned tiles = blocks_for(Hy, kPadTile);
+  dim3 grid(tiles, std::min<unsigned>(C, std::max(1u, 4096u / tiles)));
   hipStream_t s = as_stream(stream);
   if (dtype == OCNN_F32)
     pad_forward_kernel<float><<<grid, kBlock, 0, s>>>((float*)Y, Hy, C, (const float*)X, Hx, label, dval);
@@ -561,7 +673,8 @@ int ocnn_pad_backward(void* X, int Hx, int C, const void* Y, int Hy, const int* 
   OCNN_REQUIRE(label && (X || Hx == 0) && (Y || Hy == 0), OCNN_E_BADARG, "null pointer");
   OCNN_REQUIRE(Hy >= 0 && Hx >= 0 && C > 0, OCNN_E_BADARG, "Hy %d Hx %d C %d", Hy, Hx, C);
   if (Hy == 0 || Hx == 0) return OCNN_OK;
-  dim3 grid(blocks_for(Hy), (C + kChanChunk - 1) / kChanChunk);
+  const unsigned tiles = blocks_for(Hy, kPadTile), chunks = (C + kChanChunk - 1) / kChanChunk;
+  dim3 grid(tiles, std::min(chunks, std::max(1u, 2048u / tiles)));
   hipStream_t s = as_stream(stream);
   if (dtype == OCNN_F32)
     pad_backward_kernel<float><<<grid, kBlock, 0, s>>>((float*)X, Hx, C, (const float*)Y, Hy, label);

@@ -408,6 +408,54 @@ def test_pool_pad_vs_oracle(oc, orc, tree, dtype):
   assert e.value.code == -3
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_pad_any_labels(oc, orc, dtype):
+  """pad_forward / pad_backward through the C-ABI (octree_nn.cpp:163-185) with label arrays that are
+  not the ascending ranks an octree has: shuffled, with gaps, out of range, a wide spread inside one
+  tile, several tiles, unaligned rows; rows of X that no label names keep their old content."""
+  import ctypes as C
+  rng = np.random.default_rng(5)
+  P = lambda t, off=0: C.c_void_p(t.data_ptr() + off)
+  st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+  dt = 0 if dtype == torch.float32 else 1
+  Cc = 11
+  cases = []
+  Hy, Hx = 5000, 1300
+  lab = np.full(Hy, -1, np.int32)
+  pos = np.sort(rng.choice(Hy, Hx, replace=False))
+  lab[pos] = np.arange(Hx)                                   # an octree's kind of labels
+  cases.append(("ranks", lab.copy(), Hx))
+  lab2 = lab.copy(); lab2[pos] = rng.permutation(Hx)          # distinct, any order
+  cases.append(("shuffled", lab2, Hx))
+  lab3 = lab.copy(); lab3[pos[::7]] = -1; lab3[pos[3::11]] = Hx + 5   # gaps and rows outside X
+  cases.append(("gaps", lab3, Hx))
+  lab4 = np.full(Hy, -1, np.int32); lab4[pos] = np.arange(Hx) * 3     # wide spread
+  cases.append(("spread", lab4, 3 * Hx))
+  for name, l, hx in cases:
+    x = (rng.integers(-8, 8, (Cc, hx)) / 2).astype(np.float32)
+    y = (rng.integers(-8, 8, (Cc, Hy)) / 2).astype(np.float32)
+    l_d = T(l).cuda()
+    # forward, into a buffer that starts 3 elements past a line boundary
+    ybuf = torch.full((Cc * Hy + 8,), 9.0, device="cuda", dtype=dtype)
+    x_d = T(x).cuda().to(dtype)
+    es = ybuf.element_size()
+    oc.lib.call("ocnn_pad_forward", P(ybuf, 3 * es), Hy, Cc, P(x_d), hx, P(l_d), C.c_float(1.5), dt, st)
+    exp = np.where((l >= 0) & (l < hx), x[:, np.clip(l, 0, hx - 1)], np.float32(1.5))
+    got = ybuf.float().cpu().numpy()
+    assert np.array_equal(got[3:3 + Cc * Hy].reshape(Cc, Hy), exp), name
+    assert np.all(got[:3] == 9.0) and np.all(got[3 + Cc * Hy:] == 9.0), name
+    # backward: rows of X named by a label take the row of Y, the others stay
+    xbuf = torch.full((Cc * hx + 8,), 7.0, device="cuda", dtype=dtype)
+    y_d = T(y).cuda().to(dtype)
+    oc.lib.call("ocnn_pad_backward", P(xbuf, 5 * es), hx, Cc, P(y_d), Hy, P(l_d), dt, st)
+    expx = np.full((Cc, hx), 7.0, np.float32)
+    ok = (l >= 0) & (l < hx)
+    expx[:, l[ok]] = y[:, ok]
+    gotx = xbuf.float().cpu().numpy()
+    assert np.array_equal(gotx[5:5 + Cc * hx].reshape(Cc, hx), expx), name
+    assert np.all(gotx[:5] == 7.0) and np.all(gotx[5 + Cc * hx:] == 7.0), name
+
+
 def test_full_size_properties(oc, synthetic):
   """Size-independent properties on the depth-9 scene of BASELINE config 4: linearity of
   the convolution, unpool/mask-pool round trip, depad(pad(x)) == x."""
