@@ -531,7 +531,9 @@ __global__ void pack_weights_lds_f32(float* __restrict__ Wt, const float* __rest
 // 50 KiB per workgroup: three workgroups per CU.  Unit index of slot (x,y,z):
 //   (x&1) | (y&1)<<1 | (z&1)<<2 | (y>>1)<<3 | (z>>1)<<4
 // so the 8 siblings of a group (consecutive lanes) always read 8 different 16-byte units;
-// odd groups store unit u at u ^ 8 (see the kernel).
+// odd groups store unit u at u ^ 8 and the second channel half at u ^ 1 (see the kernel):
+// with that, and the staging lanes ordered by the unit bits, no read or write of the kernel
+// meets a bank conflict (SQ_LDS_BANK_CONFLICT = 0 on the depth-9 scene).
 constexpr int kB16Half = 32 * 32;  // 16-byte units per 8-channel half
 
 __device__ inline int b16_unit(int x, int y, int z) {
@@ -595,8 +597,12 @@ __global__ __launch_bounds__(256, 2) void conv_s1_bf16_lds_kernel(ConvArgs a, ui
   const int npass = (a.mtiles + MT - 1) / MT;
 
   // staging role of this lane: half s_kh, (y,z) = s_yz, groups 8*wave + 2*j + s_g (j = 0..3)
-  const int s_kh = lane & 1, s_yz = (lane >> 1) & 15, s_g = lane >> 5;
-  const int s_y = s_yz >> 2, s_z = s_yz & 3;
+  // lane bits 1..4 are (y&1, z&1, y>>1, z>>1): sixteen consecutive lanes then write sixteen
+  // different 16-byte units of one 256-byte row of banks (see the unit index above; the
+  // second channel half keeps its units with bit 0 flipped)
+  const int s_kh = lane & 1, s_g = lane >> 5;
+  const int s_y = ((lane >> 1) & 1) | (((lane >> 3) & 1) << 1), s_z = ((lane >> 2) & 1) | (((lane >> 4) & 1) << 1);
+  const int s_yz = (s_y << 2) | s_z;
   int nb[4][4];  // [j][x-layer] neighbour row (H = the zero row)
   const int group0 = (tile * kTileCols) / 8 + wave * 8;
   const int n_groups = a.N >> 3;
@@ -617,7 +623,7 @@ __global__ __launch_bounds__(256, 2) void conv_s1_bf16_lds_kernel(ConvArgs a, ui
   // Odd groups keep their units with bit 3 flipped: a 16-byte LDS read is served sixteen lanes
   // (two sibling groups) at a time, and the blocks of two groups, 512 bytes apart, would meet in
   // the same banks.
-  const int gswz = ((r >> 3) & 1) << 3;
+  const int gswz = (((r >> 3) & 1) << 3) ^ kh;
 
   for (int pass = blockIdx.y; pass < npass; pass += gridDim.y) {  // passes may be dealt out over workgroups
     floatx16 acc[MT][2];
@@ -659,7 +665,7 @@ __global__ __launch_bounds__(256, 2) void conv_s1_bf16_lds_kernel(ConvArgs a, ui
         }                                                                                      \
       }                                                                                        \
       _Pragma("unroll") for (int j = 0; j < 4; ++j)                                            \
-        sX[s_kh * kB16Half + (wave * 8 + 2 * j + s_g) * 32 + (b16_unit(L, s_y, s_z) ^ (s_g << 3))] = xr[(L) & 1][j]; \
+        sX[s_kh * kB16Half + (wave * 8 + 2 * j + s_g) * 32 + (b16_unit(L, s_y, s_z) ^ (s_g << 3) ^ s_kh)] = xr[(L) & 1][j]; \
       __syncthreads();                                                                         \
       /* weights of the next computing phase: phase L requests those of dx = L */            \
       if ((L) <= 2) OCNN_FETCH_W(SLAB, L);                                                     \
