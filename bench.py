@@ -398,6 +398,13 @@ def main():
     f16 = feat9.bfloat16()
     t = timed(lambda: oc.stacks.unet_trunk(octree, 9, up16, data=f16), max(2, reps // 2), 1)
     extra["unet_trunk_scene_d9_bf16"] = {"ms": t, "points_per_s": 250000 / (t * 1e-3)}
+    # the same trunk over the non-empty nodes only (the reference's ScanNet setting)
+    fne = F.octree_depad(feat9, octree, 9)
+    fne16 = fne.bfloat16()
+    t = timed(lambda: oc.stacks.unet_trunk(octree, 9, up, data=fne, nempty=True), max(2, reps // 2), 1)
+    extra["unet_trunk_scene_d9_f32_nempty"] = {"ms": t, "points_per_s": 250000 / (t * 1e-3)}
+    t = timed(lambda: oc.stacks.unet_trunk(octree, 9, up16, data=fne16, nempty=True), max(2, reps // 2), 1)
+    extra["unet_trunk_scene_d9_bf16_nempty"] = {"ms": t, "points_per_s": 250000 / (t * 1e-3)}
     clouds2 = [points_tensor(*oc.synthetic.shape_cloud(10000, 100 + i)) for i in range(32)]
     oct6 = F.points2octree_batch(clouds2, 6, 2)
     lch = {6: (3, 32), 5: (32, 64), 4: (64, 128), 3: (128, 256)}
