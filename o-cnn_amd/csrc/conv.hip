@@ -147,7 +147,7 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
     const float4* __restrict__ xt, const float* __restrict__ Wt, int n_tiles, int cpad) {
   constexpr int kWWords = (kRowSlab / 8) * 4 * MT * 64;  // weights of one (tap, slab)
   constexpr int kWVec = kWWords / 4 / 256;               // float4 per thread (4 for MT = 2)
-  __shared__ __attribute__((aligned(16))) float sW[kWWords];
+  __shared__ __attribute__((aligned(16))) float sW[2 * kWWords];  // double buffered: one barrier per stage
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int tile = xcd_tile(blockIdx.x, n_tiles);
   if (tile >= n_tiles) return;
@@ -191,14 +191,24 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
     int s0n = src_of(1, 0), s1n = src_of(1, 1);      // ... of the next one
     fetch_w(0);
     fetch_x(s0c, s1c, 0);
+    __syncthreads();  // the last stage of the previous pass may still be reading the weights
+#pragma unroll
+    for (int v = 0; v < kWVec; ++v) reinterpret_cast<float4*>(sW)[v * 256 + threadIdx.x] = wr[v];
+    if (1 < nstage) fetch_w(1);
     int stage = 0;
     for (int k = 0; k < a.K; ++k) {
       const int s0n2 = src_of(k + 2, 0), s1n2 = src_of(k + 2, 1);
       for (int slab = 0; slab < nslab; ++slab, ++stage) {
+        // stage - 1 is over everywhere and the weights of this stage are in place; the weights
+        // of the next stage (requested a stage ago) go into the other buffer while this one is
+        // read, those of the stage after that are requested
         __syncthreads();
+        const float* wcur = sW + (stage & 1) * kWWords;
+        if (stage + 1 < nstage) {
 #pragma unroll
-        for (int v = 0; v < kWVec; ++v) reinterpret_cast<float4*>(sW)[v * 256 + threadIdx.x] = wr[v];
-        __syncthreads();
+          for (int v = 0; v < kWVec; ++v)
+            reinterpret_cast<float4*>(sW + ((stage + 1) & 1) * kWWords)[v * 256 + threadIdx.x] = wr[v];
+        }
         // group c8 of the NEXT stage is requested right after group c8 of this one has been read
         // out of its registers, so every gather has seven eighths of a stage to arrive
         const bool more = stage + 1 < nstage;
@@ -208,7 +218,7 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
         const float4* nrow0 = xt + (int64_t)(s0x < 0 ? a.Hin : s0x) * cpad4 + kh + ((nslab_next * kRowSlab) >> 2);
         const float4* nrow1 = xt + (int64_t)(s1x < 0 ? a.Hin : s1x) * cpad4 + kh + ((nslab_next * kRowSlab) >> 2);
         const int ngroup_next = more ? (min(kRowSlab, cpad - nslab_next * kRowSlab) >> 3) : 0;
-        if (more) fetch_w(stage + 1);
+        if (stage + 2 < nstage) fetch_w(stage + 2);
         const int ngroup = min(kRowSlab, cpad - slab * kRowSlab) >> 3;
 #pragma unroll
         for (int c8 = 0; c8 < kRowSlab / 8; ++c8) {
@@ -224,7 +234,7 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
             const float v1 = j == 0 ? b1.x : j == 1 ? b1.y : j == 2 ? b1.z : b1.w;
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-              const float av = sW[((c8 * 4 + j) * MT + mt) * 64 + lane];
+              const float av = wcur[((c8 * 4 + j) * MT + mt) * 64 + lane];
               acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, v0, acc[mt][0], 0, 0, 0);
               acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, v1, acc[mt][1], 0, 0, 0);
             }
