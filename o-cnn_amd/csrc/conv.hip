@@ -384,15 +384,18 @@ __global__ void pack_weights_rows_bf16(uint16_t* __restrict__ Wt, const uint16_t
 //
 // Workgroup = 4 wavefronts = 256 columns = 32 sibling groups; wavefront w owns groups
 // 8w .. 8w+7 (its own 64 columns), stages only those, and computes all output channels of
-// a pass (MT row tiles).  The channel loop runs in slabs of kSlab = 4 input channels:
+// a pass (MT row tiles).  The channel loop runs in slabs of kSlab = 2 input channels (one MFMA
+// k-step per tap; short slabs keep a workgroup at 34 KiB of LDS and 164 VGPRs, so that three
+// workgroups share a CU and fill one another's barrier gaps):
 //   LDS X [kSlab][32 groups][80]  fp32: the neighbour blocks (wavefront-private parts)
-//   LDS W [K][2][MT][64]          fp32: the slab's weights in A-fragment order (shared)
+//   LDS W [K][kSlab/2][MT][64]    fp32: the slab's weights in A-fragment order (shared)
 // Group g sits at word 80*g + {0,2,8,10}[g&3]: with that skew the 32 lanes of a half
 // wavefront (4 groups x 8 siblings, sibling offsets {0,1,4,5,16,17,20,21}) hit 32
 // different banks for every tap.
 // The next slab's gathers and weights are issued before the MFMA loop of the current
 // slab and land in LDS after it, so their latency hides behind ~14k cycles of MFMA.
-constexpr int kSlab = 4;
+constexpr int kSlab = 2;
+constexpr int kKSteps = kSlab / 2;  // MFMA k-steps (two channels each) per slab
 constexpr int kGroupStride = 80;
 constexpr int kPlane = 32 * kGroupStride;   // words per channel plane
 
@@ -401,9 +404,9 @@ __device__ inline int group_base(int g) {
 }
 
 template <int MT, int K>
-__global__ __launch_bounds__(256, 2) void conv_s1_f32_lds_kernel(ConvArgs a, float* __restrict__ out,
+__global__ __launch_bounds__(256, 3) void conv_s1_f32_lds_kernel(ConvArgs a, float* __restrict__ out,
     const float* __restrict__ in, const float* __restrict__ Wt, int n_tiles) {
-  constexpr int kWWords = K * 2 * MT * 64;          // weight words per (pass, slab)
+  constexpr int kWWords = K * kKSteps * MT * 64;          // weight words per (pass, slab)
   constexpr int kWVec = (kWWords / 4 + 255) / 256;  // float4 loads per thread
   __shared__ float sX[kSlab * kPlane];
   __shared__ __attribute__((aligned(16))) float sW[kWWords];
@@ -490,12 +493,12 @@ __global__ __launch_bounds__(256, 2) void conv_s1_f32_lds_kernel(ConvArgs a, flo
           const int k = kxy * 3 + kz;
           const int slot = mirrored ? 42 - (s3 | kz) : (s3 | kz);
 #pragma unroll
-          for (int ks = 0; ks < 2; ++ks) {
+          for (int ks = 0; ks < kKSteps; ++ks) {
             float b0 = sX[boff[0] + ks * 2 * kPlane + slot];
             float b1 = sX[boff[1] + ks * 2 * kPlane + slot];
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-              float av = sW[((k * 2 + ks) * MT + mt) * 64 + lane];
+              float av = sW[((k * kKSteps + ks) * MT + mt) * 64 + lane];
               acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b0, acc[mt][0], 0, 0, 0);
               acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b1, acc[mt][1], 0, 0, 0);
             }
@@ -511,12 +514,12 @@ __global__ __launch_bounds__(256, 2) void conv_s1_f32_lds_kernel(ConvArgs a, flo
 __global__ void pack_weights_lds_f32(float* __restrict__ Wt, const float* __restrict__ W, int M, int Cin, int K,
     int MT, int npass, int nslab, int64_t sm, int64_t sc) {
   int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  int64_t total = (int64_t)npass * nslab * K * 2 * MT * 64;
+  int64_t total = (int64_t)npass * nslab * K * kKSteps * MT * 64;
   if (id >= total) return;
   int l = (int)(id & 63);
   int64_t f = id >> 6;
   int mt = (int)(f % MT); f /= MT;
-  int ks = (int)(f % 2); f /= 2;
+  int ks = (int)(f % kKSteps); f /= kKSteps;
   int k = (int)(f % K); f /= K;
   int slab = (int)(f % nslab);
   int pass = (int)(f / nslab);
@@ -1169,7 +1172,7 @@ int make_plan(const Info* o, int depth, int channel_in, int num_output, const in
     p->xt_general = align256(((size_t)p->btm_h + 1) * cpad * (dtype == OCNN_F32 ? 4 : 2));
   }
   if (dtype == OCNN_F32) {  // the LDS kernel pads channels to slabs of 4 and row tiles to passes
-    size_t lds_words = (size_t)((p->mtiles + 1) / 2) * ((channel_in + kSlab - 1) / kSlab) * p->taps.count * 2 * 2 * 64;
+    size_t lds_words = (size_t)((p->mtiles + 1) / 2) * ((channel_in + kSlab - 1) / kSlab) * p->taps.count * kKSteps * 2 * 64;
     p->wt_bytes = align256(lds_words * sizeof(float) > p->wt_bytes ? lds_words * sizeof(float) : p->wt_bytes);
   }
   p->ichild_bytes = nempty ? align256(sizeof(int) * (size_t)(p->ichild_h + 1)) : 0;
@@ -1303,7 +1306,7 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
   } else if (dtype == OCNN_F32 && a.mode == kModeS1 && !a.nempty && a.K == 27) {
     const int MT = a.mtiles == 1 ? 1 : 2;
     const int npass = (a.mtiles + MT - 1) / MT, nslab = (a.Cin + kSlab - 1) / kSlab;
-    int64_t total = (int64_t)npass * nslab * a.K * 2 * MT * 64;
+    int64_t total = (int64_t)npass * nslab * a.K * kKSteps * MT * 64;
     pack_weights_lds_f32<<<blocks_for(total), kBlock, 0, s>>>((float*)wsb, (const float*)weights, a.M, a.Cin, a.K,
         MT, npass, nslab, sm, sc);
     OCNN_LAUNCH_OK("pack_weights_lds");
