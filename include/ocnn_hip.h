@@ -177,8 +177,7 @@ int ocnn_octree_conv_fused(void* top, const void* btm, int channel_in, int btm_h
  * the shapes of `data_in` and `weights`.  Either result pointer may be NULL to skip it.
  * The weight gradient contracts over the octree nodes on the matrix cores without a column
  * buffer and adds its partial sums in a fixed order (reproducible); the data gradient is the
- * transposed operator with the same weight buffer.  fp32 only (OCNN_E_UNSUPPORTED otherwise);
- * a stride-2 convolution's data gradient exists for the 2x2x2 kernel only. */
+ * transposed operator with the same weight buffer.  fp32 only (OCNN_E_UNSUPPORTED otherwise). */
 int ocnn_conv_grad_workspace_bytes(const void* info, int depth, int channel_in, int num_output,
     const int* kernel_size, int stride, int nempty, int is_deconv, int dtype, size_t* workspace_bytes);
 int ocnn_octree_conv_grad(void* grad_data, void* grad_weights, const void* data_in, int channel_in,

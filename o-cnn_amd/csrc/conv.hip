@@ -21,7 +21,7 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));  // one 16-byte LDS / global unit
 
-enum { kModeS1 = 0, kModeS2Conv = 1, kModeS2Deconv = 2 };
+enum { kModeS1 = 0, kModeS2Conv = 1, kModeS2Deconv = 2, kModeS2DeconvAny = 3 };
 
 struct ConvArgs {
   int M, Cin, N, K;     // output channels, input channels, output columns, taps
@@ -48,11 +48,35 @@ constexpr int kWaveCols = 64;                 // output columns per wavefront
 constexpr int kConvWaves = 4;                 // wavefronts per workgroup
 constexpr int kTileCols = kWaveCols * kConvWaves;
 
+// Stride-2 deconvolution with any tap set, seen from an output node.  Column h (a sibling
+// group of the output level, i.e. a non-empty node of the input level) scatters through tap
+// t to the node at offset t - 1 from its first sibling (col2octree, octree_nn.cpp:216-241).
+// Per axis a node with sibling bit s is reached from its own group by tap s + 1, and, when
+// s = 1, from the group two cells further by tap 0; any other tap does not reach it.  The
+// first sibling of that other group sits in the node's own 4x4x4 block at coordinate 3.
+__device__ inline int deconv_s2_source(const int* __restrict__ neigh, int node, int tap_slot_k) {
+  const int s = node & 7;
+  int slot = 0;
+#pragma unroll
+  for (int axis = 0; axis < 3; ++axis) {
+    const int t = (tap_slot_k >> (4 - 2 * axis)) & 3, sb = (s >> (2 - axis)) & 1;
+    int c;
+    if (t == sb + 1) c = 1;
+    else if (sb == 1 && t == 0) c = 3;
+    else return -1;
+    slot = (slot << 2) | c;
+  }
+  const int q = neigh[((int64_t)(node >> 3) << 6) + slot];
+  return q >= 0 ? q >> 3 : -1;
+}
+
 // source row of output column n for tap k (-1: contributes zero)
 __device__ inline int conv_src(const ConvArgs& a, int n, int k) {
   if (n >= a.N) return -1;
   int p;
-  if (a.mode == kModeS1) {
+  if (a.mode == kModeS2DeconvAny) {
+    p = deconv_s2_source(a.neigh, a.nempty ? a.ichild[n] : n, a.slot[k]);
+  } else if (a.mode == kModeS1) {
     int node = a.nempty ? a.ichild[n] : n;
     p = a.neigh[((int64_t)(node >> 3) << 6) + sibling_slot(node & 7) + a.slot[k]];
     if (a.nempty && p >= 0) p = a.child[p];
@@ -1156,11 +1180,7 @@ int make_plan(const Info* o, int depth, int channel_in, int num_output, const in
   p->ichild_h = o->nnum_nempty[p->workspace_depth];
   if (stride == 1) p->mode = kModeS1;
   else if (!deconv) p->mode = kModeS2Conv;
-  else {
-    OCNN_REQUIRE(ks[0] == 2 && ks[1] == 2 && ks[2] == 2, OCNN_E_UNSUPPORTED,
-        "stride-2 deconvolution is implemented for the 2x2x2 kernel only");
-    p->mode = kModeS2Deconv;
-  }
+  else p->mode = (ks[0] == 2 && ks[1] == 2 && ks[2] == 2) ? kModeS2Deconv : kModeS2DeconvAny;
   p->mtiles = (num_output + 31) / 32;
   p->csteps = 0;
   {  // general row-major gather path: padded weights + the row-major copy of the input
@@ -1235,7 +1255,7 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     int tap = k < p.taps.count ? p.taps.tap[k] : 13;
     // deconvolution gathers through the mirrored offset: the rows h that scatter
     // to p through tap k are exactly the neighbours of p at the opposite offset
-    a.slot[k] = tap_slot(deconv ? 26 - tap : tap);
+    a.slot[k] = tap_slot(deconv && stride == 1 ? 26 - tap : tap);
   }
   a.neigh = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_NEIGH, p.workspace_depth));
   a.child = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_CHILD, p.workspace_depth));

@@ -28,7 +28,8 @@ def tree(oc, orc, synthetic):
 
 
 CASES = [([3, 3, 3], 1, False), ([3, 3, 3], 1, True), ([2, 2, 2], 2, False), ([2, 2, 2], 2, True),
-         ([3, 1, 1], 1, False), ([1, 1, 1], 1, False), ([3, 3, 1], 1, True)]
+         ([3, 1, 1], 1, False), ([1, 1, 1], 1, False), ([3, 3, 1], 1, True),
+         ([3, 3, 3], 2, False), ([3, 3, 3], 2, True), ([3, 1, 3], 2, False), ([1, 1, 1], 2, True)]
 
 
 @pytest.mark.parametrize("ks,stride,nempty", CASES)

@@ -218,7 +218,7 @@ def test_conv_vs_oracle(oc, orc, tree, ks, stride, nempty):
     assert relerr(got16.float().cpu().numpy().reshape(exp.shape), exp) < TOL_BF16
 
 
-DECONV_CASES = [(ks, 1, ne) for ks in KERNELS for ne in (False, True)] + [([2, 2, 2], 2, False), ([2, 2, 2], 2, True)]
+DECONV_CASES = [(ks, s, ne) for ks in KERNELS for s in (1, 2) for ne in (False, True)]
 
 
 @pytest.mark.parametrize("ks,stride,nempty", DECONV_CASES)
@@ -281,8 +281,7 @@ def test_conv_on_reference_sample_batch(oc, orc, tree):
       assert relerr(y1.detach().cpu().numpy().reshape(exp.shape), exp) < TOL_F32
       # gradients of the fused operator == gradients of octree2col + mm (the reference's own
       # comparison, pytorch/test/test_octree_conv.py:55-72)
-      # (the data gradient of a stride-2 convolution exists for the 2x2x2 kernel only)
-      want_x = stride == 1 or ks == [2, 2, 2]
+      want_x = True
       xg1 = xt.clone().requires_grad_(want_x)
       xg2 = xt.clone().requires_grad_(want_x)
       gy = torch.randn_like(y1)
