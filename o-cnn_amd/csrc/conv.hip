@@ -1685,14 +1685,12 @@ struct GradPlan {
   ConvPlan geom, data;
   WgradPlan w;
   int geom_depth, data_depth, data_cin, data_cout, wg_M, wg_C;
-  bool data_ok;
   size_t total_bytes;
 };
 int make_grad_plan(const Info* o, int is_deconv, int depth, int channel_in, int num_output, const int* ks,
     int stride, int nempty, int dtype, GradPlan* g) {
   OCNN_REQUIRE(dtype == OCNN_F32, OCNN_E_UNSUPPORTED, "gradients are computed in fp32 only");
   int e;
-  g->data_ok = true;
   if (!is_deconv) {
     // forward conv: X[Cin] at depth -> Y[Cout].  grad_w = dY * col(X)^T; grad_X = deconv(dY; W).
     g->geom_depth = depth;
@@ -1702,11 +1700,7 @@ int make_grad_plan(const Info* o, int is_deconv, int depth, int channel_in, int 
     g->data_depth = stride == 2 ? depth - 1 : depth;
     g->data_cin = num_output; g->data_cout = channel_in;
     e = make_plan(o, g->data_depth, num_output, channel_in, ks, stride, nempty, 1, dtype, &g->data);
-    if (e == OCNN_E_UNSUPPORTED) {  // only the weight gradient exists for this shape
-      g->data_ok = false;
-      g->data.total_bytes = 0;
-      e = OCNN_OK;
-    }
+    if (e) return e;
   } else {
     // forward deconv: X[Cin] at depth -> Y[Cout] at depth (+1).  grad_w = X * col(dY)^T;
     // grad_X = conv(dY; W).
@@ -1744,8 +1738,6 @@ int run_grad(int is_deconv, void* grad_data, void* grad_w, const void* data_in, 
     if (e) return e;
   }
   if (grad_data) {
-    OCNN_REQUIRE(g.data_ok, OCNN_E_UNSUPPORTED,
-        "the data gradient of a stride-2 convolution is implemented for the 2x2x2 kernel only");
     // the transposed operator with the same weight buffer; its workspace use starts after the
     // weight-gradient kernels on the same stream have finished
     e = run_conv(is_deconv ? 0 : 1, grad_data, grad_out, g.data_cin, out_h, weights, octree_dev, info, g.data_depth,
