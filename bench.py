@@ -261,9 +261,12 @@ def main():
       F.bounding_sphere(scene_pts, "sphere")
     extra["bounding_sphere_scene"] = {"ms": (time.perf_counter() - t0) / reps * 1e3}
 
-    # trilinear interpolation of 64 channels at 1 M free points (segmentation head), and
-    # octree_align of the depth-9 features onto the same octree
-    ipts = torch.cat([torch.rand(1 << 20, 3, generator=g) * 512.0, torch.zeros(1 << 20, 1)], dim=1).to(dev)
+    # trilinear interpolation of 64 channels at 1 M points on the scanned surfaces (segmentation
+    # head: the scene's own points, each four times with a jitter of a third of a cell, so that
+    # nearly every corner exists), and octree_align of the depth-9 features onto the same octree
+    base = torch.from_numpy(((pts + 1.0) * 256.0).astype(np.float32)).repeat(5, 1)[:1 << 20]
+    base = (base + (torch.rand(base.shape, generator=g) - 0.5) * 0.66).clamp(0.51, 511.49)
+    ipts = torch.cat([base, torch.zeros(1 << 20, 1)], dim=1).to(dev)
     t = timed(lambda: F.octree_interp_pts(x32, octree, 9, ipts, "linear"), reps, wu)
     extra["trilinear_1Mpts_c64_d9"] = {"ms": t, "Mpts_per_s": (1 << 20) / t / 1e3,
                                        "GBs": (1 << 20) * (64 * 4 * 9 + 16) / t / 1e6}

@@ -206,6 +206,14 @@ int ocnn_align_backward(const float* top, int top_h, int channel, float* btm, in
     ocnn_stream_t stream);
 int ocnn_octree_interp(float* out, const float* data, int channel, int H, const uint64_t* key, int n_key,
     const float* pts, int n_pts, int depth, int method, int* idx, float* weight, ocnn_stream_t stream);
+/* The same with a workspace of ocnn_octree_interp_workspace_bytes(channel, H) bytes (16-byte
+ * aligned; may be NULL): when the points ask for at least half as many rows as the level has,
+ * the features are first copied row-major into it and every corner is read as one contiguous
+ * row (several times faster for 64 channels).  Same results. */
+size_t ocnn_octree_interp_workspace_bytes(int channel, int H);
+int ocnn_octree_interp_ws(float* out, const float* data, int channel, int H, const uint64_t* key, int n_key,
+    const float* pts, int n_pts, int depth, int method, int* idx, float* weight, void* workspace_dev,
+    size_t workspace_bytes, ocnn_stream_t stream);
 int ocnn_octree_interp_backward(float* grad_data, const float* grad_out, int channel, int H, int n_pts,
     int method, const int* idx, const float* weight, ocnn_stream_t stream);
 

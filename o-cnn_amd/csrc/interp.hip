@@ -90,14 +90,18 @@ __global__ void interp_index_kernel(int* __restrict__ idx, float* __restrict__ w
 }
 
 // out[c, p] = sum_m w_m data[c, idx_m] / (sum_m w_m + 1e-10) over the corners that exist;
-// nearest: data[c, idx] or 0.  One thread per point, channels in the inner loop.
+// nearest: data[c, idx] or 0.  One thread per point, channels in the inner loop.  K is a
+// template parameter so that the corner arrays stay in registers (with a run-time bound they
+// are indexed dynamically and live in scratch memory: 10x slower).
+template <int K>
 __global__ void interp_gather_kernel(float* __restrict__ out, const float* __restrict__ data, int channel, int H,
-    const int* __restrict__ idx, const float* __restrict__ weight, int n_pts, int K, int normalise) {
+    const int* __restrict__ idx, const float* __restrict__ weight, int n_pts, int normalise) {
   const int p = blockIdx.x * kBlock + threadIdx.x;
   if (p >= n_pts) return;
-  int id[8];
-  float w[8];
+  int id[K];
+  float w[K];
   float norm = 0.0f;
+#pragma unroll
   for (int m = 0; m < K; ++m) {
     id[m] = idx[(int64_t)p * K + m];
     w[m] = (id[m] >= 0 && id[m] < H) ? weight[(int64_t)p * K + m] : 0.0f;
@@ -107,19 +111,96 @@ __global__ void interp_gather_kernel(float* __restrict__ out, const float* __res
   const float inv = normalise ? 1.0f / (norm + 1e-10f) : 1.0f;
   for (int c = 0; c < channel; ++c) {
     float acc = 0.0f;
+#pragma unroll
     for (int m = 0; m < K; ++m)
       if (id[m] >= 0) acc += w[m] * data[(int64_t)c * H + id[m]];
     out[(int64_t)c * n_pts + p] = acc * inv;
   }
 }
+// ---- the same gather through a row-major copy of the features ----------------------------------
+// In the channel-major tensor the C values of a node are C cache lines apart, so the kernel
+// above asks for 8 x C lines per point.  With a workspace the features are first copied
+// row-major ([H, Cpad], Cpad = C rounded up to 4): a corner is then one contiguous row, read by
+// 16 lanes as 16-byte vectors (two line requests per 64 channels).  The results of 64 points go
+// through an LDS tile so that the channel-major output leaves in 256-byte rows.
+__global__ void __launch_bounds__(kBlock) rows_copy_kernel(float* __restrict__ xt, const float* __restrict__ data,
+    int channel, int H, int cpad) {
+  __shared__ float tile[64][65];
+  const int h0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    const int c = c0 + i, h = h0 + tx;
+    tile[i][tx] = (c < channel && h < H) ? data[(int64_t)c * H + h] : 0.0f;
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    const int h = h0 + i, c = c0 + tx;
+    if (h < H && c < cpad) xt[(int64_t)h * cpad + c] = tile[tx][i];
+  }
+}
+
+constexpr int kInterpPts = 64;  // points per workgroup
+template <int K>
+__global__ void __launch_bounds__(kBlock) interp_gather_rows_kernel(float* __restrict__ out,
+    const float4* __restrict__ xt, int channel, int cpad4, const int* __restrict__ idx,
+    const float* __restrict__ weight, int n_pts, int normalise) {
+  __shared__ float tile[64][kInterpPts + 1];  // [channel of the chunk][point]
+  const int tid = threadIdx.x;
+  const int pl = tid >> 4, cq = tid & 15;     // point inside a pass of 16, 4-channel group
+  const int p0 = blockIdx.x * kInterpPts;
+  int id[kInterpPts / 16][K];
+  float w[kInterpPts / 16][K], inv[kInterpPts / 16];
+#pragma unroll
+  for (int pass = 0; pass < kInterpPts / 16; ++pass) {
+    const int p = p0 + pass * 16 + pl;
+    float norm = 0.0f;
+#pragma unroll
+    for (int m = 0; m < K; ++m) {
+      const int v = p < n_pts ? idx[(int64_t)p * K + m] : -1;
+      id[pass][m] = v;
+      w[pass][m] = v >= 0 ? weight[(int64_t)p * K + m] : 0.0f;
+      norm += w[pass][m];
+    }
+    inv[pass] = normalise ? 1.0f / (norm + 1e-10f) : 1.0f;
+  }
+  for (int chunk = 0; chunk * 16 < cpad4; ++chunk) {  // 64 channels at a time
+    const int q = chunk * 16 + cq;
+#pragma unroll
+    for (int pass = 0; pass < kInterpPts / 16; ++pass) {
+      float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (q < cpad4) {
+#pragma unroll
+        for (int m = 0; m < K; ++m)
+          if (id[pass][m] >= 0) {
+            const float4 v = xt[(int64_t)id[pass][m] * cpad4 + q];
+            acc.x += w[pass][m] * v.x; acc.y += w[pass][m] * v.y; acc.z += w[pass][m] * v.z; acc.w += w[pass][m] * v.w;
+          }
+      }
+      const int pt = pass * 16 + pl;
+      // the sum first, the normalisation once at the end, as the per-channel kernel does
+      tile[4 * cq + 0][pt] = acc.x * inv[pass]; tile[4 * cq + 1][pt] = acc.y * inv[pass];
+      tile[4 * cq + 2][pt] = acc.z * inv[pass]; tile[4 * cq + 3][pt] = acc.w * inv[pass];
+    }
+    __syncthreads();
+    const int lane = tid & 63, row = tid >> 6;
+    for (int c = row; c < 64; c += 4) {
+      const int ch = chunk * 64 + c;
+      if (ch < channel && p0 + lane < n_pts) out[(int64_t)ch * n_pts + p0 + lane] = tile[c][lane];
+    }
+    __syncthreads();
+  }
+}
+
 // the adjoint: grad_data[c, idx_m] += w_m / (norm + 1e-10) * grad_out[c, p]
+template <int K>
 __global__ void interp_scatter_kernel(float* __restrict__ grad_data, const float* __restrict__ grad_out, int channel,
-    int H, const int* __restrict__ idx, const float* __restrict__ weight, int n_pts, int K, int normalise) {
+    int H, const int* __restrict__ idx, const float* __restrict__ weight, int n_pts, int normalise) {
   const int p = blockIdx.x * kBlock + threadIdx.x;
   if (p >= n_pts) return;
-  int id[8];
-  float w[8];
+  int id[K];
+  float w[K];
   float norm = 0.0f;
+#pragma unroll
   for (int m = 0; m < K; ++m) {
     id[m] = idx[(int64_t)p * K + m];
     const bool ok = id[m] >= 0 && id[m] < H;
@@ -130,6 +211,7 @@ __global__ void interp_scatter_kernel(float* __restrict__ grad_data, const float
   const float inv = normalise ? 1.0f / (norm + 1e-10f) : 1.0f;
   for (int c = 0; c < channel; ++c) {
     const float g = grad_out[(int64_t)c * n_pts + p] * inv;
+#pragma unroll
     for (int m = 0; m < K; ++m)
       if (id[m] >= 0) unsafeAtomicAdd(grad_data + (int64_t)c * H + id[m], w[m] * g);
   }
@@ -162,8 +244,20 @@ int ocnn_align_backward(const float* top, int top_h, int channel, float* btm, in
   return OCNN_OK;
 }
 
+size_t ocnn_octree_interp_workspace_bytes(int channel, int H) {
+  if (channel <= 0 || H <= 0) return 0;
+  return ((size_t)H * (size_t)((channel + 3) / 4 * 4) * sizeof(float) + 255) & ~(size_t)255;
+}
+
 int ocnn_octree_interp(float* out, const float* data, int channel, int H, const uint64_t* key, int n_key,
     const float* pts, int n_pts, int depth, int method, int* idx, float* weight, ocnn_stream_t stream) {
+  return ocnn_octree_interp_ws(out, data, channel, H, key, n_key, pts, n_pts, depth, method, idx, weight, nullptr, 0,
+      stream);
+}
+
+int ocnn_octree_interp_ws(float* out, const float* data, int channel, int H, const uint64_t* key, int n_key,
+    const float* pts, int n_pts, int depth, int method, int* idx, float* weight, void* workspace_dev,
+    size_t workspace_bytes, ocnn_stream_t stream) {
   OCNN_REQUIRE(out && data && pts && idx && weight && (key || n_key == 0), OCNN_E_BADARG, "null pointer");
   OCNN_REQUIRE(channel > 0 && H >= 0 && n_key >= 0 && n_pts >= 0 && depth >= 0 && depth <= 16, OCNN_E_BADARG,
       "bad argument");
@@ -173,7 +267,25 @@ int ocnn_octree_interp(float* out, const float* data, int channel, int H, const 
   const int K = method == 0 ? 1 : 8;
   interp_index_kernel<<<blocks_for((int64_t)n_pts * K), kBlock, 0, s>>>(idx, weight, pts, n_pts, key, n_key, depth, K);
   OCNN_LAUNCH_OK("interp_index");
-  interp_gather_kernel<<<blocks_for(n_pts), kBlock, 0, s>>>(out, data, channel, H, idx, weight, n_pts, K, method);
+  // the row-major copy pays once the points ask for more rows than the level has
+  const bool rows = workspace_dev && H > 0 && workspace_bytes >= ocnn_octree_interp_workspace_bytes(channel, H) &&
+      (reinterpret_cast<uintptr_t>(workspace_dev) & 15) == 0 && (int64_t)n_pts * K >= H / 2;
+  if (rows) {
+    const int cpad = (channel + 3) / 4 * 4;
+    float* xt = static_cast<float*>(workspace_dev);
+    rows_copy_kernel<<<dim3(blocks_for(H, 64), blocks_for(cpad, 64)), kBlock, 0, s>>>(xt, data, channel, H, cpad);
+    OCNN_LAUNCH_OK("rows_copy");
+    if (K == 1)
+      interp_gather_rows_kernel<1><<<blocks_for(n_pts, kInterpPts), kBlock, 0, s>>>(out, (const float4*)xt, channel,
+          cpad / 4, idx, weight, n_pts, method);
+    else
+      interp_gather_rows_kernel<8><<<blocks_for(n_pts, kInterpPts), kBlock, 0, s>>>(out, (const float4*)xt, channel,
+          cpad / 4, idx, weight, n_pts, method);
+  } else if (K == 1) {
+    interp_gather_kernel<1><<<blocks_for(n_pts), kBlock, 0, s>>>(out, data, channel, H, idx, weight, n_pts, method);
+  } else {
+    interp_gather_kernel<8><<<blocks_for(n_pts), kBlock, 0, s>>>(out, data, channel, H, idx, weight, n_pts, method);
+  }
   OCNN_LAUNCH_OK("interp_gather");
   return OCNN_OK;
 }
@@ -186,9 +298,12 @@ int ocnn_octree_interp_backward(float* grad_data, const float* grad_out, int cha
   hipStream_t s = as_stream(stream);
   const int64_t n = (int64_t)H * channel;
   if (n > 0) zero_kernel<<<blocks_for(n), kBlock, 0, s>>>(grad_data, n);
-  if (n_pts > 0)
-    interp_scatter_kernel<<<blocks_for(n_pts), kBlock, 0, s>>>(grad_data, grad_out, channel, H, idx, weight, n_pts,
-        method == 0 ? 1 : 8, method);
+  if (n_pts > 0) {
+    if (method == 0)
+      interp_scatter_kernel<1><<<blocks_for(n_pts), kBlock, 0, s>>>(grad_data, grad_out, channel, H, idx, weight, n_pts, method);
+    else
+      interp_scatter_kernel<8><<<blocks_for(n_pts), kBlock, 0, s>>>(grad_data, grad_out, channel, H, idx, weight, n_pts, method);
+  }
   OCNN_LAUNCH_OK("interp_scatter");
   return OCNN_OK;
 }

@@ -879,8 +879,11 @@ def octree_interp_pts(data, octree, depth, pts, method="linear", nempty=False):
   out = torch.empty(1, channel, n, 1, dtype=torch.float32, device=data.device)
   idx = torch.empty(n, K, dtype=torch.int32, device=data.device)
   weight = torch.empty(n, K, dtype=torch.float32, device=data.device)
-  _lib.call("ocnn_octree_interp", _ptr(out), _ptr(data), channel, H, _ptr(key), n_key, _ptr(pts), n, depth,
-            int(method == "linear"), _ptr(idx), _ptr(weight), _stream())
+  ws_bytes = _lib.get().ocnn_octree_interp_workspace_bytes(channel, H) if n * K >= H // 2 else 0
+  ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=data.device)
+  _lib.call("ocnn_octree_interp_ws", _ptr(out), _ptr(data), channel, H, _ptr(key), n_key, _ptr(pts), n, depth,
+            int(method == "linear"), _ptr(idx), _ptr(weight), _ptr(ws) if ws_bytes else C.c_void_p(0),
+            C.c_size_t(ws_bytes), _stream())
   return out, idx, weight
 
 
