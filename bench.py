@@ -270,6 +270,11 @@ def main():
     t = timed(lambda: F.octree_interp_pts(x32, octree, 9, ipts, "linear"), reps, wu)
     extra["trilinear_1Mpts_c64_d9"] = {"ms": t, "Mpts_per_s": (1 << 20) / t / 1e3,
                                        "GBs": (1 << 20) * (64 * 4 * 9 + 16) / t / 1e6}
+    _, iidx, iw = F.octree_interp_pts(x32, octree, 9, ipts, "linear")
+    gpts = torch.randn(1, C, 1 << 20, 1, device=dev)
+    t = timed(lambda: F.octree_interp_pts_grad(gpts, iidx, iw, H9, "linear"), reps, wu)
+    extra["trilinear_grad_1Mpts_c64_d9"] = {"ms": t, "Mpts_per_s": (1 << 20) / t / 1e3}
+    del gpts, iidx, iw
     t = timed(lambda: F.octree_align(x32, octree, octree, 9), reps, wu)
     by = 2 * C * H9 * 4 + H9 * 20
     extra["octree_align_d9_c64"] = {"ms": t, "GBs": by / t / 1e6, "frac_hbm_peak": by / t / 1e6 / PEAK_HBM_GBS}

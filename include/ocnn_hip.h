@@ -216,6 +216,11 @@ int ocnn_octree_interp_ws(float* out, const float* data, int channel, int H, con
     size_t workspace_bytes, ocnn_stream_t stream);
 int ocnn_octree_interp_backward(float* grad_data, const float* grad_out, int channel, int H, int n_pts,
     int method, const int* idx, const float* weight, ocnn_stream_t stream);
+/* The backward call with the same optional workspace: the gradient is accumulated in rows
+ * (the atomics of a node fall into two cache lines) and turned channel-major at the end. */
+int ocnn_octree_interp_backward_ws(float* grad_data, const float* grad_out, int channel, int H, int n_pts,
+    int method, const int* idx, const float* weight, void* workspace_dev, size_t workspace_bytes,
+    ocnn_stream_t stream);
 
 /* ---- file formats.  A `.octree` / `.points` file is the serialized blob itself
  * (Octree::read_octree / write_octree, octree/octree/octree.cpp:41-68; Points::read_points /

@@ -191,6 +191,77 @@ __global__ void __launch_bounds__(kBlock) interp_gather_rows_kernel(float* __res
   }
 }
 
+// The adjoint through row-major storage: the gradient of a node is one contiguous row, so the
+// four atomics of a lane and those of its 15 neighbours fall into two cache lines instead of
+// 64; the rows are turned back into the channel-major tensor at the end.
+template <int K>
+__global__ void __launch_bounds__(kBlock) interp_scatter_rows_kernel(float* __restrict__ xt,
+    const float* __restrict__ grad_out, int channel, int cpad, const int* __restrict__ idx,
+    const float* __restrict__ weight, int n_pts, int normalise) {
+  __shared__ float tile[64][kInterpPts + 1];  // [channel of the chunk][point]
+  const int tid = threadIdx.x;
+  const int pl = tid >> 4, cq = tid & 15;
+  const int p0 = blockIdx.x * kInterpPts;
+  int id[kInterpPts / 16][K];
+  float w[kInterpPts / 16][K];
+#pragma unroll
+  for (int pass = 0; pass < kInterpPts / 16; ++pass) {
+    const int p = p0 + pass * 16 + pl;
+    float norm = 0.0f;
+#pragma unroll
+    for (int m = 0; m < K; ++m) {
+      const int v = p < n_pts ? idx[(int64_t)p * K + m] : -1;
+      id[pass][m] = v;
+      w[pass][m] = v >= 0 ? weight[(int64_t)p * K + m] : 0.0f;
+      norm += w[pass][m];
+    }
+    const float inv = normalise ? 1.0f / (norm + 1e-10f) : 1.0f;
+#pragma unroll
+    for (int m = 0; m < K; ++m) w[pass][m] *= inv;
+  }
+  const int lane = tid & 63, row = tid >> 6;
+  for (int chunk = 0; chunk * 64 < cpad; ++chunk) {
+    for (int c = row; c < 64; c += 4) {
+      const int ch = chunk * 64 + c;
+      tile[c][lane] = (ch < channel && p0 + lane < n_pts) ? grad_out[(int64_t)ch * n_pts + p0 + lane] : 0.0f;
+    }
+    __syncthreads();
+    const int c4 = chunk * 64 + 4 * cq;
+    if (c4 < cpad) {
+#pragma unroll
+      for (int pass = 0; pass < kInterpPts / 16; ++pass) {
+        const int pt = pass * 16 + pl;
+        const float g0 = tile[4 * cq + 0][pt], g1 = tile[4 * cq + 1][pt], g2 = tile[4 * cq + 2][pt], g3 = tile[4 * cq + 3][pt];
+#pragma unroll
+        for (int m = 0; m < K; ++m)
+          if (id[pass][m] >= 0) {
+            float* dst = xt + (int64_t)id[pass][m] * cpad + c4;
+            unsafeAtomicAdd(dst + 0, w[pass][m] * g0);
+            unsafeAtomicAdd(dst + 1, w[pass][m] * g1);
+            unsafeAtomicAdd(dst + 2, w[pass][m] * g2);
+            unsafeAtomicAdd(dst + 3, w[pass][m] * g3);
+          }
+      }
+    }
+    __syncthreads();
+  }
+}
+__global__ void __launch_bounds__(kBlock) rows_back_kernel(float* __restrict__ data, const float* __restrict__ xt,
+    int channel, int H, int cpad) {
+  __shared__ float tile[64][65];
+  const int h0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    const int h = h0 + i, c = c0 + tx;
+    tile[i][tx] = (h < H && c < cpad) ? xt[(int64_t)h * cpad + c] : 0.0f;
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    const int c = c0 + i, h = h0 + tx;
+    if (c < channel && h < H) data[(int64_t)c * H + h] = tile[tx][i];
+  }
+}
+
 // the adjoint: grad_data[c, idx_m] += w_m / (norm + 1e-10) * grad_out[c, p]
 template <int K>
 __global__ void interp_scatter_kernel(float* __restrict__ grad_data, const float* __restrict__ grad_out, int channel,
@@ -292,10 +363,32 @@ int ocnn_octree_interp_ws(float* out, const float* data, int channel, int H, con
 
 int ocnn_octree_interp_backward(float* grad_data, const float* grad_out, int channel, int H, int n_pts, int method,
     const int* idx, const float* weight, ocnn_stream_t stream) {
+  return ocnn_octree_interp_backward_ws(grad_data, grad_out, channel, H, n_pts, method, idx, weight, nullptr, 0, stream);
+}
+
+int ocnn_octree_interp_backward_ws(float* grad_data, const float* grad_out, int channel, int H, int n_pts, int method,
+    const int* idx, const float* weight, void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream) {
   OCNN_REQUIRE(grad_data && grad_out && idx && weight && channel > 0 && H >= 0 && n_pts >= 0, OCNN_E_BADARG,
       "bad argument");
   OCNN_REQUIRE(method == 0 || method == 1, OCNN_E_BADARG, "method %d", method);
   hipStream_t s = as_stream(stream);
+  const int Kc = method == 0 ? 1 : 8;
+  if (workspace_dev && H > 0 && n_pts > 0 && workspace_bytes >= ocnn_octree_interp_workspace_bytes(channel, H) &&
+      (reinterpret_cast<uintptr_t>(workspace_dev) & 15) == 0 && (int64_t)n_pts * Kc >= H / 2) {
+    const int cpad = (channel + 3) / 4 * 4;
+    float* xt = static_cast<float*>(workspace_dev);
+    const int64_t words = (int64_t)H * cpad;
+    zero_kernel<<<blocks_for(words), kBlock, 0, s>>>(xt, words);
+    if (Kc == 1)
+      interp_scatter_rows_kernel<1><<<blocks_for(n_pts, kInterpPts), kBlock, 0, s>>>(xt, grad_out, channel, cpad, idx,
+          weight, n_pts, method);
+    else
+      interp_scatter_rows_kernel<8><<<blocks_for(n_pts, kInterpPts), kBlock, 0, s>>>(xt, grad_out, channel, cpad, idx,
+          weight, n_pts, method);
+    rows_back_kernel<<<dim3(blocks_for(H, 64), blocks_for(channel, 64)), kBlock, 0, s>>>(grad_data, xt, channel, H, cpad);
+    OCNN_LAUNCH_OK("interp_scatter_rows");
+    return OCNN_OK;
+  }
   const int64_t n = (int64_t)H * channel;
   if (n > 0) zero_kernel<<<blocks_for(n), kBlock, 0, s>>>(grad_data, n);
   if (n_pts > 0) {

@@ -2,6 +2,8 @@
 point-cloud property accessors against the oracle restatements (oracle/interp.py), including the
 reference's own literal cases (pytorch/test/test_octree_align.py, test_octree_trilinear.py,
 test_points_property.py).  Indices bit-exact; fp32 values within 1e-5."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -94,6 +96,24 @@ def test_interpolation_vs_oracle(oc, orc, synthetic, nempty, key2xyz):
       lhs = float(np.vdot(got.astype(np.float64), g))
       rhs = float(np.vdot(data.astype(np.float64), back.cpu().numpy().reshape(data.shape)))
       assert abs(lhs - rhs) < 1e-4 * max(1.0, abs(lhs))
+      # element by element: the scatter written out with numpy from the returned corners
+      ii, ww = idx.cpu().numpy().reshape(len(pts), -1), w.cpu().numpy().reshape(len(pts), -1).astype(np.float64)
+      ww = np.where(ii >= 0, ww, 0.0)
+      if method == "linear":
+        ww = ww / (ww.sum(axis=1, keepdims=True) + 1e-10)
+      dense = np.zeros((6, H))
+      for m in range(ii.shape[1]):
+        ok = ii[:, m] >= 0
+        for c in range(6):
+          np.add.at(dense[c], ii[ok, m], ww[ok, m] * g.reshape(6, -1)[c, ok])
+      assert np.allclose(back.cpu().numpy().reshape(6, H), dense, atol=1e-4)
+      # the entry point without a workspace scatters channel-major: same values
+      plain = torch.empty(6, H, dtype=torch.float32, device="cuda")
+      gg = T(g).cuda().contiguous()
+      vp = lambda t: ctypes.c_void_p(t.data_ptr())
+      oc.lib.call("ocnn_octree_interp_backward", vp(plain), vp(gg), 6, H, len(pts), int(method == "linear"),
+                  vp(idx), vp(w), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+      assert np.allclose(plain.cpu().numpy(), dense, atol=1e-4)
   # the module form: points in [-1, 1], gradients through autograd
   H = int(b.nnum[5])
   x = torch.randn(1, 6, H, 1, device="cuda", requires_grad=True)
