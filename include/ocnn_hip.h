@@ -321,6 +321,22 @@ int ocnn_octree_scan(const void* octree_dev, const void* info, const float* axis
     float scale, ocnn_alloc_fn alloc, void* alloc_ctx, void* info_out, void** octree_out_dev,
     ocnn_stream_t stream);
 
+/* ---- octree_dropout, octree/octree/transform_octree.cpp:286-431 (the `OctreeDrop` op,
+ * tensorflow/libs/transform_octree_op.cc:40-56): the nodes of level `depth_dropout` whose
+ * flag is set (`flags_dev`: one byte per node of that level, device memory) leave with their
+ * whole subtrees; the levels below are compacted and the children renumbered.  The reference
+ * draws the flags on the host from an engine seeded with the clock; here the caller draws
+ * them (a Bernoulli sample of the drop ratio).  With `clear_dropped` 0 the result is
+ * bit-identical to the reference's for the same flags: at `depth_dropout` itself a dropped
+ * node then keeps its old child entry (transform_octree.cpp:422-425), which points past the
+ * compacted level below, so such a blob must not be given to anything that follows the child
+ * entries of that level (the neighbour tables of octree_batch).  With `clear_dropped` 1 those
+ * entries are -1 and the result is an ordinary octree.  Scratch and result come from `alloc`;
+ * one device-to-host copy (the node counts) is waited for. */
+int ocnn_octree_dropout(const void* octree_dev, const void* info, const unsigned char* flags_dev,
+    int depth_dropout, int clear_dropped, ocnn_alloc_fn alloc, void* alloc_ctx, void* info_out, void** octree_out_dev,
+    ocnn_stream_t stream);
+
 /* ---- octree_batch of already serialized octrees that live on the device
  * (merge_octrees, octree/octree/merge_octrees.cpp:7-198).  `out_info` (host)
  * is filled by ocnn_octree_batch_info from the n host headers; the caller

@@ -4,6 +4,7 @@
 // Header arithmetic runs on the host from the caller's host copies of the
 // headers; the payload never leaves the device.
 #include "ocnn_common.h"
+#include "octree_kernels.h"
 #include "scan.h"
 
 #include <algorithm>
@@ -434,10 +435,14 @@ int ocnn_octree_batch(void* out_dev, const void* out_info, const void* const* oc
   OCNN_REQUIRE(o.has(OCNN_CHILD), OCNN_E_FORMAT, "octrees without child links cannot get neighbour tables");
   for (int d = 1; d <= depth; ++d) {
     int* neigh = reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_NEIGH, d));
-    if (d <= fl) e = ocnn_calc_neigh_full(neigh, d, B, stream);
-    else e = ocnn_calc_neigh_sparse(neigh, reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_NEIGH, d - 1)),
-        reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_CHILD, d - 1)), o.nnum[d - 1], stream);
-    if (e) return e;
+    if (d <= fl) {
+      e = ocnn_calc_neigh_full(neigh, d, B, stream);
+      if (e) return e;
+    } else if (o.nnum[d - 1] > 0) {
+      launch_neigh_sparse(neigh, reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_NEIGH, d - 1)),
+          reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_CHILD, d - 1)), o.nnum[d - 1], s, o.nnum[d] / 8);
+      OCNN_LAUNCH_OK("calc_neigh_sparse");
+    }
   }
   return OCNN_OK;
 }
@@ -570,9 +575,12 @@ int ocnn_octree_grow(void* out_dev, const void* out_info, const void* in_dev, co
     e = ocnn_generate_key_full(reinterpret_cast<uint64_t*>(blob + key_new), target_depth, o.batch_size, stream);
     if (e) return e;
   } else {
-    e = ocnn_calc_neigh_sparse(neigh, reinterpret_cast<const int*>(in + oi.ptr_dis(OCNN_NEIGH, target_depth - 1)),
-        reinterpret_cast<const int*>(in + oi.ptr_dis(OCNN_CHILD, target_depth - 1)), o.nnum[target_depth - 1], stream);
-    if (e) return e;
+    if (o.nnum[target_depth - 1] > 0) {
+      launch_neigh_sparse(neigh, reinterpret_cast<const int*>(in + oi.ptr_dis(OCNN_NEIGH, target_depth - 1)),
+          reinterpret_cast<const int*>(in + oi.ptr_dis(OCNN_CHILD, target_depth - 1)), o.nnum[target_depth - 1], s,
+          node_num / 8);
+      OCNN_LAUNCH_OK("calc_neigh_sparse");
+    }
   }
   return OCNN_OK;
 }

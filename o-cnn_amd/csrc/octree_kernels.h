@@ -70,7 +70,7 @@ struct NeighLane {
 // GROUPS = 2 gives a small level more wavefronts and each a shorter chain.
 template <int GROUPS>
 __global__ __launch_bounds__(kBlock) void neigh_sparse_kernel(int* __restrict__ neigh_child,
-    const int* __restrict__ neigh, const int* __restrict__ children, int node_num, int iters) {
+    const int* __restrict__ neigh, const int* __restrict__ children, int node_num, int iters, int child_groups) {
   const int lane = threadIdx.x & 63;
   const int wave = (int)((blockIdx.x * (unsigned)kBlock + threadIdx.x) >> 6);
   const int groups = (node_num + 7) >> 3;
@@ -117,6 +117,7 @@ __global__ __launch_bounds__(kBlock) void neigh_sparse_kernel(int* __restrict__ 
         if (!((occ[u] >> s) & 1)) continue;   // uniform over the wavefront
         const int rank = __shfl(rank8[u], s, 64);
         const int v = __shfl(link[u], nl.parent_slot(s), 64);
+        if (rank >= child_groups) continue;   // a link past the child level (malformed input): no row to write
         neigh_child[((int64_t)rank << 6) + lane] = v >= 0 ? (v << 3) + nl.octant : -1;
       }
     }
@@ -124,8 +125,10 @@ __global__ __launch_bounds__(kBlock) void neigh_sparse_kernel(int* __restrict__ 
     for (int u = 0; u < GROUPS; ++u) { rank8[u] = next_rank8[u]; slot[u] = next_slot[u]; }
   }
 }
+// `child_groups`: sibling groups of the level written, where the caller knows it (a header);
+// links at or past it are skipped instead of followed.
 inline void launch_neigh_sparse(int* neigh_child, const int* neigh, const int* children, int node_num,
-    hipStream_t s) {
+    hipStream_t s, int child_groups = 0x7fffffff) {
   const int64_t groups = ((int64_t)node_num + 7) / 8;
   if (groups >= (1 << 16)) {
     // batches per wavefront: more than one once the wavefronts fill the device several times over
@@ -133,10 +136,10 @@ inline void launch_neigh_sparse(int* neigh_child, const int* neigh, const int* c
     int64_t iters = batches / 32768;
     iters = iters < 1 ? 1 : (iters > 8 ? 8 : iters);
     neigh_sparse_kernel<8><<<blocks_for(batches, (kBlock / 64) * iters), kBlock, 0, s>>>(neigh_child, neigh, children,
-        node_num, (int)iters);
+        node_num, (int)iters, child_groups);
   } else {
     neigh_sparse_kernel<2><<<blocks_for((groups + 1) / 2, kBlock / 64), kBlock, 0, s>>>(neigh_child, neigh, children,
-        node_num, 1);
+        node_num, 1, child_groups);
   }
 }
 

@@ -175,6 +175,56 @@ __global__ void copy_words_kernel(uint32_t* __restrict__ dst, const uint32_t* __
 
 inline size_t al(size_t v) { return (v + 255) & ~(size_t)255; }
 
+// ---- octree_dropout (octree/octree/transform_octree.cpp:286-431)
+__global__ void drop_flags_kernel(int* __restrict__ drop, const unsigned char* __restrict__ flags, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) drop[i] = flags[i] != 0;
+}
+// a dropped node takes its children along (:301-314)
+__global__ void drop_children_kernel(int* __restrict__ drop_c, const int* __restrict__ drop_p,
+    const int* __restrict__ child_p, int n_parent) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  const int i = t >> 3;
+  if (i >= n_parent) return;
+  const int c = child_p[i];
+  if (c >= 0) drop_c[(int64_t)c * 8 + (t & 7)] = drop_p[i];
+}
+struct LivePred {   // kept and non-empty: the nodes whose children are renumbered
+  const int* drop; const int* child;
+  __device__ bool operator()(int64_t i) const { return drop[i] == 0 && child[i] >= 0; }
+};
+// the kept nodes of one level below the dropout level, compacted (:365-416)
+struct DropArgs {
+  int n_in, n_out, fch;
+  const int *drop, *rank, *live_rank, *child_in;
+  const uint64_t* key_in; const float *f_in, *l_in, *s_in;
+  uint64_t* key_out; int* child_out; float *f_out, *l_out, *s_out;
+};
+__global__ void drop_gather_kernel(DropArgs a) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= a.n_in || a.drop[i] != 0) return;
+  const int j = a.rank[i];
+  a.key_out[j] = a.key_in[i];
+  const int c = a.child_in[i];
+  a.child_out[j] = c < 0 ? c : a.live_rank[i];
+  if (a.f_out)
+    for (int ch = 0; ch < a.fch; ++ch) a.f_out[(int64_t)ch * a.n_out + j] = a.f_in[(int64_t)ch * a.n_in + i];
+  if (a.l_out) a.l_out[j] = a.l_in[i];
+  if (a.s_out) a.s_out[j] = a.s_in[i];
+}
+// the dropout level itself (:419-425): a dropped node keeps its old child entry
+__global__ void drop_level_children_kernel(int* __restrict__ child_out, const int* __restrict__ child_in,
+    const int* __restrict__ drop, const int* __restrict__ live_rank, int n, int clear_dropped) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int c = child_in[i];
+  child_out[i] = (drop[i] != 0 || c < 0) ? (clear_dropped ? -1 : c) : live_rank[i];
+}
+__global__ void copy_words64_kernel(uint32_t* __restrict__ dst, const uint32_t* __restrict__ src, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = src[i];
+}
+
 }  // namespace
 }  // namespace ocnn
 
@@ -310,5 +360,129 @@ extern "C" int ocnn_octree_scan(const void* octree_dev, const void* info, const 
     if (a.n_parent > 0) trim_kernel<<<blocks_for((int64_t)a.n_parent * 8), kBlock, 0, s>>>(a);
   }
   OCNN_LAUNCH_OK("trim");
+  return OCNN_OK;
+}
+
+extern "C" int ocnn_octree_dropout(const void* octree_dev, const void* info, const unsigned char* flags_dev,
+    int depth_dropout, int clear_dropped, ocnn_alloc_fn alloc, void* alloc_ctx, void* info_out, void** octree_out_dev,
+    ocnn_stream_t stream) {
+  OCNN_REQUIRE(octree_dev && info && flags_dev && alloc && info_out && octree_out_dev, OCNN_E_BADARG, "null pointer");
+  const Info& oi = *as_info(info);
+  const int D = oi.depth, dd = depth_dropout;
+  OCNN_REQUIRE(D >= 1 && D <= 16, OCNN_E_FORMAT, "depth %d", D);
+  OCNN_REQUIRE(dd >= 0 && dd <= D, OCNN_E_BADARG, "depth_dropout %d outside [0, %d]", dd, D);
+  OCNN_REQUIRE(oi.channel(OCNN_KEY) == 1, OCNN_E_UNSUPPORTED, "octree_dropout takes one-channel keys");
+  hipStream_t s = as_stream(stream);
+  const char* in = static_cast<const char*>(octree_dev);
+
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t v = off; off += al(bytes); return v; };
+  size_t o_drop[kMaxD], o_rank[kMaxD], o_live[kMaxD];
+  int max_n = 1;
+  for (int d = dd; d <= D; ++d) {
+    o_drop[d] = take(4 * ((size_t)oi.nnum[d] + 1));
+    o_rank[d] = take(4 * ((size_t)oi.nnum[d] + 1));
+    o_live[d] = take(4 * ((size_t)oi.nnum[d] + 1));
+    if (oi.nnum[d] > max_n) max_n = oi.nnum[d];
+  }
+  const size_t o_scan = take(scan_scratch_bytes(max_n));
+  const size_t o_counts = take(sizeof(int) * 2 * kMaxD);
+  const size_t o_hdr = take(OCNN_HEADER_BYTES);
+  char* ws = static_cast<char*>(alloc(off, alloc_ctx));
+  OCNN_REQUIRE(ws, OCNN_E_BADARG, "the allocator returned no memory for %zu bytes of scratch", off);
+  OCNN_REQUIRE((reinterpret_cast<uintptr_t>(ws) & 7) == 0, OCNN_E_BADARG, "scratch not 8-byte aligned");
+  auto drop = [&](int d) { return reinterpret_cast<int*>(ws + o_drop[d]); };
+  auto rank = [&](int d) { return reinterpret_cast<int*>(ws + o_rank[d]); };
+  auto live = [&](int d) { return reinterpret_cast<int*>(ws + o_live[d]); };
+  auto child_in = [&](int d) { return reinterpret_cast<const int*>(in + oi.ptr_dis(OCNN_CHILD, d)); };
+  int* d_counts = reinterpret_cast<int*>(ws + o_counts);   // [d]: kept nodes, [kMaxD + d]: kept non-empty nodes
+
+  // ---- flags top-down, ranks of the kept nodes and of the kept non-empty nodes
+  if (oi.nnum[dd] > 0) drop_flags_kernel<<<blocks_for(oi.nnum[dd]), kBlock, 0, s>>>(drop(dd), flags_dev, oi.nnum[dd]);
+  for (int d = dd + 1; d <= D; ++d)
+    if (oi.nnum[d - 1] > 0)
+      drop_children_kernel<<<blocks_for((int64_t)oi.nnum[d - 1] * 8), kBlock, 0, s>>>(drop(d), drop(d - 1), child_in(d - 1),
+          oi.nnum[d - 1]);
+  for (int d = dd; d <= D; ++d) {
+    hipError_t e = hipSuccess;
+    if (d > dd) {
+      KeptPred kp{drop(d)};
+      KeptOut ko{rank(d)};
+      e = flag_scan(kp, ko, (int64_t)oi.nnum[d], reinterpret_cast<int*>(ws + o_scan), d_counts + d, s);
+      OCNN_REQUIRE(e == hipSuccess, OCNN_E_HIP, "scan: %s", hipGetErrorString(e));
+    }
+    LivePred lp{drop(d), child_in(d)};
+    KeptOut lo{live(d)};
+    e = flag_scan(lp, lo, (int64_t)oi.nnum[d], reinterpret_cast<int*>(ws + o_scan), d_counts + kMaxD + d, s);
+    OCNN_REQUIRE(e == hipSuccess, OCNN_E_HIP, "scan: %s", hipGetErrorString(e));
+  }
+  int h[2 * kMaxD];
+  OCNN_HIP_OK(hipMemcpyAsync(h, d_counts, sizeof(h), hipMemcpyDeviceToHost, s));
+  OCNN_HIP_OK(hipStreamSynchronize(s));
+
+  Info o = oi;
+  for (int d = dd + 1; d <= D; ++d) o.nnum[d] = h[d];
+  for (int d = dd; d <= D; ++d) o.nnum_nempty[d] = h[kMaxD + d];
+  o.set_nnum_cum();
+  OCNN_REQUIRE(o.set_ptr_dis(), OCNN_E_SHAPE, "the octree would exceed 2 GiB");
+  memcpy(info_out, &o, sizeof(Info));
+
+  // ---- the new octree: zeros, header, levels 0..depth_dropout as they are, a gather per level below
+  const size_t bytes = (size_t)o.sizeof_octree();
+  char* out = static_cast<char*>(alloc(bytes, alloc_ctx));
+  OCNN_REQUIRE(out, OCNN_E_BADARG, "the allocator returned no memory for the octree");
+  OCNN_REQUIRE((reinterpret_cast<uintptr_t>(out) & 7) == 0, OCNN_E_BADARG, "blob not 8-byte aligned");
+  *octree_out_dev = out;
+  fill_i32_kernel<<<blocks_for((int64_t)(bytes / 4)), kBlock, 0, s>>>(reinterpret_cast<int*>(out), (int64_t)(bytes / 4), 0);
+  {
+    uint32_t hdr[OCNN_HEADER_BYTES / 4];
+    memset(hdr, 0, sizeof(hdr));
+    memcpy(hdr, &o, sizeof(Info));
+    OCNN_HIP_OK(hipMemcpyAsync(ws + o_hdr, hdr, sizeof(hdr), hipMemcpyHostToDevice, s));
+    OCNN_HIP_OK(hipStreamSynchronize(s));   // `hdr` lives on this stack frame
+    copy_words_kernel<<<1, kBlock, 0, s>>>(reinterpret_cast<uint32_t*>(out), reinterpret_cast<const uint32_t*>(ws + o_hdr),
+        OCNN_HEADER_BYTES / 4);
+  }
+  const int fch = oi.channel(OCNN_FEATURE), floc = oi.location(OCNN_FEATURE);
+  const int lch = oi.channel(OCNN_LABEL), lloc = oi.location(OCNN_LABEL);
+  const int sch = oi.channel(OCNN_SPLIT), sloc = oi.location(OCNN_SPLIT);
+  const int64_t num = oi.nnum_cum[dd + 1];
+  auto copy_prefix = [&](int prop, int64_t words) {
+    if (words > 0)
+      copy_words64_kernel<<<blocks_for(words), kBlock, 0, s>>>(reinterpret_cast<uint32_t*>(out + o.ptr_dis(prop, 0)),
+          reinterpret_cast<const uint32_t*>(in + oi.ptr_dis(prop, 0)), words);
+  };
+  copy_prefix(OCNN_KEY, 2 * num);
+  copy_prefix(OCNN_CHILD, num);
+  if (oi.has(OCNN_FEATURE) && floc == -1) copy_prefix(OCNN_FEATURE, num * fch);
+  if (oi.has(OCNN_LABEL) && lloc == -1) copy_prefix(OCNN_LABEL, num * lch);
+  if (oi.has(OCNN_SPLIT) && sloc == -1) copy_prefix(OCNN_SPLIT, num * sch);
+  for (int d = dd + 1; d <= D; ++d) {
+    if (oi.nnum[d] == 0) continue;
+    DropArgs a;
+    memset(&a, 0, sizeof(a));
+    a.n_in = oi.nnum[d]; a.n_out = o.nnum[d]; a.fch = fch;
+    a.drop = drop(d); a.rank = rank(d); a.live_rank = live(d); a.child_in = child_in(d);
+    a.key_in = reinterpret_cast<const uint64_t*>(in + oi.ptr_dis(OCNN_KEY, d));
+    a.key_out = reinterpret_cast<uint64_t*>(out + o.ptr_dis(OCNN_KEY, d));
+    a.child_out = reinterpret_cast<int*>(out + o.ptr_dis(OCNN_CHILD, d));
+    if (oi.has(OCNN_FEATURE) && fch && (floc == -1 || d == D)) {
+      a.f_in = reinterpret_cast<const float*>(in + oi.ptr_dis(OCNN_FEATURE, d));
+      a.f_out = reinterpret_cast<float*>(out + o.ptr_dis(OCNN_FEATURE, d));
+    }
+    if (lch && (lloc == -1 || d == D)) {
+      a.l_in = reinterpret_cast<const float*>(in + oi.ptr_dis(OCNN_LABEL, d));
+      a.l_out = reinterpret_cast<float*>(out + o.ptr_dis(OCNN_LABEL, d));
+    }
+    if (sch && (sloc == -1 || d == D)) {
+      a.s_in = reinterpret_cast<const float*>(in + oi.ptr_dis(OCNN_SPLIT, d));
+      a.s_out = reinterpret_cast<float*>(out + o.ptr_dis(OCNN_SPLIT, d));
+    }
+    drop_gather_kernel<<<blocks_for(a.n_in), kBlock, 0, s>>>(a);
+  }
+  if (oi.nnum[dd] > 0)
+    drop_level_children_kernel<<<blocks_for(oi.nnum[dd]), kBlock, 0, s>>>(reinterpret_cast<int*>(out + o.ptr_dis(OCNN_CHILD, dd)),
+        child_in(dd), drop(dd), live(dd), oi.nnum[dd], clear_dropped);
+  OCNN_LAUNCH_OK("octree_dropout");
   return OCNN_OK;
 }

@@ -28,7 +28,7 @@ __all__ = [
     "octree_pad", "octree_depad", "octree_max_pool", "octree_max_unpool", "octree_mask_pool",
     "octree_encode_key", "octree_decode_key", "octree_xyz2key", "octree_key2xyz",
     "octree_search_key", "octree_new", "octree_grow", "octree_update", "points_new",
-    "octree_info", "octree_scan",
+    "octree_info", "octree_scan", "octree_dropout", "octree_drop",
 ]
 
 
@@ -158,14 +158,58 @@ def _points_header(points):
 _ALLOC_FN = C.CFUNCTYPE(C.c_void_p, C.c_size_t, C.c_void_p)
 
 
+_LANES = 4          # concurrent single-cloud builds: one per hardware queue of the process
+_lane_state = {}
+
+
+def _lanes(device):
+  """Side streams (default priority) and the worker threads that feed them, per device."""
+  st = _lane_state.get(device)
+  if st is None:
+    from concurrent.futures import ThreadPoolExecutor
+    st = ([torch.cuda.Stream(device=device) for _ in range(_LANES)], ThreadPoolExecutor(_LANES))
+    _lane_state[device] = st
+  return st
+
+
+def _build_each(points_list, args):
+  """Single-cloud builds of a list of clouds.  Such a build is a chain of small launches with
+  waits for node counts in between, bound by latency and not by the device: the clouds are dealt
+  over side streams, each fed by its own host thread (the C calls release the interpreter lock),
+  and the current stream takes the results when all are done."""
+  n = len(points_list)
+  if n < 2:
+    return [_build([p], False, *args) for p in points_list]
+  device = torch.cuda.current_device()
+  cur = torch.cuda.current_stream()
+  streams, pool = _lanes(device)
+  lanes = min(_LANES, n)
+  for st in streams[:lanes]:
+    st.wait_stream(cur)
+
+  def lane(k):
+    torch.cuda.set_device(device)
+    with torch.cuda.stream(streams[k]):
+      return [_build([points_list[i]], False, *args, ws_tag="build-lane%d" % k) for i in range(k, n, lanes)]
+
+  done = list(pool.map(lane, range(lanes)))
+  out = [None] * n
+  for k in range(lanes):
+    cur.wait_stream(streams[k])
+    for j, blob in enumerate(done[k]):
+      blob.record_stream(cur)     # allocated on the side stream, used on the current one from here on
+      out[k + j * lanes] = blob
+  return out
+
+
 def _build(points_list, merged, depth, full_depth, node_dis, node_feature, split_label, adaptive,
-           adp_depth, th_normal, th_distance, extrapolate, save_pts, key2xyz, bbox=None):
+           adp_depth, th_normal, th_distance, extrapolate, save_pts, key2xyz, bbox=None, ws_tag="build"):
   if merged and (node_feature or adaptive):
     # octrees with a signal at every depth are built one cloud at a time and merged afterwards,
     # as collate_octrees does (pytorch/ocnn/transforms.py:127-148)
-    return octree_batch([_build([p], False, depth, full_depth, node_dis, node_feature, split_label, adaptive,
-                                adp_depth, th_normal, th_distance, extrapolate, save_pts, key2xyz, bbox)
-                         for p in points_list])
+    return octree_batch(_build_each(list(points_list), (depth, full_depth, node_dis, node_feature, split_label,
+                                                        adaptive, adp_depth, th_normal, th_distance, extrapolate,
+                                                        save_pts, key2xyz, bbox)))
   pts = [_to_dev(p) for p in points_list]
   hdrs = [getattr(p, "_ocnn_points_info", None) for p in points_list]
   for i, h in enumerate(hdrs):
@@ -186,7 +230,7 @@ def _build(points_list, merged, depth, full_depth, node_dis, node_feature, split
   ws_bytes = L.ocnn_points2octree_workspace_bytes(total, n, eff_depth)
   if ws_bytes == 0:
     raise OcnnError(-1, "bad build arguments (points %d, clouds %d, depth %d)" % (total, n, depth))
-  ws = _workspace(ws_bytes + 256, "build")
+  ws = _workspace(ws_bytes + 256, ws_tag)
   base = (ws.data_ptr() + 255) & ~255
   dev_ptrs = (C.c_void_p * n)(*[p.data_ptr() for p in pts])
   hdr_ptrs = (C.c_void_p * n)(*[h.ctypes.data for h in hdrs])
@@ -222,6 +266,45 @@ def points2octree_batch(points_list, depth, full_depth=2, node_dis=False, node_f
   (the composition `collate_octrees` performs, pytorch/ocnn/transforms.py:127-148)."""
   return _build(list(points_list), True, depth, full_depth, node_dis, node_feature, split_label,
                 adaptive, adp_depth, th_normal, th_distance, extrapolate, save_pts, key2xyz)
+
+
+def octree_dropout(octree, depth_dropout, threshold, flags=None, generator=None, clear_dropped=False):
+  """octree/octree/transform_octree.cpp:286-431 (`octree_drop(octree, depth, ratio)`,
+  tensorflow/libs/transform_octree_op.cc:40-56): every node of level `depth_dropout` leaves
+  with probability `threshold`, together with its subtree.  The reference draws the flags from
+  an engine seeded with the clock; here they come from torch's generator on the device, or from
+  `flags` (one entry per node of the level, non-zero = dropped).  As in the reference, a dropped
+  node of level `depth_dropout` keeps its old child entry (transform_octree.cpp:422-425);
+  `clear_dropped=True` writes -1 there instead, which octree_batch needs for its neighbour
+  tables."""
+  octree = _to_dev(octree)
+  info = octree_info(octree)
+  if not 0 <= depth_dropout <= info.depth:
+    raise ValueError("depth_dropout %d outside [0, %d]" % (depth_dropout, info.depth))
+  n = int(info.nnum(depth_dropout))
+  if flags is None:
+    flags = torch.rand(n, device=_dev(), generator=generator) < float(threshold)
+  flags = torch.as_tensor(flags).to(_dev()).ne(0).to(torch.uint8).contiguous()
+  if flags.numel() != n:
+    raise ValueError("%d flags for the %d nodes of level %d" % (flags.numel(), n, depth_dropout))
+  holder = []
+
+  def alloc(nbytes, _ctx):
+    t = torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=_dev())
+    holder.append(t)
+    return t.data_ptr()
+
+  info_raw = np.zeros(INFO_BYTES, np.uint8)
+  out_ptr = C.c_void_p()
+  _lib.call("ocnn_octree_dropout", _ptr(octree), info.p, _ptr(flags), int(depth_dropout), int(bool(clear_dropped)),
+            _ALLOC_FN(alloc), None,
+            C.c_void_p(info_raw.ctypes.data), C.byref(out_ptr), _stream())
+  out = [t for t in holder if t.data_ptr() == out_ptr.value][-1]
+  out._ocnn_info = _Info(info_raw)
+  return out
+
+
+octree_drop = octree_dropout
 
 
 def octree_scan(octree, axis, scale=1.0):

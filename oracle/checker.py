@@ -126,7 +126,7 @@ class Checker:
       raise ValueError(prefix)
     for n in ("fetch", "points2octree", "octree_batch", "octree_sample",
               "octree_new", "octree_grow", "octree_update", "octree_set_property",
-              "normalize_points", "transform_points", "clip_points", "upgrade_key64", "octree_scan"):
+              "normalize_points", "transform_points", "clip_points", "upgrade_key64", "octree_scan", "octree_dropout"):
       f = getattr(self.lib, prefix + "_" + n, None)
       if f is not None:
         f.restype = C.c_int64
@@ -196,6 +196,23 @@ class Checker:
     ax = np.ascontiguousarray(axis, dtype=np.float32).reshape(-1)
     assert ax.size % 3 == 0
     return self._fetch(self.fn("octree_scan")(_p(b), _p(ax), ax.size // 3, C.c_float(scale)))
+
+  def octree_dropout(self, blob, flags, depth_dropout):
+    """The restatement: the flags of level `depth_dropout` are an argument."""
+    assert self.prefix == "orc"
+    b = np.ascontiguousarray(blob, dtype=np.uint8)
+    f = np.ascontiguousarray(flags, dtype=np.uint8)
+    assert f.size == OctreeBlob(b).nnum[depth_dropout]
+    return self._fetch(self.fn("octree_dropout")(_p(b), _p(f), int(depth_dropout)))
+
+  def octree_dropout_drawn(self, blob, depth_dropout, threshold):
+    """The compiled reference: returns its result and the flags it drew."""
+    assert self.prefix == "ref"
+    b = np.ascontiguousarray(blob, dtype=np.uint8)
+    f = np.zeros(int(OctreeBlob(b).nnum[depth_dropout]), np.uint8)
+    out = self._fetch(self.fn("octree_dropout")(_p(b), C.c_int64(b.size), int(depth_dropout), C.c_float(threshold),
+                                                _p(f), int(f.size)))
+    return out, f
 
   def upgrade_key64(self, blob32):
     b = np.ascontiguousarray(blob32, dtype=np.uint8)

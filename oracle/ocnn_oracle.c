@@ -1909,3 +1909,89 @@ int64_t orc_octree_scan(const void* blob, const float* axis, int n_axis, float s
   for (int d = 0; d <= depth; ++d) free(drop[d]);
   return sz;
 }
+
+/* octree_dropout, octree/octree/transform_octree.cpp:286-431, with the Bernoulli flags of level
+ * `depth_dropout` handed in (the reference draws them from an engine seeded with the clock).
+ * A dropped node takes its whole subtree along; the levels below are compacted, the children
+ * of the kept nodes renumbered.  At `depth_dropout` itself a dropped node KEEPS its old child
+ * index (transform_octree.cpp:422-425) while the non-empty count only counts the kept ones. */
+int64_t orc_octree_dropout(const void* blob, const unsigned char* flags, int depth_dropout) {
+  const OInfo* oi = (const OInfo*)blob;
+  const int depth = oi->depth, dd = depth_dropout;
+  if (dd < 0 || dd > depth || channel_of(oi, kKey) != 1) return ORC_E_UNSUPPORTED;
+  unsigned char* drop[17] = { 0 };
+  drop[dd] = (unsigned char*)calloc((size_t)oi->nnum[dd] + 1, 1);
+  for (int i = 0; i < oi->nnum[dd]; ++i) drop[dd][i] = flags[i] ? 1 : 0;
+  for (int d = dd + 1; d <= depth; ++d) { /* :301-314 */
+    drop[d] = (unsigned char*)calloc((size_t)oi->nnum[d] + 1, 1);
+    const int* child_p = (const int*)prop_ptr(blob, kChild, d - 1);
+    for (int i = 0; i < oi->nnum[d - 1]; ++i) {
+      const int t = child_p[i];
+      if (t < 0) continue;
+      for (int j = 0; j < 8; ++j) drop[d][t * 8 + j] = drop[d - 1][i];
+    }
+  }
+  OInfo o = *oi;
+  for (int d = dd + 1; d <= depth; ++d) { /* :318-329 */
+    int c = 0;
+    for (int i = 0; i < oi->nnum[d]; ++i) if (drop[d][i] == 0) c++;
+    o.nnum[d] = c;
+  }
+  set_nnum_cum(&o, 0);
+  set_ptr_dis(&o);
+  const int sz = sizeof_octree(&o);
+  char* out = result_alloc(sz);
+  if (!out) return ORC_E_NOMEM;
+  memset(out, 0, (size_t)sz);
+  /* levels 0..depth_dropout as they are (:339-361) */
+  const int num = oi->nnum_cum[dd + 1];
+  const int fch = channel_of(oi, kFeature), floc = location_of(oi, kFeature);
+  const int lch = channel_of(oi, kLabel), lloc = location_of(oi, kLabel);
+  const int sch = channel_of(oi, kSplit), sloc = location_of(oi, kSplit);
+  memcpy(out, &o, sizeof(o));
+  memcpy(prop_ptr(out, kKey, 0), prop_ptr(blob, kKey, 0), sizeof(uint64_t) * (size_t)num);
+  memcpy(prop_ptr(out, kChild, 0), prop_ptr(blob, kChild, 0), sizeof(int) * (size_t)num);
+  if (has_prop(oi, kFeature) && floc == -1)
+    memcpy(prop_ptr(out, kFeature, 0), prop_ptr(blob, kFeature, 0), sizeof(float) * (size_t)num * fch);
+  if (has_prop(oi, kLabel) && lloc == -1)
+    memcpy(prop_ptr(out, kLabel, 0), prop_ptr(blob, kLabel, 0), sizeof(float) * (size_t)num * lch);
+  if (has_prop(oi, kSplit) && sloc == -1)
+    memcpy(prop_ptr(out, kSplit, 0), prop_ptr(blob, kSplit, 0), sizeof(float) * (size_t)num * sch);
+  int nne[17] = { 0 };
+  for (int d = dd + 1; d <= depth; ++d) { /* :365-416 */
+    const int nnum_d = oi->nnum[d], nnum_o = o.nnum[d];
+    const int* child_src = (const int*)prop_ptr(blob, kChild, d);
+    const uint64_t* key_src = (const uint64_t*)prop_ptr(blob, kKey, d);
+    int* child_des = (int*)prop_ptr(out, kChild, d);
+    uint64_t* key_des = (uint64_t*)prop_ptr(out, kKey, d);
+    const float* f_in = (has_prop(oi, kFeature) && (floc == -1 || d == depth)) ? (const float*)prop_ptr(blob, kFeature, d) : NULL;
+    float* f_out = f_in ? (float*)prop_ptr(out, kFeature, d) : NULL;
+    const float* l_in = (lch != 0 && (lloc == -1 || d == depth)) ? (const float*)prop_ptr(blob, kLabel, d) : NULL;
+    float* l_out = l_in ? (float*)prop_ptr(out, kLabel, d) : NULL;
+    const float* s_in = (sch != 0 && (sloc == -1 || d == depth)) ? (const float*)prop_ptr(blob, kSplit, d) : NULL;
+    float* s_out = s_in ? (float*)prop_ptr(out, kSplit, d) : NULL;
+    int id = 0;
+    for (int i = 0, j = 0; i < nnum_d; ++i) {
+      if (drop[d][i] != 0) continue;
+      key_des[j] = key_src[i];
+      child_des[j] = child_src[i] < 0 ? child_src[i] : id++;
+      if (f_out) for (int c = 0; c < fch; ++c) f_out[(int64_t)c * nnum_o + j] = f_in[(int64_t)c * nnum_d + i];
+      if (l_out) l_out[j] = l_in[i];
+      if (s_out) s_out[j] = s_in[i];
+      ++j;
+    }
+    nne[d] = id;
+  }
+  { /* :419-430 */
+    int id = 0;
+    const int* child_src = (const int*)prop_ptr(blob, kChild, dd);
+    int* child_des = (int*)prop_ptr(out, kChild, dd);
+    for (int i = 0; i < o.nnum[dd]; ++i)
+      child_des[i] = (drop[dd][i] == 1 || child_src[i] < 0) ? child_src[i] : id++;
+    for (int d = 0; d < dd; ++d) nne[d] = oi->nnum_nempty[d];
+    nne[dd] = id;
+  }
+  for (int d = 0; d <= depth; ++d) ((OInfo*)out)->nnum_nempty[d] = nne[d];
+  for (int d = dd; d <= depth; ++d) free(drop[d]);
+  return sz;
+}

@@ -131,6 +131,9 @@ int orc_octree_deconv_grad(float* grad_data, float* grad_w, const float* data_in
     const float* weights, const float* grad_out, const void* blob, int depth, int num_output,
     const int* kernel_size, int stride, int nempty);
 
+/* octree_dropout, octree/octree/transform_octree.cpp:286-431, with the random flags of level
+ * `depth_dropout` (one byte per node, non-zero = dropped) as an argument. */
+int64_t orc_octree_dropout(const void* blob, const unsigned char* flags, int depth_dropout);
 /* octree_scan, pytorch/cpp/transform_octree.cpp:5-22 over ScanOctree
  * (octree/octree/transform_octree.cpp:11-297): the octree seen from n_axis directions
  * (orc_fetch).  orc_scan_frame: x, y, z axes and lower corner of one view, and its pixel width. */

@@ -19,6 +19,8 @@
 #include <transform_octree.h>
 
 #include <cmath>
+#include <ctime>
+#include <random>
 #include <string>
 
 #include <cstdint>
@@ -87,6 +89,26 @@ int64_t ref_octree_scan(const void* blob, const float* axis, int n_axis, float s
   std::vector<char> out;
   scan_octree.scan(out, parser, ax);
   return keep(out);
+}
+
+// octree/octree/transform_octree.cpp:286-431.  The reference seeds its engine with the wall
+// clock's second.  The clock is read on both sides of the call; when the second did not
+// change, the same engine and distribution are replayed here to hand the flags back, so a
+// restatement can be compared on the very flags the reference drew.
+int64_t ref_octree_dropout(const void* blob, int64_t bytes, int depth_dropout, float threshold, unsigned char* flags,
+    int n_flags) {
+  for (int attempt = 0; attempt < 8; ++attempt) {
+    const time_t t0 = time(nullptr);
+    std::string in((const char*)blob, (size_t)bytes);
+    std::vector<char> out;
+    octree_dropout(out, in, depth_dropout, threshold);
+    if (time(nullptr) != t0) continue;
+    std::default_random_engine generator(static_cast<unsigned>(t0));
+    std::bernoulli_distribution distribution(threshold);
+    for (int i = 0; i < n_flags; ++i) flags[i] = (unsigned char)static_cast<unsigned>(distribution(generator));
+    return keep(out);
+  }
+  return -1;
 }
 
 int64_t ref_upgrade_key64(const void* blob32, int64_t bytes) {
