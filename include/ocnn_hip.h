@@ -216,8 +216,12 @@ int ocnn_octree_interp_ws(float* out, const float* data, int channel, int H, con
     size_t workspace_bytes, ocnn_stream_t stream);
 int ocnn_octree_interp_backward(float* grad_data, const float* grad_out, int channel, int H, int n_pts,
     int method, const int* idx, const float* weight, ocnn_stream_t stream);
-/* The backward call with the same optional workspace: the gradient is accumulated in rows
- * (the atomics of a node fall into two cache lines) and turned channel-major at the end. */
+/* The backward call with an optional workspace of
+ * ocnn_octree_interp_backward_workspace_bytes(channel, H, n_pts, method) bytes (16-byte aligned):
+ * the (point, corner) pairs are binned by node and every node sums its pairs (a gather, no
+ * floating-point atomics); used when the points name at least half as many corners as the
+ * level has nodes, the atomic scatter otherwise or without a workspace. */
+size_t ocnn_octree_interp_backward_workspace_bytes(int channel, int H, int n_pts, int method);
 int ocnn_octree_interp_backward_ws(float* grad_data, const float* grad_out, int channel, int H, int n_pts,
     int method, const int* idx, const float* weight, void* workspace_dev, size_t workspace_bytes,
     ocnn_stream_t stream);

@@ -7,6 +7,7 @@
 //     them, assembles a sparse matrix and multiplies twice; here one kernel does key arithmetic,
 //     the eight binary searches and the weights, and a second one the weighted gather.
 #include "ocnn_common.h"
+#include "scan.h"
 
 namespace ocnn {
 namespace {
@@ -191,74 +192,107 @@ __global__ void __launch_bounds__(kBlock) interp_gather_rows_kernel(float* __res
   }
 }
 
-// The adjoint through row-major storage: the gradient of a node is one contiguous row, so the
-// four atomics of a lane and those of its 15 neighbours fall into two cache lines instead of
-// 64; the rows are turned back into the channel-major tensor at the end.
-template <int K>
-__global__ void __launch_bounds__(kBlock) interp_scatter_rows_kernel(float* __restrict__ xt,
-    const float* __restrict__ grad_out, int channel, int cpad, const int* __restrict__ idx,
-    const float* __restrict__ weight, int n_pts, int normalise) {
-  __shared__ float tile[64][kInterpPts + 1];  // [channel of the chunk][point]
-  const int tid = threadIdx.x;
-  const int pl = tid >> 4, cq = tid & 15;
-  const int p0 = blockIdx.x * kInterpPts;
-  int id[kInterpPts / 16][K];
-  float w[kInterpPts / 16][K];
+// The adjoint as a gather.  The (point, corner) pairs are binned by node with a counting sort
+// (histogram, prefix sum, fill through a cursor per node), the output gradient is copied
+// row-major ([point][channel]: a pair then reads one contiguous row), and every node sums its
+// pairs in registers and writes its row once, through an LDS tile so that the channel-major
+// result leaves in 256-byte rows.  No floating-point atomics; the order of the pairs of a node
+// (and with it the rounding of its sum) follows the order in which the cursor was taken.
+__global__ void interp_hist_kernel(int* __restrict__ count, const int* __restrict__ idx, int64_t n, int H) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int id = idx[i];
+  if ((unsigned)id < (unsigned)H) atomicAdd(&count[id], 1);
+}
+__global__ void __launch_bounds__(kBlock) seg_tile_sum_kernel(const int* __restrict__ v, int64_t n, int* __restrict__ tile_sum) {
+  const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
+  int c = 0;
 #pragma unroll
-  for (int pass = 0; pass < kInterpPts / 16; ++pass) {
-    const int p = p0 + pass * 16 + pl;
-    float norm = 0.0f;
+  for (int j = 0; j < kScanItems; ++j) c += base + j < n ? v[base + j] : 0;
+  int total;
+  block_exclusive_scan(c, &total);
+  if (threadIdx.x == 0) tile_sum[blockIdx.x] = total;
+}
+// v[i] <- sum of v[0..i) (in place)
+__global__ void __launch_bounds__(kBlock) seg_exclusive_kernel(int* __restrict__ v, int64_t n, const int* __restrict__ tile_offset) {
+  const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
+  int x[kScanItems];
+  int c = 0;
 #pragma unroll
-    for (int m = 0; m < K; ++m) {
-      const int v = p < n_pts ? idx[(int64_t)p * K + m] : -1;
-      id[pass][m] = v;
-      w[pass][m] = v >= 0 ? weight[(int64_t)p * K + m] : 0.0f;
-      norm += w[pass][m];
-    }
-    const float inv = normalise ? 1.0f / (norm + 1e-10f) : 1.0f;
+  for (int j = 0; j < kScanItems; ++j) { x[j] = base + j < n ? v[base + j] : 0; c += x[j]; }
+  int total;
+  int run = tile_offset[blockIdx.x] + block_exclusive_scan(c, &total);
 #pragma unroll
-    for (int m = 0; m < K; ++m) w[pass][m] *= inv;
-  }
-  const int lane = tid & 63, row = tid >> 6;
-  for (int chunk = 0; chunk * 64 < cpad; ++chunk) {
-    for (int c = row; c < 64; c += 4) {
-      const int ch = chunk * 64 + c;
-      tile[c][lane] = (ch < channel && p0 + lane < n_pts) ? grad_out[(int64_t)ch * n_pts + p0 + lane] : 0.0f;
-    }
-    __syncthreads();
-    const int c4 = chunk * 64 + 4 * cq;
-    if (c4 < cpad) {
-#pragma unroll
-      for (int pass = 0; pass < kInterpPts / 16; ++pass) {
-        const int pt = pass * 16 + pl;
-        const float g0 = tile[4 * cq + 0][pt], g1 = tile[4 * cq + 1][pt], g2 = tile[4 * cq + 2][pt], g3 = tile[4 * cq + 3][pt];
-#pragma unroll
-        for (int m = 0; m < K; ++m)
-          if (id[pass][m] >= 0) {
-            float* dst = xt + (int64_t)id[pass][m] * cpad + c4;
-            unsafeAtomicAdd(dst + 0, w[pass][m] * g0);
-            unsafeAtomicAdd(dst + 1, w[pass][m] * g1);
-            unsafeAtomicAdd(dst + 2, w[pass][m] * g2);
-            unsafeAtomicAdd(dst + 3, w[pass][m] * g3);
-          }
-      }
-    }
-    __syncthreads();
+  for (int j = 0; j < kScanItems; ++j) {
+    if (base + j < n) v[base + j] = run;
+    run += x[j];
   }
 }
-__global__ void __launch_bounds__(kBlock) rows_back_kernel(float* __restrict__ data, const float* __restrict__ xt,
-    int channel, int H, int cpad) {
-  __shared__ float tile[64][65];
-  const int h0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-  for (int i = ty; i < 64; i += 4) {
-    const int h = h0 + i, c = c0 + tx;
-    tile[i][tx] = (h < H && c < cpad) ? xt[(int64_t)h * cpad + c] : 0.0f;
+// cursor[id] starts at the first slot of node id and ends at the first slot of node id + 1
+template <int K>
+__global__ void interp_fill_kernel(int2* __restrict__ pairs, int* __restrict__ cursor, const int* __restrict__ idx,
+    const float* __restrict__ weight, int n_pts, int H, int normalise) {
+  const int p = blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= n_pts) return;
+  int id[K];
+  float w[K];
+  float norm = 0.0f;
+#pragma unroll
+  for (int m = 0; m < K; ++m) {
+    id[m] = idx[(int64_t)p * K + m];
+    w[m] = id[m] >= 0 ? weight[(int64_t)p * K + m] : 0.0f;
+    norm += w[m];
   }
-  __syncthreads();
-  for (int i = ty; i < 64; i += 4) {
-    const int c = c0 + i, h = h0 + tx;
-    if (c < channel && h < H) data[(int64_t)c * H + h] = tile[tx][i];
+  const float inv = normalise ? 1.0f / (norm + 1e-10f) : 1.0f;
+#pragma unroll
+  for (int m = 0; m < K; ++m)
+    if ((unsigned)id[m] < (unsigned)H) pairs[atomicAdd(&cursor[id[m]], 1)] = make_int2(p, __float_as_int(w[m] * inv));
+}
+__global__ void __launch_bounds__(kBlock) interp_reduce_kernel(float* __restrict__ grad_data,
+    const float4* __restrict__ rows, const int2* __restrict__ pairs, const int* __restrict__ ends, int channel, int cpad4,
+    int H) {
+  __shared__ float tile[64][65];   // [node][channel of the chunk]
+  const int tid = threadIdx.x;
+  const int nl = tid >> 4, cq = tid & 15;
+  const int n0 = blockIdx.x * 64;
+  const int lane = tid & 63, row = tid >> 6;
+  int b[4], e[4];
+#pragma unroll
+  for (int pass = 0; pass < 4; ++pass) {
+    const int node = n0 + pass * 16 + nl;
+    b[pass] = (node < H && node > 0) ? ends[node - 1] : 0;
+    e[pass] = node < H ? ends[node] : 0;
+  }
+  for (int chunk = 0; chunk * 16 < cpad4; ++chunk) {
+    const int c4 = chunk * 16 + cq;
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+      float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      if (c4 < cpad4) {
+        int j = b[pass];
+        for (; j + 1 < e[pass]; j += 2) {
+          const int2 p0 = pairs[j], p1 = pairs[j + 1];
+          const float4 g0 = rows[(int64_t)p0.x * cpad4 + c4], g1 = rows[(int64_t)p1.x * cpad4 + c4];
+          const float w0 = __int_as_float(p0.y), w1 = __int_as_float(p1.y);
+          acc.x += w0 * g0.x; acc.y += w0 * g0.y; acc.z += w0 * g0.z; acc.w += w0 * g0.w;
+          acc.x += w1 * g1.x; acc.y += w1 * g1.y; acc.z += w1 * g1.z; acc.w += w1 * g1.w;
+        }
+        if (j < e[pass]) {
+          const int2 p0 = pairs[j];
+          const float4 g0 = rows[(int64_t)p0.x * cpad4 + c4];
+          const float w0 = __int_as_float(p0.y);
+          acc.x += w0 * g0.x; acc.y += w0 * g0.y; acc.z += w0 * g0.z; acc.w += w0 * g0.w;
+        }
+      }
+      float* t = &tile[pass * 16 + nl][4 * cq];
+      t[0] = acc.x; t[1] = acc.y; t[2] = acc.z; t[3] = acc.w;
+    }
+    __syncthreads();
+    for (int c = row; c < 64; c += 4) {
+      const int ch = chunk * 64 + c, node = n0 + lane;
+      if (ch < channel && node < H) grad_data[(int64_t)ch * H + node] = tile[lane][c];
+    }
+    __syncthreads();
   }
 }
 
@@ -287,6 +321,21 @@ __global__ void interp_scatter_kernel(float* __restrict__ grad_data, const float
       if (id[m] >= 0) unsafeAtomicAdd(grad_data + (int64_t)c * H + id[m], w[m] * g);
   }
 }
+
+// workspace of the gathered adjoint: segment ends, (point, weight) pairs, row-major output
+// gradient, tile sums of the prefix scan
+struct InterpBackLayout {
+  size_t ends, pairs, rows, scan, total;
+  InterpBackLayout(int channel, int H, int n_pts, int K) {
+    auto al = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    size_t off = 0;
+    ends = off; off += al(sizeof(int) * ((size_t)H + 1));
+    pairs = off; off += al(sizeof(int2) * (size_t)n_pts * K);
+    rows = off; off += al(sizeof(float) * (size_t)n_pts * ((channel + 3) / 4 * 4));
+    scan = off; off += al(scan_scratch_bytes(H));
+    total = off;
+  }
+};
 
 }  // namespace
 }  // namespace ocnn
@@ -318,6 +367,11 @@ int ocnn_align_backward(const float* top, int top_h, int channel, float* btm, in
 size_t ocnn_octree_interp_workspace_bytes(int channel, int H) {
   if (channel <= 0 || H <= 0) return 0;
   return ((size_t)H * (size_t)((channel + 3) / 4 * 4) * sizeof(float) + 255) & ~(size_t)255;
+}
+
+size_t ocnn_octree_interp_backward_workspace_bytes(int channel, int H, int n_pts, int method) {
+  if (channel <= 0 || H <= 0 || n_pts <= 0 || (method != 0 && method != 1)) return 0;
+  return InterpBackLayout(channel, H, n_pts, method == 0 ? 1 : 8).total;
 }
 
 int ocnn_octree_interp(float* out, const float* data, int channel, int H, const uint64_t* key, int n_key,
@@ -373,20 +427,29 @@ int ocnn_octree_interp_backward_ws(float* grad_data, const float* grad_out, int 
   OCNN_REQUIRE(method == 0 || method == 1, OCNN_E_BADARG, "method %d", method);
   hipStream_t s = as_stream(stream);
   const int Kc = method == 0 ? 1 : 8;
-  if (workspace_dev && H > 0 && n_pts > 0 && workspace_bytes >= ocnn_octree_interp_workspace_bytes(channel, H) &&
+  const size_t need = ocnn_octree_interp_backward_workspace_bytes(channel, H, n_pts, method);
+  if (workspace_dev && H > 0 && n_pts > 0 && need > 0 && workspace_bytes >= need &&
       (reinterpret_cast<uintptr_t>(workspace_dev) & 15) == 0 && (int64_t)n_pts * Kc >= H / 2) {
     const int cpad = (channel + 3) / 4 * 4;
-    float* xt = static_cast<float*>(workspace_dev);
-    const int64_t words = (int64_t)H * cpad;
-    zero_kernel<<<blocks_for(words), kBlock, 0, s>>>(xt, words);
-    if (Kc == 1)
-      interp_scatter_rows_kernel<1><<<blocks_for(n_pts, kInterpPts), kBlock, 0, s>>>(xt, grad_out, channel, cpad, idx,
-          weight, n_pts, method);
-    else
-      interp_scatter_rows_kernel<8><<<blocks_for(n_pts, kInterpPts), kBlock, 0, s>>>(xt, grad_out, channel, cpad, idx,
-          weight, n_pts, method);
-    rows_back_kernel<<<dim3(blocks_for(H, 64), blocks_for(channel, 64)), kBlock, 0, s>>>(grad_data, xt, channel, H, cpad);
-    OCNN_LAUNCH_OK("interp_scatter_rows");
+    const InterpBackLayout L(channel, H, n_pts, Kc);
+    char* ws = static_cast<char*>(workspace_dev);
+    int* ends = reinterpret_cast<int*>(ws + L.ends);
+    int2* pairs = reinterpret_cast<int2*>(ws + L.pairs);
+    float* rows = reinterpret_cast<float*>(ws + L.rows);
+    int* tiles = reinterpret_cast<int*>(ws + L.scan);
+    const int64_t n_pairs = (int64_t)n_pts * Kc;
+    zero_kernel<<<blocks_for(H), kBlock, 0, s>>>(reinterpret_cast<float*>(ends), H);
+    interp_hist_kernel<<<blocks_for(n_pairs), kBlock, 0, s>>>(ends, idx, n_pairs, H);
+    const int n_tiles = scan_tiles(H);
+    seg_tile_sum_kernel<<<n_tiles, kBlock, 0, s>>>(ends, H, tiles);
+    scan_tiles_kernel<0><<<1, kBlock, 0, s>>>(tiles, n_tiles, nullptr);
+    seg_exclusive_kernel<<<n_tiles, kBlock, 0, s>>>(ends, H, tiles);
+    if (Kc == 1) interp_fill_kernel<1><<<blocks_for(n_pts), kBlock, 0, s>>>(pairs, ends, idx, weight, n_pts, H, method);
+    else interp_fill_kernel<8><<<blocks_for(n_pts), kBlock, 0, s>>>(pairs, ends, idx, weight, n_pts, H, method);
+    rows_copy_kernel<<<dim3(blocks_for(n_pts, 64), blocks_for(cpad, 64)), kBlock, 0, s>>>(rows, grad_out, channel, n_pts, cpad);
+    interp_reduce_kernel<<<blocks_for(H, 64), kBlock, 0, s>>>(grad_data, reinterpret_cast<const float4*>(rows), pairs, ends,
+        channel, cpad / 4, H);
+    OCNN_LAUNCH_OK("interp_reduce");
     return OCNN_OK;
   }
   const int64_t n = (int64_t)H * channel;

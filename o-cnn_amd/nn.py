@@ -975,7 +975,8 @@ def octree_interp_pts_grad(grad_out, idx, weight, H, method="linear"):
   channel, n = grad_out.size(1), grad_out.size(2)
   out = torch.empty(1, channel, H, 1, dtype=torch.float32, device=grad_out.device)
   K = 1 if method == "nearest" else 8
-  ws_bytes = _lib.get().ocnn_octree_interp_workspace_bytes(channel, H) if n * K >= H // 2 else 0
+  ws_bytes = (_lib.get().ocnn_octree_interp_backward_workspace_bytes(channel, H, n, int(method == "linear"))
+              if n * K >= H // 2 else 0)
   ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=grad_out.device)
   _lib.call("ocnn_octree_interp_backward_ws", _ptr(out), _ptr(grad_out), channel, H, n, int(method == "linear"),
             _ptr(idx), _ptr(weight), _ptr(ws) if ws_bytes else C.c_void_p(0), C.c_size_t(ws_bytes), _stream())
