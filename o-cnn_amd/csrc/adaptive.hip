@@ -115,91 +115,93 @@ __device__ inline int intersect_cube(float* V, const float* pt, const float* pt_
   return nv;
 }
 
-// Ordered sums over the non-empty leaves j0 <= j < j1.  `load(j, vals)` fetches the NV values
-// of leaf j into this lane's registers.  256 leaves at a time are requested together (the
-// chain of a node high up in the tree covers the whole finest level: memory latency must not
-// be paid per leaf), the non-empty ones are packed into the wavefront's LDS block in leaf
-// order, and then lane c adds up value c leaf after leaf: the channels run side by side, each
-// in the reference's order.  Returns the number of non-empty leaves; sum[c] / last[c] get the
-// sum and the last value of channel c on every lane.
-constexpr int kPassRounds = 4, kPassValues = 8;
-template <int NV, class Load>
-__device__ inline int ordered_sums(int j0, int j1, int lane, const int* __restrict__ child_D, float* __restrict__ lds,
-    Load load, float* sum, float* last) {
+// Ordered sums over the non-empty leaves of a range.  The non-empty leaves of the finest level
+// are packed once, in leaf order (LeafPack below; rows padded to whole 16-byte units), so a
+// node's leaves are the packed range k0 <= k < k1 of every row.  row[c] is the packed row of
+// value c (null: absent, sums to zero).  256 leaves at a time go through the wavefront's LDS
+// block (a lane moves four consecutive leaves of a value with one 16-byte load and store), and
+// lane c adds up value c leaf after leaf: the channels run side by side, each in the
+// reference's order.  Leaves outside the range enter as +0, which changes no partial sum (a
+// partial sum is never -0: the chain starts at +0).  The next 256 leaves are requested before
+// the current ones are added (the chain of a node high up in the tree covers the whole finest
+// level: memory latency must not be paid per block).  sum[c] / last[c] get the sum and the
+// last value of channel c on every lane.
+constexpr int kPassValues = 8, kPassLeaves = 256;
+template <int NV>
+__device__ inline void ordered_sums(int k0, int k1, int lane, float* __restrict__ lds, const float* const (&row)[NV],
+    float* sum, float* last) {
   static_assert(NV <= kPassValues, "LDS block too small");
-  int leaves = 0;
-  float acc = 0.0f, lastv = 0.0f;
-  for (int base = j0; base < j1; base += 64 * kPassRounds) {
-    float vals[kPassRounds][NV];
-    bool ok[kPassRounds];
+  float acc = 0.0f;
+  float4 vals[NV];
+  auto request = [&](int base) {
+    const int k = base + 4 * lane;
 #pragma unroll
-    for (int u = 0; u < kPassRounds; ++u) {
-      const int j = base + u * 64 + lane;
-      ok[u] = j < j1 && child_D[j] != -1;
+    for (int c = 0; c < NV; ++c) {
+      float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      if (row[c] && k < k1) v = *reinterpret_cast<const float4*>(row[c] + k);
+      v.x = (k >= k0 && k < k1) ? v.x : 0.0f;
+      v.y = (k + 1 >= k0 && k + 1 < k1) ? v.y : 0.0f;
+      v.z = (k + 2 >= k0 && k + 2 < k1) ? v.z : 0.0f;
+      v.w = (k + 3 >= k0 && k + 3 < k1) ? v.w : 0.0f;
+      vals[c] = v;
     }
+  };
+  const int kb = k0 < k1 ? (k0 & ~3) : k1;   // an empty range runs no block
+  if (k0 < k1) request(kb);
+  for (int base = kb; base < k1; base += kPassLeaves) {
 #pragma unroll
-    for (int u = 0; u < kPassRounds; ++u) {
-#pragma unroll
-      for (int c = 0; c < NV; ++c) vals[u][c] = 0.0f;
-      if (ok[u]) load(base + u * 64 + lane, vals[u]);
-    }
-    int total = 0;
-#pragma unroll
-    for (int u = 0; u < kPassRounds; ++u) {
-      const uint64_t mask = __ballot(ok[u]);
-      if (ok[u]) {
-        const int p = total + __popcll(mask & ((1ull << lane) - 1));
-#pragma unroll
-        for (int c = 0; c < NV; ++c) lds[p * NV + c] = vals[u][c];
-      }
-      total += __popcll(mask);
-    }
+    for (int c = 0; c < NV; ++c) *reinterpret_cast<float4*>(lds + c * kPassLeaves + 4 * lane) = vals[c];
+    if (base + kPassLeaves < k1) request(base + kPassLeaves);
     __builtin_amdgcn_wave_barrier();   // same wavefront: the LDS unit keeps its accesses in order
+    const int total = min(kPassLeaves, k1 - base);
     if (lane < NV) {
-#pragma unroll 8
-      for (int t = 0; t < total; ++t) {
-        lastv = lds[t * NV + lane];
-        acc = __fadd_rn(acc, lastv);
+      // the adds form one dependent chain; the LDS reads of the next 16 leaves are in flight
+      // while the current 16 are added
+      constexpr int kStep = 16;
+      const float4* src = reinterpret_cast<const float4*>(lds + lane * kPassLeaves);
+      float4 cur[kStep / 4];
+#pragma unroll
+      for (int i = 0; i < kStep / 4; ++i) cur[i] = src[i];
+      for (int t = 0; t < total; t += kStep) {
+        float4 nxt[kStep / 4];
+        const int tn = min(t + kStep, kPassLeaves - kStep);          // stays inside the block
+#pragma unroll
+        for (int i = 0; i < kStep / 4; ++i) nxt[i] = src[tn / 4 + i];
+#pragma unroll
+        for (int i = 0; i < kStep / 4; ++i) {
+          acc = __fadd_rn(acc, cur[i].x); acc = __fadd_rn(acc, cur[i].y);
+          acc = __fadd_rn(acc, cur[i].z); acc = __fadd_rn(acc, cur[i].w);
+        }
+#pragma unroll
+        for (int i = 0; i < kStep / 4; ++i) cur[i] = nxt[i];
       }
     }
     __builtin_amdgcn_wave_barrier();
-    leaves += total;
   }
 #pragma unroll
-  for (int c = 0; c < NV; ++c) { sum[c] = read_lane(acc, c); last[c] = read_lane(lastv, c); }
-  return leaves;
+  for (int c = 0; c < NV; ++c) {
+    sum[c] = read_lane(acc, c);
+    last[c] = (row[c] && k0 < k1) ? row[c][k1 - 1] : 0.0f;
+  }
 }
-// The same packing for a sum whose terms interleave the channels (the normal error): every lane
+// The same walk for a sum whose terms interleave the channels (the normal error): every lane
 // takes the same walk over the packed leaves, `term(vals)` gives the leaf's terms in order.
 template <int NV, class Load, class Terms>
-__device__ inline void ordered_terms(int j0, int j1, int lane, const int* __restrict__ child_D, float* __restrict__ lds,
-    Load load, Terms terms) {
-  for (int base = j0; base < j1; base += 64 * kPassRounds) {
-    float vals[kPassRounds][NV];
-    bool ok[kPassRounds];
+__device__ inline void ordered_terms(int k0, int k1, int lane, float* __restrict__ lds, Load load, Terms terms) {
+  constexpr int kPassRounds = kPassLeaves / 64;
+  for (int base = k0; base < k1; base += 64 * kPassRounds) {
 #pragma unroll
     for (int u = 0; u < kPassRounds; ++u) {
-      const int j = base + u * 64 + lane;
-      ok[u] = j < j1 && child_D[j] != -1;
-    }
+      float vals[NV];
 #pragma unroll
-    for (int u = 0; u < kPassRounds; ++u) {
+      for (int c = 0; c < NV; ++c) vals[c] = 0.0f;
+      const int k = base + u * 64 + lane;
+      if (k < k1) load(k, vals);
 #pragma unroll
-      for (int c = 0; c < NV; ++c) vals[u][c] = 0.0f;
-      if (ok[u]) load(base + u * 64 + lane, vals[u]);
-    }
-    int total = 0;
-#pragma unroll
-    for (int u = 0; u < kPassRounds; ++u) {
-      const uint64_t mask = __ballot(ok[u]);
-      if (ok[u]) {
-        const int p = total + __popcll(mask & ((1ull << lane) - 1));
-#pragma unroll
-        for (int c = 0; c < NV; ++c) lds[p * NV + c] = vals[u][c];
-      }
-      total += __popcll(mask);
+      for (int c = 0; c < NV; ++c) lds[(u * 64 + lane) * NV + c] = vals[c];
     }
     __builtin_amdgcn_wave_barrier();
+    const int total = min(64 * kPassRounds, k1 - base);
 #pragma unroll 4
     for (int t = 0; t < total; ++t) {
       float one[NV];
@@ -211,6 +213,27 @@ __device__ inline void ordered_terms(int j0, int j1, int lane, const int* __rest
   }
 }
 
+// The non-empty leaves in leaf order: rank[j] = non-empty leaves before leaf j (rank[nD] = their
+// number), and their normals / points / features side by side, channel-major rows of nD.
+struct LeafPred {
+  const int* child_D;
+  __device__ bool operator()(int64_t j) const { return child_D[j] != -1; }
+};
+struct LeafPack {
+  int* rank;
+  int64_t nD, nP;   // leaves; row stride of the packed arrays
+  int cf;
+  const float *nrm_D, *pt_D, *feat_D;
+  float *nrm_P, *pt_P, *feat_P;
+  __device__ void operator()(int64_t j, bool f, int r) const {
+    rank[j] = r;
+    if (!f) return;
+    if (nrm_D) for (int c = 0; c < 3; ++c) nrm_P[c * nP + r] = nrm_D[c * nD + j];
+    if (pt_D) for (int c = 0; c < 3; ++c) pt_P[c * nP + r] = pt_D[c * nD + j];
+    for (int c = 0; c < cf; ++c) feat_P[c * nP + r] = feat_D[c * nD + j];
+  }
+};
+
 struct SignalArgs {
   int d, depth, n, nD, cf, ch_dis, adp_layer, calc_nerr, calc_derr;
   float imul;
@@ -219,6 +242,9 @@ struct SignalArgs {
   const int *dnum, *didx;     // level d
   const int* child_D;         // finest level: structure and signal, channel-major rows of nD
   const float *nrm_D, *pt_D, *feat_D, *lab_D;
+  const int* rank_D;          // non-empty leaves before a leaf; [nD] = their number
+  const float *nrm_P, *pt_P, *feat_P;   // the non-empty leaves packed in leaf order, rows of nP
+  int64_t nP;
   float *normal, *pt, *feature, *label, *dis, *nerr, *derr;   // level d (null: absent)
 };
 
@@ -236,9 +262,9 @@ __global__ __launch_bounds__(kBlock) void signal_kernel(const SignalLevels* __re
   while (w >= levels->first_wave[d + 1]) ++d;
   const SignalArgs& a = levels->level[d];
   const int i = w - levels->first_wave[d];
-  __shared__ float s_pass[kBlock / 64][kPassRounds * 64 * kPassValues];
+  __shared__ __attribute__((aligned(16))) float s_pass[kBlock / 64][kPassLeaves * kPassValues];
   float* lds = s_pass[threadIdx.x >> 6];
-  const int64_t n = a.n, nD = a.nD;
+  const int64_t n = a.n;
   const bool has_normal = a.nrm_D != nullptr, has_pt = a.pt_D != nullptr;
   if (a.child[i] == -1) {   // empty: zero signal, no label, errors "infinite"
     if (lane == 0) {
@@ -258,10 +284,15 @@ __global__ __launch_bounds__(kBlock) void signal_kernel(const SignalLevels* __re
   // sums of normals and points over the non-empty leaves, in leaf order
   float n_avg[3] = {0.0f, 0.0f, 0.0f}, last_n[3] = {0.0f, 0.0f, 0.0f}, pt_avg[3] = {0.0f, 0.0f, 0.0f};
   float sum6[6], last6[6];
-  const int leaves = ordered_sums<6>(j0, j1, lane, a.child_D, lds, [&](int j, float* v) {
-    if (has_normal) for (int c = 0; c < 3; ++c) v[c] = a.nrm_D[c * nD + j];
-    if (has_pt) for (int c = 0; c < 3; ++c) v[3 + c] = a.pt_D[c * nD + j];
-  }, sum6, last6);
+  const int k0 = a.rank_D[j0], k1 = a.rank_D[j1];
+  const int leaves = k1 - k0;
+  const int64_t nP = a.nP;
+  {
+    const float* const rows6[6] = {has_normal ? a.nrm_P : nullptr, has_normal ? a.nrm_P + nP : nullptr,
+        has_normal ? a.nrm_P + 2 * nP : nullptr, has_pt ? a.pt_P : nullptr, has_pt ? a.pt_P + nP : nullptr,
+        has_pt ? a.pt_P + 2 * nP : nullptr};
+    ordered_sums<6>(k0, k1, lane, lds, rows6, sum6, last6);
+  }
   for (int c = 0; c < 3; ++c) { n_avg[c] = sum6[c]; last_n[c] = last6[c]; pt_avg[c] = sum6[3 + c]; }
   if (has_normal) {
     float len = norm3(n_avg);
@@ -281,9 +312,9 @@ __global__ __launch_bounds__(kBlock) void signal_kernel(const SignalLevels* __re
   for (int c0 = 0; c0 < a.cf; c0 += kPassValues) {   // features: eight channels per ordered pass
     float fsum[kPassValues], flast[kPassValues];
     const int nc = min(kPassValues, a.cf - c0);
-    ordered_sums<kPassValues>(j0, j1, lane, a.child_D, lds, [&](int j, float* v) {
-      for (int c = 0; c < kPassValues; ++c) if (c < nc) v[c] = a.feat_D[(c0 + c) * nD + j];
-    }, fsum, flast);
+    const float* rows8[kPassValues];
+    for (int c = 0; c < kPassValues; ++c) rows8[c] = c < nc ? a.feat_P + (c0 + c) * nP : nullptr;
+    ordered_sums<kPassValues>(k0, k1, lane, lds, rows8, fsum, flast);
     if (lane == 0)
       for (int c = 0; c < kPassValues; ++c) if (c < nc) a.feature[(c0 + c) * n + i] = div_rn(fsum[c], count);
   }
@@ -330,8 +361,8 @@ __global__ __launch_bounds__(kBlock) void signal_kernel(const SignalLevels* __re
     float nm_err = 1.0e20f;
     if (a.calc_nerr && has_normal && a.d >= a.adp_layer) {
       nm_err = 0.0f;
-      ordered_terms<3>(j0, j1, lane, a.child_D, lds,
-          [&](int j, float* v) { for (int c = 0; c < 3; ++c) v[c] = a.nrm_D[c * nD + j]; },
+      ordered_terms<3>(k0, k1, lane, lds,
+          [&](int k, float* v) { for (int c = 0; c < 3; ++c) v[c] = a.nrm_P[c * nP + k]; },
           [&](const float* v) {
             for (int c = 0; c < 3; ++c) {
               const float tmp = __fsub_rn(v[c], n_avg[c]);
@@ -349,10 +380,9 @@ __global__ __launch_bounds__(kBlock) void signal_kernel(const SignalLevels* __re
       float pt_avg1[3];
       for (int c = 0; c < 3; ++c) pt_avg1[c] = __fmul_rn(pt_avg[c], scale);
       float distance_max1 = -1.0f;
-      for (int j = j0 + lane; j < j1; j += 64) {
-        if (a.child_D[j] == -1) continue;
+      for (int k = k0 + lane; k < k1; k += 64) {
         float dis = 0.0f;
-        for (int c = 0; c < 3; ++c) dis = __fadd_rn(dis, __fmul_rn(__fsub_rn(a.pt_D[c * nD + j], pt_avg1[c]), n_avg[c]));
+        for (int c = 0; c < 3; ++c) dis = __fadd_rn(dis, __fmul_rn(__fsub_rn(a.pt_P[c * nP + k], pt_avg1[c]), n_avg[c]));
         distance_max1 = fmaxf(distance_max1, fabsf(dis));
       }
       distance_max1 = wave_max(distance_max1);
@@ -364,11 +394,10 @@ __global__ __launch_bounds__(kBlock) void signal_kernel(const SignalLevels* __re
         float vk[3];
         for (int c = 0; c < 3; ++c) vk[c] = __fmul_rn(vtx[3 * k + c], scale);
         float distance_min = 1.0e30f;
-        for (int j = j0 + lane; j < j1; j += 64) {
-          if (a.child_D[j] == -1) continue;
+        for (int k = k0 + lane; k < k1; k += 64) {
           float dis = 0.0f;
           for (int c = 0; c < 3; ++c) {
-            const float ptc = __fsub_rn(a.pt_D[c * nD + j], vk[c]);
+            const float ptc = __fsub_rn(a.pt_P[c * nP + k], vk[c]);
             dis = __fadd_rn(dis, __fmul_rn(ptc, ptc));
           }
           distance_min = fminf(distance_min, sqrt_rn(dis));
@@ -657,6 +686,10 @@ int adaptive_finish(const AdaptiveInput& in, ocnn_alloc_fn alloc, void* alloc_ct
     o_dnum[d] = take(4 * n); o_didx[d] = take(4 * n); o_drop[d] = take(4 * n); o_pos[d] = take(4 * n);
     o_nchild[d] = take(4 * n);
   }
+  const size_t nDp = (size_t)o0.nnum[D] + 1;
+  const size_t nP = ((size_t)o0.nnum[D] + 3) & ~(size_t)3;   // packed rows in whole 16-byte units
+  const size_t o_rank = take(4 * nDp), o_nrmP = take(4 * 3 * nP + 16), o_ptP = take(4 * 3 * nP + 16);
+  const size_t o_featP = take(4 * (size_t)(cf > 0 ? cf : 1) * nP + 16);
   const size_t o_scan = take(scan_scratch_bytes(max_n));
   const size_t o_counts = take(sizeof(int) * 64);      // [0..16] kept nodes, [17..33] kept links, [34..50] any_kept
   const size_t o_best = take(sizeof(unsigned long long) * kMaxD);
@@ -709,6 +742,16 @@ int adaptive_finish(const AdaptiveInput& in, ocnn_alloc_fn alloc, void* alloc_ct
   OCNN_LAUNCH_OK("cover");
   fill_kernel<<<blocks_for(o0.nnum[D]), kBlock, 0, s>>>(nerr[D], o0.nnum[D], 1.0e20f);
   fill_kernel<<<blocks_for(o0.nnum[D]), kBlock, 0, s>>>(derr[D], o0.nnum[D], 1.0e20f);
+  int* rank_D = reinterpret_cast<int*>(ws + o_rank);
+  float* nrm_P = reinterpret_cast<float*>(ws + o_nrmP);
+  float* pt_P = reinterpret_cast<float*>(ws + o_ptP);
+  float* feat_P = reinterpret_cast<float*>(ws + o_featP);
+  {
+    LeafPred lp{child[D]};
+    LeafPack lo{rank_D, (int64_t)o0.nnum[D], (int64_t)nP, cf, normal[D], pt[D], feature[D], nrm_P, pt_P, feat_P};
+    hipError_t e = flag_scan(lp, lo, (int64_t)o0.nnum[D], reinterpret_cast<int*>(ws + o_scan), rank_D + o0.nnum[D], s);
+    OCNN_REQUIRE(e == hipSuccess, OCNN_E_HIP, "leaf scan: %s", hipGetErrorString(e));
+  }
   {
     SignalLevels* L = new SignalLevels;
     memset(L, 0, sizeof(SignalLevels));
@@ -720,6 +763,7 @@ int adaptive_finish(const AdaptiveInput& in, ocnn_alloc_fn alloc, void* alloc_ct
       a.imul = imul;
       a.key = key[d]; a.child = child[d]; a.dnum = dnum[d]; a.didx = didx[d];
       a.child_D = child[D]; a.nrm_D = normal[D]; a.pt_D = pt[D]; a.feat_D = feature[D]; a.lab_D = label[D];
+      a.rank_D = rank_D; a.nrm_P = nrm_P; a.pt_P = pt_P; a.feat_P = feat_P; a.nP = (int64_t)nP;
       a.normal = normal[d]; a.pt = pt[d]; a.feature = feature[d]; a.label = label[d]; a.dis = dis[d];
       a.nerr = nerr[d]; a.derr = derr[d];
       L->first_wave[d] = waves;
