@@ -40,6 +40,11 @@ __device__ inline int wave_min_i(int v) {
   for (int o = 32; o > 0; o >>= 1) v = min(v, __shfl_xor(v, o, 64));
   return v;
 }
+__device__ inline int wave_max_i(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o, 64));
+  return v;
+}
 __device__ inline int wave_sum_i(int v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
@@ -223,14 +228,15 @@ struct LeafPack {
   int* rank;
   int64_t nD, nP;   // leaves; row stride of the packed arrays
   int cf;
-  const float *nrm_D, *pt_D, *feat_D;
-  float *nrm_P, *pt_P, *feat_P;
+  const float *nrm_D, *pt_D, *feat_D, *lab_D;
+  float *nrm_P, *pt_P, *feat_P, *lab_P;
   __device__ void operator()(int64_t j, bool f, int r) const {
     rank[j] = r;
     if (!f) return;
     if (nrm_D) for (int c = 0; c < 3; ++c) nrm_P[c * nP + r] = nrm_D[c * nD + j];
     if (pt_D) for (int c = 0; c < 3; ++c) pt_P[c * nP + r] = pt_D[c * nD + j];
     for (int c = 0; c < cf; ++c) feat_P[c * nP + r] = feat_D[c * nD + j];
+    if (lab_D) lab_P[r] = lab_D[j];
   }
 };
 
@@ -243,7 +249,7 @@ struct SignalArgs {
   const int* child_D;         // finest level: structure and signal, channel-major rows of nD
   const float *nrm_D, *pt_D, *feat_D, *lab_D;
   const int* rank_D;          // non-empty leaves before a leaf; [nD] = their number
-  const float *nrm_P, *pt_P, *feat_P;   // the non-empty leaves packed in leaf order, rows of nP
+  const float *nrm_P, *pt_P, *feat_P, *lab_P;   // the non-empty leaves packed in leaf order, rows of nP
   int64_t nP;
   float *normal, *pt, *feature, *label, *dis, *nerr, *derr;   // level d (null: absent)
 };
@@ -319,21 +325,46 @@ __global__ __launch_bounds__(kBlock) void signal_kernel(const SignalLevels* __re
       for (int c = 0; c < kPassValues; ++c) if (c < nc) a.feature[(c0 + c) * n + i] = div_rn(fsum[c], count);
   }
   if (a.label) {
-    // most frequent label of the range, the smallest one on a tie: walk the distinct labels upwards
-    int last = -1, best = -1, best_cnt = 0;
-    for (;;) {
-      int m = 0x7fffffff;
-      for (int j = j0 + lane; j < j1; j += 64) {
-        const int l = (int)a.lab_D[j];
-        if (l > last && l < m) m = l;
+    // most frequent label (>= 0) of the non-empty leaves, the smallest one on a tie
+    int mx = -1;
+    for (int k = k0 + lane; k < k1; k += 64) mx = max(mx, (int)a.lab_P[k]);
+    mx = wave_max_i(mx);
+    int best = -1, best_cnt = 0;
+    if (mx >= 0 && mx < kPassLeaves * kPassValues) {
+      // the labels fit the wavefront's LDS block: one counting pass
+      int* bins = reinterpret_cast<int*>(lds);
+      for (int b = lane; b <= mx; b += 64) bins[b] = 0;
+      __builtin_amdgcn_wave_barrier();
+      for (int k = k0 + lane; k < k1; k += 64) {
+        const int l = (int)a.lab_P[k];
+        if (l >= 0) atomicAdd(&bins[l], 1);
       }
-      m = wave_min_i(m);
-      if (m == 0x7fffffff) break;
-      int cnt = 0;
-      for (int j = j0 + lane; j < j1; j += 64) cnt += ((int)a.lab_D[j] == m) ? 1 : 0;
-      cnt = wave_sum_i(cnt);
-      if (cnt > best_cnt) { best = m; best_cnt = cnt; }
-      last = m;
+      __builtin_amdgcn_wave_barrier();
+      for (int b = lane; b <= mx; b += 64) {   // ascending: a lane keeps the smallest label of its best count
+        const int c = bins[b];
+        if (c > best_cnt) { best_cnt = c; best = b; }
+      }
+      const int m = wave_max_i(best_cnt);
+      best = wave_min_i((m > 0 && best_cnt == m) ? best : 0x7fffffff);
+      best_cnt = m;
+      __builtin_amdgcn_wave_barrier();
+    } else if (mx >= 0) {
+      // any label values: walk the distinct labels upwards
+      int last = -1;
+      for (;;) {
+        int m = 0x7fffffff;
+        for (int k = k0 + lane; k < k1; k += 64) {
+          const int l = (int)a.lab_P[k];
+          if (l > last && l < m) m = l;
+        }
+        m = wave_min_i(m);
+        if (m == 0x7fffffff) break;
+        int cnt = 0;
+        for (int k = k0 + lane; k < k1; k += 64) cnt += ((int)a.lab_P[k] == m) ? 1 : 0;
+        cnt = wave_sum_i(cnt);
+        if (cnt > best_cnt) { best = m; best_cnt = cnt; }
+        last = m;
+      }
     }
     if (lane == 0) a.label[i] = best_cnt > 0 ? (float)best : -1.0f;
   }
@@ -689,7 +720,7 @@ int adaptive_finish(const AdaptiveInput& in, ocnn_alloc_fn alloc, void* alloc_ct
   const size_t nDp = (size_t)o0.nnum[D] + 1;
   const size_t nP = ((size_t)o0.nnum[D] + 3) & ~(size_t)3;   // packed rows in whole 16-byte units
   const size_t o_rank = take(4 * nDp), o_nrmP = take(4 * 3 * nP + 16), o_ptP = take(4 * 3 * nP + 16);
-  const size_t o_featP = take(4 * (size_t)(cf > 0 ? cf : 1) * nP + 16);
+  const size_t o_featP = take(4 * (size_t)(cf > 0 ? cf : 1) * nP + 16), o_labP = take(4 * nP + 16);
   const size_t o_scan = take(scan_scratch_bytes(max_n));
   const size_t o_counts = take(sizeof(int) * 64);      // [0..16] kept nodes, [17..33] kept links, [34..50] any_kept
   const size_t o_best = take(sizeof(unsigned long long) * kMaxD);
@@ -746,9 +777,11 @@ int adaptive_finish(const AdaptiveInput& in, ocnn_alloc_fn alloc, void* alloc_ct
   float* nrm_P = reinterpret_cast<float*>(ws + o_nrmP);
   float* pt_P = reinterpret_cast<float*>(ws + o_ptP);
   float* feat_P = reinterpret_cast<float*>(ws + o_featP);
+  float* lab_P = reinterpret_cast<float*>(ws + o_labP);
   {
     LeafPred lp{child[D]};
-    LeafPack lo{rank_D, (int64_t)o0.nnum[D], (int64_t)nP, cf, normal[D], pt[D], feature[D], nrm_P, pt_P, feat_P};
+    LeafPack lo{rank_D, (int64_t)o0.nnum[D], (int64_t)nP, cf, normal[D], pt[D], feature[D], label[D], nrm_P, pt_P,
+        feat_P, lab_P};
     hipError_t e = flag_scan(lp, lo, (int64_t)o0.nnum[D], reinterpret_cast<int*>(ws + o_scan), rank_D + o0.nnum[D], s);
     OCNN_REQUIRE(e == hipSuccess, OCNN_E_HIP, "leaf scan: %s", hipGetErrorString(e));
   }
@@ -763,7 +796,7 @@ int adaptive_finish(const AdaptiveInput& in, ocnn_alloc_fn alloc, void* alloc_ct
       a.imul = imul;
       a.key = key[d]; a.child = child[d]; a.dnum = dnum[d]; a.didx = didx[d];
       a.child_D = child[D]; a.nrm_D = normal[D]; a.pt_D = pt[D]; a.feat_D = feature[D]; a.lab_D = label[D];
-      a.rank_D = rank_D; a.nrm_P = nrm_P; a.pt_P = pt_P; a.feat_P = feat_P; a.nP = (int64_t)nP;
+      a.rank_D = rank_D; a.nrm_P = nrm_P; a.pt_P = pt_P; a.feat_P = feat_P; a.lab_P = lab_P; a.nP = (int64_t)nP;
       a.normal = normal[d]; a.pt = pt[d]; a.feature = feature[d]; a.label = label[d]; a.dis = dis[d];
       a.nerr = nerr[d]; a.derr = derr[d];
       L->first_wave[d] = waves;

@@ -265,6 +265,8 @@ def test_adaptive_build_vs_compiled_reference(orc, ref, case):
     pts, nrm = smooth_cloud(rng, n, trial % 2)
     feat = rng.uniform(0, 1, (n, 2)).astype(np.float32) if trial >= 2 else None
     lab = rng.integers(-1, 4, n).astype(np.float32) if trial >= 3 else None
+    if trial == 4:
+      lab = np.where(lab > 0, lab * 700 + 5, lab).astype(np.float32)   # label values beyond any small table
     pb = make_points_blob(pts, nrm, feat, lab)
     depth = int(rng.integers(4, 8))
     fd = int(rng.integers(1, 3))
