@@ -28,7 +28,7 @@ __all__ = [
     "octree_pad", "octree_depad", "octree_max_pool", "octree_max_unpool", "octree_mask_pool",
     "octree_encode_key", "octree_decode_key", "octree_xyz2key", "octree_key2xyz",
     "octree_search_key", "octree_new", "octree_grow", "octree_update", "points_new",
-    "octree_info", "octree_scan", "octree_dropout", "octree_drop",
+    "octree_info", "octree_scan", "octree_dropout", "octree_drop", "octree_samples",
 ]
 
 
@@ -266,6 +266,19 @@ def points2octree_batch(points_list, depth, full_depth=2, node_dis=False, node_f
   (the composition `collate_octrees` performs, pytorch/ocnn/transforms.py:127-148)."""
   return _build(list(points_list), True, depth, full_depth, node_dis, node_feature, split_label,
                 adaptive, adp_depth, th_normal, th_distance, extrapolate, save_pts, key2xyz)
+
+
+def octree_samples(names):
+  """pytorch/cpp/octree_samples.cpp:5-18 -- the small sample octrees the reference embeds
+  (`octree_1` .. `octree_6`, 64-bit keys) as CPU uint8 tensors; data file of this package."""
+  import os
+  z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "data", "octree_samples.npz"))
+  out = []
+  for name in names:
+    if name not in z.files:
+      raise OcnnError(-1, "The specified octree does not exist : %s" % name)
+    out.append(torch.from_numpy(z[name].copy()))
+  return out
 
 
 def octree_dropout(octree, depth_dropout, threshold, flags=None, generator=None, clear_dropped=False):

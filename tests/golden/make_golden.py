@@ -38,8 +38,10 @@ def sha(a):
 
 def main():
   ref = Checker("ref")
-  np.savez_compressed(os.path.join(HERE, "octree_samples.npz"),
-                      **{"octree_%d" % i: ref.octree_sample("octree_%d" % i) for i in range(1, 7)})
+  six = {"octree_%d" % i: ref.octree_sample("octree_%d" % i) for i in range(1, 7)}
+  np.savez_compressed(os.path.join(HERE, "octree_samples.npz"), **six)
+  # the package serves the same six blobs through nn.octree_samples
+  np.savez_compressed(os.path.join(ROOT, "o-cnn_amd", "data", "octree_samples.npz"), **six)
 
   # the same six samples as the reference stores them: 32-bit keys ("_OCTREE_1.0_"), read from the
   # sample translation unit compiled without KEY64 (oracle/Makefile)

@@ -93,3 +93,13 @@ def test_library_upgrade_and_files(orc, nn, samples, samples32, synthetic, tmp_p
   open(str(tmp_path / "d.points"), "wb").write(b"nope")
   with pytest.raises(nn.OcnnError):
     nn.read_points(str(tmp_path / "d.points"))
+
+
+def test_octree_samples_match_the_reference_blobs(nn, samples):
+  """nn.octree_samples (pytorch/cpp/octree_samples.cpp:5-18): the package's data file holds the
+  six blobs of the fixture; an unknown name raises."""
+  got = nn.octree_samples(["octree_%d" % i for i in range(1, 7)])
+  for i, t in enumerate(got):
+    assert t.dtype.is_floating_point is False and np.array_equal(t.numpy(), samples["octree_%d" % (i + 1)])
+  with pytest.raises(RuntimeError):
+    nn.octree_samples(["octree_7"])
