@@ -12,8 +12,9 @@ The directory name is not a Python identifier; load the package with
   stacks    -- conv -> BatchNorm -> ReLU (folded) operator sequences of the benchmark
                configurations (LeNet trunk, U-Net encoder / decoder)
   synthetic -- seeded synthetic point clouds of the benchmark configurations
+  transforms -- NormalizePoints / TransformPoints / Points2Octree / TransformCompose / collate_octrees
 """
-from . import lib, nn, autograd, layers, stacks, synthetic  # noqa: F401
+from . import lib, nn, autograd, layers, stacks, synthetic, transforms  # noqa: F401
 from .nn import *  # noqa: F401,F403
 from .layers import (OctreeConv, OctreeDeconv, OctreeConvFast, OctreeDeconvFast,  # noqa: F401
                      OctreeMaxPool, OctreeMaxUnpool, OctreeAvgPool, OctreePad, OctreeDepad,

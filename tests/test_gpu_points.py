@@ -85,6 +85,54 @@ def test_transform_compose_on_device(oc, orc, synthetic):
   assert np.array_equal(F.octree_batch(dev_octrees).cpu().numpy(), orc.octree_batch(singles))
 
 
+def test_transform_classes_follow_the_reference_pipeline(oc, orc, synthetic):
+  """transforms.TransformCompose / collate_octrees (pytorch/ocnn/transforms.py:6-148) with numpy's
+  generator seeded: the same draws through the oracle chain give the same octrees, points and
+  masks; building the batch inside collate gives the same merged octree."""
+  tr = oc.transforms
+  flags = dict(depth=6, full_depth=2, distort=True, angle=[10, 180, 5], scale=0.2, jitter=0.125,
+               angle_interval=[1, 5, 1], uniform_scale=False, bsphere="sphere")
+  clouds = []
+  for i in range(3):
+    p, n, _ = synthetic.shape_cloud(6000, 500 + i)
+    clouds.append(make_points_blob(p * np.float32(2.0) - np.float32(0.3), n))
+  compose = tr.TransformCompose(flags)
+  np.random.seed(11)
+  samples = [compose(T(pb).cuda(), i) for i, pb in enumerate(clouds)]
+  for s, lab in zip(samples, (3, 1, 4)):
+    s["label"] = lab
+  np.random.seed(11)
+  host = []
+  for pb, s in zip(clouds, samples):
+    drawn = tr.draw_distortion(flags["angle"], flags["scale"], flags["jitter"], flags["angle_interval"], False)
+    bs = orc.bounding_sphere(pb, "sphere")
+    h = orc.normalize_points(pb, bs[0], bs[1:])
+    h = orc.transform_points(h, np.float32(drawn[0]), np.float32(drawn[1]), np.float32(drawn[2]), 0.0, "")
+    h, hm = orc.clip_points(h, [-1] * 3, [1] * 3)
+    assert np.array_equal(s["inbox_mask"].cpu().numpy(), hm)
+    assert np.array_equal(s["points"].cpu().numpy(), h)
+    host.append(orc.points2octree(h, 6, 2))
+    assert np.array_equal(s["octree"].cpu().numpy(), host[-1])
+  merged = orc.octree_batch(host)
+  out = tr.collate_octrees(samples)
+  assert np.array_equal(out["octree"].cpu().numpy(), merged) and out["label"].tolist() == [3, 1, 4]
+  assert len(out["points"]) == 3
+  # samples without octrees: the batch is built in one pass at collate time
+  late = tr.TransformCompose(flags, octree=False)
+  np.random.seed(11)
+  bare = [late(T(pb).cuda(), i) for i, pb in enumerate(clouds)]
+  assert "octree" not in bare[0]
+  out2 = tr.collate_octrees(bare, points2octree=late.points2octree)
+  assert np.array_equal(out2["octree"].cpu().numpy(), merged)
+  # no distortion: identity transform, only normalisation and clipping
+  plain = tr.TransformCompose(dict(depth=5, distort=False, radius=2.0, center=(0.1, 0.0, -0.1)))
+  s = plain(T(clouds[0]).cuda())
+  h = orc.normalize_points(clouds[0], 2.0, (0.1, 0.0, -0.1))
+  h = orc.transform_points(h, np.zeros(3, np.float32), np.ones(3, np.float32), np.zeros(3, np.float32), 0.0, "")
+  h, hm = orc.clip_points(h, [-1] * 3, [1] * 3)
+  assert np.array_equal(s["octree"].cpu().numpy(), orc.points2octree(h, 5, 2))
+
+
 def test_scene_size(oc, orc, synthetic):
   """250 000 points: the sphere's sequential growth and the compaction at full size."""
   F = oc.nn
