@@ -19,4 +19,5 @@ from .nn import *  # noqa: F401,F403
 from .layers import (OctreeConv, OctreeDeconv, OctreeConvFast, OctreeDeconvFast,  # noqa: F401
                      OctreeMaxPool, OctreeMaxUnpool, OctreeAvgPool, OctreePad, OctreeDepad,
                      OctreeTrilinear, OctreeInterp, OctreeAlign, octree_nearest_pts,
-                     octree_trilinear_pts, octree_trilinear)
+                     octree_trilinear_pts, octree_trilinear, Octree2Col, Col2Octree, OctreeTile,
+                     FullOctree2Voxel, FullOctreeGlobalPool, octree_feature)

@@ -204,3 +204,78 @@ class OctreeAlign(nn.Module):
 
   def forward(self, data, src_octree, des_octree):
     return F.octree_align(data, src_octree, des_octree, self.depth)
+
+
+class Octree2ColBase(nn.Module):
+  """pytorch/ocnn/octree2col.py:59-69."""
+
+  def __init__(self, depth, kernel_size, stride, nempty=False):
+    super().__init__()
+    self.depth, self.stride, self.nempty = depth, stride, nempty
+    self.kernel_size = resize_with_last_val(kernel_size)
+
+  def extra_repr(self):
+    return 'depth={}, kernel_size={}, stride={}, nempty={}'.format(self.depth, self.kernel_size, self.stride,
+                                                                   self.nempty)
+
+
+class Octree2Col(Octree2ColBase):
+  """pytorch/ocnn/octree2col.py:72-75."""
+
+  def forward(self, data_in, octree):
+    return F.octree2col(data_in, octree, self.depth, self.kernel_size, self.stride, self.nempty)
+
+
+class Col2Octree(Octree2ColBase):
+  """pytorch/ocnn/octree2col.py:78-81."""
+
+  def forward(self, data_in, octree):
+    return F.col2octree(data_in, octree, self.depth, self.kernel_size, self.stride, self.nempty)
+
+
+class OctreeTile(nn.Module):
+  """pytorch/ocnn/modules.py:193-206: every non-empty node hands its feature to its eight
+  children (nearest-neighbour upsampling to the next level)."""
+
+  def __init__(self, depth):
+    super().__init__()
+    self.depth = depth
+
+  def forward(self, data_in, octree):
+    out = F.octree_depad(data_in, octree, self.depth)
+    out = out.repeat(1, 1, 1, 8)
+    return out.view(1, out.shape[1], -1, 1)
+
+
+class FullOctree2Voxel(nn.Module):
+  """pytorch/ocnn/octree2voxel.py:5-16: [1, C, B * 8^depth, 1] of a full level -> [B, C, 8^depth]
+  (Morton order within a sample)."""
+
+  def __init__(self, depth):
+    super().__init__()
+    self.depth = depth
+
+  def forward(self, data):
+    height = 2 ** (3 * self.depth)
+    return data.view(data.size(1), -1, height).permute(1, 0, 2)
+
+  def extra_repr(self):
+    return 'depth={}'.format(self.depth)
+
+
+class FullOctreeGlobalPool(OctreePoolBase):
+  """pytorch/ocnn/octree_pool.py:106-115: mean over a full level, per sample."""
+
+  def __init__(self, depth):
+    super().__init__(depth)
+    self.octree2voxel = FullOctree2Voxel(depth)
+
+  def forward(self, data):
+    return self.octree2voxel(data).mean(dim=2)
+
+
+def octree_feature(octree, depth, nempty=False):
+  """pytorch/ocnn/modules.py:333-337."""
+  from . import nn as ops
+  output = ops.octree_property(octree, 'feature', depth)
+  return ops.octree_depad(output, octree, depth) if nempty else output

@@ -146,3 +146,40 @@ def test_unet_trunk(oc, orc, tree, nempty):
     x = cbr(np.concatenate([feats[d], x], 0), ("dec", d), d, [3, 3, 3], 1)
   got = oc.stacks.unet_trunk(dev, 6, params, stages=stages, nempty=nempty)
   assert relerr(got.cpu().numpy().reshape(x.shape), x) < 1e-4
+
+
+def test_thin_modules(oc, orc, tree):
+  """Octree2Col / Col2Octree, OctreeTile, FullOctree2Voxel, FullOctreeGlobalPool, octree_feature
+  (pytorch/ocnn/octree2col.py:40-55, modules.py:193-206, 333-337, octree2voxel.py, octree_pool.py:106-115)
+  against their definitions written out with numpy."""
+  host, dev, b = tree
+  rng = np.random.default_rng(8)
+  d = 5
+  H, Hn = int(b.nnum[d]), int(b.nnum_nempty[d])
+  x = rng.standard_normal((1, 3, H, 1)).astype(np.float32)
+  xd = T(x).cuda().requires_grad_(True)
+  col = oc.Octree2Col(d, [3, 3, 3], 1)(xd, dev)
+  exp = orc.octree2col(x.reshape(3, H), [3, 3, 3], 1, b.prop("neigh", d), H)
+  assert np.array_equal(col.detach().cpu().numpy(), exp.reshape(col.shape))
+  back = oc.Col2Octree(d, [3, 3, 3], 1)(col, dev)
+  expb = orc.col2octree(exp, [3, 3, 3], 1, b.prop("neigh", d), H)
+  assert relerr(back.detach().cpu().numpy().reshape(3, H), expb.reshape(3, H)) < 1e-6
+  back.sum().backward()
+  assert xd.grad is not None and xd.grad.shape == xd.shape
+  # tile: the feature of the k-th non-empty node goes to the nodes 8k .. 8k + 7 of the next level
+  tile = oc.OctreeTile(d)(T(x).cuda(), dev).cpu().numpy()
+  child = b.prop("child", d)
+  assert tile.shape == (1, 3, int(b.nnum[d + 1]), 1)
+  assert np.array_equal(tile.reshape(3, Hn, 8), np.repeat(x.reshape(3, H)[:, child >= 0][:, :, None], 8, axis=2))
+  # full level 2 of a batch of two: [1, C, 2 * 64, 1] -> [2, C, 64], mean over the level
+  f = rng.standard_normal((1, 4, 2 * 64, 1)).astype(np.float32)
+  vox = oc.FullOctree2Voxel(2)(T(f).cuda()).cpu().numpy()
+  assert np.array_equal(vox, f.reshape(4, 2, 64).transpose(1, 0, 2))
+  pooled = oc.FullOctreeGlobalPool(2)(T(f).cuda()).cpu().numpy()
+  assert np.allclose(pooled, f.reshape(4, 2, 64).transpose(1, 0, 2).mean(axis=2), atol=1e-6)
+  # the stored signal of the finest level, all nodes and non-empty nodes
+  feat = b.prop("feature", 6)
+  got = oc.octree_feature(dev, 6).cpu().numpy()
+  assert np.array_equal(got.reshape(feat.shape), feat)
+  gne = oc.octree_feature(dev, 6, nempty=True).cpu().numpy()
+  assert np.array_equal(gne.reshape(feat.shape[0], -1), feat[:, b.prop("child", 6) >= 0])
