@@ -183,3 +183,35 @@ def test_thin_modules(oc, orc, tree):
   assert np.array_equal(got.reshape(feat.shape), feat)
   gne = oc.octree_feature(dev, 6, nempty=True).cpu().numpy()
   assert np.array_equal(gne.reshape(feat.shape[0], -1), feat[:, b.prop("child", 6) >= 0])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_operator_sequence_replays_from_a_graph(oc, tree, dtype):
+  """The operators launch kernels only (no memset nodes, no waits, no allocation besides torch's
+  own): a captured LeNet trunk, replayed several times with eager work and synchronisations in
+  between, gives the eager result every time, also after its input has been rewritten."""
+  host, dev, b = tree
+  g = torch.Generator().manual_seed(3)
+  chans = {6: (3, 32), 5: (32, 64), 4: (64, 128), 3: (128, 256)}
+  params = {d: ((torch.randn(co, ci * 27, generator=g) / (ci * 27) ** 0.5).cuda().to(dtype),
+                (torch.randn(co, generator=g) * 0.1).cuda()) for d, (ci, co) in chans.items()}
+  H6 = int(b.nnum[6])
+  x = torch.randn(1, 3, H6, 1, generator=g).cuda().to(dtype)
+  run = lambda: oc.stacks.lenet_trunk(dev, 6, params, data=x)
+  side = torch.cuda.Stream()
+  side.wait_stream(torch.cuda.current_stream())
+  with torch.cuda.stream(side):
+    for _ in range(2):
+      run()
+  torch.cuda.current_stream().wait_stream(side)
+  graph = torch.cuda.CUDAGraph()
+  with torch.cuda.graph(graph):
+    out = run()
+  for rep in range(4):
+    if rep == 2:
+      x.copy_(torch.randn(1, 3, H6, 1, generator=g).cuda().to(dtype))   # new input, same graph
+    graph.replay()
+    torch.cuda.synchronize()
+    eager = run()
+    torch.cuda.synchronize()
+    assert torch.equal(out, eager), rep
