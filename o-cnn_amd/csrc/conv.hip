@@ -1582,6 +1582,115 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_f32_kernel(ConvArgs a, cons
       }
   }
 }
+// Weight gradient of the 3x3x3 stride-1 operator over all nodes, through LDS.  All 27 taps of the
+// 8 columns of a block read their source rows from the block's own 64 neighbour slots, so a
+// workgroup stages those 64 rows (32 channels each, 8 KiB) once per block, two blocks ahead of
+// their use (index -> row -> LDS, each one block apart: memory latency never meets the matrix
+// pipe), and eight wavefronts multiply from LDS: wavefront (g, h) owns the taps 7g .. 7g + 6 and
+// the 32 rows of A of half h, i.e. 7 accumulator tiles; the two wavefronts of a tap group share
+// a SIMD.  A workgroup is one slice of column blocks for one 32-channel chunk and 64 rows of A;
+// the partial sums have the layout of the kernel above and go through the same reduction.
+constexpr int kWgLdsTaps = 7;
+__global__ __launch_bounds__(512) void conv_wgrad_f32_lds_kernel(ConvArgs a, const float* __restrict__ A,
+    const float* __restrict__ xt, float* __restrict__ partial, int cpad, int mpad, int n_slices, int cpasses) {
+  __shared__ __attribute__((aligned(16))) float s_rows[3][64 * 32];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tapgroup = wave & 3, mhalf = wave >> 2;
+  const int slice = blockIdx.x;
+  const int cpass = blockIdx.y % cpasses, mpass = blockIdx.y / cpasses;
+  const int r = lane & 31, kh = lane >> 5;
+  const int tap0 = tapgroup * kWgLdsTaps;
+  floatx16 acc[kWgLdsTaps];
+#pragma unroll
+  for (int t = 0; t < kWgLdsTaps; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[t][i] = 0.0f;
+  const int nblocks = a.N >> 3;
+  const int per_slice = (nblocks + n_slices - 1) / n_slices;
+  const int b_begin = slice * per_slice, b_end = min(nblocks, b_begin + per_slice);
+  // staging: thread (slot, part) moves 16 bytes of the 128-byte row of a slot
+  const int st_slot = tid >> 3, st_part = tid & 7;
+  const float* xcol = xt + cpass * 32 + st_part * 4;
+  // neighbour of this thread's slot in block b, as stored: it is looked at only when the row is
+  // requested, one block later, so that the wavefront never waits for the index it just asked for
+  auto index_of = [&](int b) { return a.neigh[((int64_t)b << 6) + st_slot]; };
+  auto load_row = [&](int p) {   // the zero row if there is no neighbour
+    p = (p >= 0 && p < a.Hin) ? p : a.Hin;
+    return *reinterpret_cast<const float4*>(xcol + (int64_t)p * cpad);
+  };
+  auto store_row = [&](int buf, float4 v) {
+    *reinterpret_cast<float4*>(&s_rows[buf][st_slot * 32 + st_part * 4]) = v;
+  };
+  const int m = (mpass * 2 + mhalf) * 32 + r;
+  auto load_a = [&](int b) {
+    return *reinterpret_cast<const float4*>(A + (((int64_t)b * 2 + kh) * mpad + m) * 4);
+  };
+  // LDS word of this lane's B value for k-step j of tap t: row slot(sibling j + 4 kh, tap), channel r
+  int boff[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) boff[j] = sibling_slot(j + 4 * kh) * 32 + r;
+  int tslot[kWgLdsTaps];
+#pragma unroll
+  for (int t = 0; t < kWgLdsTaps; ++t) tslot[t] = a.slot[min(tap0 + t, a.K - 1)] * 32;
+  if (b_begin < b_end) {
+    const int last = b_end - 1;
+    // Three LDS buffers: while block b is multiplied from registers, the B values of block b + 1
+    // are read from LDS and the rows of block b + 2 are written to it; the rows of block b + 3
+    // and the index of block b + 4 are in flight from memory.
+    auto read_b = [&](int buf, float (&bv)[4][kWgLdsTaps]) {
+      const float* src = s_rows[buf];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int t = 0; t < kWgLdsTaps; ++t) bv[j][t] = src[boff[j] + tslot[t]];
+    };
+    store_row(0, load_row(index_of(b_begin)));
+    store_row(1, load_row(index_of(min(b_begin + 1, last))));
+    float4 rows_next = load_row(index_of(min(b_begin + 2, last)));
+    int idx_next = index_of(min(b_begin + 3, last));
+    float4 av = load_a(b_begin);
+    __syncthreads();
+    float bv[4][kWgLdsTaps];
+    read_b(0, bv);
+    int nxt = 1;                       // buffer of block b + 1
+    for (int b = b_begin; b < b_end; ++b) {
+      const float4 av_next = load_a(min(b + 1, last));
+      const float aj[4] = {av.x, av.y, av.z, av.w};
+      float bv_next[4][kWgLdsTaps];
+      read_b(nxt, bv_next);
+      // consecutive MFMAs go to different accumulators (k-step outside, tap inside); a tap past
+      // the 27th reads the slot of the last one and its tile is never written
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int t = 0; t < kWgLdsTaps; ++t)
+          acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(aj[j], bv[j][t], acc[t], 0, 0, 0);
+      const int wr = nxt == 2 ? 0 : nxt + 1;   // buffer of block b + 2
+      store_row(wr, rows_next);
+      rows_next = load_row(idx_next);
+      idx_next = index_of(min(b + 4, last));
+      av = av_next;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int t = 0; t < kWgLdsTaps; ++t) bv[j][t] = bv_next[j][t];
+      __syncthreads();
+      nxt = wr;
+    }
+  }
+  // partial[slice][tap][m][c]
+#pragma unroll
+  for (int t = 0; t < kWgLdsTaps; ++t) {
+    const int tap = tap0 + t;
+    if (tap >= a.K) continue;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int mm = (mpass * 2 + mhalf) * 32 + 8 * (i / 4) + 4 * kh + (i % 4);
+      partial[(((int64_t)slice * a.K + tap) * mpad + mm) * cpad + cpass * 32 + r] = acc[t][i];
+    }
+  }
+}
+
 __global__ void conv_wgrad_reduce_kernel(float* __restrict__ G, const float* __restrict__ partial, int n_slices,
     int M, int Cin, int K, int mpad, int cpad) {
   const int64_t per = (int64_t)K * mpad * cpad;
@@ -1659,6 +1768,20 @@ int run_wgrad(float* grad_w, const float* A, int M, const float* X, int channel_
   dim3 grid(w.n_slices / 4, w.tapgroups, w.mpasses * w.cpasses);
   // whole sibling groups (N % 8 == 0), every column a node
   const bool fast = a.mode == kModeS1 && !a.nempty && (a.N & 7) == 0;
+  if (fast && a.K == 27 && (M & 63) == 0 && (channel_in & 31) == 0 && w.mpad == M && w.cpad == channel_in) {
+    // one workgroup per compute unit, each a slice of blocks for one (32-channel, 64-row) tile
+    const int tiles = (w.cpad / 32) * (w.mpad / 64);
+    int n_slices = 256 / tiles;
+    n_slices = n_slices < 1 ? 1 : (n_slices > w.n_slices ? w.n_slices : n_slices);
+    conv_wgrad_f32_lds_kernel<<<dim3(n_slices, tiles), 512, 0, s>>>(a, aq, xt, partial, w.cpad, w.mpad, n_slices,
+        w.cpad / 32);
+    OCNN_LAUNCH_OK("conv_wgrad_lds");
+    const int64_t per = (int64_t)a.K * w.mpad * w.cpad;
+    conv_wgrad_reduce_kernel<<<blocks_for(per), kBlock, 0, s>>>(grad_w, partial, n_slices, M, channel_in, a.K, w.mpad,
+        w.cpad);
+    OCNN_LAUNCH_OK("conv_wgrad_reduce");
+    return OCNN_OK;
+  }
 #define OCNN_WGRAD(MT_, NT_)                                                                                     \
   do {                                                                                                           \
     if (fast) conv_wgrad_f32_kernel<MT_, NT_, true><<<grid, 256, 0, s>>>(a, aq, xt, partial, w.cpad, w.mpad,     \

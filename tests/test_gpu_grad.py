@@ -69,6 +69,31 @@ def test_deconv_grad_vs_oracle(oc, orc, tree, ks, stride, nempty, ci, co):
   assert relerr(gd.cpu().numpy().reshape(egd.shape), egd) < TOL
 
 
+@pytest.mark.parametrize("ci,co", [(32, 128), (128, 64)])
+def test_conv_grad_wide_channels(oc, orc, tree, ci, co):
+  """3x3x3 stride 1 over all nodes with channel counts in whole 32 / 64 blocks: the weight
+  gradient runs its LDS-staged form with several channel and row tiles per slice."""
+  host, dev, b = tree
+  d = 5
+  rng = np.random.default_rng(ci + co)
+  hin = int(b.nnum[d])
+  x = rng.standard_normal((ci, hin)).astype(np.float32)
+  w = (rng.standard_normal((co, ci * 27)) * 0.1).astype(np.float32)
+  g = rng.standard_normal((co, hin)).astype(np.float32)
+  egd, egw = orc.octree_conv_grad(x, w, g, host, d, co, [3, 3, 3], 1, False)
+  gd, gw = oc.nn.octree_conv_grad(T(x).cuda().view(1, ci, hin, 1), T(w).cuda(), dev,
+                                  T(g).cuda().view(1, co, hin, 1), d, co, [3, 3, 3], 1, False)
+  assert relerr(gw.cpu().numpy(), egw) < TOL
+  assert relerr(gd.cpu().numpy().reshape(egd.shape), egd) < TOL
+  # deconvolution: the roles of the two tensors swap in the weight gradient
+  wd = (rng.standard_normal((ci, co * 27)) * 0.1).astype(np.float32)
+  egd, egw = orc.octree_deconv_grad(x, wd, g, host, d, co, [3, 3, 3], 1, False)
+  gd, gw = oc.nn.octree_deconv_grad(T(x).cuda().view(1, ci, hin, 1), T(wd).cuda(), dev,
+                                    T(g).cuda().view(1, co, hin, 1), d, co, [3, 3, 3], 1, False)
+  assert relerr(gw.cpu().numpy(), egw) < TOL
+  assert relerr(gd.cpu().numpy().reshape(egd.shape), egd) < TOL
+
+
 def test_grad_errors(oc, tree):
   host, dev, b = tree
   x = torch.zeros(1, 4, int(b.nnum[5]), 1, device="cuda")
