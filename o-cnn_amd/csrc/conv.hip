@@ -1591,9 +1591,10 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_f32_kernel(ConvArgs a, cons
 // a SIMD.  A workgroup is one slice of column blocks for one 32-channel chunk and 64 rows of A;
 // the partial sums have the layout of the kernel above and go through the same reduction.
 constexpr int kWgLdsTaps = 7;
+constexpr int kWgLdsRow = 36;   // words per staged row: 32 channels + 4, so that the 16-byte stores of 8 lanes spread over all banks
 __global__ __launch_bounds__(512) void conv_wgrad_f32_lds_kernel(ConvArgs a, const float* __restrict__ A,
-    const float* __restrict__ xt, float* __restrict__ partial, int cpad, int mpad, int n_slices, int cpasses) {
-  __shared__ __attribute__((aligned(16))) float s_rows[3][64 * 32];
+    const float* __restrict__ X, float* __restrict__ partial, int cpad, int mpad, int n_slices, int cpasses) {
+  __shared__ __attribute__((aligned(16))) float s_rows[3][64 * kWgLdsRow];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int tapgroup = wave & 3, mhalf = wave >> 2;
   const int slice = blockIdx.x;
@@ -1608,9 +1609,10 @@ __global__ __launch_bounds__(512) void conv_wgrad_f32_lds_kernel(ConvArgs a, con
   const int nblocks = a.N >> 3;
   const int per_slice = (nblocks + n_slices - 1) / n_slices;
   const int b_begin = slice * per_slice, b_end = min(nblocks, b_begin + per_slice);
-  // staging: thread (slot, part) moves 16 bytes of the 128-byte row of a slot
+  // staging: thread (slot, part) moves 16 bytes of the 128-byte row of a slot's node in the
+  // row-major copy of the input
   const int st_slot = tid >> 3, st_part = tid & 7;
-  const float* xcol = xt + cpass * 32 + st_part * 4;
+  const float* xcol = X + cpass * 32 + st_part * 4;
   // neighbour of this thread's slot in block b, as stored: it is looked at only when the row is
   // requested, one block later, so that the wavefront never waits for the index it just asked for
   auto index_of = [&](int b) { return a.neigh[((int64_t)b << 6) + st_slot]; };
@@ -1619,19 +1621,19 @@ __global__ __launch_bounds__(512) void conv_wgrad_f32_lds_kernel(ConvArgs a, con
     return *reinterpret_cast<const float4*>(xcol + (int64_t)p * cpad);
   };
   auto store_row = [&](int buf, float4 v) {
-    *reinterpret_cast<float4*>(&s_rows[buf][st_slot * 32 + st_part * 4]) = v;
+    *reinterpret_cast<float4*>(&s_rows[buf][st_slot * kWgLdsRow + st_part * 4]) = v;
   };
+  // A in place: lane (row, kh) takes the four columns 4 kh .. 4 kh + 3 of block b of its row
   const int m = (mpass * 2 + mhalf) * 32 + r;
-  auto load_a = [&](int b) {
-    return *reinterpret_cast<const float4*>(A + (((int64_t)b * 2 + kh) * mpad + m) * 4);
-  };
+  const float* arow = A + (int64_t)m * a.N + 4 * kh;
+  auto load_a = [&](int b) { return *reinterpret_cast<const float4*>(arow + ((int64_t)b << 3)); };
   // LDS word of this lane's B value for k-step j of tap t: row slot(sibling j + 4 kh, tap), channel r
   int boff[4];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) boff[j] = sibling_slot(j + 4 * kh) * 32 + r;
+  for (int j = 0; j < 4; ++j) boff[j] = sibling_slot(j + 4 * kh) * kWgLdsRow + r;
   int tslot[kWgLdsTaps];
 #pragma unroll
-  for (int t = 0; t < kWgLdsTaps; ++t) tslot[t] = a.slot[min(tap0 + t, a.K - 1)] * 32;
+  for (int t = 0; t < kWgLdsTaps; ++t) tslot[t] = a.slot[min(tap0 + t, a.K - 1)] * kWgLdsRow;
   if (b_begin < b_end) {
     const int last = b_end - 1;
     // Three LDS buffers: while block b is multiplied from registers, the B values of block b + 1
@@ -1757,6 +1759,27 @@ int run_wgrad(float* grad_w, const float* A, int M, const float* X, int channel_
     OCNN_LAUNCH_OK("ichild");
     a.ichild = ichild;
   }
+  // whole sibling groups (N % 8 == 0), every column a node
+  const bool fast = a.mode == kModeS1 && !a.nempty && (a.N & 7) == 0;
+  if (fast && a.K == 27 && (M & 63) == 0 && (channel_in & 31) == 0 && w.mpad == M && w.cpad == channel_in &&
+      (reinterpret_cast<uintptr_t>(A) & 15) == 0) {
+    // the output gradient is read in place; one workgroup per compute unit, each a slice of blocks
+    // for one (32-channel, 64-row) tile
+    const int tiles = (w.cpad / 32) * (w.mpad / 64);
+    int n_slices = 256 / tiles;
+    n_slices = n_slices < 1 ? 1 : (n_slices > w.n_slices ? w.n_slices : n_slices);
+    dim3 tg((a.Hin + 64) / 64, (w.cpad + 63) / 64);
+    transpose_rows_f32_kernel<<<tg, 256, 0, s>>>(xt, X, channel_in, a.Hin, w.cpad);
+    OCNN_LAUNCH_OK("transpose_rows");
+    conv_wgrad_f32_lds_kernel<<<dim3(n_slices, tiles), 512, 0, s>>>(a, A, xt, partial, w.cpad, w.mpad, n_slices,
+        w.cpad / 32);
+    OCNN_LAUNCH_OK("conv_wgrad_lds");
+    const int64_t per = (int64_t)a.K * w.mpad * w.cpad;
+    conv_wgrad_reduce_kernel<<<blocks_for(per), kBlock, 0, s>>>(grad_w, partial, n_slices, M, channel_in, a.K, w.mpad,
+        w.cpad);
+    OCNN_LAUNCH_OK("conv_wgrad_reduce");
+    return OCNN_OK;
+  }
   dim3 tg((a.Hin + 64) / 64, (w.cpad + 63) / 64);
   transpose_rows_f32_kernel<<<tg, 256, 0, s>>>(xt, X, channel_in, a.Hin, w.cpad);
   OCNN_LAUNCH_OK("transpose_rows");
@@ -1766,22 +1789,6 @@ int run_wgrad(float* grad_w, const float* A, int M, const float* X, int channel_
   interleave_quads_kernel<<<qg, 256, 0, s>>>(aq, A, M, a.N, w.mpad, n_quads);
   OCNN_LAUNCH_OK("interleave_quads");
   dim3 grid(w.n_slices / 4, w.tapgroups, w.mpasses * w.cpasses);
-  // whole sibling groups (N % 8 == 0), every column a node
-  const bool fast = a.mode == kModeS1 && !a.nempty && (a.N & 7) == 0;
-  if (fast && a.K == 27 && (M & 63) == 0 && (channel_in & 31) == 0 && w.mpad == M && w.cpad == channel_in) {
-    // one workgroup per compute unit, each a slice of blocks for one (32-channel, 64-row) tile
-    const int tiles = (w.cpad / 32) * (w.mpad / 64);
-    int n_slices = 256 / tiles;
-    n_slices = n_slices < 1 ? 1 : (n_slices > w.n_slices ? w.n_slices : n_slices);
-    conv_wgrad_f32_lds_kernel<<<dim3(n_slices, tiles), 512, 0, s>>>(a, aq, xt, partial, w.cpad, w.mpad, n_slices,
-        w.cpad / 32);
-    OCNN_LAUNCH_OK("conv_wgrad_lds");
-    const int64_t per = (int64_t)a.K * w.mpad * w.cpad;
-    conv_wgrad_reduce_kernel<<<blocks_for(per), kBlock, 0, s>>>(grad_w, partial, n_slices, M, channel_in, a.K, w.mpad,
-        w.cpad);
-    OCNN_LAUNCH_OK("conv_wgrad_reduce");
-    return OCNN_OK;
-  }
 #define OCNN_WGRAD(MT_, NT_)                                                                                     \
   do {                                                                                                           \
     if (fast) conv_wgrad_f32_kernel<MT_, NT_, true><<<grid, 256, 0, s>>>(a, aq, xt, partial, w.cpad, w.mpad,     \
