@@ -1592,9 +1592,11 @@ __global__ __launch_bounds__(256, 2) void conv_wgrad_f32_kernel(ConvArgs a, cons
 // the partial sums have the layout of the kernel above and go through the same reduction.
 constexpr int kWgLdsTaps = 7;
 constexpr int kWgLdsRow = 36;   // words per staged row: 32 channels + 4, so that the 16-byte stores of 8 lanes spread over all banks
-__global__ __launch_bounds__(512) void conv_wgrad_f32_lds_kernel(ConvArgs a, const float* __restrict__ A,
+template <int HALVES>   // 2: 64 rows of A per workgroup (eight wavefronts); 1: 32 rows (four, two workgroups per unit)
+__global__ __launch_bounds__(256 * HALVES) void conv_wgrad_f32_lds_kernel(ConvArgs a, const float* __restrict__ A,
     const float* __restrict__ X, float* __restrict__ partial, int cpad, int mpad, int n_slices, int cpasses) {
   __shared__ __attribute__((aligned(16))) float s_rows[3][64 * kWgLdsRow];
+  constexpr int kVec = 2 / HALVES;   // 16-byte units a thread stages per block
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int tapgroup = wave & 3, mhalf = wave >> 2;
   const int slice = blockIdx.x;
@@ -1609,22 +1611,28 @@ __global__ __launch_bounds__(512) void conv_wgrad_f32_lds_kernel(ConvArgs a, con
   const int nblocks = a.N >> 3;
   const int per_slice = (nblocks + n_slices - 1) / n_slices;
   const int b_begin = slice * per_slice, b_end = min(nblocks, b_begin + per_slice);
-  // staging: thread (slot, part) moves 16 bytes of the 128-byte row of a slot's node in the
-  // row-major copy of the input
-  const int st_slot = tid >> 3, st_part = tid & 7;
-  const float* xcol = X + cpass * 32 + st_part * 4;
+  // staging: thread (slot, part) moves 16 * kVec bytes of the 128-byte row of a slot's node in
+  // the row-major copy of the input
+  struct Units { float4 v[kVec]; };
+  const int st_slot = tid / (8 / kVec), st_part = tid % (8 / kVec);
+  const float* xcol = X + cpass * 32 + st_part * 4 * kVec;
   // neighbour of this thread's slot in block b, as stored: it is looked at only when the row is
   // requested, one block later, so that the wavefront never waits for the index it just asked for
   auto index_of = [&](int b) { return a.neigh[((int64_t)b << 6) + st_slot]; };
   auto load_row = [&](int p) {   // the zero row if there is no neighbour
     p = (p >= 0 && p < a.Hin) ? p : a.Hin;
-    return *reinterpret_cast<const float4*>(xcol + (int64_t)p * cpad);
+    Units u;
+#pragma unroll
+    for (int v = 0; v < kVec; ++v) u.v[v] = *reinterpret_cast<const float4*>(xcol + (int64_t)p * cpad + 4 * v);
+    return u;
   };
-  auto store_row = [&](int buf, float4 v) {
-    *reinterpret_cast<float4*>(&s_rows[buf][st_slot * kWgLdsRow + st_part * 4]) = v;
+  auto store_row = [&](int buf, const Units& u) {
+#pragma unroll
+    for (int v = 0; v < kVec; ++v)
+      *reinterpret_cast<float4*>(&s_rows[buf][st_slot * kWgLdsRow + st_part * 4 * kVec + 4 * v]) = u.v[v];
   };
   // A in place: lane (row, kh) takes the four columns 4 kh .. 4 kh + 3 of block b of its row
-  const int m = (mpass * 2 + mhalf) * 32 + r;
+  const int m = (mpass * HALVES + mhalf) * 32 + r;
   const float* arow = A + (int64_t)m * a.N + 4 * kh;
   auto load_a = [&](int b) { return *reinterpret_cast<const float4*>(arow + ((int64_t)b << 3)); };
   // LDS word of this lane's B value for k-step j of tap t: row slot(sibling j + 4 kh, tap), channel r
@@ -1648,7 +1656,7 @@ __global__ __launch_bounds__(512) void conv_wgrad_f32_lds_kernel(ConvArgs a, con
     };
     store_row(0, load_row(index_of(b_begin)));
     store_row(1, load_row(index_of(min(b_begin + 1, last))));
-    float4 rows_next = load_row(index_of(min(b_begin + 2, last)));
+    Units rows_next = load_row(index_of(min(b_begin + 2, last)));
     int idx_next = index_of(min(b_begin + 3, last));
     float4 av = load_a(b_begin);
     __syncthreads();
@@ -1687,7 +1695,7 @@ __global__ __launch_bounds__(512) void conv_wgrad_f32_lds_kernel(ConvArgs a, con
     if (tap >= a.K) continue;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      const int mm = (mpass * 2 + mhalf) * 32 + 8 * (i / 4) + 4 * kh + (i % 4);
+      const int mm = (mpass * HALVES + mhalf) * 32 + 8 * (i / 4) + 4 * kh + (i % 4);
       partial[(((int64_t)slice * a.K + tap) * mpad + mm) * cpad + cpass * 32 + r] = acc[t][i];
     }
   }
@@ -1729,6 +1737,13 @@ void make_wgrad_plan(const ConvPlan& p, int M, int channel_in, int nempty, Wgrad
   if (groups > max_groups) groups = max_groups;
   if (groups < 1) groups = 1;
   w->n_slices = groups * 4;
+  // the LDS-staged kernel wants one slice per resident workgroup and tile (run_wgrad)
+  if (p.taps.count == 27 && ((M & 63) == 0 || M == 32) && (channel_in & 31) == 0) {
+    const int halves = M == 32 ? 1 : 2;
+    const int tiles = (channel_in / 32) * (M / (32 * halves));
+    const int lds_slices = ((halves == 1 ? 512 : 256) / tiles) & ~3;
+    if (lds_slices > w->n_slices) w->n_slices = lds_slices;
+  }
   w->xt_bytes = align256(((size_t)p.btm_h + 1) * w->cpad * sizeof(float));
   w->partial_bytes = align256((size_t)w->n_slices * p.taps.count * w->mpad * w->cpad * sizeof(float));
   w->ichild_bytes = nempty ? align256(sizeof(int) * (size_t)(p.ichild_h + 1)) : 0;
@@ -1761,18 +1776,23 @@ int run_wgrad(float* grad_w, const float* A, int M, const float* X, int channel_
   }
   // whole sibling groups (N % 8 == 0), every column a node
   const bool fast = a.mode == kModeS1 && !a.nempty && (a.N & 7) == 0;
-  if (fast && a.K == 27 && (M & 63) == 0 && (channel_in & 31) == 0 && w.mpad == M && w.cpad == channel_in &&
-      (reinterpret_cast<uintptr_t>(A) & 15) == 0) {
-    // the output gradient is read in place; one workgroup per compute unit, each a slice of blocks
-    // for one (32-channel, 64-row) tile
-    const int tiles = (w.cpad / 32) * (w.mpad / 64);
-    int n_slices = 256 / tiles;
+  if (fast && a.K == 27 && ((M & 63) == 0 || M == 32) && (channel_in & 31) == 0 && w.mpad == M &&
+      w.cpad == channel_in && (reinterpret_cast<uintptr_t>(A) & 15) == 0) {
+    // the output gradient is read in place; every workgroup is a slice of blocks for one tile of
+    // 32 channels and 64 rows (one workgroup per compute unit) or 32 rows (two)
+    const int halves = M == 32 ? 1 : 2;
+    const int tiles = (w.cpad / 32) * (w.mpad / (32 * halves));
+    int n_slices = (halves == 1 ? 512 : 256) / tiles;
     n_slices = n_slices < 1 ? 1 : (n_slices > w.n_slices ? w.n_slices : n_slices);
     dim3 tg((a.Hin + 64) / 64, (w.cpad + 63) / 64);
     transpose_rows_f32_kernel<<<tg, 256, 0, s>>>(xt, X, channel_in, a.Hin, w.cpad);
     OCNN_LAUNCH_OK("transpose_rows");
-    conv_wgrad_f32_lds_kernel<<<dim3(n_slices, tiles), 512, 0, s>>>(a, A, xt, partial, w.cpad, w.mpad, n_slices,
-        w.cpad / 32);
+    if (halves == 1)
+      conv_wgrad_f32_lds_kernel<1><<<dim3(n_slices, tiles), 256, 0, s>>>(a, A, xt, partial, w.cpad, w.mpad, n_slices,
+          w.cpad / 32);
+    else
+      conv_wgrad_f32_lds_kernel<2><<<dim3(n_slices, tiles), 512, 0, s>>>(a, A, xt, partial, w.cpad, w.mpad, n_slices,
+          w.cpad / 32);
     OCNN_LAUNCH_OK("conv_wgrad_lds");
     const int64_t per = (int64_t)a.K * w.mpad * w.cpad;
     conv_wgrad_reduce_kernel<<<blocks_for(per), kBlock, 0, s>>>(grad_w, partial, n_slices, M, channel_in, a.K, w.mpad,

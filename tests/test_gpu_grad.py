@@ -69,7 +69,7 @@ def test_deconv_grad_vs_oracle(oc, orc, tree, ks, stride, nempty, ci, co):
   assert relerr(gd.cpu().numpy().reshape(egd.shape), egd) < TOL
 
 
-@pytest.mark.parametrize("ci,co", [(32, 128), (128, 64)])
+@pytest.mark.parametrize("ci,co", [(32, 128), (128, 64), (32, 32), (64, 32)])
 def test_conv_grad_wide_channels(oc, orc, tree, ci, co):
   """3x3x3 stride 1 over all nodes with channel counts in whole 32 / 64 blocks: the weight
   gradient runs its LDS-staged form with several channel and row tiles per slice."""
