@@ -1715,6 +1715,7 @@ __global__ void conv_wgrad_reduce_kernel(float* __restrict__ G, const float* __r
 
 struct WgradPlan {
   int MT, NT, mpasses, cpasses, mpad, cpad, n_slices, tapgroups;
+  int lds_slices;   // slices of the LDS-staged kernel, 0 if the shape does not qualify for it
   size_t xt_bytes, partial_bytes, ichild_bytes, aq_bytes, total_bytes;
 };
 // `p` is the plan of the underlying convolution geometry (deconv = 0): M rows on the column side,
@@ -1738,14 +1739,16 @@ void make_wgrad_plan(const ConvPlan& p, int M, int channel_in, int nempty, Wgrad
   if (groups < 1) groups = 1;
   w->n_slices = groups * 4;
   // the LDS-staged kernel wants one slice per resident workgroup and tile (run_wgrad)
+  w->lds_slices = 0;
   if (p.taps.count == 27 && ((M & 63) == 0 || M == 32) && (channel_in & 31) == 0) {
     const int halves = M == 32 ? 1 : 2;
     const int tiles = (channel_in / 32) * (M / (32 * halves));
-    const int lds_slices = ((halves == 1 ? 512 : 256) / tiles) & ~3;
-    if (lds_slices > w->n_slices) w->n_slices = lds_slices;
+    w->lds_slices = (halves == 1 ? 512 : 256) / tiles;
+    if (w->lds_slices < 1) w->lds_slices = 1;
   }
   w->xt_bytes = align256(((size_t)p.btm_h + 1) * w->cpad * sizeof(float));
-  w->partial_bytes = align256((size_t)w->n_slices * p.taps.count * w->mpad * w->cpad * sizeof(float));
+  const int most_slices = w->n_slices > w->lds_slices ? w->n_slices : w->lds_slices;
+  w->partial_bytes = align256((size_t)most_slices * p.taps.count * w->mpad * w->cpad * sizeof(float));
   w->ichild_bytes = nempty ? align256(sizeof(int) * (size_t)(p.ichild_h + 1)) : 0;
   w->aq_bytes = align256((size_t)nblocks * 2 * w->mpad * 4 * sizeof(float));
   w->total_bytes = w->xt_bytes + w->partial_bytes + w->ichild_bytes + w->aq_bytes;
@@ -1776,14 +1779,12 @@ int run_wgrad(float* grad_w, const float* A, int M, const float* X, int channel_
   }
   // whole sibling groups (N % 8 == 0), every column a node
   const bool fast = a.mode == kModeS1 && !a.nempty && (a.N & 7) == 0;
-  if (fast && a.K == 27 && ((M & 63) == 0 || M == 32) && (channel_in & 31) == 0 && w.mpad == M &&
-      w.cpad == channel_in && (reinterpret_cast<uintptr_t>(A) & 15) == 0) {
+  if (fast && w.lds_slices > 0 && w.mpad == M && w.cpad == channel_in && (reinterpret_cast<uintptr_t>(A) & 15) == 0) {
     // the output gradient is read in place; every workgroup is a slice of blocks for one tile of
     // 32 channels and 64 rows (one workgroup per compute unit) or 32 rows (two)
     const int halves = M == 32 ? 1 : 2;
     const int tiles = (w.cpad / 32) * (w.mpad / (32 * halves));
-    int n_slices = (halves == 1 ? 512 : 256) / tiles;
-    n_slices = n_slices < 1 ? 1 : (n_slices > w.n_slices ? w.n_slices : n_slices);
+    const int n_slices = w.lds_slices;
     dim3 tg((a.Hin + 64) / 64, (w.cpad + 63) / 64);
     transpose_rows_f32_kernel<<<tg, 256, 0, s>>>(xt, X, channel_in, a.Hin, w.cpad);
     OCNN_LAUNCH_OK("transpose_rows");
