@@ -316,7 +316,7 @@ def main():
     # gradients of the headline conv: weight gradient (contraction over the octants) + data
     # gradient (the transposed operator); 2 x the forward flops in total
     gy = torch.randn(1, C, H9, 1, generator=g).to(dev)
-    t = timed(lambda: F.octree_conv_grad(x32, w32, octree, gy, 9, C, [3, 3, 3], 1, False), max(2, reps // 2), 1)
+    t = timed(lambda: F.octree_conv_grad(x32, w32, octree, gy, 9, C, [3, 3, 3], 1, False), max(4, reps // 2), 3)
     fl = 2 * 2.0 * H9 * 27 * C * C
     extra["conv333_s1_d9_f32_grad"] = {"ms": t, "octants_per_s": H9 / (t * 1e-3), "tflops": fl / (t * 1e-3) / 1e12,
                                        "frac_mfma_peak": fl / (t * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS["f32"]}
