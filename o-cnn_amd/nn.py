@@ -664,7 +664,7 @@ def col2octree(grad_in, octree, depth, kernel_size, stride, nempty):
 
 # ---- convolution -------------------------------------------------------------------------------
 def _conv(fn, is_deconv, data_in, weights, octree, depth, num_output, kernel_size, stride, nempty,
-          bias=None, relu=False):
+          bias=None, relu=False, out=None):
   octree = _to_dev(octree)
   info = octree_info(octree)
   ksc, _ = _ks(kernel_size)
@@ -679,7 +679,13 @@ def _conv(fn, is_deconv, data_in, weights, octree, depth, num_output, kernel_siz
             int(is_deconv), dt, C.byref(top_h), C.byref(need_h), C.byref(ws_bytes))
   ws = _workspace(ws_bytes.value + 256, "conv")
   base = (ws.data_ptr() + 255) & ~255
-  out = torch.empty(1, num_output, top_h.value, 1, dtype=data_in.dtype, device=data_in.device)
+  shape = (1, num_output, top_h.value, 1)
+  if out is None:
+    out = torch.empty(shape, dtype=data_in.dtype, device=data_in.device)
+  elif (tuple(out.shape) != shape or out.dtype != data_in.dtype or out.device != data_in.device
+        or not out.is_contiguous()):
+    # e.g. a channel slice of a larger [1, C, H, 1] tensor: the result lands there directly
+    raise OcnnError(-3, "out must be a contiguous %s %s tensor on %s" % (shape, data_in.dtype, data_in.device))
   if fn == "ocnn_octree_conv_fused":
     if bias is not None:
       bias = bias.to(torch.float32).contiguous()
@@ -708,12 +714,13 @@ def octree_deconv(data_in, weights, octree, depth, num_output, kernel_size, stri
 
 
 def octree_conv_fused(data_in, weights, bias, relu, octree, depth, num_output, kernel_size, stride,
-                      nempty, deconv=False):
+                      nempty, deconv=False, out=None):
   """conv (or deconv) + per-channel bias + optional ReLU in one kernel: the inference form of
   the reference's conv -> BatchNorm -> ReLU modules (pytorch/ocnn/modules.py:23-36) once the
-  BatchNorm statistics are folded into `weights` and `bias`."""
+  BatchNorm statistics are folded into `weights` and `bias`.  `out`: where the result goes, e.g.
+  a channel slice of the tensor a later layer reads as a concatenation."""
   return _conv("ocnn_octree_conv_fused", deconv, data_in, weights, octree, depth, num_output,
-               kernel_size, stride, nempty, bias=bias, relu=relu)
+               kernel_size, stride, nempty, bias=bias, relu=relu, out=out)
 
 
 def _conv_grad(fn, is_deconv, data_in, weights, octree, grad_in, depth, num_output, kernel_size, stride,

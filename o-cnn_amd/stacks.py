@@ -30,15 +30,16 @@ def fold_bn(weights, gamma, beta, mean, var, eps=BN_EPS, deconv=False, kdim=None
 
 
 def conv_bn_relu(data, w, b, octree, depth, cout, kernel_size=(3, 3, 3), stride=1, nempty=False,
-                 deconv=False, relu=True):
+                 deconv=False, relu=True, out=None):
   """OctreeConvBnRelu / OctreeDeConvBnRelu with folded BatchNorm, including the pad / depad the
   reference modules add around stride-2 layers (pytorch/ocnn/octree_conv.py:102-127)."""
   ks = list(kernel_size)
   if deconv and stride == 2 and not nempty:
     data = F.octree_depad(data, octree, depth)
+  padded_after = (not deconv) and stride == 2 and not nempty
   out = F.octree_conv_fused(data, w.to(data.dtype), b, relu, octree, depth, cout, ks, stride, nempty,
-                            deconv=deconv)
-  if (not deconv) and stride == 2 and not nempty:
+                            deconv=deconv, out=None if padded_after else out)
+  if padded_after:
     # a padded (empty) node holds 0 in the reference because the pad comes after conv but
     # before BatchNorm; after folding the empty nodes must receive relu(b) instead of 0:
     # the reference order is conv -> pad -> BN -> ReLU.
@@ -72,25 +73,38 @@ def unet_trunk(octree, depth, params, data=None, stages=3, nempty=False):
     data = F.octree_property(octree, "feature", depth)
     if nempty:
       data = F.octree_depad(data, octree, depth)
-  feats = {}
-  w, b = params[("conv", depth)]
-  feats[depth] = conv_bn_relu(data, w, b, octree, depth, w.shape[0], nempty=nempty)
+  # The decoder reads [encoder feature of depth d | upsampled feature] as one tensor.  That tensor
+  # is allocated when the encoder reaches depth d, and both producers write their channel slice
+  # of it directly: no concatenation copy.
+  info = F.octree_info(octree)
+  feats, joined = {}, {}
+
+  def encoder_conv(x, d, skip):
+    w, b = params[("conv", d)]
+    c_skip = w.shape[0]
+    if not skip:
+      return conv_bn_relu(x, w, b, octree, d, c_skip, nempty=nempty)
+    c_up = params[("up", d - 1)][0].shape[1] // 8
+    rows = info.nnum_nempty(d) if nempty else info.nnum(d)
+    joined[d] = torch.empty(1, c_skip + c_up, rows, 1, dtype=x.dtype, device=x.device)
+    return conv_bn_relu(x, w, b, octree, d, c_skip, nempty=nempty, out=joined[d][:, :c_skip])
+
+  feats[depth] = encoder_conv(data, depth, stages > 0)
   d = depth
-  for _ in range(stages):
+  for i in range(stages):
     w, b = params[("down", d)]
     x = conv_bn_relu(feats[d], w, b, octree, d, w.shape[0], (2, 2, 2), 2, nempty)
     d -= 1
-    w, b = params[("conv", d)]
-    feats[d] = conv_bn_relu(x, w, b, octree, d, w.shape[0], nempty=nempty)
+    feats[d] = encoder_conv(x, d, i + 1 < stages)
   x = feats[d]
   for _ in range(stages):
     w, b = params[("up", d)]
     cout = w.shape[1] // 8
-    x = conv_bn_relu(x, w, b, octree, d, cout, (2, 2, 2), 2, nempty, deconv=True)
     d += 1
-    x = torch.cat([feats[d], x], dim=1)
+    c_skip = feats[d].shape[1]
+    conv_bn_relu(x, w, b, octree, d - 1, cout, (2, 2, 2), 2, nempty, deconv=True, out=joined[d][:, c_skip:])
     w, b = params[("dec", d)]
-    x = conv_bn_relu(x, w, b, octree, d, w.shape[0], nempty=nempty)
+    x = conv_bn_relu(joined[d], w, b, octree, d, w.shape[0], nempty=nempty)
   return x
 
 
