@@ -143,7 +143,10 @@ __device__ inline void store_tiles(const ConvArgs& a, OutT* __restrict__ out, fl
 // 8-channel group and the four values feed four MFMA k-steps with k-pairs (j, 4+j).
 // Loop nest: pass over 32*MT output rows -> tap -> 64-channel slab (its weights staged in LDS
 // in A-fragment order, next slab prefetched) -> 8-channel group.
-constexpr int kRowSlab = 64;
+constexpr int kRowSlab = 64;    // channels per stage of the bf16 row kernel
+constexpr int kRowSlabF = 32;   // ... of the fp32 row kernel: with 64 the weights on their way to LDS no longer fit the
+                                // register file next to the gathers of the next stage and travel through scratch memory
+                                // (a wait for every weight load as soon as it is issued, every stage)
 
 __global__ __launch_bounds__(256) void transpose_rows_f32_kernel(float* __restrict__ dst,
     const float* __restrict__ src, int C, int H, int Cpad) {
@@ -169,7 +172,7 @@ __global__ __launch_bounds__(256) void transpose_rows_f32_kernel(float* __restri
 template <int MT>
 __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* __restrict__ out,
     const float4* __restrict__ xt, const float* __restrict__ Wt, int n_tiles, int cpad) {
-  constexpr int kWWords = (kRowSlab / 8) * 4 * MT * 64;  // weights of one (tap, slab)
+  constexpr int kWWords = (kRowSlabF / 8) * 4 * MT * 64;  // weights of one (tap, slab)
   constexpr int kWVec = kWWords / 4 / 256;               // float4 per thread (4 for MT = 2)
   __shared__ __attribute__((aligned(16))) float sW[2 * kWWords];  // double buffered: one barrier per stage
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -177,7 +180,7 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
   if (tile >= n_tiles) return;
   const int n0 = tile * kTileCols + wave * kWaveCols;
   const int r = lane & 31, kh = lane >> 5;
-  const int nslab = (cpad + kRowSlab - 1) / kRowSlab;
+  const int nslab = (cpad + kRowSlabF - 1) / kRowSlabF;
   const int npass = (a.mtiles + MT - 1) / MT;
   const int cpad4 = cpad >> 2;
   const int nstage = a.K * nslab;
@@ -189,36 +192,40 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
       for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
-    float4 wr[kWVec > 0 ? kWVec : 1];
+    // weights on their way to LDS: a value type, so that they stay in registers
+    struct WRegs { float4 v[kWVec > 0 ? kWVec : 1]; };
+    WRegs wr;
     auto fetch_w = [&](int stage) {
       const float4* wsrc = reinterpret_cast<const float4*>(Wt + ((int64_t)pass * nstage + stage) * kWWords);
+      WRegs w;
 #pragma unroll
-      for (int v = 0; v < kWVec; ++v) wr[v] = wsrc[v * 256 + threadIdx.x];
+      for (int v = 0; v < kWVec; ++v) w.v[v] = wsrc[v * 256 + threadIdx.x];
+      return w;
     };
     // Software pipeline over the stages (tap, 64-channel slab): while the MFMAs of one stage run,
     // the weights AND all gathers of the next stage (8 channel groups x 2 columns, 16 bytes each)
     // are in flight; the source rows of a tap are looked up two taps ahead.
-    float4 nx0[kRowSlab / 8], nx1[kRowSlab / 8];
+    float4 nx0[kRowSlabF / 8], nx1[kRowSlabF / 8];
     auto src_of = [&](int k, int half) { return k < a.K ? conv_src(a, n0 + half * 32 + r, k) : -1; };
     auto fetch_x = [&](int s0, int s1, int slab) {
       const float4* row0 = xt + (int64_t)(s0 < 0 ? a.Hin : s0) * cpad4 + kh;
       const float4* row1 = xt + (int64_t)(s1 < 0 ? a.Hin : s1) * cpad4 + kh;
-      const int ngroup = min(kRowSlab, cpad - slab * kRowSlab) >> 3;
+      const int ngroup = min(kRowSlabF, cpad - slab * kRowSlabF) >> 3;
 #pragma unroll
-      for (int c8 = 0; c8 < kRowSlab / 8; ++c8)
+      for (int c8 = 0; c8 < kRowSlabF / 8; ++c8)
         if (c8 < ngroup) {
-          nx0[c8] = row0[(slab * kRowSlab + c8 * 8) >> 2];
-          nx1[c8] = row1[(slab * kRowSlab + c8 * 8) >> 2];
+          nx0[c8] = row0[(slab * kRowSlabF + c8 * 8) >> 2];
+          nx1[c8] = row1[(slab * kRowSlabF + c8 * 8) >> 2];
         }
     };
     int s0c = src_of(0, 0), s1c = src_of(0, 1);      // rows of the current tap
     int s0n = src_of(1, 0), s1n = src_of(1, 1);      // ... of the next one
-    fetch_w(0);
+    wr = fetch_w(0);
     fetch_x(s0c, s1c, 0);
     __syncthreads();  // the last stage of the previous pass may still be reading the weights
 #pragma unroll
-    for (int v = 0; v < kWVec; ++v) reinterpret_cast<float4*>(sW)[v * 256 + threadIdx.x] = wr[v];
-    if (1 < nstage) fetch_w(1);
+    for (int v = 0; v < kWVec; ++v) reinterpret_cast<float4*>(sW)[v * 256 + threadIdx.x] = wr.v[v];
+    if (1 < nstage) wr = fetch_w(1);
     int stage = 0;
     for (int k = 0; k < a.K; ++k) {
       const int s0n2 = src_of(k + 2, 0), s1n2 = src_of(k + 2, 1);
@@ -231,7 +238,7 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
         if (stage + 1 < nstage) {
 #pragma unroll
           for (int v = 0; v < kWVec; ++v)
-            reinterpret_cast<float4*>(sW + ((stage + 1) & 1) * kWWords)[v * 256 + threadIdx.x] = wr[v];
+            reinterpret_cast<float4*>(sW + ((stage + 1) & 1) * kWWords)[v * 256 + threadIdx.x] = wr.v[v];
         }
         // group c8 of the NEXT stage is requested right after group c8 of this one has been read
         // out of its registers, so every gather has seven eighths of a stage to arrive
@@ -239,13 +246,13 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
         const bool same_tap = slab + 1 < nslab;
         const int nslab_next = same_tap ? slab + 1 : 0;
         const int s0x = same_tap ? s0c : s0n, s1x = same_tap ? s1c : s1n;
-        const float4* nrow0 = xt + (int64_t)(s0x < 0 ? a.Hin : s0x) * cpad4 + kh + ((nslab_next * kRowSlab) >> 2);
-        const float4* nrow1 = xt + (int64_t)(s1x < 0 ? a.Hin : s1x) * cpad4 + kh + ((nslab_next * kRowSlab) >> 2);
-        const int ngroup_next = more ? (min(kRowSlab, cpad - nslab_next * kRowSlab) >> 3) : 0;
-        if (stage + 2 < nstage) fetch_w(stage + 2);
-        const int ngroup = min(kRowSlab, cpad - slab * kRowSlab) >> 3;
+        const float4* nrow0 = xt + (int64_t)(s0x < 0 ? a.Hin : s0x) * cpad4 + kh + ((nslab_next * kRowSlabF) >> 2);
+        const float4* nrow1 = xt + (int64_t)(s1x < 0 ? a.Hin : s1x) * cpad4 + kh + ((nslab_next * kRowSlabF) >> 2);
+        const int ngroup_next = more ? (min(kRowSlabF, cpad - nslab_next * kRowSlabF) >> 3) : 0;
+        if (stage + 2 < nstage) wr = fetch_w(stage + 2);
+        const int ngroup = min(kRowSlabF, cpad - slab * kRowSlabF) >> 3;
 #pragma unroll
-        for (int c8 = 0; c8 < kRowSlab / 8; ++c8) {
+        for (int c8 = 0; c8 < kRowSlabF / 8; ++c8) {
           const float4 b0 = nx0[c8], b1 = nx1[c8];
           if (c8 < ngroup_next) {
             nx0[c8] = nrow0[c8 * 2];
@@ -274,17 +281,17 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
 __global__ void pack_weights_rows_f32(float* __restrict__ Wt, const float* __restrict__ W, int M, int Cin, int K,
     int MT, int npass, int nslab, int64_t sm, int64_t sc) {
   int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  int64_t total = (int64_t)npass * K * nslab * (kRowSlab / 8) * 4 * MT * 64;
+  int64_t total = (int64_t)npass * K * nslab * (kRowSlabF / 8) * 4 * MT * 64;
   if (id >= total) return;
   int l = (int)(id & 63);
   int64_t f = id >> 6;
   int mt = (int)(f % MT); f /= MT;
   int j = (int)(f % 4); f /= 4;
-  int c8 = (int)(f % (kRowSlab / 8)); f /= (kRowSlab / 8);
+  int c8 = (int)(f % (kRowSlabF / 8)); f /= (kRowSlabF / 8);
   int slab = (int)(f % nslab); f /= nslab;
   int k = (int)(f % K);
   int pass = (int)(f / K);
-  int m = (pass * MT + mt) * 32 + (l & 31), c = slab * kRowSlab + c8 * 8 + 4 * (l >> 5) + j;
+  int m = (pass * MT + mt) * 32 + (l & 31), c = slab * kRowSlabF + c8 * 8 + 4 * (l >> 5) + j;
   Wt[id] = (m < M && c < Cin) ? W[m * sm + c * sc + k] : 0.0f;
 }
 
@@ -1185,8 +1192,9 @@ int make_plan(const Info* o, int depth, int channel_in, int num_output, const in
   p->csteps = 0;
   {  // general row-major gather path: padded weights + the row-major copy of the input
     size_t cpad = dtype == OCNN_F32 ? ((size_t)channel_in + 7) / 8 * 8 : ((size_t)channel_in + 15) / 16 * 16;
-    size_t nslab = (cpad + kRowSlab - 1) / kRowSlab, npass = (size_t)(p->mtiles + 1) / 2;
-    size_t per_stage = dtype == OCNN_F32 ? (kRowSlab / 8) * 4 * 2 * 64 * sizeof(float)
+    const size_t slab = dtype == OCNN_F32 ? kRowSlabF : kRowSlab;
+    size_t nslab = (cpad + slab - 1) / slab, npass = (size_t)(p->mtiles + 1) / 2;
+    size_t per_stage = dtype == OCNN_F32 ? (kRowSlabF / 8) * 4 * 2 * 64 * sizeof(float)
                                          : (kRowSlab / 16) * 2 * 64 * 8 * sizeof(uint16_t);
     p->wt_bytes = align256(npass * p->taps.count * nslab * per_stage);
     p->xt_general = align256(((size_t)p->btm_h + 1) * cpad * (dtype == OCNN_F32 ? 4 : 2));
@@ -1337,8 +1345,8 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
   } else if (dtype == OCNN_F32) {
     const int MT = a.mtiles == 1 ? 1 : 2;
     const int cpad = (a.Cin + 7) / 8 * 8;
-    const int npass = (a.mtiles + MT - 1) / MT, nslab = (cpad + kRowSlab - 1) / kRowSlab;
-    int64_t total = (int64_t)npass * a.K * nslab * (kRowSlab / 8) * 4 * MT * 64;
+    const int npass = (a.mtiles + MT - 1) / MT, nslab = (cpad + kRowSlabF - 1) / kRowSlabF;
+    int64_t total = (int64_t)npass * a.K * nslab * (kRowSlabF / 8) * 4 * MT * 64;
     pack_weights_rows_f32<<<blocks_for(total), kBlock, 0, s>>>((float*)wsb, (const float*)weights, a.M, a.Cin, a.K,
         MT, npass, nslab, sm, sc);
     OCNN_LAUNCH_OK("pack_weights_rows");
