@@ -66,8 +66,12 @@ _workspaces = {}
 
 
 def _workspace(nbytes, tag="main"):
-  """A cached, growing device scratch buffer per (device, tag)."""
-  key = (torch.cuda.current_device(), tag)
+  """A cached, growing device scratch buffer per (device, stream, tag).  Calls that share a
+  workspace must not overlap, and calls on one stream never do; calls on different streams get
+  different buffers.  A buffer is allocated while its stream is current, so when it is
+  outgrown and dropped the caching allocator hands the block out again only in that stream's
+  order: kernels still queued on the stream keep their memory."""
+  key = (torch.cuda.current_device(), torch.cuda.current_stream().cuda_stream, tag)
   buf = _workspaces.get(key)
   if buf is None or buf.numel() < nbytes:
     buf = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=_dev())
