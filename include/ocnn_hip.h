@@ -171,6 +171,24 @@ int ocnn_octree_conv_fused(void* top, const void* btm, int channel_in, int btm_h
     int num_output, const int* kernel_size, int stride, int nempty, int dtype, void* workspace_dev,
     size_t workspace_bytes, ocnn_stream_t stream);
 
+/* ocnn_octree_conv_fused for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments and results minus the workspace: the packed weights, the inverted
+ * child links of the non-empty mode and, for the kernels that read one, the row-major copy of
+ * the input go into an array of OCNN_STATIC_SCRATCH_BYTES bytes that the library holds on every
+ * GPU it runs on until the process ends.  A call that needs more fails with OCNN_E_WORKSPACE and
+ * a message that says how much (fp32 convolutions over all nodes and every 2x2x2 stride-2 fp32
+ * or bf16 convolution need the packed weights only, so any octree size fits; bf16 3x3x3 and the
+ * non-empty mode also need 2 or 4 bytes x padded channels x input rows).  The call allocates
+ * nothing and waits for nothing.  All calls on one GPU share the array: calls that overlap on
+ * one GPU (two streams, two threads) race; calls on one stream are ordered and safe.
+ * ocnn_device_check(dev) resolves the array's address for `dev` ahead of time; otherwise the
+ * first call on a device does. */
+#define OCNN_STATIC_SCRATCH_BYTES (16u << 20)
+int ocnn_octree_conv_static(void* top, const void* btm, int channel_in, int btm_h, const void* weights,
+    const float* bias, int relu, int is_deconv, const void* octree_dev, const void* info, int depth,
+    int num_output, const int* kernel_size, int stride, int nempty, int dtype, ocnn_stream_t stream);
+
 /* ---- gradients: OctreeConvGradOp / OctreeDeconvGradOp, pytorch/cpp/octree_conv.cpp:159-250
  * (weight_gpu_gemm / backward_gpu_gemm / forward_gpu_gemm, octree/octree/octree_conv.cpp:276-356).
  * Arguments are those of the forward call plus `grad_out` [num_output, top_h]; the results have

@@ -14,6 +14,8 @@
 // load shared by all wavefronts through the vector L1.
 #include "ocnn_common.h"
 
+#include <mutex>
+
 namespace ocnn {
 namespace {
 
@@ -1235,7 +1237,7 @@ int make_plan(const Info* o, int depth, int channel_in, int num_output, const in
 int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, const void* weights,
     const void* octree_dev, const void* info, int depth, int num_output, const int* ks, int stride,
     int nempty, int dtype, void* ws, size_t ws_bytes, hipStream_t s, const float* bias = nullptr,
-    int relu = 0) {
+    int relu = 0, bool builtin_scratch = false) {
   OCNN_REQUIRE(top && btm && weights && octree_dev && info, OCNN_E_BADARG, "null pointer");
   const Info* o = as_info(info);
   ConvPlan p;
@@ -1243,8 +1245,8 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
   if (e) return e;
   OCNN_REQUIRE(btm_h == p.btm_h, OCNN_E_SHAPE, "input height %d, the octree has %d rows at depth %d",
       btm_h, p.btm_h, depth);
-  OCNN_REQUIRE(ws && ws_bytes >= p.total_bytes, OCNN_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes,
-      p.total_bytes);
+  OCNN_REQUIRE(ws && (builtin_scratch || ws_bytes >= p.total_bytes), OCNN_E_WORKSPACE,
+      "workspace %zu < %zu bytes", ws_bytes, p.total_bytes);
   OCNN_REQUIRE((reinterpret_cast<uintptr_t>(ws) & 15) == 0, OCNN_E_WORKSPACE, "workspace not 16-byte aligned");
 
   const char* blob = static_cast<const char*>(octree_dev);
@@ -1283,20 +1285,48 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
   }
 
   char* wsb = static_cast<char*>(ws);
-  if (nempty) {
-    int* ichild = reinterpret_cast<int*>(wsb + p.wt_bytes);
-    ichild_kernel<<<blocks_for(p.child_h), kBlock, 0, s>>>(ichild, p.ichild_h, a.child, p.child_h);
-    OCNN_LAUNCH_OK("ichild");
-    a.ichild = ichild;
-  }
   // conv: W[num_output, channel_in*K]; deconv: W[channel_in, num_output*K]
   int64_t sm = deconv ? a.K : (int64_t)channel_in * a.K;
   int64_t sc = deconv ? (int64_t)num_output * a.K : a.K;
   int n_tiles = (a.N + kTileCols - 1) / kTileCols;
   int grid = ((n_tiles + 7) / 8) * 8;
   const bool k222 = ks[0] == 2 && ks[1] == 2 && ks[2] == 2;
+  // which kernel runs, and how much of the workspace it touches: the weights in their packed
+  // order always come first, the inverted child links of the non-empty mode second, the
+  // row-major copy of the input (only some kernels read one) last
+  enum { kPathS2Conv, kPathS2Deconv, kPathS1LdsF32, kPathRowsF32, kPathS1LdsBf16, kPathRowsBf16 } path;
+  bool copies_input = true;
   if (a.mode == kModeS2Conv && !a.nempty && k222 && (a.Hin & 7) == 0 &&
       (reinterpret_cast<uintptr_t>(btm) & 15) == 0) {
+    path = kPathS2Conv;
+    copies_input = false;
+  } else if (a.mode == kModeS2Deconv && !a.nempty && (reinterpret_cast<uintptr_t>(top) & 15) == 0 &&
+             (dtype != OCNN_F32 || (reinterpret_cast<uintptr_t>(weights) & 15) == 0)) {
+    path = kPathS2Deconv;
+    copies_input = dtype != OCNN_F32;
+  } else if (dtype == OCNN_F32 && a.mode == kModeS1 && !a.nempty && a.K == 27) {
+    path = kPathS1LdsF32;
+    copies_input = false;
+  } else if (dtype == OCNN_F32) {
+    path = kPathRowsF32;
+  } else if (a.mode == kModeS1 && !a.nempty && a.K == 27) {
+    path = kPathS1LdsBf16;
+  } else {
+    path = kPathRowsBf16;
+  }
+  if (builtin_scratch) {
+    const size_t used = p.wt_bytes + p.ichild_bytes + (copies_input ? p.xt_bytes : 0);
+    OCNN_REQUIRE(used <= ws_bytes, OCNN_E_WORKSPACE,
+        "this call needs %zu bytes of scratch memory, the built-in array holds %zu: "
+        "use ocnn_octree_conv_fused with a workspace of your own", used, ws_bytes);
+  }
+  if (nempty) {
+    int* ichild = reinterpret_cast<int*>(wsb + p.wt_bytes);
+    ichild_kernel<<<blocks_for(p.child_h), kBlock, 0, s>>>(ichild, p.ichild_h, a.child, p.child_h);
+    OCNN_LAUNCH_OK("ichild");
+    a.ichild = ichild;
+  }
+  if (path == kPathS2Conv) {
     const int MT = a.mtiles == 1 ? 1 : 2;
     const int npass = (a.mtiles + MT - 1) / MT;
     if (dtype == OCNN_F32) {
@@ -1312,8 +1342,7 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
       if (MT == 1) conv_s2_bf16_kernel<1><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const uint16_t*)btm, (const uint4*)wsb, n_tiles);
       else conv_s2_bf16_kernel<2><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const uint16_t*)btm, (const uint4*)wsb, n_tiles);
     }
-  } else if (a.mode == kModeS2Deconv && !a.nempty && (reinterpret_cast<uintptr_t>(top) & 15) == 0 &&
-             (dtype != OCNN_F32 || (reinterpret_cast<uintptr_t>(weights) & 15) == 0)) {
+  } else if (path == kPathS2Deconv) {
     // columns are the parents here: one column tile writes the 8 children of 256 parents
     ConvArgs d = a;
     d.N = a.Hin;
@@ -1331,7 +1360,7 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
       transpose_rows_bf16_kernel<<<tgrid, 256, 0, s>>>(xt, (const uint16_t*)btm, a.Cin, a.Hin, cpad);
       deconv_s2_bf16_kernel<<<dim3(d_grid, pass_split(d_tiles, (d.M * 8 + 32 * kD2MT - 1) / (32 * kD2MT))), 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles, cpad / 8);
     }
-  } else if (dtype == OCNN_F32 && a.mode == kModeS1 && !a.nempty && a.K == 27) {
+  } else if (path == kPathS1LdsF32) {
     const int MT = a.mtiles == 1 ? 1 : 2;
     const int npass = (a.mtiles + MT - 1) / MT, nslab = (a.Cin + kSlab - 1) / kSlab;
     int64_t total = (int64_t)npass * nslab * a.K * kKSteps * MT * 64;
@@ -1342,7 +1371,7 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
       conv_s1_f32_lds_kernel<1, 27><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
     else
       conv_s1_f32_lds_kernel<2, 27><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
-  } else if (dtype == OCNN_F32) {
+  } else if (path == kPathRowsF32) {
     const int MT = a.mtiles == 1 ? 1 : 2;
     const int cpad = (a.Cin + 7) / 8 * 8;
     const int npass = (a.mtiles + MT - 1) / MT, nslab = (cpad + kRowSlabF - 1) / kRowSlabF;
@@ -1358,7 +1387,7 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
       conv_rows_f32_kernel<1><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (float*)top, (const float4*)xt, (const float*)wsb, n_tiles, cpad);
     else
       conv_rows_f32_kernel<2><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (float*)top, (const float4*)xt, (const float*)wsb, n_tiles, cpad);
-  } else if (a.mode == kModeS1 && !a.nempty && a.K == 27) {
+  } else if (path == kPathS1LdsBf16) {
     const int MT = a.mtiles == 1 ? 1 : 2;
     const int cpad = (a.Cin + 15) / 16 * 16;
     const int npass = (a.mtiles + MT - 1) / MT, nslab = cpad / 16;
@@ -1907,11 +1936,58 @@ int run_grad(int is_deconv, void* grad_data, void* grad_w, const void* data_in, 
 }
 
 }  // namespace
+
+// ---- scratch memory that belongs to the library ------------------------------------------
+// ocnn_octree_conv_static serves callers that cannot allocate (code under HIP graph capture,
+// serving loops, harnesses that forbid it): its workspace is this array.  Every GPU the
+// library runs on holds its own copy at its own address for the life of the process; the name
+// below is only the host-side handle of the symbol, the address kernels may use comes from
+// hipGetSymbolAddress with that GPU current.
+constexpr size_t kBuiltinScratchBytes = (size_t)OCNN_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kBuiltinScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices];
+
+// The array's address on the current device (looked up once per device), or a negative code.
+int builtin_scratch(void** out) {
+  int dev = -1;
+  OCNN_HIP_OK(hipGetDevice(&dev));
+  OCNN_REQUIRE(dev >= 0 && dev < kMaxDevices, OCNN_E_UNSUPPORTED, "device %d beyond the %d this library tracks",
+      dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    OCNN_HIP_OK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    OCNN_REQUIRE(ptr != nullptr, OCNN_E_HIP, "the scratch array has no address on device %d", dev);
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return OCNN_OK;
+}
+
+// called by ocnn_device_check so that set-up code can resolve the address ahead of the first call
+int prepare_builtin_scratch() {
+  void* ptr = nullptr;
+  return builtin_scratch(&ptr);
+}
+
 }  // namespace ocnn
 
 using namespace ocnn;
 
 extern "C" {
+
+int ocnn_octree_conv_static(void* top, const void* btm, int channel_in, int btm_h, const void* weights,
+    const float* bias, int relu, int is_deconv, const void* octree_dev, const void* info, int depth,
+    int num_output, const int* kernel_size, int stride, int nempty, int dtype, ocnn_stream_t stream) {
+  void* ptr = nullptr;
+  int e = builtin_scratch(&ptr);
+  if (e) return e;
+  return run_conv(is_deconv ? 1 : 0, top, btm, channel_in, btm_h, weights, octree_dev, info, depth, num_output,
+      kernel_size, stride, nempty, dtype, ptr, kBuiltinScratchBytes, as_stream(stream), bias, relu, true);
+}
 
 int ocnn_conv_shape(const void* info, int depth, int channel_in, int num_output, const int* kernel_size,
     int stride, int nempty, int is_deconv, int dtype, int* top_h, int* btm_h, size_t* workspace_bytes) {

@@ -114,7 +114,14 @@ int ocnn_device_check(int dev) {
   OCNN_HIP_OK(hipGetDeviceProperties(&p, dev));
   OCNN_REQUIRE(strncmp(p.gcnArchName, "gfx950", 6) == 0, OCNN_E_UNSUPPORTED,
       "device %d is %s, this library holds gfx950 code only", dev, p.gcnArchName);
-  return OCNN_OK;
+  // set-up work that must not fall into a caller's first (possibly captured) operator call:
+  // the address of the library's own scratch array on this device
+  int cur = -1;
+  OCNN_HIP_OK(hipGetDevice(&cur));
+  if (cur != dev) OCNN_HIP_OK(hipSetDevice(dev));
+  int e = ocnn::prepare_builtin_scratch();
+  if (cur != dev) OCNN_HIP_OK(hipSetDevice(cur));
+  return e;
 }
 
 int ocnn_info_check(const void* info) {  // octree_info.cpp:80-116

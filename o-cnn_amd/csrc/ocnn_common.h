@@ -99,6 +99,10 @@ int fail(int code, const char* fmt, ...);
       return ::ocnn::fail(OCNN_E_HIP, "launch %s: %s", name, hipGetErrorString(e__)); \
   } while (0)
 
+// resolves, for the current device, the address of the scratch array behind
+// ocnn_octree_conv_static (conv.hip); cheap after the first call on a device
+int prepare_builtin_scratch();
+
 inline hipStream_t as_stream(ocnn_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
 constexpr int kBlock = 256;
