@@ -171,6 +171,14 @@ int ocnn_octree_conv_fused(void* top, const void* btm, int channel_in, int btm_h
     int num_output, const int* kernel_size, int stride, int nempty, int dtype, void* workspace_dev,
     size_t workspace_bytes, ocnn_stream_t stream);
 
+/* Tuning knob, no counterpart in the reference: 3x3x3 stride-1 bf16 convolutions over all nodes
+ * run one of two kernels, chosen by the number of 1024-column tiles of the level; the
+ * register-fed kernel takes levels of at least `tiles` tiles (default 192, about 200 000
+ * octants).  0 restores the default, a negative value sends every level to it (the tests use
+ * that to run it on small octrees).  Returns the previous threshold.  Both kernels add the same
+ * products in the same order: the results do not depend on the choice. */
+int ocnn_conv_bf16_tile_threshold(int tiles);
+
 /* ocnn_octree_conv_fused for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
  * reference.  Same arguments and results minus the workspace: the packed weights, the inverted

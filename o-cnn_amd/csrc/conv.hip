@@ -14,7 +14,9 @@
 // load shared by all wavefronts through the vector L1.
 #include "ocnn_common.h"
 
+#include <atomic>
 #include <mutex>
+#include <type_traits>
 
 namespace ocnn {
 namespace {
@@ -751,6 +753,249 @@ __global__ __launch_bounds__(256, 2) void conv_s1_bf16_lds_kernel(ConvArgs a, ui
   }
 }
 
+// ---- register-fed bf16 kernel (3x3x3, stride 1, all nodes, large levels) ---------------------
+// The LDS kernel above serves every (tap, sibling) pair with its own operand read, and its phases
+// (gather -> LDS -> barrier -> compute) of two workgroups per CU do not hide one another.  Here a
+// wavefront owns 32 sibling groups and ALL 8 siblings of each: its accumulators are 8 siblings x
+// MT row tiles of 32x32 (256 registers for 64 output channels, the accumulation half of the
+// register file at one wavefront per SIMD), MFMA column n is GROUP n, and the B operand of slot
+// (x, y, z) -- lane (n, kh) holds 8 channels of the row found in that slot of group n's 4x4x4
+// neighbour block -- serves every sibling (i, j, k) whose tap (x - i, y - j, z - k) exists: 6.75
+// MFMAs per operand on average instead of 2.  So the operands come straight from the row-major
+// copy into registers: every slot row is requested once per k-step, exactly as often as the LDS
+// kernel stages it, nothing of the input passes through LDS and no barrier sits between a
+// gather and its use.  The block is walked x-layer by x-layer (16 slots = 64 registers, the next
+// layer in flight in a second set): layer L feeds the siblings with i = 0 through the taps
+// dx = L and those with i = 1 through dx = L - 1.
+// Weights: all 27 taps of one 16-channel k-step sit in LDS in A-fragment order (54 KiB for 64
+// output channels), the next k-step's are copied in during the current one (two buffers, one
+// barrier per k-step); a wavefront reads each tap's fragment twice per k-step, 0.25 KiB of LDS
+// operands per MFMA.  The neighbour rows of a wavefront's groups wait in LDS too (68 words per
+// group: 16-byte reads of 32 lanes then meet no bank twice).
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+
+// two fp32 values -> two bf16 in one word (round to nearest even, the conversion instruction of
+// this GPU; the same values as f32_to_bf16 for everything that is not a NaN)
+__device__ inline uint32_t pack_bf16x2(float lo, float hi) {
+  floatx2 f = {lo, hi};
+  bf16x2 h = __builtin_convertvector(f, bf16x2);
+  return __builtin_bit_cast(uint32_t, h);
+}
+// max(v, floor) that keeps a NaN (floor = 0 for a ReLU, -inf for none)
+__device__ inline float relu_floor(float v, float floor) { return v < floor ? floor : v; }
+
+constexpr int kRegGroups = 32;               // sibling groups (MFMA columns) per wavefront
+constexpr int kRegTileGroups = 4 * kRegGroups;
+constexpr int kNbPitch = 68;
+
+template <int MT>
+__global__ __launch_bounds__(256, 1) void conv_s1_bf16_reg_kernel(ConvArgs a, uint16_t* __restrict__ out,
+    const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles, int cpad8) {
+  constexpr int kWUnits = 27 * MT * 64;        // 16-byte units of one k-step's weights
+  constexpr int kWPiece = kWUnits / 4;         // copied per layer phase
+  constexpr int kWVec = (kWPiece + 255) / 256;
+  constexpr int kWVec0 = (kWUnits + 255) / 256;
+  __shared__ u32x4 sW[2][kWUnits];
+  __shared__ __attribute__((aligned(16))) int sNb[4][kRegGroups * kNbPitch];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = xcd_tile(blockIdx.x, n_tiles);
+  if (tile >= n_tiles) return;
+  const int n = lane & 31, kh = lane >> 5;
+  const int nks = cpad8 >> 1;                  // 16-channel k-steps
+  const int npass = (a.mtiles + MT - 1) / MT;
+  const int n_groups = a.N >> 3;
+  const int g0 = tile * kRegTileGroups + wave * kRegGroups;
+  const int row_bytes = cpad8 * 16;
+  const int half = kh * 16;
+
+  // the row-major copy and the packed weights as buffers: 32-bit offsets per lane, the k-step's
+  // column / the piece of the weights as the scalar offset (the host sends levels beyond 2 GiB
+  // to the other kernel)
+  const __amdgpu_buffer_rsrc_t xrows = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<u32x4*>(xt), 0, (int)(((int64_t)a.Hin + 1) * row_bytes), 0x00020000);
+  const __amdgpu_buffer_rsrc_t wbuf = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<u32x4*>(Wt), 0, npass * nks * kWUnits * 16, 0x00020000);
+
+  // Set-up, all requests in flight before the first is looked at: the neighbour tables of my
+  // 32 groups (8 KiB in one piece, eight 16-byte loads per lane) and the first k-step's weights
+  // of the first pass.  The tables go to LDS as byte offsets of the rows (a missing neighbour and
+  // anything beyond the level = row Hin, which is all zero).
+  int pass = blockIdx.y;
+  {
+    const int u0 = g0 * 16;                       // my first 16-byte unit of the level's table
+    const int4* nsrc = reinterpret_cast<const int4*>(a.neigh);
+    const int last = n_groups * 16 - 1;
+    int4 nv[8];
+    u32x4 w0[kWVec0];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) nv[j] = nsrc[min(u0 + j * 64 + lane, last)];
+#pragma unroll
+    for (int v = 0; v < kWVec0; ++v)
+      w0[v] = __builtin_amdgcn_raw_buffer_load_b128(wbuf, min(v * 256 + (int)threadIdx.x, kWUnits - 1) * 16,
+          pass * nks * kWUnits * 16, 0);
+    const unsigned hin = (unsigned)a.Hin;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int u = j * 64 + lane;               // group u >> 4, slots 4 (u & 15) ...
+      const unsigned gone = (unsigned)((last - (u0 + u)) >> 31);   // all ones past the end of the table
+      int4 o;
+      o.x = (int)(min((unsigned)nv[j].x | gone, hin) * (unsigned)row_bytes);
+      o.y = (int)(min((unsigned)nv[j].y | gone, hin) * (unsigned)row_bytes);
+      o.z = (int)(min((unsigned)nv[j].z | gone, hin) * (unsigned)row_bytes);
+      o.w = (int)(min((unsigned)nv[j].w | gone, hin) * (unsigned)row_bytes);
+      *reinterpret_cast<int4*>(&sNb[wave][(u >> 4) * kNbPitch + 4 * (u & 15)]) = o;
+    }
+#pragma unroll
+    for (int v = 0; v < kWVec0; ++v) sW[0][min(v * 256 + (int)threadIdx.x, kWUnits - 1)] = w0[v];
+  }
+
+  u32x4 bl[2][16];   // two x-layers of operands: [buffer][y*4 + z]
+  u32x4 wr[kWVec];
+  // requests the 4 slot rows (Y, 0..3) of layer L at k-step KS into buffer L & 1
+#define OCNN_REQ_ROW(KS, L, Y)                                                                  \
+  do {                                                                                          \
+    const int4 rows = *reinterpret_cast<const int4*>(&sNb[wave][n * kNbPitch + (L) * 16 + (Y) * 4]); \
+    const int col = (KS) * 32;                                                                  \
+    bl[(L) & 1][(Y) * 4 + 0] = __builtin_amdgcn_raw_buffer_load_b128(xrows, rows.x + half, col, 0); \
+    bl[(L) & 1][(Y) * 4 + 1] = __builtin_amdgcn_raw_buffer_load_b128(xrows, rows.y + half, col, 0); \
+    bl[(L) & 1][(Y) * 4 + 2] = __builtin_amdgcn_raw_buffer_load_b128(xrows, rows.z + half, col, 0); \
+    bl[(L) & 1][(Y) * 4 + 3] = __builtin_amdgcn_raw_buffer_load_b128(xrows, rows.w + half, col, 0); \
+  } while (0)
+  // Layer L + 2 (of this k-step, or layer L - 2 of the next) takes over the registers of layer L
+  // row by row as the rows die: row y is last used by the taps with dy = min(y, 2).  Its first
+  // rows are then under way for a phase and two thirds before the phase that multiplies them
+  // starts, the last ones for a phase and a third.
+#define OCNN_REFILL(KS, L, Y)                                                                   \
+  do {                                                                                          \
+    if ((L) < 2) OCNN_REQ_ROW(KS, (L) + 2, Y);                                                  \
+    else OCNN_REQ_ROW(ks_next, (L) - 2, Y);                                                     \
+    /* the requests stay where they are (the scheduler would sink them to their first use    \
+       to save registers) */                                                                   \
+    __builtin_amdgcn_sched_barrier(0);                                                          \
+  } while (0)
+  // One layer phase: a quarter of the next k-step's weights on their way, the layer multiplied
+  // into the siblings it reaches, the weights parked in LDS.  No branches (a thread past the end
+  // of the piece copies its last unit once more; the last k-step copies the first weights of the
+  // next pass, or its own, and requests its own first layers again): one basic block per phase,
+  // so the waits the compiler places count exactly the requests that must have landed.
+#define OCNN_LAYER_PHASE(KS, L)                                                                 \
+  do {                                                                                          \
+    {                                                                                           \
+      /* a thread's units inside a piece: computed here every time, four registers are worth   \
+         more than eight additions */                                                          \
+      int tid = threadIdx.x;                                                                    \
+      asm volatile("" : "+v"(tid));                                                             \
+      _Pragma("unroll") for (int v = 0; v < kWVec; ++v)                                         \
+        wr[v] = __builtin_amdgcn_raw_buffer_load_b128(wbuf, min(v * 256 + tid, kWPiece - 1) * 16, \
+            wsrc + (L) * kWPiece * 16, 0);                                                      \
+    }                                                                                           \
+    __builtin_amdgcn_sched_barrier(0);                                                          \
+    /* work items of the layer: (dy, dz) x the sibling halves it reaches; the weights of      \
+       item t + 1 are read from LDS before the multiplications of item t are issued */          \
+    {                                                                                           \
+      constexpr int kBoth = ((L) == 1 || (L) == 2) ? 1 : 0;                                     \
+      constexpr int kItems = kBoth ? 18 : 9;                                                    \
+      union { u32x4 q; bf16x8 v; } av[2][MT];                                                   \
+      _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                         \
+        av[0][mt].q = wcur[(((L) == 3 ? 2 : (L)) * 9 * MT + mt) * 64 + lane];                   \
+      __builtin_amdgcn_sched_group_barrier(0x100, MT, 0);                                       \
+      _Pragma("unroll") for (int it = 0; it < kItems; ++it) {                                   \
+        /* issue order: the reads of the next item, then this item's multiplications */       \
+        __builtin_amdgcn_sched_group_barrier(0x100, MT, 0);                                     \
+        __builtin_amdgcn_sched_group_barrier(0x008, 4 * MT, 0);                                 \
+        if (it + 1 < kItems) {                                                                  \
+          const int nyz = kBoth ? (it + 1) >> 1 : it + 1;                                       \
+          const int nsi = kBoth ? (it + 1) & 1 : ((L) == 3 ? 1 : 0);                            \
+          _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                     \
+            av[(it + 1) & 1][mt].q = wcur[((((L) - nsi) * 9 + nyz) * MT + mt) * 64 + lane];     \
+        }                                                                                       \
+        const int yz = kBoth ? it >> 1 : it, si = kBoth ? it & 1 : ((L) == 3 ? 1 : 0);          \
+        const int dy = yz / 3, dz = yz % 3;                                                     \
+        _Pragma("unroll") for (int sj = 0; sj < 2; ++sj)                                        \
+        _Pragma("unroll") for (int sk = 0; sk < 2; ++sk) {                                      \
+          union { u32x4 q; bf16x8 v; } bv;                                                      \
+          bv.q = bl[(L) & 1][(dy + sj) * 4 + (dz + sk)];                                        \
+          _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                     \
+            acc[si * 4 + sj * 2 + sk][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(            \
+                av[it & 1][mt].v, bv.v, acc[si * 4 + sj * 2 + sk][mt], 0, 0, 0);                \
+        }                                                                                       \
+        if (it + 1 == kItems / 3) OCNN_REFILL(KS, L, 0);                                        \
+        if (it + 1 == 2 * kItems / 3) OCNN_REFILL(KS, L, 1);                                    \
+      }                                                                                         \
+      OCNN_REFILL(KS, L, 2);                                                                    \
+      OCNN_REFILL(KS, L, 3);                                                                    \
+    }                                                                                           \
+    _Pragma("unroll") for (int v = 0; v < kWVec; ++v)                                           \
+      wnext[(L) * kWPiece + min(v * 256 + (int)threadIdx.x, kWPiece - 1)] = wr[v];              \
+  } while (0)
+
+  int wbase = 0;   // LDS buffer of a pass's first k-step
+  for (; pass < npass; pass += gridDim.y) {   // passes may be dealt out over workgroups
+#pragma unroll
+    for (int y = 0; y < 4; ++y) { OCNN_REQ_ROW(0, 0, y); }
+#pragma unroll
+    for (int y = 0; y < 4; ++y) { OCNN_REQ_ROW(0, 1, y); }
+
+    // lane (n, kh) holds rows m0 + 32 mt + 8 (i / 4) + i % 4 of columns 8 (g0 + n) .. + 7
+    const int m0 = pass * MT * 32 + 4 * kh;
+    floatx16 acc[8][MT];
+#pragma unroll
+    for (int sb = 0; sb < 8; ++sb)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[sb][mt][i] = 0.0f;
+
+    const int wpass = pass * nks * kWUnits * 16;   // byte offsets into the packed weights
+    const int wfirst = (pass + (int)gridDim.y < npass ? pass + (int)gridDim.y : pass) * nks * kWUnits * 16;
+    for (int ks = 0; ks < nks; ++ks) {
+      __syncthreads();   // this k-step's weights are in LDS; the other buffer is free
+      const u32x4* wcur = sW[(wbase + ks) & 1];
+      u32x4* wnext = sW[(wbase + ks + 1) & 1];
+      const int ks_next = min(ks + 1, nks - 1);
+      const int wsrc = ks + 1 < nks ? wpass + (ks + 1) * kWUnits * 16 : wfirst;
+      OCNN_LAYER_PHASE(ks, 0);
+      OCNN_LAYER_PHASE(ks, 1);
+      OCNN_LAYER_PHASE(ks, 2);
+      OCNN_LAYER_PHASE(ks, 3);
+    }
+    wbase = (wbase + nks) & 1;
+
+    // one 16-byte store per output channel: the 8 columns of a group are contiguous
+    const int g = g0 + n;
+    uint16_t* orow = out + (int64_t)g * 8 + (int64_t)m0 * a.Hout;
+    // Straight-line code: the biases of my rows are fetched together, the ReLU is a maximum with
+    // 0 or -inf, the conversion is the hardware's (round to nearest even).
+    const float floor = a.relu ? 0.0f : -__builtin_inff();
+    const int m_left = g < n_groups ? a.M - m0 : 0;   // rows of mine that exist
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      float bias[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) bias[i] = 0.0f;
+      if (a.bias) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) bias[i] = a.bias[min(m0 + 32 * mt + 8 * (i / 4) + (i % 4), a.M - 1)];
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int dm = 32 * mt + 8 * (i / 4) + (i % 4);
+        uint32_t w[4];
+#pragma unroll
+        for (int sp = 0; sp < 4; ++sp)
+          w[sp] = pack_bf16x2(relu_floor(acc[2 * sp][mt][i] + bias[i], floor),
+                              relu_floor(acc[2 * sp + 1][mt][i] + bias[i], floor));
+        if (dm < m_left)
+          *reinterpret_cast<uint4*>(orow + (int64_t)dm * a.Hout) = make_uint4(w[0], w[1], w[2], w[3]);
+      }
+    }
+  }
+#undef OCNN_REQ_ROW
+#undef OCNN_REFILL
+#undef OCNN_LAYER_PHASE
+}
+
 // weights for the bf16 LDS kernel: [pass][slab][dx][dy*3+dz][mt][lane][8 channels]; the tap
 // index counts geometric offsets, so a deconvolution (which gathers through the mirrored
 // offset) reads weight tap 26 - k
@@ -1143,6 +1388,11 @@ __global__ void ichild_kernel(int* __restrict__ ichild, int n_nempty, const int*
 
 // Shape rules of OctreeBaseConv::reshape (octree/octree/octree_conv.cpp:48-104)
 // and the input-height check of pytorch/cpp/octree_conv.cpp:72-78.
+// The register-fed bf16 kernel keeps one workgroup per CU busy with 1024 columns each; below
+// this many such tiles the LDS kernel (256 columns per workgroup, three workgroups per CU) fills
+// the device better.  Measured crossover on 256 CUs: between 110 and 215 tiles.
+std::atomic<int> g_bf16_reg_min_tiles{192};
+
 struct ConvPlan {
   int top_depth, workspace_depth, top_h, btm_h, workspace_h;
   int child_h, ichild_h;
@@ -1398,8 +1648,17 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     dim3 tgrid((a.Hin + 1 + 127) / 128, (cpad + 63) / 64);
     transpose_rows_bf16_kernel<<<tgrid, 256, 0, s>>>(xt, (const uint16_t*)btm, a.Cin, a.Hin, cpad);
     OCNN_LAUNCH_OK("pack/transpose");
-    // the kernel walks geometric offsets in natural order (the packer mirrored the weights)
-    if (MT == 1)
+    // the kernels walk geometric offsets in natural order (the packer mirrored the weights)
+    const int r_tiles = ((a.N >> 3) + kRegTileGroups - 1) / kRegTileGroups;
+    const bool fits32 = ((int64_t)a.Hin + 1) * cpad * 2 < ((int64_t)1 << 31);   // the kernel addresses rows with 32-bit byte offsets
+    const bool use_reg = fits32 && r_tiles >= g_bf16_reg_min_tiles.load(std::memory_order_relaxed);
+    if (use_reg) {
+      const int r_grid = ((r_tiles + 7) / 8) * 8;
+      if (MT == 1)
+        conv_s1_bf16_reg_kernel<1><<<dim3(r_grid, pass_split(r_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, r_tiles, cpad / 8);
+      else
+        conv_s1_bf16_reg_kernel<2><<<dim3(r_grid, pass_split(r_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, r_tiles, cpad / 8);
+    } else if (MT == 1)
       conv_s1_bf16_lds_kernel<1><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad / 8);
     else
       conv_s1_bf16_lds_kernel<2><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad / 8);
@@ -1987,6 +2246,12 @@ int ocnn_octree_conv_static(void* top, const void* btm, int channel_in, int btm_
   if (e) return e;
   return run_conv(is_deconv ? 1 : 0, top, btm, channel_in, btm_h, weights, octree_dev, info, depth, num_output,
       kernel_size, stride, nempty, dtype, ptr, kBuiltinScratchBytes, as_stream(stream), bias, relu, true);
+}
+
+int ocnn_conv_bf16_tile_threshold(int tiles) {
+  const int old = g_bf16_reg_min_tiles.load();
+  g_bf16_reg_min_tiles.store(tiles > 0 ? tiles : (tiles == 0 ? 192 : 1));
+  return old;
 }
 
 int ocnn_conv_shape(const void* info, int depth, int channel_in, int num_output, const int* kernel_size,

@@ -239,6 +239,42 @@ def test_deconv_vs_oracle(oc, orc, tree, ks, stride, nempty):
     assert relerr(got16.float().cpu().numpy().reshape(exp.shape), exp) < TOL_BF16
 
 
+def test_bf16_register_kernel_small_levels(oc, orc, tree):
+  """The bf16 3x3x3 stride-1 kernel for large levels (operands straight into registers, 32
+  sibling groups x 8 siblings per wavefront), forced onto small levels whose group counts are
+  no multiple of its tile: against the oracle (2e-2), and bit for bit against the LDS kernel
+  that serves these sizes by default (same products, same order).  Conv and deconv, ragged
+  channel counts, more than one pass over the output channels, fused bias + ReLU."""
+  b, dev, host = tree["blob"], tree["dev"], tree["host"]
+  L = oc.lib.get()
+  rng = np.random.default_rng(11)
+  try:
+    for d, ci, co in ((5, 3, 32), (5, 20, 70), (4, 64, 64), (6, 16, 130), (3, 40, 8), (6, 64, 64)):
+      H = int(b.nnum[d])
+      x = rng.standard_normal((ci, H)).astype(np.float32)
+      w = (rng.standard_normal((co, ci * 27)) * 0.1).astype(np.float32)
+      wd = (rng.standard_normal((ci, co * 27)) * 0.1).astype(np.float32)
+      bias = rng.standard_normal(co).astype(np.float32)
+      xt = T(x).cuda().view(1, ci, H, 1).bfloat16()
+      res = {}
+      for name, thr in (("lds", 1 << 30), ("reg", -1)):
+        L.ocnn_conv_bf16_tile_threshold(thr)
+        res[name] = (oc.nn.octree_conv(xt, T(w).cuda().bfloat16(), dev, d, co, [3, 3, 3], 1, False),
+                     oc.nn.octree_deconv(xt, T(wd).cuda().bfloat16(), dev, d, co, [3, 3, 3], 1, False),
+                     oc.nn.octree_conv_fused(xt, T(w).cuda().bfloat16(), T(bias).cuda(), True, dev, d, co,
+                                             [3, 3, 3], 1, False))
+      for got_l, got_r in zip(res["lds"], res["reg"]):
+        assert torch.equal(got_l.view(torch.int16), got_r.view(torch.int16)), (d, ci, co)
+      exp = orc.octree_conv(x, w, host, d, co, [3, 3, 3], 1, False)
+      assert relerr(res["reg"][0].float().cpu().numpy().reshape(exp.shape), exp) < TOL_BF16
+      expd = orc.octree_deconv(x, wd, host, d, co, [3, 3, 3], 1, False)
+      assert relerr(res["reg"][1].float().cpu().numpy().reshape(expd.shape), expd) < TOL_BF16
+      expf = np.maximum(exp + bias[:, None], 0)
+      assert relerr(res["reg"][2].float().cpu().numpy().reshape(expf.shape), expf) < TOL_BF16
+  finally:
+    L.ocnn_conv_bf16_tile_threshold(0)
+
+
 def test_conv_wide_channels(oc, orc, tree):
   """Channel counts of the benchmark stacks, incl. more than one pass over the output tiles."""
   b, dev, host = tree["blob"], tree["dev"], tree["host"]
