@@ -252,6 +252,37 @@ int ocnn_octree_interp_backward_ws(float* grad_data, const float* grad_out, int 
     int method, const int* idx, const float* weight, void* workspace_dev, size_t workspace_bytes,
     ocnn_stream_t stream);
 
+/* ---- octree_gather_gpu / octree_gatherbk_gpu / octree_mask_gpu, octree/octree/octree_nn.h:204-218
+ * (kernels octree_nn.cu:756-818).
+ *   gather    top[c, h] = idx[h] != -1 ? btm[c, idx[h]] : 0   (the reference's pad_forward with 0)
+ *   gatherbk  btm zero-filled, then btm[c, idx[h]] += top[c, h]; idx may name a row many times.
+ *             With a workspace of ocnn_octree_gatherbk_workspace_bytes(channel, btm_h, top_h) bytes
+ *             (16-byte aligned) the rows are binned by target and every target sums its sources,
+ *             without floating-point atomics; without one (NULL) an atomic scatter-add as in the
+ *             reference.  fp32.
+ *   mask      out[i] = label[i % height] == mask ? 0 : in[i] for i < num */
+int ocnn_octree_gather(void* top, int top_h, int channel, const void* btm, int btm_h, const int* idx, int dtype,
+    ocnn_stream_t stream);
+size_t ocnn_octree_gatherbk_workspace_bytes(int channel, int btm_h, int top_h);
+int ocnn_octree_gatherbk(const float* top, int top_h, int channel, float* btm, int btm_h, const int* idx,
+    void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream);
+int ocnn_octree_mask(float* out, const float* in, const int* label, int height, int mask, int64_t num,
+    ocnn_stream_t stream);
+
+/* ---- trilinear stencils between two levels: bilinear_neigh_gpu / bilinear_xyz_gpu,
+ * octree/octree/octree_nn.h:170-177 (kernels octree_nn.cu:491-565; the 512-entry table of
+ * NeighHelper::get_bilinear_array, octree_nn.cpp:83-108, is internal).
+ *   bilinear_neigh  bidx[(8 child[i] + j) * 8 + k] = node of the level of `neigh` in corner k of
+ *                   the interpolation cell of child j of node i, for every non-empty node i
+ *                   (node_num = nodes of that level); -1 where there is none.  Corner order
+ *                   000, 001, 010, 100, 011, 101, 110, 111 of (x, y, z): weights 27, 9, 9, 9, 3, 3, 3, 1.
+ *   bilinear_xyz    xyz0[8 i + k] = packed coordinates (x, y, z, id in 16-bit fields) of those
+ *                   cells at level d0 for cell xyz1[i] of level d1 >= d0; fracs[3 i + c] = the
+ *                   weight of the nearer cell along axis c. */
+int ocnn_bilinear_neigh(int* bidx, const int* neigh, const int* child, int node_num, ocnn_stream_t stream);
+int ocnn_bilinear_xyz(uint64_t* xyz0, float* fracs, int d0, const uint64_t* xyz1, int d1, int num,
+    ocnn_stream_t stream);
+
 /* ---- file formats.  A `.octree` / `.points` file is the serialized blob itself
  * (Octree::read_octree / write_octree, octree/octree/octree.cpp:41-68; Points::read_points /
  * write_points, points.cpp:9-37).  Files written by a 32-bit-key build carry "_OCTREE_1.0_" and

@@ -29,6 +29,27 @@ __global__ void align_backward_kernel(const float* __restrict__ top, int top_h, 
   const bool ok = j >= 0 && j < top_h;
   for (int c = 0; c < channel; ++c) btm[(int64_t)c * btm_h + h] = ok ? top[(int64_t)c * top_h + j] : 0.0f;
 }
+// octree_mask (octree_nn.cu:805-818): the rows whose label equals `mask` become zero.
+// One thread per four consecutive rows of one channel where the row count allows.
+__global__ void mask_rows_kernel(float* __restrict__ out, const float* __restrict__ in,
+    const int* __restrict__ label, int height, int mask, int64_t num) {
+  const int h = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  const int64_t base = (int64_t)blockIdx.y * height + h;
+  if (h >= height || base >= num) return;
+  if ((height & 3) == 0 && base + 3 < num) {
+    const int4 l = *reinterpret_cast<const int4*>(label + h);
+    float4 v = *reinterpret_cast<const float4*>(in + base);
+    if (l.x == mask) v.x = 0.0f;
+    if (l.y == mask) v.y = 0.0f;
+    if (l.z == mask) v.z = 0.0f;
+    if (l.w == mask) v.w = 0.0f;
+    *reinterpret_cast<float4*>(out + base) = v;
+  } else {
+    for (int j = 0; j < 4 && h + j < height && base + j < num; ++j)
+      out[base + j] = label[h + j] == mask ? 0.0f : in[base + j];
+  }
+}
+
 __global__ void zero_kernel(float* __restrict__ p, int64_t n) {
   int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (i < n) p[i] = 0.0f;
@@ -240,7 +261,7 @@ __global__ void interp_fill_kernel(int2* __restrict__ pairs, int* __restrict__ c
 #pragma unroll
   for (int m = 0; m < K; ++m) {
     id[m] = idx[(int64_t)p * K + m];
-    w[m] = id[m] >= 0 ? weight[(int64_t)p * K + m] : 0.0f;
+    w[m] = id[m] >= 0 ? (weight ? weight[(int64_t)p * K + m] : 1.0f) : 0.0f;   // no weights: a plain scatter-add
     norm += w[m];
   }
   const float inv = normalise ? 1.0f / (norm + 1e-10f) : 1.0f;
@@ -309,7 +330,7 @@ __global__ void interp_scatter_kernel(float* __restrict__ grad_data, const float
   for (int m = 0; m < K; ++m) {
     id[m] = idx[(int64_t)p * K + m];
     const bool ok = id[m] >= 0 && id[m] < H;
-    w[m] = ok ? weight[(int64_t)p * K + m] : 0.0f;
+    w[m] = ok ? (weight ? weight[(int64_t)p * K + m] : 1.0f) : 0.0f;
     if (!ok) id[m] = -1;
     norm += w[m];
   }
@@ -337,6 +358,13 @@ struct InterpBackLayout {
   }
 };
 
+}  // namespace
+}  // namespace ocnn
+
+namespace ocnn {
+namespace {
+int scatter_add_rows(float* grad_data, const float* grad_out, int channel, int H, int n_pts, int method,
+    const int* idx, const float* weight, void* workspace_dev, size_t workspace_bytes, hipStream_t s);
 }  // namespace
 }  // namespace ocnn
 
@@ -422,10 +450,56 @@ int ocnn_octree_interp_backward(float* grad_data, const float* grad_out, int cha
 
 int ocnn_octree_interp_backward_ws(float* grad_data, const float* grad_out, int channel, int H, int n_pts, int method,
     const int* idx, const float* weight, void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream) {
-  OCNN_REQUIRE(grad_data && grad_out && idx && weight && channel > 0 && H >= 0 && n_pts >= 0, OCNN_E_BADARG,
+  OCNN_REQUIRE(weight, OCNN_E_BADARG, "null weights");
+  return scatter_add_rows(grad_data, grad_out, channel, H, n_pts, method, idx, weight, workspace_dev, workspace_bytes,
+      as_stream(stream));
+}
+
+// ---- octree_gather / octree_gatherbk / octree_mask (octree/octree/octree_nn.h:204-218) -------
+int ocnn_octree_gather(void* top, int top_h, int channel, const void* btm, int btm_h, const int* idx, int dtype,
+    ocnn_stream_t stream) {
+  // the reference's own definition: pad_forward with the value 0 (octree_nn.cu:770-773)
+  return ocnn_pad_forward(top, top_h, channel, btm, btm_h, idx, 0.0f, dtype, stream);
+}
+
+size_t ocnn_octree_gatherbk_workspace_bytes(int channel, int btm_h, int top_h) {
+  return ocnn_octree_interp_backward_workspace_bytes(channel, btm_h, top_h, 0);
+}
+
+int ocnn_octree_gatherbk(const float* top, int top_h, int channel, float* btm, int btm_h, const int* idx,
+    void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream) {
+  // btm[c, idx[h]] += top[c, h] over all h with idx[h] != -1, btm zero-filled first
+  // (octree_nn.cu:782-801).  With a workspace the rows are binned by target and every target sums
+  // its sources (no floating-point atomics); without one, or for few rows, an atomic scatter.
+  return scatter_add_rows(btm, top, channel, btm_h, top_h, 0, idx, nullptr, workspace_dev, workspace_bytes,
+      as_stream(stream));
+}
+
+int ocnn_octree_mask(float* out, const float* in, const int* label, int height, int mask, int64_t num,
+    ocnn_stream_t stream) {
+  OCNN_REQUIRE(out && in && label && height > 0 && num >= 0, OCNN_E_BADARG, "bad argument");
+  if (num > 0) {
+    const int64_t rows = (num + height - 1) / height;
+    OCNN_REQUIRE(rows <= 65535, OCNN_E_BADARG, "more than 65535 channels");
+    mask_rows_kernel<<<dim3(blocks_for((height + 3) / 4), (unsigned)rows), kBlock, 0, as_stream(stream)>>>(out, in, label,
+        height, mask, num);
+  }
+  OCNN_LAUNCH_OK("octree_mask");
+  return OCNN_OK;
+}
+
+}  // extern "C"
+
+namespace ocnn {
+namespace {
+
+// grad_data[c, idx[p, m]] += w[p, m] * grad_out[c, p] (grad_data zero-filled first): the adjoint
+// of the interpolation and, with unit weights (weight == nullptr), of octree_gather.
+int scatter_add_rows(float* grad_data, const float* grad_out, int channel, int H, int n_pts, int method,
+    const int* idx, const float* weight, void* workspace_dev, size_t workspace_bytes, hipStream_t s) {
+  OCNN_REQUIRE(grad_data && grad_out && idx && channel > 0 && H >= 0 && n_pts >= 0, OCNN_E_BADARG,
       "bad argument");
   OCNN_REQUIRE(method == 0 || method == 1, OCNN_E_BADARG, "method %d", method);
-  hipStream_t s = as_stream(stream);
   const int Kc = method == 0 ? 1 : 8;
   const size_t need = ocnn_octree_interp_backward_workspace_bytes(channel, H, n_pts, method);
   if (workspace_dev && H > 0 && n_pts > 0 && need > 0 && workspace_bytes >= need &&
@@ -464,4 +538,5 @@ int ocnn_octree_interp_backward_ws(float* grad_data, const float* grad_out, int 
   return OCNN_OK;
 }
 
-}  // extern "C"
+}  // namespace
+}  // namespace ocnn

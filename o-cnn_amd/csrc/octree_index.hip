@@ -53,6 +53,61 @@ __global__ void key2idx_kernel(int* __restrict__ idx, const uint64_t* __restrict
   if (i < num) idx[i] = (int)(key[i] >> 48);
 }
 
+// ---- trilinear stencils between two levels (bilinear_neigh / bilinear_xyz) --------------------
+// The stencil of a child: the node of the parent level in each of the 8 cells around the
+// child's centre, nearest first (corner order 000, 001, 010, 100, 011, 101, 110, 111 of
+// (x, y, z): weights 27, 9, 9, 9, 3, 3, 3, 1).  Seen from the 4x4x4 neighbour block of the
+// parent's sibling group, child j of sibling i reads, per axis, slot (i + 1) and the slot one
+// step towards the child's side; the reference tabulates that in 512 entries
+// (NeighHelper, octree/octree/octree_nn.cpp:83-108), here it is computed.
+__device__ inline int stencil_slot(int sib, int child, int corner) {
+  // corner bits per axis in the order above: x = {0,0,0,1,0,1,1,1}, y = {0,0,1,0,1,0,1,1}, z = {0,1,0,0,1,1,0,1}
+  const int cx = (0xE8 >> corner) & 1, cy = (0xD4 >> corner) & 1, cz = (0xB2 >> corner) & 1;
+  const int x = ((sib >> 2) & 1) + 1 + cx * (2 * ((child >> 2) & 1) - 1);
+  const int y = ((sib >> 1) & 1) + 1 + cy * (2 * ((child >> 1) & 1) - 1);
+  const int z = (sib & 1) + 1 + cz * (2 * (child & 1) - 1);
+  return (x << 4) | (y << 2) | z;
+}
+
+// One wavefront lane per (child, corner) of a non-empty parent: 64 table reads inside the
+// parent group's 256-byte block, one 256-byte row of output per parent
+// (bilinear_neigh_cpu, octree_nn.cpp:476-492).
+__global__ void bilinear_neigh_kernel(int* __restrict__ bidx, const int* __restrict__ neigh,
+    const int* __restrict__ child, int node_num) {
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int i = (int)(id >> 6), lane = (int)(id & 63);
+  if (i >= node_num) return;
+  const int cld = child[i];
+  if (cld < 0) return;
+  bidx[((int64_t)cld << 6) + lane] = neigh[((int64_t)(i >> 3) << 6) + stencil_slot(i & 7, lane >> 3, lane & 7)];
+}
+
+// bilinear_xyz_cpu, octree_nn.cpp:494-530: cells of level d0 around the centre of a cell of
+// level d1 (packed 16-bit coordinates), and per axis the weight of the nearer cell.  Float
+// steps as in the reference (the scale is a power of two: the quotient is exact).
+__global__ void bilinear_xyz_kernel(uint64_t* __restrict__ xyz0, float* __restrict__ fracs,
+    const uint64_t* __restrict__ xyz1, float scale, int num) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= num) return;
+  const uint64_t v = xyz1[i];
+  int bnd[2][3];
+#pragma unroll
+  for (int c = 0; c < 3; ++c) {
+    const float pt = ((float)(uint32_t)((v >> (16 * c)) & 0xffff) + 0.5f) / scale - 0.5f;
+    const int b = (int)pt;
+    float frac = pt - (float)b;
+    if (frac > 0.5f) { bnd[0][c] = b + 1; bnd[1][c] = b; }
+    else { frac = 1 - frac; bnd[0][c] = b; bnd[1][c] = b + 1; }
+    fracs[3 * (int64_t)i + c] = frac;
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int cx = (0xE8 >> j) & 1, cy = (0xD4 >> j) & 1, cz = (0xB2 >> j) & 1;
+    xyz0[(int64_t)i * 8 + j] = (uint64_t)(uint16_t)bnd[cx][0] | ((uint64_t)(uint16_t)bnd[cy][1] << 16) |
+        ((uint64_t)(uint16_t)bnd[cz][2] << 32) | (v & 0xffff000000000000ull);
+  }
+}
+
 __global__ void sequence_kernel(int* __restrict__ p, int num) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < num) p[i] = i;
@@ -139,6 +194,24 @@ int ocnn_generate_label(int* label, int* count_dev, const int* btm, int btm_h, i
   LabelOut out{label};
   hipError_t e = flag_scan(pred, out, (int64_t)btm_h, (int*)scratch_dev, count_dev, as_stream(stream));
   OCNN_REQUIRE(e == hipSuccess, OCNN_E_HIP, "generate_label: %s", hipGetErrorString(e));
+  return OCNN_OK;
+}
+
+int ocnn_bilinear_neigh(int* bidx, const int* neigh, const int* child, int node_num, ocnn_stream_t stream) {
+  OCNN_REQUIRE(bidx && neigh && child && node_num >= 0, OCNN_E_BADARG, "bad argument");
+  if (node_num > 0)
+    bilinear_neigh_kernel<<<blocks_for((int64_t)node_num * 64), kBlock, 0, as_stream(stream)>>>(bidx, neigh, child, node_num);
+  OCNN_LAUNCH_OK("bilinear_neigh");
+  return OCNN_OK;
+}
+
+int ocnn_bilinear_xyz(uint64_t* xyz0, float* fracs, int d0, const uint64_t* xyz1, int d1, int num,
+    ocnn_stream_t stream) {
+  OCNN_REQUIRE(xyz0 && fracs && xyz1 && num >= 0, OCNN_E_BADARG, "bad argument");
+  OCNN_REQUIRE(d0 >= 0 && d1 >= d0 && d1 - d0 < 31, OCNN_E_BADARG, "levels %d -> %d", d1, d0);
+  if (num > 0)
+    bilinear_xyz_kernel<<<blocks_for(num), kBlock, 0, as_stream(stream)>>>(xyz0, fracs, xyz1, (float)(1 << (d1 - d0)), num);
+  OCNN_LAUNCH_OK("bilinear_xyz");
   return OCNN_OK;
 }
 

@@ -28,6 +28,7 @@ __all__ = [
     "octree_pad", "octree_depad", "octree_max_pool", "octree_max_unpool", "octree_mask_pool",
     "octree_encode_key", "octree_decode_key", "octree_xyz2key", "octree_key2xyz",
     "octree_search_key", "octree_new", "octree_grow", "octree_update", "points_new",
+    "octree_gather", "octree_gatherbk", "octree_mask", "octree_bilinear_neigh", "octree_bilinear_xyz",
     "octree_info", "octree_scan", "octree_dropout", "octree_drop", "octree_samples",
 ]
 
@@ -931,6 +932,74 @@ def octree_search_key(key, octree, depth, key_is_xyz, nempty):
   out = torch.empty(n_query, dtype=torch.int32, device=octree.device)
   _lib.call("ocnn_search_key", _ptr(out), _ptr(des), des_h, _ptr(key), n_query, _stream())
   return out
+
+
+# ---- row gathers and trilinear stencils ---------------------------------------------------------
+def octree_gather(data, index):
+  """octree_gather_gpu (octree/octree/octree_nn.h:204-207): data [1,C,H,1], index int32 [H'] ->
+  [1,C,H',1] with row h = data row index[h], or zero where index[h] is -1."""
+  data, index = data.contiguous(), _to_dev(index.contiguous().int())
+  out = torch.empty((1, data.size(1), index.numel(), 1), dtype=data.dtype, device=data.device)
+  _lib.call("ocnn_octree_gather", _ptr(out), index.numel(), data.size(1), _ptr(data), data.size(2), _ptr(index),
+            _dtype_code(data), _stream())
+  return out
+
+
+def octree_gatherbk(grad, index, height):
+  """octree_gatherbk_gpu (octree_nn.h:208-211), the adjoint of octree_gather: grad [1,C,H',1] is
+  added into [1,C,height,1] at the rows `index` names (a row may be named many times)."""
+  grad, index = grad.contiguous(), _to_dev(index.contiguous().int())
+  if grad.dtype != torch.float32:
+    raise TypeError("octree_gatherbk is fp32")
+  channel, top_h = grad.size(1), grad.size(2)
+  out = torch.empty((1, channel, height, 1), dtype=grad.dtype, device=grad.device)
+  ws_bytes = _lib.get().ocnn_octree_gatherbk_workspace_bytes(channel, height, top_h)
+  ws = _workspace(ws_bytes + 256, "gather") if ws_bytes else None
+  base = ((ws.data_ptr() + 255) & ~255) if ws is not None else 0
+  _lib.call("ocnn_octree_gatherbk", _ptr(grad), top_h, channel, _ptr(out), height, _ptr(index), C.c_void_p(base),
+            C.c_size_t(ws_bytes), _stream())
+  return out
+
+
+def octree_mask(data, label, mask):
+  """octree_mask_gpu (octree_nn.h:217-218): the rows of data [1,C,H,1] whose label equals `mask`
+  become zero."""
+  data, label = data.contiguous(), _to_dev(label.contiguous().int())
+  if data.dtype != torch.float32:
+    raise TypeError("octree_mask is fp32")
+  if label.numel() != data.size(2):
+    raise OcnnError(-3, "octree_mask: %d labels for %d rows" % (label.numel(), data.size(2)))
+  out = torch.empty_like(data)
+  _lib.call("ocnn_octree_mask", _ptr(out), _ptr(data), _ptr(label), data.size(2), int(mask), C.c_int64(data.numel()),
+            _stream())
+  return out
+
+
+def octree_bilinear_neigh(octree, depth):
+  """bilinear_neigh_gpu (octree_nn.h:170-173): int32 [nnum(depth + 1), 8], for every node of
+  level depth + 1 the nodes of level `depth` in the 8 cells around its centre, nearest first
+  (weights 27, 9, 9, 9, 3, 3, 3, 1 of 64), -1 where there is none."""
+  octree = _to_dev(octree)
+  info = octree_info(octree)
+  if not 1 <= depth < info.depth:
+    raise ValueError("depth %d outside [1, %d)" % (depth, info.depth))
+  out = torch.empty((info.nnum(depth + 1), 8), dtype=torch.int32, device=octree.device)
+  neigh = _prop_view(octree, info, NEIGH, depth, info.nnum(depth) * 8, torch.int32)
+  child = _prop_view(octree, info, CHILD, depth, info.nnum(depth), torch.int32)
+  _lib.call("ocnn_bilinear_neigh", _ptr(out), _ptr(neigh), _ptr(child), info.nnum(depth), _stream())
+  return out
+
+
+def octree_bilinear_xyz(xyz, depth_from, depth_to):
+  """bilinear_xyz_gpu (octree_nn.h:174-177): packed coordinates int64 [N] of cells of level
+  `depth_from` -> (int64 [N, 8] cells of the coarser level `depth_to` around each centre,
+  nearest first; float32 [N, 3] weight of the nearer cell per axis)."""
+  xyz = _to_dev(xyz.contiguous())
+  n = xyz.numel()
+  cells = torch.empty((n, 8), dtype=torch.int64, device=xyz.device)
+  fracs = torch.empty((n, 3), dtype=torch.float32, device=xyz.device)
+  _lib.call("ocnn_bilinear_xyz", _ptr(cells), _ptr(fracs), depth_to, _ptr(xyz), depth_from, n, _stream())
+  return cells, fracs
 
 
 # ---- feature transfer ---------------------------------------------------------------------------

@@ -48,74 +48,80 @@ class NormalizePoints:
     return F.normalize_points(points, radius, center)
 
 
+class Distortion(tuple):
+  """(rotation angles in radians, per-axis scale, per-axis shift) of one augmentation."""
+  identity = None
+
+  def __new__(cls, rotation, scale, shift):
+    return super().__new__(cls, (list(rotation), list(scale), list(shift)))
+
+
+Distortion.identity = Distortion([0.0] * 3, [1.0] * 3, [0.0] * 3)
+
+
 def draw_distortion(angle, scale, jitter, angle_interval, uniform_scale):
-  """The random part of TransformPoints (transforms.py:80-98), in the reference's order of
-  draws: per axis a whole number of `angle_interval` steps within +-angle (radians returned),
-  then three scales in [1 - scale, 1 + scale] (the first one three times if uniform), then three
-  jitters in [-jitter, jitter]."""
-  rnd_angle = [0.0, 0.0, 0.0]
-  for i in range(3):
-    steps = angle[i] // angle_interval[i]
-    rnd_angle[i] = int(np.random.randint(low=-steps, high=steps + 1, dtype=np.int32)) * angle_interval[i] * _DEG
-  rnd_scale = np.random.uniform(low=1 - scale, high=1 + scale, size=(3)).tolist()
-  if uniform_scale:
-    rnd_scale = [rnd_scale[0]] * 3
-  rnd_jitter = np.random.uniform(low=-jitter, high=jitter, size=(3)).tolist()
-  return rnd_angle, rnd_scale, rnd_jitter
+  """One random augmentation.  It consumes numpy's global generator exactly as the reference
+  does (transforms.py:80-98), so a seeded run reproduces the reference's clouds: one int32
+  `randint` per axis (a whole number of `angle_interval` steps within +-angle degrees), one
+  `uniform` of three scales in [1 - scale, 1 + scale] (only the first is used when the scale is
+  uniform), one `uniform` of three shifts in [-jitter, jitter]."""
+  def steps(axis):
+    reach = angle[axis] // angle_interval[axis]
+    return int(np.random.randint(low=-reach, high=reach + 1, dtype=np.int32))
+  rotation = [steps(axis) * angle_interval[axis] * _DEG for axis in range(3)]
+  scales = np.random.uniform(low=1 - scale, high=1 + scale, size=3).tolist()
+  shifts = np.random.uniform(low=-jitter, high=jitter, size=3).tolist()
+  return Distortion(rotation, scales[:1] * 3 if uniform_scale else scales, shifts)
 
 
 class TransformPoints:
-  """transforms.py:61-108: the augmentation of a cloud that lies in [-1, 1], and the clip back
-  into that box.  Returns (points, inbox_mask)."""
+  """transforms.py:61-108: the augmentation of a cloud that lies in [-1, 1]^3 and the clip back
+  into that box.  Returns (points, inbox_mask).  `drawn` fixes the augmentation."""
 
   def __init__(self, distort, angle=(0, 180, 0), scale=0.25, jitter=0.25, offset=0.0,
                angle_interval=(1, 1, 1), uniform_scale=False, normal_axis="", **kwargs):
-    self.distort = distort
-    self.angle, self.scale, self.jitter, self.offset = list(angle), scale, jitter, offset
-    self.angle_interval, self.uniform_scale, self.normal_axis = list(angle_interval), uniform_scale, normal_axis
+    self.distort, self.offset, self.normal_axis = distort, offset, normal_axis
+    self.ranges = (list(angle), scale, jitter, list(angle_interval), uniform_scale)
 
   def __call__(self, points, drawn=None):
     if drawn is None:
-      drawn = (draw_distortion(self.angle, self.scale, self.jitter, self.angle_interval, self.uniform_scale)
-               if self.distort else ([0.0] * 3, [1.0] * 3, [0.0] * 3))
-    rnd_angle, rnd_scale, rnd_jitter = drawn
-    points = F.transform_points(points, rnd_angle, rnd_scale, rnd_jitter, self.offset, self.normal_axis)
-    return tuple(F.clip_points(points, [-1.0] * 3, [1.0] * 3))
+      drawn = draw_distortion(*self.ranges) if self.distort else Distortion.identity
+    moved = F.transform_points(points, *drawn, self.offset, self.normal_axis)
+    return tuple(F.clip_points(moved, [-1.0] * 3, [1.0] * 3))
 
 
 class TransformCompose:
-  """transforms.py:111-130: normalise -> transform + clip -> octree.  With `octree=False` the
+  """transforms.py:111-130: normalise -> transform + clip -> octree.  With `octree=False` a
   sample keeps its points only and `collate_octrees(..., points2octree=...)` builds the whole
-  batch at once."""
+  batch in one pass."""
 
   def __init__(self, flags, octree=True):
-    self.flags = flags
+    self.flags, self.octree = flags, octree
     self.normalize_points = NormalizePoints(**flags)
     self.transform_points = TransformPoints(**flags)
     self.points2octree = Points2Octree(**flags)
-    self.octree = octree
 
   def __call__(self, points, idx=0):
-    points = self.normalize_points(points)
-    points, inbox_mask = self.transform_points(points)
-    out = {"points": points, "inbox_mask": inbox_mask}
+    points, inbox_mask = self.transform_points(self.normalize_points(points))
+    sample = {"points": points, "inbox_mask": inbox_mask}
     if self.octree:
-      out["octree"] = self.points2octree(points)
-    return out
+      sample["octree"] = self.points2octree(points)
+    return sample
 
 
 def collate_octrees(batch, points2octree=None):
-  """transforms.py:133-148: lists per key, octrees merged with octree_batch, labels as a tensor.
-  If the samples carry no octree and `points2octree` (a Points2Octree) is given, the merged
-  octree is built from the samples' points in one pass."""
-  assert type(batch) == list
-  outputs = {}
-  for key in batch[0].keys():
-    outputs[key] = [b[key] for b in batch]
+  """transforms.py:133-148: a list of samples -> one dict of lists; every entry whose key names
+  an octree is merged with octree_batch, labels additionally become the tensor `label`.  If the
+  samples carry no octree and `points2octree` (a Points2Octree) is given, the merged octree is
+  built from the samples' points in one pass."""
+  if not isinstance(batch, list):
+    raise TypeError("collate_octrees takes the list of samples of one batch")
+  merged = {key: [sample[key] for sample in batch] for key in batch[0]}
+  for key in list(merged):
     if "octree" in key:
-      outputs[key] = F.octree_batch(outputs[key])
+      merged[key] = F.octree_batch(merged[key])
     if "label" in key:
-      outputs["label"] = torch.tensor(outputs[key])
-  if points2octree is not None and "octree" not in outputs:
-    outputs["octree"] = points2octree.batch(outputs["points"])
-  return outputs
+      merged["label"] = torch.tensor(merged[key])
+  if points2octree is not None and "octree" not in merged:
+    merged["octree"] = points2octree.batch(merged["points"])
+  return merged

@@ -348,6 +348,45 @@ class Checker:
     self.fn("pad_backward")(_p(X), Hx, Cc, _p(Y), Hy, _p(label))
     return X
 
+  def octree_gather(self, btm, idx):
+    btm, idx = _f32(btm), _i32(idx)
+    Cc, Hb = btm.shape
+    top = np.empty((Cc, idx.size), np.float32)
+    self.fn("octree_gather")(_p(top), idx.size, Cc, _p(btm), Hb, _p(idx))
+    return top
+
+  def octree_gatherbk(self, top, idx, btm_h):
+    top, idx = _f32(top), _i32(idx)
+    Cc, Ht = top.shape
+    btm = np.empty((Cc, btm_h), np.float32)
+    self.fn("octree_gatherbk")(_p(top), Ht, Cc, _p(btm), btm_h, _p(idx))
+    return btm
+
+  def octree_mask(self, data, label, mask):
+    data, label = _f32(data), _i32(label)
+    out = np.empty_like(data)
+    self.fn("octree_mask")(_p(out), _p(data), _p(label), label.size, int(mask), data.size)
+    return out
+
+  # ---- trilinear stencils ------------------------------------------------------
+  def get_bilinear(self):
+    t = np.zeros(512, np.int32)
+    self.fn("get_bilinear")(_p(t))
+    return t
+
+  def bilinear_neigh(self, neigh, child, n_child_nodes):
+    neigh, child = _i32(neigh), _i32(child)
+    bidx = np.full(n_child_nodes * 8, -7, np.int32)
+    self.fn("bilinear_neigh")(_p(bidx), _p(neigh), _p(child), child.size)
+    return bidx.reshape(-1, 8)
+
+  def bilinear_xyz(self, xyz1, d0, d1):
+    xyz1 = _u64(xyz1)
+    xyz0 = np.zeros(xyz1.size * 8, np.uint64)
+    fracs = np.zeros(xyz1.size * 3, np.float32)
+    self.fn("bilinear_xyz")(_p(xyz0), _p(fracs), d0, _p(xyz1), d1, xyz1.size)
+    return xyz0.reshape(-1, 8), fracs.reshape(-1, 3)
+
   # ---- keys ------------------------------------------------------------------
   def generate_key_child(self, key, child, n_out):
     key, child = _u64(key), _i32(child)

@@ -318,6 +318,80 @@ void orc_pad_backward(float* X, int Hx, int C, const float* Y, int Hy, const int
     for (int h = 0; h < Hy; ++h)
       if (label[h] != -1) X[(int64_t)c * Hx + label[h]] = Y[(int64_t)c * Hy + h];
 }
+/* octree_gather / octree_gatherbk / octree_mask: GPU-only in the reference
+ * (octree_nn.cu:756-830, declarations octree_nn.h:204-218).  gather is pad_forward with value 0
+ * (octree_nn.cu:770-773); gatherbk zero-fills and scatter-adds, its index may repeat
+ * (:782-801); mask zeroes the rows whose label equals `mask` (:805-818). */
+void orc_octree_gather(float* top, int top_h, int channel, const float* btm, int btm_h, const int* idx) {
+  orc_pad_forward(top, top_h, channel, btm, btm_h, idx, 0.0f);
+}
+void orc_octree_gatherbk(const float* top, int top_h, int channel, float* btm, int btm_h, const int* idx) {
+  for (int64_t i = 0; i < (int64_t)channel * btm_h; ++i) btm[i] = 0.0f;
+  for (int c = 0; c < channel; ++c)
+    for (int h = 0; h < top_h; ++h)
+      if (idx[h] != -1) btm[(int64_t)c * btm_h + idx[h]] += top[(int64_t)c * top_h + h];
+}
+void orc_octree_mask(float* out, const float* in, const int* label, int height, int mask, int num) {
+  for (int i = 0; i < num; ++i) out[i] = label[i % height] == mask ? 0.0f : in[i];
+}
+
+/* Trilinear stencils between two levels.  Table: NeighHelper (octree_nn.cpp:83-108): for a node
+ * with sibling index i, its child j and corner k, the slot (x << 4 | y << 2 | z) of the
+ * parent-level node that corner k of the interpolation cell of that child falls into;
+ * corner order 000, 001, 010, 100, 011, 101, 110, 111 of (x, y, z) = weights 27, 9, 9, 9, 3, 3, 3, 1. */
+static const int kBilinearCorner[8][3] = {
+  {0, 0, 0}, {0, 0, 1}, {0, 1, 0}, {1, 0, 0}, {0, 1, 1}, {1, 0, 1}, {1, 1, 0}, {1, 1, 1}};
+void orc_get_bilinear(int* table) {
+  for (int i = 0; i < 8; ++i) {
+    int z0 = i % 2, y0 = (i / 2) % 2, x0 = i / 4;
+    for (int j = 0; j < 8; ++j) {
+      int z1 = j % 2, y1 = (j / 2) % 2, x1 = j / 4;
+      for (int k = 0; k < 8; ++k) {
+        int x2 = x0 + 1 + kBilinearCorner[k][0] * (2 * x1 - 1);
+        int y2 = y0 + 1 + kBilinearCorner[k][1] * (2 * y1 - 1);
+        int z2 = z0 + 1 + kBilinearCorner[k][2] * (2 * z1 - 1);
+        table[(i << 6) | (j << 3) | k] = (x2 << 4) | (y2 << 2) | z2;
+      }
+    }
+  }
+}
+/* bilinear_neigh_cpu, octree_nn.cpp:476-492: bidx[(8 child[i] + j) * 8 + k] for the children of
+ * every non-empty node i of the level; entries of other rows are left as they are. */
+void orc_bilinear_neigh(int* bidx, const int* neigh, const int* child, int node_num) {
+  int table[512];
+  orc_get_bilinear(table);
+  for (int i = 0; i < node_num; ++i) {
+    if (child[i] < 0) continue;
+    const int* block = neigh + ((int64_t)(i >> 3) << 6);
+    for (int j = 0; j < 8; ++j)
+      for (int k = 0; k < 8; ++k)
+        bidx[((int64_t)child[i] * 8 + j) * 8 + k] = block[table[((i % 8) << 6) | (j << 3) | k]];
+  }
+}
+/* bilinear_xyz_cpu, octree_nn.cpp:494-530 (64-bit keys: four 16-bit fields x, y, z, id): the 8
+ * cells of level d0 around the centre of a cell of level d1, nearest first, and the weights of
+ * the nearest one per axis. */
+void orc_bilinear_xyz(uint64_t* xyz0, float* fracs, int d0, const uint64_t* xyz1, int d1, int num) {
+  const float scale = (float)(1 << (d1 - d0));
+  for (int i = 0; i < num; ++i) {
+    const uint16_t* in = (const uint16_t*)(xyz1 + i);
+    int bnd[2][3];
+    for (int c = 0; c < 3; ++c) {
+      float pt = ((float)in[c] + 0.5f) / scale - 0.5f;
+      int b = (int)pt;
+      float frac = pt - (float)b;
+      if (frac > 0.5f) { bnd[0][c] = b + 1; bnd[1][c] = b; }
+      else { frac = 1 - frac; bnd[0][c] = b; bnd[1][c] = b + 1; }
+      fracs[3 * (int64_t)i + c] = frac;
+    }
+    for (int j = 0; j < 8; ++j) {
+      uint16_t* out = (uint16_t*)(xyz0 + (int64_t)i * 8 + j);
+      for (int c = 0; c < 3; ++c) out[c] = (uint16_t)bnd[kBilinearCorner[j][c]][c];
+      out[3] = in[3];
+    }
+  }
+}
+
 static void pad_backward_int(int* X, const int* Y, int Hy, const int* label) {
   for (int h = 0; h < Hy; ++h) if (label[h] != -1) X[label[h]] = Y[h];
 }

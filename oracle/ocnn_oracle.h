@@ -27,6 +27,12 @@
  *   new/grow/update ..... MD5 of the rebuilt octree_2 quoted in
  *                         pytorch/test/test_octree_grow.py
  *   search_key .......... literal vectors of pytorch/test/test_octree_key.py
+ *   bilinear neigh / xyz  compiled reference; the reference's own consistency test
+ *                         (octree/test/test_octree_nn.cpp:23-84: corner weights 27,9,9,9,3,3,3,1
+ *                         from the key geometry, and neigh stencil == xyz stencil looked up by key)
+ *   gather / gatherbk / mask  (GPU-only in the reference) gather == pad_forward with 0 (pinned
+ *                         above); gatherbk by brute force with repeated indices and the adjoint
+ *                         identity <gather x, y> == <x, gatherbk y>; mask by its closed form
  *   adaptive build ...... (all-depth signals, error metrics, extrapolation, trimming:
  *                         octree/octree/octree.cpp:454-806, 958-1178) every literal of
  *                         octree/test/test_octree.cpp:196-331 (TestOctreeTrim), compiled
@@ -88,6 +94,12 @@ void orc_pad_backward(float* X, int Hx, int C, const float* Y, int Hy, const int
 void orc_generate_key_child(uint64_t* key_child, const uint64_t* key, const int* child, int node_num);
 void orc_generate_key_full(uint64_t* key, int depth, int batch);
 int  orc_generate_label(int* label, const int* btm, int btm_h, int mask);
+void orc_octree_gather(float* top, int top_h, int channel, const float* btm, int btm_h, const int* idx);
+void orc_octree_gatherbk(const float* top, int top_h, int channel, float* btm, int btm_h, const int* idx);
+void orc_octree_mask(float* out, const float* in, const int* label, int height, int mask, int num);
+void orc_get_bilinear(int* table512);
+void orc_bilinear_neigh(int* bidx, const int* neigh, const int* child, int node_num);
+void orc_bilinear_xyz(uint64_t* xyz0, float* fracs, int d0, const uint64_t* xyz1, int d1, int num);
 void orc_search_key(int* idx, const uint64_t* key, int n_key, const uint64_t* query, int n_query);
 void orc_xyz2key(uint64_t* key, const uint64_t* xyz, int num, int depth);
 void orc_key2xyz(uint64_t* xyz, const uint64_t* key, int num, int depth);

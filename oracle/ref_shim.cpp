@@ -201,6 +201,16 @@ void ref_search_key(int* idx, const uint64_t* key, int n_key,
   search_key_cpu<uintk>(idx, (const uintk*)key, n_key, (const uintk*)query,
       n_query);
 }
+void ref_get_bilinear(int* table512) {
+  const vector<int>& t = NeighHelper::get_bilinear_array();
+  for (int i = 0; i < 512; ++i) table512[i] = t[i];
+}
+void ref_bilinear_neigh(int* bidx, const int* neigh, const int* child, int node_num) {
+  bilinear_neigh_cpu(bidx, neigh, child, node_num, NeighHelper::get_bilinear_array().data());
+}
+void ref_bilinear_xyz(uint64_t* xyz0, float* fracs, int d0, const uint64_t* xyz1, int d1, int num) {
+  bilinear_xyz_cpu((uintk*)xyz0, fracs, d0, (const uintk*)xyz1, d1, num);
+}
 void ref_xyz2key(uint64_t* key, const uint64_t* xyz, int num, int depth) {
   xyz2key_cpu<uintk>((uintk*)key, (const uintk*)xyz, num, depth);
 }

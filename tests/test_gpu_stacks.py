@@ -148,14 +148,12 @@ def test_unet_trunk(oc, orc, tree, nempty):
   assert relerr(got.cpu().numpy().reshape(x.shape), x) < 1e-4
 
 
-def test_thin_modules(oc, orc, tree):
-  """Octree2Col / Col2Octree, OctreeTile, FullOctree2Voxel, FullOctreeGlobalPool, octree_feature
-  (pytorch/ocnn/octree2col.py:40-55, modules.py:193-206, 333-337, octree2voxel.py, octree_pool.py:106-115)
-  against their definitions written out with numpy."""
+def test_column_modules(oc, orc, tree):
+  """Octree2Col / Col2Octree (pytorch/ocnn/octree2col.py:40-81) against the oracle, with gradients."""
   host, dev, b = tree
   rng = np.random.default_rng(8)
   d = 5
-  H, Hn = int(b.nnum[d]), int(b.nnum_nempty[d])
+  H = int(b.nnum[d])
   x = rng.standard_normal((1, 3, H, 1)).astype(np.float32)
   xd = T(x).cuda().requires_grad_(True)
   col = oc.Octree2Col(d, [3, 3, 3], 1)(xd, dev)
@@ -166,23 +164,6 @@ def test_thin_modules(oc, orc, tree):
   assert relerr(back.detach().cpu().numpy().reshape(3, H), expb.reshape(3, H)) < 1e-6
   back.sum().backward()
   assert xd.grad is not None and xd.grad.shape == xd.shape
-  # tile: the feature of the k-th non-empty node goes to the nodes 8k .. 8k + 7 of the next level
-  tile = oc.OctreeTile(d)(T(x).cuda(), dev).cpu().numpy()
-  child = b.prop("child", d)
-  assert tile.shape == (1, 3, int(b.nnum[d + 1]), 1)
-  assert np.array_equal(tile.reshape(3, Hn, 8), np.repeat(x.reshape(3, H)[:, child >= 0][:, :, None], 8, axis=2))
-  # full level 2 of a batch of two: [1, C, 2 * 64, 1] -> [2, C, 64], mean over the level
-  f = rng.standard_normal((1, 4, 2 * 64, 1)).astype(np.float32)
-  vox = oc.FullOctree2Voxel(2)(T(f).cuda()).cpu().numpy()
-  assert np.array_equal(vox, f.reshape(4, 2, 64).transpose(1, 0, 2))
-  pooled = oc.FullOctreeGlobalPool(2)(T(f).cuda()).cpu().numpy()
-  assert np.allclose(pooled, f.reshape(4, 2, 64).transpose(1, 0, 2).mean(axis=2), atol=1e-6)
-  # the stored signal of the finest level, all nodes and non-empty nodes
-  feat = b.prop("feature", 6)
-  got = oc.octree_feature(dev, 6).cpu().numpy()
-  assert np.array_equal(got.reshape(feat.shape), feat)
-  gne = oc.octree_feature(dev, 6, nempty=True).cpu().numpy()
-  assert np.array_equal(gne.reshape(feat.shape[0], -1), feat[:, b.prop("child", 6) >= 0])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
