@@ -19,18 +19,20 @@
 //          ONE scan for every level at once: element i starts a new node at level
 //            d iff it differs from element i-1 above bit 3*(depth-d); the
 //            per-level counts travel as 16-bit fields of four 64-bit words
-//          [one copy of the level sizes to the host: the caller must size the blob]
+//          [the level sizes reach the host through pinned memory that the scan's last
+//           workgroup writes and the host polls: the caller must size the blob]
 //   emit:  one launch writes header, keys, children, split labels and full-layer
 //            neighbour tables of every level (the children of a sibling group
-//            are found by position, nothing is scattered);
-//          one launch writes the signal of the finest level, a full row per
-//            wavefront (zeros for empty nodes);
+//            are found by position, nothing is scattered) and, in workgroups of
+//            their own, the signal of the finest level (tiles of 1024 nodes staged
+//            in LDS, full rows out, zeros for empty nodes);
 //          one launch per sparse level for the neighbour tables (each needs the
 //            level above).
 #include "build_adaptive.h"
 #include "octree_kernels.h"
 
 #include <atomic>
+#include <chrono>
 #include <type_traits>
 #include <map>
 #include <mutex>
@@ -56,9 +58,19 @@ struct Control {                 // device-resident, zeroed by init_kernel
   int nne[kMaxLevels];           // non-empty nodes per depth (valid for depth >= full_layer)
   int error;                     // a bounded wait ran out (never expected)
   unsigned ticket[kMaxPasses + 1];  // tile tickets: one per sort pass, the last for the level scan
-  int pad[5];
+  unsigned done;                 // workgroups of the level scan that have finished
+  int pad[4];
 };
 static_assert(sizeof(Control) == 128, "Control layout");
+
+// What the host needs before it can size the blob, in pinned host memory: the workgroup of the
+// level scan that finishes last writes it there, `seq` last (the host polls that word instead of
+// waiting for the stream, which costs a device-to-host copy and the wake-up of a blocked thread).
+struct HostCounts {
+  int nne[kMaxLevels];
+  int error;
+  int seq;
+};
 
 struct BuildGeom {
   int depth, full_layer, n_clouds;
@@ -228,7 +240,11 @@ __device__ inline int wait_sum(const uint32_t* __restrict__ status, int stride, 
 #pragma unroll
     for (int j = 0; j < kGroupTiles; ++j) { all &= s[j]; sum += (int)(s[j] & kCountMask); }
     if (all & kFlagSum) return sum;
-    if (++spins > spin_limit) { *error = 1; return sum; }
+    if (++spins > spin_limit) {
+      __hip_atomic_store(error, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      return sum;
+    }
     __builtin_amdgcn_s_sleep(1);
   }
 }
@@ -430,7 +446,7 @@ constexpr int kLevelTile = kBlock * kLevelItems;
 template <bool TICKETS>
 __global__ __launch_bounds__(kBlock) void levels_kernel(const uint64_t* __restrict__ key, int n, int depth,
     int full_layer, LevelOut out, uint32_t* __restrict__ status, uint32_t* __restrict__ group_status,
-    Control* __restrict__ ctl, int spin_limit) {
+    Control* __restrict__ ctl, int spin_limit, HostCounts* __restrict__ host, int seq) {
   __shared__ int s_tile;
   __shared__ int s_before[16];
   const int tid = threadIdx.x;
@@ -498,10 +514,30 @@ __global__ __launch_bounds__(kBlock) void levels_kernel(const uint64_t* __restri
       }
     });
     if (has_last) {
-      ctl->nne[d] = b0 + c0;
+      status_store(reinterpret_cast<uint32_t*>(&ctl->nne[d]), (uint32_t)(b0 + c0));
       if (f + 1 < L) first[b0 + c0] = b1 + c1;
       else out.ustart[b0 + c0] = n;
     }
+  }
+  // the workgroup that finishes last hands the counts (and whether any wait ran out, in this
+  // launch or in a sort pass before it) to the host
+  // (counts and error word are written and read with device-scope atomic accesses, which do not
+  // linger in an XCD's L2; the wait below is for their acknowledgement.  A device-wide fence
+  // here would have every workgroup write back its XCD's whole L2.)
+  __shared__ int s_last_one;
+  if (has_last) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  if (tid == 0) s_last_one = atomicAdd(&ctl->done, 1u) == gridDim.x - 1;
+  __syncthreads();
+  if (s_last_one && tid < 64) {   // one wavefront: a lane per word, then the sequence number
+    static_assert(kMaxLevels + 1 <= 64, "one lane per word");
+    const int* src = tid < kMaxLevels ? &ctl->nne[tid] : &ctl->error;
+    int* dst = tid < kMaxLevels ? &host->nne[tid] : &host->error;
+    if (tid <= kMaxLevels)
+      __hip_atomic_store(dst, __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT),
+          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    __threadfence_system();
+    if (tid == 0) __hip_atomic_store(&host->seq, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   }
 }
 
@@ -648,7 +684,7 @@ __device__ inline void leaf_signal(float* __restrict__ feature, float* __restric
 
 // The emit launch is cut into segments of whole workgroups; each segment is one kind of
 // work on one level.
-enum SegKind { kSegHeader = 0, kSegFull = 1, kSegFullNeigh = 2, kSegSparse = 3, kSegNeighSearch = 4 };
+enum SegKind { kSegHeader = 0, kSegFull = 1, kSegFullNeigh = 2, kSegSparse = 3, kSegNeighSearch = 4, kSegLeafSignal = 5 };
 // sparse levels with at most this many sibling groups get their neighbour table inside the emit
 // launch (by key search); larger ones from the table of the level above, one launch each
 constexpr int kSearchGroups = 8192;
@@ -673,14 +709,71 @@ struct EmitArgs {
 };
 static_assert(sizeof(EmitArgs) <= 3800, "kernel arguments must stay below 4 KiB");
 
+// Signal of the finest level for a tile of kSignalTile consecutive nodes, through LDS.  The
+// non-empty nodes of the tile are consecutive leaves (ranks grow with the node index), so
+// threads 0 .. count-1 take one leaf each -- dense wavefronts for the point gathers, where one
+// thread per node keeps one lane in seven busy at depth 9 -- and put the result into an LDS
+// image of the tile's rows, which is then written out in full rows (zeros, label -1, for the
+// empty nodes: every row of the block is written exactly once).  Which leaf sits in which node
+// is read off the level lists (node 8 p + octant for the leaves first[p] .. first[p + 1] of the
+// p-th sibling group), not off the child links: the tile waits for no other part of the blob
+// and runs inside the launch that writes those.  Needs channels <= kSignalStage.
+// (Tried and dropped: tiles of 512 nodes, 3-5 % slower; one thread per non-empty leaf writing a
+// compact table that a second launch expands into the rows, 15 % slower on eight scenes: the
+// expansion alone took as long as this tile kernel.)
+constexpr int kSignalTile = 1024, kSignalStage = 8;
+__device__ inline void leaf_signal_tile(char* __restrict__ blob, const EmitArgs& a, int block, unsigned char* s_raw) {
+  const SignalGeom& g = a.sg;
+  float* feature = a.off_feature >= 0 ? reinterpret_cast<float*>(blob + a.off_feature) : nullptr;
+  float* label = a.off_label >= 0 ? reinterpret_cast<float*>(blob + a.off_label) : nullptr;
+  float* s_out = reinterpret_cast<float*>(s_raw);          // [channels][kSignalTile] rows, then labels, then nodes
+  float* s_label = s_out + (size_t)g.channels * kSignalTile;
+  unsigned short* s_node = reinterpret_cast<unsigned short*>(s_label + (label ? kSignalTile : 0));
+  const int tid = threadIdx.x;
+  const int node0 = block * kSignalTile;
+  const int rows = min(kSignalTile, g.nnum_d - node0);
+  const int p0 = node0 >> 3, n_groups = rows >> 3;          // a level holds whole sibling groups
+  const int* __restrict__ first = a.first[g.depth - 1];
+  const uint64_t* __restrict__ leaf_key = a.list[g.depth];
+  const int j0 = first[p0], count = first[p0 + n_groups] - j0;
+  for (int i = tid; i < g.channels * kSignalTile; i += kBlock) s_out[i] = 0.0f;
+  if (label)
+    for (int i = tid; i < kSignalTile; i += kBlock) s_label[i] = -1.0f;
+  for (int t = tid; t < n_groups; t += kBlock) {
+    const int c0 = first[p0 + t], c1 = first[p0 + t + 1];
+    for (int j = c0; j < c1; ++j) s_node[j - j0] = (unsigned short)(t * 8 + (int)(leaf_key[j] & 7));
+  }
+  __syncthreads();
+  SignalGeom lg = g;
+  lg.nnum_d = kSignalTile;   // row length of the LDS image
+  for (int t = tid; t < count; t += kBlock) {
+    const int j = j0 + t;
+    leaf_signal(s_out, label ? s_label : nullptr, (int)s_node[t], (int)(leaf_key[j] >> (3 * g.depth)), a.ustart[j],
+        a.ustart[j + 1], a.sorted_idx, a.clouds, lg);
+  }
+  __syncthreads();
+  for (int ch = 0; ch < g.channels; ++ch)
+    for (int r = tid; r < rows; r += kBlock) feature[(int64_t)ch * g.nnum_d + node0 + r] = s_out[ch * kSignalTile + r];
+  if (label)
+    for (int r = tid; r < rows; r += kBlock) label[node0 + r] = s_label[r];
+}
+
+constexpr size_t kEmitLdsBytes = (size_t)kBlock * 8 * (sizeof(uint64_t) + sizeof(int));
+
 __global__ __launch_bounds__(kBlock) void emit_kernel(char* __restrict__ blob, const EmitArgs a) {
-  __shared__ uint64_t s_key[kBlock * 8];
-  __shared__ int s_child[kBlock * 8];
+  extern __shared__ __attribute__((aligned(16))) unsigned char s_raw[];   // max(kEmitLdsBytes, a signal tile)
+  uint64_t* s_key = reinterpret_cast<uint64_t*>(s_raw);
+  int* s_child = reinterpret_cast<int*>(s_raw + sizeof(uint64_t) * kBlock * 8);
   int seg = 0;
   while (seg + 1 < a.n_seg && (int)blockIdx.x >= a.seg_begin[seg + 1]) ++seg;
   const int kind = a.seg_kind[seg], d = a.seg_level[seg];
   const int block = blockIdx.x - a.seg_begin[seg];
   const int tid = threadIdx.x;
+
+  if (kind == kSegLeafSignal) {
+    leaf_signal_tile(blob, a, block, s_raw);
+    return;
+  }
 
   if (kind == kSegHeader) {
     // header (the tail of the 720-byte block is padding, zero); depth 0 holds no neighbour table
@@ -823,58 +916,6 @@ __global__ __launch_bounds__(kBlock) void leaf_signal_kernel(float* __restrict__
       clouds, g);
 }
 
-// The same through LDS: a workgroup takes kSignalTile consecutive nodes.  Their non-empty
-// ones are consecutive leaves (ranks grow with the node index), so threads 0 .. count-1 take
-// one leaf each -- dense wavefronts for the point gathers, where the kernel above keeps one
-// lane in seven busy at depth 9 -- and put the result into an LDS image of the tile's rows,
-// which is then written out in full rows.  Needs channels <= kSignalStage.
-constexpr int kSignalTile = 1024, kSignalStage = 8;
-__global__ __launch_bounds__(kBlock) void leaf_signal_staged_kernel(float* __restrict__ feature,
-    float* __restrict__ label, const int* __restrict__ child, const uint64_t* __restrict__ leaf_key,
-    const int* __restrict__ ustart, const uint32_t* __restrict__ sorted_idx, const CloudDesc* __restrict__ clouds,
-    SignalGeom g) {
-  extern __shared__ float s_dyn[];           // [channels][kSignalTile] rows, then labels
-  __shared__ unsigned short s_node[kSignalTile];
-  __shared__ int s_first, s_last;
-  float* s_out = s_dyn;
-  float* s_label = s_dyn + (size_t)g.channels * kSignalTile;
-  const int tid = threadIdx.x;
-  const int node0 = blockIdx.x * kSignalTile;
-  const int rows = min(kSignalTile, g.nnum_d - node0);
-  if (tid == 0) { s_first = 0x7fffffff; s_last = -1; }
-  int c[kSignalTile / kBlock];
-#pragma unroll
-  for (int q = 0; q < kSignalTile / kBlock; ++q) {
-    const int r = q * kBlock + tid;
-    c[q] = r < rows ? child[node0 + r] : -1;
-  }
-  for (int i = tid; i < g.channels * kSignalTile; i += kBlock) s_out[i] = 0.0f;
-  if (label)
-    for (int i = tid; i < kSignalTile; i += kBlock) s_label[i] = -1.0f;
-  __syncthreads();
-#pragma unroll
-  for (int q = 0; q < kSignalTile / kBlock; ++q)
-    if (c[q] >= 0) { atomicMin(&s_first, c[q]); atomicMax(&s_last, c[q]); }
-  __syncthreads();
-  const int j0 = s_first, count = s_last - s_first + 1;   // count <= 0: no leaf here
-#pragma unroll
-  for (int q = 0; q < kSignalTile / kBlock; ++q)
-    if (c[q] >= 0) s_node[c[q] - j0] = (unsigned short)(q * kBlock + tid);
-  __syncthreads();
-  SignalGeom lg = g;
-  lg.nnum_d = kSignalTile;   // row length of the LDS image
-  for (int t = tid; t < count; t += kBlock) {
-    const int j = j0 + t;
-    leaf_signal(s_out, label ? s_label : nullptr, (int)s_node[t], (int)(leaf_key[j] >> (3 * g.depth)), ustart[j],
-        ustart[j + 1], sorted_idx, clouds, lg);
-  }
-  __syncthreads();
-  for (int ch = 0; ch < g.channels; ++ch)
-    for (int r = tid; r < rows; r += kBlock) feature[(int64_t)ch * g.nnum_d + node0 + r] = s_out[ch * kSignalTile + r];
-  if (label)
-    for (int r = tid; r < rows; r += kBlock) label[node0 + r] = s_label[r];
-}
-
 __global__ void fill_f32_kernel(float* p, int64_t n, float v) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int64_t step = (int64_t)gridDim.x * blockDim.x;
@@ -940,22 +981,41 @@ constexpr int kFirstWaitLimit = 1 << 16, kTicketWaitLimit = 1 << 22;
 std::atomic<int> g_first_wait_limit{kFirstWaitLimit};
 std::atomic<int> g_ticket_reruns{0};
 
-// Pinned host slots for the one device-to-host copy of a plan (a pageable destination
-// would be staged and cost a second wait).
+// Pinned host slots that the level scan writes the node counts into (coherent host memory:
+// the device writes it in place, the host reads it in place).
 std::mutex g_slots_mutex;
-std::vector<Control*> g_free_slots;
-Control* take_slot() {
+std::vector<HostCounts*> g_free_slots;
+HostCounts* take_slot() {
   {
     std::lock_guard<std::mutex> lock(g_slots_mutex);
-    if (!g_free_slots.empty()) { Control* s = g_free_slots.back(); g_free_slots.pop_back(); return s; }
+    if (!g_free_slots.empty()) { HostCounts* s = g_free_slots.back(); g_free_slots.pop_back(); return s; }
   }
   void* p = nullptr;
-  if (hipHostMalloc(&p, sizeof(Control), hipHostMallocDefault) != hipSuccess) return nullptr;
-  return static_cast<Control*>(p);
+  if (hipHostMalloc(&p, 256, hipHostMallocCoherent) != hipSuccess) return nullptr;
+  memset(p, 0, 256);
+  return static_cast<HostCounts*>(p);
 }
-void give_slot(Control* s) {
+void give_slot(HostCounts* s) {
   std::lock_guard<std::mutex> lock(g_slots_mutex);
   g_free_slots.push_back(s);
+}
+std::atomic<int> g_plan_seq{1};
+
+// Waits until the device has written `seq` into the slot.  The host polls the word for a while
+// (the answer is a few microseconds away when the stream was idle), then falls back on the
+// stream, which also reports a launch that failed.
+int await_counts(HostCounts* h, int seq, hipStream_t s) {
+  const auto t0 = std::chrono::steady_clock::now();
+  for (int spins = 0;; ++spins) {
+    if (__atomic_load_n(&h->seq, __ATOMIC_ACQUIRE) == seq) return OCNN_OK;
+    if ((spins & 1023) == 1023 &&
+        std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(20)) break;
+  }
+  hipError_t e = hipStreamSynchronize(s);
+  OCNN_REQUIRE(e == hipSuccess, OCNN_E_HIP, "node counts: %s", hipGetErrorString(e));
+  OCNN_REQUIRE(__atomic_load_n(&h->seq, __ATOMIC_ACQUIRE) == seq, OCNN_E_HIP,
+      "the level scan finished without handing over the node counts");
+  return OCNN_OK;
 }
 
 }  // namespace
@@ -1116,18 +1176,17 @@ int ocnn_points2octree_plan(const void* const* points_dev, const void* const* po
     lo.ustart = reinterpret_cast<int*>(ws + L.ustart);
     uint32_t* level_status = reinterpret_cast<uint32_t*>(ws + L.level_status);
     uint32_t* level_groups = reinterpret_cast<uint32_t*>(ws + L.level_groups);
-    if (tickets) levels_kernel<true><<<L.level_tiles, kBlock, 0, s>>>(d_key[cur], (int)N, depth, fl, lo, level_status, level_groups, d_ctl, spin_limit);
-    else levels_kernel<false><<<L.level_tiles, kBlock, 0, s>>>(d_key[cur], (int)N, depth, fl, lo, level_status, level_groups, d_ctl, spin_limit);
-    OCNN_LAUNCH_OK("levels");
-    Control* h = take_slot();
+    HostCounts* h = take_slot();
     OCNN_REQUIRE(h, OCNN_E_HIP, "no pinned host memory for the node counts");
-    hipError_t e = hipMemcpyAsync(h, d_ctl, sizeof(Control), hipMemcpyDeviceToHost, s);
-    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    const int seq = g_plan_seq.fetch_add(1) & 0x3fffffff;
+    if (tickets) levels_kernel<true><<<L.level_tiles, kBlock, 0, s>>>(d_key[cur], (int)N, depth, fl, lo, level_status, level_groups, d_ctl, spin_limit, h, seq);
+    else levels_kernel<false><<<L.level_tiles, kBlock, 0, s>>>(d_key[cur], (int)N, depth, fl, lo, level_status, level_groups, d_ctl, spin_limit, h, seq);
+    if (hipGetLastError() != hipSuccess) { give_slot(h); return fail(OCNN_E_HIP, "launch of levels failed"); }
+    const int rc = await_counts(h, seq, s);
     for (int d = fl; d <= depth; ++d) st.nne[d] = h->nne[d];
     *wait_error = h->error;
     give_slot(h);
-    OCNN_REQUIRE(e == hipSuccess, OCNN_E_HIP, "node counts: %s", hipGetErrorString(e));
-    return OCNN_OK;
+    return rc;
   };
 
   int rc = init();
@@ -1246,6 +1305,15 @@ int ocnn_points2octree_emit(void* octree_out_dev, const void* info, void* worksp
     blocks += (int)nblocks;
   };
   add_seg(kSegHeader, 0, 1);
+  // the signal of the finest level first: its workgroups take longest
+  const bool has_signal = depth > fl && HD > 0 && (a.off_feature >= 0 || a.off_label >= 0);
+  const bool signal_inside = has_signal && fch <= kSignalStage;
+  size_t lds = kEmitLdsBytes;
+  if (signal_inside) {
+    add_seg(kSegLeafSignal, depth, blocks_for(HD, kSignalTile));
+    const size_t need = sizeof(float) * kSignalTile * (size_t)(fch + (a.off_label >= 0 ? 1 : 0)) + sizeof(unsigned short) * kSignalTile;
+    if (need > lds) lds = need;
+  }
   for (int d = depth; d > fl; --d) add_seg(kSegSparse, d, blocks_for(st.nne[d - 1]) * (st.nne[d - 1] > 0 ? 1 : 0));
   for (int d = 0; d <= fl; ++d) {
     add_seg(kSegFull, d, blocks_for(o.nnum[d]));
@@ -1259,21 +1327,15 @@ int ocnn_points2octree_emit(void* octree_out_dev, const void* info, void* worksp
     }
   a.seg_begin[n_seg] = blocks;
   a.n_seg = n_seg;
-  emit_kernel<<<blocks, kBlock, 0, s>>>(blob, a);
+  emit_kernel<<<blocks, kBlock, lds, s>>>(blob, a);
   OCNN_LAUNCH_OK("emit");
 
-  if (depth > fl && HD > 0 && (a.off_feature >= 0 || a.off_label >= 0)) {
+  if (has_signal && !signal_inside) {   // more channels than a tile stages: one thread per node, after the child links
     float* f_ptr = a.off_feature >= 0 ? reinterpret_cast<float*>(blob + a.off_feature) : nullptr;
     float* l_ptr = a.off_label >= 0 ? reinterpret_cast<float*>(blob + a.off_label) : nullptr;
     const int* c_ptr = reinterpret_cast<const int*>(blob + a.off_child[depth]);
-    if (fch <= kSignalStage) {
-      const size_t lds = sizeof(float) * kSignalTile * (size_t)(fch + (l_ptr ? 1 : 0));
-      leaf_signal_staged_kernel<<<blocks_for(HD, kSignalTile), kBlock, lds, s>>>(f_ptr, l_ptr, c_ptr, a.list[depth],
-          a.ustart, a.sorted_idx, a.clouds, a.sg);
-    } else {
-      leaf_signal_kernel<<<blocks_for(HD), kBlock, 0, s>>>(f_ptr, l_ptr, c_ptr, a.list[depth], a.ustart,
-          a.sorted_idx, a.clouds, a.sg);
-    }
+    leaf_signal_kernel<<<blocks_for(HD), kBlock, 0, s>>>(f_ptr, l_ptr, c_ptr, a.list[depth], a.ustart,
+        a.sorted_idx, a.clouds, a.sg);
     OCNN_LAUNCH_OK("leaf_signal");
   }
   if (depth == fl && HD > 0) {  // no sparse level: the finest level carries no signal
