@@ -161,6 +161,16 @@ def main():
   extra = {}
   if not args.quick:
     reps, wu = max(3, args.steps // 4), 1
+    headline_timed = timed
+
+    def timed(fn, steps, warmup):
+      """Rows of `extra`: kernels of tens of microseconds.  Warm up until the device has been
+      busy for a few milliseconds (its clocks settle), then time enough calls for the region
+      to last a few milliseconds; at least the given counts."""
+      pilot = headline_timed(fn, 2, max(1, warmup))
+      n_warm = max(warmup, min(200, int(5.0 / max(pilot, 1e-3))))
+      n_rep = max(steps, min(400, int(10.0 / max(pilot, 1e-3))))
+      return headline_timed(fn, n_rep, n_warm)
 
     def conv_case(name, oct_, d, x, w, ks, stride, nempty=False, deconv=False, n_out=C):
       fn = F.octree_deconv if deconv else F.octree_conv
@@ -457,6 +467,29 @@ def main():
                            "sample": "first %d of %d depth-9 octants: octree2col_cpu chunk + "
                                      "single-thread textbook SGEMM (64 x 1728 x %d), %.1f s"
                                      % (sample, H9, sample, t)}
+    # the host this ran on, and the same sample with the GEMM through torch.mm on all its threads
+    # (the reference's CPU path calls a BLAS GEMM there, octree/octree/octree_conv.cpp:276-325)
+    try:
+      model = [l.split(":", 1)[1].strip() for l in open("/proc/cpuinfo") if l.startswith("model name")]
+    except OSError:
+      model = []
+    out["cpu_baseline"]["host"] = {"nproc": os.cpu_count(), "cpu_model": model[0] if model else "unknown",
+                                   "usable_cpus": len(os.sched_getaffinity(0))}
+    wt, ct = torch.from_numpy(wh), torch.from_numpy(col)
+    torch.mm(wt, ct)
+    t0 = time.perf_counter()
+    n_mm = 5
+    for _ in range(n_mm):
+      ymm = torch.mm(wt, ct)
+    t_mm = (time.perf_counter() - t0) / n_mm
+    t0 = time.perf_counter()
+    orc.fn("octree2col")(P(col), P(xh), C, H9, 27, 1, P(neigh), P(ni), sample, 0)
+    t_col = time.perf_counter() - t0
+    out["cpu_baseline"]["blas_all_threads"] = {
+        "value": sample / (t_col + t_mm), "unit": "octants/s", "threads": torch.get_num_threads(),
+        "gemm_gflops": 2.0 * C * C * 27 * sample / t_mm / 1e9, "octree2col_seconds": t_col, "gemm_seconds": t_mm,
+        "max_rel_diff_vs_port": float(np.abs(ymm.numpy() - y).max() / np.abs(y).max()),
+        "sample": "the same %d columns: octree2col_cpu chunk on one core + torch.mm on all threads" % sample}
     # the sample also checks the GPU result
     yg = conv_step().cpu().numpy().reshape(C, H9)[:, :sample]
     out["cpu_baseline"]["gpu_vs_cpu_max_rel_err"] = float(np.abs(yg - y).max() / np.abs(y).max())

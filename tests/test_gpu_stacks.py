@@ -51,7 +51,7 @@ def test_fold_bn_matches_batchnorm(oc):
   assert torch.allclose((wf.t() @ x).view(cout, 8, H) + bf[:, None, None], exp, atol=1e-5)
 
 
-@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 3e-2)])
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 2e-2)])
 def test_fused_bias_relu(oc, orc, tree, dtype, tol):
   host, dev, b = tree
   rng = np.random.default_rng(1)
@@ -92,7 +92,10 @@ def test_lenet_trunk(oc, orc, tree):
   assert relerr(got.cpu().numpy().reshape(x.shape), x) < 1e-4
   p16 = {d: (w.bfloat16(), bb) for d, (w, bb) in params.items()}
   got16 = oc.stacks.lenet_trunk(dev, 6, p16, data=T(data).cuda().view(1, 3, -1, 1).bfloat16())
-  assert relerr(got16.float().cpu().numpy().reshape(x.shape), x) < 5e-2
+  # four bf16 layers against the fp32 chain: the same 2e-2 as a single operator (each layer rounds
+  # its inputs and outputs to 8 significant bits, about 4e-3 of the largest value per layer, and
+  # ReLU plus max pooling do not amplify it: the chain measures 4e-3 as well)
+  assert relerr(got16.float().cpu().numpy().reshape(x.shape), x) < 2e-2
 
 
 @pytest.mark.parametrize("nempty", [False, True])
