@@ -29,8 +29,24 @@ PEAK_MFMA_TFLOPS = {"f32": 157.3, "bf16": 2500.0}
 # HBM bytes per launch of the headline kernel, from two `rocprofv3 --pmc` runs (FETCH_SIZE,
 # WRITE_SIZE) scaled by a 1-GiB device copy: see
 # profiles/conv_s1_f32_lds_kernel__scene_depth9__hbm_traffic.md.  Counters cannot be read from
-# inside this process, so the recorded figure is reported for the workload it was taken on.
-RECORDED_TRAFFIC = {("conv_s1_f32_lds_kernel", 1494168, 64, 64): 1.018e9}
+# inside this process, so the recorded figure is reported for the workload it was taken on, and
+# only while the kernel's source file is the one it was taken from (first 16 hex digits of the
+# SHA-256 of o-cnn_amd/csrc/conv.hip); after any change to that file `traffic` is null until
+# the counters have been read again.
+RECORDED_TRAFFIC = {("conv_s1_f32_lds_kernel", 1494168, 64, 64): (1.0116e9, "b9321465653ee62a")}
+
+
+def recorded_traffic(key):
+  import hashlib
+  entry = RECORDED_TRAFFIC.get(key)
+  if entry is None:
+    return None
+  try:
+    with open(os.path.join(ROOT, "o-cnn_amd", "csrc", "conv.hip"), "rb") as fh:
+      digest = hashlib.sha256(fh.read()).hexdigest()[:16]
+  except OSError:
+    return None
+  return entry[0] if digest == entry[1] else None
 
 
 def oc_points_blob(cloud):
@@ -152,7 +168,7 @@ def main():
                  "octants_d9": H9, "octants_d8": H8, "nonempty_d9": Hne9, "points": 250000},
       "roofline": {"bound": "mfma", "achieved": achieved_tflops, "peak": PEAK_MFMA_TFLOPS["f32"],
                    "unit": "TFLOP/s", "frac": achieved_tflops / PEAK_MFMA_TFLOPS["f32"],
-                   "traffic": RECORDED_TRAFFIC.get(("conv_s1_f32_lds_kernel", H9, C, C)),
+                   "traffic": recorded_traffic(("conv_s1_f32_lds_kernel", H9, C, C)),
                    "kernel": "conv_s1_f32_lds_kernel<2,27>",
                    "algorithmic_flops_per_launch": flops},
       "wall_ms_per_step": wall_ms,
