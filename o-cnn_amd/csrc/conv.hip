@@ -1357,6 +1357,72 @@ __global__ __launch_bounds__(256) void deconv_s2_bf16_kernel(ConvArgs a, uint16_
       for (int nt = 0; nt < 2; ++nt) store_children<uint16_t>(a, out, acc[mt][nt], row_base + mt * 32, ncol[nt], kh);
   }
 }
+// The same for at most 64 input channels (KS k-steps of 16): a wavefront's 64 columns x all
+// channels stay in registers for every pass (read once, all requests in flight together), the
+// packed weights of a pass (128 rows) are staged in LDS for the four wavefronts, the next pass's
+// in flight meanwhile (two buffers, one barrier per pass), and the loop only reads LDS and
+// multiplies.  What is left is the store of the children: the kernel is bound by its output.
+template <int KS>
+__global__ __launch_bounds__(256, 2) void deconv_s2_bf16_reg_kernel(ConvArgs a, uint16_t* __restrict__ out,
+    const uint4* __restrict__ xt, const uint4* __restrict__ Wt, int n_tiles) {
+  constexpr int kUnits = KS * kD2MT * 64;            // 16-byte units of one pass's weights
+  constexpr int kVec = kUnits / 256;                 // per thread
+  __shared__ uint4 sW[2][kUnits];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = xcd_tile(blockIdx.x, n_tiles);
+  if (tile >= n_tiles) return;
+  const int n0 = tile * kTileCols + wave * kWaveCols;
+  const int r = lane & 31, kh = lane >> 5;
+  const int rows = a.M * 8;
+  const int npass = (rows + 32 * kD2MT - 1) / (32 * kD2MT);
+  int ncol[2];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) ncol[nt] = n0 + nt * 32 + r;
+  union Frag { uint4 v4; bf16x8 v; };
+  Frag b[KS][2];
+  uint4 wr[kVec];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) b[ks][nt].v4 = xt[(int64_t)min(ncol[nt], a.Hin) * (2 * KS) + 2 * ks + kh];
+#pragma unroll
+  for (int v = 0; v < kVec; ++v) wr[v] = Wt[v * 256 + threadIdx.x];
+#pragma unroll
+  for (int v = 0; v < kVec; ++v) sW[0][v * 256 + threadIdx.x] = wr[v];
+  for (int pass = 0; pass < npass; ++pass) {
+    __syncthreads();   // this pass's weights are in LDS; the other buffer is free
+    const uint4* wcur = sW[pass & 1];
+    const int nxt = min(pass + 1, npass - 1);
+#pragma unroll
+    for (int v = 0; v < kVec; ++v) wr[v] = Wt[(int64_t)nxt * kUnits + v * 256 + threadIdx.x];
+    floatx16 acc[kD2MT][2];
+#pragma unroll
+    for (int mt = 0; mt < kD2MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int mt = 0; mt < kD2MT; ++mt) {
+        Frag av;
+        av.v4 = wcur[(ks * kD2MT + mt) * 64 + lane];
+        acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b[ks][0].v, acc[mt][0], 0, 0, 0);
+        acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b[ks][1].v, acc[mt][1], 0, 0, 0);
+      }
+#pragma unroll
+    for (int v = 0; v < kVec; ++v) sW[(pass + 1) & 1][v * 256 + threadIdx.x] = wr[v];
+    if (n0 < a.N) {
+      const int row_base = pass * 32 * kD2MT;
+#pragma unroll
+      for (int mt = 0; mt < kD2MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) store_children<uint16_t>(a, out, acc[mt][nt], row_base + mt * 32, ncol[nt], kh);
+    }
+  }
+}
+
 __global__ void pack_weights_d2_bf16(uint16_t* __restrict__ Wt, const uint16_t* __restrict__ W, int rows, int Cin,
     int npass, int ksteps) {
   int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -1608,7 +1674,14 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
       uint16_t* xt = reinterpret_cast<uint16_t*>(wsb + p.wt_bytes + p.ichild_bytes);
       dim3 tgrid((a.Hin + 1 + 127) / 128, (cpad + 63) / 64);
       transpose_rows_bf16_kernel<<<tgrid, 256, 0, s>>>(xt, (const uint16_t*)btm, a.Cin, a.Hin, cpad);
-      deconv_s2_bf16_kernel<<<dim3(d_grid, pass_split(d_tiles, (d.M * 8 + 32 * kD2MT - 1) / (32 * kD2MT))), 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles, cpad / 8);
+      if (ksteps == 1)
+        deconv_s2_bf16_reg_kernel<1><<<d_grid, 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles);
+      else if (ksteps == 2)
+        deconv_s2_bf16_reg_kernel<2><<<d_grid, 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles);
+      else if (ksteps == 4)
+        deconv_s2_bf16_reg_kernel<4><<<d_grid, 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles);
+      else
+        deconv_s2_bf16_kernel<<<dim3(d_grid, pass_split(d_tiles, (d.M * 8 + 32 * kD2MT - 1) / (32 * kD2MT))), 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles, cpad / 8);
     }
   } else if (path == kPathS1LdsF32) {
     const int MT = a.mtiles == 1 ? 1 : 2;
