@@ -109,6 +109,20 @@ int ocnn_col2octreeP(const void* col, void* data, int channel, int height, int o
     const int* kernel_size, int stride, const int* neigh, const int* child, const int* ichild,
     int height_col, int n, int dtype, ocnn_stream_t stream);
 
+/* col2octree / col2octreeP (child == NULL / non-NULL) with the verdict on the table kept in a
+ * word the caller owns, no counterpart in the reference.  The gather form of col2octree is
+ * exact only for a table that maps back and forth consistently, which a check kernel verifies
+ * on the device; with the plain signatures above that check runs in every call.  Here
+ * `table_mark_dev` is an 8-byte device word that the caller zeroes once per (table, kernel
+ * size, stride, chunking): a call with check_now != 0 runs the check and leaves its verdict in
+ * the word, later calls with the same table and shape pass check_now = 0 and skip it (the
+ * kernels read the verdict from the word).  One octree level, its own NEIGH table and a fixed
+ * kernel shape -- what a Col2Octree module or a convolution's backward pass sees -- qualify. */
+int ocnn_col2octree_cached(const void* col, void* data, int channel, int height, int octree_h,
+    const int* kernel_size, int stride, const int* neigh, const int* child, const int* ichild,
+    int height_col, int n, int dtype, unsigned long long* table_mark_dev, int check_now,
+    ocnn_stream_t stream);
+
 /* ---- pooling: octree/octree/octree_nn.h:122-139, octree_nn.cu:258-327.
  * mask holds absolute row indices; the first maximum wins. */
 int ocnn_octree_max_pool(void* top, int top_h, int* mask, const void* btm, int btm_h,

@@ -342,23 +342,39 @@ __global__ void __launch_bounds__(kColTile) octree2col_block_kernel(T* __restric
   }
 }
 
-// Slots that record, per call, that a table is not symmetric.  A call owns slot
-// id % kColSlots and the value id, which no other call ever writes, so slots need no
+// Where a call records that its table is not symmetric.  Either a word the caller owns
+// (ocnn_col2octree_cached: the verdict then outlives the call and later calls with the same
+// table skip the check), or, for the reference's plain signature, a slot of a ring: a call owns
+// slot id % kColSlots and the value id, which no other call ever writes, so slots need no
 // clearing; calls overlapping on other streams only collide kColSlots calls apart.
+constexpr unsigned long long kColMarkOwned = 0xC01A5E7715BADull;   // "not symmetric" in a caller's word
 constexpr int kColSlots = 1024;
 __device__ unsigned long long g_col_asymmetric[kColSlots];
 std::atomic<unsigned long long> g_col_calls{0};
+// the ring's address on the current device (asked once per device)
+unsigned long long* col_ring() {
+  static std::atomic<unsigned long long*> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  unsigned long long* p = cached[dev].load(std::memory_order_acquire);
+  if (p) return p;
+  void* q = nullptr;
+  if (hipGetSymbolAddress(&q, HIP_SYMBOL(g_col_asymmetric)) != hipSuccess) return nullptr;
+  p = static_cast<unsigned long long*>(q);
+  cached[dev].store(p, std::memory_order_release);
+  return p;
+}
 
 // The gather form of col2octree below is exact when (column h, tap k) -> row p and
 // (row p, tap k) -> column h are inverse maps.  y = 0 walks the columns of the chunk,
 // y = 1 the rows; any pair that does not map back marks the call.
 template <bool P>
 __global__ void col_check_kernel(ColArgs a, const int* __restrict__ neigh,
-    const int* __restrict__ child, const int* __restrict__ ichild, unsigned long long id,
-    bool no_inverse) {
+    const int* __restrict__ child, const int* __restrict__ ichild, unsigned long long* __restrict__ mark,
+    unsigned long long id, bool no_inverse) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (no_inverse) {  // the caller gave no inverse child table: always scatter
-    if (i == 0 && blockIdx.y == 0) g_col_asymmetric[id % kColSlots] = id;
+    if (i == 0 && blockIdx.y == 0) *mark = id;
     return;
   }
   int lo = a.n * a.height_col, hi = min(a.height, lo + a.height_col);
@@ -380,7 +396,7 @@ __global__ void col_check_kernel(ColArgs a, const int* __restrict__ neigh,
           col_source<P>(a, col_base<P>(a, h, ichild), k, neigh, child) != p) bad = true;
     }
   }
-  if (bad) g_col_asymmetric[id % kColSlots] = id;
+  if (bad) *mark = id;
 }
 
 // Gather form: one thread per row sums its taps in ascending order, no atomics.
@@ -389,10 +405,10 @@ __global__ void col_check_kernel(ColArgs a, const int* __restrict__ neigh,
 template <bool P>
 __global__ void col2octree_kernel(const float* __restrict__ col, float* __restrict__ data, ColArgs a,
     const int* __restrict__ neigh, const int* __restrict__ child, const int* __restrict__ ichild,
-    unsigned long long id) {
+    const unsigned long long* __restrict__ mark, unsigned long long id) {
   int p = blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= a.octree_h) return;
-  bool marked = g_col_asymmetric[id % kColSlots] == id;
+  bool marked = *mark == id;
   int c0 = blockIdx.y * kChanChunk, c1 = min(a.channel, c0 + kChanChunk);
   float acc[kChanChunk];
 #pragma unroll
@@ -427,8 +443,8 @@ __global__ void col2octree_kernel(const float* __restrict__ col, float* __restri
 template <bool P>
 __global__ void col2octree_atomic_kernel(const float* __restrict__ col, float* __restrict__ data,
     ColArgs a, const int* __restrict__ neigh, const int* __restrict__ child,
-    const int* __restrict__ ichild, unsigned long long id) {
-  if (g_col_asymmetric[id % kColSlots] != id) return;
+    const int* __restrict__ ichild, const unsigned long long* __restrict__ mark, unsigned long long id) {
+  if (*mark != id) return;
   int hl = blockIdx.x * blockDim.x + threadIdx.x;
   if (hl >= a.height_col) return;
   int h = a.n * a.height_col + hl;
@@ -594,7 +610,7 @@ int run_octree2col(void* col, const void* data, int channel, int height, int oct
 template <bool P>
 int run_col2octree(const void* col, void* data, int channel, int height, int octree_h, const int* ks,
     int stride, const int* neigh, const int* child, const int* ichild, int height_col, int n,
-    int dtype, hipStream_t s) {
+    int dtype, hipStream_t s, unsigned long long* owned_mark = nullptr, bool check_now = true) {
   int e = check_col(col, data, channel, height, ks, stride, neigh, height_col, n, dtype);
   if (e) return e;
   OCNN_REQUIRE(dtype == OCNN_F32, OCNN_E_UNSUPPORTED, "col2octree accumulates in fp32 only");
@@ -604,7 +620,13 @@ int run_col2octree(const void* col, void* data, int channel, int height, int oct
   if (octree_h == 0) return OCNN_OK;
   // The first chunk (n == 0) overwrites the rows, later ones add to them
   // (octree_nn.cpp:226 clears the output before the first chunk).
-  unsigned long long id = ++g_col_calls;
+  unsigned long long id = owned_mark ? kColMarkOwned : ++g_col_calls;
+  unsigned long long* mark = owned_mark ? owned_mark : nullptr;
+  if (!mark) {
+    unsigned long long* ring = col_ring();
+    OCNN_REQUIRE(ring, OCNN_E_HIP, "no address for the table marks of this device");
+    mark = ring + id % kColSlots;
+  }
   bool can_invert = !P || ichild != nullptr;
   int chunk_cols = (int)std::max<int64_t>(0,
       std::min<int64_t>(height, ((int64_t)n + 1) * height_col) - (int64_t)n * height_col);
@@ -613,15 +635,17 @@ int run_col2octree(const void* col, void* data, int channel, int height, int oct
   // columns are found the way a column's rows are (tap k one way is the opposite tap
   // the other way), so over the whole range one direction of the check says it all.
   bool one_way = stride == 1 && ks[0] != 2 && n == 0 && chunk_cols == height && height == octree_h;
-  dim3 check_grid(blocks_for(std::max(std::max(chunk_cols, octree_h), 1)), one_way ? 1 : 2);
-  col_check_kernel<P><<<check_grid, kBlock, 0, s>>>(a, neigh, child, ichild, id, !can_invert);
-  OCNN_LAUNCH_OK("col_check");
+  if (check_now) {
+    dim3 check_grid(blocks_for(std::max(std::max(chunk_cols, octree_h), 1)), one_way ? 1 : 2);
+    col_check_kernel<P><<<check_grid, kBlock, 0, s>>>(a, neigh, child, ichild, mark, id, !can_invert);
+    OCNN_LAUNCH_OK("col_check");
+  }
   col2octree_kernel<P><<<dim3(blocks_for(octree_h), chans), kBlock, 0, s>>>((const float*)col,
-      (float*)data, a, neigh, child, ichild, id);
+      (float*)data, a, neigh, child, ichild, mark, id);
   OCNN_LAUNCH_OK("col2octree");
   if (chunk_cols > 0) {
     col2octree_atomic_kernel<P><<<dim3(blocks_for(height_col), chans), kBlock, 0, s>>>(
-        (const float*)col, (float*)data, a, neigh, child, ichild, id);
+        (const float*)col, (float*)data, a, neigh, child, ichild, mark, id);
     OCNN_LAUNCH_OK("col2octree_atomic");
   }
   return OCNN_OK;
@@ -720,6 +744,19 @@ int ocnn_col2octreeP(const void* col, void* data, int channel, int height, int o
   OCNN_REQUIRE(child && (ichild || stride == 2), OCNN_E_BADARG, "null child/ichild");
   return run_col2octree<true>(col, data, channel, height, octree_h, kernel_size, stride, neigh, child,
       ichild, height_col, n, dtype, as_stream(stream));
+}
+
+int ocnn_col2octree_cached(const void* col, void* data, int channel, int height, int octree_h,
+    const int* kernel_size, int stride, const int* neigh, const int* child, const int* ichild,
+    int height_col, int n, int dtype, unsigned long long* table_mark_dev, int check_now,
+    ocnn_stream_t stream) {
+  OCNN_REQUIRE(table_mark_dev, OCNN_E_BADARG, "null table mark");
+  OCNN_REQUIRE((reinterpret_cast<uintptr_t>(table_mark_dev) & 7) == 0, OCNN_E_BADARG, "table mark not 8-byte aligned");
+  if (child)
+    return run_col2octree<true>(col, data, channel, height, octree_h, kernel_size, stride, neigh, child,
+        ichild, height_col, n, dtype, as_stream(stream), table_mark_dev, check_now != 0);
+  return run_col2octree<false>(col, data, channel, height, octree_h, kernel_size, stride, neigh,
+      nullptr, nullptr, height_col, n, dtype, as_stream(stream), table_mark_dev, check_now != 0);
 }
 
 int ocnn_octree_max_pool(void* top, int top_h, int* mask, const void* btm, int btm_h, int channel,

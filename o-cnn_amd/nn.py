@@ -651,19 +651,30 @@ def col2octree(grad_in, octree, depth, kernel_size, stride, nempty):
   neigh = _prop_view(octree, info, NEIGH, depth, info.nnum(depth) * 8, torch.int32)
   if stride == 2 and top_h != info.nnum_nempty(depth - 1):
     raise OcnnError(-3, "col2octree: stride-2 height mismatch")
+  # The verdict on the level's table (does it map back and forth consistently, so that the sum
+  # may be gathered) is kept with the octree tensor, one device word per (depth, kernel, stride,
+  # mode): the first call checks the table on the device, later calls read the word.
+  marks = getattr(octree, "_ocnn_col_marks", None)
+  if marks is None:
+    marks = octree._ocnn_col_marks = {}
+  key = (depth, tuple(ks), stride, bool(nempty), top_h)
+  mark = marks.get(key)
+  check_now = mark is None
+  if check_now:
+    mark = marks[key] = torch.zeros(1, dtype=torch.int64, device=grad_in.device)
   if not nempty:
     btm_h = info.nnum(depth)
     out = torch.empty(1, channel, btm_h, 1, dtype=grad_in.dtype, device=grad_in.device)
-    _lib.call("ocnn_col2octree", _ptr(grad_in), _ptr(out), channel, top_h, ksc, stride, _ptr(neigh),
-              max(top_h, 1), 0, dt, _stream())
+    _lib.call("ocnn_col2octree_cached", _ptr(grad_in), _ptr(out), channel, top_h, top_h << (3 * (stride - 1)), ksc,
+              stride, _ptr(neigh), None, None, max(top_h, 1), 0, dt, _ptr(mark), int(check_now), _stream())
     return out
   btm_h = info.nnum_nempty(depth)
   if stride == 1 and top_h != btm_h:
     raise OcnnError(-3, "col2octree: height mismatch")
   child, ichild = _ichild(octree, info, depth)
   out = torch.empty(1, channel, btm_h, 1, dtype=grad_in.dtype, device=grad_in.device)
-  _lib.call("ocnn_col2octreeP", _ptr(grad_in), _ptr(out), channel, top_h, btm_h, ksc, stride,
-            _ptr(neigh), _ptr(child), _ptr(ichild), max(top_h, 1), 0, dt, _stream())
+  _lib.call("ocnn_col2octree_cached", _ptr(grad_in), _ptr(out), channel, top_h, btm_h, ksc, stride,
+            _ptr(neigh), _ptr(child), _ptr(ichild), max(top_h, 1), 0, dt, _ptr(mark), int(check_now), _stream())
   return out
 
 

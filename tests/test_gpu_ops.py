@@ -188,6 +188,20 @@ def test_col2octree_any_table_and_chunks(oc, orc, tree):
       oc.lib.call("ocnn_col2octreeP", P(colp_d), P(outp), 5, hp, Hne, ksc, stride, P(table_d), P(child_d),
                   P(ichild_d), hp, 0, 0, st)
       assert relerr(outp.cpu().numpy(), expp) < TOL_F32, (name, "P", ks, stride)
+      # the same through the entry point that keeps the verdict on the table in a word of the
+      # caller: the first call checks, the second reads the word (and must agree for a table that
+      # failed the check as much as for one that passed)
+      for mode, args, want in (("plain", (5, h, h << (3 * (stride - 1))), exp), ("P", (5, hp, Hne), expp)):
+        mark = torch.zeros(1, dtype=torch.int64, device="cuda")
+        src = T(col).cuda() if mode == "plain" else colp_d
+        for check_now in (1, 0):
+          got = torch.full((5, H if mode == "plain" else Hne), 7.0, device="cuda")
+          oc.lib.call("ocnn_col2octree_cached", P(src), P(got), *args, ksc, stride, P(table_d),
+                      P(child_d) if mode == "P" else C.c_void_p(0), P(ichild_d) if mode == "P" else C.c_void_p(0),
+                      args[1], 0, 0, P(mark), check_now, st)
+          assert relerr(got.cpu().numpy(), want) < TOL_F32, (name, mode, ks, stride, check_now)
+        if name == "own":
+          assert int(mark.item()) == 0, (mode, ks, stride)     # an octree's own table passes the check
       if stride == 2:   # without the inverse child table only the scatter form can run
         outq = torch.full((5, Hne), 7.0, device="cuda")
         oc.lib.call("ocnn_col2octreeP", P(colp_d), P(outq), 5, hp, Hne, ksc, stride, P(table_d),
