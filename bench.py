@@ -355,6 +355,12 @@ def main():
     hbm("depad_d8_f32", timed(lambda: F.octree_depad(pd8, octree, 8), reps, wu), C * (Hne8 + H8) * s + H8 * 4)
     hbm("mask_pool_d9_f32", timed(lambda: F.octree_mask_pool(x32, mask, octree, 9), reps, wu),
         C * (H9 // 8) * (2 * s + 4))
+    # the operation reads one of the eight children of every parent, i.e. 4 of every 32 bytes of
+    # the input: every line of the input is fetched.  Bytes of the lines it touches, beside the
+    # algorithmic ones (the counters agree: profiles/hbm_counters__bench_default_workloads.md)
+    lines = C * H9 * s + C * (H9 // 8) * (s + 4)
+    extra["mask_pool_d9_f32"].update({"GBs_of_touched_lines": lines / extra["mask_pool_d9_f32"]["ms"] / 1e6,
+                                      "frac_hbm_peak_of_touched_lines": lines / extra["mask_pool_d9_f32"]["ms"] / 1e6 / PEAK_HBM_GBS})
     hbm("max_pool_d9_bf16", timed(lambda: F.octree_max_pool(x16, octree, 9), reps, wu),
         C * H9 * 2 + C * (H9 // 8) * (2 + 4))
     c8 = 8
@@ -370,6 +376,9 @@ def main():
     q = key9[torch.randint(0, H9, (1 << 20,), generator=g).to(dev)]
     hbm("search_key_d9_1Mq", timed(lambda: F.octree_search_key(q, octree, 9, False, False), reps, wu),
         (1 << 20) * 12)
+    # a binary search over 1.5 M keys per query: the counters show 456 MB fetched per launch
+    # (profiles/hbm_counters__bench_default_workloads.md), 435 bytes per query
+    extra["search_key_d9_1Mq"]["GBs_fetched_by_counters"] = 460.5e6 / extra["search_key_d9_1Mq"]["ms"] / 1e6
     lab = (child8 >= 0).to(torch.int32)
     P = lambda t_: Ct.c_void_p(t_.data_ptr())
     lab_out = torch.empty_like(lab)
