@@ -393,6 +393,124 @@ __global__ __launch_bounds__(256) void conv_rows_bf16_kernel(ConvArgs a, uint16_
     if (n0 < a.N) store_tiles<uint16_t, MT>(a, out, acc, pass * MT, n0, lane);
   }
 }
+// The same operator with a deeper pipeline, for tap sets of three taps or more.  The kernel
+// above pays two barriers per (tap, 64-channel slab) for 16 MFMAs per wavefront and has one
+// stage of gathers in flight; with 27 rows to fetch per column from the L2 that leaves the
+// matrix pipe idle seven cycles in eight.  Here
+//   * the source rows of all taps of the workgroup's 256 columns are looked up once, up front and
+//     all together (two dependent trips to memory for the whole tile), and wait in LDS;
+//   * the weights come in groups of three taps (24 KiB for 64 output channels, two buffers):
+//     one barrier per three taps;
+//   * a tap's operands (64 channels x 2 column tiles = 8 loads per lane, which read each source
+//     row in full) are requested two taps ahead into a ring of three register sets;
+//   * the register budget allows two workgroups per CU, so that a second wavefront per SIMD
+//     multiplies while the first waits.
+// Non-empty 3x3x3 64 -> 64 at depth 9 (232 158 columns): 0.162 -> 0.132 ms for the operator, the
+// kernel itself 0.11 ms.  What bounds it now is the volume of the gathers: 27 rows of 128 bytes
+// per column from the L2, 0.8 GB per launch, where the matrix work is 20 microseconds; neighbouring
+// columns share most of their rows, which only a per-tile list of distinct rows staged in LDS
+// would exploit.
+template <int MT>
+__global__ __launch_bounds__(256, 2) void conv_rows_bf16_deep_kernel(ConvArgs a, uint16_t* __restrict__ out,
+    const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles, int cpad) {
+  constexpr int kG = 3;                                 // taps per weight group
+  constexpr int kKs = kRowSlab / 16;                    // k-steps per slab
+  constexpr int kWUnits = kKs * MT * 64;                // 16-byte units of one (tap, slab)
+  constexpr int kWVec = kG * kWUnits / 256;             // per thread and group
+  __shared__ u32x4 sW[2][kG * kWUnits];
+  __shared__ int sSrc[27][kTileCols];                   // source row of (tap, column), in 16-byte units of the copy
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = xcd_tile(blockIdx.x, n_tiles);
+  if (tile >= n_tiles) return;
+  const int n0 = tile * kTileCols + wave * kWaveCols;
+  const int r = lane & 31, kh = lane >> 5;
+  const int nslab = (cpad + kRowSlab - 1) / kRowSlab;
+  const int npass = (a.mtiles + MT - 1) / MT;
+  const int cpad8 = cpad >> 3;
+  const int ngroup = (a.K + kG - 1) / kG;
+  {
+    const int col = tile * kTileCols + (int)threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < 27; ++k) {
+      const int sr = k < a.K ? conv_src(a, col, k) : -1;
+      sSrc[k][threadIdx.x] = (sr < 0 ? a.Hin : sr) * cpad8;
+    }
+  }
+  const int c0 = wave * kWaveCols + r;                  // my column of the first column tile, inside the workgroup's tile
+  union Frag { u32x4 q; bf16x8 v; };
+  for (int pass = blockIdx.y; pass < npass; pass += gridDim.y) {  // passes may be dealt out over workgroups
+    floatx16 acc[MT][2];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
+    for (int slab = 0; slab < nslab; ++slab) {
+      const int nks = min(kRowSlab, cpad - slab * kRowSlab) >> 4;    // k-steps of this slab (uniform)
+      const int col16 = ((slab * kRowSlab) >> 3) + kh;               // my 16-byte unit inside a row
+      u32x4 wr[kWVec];
+      // group g of this (pass, slab): taps 3g .. 3g+2, each kWUnits units at ((pass K + tap) nslab + slab) kWUnits
+      auto fetch_w = [&](int g) {
+#pragma unroll
+        for (int v = 0; v < kWVec; ++v) {
+          const int idx = v * 256 + (int)threadIdx.x;
+          const int tap = min(g * kG + idx / kWUnits, a.K - 1);
+          wr[v] = Wt[(((int64_t)pass * a.K + tap) * nslab + slab) * kWUnits + idx % kWUnits];
+        }
+      };
+      Frag x[3][kKs][2];                                 // ring of three taps: [tap % 3][k-step][column tile]
+      auto fetch_x = [&](int tap, auto set) {
+        constexpr int S = decltype(set)::value;
+        if (tap >= a.K) return;                          // uniform
+        const int s0 = sSrc[tap][c0], s1 = sSrc[tap][c0 + 32];
+#pragma unroll
+        for (int ks = 0; ks < kKs; ++ks)
+          if (ks < nks) {
+            x[S][ks][0].q = xt[(int64_t)s0 + col16 + 2 * ks];
+            x[S][ks][1].q = xt[(int64_t)s1 + col16 + 2 * ks];
+          }
+      };
+      __syncthreads();                                   // source rows written (first time); weight buffers free
+      fetch_w(0);
+      fetch_x(0, std::integral_constant<int, 0>());
+      fetch_x(1, std::integral_constant<int, 1>());
+#pragma unroll
+      for (int v = 0; v < kWVec; ++v) sW[0][v * 256 + threadIdx.x] = wr[v];
+      for (int g = 0; g < ngroup; ++g) {
+        __syncthreads();                                 // group g's weights are in LDS; the other buffer is free
+        const u32x4* wcur = sW[g & 1];
+        if (g + 1 < ngroup) fetch_w(g + 1);
+        auto tap_step = [&](auto jc) {
+          constexpr int J = decltype(jc)::value;
+          const int tap = g * kG + J;
+          if (tap >= a.K) return;                        // uniform
+          fetch_x(tap + 2, std::integral_constant<int, (J + 2) % 3>());
+#pragma unroll
+          for (int ks = 0; ks < kKs; ++ks) {
+            if (ks >= nks) continue;                     // uniform
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+              Frag av;
+              av.q = wcur[J * kWUnits + (ks * MT + mt) * 64 + lane];
+              acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, x[J][ks][0].v, acc[mt][0], 0, 0, 0);
+              acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, x[J][ks][1].v, acc[mt][1], 0, 0, 0);
+            }
+          }
+        };
+        tap_step(std::integral_constant<int, 0>());
+        tap_step(std::integral_constant<int, 1>());
+        tap_step(std::integral_constant<int, 2>());
+        if (g + 1 < ngroup) {
+#pragma unroll
+          for (int v = 0; v < kWVec; ++v) sW[(g + 1) & 1][v * 256 + threadIdx.x] = wr[v];
+        }
+      }
+    }
+    if (n0 < a.N) store_tiles<uint16_t, MT>(a, out, acc, pass * MT, n0, lane);
+  }
+}
+
 // [pass][tap][slab][c16][mt][lane][j]: lane (m, kh), j <- W'(m, slab*64 + c16*16 + 8kh + j, tap)
 __global__ void pack_weights_rows_bf16(uint16_t* __restrict__ Wt, const uint16_t* __restrict__ W, int M, int Cin,
     int K, int MT, int npass, int nslab, int64_t sm, int64_t sc) {
@@ -1747,7 +1865,12 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     dim3 tg((a.Hin + 1 + 127) / 128, (cpad + 63) / 64);
     transpose_rows_bf16_kernel<<<tg, 256, 0, s>>>(xt, (const uint16_t*)btm, a.Cin, a.Hin, cpad);
     OCNN_LAUNCH_OK("transpose_rows");
-    if (MT == 1)
+    const bool deep = a.K >= 3;   // fewer taps than a weight group: the shallow kernel
+    if (deep && MT == 1)
+      conv_rows_bf16_deep_kernel<1><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
+    else if (deep)
+      conv_rows_bf16_deep_kernel<2><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
+    else if (MT == 1)
       conv_rows_bf16_kernel<1><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
     else
       conv_rows_bf16_kernel<2><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
