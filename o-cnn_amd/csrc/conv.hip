@@ -930,8 +930,9 @@ __global__ __launch_bounds__(256, 1) void conv_s1_bf16_reg_kernel(ConvArgs a, ui
   // the row-major copy and the packed weights as buffers: 32-bit offsets per lane, the k-step's
   // column / the piece of the weights as the scalar offset (the host sends levels beyond 2 GiB
   // to the other kernel)
+  const int xrows_bytes = (int)(((int64_t)a.Hin + 1) * row_bytes);
   const __amdgpu_buffer_rsrc_t xrows = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<u32x4*>(xt), 0, (int)(((int64_t)a.Hin + 1) * row_bytes), 0x00020000);
+      const_cast<u32x4*>(xt), 0, xrows_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t wbuf = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<u32x4*>(Wt), 0, npass * nks * kWUnits * 16, 0x00020000);
 
@@ -971,14 +972,14 @@ __global__ __launch_bounds__(256, 1) void conv_s1_bf16_reg_kernel(ConvArgs a, ui
   u32x4 bl[2][16];   // two x-layers of operands: [buffer][y*4 + z]
   u32x4 wr[kWVec];
   // requests the 4 slot rows (Y, 0..3) of layer L at k-step KS into buffer L & 1
-#define OCNN_REQ_ROW(KS, L, Y)                                                                  \
+#define OCNN_REQ_ROW(BUF, KS, L, Y)                                                             \
   do {                                                                                          \
     const int4 rows = *reinterpret_cast<const int4*>(&sNb[wave][n * kNbPitch + (L) * 16 + (Y) * 4]); \
     const int col = (KS) * 32;                                                                  \
-    bl[(L) & 1][(Y) * 4 + 0] = __builtin_amdgcn_raw_buffer_load_b128(xrows, rows.x + half, col, 0); \
-    bl[(L) & 1][(Y) * 4 + 1] = __builtin_amdgcn_raw_buffer_load_b128(xrows, rows.y + half, col, 0); \
-    bl[(L) & 1][(Y) * 4 + 2] = __builtin_amdgcn_raw_buffer_load_b128(xrows, rows.z + half, col, 0); \
-    bl[(L) & 1][(Y) * 4 + 3] = __builtin_amdgcn_raw_buffer_load_b128(xrows, rows.w + half, col, 0); \
+    bl[(L) & 1][(Y) * 4 + 0] = __builtin_amdgcn_raw_buffer_load_b128(BUF, rows.x + half, col, 0); \
+    bl[(L) & 1][(Y) * 4 + 1] = __builtin_amdgcn_raw_buffer_load_b128(BUF, rows.y + half, col, 0); \
+    bl[(L) & 1][(Y) * 4 + 2] = __builtin_amdgcn_raw_buffer_load_b128(BUF, rows.z + half, col, 0); \
+    bl[(L) & 1][(Y) * 4 + 3] = __builtin_amdgcn_raw_buffer_load_b128(BUF, rows.w + half, col, 0); \
   } while (0)
   // Layer L + 2 (of this k-step, or layer L - 2 of the next) takes over the registers of layer L
   // row by row as the rows die: row y is last used by the taps with dy = min(y, 2).  Its first
@@ -986,8 +987,8 @@ __global__ __launch_bounds__(256, 1) void conv_s1_bf16_reg_kernel(ConvArgs a, ui
   // starts, the last ones for a phase and a third.
 #define OCNN_REFILL(KS, L, Y)                                                                   \
   do {                                                                                          \
-    if ((L) < 2) OCNN_REQ_ROW(KS, (L) + 2, Y);                                                  \
-    else OCNN_REQ_ROW(ks_next, (L) - 2, Y);                                                     \
+    if ((L) < 2) OCNN_REQ_ROW(xrows, KS, (L) + 2, Y);                                           \
+    else OCNN_REQ_ROW(xnext, ks_next, (L) - 2, Y);                                              \
     /* the requests stay where they are (the scheduler would sink them to their first use    \
        to save registers) */                                                                   \
     __builtin_amdgcn_sched_barrier(0);                                                          \
@@ -995,8 +996,9 @@ __global__ __launch_bounds__(256, 1) void conv_s1_bf16_reg_kernel(ConvArgs a, ui
   // One layer phase: a quarter of the next k-step's weights on their way, the layer multiplied
   // into the siblings it reaches, the weights parked in LDS.  No branches (a thread past the end
   // of the piece copies its last unit once more; the last k-step copies the first weights of the
-  // next pass, or its own, and requests its own first layers again): one basic block per phase,
-  // so the waits the compiler places count exactly the requests that must have landed.
+  // next pass, or its own, and its requests for "the next k-step" go through a buffer of size
+  // zero: they cost an issue slot, touch no memory and return at once): one basic block per
+  // phase, so the waits the compiler places count exactly the requests that must have landed.
 #define OCNN_LAYER_PHASE(KS, L)                                                                 \
   do {                                                                                          \
     {                                                                                           \
@@ -1051,9 +1053,9 @@ __global__ __launch_bounds__(256, 1) void conv_s1_bf16_reg_kernel(ConvArgs a, ui
   int wbase = 0;   // LDS buffer of a pass's first k-step
   for (; pass < npass; pass += gridDim.y) {   // passes may be dealt out over workgroups
 #pragma unroll
-    for (int y = 0; y < 4; ++y) { OCNN_REQ_ROW(0, 0, y); }
+    for (int y = 0; y < 4; ++y) { OCNN_REQ_ROW(xrows, 0, 0, y); }
 #pragma unroll
-    for (int y = 0; y < 4; ++y) { OCNN_REQ_ROW(0, 1, y); }
+    for (int y = 0; y < 4; ++y) { OCNN_REQ_ROW(xrows, 0, 1, y); }
 
     // lane (n, kh) holds rows m0 + 32 mt + 8 (i / 4) + i % 4 of columns 8 (g0 + n) .. + 7
     const int m0 = pass * MT * 32 + 4 * kh;
@@ -1072,6 +1074,8 @@ __global__ __launch_bounds__(256, 1) void conv_s1_bf16_reg_kernel(ConvArgs a, ui
       const u32x4* wcur = sW[(wbase + ks) & 1];
       u32x4* wnext = sW[(wbase + ks + 1) & 1];
       const int ks_next = min(ks + 1, nks - 1);
+      const __amdgpu_buffer_rsrc_t xnext = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<u32x4*>(xt), 0, ks + 1 < nks ? xrows_bytes : 0, 0x00020000);
       const int wsrc = ks + 1 < nks ? wpass + (ks + 1) * kWUnits * 16 : wfirst;
       OCNN_LAYER_PHASE(ks, 0);
       OCNN_LAYER_PHASE(ks, 1);
@@ -1083,10 +1087,25 @@ __global__ __launch_bounds__(256, 1) void conv_s1_bf16_reg_kernel(ConvArgs a, ui
     // one 16-byte store per output channel: the 8 columns of a group are contiguous
     const int g = g0 + n;
     uint16_t* orow = out + (int64_t)g * 8 + (int64_t)m0 * a.Hout;
-    // Straight-line code: the biases of my rows are fetched together, the ReLU is a maximum with
-    // 0 or -inf, the conversion is the hardware's (round to nearest even).
-    const float floor = a.relu ? 0.0f : -__builtin_inff();
     const int m_left = g < n_groups ? a.M - m0 : 0;   // rows of mine that exist
+    // Straight-line code; the conversion is the hardware's (round to nearest even).  The plain
+    // operator (no bias, no ReLU: what the reference's octree_conv is) only converts and stores.
+    if (!a.bias && !a.relu) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int dm = 32 * mt + 8 * (i / 4) + (i % 4);
+          uint32_t w[4];
+#pragma unroll
+          for (int sp = 0; sp < 4; ++sp) w[sp] = pack_bf16x2(acc[2 * sp][mt][i], acc[2 * sp + 1][mt][i]);
+          if (dm < m_left)
+            *reinterpret_cast<uint4*>(orow + (int64_t)dm * a.Hout) = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+      continue;
+    }
+    // the biases of my rows are fetched together, the ReLU is a maximum with 0 or -inf
+    const float floor = a.relu ? 0.0f : -__builtin_inff();
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       float bias[16];
