@@ -688,6 +688,7 @@ enum SegKind { kSegHeader = 0, kSegFull = 1, kSegFullNeigh = 2, kSegSparse = 3, 
 // sparse levels with at most this many sibling groups get their neighbour table inside the emit
 // launch (by key search); larger ones from the table of the level above, one launch each
 constexpr int kSearchGroups = 8192;
+constexpr int kSearchPerWave = 4;
 constexpr int kMaxSeg = 56;
 struct HeaderArg { uint32_t w[OCNN_HEADER_BYTES / 4]; };
 
@@ -726,9 +727,14 @@ __device__ inline void leaf_signal_tile(char* __restrict__ blob, const EmitArgs&
   const SignalGeom& g = a.sg;
   float* feature = a.off_feature >= 0 ? reinterpret_cast<float*>(blob + a.off_feature) : nullptr;
   float* label = a.off_label >= 0 ? reinterpret_cast<float*>(blob + a.off_label) : nullptr;
-  float* s_out = reinterpret_cast<float*>(s_raw);          // [channels][kSignalTile] rows, then labels, then nodes
+  // [channels][kSignalTile] rows, labels, then per leaf: its first point (one more entry closes
+  // the last leaf), its node inside the tile and, for a batch, its cloud
+  float* s_out = reinterpret_cast<float*>(s_raw);
   float* s_label = s_out + (size_t)g.channels * kSignalTile;
-  unsigned short* s_node = reinterpret_cast<unsigned short*>(s_label + (label ? kSignalTile : 0));
+  int* s_start = reinterpret_cast<int*>(s_label + (label ? kSignalTile : 0));
+  unsigned short* s_node = reinterpret_cast<unsigned short*>(s_start + kSignalTile + 2);
+  unsigned short* s_cloud = s_node + kSignalTile;
+  const bool batch = a.n_clouds > 1;
   const int tid = threadIdx.x;
   const int node0 = block * kSignalTile;
   const int rows = min(kSignalTile, g.nnum_d - node0);
@@ -741,16 +747,21 @@ __device__ inline void leaf_signal_tile(char* __restrict__ blob, const EmitArgs&
     for (int i = tid; i < kSignalTile; i += kBlock) s_label[i] = -1.0f;
   for (int t = tid; t < n_groups; t += kBlock) {
     const int c0 = first[p0 + t], c1 = first[p0 + t + 1];
-    for (int j = c0; j < c1; ++j) s_node[j - j0] = (unsigned short)(t * 8 + (int)(leaf_key[j] & 7));
+    for (int j = c0; j < c1; ++j) {
+      const uint64_t lk = leaf_key[j];
+      s_node[j - j0] = (unsigned short)(t * 8 + (int)(lk & 7));
+      if (batch) s_cloud[j - j0] = (unsigned short)(lk >> (3 * g.depth));
+    }
   }
+  // the leaves' point ranges, requested with the keys above: a leaf then starts with its points'
+  // indices instead of with one more trip to memory
+  for (int t = tid; t <= count; t += kBlock) s_start[t] = a.ustart[j0 + t];
   __syncthreads();
   SignalGeom lg = g;
   lg.nnum_d = kSignalTile;   // row length of the LDS image
-  for (int t = tid; t < count; t += kBlock) {
-    const int j = j0 + t;
-    leaf_signal(s_out, label ? s_label : nullptr, (int)s_node[t], (int)(leaf_key[j] >> (3 * g.depth)), a.ustart[j],
-        a.ustart[j + 1], a.sorted_idx, a.clouds, lg);
-  }
+  for (int t = tid; t < count; t += kBlock)
+    leaf_signal(s_out, label ? s_label : nullptr, (int)s_node[t], batch ? (int)s_cloud[t] : 0, s_start[t],
+        s_start[t + 1], a.sorted_idx, a.clouds, lg);
   __syncthreads();
   for (int ch = 0; ch < g.channels; ++ch)
     for (int r = tid; r < rows; r += kBlock) feature[(int64_t)ch * g.nnum_d + node0 + r] = s_out[ch * kSignalTile + r];
@@ -808,28 +819,62 @@ __global__ __launch_bounds__(kBlock) void emit_kernel(char* __restrict__ blob, c
     // That node exists iff it lies inside the cube and its parent is a non-empty node of the
     // same cloud: the parent's rank r in the sorted list gives the index 8r + octant.  Equal to
     // what calc_neigh derives level by level (octree_nn.cpp:357-380).
-    const int g = block * (kBlock / 64) + (tid >> 6);
-    if (g >= a.nne[d - 1]) return;
-    const int lane = tid & 63;
+    // The 64 slots of a group have only 27 different parents (the 3x3x3 nodes around the group's
+    // own parent), so 27 lanes search and the slots pick their parent's rank up by a shuffle; a
+    // wavefront takes four groups, two in each half of its lanes, and walks the two searches of a
+    // lane side by side (the divergent loads of the search are what this segment costs).
+    const int n_par = a.nne[d - 1];
+    const int g0 = (block * (kBlock / 64) + (tid >> 6)) * kSearchPerWave;
+    if (g0 >= n_par) return;
+    const int lane = tid & 63, half = lane >> 5, pl = lane & 31;
     const int bits = 3 * (d - 1);
     const uint64_t* __restrict__ list = a.list[d - 1];
-    const uint64_t pk = list[g];
-    const uint64_t cloud_bits = (pk >> bits) << bits;
-    uint32_t px, py, pz;
-    morton_decode(pk - cloud_bits, d - 1, &px, &py, &pz);
-    const int nx = 2 * (int)px + (lane >> 4) - 1, ny = 2 * (int)py + ((lane >> 2) & 3) - 1,
-              nz = 2 * (int)pz + (lane & 3) - 1;
-    int v = -1;
-    if (nx >= 0 && ny >= 0 && nz >= 0 && ((nx | ny | nz) >> d) == 0) {
-      const uint64_t want = cloud_bits | morton_encode((uint32_t)nx >> 1, (uint32_t)ny >> 1, (uint32_t)nz >> 1, d - 1);
-      int lo = 0, hi = a.nne[d - 1];
-      while (lo < hi) {
-        const int mid = (lo + hi) >> 1;
-        if (list[mid] < want) lo = mid + 1; else hi = mid;
-      }
-      if (lo < a.nne[d - 1] && list[lo] == want) v = 8 * lo + (((nx & 1) << 2) | ((ny & 1) << 1) | (nz & 1));
+    const int ox = pl / 9 - 1, oy = (pl / 3) % 3 - 1, oz = pl % 3 - 1;   // pl < 27
+    uint64_t want[2];
+    int lo[2], hi[2];
+    bool inside[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const uint64_t pk = list[min(g0 + 2 * q + half, n_par - 1)];
+      const uint64_t cloud_bits = (pk >> bits) << bits;
+      uint32_t px, py, pz;
+      morton_decode(pk - cloud_bits, d - 1, &px, &py, &pz);
+      const int nx = (int)px + ox, ny = (int)py + oy, nz = (int)pz + oz;
+      inside[q] = pl < 27 && nx >= 0 && ny >= 0 && nz >= 0 && ((nx | ny | nz) >> (d - 1)) == 0;
+      want[q] = cloud_bits | morton_encode((uint32_t)max(nx, 0), (uint32_t)max(ny, 0), (uint32_t)max(nz, 0), d - 1);
+      lo[q] = 0;
+      hi[q] = inside[q] ? n_par : 0;   // an empty range: nothing is looked up
     }
-    reinterpret_cast<int*>(blob + a.off_neigh[d])[((int64_t)g << 6) + lane] = v;
+    for (int span = n_par; span > 0; span >>= 1) {   // enough halvings for every search
+      uint64_t v[2];
+#pragma unroll
+      for (int q = 0; q < 2; ++q) v[q] = lo[q] < hi[q] ? list[(lo[q] + hi[q]) >> 1] : 0;
+#pragma unroll
+      for (int q = 0; q < 2; ++q)
+        if (lo[q] < hi[q]) {
+          const int mid = (lo[q] + hi[q]) >> 1;
+          if (v[q] < want[q]) lo[q] = mid + 1; else hi[q] = mid;
+        }
+    }
+    int rank[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const uint64_t at = list[min(lo[q], n_par - 1)];
+      rank[q] = inside[q] && lo[q] < n_par && at == want[q] ? lo[q] : -1;
+    }
+    // slot (x, y, z) of a group = the node at (x - 1, y - 1, z - 1) from sibling 0: its parent is
+    // the one at ((x + 1) >> 1) - 1 ... from the group's parent, its octant the low bits of x + 1 ...
+    const int sx = lane >> 4, sy = (lane >> 2) & 3, sz = lane & 3;
+    const int from = ((sx + 1) >> 1) * 9 + ((sy + 1) >> 1) * 3 + ((sz + 1) >> 1);
+    const int oct = (((sx + 1) & 1) << 2) | (((sy + 1) & 1) << 1) | ((sz + 1) & 1);
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int r = __shfl(rank[q], from + 32 * h, 64);
+        const int g = g0 + 2 * q + h;
+        if (g < n_par) reinterpret_cast<int*>(blob + a.off_neigh[d])[((int64_t)g << 6) + lane] = r < 0 ? -1 : 8 * r + oct;
+      }
     return;
   }
   uint64_t* key = reinterpret_cast<uint64_t*>(blob + a.off_key[d]);
@@ -1305,13 +1350,22 @@ int ocnn_points2octree_emit(void* octree_out_dev, const void* info, void* worksp
     blocks += (int)nblocks;
   };
   add_seg(kSegHeader, 0, 1);
-  // the signal of the finest level first: its workgroups take longest
+  // the searched neighbour tables first (their divergent loads then run beside the workgroups
+  // below, which mostly wait for memory), then the signal of the finest level: its workgroups
+  // take longest
+  int searched_to = fl;  // sparse levels up to here have their neighbour table after this launch
+  if (o.has(OCNN_NEIGH))
+    for (int d = fl + 1; d <= depth && st.nne[d - 1] > 0 && st.nne[d - 1] <= kSearchGroups; ++d) {
+      add_seg(kSegNeighSearch, d, blocks_for(st.nne[d - 1], (kBlock / 64) * kSearchPerWave));
+      searched_to = d;
+    }
   const bool has_signal = depth > fl && HD > 0 && (a.off_feature >= 0 || a.off_label >= 0);
   const bool signal_inside = has_signal && fch <= kSignalStage;
   size_t lds = kEmitLdsBytes;
   if (signal_inside) {
     add_seg(kSegLeafSignal, depth, blocks_for(HD, kSignalTile));
-    const size_t need = sizeof(float) * kSignalTile * (size_t)(fch + (a.off_label >= 0 ? 1 : 0)) + sizeof(unsigned short) * kSignalTile;
+    const size_t need = sizeof(float) * kSignalTile * (size_t)(fch + (a.off_label >= 0 ? 1 : 0)) +
+        sizeof(int) * (kSignalTile + 2) + sizeof(unsigned short) * kSignalTile * (B > 1 ? 2 : 1);
     if (need > lds) lds = need;
   }
   for (int d = depth; d > fl; --d) add_seg(kSegSparse, d, blocks_for(st.nne[d - 1]) * (st.nne[d - 1] > 0 ? 1 : 0));
@@ -1319,12 +1373,6 @@ int ocnn_points2octree_emit(void* octree_out_dev, const void* info, void* worksp
     add_seg(kSegFull, d, blocks_for(o.nnum[d]));
     if (o.has(OCNN_NEIGH) && d >= 1) add_seg(kSegFullNeigh, d, blocks_for((int64_t)B << (3 * d + 3)));
   }
-  int searched_to = fl;  // sparse levels up to here have their neighbour table after this launch
-  if (o.has(OCNN_NEIGH))
-    for (int d = fl + 1; d <= depth && st.nne[d - 1] > 0 && st.nne[d - 1] <= kSearchGroups; ++d) {
-      add_seg(kSegNeighSearch, d, blocks_for(st.nne[d - 1], kBlock / 64));
-      searched_to = d;
-    }
   a.seg_begin[n_seg] = blocks;
   a.n_seg = n_seg;
   emit_kernel<<<blocks, kBlock, lds, s>>>(blob, a);
