@@ -569,7 +569,7 @@ __device__ inline void leaf_signal(float* __restrict__ feature, float* __restric
   const int64_t H = g.nnum_d;
   float* out = feature + node;  // channel c lives at out[c * H]
   // one pass over the points: every attribute of a point is requested together
-  constexpr int kRegFeatures = 8;
+  constexpr int kRegFeatures = 4;
   const int F = cd.feature ? g.ch_feature : 0;
   const bool need_pt = g.has_dis || g.save_pts;
   float acc[3] = {0.0f, 0.0f, 0.0f}, avg_pt[3] = {0.0f, 0.0f, 0.0f}, facc[kRegFeatures];
@@ -710,31 +710,40 @@ struct EmitArgs {
 };
 static_assert(sizeof(EmitArgs) <= 3800, "kernel arguments must stay below 4 KiB");
 
-// Signal of the finest level for a tile of kSignalTile consecutive nodes, through LDS.  The
-// non-empty nodes of the tile are consecutive leaves (ranks grow with the node index), so
-// threads 0 .. count-1 take one leaf each -- dense wavefronts for the point gathers, where one
-// thread per node keeps one lane in seven busy at depth 9 -- and put the result into an LDS
-// image of the tile's rows, which is then written out in full rows (zeros, label -1, for the
-// empty nodes: every row of the block is written exactly once).  Which leaf sits in which node
-// is read off the level lists (node 8 p + octant for the leaves first[p] .. first[p + 1] of the
-// p-th sibling group), not off the child links: the tile waits for no other part of the blob
-// and runs inside the launch that writes those.  Needs channels <= kSignalStage.
-// (Tried and dropped: tiles of 512 nodes, 3-5 % slower; one thread per non-empty leaf writing a
-// compact table that a second launch expands into the rows, 15 % slower on eight scenes: the
-// expansion alone took as long as this tile kernel.)
+// Signal of the finest level for a tile of kSignalTile consecutive nodes.  The non-empty nodes
+// of the tile are consecutive leaves (ranks grow with the node index), so threads 0 .. count-1
+// take one leaf each -- dense wavefronts for the point gathers, where one thread per node keeps
+// one lane in seven busy at depth 9 -- and leave the result in a compact LDS table (one column
+// per leaf, kBlock leaves a round; a tile with more leaves takes more rounds).  The rows are then
+// written out in full: every node looks up its leaf (or writes zeros, label -1), so every row of
+// the block is written exactly once.  Which leaf sits in which node is read off the level lists
+// (node 8 p + octant for the leaves first[p] .. first[p + 1] of the p-th sibling group), not off
+// the child links: the tile waits for no other part of the blob and runs inside the launch that
+// writes those.  Needs channels <= kSignalStage.  LDS per tile: 1 KiB per channel + 8-10 KiB --
+// the launch is bound by how many workgroups are resident, not by bytes.
+// (Tried and dropped: an LDS image of the tile's full rows, 4 KiB per channel: five workgroups
+// per CU; tiles of 512 nodes, 3-5 % slower; one thread per non-empty leaf writing a compact
+// table that a second launch expands into the rows, 15 % slower on eight scenes.)
 constexpr int kSignalTile = 1024, kSignalStage = 8;
+constexpr int kSignalRounds = kSignalTile / kBlock;
+__host__ __device__ inline size_t signal_lds_bytes(int channels, bool has_label, bool batch) {
+  return sizeof(float) * kBlock * (size_t)(channels + (has_label ? 1 : 0)) + sizeof(int) * (kSignalTile + 2) +
+      sizeof(int) * (kSignalRounds + 2) + sizeof(unsigned short) * kSignalTile * (batch ? 2 : 1);
+}
 __device__ inline void leaf_signal_tile(char* __restrict__ blob, const EmitArgs& a, int block, unsigned char* s_raw) {
   const SignalGeom& g = a.sg;
   float* feature = a.off_feature >= 0 ? reinterpret_cast<float*>(blob + a.off_feature) : nullptr;
   float* label = a.off_label >= 0 ? reinterpret_cast<float*>(blob + a.off_label) : nullptr;
-  // [channels][kSignalTile] rows, labels, then per leaf: its first point (one more entry closes
-  // the last leaf), its node inside the tile and, for a batch, its cloud
-  float* s_out = reinterpret_cast<float*>(s_raw);
-  float* s_label = s_out + (size_t)g.channels * kSignalTile;
-  int* s_start = reinterpret_cast<int*>(s_label + (label ? kSignalTile : 0));
-  unsigned short* s_node = reinterpret_cast<unsigned short*>(s_start + kSignalTile + 2);
-  unsigned short* s_cloud = s_node + kSignalTile;
   const bool batch = a.n_clouds > 1;
+  // [channels (+ label)][kBlock] values of a round's leaves; per leaf its first point (one more
+  // entry closes the last leaf); the node of every kBlock-th leaf; per node its leaf (0xffff:
+  // none); per leaf its cloud (batches only)
+  float* s_val = reinterpret_cast<float*>(s_raw);
+  float* s_lab = s_val + (size_t)g.channels * kBlock;
+  int* s_start = reinterpret_cast<int*>(s_lab + (label ? kBlock : 0));
+  int* s_bound = s_start + kSignalTile + 2;
+  unsigned short* s_leaf = reinterpret_cast<unsigned short*>(s_bound + kSignalRounds + 2);
+  unsigned short* s_cloud = s_leaf + kSignalTile;
   const int tid = threadIdx.x;
   const int node0 = block * kSignalTile;
   const int rows = min(kSignalTile, g.nnum_d - node0);
@@ -742,15 +751,26 @@ __device__ inline void leaf_signal_tile(char* __restrict__ blob, const EmitArgs&
   const int* __restrict__ first = a.first[g.depth - 1];
   const uint64_t* __restrict__ leaf_key = a.list[g.depth];
   const int j0 = first[p0], count = first[p0 + n_groups] - j0;
-  for (int i = tid; i < g.channels * kSignalTile; i += kBlock) s_out[i] = 0.0f;
-  if (label)
-    for (int i = tid; i < kSignalTile; i += kBlock) s_label[i] = -1.0f;
   for (int t = tid; t < n_groups; t += kBlock) {
     const int c0 = first[p0 + t], c1 = first[p0 + t + 1];
-    for (int j = c0; j < c1; ++j) {
-      const uint64_t lk = leaf_key[j];
-      s_node[j - j0] = (unsigned short)(t * 8 + (int)(lk & 7));
-      if (batch) s_cloud[j - j0] = (unsigned short)(lk >> (3 * g.depth));
+    int oct[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      oct[u] = 8;
+      if (c0 + u < c1) {
+        const uint64_t lk = leaf_key[c0 + u];
+        oct[u] = (int)(lk & 7);
+        const int l = c0 + u - j0;
+        if (batch) s_cloud[l] = (unsigned short)(lk >> (3 * g.depth));
+        if ((l & (kBlock - 1)) == 0) s_bound[l / kBlock] = t * 8 + oct[u];
+      }
+    }
+#pragma unroll
+    for (int o = 0; o < 8; ++o) {
+      int l = 0xffff;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) l = oct[u] == o ? c0 + u - j0 : l;
+      s_leaf[t * 8 + o] = (unsigned short)l;
     }
   }
   // the leaves' point ranges, requested with the keys above: a leaf then starts with its points'
@@ -758,23 +778,36 @@ __device__ inline void leaf_signal_tile(char* __restrict__ blob, const EmitArgs&
   for (int t = tid; t <= count; t += kBlock) s_start[t] = a.ustart[j0 + t];
   __syncthreads();
   SignalGeom lg = g;
-  lg.nnum_d = kSignalTile;   // row length of the LDS image
-  for (int t = tid; t < count; t += kBlock)
-    leaf_signal(s_out, label ? s_label : nullptr, (int)s_node[t], batch ? (int)s_cloud[t] : 0, s_start[t],
-        s_start[t + 1], a.sorted_idx, a.clouds, lg);
-  __syncthreads();
-  for (int ch = 0; ch < g.channels; ++ch)
-    for (int r = tid; r < rows; r += kBlock) feature[(int64_t)ch * g.nnum_d + node0 + r] = s_out[ch * kSignalTile + r];
-  if (label)
-    for (int r = tid; r < rows; r += kBlock) label[node0 + r] = s_label[r];
+  lg.nnum_d = kBlock;   // row length of the LDS table
+  for (int r0 = 0; r0 == 0 || r0 < count; r0 += kBlock) {
+    const int t = r0 + tid;
+    if (label) s_lab[tid] = -1.0f;
+    if (t < count)
+      leaf_signal(s_val, label ? s_lab : nullptr, tid, batch ? (int)s_cloud[t] : 0, s_start[t], s_start[t + 1],
+          a.sorted_idx, a.clouds, lg);
+    __syncthreads();
+    // nodes of this round: from the node of its first leaf (the tile's first node in round 0) up to
+    // the node of the next round's first leaf (the end of the tile after the last round)
+    const int n_lo = r0 == 0 ? 0 : s_bound[r0 / kBlock];
+    const int n_hi = r0 + kBlock < count ? s_bound[r0 / kBlock + 1] : rows;
+    for (int r = n_lo + tid; r < n_hi; r += kBlock) {
+      const int l = (int)s_leaf[r] - r0;          // 0xffff - r0 >= kBlock: an empty node
+      const bool leaf = l < kBlock;
+      for (int ch = 0; ch < g.channels; ++ch)
+        feature[(int64_t)ch * g.nnum_d + node0 + r] = leaf ? s_val[ch * kBlock + l] : 0.0f;
+      if (label) label[node0 + r] = leaf ? s_lab[l] : -1.0f;
+    }
+    if (r0 + kBlock < count) __syncthreads();     // the table is reused
+  }
 }
 
-constexpr size_t kEmitLdsBytes = (size_t)kBlock * 8 * (sizeof(uint64_t) + sizeof(int));
+// a sparse segment stages the parent key of each of its kBlock sibling groups and the child links
+constexpr size_t kEmitLdsBytes = (size_t)kBlock * (sizeof(uint64_t) + 8 * sizeof(int));
 
-__global__ __launch_bounds__(kBlock) void emit_kernel(char* __restrict__ blob, const EmitArgs a) {
+__global__ __launch_bounds__(kBlock, 8) void emit_kernel(char* __restrict__ blob, const EmitArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char s_raw[];   // max(kEmitLdsBytes, a signal tile)
-  uint64_t* s_key = reinterpret_cast<uint64_t*>(s_raw);
-  int* s_child = reinterpret_cast<int*>(s_raw + sizeof(uint64_t) * kBlock * 8);
+  uint64_t* s_parent = reinterpret_cast<uint64_t*>(s_raw);
+  int* s_child = reinterpret_cast<int*>(s_raw + sizeof(uint64_t) * kBlock);
   int seg = 0;
   while (seg + 1 < a.n_seg && (int)blockIdx.x >= a.seg_begin[seg + 1]) ++seg;
   const int kind = a.seg_kind[seg], d = a.seg_level[seg];
@@ -911,13 +944,12 @@ __global__ __launch_bounds__(kBlock) void emit_kernel(char* __restrict__ blob, c
   }
   // sparse layers: thread = sibling group p (the children of the p-th non-empty node of level
   // d-1): node 8p + octant, key from the parent's key; the non-empty ones are consecutive in
-  // list[d] from first[d-1][p]
+  // list[d] from first[d-1][p].  Parent keys and child links are staged in LDS so that the nodes
+  // leave in full rows.
   const int groups = a.nne[d - 1];
   const int p = block * kBlock + tid;
   if (p < groups) {
-    const uint64_t pk = a.list[d - 1][p];     // cloud << 3(d-1) | morton_{d-1}
-    const int cloud = (int)(pk >> (3 * (d - 1)));
-    const uint64_t pm = pk & ((1ull << (3 * (d - 1))) - 1);
+    s_parent[tid] = a.list[d - 1][p];     // cloud << 3(d-1) | morton_{d-1}
     const int c0 = a.first[d - 1][p], c1 = a.first[d - 1][p + 1];
     int oct[8];
 #pragma unroll
@@ -928,14 +960,15 @@ __global__ __launch_bounds__(kBlock) void emit_kernel(char* __restrict__ blob, c
 #pragma unroll
       for (int u = 0; u < 8; ++u) c = oct[u] == o ? c0 + u : c;
       s_child[tid * 8 + o] = c;
-      s_key[tid * 8 + o] = out_key((pm << 3) | (uint64_t)o, d, cloud, a.key2xyz);
     }
   }
   __syncthreads();
   const int64_t node0 = (int64_t)block * kBlock * 8;
   const int rows = min(kBlock * 8, n_d - (int)node0);  // nodes of this workgroup
+  const uint64_t pmask = (1ull << (3 * (d - 1))) - 1;
   for (int r = tid; r < rows; r += kBlock) {
-    key[node0 + r] = s_key[r];
+    const uint64_t pk = s_parent[r >> 3];
+    key[node0 + r] = out_key(((pk & pmask) << 3) | (uint64_t)(r & 7), d, (int)(pk >> (3 * (d - 1))), a.key2xyz);
     if (a.key_channel == 2) key[n_d + node0 + r] = 0;
     const int c = s_child[r];
     child[node0 + r] = c;
@@ -1364,8 +1397,7 @@ int ocnn_points2octree_emit(void* octree_out_dev, const void* info, void* worksp
   size_t lds = kEmitLdsBytes;
   if (signal_inside) {
     add_seg(kSegLeafSignal, depth, blocks_for(HD, kSignalTile));
-    const size_t need = sizeof(float) * kSignalTile * (size_t)(fch + (a.off_label >= 0 ? 1 : 0)) +
-        sizeof(int) * (kSignalTile + 2) + sizeof(unsigned short) * kSignalTile * (B > 1 ? 2 : 1);
+    const size_t need = signal_lds_bytes(fch, a.off_label >= 0, B > 1);
     if (need > lds) lds = need;
   }
   for (int d = depth; d > fl; --d) add_seg(kSegSparse, d, blocks_for(st.nne[d - 1]) * (st.nne[d - 1] > 0 ? 1 : 0));

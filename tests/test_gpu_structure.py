@@ -101,6 +101,31 @@ def test_build_wide_features_and_many_clouds(oc, orc):
   assert np.array_equal(got, orc.octree_batch([orc.points2octree(b, 5, 2) for b in blobs]))
 
 
+def test_build_dense_tiles_and_feature_overflow(oc, orc):
+  """A signal tile (1024 nodes) stages 256 leaves a round: dense levels take several rounds, with
+  labels and a batch's cloud table in LDS beside them; five feature channels are one more than
+  the leaf loop keeps in registers while the tile still stages them (at most 8 channels)."""
+  rng = np.random.default_rng(33)
+  n = 6000
+  pts = rng.uniform(-0.999, 0.999, (n, 3)).astype(np.float32)
+  nrm = rng.standard_normal((n, 3)).astype(np.float32)
+  lab = rng.integers(0, 5, n).astype(np.float32)
+  dense = make_points_blob(pts, nrm, rng.uniform(0, 1, (n, 3)).astype(np.float32), lab)
+  five = make_points_blob(pts, None, rng.uniform(0, 1, (n, 5)).astype(np.float32), lab)
+  for pb in (dense, five):
+    for depth, fd in ((4, 2), (5, 3), (4, 1)):   # 4096 / 32768 nodes at the finest level, most of them leaves at depth 4
+      got = oc.nn.points2octree(T(pb), depth, fd, node_dis=True).cpu().numpy()
+      assert np.array_equal(got, orc.points2octree(pb, depth, fd, node_dis=True)), (depth, fd)
+  blobs = []
+  for i in range(5):
+    m = int(rng.integers(2000, 5000))
+    blobs.append(make_points_blob(rng.uniform(-0.999, 0.999, (m, 3)).astype(np.float32),
+                                  rng.standard_normal((m, 3)).astype(np.float32),
+                                  rng.uniform(0, 1, (m, 2)).astype(np.float32), rng.integers(0, 3, m).astype(np.float32)))
+  got = oc.nn.points2octree_batch([T(b) for b in blobs], 4, 2).cpu().numpy()
+  assert np.array_equal(got, orc.octree_batch([orc.points2octree(b, 4, 2) for b in blobs]))
+
+
 def test_build_two_steps_and_ticket_repeat(oc, orc, synthetic):
   """The plan / emit pair gives the blob of the one-call entry point; a first attempt that is
   made to fail from the host is repeated with ticket order and gives the same blob."""
