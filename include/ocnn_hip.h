@@ -185,6 +185,28 @@ int ocnn_octree_conv_fused(void* top, const void* btm, int channel_in, int btm_h
     int num_output, const int* kernel_size, int stride, int nempty, int dtype, void* workspace_dev,
     size_t workspace_bytes, ocnn_stream_t stream);
 
+/* Row-major activations, no counterpart in the reference (whose tensors are channel-major
+ * [1, C, H, 1]): rows [H + 1][pitch] bf16, row h = the channels of node h, pitch = channels
+ * rounded up to a multiple of 16, padding channels zero, row H all zero (what a missing
+ * neighbour reads).  It is the layout the bf16 3x3x3 kernels gather from; the channel-major entry
+ * points copy their input into it on every call.  A chain of convolutions converts once
+ * (ocnn_rows_from_channels), runs ocnn_octree_conv_rows for every member, and converts back once
+ * (ocnn_channels_from_rows).
+ *   ocnn_octree_conv_rows: bf16, kernel 3x3x3, stride 1, nempty 0 (anything else:
+ *   OCNN_E_UNSUPPORTED); arithmetic and rounding as ocnn_octree_conv_fused, the results are
+ *   bit-identical.  btm_pitch = 16 * ceil(channel_in / 16); top_pitch a multiple of 16 with
+ *   num_output <= top_pitch <= 32 * ceil(num_output / 32); the call writes the padding channels
+ *   and the zero row of `top_rows` too.  Workspace: as ocnn_conv_shape says (the packed weights
+ *   are all it uses). */
+int ocnn_octree_conv_rows(void* top_rows, int top_pitch, const void* btm_rows, int btm_pitch, int channel_in,
+    int btm_h, const void* weights, const float* bias, int relu, int is_deconv, const void* octree_dev,
+    const void* info, int depth, int num_output, const int* kernel_size, int stride, int nempty, int dtype,
+    void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream);
+int ocnn_rows_from_channels(void* rows, int pitch, const void* data, int channel, int height, int dtype,
+    ocnn_stream_t stream);
+int ocnn_channels_from_rows(void* data, const void* rows, int pitch, int channel, int height, int dtype,
+    ocnn_stream_t stream);
+
 /* Tuning knob, no counterpart in the reference: 3x3x3 stride-1 bf16 convolutions over all nodes
  * run one of two kernels, chosen by the number of 1024-column tiles of the level; the
  * register-fed kernel takes levels of at least `tiles` tiles (default 192, about 200 000

@@ -747,6 +747,36 @@ __global__ __launch_bounds__(256) void transpose_rows_bf16_kernel(uint16_t* __re
   }
 }
 
+// The inverse copy: row-major src [H + 1, pitch] -> channel-major dst [C, H] (64 rows x 64
+// channels per workgroup; 16-byte reads of 8 channels of a row, 4-byte writes of two rows of a
+// channel, coalesced per channel row).
+__global__ __launch_bounds__(256) void transpose_channels_bf16_kernel(uint16_t* __restrict__ dst,
+    const uint16_t* __restrict__ src, int C, int H, int pitch) {
+  constexpr int kPitch = 66;  // halfwords per channel row of the tile
+  __shared__ uint16_t tile[64 * kPitch];
+  const int h0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+  const int t = threadIdx.x;
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int hl = pass * 32 + (t >> 3), cg = t & 7;
+    const int h = h0 + hl, c = c0 + cg * 8;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (h < H && c < pitch) v = *reinterpret_cast<const uint4*>(src + (int64_t)h * pitch + c);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      tile[(cg * 8 + 2 * j) * kPitch + hl] = (uint16_t)(w[j] & 0xffff);
+      tile[(cg * 8 + 2 * j + 1) * kPitch + hl] = (uint16_t)(w[j] >> 16);
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int pass = 0; pass < 16; ++pass) {
+    const int cl = pass * 4 + (t >> 6), c = c0 + cl, h = h0 + (t & 63);
+    if (c < C && h < H) dst[(int64_t)c * H + h] = tile[cl * kPitch + (t & 63)];
+  }
+}
+
 template <int MT>
 __global__ __launch_bounds__(256, 2) void conv_s1_bf16_lds_kernel(ConvArgs a, uint16_t* __restrict__ out,
     const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles, int cpad8) {
@@ -907,9 +937,12 @@ constexpr int kRegGroups = 32;               // sibling groups (MFMA columns) pe
 constexpr int kRegTileGroups = 4 * kRegGroups;
 constexpr int kNbPitch = 68;
 
-template <int MT>
+// ROWS_OUT: the output is written row-major as well ([Hout + 1][out_pitch] bf16, row Hout zero,
+// channels from M up to the pitch zero), the layout the next convolution of a chain gathers
+// from: 32 contiguous bytes per row and store instead of 16 bytes per channel and group.
+template <int MT, bool ROWS_OUT>
 __global__ __launch_bounds__(256, 1) void conv_s1_bf16_reg_kernel(ConvArgs a, uint16_t* __restrict__ out,
-    const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles, int cpad8) {
+    const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles, int cpad8, int out_pitch) {
   constexpr int kWUnits = 27 * MT * 64;        // 16-byte units of one k-step's weights
   constexpr int kWPiece = kWUnits / 4;         // copied per layer phase
   constexpr int kWVec = (kWPiece + 255) / 256;
@@ -1084,8 +1117,63 @@ __global__ __launch_bounds__(256, 1) void conv_s1_bf16_reg_kernel(ConvArgs a, ui
     }
     wbase = (wbase + nks) & 1;
 
-    // one 16-byte store per output channel: the 8 columns of a group are contiguous
     const int g = g0 + n;
+    if constexpr (ROWS_OUT) {
+      // Lane (n, kh) holds channels cb + 32 mt + 8 q + 4 kh + r (q, r = 0..3) of the 8 rows of its
+      // group.  The two lanes of a group swap halves (lanes 0-31 against 32-63), so that kh = 0 ends
+      // up with channels 16 j .. + 7 and kh = 1 with 16 j + 8 .. + 15 of (mt, j): one 16-byte store
+      // each, 32 contiguous bytes per row.
+      const int cb = pass * MT * 32;
+      // stores through a buffer: a lane whose group lies behind the level gets an offset past the
+      // end and the hardware drops its store (no branch per store); the offsets have 32 bits (the
+      // host sends larger outputs elsewhere)
+      const __amdgpu_buffer_rsrc_t obuf = __builtin_amdgcn_make_buffer_rsrc(
+          out, 0, (int)(((int64_t)a.Hout + 1) * out_pitch * 2), 0x00020000);
+      const int obase = g < n_groups ? (g * 8 * out_pitch + cb + 8 * kh) * 2 : 0x7fffff00;
+      auto store_rows = [&](auto value) {   // value(sb, mt, i): what goes out for accumulator i
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int sb = 0; sb < 8; ++sb) {
+            uint32_t w[4][2];
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+              for (int h = 0; h < 2; ++h)
+                w[q][h] = pack_bf16x2(value(sb, mt, 4 * q + 2 * h), value(sb, mt, 4 * q + 2 * h + 1));
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              const auto s0 = __builtin_amdgcn_permlane32_swap(w[2 * j][0], w[2 * j + 1][0], false, false);
+              const auto s1 = __builtin_amdgcn_permlane32_swap(w[2 * j][1], w[2 * j + 1][1], false, false);
+              // channels cb + 32 mt + 16 j .. + 15 (8 in each lane of the pair): inside the pitch or not
+              // for the whole wavefront
+              if (cb + 32 * mt + 16 * j < out_pitch)
+                __builtin_amdgcn_raw_buffer_store_b128(u32x4{s0[0], s1[0], s0[1], s1[1]}, obuf, obase,
+                    (sb * out_pitch + 32 * mt + 16 * j) * 2, 0);
+            }
+          }
+      };
+      if (!a.bias && !a.relu) {
+        store_rows([&](int sb, int mt, int i) { return acc[sb][mt][i]; });
+      } else {
+        const float floor = a.relu ? 0.0f : -__builtin_inff();
+        float bias[MT][16];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int ch = m0 + 32 * mt + 8 * (i / 4) + (i % 4);
+            bias[mt][i] = a.bias ? a.bias[min(ch, a.M - 1)] : 0.0f;
+            if (ch >= a.M) bias[mt][i] = 0.0f;   // the padding channels of a row stay zero
+          }
+        store_rows([&](int sb, int mt, int i) { return relu_floor(acc[sb][mt][i] + bias[mt][i], floor); });
+      }
+      // the all-zero row behind the last one (what a missing neighbour reads): once per pass range
+      if (tile == 0 && wave == 0 && lane * 8 < out_pitch && lane * 8 >= cb && lane * 8 < cb + MT * 32)
+        *reinterpret_cast<uint4*>(out + (int64_t)a.Hout * out_pitch + lane * 8) = make_uint4(0, 0, 0, 0);
+      continue;
+    }
+    // one 16-byte store per output channel: the 8 columns of a group are contiguous
     uint16_t* orow = out + (int64_t)g * 8 + (int64_t)m0 * a.Hout;
     const int m_left = g < n_groups ? a.M - m0 : 0;   // rows of mine that exist
     // Straight-line code; the conversion is the hardware's (round to nearest even).  The plain
@@ -1865,9 +1953,9 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     if (use_reg) {
       const int r_grid = ((r_tiles + 7) / 8) * 8;
       if (MT == 1)
-        conv_s1_bf16_reg_kernel<1><<<dim3(r_grid, pass_split(r_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, r_tiles, cpad / 8);
+        conv_s1_bf16_reg_kernel<1, false><<<dim3(r_grid, pass_split(r_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, r_tiles, cpad / 8, 0);
       else
-        conv_s1_bf16_reg_kernel<2><<<dim3(r_grid, pass_split(r_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, r_tiles, cpad / 8);
+        conv_s1_bf16_reg_kernel<2, false><<<dim3(r_grid, pass_split(r_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, r_tiles, cpad / 8, 0);
     } else if (MT == 1)
       conv_s1_bf16_lds_kernel<1><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad / 8);
     else
@@ -2441,6 +2529,75 @@ int builtin_scratch(void** out) {
   return OCNN_OK;
 }
 
+// 3x3x3 stride-1 convolution (or deconvolution) over all nodes of a level in bf16, input and
+// output row-major: what a chain of such convolutions keeps between its members instead of
+// copying every input row-major first.  Only the packed weights need workspace.
+int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_rows, int btm_pitch, int channel_in,
+    int btm_h, const void* weights, const float* bias, int relu, const void* octree_dev, const void* info,
+    int depth, int num_output, const int* ks, int stride, int nempty, int dtype, void* ws, size_t ws_bytes,
+    hipStream_t s) {
+  OCNN_REQUIRE(top_rows && btm_rows && weights && octree_dev && info && ks, OCNN_E_BADARG, "null pointer");
+  OCNN_REQUIRE(dtype == OCNN_BF16 && stride == 1 && !nempty && ks[0] == 3 && ks[1] == 3 && ks[2] == 3,
+      OCNN_E_UNSUPPORTED, "row-major convolutions: bf16, 3x3x3, stride 1, all nodes");
+  const Info* o = as_info(info);
+  ConvPlan p;
+  int e = make_plan(o, depth, channel_in, num_output, ks, stride, nempty, deconv, dtype, &p);
+  if (e) return e;
+  OCNN_REQUIRE(btm_h == p.btm_h, OCNN_E_SHAPE, "input height %d, the octree has %d rows at depth %d", btm_h,
+      p.btm_h, depth);
+  const int cpad = (channel_in + 15) / 16 * 16;
+  OCNN_REQUIRE(btm_pitch == cpad, OCNN_E_SHAPE, "input pitch %d: rows of %d channels are padded to %d", btm_pitch,
+      channel_in, cpad);
+  OCNN_REQUIRE(top_pitch >= num_output && top_pitch % 16 == 0 && top_pitch <= (num_output + 31) / 32 * 32,
+      OCNN_E_SHAPE, "output pitch %d for %d channels", top_pitch, num_output);
+  OCNN_REQUIRE(((reinterpret_cast<uintptr_t>(top_rows) | reinterpret_cast<uintptr_t>(btm_rows)) & 15) == 0,
+      OCNN_E_BADARG, "rows not 16-byte aligned");
+  OCNN_REQUIRE(((int64_t)btm_h + 1) * cpad * 2 < ((int64_t)1 << 31) &&
+      ((int64_t)p.top_h + 1) * top_pitch * 2 < ((int64_t)1 << 31) - (1 << 20), OCNN_E_UNSUPPORTED,
+      "level too large for 32-bit row offsets");
+  OCNN_REQUIRE(ws && ws_bytes >= p.wt_bytes, OCNN_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes, p.wt_bytes);
+  OCNN_REQUIRE((reinterpret_cast<uintptr_t>(ws) & 15) == 0, OCNN_E_WORKSPACE, "workspace not 16-byte aligned");
+  const char* blob = static_cast<const char*>(octree_dev);
+  ConvArgs a;
+  a.M = num_output;
+  a.Cin = channel_in;
+  a.N = p.top_h;
+  a.K = 27;
+  a.Hin = btm_h;
+  a.Hout = p.top_h;
+  a.mode = kModeS1;
+  a.nempty = 0;
+  a.mtiles = p.mtiles;
+  a.csteps = 0;
+  for (int k = 0; k < 27; ++k) a.slot[k] = tap_slot(deconv ? 26 - p.taps.tap[k] : p.taps.tap[k]);
+  a.neigh = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_NEIGH, depth));
+  a.child = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_CHILD, depth));
+  a.ichild = nullptr;
+  a.bias = bias;
+  a.relu = relu ? 1 : 0;
+  if (o->nnum[depth] == 0) {   // a level without nodes: one zero row, and the zero row behind it
+    zero_rows_kernel<uint16_t><<<blocks_for(2 * (int64_t)top_pitch), kBlock, 0, s>>>((uint16_t*)top_rows, 2 * (int64_t)top_pitch);
+    OCNN_LAUNCH_OK("zero_rows");
+    return OCNN_OK;
+  }
+  const int64_t sm = deconv ? 27 : (int64_t)channel_in * 27, sc = deconv ? (int64_t)num_output * 27 : 27;
+  const int MT = a.mtiles == 1 ? 1 : 2;
+  const int npass = (a.mtiles + MT - 1) / MT, nslab = cpad / 16;
+  const int64_t total = (int64_t)npass * nslab * 27 * MT * 64 * 8;
+  pack_weights_lds_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)ws, (const uint16_t*)weights, a.M, a.Cin, MT,
+      npass, nslab, sm, sc, deconv);
+  const int r_tiles = ((a.N >> 3) + kRegTileGroups - 1) / kRegTileGroups;
+  const int r_grid = ((r_tiles + 7) / 8) * 8;
+  if (MT == 1)
+    conv_s1_bf16_reg_kernel<1, true><<<dim3(r_grid, pass_split(r_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top_rows,
+        (const u32x4*)btm_rows, (const u32x4*)ws, r_tiles, cpad / 8, top_pitch);
+  else
+    conv_s1_bf16_reg_kernel<2, true><<<dim3(r_grid, pass_split(r_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top_rows,
+        (const u32x4*)btm_rows, (const u32x4*)ws, r_tiles, cpad / 8, top_pitch);
+  OCNN_LAUNCH_OK("octree_conv_rows");
+  return OCNN_OK;
+}
+
 // called by ocnn_device_check so that set-up code can resolve the address ahead of the first call
 int prepare_builtin_scratch() {
   void* ptr = nullptr;
@@ -2501,6 +2658,44 @@ int ocnn_octree_conv_fused(void* top, const void* btm, int channel_in, int btm_h
     size_t workspace_bytes, ocnn_stream_t stream) {
   return run_conv(is_deconv ? 1 : 0, top, btm, channel_in, btm_h, weights, octree_dev, info, depth, num_output,
       kernel_size, stride, nempty, dtype, workspace_dev, workspace_bytes, as_stream(stream), bias, relu);
+}
+
+int ocnn_octree_conv_rows(void* top_rows, int top_pitch, const void* btm_rows, int btm_pitch, int channel_in,
+    int btm_h, const void* weights, const float* bias, int relu, int is_deconv, const void* octree_dev,
+    const void* info, int depth, int num_output, const int* kernel_size, int stride, int nempty, int dtype,
+    void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream) {
+  return run_conv_rows(is_deconv ? 1 : 0, top_rows, top_pitch, btm_rows, btm_pitch, channel_in, btm_h, weights, bias,
+      relu, octree_dev, info, depth, num_output, kernel_size, stride, nempty, dtype, workspace_dev, workspace_bytes,
+      as_stream(stream));
+}
+
+int ocnn_rows_from_channels(void* rows, int pitch, const void* data, int channel, int height, int dtype,
+    ocnn_stream_t stream) {
+  OCNN_REQUIRE(rows && data, OCNN_E_BADARG, "null pointer");
+  OCNN_REQUIRE(dtype == OCNN_BF16, OCNN_E_UNSUPPORTED, "row-major copies: bf16");
+  OCNN_REQUIRE(channel > 0 && height >= 0 && pitch == (channel + 15) / 16 * 16, OCNN_E_SHAPE,
+      "pitch %d for %d channels", pitch, channel);
+  OCNN_REQUIRE((reinterpret_cast<uintptr_t>(rows) & 15) == 0, OCNN_E_BADARG, "rows not 16-byte aligned");
+  dim3 grid((height + 1 + 127) / 128, (pitch + 63) / 64);
+  transpose_rows_bf16_kernel<<<grid, 256, 0, as_stream(stream)>>>((uint16_t*)rows, (const uint16_t*)data, channel,
+      height, pitch);
+  OCNN_LAUNCH_OK("rows_from_channels");
+  return OCNN_OK;
+}
+
+int ocnn_channels_from_rows(void* data, const void* rows, int pitch, int channel, int height, int dtype,
+    ocnn_stream_t stream) {
+  OCNN_REQUIRE(rows && data, OCNN_E_BADARG, "null pointer");
+  OCNN_REQUIRE(dtype == OCNN_BF16, OCNN_E_UNSUPPORTED, "row-major copies: bf16");
+  OCNN_REQUIRE(channel > 0 && height >= 0 && pitch >= channel && pitch % 8 == 0, OCNN_E_SHAPE,
+      "pitch %d for %d channels", pitch, channel);
+  OCNN_REQUIRE((reinterpret_cast<uintptr_t>(rows) & 15) == 0, OCNN_E_BADARG, "rows not 16-byte aligned");
+  if (height == 0) return OCNN_OK;
+  dim3 grid((height + 63) / 64, (channel + 63) / 64);
+  transpose_channels_bf16_kernel<<<grid, 256, 0, as_stream(stream)>>>((uint16_t*)data, (const uint16_t*)rows, channel,
+      height, pitch);
+  OCNN_LAUNCH_OK("channels_from_rows");
+  return OCNN_OK;
 }
 
 int ocnn_conv_grad_workspace_bytes(const void* info, int depth, int channel_in, int num_output,

@@ -739,6 +739,67 @@ def octree_conv_fused(data_in, weights, bias, relu, octree, depth, num_output, k
                kernel_size, stride, nempty, bias=bias, relu=relu, out=out)
 
 
+def rows_pitch(channels):
+  """channels per row of the row-major layout: padded to whole 16-channel steps"""
+  return (int(channels) + 15) // 16 * 16
+
+
+def to_rows(data):
+  """[1, C, H, 1] bf16 (the reference's channel-major layout) -> rows [H + 1, pitch]: row h holds the
+  channels of node h, padding channels and row H are zero (row H is what a missing neighbour reads)."""
+  data = data.contiguous()
+  if data.dtype != torch.bfloat16:
+    raise TypeError("row-major tensors are bf16")
+  c, h = data.size(1), data.size(2)
+  rows = torch.empty(h + 1, rows_pitch(c), dtype=data.dtype, device=data.device)
+  _lib.call("ocnn_rows_from_channels", _ptr(rows), rows.size(1), _ptr(data), c, h, _dtype_code(data), _stream())
+  return rows
+
+
+def from_rows(rows, channels):
+  """rows [H + 1, pitch] -> [1, channels, H, 1]"""
+  rows = rows.contiguous()
+  h = rows.size(0) - 1
+  data = torch.empty(1, channels, h, 1, dtype=rows.dtype, device=rows.device)
+  _lib.call("ocnn_channels_from_rows", _ptr(data), _ptr(rows), rows.size(1), channels, h, _dtype_code(rows), _stream())
+  return data
+
+
+def octree_conv_rows(rows_in, channel_in, weights, octree, depth, num_output, bias=None, relu=False,
+                     deconv=False, out=None):
+  """3x3x3 stride-1 convolution over all nodes of `depth`, bf16, row-major on both sides: the same
+  arithmetic as octree_conv / octree_conv_fused (pytorch/cpp/octree_conv.cpp:131-157) on tensors
+  that a chain of convolutions keeps in the layout the kernel gathers from, so that no member of the
+  chain copies its input first.  rows_in: [H + 1, rows_pitch(channel_in)] as to_rows makes it;
+  returns [H + 1, rows_pitch(num_output)]."""
+  octree = _to_dev(octree)
+  info = octree_info(octree)
+  ksc, _ = _ks([3, 3, 3])
+  rows_in, weights = rows_in.contiguous(), weights.contiguous()
+  dt = _dtype_code(rows_in)
+  if weights.dtype != rows_in.dtype:
+    raise TypeError("weights and data must have the same dtype")
+  btm_h = rows_in.size(0) - 1
+  top_h, need_h, ws_bytes = C.c_int(), C.c_int(), C.c_size_t()
+  _lib.call("ocnn_conv_shape", info.p, depth, channel_in, num_output, ksc, 1, 0, int(deconv), dt,
+            C.byref(top_h), C.byref(need_h), C.byref(ws_bytes))
+  ws = _workspace(ws_bytes.value + 256, "conv")
+  base = (ws.data_ptr() + 255) & ~255
+  shape = (top_h.value + 1, rows_pitch(num_output))
+  if out is None:
+    out = torch.empty(shape, dtype=rows_in.dtype, device=rows_in.device)
+  elif tuple(out.shape) != shape or out.dtype != rows_in.dtype or not out.is_contiguous():
+    raise OcnnError(-3, "out must be a contiguous %s %s tensor" % (shape, rows_in.dtype))
+  if bias is not None:
+    bias = bias.to(torch.float32).contiguous()
+    if bias.numel() != num_output:
+      raise OcnnError(-3, "bias needs num_output entries")
+  _lib.call("ocnn_octree_conv_rows", _ptr(out), out.size(1), _ptr(rows_in), rows_in.size(1), channel_in, btm_h,
+            _ptr(weights), _ptr(bias), int(relu), int(deconv), _ptr(octree), info.p, depth, num_output, ksc, 1, 0,
+            dt, C.c_void_p(base), C.c_size_t(ws_bytes.value), _stream())
+  return out
+
+
 def _conv_grad(fn, is_deconv, data_in, weights, octree, grad_in, depth, num_output, kernel_size, stride,
                nempty, need_data=True, need_weights=True):
   octree = _to_dev(octree)
