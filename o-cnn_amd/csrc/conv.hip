@@ -942,7 +942,7 @@ constexpr int kNbPitch = 68;
 // from: 32 contiguous bytes per row and store instead of 16 bytes per channel and group.
 template <int MT, bool ROWS_OUT>
 __global__ __launch_bounds__(256, 1) void conv_s1_bf16_reg_kernel(ConvArgs a, uint16_t* __restrict__ out,
-    const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles, int cpad8, int out_pitch) {
+    const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles, int cpad8, int out_pitch, int out_cpad) {
   constexpr int kWUnits = 27 * MT * 64;        // 16-byte units of one k-step's weights
   constexpr int kWPiece = kWUnits / 4;         // copied per layer phase
   constexpr int kWVec = (kWPiece + 255) / 256;
@@ -1147,7 +1147,7 @@ __global__ __launch_bounds__(256, 1) void conv_s1_bf16_reg_kernel(ConvArgs a, ui
               const auto s1 = __builtin_amdgcn_permlane32_swap(w[2 * j][1], w[2 * j + 1][1], false, false);
               // channels cb + 32 mt + 16 j .. + 15 (8 in each lane of the pair): inside the pitch or not
               // for the whole wavefront
-              if (cb + 32 * mt + 16 * j < out_pitch)
+              if (cb + 32 * mt + 16 * j < out_cpad)
                 __builtin_amdgcn_raw_buffer_store_b128(u32x4{s0[0], s1[0], s0[1], s1[1]}, obuf, obase,
                     (sb * out_pitch + 32 * mt + 16 * j) * 2, 0);
             }
@@ -1169,7 +1169,7 @@ __global__ __launch_bounds__(256, 1) void conv_s1_bf16_reg_kernel(ConvArgs a, ui
         store_rows([&](int sb, int mt, int i) { return relu_floor(acc[sb][mt][i] + bias[mt][i], floor); });
       }
       // the all-zero row behind the last one (what a missing neighbour reads): once per pass range
-      if (tile == 0 && wave == 0 && lane * 8 < out_pitch && lane * 8 >= cb && lane * 8 < cb + MT * 32)
+      if (tile == 0 && wave == 0 && lane * 8 < out_cpad && lane * 8 >= cb && lane * 8 < cb + MT * 32)
         *reinterpret_cast<uint4*>(out + (int64_t)a.Hout * out_pitch + lane * 8) = make_uint4(0, 0, 0, 0);
       continue;
     }
@@ -1413,6 +1413,142 @@ __global__ void pack_weights_s2_bf16(uint16_t* __restrict__ Wt, const uint16_t* 
   int slab = (int)(f % nslab);
   int pass = (int)(f / nslab);
   int m = (pass * MT + mt) * 32 + (l & 31), c = slab * 8 + 2 * q + (l >> 5);
+  Wt[id] = (m < M && c < Cin) ? W[(int64_t)m * Cin * 8 + c * 8 + j] : (uint16_t)0;
+}
+
+// ---- 2x2x2 stride-2 convolution, row-major bf16 on both sides, padded ---------------------------
+// Column = node t of the coarser level, ALL of them: the pad that the reference's modules apply
+// after a stride-2 convolution (pytorch/ocnn/octree_conv.py:102-127) is part of the operator.
+// The operand of a column is the 8 rows of the node's children, which are consecutive rows of the
+// input: y[t] = sum_j W_j x[8 child[t] + j]; an empty node has no children, reads zeros and ends up
+// with the bias alone.  An MFMA k-step is (child j, 16 channels): lane (n, kh) loads 16 contiguous
+// bytes of row 8 child + j.  The k-steps are numbered j * ksteps + ks and staged eight at a time:
+// their weights wait in LDS (two buffers, one barrier per stage), the next stage's are on their
+// way meanwhile.  Output rows as the 3x3x3 row-major kernel writes them.
+constexpr int kS2Stage = 8;   // k-steps per weight stage
+template <int MT>
+__global__ __launch_bounds__(256) void conv_s2_rows_bf16_kernel(ConvArgs a, uint16_t* __restrict__ out,
+    int out_pitch, int out_cpad, const u32x4* __restrict__ xt, int in_pitch, int in_cpad,
+    const u32x4* __restrict__ Wt, int n_tiles) {
+  constexpr int kStageUnits = kS2Stage * MT * 64;
+  constexpr int kWVec = kStageUnits / 256;
+  __shared__ u32x4 sW[2][kStageUnits];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = xcd_tile(blockIdx.x, n_tiles);
+  if (tile >= n_tiles) return;
+  const int n0 = tile * kTileCols + wave * kWaveCols;
+  const int r = lane & 31, kh = lane >> 5;
+  const int row_bytes = in_pitch * 2;
+  const int ksteps = in_cpad >> 4;           // 16-channel k-steps per child = stages (8 children)
+  const int npass = (a.mtiles + MT - 1) / MT;
+  const __amdgpu_buffer_rsrc_t xrows = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<u32x4*>(xt), 0, (int)(((int64_t)a.Hin + 1) * row_bytes), 0x00020000);
+  const __amdgpu_buffer_rsrc_t obuf = __builtin_amdgcn_make_buffer_rsrc(
+      out, 0, (int)(((int64_t)a.Hout + 1) * out_pitch * 2), 0x00020000);
+  // byte offset of the first child's row; a column without children (or behind the level) reads
+  // past the end of the buffer, which yields zeros
+  int xoff[2], ooff[2];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+    const int n = n0 + nt * 32 + r;
+    const int c = n < a.N ? a.child[n] : -1;
+    xoff[nt] = c >= 0 ? c * 8 * row_bytes + kh * 16 : 0x7fffff00;
+    ooff[nt] = n < a.N ? (n * out_pitch + 8 * kh) * 2 : 0x7fffff00;
+  }
+  for (int pass = blockIdx.y; pass < npass; pass += gridDim.y) {
+    floatx16 acc[MT][2];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
+    const u32x4* wpass = Wt + (int64_t)pass * ksteps * kStageUnits;
+    u32x4 wr[kWVec];
+#pragma unroll
+    for (int v = 0; v < kWVec; ++v) wr[v] = wpass[v * 256 + threadIdx.x];
+    __syncthreads();   // the previous pass has left the buffers
+#pragma unroll
+    for (int v = 0; v < kWVec; ++v) sW[0][v * 256 + threadIdx.x] = wr[v];
+    int j = 0, ks = 0;   // child and channel step of the stage's first k-step
+    for (int st = 0; st < ksteps; ++st) {
+      __syncthreads();   // this stage's weights are in LDS; the other buffer is free
+      const u32x4* wnext = wpass + (int64_t)min(st + 1, ksteps - 1) * kStageUnits;
+#pragma unroll
+      for (int v = 0; v < kWVec; ++v) wr[v] = wnext[v * 256 + threadIdx.x];
+      union { u32x4 q; bf16x8 v; } b[kS2Stage][2];
+#pragma unroll
+      for (int t = 0; t < kS2Stage; ++t) {
+        const int so = j * row_bytes + ks * 32;
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) b[t][nt].q = __builtin_amdgcn_raw_buffer_load_b128(xrows, xoff[nt], so, 0);
+        if (++ks == ksteps) { ks = 0; ++j; }
+      }
+      const u32x4* wcur = sW[st & 1];
+#pragma unroll
+      for (int t = 0; t < kS2Stage; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          union { u32x4 q; bf16x8 v; } av;
+          av.q = wcur[(t * MT + mt) * 64 + lane];
+          acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b[t][0].v, acc[mt][0], 0, 0, 0);
+          acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b[t][1].v, acc[mt][1], 0, 0, 0);
+        }
+#pragma unroll
+      for (int v = 0; v < kWVec; ++v) sW[(st + 1) & 1][v * 256 + threadIdx.x] = wr[v];
+    }
+    // rows out: lane (r, kh) holds channels cb + 32 mt + 8 q + 4 kh + e of its two nodes; the lanes
+    // of a pair swap halves and store 16 bytes each (see conv_s1_bf16_reg_kernel)
+    const int cb = pass * MT * 32;
+    const float floor = a.relu ? 0.0f : -__builtin_inff();
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      float bias[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int ch = cb + 32 * mt + 8 * (i / 4) + 4 * kh + (i % 4);
+        bias[i] = a.bias ? a.bias[min(ch, a.M - 1)] : 0.0f;
+        if (ch >= a.M) bias[i] = 0.0f;
+      }
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) {
+        uint32_t w[4][2];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const int i = 4 * q + 2 * h;
+            w[q][h] = pack_bf16x2(relu_floor(acc[mt][nt][i] + bias[i], floor),
+                                  relu_floor(acc[mt][nt][i + 1] + bias[i + 1], floor));
+          }
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+          const auto s0 = __builtin_amdgcn_permlane32_swap(w[2 * jj][0], w[2 * jj + 1][0], false, false);
+          const auto s1 = __builtin_amdgcn_permlane32_swap(w[2 * jj][1], w[2 * jj + 1][1], false, false);
+          if (cb + 32 * mt + 16 * jj < out_cpad)
+            __builtin_amdgcn_raw_buffer_store_b128(u32x4{s0[0], s1[0], s0[1], s1[1]}, obuf, ooff[nt],
+                (cb + 32 * mt + 16 * jj) * 2, 0);
+        }
+      }
+    }
+    if (tile == 0 && wave == 0 && lane * 8 >= cb && lane * 8 < min(cb + MT * 32, out_cpad))
+      *reinterpret_cast<uint4*>(out + (int64_t)a.Hout * out_pitch + lane * 8) = make_uint4(0, 0, 0, 0);
+  }
+}
+// [pass][t = j * ksteps + ks][mt][lane][e]: lane (m, kh) <- W[m][(16 ks + 8 kh + e) * 8 + j]
+__global__ void pack_weights_s2_rows_bf16(uint16_t* __restrict__ Wt, const uint16_t* __restrict__ W, int M, int Cin,
+    int MT, int npass, int ksteps) {
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t total = (int64_t)npass * 8 * ksteps * MT * 64 * 8;
+  if (id >= total) return;
+  const int e = (int)(id & 7);
+  const int l = (int)((id >> 3) & 63);
+  int64_t f = id >> 9;
+  const int mt = (int)(f % MT); f /= MT;
+  const int t = (int)(f % (8 * ksteps));
+  const int pass = (int)(f / (8 * ksteps));
+  const int j = t / ksteps, ks = t % ksteps;
+  const int m = (pass * MT + mt) * 32 + (l & 31), c = 16 * ks + 8 * (l >> 5) + e;
   Wt[id] = (m < M && c < Cin) ? W[(int64_t)m * Cin * 8 + c * 8 + j] : (uint16_t)0;
 }
 
@@ -1661,6 +1797,129 @@ __global__ void pack_weights_d2_bf16(uint16_t* __restrict__ Wt, const uint16_t* 
   int pass = (int)(f / ksteps);
   int m = (pass * kD2MT + mt) * 32 + (l & 31), c = 16 * ks + 8 * (l >> 5) + j;
   Wt[id] = (m < rows && c < Cin) ? W[(int64_t)c * rows + m] : (uint16_t)0;
+}
+
+// ---- 2x2x2 stride-2 deconvolution, row-major bf16 on both sides, depad folded in -------------------
+// Column = p-th non-empty node of the level; its operand is that node's row of the input (all
+// nodes of the level, row ichild[p]: the depad the reference's modules apply before a stride-2
+// deconvolution, pytorch/ocnn/octree_conv.py:102-127, is part of the operator).  GEMM rows are
+// ordered (child s, output channel): a 32-row tile is 32 channels of one child and goes out as
+// 16-byte pieces of row 8 p + s, like the convolutions above.  The columns' operands stay in
+// registers for every pass, the packed weights of a pass are staged in LDS (two buffers, one
+// barrier per pass).
+template <int KS, int MT2>
+__global__ __launch_bounds__(256) void deconv_s2_rows_bf16_kernel(ConvArgs a, uint16_t* __restrict__ out,
+    int out_pitch, int out_cpad, const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles) {
+  constexpr int kUnits = KS * MT2 * 64;
+  constexpr int kVec = kUnits / 256;
+  __shared__ u32x4 sW[2][kUnits];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = xcd_tile(blockIdx.x, n_tiles);
+  if (tile >= n_tiles) return;
+  const int n0 = tile * kTileCols + wave * kWaveCols;
+  const int r = lane & 31, kh = lane >> 5;
+  const int ctiles = (a.M + 31) / 32;                 // 32-channel tiles per child
+  const int npass = (8 * ctiles + MT2 - 1) / MT2;
+  const __amdgpu_buffer_rsrc_t xrows = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<u32x4*>(xt), 0, (int)(((int64_t)a.Hin + 1) * KS * 32), 0x00020000);
+  const __amdgpu_buffer_rsrc_t obuf = __builtin_amdgcn_make_buffer_rsrc(
+      out, 0, (int)(((int64_t)a.Hout + 1) * out_pitch * 2), 0x00020000);
+  union Frag { u32x4 q; bf16x8 v; };
+  Frag b[KS][2];
+  int ooff[2];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+    const int n = n0 + nt * 32 + r;
+    const int src = n < a.N ? a.ichild[n] : -1;
+    const int xoff = src >= 0 ? src * KS * 32 + kh * 16 : 0x7fffff00;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) b[ks][nt].q = __builtin_amdgcn_raw_buffer_load_b128(xrows, xoff, ks * 32, 0);
+    ooff[nt] = n < a.N ? (n * 8 * out_pitch + 8 * kh) * 2 : 0x7fffff00;
+  }
+  u32x4 wr[kVec];
+#pragma unroll
+  for (int v = 0; v < kVec; ++v) wr[v] = Wt[v * 256 + threadIdx.x];
+#pragma unroll
+  for (int v = 0; v < kVec; ++v) sW[0][v * 256 + threadIdx.x] = wr[v];
+  const float floor = a.relu ? 0.0f : -__builtin_inff();
+  for (int pass = 0; pass < npass; ++pass) {
+    __syncthreads();   // this pass's weights are in LDS; the other buffer is free
+    const u32x4* wcur = sW[pass & 1];
+    const int nxt = min(pass + 1, npass - 1);
+#pragma unroll
+    for (int v = 0; v < kVec; ++v) wr[v] = Wt[(int64_t)nxt * kUnits + v * 256 + threadIdx.x];
+    floatx16 acc[MT2][2];
+#pragma unroll
+    for (int mt = 0; mt < MT2; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int mt = 0; mt < MT2; ++mt) {
+        Frag av;
+        av.q = wcur[(ks * MT2 + mt) * 64 + lane];
+        acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b[ks][0].v, acc[mt][0], 0, 0, 0);
+        acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b[ks][1].v, acc[mt][1], 0, 0, 0);
+      }
+#pragma unroll
+    for (int v = 0; v < kVec; ++v) sW[(pass + 1) & 1][v * 256 + threadIdx.x] = wr[v];
+#pragma unroll
+    for (int mt = 0; mt < MT2; ++mt) {
+      const int t = pass * MT2 + mt;                  // tile = (child, 32-channel block)
+      if (t >= 8 * ctiles) break;
+      const int child = t / ctiles, cb = (t % ctiles) * 32;
+      float bias[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int ch = cb + 8 * (i / 4) + 4 * kh + (i % 4);
+        bias[i] = a.bias ? a.bias[min(ch, a.M - 1)] : 0.0f;
+        if (ch >= a.M) bias[i] = 0.0f;
+      }
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) {
+        uint32_t w[4][2];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const int i = 4 * q + 2 * h;
+            w[q][h] = pack_bf16x2(relu_floor(acc[mt][nt][i] + bias[i], floor),
+                                  relu_floor(acc[mt][nt][i + 1] + bias[i + 1], floor));
+          }
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+          const auto s0 = __builtin_amdgcn_permlane32_swap(w[2 * jj][0], w[2 * jj + 1][0], false, false);
+          const auto s1 = __builtin_amdgcn_permlane32_swap(w[2 * jj][1], w[2 * jj + 1][1], false, false);
+          if (cb + 16 * jj < out_cpad)
+            __builtin_amdgcn_raw_buffer_store_b128(u32x4{s0[0], s1[0], s0[1], s1[1]}, obuf, ooff[nt],
+                (child * out_pitch + cb + 16 * jj) * 2, 0);
+        }
+      }
+      if (tile == 0 && wave == 0 && child == 0 && lane * 8 >= cb && lane * 8 < min(cb + 32, out_cpad))
+        *reinterpret_cast<uint4*>(out + (int64_t)a.Hout * out_pitch + lane * 8) = make_uint4(0, 0, 0, 0);
+    }
+  }
+}
+// [pass][ks][mt][lane][e]: tile t = pass * MT2 + mt = (child s, channel block cbk); lane (m, kh) <-
+// W[16 ks + 8 kh + e][(32 cbk + m) * 8 + s]   (deconvolution weights are [Cin, Cout * 8])
+__global__ void pack_weights_d2_rows_bf16(uint16_t* __restrict__ Wt, const uint16_t* __restrict__ W, int Cout, int Cin,
+    int MT2, int npass, int ksteps) {
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t total = (int64_t)npass * ksteps * MT2 * 64 * 8;
+  if (id >= total) return;
+  const int e = (int)(id & 7);
+  const int l = (int)((id >> 3) & 63);
+  int64_t f = id >> 9;
+  const int mt = (int)(f % MT2); f /= MT2;
+  const int ks = (int)(f % ksteps);
+  const int pass = (int)(f / ksteps);
+  const int ctiles = (Cout + 31) / 32;
+  const int t = pass * MT2 + mt;
+  const int child = t / ctiles, co = (t % ctiles) * 32 + (l & 31), c = 16 * ks + 8 * (l >> 5) + e;
+  Wt[id] = (t < 8 * ctiles && co < Cout && c < Cin) ? W[(int64_t)c * Cout * 8 + co * 8 + child] : (uint16_t)0;
 }
 
 template <typename T>
@@ -1953,9 +2212,9 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     if (use_reg) {
       const int r_grid = ((r_tiles + 7) / 8) * 8;
       if (MT == 1)
-        conv_s1_bf16_reg_kernel<1, false><<<dim3(r_grid, pass_split(r_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, r_tiles, cpad / 8, 0);
+        conv_s1_bf16_reg_kernel<1, false><<<dim3(r_grid, pass_split(r_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, r_tiles, cpad / 8, 0, 0);
       else
-        conv_s1_bf16_reg_kernel<2, false><<<dim3(r_grid, pass_split(r_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, r_tiles, cpad / 8, 0);
+        conv_s1_bf16_reg_kernel<2, false><<<dim3(r_grid, pass_split(r_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, r_tiles, cpad / 8, 0, 0);
     } else if (MT == 1)
       conv_s1_bf16_lds_kernel<1><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad / 8);
     else
@@ -2529,71 +2788,172 @@ int builtin_scratch(void** out) {
   return OCNN_OK;
 }
 
-// 3x3x3 stride-1 convolution (or deconvolution) over all nodes of a level in bf16, input and
-// output row-major: what a chain of such convolutions keeps between its members instead of
-// copying every input row-major first.  Only the packed weights need workspace.
+// Row-major bf16 operators over all nodes of a level: what a chain of convolutions keeps between
+// its members instead of copying every input row-major first.
+//   3x3x3 stride 1 (conv / deconv): rows of depth d in, rows of depth d out
+//   2x2x2 stride 2 conv:   rows of depth d in, rows of ALL nodes of depth d-1 out (pad folded in)
+//   2x2x2 stride 2 deconv: rows of ALL nodes of depth d in (depad folded in), rows of depth d+1 out
+struct RowsPlan {
+  int kind;            // 0: 3x3x3 s1, 1: 2x2x2 s2 conv, 2: 2x2x2 s2 deconv
+  int btm_h, top_h, cols, cpad, out_cpad;
+  int MT, npass, ksteps;
+  size_t wt_bytes, ichild_bytes, total_bytes;
+};
+int make_rows_plan(const Info* o, int depth, int channel_in, int num_output, const int* ks, int stride, int nempty,
+    int deconv, int dtype, RowsPlan* r) {
+  OCNN_REQUIRE(o && ks, OCNN_E_BADARG, "null pointer");
+  int e = ocnn_info_check(o);
+  if (e) return e;
+  OCNN_REQUIRE(dtype == OCNN_BF16 && !nempty, OCNN_E_UNSUPPORTED, "row-major operators: bf16, all nodes");
+  OCNN_REQUIRE(depth > 0 && depth <= o->depth, OCNN_E_BADARG, "depth %d not in [1,%d]", depth, o->depth);
+  OCNN_REQUIRE(num_output > 0 && channel_in > 0, OCNN_E_BADARG, "channels %d -> %d", channel_in, num_output);
+  OCNN_REQUIRE(o->has(OCNN_NEIGH) && o->has(OCNN_CHILD), OCNN_E_FORMAT,
+      "the octree holds no neighbour table (not an octree_batch result)");
+  const bool k333 = ks[0] == 3 && ks[1] == 3 && ks[2] == 3, k222 = ks[0] == 2 && ks[1] == 2 && ks[2] == 2;
+  r->cpad = (channel_in + 15) / 16 * 16;
+  r->out_cpad = (num_output + 15) / 16 * 16;
+  r->ksteps = r->cpad / 16;
+  r->ichild_bytes = 0;
+  const int mtiles = (num_output + 31) / 32;
+  if (stride == 1 && k333) {
+    r->kind = 0;
+    r->btm_h = r->top_h = r->cols = o->nnum[depth];
+    r->MT = mtiles == 1 ? 1 : 2;
+    r->npass = (mtiles + r->MT - 1) / r->MT;
+    r->wt_bytes = align256((size_t)r->npass * r->ksteps * 27 * r->MT * 64 * 16);
+  } else if (stride == 2 && k222 && !deconv) {
+    r->kind = 1;
+    r->btm_h = o->nnum[depth];
+    r->top_h = r->cols = o->nnum[depth - 1];
+    r->MT = mtiles == 1 ? 1 : 2;
+    r->npass = (mtiles + r->MT - 1) / r->MT;
+    r->wt_bytes = align256((size_t)r->npass * 8 * r->ksteps * r->MT * 64 * 16);
+  } else if (stride == 2 && k222 && deconv) {
+    OCNN_REQUIRE(depth < o->depth, OCNN_E_BADARG, "output depth %d outside the octree", depth + 1);
+    OCNN_REQUIRE(r->ksteps == 1 || r->ksteps == 2 || r->ksteps == 4 || r->ksteps == 8 || r->ksteps == 16,
+        OCNN_E_UNSUPPORTED, "row-major stride-2 deconvolution: input channels padded to 16, 32, 64, 128 or 256");
+    r->kind = 2;
+    r->btm_h = o->nnum[depth];
+    r->cols = o->nnum_nempty[depth];
+    r->top_h = o->nnum[depth + 1];
+    r->MT = r->ksteps <= 4 ? 4 : 2;
+    r->npass = (8 * mtiles + r->MT - 1) / r->MT;
+    r->wt_bytes = align256((size_t)r->npass * r->ksteps * r->MT * 64 * 16);
+    r->ichild_bytes = align256(sizeof(int) * (size_t)(r->cols + 1));
+  } else {
+    return fail(OCNN_E_UNSUPPORTED, "row-major operators: 3x3x3 stride 1, 2x2x2 stride 2");
+  }
+  r->total_bytes = r->wt_bytes + r->ichild_bytes;
+  return OCNN_OK;
+}
+
 int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_rows, int btm_pitch, int channel_in,
     int btm_h, const void* weights, const float* bias, int relu, const void* octree_dev, const void* info,
     int depth, int num_output, const int* ks, int stride, int nempty, int dtype, void* ws, size_t ws_bytes,
     hipStream_t s) {
   OCNN_REQUIRE(top_rows && btm_rows && weights && octree_dev && info && ks, OCNN_E_BADARG, "null pointer");
-  OCNN_REQUIRE(dtype == OCNN_BF16 && stride == 1 && !nempty && ks[0] == 3 && ks[1] == 3 && ks[2] == 3,
-      OCNN_E_UNSUPPORTED, "row-major convolutions: bf16, 3x3x3, stride 1, all nodes");
   const Info* o = as_info(info);
-  ConvPlan p;
-  int e = make_plan(o, depth, channel_in, num_output, ks, stride, nempty, deconv, dtype, &p);
+  RowsPlan r;
+  int e = make_rows_plan(o, depth, channel_in, num_output, ks, stride, nempty, deconv, dtype, &r);
   if (e) return e;
-  OCNN_REQUIRE(btm_h == p.btm_h, OCNN_E_SHAPE, "input height %d, the octree has %d rows at depth %d", btm_h,
-      p.btm_h, depth);
-  const int cpad = (channel_in + 15) / 16 * 16;
-  OCNN_REQUIRE(btm_pitch == cpad, OCNN_E_SHAPE, "input pitch %d: rows of %d channels are padded to %d", btm_pitch,
-      channel_in, cpad);
-  OCNN_REQUIRE(top_pitch >= num_output && top_pitch % 16 == 0 && top_pitch <= (num_output + 31) / 32 * 32,
-      OCNN_E_SHAPE, "output pitch %d for %d channels", top_pitch, num_output);
+  OCNN_REQUIRE(btm_h == r.btm_h, OCNN_E_SHAPE, "input height %d, the octree has %d rows at depth %d", btm_h,
+      r.btm_h, depth);
+  // the stride-2 convolution also reads a channel slice of a wider tensor (an encoder feature that
+  // sits in the tensor the decoder reads as a concatenation)
+  OCNN_REQUIRE(btm_pitch == r.cpad || (r.kind == 1 && btm_pitch > r.cpad && btm_pitch % 8 == 0), OCNN_E_SHAPE,
+      "input pitch %d: rows of %d channels are padded to %d", btm_pitch, channel_in, r.cpad);
+  OCNN_REQUIRE(top_pitch >= r.out_cpad && top_pitch % 8 == 0, OCNN_E_SHAPE, "output pitch %d for %d channels",
+      top_pitch, num_output);
   OCNN_REQUIRE(((reinterpret_cast<uintptr_t>(top_rows) | reinterpret_cast<uintptr_t>(btm_rows)) & 15) == 0,
       OCNN_E_BADARG, "rows not 16-byte aligned");
-  OCNN_REQUIRE(((int64_t)btm_h + 1) * cpad * 2 < ((int64_t)1 << 31) &&
-      ((int64_t)p.top_h + 1) * top_pitch * 2 < ((int64_t)1 << 31) - (1 << 20), OCNN_E_UNSUPPORTED,
+  OCNN_REQUIRE(((int64_t)btm_h + 1) * btm_pitch * 2 < ((int64_t)1 << 31) - (1 << 20) &&
+      ((int64_t)r.top_h + 1) * top_pitch * 2 < ((int64_t)1 << 31) - (1 << 20), OCNN_E_UNSUPPORTED,
       "level too large for 32-bit row offsets");
-  OCNN_REQUIRE(ws && ws_bytes >= p.wt_bytes, OCNN_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes, p.wt_bytes);
+  OCNN_REQUIRE(ws && ws_bytes >= r.total_bytes, OCNN_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes, r.total_bytes);
   OCNN_REQUIRE((reinterpret_cast<uintptr_t>(ws) & 15) == 0, OCNN_E_WORKSPACE, "workspace not 16-byte aligned");
   const char* blob = static_cast<const char*>(octree_dev);
+  char* wsb = static_cast<char*>(ws);
   ConvArgs a;
   a.M = num_output;
   a.Cin = channel_in;
-  a.N = p.top_h;
-  a.K = 27;
+  a.N = r.cols;
   a.Hin = btm_h;
-  a.Hout = p.top_h;
-  a.mode = kModeS1;
+  a.Hout = r.top_h;
   a.nempty = 0;
-  a.mtiles = p.mtiles;
+  a.mtiles = (num_output + 31) / 32;
   a.csteps = 0;
-  for (int k = 0; k < 27; ++k) a.slot[k] = tap_slot(deconv ? 26 - p.taps.tap[k] : p.taps.tap[k]);
-  a.neigh = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_NEIGH, depth));
-  a.child = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_CHILD, depth));
   a.ichild = nullptr;
   a.bias = bias;
   a.relu = relu ? 1 : 0;
-  if (o->nnum[depth] == 0) {   // a level without nodes: one zero row, and the zero row behind it
-    zero_rows_kernel<uint16_t><<<blocks_for(2 * (int64_t)top_pitch), kBlock, 0, s>>>((uint16_t*)top_rows, 2 * (int64_t)top_pitch);
+  for (int k = 0; k < 27; ++k) a.slot[k] = 0;
+  if (r.top_h == 0 || r.cols == 0) {   // nothing to convolve: zero rows (one data row at least, and the zero row)
+    const int64_t cnt = ((int64_t)r.top_h + 1) * top_pitch;
+    OCNN_REQUIRE(top_pitch == r.out_cpad, OCNN_E_UNSUPPORTED, "empty level into a channel slice");
+    zero_rows_kernel<uint16_t><<<blocks_for(cnt), kBlock, 0, s>>>((uint16_t*)top_rows, cnt);
     OCNN_LAUNCH_OK("zero_rows");
     return OCNN_OK;
   }
-  const int64_t sm = deconv ? 27 : (int64_t)channel_in * 27, sc = deconv ? (int64_t)num_output * 27 : 27;
-  const int MT = a.mtiles == 1 ? 1 : 2;
-  const int npass = (a.mtiles + MT - 1) / MT, nslab = cpad / 16;
-  const int64_t total = (int64_t)npass * nslab * 27 * MT * 64 * 8;
-  pack_weights_lds_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)ws, (const uint16_t*)weights, a.M, a.Cin, MT,
-      npass, nslab, sm, sc, deconv);
-  const int r_tiles = ((a.N >> 3) + kRegTileGroups - 1) / kRegTileGroups;
-  const int r_grid = ((r_tiles + 7) / 8) * 8;
-  if (MT == 1)
-    conv_s1_bf16_reg_kernel<1, true><<<dim3(r_grid, pass_split(r_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top_rows,
-        (const u32x4*)btm_rows, (const u32x4*)ws, r_tiles, cpad / 8, top_pitch);
-  else
-    conv_s1_bf16_reg_kernel<2, true><<<dim3(r_grid, pass_split(r_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top_rows,
-        (const u32x4*)btm_rows, (const u32x4*)ws, r_tiles, cpad / 8, top_pitch);
+  if (r.kind == 0) {
+    KernelTaps taps;
+    kernel_taps(ks, &taps);
+    a.K = 27;
+    a.mode = kModeS1;
+    for (int k = 0; k < 27; ++k) a.slot[k] = tap_slot(deconv ? 26 - taps.tap[k] : taps.tap[k]);
+    a.neigh = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_NEIGH, depth));
+    a.child = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_CHILD, depth));
+    const int64_t sm = deconv ? 27 : (int64_t)channel_in * 27, sc = deconv ? (int64_t)num_output * 27 : 27;
+    const int64_t total = (int64_t)r.npass * r.ksteps * 27 * r.MT * 64 * 8;
+    pack_weights_lds_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)ws, (const uint16_t*)weights, a.M, a.Cin,
+        r.MT, r.npass, r.ksteps, sm, sc, deconv);
+    const int r_tiles = ((a.N >> 3) + kRegTileGroups - 1) / kRegTileGroups;
+    const dim3 grid(((r_tiles + 7) / 8) * 8, pass_split(r_tiles, r.npass));
+    if (r.MT == 1)
+      conv_s1_bf16_reg_kernel<1, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
+          (const u32x4*)ws, r_tiles, r.cpad / 8, top_pitch, r.out_cpad);
+    else
+      conv_s1_bf16_reg_kernel<2, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
+          (const u32x4*)ws, r_tiles, r.cpad / 8, top_pitch, r.out_cpad);
+  } else if (r.kind == 1) {
+    a.K = 8;
+    a.mode = kModeS2Conv;
+    a.neigh = nullptr;
+    a.child = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_CHILD, depth - 1));
+    const int64_t total = (int64_t)r.npass * 8 * r.ksteps * r.MT * 64 * 8;
+    pack_weights_s2_rows_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)ws, (const uint16_t*)weights, a.M,
+        a.Cin, r.MT, r.npass, r.ksteps);
+    const int n_tiles = (a.N + kTileCols - 1) / kTileCols;
+    const dim3 grid(((n_tiles + 7) / 8) * 8, pass_split(n_tiles, r.npass));
+    if (r.MT == 1)
+      conv_s2_rows_bf16_kernel<1><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, top_pitch, r.out_cpad,
+          (const u32x4*)btm_rows, btm_pitch, r.cpad, (const u32x4*)ws, n_tiles);
+    else
+      conv_s2_rows_bf16_kernel<2><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, top_pitch, r.out_cpad,
+          (const u32x4*)btm_rows, btm_pitch, r.cpad, (const u32x4*)ws, n_tiles);
+  } else {
+    a.K = 8;
+    a.mode = kModeS2Deconv;
+    a.neigh = nullptr;
+    a.child = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_CHILD, depth));
+    int* ichild = reinterpret_cast<int*>(wsb + r.wt_bytes);
+    ichild_kernel<<<blocks_for(btm_h), kBlock, 0, s>>>(ichild, r.cols, a.child, btm_h);
+    a.ichild = ichild;
+    const int64_t total = (int64_t)r.npass * r.ksteps * r.MT * 64 * 8;
+    pack_weights_d2_rows_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)ws, (const uint16_t*)weights, a.M,
+        a.Cin, r.MT, r.npass, r.ksteps);
+    const int n_tiles = (a.N + kTileCols - 1) / kTileCols;
+    const int grid = ((n_tiles + 7) / 8) * 8;
+#define OCNN_D2_ROWS(KS, MT2)                                                                         \
+    deconv_s2_rows_bf16_kernel<KS, MT2><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, top_pitch, r.out_cpad, \
+        (const u32x4*)btm_rows, (const u32x4*)ws, n_tiles)
+    switch (r.ksteps) {
+      case 1: OCNN_D2_ROWS(1, 4); break;
+      case 2: OCNN_D2_ROWS(2, 4); break;
+      case 4: OCNN_D2_ROWS(4, 4); break;
+      case 8: OCNN_D2_ROWS(8, 2); break;
+      default: OCNN_D2_ROWS(16, 2); break;
+    }
+#undef OCNN_D2_ROWS
+  }
   OCNN_LAUNCH_OK("octree_conv_rows");
   return OCNN_OK;
 }
@@ -2667,6 +3027,17 @@ int ocnn_octree_conv_rows(void* top_rows, int top_pitch, const void* btm_rows, i
   return run_conv_rows(is_deconv ? 1 : 0, top_rows, top_pitch, btm_rows, btm_pitch, channel_in, btm_h, weights, bias,
       relu, octree_dev, info, depth, num_output, kernel_size, stride, nempty, dtype, workspace_dev, workspace_bytes,
       as_stream(stream));
+}
+
+int ocnn_conv_rows_shape(const void* info, int depth, int channel_in, int num_output, const int* kernel_size,
+    int stride, int is_deconv, int dtype, int* top_h, int* btm_h, size_t* workspace_bytes) {
+  RowsPlan r;
+  int e = make_rows_plan(as_info(info), depth, channel_in, num_output, kernel_size, stride, 0, is_deconv, dtype, &r);
+  if (e) return e;
+  if (top_h) *top_h = r.top_h;
+  if (btm_h) *btm_h = r.btm_h;
+  if (workspace_bytes) *workspace_bytes = r.total_bytes;
+  return OCNN_OK;
 }
 
 int ocnn_rows_from_channels(void* rows, int pitch, const void* data, int channel, int height, int dtype,

@@ -766,37 +766,47 @@ def from_rows(rows, channels):
 
 
 def octree_conv_rows(rows_in, channel_in, weights, octree, depth, num_output, bias=None, relu=False,
-                     deconv=False, out=None):
-  """3x3x3 stride-1 convolution over all nodes of `depth`, bf16, row-major on both sides: the same
-  arithmetic as octree_conv / octree_conv_fused (pytorch/cpp/octree_conv.cpp:131-157) on tensors
-  that a chain of convolutions keeps in the layout the kernel gathers from, so that no member of the
-  chain copies its input first.  rows_in: [H + 1, rows_pitch(channel_in)] as to_rows makes it;
-  returns [H + 1, rows_pitch(num_output)]."""
+                     deconv=False, out=None, kernel_size=(3, 3, 3), stride=1):
+  """Convolutions over all nodes in bf16, row-major on both sides: the arithmetic of octree_conv /
+  octree_conv_fused (pytorch/cpp/octree_conv.cpp:131-216) on tensors that a chain of convolutions
+  keeps in the layout the kernels gather from, so that no member of the chain copies its input.
+    3x3x3 stride 1: rows of `depth` in and out (bit-identical to the channel-major operator);
+    2x2x2 stride 2 conv: rows of `depth` in, rows of ALL nodes of depth-1 out -- the octree_pad of
+      the reference's modules (pytorch/ocnn/octree_conv.py:102-127) is folded in, an empty node
+      receives the bias alone;
+    2x2x2 stride 2 deconv: rows of ALL nodes of `depth` in (the octree_depad of those modules is
+      folded in), rows of depth+1 out.
+  rows_in: [H + 1, rows_pitch(channel_in)] as to_rows makes it.  `out`: [top_h + 1, P] with
+  P >= rows_pitch(num_output), or columns c0 .. c0 + rows_pitch(num_output) of such a tensor (a
+  slice of what a later layer reads as a concatenation); returns `out`."""
   octree = _to_dev(octree)
   info = octree_info(octree)
-  ksc, _ = _ks([3, 3, 3])
-  rows_in, weights = rows_in.contiguous(), weights.contiguous()
+  ksc, _ = _ks(kernel_size)
+  weights = weights.contiguous()
+  if rows_in.dim() != 2 or rows_in.stride(1) != 1:
+    raise OcnnError(-3, "rows_in must be [H + 1, pitch] with unit channel stride")
   dt = _dtype_code(rows_in)
   if weights.dtype != rows_in.dtype:
     raise TypeError("weights and data must have the same dtype")
   btm_h = rows_in.size(0) - 1
   top_h, need_h, ws_bytes = C.c_int(), C.c_int(), C.c_size_t()
-  _lib.call("ocnn_conv_shape", info.p, depth, channel_in, num_output, ksc, 1, 0, int(deconv), dt,
+  _lib.call("ocnn_conv_rows_shape", info.p, depth, channel_in, num_output, ksc, stride, int(deconv), dt,
             C.byref(top_h), C.byref(need_h), C.byref(ws_bytes))
   ws = _workspace(ws_bytes.value + 256, "conv")
   base = (ws.data_ptr() + 255) & ~255
-  shape = (top_h.value + 1, rows_pitch(num_output))
+  cpad = rows_pitch(num_output)
   if out is None:
-    out = torch.empty(shape, dtype=rows_in.dtype, device=rows_in.device)
-  elif tuple(out.shape) != shape or out.dtype != rows_in.dtype or not out.is_contiguous():
-    raise OcnnError(-3, "out must be a contiguous %s %s tensor" % (shape, rows_in.dtype))
+    out = torch.empty(top_h.value + 1, cpad, dtype=rows_in.dtype, device=rows_in.device)
+  elif (out.dim() != 2 or out.size(0) != top_h.value + 1 or out.size(1) < cpad or out.stride(1) != 1
+        or out.dtype != rows_in.dtype or out.device != rows_in.device):
+    raise OcnnError(-3, "out must be [%d, >= %d] %s with unit channel stride" % (top_h.value + 1, cpad, rows_in.dtype))
   if bias is not None:
     bias = bias.to(torch.float32).contiguous()
     if bias.numel() != num_output:
       raise OcnnError(-3, "bias needs num_output entries")
-  _lib.call("ocnn_octree_conv_rows", _ptr(out), out.size(1), _ptr(rows_in), rows_in.size(1), channel_in, btm_h,
-            _ptr(weights), _ptr(bias), int(relu), int(deconv), _ptr(octree), info.p, depth, num_output, ksc, 1, 0,
-            dt, C.c_void_p(base), C.c_size_t(ws_bytes.value), _stream())
+  _lib.call("ocnn_octree_conv_rows", _ptr(out), out.stride(0), _ptr(rows_in), rows_in.stride(0), channel_in, btm_h,
+            _ptr(weights), _ptr(bias), int(relu), int(deconv), _ptr(octree), info.p, depth, num_output, ksc, stride,
+            0, dt, C.c_void_p(base), C.c_size_t(ws_bytes.value), _stream())
   return out
 
 

@@ -84,3 +84,89 @@ def test_conv_rows_rejects(oc, octree):
     F.octree_conv_rows(x[:-1].contiguous(), 16, w, octree, 6, 32)       # one row short
   with pytest.raises(oc.nn.OcnnError):
     F.octree_conv_rows(x, 20, w, octree, 6, 32)                         # pitch does not match the channels
+
+
+def bf16_round(a):
+  return T(a).bfloat16().float().numpy()
+
+
+def close(got, exp, tol, what):
+  """largest error against the largest magnitude, and element-wise against |exp| + the channel's rms"""
+  assert got.shape == exp.shape, what
+  assert float(np.abs(got - exp).max()) / float(np.abs(exp).max()) < tol, what
+  rms = np.sqrt((exp.astype(np.float64) ** 2).mean(axis=1, keepdims=True)).astype(np.float32)
+  bad = np.abs(got - exp) > tol * (np.abs(exp) + rms)
+  assert not bad.any(), (what, int(bad.sum()))
+
+
+@pytest.fixture(scope="module")
+def small(oc, orc, synthetic):
+  from oracle.checker import OctreeBlob
+  pbs = [make_points_blob(*synthetic.shape_cloud(3000, 61 + i)[:2]) for i in range(2)]
+  host = orc.octree_batch([orc.points2octree(p, 6, 2) for p in pbs])
+  return host, T(host).cuda(), OctreeBlob(host)
+
+
+@pytest.mark.parametrize("cin,cout", [(16, 32), (32, 64), (24, 40), (128, 256), (64, 16)])
+def test_stride2_rows_against_oracle(oc, orc, small, cin, cout):
+  """2x2x2 stride 2 with the pad / depad of the reference's modules folded in
+  (pytorch/ocnn/octree_conv.py:102-127), bias and ReLU fused: 2e-2 against the oracle in fp32 on
+  bf16-rounded operands."""
+  host, dev, b = small
+  F = oc.nn
+  rng = np.random.default_rng(cin * 7 + cout)
+  d = 6
+  H = int(b.nnum[d])
+  x = bf16_round(rng.standard_normal((cin, H)).astype(np.float32))
+  bias = (rng.standard_normal(cout) * 0.2).astype(np.float32)
+  xr = F.to_rows(T(x).cuda().view(1, cin, H, 1).bfloat16())
+  # convolution: nodes of depth 5 out, an empty node holds relu(bias)
+  w = bf16_round((rng.standard_normal((cout, cin * 8)) / np.sqrt(cin * 8)).astype(np.float32))
+  y = orc.pad(orc.octree_conv(x, w, host, d, cout, [2, 2, 2], 2, False), b.prop("child", d - 1))
+  exp = np.maximum(y + bias[:, None], 0)
+  rows = F.octree_conv_rows(xr, cin, T(w).cuda().bfloat16(), dev, d, cout, bias=T(bias).cuda(), relu=True,
+                            kernel_size=(2, 2, 2), stride=2)
+  assert rows.shape == (int(b.nnum[d - 1]) + 1, F.rows_pitch(cout))
+  assert not rows[-1].any() and not rows[:, cout:].any()
+  close(F.from_rows(rows, cout).float().cpu().numpy().reshape(exp.shape), exp, 2e-2, ("conv", cin, cout))
+  # deconvolution from depth 5 to depth 6: rows of all nodes of depth 5 in, the non-empty ones are used
+  d = 5
+  H = int(b.nnum[d])
+  x = bf16_round(rng.standard_normal((cin, H)).astype(np.float32))
+  w = bf16_round((rng.standard_normal((cin, cout * 8)) / np.sqrt(cin)).astype(np.float32))
+  xne = orc.depad(x, b.prop("child", d), int(b.nnum_nempty[d]))
+  exp = orc.octree_deconv(xne, w, host, d, cout, [2, 2, 2], 2, False) + bias[:, None]
+  xr = F.to_rows(T(x).cuda().view(1, cin, H, 1).bfloat16())
+  wide = torch.full((int(b.nnum[d + 1]) + 1, F.rows_pitch(cout) + 32), 7.0, dtype=torch.bfloat16, device="cuda")
+  rows = F.octree_conv_rows(xr, cin, T(w).cuda().bfloat16(), dev, d, cout, bias=T(bias).cuda(), relu=False,
+                            deconv=True, kernel_size=(2, 2, 2), stride=2, out=wide[:, 16:16 + F.rows_pitch(cout)])
+  assert (wide[:, :16] == 7).all() and (wide[:, 16 + F.rows_pitch(cout):] == 7).all(), "wrote outside its slice"
+  assert not rows[-1].any() and not rows[:, cout:].any()
+  close(F.from_rows(rows.contiguous(), cout).float().cpu().numpy().reshape(exp.shape), exp, 2e-2, ("deconv", cin, cout))
+
+
+def test_unet_trunk_rows(oc, small):
+  """the row-major trunk against the channel-major bf16 trunk (same operators, the 3x3x3 ones
+  bit-identical, the stride-2 ones summed in another order): 2e-2 over the whole chain, as for a
+  single bf16 operator (measured: below 1e-2)"""
+  host, dev, b = small
+  rng = np.random.default_rng(3)
+  ch = {6: 16, 5: 32, 4: 64}
+  params = {}
+
+  def mk(key, shape, fan):
+    w = (rng.standard_normal(shape) / np.sqrt(fan)).astype(np.float32)
+    bias = (rng.standard_normal(shape[0] if key[0] != "up" else shape[1] // 8) * 0.1).astype(np.float32)
+    params[key] = (T(w).cuda().bfloat16(), T(bias).cuda())
+
+  mk(("conv", 6), (ch[6], 3 * 27), 81)
+  for d in (6, 5):
+    mk(("down", d), (ch[d - 1], ch[d] * 8), ch[d] * 8)
+    mk(("conv", d - 1), (ch[d - 1], ch[d - 1] * 27), ch[d - 1] * 27)
+  for d in (4, 5):
+    mk(("up", d), (ch[d], ch[d + 1] * 8), ch[d])
+    mk(("dec", d + 1), (ch[d + 1], 2 * ch[d + 1] * 27), 2 * ch[d + 1] * 27)
+  data = oc.nn.octree_property(dev, "feature", 6).bfloat16()
+  exp = oc.stacks.unet_trunk(dev, 6, params, data=data, stages=2).float().cpu().numpy()
+  got = oc.stacks.unet_trunk_rows(dev, 6, params, data=data, stages=2).float().cpu().numpy()
+  close(got.reshape(got.shape[1], -1), exp.reshape(exp.shape[1], -1), 2e-2, "unet trunk")
