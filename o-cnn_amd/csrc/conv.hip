@@ -920,6 +920,12 @@ __global__ __launch_bounds__(256, 2) void conv_s1_bf16_lds_kernel(ConvArgs a, ui
 // barrier per k-step); a wavefront reads each tap's fragment twice per k-step, 0.25 KiB of LDS
 // operands per MFMA.  The neighbour rows of a wavefront's groups wait in LDS too (68 words per
 // group: 16-byte reads of 32 lanes then meet no bank twice).
+// A 16-byte store reads its four data registers for a while after it has issued, and the next
+// instruction that writes one of them has to keep two wait states' distance.  The compiler puts
+// them in when store and writer share a basic block; the stores below sit in conditional blocks of
+// their own, and the value computed for the next store landed in a register the store was
+// still reading (seen as a few wrong words per million).  So the wait goes in by hand.
+#define OCNN_STORE_DATA_WAIT() asm volatile("s_nop 1")
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
 
@@ -1147,9 +1153,11 @@ __global__ __launch_bounds__(256, 1) void conv_s1_bf16_reg_kernel(ConvArgs a, ui
               const auto s1 = __builtin_amdgcn_permlane32_swap(w[2 * j][1], w[2 * j + 1][1], false, false);
               // channels cb + 32 mt + 16 j .. + 15 (8 in each lane of the pair): inside the pitch or not
               // for the whole wavefront
-              if (cb + 32 * mt + 16 * j < out_cpad)
+              if (cb + 32 * mt + 16 * j < out_cpad) {
                 __builtin_amdgcn_raw_buffer_store_b128(u32x4{s0[0], s1[0], s0[1], s1[1]}, obuf, obase,
                     (sb * out_pitch + 32 * mt + 16 * j) * 2, 0);
+                OCNN_STORE_DATA_WAIT();
+              }
             }
           }
       };
@@ -1525,9 +1533,11 @@ __global__ __launch_bounds__(256) void conv_s2_rows_bf16_kernel(ConvArgs a, uint
         for (int jj = 0; jj < 2; ++jj) {
           const auto s0 = __builtin_amdgcn_permlane32_swap(w[2 * jj][0], w[2 * jj + 1][0], false, false);
           const auto s1 = __builtin_amdgcn_permlane32_swap(w[2 * jj][1], w[2 * jj + 1][1], false, false);
-          if (cb + 32 * mt + 16 * jj < out_cpad)
+          if (cb + 32 * mt + 16 * jj < out_cpad) {
             __builtin_amdgcn_raw_buffer_store_b128(u32x4{s0[0], s1[0], s0[1], s1[1]}, obuf, ooff[nt],
                 (cb + 32 * mt + 16 * jj) * 2, 0);
+            OCNN_STORE_DATA_WAIT();
+          }
         }
       }
     }
@@ -1893,9 +1903,11 @@ __global__ __launch_bounds__(256) void deconv_s2_rows_bf16_kernel(ConvArgs a, ui
         for (int jj = 0; jj < 2; ++jj) {
           const auto s0 = __builtin_amdgcn_permlane32_swap(w[2 * jj][0], w[2 * jj + 1][0], false, false);
           const auto s1 = __builtin_amdgcn_permlane32_swap(w[2 * jj][1], w[2 * jj + 1][1], false, false);
-          if (cb + 16 * jj < out_cpad)
+          if (cb + 16 * jj < out_cpad) {
             __builtin_amdgcn_raw_buffer_store_b128(u32x4{s0[0], s1[0], s0[1], s1[1]}, obuf, ooff[nt],
                 (child * out_pitch + cb + 16 * jj) * 2, 0);
+            OCNN_STORE_DATA_WAIT();
+          }
         }
       }
       if (tile == 0 && wave == 0 && child == 0 && lane * 8 >= cb && lane * 8 < min(cb + 32, out_cpad))

@@ -170,3 +170,39 @@ def test_unet_trunk_rows(oc, small):
   exp = oc.stacks.unet_trunk(dev, 6, params, data=data, stages=2).float().cpu().numpy()
   got = oc.stacks.unet_trunk_rows(dev, 6, params, data=data, stages=2).float().cpu().numpy()
   close(got.reshape(got.shape[1], -1), exp.reshape(exp.shape[1], -1), 2e-2, "unet trunk")
+
+
+def test_rows_operators_full_size(oc, synthetic):
+  """The depth-9 scene (1.5 M octants): 3x3x3 bit-identical to the channel-major operator, the
+  stride-2 pair within 2e-2 of it, and every operator the same on a second run (a store whose data
+  registers were overwritten too early showed up only at this size, as a few words that changed
+  from run to run)."""
+  F, S = oc.nn, oc.stacks
+  p, n, f = synthetic.room_cloud(250000, 3)
+  octree = F.points2octree_batch([T(make_points_blob(p, n, f)).cuda()], 9, 2)
+  info = F.octree_info(octree)
+  g = torch.Generator().manual_seed(4)
+  H9 = info.nnum(9)
+  x = torch.randn(1, 32, H9, 1, generator=g).bfloat16().cuda()
+  w3 = (torch.randn(32, 32 * 27, generator=g) * 0.05).bfloat16().cuda()
+  wd = (torch.randn(64, 32 * 8, generator=g) * 0.08).bfloat16().cuda()
+  wu = (torch.randn(64, 32 * 8, generator=g) * 0.1).bfloat16().cuda()
+  b32, b64 = torch.randn(32, generator=g).cuda() * 0.2, torch.randn(64, generator=g).cuda() * 0.2
+  xr = F.to_rows(x)
+
+  def same(fn):
+    a = fn()
+    for _ in range(2):
+      assert torch.equal(a, fn()), "results change from run to run"
+    return a
+
+  y = same(lambda: F.octree_conv_rows(xr, 32, w3, octree, 9, 32, bias=b32, relu=True))
+  y_ref = F.octree_conv_fused(x, w3, b32, True, octree, 9, 32, [3, 3, 3], 1, False)
+  assert torch.equal(F.from_rows(y, 32), y_ref)
+  dn = same(lambda: F.octree_conv_rows(y, 32, wd, octree, 9, 64, bias=b64, relu=True, kernel_size=(2, 2, 2), stride=2))
+  dn_ref = S.conv_bn_relu(y_ref, wd, b64, octree, 9, 64, (2, 2, 2), 2)
+  close(F.from_rows(dn, 64).float().cpu().numpy().reshape(64, -1), dn_ref.float().cpu().numpy().reshape(64, -1), 2e-2, "down")
+  up = same(lambda: F.octree_conv_rows(dn, 64, wu, octree, 8, 32, bias=b32, relu=True, deconv=True,
+                                       kernel_size=(2, 2, 2), stride=2))
+  up_ref = S.conv_bn_relu(dn_ref, wu, b32, octree, 8, 32, (2, 2, 2), 2, deconv=True)
+  close(F.from_rows(up, 32).float().cpu().numpy().reshape(32, -1), up_ref.float().cpu().numpy().reshape(32, -1), 2e-2, "up")
