@@ -201,7 +201,29 @@ def main():
 
     x16, w16 = x32.bfloat16(), w32.bfloat16()
     conv_case("conv333_s1_d9_bf16", octree, 9, x16, w16, [3, 3, 3], 1)
+    # the same operator on row-major activations (input and output [H + 1][pitch] bf16): what a
+    # member of a chain of convolutions costs once the chain keeps that layout between its members
+    # (bit-identical results; the channel-major entry above copies its input row-major first)
+    rows16 = F.to_rows(x16)
+    rows_out = torch.empty(H9 + 1, F.rows_pitch(C), dtype=torch.bfloat16, device=dev)
+    t = timed(lambda: F.octree_conv_rows(rows16, C, w16, octree, 9, C, out=rows_out), reps, wu)
+    extra["conv333_s1_d9_bf16_rows"] = {
+        "ms": t, "octants_per_s": H9 / (t * 1e-3), "tflops": flops / (t * 1e-3) / 1e12,
+        "frac_mfma_peak": flops / (t * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS["bf16"],
+        "layout": "row-major in and out, no copy"}
     w2 = (torch.randn(C, C * 8, generator=g) * 0.02).to(dev)
+    # 2x2x2 stride 2, row-major, with the pad (conv) / depad (deconv) of the reference's modules folded in
+    t = timed(lambda: F.octree_conv_rows(rows16, C, w2.bfloat16(), octree, 9, C, kernel_size=(2, 2, 2), stride=2), reps, wu)
+    by = (H9 * C + H8 * C) * 2 + H8 * 4
+    extra["conv222_s2_d9_bf16_rows_padded"] = {"ms": t, "GBs": by / t / 1e6, "frac_hbm_peak": by / t / 1e6 / PEAK_HBM_GBS,
+                                               "tflops": 2.0 * Hne8 * 8 * C * C / (t * 1e-3) / 1e12}
+    rows8 = torch.randn(H8 + 1, C, generator=g).bfloat16().to(dev)
+    t = timed(lambda: F.octree_conv_rows(rows8, C, w2.bfloat16(), octree, 8, C, deconv=True, kernel_size=(2, 2, 2),
+                                         stride=2, out=rows_out), reps, wu)
+    by = (Hne8 * C + H9 * C) * 2 + H8 * 4 + Hne8 * 4
+    extra["deconv222_s2_d8to9_bf16_rows_depadded"] = {"ms": t, "GBs": by / t / 1e6, "frac_hbm_peak": by / t / 1e6 / PEAK_HBM_GBS,
+                                                      "tflops": 2.0 * Hne8 * 8 * C * C / (t * 1e-3) / 1e12}
+    del rows16, rows8, rows_out
     conv_case("conv222_s2_d9_f32", octree, 9, x32, w2, [2, 2, 2], 2)
     conv_case("conv222_s2_d9_bf16", octree, 9, x16, w2.bfloat16(), [2, 2, 2], 2)
     xne = torch.randn(1, C, Hne9, 1, generator=g).to(dev)
@@ -441,6 +463,9 @@ def main():
     f16 = feat9.bfloat16()
     t = timed(lambda: oc.stacks.unet_trunk(octree, 9, up16, data=f16), max(2, reps // 2), 1)
     extra["unet_trunk_scene_d9_bf16"] = {"ms": t, "points_per_s": 250000 / (t * 1e-3)}
+    # the same trunk with row-major activations between the operators (converted once at each end)
+    t = timed(lambda: oc.stacks.unet_trunk_rows(octree, 9, up16, data=f16), max(2, reps // 2), 1)
+    extra["unet_trunk_scene_d9_bf16_rows"] = {"ms": t, "points_per_s": 250000 / (t * 1e-3)}
     # the same trunk over the non-empty nodes only (the reference's ScanNet setting)
     fne = F.octree_depad(feat9, octree, 9)
     fne16 = fne.bfloat16()
