@@ -119,6 +119,31 @@ template <typename OutT, int MT>
 __device__ inline void store_tiles(const ConvArgs& a, OutT* __restrict__ out, floatx16 (&acc)[MT][2],
     int mt0, int n0, int lane) {
   const int r = lane & 31, kh = lane >> 5;
+  if (sizeof(OutT) == 2 && (a.Hout & 1) == 0 && (a.N & 1) == 0 && (reinterpret_cast<uintptr_t>(out) & 3) == 0) {
+    // bf16 with an even row length: neighbouring lanes (columns n, n + 1) swap one value of each
+    // channel pair (m, m + 1), so the even lane stores both columns of channel m and the odd lane
+    // both columns of channel m + 1 as one aligned word: half the store instructions
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) {
+        const int n = n0 + nt * 32 + r;           // N is even: a column and its partner exist together
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+          const int m = (mt0 + mt) * 32 + 8 * (i / 4) + 4 * kh + (i % 4);
+          const float v0 = finish(a, acc[mt][nt][i], min(m, a.M - 1));
+          const float v1 = finish(a, acc[mt][nt][i + 1], min(m + 1, a.M - 1));
+          const uint32_t mine = (r & 1) ? f32_to_bf16(v1) : f32_to_bf16(v0);
+          const uint32_t send = (r & 1) ? f32_to_bf16(v0) : f32_to_bf16(v1);
+          const uint32_t got = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send, 0xB1, 0xf, 0xf, true);  // lane ^ 1
+          const int mm = m + (r & 1);
+          if (n < a.N && mm < a.M)
+            *reinterpret_cast<uint32_t*>(reinterpret_cast<uint16_t*>(out) + (int64_t)mm * a.Hout + (n & ~1)) =
+                (r & 1) ? (got | (mine << 16)) : (mine | (got << 16));
+        }
+      }
+    return;
+  }
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -430,14 +455,53 @@ __global__ __launch_bounds__(256, 2) void conv_rows_bf16_deep_kernel(ConvArgs a,
   const int ngroup = (a.K + kG - 1) / kG;
   {
     const int col = tile * kTileCols + (int)threadIdx.x;
+    if (a.mode == kModeS1) {
+      // three dependent trips for all taps together: my node, its 27 neighbours (all in the 256-byte
+      // block of the node's sibling group), their ranks among the non-empty nodes
+      const bool mine = col < a.N;
+      const int node = mine ? (a.nempty ? a.ichild[col] : col) : 0;
+      const int* __restrict__ block = a.neigh + ((int64_t)(node >> 3) << 6) + sibling_slot(node & 7);
+      int nb[27];
 #pragma unroll
-    for (int k = 0; k < 27; ++k) {
-      const int sr = k < a.K ? conv_src(a, col, k) : -1;
-      sSrc[k][threadIdx.x] = (sr < 0 ? a.Hin : sr) * cpad8;
+      for (int k = 0; k < 27; ++k) nb[k] = (mine && k < a.K) ? block[a.slot[k]] : -1;
+      if (a.nempty) {
+        int rank[27];
+#pragma unroll
+        for (int k = 0; k < 27; ++k) rank[k] = a.child[max(nb[k], 0)];
+#pragma unroll
+        for (int k = 0; k < 27; ++k) nb[k] = nb[k] >= 0 ? rank[k] : -1;
+      }
+#pragma unroll
+      for (int k = 0; k < 27; ++k) sSrc[k][threadIdx.x] = ((nb[k] >= 0 && nb[k] < a.Hin) ? nb[k] : a.Hin) * cpad8;
+    } else {
+#pragma unroll
+      for (int k = 0; k < 27; ++k) {
+        const int sr = k < a.K ? conv_src(a, col, k) : -1;
+        sSrc[k][threadIdx.x] = (sr < 0 ? a.Hin : sr) * cpad8;
+      }
     }
   }
   const int c0 = wave * kWaveCols + r;                  // my column of the first column tile, inside the workgroup's tile
   union Frag { u32x4 q; bf16x8 v; };
+  // Taps whose neighbour is missing for all 32 columns of a column tile add nothing: their
+  // operands are not requested and their products not formed.  Over the non-empty nodes of a
+  // surface that is most taps (the columns of a wavefront lie on one patch of the surface, and
+  // the nodes off that patch are empty for all of them).  live[nt]: bit k = tap k has a
+  // neighbour in column tile nt of this wavefront.
+  unsigned live[2] = {0, 0};
+  __syncthreads();                                       // source rows written
+  {
+    const int none = a.Hin * cpad8;
+#pragma unroll
+    for (int k = 0; k < 27; ++k) {
+      if (k >= a.K) break;
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+        if (__ballot(sSrc[k][c0 + 32 * nt] != none) != 0) live[nt] |= 1u << k;
+    }
+    live[0] = __builtin_amdgcn_readfirstlane(live[0]);
+    live[1] = __builtin_amdgcn_readfirstlane(live[1]);
+  }
   for (int pass = blockIdx.y; pass < npass; pass += gridDim.y) {  // passes may be dealt out over workgroups
     floatx16 acc[MT][2];
 #pragma unroll
@@ -464,12 +528,16 @@ __global__ __launch_bounds__(256, 2) void conv_rows_bf16_deep_kernel(ConvArgs a,
         constexpr int S = decltype(set)::value;
         if (tap >= a.K) return;                          // uniform
         const int s0 = sSrc[tap][c0], s1 = sSrc[tap][c0 + 32];
+        if ((live[0] >> tap) & 1) {                      // uniform over the wavefront
 #pragma unroll
-        for (int ks = 0; ks < kKs; ++ks)
-          if (ks < nks) {
-            x[S][ks][0].q = xt[(int64_t)s0 + col16 + 2 * ks];
-            x[S][ks][1].q = xt[(int64_t)s1 + col16 + 2 * ks];
-          }
+          for (int ks = 0; ks < kKs; ++ks)
+            if (ks < nks) x[S][ks][0].q = xt[(int64_t)s0 + col16 + 2 * ks];
+        }
+        if ((live[1] >> tap) & 1) {
+#pragma unroll
+          for (int ks = 0; ks < kKs; ++ks)
+            if (ks < nks) x[S][ks][1].q = xt[(int64_t)s1 + col16 + 2 * ks];
+        }
       };
       __syncthreads();                                   // source rows written (first time); weight buffers free
       fetch_w(0);
@@ -486,6 +554,8 @@ __global__ __launch_bounds__(256, 2) void conv_rows_bf16_deep_kernel(ConvArgs a,
           const int tap = g * kG + J;
           if (tap >= a.K) return;                        // uniform
           fetch_x(tap + 2, std::integral_constant<int, (J + 2) % 3>());
+          const bool l0 = (live[0] >> tap) & 1, l1 = (live[1] >> tap) & 1;   // uniform over the wavefront
+          if (!l0 && !l1) return;
 #pragma unroll
           for (int ks = 0; ks < kKs; ++ks) {
             if (ks >= nks) continue;                     // uniform
@@ -493,8 +563,8 @@ __global__ __launch_bounds__(256, 2) void conv_rows_bf16_deep_kernel(ConvArgs a,
             for (int mt = 0; mt < MT; ++mt) {
               Frag av;
               av.q = wcur[J * kWUnits + (ks * MT + mt) * 64 + lane];
-              acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, x[J][ks][0].v, acc[mt][0], 0, 0, 0);
-              acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, x[J][ks][1].v, acc[mt][1], 0, 0, 0);
+              if (l0) acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, x[J][ks][0].v, acc[mt][0], 0, 0, 0);
+              if (l1) acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, x[J][ks][1].v, acc[mt][1], 0, 0, 0);
             }
           }
         };
