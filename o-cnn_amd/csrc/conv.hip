@@ -198,6 +198,33 @@ __global__ __launch_bounds__(256) void transpose_rows_f32_kernel(float* __restri
   }
 }
 
+// Source rows of one output column for all taps (-1: contributes zero), handed to `put(tap, row)`.
+// Stride-1 modes: three dependent trips for all taps together -- the node, its neighbours (all in
+// the 256-byte block of the node's sibling group), their ranks among the non-empty nodes.
+template <class Put>
+__device__ inline void lookup_sources(const ConvArgs& a, int col, Put put) {
+  if (a.mode == kModeS1) {
+    const bool mine = col < a.N;
+    const int node = mine ? (a.nempty ? a.ichild[col] : col) : 0;
+    const int* __restrict__ block = a.neigh + ((int64_t)(node >> 3) << 6) + sibling_slot(node & 7);
+    int nb[27];
+#pragma unroll
+    for (int k = 0; k < 27; ++k) nb[k] = (mine && k < a.K) ? block[a.slot[k]] : -1;
+    if (a.nempty) {
+      int rank[27];
+#pragma unroll
+      for (int k = 0; k < 27; ++k) rank[k] = a.child[max(nb[k], 0)];
+#pragma unroll
+      for (int k = 0; k < 27; ++k) nb[k] = nb[k] >= 0 ? rank[k] : -1;
+    }
+#pragma unroll
+    for (int k = 0; k < 27; ++k) put(k, (nb[k] >= 0 && nb[k] < a.Hin) ? nb[k] : -1);
+  } else {
+#pragma unroll
+    for (int k = 0; k < 27; ++k) put(k, k < a.K ? conv_src(a, col, k) : -1);
+  }
+}
+
 template <int MT>
 __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* __restrict__ out,
     const float4* __restrict__ xt, const float* __restrict__ Wt, int n_tiles, int cpad) {
@@ -213,6 +240,11 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
   const int npass = (a.mtiles + MT - 1) / MT;
   const int cpad4 = cpad >> 2;
   const int nstage = a.K * nslab;
+  // source rows of all taps of the workgroup's 256 columns, looked up once and all together
+  // (inside the tap loop a look-up is a chain of two or three trips to memory per tap)
+  __shared__ int sSrc[27][kTileCols];
+  lookup_sources(a, tile * kTileCols + (int)threadIdx.x, [&](int k, int row) { sSrc[k][threadIdx.x] = row; });
+  __syncthreads();
   for (int pass = blockIdx.y; pass < npass; pass += gridDim.y) {  // passes may be dealt out over workgroups
     floatx16 acc[MT][2];
 #pragma unroll
@@ -235,7 +267,7 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
     // the weights AND all gathers of the next stage (8 channel groups x 2 columns, 16 bytes each)
     // are in flight; the source rows of a tap are looked up two taps ahead.
     float4 nx0[kRowSlabF / 8], nx1[kRowSlabF / 8];
-    auto src_of = [&](int k, int half) { return k < a.K ? conv_src(a, n0 + half * 32 + r, k) : -1; };
+    auto src_of = [&](int k, int half) { return k < a.K ? sSrc[k][wave * kWaveCols + half * 32 + r] : -1; };
     auto fetch_x = [&](int s0, int s1, int slab) {
       const float4* row0 = xt + (int64_t)(s0 < 0 ? a.Hin : s0) * cpad4 + kh;
       const float4* row1 = xt + (int64_t)(s1 < 0 ? a.Hin : s1) * cpad4 + kh;
@@ -249,6 +281,11 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
     };
     int s0c = src_of(0, 0), s1c = src_of(0, 1);      // rows of the current tap
     int s0n = src_of(1, 0), s1n = src_of(1, 1);      // ... of the next one
+    // A tap whose neighbour is missing for all 32 columns of a column tile adds nothing: its
+    // operands are not requested and its products not formed (over the non-empty nodes of a
+    // surface that is more than half of the (column tile, tap) pairs).  Uniform over the wavefront.
+    auto any_row = [](int src) { return __ballot(src >= 0) != 0; };
+    bool l0c = any_row(s0c), l1c = any_row(s1c), l0n = any_row(s0n), l1n = any_row(s1n);
     wr = fetch_w(0);
     fetch_x(s0c, s1c, 0);
     __syncthreads();  // the last stage of the previous pass may still be reading the weights
@@ -258,6 +295,7 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
     int stage = 0;
     for (int k = 0; k < a.K; ++k) {
       const int s0n2 = src_of(k + 2, 0), s1n2 = src_of(k + 2, 1);
+      const bool l0n2 = any_row(s0n2), l1n2 = any_row(s1n2);
       for (int slab = 0; slab < nslab; ++slab, ++stage) {
         // stage - 1 is over everywhere and the weights of this stage are in place; the weights
         // of the next stage (requested a stage ago) go into the other buffer while this one is
@@ -275,6 +313,7 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
         const bool same_tap = slab + 1 < nslab;
         const int nslab_next = same_tap ? slab + 1 : 0;
         const int s0x = same_tap ? s0c : s0n, s1x = same_tap ? s1c : s1n;
+        const bool l0x = same_tap ? l0c : l0n, l1x = same_tap ? l1c : l1n;
         const float4* nrow0 = xt + (int64_t)(s0x < 0 ? a.Hin : s0x) * cpad4 + kh + ((nslab_next * kRowSlabF) >> 2);
         const float4* nrow1 = xt + (int64_t)(s1x < 0 ? a.Hin : s1x) * cpad4 + kh + ((nslab_next * kRowSlabF) >> 2);
         const int ngroup_next = more ? (min(kRowSlabF, cpad - nslab_next * kRowSlabF) >> 3) : 0;
@@ -284,10 +323,10 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
         for (int c8 = 0; c8 < kRowSlabF / 8; ++c8) {
           const float4 b0 = nx0[c8], b1 = nx1[c8];
           if (c8 < ngroup_next) {
-            nx0[c8] = nrow0[c8 * 2];
-            nx1[c8] = nrow1[c8 * 2];
+            if (l0x) nx0[c8] = nrow0[c8 * 2];
+            if (l1x) nx1[c8] = nrow1[c8 * 2];
           }
-          if (c8 >= ngroup) continue;  // uniform
+          if (c8 >= ngroup || (!l0c && !l1c)) continue;  // uniform
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const float v0 = j == 0 ? b0.x : j == 1 ? b0.y : j == 2 ? b0.z : b0.w;
@@ -295,13 +334,14 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
               const float av = wcur[((c8 * 4 + j) * MT + mt) * 64 + lane];
-              acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, v0, acc[mt][0], 0, 0, 0);
-              acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, v1, acc[mt][1], 0, 0, 0);
+              if (l0c) acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, v0, acc[mt][0], 0, 0, 0);
+              if (l1c) acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, v1, acc[mt][1], 0, 0, 0);
             }
           }
         }
       }
       s0c = s0n; s1c = s1n; s0n = s0n2; s1n = s1n2;
+      l0c = l0n; l1c = l1n; l0n = l0n2; l1n = l1n2;
     }
     if (n0 < a.N) store_tiles<float, MT>(a, out, acc, pass * MT, n0, lane);
   }
@@ -454,32 +494,8 @@ __global__ __launch_bounds__(256, 2) void conv_rows_bf16_deep_kernel(ConvArgs a,
   const int cpad8 = cpad >> 3;
   const int ngroup = (a.K + kG - 1) / kG;
   {
-    const int col = tile * kTileCols + (int)threadIdx.x;
-    if (a.mode == kModeS1) {
-      // three dependent trips for all taps together: my node, its 27 neighbours (all in the 256-byte
-      // block of the node's sibling group), their ranks among the non-empty nodes
-      const bool mine = col < a.N;
-      const int node = mine ? (a.nempty ? a.ichild[col] : col) : 0;
-      const int* __restrict__ block = a.neigh + ((int64_t)(node >> 3) << 6) + sibling_slot(node & 7);
-      int nb[27];
-#pragma unroll
-      for (int k = 0; k < 27; ++k) nb[k] = (mine && k < a.K) ? block[a.slot[k]] : -1;
-      if (a.nempty) {
-        int rank[27];
-#pragma unroll
-        for (int k = 0; k < 27; ++k) rank[k] = a.child[max(nb[k], 0)];
-#pragma unroll
-        for (int k = 0; k < 27; ++k) nb[k] = nb[k] >= 0 ? rank[k] : -1;
-      }
-#pragma unroll
-      for (int k = 0; k < 27; ++k) sSrc[k][threadIdx.x] = ((nb[k] >= 0 && nb[k] < a.Hin) ? nb[k] : a.Hin) * cpad8;
-    } else {
-#pragma unroll
-      for (int k = 0; k < 27; ++k) {
-        const int sr = k < a.K ? conv_src(a, col, k) : -1;
-        sSrc[k][threadIdx.x] = (sr < 0 ? a.Hin : sr) * cpad8;
-      }
-    }
+    lookup_sources(a, tile * kTileCols + (int)threadIdx.x,
+        [&](int k, int row) { sSrc[k][threadIdx.x] = (row < 0 ? a.Hin : row) * cpad8; });
   }
   const int c0 = wave * kWaveCols + r;                  // my column of the first column tile, inside the workgroup's tile
   union Frag { u32x4 q; bf16x8 v; };
