@@ -281,9 +281,9 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
     };
     int s0c = src_of(0, 0), s1c = src_of(0, 1);      // rows of the current tap
     int s0n = src_of(1, 0), s1n = src_of(1, 1);      // ... of the next one
-    // A tap whose neighbour is missing for all 32 columns of a column tile adds nothing: its
-    // operands are not requested and its products not formed (over the non-empty nodes of a
-    // surface that is more than half of the (column tile, tap) pairs).  Uniform over the wavefront.
+    // A tap whose neighbour is missing for all 64 columns of the wavefront adds nothing: its
+    // products are not formed (over the non-empty nodes of a surface that is about half of the
+    // (wavefront, tap) pairs).  Uniform over the wavefront.
     auto any_row = [](int src) { return __ballot(src >= 0) != 0; };
     bool l0c = any_row(s0c), l1c = any_row(s1c), l0n = any_row(s0n), l1n = any_row(s1n);
     wr = fetch_w(0);
@@ -313,20 +313,23 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
         const bool same_tap = slab + 1 < nslab;
         const int nslab_next = same_tap ? slab + 1 : 0;
         const int s0x = same_tap ? s0c : s0n, s1x = same_tap ? s1c : s1n;
-        const bool l0x = same_tap ? l0c : l0n, l1x = same_tap ? l1c : l1n;
         const float4* nrow0 = xt + (int64_t)(s0x < 0 ? a.Hin : s0x) * cpad4 + kh + ((nslab_next * kRowSlabF) >> 2);
         const float4* nrow1 = xt + (int64_t)(s1x < 0 ? a.Hin : s1x) * cpad4 + kh + ((nslab_next * kRowSlabF) >> 2);
         const int ngroup_next = more ? (min(kRowSlabF, cpad - nslab_next * kRowSlabF) >> 3) : 0;
         if (stage + 2 < nstage) wr = fetch_w(stage + 2);
         const int ngroup = min(kRowSlabF, cpad - slab * kRowSlabF) >> 3;
+        // Both column tiles or none: the test is made once per stage and the MFMAs stay one
+        // straight-line block (a body per case of (tile 0 live, tile 1 live) made the compiler
+        // move the 64 accumulator registers at every join; a branch per MFMA breaks up their issue).
+        const bool live = l0c || l1c;
 #pragma unroll
         for (int c8 = 0; c8 < kRowSlabF / 8; ++c8) {
           const float4 b0 = nx0[c8], b1 = nx1[c8];
-          if (c8 < ngroup_next) {
-            if (l0x) nx0[c8] = nrow0[c8 * 2];
-            if (l1x) nx1[c8] = nrow1[c8 * 2];
+          if (c8 < ngroup_next) {   // requested whether live or not (a dead tile reads the zero row, which
+            nx0[c8] = nrow0[c8 * 2];  // stays in the L1): a branch per request would cost the waits their order
+            nx1[c8] = nrow1[c8 * 2];
           }
-          if (c8 >= ngroup || (!l0c && !l1c)) continue;  // uniform
+          if (c8 >= ngroup || !live) continue;  // uniform
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const float v0 = j == 0 ? b0.x : j == 1 ? b0.y : j == 2 ? b0.z : b0.w;
@@ -334,8 +337,8 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
               const float av = wcur[((c8 * 4 + j) * MT + mt) * 64 + lane];
-              if (l0c) acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, v0, acc[mt][0], 0, 0, 0);
-              if (l1c) acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, v1, acc[mt][1], 0, 0, 0);
+              acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, v0, acc[mt][0], 0, 0, 0);
+              acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, v1, acc[mt][1], 0, 0, 0);
             }
           }
         }
