@@ -478,11 +478,14 @@ __global__ __launch_bounds__(256) void conv_rows_bf16_kernel(ConvArgs a, uint16_
 // per column from the L2, 0.8 GB per launch, where the matrix work is 20 microseconds; neighbouring
 // columns share most of their rows, which only a per-tile list of distinct rows staged in LDS
 // would exploit.
-template <int MT>
+// SLAB: input channels per stage.  MT = 4 (128 output channels a pass) with 32-channel stages halves the
+// operand bytes per MFMA against MT = 2 with 64-channel stages at the same LDS and register budget: two
+// row tiles share a gathered operand at MT = 2, four at MT = 4, and the L1 delivers 64 bytes a cycle.
+template <int MT, int SLAB>
 __global__ __launch_bounds__(256, 2) void conv_rows_bf16_deep_kernel(ConvArgs a, uint16_t* __restrict__ out,
     const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles, int cpad) {
   constexpr int kG = 3;                                 // taps per weight group
-  constexpr int kKs = kRowSlab / 16;                    // k-steps per slab
+  constexpr int kKs = SLAB / 16;                    // k-steps per slab
   constexpr int kWUnits = kKs * MT * 64;                // 16-byte units of one (tap, slab)
   constexpr int kWVec = kG * kWUnits / 256;             // per thread and group
   __shared__ u32x4 sW[2][kG * kWUnits];
@@ -492,7 +495,7 @@ __global__ __launch_bounds__(256, 2) void conv_rows_bf16_deep_kernel(ConvArgs a,
   if (tile >= n_tiles) return;
   const int n0 = tile * kTileCols + wave * kWaveCols;
   const int r = lane & 31, kh = lane >> 5;
-  const int nslab = (cpad + kRowSlab - 1) / kRowSlab;
+  const int nslab = (cpad + SLAB - 1) / SLAB;
   const int npass = (a.mtiles + MT - 1) / MT;
   const int cpad8 = cpad >> 3;
   const int ngroup = (a.K + kG - 1) / kG;
@@ -530,8 +533,8 @@ __global__ __launch_bounds__(256, 2) void conv_rows_bf16_deep_kernel(ConvArgs a,
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
     for (int slab = 0; slab < nslab; ++slab) {
-      const int nks = min(kRowSlab, cpad - slab * kRowSlab) >> 4;    // k-steps of this slab (uniform)
-      const int col16 = ((slab * kRowSlab) >> 3) + kh;               // my 16-byte unit inside a row
+      const int nks = min(SLAB, cpad - slab * SLAB) >> 4;    // k-steps of this slab (uniform)
+      const int col16 = ((slab * SLAB) >> 3) + kh;               // my 16-byte unit inside a row
       u32x4 wr[kWVec];
       // group g of this (pass, slab): taps 3g .. 3g+2, each kWUnits units at ((pass K + tap) nslab + slab) kWUnits
       auto fetch_w = [&](int g) {
@@ -602,19 +605,19 @@ __global__ __launch_bounds__(256, 2) void conv_rows_bf16_deep_kernel(ConvArgs a,
 
 // [pass][tap][slab][c16][mt][lane][j]: lane (m, kh), j <- W'(m, slab*64 + c16*16 + 8kh + j, tap)
 __global__ void pack_weights_rows_bf16(uint16_t* __restrict__ Wt, const uint16_t* __restrict__ W, int M, int Cin,
-    int K, int MT, int npass, int nslab, int64_t sm, int64_t sc) {
+    int K, int MT, int npass, int nslab, int64_t sm, int64_t sc, int slab_ch) {
   int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  int64_t total = (int64_t)npass * K * nslab * (kRowSlab / 16) * MT * 64 * 8;
+  int64_t total = (int64_t)npass * K * nslab * (slab_ch / 16) * MT * 64 * 8;
   if (id >= total) return;
   int j = (int)(id & 7);
   int l = (int)((id >> 3) & 63);
   int64_t f = id >> 9;
   int mt = (int)(f % MT); f /= MT;
-  int c16 = (int)(f % (kRowSlab / 16)); f /= (kRowSlab / 16);
+  int c16 = (int)(f % (slab_ch / 16)); f /= (slab_ch / 16);
   int slab = (int)(f % nslab); f /= nslab;
   int k = (int)(f % K);
   int pass = (int)(f / K);
-  int m = (pass * MT + mt) * 32 + (l & 31), c = slab * kRowSlab + c16 * 16 + 8 * (l >> 5) + j;
+  int m = (pass * MT + mt) * 32 + (l & 31), c = slab * slab_ch + c16 * 16 + 8 * (l >> 5) + j;
   Wt[id] = (m < M && c < Cin) ? W[m * sm + c * sc + k] : (uint16_t)0;
 }
 
@@ -2321,26 +2324,32 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     else
       conv_s1_bf16_lds_kernel<2><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad / 8);
   } else {
-    const int MT = a.mtiles == 1 ? 1 : 2;
+    const bool deep = a.K >= 3;   // fewer taps than a weight group: the shallow kernel
+    // 128 output channels a pass where the operator has whole blocks of them (see the kernel)
+    const bool wide = deep && a.mtiles % 4 == 0;
+    const int MT = a.mtiles == 1 ? 1 : (wide ? 4 : 2);
+    const int slab_ch = wide ? 32 : kRowSlab;
     const int cpad = (a.Cin + 15) / 16 * 16;
-    const int npass = (a.mtiles + MT - 1) / MT, nslab = (cpad + kRowSlab - 1) / kRowSlab;
-    int64_t total = (int64_t)npass * a.K * nslab * (kRowSlab / 16) * MT * 64 * 8;
+    const int npass = (a.mtiles + MT - 1) / MT, nslab = (cpad + slab_ch - 1) / slab_ch;
+    int64_t total = (int64_t)npass * a.K * nslab * (slab_ch / 16) * MT * 64 * 8;
     pack_weights_rows_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)wsb, (const uint16_t*)weights, a.M,
-        a.Cin, a.K, MT, npass, nslab, sm, sc);
+        a.Cin, a.K, MT, npass, nslab, sm, sc, slab_ch);
     OCNN_LAUNCH_OK("pack_weights_rows");
     uint16_t* xt = (uint16_t*)(wsb + p.wt_bytes + p.ichild_bytes);
     dim3 tg((a.Hin + 1 + 127) / 128, (cpad + 63) / 64);
     transpose_rows_bf16_kernel<<<tg, 256, 0, s>>>(xt, (const uint16_t*)btm, a.Cin, a.Hin, cpad);
     OCNN_LAUNCH_OK("transpose_rows");
-    const bool deep = a.K >= 3;   // fewer taps than a weight group: the shallow kernel
-    if (deep && MT == 1)
-      conv_rows_bf16_deep_kernel<1><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
+    const dim3 rgrid(grid, pass_split(n_tiles, npass));
+    if (wide)
+      conv_rows_bf16_deep_kernel<4, 32><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
+    else if (deep && MT == 1)
+      conv_rows_bf16_deep_kernel<1, kRowSlab><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
     else if (deep)
-      conv_rows_bf16_deep_kernel<2><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
+      conv_rows_bf16_deep_kernel<2, kRowSlab><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
     else if (MT == 1)
-      conv_rows_bf16_kernel<1><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
+      conv_rows_bf16_kernel<1><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
     else
-      conv_rows_bf16_kernel<2><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
+      conv_rows_bf16_kernel<2><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
   }
   OCNN_LAUNCH_OK("octree_conv");
   return OCNN_OK;

@@ -305,6 +305,35 @@ def test_conv_wide_channels(oc, orc, tree):
     assert relerr(got16.float().cpu().numpy().reshape(exp.shape), exp) < TOL_BF16, (d, ci, co)
 
 
+def test_conv_wide_channels_nonempty(oc, orc, tree):
+  """The row kernels with whole blocks of 128 output channels (four row tiles a pass, 32-channel
+  stages in bf16), input channel counts that leave a partial last stage, more than one pass, and
+  the stride-2 shapes of the U-Net trunk, over the non-empty nodes."""
+  b, dev, host = tree["blob"], tree["dev"], tree["host"]
+  rng = np.random.default_rng(6)
+  for d, ci, co, ks, stride in ((5, 64, 128, [3, 3, 3], 1), (4, 48, 256, [3, 3, 3], 1), (4, 80, 128, [3, 3, 3], 1),
+                                (5, 128, 384, [3, 1, 1], 1), (5, 64, 128, [2, 2, 2], 2), (4, 256, 128, [3, 3, 3], 1)):
+    K = ks[0] * ks[1] * ks[2]
+    hin = int(b.nnum_nempty[d])
+    x = rng.standard_normal((ci, hin)).astype(np.float32)
+    w = (rng.standard_normal((co, ci * K)) * 0.02).astype(np.float32)
+    exp = orc.octree_conv(x, w, host, d, co, ks, stride, True)
+    xt, wt = T(x).cuda().view(1, ci, hin, 1), T(w).cuda()
+    got = oc.nn.octree_conv(xt, wt, dev, d, co, ks, stride, True)
+    assert relerr(got.cpu().numpy().reshape(exp.shape), exp) < TOL_F32, (d, ci, co, ks)
+    got16 = oc.nn.octree_conv(xt.bfloat16(), wt.bfloat16(), dev, d, co, ks, stride, True)
+    assert relerr(got16.float().cpu().numpy().reshape(exp.shape), exp) < TOL_BF16, (d, ci, co, ks)
+  # deconvolution over the non-empty nodes with 128 output channels
+  d, ci, co = 4, 64, 128
+  hin = int(b.nnum_nempty[d])
+  x = rng.standard_normal((ci, hin)).astype(np.float32)
+  w = (rng.standard_normal((ci, co * 8)) * 0.05).astype(np.float32)
+  exp = orc.octree_deconv(x, w, host, d, co, [2, 2, 2], 2, True)
+  got16 = oc.nn.octree_deconv(T(x).cuda().view(1, ci, hin, 1).bfloat16(), T(w).cuda().bfloat16(), dev, d, co,
+                              [2, 2, 2], 2, True)
+  assert relerr(got16.float().cpu().numpy().reshape(exp.shape), exp) < TOL_BF16
+
+
 def test_conv_on_reference_sample_batch(oc, orc, tree):
   """The shapes of pytorch/test/test_octree_conv.py: depth 4, 3 -> 5 channels."""
   sb, sdev, shost = tree["sblob"], tree["sdev"], tree["shost"]
