@@ -229,6 +229,14 @@ def main():
     xne = torch.randn(1, C, Hne9, 1, generator=g).to(dev)
     conv_case("conv333_s1_d9_f32_nempty", octree, 9, xne, w32, [3, 3, 3], 1, nempty=True)
     conv_case("conv333_s1_d9_bf16_nempty", octree, 9, xne.bfloat16(), w16, [3, 3, 3], 1, nempty=True)
+    rows_ne = F.to_rows(xne.bfloat16())
+    rows_ne_out = torch.empty(Hne9 + 1, F.rows_pitch(C), dtype=torch.bfloat16, device=dev)
+    t = timed(lambda: F.octree_conv_rows(rows_ne, C, w16, octree, 9, C, out=rows_ne_out, nempty=True), reps, wu)
+    fl = 2.0 * Hne9 * 27 * C * C
+    extra["conv333_s1_d9_bf16_nempty_rows"] = {"ms": t, "octants_per_s": Hne9 / (t * 1e-3), "tflops": fl / (t * 1e-3) / 1e12,
+                                               "frac_mfma_peak": fl / (t * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS["bf16"],
+                                               "layout": "row-major in and out, no copy; flops counted densely (27 taps a column)"}
+    del rows_ne, rows_ne_out
     x8 = torch.randn(1, C, Hne8, 1, generator=g).to(dev)
     conv_case("deconv222_s2_d8to9_f32", octree, 8, x8, w2, [2, 2, 2], 2, deconv=True)
 
@@ -478,6 +486,8 @@ def main():
     extra["unet_trunk_scene_d9_f32_nempty"] = {"ms": t, "points_per_s": 250000 / (t * 1e-3)}
     t = timed(lambda: oc.stacks.unet_trunk(octree, 9, up16, data=fne16, nempty=True), max(2, reps // 2), 1)
     extra["unet_trunk_scene_d9_bf16_nempty"] = {"ms": t, "points_per_s": 250000 / (t * 1e-3)}
+    t = timed(lambda: oc.stacks.unet_trunk_rows(octree, 9, up16, data=fne16, nempty=True), max(2, reps // 2), 1)
+    extra["unet_trunk_scene_d9_bf16_nempty_rows"] = {"ms": t, "points_per_s": 250000 / (t * 1e-3)}
     clouds2 = [points_tensor(*oc.synthetic.shape_cloud(10000, 100 + i)) for i in range(32)]
     oct6 = F.points2octree_batch(clouds2, 6, 2)
     lch = {6: (3, 32), 5: (32, 64), 4: (64, 128), 3: (128, 256)}

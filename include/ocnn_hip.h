@@ -192,7 +192,7 @@ int ocnn_octree_conv_fused(void* top, const void* btm, int channel_in, int btm_h
  * points copy their input into it on every call.  A chain of convolutions converts once
  * (ocnn_rows_from_channels), runs ocnn_octree_conv_rows for every member, and converts back once
  * (ocnn_channels_from_rows).
- *   ocnn_octree_conv_rows: bf16, nempty 0, and
+ *   ocnn_octree_conv_rows: bf16; with nempty 0
  *     kernel 3x3x3 stride 1 (conv or deconv): rows of `depth` in and out; arithmetic and rounding
  *       as ocnn_octree_conv_fused, the results are bit-identical;
  *     kernel 2x2x2 stride 2, conv: rows of `depth` in, rows of ALL nodes of depth-1 out: the
@@ -200,15 +200,18 @@ int ocnn_octree_conv_fused(void* top, const void* btm, int channel_in, int btm_h
  *       (pytorch/ocnn/octree_conv.py:102-127) is folded in, an empty node receives the bias alone;
  *     kernel 2x2x2 stride 2, deconv: rows of ALL nodes of `depth` in (the octree_depad of those
  *       modules is folded in), rows of depth+1 out; input channels padded to 16 .. 256;
- *     anything else: OCNN_E_UNSUPPORTED.
+ *   with nempty 1 (rows = ranks of the non-empty nodes on both sides, the operator of the
+ *   channel-major entry points, pytorch/cpp/octree_conv.cpp:131-216): kernel 3x3x3 stride 1 and
+ *   kernel 2x2x2 stride 2, conv and deconv;
+ *   anything else: OCNN_E_UNSUPPORTED.
  *   btm_pitch = 16 * ceil(channel_in / 16) (the stride-2 convolution also takes a larger multiple
- *   of 8: its input may be a channel slice of a wider tensor).  top_pitch: channels per row of the tensor `top_rows`
+ *   of 8: its input may be a channel slice of a wider tensor; so do the nempty operators).  top_pitch: channels per row of the tensor `top_rows`
  *   points into, a multiple of 8, at least 16 * ceil(num_output / 16); the call writes channels
  *   0 .. 16 * ceil(num_output / 16) - 1 of every row and of the zero row and nothing else, so
  *   `top_rows` may be a channel slice of a wider tensor.  ocnn_conv_rows_shape: row counts and
  *   workspace bytes of such a call. */
 int ocnn_conv_rows_shape(const void* info, int depth, int channel_in, int num_output, const int* kernel_size,
-    int stride, int is_deconv, int dtype, int* top_h, int* btm_h, size_t* workspace_bytes);
+    int stride, int nempty, int is_deconv, int dtype, int* top_h, int* btm_h, size_t* workspace_bytes);
 int ocnn_octree_conv_rows(void* top_rows, int top_pitch, const void* btm_rows, int btm_pitch, int channel_in,
     int btm_h, const void* weights, const float* bias, int relu, int is_deconv, const void* octree_dev,
     const void* info, int depth, int num_output, const int* kernel_size, int stride, int nempty, int dtype,

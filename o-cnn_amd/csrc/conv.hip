@@ -461,6 +461,68 @@ __global__ __launch_bounds__(256) void conv_rows_bf16_kernel(ConvArgs a, uint16_
     if (n0 < a.N) store_tiles<uint16_t, MT>(a, out, acc, pass * MT, n0, lane);
   }
 }
+// A 16-byte store reads its four data registers for a while after it has issued, and the next
+// instruction that writes one of them has to keep two wait states' distance.  The compiler puts
+// them in when store and writer share a basic block; the row-major stores sit in conditional blocks
+// of their own, and the value computed for the next store landed in a register the store was
+// still reading (seen as a few wrong words per million).  So the wait goes in by hand.
+#define OCNN_STORE_DATA_WAIT() asm volatile("s_nop 1")
+
+// Row-major epilogue of the 32x32 accumulator tiles acc[MT][2] of a wavefront (columns n0 .. n0 + 63,
+// channels cb + 32 mt ..): lane (r, kh) holds channels cb + 32 mt + 8 q + 4 kh + e of its two
+// columns; the lanes r and r + 32 swap halves, so that each ends up with 8 consecutive channels and
+// stores 16 bytes (32 contiguous bytes per row and store).  A column behind the level gets an
+// offset past the end of the buffer and the hardware drops its store.
+template <int MT>
+__device__ inline void rows_out_tiles(const ConvArgs& a, uint16_t* __restrict__ out, int out_pitch, int out_cpad,
+    floatx16 (&acc)[MT][2], int cb, int n0, int lane) {
+  typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  typedef float floatx2_t __attribute__((ext_vector_type(2)));
+  const int r = lane & 31, kh = lane >> 5;
+  const __amdgpu_buffer_rsrc_t obuf = __builtin_amdgcn_make_buffer_rsrc(
+      out, 0, (int)(((int64_t)a.Hout + 1) * out_pitch * 2), 0x00020000);
+  const float floor = a.relu ? 0.0f : -__builtin_inff();
+  auto pack = [](float lo, float hi) {
+    floatx2_t f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+  };
+  auto clamp = [&](float v) { return v < floor ? floor : v; };   // keeps a NaN
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    float bias[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int ch = cb + 32 * mt + 8 * (i / 4) + 4 * kh + (i % 4);
+      bias[i] = a.bias ? a.bias[min(ch, a.M - 1)] : 0.0f;
+      if (ch >= a.M) bias[i] = 0.0f;   // the padding channels of a row stay zero
+    }
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      const int n = n0 + nt * 32 + r;
+      const int ooff = n < a.N ? (n * out_pitch + 8 * kh) * 2 : 0x7fffff00;
+      uint32_t w[4][2];
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int i = 4 * q + 2 * h;
+          w[q][h] = pack(clamp(acc[mt][nt][i] + bias[i]), clamp(acc[mt][nt][i + 1] + bias[i + 1]));
+        }
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj) {
+        const auto s0 = __builtin_amdgcn_permlane32_swap(w[2 * jj][0], w[2 * jj + 1][0], false, false);
+        const auto s1 = __builtin_amdgcn_permlane32_swap(w[2 * jj][1], w[2 * jj + 1][1], false, false);
+        if (cb + 32 * mt + 16 * jj < out_cpad) {
+          __builtin_amdgcn_raw_buffer_store_b128(u32x4_t{s0[0], s1[0], s0[1], s1[1]}, obuf, ooff,
+              (cb + 32 * mt + 16 * jj) * 2, 0);
+          OCNN_STORE_DATA_WAIT();
+        }
+      }
+    }
+  }
+}
+
 // The same operator with a deeper pipeline, for tap sets of three taps or more.  The kernel
 // above pays two barriers per (tap, 64-channel slab) for 16 MFMAs per wavefront and has one
 // stage of gathers in flight; with 27 rows to fetch per column from the L2 that leaves the
@@ -481,9 +543,11 @@ __global__ __launch_bounds__(256) void conv_rows_bf16_kernel(ConvArgs a, uint16_
 // SLAB: input channels per stage.  MT = 4 (128 output channels a pass) with 32-channel stages halves the
 // operand bytes per MFMA against MT = 2 with 64-channel stages at the same LDS and register budget: two
 // row tiles share a gathered operand at MT = 2, four at MT = 4, and the L1 delivers 64 bytes a cycle.
-template <int MT, int SLAB>
+// ROWS_OUT: row-major output ([Hout + 1][out_pitch], channels below out_cpad and the zero row written),
+// as the row-major kernels further down write it.
+template <int MT, int SLAB, bool ROWS_OUT>
 __global__ __launch_bounds__(256, 2) void conv_rows_bf16_deep_kernel(ConvArgs a, uint16_t* __restrict__ out,
-    const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles, int cpad) {
+    const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles, int cpad, int in_pitch, int out_pitch, int out_cpad) {
   constexpr int kG = 3;                                 // taps per weight group
   constexpr int kKs = SLAB / 16;                    // k-steps per slab
   constexpr int kWUnits = kKs * MT * 64;                // 16-byte units of one (tap, slab)
@@ -497,7 +561,7 @@ __global__ __launch_bounds__(256, 2) void conv_rows_bf16_deep_kernel(ConvArgs a,
   const int r = lane & 31, kh = lane >> 5;
   const int nslab = (cpad + SLAB - 1) / SLAB;
   const int npass = (a.mtiles + MT - 1) / MT;
-  const int cpad8 = cpad >> 3;
+  const int cpad8 = in_pitch >> 3;   // 16-byte units per input row (the pitch; the channels read are below cpad)
   const int ngroup = (a.K + kG - 1) / kG;
   {
     lookup_sources(a, tile * kTileCols + (int)threadIdx.x,
@@ -599,7 +663,13 @@ __global__ __launch_bounds__(256, 2) void conv_rows_bf16_deep_kernel(ConvArgs a,
         }
       }
     }
-    if (n0 < a.N) store_tiles<uint16_t, MT>(a, out, acc, pass * MT, n0, lane);
+    if constexpr (ROWS_OUT) {
+      rows_out_tiles<MT>(a, out, out_pitch, out_cpad, acc, pass * MT * 32, n0, lane);
+      if (tile == 0 && wave == 0 && lane * 8 >= pass * MT * 32 && lane * 8 < min((pass + 1) * MT * 32, out_cpad))
+        *reinterpret_cast<uint4*>(out + (int64_t)a.Hout * out_pitch + lane * 8) = make_uint4(0, 0, 0, 0);
+    } else {
+      if (n0 < a.N) store_tiles<uint16_t, MT>(a, out, acc, pass * MT, n0, lane);
+    }
   }
 }
 
@@ -1012,12 +1082,6 @@ __global__ __launch_bounds__(256, 2) void conv_s1_bf16_lds_kernel(ConvArgs a, ui
 // barrier per k-step); a wavefront reads each tap's fragment twice per k-step, 0.25 KiB of LDS
 // operands per MFMA.  The neighbour rows of a wavefront's groups wait in LDS too (68 words per
 // group: 16-byte reads of 32 lanes then meet no bank twice).
-// A 16-byte store reads its four data registers for a while after it has issued, and the next
-// instruction that writes one of them has to keep two wait states' distance.  The compiler puts
-// them in when store and writer share a basic block; the stores below sit in conditional blocks of
-// their own, and the value computed for the next store landed in a register the store was
-// still reading (seen as a few wrong words per million).  So the wait goes in by hand.
-#define OCNN_STORE_DATA_WAIT() asm volatile("s_nop 1")
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
 
@@ -2341,11 +2405,11 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     OCNN_LAUNCH_OK("transpose_rows");
     const dim3 rgrid(grid, pass_split(n_tiles, npass));
     if (wide)
-      conv_rows_bf16_deep_kernel<4, 32><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
+      conv_rows_bf16_deep_kernel<4, 32, false><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad, cpad, 0, 0);
     else if (deep && MT == 1)
-      conv_rows_bf16_deep_kernel<1, kRowSlab><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
+      conv_rows_bf16_deep_kernel<1, kRowSlab, false><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad, cpad, 0, 0);
     else if (deep)
-      conv_rows_bf16_deep_kernel<2, kRowSlab><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
+      conv_rows_bf16_deep_kernel<2, kRowSlab, false><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad, cpad, 0, 0);
     else if (MT == 1)
       conv_rows_bf16_kernel<1><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad);
     else
@@ -2914,7 +2978,7 @@ int make_rows_plan(const Info* o, int depth, int channel_in, int num_output, con
   OCNN_REQUIRE(o && ks, OCNN_E_BADARG, "null pointer");
   int e = ocnn_info_check(o);
   if (e) return e;
-  OCNN_REQUIRE(dtype == OCNN_BF16 && !nempty, OCNN_E_UNSUPPORTED, "row-major operators: bf16, all nodes");
+  OCNN_REQUIRE(dtype == OCNN_BF16, OCNN_E_UNSUPPORTED, "row-major operators: bf16");
   OCNN_REQUIRE(depth > 0 && depth <= o->depth, OCNN_E_BADARG, "depth %d not in [1,%d]", depth, o->depth);
   OCNN_REQUIRE(num_output > 0 && channel_in > 0, OCNN_E_BADARG, "channels %d -> %d", channel_in, num_output);
   OCNN_REQUIRE(o->has(OCNN_NEIGH) && o->has(OCNN_CHILD), OCNN_E_FORMAT,
@@ -2925,7 +2989,23 @@ int make_rows_plan(const Info* o, int depth, int channel_in, int num_output, con
   r->ksteps = r->cpad / 16;
   r->ichild_bytes = 0;
   const int mtiles = (num_output + 31) / 32;
-  if (stride == 1 && k333) {
+  if (nempty) {
+    // over the non-empty nodes: the general row kernel (rows = ranks of the non-empty nodes on
+    // both sides, exactly the operator of the channel-major entry points)
+    OCNN_REQUIRE((stride == 1 && k333) || (stride == 2 && k222), OCNN_E_UNSUPPORTED,
+        "row-major operators: 3x3x3 stride 1, 2x2x2 stride 2");
+    ConvPlan p;
+    e = make_plan(o, depth, channel_in, num_output, ks, stride, 1, deconv, dtype, &p);
+    if (e) return e;
+    r->kind = 3;
+    r->btm_h = p.btm_h;
+    r->top_h = r->cols = p.top_h;
+    const bool wide = mtiles % 4 == 0;
+    r->MT = mtiles == 1 ? 1 : (wide ? 4 : 2);
+    r->npass = (mtiles + r->MT - 1) / r->MT;
+    r->wt_bytes = p.wt_bytes;
+    r->ichild_bytes = p.ichild_bytes;
+  } else if (stride == 1 && k333) {
     r->kind = 0;
     r->btm_h = r->top_h = r->cols = o->nnum[depth];
     r->MT = mtiles == 1 ? 1 : 2;
@@ -2970,7 +3050,7 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
       r.btm_h, depth);
   // the stride-2 convolution also reads a channel slice of a wider tensor (an encoder feature that
   // sits in the tensor the decoder reads as a concatenation)
-  OCNN_REQUIRE(btm_pitch == r.cpad || (r.kind == 1 && btm_pitch > r.cpad && btm_pitch % 8 == 0), OCNN_E_SHAPE,
+  OCNN_REQUIRE(btm_pitch == r.cpad || ((r.kind == 1 || r.kind == 3) && btm_pitch > r.cpad && btm_pitch % 8 == 0), OCNN_E_SHAPE,
       "input pitch %d: rows of %d channels are padded to %d", btm_pitch, channel_in, r.cpad);
   OCNN_REQUIRE(top_pitch >= r.out_cpad && top_pitch % 8 == 0, OCNN_E_SHAPE, "output pitch %d for %d channels",
       top_pitch, num_output);
@@ -2996,6 +3076,50 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
   a.bias = bias;
   a.relu = relu ? 1 : 0;
   for (int k = 0; k < 27; ++k) a.slot[k] = 0;
+  if (r.kind == 3) {
+    ConvPlan p;
+    e = make_plan(o, depth, channel_in, num_output, ks, stride, 1, deconv, dtype, &p);
+    if (e) return e;
+    const bool empty_level = o->nnum_nempty[p.top_depth] == 0;
+    if (empty_level) {   // one zero row (octree_conv.cpp:82) and the zero row behind it
+      OCNN_REQUIRE(top_pitch == r.out_cpad, OCNN_E_UNSUPPORTED, "empty level into a channel slice");
+      const int64_t cnt = ((int64_t)r.top_h + 1) * top_pitch;
+      zero_rows_kernel<uint16_t><<<blocks_for(cnt), kBlock, 0, s>>>((uint16_t*)top_rows, cnt);
+      OCNN_LAUNCH_OK("zero_rows");
+      return OCNN_OK;
+    }
+    a.K = p.taps.count;
+    a.mode = p.mode;
+    a.nempty = 1;
+    for (int k = 0; k < 27; ++k) {
+      const int tap = k < p.taps.count ? p.taps.tap[k] : 13;
+      a.slot[k] = tap_slot(deconv && stride == 1 ? 26 - tap : tap);
+    }
+    a.neigh = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_NEIGH, p.workspace_depth));
+    a.child = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_CHILD, p.workspace_depth));
+    int* ichild = reinterpret_cast<int*>(wsb + p.wt_bytes);
+    ichild_kernel<<<blocks_for(p.child_h), kBlock, 0, s>>>(ichild, p.ichild_h, a.child, p.child_h);
+    a.ichild = ichild;
+    const int64_t sm = deconv ? a.K : (int64_t)channel_in * a.K, sc = deconv ? (int64_t)num_output * a.K : a.K;
+    const int slab_ch = r.MT == 4 ? 32 : kRowSlab;
+    const int nslab = (r.cpad + slab_ch - 1) / slab_ch;
+    const int64_t total = (int64_t)r.npass * a.K * nslab * (slab_ch / 16) * r.MT * 64 * 8;
+    pack_weights_rows_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)ws, (const uint16_t*)weights, a.M, a.Cin,
+        a.K, r.MT, r.npass, nslab, sm, sc, slab_ch);
+    const int n_tiles = (a.N + kTileCols - 1) / kTileCols;
+    const dim3 grid(((n_tiles + 7) / 8) * 8, pass_split(n_tiles, r.npass));
+    if (r.MT == 4)
+      conv_rows_bf16_deep_kernel<4, 32, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
+          (const u32x4*)ws, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
+    else if (r.MT == 2)
+      conv_rows_bf16_deep_kernel<2, kRowSlab, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
+          (const u32x4*)ws, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
+    else
+      conv_rows_bf16_deep_kernel<1, kRowSlab, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
+          (const u32x4*)ws, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
+    OCNN_LAUNCH_OK("octree_conv_rows");
+    return OCNN_OK;
+  }
   if (r.top_h == 0 || r.cols == 0) {   // nothing to convolve: zero rows (one data row at least, and the zero row)
     const int64_t cnt = ((int64_t)r.top_h + 1) * top_pitch;
     OCNN_REQUIRE(top_pitch == r.out_cpad, OCNN_E_UNSUPPORTED, "empty level into a channel slice");
@@ -3140,9 +3264,9 @@ int ocnn_octree_conv_rows(void* top_rows, int top_pitch, const void* btm_rows, i
 }
 
 int ocnn_conv_rows_shape(const void* info, int depth, int channel_in, int num_output, const int* kernel_size,
-    int stride, int is_deconv, int dtype, int* top_h, int* btm_h, size_t* workspace_bytes) {
+    int stride, int nempty, int is_deconv, int dtype, int* top_h, int* btm_h, size_t* workspace_bytes) {
   RowsPlan r;
-  int e = make_rows_plan(as_info(info), depth, channel_in, num_output, kernel_size, stride, 0, is_deconv, dtype, &r);
+  int e = make_rows_plan(as_info(info), depth, channel_in, num_output, kernel_size, stride, nempty, is_deconv, dtype, &r);
   if (e) return e;
   if (top_h) *top_h = r.top_h;
   if (btm_h) *btm_h = r.btm_h;

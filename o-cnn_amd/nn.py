@@ -766,7 +766,7 @@ def from_rows(rows, channels):
 
 
 def octree_conv_rows(rows_in, channel_in, weights, octree, depth, num_output, bias=None, relu=False,
-                     deconv=False, out=None, kernel_size=(3, 3, 3), stride=1):
+                     deconv=False, out=None, kernel_size=(3, 3, 3), stride=1, nempty=False):
   """Convolutions over all nodes in bf16, row-major on both sides: the arithmetic of octree_conv /
   octree_conv_fused (pytorch/cpp/octree_conv.cpp:131-216) on tensors that a chain of convolutions
   keeps in the layout the kernels gather from, so that no member of the chain copies its input.
@@ -776,6 +776,8 @@ def octree_conv_rows(rows_in, channel_in, weights, octree, depth, num_output, bi
       receives the bias alone;
     2x2x2 stride 2 deconv: rows of ALL nodes of `depth` in (the octree_depad of those modules is
       folded in), rows of depth+1 out.
+  With nempty=True the rows on both sides are the ranks of the non-empty nodes, as in the
+  channel-major operators (3x3x3 stride 1 and 2x2x2 stride 2, conv and deconv).
   rows_in: [H + 1, rows_pitch(channel_in)] as to_rows makes it.  `out`: [top_h + 1, P] with
   P >= rows_pitch(num_output), or columns c0 .. c0 + rows_pitch(num_output) of such a tensor (a
   slice of what a later layer reads as a concatenation); returns `out`."""
@@ -790,7 +792,7 @@ def octree_conv_rows(rows_in, channel_in, weights, octree, depth, num_output, bi
     raise TypeError("weights and data must have the same dtype")
   btm_h = rows_in.size(0) - 1
   top_h, need_h, ws_bytes = C.c_int(), C.c_int(), C.c_size_t()
-  _lib.call("ocnn_conv_rows_shape", info.p, depth, channel_in, num_output, ksc, stride, int(deconv), dt,
+  _lib.call("ocnn_conv_rows_shape", info.p, depth, channel_in, num_output, ksc, stride, int(nempty), int(deconv), dt,
             C.byref(top_h), C.byref(need_h), C.byref(ws_bytes))
   ws = _workspace(ws_bytes.value + 256, "conv")
   base = (ws.data_ptr() + 255) & ~255
@@ -806,7 +808,7 @@ def octree_conv_rows(rows_in, channel_in, weights, octree, depth, num_output, bi
       raise OcnnError(-3, "bias needs num_output entries")
   _lib.call("ocnn_octree_conv_rows", _ptr(out), out.stride(0), _ptr(rows_in), rows_in.stride(0), channel_in, btm_h,
             _ptr(weights), _ptr(bias), int(relu), int(deconv), _ptr(octree), info.p, depth, num_output, ksc, stride,
-            0, dt, C.c_void_p(base), C.c_size_t(ws_bytes.value), _stream())
+            int(nempty), dt, C.c_void_p(base), C.c_size_t(ws_bytes.value), _stream())
   return out
 
 

@@ -108,36 +108,42 @@ def unet_trunk(octree, depth, params, data=None, stages=3, nempty=False):
   return x
 
 
-def unet_trunk_rows(octree, depth, params, data=None, stages=3):
-  """unet_trunk over all nodes in bf16 with row-major activations between the operators: the
-  input is converted once, every convolution reads the layout its kernel gathers from and writes
-  it for the next one (pad and depad around the stride-2 layers are part of those operators,
-  both halves of a concatenation are written in place), and the result is converted back once.
+def unet_trunk_rows(octree, depth, params, data=None, stages=3, nempty=False):
+  """unet_trunk in bf16 with row-major activations between the operators: the input is converted
+  once, every convolution reads the layout its kernel gathers from and writes it for the next one
+  (over all nodes the pad and depad around the stride-2 layers are part of those operators; both
+  halves of a concatenation are written in place), and the result is converted back once.
   Same operators in the same order as unet_trunk (pytorch/ocnn/unet.py:61-92 with one
   convolution per stage); channel counts of the concatenated features must be multiples of 16."""
   if data is None:
     data = F.octree_property(octree, "feature", depth).bfloat16()
+    if nempty:
+      data = F.octree_depad(data, octree, depth)
   info = F.octree_info(octree)
   x, cin = F.to_rows(data), data.size(1)
   feats, joined = {}, {}
+
+  def conv(x, cin, w, b, d, cout, out=None, **kw):
+    return F.octree_conv_rows(x, cin, w, octree, d, cout, bias=b, relu=True, out=out, nempty=nempty, **kw)
 
   def encoder_conv(x, cin, d, skip):
     w, b = params[("conv", d)]
     c_skip = w.shape[0]
     if not skip:
-      return F.octree_conv_rows(x, cin, w, octree, d, c_skip, bias=b, relu=True), c_skip
+      return conv(x, cin, w, b, d, c_skip), c_skip
     c_up = params[("up", d - 1)][0].shape[1] // 8
     if c_skip % 16 or c_up % 16:
       raise ValueError("concatenated features need channel counts that are multiples of 16")
-    joined[d] = torch.empty(info.nnum(d) + 1, c_skip + c_up, dtype=x.dtype, device=x.device)
-    return F.octree_conv_rows(x, cin, w, octree, d, c_skip, bias=b, relu=True, out=joined[d][:, :c_skip]), c_skip
+    rows = info.nnum_nempty(d) if nempty else info.nnum(d)
+    joined[d] = torch.empty(rows + 1, c_skip + c_up, dtype=x.dtype, device=x.device)
+    return conv(x, cin, w, b, d, c_skip, out=joined[d][:, :c_skip]), c_skip
 
   feats[depth] = encoder_conv(x, cin, depth, stages > 0)
   d = depth
   for i in range(stages):
     w, b = params[("down", d)]
     x, cin = feats[d]
-    x = F.octree_conv_rows(x, cin, w, octree, d, w.shape[0], bias=b, relu=True, kernel_size=(2, 2, 2), stride=2)
+    x = conv(x, cin, w, b, d, w.shape[0], kernel_size=(2, 2, 2), stride=2)
     d -= 1
     feats[d] = encoder_conv(x, w.shape[0], d, i + 1 < stages)
   x, cin = feats[d]
@@ -145,11 +151,10 @@ def unet_trunk_rows(octree, depth, params, data=None, stages=3):
     w, b = params[("up", d)]
     cout = w.shape[1] // 8
     c_skip = feats[d + 1][1]
-    F.octree_conv_rows(x, cin, w, octree, d, cout, bias=b, relu=True, deconv=True, kernel_size=(2, 2, 2), stride=2,
-                       out=joined[d + 1][:, c_skip:])
+    conv(x, cin, w, b, d, cout, out=joined[d + 1][:, c_skip:], deconv=True, kernel_size=(2, 2, 2), stride=2)
     d += 1
     w, b = params[("dec", d)]
-    x, cin = F.octree_conv_rows(joined[d], c_skip + cout, w, octree, d, w.shape[0], bias=b, relu=True), w.shape[0]
+    x, cin = conv(joined[d], c_skip + cout, w, b, d, w.shape[0]), w.shape[0]
   return F.from_rows(x, cin)
 
 

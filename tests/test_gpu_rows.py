@@ -206,3 +206,55 @@ def test_rows_operators_full_size(oc, synthetic):
                                        kernel_size=(2, 2, 2), stride=2))
   up_ref = S.conv_bn_relu(dn_ref, wu, b32, octree, 8, 32, (2, 2, 2), 2, deconv=True)
   close(F.from_rows(up, 32).float().cpu().numpy().reshape(32, -1), up_ref.float().cpu().numpy().reshape(32, -1), 2e-2, "up")
+
+
+@pytest.mark.parametrize("cin,cout", [(3, 32), (64, 64), (24, 40), (48, 128), (128, 256)])
+def test_nonempty_rows_equal_channel_major(oc, octree, cin, cout):
+  """over the non-empty nodes the row-major operators run the kernel of the channel-major entry
+  points on the same operands in the same order: equal bits, for 3x3x3 stride 1 and for 2x2x2
+  stride 2, convolution and deconvolution"""
+  F = oc.nn
+  info = F.octree_info(octree)
+  g = torch.Generator().manual_seed(cin * 31 + cout)
+  bias = torch.randn(cout, generator=g).cuda()
+  for depth in (6, 5):
+    Hne = info.nnum_nempty(depth)
+    x = torch.randn(1, cin, Hne, 1, generator=g).bfloat16().cuda()
+    xr = F.to_rows(x)
+    for ks, stride, deconv in (([3, 3, 3], 1, False), ([3, 3, 3], 1, True), ([2, 2, 2], 2, False), ([2, 2, 2], 2, True)):
+      if deconv and stride == 2 and depth == 6:
+        continue   # no level below the finest one
+      K = ks[0] * ks[1] * ks[2]
+      shape = (cin, cout * K) if deconv else (cout, cin * K)
+      w = (torch.randn(*shape, generator=g) * 0.05).bfloat16().cuda()
+      for b, relu in ((None, False), (bias, True)):
+        exp = F.octree_conv_fused(x, w, b, relu, octree, depth, cout, ks, stride, True, deconv=deconv)
+        rows = F.octree_conv_rows(xr, cin, w, octree, depth, cout, bias=b, relu=relu, deconv=deconv,
+                                  kernel_size=tuple(ks), stride=stride, nempty=True)
+        assert rows.shape == (exp.size(2) + 1, F.rows_pitch(cout))
+        assert not rows[-1].any() and not rows[:, cout:].any()
+        assert torch.equal(F.from_rows(rows, cout), exp), (depth, ks, stride, deconv, relu)
+
+
+def test_unet_trunk_rows_nonempty(oc, small):
+  host, dev, b = small
+  rng = np.random.default_rng(5)
+  ch = {6: 16, 5: 32, 4: 64}
+  params = {}
+
+  def mk(key, shape, fan):
+    w = (rng.standard_normal(shape) / np.sqrt(fan)).astype(np.float32)
+    bias = (rng.standard_normal(shape[0] if key[0] != "up" else shape[1] // 8) * 0.1).astype(np.float32)
+    params[key] = (T(w).cuda().bfloat16(), T(bias).cuda())
+
+  mk(("conv", 6), (ch[6], 3 * 27), 81)
+  for d in (6, 5):
+    mk(("down", d), (ch[d - 1], ch[d] * 8), ch[d] * 8)
+    mk(("conv", d - 1), (ch[d - 1], ch[d - 1] * 27), ch[d - 1] * 27)
+  for d in (4, 5):
+    mk(("up", d), (ch[d], ch[d + 1] * 8), ch[d])
+    mk(("dec", d + 1), (ch[d + 1], 2 * ch[d + 1] * 27), 2 * ch[d + 1] * 27)
+  data = oc.nn.octree_depad(oc.nn.octree_property(dev, "feature", 6).bfloat16(), dev, 6)
+  exp = oc.stacks.unet_trunk(dev, 6, params, data=data, stages=2, nempty=True)
+  got = oc.stacks.unet_trunk_rows(dev, 6, params, data=data, stages=2, nempty=True)
+  assert torch.equal(got, exp)   # every member is bit-identical to its channel-major counterpart
