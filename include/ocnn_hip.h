@@ -216,6 +216,23 @@ int ocnn_octree_conv_rows(void* top_rows, int top_pitch, const void* btm_rows, i
     int btm_h, const void* weights, const float* bias, int relu, int is_deconv, const void* octree_dev,
     const void* info, int depth, int num_output, const int* kernel_size, int stride, int nempty, int dtype,
     void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream);
+/* The same operator for weights that do not change from call to call (inference): pack them once
+ * (ocnn_conv_rows_packed_bytes bytes, 16-byte aligned; the order depends on the channel counts, the
+ * kernel, the stride, nempty and is_deconv only) and pass the packed form; `ichild_dev`: the
+ * inverted child links from ocnn_make_ichild for the operators that use them -- every nempty
+ * operator (links of `depth`; of depth+1 for the stride-2 deconvolution) and the all-nodes stride-2
+ * deconvolution (links of `depth`) -- or NULL, then the call computes them into the workspace
+ * (ocnn_conv_rows_shape bytes are enough).  With both, no workspace is needed and the call launches
+ * the convolution kernel alone. */
+int ocnn_conv_rows_packed_bytes(const void* info, int depth, int channel_in, int num_output, const int* kernel_size,
+    int stride, int nempty, int is_deconv, int dtype, size_t* packed_bytes);
+int ocnn_conv_rows_pack(void* packed_dev, size_t packed_bytes, const void* weights, const void* octree_dev,
+    const void* info, int depth, int channel_in, int num_output, const int* kernel_size, int stride, int nempty,
+    int is_deconv, int dtype, ocnn_stream_t stream);
+int ocnn_octree_conv_rows_packed(void* top_rows, int top_pitch, const void* btm_rows, int btm_pitch, int channel_in,
+    int btm_h, const void* packed_weights, const int* ichild_dev, const float* bias, int relu, int is_deconv,
+    const void* octree_dev, const void* info, int depth, int num_output, const int* kernel_size, int stride, int nempty,
+    int dtype, void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream);
 int ocnn_rows_from_channels(void* rows, int pitch, const void* data, int channel, int height, int dtype,
     ocnn_stream_t stream);
 int ocnn_channels_from_rows(void* data, const void* rows, int pitch, int channel, int height, int dtype,

@@ -3003,7 +3003,11 @@ int make_rows_plan(const Info* o, int depth, int channel_in, int num_output, con
     const bool wide = mtiles % 4 == 0;
     r->MT = mtiles == 1 ? 1 : (wide ? 4 : 2);
     r->npass = (mtiles + r->MT - 1) / r->MT;
-    r->wt_bytes = p.wt_bytes;
+    {
+      const int slab_ch = r->MT == 4 ? 32 : kRowSlab;
+      const int nslab = (r->cpad + slab_ch - 1) / slab_ch;
+      r->wt_bytes = align256((size_t)r->npass * p.taps.count * nslab * (slab_ch / 16) * r->MT * 64 * 16);
+    }
     r->ichild_bytes = p.ichild_bytes;
   } else if (stride == 1 && k333) {
     r->kind = 0;
@@ -3037,15 +3041,56 @@ int make_rows_plan(const Info* o, int depth, int channel_in, int num_output, con
   return OCNN_OK;
 }
 
+// `packed` (optional): the weights as ocnn_conv_rows_pack left them -- then `weights` is not read and no
+// packing kernel runs; `ichild_in` (optional): the inverted child links the operator needs -- then
+// none are computed.  With both (or with `packed` for an operator that needs no links) the call needs
+// no workspace.  `only_pack`: pack `weights` into `ws` and return.
 int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_rows, int btm_pitch, int channel_in,
     int btm_h, const void* weights, const float* bias, int relu, const void* octree_dev, const void* info,
     int depth, int num_output, const int* ks, int stride, int nempty, int dtype, void* ws, size_t ws_bytes,
-    hipStream_t s) {
-  OCNN_REQUIRE(top_rows && btm_rows && weights && octree_dev && info && ks, OCNN_E_BADARG, "null pointer");
+    hipStream_t s, const void* packed = nullptr, const int* ichild_in = nullptr, bool only_pack = false) {
+  OCNN_REQUIRE((only_pack || (top_rows && btm_rows)) && (weights || packed) && octree_dev && info && ks,
+      OCNN_E_BADARG, "null pointer");
   const Info* o = as_info(info);
   RowsPlan r;
   int e = make_rows_plan(o, depth, channel_in, num_output, ks, stride, nempty, deconv, dtype, &r);
   if (e) return e;
+  const bool need_links = r.ichild_bytes > 0 && !ichild_in && !only_pack;
+  const size_t ws_need = (packed ? 0 : r.wt_bytes) + (need_links ? r.ichild_bytes : 0);
+  OCNN_REQUIRE(ws_need == 0 || (ws && ws_bytes >= ws_need), OCNN_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes, ws_need);
+  OCNN_REQUIRE(ws_need == 0 || (reinterpret_cast<uintptr_t>(ws) & 15) == 0, OCNN_E_WORKSPACE, "workspace not 16-byte aligned");
+  OCNN_REQUIRE(!packed || (reinterpret_cast<uintptr_t>(packed) & 15) == 0, OCNN_E_BADARG, "packed weights not 16-byte aligned");
+  char* wsb = static_cast<char*>(ws);
+  if (!packed) {   // the weights in the order the kernel of this operator reads them
+    const int mtiles_w = (num_output + 31) / 32;
+    if (r.kind == 0) {
+      const int64_t sm = deconv ? 27 : (int64_t)channel_in * 27, sc = deconv ? (int64_t)num_output * 27 : 27;
+      const int64_t total = (int64_t)r.npass * r.ksteps * 27 * r.MT * 64 * 8;
+      pack_weights_lds_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)ws, (const uint16_t*)weights, num_output,
+          channel_in, r.MT, r.npass, r.ksteps, sm, sc, deconv);
+    } else if (r.kind == 1) {
+      const int64_t total = (int64_t)r.npass * 8 * r.ksteps * r.MT * 64 * 8;
+      pack_weights_s2_rows_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)ws, (const uint16_t*)weights, num_output,
+          channel_in, r.MT, r.npass, r.ksteps);
+    } else if (r.kind == 2) {
+      const int64_t total = (int64_t)r.npass * r.ksteps * r.MT * 64 * 8;
+      pack_weights_d2_rows_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)ws, (const uint16_t*)weights, num_output,
+          channel_in, r.MT, r.npass, r.ksteps);
+    } else {
+      const int K = stride == 1 ? 27 : 8;
+      const int64_t sm = deconv ? K : (int64_t)channel_in * K, sc = deconv ? (int64_t)num_output * K : K;
+      const int slab_ch = r.MT == 4 ? 32 : kRowSlab;
+      const int nslab = (r.cpad + slab_ch - 1) / slab_ch;
+      const int64_t total = (int64_t)r.npass * K * nslab * (slab_ch / 16) * r.MT * 64 * 8;
+      pack_weights_rows_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)ws, (const uint16_t*)weights, num_output,
+          channel_in, K, r.MT, r.npass, nslab, sm, sc, slab_ch);
+    }
+    (void)mtiles_w;
+    OCNN_LAUNCH_OK("pack_weights");
+    if (only_pack) return OCNN_OK;
+  }
+  const void* wpk = packed ? packed : ws;
+  int* links_ws = reinterpret_cast<int*>(wsb + (packed ? 0 : r.wt_bytes));
   OCNN_REQUIRE(btm_h == r.btm_h, OCNN_E_SHAPE, "input height %d, the octree has %d rows at depth %d", btm_h,
       r.btm_h, depth);
   // the stride-2 convolution also reads a channel slice of a wider tensor (an encoder feature that
@@ -3059,10 +3104,7 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
   OCNN_REQUIRE(((int64_t)btm_h + 1) * btm_pitch * 2 < ((int64_t)1 << 31) - (1 << 20) &&
       ((int64_t)r.top_h + 1) * top_pitch * 2 < ((int64_t)1 << 31) - (1 << 20), OCNN_E_UNSUPPORTED,
       "level too large for 32-bit row offsets");
-  OCNN_REQUIRE(ws && ws_bytes >= r.total_bytes, OCNN_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes, r.total_bytes);
-  OCNN_REQUIRE((reinterpret_cast<uintptr_t>(ws) & 15) == 0, OCNN_E_WORKSPACE, "workspace not 16-byte aligned");
   const char* blob = static_cast<const char*>(octree_dev);
-  char* wsb = static_cast<char*>(ws);
   ConvArgs a;
   a.M = num_output;
   a.Cin = channel_in;
@@ -3097,26 +3139,23 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
     }
     a.neigh = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_NEIGH, p.workspace_depth));
     a.child = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_CHILD, p.workspace_depth));
-    int* ichild = reinterpret_cast<int*>(wsb + p.wt_bytes);
-    ichild_kernel<<<blocks_for(p.child_h), kBlock, 0, s>>>(ichild, p.ichild_h, a.child, p.child_h);
-    a.ichild = ichild;
-    const int64_t sm = deconv ? a.K : (int64_t)channel_in * a.K, sc = deconv ? (int64_t)num_output * a.K : a.K;
-    const int slab_ch = r.MT == 4 ? 32 : kRowSlab;
-    const int nslab = (r.cpad + slab_ch - 1) / slab_ch;
-    const int64_t total = (int64_t)r.npass * a.K * nslab * (slab_ch / 16) * r.MT * 64 * 8;
-    pack_weights_rows_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)ws, (const uint16_t*)weights, a.M, a.Cin,
-        a.K, r.MT, r.npass, nslab, sm, sc, slab_ch);
+    if (ichild_in) {
+      a.ichild = ichild_in;
+    } else {
+      ichild_kernel<<<blocks_for(p.child_h), kBlock, 0, s>>>(links_ws, p.ichild_h, a.child, p.child_h);
+      a.ichild = links_ws;
+    }
     const int n_tiles = (a.N + kTileCols - 1) / kTileCols;
     const dim3 grid(((n_tiles + 7) / 8) * 8, pass_split(n_tiles, r.npass));
     if (r.MT == 4)
       conv_rows_bf16_deep_kernel<4, 32, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
-          (const u32x4*)ws, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
+          (const u32x4*)wpk, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
     else if (r.MT == 2)
       conv_rows_bf16_deep_kernel<2, kRowSlab, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
-          (const u32x4*)ws, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
+          (const u32x4*)wpk, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
     else
       conv_rows_bf16_deep_kernel<1, kRowSlab, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
-          (const u32x4*)ws, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
+          (const u32x4*)wpk, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
     OCNN_LAUNCH_OK("octree_conv_rows");
     return OCNN_OK;
   }
@@ -3135,50 +3174,43 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
     for (int k = 0; k < 27; ++k) a.slot[k] = tap_slot(deconv ? 26 - taps.tap[k] : taps.tap[k]);
     a.neigh = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_NEIGH, depth));
     a.child = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_CHILD, depth));
-    const int64_t sm = deconv ? 27 : (int64_t)channel_in * 27, sc = deconv ? (int64_t)num_output * 27 : 27;
-    const int64_t total = (int64_t)r.npass * r.ksteps * 27 * r.MT * 64 * 8;
-    pack_weights_lds_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)ws, (const uint16_t*)weights, a.M, a.Cin,
-        r.MT, r.npass, r.ksteps, sm, sc, deconv);
     const int r_tiles = ((a.N >> 3) + kRegTileGroups - 1) / kRegTileGroups;
     const dim3 grid(((r_tiles + 7) / 8) * 8, pass_split(r_tiles, r.npass));
     if (r.MT == 1)
       conv_s1_bf16_reg_kernel<1, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
-          (const u32x4*)ws, r_tiles, r.cpad / 8, top_pitch, r.out_cpad);
+          (const u32x4*)wpk, r_tiles, r.cpad / 8, top_pitch, r.out_cpad);
     else
       conv_s1_bf16_reg_kernel<2, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
-          (const u32x4*)ws, r_tiles, r.cpad / 8, top_pitch, r.out_cpad);
+          (const u32x4*)wpk, r_tiles, r.cpad / 8, top_pitch, r.out_cpad);
   } else if (r.kind == 1) {
     a.K = 8;
     a.mode = kModeS2Conv;
     a.neigh = nullptr;
     a.child = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_CHILD, depth - 1));
-    const int64_t total = (int64_t)r.npass * 8 * r.ksteps * r.MT * 64 * 8;
-    pack_weights_s2_rows_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)ws, (const uint16_t*)weights, a.M,
-        a.Cin, r.MT, r.npass, r.ksteps);
     const int n_tiles = (a.N + kTileCols - 1) / kTileCols;
     const dim3 grid(((n_tiles + 7) / 8) * 8, pass_split(n_tiles, r.npass));
     if (r.MT == 1)
       conv_s2_rows_bf16_kernel<1><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, top_pitch, r.out_cpad,
-          (const u32x4*)btm_rows, btm_pitch, r.cpad, (const u32x4*)ws, n_tiles);
+          (const u32x4*)btm_rows, btm_pitch, r.cpad, (const u32x4*)wpk, n_tiles);
     else
       conv_s2_rows_bf16_kernel<2><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, top_pitch, r.out_cpad,
-          (const u32x4*)btm_rows, btm_pitch, r.cpad, (const u32x4*)ws, n_tiles);
+          (const u32x4*)btm_rows, btm_pitch, r.cpad, (const u32x4*)wpk, n_tiles);
   } else {
     a.K = 8;
     a.mode = kModeS2Deconv;
     a.neigh = nullptr;
     a.child = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_CHILD, depth));
-    int* ichild = reinterpret_cast<int*>(wsb + r.wt_bytes);
-    ichild_kernel<<<blocks_for(btm_h), kBlock, 0, s>>>(ichild, r.cols, a.child, btm_h);
-    a.ichild = ichild;
-    const int64_t total = (int64_t)r.npass * r.ksteps * r.MT * 64 * 8;
-    pack_weights_d2_rows_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)ws, (const uint16_t*)weights, a.M,
-        a.Cin, r.MT, r.npass, r.ksteps);
+    if (ichild_in) {
+      a.ichild = ichild_in;
+    } else {
+      ichild_kernel<<<blocks_for(btm_h), kBlock, 0, s>>>(links_ws, r.cols, a.child, btm_h);
+      a.ichild = links_ws;
+    }
     const int n_tiles = (a.N + kTileCols - 1) / kTileCols;
     const int grid = ((n_tiles + 7) / 8) * 8;
 #define OCNN_D2_ROWS(KS, MT2)                                                                         \
     deconv_s2_rows_bf16_kernel<KS, MT2><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, top_pitch, r.out_cpad, \
-        (const u32x4*)btm_rows, (const u32x4*)ws, n_tiles)
+        (const u32x4*)btm_rows, (const u32x4*)wpk, n_tiles)
     switch (r.ksteps) {
       case 1: OCNN_D2_ROWS(1, 4); break;
       case 2: OCNN_D2_ROWS(2, 4); break;
@@ -3272,6 +3304,34 @@ int ocnn_conv_rows_shape(const void* info, int depth, int channel_in, int num_ou
   if (btm_h) *btm_h = r.btm_h;
   if (workspace_bytes) *workspace_bytes = r.total_bytes;
   return OCNN_OK;
+}
+
+int ocnn_conv_rows_packed_bytes(const void* info, int depth, int channel_in, int num_output, const int* kernel_size,
+    int stride, int nempty, int is_deconv, int dtype, size_t* packed_bytes) {
+  RowsPlan r;
+  int e = make_rows_plan(as_info(info), depth, channel_in, num_output, kernel_size, stride, nempty, is_deconv, dtype, &r);
+  if (e) return e;
+  if (packed_bytes) *packed_bytes = r.wt_bytes;
+  return OCNN_OK;
+}
+
+int ocnn_conv_rows_pack(void* packed_dev, size_t packed_bytes, const void* weights, const void* octree_dev,
+    const void* info, int depth, int channel_in, int num_output, const int* kernel_size, int stride, int nempty,
+    int is_deconv, int dtype, ocnn_stream_t stream) {
+  OCNN_REQUIRE(packed_dev && weights, OCNN_E_BADARG, "null pointer");
+  return run_conv_rows(is_deconv ? 1 : 0, nullptr, 0, nullptr, 0, channel_in, 0, weights, nullptr, 0, octree_dev, info,
+      depth, num_output, kernel_size, stride, nempty, dtype, packed_dev, packed_bytes, as_stream(stream), nullptr, nullptr,
+      true);
+}
+
+int ocnn_octree_conv_rows_packed(void* top_rows, int top_pitch, const void* btm_rows, int btm_pitch, int channel_in,
+    int btm_h, const void* packed_weights, const int* ichild_dev, const float* bias, int relu, int is_deconv,
+    const void* octree_dev, const void* info, int depth, int num_output, const int* kernel_size, int stride, int nempty,
+    int dtype, void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream) {
+  OCNN_REQUIRE(packed_weights, OCNN_E_BADARG, "null pointer");
+  return run_conv_rows(is_deconv ? 1 : 0, top_rows, top_pitch, btm_rows, btm_pitch, channel_in, btm_h, nullptr, bias,
+      relu, octree_dev, info, depth, num_output, kernel_size, stride, nempty, dtype, workspace_dev, workspace_bytes,
+      as_stream(stream), packed_weights, ichild_dev);
 }
 
 int ocnn_rows_from_channels(void* rows, int pitch, const void* data, int channel, int height, int dtype,

@@ -766,7 +766,7 @@ def from_rows(rows, channels):
 
 
 def octree_conv_rows(rows_in, channel_in, weights, octree, depth, num_output, bias=None, relu=False,
-                     deconv=False, out=None, kernel_size=(3, 3, 3), stride=1, nempty=False):
+                     deconv=False, out=None, kernel_size=(3, 3, 3), stride=1, nempty=False, constant_weights=False):
   """Convolutions over all nodes in bf16, row-major on both sides: the arithmetic of octree_conv /
   octree_conv_fused (pytorch/cpp/octree_conv.cpp:131-216) on tensors that a chain of convolutions
   keeps in the layout the kernels gather from, so that no member of the chain copies its input.
@@ -778,6 +778,9 @@ def octree_conv_rows(rows_in, channel_in, weights, octree, depth, num_output, bi
       folded in), rows of depth+1 out.
   With nempty=True the rows on both sides are the ranks of the non-empty nodes, as in the
   channel-major operators (3x3x3 stride 1 and 2x2x2 stride 2, conv and deconv).
+  constant_weights=True (inference): the packed form of `weights` is kept with the tensor (and
+  packed again when the tensor is written to), the inverted child links with the octree, so that a
+  call launches the convolution kernel alone.
   rows_in: [H + 1, rows_pitch(channel_in)] as to_rows makes it.  `out`: [top_h + 1, P] with
   P >= rows_pitch(num_output), or columns c0 .. c0 + rows_pitch(num_output) of such a tensor (a
   slice of what a later layer reads as a concatenation); returns `out`."""
@@ -806,6 +809,32 @@ def octree_conv_rows(rows_in, channel_in, weights, octree, depth, num_output, bi
     bias = bias.to(torch.float32).contiguous()
     if bias.numel() != num_output:
       raise OcnnError(-3, "bias needs num_output entries")
+  if constant_weights:
+    key = (channel_in, num_output, tuple(kernel_size), stride, bool(nempty), bool(deconv))
+    cache = weights.__dict__.setdefault("_ocnn_rows_packed", {})
+    ent = cache.get(key)
+    if ent is None or ent[0] != weights._version:
+      nbytes = C.c_size_t()
+      _lib.call("ocnn_conv_rows_packed_bytes", info.p, depth, channel_in, num_output, ksc, stride, int(nempty),
+                int(deconv), dt, C.byref(nbytes))
+      packed = torch.empty(nbytes.value, dtype=torch.uint8, device=weights.device)
+      _lib.call("ocnn_conv_rows_pack", _ptr(packed), C.c_size_t(nbytes.value), _ptr(weights), _ptr(octree), info.p, depth,
+                channel_in, num_output, ksc, stride, int(nempty), int(deconv), dt, _stream())
+      ent = cache[key] = (weights._version, packed)
+    links = None
+    link_depth = depth + 1 if (deconv and stride == 2 and nempty) else depth
+    if nempty or (deconv and stride == 2):
+      links_of = octree.__dict__.setdefault("_ocnn_ichild", {})
+      links = links_of.get(link_depth)
+      if links is None:
+        child = octree_property(octree, "child", link_depth).view(-1)
+        links = torch.empty(info.nnum_nempty(link_depth) + 1, dtype=torch.int32, device=octree.device)
+        _lib.call("ocnn_make_ichild", _ptr(links), info.nnum_nempty(link_depth), _ptr(child), child.numel(), _stream())
+        links_of[link_depth] = links
+    _lib.call("ocnn_octree_conv_rows_packed", _ptr(out), out.stride(0), _ptr(rows_in), rows_in.stride(0), channel_in,
+              btm_h, _ptr(ent[1]), _ptr(links), _ptr(bias), int(relu), int(deconv), _ptr(octree), info.p, depth,
+              num_output, ksc, stride, int(nempty), dt, C.c_void_p(base), C.c_size_t(ws_bytes.value), _stream())
+    return out
   _lib.call("ocnn_octree_conv_rows", _ptr(out), out.stride(0), _ptr(rows_in), rows_in.stride(0), channel_in, btm_h,
             _ptr(weights), _ptr(bias), int(relu), int(deconv), _ptr(octree), info.p, depth, num_output, ksc, stride,
             int(nempty), dt, C.c_void_p(base), C.c_size_t(ws_bytes.value), _stream())

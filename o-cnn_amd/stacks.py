@@ -108,13 +108,15 @@ def unet_trunk(octree, depth, params, data=None, stages=3, nempty=False):
   return x
 
 
-def unet_trunk_rows(octree, depth, params, data=None, stages=3, nempty=False):
+def unet_trunk_rows(octree, depth, params, data=None, stages=3, nempty=False, constant_weights=True):
   """unet_trunk in bf16 with row-major activations between the operators: the input is converted
   once, every convolution reads the layout its kernel gathers from and writes it for the next one
   (over all nodes the pad and depad around the stride-2 layers are part of those operators; both
   halves of a concatenation are written in place), and the result is converted back once.
   Same operators in the same order as unet_trunk (pytorch/ocnn/unet.py:61-92 with one
-  convolution per stage); channel counts of the concatenated features must be multiples of 16."""
+  convolution per stage); channel counts of the concatenated features must be multiples of 16.
+  constant_weights (the inference case): packed weights and inverted child links are kept between
+  calls, see octree_conv_rows."""
   if data is None:
     data = F.octree_property(octree, "feature", depth).bfloat16()
     if nempty:
@@ -124,7 +126,8 @@ def unet_trunk_rows(octree, depth, params, data=None, stages=3, nempty=False):
   feats, joined = {}, {}
 
   def conv(x, cin, w, b, d, cout, out=None, **kw):
-    return F.octree_conv_rows(x, cin, w, octree, d, cout, bias=b, relu=True, out=out, nempty=nempty, **kw)
+    return F.octree_conv_rows(x, cin, w, octree, d, cout, bias=b, relu=True, out=out, nempty=nempty,
+                              constant_weights=constant_weights, **kw)
 
   def encoder_conv(x, cin, d, skip):
     w, b = params[("conv", d)]

@@ -258,3 +258,26 @@ def test_unet_trunk_rows_nonempty(oc, small):
   exp = oc.stacks.unet_trunk(dev, 6, params, data=data, stages=2, nempty=True)
   got = oc.stacks.unet_trunk_rows(dev, 6, params, data=data, stages=2, nempty=True)
   assert torch.equal(got, exp)   # every member is bit-identical to its channel-major counterpart
+
+
+def test_packed_weights_and_cached_links(oc, octree):
+  """constant_weights=True keeps the packed weights with the weight tensor and the inverted child
+  links with the octree: the same bits as the plain call, also after the weights were written to"""
+  F = oc.nn
+  info = F.octree_info(octree)
+  g = torch.Generator().manual_seed(77)
+  bias = torch.randn(48, generator=g).cuda()
+  for nempty in (False, True):
+    for ks, stride, deconv, depth in (((3, 3, 3), 1, False, 6), ((2, 2, 2), 2, False, 6), ((2, 2, 2), 2, True, 5)):
+      K = ks[0] * ks[1] * ks[2]
+      H = info.nnum_nempty(depth) if nempty else info.nnum(depth)
+      x = F.to_rows(torch.randn(1, 32, H, 1, generator=g).bfloat16().cuda())
+      shape = (32, 48 * K) if deconv else (48, 32 * K)
+      w = (torch.randn(*shape, generator=g) * 0.05).bfloat16().cuda()
+      kw = dict(bias=bias, relu=True, deconv=deconv, kernel_size=ks, stride=stride, nempty=nempty)
+      for _ in range(2):
+        exp = F.octree_conv_rows(x, 32, w, octree, depth, 48, **kw)
+        for _ in range(2):   # the second call finds everything in place
+          got = F.octree_conv_rows(x, 32, w, octree, depth, 48, constant_weights=True, **kw)
+          assert torch.equal(got, exp), (nempty, ks, stride, deconv)
+        w.mul_(1.5)        # a write to the tensor: the next call packs again
