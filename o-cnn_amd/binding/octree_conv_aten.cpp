@@ -126,10 +126,58 @@ Tensor octree_conv_bn_relu(Tensor data_in, Tensor weights, Tensor bias, Tensor o
   return conv_forward(data_in, weights, octree, depth, num_output, kernel_size, stride, nempty, deconv, &bias, relu);
 }
 
+// ---- row-major bf16 activations (no counterpart in the reference): rows [H + 1, pitch] ----------------
+Tensor rows_from_channels(Tensor data) {
+  data = data.contiguous();
+  const int c = (int)data.size(1), h = (int)data.size(2), pitch = (c + 15) / 16 * 16;
+  Tensor rows = torch::empty({h + 1, pitch}, data.options());
+  int rc = ocnn_rows_from_channels(rows.data_ptr(), pitch, data.data_ptr(), c, h, dtype_of(data), current_stream());
+  TORCH_CHECK(rc == OCNN_OK, ocnn_last_error());
+  return rows;
+}
+
+Tensor channels_from_rows(Tensor rows, int channels) {
+  rows = rows.contiguous();
+  const int h = (int)rows.size(0) - 1;
+  Tensor data = torch::empty({1, channels, h, 1}, rows.options());
+  int rc = ocnn_channels_from_rows(data.data_ptr(), rows.data_ptr(), (int)rows.size(1), channels, h, dtype_of(rows),
+      current_stream());
+  TORCH_CHECK(rc == OCNN_OK, ocnn_last_error());
+  return data;
+}
+
+// conv / deconv + bias + ReLU on row-major tensors; rows_in [H + 1, pitch(channel_in)] -> [top_h + 1, pitch(num_output)]
+Tensor octree_conv_rows(Tensor rows_in, int channel_in, Tensor weights, Tensor bias, bool relu, Tensor octree,
+    int depth, int num_output, vector<int> kernel_size, int stride, bool nempty, bool deconv) {
+  TORCH_CHECK(kernel_size.size() == 3, "kernel_size holds three numbers");
+  TORCH_CHECK(rows_in.dim() == 2 && rows_in.stride(1) == 1, "rows_in is [H + 1, pitch] with unit channel stride");
+  weights = weights.contiguous();
+  const void* info = host_info(octree);
+  const int dt = dtype_of(rows_in);
+  int top_h = 0, btm_h = 0;
+  size_t ws_bytes = 0;
+  int rc = ocnn_conv_rows_shape(info, depth, channel_in, num_output, kernel_size.data(), stride, nempty ? 1 : 0,
+      deconv ? 1 : 0, dt, &top_h, &btm_h, &ws_bytes);
+  TORCH_CHECK(rc == OCNN_OK, ocnn_last_error());
+  Tensor ws = torch::empty({(int64_t)ws_bytes + 16}, octree.options().dtype(torch::kUInt8));
+  Tensor out = torch::empty({top_h + 1, (num_output + 15) / 16 * 16}, rows_in.options());
+  Tensor b;
+  if (bias.defined() && bias.numel() > 0) b = bias.to(torch::kFloat32).contiguous();
+  rc = ocnn_octree_conv_rows(out.data_ptr(), (int)out.stride(0), rows_in.data_ptr(), (int)rows_in.stride(0), channel_in,
+      (int)rows_in.size(0) - 1, weights.data_ptr(), b.defined() ? b.data_ptr<float>() : nullptr, relu ? 1 : 0,
+      deconv ? 1 : 0, octree.data_ptr(), info, depth, num_output, kernel_size.data(), stride, nempty ? 1 : 0, dt,
+      ws.data_ptr(), ws_bytes, current_stream());
+  TORCH_CHECK(rc == OCNN_OK, ocnn_last_error());
+  return out;
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("octree_conv", &octree_conv, "octree based convolution");
   m.def("octree_deconv", &octree_deconv, "octree based deconvolution");
   m.def("octree_conv_grad", &octree_conv_grad, "octree based convolution, gradients");
   m.def("octree_deconv_grad", &octree_deconv_grad, "octree based deconvolution, gradients");
   m.def("octree_conv_bn_relu", &octree_conv_bn_relu, "convolution with folded BatchNorm and ReLU");
+  m.def("rows_from_channels", &rows_from_channels, "[1, C, H, 1] bf16 -> rows [H + 1, pitch]");
+  m.def("channels_from_rows", &channels_from_rows, "rows [H + 1, pitch] -> [1, C, H, 1]");
+  m.def("octree_conv_rows", &octree_conv_rows, "convolution on row-major bf16 activations");
 }
