@@ -15,6 +15,7 @@ namespace ocnn {
 namespace {
 
 constexpr int kChanChunk = 8;  // channels handled per thread in the gather ops
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));  // one 16-byte LDS / global unit
 
 template <typename T> __device__ inline T zero_of();
 template <> __device__ inline float zero_of<float>() { return 0.0f; }
@@ -439,6 +440,132 @@ __global__ void col2octree_kernel(const float* __restrict__ col, float* __restri
     }
 }
 
+// Gather form for the 27 taps at stride 1 over all nodes, where columns and rows are the same
+// nodes: a workgroup owns kGatherTile consecutive rows and streams the same range of the 27
+// col rows of a channel through LDS with coalesced 16-byte loads, the next channel flying
+// while this one is summed.  A row finds the column of a tap in LDS when that column lies
+// inside the tile (19 of 20 do in a depth-9 scene, neighbours being close in z-order); for the
+// others the thread asks global memory, in a wavefront that has such a tap at all, before the
+// tile is written to LDS.  Taps are summed in ascending order as above.
+constexpr int kGatherTile = 1024, kGatherUnits = kGatherTile / 4;  // rows of a tile, 16-byte units of a staged row
+constexpr int kGatherLoads = (27 * kGatherUnits + kGatherTile - 1) / kGatherTile;  // 16-byte loads a thread and channel
+
+__global__ void __launch_bounds__(kGatherTile, 4) col2octree_tile_kernel(const float* __restrict__ col,
+    float* __restrict__ data, ColArgs a, const int* __restrict__ neigh,
+    const unsigned long long* __restrict__ mark, unsigned long long id) {
+  extern __shared__ __attribute__((aligned(16))) float s_col[];  // [27][kGatherTile] and one word that stays zero
+  const int tid = threadIdx.x;
+  const int r0 = blockIdx.x * kGatherTile, p = r0 + tid;
+  const int c0 = blockIdx.y * kChanChunk, c1 = min(a.channel, c0 + kChanChunk);
+  const int lo = a.n * a.height_col, hi = min(a.height, lo + a.height_col);  // lo is a multiple of 4 (host)
+  // The col rows of a channel are one buffer (the host checks that they fit 2 GiB), a tap is a
+  // scalar offset into it, and a column is a 32-bit offset; an offset past any buffer reads as
+  // zero, and so does each word of a 16-byte load that lies past the end.
+  constexpr int kNoColumn = (int)0x80000000u;
+  const int row_bytes = a.height_col * 4;
+  auto rows_of = [&](int c) {
+    return __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(col) + (int64_t)c * 27 * a.height_col, 0, 27 * row_bytes, 0x00020000);
+  };
+  // staging: load j of the thread is tap tid / kGatherUnits + 4 j, columns 4 (tid % kGatherUnits) .. + 3 of the tile
+  const int tap0 = __builtin_amdgcn_readfirstlane(tid / kGatherUnits);
+  const int group = (tid % kGatherUnits) * 4;
+  const int mine = (r0 + group >= lo && r0 + group < hi) ? (r0 + group - lo) * 4 : kNoColumn;
+  u32x4 next[kGatherLoads];
+  auto fetch = [&](int c) {
+    if (c >= c1) return;
+    const __amdgpu_buffer_rsrc_t rows = rows_of(c);
+#pragma unroll
+    for (int j = 0; j < kGatherLoads; ++j) {
+      const int k = tap0 + 4 * j;
+      next[j] = __builtin_amdgcn_raw_buffer_load_b128(rows, k < 27 ? mine : kNoColumn, min(k, 26) * row_bytes, 0);
+    }
+  };
+  // Set-up, everything asked for at once: the first tile, the neighbour blocks of the tile's
+  // sibling groups (one contiguous piece of the table, read in 16-byte units and laid out in
+  // LDS as octree2col_block_kernel does, so that the 8 siblings of 8 groups hit 64 banks) and
+  // the mark of the call.
+  fetch(c0);
+  constexpr int kBlockUnits = kGatherTile / 8 * 64 / 4;  // 16-byte units of the tile's neighbour blocks
+  const int table_units = (int)(((int64_t)a.octree_h + 7) / 8 * 16);  // units of the whole table
+  const u32x4* table = reinterpret_cast<const u32x4*>(neigh) + (int64_t)(r0 >> 3) * 16;
+  u32x4 block[kBlockUnits / kGatherTile];
+#pragma unroll
+  for (int j = 0; j < kBlockUnits / kGatherTile; ++j) {
+    const int u = tid + j * kGatherTile;
+    block[j] = (int64_t)(r0 >> 3) * 16 + u < table_units ? table[u] : u32x4{~0u, ~0u, ~0u, ~0u};
+  }
+  if (*mark == id) {  // the scatter kernel does the work; the first chunk clears the rows for it
+    if (a.n == 0 && p < a.octree_h)
+      for (int c = c0; c < c1; ++c) data[(int64_t)c * a.octree_h + p] = 0.0f;
+    return;
+  }
+  int* s_block = reinterpret_cast<int*>(s_col);
+#pragma unroll
+  for (int j = 0; j < kBlockUnits / kGatherTile; ++j) {
+    const int u = tid + j * kGatherTile;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) s_block[stage_index(u >> 4, (u & 15) * 4 + e)] = (int)block[j][e];
+  }
+  __syncthreads();
+  // per tap: the column's place in the staged tile, or kFar + its place in the chunk when it
+  // lies outside the tile, or -1 when there is no column
+  constexpr int kFar = 1 << 30;
+  int where[27];
+#pragma unroll
+  for (int k = 0; k < 27; ++k) {
+    int h = s_block[stage_index(tid >> 3, sibling_slot(tid & 7) + a.rslot[k])];
+    bool have = p < a.octree_h && h >= lo && h < hi;  // h < height = octree_h here
+    bool inside = have && h >= r0 && h < r0 + kGatherTile;
+    where[k] = inside ? h - r0 : (have ? kFar + (h - lo) : -1);
+  }
+  __syncthreads();  // the blocks make room for the first tile
+  auto fetch_far = [&](int c, float (&ask)[27]) {
+    if (c >= c1) return;
+    const __amdgpu_buffer_rsrc_t rows = rows_of(c);
+#pragma unroll
+    for (int k = 0; k < 27; ++k) {
+      ask[k] = 0.0f;
+      if (where[k] >= kFar)  // only the lanes that ask take part in the load
+        ask[k] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rows, (where[k] - kFar) * 4, k * row_bytes, 0));
+    }
+  };
+  // One channel: the far columns are asked for, the tile goes from registers to LDS, the loads of
+  // the next channel's tile start, then the taps are summed.
+  float ask[27];
+  if (tid == 0) s_col[27 * kGatherTile] = 0.0f;
+  for (int c = c0; c < c1; ++c) {
+    fetch_far(c, ask);
+    if (c > c0) __syncthreads();  // every wavefront has summed the previous channel
+#pragma unroll
+    for (int j = 0; j < kGatherLoads; ++j) {
+      const int k = tap0 + 4 * j;
+      if (k < 27) *reinterpret_cast<u32x4*>(&s_col[k * kGatherTile + group]) = next[j];
+    }
+    // The far loads sit in branches, where the compiler cannot count them: without this wait for
+    // all loads it waits for all of them at the first far value below, when the next tile flies.
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    fetch(c + 1);  // before the barrier: a wavefront whose part of the tile has arrived early asks early
+    __syncthreads();
+    float acc = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 27; ++k) {
+      // Every lane reads LDS (the zero word when its column is not in the tile) and takes the bits
+      // of the far value on top, which are zero when it did not ask.  A select between the two
+      // the compiler turns into an LDS read under a lane mask into the register of the far value,
+      // with a wait for every load in flight before each read.
+      const unsigned near = __float_as_uint(s_col[(unsigned)where[k] < (unsigned)kGatherTile
+                                                      ? k * kGatherTile + where[k] : 27 * kGatherTile]);
+      const float v = __uint_as_float(near | __float_as_uint(ask[k]));
+      acc = where[k] < 0 ? acc : acc + v;
+    }
+    if (p < a.octree_h) {
+      float* dst = &data[(int64_t)c * a.octree_h + p];
+      *dst = a.n == 0 ? acc : *dst + acc;
+    }
+  }
+}
+
 // Scatter form, for any table (octree_nn.cu:130-174); runs only for a marked call.
 template <bool P>
 __global__ void col2octree_atomic_kernel(const float* __restrict__ col, float* __restrict__ data,
@@ -640,8 +767,15 @@ int run_col2octree(const void* col, void* data, int channel, int height, int oct
     col_check_kernel<P><<<check_grid, kBlock, 0, s>>>(a, neigh, child, ichild, mark, id, !can_invert);
     OCNN_LAUNCH_OK("col_check");
   }
-  col2octree_kernel<P><<<dim3(blocks_for(octree_h), chans), kBlock, 0, s>>>((const float*)col,
-      (float*)data, a, neigh, child, ichild, mark, id);
+  if (!P && stride == 1 && a.K == 27 && height == octree_h && ((int64_t)n * height_col) % 4 == 0 &&
+      (int64_t)27 * height_col * 4 < (int64_t(1) << 31)) {
+    col2octree_tile_kernel<<<dim3(blocks_for(octree_h, kGatherTile), chans), kGatherTile,
+        (27 * kGatherTile + 1) * sizeof(float), s>>>(
+        (const float*)col, (float*)data, a, neigh, mark, id);
+  } else {
+    col2octree_kernel<P><<<dim3(blocks_for(octree_h), chans), kBlock, 0, s>>>((const float*)col,
+        (float*)data, a, neigh, child, ichild, mark, id);
+  }
   OCNN_LAUNCH_OK("col2octree");
   if (chunk_cols > 0) {
     col2octree_atomic_kernel<P><<<dim3(blocks_for(height_col), chans), kBlock, 0, s>>>(

@@ -171,15 +171,17 @@ def test_col2octree_any_table_and_chunks(oc, orc, tree):
       h = H if stride == 1 else H // 8
       col = rng.standard_normal((5, K, h)).astype(np.float32)
       exp = orc.col2octree(col, ks, stride, table, h)
-      hc = (h + 2) // 3                                  # three chunks, the last one ragged
-      out = torch.full((5, H), 7.0, device="cuda")       # stale values the first chunk must replace
-      for n in range(3):
-        piece = np.zeros((5, K, hc), np.float32)
-        w = max(0, min(h, (n + 1) * hc) - n * hc)
-        piece[:, :, :w] = col[:, :, n * hc:n * hc + w]
-        piece_d = T(piece).cuda()
-        oc.lib.call("ocnn_col2octree", P(piece_d), P(out), 5, h, ksc, stride, P(table_d), hc, n, 0, st)
-      assert relerr(out.cpu().numpy(), exp) < TOL_F32, (name, ks, stride)
+      # three chunks, the last one ragged; the second height is a multiple of 4, which the tiled
+      # gather kernel of the 27 taps asks of a chunk's first column
+      for hc in ((h + 2) // 3, (h // 3 + 4) // 4 * 4):
+        out = torch.full((5, H), 7.0, device="cuda")       # stale values the first chunk must replace
+        for n in range(3):
+          piece = np.zeros((5, K, hc), np.float32)
+          w = max(0, min(h, (n + 1) * hc) - n * hc)
+          piece[:, :, :w] = col[:, :, n * hc:n * hc + w]
+          piece_d = T(piece).cuda()
+          oc.lib.call("ocnn_col2octree", P(piece_d), P(out), 5, h, ksc, stride, P(table_d), hc, n, 0, st)
+        assert relerr(out.cpu().numpy(), exp) < TOL_F32, (name, ks, stride, hc)
       hp = Hne if stride == 1 else H // 8
       colp = rng.standard_normal((5, K, hp)).astype(np.float32)
       expp = orc.col2octreeP(colp, ks, stride, table, child, ichild, hp, Hne)
@@ -207,6 +209,24 @@ def test_col2octree_any_table_and_chunks(oc, orc, tree):
         oc.lib.call("ocnn_col2octreeP", P(colp_d), P(outq), 5, hp, Hne, ksc, stride, P(table_d),
                     P(child_d), C.c_void_p(0), hp, 0, 0, st)
         assert relerr(outq.cpu().numpy(), expp) < TOL_F32, (name, "P, no ichild", ks, stride)
+
+
+def test_col2octree_sums_in_the_reference_order(oc, orc, tree):
+  """The gather forms add the taps of a row in ascending order, which is the order in which the
+  reference's loops (channel, tap, column: octree_nn.cpp:216-241) reach that row: the sums are
+  equal bit for bit, on random col entries (not an octree2col image) so that every tap counts.
+  Depth 6 of the tree spans several 1024-row tiles of the 27-tap kernel."""
+  b, dev = tree["blob"], tree["dev"]
+  rng = np.random.default_rng(21)
+  for d in (4, 6):
+    H = int(b.nnum[d])
+    neigh = b.prop("neigh", d).reshape(-1)
+    for ks in ([3, 3, 3], [3, 1, 3]):
+      K = int(np.prod(ks))
+      col = rng.standard_normal((11, K, H)).astype(np.float32)
+      exp = orc.col2octree(col, ks, 1, neigh, H)
+      got = oc.nn.col2octree(T(col).cuda(), dev, d, ks, 1, False)
+      assert np.array_equal(got.cpu().numpy().reshape(11, H), exp), (d, ks)
 
 
 CONV_CASES = [(ks, s, ne) for ks in KERNELS for s in (1, 2) for ne in (False, True)]
