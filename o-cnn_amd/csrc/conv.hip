@@ -700,8 +700,10 @@ __global__ void pack_weights_rows_bf16(uint16_t* __restrict__ Wt, const uint16_t
 // Workgroup = 4 wavefronts = 256 columns = 32 sibling groups; wavefront w owns groups
 // 8w .. 8w+7 (its own 64 columns), stages only those, and computes all output channels of
 // a pass (MT row tiles).  The channel loop runs in slabs of kSlab = 2 input channels (one MFMA
-// k-step per tap; short slabs keep a workgroup at 34 KiB of LDS and 164 VGPRs, so that three
-// workgroups share a CU and fill one another's barrier gaps):
+// k-step per tap; short slabs keep a workgroup at 34 KiB of LDS, and with buffer loads (scalar
+// base, one 32-bit offset a lane, nothing to mask) the kernel fits 128 VGPRs, so that four
+// workgroups share a CU and fill one another's barrier gaps; with 64-bit addresses in registers
+// it took 164 VGPRs and three workgroups, 6 % slower):
 //   LDS X [kSlab][32 groups][80]  fp32: the neighbour blocks (wavefront-private parts)
 //   LDS W [K][kSlab/2][MT][64]    fp32: the slab's weights in A-fragment order (shared)
 // Group g sits at word 80*g + {0,2,8,10}[g&3]: with that skew the 32 lanes of a half
@@ -719,7 +721,7 @@ __device__ inline int group_base(int g) {
 }
 
 template <int MT, int K>
-__global__ __launch_bounds__(256, 3) void conv_s1_f32_lds_kernel(ConvArgs a, float* __restrict__ out,
+__global__ __launch_bounds__(256, 4) void conv_s1_f32_lds_kernel(ConvArgs a, float* __restrict__ out,
     const float* __restrict__ in, const float* __restrict__ Wt, int n_tiles) {
   constexpr int kWWords = K * kKSteps * MT * 64;          // weight words per (pass, slab)
   constexpr int kWVec = (kWWords / 4 + 255) / 256;  // float4 loads per thread
@@ -734,7 +736,8 @@ __global__ __launch_bounds__(256, 3) void conv_s1_f32_lds_kernel(ConvArgs a, flo
   const int npass = (a.mtiles + MT - 1) / MT;
   const bool mirrored = a.slot[0] != 0;  // deconvolution walks the taps through the opposite offsets
 
-  // neighbour rows of slot `lane` of my eight groups (kept for all slabs and passes)
+  // neighbour rows of slot `lane` of my eight groups (kept for all slabs and passes), as byte
+  // offsets into a channel of the input; a missing neighbour lies past any channel and reads as zero
   int nb[8];
   const int group0 = (tile * kTileCols) / 8 + wave * 8;
   const int n_groups = a.N >> 3;
@@ -742,7 +745,7 @@ __global__ __launch_bounds__(256, 3) void conv_s1_f32_lds_kernel(ConvArgs a, flo
   for (int j = 0; j < 8; ++j) {
     int g = group0 + j;
     int v = g < n_groups ? a.neigh[((int64_t)g << 6) + lane] : -1;
-    nb[j] = (v >= 0 && v < a.Hin) ? v : -1;
+    nb[j] = (v >= 0 && v < a.Hin) ? v * 4 : (int)0x80000000u;
   }
   // LDS word offsets of my two B columns (channel plane and tap slot are added per read)
   int boff[2];
@@ -761,24 +764,24 @@ __global__ __launch_bounds__(256, 3) void conv_s1_f32_lds_kernel(ConvArgs a, flo
 
     float xr[8][kSlab];
     float4 wr[kWVec];
+    // Buffer loads: a scalar base and one 32-bit offset a lane, no 64-bit addresses in registers;
+    // what lies past a buffer (a piece behind the slab's weights, a channel behind the last) reads as zero.
     auto fetch = [&](int slab) {
-      const float4* wsrc = reinterpret_cast<const float4*>(Wt + ((int64_t)pass * nslab + slab) * kWWords);
+      const __amdgpu_buffer_rsrc_t wsrc = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<float*>(Wt) + ((int64_t)pass * nslab + slab) * kWWords, 0, kWWords * 4, 0x00020000);
 #pragma unroll
       for (int v = 0; v < kWVec; ++v) {
-        int idx = v * 256 + threadIdx.x;
-        wr[v] = idx < kWWords / 4 ? wsrc[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+        const u32x4 w4 = __builtin_amdgcn_raw_buffer_load_b128(wsrc, (v * 256 + (int)threadIdx.x) * 16, 0, 0);
+        wr[v] = make_float4(__uint_as_float(w4[0]), __uint_as_float(w4[1]), __uint_as_float(w4[2]), __uint_as_float(w4[3]));
       }
 #pragma unroll
       for (int cc = 0; cc < kSlab; ++cc) {
         const int c = slab * kSlab + cc;
-        if (c < a.Cin) {
-          const float* pc = in + (int64_t)c * a.Hin;
+        const __amdgpu_buffer_rsrc_t plane = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float*>(in) + (int64_t)c * a.Hin, 0, c < a.Cin ? a.Hin * 4 : 0, 0x00020000);
 #pragma unroll
-          for (int j = 0; j < 8; ++j) xr[j][cc] = pc[(uint32_t)max(nb[j], 0)];  // masked when staged
-        } else {
-#pragma unroll
-          for (int j = 0; j < 8; ++j) xr[j][cc] = 0.0f;
-        }
+        for (int j = 0; j < 8; ++j)
+          xr[j][cc] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(plane, nb[j], 0, 0));
       }
     };
     fetch(0);
@@ -792,8 +795,8 @@ __global__ __launch_bounds__(256, 3) void conv_s1_f32_lds_kernel(ConvArgs a, flo
 #pragma unroll
       for (int cc = 0; cc < kSlab; ++cc)
 #pragma unroll
-        for (int j = 0; j < 8; ++j)  // the mask is applied here so that nothing waits for the gathers earlier
-          sX[cc * kPlane + group_base(wave * 8 + j) + lane] = nb[j] >= 0 ? xr[j][cc] : 0.0f;
+        for (int j = 0; j < 8; ++j)
+          sX[cc * kPlane + group_base(wave * 8 + j) + lane] = xr[j][cc];
       __syncthreads();
       if (slab + 1 < nslab) fetch(slab + 1);
       // taps in (dx, dy) pairs of three dz each: the slot of tap (dx, dy, dz) is dx<<4 | dy<<2 | dz
@@ -2272,7 +2275,8 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
              (dtype != OCNN_F32 || (reinterpret_cast<uintptr_t>(weights) & 15) == 0)) {
     path = kPathS2Deconv;
     copies_input = dtype != OCNN_F32;
-  } else if (dtype == OCNN_F32 && a.mode == kModeS1 && !a.nempty && a.K == 27) {
+  } else if (dtype == OCNN_F32 && a.mode == kModeS1 && !a.nempty && a.K == 27 &&
+             a.Hin < (1 << 29)) {  // its gathers address a channel with 32-bit byte offsets
     path = kPathS1LdsF32;
     copies_input = false;
   } else if (dtype == OCNN_F32) {
