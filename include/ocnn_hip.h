@@ -287,6 +287,10 @@ int ocnn_octree_deconv_grad(void* grad_data, void* grad_weights, const void* dat
  * (octree/octree/octree_nn.h:196-201, octree_nn.cu:710-752): top[c, idx[h]] = btm[c, h] for
  * idx[h] != -1 (top is zero-filled first); backward gathers.  `octree_align`
  * (pytorch/cpp/octree_align.cpp:9-83) = key arrays of both octrees -> ocnn_search_key -> this.
+ * ocnn_align_forward_ws: the same result with `inverse_ws` (top_h ints of device memory, contents
+ * ignored and overwritten): idx is inverted there and every row of top is written once, its
+ * source row or zero, instead of twice.  Where two rows of btm name one row of top (keys of an
+ * octree never do) one of them wins, as in the scatter.
  * ocnn_octree_interp: octree_nearest_pts (method 0) / octree_trilinear_pts (method 1) of
  * pytorch/ocnn/modules.py:209-275 in two kernels.  key[n_key]: the sorted Morton keys of the
  * searched depth (de-padded by the caller for nempty, as octree_search_key does,
@@ -295,6 +299,8 @@ int ocnn_octree_deconv_grad(void* grad_data, void* grad_weights, const void* dat
  * backward call, which zero-fills grad_data [channel, H] and scatters with fp32 atomics. */
 int ocnn_align_forward(float* top, int top_h, int channel, const float* btm, int btm_h, const int* idx,
     ocnn_stream_t stream);
+int ocnn_align_forward_ws(float* top, int top_h, int channel, const float* btm, int btm_h, const int* idx,
+    int* inverse_ws, ocnn_stream_t stream);
 int ocnn_align_backward(const float* top, int top_h, int channel, float* btm, int btm_h, const int* idx,
     ocnn_stream_t stream);
 int ocnn_octree_interp(float* out, const float* data, int channel, int H, const uint64_t* key, int n_key,

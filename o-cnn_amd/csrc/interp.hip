@@ -29,6 +29,17 @@ __global__ void align_backward_kernel(const float* __restrict__ top, int top_h, 
   const bool ok = j >= 0 && j < top_h;
   for (int c = 0; c < channel; ++c) btm[(int64_t)c * btm_h + h] = ok ? top[(int64_t)c * top_h + j] : 0.0f;
 }
+__global__ void fill_i32_kernel(int* __restrict__ p, int n, int v) {
+  const int i = blockIdx.x * kBlock + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+// inverse[index[h]] = h over the valid entries of index; inverse was filled with -1 first
+__global__ void align_invert_kernel(int* __restrict__ inverse, int top_h, const int* __restrict__ index, int btm_h) {
+  const int h = blockIdx.x * kBlock + threadIdx.x;
+  if (h >= btm_h) return;
+  const int j = index[h];
+  if (j >= 0 && j < top_h) inverse[j] = h;
+}
 // octree_mask (octree_nn.cu:805-818): the rows whose label equals `mask` become zero.
 // One thread per four consecutive rows of one channel where the row count allows.
 __global__ void mask_rows_kernel(float* __restrict__ out, const float* __restrict__ in,
@@ -380,6 +391,21 @@ int ocnn_align_forward(float* top, int top_h, int channel, const float* btm, int
   if (n > 0) zero_kernel<<<blocks_for(n), kBlock, 0, s>>>(top, n);
   if (btm_h > 0) align_forward_kernel<<<blocks_for(btm_h), kBlock, 0, s>>>(top, top_h, btm, btm_h, idx, channel);
   OCNN_LAUNCH_OK("align_forward");
+  return OCNN_OK;
+}
+
+int ocnn_align_forward_ws(float* top, int top_h, int channel, const float* btm, int btm_h, const int* idx,
+    int* inverse_ws, ocnn_stream_t stream) {
+  OCNN_REQUIRE(top && btm && idx && inverse_ws && top_h >= 0 && btm_h >= 0 && channel > 0, OCNN_E_BADARG,
+      "bad argument");
+  hipStream_t s = as_stream(stream);
+  if (top_h == 0) return OCNN_OK;
+  // Every row of top is written once, by the thread of that row: its source row through the
+  // inverted index, or zero.  (The scatter form writes top twice, the zeros and the rows.)
+  fill_i32_kernel<<<blocks_for(top_h), kBlock, 0, s>>>(inverse_ws, top_h, -1);
+  if (btm_h > 0) align_invert_kernel<<<blocks_for(btm_h), kBlock, 0, s>>>(inverse_ws, top_h, idx, btm_h);
+  align_backward_kernel<<<blocks_for(top_h), kBlock, 0, s>>>(btm, btm_h, top, top_h, inverse_ws, channel);
+  OCNN_LAUNCH_OK("align_forward_ws");
   return OCNN_OK;
 }
 

@@ -1133,7 +1133,9 @@ def octree_align(src_data, src_octree, des_octree, depth):
   idx = torch.empty(src_h, dtype=torch.int32, device=src_data.device)
   _lib.call("ocnn_search_key", _ptr(idx), _ptr(des_key), des_h, _ptr(src_key), src_h, _stream())
   out = torch.empty(1, channel, des_h, 1, dtype=torch.float32, device=src_data.device)
-  _lib.call("ocnn_align_forward", _ptr(out), des_h, channel, _ptr(src_data), src_h, _ptr(idx), _stream())
+  inverse = torch.empty(max(des_h, 1), dtype=torch.int32, device=src_data.device)
+  _lib.call("ocnn_align_forward_ws", _ptr(out), des_h, channel, _ptr(src_data), src_h, _ptr(idx), _ptr(inverse),
+            _stream())
   return [out, idx]
 
 

@@ -57,6 +57,37 @@ def test_align_between_different_octrees(oc, orc, synthetic):
     assert np.array_equal(back.cpu().numpy().reshape(x.shape), interp.octree_align_grad(g, eidx))
 
 
+def test_align_forward_forms_agree(oc):
+  """ocnn_align_forward (zero fill + scatter, the reference's form, octree_nn.cu:710-730) and
+  ocnn_align_forward_ws (inverted index, every row written once) through the C-ABI: equal bits on an
+  index with holes on both sides, stale values in the output, and empty inputs."""
+  import ctypes as C
+  P = lambda t: C.c_void_p(t.data_ptr())
+  st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+  g = torch.Generator().manual_seed(5)
+  for btm_h, top_h in ((1000, 1500), (1500, 700), (64, 64), (0, 40), (40, 0)):
+    keep = torch.rand(btm_h, generator=g) < 0.7
+    target = torch.randperm(max(top_h, 1), generator=g)[:btm_h] if top_h else torch.zeros(0, dtype=torch.int64)
+    idx = torch.full((btm_h,), -1, dtype=torch.int32)
+    n = min(btm_h, target.numel())
+    idx[:n] = torch.where(keep[:n], target[:n].to(torch.int32), torch.tensor(-1, dtype=torch.int32))
+    x = torch.randn(5, btm_h, generator=g)
+    # (an empty tensor has no address: every buffer holds one element more than it needs)
+    x_d = torch.cat([x.reshape(-1), torch.zeros(1)]).cuda()
+    idx_d = torch.cat([idx, torch.zeros(1, dtype=torch.int32)]).cuda()
+    a = torch.full((5 * top_h + 1,), 7.0, device="cuda")
+    b = torch.full((5 * top_h + 1,), 9.0, device="cuda")
+    inv = torch.full((top_h + 1,), 123, dtype=torch.int32, device="cuda")
+    oc.lib.call("ocnn_align_forward", P(a), top_h, 5, P(x_d), btm_h, P(idx_d), st)
+    oc.lib.call("ocnn_align_forward_ws", P(b), top_h, 5, P(x_d), btm_h, P(idx_d), P(inv), st)
+    assert torch.equal(a[:-1], b[:-1]), (btm_h, top_h)
+    assert float(a[-1]) == 7.0 and float(b[-1]) == 9.0 and int(inv[-1]) == 123   # nothing written past the end
+    exp = torch.zeros(5, top_h)
+    ok = idx >= 0
+    exp[:, idx[ok].long()] = x[:, ok]
+    assert torch.equal(a[:-1].cpu().view(5, top_h), exp), (btm_h, top_h)
+
+
 def test_trilinear_reference_case(oc, samples):
   octree = oc.nn.octree_batch([T(samples["octree_1"]), T(samples["octree_1"])])
   data = torch.ones(1, 3, 16, 1).cuda()
