@@ -118,7 +118,7 @@ __device__ inline float scale_coord(float p, float bbmin, float mul) {
 // themselves then need no counting launch).  Neighbouring points mostly share their high
 // digits: a wavefront whose lanes all hold the same digit adds its count once instead of
 // serialising 64 LDS atomics on one address.
-constexpr int kKeyItems = 8;
+constexpr int kKeyItems = 4;   // points per thread: 250 k points then make 244 workgroups (with 8, half the CUs had none)
 constexpr int kKeyGrid = 512;   // workgroups at most: each adds its histograms to the global ones once
 constexpr int kHistCopies = 16; // global histogram copies: atomics on one address are served one by one
 __global__ __launch_bounds__(kBlock) void keygen_kernel(uint64_t* __restrict__ key, uint32_t* __restrict__ val,
