@@ -440,7 +440,7 @@ struct LevelOut {
   int* ustart;                  // first sorted point of each leaf; [n_leaf] = n_points
 };
 
-constexpr int kLevelItems = 8;
+constexpr int kLevelItems = 4;   // keys per thread (8 left half the CUs without a workgroup on a 250 k cloud)
 constexpr int kLevelTile = kBlock * kLevelItems;
 
 template <bool TICKETS>
