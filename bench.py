@@ -495,6 +495,23 @@ def main():
               (torch.randn(co, generator=g) * 0.1).to(dev)) for d, (ci, co) in lch.items()}
     t = timed(lambda: oc.stacks.lenet_trunk(oct6, 6, lp), reps, wu)
     extra["lenet_trunk_batch32_d6_f32"] = {"ms": t, "shapes_per_s": 32 / (t * 1e-3)}
+    # the same trunk captured once in a HIP graph and replayed: its twelve operators are short
+    # kernels, and the eager time is mostly the host getting from one launch to the next
+    feat6 = F.octree_property(oct6, "feature", 6)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+      for _ in range(2):
+        oc.stacks.lenet_trunk(oct6, 6, lp, data=feat6)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+      graph_out = oc.stacks.lenet_trunk(oct6, 6, lp, data=feat6)
+    t = timed(graph.replay, reps, wu)
+    torch.cuda.synchronize()
+    same = bool(torch.equal(graph_out, oc.stacks.lenet_trunk(oct6, 6, lp, data=feat6)))
+    extra["lenet_trunk_batch32_d6_f32_graph"] = {"ms": t, "shapes_per_s": 32 / (t * 1e-3), "equals_eager": same}
+    del graph, graph_out
     # completion decoder loop (configs[4] shape): 16 octrees at depth 7 regrown from depth 2 with
     # the split labels of the built batch, deconv up + 3x3x3 conv per depth, channels 256 -> 32
     dch = {2: 256, 3: 128, 4: 64, 5: 32, 6: 32, 7: 32}

@@ -2340,7 +2340,10 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
         deconv_s2_bf16_kernel<<<dim3(d_grid, pass_split(d_tiles, (d.M * 8 + 32 * kD2MT - 1) / (32 * kD2MT))), 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles, cpad / 8);
     }
   } else if (path == kPathS1LdsF32) {
-    const int MT = a.mtiles == 1 ? 1 : 2;
+    // Two row tiles a workgroup halve the gathers per product, one row tile doubles the number of
+    // workgroups: the latter where a level is so small that the former leaves the CUs short of work
+    // (12 824 columns, 128 -> 256 channels: 0.31 -> 0.285 ms).
+    const int MT = (a.mtiles == 1 || (int64_t)n_tiles * ((a.mtiles + 1) / 2) < 512) ? 1 : 2;
     const int npass = (a.mtiles + MT - 1) / MT, nslab = (a.Cin + kSlab - 1) / kSlab;
     int64_t total = (int64_t)npass * nslab * a.K * kKSteps * MT * 64;
     pack_weights_lds_f32<<<blocks_for(total), kBlock, 0, s>>>((float*)wsb, (const float*)weights, a.M, a.Cin, a.K,
