@@ -495,8 +495,8 @@ def main():
               (torch.randn(co, generator=g) * 0.1).to(dev)) for d, (ci, co) in lch.items()}
     t = timed(lambda: oc.stacks.lenet_trunk(oct6, 6, lp), reps, wu)
     extra["lenet_trunk_batch32_d6_f32"] = {"ms": t, "shapes_per_s": 32 / (t * 1e-3)}
-    # the same trunk captured once in a HIP graph and replayed: its twelve operators are short
-    # kernels, and the eager time is mostly the host getting from one launch to the next
+    # the same trunk captured once in a HIP graph and replayed: what of the eager time is the host
+    # getting from one launch to the next (little: the convolutions of the small levels take it)
     feat6 = F.octree_property(oct6, "feature", 6)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
