@@ -1762,7 +1762,7 @@ constexpr int kD2MT = 4;  // row tiles per pass: 128 rows = 16 output channels x
 constexpr int kD2fMT = 2;
 constexpr int kD2fChunk = 64;
 
-__global__ __launch_bounds__(256, 2) void deconv_s2_f32_kernel(ConvArgs a, float* __restrict__ out,
+__global__ __launch_bounds__(256, 3) void deconv_s2_f32_kernel(ConvArgs a, float* __restrict__ out,
     const float* __restrict__ in, const float* __restrict__ W, int n_tiles) {
   __shared__ __attribute__((aligned(16))) float sW[kD2fChunk * 32 * kD2fMT];
   constexpr int kWVec = kD2fChunk * 32 * kD2fMT / 4 / 256;  // float4 per thread and stage
