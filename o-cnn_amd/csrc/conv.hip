@@ -1515,8 +1515,12 @@ __global__ void pack_weights_s2_f32(float* __restrict__ Wt, const float* __restr
 
 // bf16: one 16-byte load = all 8 taps of (channel ci0 + kh, column n); an MFMA k-step of 16
 // covers two input channels.  Slab = 8 channels = 4 k-steps.
+// (The occupancy asked for in the launch bounds matters: left to itself the compiler puts the
+// accumulators into the second register file beside 114 registers of the first and two wavefronts
+// fit a SIMD; asked for three it keeps everything in 114 registers, four fit, and the kernel is a
+// quarter faster.  The same holds for the wide-channel stride-2 deconvolution below.)
 template <int MT>
-__global__ __launch_bounds__(256) void conv_s2_bf16_kernel(ConvArgs a, uint16_t* __restrict__ out,
+__global__ __launch_bounds__(256, 3) void conv_s2_bf16_kernel(ConvArgs a, uint16_t* __restrict__ out,
     const uint16_t* __restrict__ in, const uint4* __restrict__ Wt, int n_tiles) {
   constexpr int kWUnits = 4 * MT * 64;
   __shared__ uint4 sW[kWUnits];
@@ -1594,7 +1598,7 @@ __global__ void pack_weights_s2_bf16(uint16_t* __restrict__ Wt, const uint16_t* 
 // way meanwhile.  Output rows as the 3x3x3 row-major kernel writes them.
 constexpr int kS2Stage = 8;   // k-steps per weight stage
 template <int MT>
-__global__ __launch_bounds__(256) void conv_s2_rows_bf16_kernel(ConvArgs a, uint16_t* __restrict__ out,
+__global__ __launch_bounds__(256, 3) void conv_s2_rows_bf16_kernel(ConvArgs a, uint16_t* __restrict__ out,
     int out_pitch, int out_cpad, const u32x4* __restrict__ xt, int in_pitch, int in_cpad,
     const u32x4* __restrict__ Wt, int n_tiles) {
   constexpr int kStageUnits = kS2Stage * MT * 64;
@@ -1845,7 +1849,7 @@ __global__ __launch_bounds__(256, 3) void deconv_s2_f32_kernel(ConvArgs a, float
 
 // bf16: activations come from the row-major copy [H + 1, Cpad] (16-byte operand loads); weights
 // packed [pass][kstep][mt][lane][8]: lane (m', kh), j <- W[16*kstep + 8kh + j][m']
-__global__ __launch_bounds__(256) void deconv_s2_bf16_kernel(ConvArgs a, uint16_t* __restrict__ out,
+__global__ __launch_bounds__(256, 2) void deconv_s2_bf16_kernel(ConvArgs a, uint16_t* __restrict__ out,
     const uint4* __restrict__ xt, const uint4* __restrict__ Wt, int n_tiles, int cpad8) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int tile = xcd_tile(blockIdx.x, n_tiles);
