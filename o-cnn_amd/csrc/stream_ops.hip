@@ -445,8 +445,8 @@ __global__ void col2octree_kernel(const float* __restrict__ col, float* __restri
 // col rows of a channel through LDS with coalesced 16-byte loads, the next channel flying
 // while this one is summed.  A row finds the column of a tap in LDS when that column lies
 // inside the tile (19 of 20 do in a depth-9 scene, neighbours being close in z-order); for the
-// others the thread asks global memory, in a wavefront that has such a tap at all, before the
-// tile is written to LDS.  Taps are summed in ascending order as above.
+// others the thread asks global memory (a load under a lane mask) before the tile is written to
+// LDS.  Taps are summed in ascending order as above.
 constexpr int kGatherTile = 1024, kGatherUnits = kGatherTile / 4;  // rows of a tile, 16-byte units of a staged row
 constexpr int kGatherLoads = (27 * kGatherUnits + kGatherTile - 1) / kGatherTile;  // 16-byte loads a thread and channel
 
