@@ -532,7 +532,7 @@ def main():
     orc = Checker("orc")
     blob_host = octree.cpu().numpy()
     ob = OctreeBlob(blob_host)
-    sample = 32768
+    sample = 327680   # about 10 s of single-thread work
     neigh = ob.prop("neigh", 9).reshape(-1)
     xh = x32.cpu().numpy().reshape(C, H9)
     wh = w32.cpu().numpy()
