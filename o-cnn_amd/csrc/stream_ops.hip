@@ -279,68 +279,260 @@ __global__ void __launch_bounds__(kColTile) octree2col_kernel(T* __restrict__ co
 }
 
 // Stride 1 over all nodes: the 27 taps of the 8 columns of a sibling group all lie in
-// the group's 64-entry block, so a workgroup gathers each block of its tile once per
-// channel (64 reads per group instead of 8 x 27) into LDS and serves every tap from
+// the group's 64-entry block, so a workgroup stages the blocks of its tile once per
+// channel in LDS (64 values per group instead of 8 x 27) and serves every tap from
 // there, with the same per-row shift for aligned stores.  Entry s of staged group g
 // sits at g * 64 + (s ^ spread(g)), spread() moving the low bits of g to bits 1, 3, 5:
 // the 8 columns of a group differ in bits 0, 2, 4 of s, so a wavefront's 64 reads hit
 // 64 different banks.
-constexpr int kStageGroups = (kColTile + kColApron) / 8 + 1;  // + 1: a chunk may start inside a group
+constexpr int kBlockTile = 256;  // columns and threads of a workgroup
+constexpr int kStageGroups = (kBlockTile + kColApron) / 8 + 1;  // + 1: a chunk may start inside a group
 constexpr int kStageSlots = kStageGroups * 64;
-constexpr int kStagePerThread = (kStageSlots + kColTile - 1) / kColTile;
+constexpr int kStagePerThread = (kStageSlots + kBlockTile - 1) / kBlockTile;
+constexpr int kOctCap = 128;  // octets a tile may copy (a tile of the scenes measured names 66 on average, 132 at most)
+constexpr int kOctTab = 512;  // slots of the hash table that finds them (a quarter full at most)
 
 __device__ inline int stage_index(int g, int s) {
   return g * 64 + (s ^ (((g & 1) << 1) | ((g & 2) << 2) | ((g & 4) << 3)));
 }
 
-template <typename T>
-__global__ void __launch_bounds__(kColTile) octree2col_block_kernel(T* __restrict__ col,
+template <typename T, int KC>  // KC: the taps when known (27), which lets the waits count the stores; 0: a.K
+__global__ void __launch_bounds__(kBlockTile) octree2col_block_kernel(T* __restrict__ col,
     const T* __restrict__ data, ColArgs a, const int* __restrict__ neigh) {
   __shared__ T s_val[2][kStageSlots];
   const int tid = threadIdx.x;
   const int lo = a.n * a.height_col;
-  const int first = blockIdx.x * kColTile - kColApron;  // first column the tile may store
+  const int first = blockIdx.x * kBlockTile - kColApron;  // first column the tile may store
   const int g0 = (lo + first) >> 3;                      // first staged group (may be negative)
-  int src[kStagePerThread];  // rows behind this thread's staged entries, the same for every channel
+  // Loads and stores go through buffers (a channel of the input, a row of col): what is not there
+  // gets an offset past the end, reads as zero and is not stored, so that neither sits in a branch
+  // and the waits are exact: the gathers of the next channel are waited for while the stores of
+  // this one are still on their way (with branches the compiler waits for everything in flight).
+  constexpr int kNone = (int)0x80000000u;
+  int src[kStagePerThread];  // byte offsets of the rows behind this thread's staged entries, the same for every channel
 #pragma unroll
   for (int j = 0; j < kStagePerThread; ++j) {
-    int i = tid + j * kColTile, g = g0 + (i >> 6);
+    int i = tid + j * kBlockTile, g = g0 + (i >> 6);
     int p = -1;
     if (i < kStageSlots && g >= 0 && (int64_t)g * 8 < a.height) p = neigh[((int64_t)g << 6) + (i & 63)];
-    src[j] = (p >= 0 && p < a.octree_h) ? p : -1;
+    src[j] = (p >= 0 && p < a.octree_h) ? p * (int)sizeof(T) : kNone;
   }
   const uint64_t col_elem = reinterpret_cast<uintptr_t>(col) / sizeof(T);
   // The rows of the next channel are gathered into registers while the taps of this
   // one are stored.
   T next[kStagePerThread];
   auto gather = [&](int c) {
-    const T* row_in = data + (int64_t)c * a.octree_h;
+    const __amdgpu_buffer_rsrc_t plane = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T*>(data) + (int64_t)c * a.octree_h, 0, a.octree_h * (int)sizeof(T), 0x00020000);
 #pragma unroll
-    for (int j = 0; j < kStagePerThread; ++j) next[j] = src[j] < 0 ? zero_of<T>() : row_in[src[j]];
+    for (int j = 0; j < kStagePerThread; ++j) {
+      if constexpr (sizeof(T) == 4) next[j] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(plane, src[j], 0, 0));
+      else next[j] = (T)__builtin_amdgcn_raw_buffer_load_b16(plane, src[j], 0, 0);
+    }
   };
-  if ((int)blockIdx.y < a.channel) gather(blockIdx.y);
-  int turn = 0;
-  for (int c = blockIdx.y; c < a.channel; c += gridDim.y, turn ^= 1) {  // few tiles: channels dealt out
+  auto pass = [&](int c, int turn) __attribute__((always_inline)) {
     T* val = s_val[turn];
 #pragma unroll
     for (int j = 0; j < kStagePerThread; ++j) {
-      int i = tid + j * kColTile;
+      int i = tid + j * kBlockTile;
       if (i < kStageSlots) val[stage_index(i >> 6, i & 63)] = next[j];
     }
     __syncthreads();  // one barrier per channel: the other buffer is still being read
     if (c + (int)gridDim.y < a.channel) gather(c + gridDim.y);
-#pragma unroll 9
-    for (int k = 0; k < a.K; ++k) {
+    auto put = [&](int k) {
       int64_t row = ((int64_t)c * a.K + k) * a.height_col;
       int shift = (int)((col_elem + (uint64_t)row) & (kColApron - 1));
       int hl = first + kColApron + tid - shift;
-      if (hl < 0 || hl >= a.height_col) continue;
+      const bool inside = hl >= 0 && hl < a.height_col;
       int h = lo + hl;
       T v = zero_of<T>();
-      if (h < a.height) v = val[stage_index((h >> 3) - g0, sibling_slot(h & 7) + a.slot[k])];
-      col[row + hl] = v;
+      if (inside && h < a.height) v = val[stage_index((h >> 3) - g0, sibling_slot(h & 7) + a.slot[k])];
+      const __amdgpu_buffer_rsrc_t out_row = __builtin_amdgcn_make_buffer_rsrc(
+          col + row, 0, a.height_col * (int)sizeof(T), 0x00020000);
+      const int at = inside ? hl * (int)sizeof(T) : kNone;
+      if constexpr (sizeof(T) == 4) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), out_row, at, 0, 0);
+      else __builtin_amdgcn_raw_buffer_store_b16((short)v, out_row, at, 0, 0);
+    };
+    if constexpr (KC > 0) {
+#pragma unroll
+      for (int k = 0; k < KC; ++k) put(k);
+    } else {
+#pragma unroll 9
+      for (int k = 0; k < a.K; ++k) put(k);
     }
+  };
+  // Few tiles: channels dealt out over blockIdx.y.  The first channel stands outside the loop so
+  // that every turn of the loop starts in the same state (a gather under way and, after it, the
+  // stores of the channel before): the wait for the gather can then leave those stores in flight.
+  int c = blockIdx.y;
+  if (c >= a.channel) return;
+  gather(c);
+  pass(c, 0);
+  int turn = 1;
+  for (c += gridDim.y; c < a.channel; c += gridDim.y, turn ^= 1) pass(c, turn);
+}
+
+// The same with each value loaded once.  The blocks of neighbouring groups overlap: the 64
+// entries of a block lie in 27 sibling octets (rows p with the same p >> 3, 32 contiguous
+// bytes of a float channel), and the 41 blocks of a tile name about 70 different octets of a
+// scene, not 41 x 27.  A load instruction costs by the cache lines its lanes touch, so the
+// tile finds its octets once (a hash table in LDS), loads each of them once per channel in
+// 16-byte units, and fills the blocks from that copy.  A tile with more octets than the copy
+// holds gathers every entry from memory as above (same results).  Finding the octets costs
+// about as much as two channels, and the units need channels that start on 16-byte
+// boundaries: other calls go to the kernel above.
+template <typename T, int KC>
+__global__ void __launch_bounds__(kBlockTile) octree2col_octet_kernel(T* __restrict__ col,
+    const T* __restrict__ data, ColArgs a, const int* __restrict__ neigh) {
+  constexpr int kUnitElems = 16 / (int)sizeof(T);       // elements of a 16-byte unit
+  constexpr int kOctUnits = 8 / kUnitElems;             // units of an octet
+  constexpr int kUnits = kOctCap * kOctUnits;           // units of a copy
+  constexpr int kUnitLoads = (kUnits + kBlockTile - 1) / kBlockTile;  // units a thread loads per channel
+  constexpr int kZeroOct = kOctCap * 8;                 // an octet of zeros behind the copy
+  static_assert(kStageSlots % kUnitElems == 0, "the copies start on a 16-byte boundary");
+  __shared__ __align__(16) T s_mem[kStageSlots + 2 * (kZeroOct + 8)];
+  __shared__ int s_count, s_over;
+  T* const val = s_mem;                // the staged blocks
+  T* const oct = s_mem + kStageSlots;  // two copies of the octets (this channel's, the next one's), each followed by the zeros
+  // The tables of the set-up lie over both and are dead before the first channel.
+  int* const s_key = reinterpret_cast<int*>(s_mem);                                  // octet in a slot, or -1
+  unsigned short* const s_id = reinterpret_cast<unsigned short*>(s_key + kOctTab);   // its place in the copy
+  int* const s_list = reinterpret_cast<int*>(s_id + kOctTab);                        // octet at a place
+  static_assert(kOctTab * 6 + kOctCap * 4 <= (int)sizeof(s_mem), "set-up tables");
+  const int tid = threadIdx.x;
+  const int lo = a.n * a.height_col;
+  const int first = blockIdx.x * kBlockTile - kColApron;  // first column the tile may store
+  const int g0 = (lo + first) >> 3;                      // first staged group (may be negative)
+  // Loads and stores go through buffers (a channel of the input, a row of col): what is not there
+  // gets an offset past the end, reads as zero and is not stored, so that neither sits in a branch
+  // and the waits are exact: the loads of the next channel are waited for while the stores of
+  // this one are still on their way (with branches the compiler waits for everything in flight).
+  constexpr int kNone = (int)0x80000000u;
+  for (int i = tid; i < kOctTab; i += kBlockTile) s_key[i] = -1;
+  if (tid == 0) { s_count = 0; s_over = 0; }
+  __syncthreads();
+  auto slot_of = [&](int o, bool insert) {  // linear probing; -1: no room (insert) or not there
+    const unsigned at = ((unsigned)o * 2654435761u) >> 23;
+    for (int probe = 0; probe < 32; ++probe) {
+      const int slot = (at + probe) & (kOctTab - 1);
+      const int old = insert ? atomicCAS(&s_key[slot], -1, o) : s_key[slot];
+      if (old == o || (insert && old == -1)) return slot;
+      if (old == -1) return -1;
+    }
+    return -1;
+  };
+  // Per staged entry of this thread: first its row, then where its value comes from, the same
+  // for every channel (an index into oct, or a byte offset into the channel when gathering).
+  int from[kStagePerThread];
+#pragma unroll
+  for (int j = 0; j < kStagePerThread; ++j) {
+    int i = tid + j * kBlockTile, g = g0 + (i >> 6);
+    int p = -1;
+    if (i < kStageSlots && g >= 0 && (int64_t)g * 8 < a.height) p = neigh[((int64_t)g << 6) + (i & 63)];
+    from[j] = (p >= 0 && p < a.octree_h) ? p : -1;
+    if (from[j] >= 0 && slot_of(p >> 3, true) < 0) s_over = 1;
   }
+  __syncthreads();
+  for (int i = tid; i < kOctTab; i += kBlockTile) {
+    const int o = s_key[i];
+    if (o < 0) continue;
+    const int id = atomicAdd(&s_count, 1);  // any order: the places only say where a value waits
+    if (id < kOctCap) { s_list[id] = o; s_id[i] = (unsigned short)id; }
+  }
+  __syncthreads();
+  const int n_oct = s_count;
+  const bool gathers = s_over != 0 || n_oct > kOctCap;  // the same for the whole workgroup
+  int unit_at[kUnitLoads];  // byte offsets, within a channel, of the units this thread copies
+#pragma unroll
+  for (int l = 0; l < kUnitLoads; ++l) {
+    const int u = tid + l * kBlockTile, o = u / kOctUnits;
+    unit_at[l] = (!gathers && o < n_oct) ? (s_list[o] * 8 + (u % kOctUnits) * kUnitElems) * (int)sizeof(T) : kNone;
+  }
+#pragma unroll
+  for (int j = 0; j < kStagePerThread; ++j) {
+    const int p = from[j];
+    if (gathers) from[j] = p >= 0 ? p * (int)sizeof(T) : kNone;
+    else from[j] = p >= 0 ? s_id[slot_of(p >> 3, false)] * 8 + (p & 7) : kZeroOct;
+  }
+  __syncthreads();  // the tables have been read
+  if (tid < 16) oct[(tid >> 3) * (kZeroOct + 8) + kZeroOct + (tid & 7)] = zero_of<T>();
+  const uint64_t col_elem = reinterpret_cast<uintptr_t>(col) / sizeof(T);
+  // What the next channel needs is loaded into registers while the taps of this one are stored.
+  u32x4 unit[kUnitLoads];
+  T next[kStagePerThread];
+  auto fetch = [&](int c) {
+    const __amdgpu_buffer_rsrc_t plane = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T*>(data) + (int64_t)c * a.octree_h, 0, a.octree_h * (int)sizeof(T), 0x00020000);
+    if (gathers) {
+#pragma unroll
+      for (int j = 0; j < kStagePerThread; ++j) {
+        if constexpr (sizeof(T) == 4) next[j] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(plane, from[j], 0, 0));
+        else next[j] = (T)__builtin_amdgcn_raw_buffer_load_b16(plane, from[j], 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int l = 0; l < kUnitLoads; ++l) unit[l] = __builtin_amdgcn_raw_buffer_load_b128(plane, unit_at[l], 0, 0);
+    }
+  };
+  // Copy b holds the octets of the channel being stored; those of the next channel are written
+  // into the other copy at the top of a pass, a whole pass after their loads were issued, and the
+  // loads of the channel after that are issued right behind.
+  auto land = [&](int b) {
+#pragma unroll
+    for (int l = 0; l < kUnitLoads; ++l)
+      if (tid + l * kBlockTile < kUnits) reinterpret_cast<u32x4*>(oct + b * (kZeroOct + 8))[tid + l * kBlockTile] = unit[l];
+  };
+  auto pass = [&](int c, int b) __attribute__((always_inline)) {
+    const int step = gridDim.y;
+    if (!gathers) {
+      if (c + step < a.channel) land(b ^ 1);
+      if (c + 2 * step < a.channel) fetch(c + 2 * step);
+    }
+    __syncthreads();  // the octets are in place, and nobody reads the blocks of the channel before
+    const T* const here = oct + b * (kZeroOct + 8);
+#pragma unroll
+    for (int j = 0; j < kStagePerThread; ++j) {
+      int i = tid + j * kBlockTile;
+      T v = gathers ? next[j] : here[from[j]];
+      if (i < kStageSlots) val[stage_index(i >> 6, i & 63)] = v;
+    }
+    if (gathers && c + step < a.channel) fetch(c + step);
+    __syncthreads();  // the blocks are in place
+    auto put = [&](int k) {
+      int64_t row = ((int64_t)c * a.K + k) * a.height_col;
+      int shift = (int)((col_elem + (uint64_t)row) & (kColApron - 1));
+      int hl = first + kColApron + tid - shift;
+      const bool inside = hl >= 0 && hl < a.height_col;
+      int h = lo + hl;
+      T v = zero_of<T>();
+      if (inside && h < a.height) v = val[stage_index((h >> 3) - g0, sibling_slot(h & 7) + a.slot[k])];
+      const __amdgpu_buffer_rsrc_t out_row = __builtin_amdgcn_make_buffer_rsrc(
+          col + row, 0, a.height_col * (int)sizeof(T), 0x00020000);
+      const int at = inside ? hl * (int)sizeof(T) : kNone;
+      if constexpr (sizeof(T) == 4) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), out_row, at, 0, 0);
+      else __builtin_amdgcn_raw_buffer_store_b16((short)v, out_row, at, 0, 0);
+    };
+    if constexpr (KC > 0) {
+#pragma unroll
+      for (int k = 0; k < KC; ++k) put(k);
+    } else {
+#pragma unroll 9
+      for (int k = 0; k < a.K; ++k) put(k);
+    }
+  };
+  // Few tiles: channels dealt out over blockIdx.y.  The first channel stands outside the loop so
+  // that every turn of the loop starts in the same state (loads under way and, after them, the
+  // stores of the channel before): the wait for the loads can then leave those stores in flight.
+  int c = blockIdx.y;
+  if (c >= a.channel) return;
+  fetch(c);
+  if (!gathers) {
+    land(0);
+    if (c + (int)gridDim.y < a.channel) fetch(c + gridDim.y);
+  }
+  pass(c, 0);
+  int b = 1;
+  for (c += gridDim.y; c < a.channel; c += gridDim.y, b ^= 1) pass(c, b);
 }
 
 // Where a call records that its table is not symmetric.  Either a word the caller owns
@@ -715,16 +907,27 @@ int run_octree2col(void* col, const void* data, int channel, int height, int oct
   ColArgs a;
   OCNN_REQUIRE(fill_col_args(&a, channel, height, octree_h, ks, stride, height_col, n),
       OCNN_E_UNSUPPORTED, "kernel size %d%d%d", ks[0], ks[1], ks[2]);
-  unsigned tiles = blocks_for((int64_t)height_col + kColApron - 1, kColTile);
-  if (!P && stride == 1) {
+  if (!P && stride == 1 && (int64_t)octree_h * 4 < (int64_t(1) << 31) && (int64_t)height_col * 4 < (int64_t(1) << 31)) {
+    unsigned tiles = blocks_for((int64_t)height_col + kColApron - 1, kBlockTile);
     dim3 grid(tiles, std::min<unsigned>(channel, std::max(1u, 2048u / tiles)));
-    if (dtype == OCNN_F32)
-      octree2col_block_kernel<float><<<grid, kColTile, 0, s>>>((float*)col, (const float*)data, a, neigh);
-    else
-      octree2col_block_kernel<uint16_t><<<grid, kColTile, 0, s>>>((uint16_t*)col, (const uint16_t*)data, a, neigh);
+    // The octet kernel loads 16-byte units, so every channel must start on a 16-byte boundary,
+    // and it pays from about 5 channels per workgroup on.
+    const size_t esize = dtype == OCNN_F32 ? 4 : 2;
+    const bool octets = reinterpret_cast<uintptr_t>(data) % 16 == 0 && (size_t)octree_h * esize % 16 == 0 &&
+        channel / grid.y >= 5;
+#define OCNN_O2C(kernel, T, KC) kernel<T, KC><<<grid, kBlockTile, 0, s>>>((T*)col, (const T*)data, a, neigh)
+#define OCNN_O2C_TAPS(kernel, T) do { if (a.K == 27) OCNN_O2C(kernel, T, 27); else OCNN_O2C(kernel, T, 0); } while (0)
+    if (dtype == OCNN_F32) {
+      if (octets) OCNN_O2C_TAPS(octree2col_octet_kernel, float); else OCNN_O2C_TAPS(octree2col_block_kernel, float);
+    } else {
+      if (octets) OCNN_O2C_TAPS(octree2col_octet_kernel, uint16_t); else OCNN_O2C_TAPS(octree2col_block_kernel, uint16_t);
+    }
+#undef OCNN_O2C_TAPS
+#undef OCNN_O2C
     OCNN_LAUNCH_OK("octree2col");
     return OCNN_OK;
   }
+  unsigned tiles = blocks_for((int64_t)height_col + kColApron - 1, kColTile);
   dim3 grid(tiles, (channel + kChanChunk - 1) / kChanChunk);
   if (dtype == OCNN_F32)
     octree2col_kernel<float, P><<<grid, kColTile, 0, s>>>((float*)col, (const float*)data, a, neigh, child, ichild);

@@ -143,6 +143,60 @@ def test_octree2col_chunks_and_unaligned_rows(oc, orc, tree):
         assert np.all(got[:5] == 9.0) and np.all(got[5 + Cc * K * hc:] == 9.0), "wrote outside the chunk"
 
 
+def test_octree2col_many_channels_large_level(oc, orc, synthetic):
+  """From about 5 channels per workgroup on (levels of 100 000 nodes and more), stride 1 over all
+  nodes runs the kernel that copies each sibling octet of a tile once per channel.  A room at
+  depth 8 against the oracle, bit exact, fp32 and bf16: with the level's own table, with a table
+  whose groups partly name random rows (those tiles name more octets than the copy holds and
+  gather from memory) and in two column chunks through the C-ABI (octree_nn.cpp:188-214)."""
+  import ctypes as C
+  d = 8
+  p, n, f = synthetic.room_cloud(60000, 5)
+  host = orc.octree_batch([orc.points2octree(make_points_blob(p, n, f), d, 2)])
+  b, dev = OctreeBlob(host), T(host).cuda()
+  H = int(b.nnum[d])
+  assert H >= 100000, H
+  neigh = b.prop("neigh", d).reshape(-1, 64)
+  rng = np.random.default_rng(21)
+  tiles = (H + 63 + 255) // 256
+  Cc = 5 * max(1, 2048 // tiles)
+  x = rng.standard_normal((Cc, H)).astype(np.float32)
+  for tt in (torch.float32, torch.bfloat16):
+    x_d = T(x).cuda().to(tt)
+    xr = x_d.float().cpu().numpy()
+    for ks in ([3, 3, 3], [3, 1, 3]):
+      col = oc.nn.octree2col(x_d.view(1, Cc, H, 1), dev, d, ks, 1, False)
+      exp = orc.octree2col(xr, ks, 1, neigh.reshape(-1), H)
+      assert np.array_equal(col.float().cpu().numpy(), exp), (tt, ks)
+      del col, exp
+  # any table: a third of the groups name random rows or nothing
+  odd = neigh.copy()
+  pick = np.nonzero(np.arange(len(odd)) % 96 < 32)[0]
+  odd[pick] = rng.integers(-1, H, (len(pick), 64))
+  Pp = lambda t, off=0: C.c_void_p(t.data_ptr() + off)
+  st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+  ksc = (C.c_int * 3)(3, 3, 3)
+  x_d, odd_d = T(x).cuda(), T(odd.reshape(-1)).cuda()
+  exp = orc.octree2col(x, [3, 3, 3], 1, odd.reshape(-1), H)
+  out = torch.empty(Cc * 27 * H, device="cuda")
+  oc.lib.call("ocnn_octree2col", Pp(out), Pp(x_d), Cc, H, ksc, 1, Pp(odd_d), H, 0, 0, st)
+  assert np.array_equal(out.cpu().numpy().reshape(Cc, 27, H), exp)
+  Cc2 = 2 * Cc                      # half the tiles per chunk: twice the channels to stay on that kernel
+  x2 = np.concatenate([x, x[::-1]])
+  exp2 = np.concatenate([exp, exp[::-1]])
+  x2_d = T(x2).cuda()
+  hc = (H + 1) // 2 + 3
+  for n in range(2):
+    want = np.zeros((Cc2, 27, hc), np.float32)
+    w = min(H, (n + 1) * hc) - n * hc
+    want[:, :, :w] = exp2[:, :, n * hc:n * hc + w]
+    buf = torch.full((Cc2 * 27 * hc + 64,), 9.0, device="cuda")
+    oc.lib.call("ocnn_octree2col", Pp(buf, 12), Pp(x2_d), Cc2, H, ksc, 1, Pp(odd_d), hc, n, 0, st)
+    got = buf.cpu().numpy()
+    assert np.array_equal(got[3:3 + Cc2 * 27 * hc].reshape(Cc2, 27, hc), want), n
+    assert np.all(got[:3] == 9.0) and np.all(got[3 + Cc2 * 27 * hc:] == 9.0), "wrote outside the chunk"
+
+
 def test_col2octree_any_table_and_chunks(oc, orc, tree):
   """col2octree through the C-ABI in column chunks (octree_nn.cpp:216-241 adds chunk n to the
   rows the earlier chunks left), on the octree's own table and on tables that are not
