@@ -21,13 +21,25 @@ __global__ void align_forward_kernel(float* __restrict__ top, int top_h, const f
   if (j < 0 || j >= top_h) return;
   for (int c = 0; c < channel; ++c) top[(int64_t)c * top_h + j] = btm[(int64_t)c * btm_h + h];
 }
+// btm[c][h] = top[c][index[h]], or zero where the index names no row.  A thread serves one row in
+// kAlignChunk channels (blockIdx.y): their loads are issued together and outside any per-lane
+// branch (a row without a source reads row 0 and stores zero), so they are all in flight at once.
+constexpr int kAlignChunk = 8;
 __global__ void align_backward_kernel(const float* __restrict__ top, int top_h, float* __restrict__ btm, int btm_h,
     const int* __restrict__ index, int channel) {
   const int h = blockIdx.x * kBlock + threadIdx.x;
   if (h >= btm_h) return;
+  const int c0 = blockIdx.y * kAlignChunk;
   const int j = index[h];
   const bool ok = j >= 0 && j < top_h;
-  for (int c = 0; c < channel; ++c) btm[(int64_t)c * btm_h + h] = ok ? top[(int64_t)c * top_h + j] : 0.0f;
+  const int from = ok ? j : 0;
+  float v[kAlignChunk];
+#pragma unroll
+  for (int i = 0; i < kAlignChunk; ++i)
+    v[i] = (top_h > 0 && c0 + i < channel) ? top[(int64_t)(c0 + i) * top_h + from] : 0.0f;  // the same for the whole grid row
+#pragma unroll
+  for (int i = 0; i < kAlignChunk; ++i)
+    if (c0 + i < channel) btm[(int64_t)(c0 + i) * btm_h + h] = ok ? v[i] : 0.0f;
 }
 __global__ void fill_i32_kernel(int* __restrict__ p, int n, int v) {
   const int i = blockIdx.x * kBlock + threadIdx.x;
@@ -404,7 +416,8 @@ int ocnn_align_forward_ws(float* top, int top_h, int channel, const float* btm, 
   // inverted index, or zero.  (The scatter form writes top twice, the zeros and the rows.)
   fill_i32_kernel<<<blocks_for(top_h), kBlock, 0, s>>>(inverse_ws, top_h, -1);
   if (btm_h > 0) align_invert_kernel<<<blocks_for(btm_h), kBlock, 0, s>>>(inverse_ws, top_h, idx, btm_h);
-  align_backward_kernel<<<blocks_for(top_h), kBlock, 0, s>>>(btm, btm_h, top, top_h, inverse_ws, channel);
+  align_backward_kernel<<<dim3(blocks_for(top_h), (channel + kAlignChunk - 1) / kAlignChunk), kBlock, 0, s>>>(
+      btm, btm_h, top, top_h, inverse_ws, channel);
   OCNN_LAUNCH_OK("align_forward_ws");
   return OCNN_OK;
 }
@@ -413,7 +426,8 @@ int ocnn_align_backward(const float* top, int top_h, int channel, float* btm, in
     ocnn_stream_t stream) {
   OCNN_REQUIRE(top && btm && idx && top_h >= 0 && btm_h >= 0 && channel > 0, OCNN_E_BADARG, "bad argument");
   if (btm_h > 0)
-    align_backward_kernel<<<blocks_for(btm_h), kBlock, 0, as_stream(stream)>>>(top, top_h, btm, btm_h, idx, channel);
+    align_backward_kernel<<<dim3(blocks_for(btm_h), (channel + kAlignChunk - 1) / kAlignChunk), kBlock, 0,
+        as_stream(stream)>>>(top, top_h, btm, btm_h, idx, channel);
   OCNN_LAUNCH_OK("align_backward");
   return OCNN_OK;
 }
