@@ -461,12 +461,26 @@ __global__ __launch_bounds__(256) void conv_rows_bf16_kernel(ConvArgs a, uint16_
     if (n0 < a.N) store_tiles<uint16_t, MT>(a, out, acc, pass * MT, n0, lane);
   }
 }
-// A 16-byte store reads its four data registers for a while after it has issued, and the next
-// instruction that writes one of them has to keep two wait states' distance.  The compiler puts
-// them in when store and writer share a basic block; the row-major stores sit in conditional blocks
-// of their own, and the value computed for the next store landed in a register the store was
-// still reading (seen as a few wrong words per million).  So the wait goes in by hand.
-#define OCNN_STORE_DATA_WAIT() asm volatile("s_nop 1")
+// Every 16-byte store of the row-major epilogues goes through this one function.  At depth 9 a
+// few words per million outputs held the value computed for the NEXT store, different from run to
+// run, while these stores sat in conditional blocks of their own (channel piece inside the pitch or
+// not) with nothing between them and the next writer of their data registers; two wait states
+// behind each store cured it.  The cause is established by that experiment, not by a rule of the
+// instruction set that could be relied on elsewhere, so the cure is applied to every such store:
+//   * the store is unconditional: a piece outside the pitch (`inside` false, uniform) gets the
+//     out-of-range offset that columns behind the level use, and the hardware drops it, so no
+//     store stands alone in a block;
+//   * the wait states are tied to the store's data registers: the asm statement takes the four
+//     registers as read-write operands, so the register allocator keeps them (and nothing else
+//     in them) until the two wait states have passed.
+// tests/test_gpu_rows.py::test_rows_operators_full_size is the regression test (equal bits
+// over repeated runs at full size).
+typedef uint32_t store16_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void store16_then_wait(store16_t v, __amdgpu_buffer_rsrc_t buf, int voffset, int soffset,
+    bool inside) {
+  __builtin_amdgcn_raw_buffer_store_b128(v, buf, inside ? voffset : 0x7fffff00, soffset, 0);
+  asm volatile("s_nop 1" : "+v"(v) : : "memory");
+}
 
 // Row-major epilogue of the 32x32 accumulator tiles acc[MT][2] of a wavefront (columns n0 .. n0 + 63,
 // channels cb + 32 mt ..): lane (r, kh) holds channels cb + 32 mt + 8 q + 4 kh + e of its two
@@ -476,7 +490,6 @@ __global__ __launch_bounds__(256) void conv_rows_bf16_kernel(ConvArgs a, uint16_
 template <int MT>
 __device__ inline void rows_out_tiles(const ConvArgs& a, uint16_t* __restrict__ out, int out_pitch, int out_cpad,
     floatx16 (&acc)[MT][2], int cb, int n0, int lane) {
-  typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
   typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
   typedef float floatx2_t __attribute__((ext_vector_type(2)));
   const int r = lane & 31, kh = lane >> 5;
@@ -513,11 +526,8 @@ __device__ inline void rows_out_tiles(const ConvArgs& a, uint16_t* __restrict__ 
       for (int jj = 0; jj < 2; ++jj) {
         const auto s0 = __builtin_amdgcn_permlane32_swap(w[2 * jj][0], w[2 * jj + 1][0], false, false);
         const auto s1 = __builtin_amdgcn_permlane32_swap(w[2 * jj][1], w[2 * jj + 1][1], false, false);
-        if (cb + 32 * mt + 16 * jj < out_cpad) {
-          __builtin_amdgcn_raw_buffer_store_b128(u32x4_t{s0[0], s1[0], s0[1], s1[1]}, obuf, ooff,
-              (cb + 32 * mt + 16 * jj) * 2, 0);
-          OCNN_STORE_DATA_WAIT();
-        }
+        store16_then_wait(store16_t{s0[0], s1[0], s0[1], s1[1]}, obuf, ooff, (cb + 32 * mt + 16 * jj) * 2,
+            cb + 32 * mt + 16 * jj < out_cpad);
       }
     }
   }
@@ -1312,11 +1322,8 @@ __global__ __launch_bounds__(256, 1) void conv_s1_bf16_reg_kernel(ConvArgs a, ui
               const auto s1 = __builtin_amdgcn_permlane32_swap(w[2 * j][1], w[2 * j + 1][1], false, false);
               // channels cb + 32 mt + 16 j .. + 15 (8 in each lane of the pair): inside the pitch or not
               // for the whole wavefront
-              if (cb + 32 * mt + 16 * j < out_cpad) {
-                __builtin_amdgcn_raw_buffer_store_b128(u32x4{s0[0], s1[0], s0[1], s1[1]}, obuf, obase,
-                    (sb * out_pitch + 32 * mt + 16 * j) * 2, 0);
-                OCNN_STORE_DATA_WAIT();
-              }
+              store16_then_wait(store16_t{s0[0], s1[0], s0[1], s1[1]}, obuf, obase,
+                  (sb * out_pitch + 32 * mt + 16 * j) * 2, cb + 32 * mt + 16 * j < out_cpad);
             }
           }
       };
@@ -1697,11 +1704,8 @@ __global__ __launch_bounds__(256, 3) void conv_s2_rows_bf16_kernel(ConvArgs a, u
         for (int jj = 0; jj < 2; ++jj) {
           const auto s0 = __builtin_amdgcn_permlane32_swap(w[2 * jj][0], w[2 * jj + 1][0], false, false);
           const auto s1 = __builtin_amdgcn_permlane32_swap(w[2 * jj][1], w[2 * jj + 1][1], false, false);
-          if (cb + 32 * mt + 16 * jj < out_cpad) {
-            __builtin_amdgcn_raw_buffer_store_b128(u32x4{s0[0], s1[0], s0[1], s1[1]}, obuf, ooff[nt],
-                (cb + 32 * mt + 16 * jj) * 2, 0);
-            OCNN_STORE_DATA_WAIT();
-          }
+          store16_then_wait(store16_t{s0[0], s1[0], s0[1], s1[1]}, obuf, ooff[nt], (cb + 32 * mt + 16 * jj) * 2,
+              cb + 32 * mt + 16 * jj < out_cpad);
         }
       }
     }
@@ -2067,11 +2071,8 @@ __global__ __launch_bounds__(256) void deconv_s2_rows_bf16_kernel(ConvArgs a, ui
         for (int jj = 0; jj < 2; ++jj) {
           const auto s0 = __builtin_amdgcn_permlane32_swap(w[2 * jj][0], w[2 * jj + 1][0], false, false);
           const auto s1 = __builtin_amdgcn_permlane32_swap(w[2 * jj][1], w[2 * jj + 1][1], false, false);
-          if (cb + 16 * jj < out_cpad) {
-            __builtin_amdgcn_raw_buffer_store_b128(u32x4{s0[0], s1[0], s0[1], s1[1]}, obuf, ooff[nt],
-                (child * out_pitch + cb + 16 * jj) * 2, 0);
-            OCNN_STORE_DATA_WAIT();
-          }
+          store16_then_wait(store16_t{s0[0], s1[0], s0[1], s1[1]}, obuf, ooff[nt],
+              (child * out_pitch + cb + 16 * jj) * 2, cb + 16 * jj < out_cpad);
         }
       }
       if (tile == 0 && wave == 0 && child == 0 && lane * 8 >= cb && lane * 8 < min(cb + 32, out_cpad))

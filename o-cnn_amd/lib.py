@@ -33,6 +33,25 @@ class BuildParams(C.Structure):
 
 
 _lib = None
+_aten = None
+ATEN_PATH = os.path.join(HERE, "binding", "ocnn_aten.so")
+
+
+def aten():
+  """The ATen binding (binding/ocnn_aten.cpp built by binding/Makefile): the reference's operator
+  signatures over the same C interface, as a compiled Python module."""
+  global _aten
+  if _aten is None:
+    if not os.path.exists(ATEN_PATH):
+      raise ImportError("%s is missing: run `make -C o-cnn_amd/binding` (or __graft_entry__.build())" % ATEN_PATH)
+    import importlib.util
+    import torch  # noqa: F401  (the module links against PyTorch's libraries)
+    get()
+    spec = importlib.util.spec_from_file_location("ocnn_aten", ATEN_PATH)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    _aten = mod
+  return _aten
 
 
 def build():

@@ -169,20 +169,37 @@ def create_full_octree(depth, channel, batch_size=1, node_dis=True):
   return octree
 
 
+def predict_head(x, head, octree, depth):
+  """The prediction module of pytorch/ocnn/ounet.py:46-49: a 1x1x1 conv -> BN -> ReLU to the hidden
+  width and a 1x1x1 convolution with bias; head = ((w1, b1), (w2, b2)) with the BatchNorm folded
+  into (w1, b1).  Returns the logits [1, n_out, H, 1]."""
+  (w1, b1), (w2, b2) = head
+  hidden = conv_bn_relu(x, w1, b1, octree, depth, w1.shape[0], (1, 1, 1))
+  return conv_bn_relu(hidden, w2, b2, octree, depth, w2.shape[0], (1, 1, 1), relu=False)
+
+
 def completion_decoder(code, params, split_labels, depth, full_depth, batch_size=1, channel_out=4,
-                       signal=None):
-  """The shape-decoding loop of pytorch/ocnn/ounet.py:103-131 (`decode_shape`) without the skip
-  connections: starting from a full octree at `full_depth`, per depth a 2x2x2 stride-2
-  deconvolution up, a 3x3x3 convolution, the split decision, `octree_update` (child links from
+                       signal=None, skips=None, octree_in=None):
+  """The shape-decoding loop of pytorch/ocnn/ounet.py:72-131 (`ocnn_decoder` / `decode_shape`):
+  starting from a full octree at `full_depth`, per depth a 2x2x2 stride-2 deconvolution up, the
+  encoder's feature of that depth moved onto the growing octree (`octree_align`) and added, a
+  3x3x3 convolution, the split prediction (1x1x1 head -> argmax), `octree_update` (child links from
   the labels) and `octree_grow` (keys / children / neighbours of the next depth).
 
   code          features at full_depth, [1, C, batch*8^full_depth, 1]
-  params        {('up', d): (w, b), ('conv', d): (w, b)} for d in full_depth+1 .. depth
-  split_labels  {d: int32[H_d]}; label 1 = split.  A callable `f(d, features) -> labels` stands
-                for the reference's prediction head.
+  params        {('up', d): (w, b), ('conv', d): (w, b)} for d in full_depth+1 .. depth, and
+                optionally {('predict', d): ((w1, b1), (w2, b2))} for d in full_depth .. depth
+  split_labels  {d: int32[H_d]}; label 1 = split: the labels that decide the structure (the
+                ground truth's when training, ounet.py:89-90).  A callable `f(d, features) ->
+                labels` may stand for them; None takes the predicted labels (`decode_shape`,
+                ounet.py:118-119).  With a prediction head the logits and their argmax are
+                computed at every depth either way.
+  skips, octree_in  optional encoder features {d: [1, C_d, H_d(octree_in), 1]} and the octree
+                they live on (ounet.py:109-111)
   signal        optional callable `f(features) -> [1, channel_out, H_depth, 1]` written as the
                 finest-level feature of the result
-  Returns (octree, {d: features}).
+  Returns (octree, feats): feats[d] = decoder features, feats[('logit', d)] / feats[('label', d)]
+  = the head's output and its argmax (int32 [H_d]) where a head was given.
   """
   octree = create_full_octree(full_depth, channel_out, batch_size)
   feats = {full_depth: code}
@@ -190,9 +207,22 @@ def completion_decoder(code, params, split_labels, depth, full_depth, batch_size
     if d > full_depth:
       w, b = params[("up", d)]
       x = conv_bn_relu(feats[d - 1], w, b, octree, d - 1, w.shape[1] // 8, (2, 2, 2), 2, deconv=True)
+      if skips is not None and d in skips:
+        skip, _ = F.octree_align(skips[d], octree_in, octree, d)
+        x = x + skip
       w, b = params[("conv", d)]
       feats[d] = conv_bn_relu(x, w, b, octree, d, w.shape[0])
-    label = split_labels(d, feats[d]) if callable(split_labels) else split_labels[d]
+    predicted = None
+    if ("predict", d) in params:
+      logit = predict_head(feats[d], params[("predict", d)], octree, d)
+      predicted = logit.view(logit.shape[1], -1).argmax(0).to(torch.int32)
+      feats[("logit", d)], feats[("label", d)] = logit, predicted
+    if split_labels is None:
+      if predicted is None:
+        raise ValueError("no split labels and no prediction head at depth %d" % d)
+      label = predicted
+    else:
+      label = split_labels(d, feats[d]) if callable(split_labels) else split_labels[d]
     octree = F.octree_update(octree, label.to(torch.int32), d, 1)
     if d < depth:
       octree = F.octree_grow(octree, d + 1, False)
