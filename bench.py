@@ -512,8 +512,10 @@ def main():
     same = bool(torch.equal(graph_out, oc.stacks.lenet_trunk(oct6, 6, lp, data=feat6)))
     extra["lenet_trunk_batch32_d6_f32_graph"] = {"ms": t, "shapes_per_s": 32 / (t * 1e-3), "equals_eager": same}
     del graph, graph_out
-    # completion decoder loop (configs[4] shape): 16 octrees at depth 7 regrown from depth 2 with
-    # the split labels of the built batch, deconv up + 3x3x3 conv per depth, channels 256 -> 32
+    # completion decoder loop (configs[4] shape, pytorch/ocnn/ounet.py:72-131): 16 octrees at depth 7
+    # regrown from depth 2 with the split labels of the built batch; per depth a deconv up, the
+    # encoder's feature moved onto the growing octree (octree_align) and added, a 3x3x3 conv, the
+    # split head (1x1x1 -> 32 -> 2, argmax), octree_update and octree_grow; channels 256 -> 32
     dch = {2: 256, 3: 128, 4: 64, 5: 32, 6: 32, 7: 32}
     dspec = {}
     for d in range(3, 8):
@@ -523,7 +525,18 @@ def main():
     dlabels = {d: (F.octree_property(oct7, "child", d) >= 0).to(torch.int32) for d in range(2, 8)}
     code = torch.randn(1, 256, 16 * 64, 1, generator=g).to(dev)
     t = timed(lambda: oc.stacks.completion_decoder(code, dp, dlabels, 7, 2, batch_size=16), max(2, reps // 2), 1)
-    extra["completion_decoder_batch16_d7_f32"] = {"ms": t, "octants_d7": H7, "octrees_per_s": 16 / (t * 1e-3)}
+    extra["completion_decoder_batch16_d7_f32_plain"] = {"ms": t, "octants_d7": H7, "octrees_per_s": 16 / (t * 1e-3),
+                                                        "ops": "deconv, conv, update, grow (no skips, no heads)"}
+    heads = rand_params({("h1", d): (32, dch[d]) for d in range(2, 8)})
+    heads2 = rand_params({("h2", d): (2, 32) for d in range(2, 8)})
+    for d in range(2, 8):
+      dp[("predict", d)] = (heads[("h1", d)], heads2[("h2", d)])
+    i7 = F.octree_info(oct7)
+    dskips = {d: torch.randn(1, dch[d], i7.nnum(d), 1, generator=g).to(dev) for d in range(3, 8)}
+    t = timed(lambda: oc.stacks.completion_decoder(code, dp, dlabels, 7, 2, batch_size=16, skips=dskips, octree_in=oct7),
+              max(2, reps // 2), 1)
+    extra["completion_decoder_batch16_d7_f32"] = {"ms": t, "octants_d7": H7, "octrees_per_s": 16 / (t * 1e-3),
+                                                  "ops": "deconv, octree_align skip, conv, split head + argmax, update, grow"}
   out["extra"] = extra
 
   # ---- CPU baseline (reported, not the target) -----------------------------------------------

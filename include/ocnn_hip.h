@@ -97,7 +97,14 @@ int ocnn_make_ichild(int* ichild, int n_nempty, const int* child, int n_node, oc
  * (no atomics, same result on every run); the call first checks on the device that the
  * table maps back and forth consistently and otherwise scatter-adds as the reference
  * does, so any table gives the reference's result.  col2octreeP with stride 2 and a null
- * `ichild` always scatter-adds. */
+ * `ichild` always scatter-adds.
+ * With these plain signatures the verdict of the check travels from the check kernel to the
+ * summing kernels of the same call through one of 1024 words that the library holds per device,
+ * chosen by a per-call counter: calls on ONE stream never share a live word; calls that overlap on
+ * different streams share one only when 1024 or more col2octree calls were issued between them
+ * (then a call may sum by the other's verdict: still the reference's result for octree tables,
+ * wrong only if exactly one of the two tables is inconsistent).  ocnn_col2octree_cached below has
+ * no such bound: the word is the caller's. */
 int ocnn_octree2col(void* col, const void* data, int channel, int height, const int* kernel_size,
     int stride, const int* neigh, int height_col, int n, int dtype, ocnn_stream_t stream);
 int ocnn_col2octree(const void* col, void* data, int channel, int height, const int* kernel_size,
@@ -223,22 +230,37 @@ int ocnn_octree_conv_rows(void* top_rows, int top_pitch, const void* btm_rows, i
  * operator (links of `depth`; of depth+1 for the stride-2 deconvolution) and the all-nodes stride-2
  * deconvolution (links of `depth`) -- or NULL, then the call computes them into the workspace
  * (ocnn_conv_rows_shape bytes are enough).  With both, no workspace is needed and the call launches
- * the convolution kernel alone. */
+ * the convolution kernel alone.  `packed_bytes` must be what ocnn_conv_rows_packed_bytes returns for
+ * the very operator of the call (OCNN_E_WORKSPACE otherwise: a buffer packed for another shape). */
 int ocnn_conv_rows_packed_bytes(const void* info, int depth, int channel_in, int num_output, const int* kernel_size,
     int stride, int nempty, int is_deconv, int dtype, size_t* packed_bytes);
 int ocnn_conv_rows_pack(void* packed_dev, size_t packed_bytes, const void* weights, const void* octree_dev,
     const void* info, int depth, int channel_in, int num_output, const int* kernel_size, int stride, int nempty,
     int is_deconv, int dtype, ocnn_stream_t stream);
 int ocnn_octree_conv_rows_packed(void* top_rows, int top_pitch, const void* btm_rows, int btm_pitch, int channel_in,
-    int btm_h, const void* packed_weights, const int* ichild_dev, const float* bias, int relu, int is_deconv,
-    const void* octree_dev, const void* info, int depth, int num_output, const int* kernel_size, int stride, int nempty,
-    int dtype, void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream);
+    int btm_h, const void* packed_weights, size_t packed_bytes, const int* ichild_dev, const float* bias, int relu,
+    int is_deconv, const void* octree_dev, const void* info, int depth, int num_output, const int* kernel_size, int stride,
+    int nempty, int dtype, void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream);
 int ocnn_rows_from_channels(void* rows, int pitch, const void* data, int channel, int height, int dtype,
     ocnn_stream_t stream);
 int ocnn_channels_from_rows(void* data, const void* rows, int pitch, int channel, int height, int dtype,
     ocnn_stream_t stream);
 
-/* Tuning knob, no counterpart in the reference: 3x3x3 stride-1 bf16 convolutions over all nodes
+/* OctreeMaxPool on row-major activations (pytorch/ocnn/octree_pool.py:79-86: octree_max_pool at
+ * `depth` followed by octree_pad at depth-1; no row-major counterpart in the reference): rows of
+ * `depth` in, rows of ALL nodes of depth-1 out; a node with children takes the channel-wise
+ * maximum of their eight rows (the first maximum wins), a node without gets zeros; the zero row
+ * behind the last one and the padding channels are written.  mask_rows (may be NULL): int32
+ * [nnum(depth-1) + 1][top_pitch], the absolute row of each maximum, -1 for an empty node.
+ * Values and mask equal the channel-major pair bit for bit.  bf16; pitches as in
+ * ocnn_octree_conv_rows, so that a conv -> pool -> conv chain (pytorch/ocnn/lenet.py:24-32) stays
+ * in this layout. */
+int ocnn_octree_max_pool_rows(void* top_rows, int top_pitch, int* mask_rows, const void* btm_rows, int btm_pitch,
+    int channel, const void* octree_dev, const void* info, int depth, int dtype, ocnn_stream_t stream);
+
+/* Test hook and tuning knob, no counterpart in the reference (process-wide: a thread that flips it
+ * changes the kernel other threads' bf16 convolutions run from then on; their results do not
+ * change, only their timing): 3x3x3 stride-1 bf16 convolutions over all nodes
  * run one of two kernels, chosen by the number of 1024-column tiles of the level; the
  * register-fed kernel takes levels of at least `tiles` tiles (default 192, about 200 000
  * octants).  0 restores the default, a negative value sends every level to it (the tests use
@@ -444,6 +466,17 @@ int ocnn_points2octree(const void* const* points_dev, const void* const* points_
     int n_clouds, const ocnn_build_params* params, void* workspace_dev, size_t workspace_bytes,
     ocnn_alloc_fn alloc, void* alloc_ctx, void* info_out, void** octree_out_dev,
     ocnn_stream_t stream);
+
+/* Both steps in one call for a caller that obtains the blob's memory BEFORE its size is known (a
+ * guess from earlier builds of similar clouds): between the level scan and the emit launch the
+ * device then waits for the host's look at the node counts only, not for an allocation.  Plain
+ * octrees only (as ocnn_points2octree_plan).  OCNN_OK: the blob is the first
+ * ocnn_info_sizeof_octree(info_out) bytes of `octree_buf_dev`.  OCNN_E_WORKSPACE: `capacity` is too
+ * small; info_out is filled and the plan is kept, the caller allocates and calls
+ * ocnn_points2octree_emit.  No counterpart in the reference. */
+int ocnn_points2octree_into(const void* const* points_dev, const void* const* points_info, int n_clouds,
+    const ocnn_build_params* params, void* workspace_dev, size_t workspace_bytes, void* octree_buf_dev,
+    size_t capacity, void* info_out, ocnn_stream_t stream);
 
 /* ---- octree_scan, pytorch/cpp/transform_octree.cpp:5-22 over ScanOctree
  * (octree/octree/transform_octree.cpp:11-297): the part of a single octree that is visible

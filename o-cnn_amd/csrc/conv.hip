@@ -3338,10 +3338,17 @@ int ocnn_conv_rows_pack(void* packed_dev, size_t packed_bytes, const void* weigh
 }
 
 int ocnn_octree_conv_rows_packed(void* top_rows, int top_pitch, const void* btm_rows, int btm_pitch, int channel_in,
-    int btm_h, const void* packed_weights, const int* ichild_dev, const float* bias, int relu, int is_deconv,
-    const void* octree_dev, const void* info, int depth, int num_output, const int* kernel_size, int stride, int nempty,
-    int dtype, void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream) {
+    int btm_h, const void* packed_weights, size_t packed_bytes, const int* ichild_dev, const float* bias, int relu,
+    int is_deconv, const void* octree_dev, const void* info, int depth, int num_output, const int* kernel_size, int stride,
+    int nempty, int dtype, void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream) {
   OCNN_REQUIRE(packed_weights, OCNN_E_BADARG, "null pointer");
+  {   // a buffer packed for another operator has another size: refused, not read out of bounds
+    RowsPlan r;
+    int e = make_rows_plan(as_info(info), depth, channel_in, num_output, kernel_size, stride, nempty, is_deconv, dtype, &r);
+    if (e) return e;
+    OCNN_REQUIRE(packed_bytes == r.wt_bytes, OCNN_E_WORKSPACE,
+        "the packed weights hold %zu bytes, this operator reads %zu (packed for another shape?)", packed_bytes, (size_t)r.wt_bytes);
+  }
   return run_conv_rows(is_deconv ? 1 : 0, top_rows, top_pitch, btm_rows, btm_pitch, channel_in, btm_h, nullptr, bias,
       relu, octree_dev, info, depth, num_output, kernel_size, stride, nempty, dtype, workspace_dev, workspace_bytes,
       as_stream(stream), packed_weights, ichild_dev);

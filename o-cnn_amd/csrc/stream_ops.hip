@@ -814,6 +814,57 @@ __global__ void max_pool_kernel(T* __restrict__ top, int top_h, int* __restrict_
   mask[i] = 8 * h + arg;
 }
 
+// Row-major activations ([H + 1][pitch] bf16, row H zero): max pooling with the pad behind it.
+// Thread = (node p of the coarser level, 8-channel piece): the node's child link c names the rows
+// 8c .. 8c + 7 of the finer level; the eight 16-byte pieces are requested together, the maximum is
+// taken channel by channel in row order (the first maximum wins, as in max_pool_kernel), and an
+// empty node writes zeros.  Row `top_h` (what a missing neighbour reads) is written as zeros too.
+// mask (optional, [top_h + 1][pitch] int32): the absolute row of the maximum, -1 for an empty node.
+__global__ __launch_bounds__(kBlock) void max_pool_rows_kernel(uint16_t* __restrict__ top, int top_pitch,
+    int* __restrict__ mask, const uint16_t* __restrict__ btm, int btm_pitch, int pieces, const int* __restrict__ child,
+    int top_h, int btm_h) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int p = (int)(i / pieces), j = (int)(i % pieces);
+  if (p > top_h) return;
+  const int c = p < top_h ? child[p] : -1;
+  uint4 v[8];
+  if (c >= 0 && 8 * (int64_t)c + 7 < btm_h) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+      v[r] = *reinterpret_cast<const uint4*>(btm + (8 * (int64_t)c + r) * btm_pitch + 8 * j);
+  } else {
+#pragma unroll
+    for (int r = 0; r < 8; ++r) v[r] = make_uint4(0, 0, 0, 0);
+  }
+  uint16_t best[8];
+  int arg[8];
+  {
+    uint16_t h[8];
+    memcpy(h, &v[0], 16);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { best[e] = h[e]; arg[e] = 0; }
+  }
+#pragma unroll
+  for (int r = 1; r < 8; ++r) {
+    uint16_t h[8];
+    memcpy(h, &v[r], 16);
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      if (bf16_to_f32(h[e]) > bf16_to_f32(best[e])) { best[e] = h[e]; arg[e] = r; }
+  }
+  uint4 o;
+  memcpy(&o, best, 16);
+  *reinterpret_cast<uint4*>(top + (int64_t)p * top_pitch + 8 * j) = o;
+  if (mask) {
+    int m[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) m[e] = c >= 0 ? 8 * c + arg[e] : -1;
+    int4* dst = reinterpret_cast<int4*>(mask + (int64_t)p * top_pitch + 8 * j);
+    dst[0] = make_int4(m[0], m[1], m[2], m[3]);
+    dst[1] = make_int4(m[4], m[5], m[6], m[7]);
+  }
+}
+
 // Writes every row of the sibling group: the pooled value where the mask points,
 // zero elsewhere, so no separate zero fill is needed.  A mask that points outside
 // its own group (never produced by max_pool) is left to unpool_foreign_kernel.
@@ -1109,6 +1160,29 @@ int ocnn_octree_max_pool(void* top, int top_h, int* mask, const void* btm, int b
   else
     max_pool_kernel<uint16_t><<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)top, top_h, mask, (const uint16_t*)btm, btm_h, total);
   OCNN_LAUNCH_OK("max_pool");
+  return OCNN_OK;
+}
+
+int ocnn_octree_max_pool_rows(void* top_rows, int top_pitch, int* mask_rows, const void* btm_rows, int btm_pitch,
+    int channel, const void* octree_dev, const void* info, int depth, int dtype, ocnn_stream_t stream) {
+  OCNN_REQUIRE(top_rows && btm_rows && octree_dev && info, OCNN_E_BADARG, "null pointer");
+  OCNN_REQUIRE(dtype == OCNN_BF16, OCNN_E_UNSUPPORTED, "row-major activations: bf16");
+  const Info* o = as_info(info);
+  int e = ocnn_info_check(o);
+  if (e) return e;
+  OCNN_REQUIRE(depth > 1 && depth <= o->depth, OCNN_E_BADARG, "depth %d not in [2,%d]", depth, o->depth);
+  const int pitch = (channel + 15) / 16 * 16;
+  OCNN_REQUIRE(channel > 0 && top_pitch >= pitch && btm_pitch >= pitch && top_pitch % 8 == 0 && btm_pitch % 8 == 0,
+      OCNN_E_SHAPE, "pitches %d / %d for %d channels", top_pitch, btm_pitch, channel);
+  OCNN_REQUIRE(((reinterpret_cast<uintptr_t>(top_rows) | reinterpret_cast<uintptr_t>(btm_rows) |
+      reinterpret_cast<uintptr_t>(mask_rows)) & 15) == 0, OCNN_E_BADARG, "rows not 16-byte aligned");
+  const int top_h = o->nnum[depth - 1], btm_h = o->nnum[depth];
+  const int pieces = pitch / 8;
+  const int* child = reinterpret_cast<const int*>(static_cast<const char*>(octree_dev) + o->ptr_dis(OCNN_CHILD, depth - 1));
+  const int64_t total = ((int64_t)top_h + 1) * pieces;
+  max_pool_rows_kernel<<<blocks_for(total), kBlock, 0, as_stream(stream)>>>((uint16_t*)top_rows, top_pitch, mask_rows,
+      (const uint16_t*)btm_rows, btm_pitch, pieces, child, top_h, btm_h);
+  OCNN_LAUNCH_OK("max_pool_rows");
   return OCNN_OK;
 }
 

@@ -29,7 +29,7 @@ __all__ = [
     "octree_encode_key", "octree_decode_key", "octree_xyz2key", "octree_key2xyz",
     "octree_search_key", "octree_new", "octree_grow", "octree_update", "points_new",
     "octree_gather", "octree_gatherbk", "octree_mask", "octree_bilinear_neigh", "octree_bilinear_xyz",
-    "octree_info", "octree_scan", "octree_dropout", "octree_drop", "octree_samples",
+    "octree_info", "forget_cached", "octree_max_pool_rows", "octree_scan", "octree_dropout", "octree_drop", "octree_samples",
 ]
 
 
@@ -163,6 +163,8 @@ def _points_header(points):
 _ALLOC_FN = C.CFUNCTYPE(C.c_void_p, C.c_size_t, C.c_void_p)
 
 
+_blob_bytes_per_point = {}   # build settings -> bytes of blob per input point, from earlier builds
+
 _LANES = 4          # concurrent single-cloud builds: one per hardware queue of the process
 _lane_state = {}
 
@@ -240,6 +242,34 @@ def _build(points_list, merged, depth, full_depth, node_dis, node_feature, split
   dev_ptrs = (C.c_void_p * n)(*[p.data_ptr() for p in pts])
   hdr_ptrs = (C.c_void_p * n)(*[h.ctypes.data for h in hdrs])
   info_raw = np.zeros(INFO_BYTES, np.uint8)
+  if not (node_feature or adaptive):
+    # A plain octree: the blob's memory is obtained before the build, sized from the bytes per point
+    # that earlier builds with these settings took, so that the device does not sit idle while the
+    # interpreter allocates between the level scan and the emit step.  A guess that turns out too
+    # small costs one more allocation; the blob is a view of the (slightly larger) buffer.
+    key = (n, depth, full_depth, bool(node_dis), bool(split_label), bool(save_pts), bool(key2xyz), bool(merged),
+           hdrs[0][20:24].tobytes(), hdrs[0][24:56].tobytes())
+    ratio = _blob_bytes_per_point.get(key)
+    cap = int(ratio * total * 1.125) + (1 << 16) if ratio else 0
+    if cap:
+      buf = torch.empty(cap, dtype=torch.uint8, device=_dev())
+      rc = L.ocnn_points2octree_into(dev_ptrs, hdr_ptrs, n, C.byref(bp), C.c_void_p(base), C.c_size_t(ws_bytes),
+                                     _ptr(buf), C.c_size_t(cap), C.c_void_p(info_raw.ctypes.data), _stream())
+      if rc not in (0, -4):
+        _lib.check(rc)
+    else:
+      _lib.call("ocnn_points2octree_plan", dev_ptrs, hdr_ptrs, n, C.byref(bp), C.c_void_p(base),
+                C.c_size_t(ws_bytes), C.c_void_p(info_raw.ctypes.data), _stream())
+      rc = -4
+    info = _Info(info_raw)
+    size = info.size()
+    if rc == -4:
+      buf = torch.empty(size, dtype=torch.uint8, device=_dev())
+      _lib.call("ocnn_points2octree_emit", _ptr(buf), info.p, C.c_void_p(base), C.c_size_t(ws_bytes), _stream())
+    _blob_bytes_per_point[key] = max(size / max(total, 1), 0.9 * ratio if ratio else 0.0)
+    out = buf[:size]
+    out._ocnn_info = info
+    return out
   holder = []
 
   def alloc(nbytes, _ctx):
@@ -657,7 +687,9 @@ def col2octree(grad_in, octree, depth, kernel_size, stride, nempty):
   marks = getattr(octree, "_ocnn_col_marks", None)
   if marks is None:
     marks = octree._ocnn_col_marks = {}
-  key = (depth, tuple(ks), stride, bool(nempty), top_h)
+  # one word per (table, shape, version of the blob) AND stream: the first call on a stream checks
+  # the table on that stream, so no call reads a word whose check is still queued on another stream
+  key = (depth, tuple(ks), stride, bool(nempty), top_h, octree._version, torch.cuda.current_stream().cuda_stream)
   mark = marks.get(key)
   check_now = mark is None
   if check_now:
@@ -739,6 +771,15 @@ def octree_conv_fused(data_in, weights, bias, relu, octree, depth, num_output, k
                kernel_size, stride, nempty, bias=bias, relu=relu, out=out)
 
 
+def forget_cached(tensor):
+  """Drops what this module keeps with a tensor between calls: the packed weights of
+  octree_conv_rows(constant_weights=True), and for an octree blob the inverted child links, the
+  col2octree table verdicts and the host copy of the header.  For writes that the tensor's version
+  counter does not see."""
+  for name in ("_ocnn_rows_packed", "_ocnn_ichild", "_ocnn_col_marks", "_ocnn_info"):
+    tensor.__dict__.pop(name, None)
+
+
 def rows_pitch(channels):
   """channels per row of the row-major layout: padded to whole 16-channel steps"""
   return (int(channels) + 15) // 16 * 16
@@ -779,8 +820,11 @@ def octree_conv_rows(rows_in, channel_in, weights, octree, depth, num_output, bi
   With nempty=True the rows on both sides are the ranks of the non-empty nodes, as in the
   channel-major operators (3x3x3 stride 1 and 2x2x2 stride 2, conv and deconv).
   constant_weights=True (inference): the packed form of `weights` is kept with the tensor (and
-  packed again when the tensor is written to), the inverted child links with the octree, so that a
-  call launches the convolution kernel alone.
+  packed again when the tensor's version counter or address changes), the inverted child links
+  with the octree, so that a call launches the convolution kernel alone.  A write that bypasses
+  the version counter (`weights.data.copy_(...)`, a raw-pointer write into the octree) is not
+  seen: pass constant_weights=False then, or call forget_cached(weights) / forget_cached(octree)
+  after such a write.
   rows_in: [H + 1, rows_pitch(channel_in)] as to_rows makes it.  `out`: [top_h + 1, P] with
   P >= rows_pitch(num_output), or columns c0 .. c0 + rows_pitch(num_output) of such a tensor (a
   slice of what a later layer reads as a concatenation); returns `out`."""
@@ -813,18 +857,22 @@ def octree_conv_rows(rows_in, channel_in, weights, octree, depth, num_output, bi
     key = (channel_in, num_output, tuple(kernel_size), stride, bool(nempty), bool(deconv))
     cache = weights.__dict__.setdefault("_ocnn_rows_packed", {})
     ent = cache.get(key)
-    if ent is None or ent[0] != weights._version:
+    stamp = (weights._version, weights.data_ptr())
+    if ent is None or ent[0] != stamp:
       nbytes = C.c_size_t()
       _lib.call("ocnn_conv_rows_packed_bytes", info.p, depth, channel_in, num_output, ksc, stride, int(nempty),
                 int(deconv), dt, C.byref(nbytes))
       packed = torch.empty(nbytes.value, dtype=torch.uint8, device=weights.device)
       _lib.call("ocnn_conv_rows_pack", _ptr(packed), C.c_size_t(nbytes.value), _ptr(weights), _ptr(octree), info.p, depth,
                 channel_in, num_output, ksc, stride, int(nempty), int(deconv), dt, _stream())
-      ent = cache[key] = (weights._version, packed)
+      ent = cache[key] = (stamp, packed)
     links = None
     link_depth = depth + 1 if (deconv and stride == 2 and nempty) else depth
     if nempty or (deconv and stride == 2):
       links_of = octree.__dict__.setdefault("_ocnn_ichild", {})
+      if links_of.get("version") != octree._version:      # the blob was written to through torch
+        links_of.clear()
+        links_of["version"] = octree._version
       links = links_of.get(link_depth)
       if links is None:
         child = octree_property(octree, "child", link_depth).view(-1)
@@ -832,13 +880,31 @@ def octree_conv_rows(rows_in, channel_in, weights, octree, depth, num_output, bi
         _lib.call("ocnn_make_ichild", _ptr(links), info.nnum_nempty(link_depth), _ptr(child), child.numel(), _stream())
         links_of[link_depth] = links
     _lib.call("ocnn_octree_conv_rows_packed", _ptr(out), out.stride(0), _ptr(rows_in), rows_in.stride(0), channel_in,
-              btm_h, _ptr(ent[1]), _ptr(links), _ptr(bias), int(relu), int(deconv), _ptr(octree), info.p, depth,
+              btm_h, _ptr(ent[1]), C.c_size_t(ent[1].numel()), _ptr(links), _ptr(bias), int(relu), int(deconv), _ptr(octree), info.p, depth,
               num_output, ksc, stride, int(nempty), dt, C.c_void_p(base), C.c_size_t(ws_bytes.value), _stream())
     return out
   _lib.call("ocnn_octree_conv_rows", _ptr(out), out.stride(0), _ptr(rows_in), rows_in.stride(0), channel_in, btm_h,
             _ptr(weights), _ptr(bias), int(relu), int(deconv), _ptr(octree), info.p, depth, num_output, ksc, stride,
             int(nempty), dt, C.c_void_p(base), C.c_size_t(ws_bytes.value), _stream())
   return out
+
+
+def octree_max_pool_rows(rows_in, channels, octree, depth, return_mask=False):
+  """OctreeMaxPool (pytorch/ocnn/octree_pool.py:79-86: max_pool at `depth`, then pad at depth-1)
+  on row-major bf16 activations: [H_depth + 1, pitch] -> [H_{depth-1} + 1, pitch], empty nodes
+  zero; with return_mask also the int32 rows of the maxima ([H_{depth-1} + 1, pitch], -1 for an
+  empty node).  Bit-equal to the channel-major pair."""
+  octree = _to_dev(octree)
+  info = octree_info(octree)
+  if rows_in.dim() != 2 or rows_in.stride(1) != 1 or rows_in.size(0) != info.nnum(depth) + 1:
+    raise OcnnError(-3, "rows_in must be [%d, pitch] with unit channel stride" % (info.nnum(depth) + 1))
+  top_h = info.nnum(depth - 1)
+  pitch = rows_pitch(channels)
+  out = torch.empty(top_h + 1, pitch, dtype=rows_in.dtype, device=rows_in.device)
+  mask = torch.empty(top_h + 1, pitch, dtype=torch.int32, device=rows_in.device) if return_mask else None
+  _lib.call("ocnn_octree_max_pool_rows", _ptr(out), pitch, _ptr(mask), _ptr(rows_in), rows_in.stride(0), channels,
+            _ptr(octree), info.p, depth, _dtype_code(rows_in), _stream())
+  return (out, mask) if return_mask else out
 
 
 def _conv_grad(fn, is_deconv, data_in, weights, octree, grad_in, depth, num_output, kernel_size, stride,

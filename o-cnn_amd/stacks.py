@@ -6,6 +6,7 @@ affine map per output channel, so it folds into the weights and a bias; the fuse
 applies bias and ReLU to the accumulator before the store.
 
   lenet_trunk  conv -> BN -> ReLU -> max_pool (+pad) per depth, as pytorch/ocnn/lenet.py:24-32
+               (lenet_trunk_rows: the same in bf16 on row-major activations)
   unet_trunk   encoder / decoder with 2x2x2 stride-2 down-convolutions and deconvolutions and
                skip concatenations, the op order of pytorch/ocnn/unet.py:61-92 with one
                convolution per stage
@@ -62,6 +63,21 @@ def lenet_trunk(octree, depth, params, data=None, to_depth=2):
     pool, _ = F.octree_max_pool(data, octree, d)
     data = F.octree_pad(pool, octree, d - 1)
   return data
+
+
+def lenet_trunk_rows(octree, depth, params, data=None, to_depth=2, constant_weights=True):
+  """lenet_trunk in bf16 with row-major activations between the operators: the input is converted
+  once, every convolution and every pooling step (max_pool with the pad behind it) reads and
+  writes the layout the convolution kernels gather from, the result is converted back once."""
+  if data is None:
+    data = F.octree_property(octree, "feature", depth).bfloat16()
+  x, cin = F.to_rows(data), data.size(1)
+  for d in range(depth, to_depth, -1):
+    w, b = params[d]
+    x = F.octree_conv_rows(x, cin, w, octree, d, w.shape[0], bias=b, relu=True, constant_weights=constant_weights)
+    cin = w.shape[0]
+    x = F.octree_max_pool_rows(x, cin, octree, d)
+  return F.from_rows(x, cin)
 
 
 def unet_trunk(octree, depth, params, data=None, stages=3, nempty=False):

@@ -281,3 +281,74 @@ def test_packed_weights_and_cached_links(oc, octree):
           got = F.octree_conv_rows(x, 32, w, octree, depth, 48, constant_weights=True, **kw)
           assert torch.equal(got, exp), (nempty, ks, stride, deconv)
         w.mul_(1.5)        # a write to the tensor: the next call packs again
+
+
+def test_packed_weights_of_another_shape_are_refused(oc, octree):
+  """The packed form carries no shape: the call checks its byte count against the operator it is
+  asked to run, and a write that bypasses the version counter needs forget_cached."""
+  import ctypes as C
+  F = oc.nn
+  info = F.octree_info(octree)
+  H = info.nnum(6)
+  g = torch.Generator().manual_seed(78)
+  x = F.to_rows(torch.randn(1, 32, H, 1, generator=g).bfloat16().cuda())
+  w = (torch.randn(48, 32 * 27, generator=g) * 0.05).bfloat16().cuda()
+  F.octree_conv_rows(x, 32, w, octree, 6, 48, constant_weights=True)
+  (stamp, packed), = w._ocnn_rows_packed.values()
+  out = torch.empty(H + 1, 128, dtype=torch.bfloat16, device="cuda")
+  ks = (C.c_int * 3)(3, 3, 3)
+  P = lambda t: C.c_void_p(t.data_ptr())
+  args = lambda cout, nbytes: (P(out), 128, P(x), x.stride(0), 32, H, P(packed), C.c_size_t(nbytes), None, None, 0, 0,
+                               P(octree), info.p, 6, cout, ks, 1, 0, 1, None, C.c_size_t(0),
+                               C.c_void_p(torch.cuda.current_stream().cuda_stream))
+  L = oc.lib.get()
+  assert L.ocnn_octree_conv_rows_packed(*args(48, packed.numel())) == 0
+  assert L.ocnn_octree_conv_rows_packed(*args(128, packed.numel())) == -4       # packed for 48 output channels
+  assert L.ocnn_octree_conv_rows_packed(*args(48, packed.numel() - 16)) == -4
+  # a write through .data is invisible to the version counter: the stale pack is used until forgotten
+  exp_old = F.octree_conv_rows(x, 32, w, octree, 6, 48, constant_weights=True)
+  w.data.mul_(2.0)
+  assert w._version == stamp[0]
+  assert torch.equal(F.octree_conv_rows(x, 32, w, octree, 6, 48, constant_weights=True), exp_old)
+  F.forget_cached(w)
+  assert torch.equal(F.octree_conv_rows(x, 32, w, octree, 6, 48, constant_weights=True),
+                     F.octree_conv_rows(x, 32, w, octree, 6, 48))
+
+
+def test_max_pool_rows_equals_channel_major(oc, octree):
+  """max_pool + pad on row-major activations: values and mask bit-equal to the channel-major pair
+  (which the oracle checks in test_gpu_ops.py), zero row and padding channels written."""
+  F = oc.nn
+  info = F.octree_info(octree)
+  g = torch.Generator().manual_seed(91)
+  for depth in (6, 4, 3):
+    for c in (3, 16, 40, 64):
+      H, Hp = info.nnum(depth), info.nnum(depth - 1)
+      x = torch.randn(1, c, H, 1, generator=g).bfloat16().cuda()
+      x[0, :, 1::8] = x[0, :, 0::8]      # ties between siblings 0 and 1: the first maximum must win
+      top, mask = F.octree_max_pool(x, octree, depth)
+      exp = F.octree_pad(top, octree, depth - 1)
+      rows, mrows = F.octree_max_pool_rows(F.to_rows(x), c, octree, depth, return_mask=True)
+      assert rows.shape == (Hp + 1, F.rows_pitch(c))
+      assert torch.equal(F.from_rows(rows, c), exp), (depth, c)
+      assert not rows[Hp].any() and not rows[:, c:].any()
+      child = F.octree_property(octree, "child", depth - 1)
+      exp_mask = torch.full((c, Hp), -1, dtype=torch.int32, device="cuda")
+      exp_mask[:, child >= 0] = mask.view(c, -1)
+      assert torch.equal(mrows[:Hp, :c].t(), exp_mask), (depth, c)
+      assert torch.equal(F.octree_max_pool_rows(F.to_rows(x), c, octree, depth), rows)
+
+
+def test_lenet_trunk_rows(oc, octree):
+  """conv -> ReLU -> max_pool (+pad) from depth 6 down to depth 2 on row-major activations == the
+  channel-major bf16 trunk, bit for bit (same kernels, same operands, same order)."""
+  g = torch.Generator().manual_seed(92)
+  chans = {6: (3, 32), 5: (32, 64), 4: (64, 128), 3: (128, 256)}
+  params = {d: ((torch.randn(co, ci * 27, generator=g) / (ci * 27) ** 0.5).bfloat16().cuda(),
+                (torch.randn(co, generator=g) * 0.1).cuda()) for d, (ci, co) in chans.items()}
+  info = oc.nn.octree_info(octree)
+  x = torch.randn(1, 3, info.nnum(6), 1, generator=g).bfloat16().cuda()
+  exp = oc.stacks.lenet_trunk(octree, 6, params, data=x)
+  for cw in (False, True, True):
+    got = oc.stacks.lenet_trunk_rows(octree, 6, params, data=x, constant_weights=cw)
+    assert torch.equal(got, exp)

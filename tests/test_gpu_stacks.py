@@ -122,33 +122,53 @@ def test_unet_trunk(oc, orc, tree, nempty):
     mk(("up", d), (ch[d], ch[d + 1] * 8), ch[d])
     mk(("dec", d + 1), (ch[d + 1], 2 * ch[d + 1] * 27), 2 * ch[d + 1] * 27)
 
-  def cbr(x, key, d, ks, stride, deconv=False):
-    w, bias = P[key]
-    cout = w.shape[1] // 8 if deconv else w.shape[0]
-    if deconv and not nempty:
-      x = orc.depad(x, b.prop("child", d), int(b.nnum_nempty[d]))
-    fn = orc.octree_deconv if deconv else orc.octree_conv
-    y = fn(x, w, host, d, cout, ks, stride, nempty)
-    if (not deconv) and stride == 2 and not nempty:
-      y = orc.pad(y, b.prop("child", d - 1))          # conv -> pad -> BN -> ReLU
-    return np.maximum(y + bias[:, None], 0)
+  def chain(rnd):
+    """the operator sequence through the oracle; `rnd` rounds weights and every stored activation
+    (identity for fp32, round-to-bf16 for the bf16 trunks, which store bf16 between operators)"""
+    def cbr(x, key, d, ks, stride, deconv=False):
+      w, bias = P[key]
+      w = rnd(w)
+      cout = w.shape[1] // 8 if deconv else w.shape[0]
+      if deconv and not nempty:
+        x = orc.depad(x, b.prop("child", d), int(b.nnum_nempty[d]))
+      fn = orc.octree_deconv if deconv else orc.octree_conv
+      y = fn(x, w, host, d, cout, ks, stride, nempty)
+      if (not deconv) and stride == 2 and not nempty:
+        y = orc.pad(y, b.prop("child", d - 1))          # conv -> pad -> BN -> ReLU
+      return rnd(np.maximum(y + bias[:, None], 0))
 
-  x0 = b.prop("feature", 6).copy()
-  if nempty:
-    x0 = x0[:, b.prop("child", 6) >= 0]
-  feats = {6: cbr(x0, ("conv", 6), 6, [3, 3, 3], 1)}
-  d = 6
-  for _ in range(stages):
-    x = cbr(feats[d], ("down", d), d, [2, 2, 2], 2)
-    d -= 1
-    feats[d] = cbr(x, ("conv", d), d, [3, 3, 3], 1)
-  x = feats[d]
-  for _ in range(stages):
-    x = cbr(x, ("up", d), d, [2, 2, 2], 2, deconv=True)
-    d += 1
-    x = cbr(np.concatenate([feats[d], x], 0), ("dec", d), d, [3, 3, 3], 1)
+    x0 = rnd(b.prop("feature", 6).copy())
+    if nempty:
+      x0 = x0[:, b.prop("child", 6) >= 0]
+    feats = {6: cbr(x0, ("conv", 6), 6, [3, 3, 3], 1)}
+    d = 6
+    for _ in range(stages):
+      x = cbr(feats[d], ("down", d), d, [2, 2, 2], 2)
+      d -= 1
+      feats[d] = cbr(x, ("conv", d), d, [3, 3, 3], 1)
+    x = feats[d]
+    for _ in range(stages):
+      x = cbr(x, ("up", d), d, [2, 2, 2], 2, deconv=True)
+      d += 1
+      x = cbr(np.concatenate([feats[d], x], 0), ("dec", d), d, [3, 3, 3], 1)
+    return x
+
+  x = chain(lambda a: a)
   got = oc.stacks.unet_trunk(dev, 6, params, stages=stages, nempty=nempty)
   assert relerr(got.cpu().numpy().reshape(x.shape), x) < 1e-4
+  # bf16, channel-major and row-major between the operators, against the oracle chain that rounds
+  # what those trunks round (weights, input, every stored activation); what is left is the order
+  # of the fp32 sums and the occasional value that rounds the other way, far inside 2e-2
+  x16 = chain(lambda a: T(a).bfloat16().float().numpy())
+  p16 = {k: (w.bfloat16(), bias) for k, (w, bias) in params.items()}
+  data16 = T(b.prop("feature", 6)).cuda().view(1, 3, -1, 1).bfloat16()
+  if nempty:
+    data16 = oc.nn.octree_depad(data16, dev, 6)
+  got16 = oc.stacks.unet_trunk(dev, 6, p16, data=data16, stages=stages, nempty=nempty)
+  assert relerr(got16.float().cpu().numpy().reshape(x16.shape), x16) < 2e-2
+  rows16 = oc.stacks.unet_trunk_rows(dev, 6, p16, data=data16, stages=stages, nempty=nempty)
+  assert relerr(rows16.float().cpu().numpy().reshape(x16.shape), x16) < 2e-2
+  assert relerr(x16, x) < 2e-2          # and the rounded chain stays near the fp32 chain
 
 
 def test_column_modules(oc, orc, tree):
