@@ -86,6 +86,12 @@ int ocnn_pad_forward(void* Y, int Hy, int C, const void* X, int Hx, const int* l
     float dval, int dtype, ocnn_stream_t stream);
 int ocnn_pad_backward(void* X, int Hx, int C, const void* Y, int Hy, const int* label,
     int dtype, ocnn_stream_t stream);
+/* pad_forward with one value per channel for the rows without a source (`fill`: device, fp32 [C],
+ * rounded to `dtype`), no counterpart in the reference: what conv -> pad -> BatchNorm -> ReLU
+ * (pytorch/ocnn/octree_conv.py:102-113 inside pytorch/ocnn/modules.py:23-36) leaves in an empty node
+ * once the BatchNorm is folded into the convolution, relu(shift), in the same pass as the pad. */
+int ocnn_pad_forward_fill(void* Y, int Hy, int C, const void* X, int Hx, const int* label,
+    const float* fill, int dtype, ocnn_stream_t stream);
 /* int32 variant used to invert `children` into `ichild`
  * (pytorch/cpp/octree2col.cpp:10-20): ichild[child[h]] = h. */
 int ocnn_make_ichild(int* ichild, int n_nempty, const int* child, int n_node, ocnn_stream_t stream);

@@ -47,9 +47,10 @@ __device__ inline int line_rotation(const T* row) {  // elements up to the next 
   return (int)((0 - (reinterpret_cast<uintptr_t>(row) / sizeof(T))) & 63);
 }
 
+// fill: optional fp32 value per channel for the rows without a source (rounded to T), instead of dval
 template <typename T>
 __global__ void __launch_bounds__(kBlock) pad_forward_kernel(T* __restrict__ Y, int Hy, int C,
-    const T* __restrict__ X, int Hx, const int* __restrict__ label, T dval) {
+    const T* __restrict__ X, int Hx, const int* __restrict__ label, T dval, const float* __restrict__ fill) {
   __shared__ int s_l[kPadTile];
   const int tid = threadIdx.x;
   const int tile0 = blockIdx.x * kPadTile;
@@ -67,12 +68,17 @@ __global__ void __launch_bounds__(kBlock) pad_forward_kernel(T* __restrict__ Y, 
     const int rot = line_rotation(row);
     T v[kPadTile / kBlock];
     int at[kPadTile / kBlock];
+    T none = dval;
+    if (fill) {
+      if constexpr (sizeof(T) == 4) none = fill[c];
+      else none = f32_to_bf16(fill[c]);
+    }
 #pragma unroll
     for (int q = 0; q < kPadTile / kBlock; ++q) {
       const int r = (q * kBlock + tid + rot) & (kPadTile - 1);
       at[q] = r < rows ? r : -1;
       const int l = r < rows ? s_l[r] : -1;
-      v[q] = l < 0 ? dval : xin[l];
+      v[q] = l < 0 ? none : xin[l];
     }
 #pragma unroll
     for (int q = 0; q < kPadTile / kBlock; ++q)
@@ -1055,8 +1061,22 @@ using namespace ocnn;
 
 extern "C" {
 
+static int run_pad_forward(void* Y, int Hy, int C, const void* X, int Hx, const int* label, float dval,
+    const float* fill, int dtype, ocnn_stream_t stream);
+
 int ocnn_pad_forward(void* Y, int Hy, int C, const void* X, int Hx, const int* label, float dval,
     int dtype, ocnn_stream_t stream) {
+  return run_pad_forward(Y, Hy, C, X, Hx, label, dval, nullptr, dtype, stream);
+}
+
+int ocnn_pad_forward_fill(void* Y, int Hy, int C, const void* X, int Hx, const int* label, const float* fill,
+    int dtype, ocnn_stream_t stream) {
+  OCNN_REQUIRE(fill, OCNN_E_BADARG, "null pointer");
+  return run_pad_forward(Y, Hy, C, X, Hx, label, 0.0f, fill, dtype, stream);
+}
+
+static int run_pad_forward(void* Y, int Hy, int C, const void* X, int Hx, const int* label, float dval,
+    const float* fill, int dtype, ocnn_stream_t stream) {
   OCNN_REQUIRE(Y && label && (X || Hx == 0), OCNN_E_BADARG, "null pointer");
   OCNN_REQUIRE(Hy >= 0 && Hx >= 0 && C > 0, OCNN_E_BADARG, "Hy %d Hx %d C %d", Hy, Hx, C);
   if (Hy == 0) return OCNN_OK;
@@ -1066,14 +1086,14 @@ int ocnn_pad_forward(void* Y, int Hy, int C, const void* X, int Hx, const int* l
   dim3 grid(tiles, std::min<unsigned>(C, std::max(1u, 4096u / tiles)));
   hipStream_t s = as_stream(stream);
   if (dtype == OCNN_F32)
-    pad_forward_kernel<float><<<grid, kBlock, 0, s>>>((float*)Y, Hy, C, (const float*)X, Hx, label, dval);
+    pad_forward_kernel<float><<<grid, kBlock, 0, s>>>((float*)Y, Hy, C, (const float*)X, Hx, label, dval, fill);
   else if (dtype == OCNN_BF16) {
     // the pad value is rounded to bf16 on the host side of the launch
     uint32_t u;
     memcpy(&u, &dval, 4);
     u += 0x7fffu + ((u >> 16) & 1u);
     pad_forward_kernel<uint16_t><<<grid, kBlock, 0, s>>>((uint16_t*)Y, Hy, C, (const uint16_t*)X, Hx,
-        label, (uint16_t)(u >> 16));
+        label, (uint16_t)(u >> 16), fill);
   } else
     return fail(OCNN_E_BADARG, "dtype %d", dtype);
   OCNN_LAUNCH_OK("pad_forward");

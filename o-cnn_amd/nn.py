@@ -29,7 +29,7 @@ __all__ = [
     "octree_encode_key", "octree_decode_key", "octree_xyz2key", "octree_key2xyz",
     "octree_search_key", "octree_new", "octree_grow", "octree_update", "points_new",
     "octree_gather", "octree_gatherbk", "octree_mask", "octree_bilinear_neigh", "octree_bilinear_xyz",
-    "octree_info", "forget_cached", "octree_max_pool_rows", "octree_scan", "octree_dropout", "octree_drop", "octree_samples",
+    "octree_info", "octree_pad_fill", "forget_cached", "octree_max_pool_rows", "octree_scan", "octree_dropout", "octree_drop", "octree_samples",
 ]
 
 
@@ -969,6 +969,25 @@ def octree_pad(data_in, octree, depth, val=0.0):
   out = torch.empty(1, channel, top_h, 1, dtype=data_in.dtype, device=data_in.device)
   _lib.call("ocnn_pad_forward", _ptr(out), top_h, channel, _ptr(data_in), btm_h, _ptr(child),
             C.c_float(val), _dtype_code(data_in), _stream())
+  return out
+
+
+def octree_pad_fill(data_in, octree, depth, fill):
+  """octree_pad with one value per channel (`fill`, fp32 [C]) in the empty nodes instead of a scalar."""
+  octree = _to_dev(octree)
+  info = octree_info(octree)
+  data_in = data_in.contiguous()
+  channel, btm_h = data_in.size(1), data_in.size(2)
+  if btm_h != info.nnum_nempty(depth):
+    raise OcnnError(-3, "pad, d = %d, channel = %d: height %d != %d" % (depth, channel, btm_h, info.nnum_nempty(depth)))
+  fill = fill.to(torch.float32).contiguous()
+  if fill.numel() != channel:
+    raise OcnnError(-3, "fill needs one value per channel")
+  top_h = info.nnum(depth)
+  child = _prop_view(octree, info, CHILD, depth, top_h, torch.int32)
+  out = torch.empty(1, channel, top_h, 1, dtype=data_in.dtype, device=data_in.device)
+  _lib.call("ocnn_pad_forward_fill", _ptr(out), top_h, channel, _ptr(data_in), btm_h, _ptr(child), _ptr(fill),
+            _dtype_code(data_in), _stream())
   return out
 
 

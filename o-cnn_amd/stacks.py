@@ -44,11 +44,8 @@ def conv_bn_relu(data, w, b, octree, depth, cout, kernel_size=(3, 3, 3), stride=
     # a padded (empty) node holds 0 in the reference because the pad comes after conv but
     # before BatchNorm; after folding the empty nodes must receive relu(b) instead of 0:
     # the reference order is conv -> pad -> BN -> ReLU.
-    padded = F.octree_pad(out, octree, depth - 1, 0.0)
-    child = F.octree_property(octree, "child", depth - 1)
-    fill = torch.relu(b) if relu else b
-    empty = (child < 0).view(1, 1, -1, 1)
-    out = torch.where(empty, fill.to(out.dtype).view(1, -1, 1, 1), padded)
+    # (one pass: the pad writes the per-channel value where a node has no source row)
+    out = F.octree_pad_fill(out, octree, depth - 1, torch.relu(b) if relu else b)
   return out
 
 

@@ -638,3 +638,20 @@ def test_full_size_properties(oc, synthetic):
   assert down.shape[2] == info.nnum_nempty(8)
   up = oc.nn.octree_deconv(down, w2, octree, 8, C, [2, 2, 2], 2, False)
   assert up.shape[2] == H
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_pad_with_a_value_per_channel(oc, orc, tree, dtype):
+  """ocnn_pad_forward_fill: the oracle's pad where a node has a source row, the channel's own value
+  (rounded to the tensor's type) where it has none."""
+  b, dev = tree["blob"], tree["dev"]
+  rng = np.random.default_rng(17)
+  for d, Cc in ((5, 7), (4, 64), (3, 130)):
+    child = b.prop("child", d)
+    Hne = int(b.nnum_nempty[d])
+    x = T(rng.standard_normal((Cc, Hne)).astype(np.float32)).to(dtype)
+    fill = T(rng.standard_normal(Cc).astype(np.float32))
+    got = oc.nn.octree_pad_fill(x.cuda().view(1, Cc, Hne, 1), dev, d, fill.cuda())
+    exp = T(orc.pad(x.float().numpy(), child)).to(dtype)
+    exp[:, child < 0] = fill.to(dtype)[:, None]
+    assert got.dtype == dtype and torch.equal(got.cpu().view(Cc, -1), exp), (d, Cc)
