@@ -1761,6 +1761,32 @@ __device__ inline void store_children(const ConvArgs& a, OutT* __restrict__ out,
   }
 }
 
+// bf16: lane (n, kh) holds children 4kh .. 4kh + 3 (8 bytes) of four output channels.  The two
+// lanes of a parent swap halves (lanes 0-31 against 32-63) for a pair of channels, so that kh = 0
+// ends up with all eight children of the pair's first channel and kh = 1 with those of the second:
+// one 16-byte store a lane, 512 contiguous bytes per half wavefront, half the store instructions
+// and twice the bytes per request of the 8-byte form.
+__device__ inline void store_children_bf16(const ConvArgs& a, uint16_t* __restrict__ out, const floatx16& acc,
+    int row0, int n, int kh) {
+  if (n >= a.N) return;          // both lanes of a parent leave together
+  const int co0 = row0 >> 3;
+#pragma unroll
+  for (int qp = 0; qp < 2; ++qp) {
+    uint32_t w[2][2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int q = 2 * qp + h, co = min(co0 + q, a.M - 1);
+      w[h][0] = pack_bf16x2(finish(a, acc[4 * q], co), finish(a, acc[4 * q + 1], co));
+      w[h][1] = pack_bf16x2(finish(a, acc[4 * q + 2], co), finish(a, acc[4 * q + 3], co));
+    }
+    const auto s0 = __builtin_amdgcn_permlane32_swap(w[0][0], w[1][0], false, false);
+    const auto s1 = __builtin_amdgcn_permlane32_swap(w[0][1], w[1][1], false, false);
+    const int co = co0 + 2 * qp + kh;
+    if (co < a.M)
+      *reinterpret_cast<uint4*>(out + (int64_t)co * a.Hout + (int64_t)n * 8) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+  }
+}
+
 constexpr int kD2MT = 4;  // row tiles per pass: 128 rows = 16 output channels x 8 children
 
 // fp32: a wavefront keeps its 64 columns x 64 input channels in registers (read once, coalesced,
@@ -1893,7 +1919,7 @@ __global__ __launch_bounds__(256, 2) void deconv_s2_bf16_kernel(ConvArgs a, uint
 #pragma unroll
     for (int mt = 0; mt < kD2MT; ++mt)
 #pragma unroll
-      for (int nt = 0; nt < 2; ++nt) store_children<uint16_t>(a, out, acc[mt][nt], row_base + mt * 32, ncol[nt], kh);
+      for (int nt = 0; nt < 2; ++nt) store_children_bf16(a, out, acc[mt][nt], row_base + mt * 32, ncol[nt], kh);
   }
 }
 // The same for at most 64 input channels (KS k-steps of 16): a wavefront's 64 columns x all
@@ -1957,7 +1983,7 @@ __global__ __launch_bounds__(256, 2) void deconv_s2_bf16_reg_kernel(ConvArgs a, 
 #pragma unroll
       for (int mt = 0; mt < kD2MT; ++mt)
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) store_children<uint16_t>(a, out, acc[mt][nt], row_base + mt * 32, ncol[nt], kh);
+        for (int nt = 0; nt < 2; ++nt) store_children_bf16(a, out, acc[mt][nt], row_base + mt * 32, ncol[nt], kh);
     }
   }
 }
@@ -2342,6 +2368,8 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
         deconv_s2_bf16_reg_kernel<2><<<d_grid, 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles);
       else if (ksteps == 4)
         deconv_s2_bf16_reg_kernel<4><<<d_grid, 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles);
+      else if (ksteps == 8)
+        deconv_s2_bf16_reg_kernel<8><<<d_grid, 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles);
       else
         deconv_s2_bf16_kernel<<<dim3(d_grid, pass_split(d_tiles, (d.M * 8 + 32 * kD2MT - 1) / (32 * kD2MT))), 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles, cpad / 8);
     }

@@ -327,6 +327,28 @@ def test_deconv_vs_oracle(oc, orc, tree, ks, stride, nempty):
     assert relerr(got16.float().cpu().numpy().reshape(exp.shape), exp) < TOL_BF16
 
 
+@pytest.mark.parametrize("ci,co", [(16, 24), (32, 7), (64, 64), (128, 40), (120, 64), (48, 16), (256, 32)])
+def test_deconv_stride2_bf16_channel_widths(oc, orc, tree, ci, co):
+  """The 2x2x2 stride-2 bf16 deconvolution over all nodes picks its kernel by the number of
+  16-channel k-steps of the input (1, 2, 4, 8: columns held in registers; anything else: the
+  general form) and stores the eight children of a (parent, channel) pair as one 16-byte piece
+  after a swap between the two lanes of the parent: every width against the oracle, odd output
+  channel counts included, with and without bias + ReLU."""
+  b, dev, host = tree["blob"], tree["dev"], tree["host"]
+  rng = np.random.default_rng(100 + ci + co)
+  d = 4
+  hin = int(b.nnum_nempty[d])
+  x = T(rng.standard_normal((ci, hin)).astype(np.float32)).bfloat16()
+  w = T((rng.standard_normal((ci, co * 8)) * 0.1).astype(np.float32)).bfloat16()
+  bias = rng.standard_normal(co).astype(np.float32)
+  exp = orc.octree_deconv(x.float().numpy(), w.float().numpy(), host, d, co, [2, 2, 2], 2, False)
+  got = oc.nn.octree_deconv(x.cuda().view(1, ci, hin, 1), w.cuda(), dev, d, co, [2, 2, 2], 2, False)
+  assert relerr(got.float().cpu().numpy().reshape(exp.shape), exp) < TOL_BF16
+  gotf = oc.nn.octree_conv_fused(x.cuda().view(1, ci, hin, 1), w.cuda(), T(bias).cuda(), True, dev, d, co, [2, 2, 2], 2,
+                                 False, deconv=True)
+  assert relerr(gotf.float().cpu().numpy().reshape(exp.shape), np.maximum(exp + bias[:, None], 0)) < TOL_BF16
+
+
 def test_bf16_register_kernel_small_levels(oc, orc, tree):
   """The bf16 3x3x3 stride-1 kernel for large levels (operands straight into registers, 32
   sibling groups x 8 siblings per wavefront), forced onto small levels whose group counts are
