@@ -244,9 +244,24 @@ int ocnn_conv_rows_pack(void* packed_dev, size_t packed_bytes, const void* weigh
     const void* info, int depth, int channel_in, int num_output, const int* kernel_size, int stride, int nempty,
     int is_deconv, int dtype, ocnn_stream_t stream);
 int ocnn_octree_conv_rows_packed(void* top_rows, int top_pitch, const void* btm_rows, int btm_pitch, int channel_in,
-    int btm_h, const void* packed_weights, size_t packed_bytes, const int* ichild_dev, const float* bias, int relu,
-    int is_deconv, const void* octree_dev, const void* info, int depth, int num_output, const int* kernel_size, int stride,
-    int nempty, int dtype, void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream);
+    int btm_h, const void* packed_weights, size_t packed_bytes, const int* ichild_dev, const int* sources_dev,
+    const float* bias, int relu, int is_deconv, const void* octree_dev, const void* info, int depth, int num_output,
+    const int* kernel_size, int stride, int nempty, int dtype, void* workspace_dev, size_t workspace_bytes,
+    ocnn_stream_t stream);
+/* The nempty operators first look up, for every output column, the source row of each tap (through
+ * the neighbour table and the child links).  The result depends on the octree, the depth, the
+ * kernel shape, the stride and is_deconv only -- not on channels or weights -- so the layers of a
+ * network that work on one level share it: ocnn_conv_rows_sources writes that table
+ * (ocnn_conv_rows_sources_bytes bytes, int32; `ichild_dev` as above or NULL with a workspace of
+ * ocnn_conv_rows_shape bytes), and ocnn_octree_conv_rows_packed takes it as `sources_dev` (NULL:
+ * the call makes the table itself when the workspace has room for it, as ocnn_conv_rows_shape
+ * asks, and otherwise looks the rows up tile by tile inside the convolution kernel).  With a table
+ * the call needs no `ichild_dev`.  Same results in every case. */
+int ocnn_conv_rows_sources_bytes(const void* info, int depth, const int* kernel_size, int stride, int nempty,
+    int is_deconv, size_t* sources_bytes);
+int ocnn_conv_rows_sources(int* sources_dev, size_t sources_bytes, const int* ichild_dev, const void* octree_dev,
+    const void* info, int depth, const int* kernel_size, int stride, int nempty, int is_deconv, void* workspace_dev,
+    size_t workspace_bytes, ocnn_stream_t stream);
 int ocnn_rows_from_channels(void* rows, int pitch, const void* data, int channel, int height, int dtype,
     ocnn_stream_t stream);
 int ocnn_channels_from_rows(void* data, const void* rows, int pitch, int channel, int height, int dtype,
@@ -273,6 +288,14 @@ int ocnn_octree_max_pool_rows(void* top_rows, int top_pitch, int* mask_rows, con
  * that to run it on small octrees).  Returns the previous threshold.  Both kernels add the same
  * products in the same order: the results do not depend on the choice. */
 int ocnn_conv_bf16_tile_threshold(int tiles);
+
+/* Test hook, no counterpart in the reference (process-wide, like the knob above): the bf16 row
+ * kernels for tap sets of three taps or more exist in two forms that add the same products in the
+ * same order -- weights staged in LDS for all taps of a tile, or read per live tap straight from
+ * the packed weights (the default where it is faster: everywhere but the channel-major operators
+ * with whole blocks of 128 output channels).  0 sends every call to the staged form, 1 restores
+ * the default.  Returns the previous setting. */
+int ocnn_conv_rows_direct(int on);
 
 /* ocnn_octree_conv_fused for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the

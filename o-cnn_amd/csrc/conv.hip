@@ -39,6 +39,10 @@ struct ConvArgs {
   const int* ichild;
   const float* bias;    // optional per-output-channel bias (fp32), added before the store
   int relu;             // optional max(., 0) before the store
+  // optional: the source rows of every (tap, column), made ahead of the convolution by
+  // conv_sources_kernel: table[k * src_pitch + column] = row, -1 for none
+  const int* src_table = nullptr;
+  int src_pitch = 0;
 };
 
 // epilogue shared by every kernel: bias and ReLU are applied to the fp32 accumulator
@@ -225,6 +229,31 @@ __device__ inline void lookup_sources(const ConvArgs& a, int col, Put put) {
   }
 }
 
+// The source rows of all taps of all columns, one thread a column, into table[27][pitch].  Inside
+// a convolution kernel the look-up is two or three dependent trips to memory per tile in front of
+// everything else, run by the two or three workgroups that fit a compute unit beside their
+// accumulators (about 10 of the 40 microseconds a 256-column tile of a 64 -> 64 bf16 convolution over
+// the non-empty nodes lives); here it runs at full occupancy, and a caller that convolves the same
+// level again (the next layer of the same depth) keeps the table.
+__global__ __launch_bounds__(kBlock) void conv_sources_kernel(ConvArgs a, int* __restrict__ table, int pitch) {
+  const int col = blockIdx.x * kBlock + threadIdx.x;
+  if (col >= pitch) return;
+  lookup_sources(a, col, [&](int k, int row) { table[(int64_t)k * pitch + col] = row; });
+}
+// a tile's part of the table, or the look-up itself: put(k, row) for the 27 taps of column `col`
+template <class Put>
+__device__ inline void tile_sources(const ConvArgs& a, int col, Put put) {
+  if (a.src_table) {
+    int row[27];
+#pragma unroll
+    for (int k = 0; k < 27; ++k) row[k] = a.src_table[(int64_t)k * a.src_pitch + col];
+#pragma unroll
+    for (int k = 0; k < 27; ++k) put(k, row[k]);
+  } else {
+    lookup_sources(a, col, put);
+  }
+}
+
 template <int MT>
 __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* __restrict__ out,
     const float4* __restrict__ xt, const float* __restrict__ Wt, int n_tiles, int cpad) {
@@ -243,7 +272,7 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
   // source rows of all taps of the workgroup's 256 columns, looked up once and all together
   // (inside the tap loop a look-up is a chain of two or three trips to memory per tap)
   __shared__ int sSrc[27][kTileCols];
-  lookup_sources(a, tile * kTileCols + (int)threadIdx.x, [&](int k, int row) { sSrc[k][threadIdx.x] = row; });
+  tile_sources(a, tile * kTileCols + (int)threadIdx.x, [&](int k, int row) { sSrc[k][threadIdx.x] = row; });
   __syncthreads();
   for (int pass = blockIdx.y; pass < npass; pass += gridDim.y) {  // passes may be dealt out over workgroups
     floatx16 acc[MT][2];
@@ -574,7 +603,7 @@ __global__ __launch_bounds__(256, 2) void conv_rows_bf16_deep_kernel(ConvArgs a,
   const int cpad8 = in_pitch >> 3;   // 16-byte units per input row (the pitch; the channels read are below cpad)
   const int ngroup = (a.K + kG - 1) / kG;
   {
-    lookup_sources(a, tile * kTileCols + (int)threadIdx.x,
+    tile_sources(a, tile * kTileCols + (int)threadIdx.x,
         [&](int k, int row) { sSrc[k][threadIdx.x] = (row < 0 ? a.Hin : row) * cpad8; });
   }
   const int c0 = wave * kWaveCols + r;                  // my column of the first column tile, inside the workgroup's tile
@@ -671,6 +700,125 @@ __global__ __launch_bounds__(256, 2) void conv_rows_bf16_deep_kernel(ConvArgs a,
 #pragma unroll
           for (int v = 0; v < kWVec; ++v) sW[(g + 1) & 1][v * 256 + threadIdx.x] = wr[v];
         }
+      }
+    }
+    if constexpr (ROWS_OUT) {
+      rows_out_tiles<MT>(a, out, out_pitch, out_cpad, acc, pass * MT * 32, n0, lane);
+      if (tile == 0 && wave == 0 && lane * 8 >= pass * MT * 32 && lane * 8 < min((pass + 1) * MT * 32, out_cpad))
+        *reinterpret_cast<uint4*>(out + (int64_t)a.Hout * out_pitch + lane * 8) = make_uint4(0, 0, 0, 0);
+    } else {
+      if (n0 < a.N) store_tiles<uint16_t, MT>(a, out, acc, pass * MT, n0, lane);
+    }
+  }
+}
+
+// The same operator without LDS for the weights and without barriers: a wavefront reads the A
+// fragments of a tap straight from the packed weights (1 KiB coalesced per fragment, served by the
+// L1 / L2: the four wavefronts of a workgroup and the workgroups of a compute unit read the same
+// bytes) and only for the taps that are live for its own 64 columns.  Over the non-empty nodes of
+// a surface most (wavefront, tap) pairs are dead (12 of 27 taps live per 32 columns at depth 9 of
+// the scene), but the LDS-staged kernel moves the weights of all 27 taps through LDS for every
+// tile, 216 KiB for 64 -> 64, more than the rows it gathers, and synchronises its wavefronts nine
+// times a slab.  Here a wavefront walks its live taps in ascending order with the next live tap's
+// weights and rows in flight (two register sets), at its own pace.  Same products in the same order
+// as conv_rows_bf16_deep_kernel: the results are bit-identical.
+template <int MT, int SLAB, bool ROWS_OUT>
+__global__ __launch_bounds__(256, 2) void conv_rows_bf16_direct_kernel(ConvArgs a, uint16_t* __restrict__ out,
+    const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles, int cpad, int in_pitch, int out_pitch, int out_cpad) {
+  constexpr int kKs = SLAB / 16;                        // k-steps per slab
+  constexpr int kWUnits = kKs * MT * 64;                // 16-byte units of one (tap, slab)
+  __shared__ int sSrc[27][kTileCols];                   // source row of (tap, column), in 16-byte units of the copy
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = xcd_tile(blockIdx.x, n_tiles);
+  if (tile >= n_tiles) return;
+  const int n0 = tile * kTileCols + wave * kWaveCols;
+  const int r = lane & 31, kh = lane >> 5;
+  const int nslab = (cpad + SLAB - 1) / SLAB;
+  const int npass = (a.mtiles + MT - 1) / MT;
+  const int cpad8 = in_pitch >> 3;
+  tile_sources(a, tile * kTileCols + (int)threadIdx.x,
+      [&](int k, int row) { sSrc[k][threadIdx.x] = (row < 0 ? a.Hin : row) * cpad8; });
+  const int c0 = wave * kWaveCols + r;
+  union Frag { u32x4 q; bf16x8 v; };
+  unsigned live[2] = {0, 0};
+  __syncthreads();                                       // source rows written
+  {
+    const int none = a.Hin * cpad8;
+#pragma unroll
+    for (int k = 0; k < 27; ++k) {
+      if (k >= a.K) break;
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+        if (__ballot(sSrc[k][c0 + 32 * nt] != none) != 0) live[nt] |= 1u << k;
+    }
+    live[0] = __builtin_amdgcn_readfirstlane(live[0]);
+    live[1] = __builtin_amdgcn_readfirstlane(live[1]);
+  }
+  const unsigned live_any = live[0] | live[1];
+  for (int pass = blockIdx.y; pass < npass; pass += gridDim.y) {
+    floatx16 acc[MT][2];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
+    for (int slab = 0; slab < nslab; ++slab) {
+      const int nks = min(SLAB, cpad - slab * SLAB) >> 4;    // k-steps of this slab (uniform)
+      const int col16 = ((slab * SLAB) >> 3) + kh;               // my 16-byte unit inside a row
+      Frag wa[2][kKs][MT], x[2][kKs][2];                     // two register sets: [set][k-step][row tile / column tile]
+      auto fetch = [&](int tap, auto set) {
+        constexpr int S = decltype(set)::value;
+        if (tap < 0) return;                              // uniform
+        const u32x4* wsrc = Wt + (((int64_t)pass * a.K + tap) * nslab + slab) * kWUnits + lane;
+#pragma unroll
+        for (int ks = 0; ks < kKs; ++ks)
+          if (ks < nks) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) wa[S][ks][mt].q = wsrc[(ks * MT + mt) * 64];
+          }
+        const int s0 = sSrc[tap][c0], s1 = sSrc[tap][c0 + 32];
+        if ((live[0] >> tap) & 1) {                      // uniform over the wavefront
+#pragma unroll
+          for (int ks = 0; ks < kKs; ++ks)
+            if (ks < nks) x[S][ks][0].q = xt[(int64_t)s0 + col16 + 2 * ks];
+        }
+        if ((live[1] >> tap) & 1) {
+#pragma unroll
+          for (int ks = 0; ks < kKs; ++ks)
+            if (ks < nks) x[S][ks][1].q = xt[(int64_t)s1 + col16 + 2 * ks];
+        }
+      };
+      auto compute = [&](int tap, auto set) {
+        constexpr int S = decltype(set)::value;
+        const bool l0 = (live[0] >> tap) & 1, l1 = (live[1] >> tap) & 1;   // uniform over the wavefront
+#pragma unroll
+        for (int ks = 0; ks < kKs; ++ks) {
+          if (ks >= nks) continue;                       // uniform
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            if (l0) acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wa[S][ks][mt].v, x[S][ks][0].v, acc[mt][0], 0, 0, 0);
+            if (l1) acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wa[S][ks][mt].v, x[S][ks][1].v, acc[mt][1], 0, 0, 0);
+          }
+        }
+      };
+      unsigned todo = live_any;                          // live taps not yet requested (uniform)
+      auto next_tap = [&]() {
+        if (todo == 0) return -1;
+        const int t = __builtin_ctz(todo);
+        todo &= todo - 1;
+        return t;
+      };
+      int t0 = next_tap();
+      fetch(t0, std::integral_constant<int, 0>());
+      while (t0 >= 0) {
+        const int t1 = next_tap();
+        fetch(t1, std::integral_constant<int, 1>());
+        compute(t0, std::integral_constant<int, 0>());
+        if (t1 < 0) break;
+        t0 = next_tap();
+        fetch(t0, std::integral_constant<int, 0>());
+        compute(t1, std::integral_constant<int, 1>());
       }
     }
     if constexpr (ROWS_OUT) {
@@ -2145,6 +2293,7 @@ __global__ void ichild_kernel(int* __restrict__ ichild, int n_nempty, const int*
 // this many such tiles the LDS kernel (256 columns per workgroup, three workgroups per CU) fills
 // the device better.  Measured crossover on 256 CUs: between 110 and 215 tiles.
 std::atomic<int> g_bf16_reg_min_tiles{192};
+std::atomic<int> g_rows_direct{1};   // bf16 row kernels with three taps or more: 1 = weights straight from memory per live tap
 
 struct ConvPlan {
   int top_depth, workspace_depth, top_h, btm_h, workspace_h;
@@ -2153,6 +2302,8 @@ struct ConvPlan {
   KernelTaps taps;
   int mtiles, csteps;
   size_t wt_bytes, ichild_bytes, xt_bytes, xt_general, total_bytes;
+  size_t src_bytes;    // table of source rows (non-empty mode), behind everything else; optional
+  int src_pitch;
 };
 
 inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -2233,7 +2384,11 @@ int make_plan(const Info* o, int depth, int channel_in, int num_output, const in
     p->xt_bytes = align256(((size_t)p->btm_h + 1) * cpad * sizeof(uint16_t));
   }
   if (p->xt_general > p->xt_bytes) p->xt_bytes = p->xt_general;  // one buffer serves whichever path runs
-  p->total_bytes = p->wt_bytes + p->ichild_bytes + p->xt_bytes;
+  // non-empty mode: room for the table of source rows (27 taps x the column tiles), which the call
+  // then makes in a launch of its own at full occupancy instead of tile by tile inside the kernel
+  p->src_pitch = nempty ? (top_h + kTileCols - 1) / kTileCols * kTileCols : 0;
+  p->src_bytes = nempty ? align256(sizeof(int) * 27 * (size_t)p->src_pitch) : 0;
+  p->total_bytes = p->wt_bytes + p->ichild_bytes + p->xt_bytes + p->src_bytes;
   return OCNN_OK;
 }
 
@@ -2248,7 +2403,8 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
   if (e) return e;
   OCNN_REQUIRE(btm_h == p.btm_h, OCNN_E_SHAPE, "input height %d, the octree has %d rows at depth %d",
       btm_h, p.btm_h, depth);
-  OCNN_REQUIRE(ws && (builtin_scratch || ws_bytes >= p.total_bytes), OCNN_E_WORKSPACE,
+  // (the table of source rows is optional: a workspace without room for it still serves)
+  OCNN_REQUIRE(ws && (builtin_scratch || ws_bytes >= p.total_bytes - p.src_bytes), OCNN_E_WORKSPACE,
       "workspace %zu < %zu bytes", ws_bytes, p.total_bytes);
   OCNN_REQUIRE((reinterpret_cast<uintptr_t>(ws) & 15) == 0, OCNN_E_WORKSPACE, "workspace not 16-byte aligned");
 
@@ -2329,6 +2485,14 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     ichild_kernel<<<blocks_for(p.child_h), kBlock, 0, s>>>(ichild, p.ichild_h, a.child, p.child_h);
     OCNN_LAUNCH_OK("ichild");
     a.ichild = ichild;
+    const size_t before = p.wt_bytes + p.ichild_bytes + p.xt_bytes;
+    if ((path == kPathRowsBf16 || path == kPathRowsF32) && p.src_bytes > 0 && ws_bytes >= before + p.src_bytes) {
+      int* table = reinterpret_cast<int*>(wsb + before);
+      conv_sources_kernel<<<blocks_for(p.src_pitch), kBlock, 0, s>>>(a, table, p.src_pitch);
+      OCNN_LAUNCH_OK("conv_sources");
+      a.src_table = table;
+      a.src_pitch = p.src_pitch;
+    }
   }
   if (path == kPathS2Conv) {
     const int MT = a.mtiles == 1 ? 1 : 2;
@@ -2445,7 +2609,15 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     transpose_rows_bf16_kernel<<<tg, 256, 0, s>>>(xt, (const uint16_t*)btm, a.Cin, a.Hin, cpad);
     OCNN_LAUNCH_OK("transpose_rows");
     const dim3 rgrid(grid, pass_split(n_tiles, npass));
-    if (wide)
+    // (with whole blocks of 128 output channels and a channel-major store the staged kernel is ahead)
+    const bool direct = deep && !wide && g_rows_direct.load() != 0;
+    if (direct && wide)
+      conv_rows_bf16_direct_kernel<4, 32, false><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad, cpad, 0, 0);
+    else if (direct && MT == 1)
+      conv_rows_bf16_direct_kernel<1, kRowSlab, false><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad, cpad, 0, 0);
+    else if (direct)
+      conv_rows_bf16_direct_kernel<2, kRowSlab, false><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad, cpad, 0, 0);
+    else if (wide)
       conv_rows_bf16_deep_kernel<4, 32, false><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad, cpad, 0, 0);
     else if (deep && MT == 1)
       conv_rows_bf16_deep_kernel<1, kRowSlab, false><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad, cpad, 0, 0);
@@ -3012,7 +3184,8 @@ struct RowsPlan {
   int kind;            // 0: 3x3x3 s1, 1: 2x2x2 s2 conv, 2: 2x2x2 s2 deconv
   int btm_h, top_h, cols, cpad, out_cpad;
   int MT, npass, ksteps;
-  size_t wt_bytes, ichild_bytes, total_bytes;
+  size_t wt_bytes, ichild_bytes, src_bytes, total_bytes;
+  int src_pitch;       // columns of the source table (kind 3): the column tiles, whole
 };
 int make_rows_plan(const Info* o, int depth, int channel_in, int num_output, const int* ks, int stride, int nempty,
     int deconv, int dtype, RowsPlan* r) {
@@ -3029,6 +3202,8 @@ int make_rows_plan(const Info* o, int depth, int channel_in, int num_output, con
   r->out_cpad = (num_output + 15) / 16 * 16;
   r->ksteps = r->cpad / 16;
   r->ichild_bytes = 0;
+  r->src_bytes = 0;
+  r->src_pitch = 0;
   const int mtiles = (num_output + 31) / 32;
   if (nempty) {
     // over the non-empty nodes: the general row kernel (rows = ranks of the non-empty nodes on
@@ -3050,6 +3225,8 @@ int make_rows_plan(const Info* o, int depth, int channel_in, int num_output, con
       r->wt_bytes = align256((size_t)r->npass * p.taps.count * nslab * (slab_ch / 16) * r->MT * 64 * 16);
     }
     r->ichild_bytes = p.ichild_bytes;
+    r->src_pitch = (r->cols + kTileCols - 1) / kTileCols * kTileCols;
+    r->src_bytes = align256(sizeof(int) * 27 * (size_t)(r->src_pitch > 0 ? r->src_pitch : kTileCols));
   } else if (stride == 1 && k333) {
     r->kind = 0;
     r->btm_h = r->top_h = r->cols = o->nnum[depth];
@@ -3078,7 +3255,7 @@ int make_rows_plan(const Info* o, int depth, int channel_in, int num_output, con
   } else {
     return fail(OCNN_E_UNSUPPORTED, "row-major operators: 3x3x3 stride 1, 2x2x2 stride 2");
   }
-  r->total_bytes = r->wt_bytes + r->ichild_bytes;
+  r->total_bytes = r->wt_bytes + r->ichild_bytes + r->src_bytes;
   return OCNN_OK;
 }
 
@@ -3089,20 +3266,23 @@ int make_rows_plan(const Info* o, int depth, int channel_in, int num_output, con
 int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_rows, int btm_pitch, int channel_in,
     int btm_h, const void* weights, const float* bias, int relu, const void* octree_dev, const void* info,
     int depth, int num_output, const int* ks, int stride, int nempty, int dtype, void* ws, size_t ws_bytes,
-    hipStream_t s, const void* packed = nullptr, const int* ichild_in = nullptr, bool only_pack = false) {
-  OCNN_REQUIRE((only_pack || (top_rows && btm_rows)) && (weights || packed) && octree_dev && info && ks,
-      OCNN_E_BADARG, "null pointer");
+    hipStream_t s, const void* packed = nullptr, const int* ichild_in = nullptr, bool only_pack = false,
+    const int* sources_in = nullptr, int* sources_out = nullptr) {
+  OCNN_REQUIRE((only_pack || sources_out || (top_rows && btm_rows)) && (weights || packed || sources_out) && octree_dev &&
+      info && ks, OCNN_E_BADARG, "null pointer");
   const Info* o = as_info(info);
   RowsPlan r;
   int e = make_rows_plan(o, depth, channel_in, num_output, ks, stride, nempty, deconv, dtype, &r);
   if (e) return e;
-  const bool need_links = r.ichild_bytes > 0 && !ichild_in && !only_pack;
-  const size_t ws_need = (packed ? 0 : r.wt_bytes) + (need_links ? r.ichild_bytes : 0);
+  // the inverted child links serve the look-up of the source rows only: a caller that brings the
+  // table of sources needs none
+  const bool need_links = r.ichild_bytes > 0 && !ichild_in && !only_pack && !(sources_in && r.kind == 3);
+  const size_t ws_need = (packed || sources_out ? 0 : r.wt_bytes) + (need_links ? r.ichild_bytes : 0);
   OCNN_REQUIRE(ws_need == 0 || (ws && ws_bytes >= ws_need), OCNN_E_WORKSPACE, "workspace %zu < %zu bytes", ws_bytes, ws_need);
   OCNN_REQUIRE(ws_need == 0 || (reinterpret_cast<uintptr_t>(ws) & 15) == 0, OCNN_E_WORKSPACE, "workspace not 16-byte aligned");
   OCNN_REQUIRE(!packed || (reinterpret_cast<uintptr_t>(packed) & 15) == 0, OCNN_E_BADARG, "packed weights not 16-byte aligned");
   char* wsb = static_cast<char*>(ws);
-  if (!packed) {   // the weights in the order the kernel of this operator reads them
+  if (!packed && !sources_out) {   // the weights in the order the kernel of this operator reads them
     const int mtiles_w = (num_output + 31) / 32;
     if (r.kind == 0) {
       const int64_t sm = deconv ? 27 : (int64_t)channel_in * 27, sc = deconv ? (int64_t)num_output * 27 : 27;
@@ -3131,8 +3311,8 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
     if (only_pack) return OCNN_OK;
   }
   const void* wpk = packed ? packed : ws;
-  int* links_ws = reinterpret_cast<int*>(wsb + (packed ? 0 : r.wt_bytes));
-  OCNN_REQUIRE(btm_h == r.btm_h, OCNN_E_SHAPE, "input height %d, the octree has %d rows at depth %d", btm_h,
+  int* links_ws = reinterpret_cast<int*>(wsb + (packed || sources_out ? 0 : r.wt_bytes));
+  OCNN_REQUIRE(sources_out || btm_h == r.btm_h, OCNN_E_SHAPE, "input height %d, the octree has %d rows at depth %d", btm_h,
       r.btm_h, depth);
   // the stride-2 convolution also reads a channel slice of a wider tensor (an encoder feature that
   // sits in the tensor the decoder reads as a concatenation)
@@ -3182,13 +3362,40 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
     a.child = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_CHILD, p.workspace_depth));
     if (ichild_in) {
       a.ichild = ichild_in;
-    } else {
+    } else if (need_links) {
       ichild_kernel<<<blocks_for(p.child_h), kBlock, 0, s>>>(links_ws, p.ichild_h, a.child, p.child_h);
       a.ichild = links_ws;
     }
+    // the source rows of every (tap, column): the caller's table, or one made now when the
+    // workspace has room for it (ocnn_conv_rows_shape asks for that room), or looked up per tile
+    if (sources_out) {
+      a.Hin = r.btm_h;
+      conv_sources_kernel<<<blocks_for(r.src_pitch), kBlock, 0, s>>>(a, sources_out, r.src_pitch);
+      OCNN_LAUNCH_OK("conv_sources");
+      return OCNN_OK;
+    }
+    if (sources_in) {
+      a.src_table = sources_in;
+      a.src_pitch = r.src_pitch;
+    } else if (ws && ws_bytes >= ws_need + r.src_bytes) {
+      int* table = reinterpret_cast<int*>(wsb + ws_need);
+      conv_sources_kernel<<<blocks_for(r.src_pitch), kBlock, 0, s>>>(a, table, r.src_pitch);
+      a.src_table = table;
+      a.src_pitch = r.src_pitch;
+    }
     const int n_tiles = (a.N + kTileCols - 1) / kTileCols;
     const dim3 grid(((n_tiles + 7) / 8) * 8, pass_split(n_tiles, r.npass));
-    if (r.MT == 4)
+    const bool direct = a.K >= 3 && g_rows_direct.load() != 0;
+    if (direct && r.MT == 4)
+      conv_rows_bf16_direct_kernel<4, 32, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
+          (const u32x4*)wpk, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
+    else if (direct && r.MT == 2)
+      conv_rows_bf16_direct_kernel<2, kRowSlab, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
+          (const u32x4*)wpk, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
+    else if (direct)
+      conv_rows_bf16_direct_kernel<1, kRowSlab, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
+          (const u32x4*)wpk, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
+    else if (r.MT == 4)
       conv_rows_bf16_deep_kernel<4, 32, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
           (const u32x4*)wpk, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
     else if (r.MT == 2)
@@ -3287,6 +3494,8 @@ int ocnn_octree_conv_static(void* top, const void* btm, int channel_in, int btm_
       kernel_size, stride, nempty, dtype, ptr, kBuiltinScratchBytes, as_stream(stream), bias, relu, true);
 }
 
+int ocnn_conv_rows_direct(int on) { return g_rows_direct.exchange(on ? 1 : 0); }
+
 int ocnn_conv_bf16_tile_threshold(int tiles) {
   const int old = g_bf16_reg_min_tiles.load();
   g_bf16_reg_min_tiles.store(tiles > 0 ? tiles : (tiles == 0 ? 192 : 1));
@@ -3365,10 +3574,35 @@ int ocnn_conv_rows_pack(void* packed_dev, size_t packed_bytes, const void* weigh
       true);
 }
 
+int ocnn_conv_rows_sources_bytes(const void* info, int depth, const int* kernel_size, int stride, int nempty,
+    int is_deconv, size_t* sources_bytes) {
+  RowsPlan r;
+  int e = make_rows_plan(as_info(info), depth, 16, 16, kernel_size, stride, nempty, is_deconv, OCNN_BF16, &r);
+  if (e) return e;
+  if (sources_bytes) *sources_bytes = r.src_bytes;
+  return OCNN_OK;
+}
+
+int ocnn_conv_rows_sources(int* sources_dev, size_t sources_bytes, const int* ichild_dev, const void* octree_dev,
+    const void* info, int depth, const int* kernel_size, int stride, int nempty, int is_deconv, void* workspace_dev,
+    size_t workspace_bytes, ocnn_stream_t stream) {
+  OCNN_REQUIRE(sources_dev, OCNN_E_BADARG, "null pointer");
+  RowsPlan r;
+  int e = make_rows_plan(as_info(info), depth, 16, 16, kernel_size, stride, nempty, is_deconv, OCNN_BF16, &r);
+  if (e) return e;
+  OCNN_REQUIRE(r.src_bytes > 0, OCNN_E_UNSUPPORTED, "this operator looks no source rows up (nempty operators do)");
+  OCNN_REQUIRE(sources_bytes >= r.src_bytes, OCNN_E_WORKSPACE, "the table takes %zu bytes, the buffer holds %zu",
+      (size_t)r.src_bytes, sources_bytes);
+  return run_conv_rows(is_deconv ? 1 : 0, nullptr, 16, nullptr, 16, 16, r.btm_h, nullptr, nullptr, 0, octree_dev, info,
+      depth, 16, kernel_size, stride, nempty, OCNN_BF16, workspace_dev, workspace_bytes, as_stream(stream), nullptr,
+      ichild_dev, false, nullptr, sources_dev);   // (pitches of 16 channels: only the look-up runs)
+}
+
 int ocnn_octree_conv_rows_packed(void* top_rows, int top_pitch, const void* btm_rows, int btm_pitch, int channel_in,
-    int btm_h, const void* packed_weights, size_t packed_bytes, const int* ichild_dev, const float* bias, int relu,
-    int is_deconv, const void* octree_dev, const void* info, int depth, int num_output, const int* kernel_size, int stride,
-    int nempty, int dtype, void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream) {
+    int btm_h, const void* packed_weights, size_t packed_bytes, const int* ichild_dev, const int* sources_dev,
+    const float* bias, int relu, int is_deconv, const void* octree_dev, const void* info, int depth, int num_output,
+    const int* kernel_size, int stride, int nempty, int dtype, void* workspace_dev, size_t workspace_bytes,
+    ocnn_stream_t stream) {
   OCNN_REQUIRE(packed_weights, OCNN_E_BADARG, "null pointer");
   {   // a buffer packed for another operator has another size: refused, not read out of bounds
     RowsPlan r;
@@ -3379,7 +3613,7 @@ int ocnn_octree_conv_rows_packed(void* top_rows, int top_pitch, const void* btm_
   }
   return run_conv_rows(is_deconv ? 1 : 0, top_rows, top_pitch, btm_rows, btm_pitch, channel_in, btm_h, nullptr, bias,
       relu, octree_dev, info, depth, num_output, kernel_size, stride, nempty, dtype, workspace_dev, workspace_bytes,
-      as_stream(stream), packed_weights, ichild_dev);
+      as_stream(stream), packed_weights, ichild_dev, false, sources_dev);
 }
 
 int ocnn_rows_from_channels(void* rows, int pitch, const void* data, int channel, int height, int dtype,

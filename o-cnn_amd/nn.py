@@ -776,7 +776,7 @@ def forget_cached(tensor):
   octree_conv_rows(constant_weights=True), and for an octree blob the inverted child links, the
   col2octree table verdicts and the host copy of the header.  For writes that the tensor's version
   counter does not see."""
-  for name in ("_ocnn_rows_packed", "_ocnn_ichild", "_ocnn_col_marks", "_ocnn_info"):
+  for name in ("_ocnn_rows_packed", "_ocnn_ichild", "_ocnn_sources", "_ocnn_col_marks", "_ocnn_info"):
     tensor.__dict__.pop(name, None)
 
 
@@ -867,8 +867,25 @@ def octree_conv_rows(rows_in, channel_in, weights, octree, depth, num_output, bi
                 channel_in, num_output, ksc, stride, int(nempty), int(deconv), dt, _stream())
       ent = cache[key] = (stamp, packed)
     links = None
+    sources = None
     link_depth = depth + 1 if (deconv and stride == 2 and nempty) else depth
-    if nempty or (deconv and stride == 2):
+    if nempty:
+      # the source row of every (tap, column): the same for every layer on this level with this
+      # kernel shape, kept with the octree
+      tables = octree.__dict__.setdefault("_ocnn_sources", {})
+      if tables.get("version") != octree._version:
+        tables.clear()
+        tables["version"] = octree._version
+      skey = (depth, tuple(kernel_size), stride, bool(deconv))
+      sources = tables.get(skey)
+      if sources is None:
+        nb = C.c_size_t()
+        _lib.call("ocnn_conv_rows_sources_bytes", info.p, depth, ksc, stride, 1, int(deconv), C.byref(nb))
+        sources = torch.empty(nb.value // 4, dtype=torch.int32, device=octree.device)
+        _lib.call("ocnn_conv_rows_sources", _ptr(sources), C.c_size_t(nb.value), None, _ptr(octree), info.p, depth, ksc,
+                  stride, 1, int(deconv), C.c_void_p(base), C.c_size_t(ws_bytes.value), _stream())
+        tables[skey] = sources
+    elif deconv and stride == 2:
       links_of = octree.__dict__.setdefault("_ocnn_ichild", {})
       if links_of.get("version") != octree._version:      # the blob was written to through torch
         links_of.clear()
@@ -880,7 +897,7 @@ def octree_conv_rows(rows_in, channel_in, weights, octree, depth, num_output, bi
         _lib.call("ocnn_make_ichild", _ptr(links), info.nnum_nempty(link_depth), _ptr(child), child.numel(), _stream())
         links_of[link_depth] = links
     _lib.call("ocnn_octree_conv_rows_packed", _ptr(out), out.stride(0), _ptr(rows_in), rows_in.stride(0), channel_in,
-              btm_h, _ptr(ent[1]), C.c_size_t(ent[1].numel()), _ptr(links), _ptr(bias), int(relu), int(deconv), _ptr(octree), info.p, depth,
+              btm_h, _ptr(ent[1]), C.c_size_t(ent[1].numel()), _ptr(links), _ptr(sources), _ptr(bias), int(relu), int(deconv), _ptr(octree), info.p, depth,
               num_output, ksc, stride, int(nempty), dt, C.c_void_p(base), C.c_size_t(ws_bytes.value), _stream())
     return out
   _lib.call("ocnn_octree_conv_rows", _ptr(out), out.stride(0), _ptr(rows_in), rows_in.stride(0), channel_in, btm_h,
