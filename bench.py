@@ -236,6 +236,15 @@ def main():
     extra["conv333_s1_d9_bf16_nempty_rows"] = {"ms": t, "octants_per_s": Hne9 / (t * 1e-3), "tflops": fl / (t * 1e-3) / 1e12,
                                                "frac_mfma_peak": fl / (t * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS["bf16"],
                                                "layout": "row-major in and out, no copy; flops counted densely (27 taps a column)"}
+    # the same as a layer of a network at inference sees it: the weights packed once, the table of
+    # source rows of this level (octree, depth and kernel shape only) made once and kept
+    t = timed(lambda: F.octree_conv_rows(rows_ne, C, w16, octree, 9, C, out=rows_ne_out, nempty=True,
+                                         constant_weights=True), reps, wu)
+    extra["conv333_s1_d9_bf16_nempty_rows_kept_tables"] = {
+        "ms": t, "octants_per_s": Hne9 / (t * 1e-3), "tflops": fl / (t * 1e-3) / 1e12,
+        "frac_mfma_peak": fl / (t * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS["bf16"],
+        "layout": "row-major in and out; packed weights and the level's source rows kept between calls; "
+                  "flops counted densely (27 taps a column)"}
     del rows_ne, rows_ne_out
     x8 = torch.randn(1, C, Hne8, 1, generator=g).to(dev)
     conv_case("deconv222_s2_d8to9_f32", octree, 8, x8, w2, [2, 2, 2], 2, deconv=True)
@@ -495,6 +504,13 @@ def main():
               (torch.randn(co, generator=g) * 0.1).to(dev)) for d, (ci, co) in lch.items()}
     t = timed(lambda: oc.stacks.lenet_trunk(oct6, 6, lp), reps, wu)
     extra["lenet_trunk_batch32_d6_f32"] = {"ms": t, "shapes_per_s": 32 / (t * 1e-3)}
+    lp16 = {d: (w.bfloat16(), b) for d, (w, b) in lp.items()}
+    feat6_16 = F.octree_property(oct6, "feature", 6).bfloat16()
+    t = timed(lambda: oc.stacks.lenet_trunk(oct6, 6, lp16, data=feat6_16), reps, wu)
+    extra["lenet_trunk_batch32_d6_bf16"] = {"ms": t, "shapes_per_s": 32 / (t * 1e-3)}
+    t = timed(lambda: oc.stacks.lenet_trunk_rows(oct6, 6, lp16, data=feat6_16), reps, wu)
+    extra["lenet_trunk_batch32_d6_bf16_rows"] = {"ms": t, "shapes_per_s": 32 / (t * 1e-3),
+                                                 "layout": "row-major between conv and pool (pool + pad in one kernel)"}
     # the same trunk captured once in a HIP graph and replayed: what of the eager time is the host
     # getting from one launch to the next (little: the convolutions of the small levels take it)
     feat6 = F.octree_property(oct6, "feature", 6)

@@ -233,8 +233,8 @@ __device__ inline void lookup_sources(const ConvArgs& a, int col, Put put) {
 // a convolution kernel the look-up is two or three dependent trips to memory per tile in front of
 // everything else, run by the two or three workgroups that fit a compute unit beside their
 // accumulators (about 10 of the 40 microseconds a 256-column tile of a 64 -> 64 bf16 convolution over
-// the non-empty nodes lives); here it runs at full occupancy, and a caller that convolves the same
-// level again (the next layer of the same depth) keeps the table.
+// the non-empty nodes lives).  The table depends on the octree level and the kernel shape only: a
+// caller that convolves the same level again (the other layers of that depth) makes it once.
 __global__ __launch_bounds__(kBlock) void conv_sources_kernel(ConvArgs a, int* __restrict__ table, int pitch) {
   const int col = blockIdx.x * kBlock + threadIdx.x;
   if (col >= pitch) return;
@@ -2302,8 +2302,6 @@ struct ConvPlan {
   KernelTaps taps;
   int mtiles, csteps;
   size_t wt_bytes, ichild_bytes, xt_bytes, xt_general, total_bytes;
-  size_t src_bytes;    // table of source rows (non-empty mode), behind everything else; optional
-  int src_pitch;
 };
 
 inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -2384,11 +2382,7 @@ int make_plan(const Info* o, int depth, int channel_in, int num_output, const in
     p->xt_bytes = align256(((size_t)p->btm_h + 1) * cpad * sizeof(uint16_t));
   }
   if (p->xt_general > p->xt_bytes) p->xt_bytes = p->xt_general;  // one buffer serves whichever path runs
-  // non-empty mode: room for the table of source rows (27 taps x the column tiles), which the call
-  // then makes in a launch of its own at full occupancy instead of tile by tile inside the kernel
-  p->src_pitch = nempty ? (top_h + kTileCols - 1) / kTileCols * kTileCols : 0;
-  p->src_bytes = nempty ? align256(sizeof(int) * 27 * (size_t)p->src_pitch) : 0;
-  p->total_bytes = p->wt_bytes + p->ichild_bytes + p->xt_bytes + p->src_bytes;
+  p->total_bytes = p->wt_bytes + p->ichild_bytes + p->xt_bytes;
   return OCNN_OK;
 }
 
@@ -2403,8 +2397,7 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
   if (e) return e;
   OCNN_REQUIRE(btm_h == p.btm_h, OCNN_E_SHAPE, "input height %d, the octree has %d rows at depth %d",
       btm_h, p.btm_h, depth);
-  // (the table of source rows is optional: a workspace without room for it still serves)
-  OCNN_REQUIRE(ws && (builtin_scratch || ws_bytes >= p.total_bytes - p.src_bytes), OCNN_E_WORKSPACE,
+  OCNN_REQUIRE(ws && (builtin_scratch || ws_bytes >= p.total_bytes), OCNN_E_WORKSPACE,
       "workspace %zu < %zu bytes", ws_bytes, p.total_bytes);
   OCNN_REQUIRE((reinterpret_cast<uintptr_t>(ws) & 15) == 0, OCNN_E_WORKSPACE, "workspace not 16-byte aligned");
 
@@ -2485,14 +2478,6 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     ichild_kernel<<<blocks_for(p.child_h), kBlock, 0, s>>>(ichild, p.ichild_h, a.child, p.child_h);
     OCNN_LAUNCH_OK("ichild");
     a.ichild = ichild;
-    const size_t before = p.wt_bytes + p.ichild_bytes + p.xt_bytes;
-    if ((path == kPathRowsBf16 || path == kPathRowsF32) && p.src_bytes > 0 && ws_bytes >= before + p.src_bytes) {
-      int* table = reinterpret_cast<int*>(wsb + before);
-      conv_sources_kernel<<<blocks_for(p.src_pitch), kBlock, 0, s>>>(a, table, p.src_pitch);
-      OCNN_LAUNCH_OK("conv_sources");
-      a.src_table = table;
-      a.src_pitch = p.src_pitch;
-    }
   }
   if (path == kPathS2Conv) {
     const int MT = a.mtiles == 1 ? 1 : 2;
@@ -3255,7 +3240,7 @@ int make_rows_plan(const Info* o, int depth, int channel_in, int num_output, con
   } else {
     return fail(OCNN_E_UNSUPPORTED, "row-major operators: 3x3x3 stride 1, 2x2x2 stride 2");
   }
-  r->total_bytes = r->wt_bytes + r->ichild_bytes + r->src_bytes;
+  r->total_bytes = r->wt_bytes + r->ichild_bytes;   // (the table of sources is the caller's, see ocnn_conv_rows_sources)
   return OCNN_OK;
 }
 
@@ -3366,8 +3351,8 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
       ichild_kernel<<<blocks_for(p.child_h), kBlock, 0, s>>>(links_ws, p.ichild_h, a.child, p.child_h);
       a.ichild = links_ws;
     }
-    // the source rows of every (tap, column): the caller's table, or one made now when the
-    // workspace has room for it (ocnn_conv_rows_shape asks for that room), or looked up per tile
+    // the source rows of every (tap, column): the caller's table, or looked up per tile inside the
+    // kernel (a table made for one call costs more than it saves: 0.087 -> 0.095 ms at depth 9)
     if (sources_out) {
       a.Hin = r.btm_h;
       conv_sources_kernel<<<blocks_for(r.src_pitch), kBlock, 0, s>>>(a, sources_out, r.src_pitch);
@@ -3376,11 +3361,6 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
     }
     if (sources_in) {
       a.src_table = sources_in;
-      a.src_pitch = r.src_pitch;
-    } else if (ws && ws_bytes >= ws_need + r.src_bytes) {
-      int* table = reinterpret_cast<int*>(wsb + ws_need);
-      conv_sources_kernel<<<blocks_for(r.src_pitch), kBlock, 0, s>>>(a, table, r.src_pitch);
-      a.src_table = table;
       a.src_pitch = r.src_pitch;
     }
     const int n_tiles = (a.N + kTileCols - 1) / kTileCols;

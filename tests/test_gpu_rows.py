@@ -357,9 +357,8 @@ def test_lenet_trunk_rows(oc, octree):
 def test_row_kernel_forms_and_source_tables_agree(oc, octree):
   """Over the non-empty nodes the bf16 row kernels exist in two forms (weights staged in LDS /
   read per live tap), and the source rows of a tile come from a table made ahead (kept with the
-  octree under constant_weights, made per call when the workspace has room) or from the look-up
-  inside the kernel: every combination gives the same bits."""
-  import ctypes as C
+  octree under constant_weights) or from the look-up inside the kernel: every combination gives
+  the same bits."""
   F = oc.nn
   L = oc.lib.get()
   info = F.octree_info(octree)
@@ -378,27 +377,11 @@ def test_row_kernel_forms_and_source_tables_agree(oc, octree):
       for form in (0, 1):
         L.ocnn_conv_rows_direct(form)
         F.forget_cached(octree)
-        results.append(F.octree_conv_rows(xr, cin, w, octree, depth, cout, **kw))                          # table per call
+        results.append(F.octree_conv_rows(xr, cin, w, octree, depth, cout, **kw))                          # look-up in the kernel
         results.append(F.octree_conv_rows(xr, cin, w, octree, depth, cout, constant_weights=True, **kw))   # table kept
         results.append(F.octree_conv_rows(xr, cin, w, octree, depth, cout, constant_weights=True, **kw))
         fn = F.octree_deconv if deconv else F.octree_conv
         results.append(F.to_rows(fn(x, w, octree, depth, cout, list(ks), stride, True)))                     # channel-major
-        # no room for a table: the look-up inside the kernel
-        top_h, need_h, ws_bytes = C.c_int(), C.c_int(), C.c_size_t()
-        ksc = (C.c_int * 3)(*ks)
-        L.ocnn_conv_rows_shape(info.p, depth, cin, cout, ksc, stride, 1, int(deconv), 1, C.byref(top_h), C.byref(need_h),
-                               C.byref(ws_bytes))
-        nb = C.c_size_t()
-        L.ocnn_conv_rows_sources_bytes(info.p, depth, ksc, stride, 1, int(deconv), C.byref(nb))
-        small = ws_bytes.value - nb.value
-        ws = torch.empty(small, dtype=torch.uint8, device="cuda")
-        out = torch.empty(top_h.value + 1, F.rows_pitch(cout), dtype=torch.bfloat16, device="cuda")
-        P = lambda t: C.c_void_p(t.data_ptr())
-        rc = L.ocnn_octree_conv_rows(P(out), out.stride(0), P(xr), xr.stride(0), cin, H, P(w), None, 0, int(deconv), P(octree),
-                                     info.p, depth, cout, ksc, stride, 1, 1, P(ws), C.c_size_t(small),
-                                     C.c_void_p(torch.cuda.current_stream().cuda_stream))
-        assert rc == 0
-        results.append(out)
       for r in results[1:]:
         assert torch.equal(r, results[0]), (depth, cin, cout, ks, stride, deconv)
   finally:
