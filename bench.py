@@ -559,25 +559,32 @@ def main():
   if not (args.quick or args.no_cpu):
     from oracle.checker import Checker, OctreeBlob
     orc = Checker("orc")
+    # the reference's own CPU functions where oracle/_ref holds them compiled (octree2col_cpu, the
+    # pooling and padding loops, the build); the GEMM is the oracle's textbook one either way: the
+    # reference has no CPU GEMM of its own (its CPU path calls a BLAS, octree_conv.cpp:276-325)
+    ref_ok = os.path.exists(os.path.join(ROOT, "oracle", "_ref", "libocnn_ref.so"))
+    chk = Checker("ref") if ref_ok else orc
+    kind = "reference" if ref_ok else "port"
     blob_host = octree.cpu().numpy()
     ob = OctreeBlob(blob_host)
     sample = 327680   # about 10 s of single-thread work
     neigh = ob.prop("neigh", 9).reshape(-1)
     xh = x32.cpu().numpy().reshape(C, H9)
     wh = w32.cpu().numpy()
-    ni = orc.get_ni([3, 3, 3])
+    ni = chk.get_ni([3, 3, 3])
     col = np.empty((C * 27, sample), np.float32)
     import ctypes as Ct
     P = lambda a: a.ctypes.data_as(Ct.c_void_p)
     t0 = time.perf_counter()
     # first chunk of `sample` columns: octree2col_cpu chunk + single-thread SGEMM
-    orc.fn("octree2col")(P(col), P(xh), C, H9, 27, 1, P(neigh), P(ni), sample, 0)
+    chk.fn("octree2col")(P(col), P(xh), C, H9, 27, 1, P(neigh), P(ni), sample, 0)
     y = orc.sgemm(wh, col)
     t = time.perf_counter() - t0
-    out["cpu_baseline"] = {"value": sample / t, "unit": "octants/s", "cores": 1, "kind": "port",
-                           "sample": "first %d of %d depth-9 octants: octree2col_cpu chunk + "
-                                     "single-thread textbook SGEMM (64 x 1728 x %d), %.1f s"
-                                     % (sample, H9, sample, t)}
+    out["cpu_baseline"] = {"value": sample / t, "unit": "octants/s", "cores": 1, "kind": kind,
+                           "sample": "first %d of %d depth-9 octants: %s octree2col_cpu chunk + "
+                                     "single-thread textbook SGEMM (64 x 1728 x %d; the reference has no CPU GEMM "
+                                     "of its own), %.1f s"
+                                     % (sample, H9, "the compiled reference's" if ref_ok else "the oracle's", sample, t)}
     # the host this ran on, and the same sample with the GEMM through torch.mm on all its threads
     # (the reference's CPU path calls a BLAS GEMM there, octree/octree/octree_conv.cpp:276-325)
     try:
@@ -594,7 +601,7 @@ def main():
       ymm = torch.mm(wt, ct)
     t_mm = (time.perf_counter() - t0) / n_mm
     t0 = time.perf_counter()
-    orc.fn("octree2col")(P(col), P(xh), C, H9, 27, 1, P(neigh), P(ni), sample, 0)
+    chk.fn("octree2col")(P(col), P(xh), C, H9, 27, 1, P(neigh), P(ni), sample, 0)
     t_col = time.perf_counter() - t0
     out["cpu_baseline"]["blas_all_threads"] = {
         "value": sample / (t_col + t_mm), "unit": "octants/s", "threads": torch.get_num_threads(),
@@ -604,8 +611,6 @@ def main():
     # the sample also checks the GPU result
     yg = conv_step().cpu().numpy().reshape(C, H9)[:, :sample]
     out["cpu_baseline"]["gpu_vs_cpu_max_rel_err"] = float(np.abs(yg - y).max() / np.abs(y).max())
-    ref_ok = os.path.exists(os.path.join(ROOT, "oracle", "_ref", "libocnn_ref.so"))
-    chk = Checker("ref") if ref_ok else orc
     pb = scene_pts.cpu().numpy()
     t0 = time.perf_counter()
     single = chk.points2octree(pb, 9, 2)
@@ -621,18 +626,20 @@ def main():
       t0 = time.perf_counter()
       r = fn()
       dt = time.perf_counter() - t0
-      rows[name] = {"seconds": dt, unit: units / dt, "cores": 1, "kind": "port"}
+      rows[name] = {"seconds": dt, unit: units / dt, "cores": 1, "kind": kind if name not in port_only else "port"}
       return r
+
+    port_only = ("octree_update_d8",)   # pytorch/cpp/octree_grow.cpp is part of the extension, not of the compiled library
 
     Cs = 16  # channels of the streaming samples
     xs = xh[:Cs]
-    pooled, maskh = cpu_row("max_pool_d9", lambda: orc.max_pool(xs), H9, "octants_per_s")
-    cpu_row("max_unpool_d9", lambda: orc.max_unpool(pooled, maskh), H9, "octants_per_s")
-    cpu_row("mask_pool_d9", lambda: orc.mask_pool(xs, maskh), H9, "octants_per_s")
+    pooled, maskh = cpu_row("max_pool_d9", lambda: chk.max_pool(xs), H9, "octants_per_s")
+    cpu_row("max_unpool_d9", lambda: chk.max_unpool(pooled, maskh), H9, "octants_per_s")
+    cpu_row("mask_pool_d9", lambda: chk.mask_pool(xs, maskh), H9, "octants_per_s")
     child8 = ob.prop("child", 8)
-    padded = cpu_row("pad_d8", lambda: orc.pad(pooled, child8), H8, "octants_per_s")
-    cpu_row("depad_d8", lambda: orc.depad(padded, child8, pooled.shape[1]), H8, "octants_per_s")
-    cpu_row("octree_batch_with_calc_neigh", lambda: orc.octree_batch([single]), sum(ob.nnum[:10]), "nodes_per_s")
+    padded = cpu_row("pad_d8", lambda: chk.pad(pooled, child8), H8, "octants_per_s")
+    cpu_row("depad_d8", lambda: chk.depad(padded, child8, pooled.shape[1]), H8, "octants_per_s")
+    cpu_row("octree_batch_with_calc_neigh", lambda: chk.octree_batch([single]), sum(ob.nnum[:10]), "nodes_per_s")
     lab8 = (child8 >= 0).astype(np.int32)
     upd = cpu_row("octree_update_d8", lambda: orc.octree_update(merged, lab8, 8, 1), H8, "nodes_per_s")
     del upd

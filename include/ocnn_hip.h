@@ -231,7 +231,9 @@ int ocnn_octree_conv_rows(void* top_rows, int top_pitch, const void* btm_rows, i
     void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream);
 /* The same operator for weights that do not change from call to call (inference): pack them once
  * (ocnn_conv_rows_packed_bytes bytes, 16-byte aligned; the order depends on the channel counts, the
- * kernel, the stride, nempty and is_deconv only) and pass the packed form; `ichild_dev`: the
+ * kernel, the stride, nempty, is_deconv and, for nempty operators, on whether at least one node in
+ * five of the level of the columns is non-empty: pack with the header of the octree the call will run on,
+ * or of one like it) and pass the packed form; `ichild_dev`: the
  * inverted child links from ocnn_make_ichild for the operators that use them -- every nempty
  * operator (links of `depth`; of depth+1 for the stride-2 deconvolution) and the all-nodes stride-2
  * deconvolution (links of `depth`) -- or NULL, then the call computes them into the workspace

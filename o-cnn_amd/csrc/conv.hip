@@ -722,8 +722,8 @@ __global__ __launch_bounds__(256, 2) void conv_rows_bf16_deep_kernel(ConvArgs a,
 // times a slab.  Here a wavefront walks its live taps in ascending order with the next live tap's
 // weights and rows in flight (two register sets), at its own pace.  Same products in the same order
 // as conv_rows_bf16_deep_kernel: the results are bit-identical.
-template <int MT, int SLAB, bool ROWS_OUT>
-__global__ __launch_bounds__(256, 2) void conv_rows_bf16_direct_kernel(ConvArgs a, uint16_t* __restrict__ out,
+template <int MT, int SLAB, bool ROWS_OUT, int WPS = 2>
+__global__ __launch_bounds__(256, WPS) void conv_rows_bf16_direct_kernel(ConvArgs a, uint16_t* __restrict__ out,
     const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles, int cpad, int in_pitch, int out_pitch, int out_cpad) {
   constexpr int kKs = SLAB / 16;                        // k-steps per slab
   constexpr int kWUnits = kKs * MT * 64;                // 16-byte units of one (tap, slab)
@@ -2582,7 +2582,10 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     // 128 output channels a pass where the operator has whole blocks of them (see the kernel)
     const bool wide = deep && a.mtiles % 4 == 0;
     const int MT = a.mtiles == 1 ? 1 : (wide ? 4 : 2);
-    const int slab_ch = wide ? 32 : kRowSlab;
+    // (the rule of make_rows_plan: 32-channel stages at three wavefronts a SIMD on a level where one
+    // node in five or more is non-empty)
+    const bool dense_level = nempty && deep && MT == 2 && (int64_t)o->nnum_nempty[p.top_depth] * 5 >= o->nnum[p.top_depth];
+    const int slab_ch = wide || dense_level ? 32 : kRowSlab;
     const int cpad = (a.Cin + 15) / 16 * 16;
     const int npass = (a.mtiles + MT - 1) / MT, nslab = (cpad + slab_ch - 1) / slab_ch;
     int64_t total = (int64_t)npass * a.K * nslab * (slab_ch / 16) * MT * 64 * 8;
@@ -2596,7 +2599,12 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     const dim3 rgrid(grid, pass_split(n_tiles, npass));
     // (with whole blocks of 128 output channels and a channel-major store the staged kernel is ahead)
     const bool direct = deep && !wide && g_rows_direct.load() != 0;
-    if (direct && wide)
+    const bool staged = dense_level && (int64_t)o->nnum_nempty[p.top_depth] * 5 >= (int64_t)o->nnum[p.top_depth] * 2;
+    if (dense_level && direct && !staged)
+      conv_rows_bf16_direct_kernel<2, 32, false, 3><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad, cpad, 0, 0);
+    else if (dense_level)
+      conv_rows_bf16_deep_kernel<2, 32, false><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad, cpad, 0, 0);
+    else if (direct && wide)
       conv_rows_bf16_direct_kernel<4, 32, false><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad, cpad, 0, 0);
     else if (direct && MT == 1)
       conv_rows_bf16_direct_kernel<1, kRowSlab, false><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad, cpad, 0, 0);
@@ -3171,6 +3179,8 @@ struct RowsPlan {
   int MT, npass, ksteps;
   size_t wt_bytes, ichild_bytes, src_bytes, total_bytes;
   int src_pitch;       // columns of the source table (kind 3): the column tiles, whole
+  int slab_ch;         // input channels per stage of the row kernels (kind 3)
+  bool staged;         // 64 output channels a pass on a level where most taps of a tile are live: weights through LDS
 };
 int make_rows_plan(const Info* o, int depth, int channel_in, int num_output, const int* ks, int stride, int nempty,
     int deconv, int dtype, RowsPlan* r) {
@@ -3189,6 +3199,8 @@ int make_rows_plan(const Info* o, int depth, int channel_in, int num_output, con
   r->ichild_bytes = 0;
   r->src_bytes = 0;
   r->src_pitch = 0;
+  r->slab_ch = kRowSlab;
+  r->staged = false;
   const int mtiles = (num_output + 31) / 32;
   if (nempty) {
     // over the non-empty nodes: the general row kernel (rows = ranks of the non-empty nodes on
@@ -3205,9 +3217,23 @@ int make_rows_plan(const Info* o, int depth, int channel_in, int num_output, con
     r->MT = mtiles == 1 ? 1 : (wide ? 4 : 2);
     r->npass = (mtiles + r->MT - 1) / r->MT;
     {
-      const int slab_ch = r->MT == 4 ? 32 : kRowSlab;
+      // 64 output channels a pass: on a level where one node in five or more is non-empty (about
+      // five neighbours a column and up) 32-channel stages, whose two register sets leave room for
+      // three wavefronts a SIMD; on a sparser level (2.2 neighbours a column at depth 9 of a scanned
+      // room) 64-channel stages at two wavefronts.  Measured, 64 -> 64 with kept tables: depth 8
+      // 0.075 -> 0.060 ms with the first, depth 9 0.062 -> 0.067 ms.
+      // Where two nodes in five or more are non-empty (about ten neighbours a column) most taps are
+      // live for every wavefront, and weights staged once in LDS for the four wavefronts win again:
+      // depth 7, 64 -> 64: 0.050 ms staged against 0.054 ms.
+      const bool dense_level = (int64_t)o->nnum_nempty[p.top_depth] * 5 >= o->nnum[p.top_depth];
+      const int slab_ch = r->MT == 4 || (r->MT == 2 && dense_level) ? 32 : kRowSlab;
+      r->slab_ch = slab_ch;
+      r->staged = r->MT == 2 && (int64_t)o->nnum_nempty[p.top_depth] * 5 >= (int64_t)o->nnum[p.top_depth] * 2;
       const int nslab = (r->cpad + slab_ch - 1) / slab_ch;
       r->wt_bytes = align256((size_t)r->npass * p.taps.count * nslab * (slab_ch / 16) * r->MT * 64 * 16);
+      // the two orders of a 64-channel pass take the same room: one more line tells them apart, so
+      // that weights packed for one are refused by a call that would read them in the other
+      if (r->MT == 2 && slab_ch == 32) r->wt_bytes += 256;
     }
     r->ichild_bytes = p.ichild_bytes;
     r->src_pitch = (r->cols + kTileCols - 1) / kTileCols * kTileCols;
@@ -3285,7 +3311,7 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
     } else {
       const int K = stride == 1 ? 27 : 8;
       const int64_t sm = deconv ? K : (int64_t)channel_in * K, sc = deconv ? (int64_t)num_output * K : K;
-      const int slab_ch = r.MT == 4 ? 32 : kRowSlab;
+      const int slab_ch = r.slab_ch;
       const int nslab = (r.cpad + slab_ch - 1) / slab_ch;
       const int64_t total = (int64_t)r.npass * K * nslab * (slab_ch / 16) * r.MT * 64 * 8;
       pack_weights_rows_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)ws, (const uint16_t*)weights, num_output,
@@ -3366,7 +3392,13 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
     const int n_tiles = (a.N + kTileCols - 1) / kTileCols;
     const dim3 grid(((n_tiles + 7) / 8) * 8, pass_split(n_tiles, r.npass));
     const bool direct = a.K >= 3 && g_rows_direct.load() != 0;
-    if (direct && r.MT == 4)
+    if (r.slab_ch == 32 && r.MT == 2 && direct && !r.staged)
+      conv_rows_bf16_direct_kernel<2, 32, true, 3><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
+          (const u32x4*)wpk, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
+    else if (r.slab_ch == 32 && r.MT == 2)
+      conv_rows_bf16_deep_kernel<2, 32, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
+          (const u32x4*)wpk, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
+    else if (direct && r.MT == 4)
       conv_rows_bf16_direct_kernel<4, 32, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
           (const u32x4*)wpk, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
     else if (direct && r.MT == 2)

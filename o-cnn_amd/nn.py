@@ -854,14 +854,16 @@ def octree_conv_rows(rows_in, channel_in, weights, octree, depth, num_output, bi
     if bias.numel() != num_output:
       raise OcnnError(-3, "bias needs num_output entries")
   if constant_weights:
-    key = (channel_in, num_output, tuple(kernel_size), stride, bool(nempty), bool(deconv))
+    # (the byte count is part of the key: it also tells the two orders apart that a 64-channel
+    # pass over the non-empty nodes can be packed in, which one depends on the level)
+    nbytes = C.c_size_t()
+    _lib.call("ocnn_conv_rows_packed_bytes", info.p, depth, channel_in, num_output, ksc, stride, int(nempty),
+              int(deconv), dt, C.byref(nbytes))
+    key = (channel_in, num_output, tuple(kernel_size), stride, bool(nempty), bool(deconv), nbytes.value)
     cache = weights.__dict__.setdefault("_ocnn_rows_packed", {})
     ent = cache.get(key)
     stamp = (weights._version, weights.data_ptr())
     if ent is None or ent[0] != stamp:
-      nbytes = C.c_size_t()
-      _lib.call("ocnn_conv_rows_packed_bytes", info.p, depth, channel_in, num_output, ksc, stride, int(nempty),
-                int(deconv), dt, C.byref(nbytes))
       packed = torch.empty(nbytes.value, dtype=torch.uint8, device=weights.device)
       _lib.call("ocnn_conv_rows_pack", _ptr(packed), C.c_size_t(nbytes.value), _ptr(weights), _ptr(octree), info.p, depth,
                 channel_in, num_output, ksc, stride, int(nempty), int(deconv), dt, _stream())
