@@ -2159,12 +2159,19 @@ __global__ void pack_weights_d2_bf16(uint16_t* __restrict__ Wt, const uint16_t* 
 // 16-byte pieces of row 8 p + s, like the convolutions above.  The columns' operands stay in
 // registers for every pass, the packed weights of a pass are staged in LDS (two buffers, one
 // barrier per pass).
-template <int KS, int MT2>
+// NE: the operator over the non-empty nodes.  The columns are then the rows of the input as they
+// come (rank p of the non-empty nodes of the level), and child s of column p goes to the row that
+// the child links of the finer level name for node 8 p + s, or nowhere when that node is empty.
+// (The general row kernel serves this operator too, one live tap in eight per column and the
+// weights of all eight taps read by every tile: 0.074 ms for 256 -> 128 from 24 730 nodes, where
+// this kernel takes the time of its stores.)
+template <int KS, int MT2, bool NE = false>
 __global__ __launch_bounds__(256) void deconv_s2_rows_bf16_kernel(ConvArgs a, uint16_t* __restrict__ out,
-    int out_pitch, int out_cpad, const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles) {
+    int out_pitch, int out_cpad, const u32x4* __restrict__ xt, int in_pitch, const u32x4* __restrict__ Wt, int n_tiles) {
   constexpr int kUnits = KS * MT2 * 64;
   constexpr int kVec = kUnits / 256;
   __shared__ u32x4 sW[2][kUnits];
+  __shared__ int sRow[NE ? kTileCols * 8 : 1];        // NE: byte offset of the output row of (column, child)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int tile = xcd_tile(blockIdx.x, n_tiles);
   if (tile >= n_tiles) return;
@@ -2173,31 +2180,43 @@ __global__ __launch_bounds__(256) void deconv_s2_rows_bf16_kernel(ConvArgs a, ui
   const int ctiles = (a.M + 31) / 32;                 // 32-channel tiles per child
   const int npass = (8 * ctiles + MT2 - 1) / MT2;
   const __amdgpu_buffer_rsrc_t xrows = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<u32x4*>(xt), 0, (int)(((int64_t)a.Hin + 1) * KS * 32), 0x00020000);
+      const_cast<u32x4*>(xt), 0, (int)(((int64_t)a.Hin + 1) * in_pitch * 2), 0x00020000);
   const __amdgpu_buffer_rsrc_t obuf = __builtin_amdgcn_make_buffer_rsrc(
       out, 0, (int)(((int64_t)a.Hout + 1) * out_pitch * 2), 0x00020000);
   union Frag { u32x4 q; bf16x8 v; };
   Frag b[KS][2];
   int ooff[2];
+  if constexpr (NE) {
+    // the ranks of the children of the tile's columns: eight child links a column, contiguous
+    for (int i = threadIdx.x; i < kTileCols * 8; i += 256) {
+      const int node = tile * kTileCols * 8 + i;         // node 8 p + s of the finer level
+      const int rank = (node >> 3) < a.N ? a.child[node] : -1;
+      sRow[i] = rank >= 0 && rank < a.Hout ? rank * out_pitch * 2 : 0x7fffff00;
+    }
+  }
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) {
     const int n = n0 + nt * 32 + r;
-    const int src = n < a.N ? a.ichild[n] : -1;
-    const int xoff = src >= 0 ? src * KS * 32 + kh * 16 : 0x7fffff00;
+    const int src = n < a.N ? (NE ? n : a.ichild[n]) : -1;
+    const int xoff = src >= 0 ? src * in_pitch * 2 + kh * 16 : 0x7fffff00;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) b[ks][nt].q = __builtin_amdgcn_raw_buffer_load_b128(xrows, xoff, ks * 32, 0);
     ooff[nt] = n < a.N ? (n * 8 * out_pitch + 8 * kh) * 2 : 0x7fffff00;
   }
   u32x4 wr[kVec];
+  // passes may be dealt out over workgroups (blockIdx.y) where the level has few column tiles
+  const int pass0 = blockIdx.y, pstep = gridDim.y;
+  if (pass0 >= npass) return;
 #pragma unroll
-  for (int v = 0; v < kVec; ++v) wr[v] = Wt[v * 256 + threadIdx.x];
+  for (int v = 0; v < kVec; ++v) wr[v] = Wt[(int64_t)pass0 * kUnits + v * 256 + threadIdx.x];
 #pragma unroll
   for (int v = 0; v < kVec; ++v) sW[0][v * 256 + threadIdx.x] = wr[v];
   const float floor = a.relu ? 0.0f : -__builtin_inff();
-  for (int pass = 0; pass < npass; ++pass) {
+  int buf = 0;
+  for (int pass = pass0; pass < npass; pass += pstep, buf ^= 1) {
     __syncthreads();   // this pass's weights are in LDS; the other buffer is free
-    const u32x4* wcur = sW[pass & 1];
-    const int nxt = min(pass + 1, npass - 1);
+    const u32x4* wcur = sW[buf];
+    const int nxt = pass + pstep < npass ? pass + pstep : pass;
 #pragma unroll
     for (int v = 0; v < kVec; ++v) wr[v] = Wt[(int64_t)nxt * kUnits + v * 256 + threadIdx.x];
     floatx16 acc[MT2][2];
@@ -2217,7 +2236,7 @@ __global__ __launch_bounds__(256) void deconv_s2_rows_bf16_kernel(ConvArgs a, ui
         acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b[ks][1].v, acc[mt][1], 0, 0, 0);
       }
 #pragma unroll
-    for (int v = 0; v < kVec; ++v) sW[(pass + 1) & 1][v * 256 + threadIdx.x] = wr[v];
+    for (int v = 0; v < kVec; ++v) sW[buf ^ 1][v * 256 + threadIdx.x] = wr[v];
 #pragma unroll
     for (int mt = 0; mt < MT2; ++mt) {
       const int t = pass * MT2 + mt;                  // tile = (child, 32-channel block)
@@ -2245,8 +2264,14 @@ __global__ __launch_bounds__(256) void deconv_s2_rows_bf16_kernel(ConvArgs a, ui
         for (int jj = 0; jj < 2; ++jj) {
           const auto s0 = __builtin_amdgcn_permlane32_swap(w[2 * jj][0], w[2 * jj + 1][0], false, false);
           const auto s1 = __builtin_amdgcn_permlane32_swap(w[2 * jj][1], w[2 * jj + 1][1], false, false);
-          store16_then_wait(store16_t{s0[0], s1[0], s0[1], s1[1]}, obuf, ooff[nt],
-              (child * out_pitch + cb + 16 * jj) * 2, cb + 16 * jj < out_cpad);
+          if constexpr (NE) {
+            const int row = sRow[(wave * kWaveCols + nt * 32 + r) * 8 + child];   // written before the first barrier
+            store16_then_wait(store16_t{s0[0], s1[0], s0[1], s1[1]}, obuf, row == 0x7fffff00 ? row : row + 16 * kh,
+                (cb + 16 * jj) * 2, cb + 16 * jj < out_cpad);
+          } else {
+            store16_then_wait(store16_t{s0[0], s1[0], s0[1], s1[1]}, obuf, ooff[nt],
+                (child * out_pitch + cb + 16 * jj) * 2, cb + 16 * jj < out_cpad);
+          }
         }
       }
       if (tile == 0 && wave == 0 && child == 0 && lane * 8 >= cb && lane * 8 < min(cb + 32, out_cpad))
@@ -3202,7 +3227,22 @@ int make_rows_plan(const Info* o, int depth, int channel_in, int num_output, con
   r->slab_ch = kRowSlab;
   r->staged = false;
   const int mtiles = (num_output + 31) / 32;
-  if (nempty) {
+  if (nempty && stride == 2 && k222 && deconv && depth < o->depth &&
+      (r->ksteps == 1 || r->ksteps == 2 || r->ksteps == 4 || r->ksteps == 8 || r->ksteps == 16) &&
+      (int64_t)o->nnum_nempty[depth + 1] * 5 >= (int64_t)o->nnum[depth + 1] * 2) {
+    // 2x2x2 stride-2 deconvolution over the non-empty nodes: the all-nodes kernel with the rows of
+    // the input as its columns and the child links of the finer level as the map of its output rows.
+    // It forms all eight children of a column and drops the empty ones, so it pays where two
+    // children in five or more exist (256 -> 128 from depth 6 of the scene: 0.074 -> 0.05 ms); on a
+    // sparser level the general row kernel, which forms the non-empty rows only, is ahead (64 -> 32
+    // onto depth 9, one child in six: 0.023 against 0.031 ms)
+    r->kind = 4;
+    r->btm_h = r->cols = o->nnum_nempty[depth];
+    r->top_h = o->nnum_nempty[depth + 1];
+    r->MT = r->ksteps <= 4 ? 4 : 2;
+    r->npass = (8 * mtiles + r->MT - 1) / r->MT;
+    r->wt_bytes = align256((size_t)r->npass * r->ksteps * r->MT * 64 * 16);
+  } else if (nempty) {
     // over the non-empty nodes: the general row kernel (rows = ranks of the non-empty nodes on
     // both sides, exactly the operator of the channel-major entry points)
     OCNN_REQUIRE((stride == 1 && k333) || (stride == 2 && k222), OCNN_E_UNSUPPORTED,
@@ -3304,7 +3344,7 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
       const int64_t total = (int64_t)r.npass * 8 * r.ksteps * r.MT * 64 * 8;
       pack_weights_s2_rows_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)ws, (const uint16_t*)weights, num_output,
           channel_in, r.MT, r.npass, r.ksteps);
-    } else if (r.kind == 2) {
+    } else if (r.kind == 2 || r.kind == 4) {
       const int64_t total = (int64_t)r.npass * r.ksteps * r.MT * 64 * 8;
       pack_weights_d2_rows_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)ws, (const uint16_t*)weights, num_output,
           channel_in, r.MT, r.npass, r.ksteps);
@@ -3327,7 +3367,7 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
       r.btm_h, depth);
   // the stride-2 convolution also reads a channel slice of a wider tensor (an encoder feature that
   // sits in the tensor the decoder reads as a concatenation)
-  OCNN_REQUIRE(btm_pitch == r.cpad || ((r.kind == 1 || r.kind == 3) && btm_pitch > r.cpad && btm_pitch % 8 == 0), OCNN_E_SHAPE,
+  OCNN_REQUIRE(btm_pitch == r.cpad || ((r.kind == 1 || r.kind == 3 || r.kind == 4) && btm_pitch > r.cpad && btm_pitch % 8 == 0), OCNN_E_SHAPE,
       "input pitch %d: rows of %d channels are padded to %d", btm_pitch, channel_in, r.cpad);
   OCNN_REQUIRE(top_pitch >= r.out_cpad && top_pitch % 8 == 0, OCNN_E_SHAPE, "output pitch %d for %d channels",
       top_pitch, num_output);
@@ -3455,6 +3495,33 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
     else
       conv_s2_rows_bf16_kernel<2><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, top_pitch, r.out_cpad,
           (const u32x4*)btm_rows, btm_pitch, r.cpad, (const u32x4*)wpk, n_tiles);
+  } else if (r.kind == 4) {
+    a.K = 8;
+    a.mode = kModeS2Deconv;
+    a.neigh = nullptr;
+    a.child = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_CHILD, depth + 1));
+    OCNN_REQUIRE(o->nnum[depth + 1] == 8 * r.cols, OCNN_E_FORMAT, "depth %d holds %d nodes for %d non-empty parents",
+        depth + 1, o->nnum[depth + 1], r.cols);
+    if (r.top_h == 0 || r.cols == 0) {
+      OCNN_REQUIRE(top_pitch == r.out_cpad, OCNN_E_UNSUPPORTED, "empty level into a channel slice");
+      const int64_t cnt = ((int64_t)r.top_h + 1) * top_pitch;
+      zero_rows_kernel<uint16_t><<<blocks_for(cnt), kBlock, 0, s>>>((uint16_t*)top_rows, cnt);
+      OCNN_LAUNCH_OK("zero_rows");
+      return OCNN_OK;
+    }
+    const int n_tiles = (a.N + kTileCols - 1) / kTileCols;
+    const dim3 grid(((n_tiles + 7) / 8) * 8, pass_split(n_tiles, r.npass));
+#define OCNN_D2_ROWS_NE(KS, MT2)                                                                      \
+    deconv_s2_rows_bf16_kernel<KS, MT2, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, top_pitch, r.out_cpad, \
+        (const u32x4*)btm_rows, btm_pitch, (const u32x4*)wpk, n_tiles)
+    switch (r.ksteps) {
+      case 1: OCNN_D2_ROWS_NE(1, 4); break;
+      case 2: OCNN_D2_ROWS_NE(2, 4); break;
+      case 4: OCNN_D2_ROWS_NE(4, 4); break;
+      case 8: OCNN_D2_ROWS_NE(8, 2); break;
+      default: OCNN_D2_ROWS_NE(16, 2); break;
+    }
+#undef OCNN_D2_ROWS_NE
   } else {
     a.K = 8;
     a.mode = kModeS2Deconv;
@@ -3467,10 +3534,10 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
       a.ichild = links_ws;
     }
     const int n_tiles = (a.N + kTileCols - 1) / kTileCols;
-    const int grid = ((n_tiles + 7) / 8) * 8;
+    const dim3 grid(((n_tiles + 7) / 8) * 8, pass_split(n_tiles, r.npass));
 #define OCNN_D2_ROWS(KS, MT2)                                                                         \
     deconv_s2_rows_bf16_kernel<KS, MT2><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, top_pitch, r.out_cpad, \
-        (const u32x4*)btm_rows, (const u32x4*)wpk, n_tiles)
+        (const u32x4*)btm_rows, btm_pitch, (const u32x4*)wpk, n_tiles)
     switch (r.ksteps) {
       case 1: OCNN_D2_ROWS(1, 4); break;
       case 2: OCNN_D2_ROWS(2, 4); break;

@@ -879,13 +879,15 @@ def octree_conv_rows(rows_in, channel_in, weights, octree, depth, num_output, bi
         tables.clear()
         tables["version"] = octree._version
       skey = (depth, tuple(kernel_size), stride, bool(deconv))
-      sources = tables.get(skey)
-      if sources is None:
+      sources = tables.get(skey, False)
+      if sources is False:
         nb = C.c_size_t()
         _lib.call("ocnn_conv_rows_sources_bytes", info.p, depth, ksc, stride, 1, int(deconv), C.byref(nb))
-        sources = torch.empty(nb.value // 4, dtype=torch.int32, device=octree.device)
-        _lib.call("ocnn_conv_rows_sources", _ptr(sources), C.c_size_t(nb.value), None, _ptr(octree), info.p, depth, ksc,
-                  stride, 1, int(deconv), C.c_void_p(base), C.c_size_t(ws_bytes.value), _stream())
+        sources = None       # an operator that looks nothing up (the 2x2x2 stride-2 deconvolution)
+        if nb.value:
+          sources = torch.empty(nb.value // 4, dtype=torch.int32, device=octree.device)
+          _lib.call("ocnn_conv_rows_sources", _ptr(sources), C.c_size_t(nb.value), None, _ptr(octree), info.p, depth, ksc,
+                    stride, 1, int(deconv), C.c_void_p(base), C.c_size_t(ws_bytes.value), _stream())
         tables[skey] = sources
     elif deconv and stride == 2:
       links_of = octree.__dict__.setdefault("_ocnn_ichild", {})
