@@ -13,6 +13,7 @@
 #include "build_adaptive.h"
 #include "octree_kernels.h"
 
+#include <algorithm>
 #include <vector>
 
 namespace ocnn {
@@ -56,27 +57,52 @@ __device__ inline float norm3(const float* v) {  // math_functions.cpp:257-263
   return sqrt_rn(len);
 }
 
-// ---- covered_depth_nodes (octree.cpp:958-1002): range of finest-level nodes under a node
-// mode 0: finest level, 1: the level above, 2: any other level
-__global__ void cover_kernel(int* __restrict__ dnum, int* __restrict__ didx, const int* __restrict__ child,
-    const int* __restrict__ dnum_c, const int* __restrict__ didx_c, int n, int mode) {
+// ---- covered_depth_nodes (octree.cpp:958-1002): range of finest-level nodes under a node.
+// The finest level itself needs no table (a node covers itself).  The level above it covers
+// its eight children, and every node of the finest level is such a child: its error terms start
+// "infinite" here (calc_signal leaves them at 1.0e20f, octree.cpp:456-470).
+__global__ void cover_first_kernel(int* __restrict__ dnum, int* __restrict__ didx, const int* __restrict__ child,
+    float* __restrict__ nerr_c, float* __restrict__ derr_c, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
+  const int c = child[i];
+  dnum[i] = c >= 0 ? 8 : 0;
+  didx[i] = c >= 0 ? c * 8 : -1;
+  if (c >= 0) {
+    const float4 big = make_float4(1.0e20f, 1.0e20f, 1.0e20f, 1.0e20f);
+    float4* e0 = reinterpret_cast<float4*>(nerr_c + c * 8);
+    float4* e1 = reinterpret_cast<float4*>(derr_c + c * 8);
+    e0[0] = big; e0[1] = big; e1[0] = big; e1[1] = big;
+  }
+}
+__device__ inline void cover_node(int* __restrict__ dnum, int* __restrict__ didx, const int* __restrict__ child,
+    const int* dnum_c, const int* didx_c, int i) {
   int num = 0, idx = -1;
-  if (mode == 0) { num = 1; idx = i; }
-  else {
-    const int c = child[i];
-    if (c >= 0) {
-      if (mode == 1) { num = 8; idx = c * 8; }
-      else {
-        for (int j = 0; j < 8; ++j) num += dnum_c[c * 8 + j];
-        for (int j = 0; j < 8; ++j)
-          if (didx_c[c * 8 + j] != -1) { idx = didx_c[c * 8 + j]; break; }
-      }
-    }
+  const int c = child[i];
+  if (c >= 0) {
+    for (int j = 0; j < 8; ++j) num += dnum_c[c * 8 + j];
+    for (int j = 0; j < 8; ++j)
+      if (didx_c[c * 8 + j] != -1) { idx = didx_c[c * 8 + j]; break; }
   }
   dnum[i] = num;
   didx[i] = idx;
+}
+__global__ void cover_kernel(int* __restrict__ dnum, int* __restrict__ didx, const int* __restrict__ child,
+    const int* __restrict__ dnum_c, const int* __restrict__ didx_c, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) cover_node(dnum, didx, child, dnum_c, didx_c, i);
+}
+// the small levels at the top, one after the other in one workgroup
+struct CoverTop {
+  int d_top;   // levels d_top .. 0; level d_top + 1 is complete
+  int n[kMaxD];
+  int* dnum[kMaxD]; int* didx[kMaxD]; const int* child[kMaxD];
+};
+__global__ __launch_bounds__(1024) void cover_top_kernel(const CoverTop t) {
+  for (int d = t.d_top; d >= 0; --d) {
+    for (int i = threadIdx.x; i < t.n[d]; i += 1024) cover_node(t.dnum[d], t.didx[d], t.child[d], t.dnum[d + 1], t.didx[d + 1], i);
+    __syncthreads();   // the level's tables are read by the next one (same workgroup: its writes are visible after the barrier)
+  }
 }
 
 __global__ void fill_kernel(float* __restrict__ p, int64_t n, float v) {
@@ -127,9 +153,10 @@ __device__ inline int intersect_cube(float* V, const float* pt, const float* pt_
 // block (a lane moves four consecutive leaves of a value with one 16-byte load and store), and
 // lane c adds up value c leaf after leaf: the channels run side by side, each in the
 // reference's order.  Leaves outside the range enter as +0, which changes no partial sum (a
-// partial sum is never -0: the chain starts at +0).  The next 256 leaves are requested before
-// the current ones are added (the chain of a node high up in the tree covers the whole finest
-// level: memory latency must not be paid per block).  sum[c] / last[c] get the sum and the
+// partial sum is never -0: the chain starts at +0).  Three blocks of 256 leaves are requested
+// ahead of the one being added (the chain of a node high up in the tree covers the whole finest
+// level, adding a block takes less time than a load from memory: the latency must not be paid
+// per block).  sum[c] / last[c] get the sum and the
 // last value of channel c on every lane.
 constexpr int kPassValues = 8, kPassLeaves = 256;
 template <int NV>
@@ -137,8 +164,9 @@ __device__ inline void ordered_sums(int k0, int k1, int lane, float* __restrict_
     float* sum, float* last) {
   static_assert(NV <= kPassValues, "LDS block too small");
   float acc = 0.0f;
-  float4 vals[NV];
-  auto request = [&](int base) {
+  constexpr int kAhead = 3;      // blocks requested before they are needed
+  float4 vals[kAhead][NV];
+  auto request = [&](float4 (&dst)[NV], int base) {
     const int k = base + 4 * lane;
 #pragma unroll
     for (int c = 0; c < NV; ++c) {
@@ -148,40 +176,63 @@ __device__ inline void ordered_sums(int k0, int k1, int lane, float* __restrict_
       v.y = (k + 1 >= k0 && k + 1 < k1) ? v.y : 0.0f;
       v.z = (k + 2 >= k0 && k + 2 < k1) ? v.z : 0.0f;
       v.w = (k + 3 >= k0 && k + 3 < k1) ? v.w : 0.0f;
-      vals[c] = v;
+      dst[c] = v;
     }
   };
-  const int kb = k0 < k1 ? (k0 & ~3) : k1;   // an empty range runs no block
-  if (k0 < k1) request(kb);
-  for (int base = kb; base < k1; base += kPassLeaves) {
+  auto add_block = [&](const float4 (&cur_vals)[NV], int base) {
 #pragma unroll
-    for (int c = 0; c < NV; ++c) *reinterpret_cast<float4*>(lds + c * kPassLeaves + 4 * lane) = vals[c];
-    if (base + kPassLeaves < k1) request(base + kPassLeaves);
+    for (int c = 0; c < NV; ++c) *reinterpret_cast<float4*>(lds + c * kPassLeaves + 4 * lane) = cur_vals[c];
     __builtin_amdgcn_wave_barrier();   // same wavefront: the LDS unit keeps its accesses in order
     const int total = min(kPassLeaves, k1 - base);
     if (lane < NV) {
-      // the adds form one dependent chain; the LDS reads of the next 16 leaves are in flight
-      // while the current 16 are added
-      constexpr int kStep = 16;
+      // the adds form one dependent chain, and one wavefront issues an instruction every few
+      // cycles: nothing but the adds and the LDS reads may sit in the loop.  Two register sets
+      // take turns (the reads of the next 32 leaves are in flight while the current 32 are
+      // added, an LDS read takes longer than 16 adds), every offset is a constant.
+      constexpr int kStep = 32, kChunks = kPassLeaves / kStep;
       const float4* src = reinterpret_cast<const float4*>(lds + lane * kPassLeaves);
-      float4 cur[kStep / 4];
+      float4 ra[kStep / 4], rb[kStep / 4];
+      auto read = [&](float4 (&r)[kStep / 4], int chunk) {
 #pragma unroll
-      for (int i = 0; i < kStep / 4; ++i) cur[i] = src[i];
-      for (int t = 0; t < total; t += kStep) {
-        float4 nxt[kStep / 4];
-        const int tn = min(t + kStep, kPassLeaves - kStep);          // stays inside the block
-#pragma unroll
-        for (int i = 0; i < kStep / 4; ++i) nxt[i] = src[tn / 4 + i];
+        for (int i = 0; i < kStep / 4; ++i) r[i] = src[chunk * (kStep / 4) + i];
+      };
+      auto add = [&](const float4 (&r)[kStep / 4]) {
 #pragma unroll
         for (int i = 0; i < kStep / 4; ++i) {
-          acc = __fadd_rn(acc, cur[i].x); acc = __fadd_rn(acc, cur[i].y);
-          acc = __fadd_rn(acc, cur[i].z); acc = __fadd_rn(acc, cur[i].w);
+          acc = __fadd_rn(acc, r[i].x); acc = __fadd_rn(acc, r[i].y);
+          acc = __fadd_rn(acc, r[i].z); acc = __fadd_rn(acc, r[i].w);
         }
+      };
+      read(ra, 0);
 #pragma unroll
-        for (int i = 0; i < kStep / 4; ++i) cur[i] = nxt[i];
+      for (int ch = 0; ch < kChunks; ch += 2) {
+        if (ch * kStep >= total) break;
+        read(rb, ch + 1);
+        add(ra);
+        if ((ch + 1) * kStep >= total) break;
+        if (ch + 2 < kChunks) read(ra, ch + 2);
+        add(rb);
       }
     }
     __builtin_amdgcn_wave_barrier();
+  };
+  const int kb = k0 < k1 ? (k0 & ~3) : k1;   // an empty range runs no block
+#pragma unroll
+  for (int u = 0; u < kAhead; ++u)
+    if (kb + u * kPassLeaves < k1) request(vals[u], kb + u * kPassLeaves);
+  for (int base = kb; base < k1; base += kAhead * kPassLeaves) {
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      const int b = base + u * kPassLeaves;
+      if (b < k1) {
+        // a block's registers are free once it sits in LDS: the block kAhead further on takes them
+        float4 now[NV];
+#pragma unroll
+        for (int c = 0; c < NV; ++c) now[c] = vals[u][c];
+        if (b + kAhead * kPassLeaves < k1) request(vals[u], b + kAhead * kPassLeaves);
+        add_block(now, b);
+      }
+    }
   }
 #pragma unroll
   for (int c = 0; c < NV; ++c) {
@@ -240,6 +291,7 @@ struct LeafPack {
   }
 };
 
+// what a node's signal is computed from: the level's own rows and the finest level
 struct SignalArgs {
   int d, depth, n, nD, cf, ch_dis, adp_layer, calc_nerr, calc_derr;
   float imul;
@@ -253,21 +305,41 @@ struct SignalArgs {
   int64_t nP;
   float *normal, *pt, *feature, *label, *dis, *nerr, *derr;   // level d (null: absent)
 };
+struct SignalLevel {   // the part of SignalArgs that differs from level to level
+  int n;
+  const uint64_t* key;
+  const int *child, *dnum, *didx;
+  float *normal, *pt, *feature, *label, *dis, *nerr, *derr;
+};
 
 // One wavefront per node; every level above the finest in one launch, the root first (its
 // chain is the longest, the others run beside it).
+// The two levels above the finest (at most 8 and 64 leaves to a node, and nine nodes in ten of
+// the levels above the finest) go one THREAD per node in a launch of their own: a wavefront
+// per node spends its time on the fixed cost of a node there, not on leaves.
+// The table travels as a kernel argument (under 2 KB): no copy, no wait.
 struct SignalLevels {
-  int first_wave[kMaxD + 1];     // of level d; [depth] = total
-  SignalArgs level[kMaxD - 1];
+  int first_wave[kMaxD + 1];     // of level d among the levels that go one wavefront per node; [depth] = total
+  int first_thread[kMaxD + 1];   // of level d among the levels that go one thread per node; [depth] = total
+  SignalArgs common;             // the level fields are filled per node from `level`
+  SignalLevel level[kMaxD - 1];
 };
-__global__ __launch_bounds__(kBlock) void signal_kernel(const SignalLevels* __restrict__ levels, int depth) {
+__device__ inline SignalArgs signal_args(const SignalLevels& L, int d) {
+  SignalArgs a = L.common;
+  const SignalLevel& l = L.level[d];
+  a.d = d; a.n = l.n; a.key = l.key; a.child = l.child; a.dnum = l.dnum; a.didx = l.didx;
+  a.normal = l.normal; a.pt = l.pt; a.feature = l.feature; a.label = l.label; a.dis = l.dis;
+  a.nerr = l.nerr; a.derr = l.derr;
+  return a;
+}
+__global__ __launch_bounds__(kBlock) void signal_kernel(const SignalLevels levels, int depth) {
   const int lane = threadIdx.x & 63;
   const int w = (int)((blockIdx.x * (unsigned)kBlock + threadIdx.x) >> 6);
-  if (w >= levels->first_wave[depth]) return;
+  if (w >= levels.first_wave[depth]) return;
   int d = 0;
-  while (w >= levels->first_wave[d + 1]) ++d;
-  const SignalArgs& a = levels->level[d];
-  const int i = w - levels->first_wave[d];
+  while (w >= levels.first_wave[d + 1]) ++d;
+  const SignalArgs a = signal_args(levels, d);
+  const int i = w - levels.first_wave[d];
   __shared__ __attribute__((aligned(16))) float s_pass[kBlock / 64][kPassLeaves * kPassValues];
   float* lds = s_pass[threadIdx.x >> 6];
   const int64_t n = a.n;
@@ -442,6 +514,135 @@ __global__ __launch_bounds__(kBlock) void signal_kernel(const SignalLevels* __re
   }
 }
 
+// One thread per node: calc_signal as the reference writes it, leaf after leaf (the sums are
+// the same chains as in signal_kernel, so both forms give the same bits).
+__global__ __launch_bounds__(kBlock) void signal_small_kernel(const SignalLevels levels, int depth) {
+  const int t = blockIdx.x * kBlock + threadIdx.x;
+  if (t >= levels.first_thread[depth]) return;
+  int d = 0;
+  while (t >= levels.first_thread[d + 1]) ++d;
+  const SignalArgs a = signal_args(levels, d);
+  const int i = t - levels.first_thread[d];
+  const int64_t n = a.n;
+  const bool has_normal = a.nrm_D != nullptr, has_pt = a.pt_D != nullptr;
+  if (a.child[i] == -1) {   // empty: zero signal, no label, errors "infinite"
+    if (a.normal) for (int c = 0; c < 3; ++c) a.normal[c * n + i] = 0.0f;
+    if (a.pt) for (int c = 0; c < 3; ++c) a.pt[c * n + i] = 0.0f;
+    for (int c = 0; c < a.cf; ++c) a.feature[c * n + i] = 0.0f;
+    if (a.label) a.label[i] = -1.0f;
+    if (a.dis) for (int c = 0; c < a.ch_dis; ++c) a.dis[c * n + i] = 0.0f;
+    if (a.nerr) a.nerr[i] = 1.0e20f;
+    if (a.derr) a.derr[i] = 1.0e20f;
+    return;
+  }
+  const int j0 = a.didx[i], j1 = j0 + a.dnum[i];
+  const float scale = (float)(1 << (a.depth - a.d));
+  const int k0 = a.rank_D[j0], k1 = a.rank_D[j1];
+  const int leaves = k1 - k0;
+  const int64_t nP = a.nP;
+  float n_avg[3] = {0.0f, 0.0f, 0.0f}, last_n[3] = {0.0f, 0.0f, 0.0f}, pt_avg[3] = {0.0f, 0.0f, 0.0f};
+  for (int k = k0; k < k1; ++k) {
+    if (has_normal) for (int c = 0; c < 3; ++c) n_avg[c] = __fadd_rn(n_avg[c], a.nrm_P[c * nP + k]);
+    if (has_pt) for (int c = 0; c < 3; ++c) pt_avg[c] = __fadd_rn(pt_avg[c], a.pt_P[c * nP + k]);
+  }
+  if (has_normal && k0 < k1) for (int c = 0; c < 3; ++c) last_n[c] = a.nrm_P[c * nP + k1 - 1];
+  if (has_normal) {
+    float len = norm3(n_avg);
+    if (len < 1.0e-6f) {
+      for (int c = 0; c < 3; ++c) n_avg[c] = last_n[c];
+      len = __fadd_rn(norm3(n_avg), 1.0e-30f);
+    }
+    for (int c = 0; c < 3; ++c) n_avg[c] = div_rn(n_avg[c], len);
+    for (int c = 0; c < 3; ++c) a.normal[c * n + i] = n_avg[c];
+  }
+  const float count = leaves > 0 ? (float)leaves : 1.0e-30f;   // 1e-30f + 1 + 1 + ... in float
+  if (has_pt) {
+    const float div = __fmul_rn(count, scale);
+    for (int c = 0; c < 3; ++c) pt_avg[c] = div_rn(pt_avg[c], div);
+    for (int c = 0; c < 3; ++c) a.pt[c * n + i] = pt_avg[c];
+  }
+  for (int c = 0; c < a.cf; ++c) {
+    float f = 0.0f;
+    for (int k = k0; k < k1; ++k) f = __fadd_rn(f, a.feat_P[c * nP + k]);
+    a.feature[c * n + i] = div_rn(f, count);
+  }
+  if (a.label) {
+    // most frequent label (>= 0) of the non-empty leaves, the smallest one on a tie
+    int best = -1, best_cnt = 0;
+    for (int u = k0; u < k1; ++u) {
+      const int l = (int)a.lab_P[u];
+      if (l < 0) continue;
+      int cnt = 0;
+      for (int k = k0; k < k1; ++k) cnt += ((int)a.lab_P[k] == l) ? 1 : 0;
+      if (cnt > best_cnt || (cnt == best_cnt && l < best)) { best = l; best_cnt = cnt; }
+    }
+    a.label[i] = best_cnt > 0 ? (float)best : -1.0f;
+  }
+  uint32_t bx, by, bz;
+  morton_decode(a.key[i], a.d, &bx, &by, &bz);
+  const float pt_base[3] = {(float)bx, (float)by, (float)bz};
+  if (a.dis) {
+    float dis_avg[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int c = 0; c < 3; ++c) {
+      const float fract = __fsub_rn(pt_avg[c], pt_base[c]);
+      dis_avg[c] = __fsub_rn(fract, 0.5f);
+      if (has_normal) dis_avg[3] = __fadd_rn(dis_avg[3], __fmul_rn(dis_avg[c], n_avg[c]));
+      else dis_avg[3] = 1.0f;
+    }
+    if (!has_normal) {
+      for (int c = 0; c < 3; ++c) a.dis[c * n + i] = dis_avg[c];
+      a.dis[3 * n + i] = __fmul_rn(dis_avg[3], a.imul);
+    } else {
+      a.dis[i] = __fmul_rn(dis_avg[3], a.imul);
+    }
+  }
+  if (a.nerr) {
+    float nm_err = 1.0e20f;
+    if (a.calc_nerr && has_normal && a.d >= a.adp_layer) {
+      nm_err = 0.0f;
+      for (int k = k0; k < k1; ++k)
+        for (int c = 0; c < 3; ++c) {
+          const float tmp = __fsub_rn(a.nrm_P[c * nP + k], n_avg[c]);
+          nm_err = __fadd_rn(nm_err, __fmul_rn(tmp, tmp));
+        }
+      nm_err = div_rn(nm_err, count);
+    }
+    a.nerr[i] = nm_err;
+  }
+  if (a.derr) {
+    float err = 1.0e20f;
+    if (a.calc_derr && has_pt && a.d >= a.adp_layer) {
+      float pt_avg1[3];
+      for (int c = 0; c < 3; ++c) pt_avg1[c] = __fmul_rn(pt_avg[c], scale);
+      float distance_max1 = -1.0f;
+      for (int k = k0; k < k1; ++k) {
+        float dis = 0.0f;
+        for (int c = 0; c < 3; ++c) dis = __fadd_rn(dis, __fmul_rn(__fsub_rn(a.pt_P[c * nP + k], pt_avg1[c]), n_avg[c]));
+        distance_max1 = fmaxf(distance_max1, fabsf(dis));
+      }
+      float vtx[36];
+      const int nv = intersect_cube(vtx, pt_avg, pt_base, n_avg);
+      float distance_max2 = nv == 0 ? 5.0e10f : -1.0f;
+      for (int v = 0; v < nv; ++v) {
+        float vk[3];
+        for (int c = 0; c < 3; ++c) vk[c] = __fmul_rn(vtx[3 * v + c], scale);
+        float distance_min = 1.0e30f;
+        for (int k = k0; k < k1; ++k) {
+          float dis = 0.0f;
+          for (int c = 0; c < 3; ++c) {
+            const float ptc = __fsub_rn(a.pt_P[c * nP + k], vk[c]);
+            dis = __fadd_rn(dis, __fmul_rn(ptc, ptc));
+          }
+          distance_min = fminf(distance_min, sqrt_rn(dis));
+        }
+        if (distance_min > distance_max2) distance_max2 = distance_min;
+      }
+      err = distance_max2 > distance_max1 ? distance_max2 : distance_max1;
+    }
+    a.derr[i] = err;
+  }
+}
+
 // ---- extrapolate_signal (octree.cpp:666-806): one thread per sibling group ------------------
 // OctreeParser::key2xyz<float> (octree_parser.cpp:151-165) on the builder's keys: they are still
 // Morton codes at this point, and with the key2xyz option the reference reads them as packed
@@ -458,6 +659,7 @@ __device__ inline void node_xyz(float* xyz, uint64_t key, int depth, int packed)
 
 struct ExtrapolateArgs {
   int n, cf, has_dis, d, key2xyz;
+  int per_octree;     // nodes of one octree on this level where the level is full (else n)
   float imul;
   const uint64_t* key;
   const int* child;
@@ -475,14 +677,16 @@ __global__ void extrapolate_kernel(ExtrapolateArgs a) {
   if (cnt == 0) {
     // No non-empty sibling (happens on the last full layer only): normals, features and labels
     // stay as they are; the displacement comes from the nearest non-empty node of the level
-    // (L1 distance, the first one on a tie), octree.cpp:776-803.
+    // (L1 distance, the first one on a tie), octree.cpp:776-803.  In a batch "the level" is
+    // the level of the node's own octree: on a full layer its nodes are one block of the row.
     if (!(a.has_dis && a.dis)) return;
+    const int j_first = (i_base / a.per_octree) * a.per_octree, j_end = min(a.n, j_first + a.per_octree);
     for (int id = 0; id < 8; ++id) {
       const int i = i_base + id;
       float pti[3], ptj[3], dis_min = 1.0e30f;
       node_xyz(pti, a.key[i], a.d, a.key2xyz);
       int j_min = -1;
-      for (int j = 0; j < a.n; ++j) {
+      for (int j = j_first; j < j_end; ++j) {
         if (a.child[j] == -1) continue;
         node_xyz(ptj, a.key[j], a.d, a.key2xyz);
         const float dd = __fadd_rn(__fadd_rn(fabsf(__fsub_rn(pti[0], ptj[0])), fabsf(__fsub_rn(pti[1], ptj[1]))),
@@ -573,120 +777,232 @@ __global__ void extrapolate_kernel(ExtrapolateArgs a) {
 // ---- trim_octree (octree.cpp:1004-1135) ------------------------------------------------------
 enum { kDrop = 0, kDropChildren = 1, kKeep = 2 };
 
-// one thread per node of level d-1: flags of its children at level d
-__global__ void trim_flag_kernel(int* __restrict__ drop_d, const int* __restrict__ drop_p, const int* __restrict__ child_p,
-    const int* __restrict__ child_d, const float* __restrict__ nerr, const float* __restrict__ derr, int n_p,
-    int has_dis, float th_dist, float th_norm, int* __restrict__ any_kept) {
+// one thread per node of level d-1: flags of its children at level d.  The test "was any
+// non-empty node of the level kept" is taken per octree (trim_octree runs on one octree at a
+// time, and a batch is trimmed octree by octree before merge_octrees joins them): the octree
+// of a node is the index in the top 16 bits of its key, and `any_kept` / `best` hold one entry
+// per octree.
+__global__ __launch_bounds__(kBlock) void trim_flag_kernel(int* __restrict__ drop_d, const int* __restrict__ drop_p,
+    const int* __restrict__ child_p, const int* __restrict__ child_d, const uint64_t* __restrict__ key_p,
+    const float* __restrict__ nerr, const float* __restrict__ derr, int n_p, int has_dis, float th_dist, float th_norm,
+    int* __restrict__ any_kept, unsigned long long* __restrict__ best) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n_p) return;
-  const int c = child_p[i];
-  if (c == -1) return;
-  const bool parent_kept = drop_p == nullptr || drop_p[i] == kKeep;
-  bool kept = false;
-  for (int j = 0; j < 8; ++j) {
-    const int idx = c * 8 + j;
-    int f = kKeep;
-    if (parent_kept) {
-      if ((!has_dis || derr[idx] < th_dist) && nerr[idx] < th_norm) f = kDropChildren;
-    } else {
-      f = kDrop;
+  const int c = i < n_p ? child_p[i] : -1;
+  const bool active = c != -1;
+  const int b = active ? (int)(key_p[i] >> 48) : -1;
+  // In case no non-empty node of the octree's level is kept, the candidate that is kept all the
+  // same: a non-empty child of a kept parent with the largest normal error, the first one on a
+  // tie (octree.cpp:1057-1073), as (error bits, ~index) so that one atomic maximum finds it.
+  unsigned long long cand = 0;
+  if (active) {
+    const bool parent_kept = drop_p == nullptr || drop_p[i] == kKeep;
+    bool kept = false;
+    for (int j = 0; j < 8; ++j) {
+      const int idx = c * 8 + j;
+      int f = kKeep;
+      const float e = nerr[idx];
+      if (parent_kept) {
+        if ((!has_dis || derr[idx] < th_dist) && e < th_norm) f = kDropChildren;
+      } else {
+        f = kDrop;
+      }
+      drop_d[idx] = f;
+      const bool inner = child_d[idx] != -1;
+      kept = kept || (f == kKeep && inner);
+      if (parent_kept && inner && e > -1.0f) {
+        const unsigned long long v = ((unsigned long long)__float_as_uint(e) << 32) | (unsigned long long)(0xffffffffu - (unsigned)idx);
+        cand = v > cand ? v : cand;
+      }
     }
-    drop_d[idx] = f;
-    kept = kept || (f == kKeep && child_d[idx] != -1);
+    if (kept) any_kept[b] = 1;
   }
-  if (kept) *any_kept = 1;
-}
-// if no non-empty node of the level was kept: the candidate with the largest normal error
-// (the first one on a tie) is found ...
-__global__ void trim_argmax_kernel(unsigned long long* __restrict__ best, const int* __restrict__ drop_p,
-    const int* __restrict__ child_p, const int* __restrict__ child_d, const float* __restrict__ nerr, int n_p,
-    const int* __restrict__ any_kept) {
-  if (*any_kept) return;
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n_p) return;
-  const int c = child_p[i];
-  if (c == -1 || (drop_p != nullptr && drop_p[i] != kKeep)) return;
-  for (int j = 0; j < 8; ++j) {
-    const int idx = c * 8 + j;
-    if (child_d[idx] == -1) continue;
-    const float e = nerr[idx];
-    if (!(e > -1.0f)) continue;
-    atomicMax(best, ((unsigned long long)__float_as_uint(e) << 32) | (unsigned long long)(0xffffffffu - (unsigned)idx));
+  // one atomic per wavefront where its nodes are of one octree (nearly always)
+  const unsigned long long act = __ballot(active);
+  if (act == 0) return;
+  const int b0 = __builtin_amdgcn_readlane(b, __builtin_ctzll(act));
+  if (__all(!active || b == b0)) {
+    unsigned long long m = cand;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const unsigned long long other = __shfl_xor(m, o, 64);
+      m = other > m ? other : m;
+    }
+    // both words only grow: a candidate that an earlier value already beats, or an octree that
+    // already has a kept node, needs no atomic (a stale read costs one atomic, never a result)
+    if ((threadIdx.x & 63) == 0 && m != 0 && any_kept[b0] == 0 && m > best[b0]) atomicMax(best + b0, m);
+  } else if (cand != 0) {
+    atomicMax(best + b, cand);
   }
 }
-// ... and kept
+// An octree without a kept non-empty node on the level keeps its candidate; without a candidate
+// it is the octree's first node of the level (max_idx starts at 0, octree.cpp:1059).  One thread
+// per octree.
 __global__ void trim_fix_kernel(int* __restrict__ drop_d, const unsigned long long* __restrict__ best,
-    const int* __restrict__ any_kept) {
-  if (*any_kept) return;
-  const unsigned long long b = *best;
-  const int idx = b == 0 ? 0 : (int)(0xffffffffu - (unsigned)(b & 0xffffffffull));
+    const int* __restrict__ any_kept, const uint64_t* __restrict__ key_d, int n_d, int n_octrees) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= n_octrees || any_kept[b]) return;
+  const unsigned long long v = best[b];
+  int idx;
+  if (v != 0) {
+    idx = (int)(0xffffffffu - (unsigned)(v & 0xffffffffull));
+  } else {   // the level's keys ascend with the octree index on top: first node of octree b
+    int lo = 0, hi = n_d;
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if ((int)(key_d[mid] >> 48) < b) lo = mid + 1; else hi = mid;
+    }
+    if (lo >= n_d || (int)(key_d[lo] >> 48) != b) return;   // the octree has no node here
+    idx = lo;
+  }
   drop_d[idx] = kKeep;
 }
 
-struct KeepPred {
-  const int* drop;
-  __device__ bool operator()(int64_t i) const { return drop[i] != kDrop; }
-};
-struct KeepOut {
-  int* pos;
-  __device__ void operator()(int64_t i, bool f, int rank) const { pos[i] = f ? rank : -1; }
-};
-struct LinkPred {
+// New positions of the kept nodes and new child links of every trimmed level in three launches
+// (tile counts, their prefix per level, ranks): a node stays unless its flag is kDrop, and keeps
+// its children if it is kKeep and has any.
+struct TrimScanLevel {
+  int n, first_tile;
   const int* drop; const int* child;
-  __device__ bool operator()(int64_t i) const { return drop[i] == kKeep && child[i] != -1; }
+  int* pos;        // new index, -1: dropped
+  int* nchild;     // new child link, -1: none
+  int* total_keep; int* total_link;
 };
-struct LinkOut {
-  const int* drop; int* nchild;
-  __device__ void operator()(int64_t i, bool f, int rank) const { nchild[i] = f ? rank : -1; }
+struct TrimScanLevels {
+  int n_levels, n_tiles;
+  int* tile_count;     // [2][n_tiles]: kept nodes, kept links
+  TrimScanLevel level[kMaxD];
 };
+__device__ inline int trim_scan_level(const TrimScanLevels& t, int tile) {
+  int l = 0;
+  while (l + 1 < t.n_levels && tile >= t.level[l + 1].first_tile) ++l;
+  return l;
+}
+__global__ __launch_bounds__(kBlock) void trim_count_kernel(const TrimScanLevels t) {
+  const TrimScanLevel& a = t.level[trim_scan_level(t, blockIdx.x)];
+  const int base = ((int)blockIdx.x - a.first_tile) * kScanTile + threadIdx.x * kScanItems;
+  int ck = 0, cl = 0;
+#pragma unroll
+  for (int j = 0; j < kScanItems; ++j) {
+    if (base + j >= a.n) continue;
+    const int f = a.drop[base + j];
+    ck += f != kDrop ? 1 : 0;
+    cl += (f == kKeep && a.child[base + j] != -1) ? 1 : 0;
+  }
+  int tk, tl;
+  block_exclusive_scan(ck, &tk);
+  block_exclusive_scan(cl, &tl);
+  if (threadIdx.x == 0) { t.tile_count[blockIdx.x] = tk; t.tile_count[t.n_tiles + blockIdx.x] = tl; }
+}
+// one workgroup per (level, count): tile counts -> exclusive offsets within the level, and the total
+__global__ __launch_bounds__(kBlock) void trim_tiles_kernel(const TrimScanLevels t) {
+  const int l = blockIdx.x >> 1, which = blockIdx.x & 1;
+  const TrimScanLevel& a = t.level[l];
+  const int n_tiles = (l + 1 < t.n_levels ? t.level[l + 1].first_tile : t.n_tiles) - a.first_tile;
+  int* tc = t.tile_count + which * t.n_tiles + a.first_tile;
+  __shared__ int carry;
+  if (threadIdx.x == 0) carry = 0;
+  __syncthreads();
+  for (int start = 0; start < n_tiles; start += kBlock) {
+    const int i = start + threadIdx.x;
+    const int v = i < n_tiles ? tc[i] : 0;
+    int total;
+    const int ex = block_exclusive_scan(v, &total);
+    const int c = carry;
+    if (i < n_tiles) tc[i] = c + ex;
+    __syncthreads();
+    if (threadIdx.x == 0) carry = c + total;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) *(which ? a.total_link : a.total_keep) = carry;
+}
+__global__ __launch_bounds__(kBlock) void trim_apply_kernel(const TrimScanLevels t) {
+  const TrimScanLevel& a = t.level[trim_scan_level(t, blockIdx.x)];
+  const int base = ((int)blockIdx.x - a.first_tile) * kScanTile + threadIdx.x * kScanItems;
+  bool fk[kScanItems], fl[kScanItems];
+  int ck = 0, cl = 0;
+#pragma unroll
+  for (int j = 0; j < kScanItems; ++j) {
+    fk[j] = fl[j] = false;
+    if (base + j < a.n) {
+      const int f = a.drop[base + j];
+      fk[j] = f != kDrop;
+      fl[j] = f == kKeep && a.child[base + j] != -1;
+    }
+    ck += fk[j] ? 1 : 0;
+    cl += fl[j] ? 1 : 0;
+  }
+  int total;
+  int rk = t.tile_count[blockIdx.x] + block_exclusive_scan(ck, &total);
+  int rl = t.tile_count[t.n_tiles + blockIdx.x] + block_exclusive_scan(cl, &total);
+#pragma unroll
+  for (int j = 0; j < kScanItems; ++j) {
+    if (base + j < a.n) {
+      a.pos[base + j] = fk[j] ? rk : -1;
+      a.nchild[base + j] = fl[j] ? rl : -1;
+    }
+    rk += fk[j] ? 1 : 0;
+    rl += fl[j] ? 1 : 0;
+  }
+}
 
 // ---- serialization (octree.cpp:907-956) -----------------------------------------------------
-struct GatherArgs {
-  int d, n_old, n_new, key2xyz, key_channel, adaptive_split;
+// every level in one launch: the table is a kernel argument (about 2 KB)
+struct GatherLevel {
+  int n_old, n_new;
   const int* pos;            // new index of an old node, -1: dropped; null: identity
   const int* nchild;         // new child link; null: the old one
   const uint64_t* key; const int* child;
   const float *normal, *dis, *feature, *label, *pt;   // per-level signals (null: not stored)
-  int cn, ch_dis, cf, cp;
   uint64_t* key_out; int* child_out; float* feature_out; float* label_out; float* split_out;
 };
-__global__ void gather_kernel(GatherArgs a) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+struct GatherLevels {
+  int first_block[kMaxD + 1];   // of level d; [depth + 1] = all blocks
+  int depth, key2xyz, key_channel, adaptive_split;
+  int cn, ch_dis, cf, cp;
+  GatherLevel level[kMaxD];
+};
+__global__ __launch_bounds__(kBlock) void gather_kernel(const GatherLevels g) {
+  int d = 0;
+  while (d < g.depth && (int)blockIdx.x >= g.first_block[d + 1]) ++d;
+  const GatherLevel& a = g.level[d];
+  const int i = ((int)blockIdx.x - g.first_block[d]) * kBlock + threadIdx.x;
   if (i >= a.n_old) return;
   const int k = a.pos ? a.pos[i] : i;
   if (k < 0) return;
   const int64_t no = a.n_old, nn = a.n_new;
   uint64_t key = a.key[i];
-  if (a.key2xyz) {  // Octree::key_to_xyz, octree.cpp:1137-1156
+  if (g.key2xyz) {  // Octree::key_to_xyz, octree.cpp:1137-1156
     uint32_t x, y, z;
-    morton_decode(key, a.d, &x, &y, &z);
-    key = (uint64_t)(x & 0xffff) | ((uint64_t)(y & 0xffff) << 16) | ((uint64_t)(z & 0xffff) << 32);
+    morton_decode(key, d, &x, &y, &z);
+    // the octree index of a batch stays in the top 16 bits (merge_octrees.cpp:126-131)
+    key = (uint64_t)(x & 0xffff) | ((uint64_t)(y & 0xffff) << 16) | ((uint64_t)(z & 0xffff) << 32) | (key & 0xffff000000000000ull);
   }
   a.key_out[k] = key;
-  if (a.key_channel == 2) a.key_out[nn + k] = 0;
+  if (g.key_channel == 2) a.key_out[nn + k] = 0;
   const int ch = a.nchild ? a.nchild[i] : a.child[i];
   a.child_out[k] = ch;
   float* f = a.feature_out;
   float nsum = 0.0f;
   if (f) {
-    for (int c = 0; c < a.cn; ++c) { const float v = a.normal[c * no + i]; f[c * nn + k] = v; if (c < 3) nsum = __fadd_rn(nsum, fabsf(v)); }
-    f += a.cn * nn;
-    for (int c = 0; c < a.ch_dis; ++c) f[c * nn + k] = a.dis[c * no + i];
-    f += a.ch_dis * nn;
-    for (int c = 0; c < a.cf; ++c) f[c * nn + k] = a.feature[c * no + i];
-    f += a.cf * nn;
-    for (int c = 0; c < a.cp; ++c) f[c * nn + k] = a.pt[c * no + i];
+    for (int c = 0; c < g.cn; ++c) { const float v = a.normal[c * no + i]; f[c * nn + k] = v; if (c < 3) nsum = __fadd_rn(nsum, fabsf(v)); }
+    f += g.cn * nn;
+    for (int c = 0; c < g.ch_dis; ++c) f[c * nn + k] = a.dis[c * no + i];
+    f += g.ch_dis * nn;
+    for (int c = 0; c < g.cf; ++c) f[c * nn + k] = a.feature[c * no + i];
+    f += g.cf * nn;
+    for (int c = 0; c < g.cp; ++c) f[c * nn + k] = a.pt[c * no + i];
   }
   if (a.label_out) a.label_out[k] = a.label[i];
   if (a.split_out) {  // calc_split_label, octree.cpp:1158-1178
     float s = 1.0f;
-    if (ch == -1) s = (a.adaptive_split && nsum != 0.0f) ? 2.0f : 0.0f;
+    if (ch == -1) s = (g.adaptive_split && nsum != 0.0f) ? 2.0f : 0.0f;
     a.split_out[k] = s;
   }
 }
-__global__ void header_kernel(uint32_t* __restrict__ dst, const uint32_t* __restrict__ src_words, int n) {
+struct HeaderWords { uint32_t w[OCNN_HEADER_BYTES / 4]; };
+__global__ void header_kernel(uint32_t* __restrict__ dst, const HeaderWords h) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) dst[i] = src_words[i];
+  if (i < OCNN_HEADER_BYTES / 4) dst[i] = h.w[i];
 }
 
 inline size_t al(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -721,11 +1037,15 @@ int adaptive_finish(const AdaptiveInput& in, ocnn_alloc_fn alloc, void* alloc_ct
   const size_t nP = ((size_t)o0.nnum[D] + 3) & ~(size_t)3;   // packed rows in whole 16-byte units
   const size_t o_rank = take(4 * nDp), o_nrmP = take(4 * 3 * nP + 16), o_ptP = take(4 * 3 * nP + 16);
   const size_t o_featP = take(4 * (size_t)(cf > 0 ? cf : 1) * nP + 16), o_labP = take(4 * nP + 16);
-  const size_t o_scan = take(scan_scratch_bytes(max_n));
-  const size_t o_counts = take(sizeof(int) * 64);      // [0..16] kept nodes, [17..33] kept links, [34..50] any_kept
-  const size_t o_best = take(sizeof(unsigned long long) * kMaxD);
-  const size_t o_hdr = take(OCNN_HEADER_BYTES);
-  const size_t o_levels = take(sizeof(SignalLevels));
+  size_t level_tiles = 0;
+  for (int d = 0; d <= D; ++d) level_tiles += (size_t)scan_tiles(o0.nnum[d]);
+  const size_t o_scan = take(std::max(scan_scratch_bytes(max_n), sizeof(int) * 2 * (level_tiles + 1)));
+  const int B = o0.batch_size;
+  OCNN_REQUIRE(B >= 1 && B <= 65535, OCNN_E_BADARG, "batch size %d", B);
+  const size_t o_counts = take(sizeof(int) * 64);      // [0..16] kept nodes, [17..33] kept links
+  const size_t o_any = take(sizeof(int) * kMaxD * (size_t)B);                    // [d * B + octree]
+  const size_t o_best = take(sizeof(unsigned long long) * kMaxD * (size_t)B);    // [d * B + octree]
+  const size_t o_hdr = take(256);   // end of the block that starts cleared
   char* ws = static_cast<char*>(alloc(off, alloc_ctx));
   OCNN_REQUIRE(ws, OCNN_E_BADARG, "the allocator returned no memory for %zu bytes of scratch", off);
   OCNN_REQUIRE((reinterpret_cast<uintptr_t>(ws) & 7) == 0, OCNN_E_BADARG, "scratch not 8-byte aligned");
@@ -762,17 +1082,26 @@ int adaptive_finish(const AdaptiveInput& in, ocnn_alloc_fn alloc, void* alloc_ct
     if (has_label) label[D] = reinterpret_cast<float*>(b0 + o0.ptr_dis(OCNN_LABEL, D));
   }
   int* d_counts = reinterpret_cast<int*>(ws + o_counts);
+  int* d_any = reinterpret_cast<int*>(ws + o_any);
   unsigned long long* d_best = reinterpret_cast<unsigned long long*>(ws + o_best);
 
   // ---- covered ranges and signals of every depth
-  for (int d = D; d >= 0; --d) {
-    const int n = o0.nnum[d];
-    cover_kernel<<<blocks_for(n), kBlock, 0, s>>>(dnum[d], didx[d], child[d], d < D ? dnum[d + 1] : nullptr,
-        d < D ? didx[d + 1] : nullptr, n, d == D ? 0 : (d == D - 1 ? 1 : 2));
+  {
+    const int nD1 = D >= 1 ? o0.nnum[D - 1] : 0;
+    if (nD1 > 0)
+      cover_first_kernel<<<blocks_for(nD1), kBlock, 0, s>>>(dnum[D - 1], didx[D - 1], child[D - 1], nerr[D], derr[D], nD1);
+    int d = D - 2;
+    for (; d >= 0 && o0.nnum[d] > 8192; --d)
+      cover_kernel<<<blocks_for(o0.nnum[d]), kBlock, 0, s>>>(dnum[d], didx[d], child[d], dnum[d + 1], didx[d + 1], o0.nnum[d]);
+    if (d >= 0) {
+      CoverTop t;
+      memset(&t, 0, sizeof(t));
+      t.d_top = d;
+      for (int q = 0; q <= d + 1; ++q) { t.n[q] = o0.nnum[q]; t.dnum[q] = dnum[q]; t.didx[q] = didx[q]; t.child[q] = child[q]; }
+      cover_top_kernel<<<1, 1024, 0, s>>>(t);
+    }
   }
   OCNN_LAUNCH_OK("cover");
-  fill_kernel<<<blocks_for(o0.nnum[D]), kBlock, 0, s>>>(nerr[D], o0.nnum[D], 1.0e20f);
-  fill_kernel<<<blocks_for(o0.nnum[D]), kBlock, 0, s>>>(derr[D], o0.nnum[D], 1.0e20f);
   int* rank_D = reinterpret_cast<int*>(ws + o_rank);
   float* nrm_P = reinterpret_cast<float*>(ws + o_nrmP);
   float* pt_P = reinterpret_cast<float*>(ws + o_ptP);
@@ -786,29 +1115,32 @@ int adaptive_finish(const AdaptiveInput& in, ocnn_alloc_fn alloc, void* alloc_ct
     OCNN_REQUIRE(e == hipSuccess, OCNN_E_HIP, "leaf scan: %s", hipGetErrorString(e));
   }
   {
-    SignalLevels* L = new SignalLevels;
-    memset(L, 0, sizeof(SignalLevels));
-    int waves = 0;
-    for (int d = 0; d < D; ++d) {
-      SignalArgs& a = L->level[d];
-      a.d = d; a.depth = D; a.n = o0.nnum[d]; a.nD = o0.nnum[D]; a.cf = cf; a.ch_dis = ch_dis;
+    SignalLevels L;
+    memset(&L, 0, sizeof(L));
+    static_assert(sizeof(SignalLevels) <= 2048, "the level table is passed as a kernel argument");
+    int waves = 0, threads = 0;
+    const int d_small = D - 2 > 0 ? D - 2 : 0;   // levels from here on: one thread per node
+    {
+      SignalArgs& a = L.common;
+      a.depth = D; a.nD = o0.nnum[D]; a.cf = cf; a.ch_dis = ch_dis;
       a.adp_layer = o0.adp_layer; a.calc_nerr = adaptive && cn; a.calc_derr = adaptive && P.node_dis && cn;
       a.imul = imul;
-      a.key = key[d]; a.child = child[d]; a.dnum = dnum[d]; a.didx = didx[d];
       a.child_D = child[D]; a.nrm_D = normal[D]; a.pt_D = pt[D]; a.feat_D = feature[D]; a.lab_D = label[D];
       a.rank_D = rank_D; a.nrm_P = nrm_P; a.pt_P = pt_P; a.feat_P = feat_P; a.lab_P = lab_P; a.nP = (int64_t)nP;
-      a.normal = normal[d]; a.pt = pt[d]; a.feature = feature[d]; a.label = label[d]; a.dis = dis[d];
-      a.nerr = nerr[d]; a.derr = derr[d];
-      L->first_wave[d] = waves;
-      waves += a.n;
     }
-    for (int d = D; d <= kMaxD; ++d) L->first_wave[d] = waves;
-    hipError_t e = hipMemcpyAsync(ws + o_levels, L, sizeof(SignalLevels), hipMemcpyHostToDevice, s);
-    if (e == hipSuccess) e = hipStreamSynchronize(s);   // the table is host memory of this call
-    delete L;
-    OCNN_REQUIRE(e == hipSuccess, OCNN_E_HIP, "level table: %s", hipGetErrorString(e));
-    if (waves > 0)
-      signal_kernel<<<blocks_for((int64_t)waves * 64), kBlock, 0, s>>>(reinterpret_cast<const SignalLevels*>(ws + o_levels), D);
+    for (int d = 0; d < D; ++d) {
+      SignalLevel& l = L.level[d];
+      l.n = o0.nnum[d];
+      l.key = key[d]; l.child = child[d]; l.dnum = dnum[d]; l.didx = didx[d];
+      l.normal = normal[d]; l.pt = pt[d]; l.feature = feature[d]; l.label = label[d]; l.dis = dis[d];
+      l.nerr = nerr[d]; l.derr = derr[d];
+      L.first_wave[d] = waves;
+      L.first_thread[d] = threads;
+      if (d < d_small) waves += l.n; else threads += l.n;
+    }
+    for (int d = D; d <= kMaxD; ++d) { L.first_wave[d] = waves; L.first_thread[d] = threads; }
+    if (waves > 0) signal_kernel<<<blocks_for((int64_t)waves * 64), kBlock, 0, s>>>(L, D);
+    if (threads > 0) signal_small_kernel<<<blocks_for(threads), kBlock, 0, s>>>(L, D);
   }
   OCNN_LAUNCH_OK("signal");
 
@@ -817,6 +1149,7 @@ int adaptive_finish(const AdaptiveInput& in, ocnn_alloc_fn alloc, void* alloc_ct
     for (int d = D; d >= fl; --d) {
       ExtrapolateArgs a;
       a.n = o0.nnum[d]; a.cf = cf; a.has_dis = ch_dis != 0; a.imul = imul; a.d = d; a.key2xyz = P.key2xyz ? 1 : 0;
+      a.per_octree = (d <= fl && a.n >= B) ? a.n / B : (a.n > 0 ? a.n : 1);
       a.key = key[d]; a.child = child[d]; a.normal = normal[d]; a.feature = feature[d]; a.label = label[d]; a.dis = dis[d];
       extrapolate_kernel<<<blocks_for((a.n + 7) / 8), kBlock, 0, s>>>(a);
     }
@@ -837,30 +1170,42 @@ int adaptive_finish(const AdaptiveInput& in, ocnn_alloc_fn alloc, void* alloc_ct
   o.set_channel(OCNN_FEATURE, cn + out_dis + cf + out_pt);
   o.set_location(OCNN_FEATURE, -1);
   if (has_label) o.set_property(OCNN_LABEL, 1, -1);
+  if (in.merged) {   // the header of merge_octrees (merge_octrees.cpp:92-107): neighbour tables at every depth
+    OCNN_REQUIRE(o.channel(OCNN_KEY) == 1, OCNN_E_UNSUPPORTED, "octree_batch of two-channel keys (key2xyz with depth > 8)");
+    o.set_property(OCNN_NEIGH, 8, -1);
+  }
   const int A = o.adp_layer;
   if (adaptive) {
     OCNN_REQUIRE(A >= 1 && A <= D, OCNN_E_BADARG, "adp_depth %d", A);
     for (int d = A; d <= D; ++d) {
       const int n_p = o0.nnum[d - 1];
       const int* drop_p = d - 1 >= A ? drop[d - 1] : nullptr;
-      int* any_kept = d_counts + 34 + d;
+      int* any_kept = d_any + (size_t)d * B;
       // nodes whose parent is empty do not exist; every node of level d has a flag after this
-      trim_flag_kernel<<<blocks_for(n_p), kBlock, 0, s>>>(drop[d], drop_p, child[d - 1], child[d], nerr[d], derr[d], n_p,
-          P.node_dis ? 1 : 0, P.th_distance, P.th_normal, any_kept);
-      trim_argmax_kernel<<<blocks_for(n_p), kBlock, 0, s>>>(d_best + d, drop_p, child[d - 1], child[d], nerr[d], n_p, any_kept);
-      trim_fix_kernel<<<1, 1, 0, s>>>(drop[d], d_best + d, any_kept);
+      trim_flag_kernel<<<blocks_for(n_p), kBlock, 0, s>>>(drop[d], drop_p, child[d - 1], child[d], key[d - 1], nerr[d],
+          derr[d], n_p, P.node_dis ? 1 : 0, P.th_distance, P.th_normal, any_kept, d_best + (size_t)d * B);
+      trim_fix_kernel<<<blocks_for(B), kBlock, 0, s>>>(drop[d], d_best + (size_t)d * B, any_kept, key[d], o0.nnum[d], B);
     }
     OCNN_LAUNCH_OK("trim flags");
-    for (int d = A; d <= D; ++d) {
-      const int n = o0.nnum[d];
-      KeepPred kp{drop[d]};
-      KeepOut ko{pos[d]};
-      hipError_t e = flag_scan(kp, ko, (int64_t)n, reinterpret_cast<int*>(ws + o_scan), d_counts + d, s);
-      OCNN_REQUIRE(e == hipSuccess, OCNN_E_HIP, "keep scan: %s", hipGetErrorString(e));
-      LinkPred lp{drop[d], child[d]};
-      LinkOut lo{drop[d], nchild[d]};
-      e = flag_scan(lp, lo, (int64_t)n, reinterpret_cast<int*>(ws + o_scan), d_counts + 17 + d, s);
-      OCNN_REQUIRE(e == hipSuccess, OCNN_E_HIP, "link scan: %s", hipGetErrorString(e));
+    {
+      TrimScanLevels t;
+      memset(&t, 0, sizeof(t));
+      static_assert(sizeof(TrimScanLevels) <= 2048, "the level table is passed as a kernel argument");
+      int tiles = 0;
+      for (int d = A; d <= D; ++d) {
+        TrimScanLevel& l = t.level[t.n_levels++];
+        l.n = o0.nnum[d]; l.first_tile = tiles;
+        l.drop = drop[d]; l.child = child[d]; l.pos = pos[d]; l.nchild = nchild[d];
+        l.total_keep = d_counts + d; l.total_link = d_counts + 17 + d;
+        tiles += scan_tiles(l.n);
+      }
+      t.n_tiles = tiles;
+      t.tile_count = reinterpret_cast<int*>(ws + o_scan);
+      if (tiles > 0) {
+        trim_count_kernel<<<tiles, kBlock, 0, s>>>(t);
+        trim_tiles_kernel<<<2 * t.n_levels, kBlock, 0, s>>>(t);
+        trim_apply_kernel<<<tiles, kBlock, 0, s>>>(t);
+      }
     }
     int h[64];
     OCNN_HIP_OK(hipMemcpyAsync(h, d_counts, sizeof(h), hipMemcpyDeviceToHost, s));
@@ -877,35 +1222,55 @@ int adaptive_finish(const AdaptiveInput& in, ocnn_alloc_fn alloc, void* alloc_ct
   OCNN_REQUIRE((reinterpret_cast<uintptr_t>(out) & 7) == 0, OCNN_E_BADARG, "blob not 8-byte aligned");
   *blob_out = out;
   {
-    uint32_t hdr[OCNN_HEADER_BYTES / 4];
-    memset(hdr, 0, sizeof(hdr));
-    memcpy(hdr, &o, sizeof(Info));
-    // the words travel through the scratch block: a kernel argument of 720 bytes per launch
-    // would do as well, but this launch is not on any critical path
-    OCNN_HIP_OK(hipMemcpyAsync(ws + o_hdr, hdr, sizeof(hdr), hipMemcpyHostToDevice, s));
-    OCNN_HIP_OK(hipStreamSynchronize(s));   // `hdr` lives on this stack frame
-    header_kernel<<<1, kBlock, 0, s>>>(reinterpret_cast<uint32_t*>(out), reinterpret_cast<const uint32_t*>(ws + o_hdr),
-        OCNN_HEADER_BYTES / 4);
+    HeaderWords hdr;   // 720 bytes as a kernel argument: no copy, no wait
+    memset(&hdr, 0, sizeof(hdr));
+    memcpy(&hdr, &o, sizeof(Info));
+    header_kernel<<<1, kBlock, 0, s>>>(reinterpret_cast<uint32_t*>(out), hdr);
   }
-  for (int d = 0; d <= D; ++d) {
-    const bool trimmed = adaptive && d >= A;
-    GatherArgs g;
+  {
+    GatherLevels g;
     memset(&g, 0, sizeof(g));
-    g.d = d; g.n_old = o0.nnum[d]; g.n_new = o.nnum[d]; g.key2xyz = o.key2xyz; g.key_channel = o.channel(OCNN_KEY);
-    g.adaptive_split = adaptive ? 1 : 0;
-    g.pos = trimmed ? pos[d] : nullptr;
-    g.nchild = trimmed ? nchild[d] : nullptr;
-    g.key = key[d]; g.child = child[d];
-    g.normal = normal[d]; g.dis = dis[d]; g.feature = feature[d]; g.label = label[d]; g.pt = pt[d];
+    static_assert(sizeof(GatherLevels) <= 3072, "the level table is passed as a kernel argument");
+    g.depth = D; g.key2xyz = o.key2xyz; g.key_channel = o.channel(OCNN_KEY); g.adaptive_split = adaptive ? 1 : 0;
     g.cn = cn; g.ch_dis = out_dis; g.cf = cf; g.cp = out_pt;
-    g.key_out = reinterpret_cast<uint64_t*>(out + o.ptr_dis(OCNN_KEY, d));
-    g.child_out = reinterpret_cast<int*>(out + o.ptr_dis(OCNN_CHILD, d));
-    g.feature_out = o.channel(OCNN_FEATURE) > 0 ? reinterpret_cast<float*>(out + o.ptr_dis(OCNN_FEATURE, d)) : nullptr;
-    g.label_out = o.has(OCNN_LABEL) ? reinterpret_cast<float*>(out + o.ptr_dis(OCNN_LABEL, d)) : nullptr;
-    g.split_out = o.has(OCNN_SPLIT) ? reinterpret_cast<float*>(out + o.ptr_dis(OCNN_SPLIT, d)) : nullptr;
-    if (g.n_old > 0) gather_kernel<<<blocks_for(g.n_old), kBlock, 0, s>>>(g);
+    int blocks = 0;
+    for (int d = 0; d <= D; ++d) {
+      const bool trimmed = adaptive && d >= A;
+      GatherLevel& l = g.level[d];
+      l.n_old = o0.nnum[d]; l.n_new = o.nnum[d];
+      l.pos = trimmed ? pos[d] : nullptr;
+      l.nchild = trimmed ? nchild[d] : nullptr;
+      l.key = key[d]; l.child = child[d];
+      l.normal = normal[d]; l.dis = dis[d]; l.feature = feature[d]; l.label = label[d]; l.pt = pt[d];
+      l.key_out = reinterpret_cast<uint64_t*>(out + o.ptr_dis(OCNN_KEY, d));
+      l.child_out = reinterpret_cast<int*>(out + o.ptr_dis(OCNN_CHILD, d));
+      l.feature_out = o.channel(OCNN_FEATURE) > 0 ? reinterpret_cast<float*>(out + o.ptr_dis(OCNN_FEATURE, d)) : nullptr;
+      l.label_out = o.has(OCNN_LABEL) ? reinterpret_cast<float*>(out + o.ptr_dis(OCNN_LABEL, d)) : nullptr;
+      l.split_out = o.has(OCNN_SPLIT) ? reinterpret_cast<float*>(out + o.ptr_dis(OCNN_SPLIT, d)) : nullptr;
+      g.first_block[d] = blocks;
+      blocks += (int)blocks_for(l.n_old);
+    }
+    for (int d = D + 1; d <= kMaxD; ++d) g.first_block[d] = blocks;
+    if (blocks > 0) gather_kernel<<<blocks, kBlock, 0, s>>>(g);
   }
   OCNN_LAUNCH_OK("serialize");
+  if (in.merged) {
+    // neighbour tables of the final structure (merge_octrees.cpp:185-197); the root level has
+    // none and stays zero as in the reference's zero-initialised buffer
+    fill_kernel<<<blocks_for((int64_t)o.nnum[0] * 8), kBlock, 0, s>>>(
+        reinterpret_cast<float*>(out + o.ptr_dis(OCNN_NEIGH, 0)), (int64_t)o.nnum[0] * 8, 0.0f);
+    for (int d = 1; d <= D; ++d) {
+      int* neigh = reinterpret_cast<int*>(out + o.ptr_dis(OCNN_NEIGH, d));
+      if (d <= fl) {
+        const int e = ocnn_calc_neigh_full(neigh, d, B, s);
+        if (e) return e;
+      } else if (o.nnum[d - 1] > 0) {
+        launch_neigh_sparse(neigh, reinterpret_cast<const int*>(out + o.ptr_dis(OCNN_NEIGH, d - 1)),
+            reinterpret_cast<const int*>(out + o.ptr_dis(OCNN_CHILD, d - 1)), o.nnum[d - 1], s, o.nnum[d] / 8);
+      }
+    }
+    OCNN_LAUNCH_OK("neighbours");
+  }
   return OCNN_OK;
 }
 

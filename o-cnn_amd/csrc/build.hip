@@ -50,6 +50,7 @@ struct CloudDesc {
 };
 
 constexpr int kMaxLevels = 17;
+constexpr int kMergedNoNeigh = 2;   // ocnn_build_params::merged: batch layout, no neighbour tables (first stage of a two-stage build)
 constexpr int kMaxPasses = 8;
 constexpr uint32_t kFlagSum = 1u << 30;    // status word: published (the count is in the low bits)
 constexpr uint32_t kCountMask = (1u << 30) - 1;
@@ -1291,7 +1292,7 @@ int ocnn_points2octree_plan(const void* const* points_dev, const void* const* po
   }
   if (params->merged) {
     o.set_batch_size(n_clouds);
-    o.set_property(OCNN_NEIGH, 8, -1);
+    if (params->merged != kMergedNoNeigh) o.set_property(OCNN_NEIGH, 8, -1);
   }
   o.set_nnum_cum();
   OCNN_REQUIRE(o.set_ptr_dis(), OCNN_E_SHAPE,
@@ -1463,10 +1464,13 @@ int ocnn_points2octree(const void* const* points_dev, const void* const* points_
     void* alloc_ctx, void* info_out, void** octree_out_dev, ocnn_stream_t stream) {
   OCNN_REQUIRE(alloc && octree_out_dev && params && points_info && points_dev, OCNN_E_BADARG, "null pointer");
   if (params->node_feature || params->adaptive) {
-    // Signals at every depth / trimming: a plain single octree first (raw Morton keys, average
-    // points kept whenever the displacement is), then the second stage on top of it.
-    OCNN_REQUIRE(n_clouds == 1 && !params->merged, OCNN_E_UNSUPPORTED,
-        "node_feature / adaptive octrees are built one cloud at a time (batch them with ocnn_octree_batch)");
+    // Signals at every depth / trimming: a plain octree first (raw Morton keys, average points
+    // kept whenever the displacement is), then the second stage on top of it.  A batch goes
+    // through both stages as ONE octree in merged layout: every step of the second stage works
+    // within a sibling group or over a node's own leaves, except the trimming rule that keeps
+    // one node per level, which is applied per octree (the index in the top bits of the keys).
+    OCNN_REQUIRE(params->merged == 0 || params->merged == 1, OCNN_E_BADARG, "merged %d", params->merged);
+    OCNN_REQUIRE(n_clouds == 1 || params->merged, OCNN_E_BADARG, "a single-octree blob holds one cloud");
     const PointsInfo* pi = static_cast<const PointsInfo*>(points_info[0]);
     OCNN_REQUIRE(pi, OCNN_E_BADARG, "null cloud header");
     const bool has_normal = (pi->content_flags & 2) != 0;
@@ -1477,8 +1481,10 @@ int ocnn_points2octree(const void* const* points_dev, const void* const* points_
     ocnn_build_params p0 = *params;
     p0.node_feature = p0.adaptive = p0.key2xyz = p0.split_label = p0.extrapolate = 0;
     p0.save_pts = (params->node_dis || params->save_pts) ? 1 : 0;
+    p0.merged = params->merged ? kMergedNoNeigh : 0;   // the first stage's neighbour tables would be thrown away
     AdaptiveInput in;
-    int e = ocnn_points2octree_plan(points_dev, points_info, 1, &p0, workspace_dev, workspace_bytes, &in.info0, stream);
+    in.merged = params->merged ? 1 : 0;
+    int e = ocnn_points2octree_plan(points_dev, points_info, n_clouds, &p0, workspace_dev, workspace_bytes, &in.info0, stream);
     if (e != OCNN_OK) return e;
     in.blob0 = static_cast<char*>(alloc((size_t)in.info0.sizeof_octree(), alloc_ctx));
     if (!in.blob0) {

@@ -8,8 +8,11 @@
 namespace ocnn {
 
 struct AdaptiveInput {
-  char* blob0;          // device: single octree, raw Morton keys, finest-level signal
+  char* blob0;          // device: first-stage octree (one cloud, or a batch in merged layout:
+                        //         octree index in the top 16 bits of the keys, child links
+                        //         counted over the batch), raw Morton keys, finest-level signal
                         //         normals | displacement | features | average points
+  int merged;           // 0: single-octree blob out; 1: octree_batch blob out (neighbour tables)
   Info info0;           // its header (host)
   int ch_normal, ch_feature, ch_dis, has_pt, has_label;
   ocnn_build_params params;   // what the caller asked for

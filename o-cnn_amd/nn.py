@@ -165,58 +165,9 @@ _ALLOC_FN = C.CFUNCTYPE(C.c_void_p, C.c_size_t, C.c_void_p)
 
 _blob_bytes_per_point = {}   # build settings -> bytes of blob per input point, from earlier builds
 
-_LANES = 4          # concurrent single-cloud builds: one per hardware queue of the process
-_lane_state = {}
-
-
-def _lanes(device):
-  """Side streams (default priority) and the worker threads that feed them, per device."""
-  st = _lane_state.get(device)
-  if st is None:
-    from concurrent.futures import ThreadPoolExecutor
-    st = ([torch.cuda.Stream(device=device) for _ in range(_LANES)], ThreadPoolExecutor(_LANES))
-    _lane_state[device] = st
-  return st
-
-
-def _build_each(points_list, args):
-  """Single-cloud builds of a list of clouds.  Such a build is a chain of small launches with
-  waits for node counts in between, bound by latency and not by the device: the clouds are dealt
-  over side streams, each fed by its own host thread (the C calls release the interpreter lock),
-  and the current stream takes the results when all are done."""
-  n = len(points_list)
-  if n < 2:
-    return [_build([p], False, *args) for p in points_list]
-  device = torch.cuda.current_device()
-  cur = torch.cuda.current_stream()
-  streams, pool = _lanes(device)
-  lanes = min(_LANES, n)
-  for st in streams[:lanes]:
-    st.wait_stream(cur)
-
-  def lane(k):
-    torch.cuda.set_device(device)
-    with torch.cuda.stream(streams[k]):
-      return [_build([points_list[i]], False, *args, ws_tag="build-lane%d" % k) for i in range(k, n, lanes)]
-
-  done = list(pool.map(lane, range(lanes)))
-  out = [None] * n
-  for k in range(lanes):
-    cur.wait_stream(streams[k])
-    for j, blob in enumerate(done[k]):
-      blob.record_stream(cur)     # allocated on the side stream, used on the current one from here on
-      out[k + j * lanes] = blob
-  return out
-
 
 def _build(points_list, merged, depth, full_depth, node_dis, node_feature, split_label, adaptive,
            adp_depth, th_normal, th_distance, extrapolate, save_pts, key2xyz, bbox=None, ws_tag="build"):
-  if merged and (node_feature or adaptive):
-    # octrees with a signal at every depth are built one cloud at a time and merged afterwards,
-    # as collate_octrees does (pytorch/ocnn/transforms.py:127-148)
-    return octree_batch(_build_each(list(points_list), (depth, full_depth, node_dis, node_feature, split_label,
-                                                        adaptive, adp_depth, th_normal, th_distance, extrapolate,
-                                                        save_pts, key2xyz, bbox)))
   pts = [_to_dev(p) for p in points_list]
   hdrs = [getattr(p, "_ocnn_points_info", None) for p in points_list]
   for i, h in enumerate(hdrs):

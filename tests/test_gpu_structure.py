@@ -263,6 +263,39 @@ def test_adaptive_build_vs_oracle(oc, orc, case):
     assert got.size == exp.size and np.array_equal(got, exp), (trial, n, depth, fd, extra, kw)
 
 
+@pytest.mark.parametrize("case", range(len(ADAPTIVE_CASES)))
+def test_adaptive_batch_in_one_pass_vs_oracle(oc, orc, case):
+  """A batch of clouds through both stages of the builder as ONE octree in merged layout: the
+  blob equals merge_octrees over the octrees the oracle builds cloud by cloud.  The clouds
+  differ in size and smoothness, so with the loose thresholds some octrees of a batch fall
+  under the "keep one node per level" rule of trim_octree (octree.cpp:1055-1073) and others do
+  not: that rule is the one step that is taken per octree."""
+  kw = ADAPTIVE_CASES[case]   # depth <= 7 below: one key channel also with key2xyz, which merge_octrees needs
+  rng = np.random.default_rng(900 + case)
+  for trial in range(4):
+    n_clouds = int(rng.integers(2, 6))
+    depth = int(rng.integers(4, 8))
+    fd = int(rng.integers(1, 3))
+    extra = dict(adp_depth=int(rng.integers(fd + 1, depth + 1)), th_normal=float(rng.choice([0.1, 0.3, 5.0])),
+                 th_distance=float(rng.choice([0.5, 2.0, 3.0])))
+    pbs = []
+    for c in range(n_clouds):
+      n = int(rng.integers(1, 40)) if (trial == 3 and c == 1) else int(rng.integers(200, 5000))
+      pts, nrm = smooth_cloud(rng, n, int(rng.integers(0, 2)))
+      if c % 2 == 1:   # a rough cloud next to the smooth ones
+        nrm = rng.standard_normal((n, 3)).astype(np.float32)
+        nrm /= np.linalg.norm(nrm, axis=1, keepdims=True)
+      feat = rng.uniform(0, 1, (n, 2)).astype(np.float32) if trial >= 2 else None
+      lab = rng.integers(-1, 4, n).astype(np.float32) if trial >= 3 else None
+      pbs.append(make_points_blob(pts, nrm, feat, lab))
+    got = oc.nn.points2octree_batch([T(pb) for pb in pbs], depth, fd, **extra, **kw).cpu().numpy()
+    exp = orc.octree_batch([orc.points2octree(pb, depth, fd, **extra, **kw) for pb in pbs])
+    assert got.size == exp.size and np.array_equal(got, exp), (trial, n_clouds, depth, fd, extra, kw)
+    if trial == 0:   # a batch of one is still a batch blob (neighbour tables, batch header)
+      one = oc.nn.points2octree_batch([T(pbs[0])], depth, fd, **extra, **kw).cpu().numpy()
+      assert np.array_equal(one, orc.octree_batch([orc.points2octree(pbs[0], depth, fd, **extra, **kw)]))
+
+
 def test_adaptive_golden_and_config5_on_gpu(oc, synthetic, hashes):
   """The committed hashes were written from the compiled reference: one small adaptive octree
   and BASELINE config 5's input (16 adaptive octrees at depth 7, merged), built on the device."""
