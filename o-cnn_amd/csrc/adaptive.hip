@@ -161,34 +161,43 @@ __device__ inline int intersect_cube(float* V, const float* pt, const float* pt_
 constexpr int kPassValues = 8, kPassLeaves = 256;
 template <int NV>
 __device__ inline void ordered_sums(int k0, int k1, int lane, float* __restrict__ lds, const float* const (&row)[NV],
-    float* sum, float* last) {
+    const float* __restrict__ any_row, int64_t row_len, float* sum, float* last) {
   static_assert(NV <= kPassValues, "LDS block too small");
   float acc = 0.0f;
   constexpr int kAhead = 3;      // blocks requested before they are needed
   float4 vals[kAhead][NV];
-  auto request = [&](float4 (&dst)[NV], int base) {
+  // Every request issues the same NV loads whatever the range (an absent row reads `any_row`,
+  // a block past the end reads the last four values of the row, both become zeros): the number
+  // of loads in flight behind a block is then a constant, and waiting for one block does not
+  // wait for the blocks requested after it.
+  const int k_last = (int)row_len - 4;
+  auto request = [&](float4 (&dst)[NV], int base) {   // loads only: nothing here waits for them
+    const int kk = min(base + 4 * lane, k_last);
+#pragma unroll
+    for (int c = 0; c < NV; ++c) dst[c] = *reinterpret_cast<const float4*>((row[c] ? row[c] : any_row) + kk);
+  };
+  auto stage = [&](const float4 (&raw)[NV], int base) {   // a block's values, zeros outside the range, to LDS
     const int k = base + 4 * lane;
 #pragma unroll
     for (int c = 0; c < NV; ++c) {
-      float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-      if (row[c] && k < k1) v = *reinterpret_cast<const float4*>(row[c] + k);
-      v.x = (k >= k0 && k < k1) ? v.x : 0.0f;
-      v.y = (k + 1 >= k0 && k + 1 < k1) ? v.y : 0.0f;
-      v.z = (k + 2 >= k0 && k + 2 < k1) ? v.z : 0.0f;
-      v.w = (k + 3 >= k0 && k + 3 < k1) ? v.w : 0.0f;
-      dst[c] = v;
+      const bool have = row[c] != nullptr;
+      float4 v = raw[c];
+      v.x = (have && k >= k0 && k < k1) ? v.x : 0.0f;
+      v.y = (have && k + 1 >= k0 && k + 1 < k1) ? v.y : 0.0f;
+      v.z = (have && k + 2 >= k0 && k + 2 < k1) ? v.z : 0.0f;
+      v.w = (have && k + 3 >= k0 && k + 3 < k1) ? v.w : 0.0f;
+      *reinterpret_cast<float4*>(lds + c * kPassLeaves + 4 * lane) = v;
     }
-  };
-  auto add_block = [&](const float4 (&cur_vals)[NV], int base) {
-#pragma unroll
-    for (int c = 0; c < NV; ++c) *reinterpret_cast<float4*>(lds + c * kPassLeaves + 4 * lane) = cur_vals[c];
     __builtin_amdgcn_wave_barrier();   // same wavefront: the LDS unit keeps its accesses in order
+  };
+  auto chain = [&](int base) {
     const int total = min(kPassLeaves, k1 - base);
     if (lane < NV) {
       // the adds form one dependent chain, and one wavefront issues an instruction every few
       // cycles: nothing but the adds and the LDS reads may sit in the loop.  Two register sets
       // take turns (the reads of the next 32 leaves are in flight while the current 32 are
-      // added, an LDS read takes longer than 16 adds), every offset is a constant.
+      // added, an LDS read takes longer than 16 adds; the scheduler is told to keep that
+      // order), every offset is a constant.
       constexpr int kStep = 32, kChunks = kPassLeaves / kStep;
       const float4* src = reinterpret_cast<const float4*>(lds + lane * kPassLeaves);
       float4 ra[kStep / 4], rb[kStep / 4];
@@ -208,29 +217,35 @@ __device__ inline void ordered_sums(int k0, int k1, int lane, float* __restrict_
       for (int ch = 0; ch < kChunks; ch += 2) {
         if (ch * kStep >= total) break;
         read(rb, ch + 1);
+        __builtin_amdgcn_sched_barrier(0);
         add(ra);
+        __builtin_amdgcn_sched_barrier(0);
         if ((ch + 1) * kStep >= total) break;
         if (ch + 2 < kChunks) read(ra, ch + 2);
+        __builtin_amdgcn_sched_barrier(0);
         add(rb);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
     __builtin_amdgcn_wave_barrier();
   };
-  const int kb = k0 < k1 ? (k0 & ~3) : k1;   // an empty range runs no block
-#pragma unroll
-  for (int u = 0; u < kAhead; ++u)
-    if (kb + u * kPassLeaves < k1) request(vals[u], kb + u * kPassLeaves);
-  for (int base = kb; base < k1; base += kAhead * kPassLeaves) {
+  if (k0 < k1) {
+    const int kb = k0 & ~3;
 #pragma unroll
     for (int u = 0; u < kAhead; ++u) {
-      const int b = base + u * kPassLeaves;
-      if (b < k1) {
-        // a block's registers are free once it sits in LDS: the block kAhead further on takes them
-        float4 now[NV];
+      request(vals[u], kb + u * kPassLeaves);
+      __builtin_amdgcn_sched_barrier(0);   // block after block, as in the loop: the wait below counts on the order
+    }
+    // kAhead blocks a turn, without a way out in between (a block past the end adds nothing):
+    // straight-line code keeps the count of loads in flight a constant
+    for (int base = kb; base < k1; base += kAhead * kPassLeaves) {
 #pragma unroll
-        for (int c = 0; c < NV; ++c) now[c] = vals[u][c];
-        if (b + kAhead * kPassLeaves < k1) request(vals[u], b + kAhead * kPassLeaves);
-        add_block(now, b);
+      for (int u = 0; u < kAhead; ++u) {
+        const int b = base + u * kPassLeaves;
+        stage(vals[u], b);
+        request(vals[u], b + kAhead * kPassLeaves);   // its registers are free once the block sits in LDS
+        __builtin_amdgcn_sched_barrier(0);
+        chain(b);
       }
     }
   }
@@ -302,6 +317,7 @@ struct SignalArgs {
   const float *nrm_D, *pt_D, *feat_D, *lab_D;
   const int* rank_D;          // non-empty leaves before a leaf; [nD] = their number
   const float *nrm_P, *pt_P, *feat_P, *lab_P;   // the non-empty leaves packed in leaf order, rows of nP
+  const float* any_P;         // nP floats that may be read (whatever they hold)
   int64_t nP;
   float *normal, *pt, *feature, *label, *dis, *nerr, *derr;   // level d (null: absent)
 };
@@ -369,7 +385,7 @@ __global__ __launch_bounds__(kBlock) void signal_kernel(const SignalLevels level
     const float* const rows6[6] = {has_normal ? a.nrm_P : nullptr, has_normal ? a.nrm_P + nP : nullptr,
         has_normal ? a.nrm_P + 2 * nP : nullptr, has_pt ? a.pt_P : nullptr, has_pt ? a.pt_P + nP : nullptr,
         has_pt ? a.pt_P + 2 * nP : nullptr};
-    ordered_sums<6>(k0, k1, lane, lds, rows6, sum6, last6);
+    ordered_sums<6>(k0, k1, lane, lds, rows6, a.any_P, nP, sum6, last6);
   }
   for (int c = 0; c < 3; ++c) { n_avg[c] = sum6[c]; last_n[c] = last6[c]; pt_avg[c] = sum6[3 + c]; }
   if (has_normal) {
@@ -392,7 +408,7 @@ __global__ __launch_bounds__(kBlock) void signal_kernel(const SignalLevels level
     const int nc = min(kPassValues, a.cf - c0);
     const float* rows8[kPassValues];
     for (int c = 0; c < kPassValues; ++c) rows8[c] = c < nc ? a.feat_P + (c0 + c) * nP : nullptr;
-    ordered_sums<kPassValues>(k0, k1, lane, lds, rows8, fsum, flast);
+    ordered_sums<kPassValues>(k0, k1, lane, lds, rows8, a.any_P, nP, fsum, flast);
     if (lane == 0)
       for (int c = 0; c < kPassValues; ++c) if (c < nc) a.feature[(c0 + c) * n + i] = div_rn(fsum[c], count);
   }
@@ -496,22 +512,65 @@ __global__ __launch_bounds__(kBlock) void signal_kernel(const SignalLevels level
       for (int k = 0; k < nv; ++k) {
         float vk[3];
         for (int c = 0; c < 3; ++c) vk[c] = __fmul_rn(vtx[3 * k + c], scale);
-        float distance_min = 1.0e30f;
+        // the correctly rounded root is monotonic: the smallest root is the root of the smallest square
+        float sq_min = __builtin_inff();   // (no leaf, or only infinite squares: 1.0e30f as before)
         for (int k = k0 + lane; k < k1; k += 64) {
           float dis = 0.0f;
           for (int c = 0; c < 3; ++c) {
             const float ptc = __fsub_rn(a.pt_P[c * nP + k], vk[c]);
             dis = __fadd_rn(dis, __fmul_rn(ptc, ptc));
           }
-          distance_min = fminf(distance_min, sqrt_rn(dis));
+          sq_min = fminf(sq_min, dis);
         }
-        distance_min = wave_min(distance_min);
+        sq_min = wave_min(sq_min);
+        const float distance_min = fminf(1.0e30f, sqrt_rn(sq_min));
         if (distance_min > distance_max2) distance_max2 = distance_min;
       }
       err = distance_max2 > distance_max1 ? distance_max2 : distance_max1;
     }
     if (lane == 0) a.derr[i] = err;
   }
+}
+
+// intersect_cube for one thread: the same vertices in the same order, kept in registers (every
+// index below is a constant once the loops are unrolled; a vertex goes to slot `nv` through
+// selects).  At most six edges of a cube are cut by a plane.
+__device__ inline int intersect_cube_regs(float (&vx)[6], float (&vy)[6], float (&vz)[6], const float* pt,
+    const float* pt_base, const float* normal) {
+  constexpr float kC[8][3] = {{0, 0, 0}, {0, 0, 1}, {0, 1, 1}, {0, 1, 0}, {1, 0, 0}, {1, 0, 1}, {1, 1, 1}, {1, 1, 0}};
+  constexpr int kE[12][2] = {{0, 1}, {1, 2}, {2, 3}, {3, 0}, {4, 5}, {5, 6}, {6, 7}, {7, 4}, {0, 4}, {1, 5}, {2, 6}, {3, 7}};
+  float fval[8];
+  unsigned cube_case = 0;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    float f = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 3; ++j)
+      f = __fadd_rn(f, __fmul_rn(__fsub_rn(__fadd_rn(kC[k][j], pt_base[j]), pt[j]), normal[j]));
+    fval[k] = f;
+    if (f < 0.0f) cube_case |= 1u << k;
+  }
+#pragma unroll
+  for (int q = 0; q < 6; ++q) { vx[q] = 0.0f; vy[q] = 0.0f; vz[q] = 0.0f; }
+  int nv = 0;
+#pragma unroll
+  for (int e = 0; e < 12; ++e) {
+    const int v1 = kE[e][0], v2 = kE[e][1];
+    if ((((cube_case >> v1) ^ (cube_case >> v2)) & 1u) == 0) continue;
+    const float f1 = fval[v1], f2 = fval[v2];
+    float df = __fsub_rn(f2, f1);
+    if (df == 0) df = __fadd_rn(df, 1.0e-10f);
+    const float t = div_rn(-f1, df);
+    float p[3];
+#pragma unroll
+    for (int j = 0; j < 3; ++j)
+      p[j] = __fadd_rn(__fadd_rn(kC[v1][j], __fmul_rn(t, __fsub_rn(kC[v2][j], kC[v1][j]))), pt_base[j]);
+#pragma unroll
+    for (int q = 0; q < 6; ++q)
+      if (nv == q) { vx[q] = p[0]; vy[q] = p[1]; vz[q] = p[2]; }
+    nv++;
+  }
+  return nv;
 }
 
 // One thread per node: calc_signal as the reference writes it, leaf after leaf (the sums are
@@ -540,12 +599,31 @@ __global__ __launch_bounds__(kBlock) void signal_small_kernel(const SignalLevels
   const int k0 = a.rank_D[j0], k1 = a.rank_D[j1];
   const int leaves = k1 - k0;
   const int64_t nP = a.nP;
+  // A sweep over the node's leaves takes them eight at a time: the loads of a group are issued
+  // together (the adds of a chain wait for one another, the loads need not), `leaf(nrm, pt)`
+  // then sees the leaves in order.  An absent row reads a row that exists; its values are unused.
+  const float* nrm_row = has_normal ? a.nrm_P : a.any_P;
+  const float* pt_row = has_pt ? a.pt_P : a.any_P;
+  const int64_t nrm_step = has_normal ? nP : 0, pt_step = has_pt ? nP : 0;
+  auto sweep = [&](auto leaf) {
+    for (int k = k0; k < k1; k += 8) {
+      float vn[8][3], vp[8][3];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int kk = min(k + j, k1 - 1);
+#pragma unroll
+        for (int c = 0; c < 3; ++c) { vn[j][c] = nrm_row[c * nrm_step + kk]; vp[j][c] = pt_row[c * pt_step + kk]; }
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (k + j < k1) leaf(vn[j], vp[j]);
+    }
+  };
   float n_avg[3] = {0.0f, 0.0f, 0.0f}, last_n[3] = {0.0f, 0.0f, 0.0f}, pt_avg[3] = {0.0f, 0.0f, 0.0f};
-  for (int k = k0; k < k1; ++k) {
-    if (has_normal) for (int c = 0; c < 3; ++c) n_avg[c] = __fadd_rn(n_avg[c], a.nrm_P[c * nP + k]);
-    if (has_pt) for (int c = 0; c < 3; ++c) pt_avg[c] = __fadd_rn(pt_avg[c], a.pt_P[c * nP + k]);
-  }
-  if (has_normal && k0 < k1) for (int c = 0; c < 3; ++c) last_n[c] = a.nrm_P[c * nP + k1 - 1];
+  sweep([&](const float* vn, const float* vp) {
+    if (has_normal) for (int c = 0; c < 3; ++c) { n_avg[c] = __fadd_rn(n_avg[c], vn[c]); last_n[c] = vn[c]; }
+    if (has_pt) for (int c = 0; c < 3; ++c) pt_avg[c] = __fadd_rn(pt_avg[c], vp[c]);
+  });
   if (has_normal) {
     float len = norm3(n_avg);
     if (len < 1.0e-6f) {
@@ -596,46 +674,55 @@ __global__ __launch_bounds__(kBlock) void signal_small_kernel(const SignalLevels
       a.dis[i] = __fmul_rn(dis_avg[3], a.imul);
     }
   }
-  if (a.nerr) {
-    float nm_err = 1.0e20f;
-    if (a.calc_nerr && has_normal && a.d >= a.adp_layer) {
-      nm_err = 0.0f;
-      for (int k = k0; k < k1; ++k)
+  const bool do_nerr = a.nerr && a.calc_nerr && has_normal && a.d >= a.adp_layer;
+  const bool do_derr = a.derr && a.calc_derr && has_pt && a.d >= a.adp_layer;
+  float nm_err = 0.0f, distance_max1 = -1.0f;
+  float pt_avg1[3];
+  for (int c = 0; c < 3; ++c) pt_avg1[c] = __fmul_rn(pt_avg[c], scale);
+  if (do_nerr || do_derr) {
+    // one sweep for both: the chain of the normal error, and the largest distance of a leaf
+    // point from the plane
+    sweep([&](const float* vn, const float* vp) {
+      if (do_nerr)
         for (int c = 0; c < 3; ++c) {
-          const float tmp = __fsub_rn(a.nrm_P[c * nP + k], n_avg[c]);
+          const float tmp = __fsub_rn(vn[c], n_avg[c]);
           nm_err = __fadd_rn(nm_err, __fmul_rn(tmp, tmp));
         }
-      nm_err = div_rn(nm_err, count);
-    }
-    a.nerr[i] = nm_err;
-  }
-  if (a.derr) {
-    float err = 1.0e20f;
-    if (a.calc_derr && has_pt && a.d >= a.adp_layer) {
-      float pt_avg1[3];
-      for (int c = 0; c < 3; ++c) pt_avg1[c] = __fmul_rn(pt_avg[c], scale);
-      float distance_max1 = -1.0f;
-      for (int k = k0; k < k1; ++k) {
+      if (do_derr) {
         float dis = 0.0f;
-        for (int c = 0; c < 3; ++c) dis = __fadd_rn(dis, __fmul_rn(__fsub_rn(a.pt_P[c * nP + k], pt_avg1[c]), n_avg[c]));
+        for (int c = 0; c < 3; ++c) dis = __fadd_rn(dis, __fmul_rn(__fsub_rn(vp[c], pt_avg1[c]), n_avg[c]));
         distance_max1 = fmaxf(distance_max1, fabsf(dis));
       }
-      float vtx[36];
-      const int nv = intersect_cube(vtx, pt_avg, pt_base, n_avg);
-      float distance_max2 = nv == 0 ? 5.0e10f : -1.0f;
-      for (int v = 0; v < nv; ++v) {
-        float vk[3];
-        for (int c = 0; c < 3; ++c) vk[c] = __fmul_rn(vtx[3 * v + c], scale);
-        float distance_min = 1.0e30f;
-        for (int k = k0; k < k1; ++k) {
-          float dis = 0.0f;
-          for (int c = 0; c < 3; ++c) {
-            const float ptc = __fsub_rn(a.pt_P[c * nP + k], vk[c]);
-            dis = __fadd_rn(dis, __fmul_rn(ptc, ptc));
+    });
+  }
+  if (a.nerr) a.nerr[i] = do_nerr ? div_rn(nm_err, count) : 1.0e20f;
+  if (a.derr) {
+    float err = 1.0e20f;
+    if (do_derr) {
+      // ... and of a vertex of the plane's polygon inside the node from its nearest leaf point:
+      // every vertex in the same sweep.  The correctly rounded root is monotonic: the smallest
+      // root is the root of the smallest square.
+      float vx[6], vy[6], vz[6], sq_min[6];
+      const int nv = intersect_cube_regs(vx, vy, vz, pt_avg, pt_base, n_avg);
+#pragma unroll
+      for (int q = 0; q < 6; ++q) {
+        vx[q] = __fmul_rn(vx[q], scale); vy[q] = __fmul_rn(vy[q], scale); vz[q] = __fmul_rn(vz[q], scale);
+        sq_min[q] = __builtin_inff();   // (no leaf, or only infinite squares: 1.0e30f as the reference starts from)
+      }
+      if (nv > 0)
+        sweep([&](const float*, const float* vp) {
+#pragma unroll
+          for (int q = 0; q < 6; ++q) {
+            const float px = __fsub_rn(vp[0], vx[q]), py = __fsub_rn(vp[1], vy[q]), pz = __fsub_rn(vp[2], vz[q]);
+            const float dis = __fadd_rn(__fadd_rn(__fadd_rn(0.0f, __fmul_rn(px, px)), __fmul_rn(py, py)), __fmul_rn(pz, pz));
+            sq_min[q] = fminf(sq_min[q], dis);
           }
-          distance_min = fminf(distance_min, sqrt_rn(dis));
-        }
-        if (distance_min > distance_max2) distance_max2 = distance_min;
+        });
+      float distance_max2 = nv == 0 ? 5.0e10f : -1.0f;
+#pragma unroll
+      for (int q = 0; q < 6; ++q) {
+        const float distance_min = fminf(1.0e30f, sqrt_rn(sq_min[q]));
+        if (q < nv && distance_min > distance_max2) distance_max2 = distance_min;
       }
       err = distance_max2 > distance_max1 ? distance_max2 : distance_max1;
     }
@@ -1127,6 +1214,7 @@ int adaptive_finish(const AdaptiveInput& in, ocnn_alloc_fn alloc, void* alloc_ct
       a.imul = imul;
       a.child_D = child[D]; a.nrm_D = normal[D]; a.pt_D = pt[D]; a.feat_D = feature[D]; a.lab_D = label[D];
       a.rank_D = rank_D; a.nrm_P = nrm_P; a.pt_P = pt_P; a.feat_P = feat_P; a.lab_P = lab_P; a.nP = (int64_t)nP;
+      a.any_P = nrm_P;   // allocated whether or not the cloud has normals
     }
     for (int d = 0; d < D; ++d) {
       SignalLevel& l = L.level[d];
