@@ -363,7 +363,7 @@ def main():
     t = (time.perf_counter() - t0) / reps
     extra["points2octree_batch16_d7"] = {"ms": t * 1e3, "Mpts_per_s": 0.8 / t}
     # the adaptive build of configs[4]'s input: all-depth signals, plane-fit errors, trimming,
-    # one cloud at a time, then octree_batch (summation order of the reference kept: bit-exact)
+    # the whole batch as one octree in merged layout (summation order of the reference kept: bit-exact)
     adp = dict(node_dis=True, split_label=True, adaptive=True, adp_depth=4, th_normal=0.1, th_distance=2.0)
     F.points2octree_batch(cl, 7, 2, **adp)
     torch.cuda.synchronize()

@@ -461,13 +461,21 @@ int ocnn_clip_points(void* out_dev, void* out_info, int* inbox_mask_dev, const v
  * (ocnn_points2octree_emit) writes the blob.  The workspace must stay
  * untouched between the two steps.
  * The adaptive / node_feature / extrapolate options of the reference
- * (octree.cpp:454-806, 958-1135) are not implemented: OCNN_E_UNSUPPORTED. */
+ * (octree.cpp:454-806, 958-1135) take two rounds of allocation and go through
+ * ocnn_points2octree only (the two-step form answers OCNN_E_UNSUPPORTED).  A
+ * batch (n_clouds > 1, merged == 1) goes through both stages as one octree in
+ * merged layout; the result equals octree_batch over the octrees built cloud by
+ * cloud (the rule of trim_octree that keeps one node per level, octree.cpp:1055-1073,
+ * and the nearest-node search of extrapolate_signal, octree.cpp:776-803, are
+ * applied per octree).  Two-channel keys (key2xyz with depth > 8) cannot be
+ * batched, as in merge_octrees. */
 typedef struct {
   int depth, full_depth;
   int node_dis, node_feature, split_label, adaptive, adp_depth;
   float th_normal, th_distance;
   int extrapolate, save_pts, key2xyz;
-  int merged;          /* 0: single-octree blob (n_clouds must be 1); 1: octree_batch blob */
+  int merged;          /* 0: single-octree blob (n_clouds must be 1); 1: octree_batch blob;
+                          2 (plan/emit only): batch layout without neighbour tables */
   int has_bbox;        /* 0: [-1,1]^3 as pytorch/cpp does (octree_info.cpp:68-69) */
   float bbmin[3], bbmax[3];
 } ocnn_build_params;
