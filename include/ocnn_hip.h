@@ -299,6 +299,14 @@ int ocnn_conv_bf16_tile_threshold(int tiles);
  * the default.  Returns the previous setting. */
 int ocnn_conv_rows_direct(int on);
 
+/* Test hook, no counterpart in the reference (process-wide): the weight gradient of the shapes
+ * other than 3x3x3 stride 1 over all nodes (non-empty nodes, stride 2, smaller tap sets) with whole
+ * 32-channel blocks and 32 or whole 64 output channels stages its source rows in LDS from a table
+ * of row numbers; 0 sends these shapes to the register-fed kernel that serves every other channel
+ * count, 1 restores the default.  Both add the same products, in different orders (fp32, 1e-4).
+ * Returns the previous setting. */
+int ocnn_conv_wgrad_staged(int on);
+
 /* ocnn_octree_conv_fused for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
  * reference.  Same arguments and results minus the workspace: the packed weights, the inverted

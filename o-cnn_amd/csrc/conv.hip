@@ -2964,22 +2964,234 @@ __global__ __launch_bounds__(256 * HALVES) void conv_wgrad_f32_lds_kernel(ConvAr
   }
 }
 
-__global__ void conv_wgrad_reduce_kernel(float* __restrict__ G, const float* __restrict__ partial, int n_slices,
-    int M, int Cin, int K, int mpad, int cpad) {
+// The LDS-staged weight gradient for every other shape (non-empty nodes, stride 2, the smaller tap
+// sets, the deconvolution's geometry): a block of 8 columns reads 8 K source rows, one per
+// (tap, column), whose numbers a small launch writes down beforehand (src[block][tap][column],
+// wgrad_src: the zero row where there is nothing).  A workgroup stages these rows (32 channels
+// each) two blocks ahead of their use, as the kernel above does with the 64 rows of a sibling
+// group, and wavefront (g, h) multiplies the taps T g .. T g + T - 1 with the 32 rows of A of
+// half h.  A comes from its quad-interleaved copy (any number of columns, zero past the end).
+__global__ void wgrad_sources_kernel(ConvArgs a, int* __restrict__ src, int nblocks, int row_bytes) {
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= (int64_t)nblocks * a.K * 8) return;
+  const int j = (int)(id & 7), k = (int)((id >> 3) % a.K), b = (int)((id >> 3) / a.K);
+  src[id] = wgrad_src(a, b * 8 + j, k) * row_bytes;   // where the row starts in the row-major copy
+}
+// LDS rows of the kernel below: three buffers of 8 K rows, the rows that the taps past the K-th
+// of the last wavefront read behind the third buffer (never used), and a spare row
+__host__ __device__ inline int wgrad_src_lds_rows(int K, int T) { return 3 * K * 8 + (32 * T - 8 * K) + 1; }
+// DIRECT: the 2x2x2 stride-2 operator over all nodes.  The eight source rows of column n are the
+// eight children 8 n .. 8 n + 7 (tap k = child k), so a block's 64 rows are 64 consecutive rows of
+// the finer level and X is read as it lies, channel-major [C][hin]: thread (channel, quad) moves
+// four consecutive rows of a channel (16 bytes, a channel's 64 rows are 256 contiguous bytes) and
+// scatters them over the staged rows.  No row-major copy of X, no table of row numbers.
+template <int HALVES, int T, bool DIRECT>
+__global__ __launch_bounds__(256 * HALVES) void conv_wgrad_f32_lds_src_kernel(int K, int nblocks,
+    const float* __restrict__ aq, const float* __restrict__ X, int x_bytes, int hin, const int* __restrict__ src,
+    float* __restrict__ partial, int cpad, int mpad, int n_slices, int cpasses) {
+  static_assert(!DIRECT || (HALVES == 2 && T == 2), "the direct form stages 32 channels x 16 quads with 512 threads");
+  extern __shared__ __attribute__((aligned(16))) float s_dyn[];
+  constexpr int kThreads = 256 * HALVES;
+  constexpr int kUnits = (T + HALVES - 1) / HALVES;   // 16-byte units a thread stages per block (K <= 4 T)
+  const int rows = K * 8, buf_words = rows * kWgLdsRow;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tapgroup = wave & 3, mhalf = wave >> 2;
+  const int slice = blockIdx.x;
+  const int cpass = blockIdx.y % cpasses, mpass = blockIdx.y / cpasses;
+  const int r = lane & 31, kh = lane >> 5;
+  const int tap0 = tapgroup * T;
+  floatx16 acc[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[t][i] = 0.0f;
+  const int per_slice = (nblocks + n_slices - 1) / n_slices;
+  const int b_begin = slice * per_slice, b_end = min(nblocks, b_begin + per_slice);
+  // Everything the loop reads from memory goes through buffers with 32-bit offsets: a lane's part
+  // of the offset is fixed, the block's part is a scalar, so that a turn of the loop spends next
+  // to no vector instructions on addresses (they share the issue port with the MFMAs).
+  const __amdgpu_buffer_rsrc_t xbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(X), 0, x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t sbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<int*>(DIRECT ? (const int*)X : src), 0,
+      DIRECT ? 0 : nblocks * rows * 4, 0x00020000);
+  const __amdgpu_buffer_rsrc_t abuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(aq), 0, nblocks * 2 * mpad * 16, 0x00020000);
+  // staging: unit u of a block = 16 bytes `part` of row u / 8; a thread takes the units
+  // tid, tid + kThreads, ... (a unit past the block's rows repeats the last row and lands in the
+  // spare row: no branch in the loop, which the instruction order below relies on)
+  const int spare = (wgrad_src_lds_rows(K, T) - 1) * kWgLdsRow;
+  int st_src[kUnits], st_lds[kUnits], st_step[kUnits], st_col[kUnits];
+#pragma unroll
+  for (int v = 0; v < kUnits; ++v) {
+    const bool real = tid + v * kThreads < rows * 8;
+    const int u = min(tid + v * kThreads, rows * 8 - 1);
+    st_src[v] = (u >> 3) * 4;
+    st_lds[v] = real ? (u >> 3) * kWgLdsRow + (u & 7) * 4 : spare + (u & 7) * 4;
+    st_step[v] = real ? buf_words : 0;
+    st_col[v] = (cpass * 32 + (u & 7) * 4) * 4;
+  }
+  struct Idx { int p[kUnits]; };
+  struct Units { u32x4 v[kUnits]; };
+  // direct form: thread (channel, quad) = (tid >> 4, tid & 15); fine row 4 quad + i of the block is
+  // child (row & 7) of column (row >> 3), i.e. staged row (row & 7) * 8 + (row >> 3)
+  const int d_off = ((cpass * 32 + (tid >> 4)) * hin + 4 * (tid & 15)) * 4;
+  int d_lds[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = 4 * (tid & 15) + i;
+    d_lds[i] = ((row & 7) * 8 + (row >> 3)) * kWgLdsRow + (tid >> 4);
+  }
+  auto index_of = [&](int b) {
+    Idx x;
+#pragma unroll
+    for (int v = 0; v < kUnits; ++v)
+      x.p[v] = DIRECT ? b : (int)__builtin_amdgcn_raw_buffer_load_b32(sbuf, st_src[v], b * rows * 4, 0);
+    return x;
+  };
+  auto load_rows = [&](const Idx& x) {
+    Units u;
+    if (DIRECT) {
+      u32x4 q = __builtin_amdgcn_raw_buffer_load_b128(xbuf, d_off, x.p[0] * 256, 0);
+      const bool inside = x.p[0] * 64 + 4 * (tid & 15) < hin;   // whole quads: the level has a multiple of 8 rows
+      q.x = inside ? q.x : 0u; q.y = inside ? q.y : 0u; q.z = inside ? q.z : 0u; q.w = inside ? q.w : 0u;
+      u.v[0] = q;
+      return u;
+    }
+#pragma unroll
+    for (int v = 0; v < kUnits; ++v) u.v[v] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, x.p[v] + st_col[v], 0, 0);
+    return u;
+  };
+  auto store_rows = [&](int buf, const Units& u) {
+    if (DIRECT) {
+      float* base = s_dyn + buf * buf_words;
+      base[d_lds[0]] = __uint_as_float(u.v[0].x); base[d_lds[1]] = __uint_as_float(u.v[0].y);
+      base[d_lds[2]] = __uint_as_float(u.v[0].z); base[d_lds[3]] = __uint_as_float(u.v[0].w);
+      return;
+    }
+#pragma unroll
+    for (int v = 0; v < kUnits; ++v) *reinterpret_cast<u32x4*>(&s_dyn[buf * st_step[v] + st_lds[v]]) = u.v[v];
+  };
+  const int m = (mpass * HALVES + mhalf) * 32 + r;
+  const int a_lane = (kh * mpad + m) * 16;
+  auto load_a = [&](int b) { return __builtin_amdgcn_raw_buffer_load_b128(abuf, a_lane, b * 2 * mpad * 16, 0); };
+  // LDS word of this lane's B value for k-step j of tap t: row (tap, column j + 4 kh), channel r;
+  // the tap and the k-step are constant offsets from the lane's own word
+  const int lane_word = (tap0 * 8 + 4 * kh) * kWgLdsRow + r;
+  if (b_begin < b_end) {
+    const int last = b_end - 1;
+    auto read_b = [&](int buf, float (&bv)[4][T]) {
+      const float* base = s_dyn + buf * buf_words + lane_word;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int t = 0; t < T; ++t) bv[j][t] = base[(t * 8 + j) * kWgLdsRow];
+    };
+    store_rows(0, load_rows(index_of(b_begin)));
+    store_rows(1, load_rows(index_of(min(b_begin + 1, last))));
+    Units rows_next = load_rows(index_of(min(b_begin + 2, last)));
+    Idx idx_next = index_of(min(b_begin + 3, last));
+    u32x4 av = load_a(b_begin);
+    __syncthreads();
+    // One block: the MFMAs of block b from registers, with everything else of the turn spread
+    // between them (the two wavefronts of a SIMD meet at the barrier every turn, so work that
+    // follows the last MFMA of one finds the matrix pipe idle in the other as well): B values of
+    // block b + 1 out of LDS, rows of block b + 2 into LDS, rows of block b + 3 and the numbers of
+    // block b + 4 requested.
+    auto turn = [&](int b, int rd, int wr, const float (&cur)[4][T], float (&nxtv)[4][T]) {
+      const u32x4 av_next = load_a(min(b + 1, last));
+      const float aj[4] = {__uint_as_float(av.x), __uint_as_float(av.y), __uint_as_float(av.z), __uint_as_float(av.w)};
+      read_b(rd, nxtv);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int t = 0; t < T; ++t)
+          acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(aj[j], cur[j][t], acc[t], 0, 0, 0);
+      store_rows(wr, rows_next);
+      rows_next = load_rows(idx_next);
+      idx_next = index_of(min(b + 4, last));
+      av = av_next;
+#pragma unroll
+      for (int i = 0; i < 4 * T; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+        if (i % 4 == 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // a load from memory
+        if (DIRECT || i % 4 == 3) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // an LDS write
+        __builtin_amdgcn_sched_group_barrier(0x006, 2, 0);   // what is left of address arithmetic
+      }
+      __syncthreads();
+    };
+    float bva[4][T], bvb[4][T];
+    read_b(0, bva);
+    int rd = 1;                        // buffer of block b + 1
+    for (int b = b_begin; b < b_end; b += 2) {
+      int wr = rd == 2 ? 0 : rd + 1;   // buffer of block b + 2
+      turn(b, rd, wr, bva, bvb);
+      rd = wr;
+      if (b + 1 < b_end) {
+        wr = rd == 2 ? 0 : rd + 1;
+        turn(b + 1, rd, wr, bvb, bva);
+        rd = wr;
+      }
+    }
+  }
+  // partial[slice][tap][m][c]
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    const int tap = tap0 + t;
+    if (tap >= K) continue;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int mm = (mpass * HALVES + mhalf) * 32 + 8 * (i / 4) + 4 * kh + (i % 4);
+      partial[(((int64_t)slice * K + tap) * mpad + mm) * cpad + cpass * 32 + r] = acc[t][i];
+    }
+  }
+}
+
+// G <- the slices added up in a fixed order: eight groups of consecutive slices side by side (one
+// per 32 threads of a workgroup, each adding its slices in order), then the eight sums in order.
+__global__ __launch_bounds__(256) void conv_wgrad_reduce_kernel(float* __restrict__ G, const float* __restrict__ partial,
+    int n_slices, int M, int Cin, int K, int mpad, int cpad) {
+  __shared__ float s_sum[8][32];
   const int64_t per = (int64_t)K * mpad * cpad;
-  int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (id >= per) return;
+  const int e = threadIdx.x & 31, grp = threadIdx.x >> 5;
+  const int64_t id = (int64_t)blockIdx.x * 32 + e;
+  const int per_group = (n_slices + 7) / 8;
+  const int s0 = grp * per_group, s1 = min(n_slices, s0 + per_group);
+  float sum = 0.0f;
+  if (id < per)
+    for (int sl = s0; sl < s1; ++sl) sum += partial[sl * per + id];
+  s_sum[grp][e] = sum;
+  __syncthreads();
+  if (grp != 0 || id >= per) return;
+  float total = 0.0f;
+#pragma unroll
+  for (int g = 0; g < 8; ++g) total += s_sum[g][e];
   const int c = (int)(id % cpad), m = (int)((id / cpad) % mpad), k = (int)(id / ((int64_t)cpad * mpad));
   if (m >= M || c >= Cin) return;
-  float sum = 0.0f;
-  for (int sl = 0; sl < n_slices; ++sl) sum += partial[sl * per + id];
-  G[((int64_t)m * Cin + c) * K + k] = sum;
+  G[((int64_t)m * Cin + c) * K + k] = total;
 }
+
+// The staging buffers of the larger tap sets pass the 64 KiB a kernel may use without asking.
+template <int HALVES, int T, bool DIRECT = false>
+int launch_wgrad_src(dim3 grid, size_t lds, hipStream_t s, int K, int nblocks, const float* aq, const float* xt,
+    int x_bytes, int hin, const int* src, float* partial, int cpad, int mpad, int n_slices, int cpasses) {
+  static std::atomic<size_t> allowed{0};
+  if (lds > 64 * 1024 && allowed.load() < lds) {
+    OCNN_HIP_OK(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_wgrad_f32_lds_src_kernel<HALVES, T, DIRECT>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    allowed.store(lds);
+  }
+  conv_wgrad_f32_lds_src_kernel<HALVES, T, DIRECT><<<grid, 256 * HALVES, lds, s>>>(K, nblocks, aq, xt, x_bytes, hin, src,
+      partial, cpad, mpad, n_slices, cpasses);
+  OCNN_LAUNCH_OK("conv_wgrad_lds_src");
+  return OCNN_OK;
+}
+std::atomic<int> g_wgrad_lds{1};   // test hook: 0 sends every shape but 3x3x3 stride 1 over all nodes to the register-fed kernel
 
 struct WgradPlan {
   int MT, NT, mpasses, cpasses, mpad, cpad, n_slices, tapgroups;
   int lds_slices;   // slices of the LDS-staged kernel, 0 if the shape does not qualify for it
-  size_t xt_bytes, partial_bytes, ichild_bytes, aq_bytes, total_bytes;
+  int src_taps;     // taps per wavefront of the LDS-staged kernel with a source table, 0 if the shape does not qualify
+  int src_slices;
+  size_t xt_bytes, partial_bytes, ichild_bytes, aq_bytes, src_bytes, total_bytes;
 };
 // `p` is the plan of the underlying convolution geometry (deconv = 0): M rows on the column side,
 // channel_in channels on the gathered side.
@@ -3009,12 +3221,28 @@ void make_wgrad_plan(const ConvPlan& p, int M, int channel_in, int nempty, Wgrad
     w->lds_slices = (halves == 1 ? 512 : 256) / tiles;
     if (w->lds_slices < 1) w->lds_slices = 1;
   }
+  // every other shape with whole 32-channel chunks and 32 / 64-row tiles of A: the LDS-staged kernel
+  // with a source table (a single tap is a plain product, left to the register-fed kernel)
+  w->src_taps = 0; w->src_slices = 0; w->src_bytes = 0;
+  const int K = p.taps.count;
+  if (K >= 2 && K <= 28 && ((M & 63) == 0 || M == 32) && (channel_in & 31) == 0) {
+    const int halves = M == 32 ? 1 : 2;
+    w->src_taps = K > 12 ? 7 : K > 8 ? 3 : K > 4 ? 2 : 1;
+    const int tiles = (channel_in / 32) * (M / (32 * halves));
+    const size_t lds = (size_t)wgrad_src_lds_rows(K, w->src_taps) * kWgLdsRow * sizeof(float);
+    const int per_cu = (lds > 80 * 1024 ? 1 : 2) * (halves == 1 ? 2 : 1);
+    w->src_slices = 256 * per_cu / tiles;
+    if (w->src_slices < 1) w->src_slices = 1;
+    if (w->src_slices > nblocks) w->src_slices = nblocks;
+    w->src_bytes = align256((size_t)nblocks * K * 8 * sizeof(int));
+  }
   w->xt_bytes = align256(((size_t)p.btm_h + 1) * w->cpad * sizeof(float));
-  const int most_slices = w->n_slices > w->lds_slices ? w->n_slices : w->lds_slices;
+  int most_slices = w->n_slices > w->lds_slices ? w->n_slices : w->lds_slices;
+  if (w->src_slices > most_slices) most_slices = w->src_slices;
   w->partial_bytes = align256((size_t)most_slices * p.taps.count * w->mpad * w->cpad * sizeof(float));
   w->ichild_bytes = nempty ? align256(sizeof(int) * (size_t)(p.ichild_h + 1)) : 0;
   w->aq_bytes = align256((size_t)nblocks * 2 * w->mpad * 4 * sizeof(float));
-  w->total_bytes = w->xt_bytes + w->partial_bytes + w->ichild_bytes + w->aq_bytes;
+  w->total_bytes = w->xt_bytes + w->partial_bytes + w->ichild_bytes + w->aq_bytes + w->src_bytes;
 }
 
 // grad_w[M, channel_in * K] from A [M, top_h] (column side) and X [channel_in, btm_h] (gathered side)
@@ -3059,19 +3287,64 @@ int run_wgrad(float* grad_w, const float* A, int M, const float* X, int channel_
           w.cpad / 32);
     OCNN_LAUNCH_OK("conv_wgrad_lds");
     const int64_t per = (int64_t)a.K * w.mpad * w.cpad;
-    conv_wgrad_reduce_kernel<<<blocks_for(per), kBlock, 0, s>>>(grad_w, partial, n_slices, M, channel_in, a.K, w.mpad,
+    conv_wgrad_reduce_kernel<<<blocks_for(per, 32), 256, 0, s>>>(grad_w, partial, n_slices, M, channel_in, a.K, w.mpad,
         w.cpad);
+    OCNN_LAUNCH_OK("conv_wgrad_reduce");
+    return OCNN_OK;
+  }
+  float* aq = reinterpret_cast<float*>(wsb + w.xt_bytes + w.partial_bytes + w.ichild_bytes);
+  const int n_quads = ((a.N + 7) / 8) * 2;
+  dim3 qg((n_quads * 4 + 63) / 64, (w.mpad + 63) / 64);
+  interleave_quads_kernel<<<qg, 256, 0, s>>>(aq, A, M, a.N, w.mpad, n_quads);
+  OCNN_LAUNCH_OK("interleave_quads");
+  // 2x2x2 stride 2 over all nodes: the children of column n are the rows 8 n .. 8 n + 7, X is read in place
+  if (a.mode == kModeS2Conv && a.K == 8 && !a.nempty && w.src_taps == 2 && (M & 63) == 0 && w.mpad == M &&
+      w.cpad == channel_in && a.Hin == 8 * a.N && (int64_t)channel_in * a.Hin * 4 < (1ll << 31) &&
+      (int64_t)n_quads * w.mpad * 16 < (1ll << 31) && (reinterpret_cast<uintptr_t>(X) & 15) == 0 && g_wgrad_lds.load()) {
+    const int nblocks = (a.N + 7) / 8;
+    const int tiles = (w.cpad / 32) * (w.mpad / 64);
+    const size_t lds = (size_t)wgrad_src_lds_rows(a.K, 2) * kWgLdsRow * sizeof(float);
+    int e = launch_wgrad_src<2, 2, true>(dim3(w.src_slices, tiles), lds, s, a.K, nblocks, aq, X, channel_in * a.Hin * 4,
+        a.Hin, nullptr, partial, w.cpad, w.mpad, w.src_slices, w.cpad / 32);
+    if (e) return e;
+    const int64_t per = (int64_t)a.K * w.mpad * w.cpad;
+    conv_wgrad_reduce_kernel<<<blocks_for(per, 32), 256, 0, s>>>(grad_w, partial, w.src_slices, M, channel_in, a.K,
+        w.mpad, w.cpad);
     OCNN_LAUNCH_OK("conv_wgrad_reduce");
     return OCNN_OK;
   }
   dim3 tg((a.Hin + 64) / 64, (w.cpad + 63) / 64);
   transpose_rows_f32_kernel<<<tg, 256, 0, s>>>(xt, X, channel_in, a.Hin, w.cpad);
   OCNN_LAUNCH_OK("transpose_rows");
-  float* aq = reinterpret_cast<float*>(wsb + w.xt_bytes + w.partial_bytes + w.ichild_bytes);
-  const int n_quads = ((a.N + 7) / 8) * 2;
-  dim3 qg((n_quads * 4 + 63) / 64, (w.mpad + 63) / 64);
-  interleave_quads_kernel<<<qg, 256, 0, s>>>(aq, A, M, a.N, w.mpad, n_quads);
-  OCNN_LAUNCH_OK("interleave_quads");
+  const int64_t x_bytes = ((int64_t)a.Hin + 1) * w.cpad * 4;
+  const int64_t most_bytes = std::max(x_bytes, std::max((int64_t)((a.N + 7) / 8) * a.K * 32, (int64_t)((a.N + 7) / 8) * 2 * w.mpad * 16));
+  if (w.src_taps > 0 && w.mpad == M && w.cpad == channel_in && most_bytes < (1ll << 31) && g_wgrad_lds.load()) {
+    const int nblocks = (a.N + 7) / 8;
+    int* src = reinterpret_cast<int*>(wsb + w.xt_bytes + w.partial_bytes + w.ichild_bytes + w.aq_bytes);
+    wgrad_sources_kernel<<<blocks_for((int64_t)nblocks * a.K * 8), kBlock, 0, s>>>(a, src, nblocks, w.cpad * 4);
+    OCNN_LAUNCH_OK("wgrad_sources");
+    const int halves = M == 32 ? 1 : 2;
+    const int tiles = (w.cpad / 32) * (w.mpad / (32 * halves));
+    const size_t lds = (size_t)wgrad_src_lds_rows(a.K, w.src_taps) * kWgLdsRow * sizeof(float);
+    int e = OCNN_OK;
+#define OCNN_WGRAD_SRC(H_, T_)                                                                                    \
+    e = launch_wgrad_src<H_, T_>(dim3(w.src_slices, tiles), lds, s, a.K, nblocks, aq, xt, (int)x_bytes, a.Hin,    \
+        src, partial, w.cpad, w.mpad, w.src_slices, w.cpad / 32)
+    if (halves == 2) {
+      if (w.src_taps == 7) OCNN_WGRAD_SRC(2, 7); else if (w.src_taps == 3) OCNN_WGRAD_SRC(2, 3);
+      else if (w.src_taps == 2) OCNN_WGRAD_SRC(2, 2); else OCNN_WGRAD_SRC(2, 1);
+    } else {
+      if (w.src_taps == 7) OCNN_WGRAD_SRC(1, 7); else if (w.src_taps == 3) OCNN_WGRAD_SRC(1, 3);
+      else if (w.src_taps == 2) OCNN_WGRAD_SRC(1, 2); else OCNN_WGRAD_SRC(1, 1);
+    }
+#undef OCNN_WGRAD_SRC
+    if (e) return e;
+    const int64_t per = (int64_t)a.K * w.mpad * w.cpad;
+    conv_wgrad_reduce_kernel<<<blocks_for(per, 32), 256, 0, s>>>(grad_w, partial, w.src_slices, M, channel_in, a.K,
+        w.mpad, w.cpad);
+    OCNN_LAUNCH_OK("conv_wgrad_reduce");
+    return OCNN_OK;
+  }
   dim3 grid(w.n_slices / 4, w.tapgroups, w.mpasses * w.cpasses);
 #define OCNN_WGRAD(MT_, NT_)                                                                                     \
   do {                                                                                                           \
@@ -3087,7 +3360,7 @@ int run_wgrad(float* grad_w, const float* A, int M, const float* X, int channel_
 #undef OCNN_WGRAD
   OCNN_LAUNCH_OK("conv_wgrad");
   int64_t per = (int64_t)a.K * w.mpad * w.cpad;
-  conv_wgrad_reduce_kernel<<<blocks_for(per), kBlock, 0, s>>>(grad_w, partial, w.n_slices, M, channel_in, a.K,
+  conv_wgrad_reduce_kernel<<<blocks_for(per, 32), 256, 0, s>>>(grad_w, partial, w.n_slices, M, channel_in, a.K,
       w.mpad, w.cpad);
   OCNN_LAUNCH_OK("conv_wgrad_reduce");
   return OCNN_OK;
@@ -3574,6 +3847,7 @@ int ocnn_octree_conv_static(void* top, const void* btm, int channel_in, int btm_
 }
 
 int ocnn_conv_rows_direct(int on) { return g_rows_direct.exchange(on ? 1 : 0); }
+int ocnn_conv_wgrad_staged(int on) { return g_wgrad_lds.exchange(on ? 1 : 0); }
 
 int ocnn_conv_bf16_tile_threshold(int tiles) {
   const int old = g_bf16_reg_min_tiles.load();
