@@ -391,6 +391,19 @@ def main():
     extra["conv333_s1_d9_f32_grad"] = {"ms": t, "octants_per_s": H9 / (t * 1e-3), "tflops": fl / (t * 1e-3) / 1e12,
                                        "frac_mfma_peak": fl / (t * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS["f32"]}
 
+    # the weight gradient alone, for the shapes a network over the non-empty nodes trains with
+    # (3x3x3 over the non-empty nodes, 2x2x2 stride 2 down and its deconvolution up)
+    def wgrad_case(name, fn, x, w_, gy_, depth, ks, stride, nempty, cols):
+      t = timed(lambda: fn(x, w_, octree, gy_, depth, C, ks, stride, nempty, need_data=False), max(4, reps // 2), 3)
+      fl = 2.0 * cols * ks[0] * ks[1] * ks[2] * C * C
+      extra[name] = {"ms": t, "tflops": fl / (t * 1e-3) / 1e12, "frac_mfma_peak": fl / (t * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS["f32"]}
+    gne = torch.randn(1, C, Hne9, 1, generator=g).to(dev)
+    wgrad_case("conv333_s1_d9_f32_nempty_wgrad", F.octree_conv_grad, xne, w32, gne, 9, [3, 3, 3], 1, True, Hne9)
+    g8 = torch.randn(1, C, Hne8, 1, generator=g).to(dev)
+    wgrad_case("conv222_s2_d9_f32_wgrad", F.octree_conv_grad, x32, w2, g8, 9, [2, 2, 2], 2, False, Hne8)
+    wgrad_case("deconv222_s2_d8to9_f32_wgrad", F.octree_deconv_grad, x8, w2, gy, 8, [2, 2, 2], 2, False, Hne8)
+    del gne, g8
+
     def hbm(name, t, by):
       extra[name] = {"ms": t, "GBs": by / t / 1e6, "frac_hbm_peak": by / t / 1e6 / PEAK_HBM_GBS}
 

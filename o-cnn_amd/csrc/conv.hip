@@ -2977,23 +2977,31 @@ __global__ void wgrad_sources_kernel(ConvArgs a, int* __restrict__ src, int nblo
   const int j = (int)(id & 7), k = (int)((id >> 3) % a.K), b = (int)((id >> 3) / a.K);
   src[id] = wgrad_src(a, b * 8 + j, k) * row_bytes;   // where the row starts in the row-major copy
 }
-// LDS rows of the kernel below: three buffers of 8 K rows, the rows that the taps past the K-th
+// Blocks of 8 columns a turn of the kernel below takes at once: a turn ends in a barrier, so a tap
+// set with few taps per wavefront takes several blocks to keep the matrix pipe fed between two.
+__host__ __device__ constexpr int wgrad_src_blocks(int T) { return T >= 7 ? 1 : T == 1 ? 4 : 2; }
+// LDS rows of the kernel below: three buffers of a turn's rows, the rows that the taps past the K-th
 // of the last wavefront read behind the third buffer (never used), and a spare row
-__host__ __device__ inline int wgrad_src_lds_rows(int K, int T) { return 3 * K * 8 + (32 * T - 8 * K) + 1; }
+__host__ __device__ inline int wgrad_src_lds_rows(int K, int T) {
+  return 3 * K * 8 * wgrad_src_blocks(T) + (32 * T - 8 * K) + 1;
+}
 // DIRECT: the 2x2x2 stride-2 operator over all nodes.  The eight source rows of column n are the
 // eight children 8 n .. 8 n + 7 (tap k = child k), so a block's 64 rows are 64 consecutive rows of
 // the finer level and X is read as it lies, channel-major [C][hin]: thread (channel, quad) moves
 // four consecutive rows of a channel (16 bytes, a channel's 64 rows are 256 contiguous bytes) and
 // scatters them over the staged rows.  No row-major copy of X, no table of row numbers.
+// `nturns` turns of wgrad_src_blocks(T) blocks each; aq and src cover whole turns (zero columns /
+// the zero row past the last column).
 template <int HALVES, int T, bool DIRECT>
-__global__ __launch_bounds__(256 * HALVES) void conv_wgrad_f32_lds_src_kernel(int K, int nblocks,
+__global__ __launch_bounds__(256 * HALVES) void conv_wgrad_f32_lds_src_kernel(int K, int nturns,
     const float* __restrict__ aq, const float* __restrict__ X, int x_bytes, int hin, const int* __restrict__ src,
     float* __restrict__ partial, int cpad, int mpad, int n_slices, int cpasses) {
-  static_assert(!DIRECT || (HALVES == 2 && T == 2), "the direct form stages 32 channels x 16 quads with 512 threads");
+  static_assert(!DIRECT || (HALVES == 2 && T == 2), "the direct form stages 32 channels x 16 quads a block with 512 threads");
   extern __shared__ __attribute__((aligned(16))) float s_dyn[];
   constexpr int kThreads = 256 * HALVES;
-  constexpr int kUnits = (T + HALVES - 1) / HALVES;   // 16-byte units a thread stages per block (K <= 4 T)
-  const int rows = K * 8, buf_words = rows * kWgLdsRow;
+  constexpr int BPT = wgrad_src_blocks(T);
+  constexpr int kUnits = DIRECT ? BPT : (T * BPT + HALVES - 1) / HALVES;   // 16-byte units a thread stages per turn (K <= 4 T)
+  const int rows8 = K * 8, rows = rows8 * BPT, buf_words = rows * kWgLdsRow;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int tapgroup = wave & 3, mhalf = wave >> 2;
   const int slice = blockIdx.x;
@@ -3005,17 +3013,18 @@ __global__ __launch_bounds__(256 * HALVES) void conv_wgrad_f32_lds_src_kernel(in
   for (int t = 0; t < T; ++t)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[t][i] = 0.0f;
-  const int per_slice = (nblocks + n_slices - 1) / n_slices;
-  const int b_begin = slice * per_slice, b_end = min(nblocks, b_begin + per_slice);
+  const int per_slice = (nturns + n_slices - 1) / n_slices;
+  const int b_begin = slice * per_slice, b_end = min(nturns, b_begin + per_slice);
   // Everything the loop reads from memory goes through buffers with 32-bit offsets: a lane's part
-  // of the offset is fixed, the block's part is a scalar, so that a turn of the loop spends next
+  // of the offset is fixed, the turn's part is a scalar, so that a turn of the loop spends next
   // to no vector instructions on addresses (they share the issue port with the MFMAs).
   const __amdgpu_buffer_rsrc_t xbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(X), 0, x_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t sbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<int*>(DIRECT ? (const int*)X : src), 0,
-      DIRECT ? 0 : nblocks * rows * 4, 0x00020000);
-  const __amdgpu_buffer_rsrc_t abuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(aq), 0, nblocks * 2 * mpad * 16, 0x00020000);
-  // staging: unit u of a block = 16 bytes `part` of row u / 8; a thread takes the units
-  // tid, tid + kThreads, ... (a unit past the block's rows repeats the last row and lands in the
+      DIRECT ? 0 : nturns * rows * 4, 0x00020000);
+  const __amdgpu_buffer_rsrc_t abuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(aq), 0,
+      nturns * BPT * 2 * mpad * 16, 0x00020000);
+  // staging: unit u of a turn = 16 bytes `part` of row u / 8; a thread takes the units
+  // tid, tid + kThreads, ... (a unit past the turn's rows repeats the last row and lands in the
   // spare row: no branch in the loop, which the instruction order below relies on)
   const int spare = (wgrad_src_lds_rows(K, T) - 1) * kWgLdsRow;
   int st_src[kUnits], st_lds[kUnits], st_step[kUnits], st_col[kUnits];
@@ -3030,8 +3039,9 @@ __global__ __launch_bounds__(256 * HALVES) void conv_wgrad_f32_lds_src_kernel(in
   }
   struct Idx { int p[kUnits]; };
   struct Units { u32x4 v[kUnits]; };
-  // direct form: thread (channel, quad) = (tid >> 4, tid & 15); fine row 4 quad + i of the block is
-  // child (row & 7) of column (row >> 3), i.e. staged row (row & 7) * 8 + (row >> 3)
+  // direct form: thread (channel, quad) = (tid >> 4, tid & 15) of every block of the turn; fine row
+  // 4 quad + i of a block is child (row & 7) of column (row >> 3), i.e. staged row
+  // (row & 7) * 8 + (row >> 3)
   const int d_off = ((cpass * 32 + (tid >> 4)) * hin + 4 * (tid & 15)) * 4;
   int d_lds[4];
 #pragma unroll
@@ -3043,86 +3053,107 @@ __global__ __launch_bounds__(256 * HALVES) void conv_wgrad_f32_lds_src_kernel(in
     Idx x;
 #pragma unroll
     for (int v = 0; v < kUnits; ++v)
-      x.p[v] = DIRECT ? b : (int)__builtin_amdgcn_raw_buffer_load_b32(sbuf, st_src[v], b * rows * 4, 0);
+      x.p[v] = DIRECT ? b * BPT + v : (int)__builtin_amdgcn_raw_buffer_load_b32(sbuf, st_src[v], b * rows * 4, 0);
     return x;
   };
   auto load_rows = [&](const Idx& x) {
     Units u;
-    if (DIRECT) {
-      u32x4 q = __builtin_amdgcn_raw_buffer_load_b128(xbuf, d_off, x.p[0] * 256, 0);
-      const bool inside = x.p[0] * 64 + 4 * (tid & 15) < hin;   // whole quads: the level has a multiple of 8 rows
-      q.x = inside ? q.x : 0u; q.y = inside ? q.y : 0u; q.z = inside ? q.z : 0u; q.w = inside ? q.w : 0u;
-      u.v[0] = q;
-      return u;
-    }
 #pragma unroll
-    for (int v = 0; v < kUnits; ++v) u.v[v] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, x.p[v] + st_col[v], 0, 0);
+    for (int v = 0; v < kUnits; ++v) {
+      if (DIRECT) {
+        u32x4 q = __builtin_amdgcn_raw_buffer_load_b128(xbuf, d_off, x.p[v] * 256, 0);
+        const bool inside = x.p[v] * 64 + 4 * (tid & 15) < hin;   // whole quads: the level has a multiple of 8 rows
+        q.x = inside ? q.x : 0u; q.y = inside ? q.y : 0u; q.z = inside ? q.z : 0u; q.w = inside ? q.w : 0u;
+        u.v[v] = q;
+      } else {
+        u.v[v] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, x.p[v] + st_col[v], 0, 0);
+      }
+    }
     return u;
   };
   auto store_rows = [&](int buf, const Units& u) {
-    if (DIRECT) {
-      float* base = s_dyn + buf * buf_words;
-      base[d_lds[0]] = __uint_as_float(u.v[0].x); base[d_lds[1]] = __uint_as_float(u.v[0].y);
-      base[d_lds[2]] = __uint_as_float(u.v[0].z); base[d_lds[3]] = __uint_as_float(u.v[0].w);
-      return;
-    }
 #pragma unroll
-    for (int v = 0; v < kUnits; ++v) *reinterpret_cast<u32x4*>(&s_dyn[buf * st_step[v] + st_lds[v]]) = u.v[v];
+    for (int v = 0; v < kUnits; ++v) {
+      if (DIRECT) {
+        float* base = s_dyn + buf * buf_words + v * rows8 * kWgLdsRow;
+        base[d_lds[0]] = __uint_as_float(u.v[v].x); base[d_lds[1]] = __uint_as_float(u.v[v].y);
+        base[d_lds[2]] = __uint_as_float(u.v[v].z); base[d_lds[3]] = __uint_as_float(u.v[v].w);
+      } else {
+        *reinterpret_cast<u32x4*>(&s_dyn[buf * st_step[v] + st_lds[v]]) = u.v[v];
+      }
+    }
   };
   const int m = (mpass * HALVES + mhalf) * 32 + r;
   const int a_lane = (kh * mpad + m) * 16;
-  auto load_a = [&](int b) { return __builtin_amdgcn_raw_buffer_load_b128(abuf, a_lane, b * 2 * mpad * 16, 0); };
+  struct AVals { u32x4 v[BPT]; };
+  auto load_a = [&](int b) {
+    AVals a4;
+#pragma unroll
+    for (int bb = 0; bb < BPT; ++bb)
+      a4.v[bb] = __builtin_amdgcn_raw_buffer_load_b128(abuf, a_lane, (b * BPT + bb) * 2 * mpad * 16, 0);
+    return a4;
+  };
   // LDS word of this lane's B value for k-step j of tap t: row (tap, column j + 4 kh), channel r;
-  // the tap and the k-step are constant offsets from the lane's own word
+  // the block of the turn, the tap and the k-step are constant offsets from the lane's own word
   const int lane_word = (tap0 * 8 + 4 * kh) * kWgLdsRow + r;
   if (b_begin < b_end) {
     const int last = b_end - 1;
-    auto read_b = [&](int buf, float (&bv)[4][T]) {
+    auto read_b = [&](int buf, float (&bv)[BPT][4][T]) {
       const float* base = s_dyn + buf * buf_words + lane_word;
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int bb = 0; bb < BPT; ++bb) {
+        const float* sub = base + bb * rows8 * kWgLdsRow;
 #pragma unroll
-        for (int t = 0; t < T; ++t) bv[j][t] = base[(t * 8 + j) * kWgLdsRow];
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int t = 0; t < T; ++t) bv[bb][j][t] = sub[(t * 8 + j) * kWgLdsRow];
+      }
     };
     store_rows(0, load_rows(index_of(b_begin)));
     store_rows(1, load_rows(index_of(min(b_begin + 1, last))));
     Units rows_next = load_rows(index_of(min(b_begin + 2, last)));
     Idx idx_next = index_of(min(b_begin + 3, last));
-    u32x4 av = load_a(b_begin);
+    AVals av = load_a(b_begin);
     __syncthreads();
-    // One block: the MFMAs of block b from registers, with everything else of the turn spread
+    // One turn: the MFMAs of turn b from registers, with everything else of the turn spread
     // between them (the two wavefronts of a SIMD meet at the barrier every turn, so work that
     // follows the last MFMA of one finds the matrix pipe idle in the other as well): B values of
-    // block b + 1 out of LDS, rows of block b + 2 into LDS, rows of block b + 3 and the numbers of
-    // block b + 4 requested.
-    auto turn = [&](int b, int rd, int wr, const float (&cur)[4][T], float (&nxtv)[4][T]) {
-      const u32x4 av_next = load_a(min(b + 1, last));
-      const float aj[4] = {__uint_as_float(av.x), __uint_as_float(av.y), __uint_as_float(av.z), __uint_as_float(av.w)};
+    // turn b + 1 out of LDS, rows of turn b + 2 into LDS, rows of turn b + 3 and the numbers of
+    // turn b + 4 requested.
+    auto turn = [&](int b, int rd, int wr, const float (&cur)[BPT][4][T], float (&nxtv)[BPT][4][T]) {
+      const AVals av_next = load_a(min(b + 1, last));
       read_b(rd, nxtv);
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int bb = 0; bb < BPT; ++bb) {
+        const float aj[4] = {__uint_as_float(av.v[bb].x), __uint_as_float(av.v[bb].y), __uint_as_float(av.v[bb].z),
+            __uint_as_float(av.v[bb].w)};
 #pragma unroll
-        for (int t = 0; t < T; ++t)
-          acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(aj[j], cur[j][t], acc[t], 0, 0, 0);
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int t = 0; t < T; ++t)
+            acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(aj[j], cur[bb][j][t], acc[t], 0, 0, 0);
+      }
       store_rows(wr, rows_next);
       rows_next = load_rows(idx_next);
       idx_next = index_of(min(b + 4, last));
       av = av_next;
+      constexpr int kMfma = 4 * T * BPT;
+      constexpr int kLoads = (DIRECT ? kUnits : 2 * kUnits) + BPT, kWrites = DIRECT ? 4 * kUnits : kUnits;
 #pragma unroll
-      for (int i = 0; i < 4 * T; ++i) {
+      for (int i = 0; i < kMfma; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
-        if (i % 4 == 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // a load from memory
-        if (DIRECT || i % 4 == 3) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // an LDS write
+        if ((i * kLoads) / kMfma != ((i + 1) * kLoads) / kMfma) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // a load from memory
+        if ((i * kWrites) / kMfma != ((i + 1) * kWrites) / kMfma) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // an LDS write
         __builtin_amdgcn_sched_group_barrier(0x006, 2, 0);   // what is left of address arithmetic
       }
       __syncthreads();
     };
-    float bva[4][T], bvb[4][T];
+    float bva[BPT][4][T], bvb[BPT][4][T];
     read_b(0, bva);
-    int rd = 1;                        // buffer of block b + 1
+    int rd = 1;                        // buffer of turn b + 1
     for (int b = b_begin; b < b_end; b += 2) {
-      int wr = rd == 2 ? 0 : rd + 1;   // buffer of block b + 2
+      int wr = rd == 2 ? 0 : rd + 1;   // buffer of turn b + 2
       turn(b, rd, wr, bva, bvb);
       rd = wr;
       if (b + 1 < b_end) {
@@ -3171,7 +3202,7 @@ __global__ __launch_bounds__(256) void conv_wgrad_reduce_kernel(float* __restric
 
 // The staging buffers of the larger tap sets pass the 64 KiB a kernel may use without asking.
 template <int HALVES, int T, bool DIRECT = false>
-int launch_wgrad_src(dim3 grid, size_t lds, hipStream_t s, int K, int nblocks, const float* aq, const float* xt,
+int launch_wgrad_src(dim3 grid, size_t lds, hipStream_t s, int K, int nturns, const float* aq, const float* xt,
     int x_bytes, int hin, const int* src, float* partial, int cpad, int mpad, int n_slices, int cpasses) {
   static std::atomic<size_t> allowed{0};
   if (lds > 64 * 1024 && allowed.load() < lds) {
@@ -3179,7 +3210,7 @@ int launch_wgrad_src(dim3 grid, size_t lds, hipStream_t s, int K, int nblocks, c
         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     allowed.store(lds);
   }
-  conv_wgrad_f32_lds_src_kernel<HALVES, T, DIRECT><<<grid, 256 * HALVES, lds, s>>>(K, nblocks, aq, xt, x_bytes, hin, src,
+  conv_wgrad_f32_lds_src_kernel<HALVES, T, DIRECT><<<grid, 256 * HALVES, lds, s>>>(K, nturns, aq, xt, x_bytes, hin, src,
       partial, cpad, mpad, n_slices, cpasses);
   OCNN_LAUNCH_OK("conv_wgrad_lds_src");
   return OCNN_OK;
@@ -3234,14 +3265,14 @@ void make_wgrad_plan(const ConvPlan& p, int M, int channel_in, int nempty, Wgrad
     w->src_slices = 256 * per_cu / tiles;
     if (w->src_slices < 1) w->src_slices = 1;
     if (w->src_slices > nblocks) w->src_slices = nblocks;
-    w->src_bytes = align256((size_t)nblocks * K * 8 * sizeof(int));
+    w->src_bytes = align256((size_t)(nblocks + 3) * K * 8 * sizeof(int));   // whole turns of up to four blocks
   }
   w->xt_bytes = align256(((size_t)p.btm_h + 1) * w->cpad * sizeof(float));
   int most_slices = w->n_slices > w->lds_slices ? w->n_slices : w->lds_slices;
   if (w->src_slices > most_slices) most_slices = w->src_slices;
   w->partial_bytes = align256((size_t)most_slices * p.taps.count * w->mpad * w->cpad * sizeof(float));
   w->ichild_bytes = nempty ? align256(sizeof(int) * (size_t)(p.ichild_h + 1)) : 0;
-  w->aq_bytes = align256((size_t)nblocks * 2 * w->mpad * 4 * sizeof(float));
+  w->aq_bytes = align256((size_t)(nblocks + 3) * 2 * w->mpad * 4 * sizeof(float));   // zero columns up to a whole turn
   w->total_bytes = w->xt_bytes + w->partial_bytes + w->ichild_bytes + w->aq_bytes + w->src_bytes;
 }
 
@@ -3293,7 +3324,10 @@ int run_wgrad(float* grad_w, const float* A, int M, const float* X, int channel_
     return OCNN_OK;
   }
   float* aq = reinterpret_cast<float*>(wsb + w.xt_bytes + w.partial_bytes + w.ichild_bytes);
-  const int n_quads = ((a.N + 7) / 8) * 2;
+  // whole turns of the LDS-staged kernel (columns past the last one are zero)
+  const int bpt = w.src_taps > 0 ? wgrad_src_blocks(w.src_taps) : 1;
+  const int nturns = ((a.N + 7) / 8 + bpt - 1) / bpt, nblocks_pad = nturns * bpt;
+  const int n_quads = nblocks_pad * 2;
   dim3 qg((n_quads * 4 + 63) / 64, (w.mpad + 63) / 64);
   interleave_quads_kernel<<<qg, 256, 0, s>>>(aq, A, M, a.N, w.mpad, n_quads);
   OCNN_LAUNCH_OK("interleave_quads");
@@ -3301,14 +3335,14 @@ int run_wgrad(float* grad_w, const float* A, int M, const float* X, int channel_
   if (a.mode == kModeS2Conv && a.K == 8 && !a.nempty && w.src_taps == 2 && (M & 63) == 0 && w.mpad == M &&
       w.cpad == channel_in && a.Hin == 8 * a.N && (int64_t)channel_in * a.Hin * 4 < (1ll << 31) &&
       (int64_t)n_quads * w.mpad * 16 < (1ll << 31) && (reinterpret_cast<uintptr_t>(X) & 15) == 0 && g_wgrad_lds.load()) {
-    const int nblocks = (a.N + 7) / 8;
     const int tiles = (w.cpad / 32) * (w.mpad / 64);
     const size_t lds = (size_t)wgrad_src_lds_rows(a.K, 2) * kWgLdsRow * sizeof(float);
-    int e = launch_wgrad_src<2, 2, true>(dim3(w.src_slices, tiles), lds, s, a.K, nblocks, aq, X, channel_in * a.Hin * 4,
-        a.Hin, nullptr, partial, w.cpad, w.mpad, w.src_slices, w.cpad / 32);
+    const int slices = std::min(w.src_slices, nturns);
+    int e = launch_wgrad_src<2, 2, true>(dim3(slices, tiles), lds, s, a.K, nturns, aq, X, channel_in * a.Hin * 4,
+        a.Hin, nullptr, partial, w.cpad, w.mpad, slices, w.cpad / 32);
     if (e) return e;
     const int64_t per = (int64_t)a.K * w.mpad * w.cpad;
-    conv_wgrad_reduce_kernel<<<blocks_for(per, 32), 256, 0, s>>>(grad_w, partial, w.src_slices, M, channel_in, a.K,
+    conv_wgrad_reduce_kernel<<<blocks_for(per, 32), 256, 0, s>>>(grad_w, partial, slices, M, channel_in, a.K,
         w.mpad, w.cpad);
     OCNN_LAUNCH_OK("conv_wgrad_reduce");
     return OCNN_OK;
@@ -3317,19 +3351,19 @@ int run_wgrad(float* grad_w, const float* A, int M, const float* X, int channel_
   transpose_rows_f32_kernel<<<tg, 256, 0, s>>>(xt, X, channel_in, a.Hin, w.cpad);
   OCNN_LAUNCH_OK("transpose_rows");
   const int64_t x_bytes = ((int64_t)a.Hin + 1) * w.cpad * 4;
-  const int64_t most_bytes = std::max(x_bytes, std::max((int64_t)((a.N + 7) / 8) * a.K * 32, (int64_t)((a.N + 7) / 8) * 2 * w.mpad * 16));
+  const int64_t most_bytes = std::max(x_bytes, std::max((int64_t)nblocks_pad * a.K * 32, (int64_t)nblocks_pad * 2 * w.mpad * 16));
   if (w.src_taps > 0 && w.mpad == M && w.cpad == channel_in && most_bytes < (1ll << 31) && g_wgrad_lds.load()) {
-    const int nblocks = (a.N + 7) / 8;
     int* src = reinterpret_cast<int*>(wsb + w.xt_bytes + w.partial_bytes + w.ichild_bytes + w.aq_bytes);
-    wgrad_sources_kernel<<<blocks_for((int64_t)nblocks * a.K * 8), kBlock, 0, s>>>(a, src, nblocks, w.cpad * 4);
+    const int slices = std::min(w.src_slices, nturns);
+    wgrad_sources_kernel<<<blocks_for((int64_t)nblocks_pad * a.K * 8), kBlock, 0, s>>>(a, src, nblocks_pad, w.cpad * 4);
     OCNN_LAUNCH_OK("wgrad_sources");
     const int halves = M == 32 ? 1 : 2;
     const int tiles = (w.cpad / 32) * (w.mpad / (32 * halves));
     const size_t lds = (size_t)wgrad_src_lds_rows(a.K, w.src_taps) * kWgLdsRow * sizeof(float);
     int e = OCNN_OK;
 #define OCNN_WGRAD_SRC(H_, T_)                                                                                    \
-    e = launch_wgrad_src<H_, T_>(dim3(w.src_slices, tiles), lds, s, a.K, nblocks, aq, xt, (int)x_bytes, a.Hin,    \
-        src, partial, w.cpad, w.mpad, w.src_slices, w.cpad / 32)
+    e = launch_wgrad_src<H_, T_>(dim3(slices, tiles), lds, s, a.K, nturns, aq, xt, (int)x_bytes, a.Hin,           \
+        src, partial, w.cpad, w.mpad, slices, w.cpad / 32)
     if (halves == 2) {
       if (w.src_taps == 7) OCNN_WGRAD_SRC(2, 7); else if (w.src_taps == 3) OCNN_WGRAD_SRC(2, 3);
       else if (w.src_taps == 2) OCNN_WGRAD_SRC(2, 2); else OCNN_WGRAD_SRC(2, 1);
@@ -3340,7 +3374,7 @@ int run_wgrad(float* grad_w, const float* A, int M, const float* X, int channel_
 #undef OCNN_WGRAD_SRC
     if (e) return e;
     const int64_t per = (int64_t)a.K * w.mpad * w.cpad;
-    conv_wgrad_reduce_kernel<<<blocks_for(per, 32), 256, 0, s>>>(grad_w, partial, w.src_slices, M, channel_in, a.K,
+    conv_wgrad_reduce_kernel<<<blocks_for(per, 32), 256, 0, s>>>(grad_w, partial, slices, M, channel_in, a.K,
         w.mpad, w.cpad);
     OCNN_LAUNCH_OK("conv_wgrad_reduce");
     return OCNN_OK;

@@ -94,6 +94,50 @@ def test_conv_grad_wide_channels(oc, orc, tree, ci, co):
   assert relerr(gd.cpu().numpy().reshape(egd.shape), egd) < TOL
 
 
+@pytest.mark.parametrize("ks,stride,nempty", [([3, 3, 3], 1, True), ([2, 2, 2], 2, False), ([2, 2, 2], 2, True),
+                                              ([3, 1, 1], 1, False), ([3, 3, 1], 1, True), ([3, 3, 3], 2, False)])
+@pytest.mark.parametrize("ci,co", [(32, 64), (64, 32), (96, 128)])
+def test_weight_gradient_staged_forms(oc, orc, tree, ks, stride, nempty, ci, co):
+  """The shapes other than 3x3x3 stride 1 over all nodes with whole 32-channel blocks: the weight
+  gradient stages its source rows in LDS from a table of row offsets (2x2x2 stride 2 over all nodes
+  reads the finer level in place).  Against the oracle, and against the register-fed kernel that
+  serves every other channel count (same products, another order of addition); both for the
+  convolution and for the deconvolution, whose weight gradient swaps the two tensors."""
+  host, dev, b = tree
+  L = oc.lib.get()
+  d, K = 5, ks[0] * ks[1] * ks[2]
+  rng = np.random.default_rng(ci * 7 + co + K)
+  hin = int(b.nnum_nempty[d] if nempty else b.nnum[d])
+  x = rng.standard_normal((ci, hin)).astype(np.float32)
+  w = (rng.standard_normal((co, ci * K)) * 0.1).astype(np.float32)
+  top_h = orc.octree_conv(x, w, host, d, co, ks, stride, nempty).shape[1]
+  g = rng.standard_normal((co, top_h)).astype(np.float32)
+  _, egw = orc.octree_conv_grad(x, w, g, host, d, co, ks, stride, nempty)
+  args = (T(x).cuda().view(1, ci, hin, 1), T(w).cuda(), dev, T(g).cuda().view(1, co, top_h, 1), d, co, ks, stride, nempty)
+  _, gw = oc.nn.octree_conv_grad(*args, need_data=False)
+  assert relerr(gw.cpu().numpy(), egw) < TOL
+  before = L.ocnn_conv_wgrad_staged(0)
+  try:
+    _, gw_reg = oc.nn.octree_conv_grad(*args, need_data=False)
+  finally:
+    L.ocnn_conv_wgrad_staged(before)
+  assert relerr(gw_reg.cpu().numpy(), egw) < TOL
+  assert relerr(gw.cpu().numpy(), gw_reg.cpu().numpy().astype(np.float64)) < TOL
+  _, again = oc.nn.octree_conv_grad(*args, need_data=False)
+  assert torch.equal(gw, again)   # fixed order of addition: the same bits run to run
+  # deconvolution at stride 2 lives one level up
+  dd = d - 1 if stride == 2 else d
+  hd = int(b.nnum_nempty[dd] if (nempty or stride == 2) else b.nnum[dd])
+  xd = rng.standard_normal((ci, hd)).astype(np.float32)
+  wd = (rng.standard_normal((ci, co * K)) * 0.1).astype(np.float32)
+  top_d = orc.octree_deconv(xd, wd, host, dd, co, ks, stride, nempty).shape[1]
+  gd_ = rng.standard_normal((co, top_d)).astype(np.float32)
+  _, egw = orc.octree_deconv_grad(xd, wd, gd_, host, dd, co, ks, stride, nempty)
+  _, gw = oc.nn.octree_deconv_grad(T(xd).cuda().view(1, ci, hd, 1), T(wd).cuda(), dev, T(gd_).cuda().view(1, co, top_d, 1),
+                                   dd, co, ks, stride, nempty, need_data=False)
+  assert relerr(gw.cpu().numpy(), egw) < TOL
+
+
 def test_grad_errors(oc, tree):
   host, dev, b = tree
   x = torch.zeros(1, 4, int(b.nnum[5]), 1, device="cuda")
