@@ -433,9 +433,9 @@ def main():
     q = key9[torch.randint(0, H9, (1 << 20,), generator=g).to(dev)]
     hbm("search_key_d9_1Mq", timed(lambda: F.octree_search_key(q, octree, 9, False, False), reps, wu),
         (1 << 20) * 12)
-    # a binary search over 1.5 M keys per query: the counters show 456 MB fetched per launch
-    # (profiles/hbm_counters__bench_default_workloads.md), 435 bytes per query
-    extra["search_key_d9_1Mq"]["GBs_fetched_by_counters"] = 460.5e6 / extra["search_key_d9_1Mq"]["ms"] / 1e6
+    # 1 M random queries in 1.5 M keys through the sample tables of ocnn_search_key_indexed: a line
+    # of the fine table (L2) and a line of keys per query; the plain binary search took 0.086 ms and
+    # fetched 435 bytes per query (profiles/hbm_counters__bench_default_workloads.md has the counters)
     lab = (child8 >= 0).to(torch.int32)
     P = lambda t_: Ct.c_void_p(t_.data_ptr())
     lab_out = torch.empty_like(lab)

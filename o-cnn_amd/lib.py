@@ -13,7 +13,7 @@ INFO_BYTES, HEADER_BYTES, POINTS_INFO_BYTES = 716, 720, 88
 _SIZE_T = ("ocnn_generate_label_scratch_bytes", "ocnn_points2octree_workspace_bytes",
            "ocnn_octree_batch_workspace_bytes", "ocnn_octree_update_scratch_bytes",
            "ocnn_points_workspace_bytes", "ocnn_octree_interp_workspace_bytes", "ocnn_octree_interp_backward_workspace_bytes",
-           "ocnn_octree_gatherbk_workspace_bytes")
+           "ocnn_octree_gatherbk_workspace_bytes", "ocnn_search_key_workspace_bytes")
 _INT64 = ("ocnn_info_ptr_dis", "ocnn_info_sizeof_octree")
 
 

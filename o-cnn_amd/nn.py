@@ -1086,6 +1086,17 @@ def _morton_keys(octree, info, depth, nempty=False):
   return des, des_h
 
 
+def _search_key(out, keys, n_key, query, n_query):
+  """Position of each query in the sorted `keys`, -1 on a miss; many queries in a large array go
+  through sample tables in the workspace (ocnn_search_key_indexed decides)."""
+  L = _lib.get()
+  nbytes = L.ocnn_search_key_workspace_bytes(n_key)
+  ws = _workspace(nbytes + 16, "search")
+  base = (ws.data_ptr() + 15) & ~15
+  _lib.call("ocnn_search_key_indexed", _ptr(out), _ptr(keys), n_key, _ptr(query), n_query, C.c_void_p(base),
+            C.c_size_t(nbytes), _stream())
+
+
 def octree_search_key(key, octree, depth, key_is_xyz, nempty):
   """pytorch/cpp/octree_key.cpp:83-132: index of each query key at `depth`, -1 on a miss."""
   octree = _to_dev(octree)
@@ -1100,7 +1111,7 @@ def octree_search_key(key, octree, depth, key_is_xyz, nempty):
     key = tmp
   des, des_h = _morton_keys(octree, info, depth, nempty)
   out = torch.empty(n_query, dtype=torch.int32, device=octree.device)
-  _lib.call("ocnn_search_key", _ptr(out), _ptr(des), des_h, _ptr(key), n_query, _stream())
+  _search_key(out, des, des_h, key, n_query)
   return out
 
 
@@ -1188,7 +1199,7 @@ def octree_align(src_data, src_octree, des_octree, depth):
   src_key, _ = _morton_keys(src_octree, sinfo, depth)
   des_key, des_h = _morton_keys(des_octree, dinfo, depth)
   idx = torch.empty(src_h, dtype=torch.int32, device=src_data.device)
-  _lib.call("ocnn_search_key", _ptr(idx), _ptr(des_key), des_h, _ptr(src_key), src_h, _stream())
+  _search_key(idx, des_key, des_h, src_key, src_h)
   out = torch.empty(1, channel, des_h, 1, dtype=torch.float32, device=src_data.device)
   inverse = torch.empty(max(des_h, 1), dtype=torch.int32, device=src_data.device)
   _lib.call("ocnn_align_forward_ws", _ptr(out), des_h, channel, _ptr(src_data), src_h, _ptr(idx), _ptr(inverse),

@@ -463,6 +463,45 @@ def test_generate_key_label_search(oc, orc):
   assert np.array_equal(idx.cpu().numpy(), orc.search_key(keys, q))
 
 
+@pytest.mark.parametrize("n_key", [16384, 16385, 40000, 65536 + 17, 1 << 20])
+def test_search_key_through_sample_tables(oc, orc, n_key):
+  """search_key_gpu (octree_nn.h:180-181) for many queries in a large array: two tables of samples
+  (every 256th and every 16th key) written per call, the same positions as the plain search.
+  Sizes around the table strides, queries below the first and above the last key, every sampled
+  key and its neighbours, runs of equal keys (the first one is the answer, as lower_bound gives)."""
+  import ctypes as C
+  st = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)
+  P = lambda t: C.c_void_p(t.data_ptr())
+  rng = np.random.default_rng(n_key)
+  keys = np.sort(rng.integers(1000, 1 << 50, n_key).astype(np.uint64))
+  if n_key == 40000:   # runs of equal keys across the sample boundaries
+    keys[240:300] = keys[240]
+    keys[4090:4100] = keys[4090]
+    keys = np.sort(keys)
+  hits = np.concatenate([keys[::16], keys[15::16], keys[1::256], keys[-3:], keys[:3]])
+  q = np.concatenate([hits, hits + np.uint64(1), rng.integers(0, 1 << 50, 30000).astype(np.uint64),
+                      np.array([0, 999, keys[-1] + np.uint64(5), (1 << 63)], dtype=np.uint64)])
+  q = q[rng.permutation(q.size)]
+  assert q.size >= 16384
+  keys_d, q_d = T(keys.view(np.int64)).cuda(), T(q.view(np.int64)).cuda()
+  idx = torch.full((q.size,), -7, dtype=torch.int32, device="cuda")
+  nb = oc.lib.get().ocnn_search_key_workspace_bytes(n_key)
+  ws = torch.empty(nb, dtype=torch.uint8, device="cuda")
+  oc.lib.call("ocnn_search_key_indexed", P(idx), P(keys_d), n_key, P(q_d), q.size, P(ws), C.c_size_t(nb), st())
+  exp = orc.search_key(keys, q)
+  assert np.array_equal(idx.cpu().numpy(), exp)
+  plain = torch.empty_like(idx)
+  oc.lib.call("ocnn_search_key", P(plain), P(keys_d), n_key, P(q_d), q.size, st())
+  assert torch.equal(idx, plain)
+  # few queries: the call is the plain search and needs no workspace
+  few = torch.empty(100, dtype=torch.int32, device="cuda")
+  oc.lib.call("ocnn_search_key_indexed", P(few), P(keys_d), n_key, P(q_d), 100, None, C.c_size_t(0), st())
+  assert np.array_equal(few.cpu().numpy(), exp[:100])
+  with pytest.raises(oc.lib.OcnnError) as e:
+    oc.lib.call("ocnn_search_key_indexed", P(idx), P(keys_d), n_key, P(q_d), q.size, P(ws), C.c_size_t(64), st())
+  assert e.value.code == -4
+
+
 def test_grow_md5_on_gpu(oc, samples):
   """pytorch/test/test_octree_grow.py: rebuild octree_2 with new/grow/update/set_property."""
   F = oc.nn
