@@ -167,7 +167,7 @@ int ocnn_search_key(int* idx, const uint64_t* key, int n_key, const uint64_t* qu
 /* search_key_gpu (octree/octree/octree_nn.h:180-181) for many queries in a large array: the same
  * result (position of the first equal key, -1 on a miss), through two tables of samples of `key`
  * that the call writes into workspace_dev (every 256th and every 16th key;
- * ocnn_search_key_workspace_bytes(n_key) bytes, 16-byte aligned).  With fewer than 16384 queries or
+ * ocnn_search_key_workspace_bytes(n_key) bytes, 128-byte aligned).  With fewer than 16384 queries or
  * keys, or more than 3.1 M keys, the call is ocnn_search_key and the workspace may be null. */
 size_t ocnn_search_key_workspace_bytes(int n_key);
 int ocnn_search_key_indexed(int* idx, const uint64_t* key, int n_key, const uint64_t* query,

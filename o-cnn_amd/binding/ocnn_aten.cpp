@@ -391,8 +391,8 @@ Tensor octree_search_key(Tensor key, Tensor octree, int depth, bool key_is_xyz, 
   if (ocnn_info_is_key2xyz(info.p()) && des_h > 0) des = key_op(des, depth, true);
   Tensor out = torch::empty({key.numel()}, octree.options().dtype(torch::kInt32));
   // many queries in a large array go through sample tables in a scratch tensor of this call
-  Tensor ws = torch::empty({(int64_t)ocnn_search_key_workspace_bytes(des_h) + 16}, octree.options().dtype(torch::kUInt8));
-  void* base = reinterpret_cast<void*>((reinterpret_cast<uintptr_t>(ws.data_ptr()) + 15) & ~(uintptr_t)15);
+  Tensor ws = torch::empty({(int64_t)ocnn_search_key_workspace_bytes(des_h) + 128}, octree.options().dtype(torch::kUInt8));
+  void* base = reinterpret_cast<void*>((reinterpret_cast<uintptr_t>(ws.data_ptr()) + 127) & ~(uintptr_t)127);
   check(ocnn_search_key_indexed(out.data_ptr<int>(), reinterpret_cast<const uint64_t*>(des.data_ptr<int64_t>()), des_h,
       reinterpret_cast<const uint64_t*>(key.data_ptr<int64_t>()), (int)key.numel(), base,
       ocnn_search_key_workspace_bytes(des_h), current_stream()));

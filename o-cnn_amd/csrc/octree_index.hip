@@ -136,11 +136,14 @@ __global__ void search_key_kernel(int* __restrict__ idx, const uint64_t* __restr
 // one line of keys, each line once (16 lanes read a window together).  A window starts at the
 // last sample BELOW the query, so the first of several equal keys is found as lower_bound does.
 constexpr int kSearchFine = 16, kSearchCoarse = 256, kSearchLdsMax = 96 * 1024;
+// `shift` = elements between the 128-byte line that holds key[0] and key[0]: the windows of 16
+// keys are cut at line boundaries of the array as it lies in memory, sample e is the first key of
+// window e (the first window is short), so that a window is one line whatever the array's address.
 __global__ void search_tables_kernel(uint64_t* __restrict__ t1, int n1, uint64_t* __restrict__ t2, int n2,
-    const uint64_t* __restrict__ key) {
+    const uint64_t* __restrict__ key, int shift) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n2) t2[i] = key[(int64_t)i * kSearchFine];
-  if (i < n1) t1[i] = key[(int64_t)i * kSearchCoarse];
+  if (i < n2) t2[i] = key[max(i * kSearchFine - shift, 0)];
+  if (i < n1) t1[i] = key[max(i * kSearchCoarse - shift, 0)];
 }
 // number of elements below q in a[lo, hi)
 __device__ inline int count_below(const uint64_t* a, int lo, int hi, uint64_t q) {
@@ -151,8 +154,8 @@ __device__ inline int count_below(const uint64_t* a, int lo, int hi, uint64_t q)
   return lo;
 }
 // For every lane of the wavefront: the number of elements below the lane's q among the 16 elements
-// a[base .. base + 15] (base a multiple of 16: one 128-byte line; elements from n on count as not
-// below).  A wavefront's loads cost by the lines they touch, and a lane that walks its own window
+// a[base .. base + 15] (one 128-byte line; places in front of the array count as below, elements
+// from n on as not below).  A wavefront's loads cost by the lines they touch, and a lane that walks its own window
 // touches a line per probe; here 16 lanes read one window together, four windows a round, and the
 // 16 rounds of a wavefront are independent of one another.  Every lane must call.
 constexpr int kSearchBlock = 1024;
@@ -166,15 +169,15 @@ __device__ inline int window_count(const uint64_t* __restrict__ a, int base, int
     const int b = __shfl(base, owner, 64);
     const uint64_t qq = ((uint64_t)(uint32_t)__shfl((int)q_hi, owner, 64) << 32) | (uint32_t)__shfl((int)q_lo, owner, 64);
     const int at = b + sub;
-    const uint64_t v = a[min(at, n - 1)];
-    const unsigned long long below = __ballot(at < n && v < qq);
+    const uint64_t v = a[min(max(at, 0), n - 1)];
+    const unsigned long long below = __ballot(at < 0 || (at < n && v < qq));   // (places in front of the array: below)
     if ((lane >> 2) == r) mine = __popcll((below >> (16 * (lane & 3))) & 0xffffull);
   }
   return mine;
 }
 __global__ __launch_bounds__(kSearchBlock) void search_key_indexed_kernel(int* __restrict__ idx,
     const uint64_t* __restrict__ key, int n_key, const uint64_t* __restrict__ t1, int n1, const uint64_t* __restrict__ t2,
-    int n2, const uint64_t* __restrict__ query, int n_query, int per_block) {
+    int n2, const uint64_t* __restrict__ query, int n_query, int per_block, int shift) {
   extern __shared__ __attribute__((aligned(16))) uint64_t s_t1[];
   {   // the coarse table, 16 bytes a lane (its row is padded to whole units)
     const ulonglong2* src = reinterpret_cast<const ulonglong2*>(t1);
@@ -192,7 +195,7 @@ __global__ __launch_bounds__(kSearchBlock) void search_key_indexed_kernel(int* _
     // the sample below q bounds the window from the left, the next sample (not below q) from the right
     const int e0 = max(count_below(s_t1, 0, n1, q) - 1, 0) * (kSearchCoarse / kSearchFine);
     const int e2 = max(e0 + window_count(t2, e0, n2, q) - 1, e0);
-    const int k0 = e2 * kSearchFine;
+    const int k0 = e2 * kSearchFine - shift;
     const int lo = k0 + window_count(key, k0, n_key, q);
     if (i < end) idx[i] = (lo < n_key && key[lo] == q) ? lo : -1;
   }
@@ -305,7 +308,7 @@ int ocnn_search_key(int* idx, const uint64_t* key, int n_key, const uint64_t* qu
 
 size_t ocnn_search_key_workspace_bytes(int n_key) {
   if (n_key < 0) return 0;
-  const size_t n1 = ((size_t)n_key + kSearchCoarse - 1) / kSearchCoarse, n2 = ((size_t)n_key + kSearchFine - 1) / kSearchFine;
+  const size_t n1 = ((size_t)n_key + 15 + kSearchCoarse - 1) / kSearchCoarse, n2 = ((size_t)n_key + 15 + kSearchFine - 1) / kSearchFine;
   return (n1 + n2) * sizeof(uint64_t) + 512;
 }
 
@@ -313,18 +316,19 @@ int ocnn_search_key_indexed(int* idx, const uint64_t* key, int n_key, const uint
     void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream) {
   OCNN_REQUIRE(idx && query && (key || n_key == 0) && n_key >= 0 && n_query >= 0, OCNN_E_BADARG, "bad argument");
   if (n_query == 0) return OCNN_OK;
-  const int n1 = (n_key + kSearchCoarse - 1) / kSearchCoarse, n2 = (n_key + kSearchFine - 1) / kSearchFine;
+  const int shift = (int)((reinterpret_cast<uintptr_t>(key) & 127) / sizeof(uint64_t));
+  const int n1 = (n_key + shift + kSearchCoarse - 1) / kSearchCoarse, n2 = (n_key + shift + kSearchFine - 1) / kSearchFine;
   const size_t lds = (size_t)n1 * sizeof(uint64_t);
   // few queries, few keys, or more coarse samples than a workgroup can hold: the plain search
   if (n_query < 16384 || n_key < 16384 || lds > (size_t)kSearchLdsMax)
     return ocnn_search_key(idx, key, n_key, query, n_query, stream);
   OCNN_REQUIRE(workspace_dev && workspace_bytes >= ocnn_search_key_workspace_bytes(n_key), OCNN_E_WORKSPACE,
       "workspace %zu < %zu bytes", workspace_bytes, ocnn_search_key_workspace_bytes(n_key));
-  OCNN_REQUIRE((reinterpret_cast<uintptr_t>(workspace_dev) & 15) == 0, OCNN_E_WORKSPACE, "workspace not 16-byte aligned");
+  OCNN_REQUIRE((reinterpret_cast<uintptr_t>(workspace_dev) & 127) == 0, OCNN_E_WORKSPACE, "workspace not 128-byte aligned");
   hipStream_t s = as_stream(stream);
   uint64_t* t1 = static_cast<uint64_t*>(workspace_dev);
-  uint64_t* t2 = t1 + ((n1 + 31) & ~31);
-  search_tables_kernel<<<blocks_for(n2), kBlock, 0, s>>>(t1, n1, t2, n2, key);
+  uint64_t* t2 = t1 + ((n1 + 31) & ~31);    // on a line boundary as well
+  search_tables_kernel<<<blocks_for(n2), kBlock, 0, s>>>(t1, n1, t2, n2, key, shift);
   OCNN_LAUNCH_OK("search_tables");
   static std::atomic<size_t> allowed{0};
   if (lds > 64 * 1024 && allowed.load() < lds) {
@@ -338,7 +342,7 @@ int ocnn_search_key_indexed(int* idx, const uint64_t* key, int n_key, const uint
   while (per_block > kSearchBlock && (n_query + per_block - 1) / per_block < 512) per_block >>= 1;
   const int blocks = (n_query + per_block - 1) / per_block;
   search_key_indexed_kernel<<<blocks, kSearchBlock, (lds + 15) & ~(size_t)15, s>>>(idx, key, n_key, t1, n1, t2, n2, query,
-      n_query, per_block);
+      n_query, per_block, shift);
   OCNN_LAUNCH_OK("search_key_indexed");
   return OCNN_OK;
 }

@@ -1091,8 +1091,8 @@ def _search_key(out, keys, n_key, query, n_query):
   through sample tables in the workspace (ocnn_search_key_indexed decides)."""
   L = _lib.get()
   nbytes = L.ocnn_search_key_workspace_bytes(n_key)
-  ws = _workspace(nbytes + 16, "search")
-  base = (ws.data_ptr() + 15) & ~15
+  ws = _workspace(nbytes + 128, "search")
+  base = (ws.data_ptr() + 127) & ~127
   _lib.call("ocnn_search_key_indexed", _ptr(out), _ptr(keys), n_key, _ptr(query), n_query, C.c_void_p(base),
             C.c_size_t(nbytes), _stream())
 

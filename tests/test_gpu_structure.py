@@ -483,13 +483,20 @@ def test_search_key_through_sample_tables(oc, orc, n_key):
                       np.array([0, 999, keys[-1] + np.uint64(5), (1 << 63)], dtype=np.uint64)])
   q = q[rng.permutation(q.size)]
   assert q.size >= 16384
-  keys_d, q_d = T(keys.view(np.int64)).cuda(), T(q.view(np.int64)).cuda()
-  idx = torch.full((q.size,), -7, dtype=torch.int32, device="cuda")
+  q_d = T(q.view(np.int64)).cuda()
   nb = oc.lib.get().ocnn_search_key_workspace_bytes(n_key)
   ws = torch.empty(nb, dtype=torch.uint8, device="cuda")
-  oc.lib.call("ocnn_search_key_indexed", P(idx), P(keys_d), n_key, P(q_d), q.size, P(ws), C.c_size_t(nb), st())
   exp = orc.search_key(keys, q)
-  assert np.array_equal(idx.cpu().numpy(), exp)
+  # the windows are cut at the 128-byte lines of the array as it lies in memory: every offset of
+  # its first key inside a line (a key array inside an octree blob starts anywhere)
+  padded = torch.zeros(n_key + 16, dtype=torch.int64, device="cuda")
+  for off in (0, 1, 7, 15):
+    keys_d = padded[off:off + n_key]
+    keys_d.copy_(T(keys.view(np.int64)))
+    assert (keys_d.data_ptr() & 127) == 8 * off
+    idx = torch.full((q.size,), -7, dtype=torch.int32, device="cuda")
+    oc.lib.call("ocnn_search_key_indexed", P(idx), P(keys_d), n_key, P(q_d), q.size, P(ws), C.c_size_t(nb), st())
+    assert np.array_equal(idx.cpu().numpy(), exp), off
   plain = torch.empty_like(idx)
   oc.lib.call("ocnn_search_key", P(plain), P(keys_d), n_key, P(q_d), q.size, st())
   assert torch.equal(idx, plain)
