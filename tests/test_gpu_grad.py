@@ -218,3 +218,45 @@ def test_weight_gradient_identity_at_full_size(oc, synthetic):
   assert abs(lhs - rhs) < 1e-4 * max(abs(lhs), abs(rhs), (gd.double().norm() * x2.double().norm()).item() * 1e-2)
   _, gw_again = F.octree_conv_grad(x, w, octree, gy, 7, 64, [3, 3, 3], 1, False)
   assert torch.equal(gw, gw_again)
+
+
+@pytest.mark.parametrize("ks,stride,nempty", [([3, 3, 3], 1, True), ([2, 2, 2], 2, False), ([2, 2, 2], 2, True)])
+def test_staged_weight_gradient_identity_at_full_size(oc, synthetic, ks, stride, nempty):
+  """Depth-7 batch of four 50 k clouds, 64 -> 64: <grad_w, W'> == <grad_out, conv(x; W')> for the
+  shapes whose weight gradient stages its rows from a table (or reads the finer level in place),
+  both sides on the GPU, and the same bits run to run."""
+  F = oc.nn
+  clouds = []
+  for i in range(4):
+    p, n, _ = synthetic.shape_cloud(50000, 200 + i)
+    blob = make_points_blob(p, n)
+    t = T(blob).cuda()
+    t._ocnn_points_info = blob[:88].copy()
+    clouds.append(t)
+  octree = F.points2octree_batch(clouds, 7, 2)
+  info = F.octree_info(octree)
+  K = ks[0] * ks[1] * ks[2]
+  hin = info.nnum_nempty(7) if nempty else info.nnum(7)
+  g = torch.Generator().manual_seed(4)
+  x = torch.randn(1, 64, hin, 1, generator=g).cuda()
+  w = (torch.randn(64, 64 * K, generator=g) * 0.02).cuda()
+  w2 = torch.randn(64, 64 * K, generator=g).cuda()
+  y = F.octree_conv(x, w2, octree, 7, 64, ks, stride, nempty)
+  gy = torch.randn(y.shape, generator=g).cuda()
+  _, gw = F.octree_conv_grad(x, w, octree, gy, 7, 64, ks, stride, nempty, need_data=False)
+  lhs = (gw.double() * w2.double()).sum().item()
+  rhs = (gy.double() * y.double()).sum().item()
+  assert abs(lhs - rhs) < 1e-4 * max(abs(lhs), abs(rhs), (gw.double().norm() * w2.double().norm()).item() * 1e-2)
+  _, again = F.octree_conv_grad(x, w, octree, gy, 7, 64, ks, stride, nempty, need_data=False)
+  assert torch.equal(gw, again)
+  # the deconvolution's weight gradient: the same geometry with the tensors swapped
+  d = 6 if stride == 2 else 7
+  hd = info.nnum_nempty(d) if (nempty or stride == 2) else info.nnum(d)
+  xd = torch.randn(1, 64, hd, 1, generator=g).cuda()
+  wd2 = torch.randn(64, 64 * K, generator=g).cuda()
+  yd = F.octree_deconv(xd, wd2, octree, d, 64, ks, stride, nempty)
+  gyd = torch.randn(yd.shape, generator=g).cuda()
+  _, gwd = F.octree_deconv_grad(xd, w, octree, gyd, d, 64, ks, stride, nempty, need_data=False)
+  lhs = (gwd.double() * wd2.double()).sum().item()
+  rhs = (gyd.double() * yd.double()).sum().item()
+  assert abs(lhs - rhs) < 1e-4 * max(abs(lhs), abs(rhs), (gwd.double().norm() * wd2.double().norm()).item() * 1e-2)
