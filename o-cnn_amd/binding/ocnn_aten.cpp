@@ -10,6 +10,8 @@
 #include <c10/hip/HIPStream.h>
 #include <c10/util/intrusive_ptr.h>
 
+#include <dlfcn.h>
+
 #include <cstring>
 #include <mutex>
 #include <unordered_map>
@@ -541,6 +543,361 @@ Tensor octree_conv_rows(Tensor rows_in, int channel_in, Tensor weights, Tensor b
   return out;
 }
 
+// ---- serialized point clouds (octree/octree/points_info.h:35-39: 88-byte header, then the xyz, normal,
+// feature and label arrays, point-major) -------------------------------------------------------------------------
+namespace {
+struct PointsHeader {   // host copy of a cloud's header: a blocking read when the cloud lives on the device
+  unsigned char bytes[OCNN_POINTS_INFO_BYTES];
+  explicit PointsHeader(const Tensor& points) {
+    TORCH_CHECK(points.scalar_type() == torch::kUInt8 && points.dim() == 1 && points.is_contiguous() &&
+        points.numel() >= OCNN_POINTS_INFO_BYTES, "a point cloud is a contiguous 1-D uint8 tensor of at least ",
+        OCNN_POINTS_INFO_BYTES, " bytes");
+    Tensor head = points.slice(0, 0, OCNN_POINTS_INFO_BYTES).cpu();
+    std::memcpy(bytes, head.data_ptr(), OCNN_POINTS_INFO_BYTES);
+    TORCH_CHECK(std::memcmp(bytes, "_POINTS_1.0_", 12) == 0, "The version of points format is not _POINTS_1.0_");
+    TORCH_CHECK(pt_num() > 0 && offset(4) <= points.numel(), "point cloud tensor shorter than its header says");
+  }
+  int word(int i) const { int v; std::memcpy(&v, bytes + 16 + 4 * i, 4); return v; }
+  int pt_num() const { return word(0); }
+  bool has(int t) const { return (word(1) >> t & 1) && word(2 + t) > 0; }
+  int channel(int t) const { return word(2 + t); }
+  int64_t offset(int t) const { return word(10 + t); }   // t = 4: the size of the cloud
+};
+
+Tensor on_device(const Tensor& t) {
+  return t.is_cuda() ? t.contiguous() : t.contiguous().to(torch::Device(torch::kCUDA, c10::hip::current_device()));
+}
+
+int points_ptype(const string& property) {   // get_ptype, pytorch/cpp/points_property.cpp:9-24
+  if (property == "xyz" || property == "xyzi") return 0;
+  if (property == "normal") return 1;
+  if (property == "feature") return 2;
+  if (property == "label") return 3;
+  TORCH_CHECK(false, "Unsupported Property: ", property);
+}
+
+// [pt_num, channel] float view of a property inside the cloud, undefined when the cloud has none
+Tensor points_array(const Tensor& points, const PointsHeader& h, int t) {
+  if (!h.has(t)) return Tensor();
+  return torch::from_blob(static_cast<unsigned char*>(points.data_ptr()) + h.offset(t), {h.pt_num(), h.channel(t)},
+      points.options().dtype(torch::kFloat32));
+}
+
+const float* three_floats(vector<float>& v, const char* what) {   // resize_with_last_val on floats
+  TORCH_CHECK(!v.empty() && v.size() <= 3, what, " holds one to three numbers");
+  while (v.size() < 3) v.push_back(v.back());
+  return v.data();
+}
+
+struct Aligned {   // scratch bytes of one call, 256-byte aligned
+  Tensor t;
+  void* p;
+  Aligned(const Tensor& like, size_t n) : t(torch::empty({(int64_t)n + 256}, like.options().dtype(torch::kUInt8))) {
+    p = reinterpret_cast<void*>((reinterpret_cast<uintptr_t>(t.data_ptr()) + 255) & ~(uintptr_t)255);
+  }
+};
+
+// the allocator the library calls back for scratch blocks and the result of a build or a scan
+struct TensorPool {
+  torch::TensorOptions options;
+  vector<Tensor> blocks;
+  static void* alloc(size_t bytes, void* ctx) {
+    TensorPool* self = static_cast<TensorPool*>(ctx);
+    self->blocks.push_back(torch::empty({(int64_t)std::max<size_t>(bytes, 1)}, self->options));
+    return self->blocks.back().data_ptr();
+  }
+  Tensor take(void* p) const {   // (scratch blocks come first: the last match is the result)
+    for (auto it = blocks.rbegin(); it != blocks.rend(); ++it)
+      if (it->data_ptr() == p) return *it;
+    TORCH_CHECK(false, "the library returned memory that its allocator did not hand out");
+  }
+};
+}  // namespace
+
+// ---- pytorch/cpp/points_property.cpp:38-165 ------------------------------------------------------------------
+Tensor points_new(Tensor pts, Tensor normals, Tensor features, Tensor labels) {
+  TORCH_CHECK(pts.defined() && pts.numel() > 0 && pts.numel() % 3 == 0, "Error occurs when setting points");
+  pts = pts.reshape({-1, 3}).to(torch::kFloat32).contiguous();
+  const int64_t n = pts.size(0);
+  vector<Tensor> parts;
+  int chans[4] = {3, 0, 0, 0}, flags = 1;
+  const Tensor* rest[3] = {&normals, &features, &labels};
+  parts.push_back(Tensor());   // the header's place
+  parts.push_back(pts.reshape({-1}).view(torch::kUInt8));
+  for (int i = 1; i < 4; ++i) {
+    const Tensor& a = *rest[i - 1];
+    if (!a.defined() || a.numel() == 0) continue;
+    TORCH_CHECK(a.numel() % n == 0, "Error occurs when setting points");
+    Tensor b = a.reshape({n, -1}).to(torch::kFloat32).to(pts.device()).contiguous();
+    TORCH_CHECK((i != 1 || b.size(1) == 3) && (i != 3 || b.size(1) == 1), "normals need 3 channels and labels 1");
+    chans[i] = (int)b.size(1);
+    flags |= 1 << i;
+    parts.push_back(b.reshape({-1}).view(torch::kUInt8));
+  }
+  Tensor hdr = torch::zeros({OCNN_POINTS_INFO_BYTES}, torch::TensorOptions().dtype(torch::kUInt8));
+  unsigned char* h = hdr.data_ptr<uint8_t>();
+  std::memcpy(h, "_POINTS_1.0_", 12);
+  int words[18] = {0};
+  words[0] = (int)n;
+  words[1] = flags;
+  int64_t dis = OCNN_POINTS_INFO_BYTES;
+  for (int t = 0; t < 4; ++t) {
+    words[2 + t] = chans[t];
+    words[10 + t] = (int)dis;
+    dis += 4 * n * chans[t];
+  }
+  words[14] = (int)dis;
+  std::memcpy(h + 16, words, sizeof(words));
+  parts[0] = hdr.to(pts.device());
+  return torch::cat(parts);
+}
+
+Tensor points_property(Tensor points, string property) {
+  points = points.contiguous();
+  PointsHeader h(points);
+  Tensor a = points_array(points, h, points_ptype(property));
+  return a.defined() ? a.clone() : a;
+}
+
+Tensor points_batch_property(vector<Tensor> tensors_in, string property) {
+  const int t = points_ptype(property);
+  vector<Tensor> parts;
+  int channel = -1;
+  for (size_t i = 0; i < tensors_in.size(); ++i) {
+    Tensor p = tensors_in[i].contiguous();
+    PointsHeader h(p);
+    Tensor a = points_array(p, h, t);
+    TORCH_CHECK(a.defined(), "The specified property does not exist.");
+    if (channel < 0) channel = h.channel(t);
+    TORCH_CHECK(h.channel(t) == channel, "The specified channel_out is wrong.");
+    if (property == "xyzi") a = torch::cat({a, torch::full({h.pt_num(), 1}, (float)i, a.options())}, 1);
+    parts.push_back(a);
+  }
+  return torch::cat(parts, 0);
+}
+
+Tensor points_set_property(Tensor points, Tensor data, string property) {
+  TORCH_CHECK(data.dim() == 2, "data is [pt_num, channel]");
+  points = points.contiguous();
+  PointsHeader h(points);
+  const int t = points_ptype(property);
+  TORCH_CHECK(h.has(t), "The property does not exist.");
+  TORCH_CHECK(data.size(1) == h.channel(t), "The channel is wrong.");
+  TORCH_CHECK(data.size(0) == h.pt_num(), "The point number is wrong.");
+  Tensor out = points.clone();
+  points_array(out, h, t).copy_(data.to(torch::kFloat32));
+  return out;
+}
+
+// ---- pytorch/cpp/transform_points.cpp:7-125, on the device ------------------------------------------------------
+vector<float> bounding_sphere(Tensor data_in, string method) {
+  Tensor points = on_device(data_in);
+  PointsHeader h(data_in.is_cuda() ? points : data_in.contiguous());
+  const size_t wb = ocnn_points_workspace_bytes(h.pt_num());
+  Aligned ws(points, wb);
+  vector<float> out(4);
+  check(ocnn_bounding_sphere(points.data_ptr(), h.bytes, method == "sphere" ? 0 : 1, out.data(), ws.p, wb,
+      current_stream()));
+  return out;
+}
+
+Tensor normalize_points(Tensor data_in, float radius, vector<float> center) {
+  Tensor points = on_device(data_in);
+  PointsHeader h(data_in.is_cuda() ? points : data_in.contiguous());
+  Tensor out = torch::empty_like(points);
+  check(ocnn_normalize_points(out.data_ptr(), points.data_ptr(), h.bytes, radius, three_floats(center, "center"),
+      current_stream()));
+  return out;
+}
+
+Tensor transform_points(Tensor data_in, vector<float> angle, vector<float> scale, vector<float> jitter, float offset,
+    string normal_axis) {
+  Tensor points = on_device(data_in);
+  PointsHeader h(data_in.is_cuda() ? points : data_in.contiguous());
+  Tensor out = torch::empty_like(points);
+  check(ocnn_transform_points(out.data_ptr(), points.data_ptr(), h.bytes, three_floats(angle, "angle"),
+      three_floats(scale, "scale"), three_floats(jitter, "jitter"), offset, normal_axis.c_str(), current_stream()));
+  return out;
+}
+
+vector<Tensor> clip_points(Tensor data_in, vector<float> bbmin, vector<float> bbmax) {
+  Tensor points = on_device(data_in);
+  PointsHeader h(data_in.is_cuda() ? points : data_in.contiguous());
+  Tensor out = torch::empty_like(points);
+  Tensor mask = torch::empty({h.pt_num()}, points.options().dtype(torch::kInt32));
+  unsigned char new_hdr[OCNN_POINTS_INFO_BYTES];
+  const size_t wb = ocnn_points_workspace_bytes(h.pt_num());
+  Aligned ws(points, wb);
+  check(ocnn_clip_points(out.data_ptr(), new_hdr, mask.data_ptr<int>(), points.data_ptr(), h.bytes,
+      three_floats(bbmin, "bbmin"), three_floats(bbmax, "bbmax"), ws.p, wb, current_stream()));
+  return {out, mask};
+}
+
+// ---- pytorch/cpp/point2octree.cpp:5-34 ----------------------------------------------------------------------------
+Tensor points2octree(Tensor points_in, int depth, int full_depth, bool node_dis, bool node_feature, bool split_label,
+    bool adaptive, int adp_depth, float th_normal, float th_distance, bool extrapolate, bool save_pts, bool key2xyz) {
+  Tensor points = on_device(points_in);
+  PointsHeader h(points_in.is_cuda() ? points : points_in.contiguous());
+  ocnn_build_params bp;
+  std::memset(&bp, 0, sizeof(bp));
+  bp.depth = depth;
+  bp.full_depth = full_depth;
+  bp.node_dis = node_dis;
+  bp.node_feature = node_feature;
+  bp.split_label = split_label;
+  bp.adaptive = adaptive;
+  bp.adp_depth = adp_depth;
+  bp.th_normal = th_normal;
+  bp.th_distance = th_distance;
+  bp.extrapolate = extrapolate;
+  bp.save_pts = save_pts;
+  bp.key2xyz = key2xyz;
+  const size_t wb = ocnn_points2octree_workspace_bytes(h.pt_num(), 1, std::max(depth, std::max(full_depth, 1)));
+  TORCH_CHECK(wb > 0, "bad build arguments (points ", h.pt_num(), ", depth ", depth, ")");
+  Aligned ws(points, wb);
+  TensorPool pool{points.options(), {}};
+  const void* dev[1] = {points.data_ptr()};
+  const void* hdr[1] = {h.bytes};
+  unsigned char info[OCNN_HEADER_BYTES] = {0};
+  void* out_ptr = nullptr;
+  check(ocnn_points2octree(dev, hdr, 1, &bp, ws.p, wb, &TensorPool::alloc, &pool, info, &out_ptr, current_stream()));
+  Tensor out = pool.take(out_ptr);
+  headers().put(out, info);
+  return out;
+}
+
+// ---- pytorch/cpp/octree_batch.cpp:5-22 ------------------------------------------------------------------------------
+Tensor octree_batch(vector<Tensor> tensors_in) {
+  const int n = (int)tensors_in.size();
+  TORCH_CHECK(n > 0, "octree_batch of nothing");
+  vector<Tensor> octs;
+  vector<Info> infos;
+  vector<const void*> info_ptrs, dev_ptrs;
+  octs.reserve(n);
+  infos.reserve(n);
+  for (const Tensor& t : tensors_in) {
+    octs.push_back(on_device(t));
+    infos.emplace_back(octs.back());
+  }
+  for (int i = 0; i < n; ++i) {
+    info_ptrs.push_back(infos[i].p());
+    dev_ptrs.push_back(octs[i].data_ptr());
+  }
+  unsigned char hdr[OCNN_HEADER_BYTES] = {0};
+  check(ocnn_octree_batch_info(info_ptrs.data(), n, hdr));
+  Tensor out = torch::empty({ocnn_info_sizeof_octree(hdr)}, octs[0].options());
+  const size_t wb = ocnn_octree_batch_workspace_bytes(n, ocnn_info_depth(hdr));
+  Tensor ws = bytes_on(out, wb);
+  check(ocnn_octree_batch(out.data_ptr(), hdr, dev_ptrs.data(), info_ptrs.data(), n, ws.data_ptr(), wb,
+      current_stream()));
+  headers().put(out, hdr);
+  return out;
+}
+
+// ---- pytorch/cpp/octree_samples.cpp:5-18: `octree_1` .. `octree_6` as CPU uint8 tensors, from the package's data
+// file (data/octree_samples.npz beside this module's folder; numpy reads it) ---------------------------------------
+int64_t octree_header_copies();
+vector<Tensor> octree_samples(vector<string> names) {
+  namespace py = pybind11;
+  Dl_info self;   // where this shared object was loaded from
+  TORCH_CHECK(dladdr(reinterpret_cast<const void*>(&octree_header_copies), &self) != 0 && self.dli_fname,
+      "cannot locate the module's file");
+  string path(self.dli_fname);
+  const size_t slash = path.rfind('/');
+  path = (slash == string::npos ? string(".") : path.substr(0, slash)) + "/../data/octree_samples.npz";
+  py::object z = py::module_::import("numpy").attr("load")(path);
+  py::object from_numpy = py::module_::import("torch").attr("from_numpy");
+  vector<Tensor> out;
+  for (const string& name : names) {
+    TORCH_CHECK(z.attr("files").attr("__contains__")(name).cast<bool>(), "The specified octree does not exist : ", name);
+    out.push_back(from_numpy(z.attr("__getitem__")(name).attr("copy")()).cast<Tensor>());
+  }
+  return out;
+}
+
+// ---- pytorch/cpp/octree_property.cpp:308-325: a copy with the features of one depth replaced -------------------------
+Tensor octree_set_property(Tensor octree_in, Tensor data_in, int depth) {
+  Info info(octree_in);
+  const int64_t count = (int64_t)info.nnum(depth) * ocnn_info_channel(info.p(), OCNN_FEATURE);
+  TORCH_CHECK(data_in.numel() == count, "Wrong Property Size");
+  const int64_t off = ocnn_info_ptr_dis(info.p(), OCNN_FEATURE, depth);
+  TORCH_CHECK(off >= 0, "The octree has no feature: d = ", depth);
+  Tensor out = octree_in.clone();
+  torch::from_blob(static_cast<unsigned char*>(out.data_ptr()) + off, {count}, out.options().dtype(torch::kFloat32))
+      .copy_(data_in.to(torch::kFloat32).reshape({-1}));
+  headers().put(out, info.bytes);
+  return out;
+}
+
+// ---- pytorch/cpp/octree_key.cpp:11-47: int16 [N, 4] (x, y, z, id) <-> int64 [N], a copy of the bits -------------------
+Tensor octree_encode_key(Tensor xyz) {
+  TORCH_CHECK(xyz.dim() == 2 && xyz.size(1) == 4, "The input must be [N, 4]");
+  return xyz.to(torch::kInt16).contiguous().view(torch::kInt64).reshape({-1}).clone();
+}
+
+Tensor octree_decode_key(Tensor key) {
+  TORCH_CHECK(key.dim() == 1 && key.scalar_type() == torch::kInt64, "The dim of input tensor must be 1.");
+  return key.contiguous().view(torch::kInt16).reshape({-1, 4}).clone();
+}
+
+// ---- pytorch/cpp/transform_octree.cpp:5-22 ------------------------------------------------------------------------------
+Tensor octree_scan(Tensor octree_in, vector<float> axis, float scale) {
+  Tensor octree = on_device(octree_in);
+  Info info(octree);
+  TORCH_CHECK(!axis.empty() && axis.size() % 3 == 0, "axis needs 3 floats per direction");
+  TensorPool pool{octree.options(), {}};
+  unsigned char hdr[OCNN_HEADER_BYTES] = {0};
+  void* out_ptr = nullptr;
+  check(ocnn_octree_scan(octree.data_ptr(), info.p(), axis.data(), (int)axis.size() / 3, scale, &TensorPool::alloc, &pool,
+      hdr, &out_ptr, current_stream()));
+  Tensor out = pool.take(out_ptr);
+  headers().put(out, hdr);
+  return out;
+}
+
+// ---- pytorch/cpp/octree_align.cpp:9-83 -------------------------------------------------------------------------------------
+namespace {
+// sorted Morton keys of a depth (converted from packed xyz where the octree stores those)
+Tensor morton_keys(const Tensor& octree, const Info& info, int depth) {
+  const int h = info.nnum(depth);
+  Tensor key = torch::from_blob(const_cast<int64_t*>(info.prop<int64_t>(octree, OCNN_KEY, depth)), {h},
+      octree.options().dtype(torch::kInt64));
+  if (ocnn_info_is_key2xyz(info.p()) && h > 0) key = key_op(key, depth, true);
+  return key;
+}
+}  // namespace
+
+vector<Tensor> octree_align(Tensor src_data, Tensor src_octree, Tensor des_octree, int depth) {
+  src_data = src_data.contiguous();
+  TORCH_CHECK(src_data.scalar_type() == torch::kFloat32, "octree_align is fp32");
+  Info sinfo(src_octree), dinfo(des_octree);
+  const int channel = (int)src_data.size(1), src_h = (int)src_data.size(2), des_h = dinfo.nnum(depth);
+  TORCH_CHECK(sinfo.nnum(depth) == src_h, "octree_align: ", src_h, " rows, the source octree has ", sinfo.nnum(depth),
+      " nodes at depth ", depth);
+  Tensor src_key = morton_keys(src_octree, sinfo, depth), des_key = morton_keys(des_octree, dinfo, depth);
+  Tensor idx = torch::empty({src_h}, src_data.options().dtype(torch::kInt32));
+  // the queries are sorted themselves: the plain search walks the same cache lines lane by lane
+  check(ocnn_search_key(idx.data_ptr<int>(), reinterpret_cast<const uint64_t*>(des_key.data_ptr<int64_t>()), des_h,
+      reinterpret_cast<const uint64_t*>(src_key.data_ptr<int64_t>()), src_h, current_stream()));
+  Tensor out = torch::empty({1, channel, des_h, 1}, src_data.options());
+  Tensor inverse = torch::empty({std::max(des_h, 1)}, idx.options());
+  check(ocnn_align_forward_ws(out.data_ptr<float>(), des_h, channel, src_data.data_ptr<float>(), src_h,
+      idx.data_ptr<int>(), inverse.data_ptr<int>(), current_stream()));
+  return {out, idx};
+}
+
+Tensor octree_align_grad(Tensor des_grad, Tensor idx_tensor) {
+  des_grad = des_grad.contiguous();
+  idx_tensor = idx_tensor.contiguous();
+  TORCH_CHECK(des_grad.scalar_type() == torch::kFloat32 && idx_tensor.scalar_type() == torch::kInt32,
+      "octree_align_grad: fp32 gradients, int32 indices");
+  const int channel = (int)des_grad.size(1), des_h = (int)des_grad.size(2), src_h = (int)idx_tensor.numel();
+  Tensor out = torch::empty({1, channel, src_h, 1}, des_grad.options());
+  check(ocnn_align_backward(des_grad.data_ptr<float>(), des_h, channel, out.data_ptr<float>(), src_h,
+      idx_tensor.data_ptr<int>(), current_stream()));
+  return out;
+}
+
 // Test hooks for the header copies: the bytes this file would use for `octree`, and how many
 // copies are alive (entries of dead tensors are dropped first).
 Tensor octree_header(Tensor octree) {
@@ -566,10 +923,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("octree_mask_pool", &octree_mask_pool, "pooling through a given mask");
   m.def("octree_xyz2key", &octree_xyz2key, "packed xyz -> Morton key");
   m.def("octree_key2xyz", &octree_key2xyz, "Morton key -> packed xyz");
-  m.def("octree_search_key", &octree_search_key, "index of keys in an octree level");
-  m.def("octree_new", &octree_new, "an octree with the root level only");
-  m.def("octree_grow", &octree_grow, "add one level");
-  m.def("octree_update", &octree_update, "children of a level from split labels");
+  m.def("octree_search_key", &octree_search_key, "index of keys in an octree level", py::arg("key"), py::arg("octree"),
+      py::arg("depth"), py::arg("key_is_xyz") = true, py::arg("nempty") = false);
+  m.def("octree_new", &octree_new, "an octree with the root level only", py::arg("batch_size") = 1, py::arg("channel") = 4,
+      py::arg("node_dis") = true, py::arg("adaptive_layer") = 0);
+  m.def("octree_grow", &octree_grow, "add one level", py::arg("octree"), py::arg("target_depth"),
+      py::arg("full_octree") = false);
+  m.def("octree_update", &octree_update, "children of a level from split labels", py::arg("octree"), py::arg("label"),
+      py::arg("depth"), py::arg("split") = 1);
   m.def("octree_update_", &octree_update_, "octree_update on the blob itself");
   m.def("octree_property", &octree_property, "a property of an octree", py::arg("octree"), py::arg("property"),
       py::arg("depth") = 0);
@@ -577,6 +938,26 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("rows_from_channels", &rows_from_channels, "[1, C, H, 1] bf16 -> rows [H + 1, pitch]");
   m.def("channels_from_rows", &channels_from_rows, "rows [H + 1, pitch] -> [1, C, H, 1]");
   m.def("octree_conv_rows", &octree_conv_rows, "convolution on row-major bf16 activations");
+  m.def("octree_batch", &octree_batch, "merge a batch of octrees");
+  m.def("octree_samples", &octree_samples, "the sample octrees of the package");
+  m.def("points2octree", &points2octree, "one octree from one point cloud");
+  m.def("octree_set_property", &octree_set_property, "a copy with the features of one depth replaced", py::arg("octree"),
+      py::arg("data"), py::arg("depth"));
+  m.def("transform_points", &transform_points, "rotate, scale, jitter a point cloud");
+  m.def("clip_points", &clip_points, "keep the points inside a box");
+  m.def("normalize_points", &normalize_points, "move to a centre and scale by 1 / radius");
+  m.def("bounding_sphere", &bounding_sphere, "radius and centre of a bounding sphere");
+  m.def("octree_encode_key", &octree_encode_key, "int16 (x, y, z, id) -> int64 key");
+  m.def("octree_decode_key", &octree_decode_key, "int64 key -> int16 (x, y, z, id)");
+  m.def("octree_scan", &octree_scan, "the part of an octree seen from given directions", py::arg("octree"),
+      py::arg("axis"), py::arg("scale") = 1.0f);
+  m.def("octree_align", &octree_align, "features moved to the nodes of another octree", py::arg("src_data"),
+      py::arg("src_octree"), py::arg("des_octree"), py::arg("depth"));
+  m.def("octree_align_grad", &octree_align_grad, "backward of octree_align");
+  m.def("points_batch_property", &points_batch_property, "a property of several point clouds, stacked");
+  m.def("points_property", &points_property, "a property of a point cloud");
+  m.def("points_set_property", &points_set_property, "a copy of a point cloud with one property replaced");
+  m.def("points_new", &points_new, "a serialized point cloud from its arrays");
   m.def("octree_header", &octree_header, "the host copy of an octree's header (test hook)");
   m.def("octree_header_copies", &octree_header_copies, "live header copies (test hook)");
 }

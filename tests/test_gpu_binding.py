@@ -185,3 +185,122 @@ def test_header_copy_follows_the_tensor_on_the_device(oc, orc, aten, tree, sampl
   b_full.copy_(T(host_a))
   assert np.array_equal(aten.octree_header(b_full).numpy(), host_a[:716])
   conv_on(b_full, ia, 4)
+
+
+def cloud(synthetic, n, seed, features=False, labels=False):
+  pts, nrm = synthetic.shape_cloud(n, seed)[:2]
+  rng = np.random.default_rng(seed)
+  feat = rng.standard_normal((pts.shape[0], 2)).astype(np.float32) if features else None
+  lab = rng.integers(0, 5, (pts.shape[0], 1)).astype(np.float32) if labels else None
+  return pts, nrm, feat, lab
+
+
+def test_points_ops_equal_the_mirror(oc, aten, synthetic):
+  pts, nrm, feat, lab = cloud(synthetic, 3000, 61, features=True, labels=True)
+  args = [T(a).cuda() for a in (pts, nrm, feat, lab)]
+  p = aten.points_new(*args)
+  assert same(p, oc.nn.points_new(*args))
+  assert np.array_equal(p.cpu().numpy(), make_points_blob(pts, nrm, feat, lab))
+  # without the optional arrays: empty tensors, as the reference's Python side passes them
+  none = torch.zeros(0)
+  p2 = aten.points_new(args[0], args[1], none, none)
+  assert np.array_equal(p2.cpu().numpy(), make_points_blob(pts, nrm))
+  for name in ("xyz", "normal", "feature", "label"):
+    assert same(aten.points_property(p, name), oc.nn.points_property(p, name)), name
+  assert aten.points_property(p2, "feature") is None and aten.points_property(p2, "label") is None
+  for name in ("xyz", "xyzi", "normal"):
+    assert same(aten.points_batch_property([p, p2, p], name), oc.nn.points_batch_property([p, p2, p], name)), name
+  with pytest.raises(RuntimeError):
+    aten.points_batch_property([p, p2], "feature")
+  new_nrm = torch.randn(pts.shape[0], 3, device="cuda")
+  assert same(aten.points_set_property(p, new_nrm, "normal"), oc.nn.points_set_property(p, new_nrm, "normal"))
+  with pytest.raises(RuntimeError):
+    aten.points_set_property(p2, torch.zeros(pts.shape[0], 2, device="cuda"), "feature")
+  with pytest.raises(RuntimeError):
+    aten.points_set_property(p, torch.zeros(pts.shape[0] - 1, 3, device="cuda"), "normal")
+  # transforms: device clouds and host clouds (the reference keeps clouds on the host) give the same bytes
+  for src in (p, p.cpu()):
+    for method in ("sphere", "box"):
+      assert aten.bounding_sphere(src, method) == oc.nn.bounding_sphere(p, method)
+    r, c = 0.8, [0.1, -0.05, 0.02]
+    assert same(aten.normalize_points(src, r, c), oc.nn.normalize_points(p, r, c))
+    for axis in ("", "y", "xyz"):
+      tr = ([0.3, -0.2, 1.1], [1.1, 0.9, 1.0], [0.05, 0.0, -0.02], 0.01, axis)
+      assert same(aten.transform_points(src, *tr), oc.nn.transform_points(p, *tr)), axis
+    assert same(aten.transform_points(src, [0.5], [0.9], [0.0], 0.0, ""), oc.nn.transform_points(p, [0.5], [0.9], [0.0], 0.0, ""))
+    got, exp = aten.clip_points(src, [-0.5, -0.4, -0.6], [0.5, 0.6, 0.3]), oc.nn.clip_points(p, [-0.5, -0.4, -0.6], [0.5, 0.6, 0.3])
+    assert same(got[0], exp[0]) and same(got[1], exp[1]) and 0 < int(got[1].sum()) < pts.shape[0]
+  with pytest.raises(RuntimeError):
+    aten.points_property(torch.zeros(200, dtype=torch.uint8), "xyz")   # no magic string
+
+
+@pytest.mark.parametrize("opts", [
+    dict(depth=6, full_depth=2),
+    dict(depth=5, full_depth=3, node_dis=True, split_label=True, save_pts=True),
+    dict(depth=6, full_depth=2, key2xyz=True),
+    dict(depth=6, full_depth=2, node_dis=True, node_feature=True),
+    dict(depth=6, full_depth=2, node_dis=True, adaptive=True, adp_depth=3, th_normal=0.2, th_distance=1.5),
+    dict(depth=6, full_depth=2, node_dis=True, adaptive=True, adp_depth=3, extrapolate=True),
+], ids=["plain", "dis_split_pts", "key2xyz", "node_feature", "adaptive", "adaptive_extrapolate"])
+def test_build_and_batch_equal_the_mirror(oc, aten, synthetic, opts):
+  order = ("depth", "full_depth", "node_dis", "node_feature", "split_label", "adaptive", "adp_depth", "th_normal",
+           "th_distance", "extrapolate", "save_pts", "key2xyz")
+  full = dict(full_depth=2, node_dis=False, node_feature=False, split_label=False, adaptive=False, adp_depth=4,
+              th_normal=0.1, th_distance=2.0, extrapolate=False, save_pts=False, key2xyz=False)
+  full.update(opts)
+  clouds = [T(make_points_blob(*cloud(synthetic, 2500 + 300 * i, 70 + i)[:2])) for i in range(3)]
+  got, exp = [], []
+  for i, c in enumerate(clouds):
+    src = c.cuda() if i != 1 else c                     # one cloud comes from the host
+    got.append(aten.points2octree(src, *[full[k] for k in order]))
+    exp.append(oc.nn.points2octree(c.cuda(), **full))
+    assert same(got[-1], exp[-1]), i
+    assert np.array_equal(aten.octree_header(got[-1]).numpy(), exp[-1][:716].cpu().numpy())
+  merged, merged_exp = aten.octree_batch(got), oc.nn.octree_batch(exp)
+  assert same(merged, merged_exp)
+  assert np.array_equal(aten.octree_header(merged).numpy(), merged_exp[:716].cpu().numpy())
+  assert same(aten.octree_batch([g.cpu() for g in got]), merged_exp)   # host blobs, as a data loader hands them over
+  d = full["depth"]
+  assert same(aten.octree_property(merged, "feature", d), oc.nn.octree_property(merged_exp, "feature", d))
+  with pytest.raises(RuntimeError):
+    aten.points2octree(clouds[0].cuda(), 0, 2, False, False, False, False, 4, 0.1, 2.0, False, False, False)
+
+
+def test_samples_set_property_keys_scan_align_equal_the_mirror(oc, aten, samples, tree, synthetic):
+  names = ["octree_%d" % i for i in range(1, 7)]
+  for a, r, n in zip(aten.octree_samples(names), oc.nn.octree_samples(names), names):
+    assert same(a, r) and np.array_equal(a.numpy(), samples[n]), n
+  with pytest.raises(RuntimeError):
+    aten.octree_samples(["octree_7"])
+  dev, b = tree["dev"], tree["blob"]
+  d = 6
+  feat = oc.nn.octree_property(dev, "feature", d)
+  new = torch.randn_like(feat)
+  got = aten.octree_set_property(dev, new, d)
+  assert same(got, oc.nn.octree_set_property(dev, new, d))
+  assert same(aten.octree_property(got, "feature", d), new) and same(aten.octree_property(dev, "feature", d), feat)
+  with pytest.raises(RuntimeError):
+    aten.octree_set_property(dev, new[:, :, :-1], d)
+  xyz = torch.randint(0, 64, (500, 4), dtype=torch.int16, device="cuda")
+  key = aten.octree_encode_key(xyz)
+  assert same(key, oc.nn.octree_encode_key(xyz)) and same(aten.octree_decode_key(key), xyz)
+  with pytest.raises(RuntimeError):
+    aten.octree_encode_key(xyz[:, :3])
+  # scan: one octree, two view directions; then features of the scanned octree on the nodes of the whole one
+  single = aten.points2octree(T(make_points_blob(*cloud(synthetic, 6000, 81)[:2])).cuda(), 6, 2, True, False, False, False,
+                              4, 0.1, 2.0, False, False, False)
+  axis = [0.0, 0.0, 1.0, 0.6, 0.0, 0.8]
+  part = aten.octree_scan(single, axis, 1.0)
+  assert same(part, oc.nn.octree_scan(single, axis, 1.0)) and same(aten.octree_scan(single, axis[:3]), oc.nn.octree_scan(single, axis[:3]))
+  assert np.array_equal(aten.octree_header(part).numpy(), part[:716].cpu().numpy())
+  whole, part_b = aten.octree_batch([single]), aten.octree_batch([part])
+  for dep in (4, 6):
+    h = int(aten.octree_property(part_b, "node_num", dep)[0])
+    assert 0 < h < int(aten.octree_property(whole, "node_num", dep)[0]) or dep == 4
+    x = torch.randn(1, 5, h, 1, device="cuda")
+    (ga, gi), (ea, ei) = aten.octree_align(x, part_b, whole, dep), oc.nn.octree_align(x, part_b, whole, dep)
+    assert same(ga, ea) and same(gi, ei) and int((gi >= 0).sum()) == h
+    grad = torch.randn_like(ga)
+    assert same(aten.octree_align_grad(grad, gi), oc.nn.octree_align_grad(grad, gi))
+  with pytest.raises(RuntimeError):
+    aten.octree_align(torch.randn(1, 5, 7, 1, device="cuda"), part_b, whole, 6)
