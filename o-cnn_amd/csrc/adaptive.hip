@@ -1347,15 +1347,27 @@ int adaptive_finish(const AdaptiveInput& in, ocnn_alloc_fn alloc, void* alloc_ct
     // none and stays zero as in the reference's zero-initialised buffer
     fill_kernel<<<blocks_for((int64_t)o.nnum[0] * 8), kBlock, 0, s>>>(
         reinterpret_cast<float*>(out + o.ptr_dis(OCNN_NEIGH, 0)), (int64_t)o.nnum[0] * 8, 0.0f);
-    for (int d = 1; d <= D; ++d) {
+    for (int d = 1; d <= D;) {
       int* neigh = reinterpret_cast<int*>(out + o.ptr_dis(OCNN_NEIGH, d));
       if (d <= fl) {
         const int e = ocnn_calc_neigh_full(neigh, d, B, s);
         if (e) return e;
-      } else if (o.nnum[d - 1] > 0) {
-        launch_neigh_sparse(neigh, reinterpret_cast<const int*>(out + o.ptr_dis(OCNN_NEIGH, d - 1)),
-            reinterpret_cast<const int*>(out + o.ptr_dis(OCNN_CHILD, d - 1)), o.nnum[d - 1], s, o.nnum[d] / 8);
+        ++d;
+        continue;
       }
+      if (o.nnum[d - 1] <= 0) { ++d; continue; }
+      // the last levels in one launch (small levels: the chain of launches is what they cost)
+      int count = 1;
+      if (D - d < kNeighLevels && o.nnum[D] <= (1 << 21)) while (d + count <= D && o.nnum[d + count - 1] > 0) ++count;
+      int* tables[kNeighLevels] = {nullptr, nullptr, nullptr};
+      const int* links[kNeighLevels] = {nullptr, nullptr, nullptr};
+      for (int i = 0; i < count; ++i) {
+        tables[i] = reinterpret_cast<int*>(out + o.ptr_dis(OCNN_NEIGH, d + i));
+        links[i] = reinterpret_cast<const int*>(out + o.ptr_dis(OCNN_CHILD, d + i - 1));
+      }
+      launch_neigh_sparse_levels(count, tables, reinterpret_cast<const int*>(out + o.ptr_dis(OCNN_NEIGH, d - 1)), links,
+          o.nnum[d - 1], s);
+      d += count;
     }
     OCNN_LAUNCH_OK("neighbours");
   }

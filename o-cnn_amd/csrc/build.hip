@@ -1426,13 +1426,27 @@ int ocnn_points2octree_emit(void* octree_out_dev, const void* info, void* worksp
       fill_f32_kernel<<<blocks_for(HD, kBlock * 4), kBlock, 0, s>>>(reinterpret_cast<float*>(blob + a.off_label), HD, -1.0f);
     OCNN_LAUNCH_OK("fill");
   }
-  if (o.has(OCNN_NEIGH)) {  // merge_octrees.cpp:185-197: sparse levels, each from the level above
-    for (int d = searched_to + 1; d <= depth; ++d) {
-      if (o.nnum[d - 1] <= 0) continue;
-      launch_neigh_sparse(reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_NEIGH, d)),
-          reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_NEIGH, d - 1)),
-          reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_CHILD, d - 1)), o.nnum[d - 1], s);
+  if (o.has(OCNN_NEIGH)) {
+    // merge_octrees.cpp:185-197: the remaining sparse levels, each from the level above; the last
+    // (and largest) two or three in one launch while the tables are bound by the chain of dependent
+    // trips to memory rather than by their bytes (measured on depth-9 scenes of 250 k points, levels
+    // fused 1 / 2 / 3: one scene 0.121 / 0.113 / 0.112 ms, four 0.310 / 0.290 / 0.295, eight 0.575 /
+    // 0.579 / 0.608)
+    const int fuse = o.nnum[depth] <= (1 << 21) ? 3 : (o.nnum[depth] <= (1 << 23) ? 2 : 1);
+    for (int d = searched_to + 1; d <= depth;) {
+      if (o.nnum[d - 1] <= 0) { ++d; continue; }
+      int count = 1;
+      if (depth - d < fuse) while (d + count <= depth && o.nnum[d + count - 1] > 0) ++count;
+      int* out[kNeighLevels] = {nullptr, nullptr, nullptr};
+      const int* children[kNeighLevels] = {nullptr, nullptr, nullptr};
+      for (int i = 0; i < count; ++i) {
+        out[i] = reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_NEIGH, d + i));
+        children[i] = reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_CHILD, d + i - 1));
+      }
+      launch_neigh_sparse_levels(count, out, reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_NEIGH, d - 1)), children,
+          o.nnum[d - 1], s);
       OCNN_LAUNCH_OK("neigh");
+      d += count;
     }
   }
   return OCNN_OK;

@@ -68,24 +68,27 @@ struct NeighLane {
 // links while the current batch is gathered and written.  GROUPS = 8 keeps enough bytes in
 // flight per wavefront for a large level (the kernel is bound by that, not by bandwidth);
 // GROUPS = 2 gives a small level more wavefronts and each a shorter chain.
+// members (bit s = sibling s) whose 3x3x3 window of the group's 4x4x4 block contains this lane's slot
+__device__ inline int neigh_wanted_by(int lane) {
+  int wants = 0;
+  const int x = lane >> 4, y = (lane >> 2) & 3, z = lane & 3;
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    const int dx = x - (s >> 2), dy = y - ((s >> 1) & 1), dz = z - (s & 1);
+    if (dx >= 0 && dx <= 2 && dy >= 0 && dy <= 2 && dz >= 0 && dz <= 2) wants |= 1 << s;
+  }
+  return wants;
+}
+
+// the work of wavefront `wave` out of `stride` wavefronts
 template <int GROUPS>
-__global__ __launch_bounds__(kBlock) void neigh_sparse_kernel(int* __restrict__ neigh_child,
-    const int* __restrict__ neigh, const int* __restrict__ children, int node_num, int iters, int child_groups) {
+__device__ inline void neigh_sparse_wave(int* __restrict__ neigh_child, const int* __restrict__ neigh,
+    const int* __restrict__ children, int node_num, int iters, int child_groups, int wave, int stride) {
   const int lane = threadIdx.x & 63;
-  const int wave = (int)((blockIdx.x * (unsigned)kBlock + threadIdx.x) >> 6);
   const int groups = (node_num + 7) >> 3;
   const int64_t slots = (int64_t)node_num * 8;
   const NeighLane nl(lane);
-  // members (bit s = sibling s) whose 3x3x3 window of the block contains this lane's slot
-  int wants = 0;
-  {
-    const int x = lane >> 4, y = (lane >> 2) & 3, z = lane & 3;
-#pragma unroll
-    for (int s = 0; s < 8; ++s) {
-      const int dx = x - (s >> 2), dy = y - ((s >> 1) & 1), dz = z - (s & 1);
-      if (dx >= 0 && dx <= 2 && dy >= 0 && dy <= 2 && dz >= 0 && dz <= 2) wants |= 1 << s;
-    }
-  }
+  const int wants = neigh_wanted_by(lane);
   int rank8[GROUPS], slot[GROUPS];
   auto request = [&](int batch, int* r8, int* sl) {
 #pragma unroll
@@ -98,7 +101,6 @@ __global__ __launch_bounds__(kBlock) void neigh_sparse_kernel(int* __restrict__ 
   };
   // batch it of wavefront w is w + it * (number of wavefronts): at any moment the wavefronts of
   // the device work on one contiguous window of the level
-  const int stride = (int)(gridDim.x * (unsigned)(kBlock / 64));
   request(wave, rank8, slot);
   for (int it = 0; it < iters; ++it) {
     if ((int64_t)(wave + (int64_t)it * stride) * GROUPS >= groups) break;
@@ -115,15 +117,102 @@ __global__ __launch_bounds__(kBlock) void neigh_sparse_kernel(int* __restrict__ 
     for (int u = 0; u < GROUPS; ++u) {
       for (int s = 0; s < 8; ++s) {
         if (!((occ[u] >> s) & 1)) continue;   // uniform over the wavefront
-        const int rank = __shfl(rank8[u], s, 64);
+        const int rank = __builtin_amdgcn_readlane(rank8[u], s);   // a scalar: the row's address is base + lane
         const int v = __shfl(link[u], nl.parent_slot(s), 64);
         if (rank >= child_groups) continue;   // a link past the child level (malformed input): no row to write
-        neigh_child[((int64_t)rank << 6) + lane] = v >= 0 ? (v << 3) + nl.octant : -1;
+        (neigh_child + ((int64_t)rank << 6))[lane] = v >= 0 ? (v << 3) + nl.octant : -1;
       }
     }
 #pragma unroll
     for (int u = 0; u < GROUPS; ++u) { rank8[u] = next_rank8[u]; slot[u] = next_slot[u]; }
   }
+}
+template <int GROUPS>
+__global__ __launch_bounds__(kBlock) void neigh_sparse_kernel(int* __restrict__ neigh_child,
+    const int* __restrict__ neigh, const int* __restrict__ children, int node_num, int iters, int child_groups) {
+  neigh_sparse_wave<GROUPS>(neigh_child, neigh, children, node_num, iters, child_groups,
+      (int)((blockIdx.x * (unsigned)kBlock + threadIdx.x) >> 6), (int)(gridDim.x * (unsigned)(kBlock / 64)));
+}
+
+// Two levels from one sibling group whose 4x4x4 block is in registers (`slot`: this lane's entry,
+// `rank8`: the child link of member `lane`, lanes 0 .. 7): the rows of the non-empty members'
+// children (level + 1, as above) and, from those rows while they are still in registers, the rows
+// of the grandchildren (level + 2): the larger level does not wait for a launch of the smaller
+// one, and the smaller one's rows are not read back.  `children` / `children_c`: the child links
+// of the level and of level + 1 (consistent: every link is a sibling group of the next level).
+// The loads of the eight members are requested together (an empty member reads index 0), so this
+// is three dependent trips to memory.
+__device__ inline void neigh_sparse2_rows(int* __restrict__ neigh_c, int* __restrict__ neigh_cc, int slot, int rank8,
+    const int* __restrict__ children, const int* __restrict__ children_c) {
+  const int lane = threadIdx.x & 63;
+  const NeighLane nl(lane);
+  const int wants = neigh_wanted_by(lane);
+  const int from0 = nl.parent_slot(0);   // parent_slot(s) = from0 + the offsets of s (no carries: hx + 1 <= 3)
+  const int occ = (int)(__ballot(lane < 8 && rank8 >= 0) & 0xff);
+  if (occ == 0) return;
+  const int t = (wants & occ) ? slot : -1;
+  const int link = t >= 0 ? children[t] : -1;
+  // (ranks are the same for every lane: read through readlane they stay in scalar registers and
+  // the row addresses are scalar base + lane)
+  int row[8], rank8_c[8];
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    const bool live = (occ >> s) & 1;
+    const int rank = live ? __builtin_amdgcn_readlane(rank8, s) : 0;
+    const int v = __shfl(link, from0 + ((s >> 2) << 4) + (((s >> 1) & 1) << 2) + (s & 1), 64);
+    row[s] = live && v >= 0 ? (v << 3) + nl.octant : -1;
+    rank8_c[s] = (children_c + rank * 8)[lane & 7];   // (every lane: lanes 8 .. 63 read the same line)
+  }
+  int link_c[8], occ_c[8];
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    const bool live = (occ >> s) & 1;
+    occ_c[s] = live ? (int)(__ballot(lane < 8 && rank8_c[s] >= 0) & 0xff) : 0;
+    const int tc = (wants & occ_c[s]) ? row[s] : -1;
+    link_c[s] = children_c[max(tc, 0)];
+    if (tc < 0) link_c[s] = -1;
+  }
+#pragma unroll
+  for (int s = 0; s < 8; ++s)
+    if ((occ >> s) & 1) (neigh_c + ((int64_t)__builtin_amdgcn_readlane(rank8, s) << 6))[lane] = row[s];
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    for (int m = occ_c[s]; m != 0; m &= m - 1) {   // uniform over the wavefront
+      const int u = __builtin_ctz(m);
+      const int r = __builtin_amdgcn_readlane(rank8_c[s], u);
+      const int v = __shfl(link_c[s], from0 + ((u >> 2) << 4) + (((u >> 1) & 1) << 2) + (u & 1), 64);
+      (neigh_cc + ((int64_t)r << 6))[lane] = v >= 0 ? (v << 3) + nl.octant : -1;
+    }
+  }
+}
+// levels + 1 and + 2 from sibling group `g` of a level whose table `neigh` exists
+__device__ inline void neigh_sparse2_wave(int* __restrict__ neigh_c, int* __restrict__ neigh_cc,
+    const int* __restrict__ neigh, const int* __restrict__ children, const int* __restrict__ children_c,
+    int node_num, int g) {
+  const int lane = threadIdx.x & 63;
+  if (g * 8 >= node_num) return;
+  const int node = g * 8 + lane;
+  const int rank8 = (lane < 8 && node < node_num) ? children[node] : -1;
+  const int slot = ((int64_t)g << 6) + lane < (int64_t)node_num * 8 ? neigh[((int64_t)g << 6) + lane] : -1;
+  neigh_sparse2_rows(neigh_c, neigh_cc, slot, rank8, children, children_c);
+}
+// levels + 1, + 2 and + 3 from node `node` of a level whose table `neigh` exists: the node's own
+// row of level + 1 (every member of a group reads the group's block again), then the two levels
+// below from that row
+__device__ inline void neigh_sparse3_wave(int* __restrict__ neigh_c, int* __restrict__ neigh_cc,
+    int* __restrict__ neigh_ccc, const int* __restrict__ neigh, const int* __restrict__ children,
+    const int* __restrict__ children_c, const int* __restrict__ children_cc, int node_num, int node) {
+  const int lane = threadIdx.x & 63;
+  if (node >= node_num) return;
+  const int rank = children[node];
+  if (rank < 0) return;   // uniform over the wavefront
+  const NeighLane nl(lane);
+  const int s = node & 7;
+  const int slot = neigh[((int64_t)(node >> 3) << 6) + nl.parent_slot(s)];   // the entry this lane's value comes from
+  const int v = slot >= 0 ? children[slot] : -1;
+  const int row = v >= 0 ? (v << 3) + nl.octant : -1;
+  neigh_c[((int64_t)rank << 6) + lane] = row;
+  neigh_sparse2_rows(neigh_cc, neigh_ccc, row, children_c[rank * 8 + (lane & 7)], children_c, children_cc);
 }
 // `child_groups`: sibling groups of the level written, where the caller knows it (a header);
 // links at or past it are skipped instead of followed.
@@ -141,6 +230,35 @@ inline void launch_neigh_sparse(int* neigh_child, const int* neigh, const int* c
     neigh_sparse_kernel<2><<<blocks_for((groups + 1) / 2, kBlock / 64), kBlock, 0, s>>>(neigh_child, neigh, children,
         node_num, 1, child_groups);
   }
+}
+
+// The tables of `count` (1 .. kNeighLevels) consecutive sparse levels in one launch, from the level
+// above the first: out[i] is the table of the i-th level written, children[i] the child links of
+// the level above it (consistent links: a fresh octree's own), `neigh` / `node_num` the table and
+// node count of the level above the first.  The same rows as one launch_neigh_sparse per level.
+constexpr int kNeighLevels = 3;
+struct NeighLevels {
+  int* out[kNeighLevels];
+  const int* children[kNeighLevels];
+};
+template <int COUNT>
+__global__ __launch_bounds__(kBlock) void neigh_sparse_levels_kernel(NeighLevels a, const int* __restrict__ neigh, int node_num) {
+  const int wave = (int)((blockIdx.x * (unsigned)kBlock + threadIdx.x) >> 6);
+  if (COUNT == 2) neigh_sparse2_wave(a.out[0], a.out[1], neigh, a.children[0], a.children[1], node_num, wave);
+  else neigh_sparse3_wave(a.out[0], a.out[1], a.out[2], neigh, a.children[0], a.children[1], a.children[2], node_num, wave);
+}
+inline void launch_neigh_sparse_levels(int count, int* const* out, const int* neigh, const int* const* children,
+    int node_num, hipStream_t s) {
+  if (count <= 1) {
+    launch_neigh_sparse(out[0], neigh, children[0], node_num, s);
+    return;
+  }
+  NeighLevels a;
+  for (int i = 0; i < kNeighLevels; ++i) { a.out[i] = i < count ? out[i] : nullptr; a.children[i] = i < count ? children[i] : nullptr; }
+  if (count == 2)
+    neigh_sparse_levels_kernel<2><<<blocks_for(((int64_t)node_num + 7) / 8, kBlock / 64), kBlock, 0, s>>>(a, neigh, node_num);
+  else
+    neigh_sparse_levels_kernel<3><<<blocks_for(node_num, kBlock / 64), kBlock, 0, s>>>(a, neigh, node_num);
 }
 
 // Full layer: closed form through Morton decode / encode (octree_nn.cpp:382-424).
