@@ -116,6 +116,25 @@ inline int pass_split(int n_tiles, int npass) {
   return p < npass ? p : npass;
 }
 
+// Wavefronts per workgroup (64 columns each) of a kernel whose wavefronts share nothing but a table:
+// a level of a few hundred 256-column tiles leaves some compute units with two workgroups and others
+// with one (363 tiles on 256 units: the launch lasts as long as two), and smaller workgroups spread
+// evenly.  The pick is the size whose most loaded unit holds the fewest wavefronts' work; on a tie
+// the larger (neighbouring columns share rows and the weights in the L1).  Measured at depth 7 of
+// the scene (92 723 columns): 256 -> 128 channels 0.248 -> 0.202 ms, 128 -> 128 0.131 -> 0.107 ms.
+inline int direct_waves(int cols, int npass) {
+  constexpr int kUnits = 256;   // compute units of the device
+  int best = kConvWaves;
+  int64_t best_load = INT64_MAX;
+  for (int w = kConvWaves; w >= 1; w >>= 1) {
+    const int tiles = (cols + kWaveCols * w - 1) / (kWaveCols * w);
+    const int split = pass_split(tiles, npass);
+    const int64_t load = (((int64_t)tiles * split + kUnits - 1) / kUnits) * w * ((npass + split - 1) / split);
+    if (load < best_load) { best_load = load; best = w; }
+  }
+  return best;
+}
+
 // ---- main kernels ----------------------------------------------------------------
 // Accumulator layout of the 32x32 MFMA: lane l, register i holds
 // D[row = 8*(i/4) + 4*(l>>5) + (i%4)][col = l&31].
@@ -722,21 +741,22 @@ __global__ __launch_bounds__(256, 2) void conv_rows_bf16_deep_kernel(ConvArgs a,
 // times a slab.  Here a wavefront walks its live taps in ascending order with the next live tap's
 // weights and rows in flight (two register sets), at its own pace.  Same products in the same order
 // as conv_rows_bf16_deep_kernel: the results are bit-identical.
-template <int MT, int SLAB, bool ROWS_OUT, int WPS = 2>
-__global__ __launch_bounds__(256, WPS) void conv_rows_bf16_direct_kernel(ConvArgs a, uint16_t* __restrict__ out,
+template <int MT, int SLAB, bool ROWS_OUT, int WPS = 2, int WAVES = kConvWaves>
+__global__ __launch_bounds__(64 * WAVES, WPS) void conv_rows_bf16_direct_kernel(ConvArgs a, uint16_t* __restrict__ out,
     const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles, int cpad, int in_pitch, int out_pitch, int out_cpad) {
   constexpr int kKs = SLAB / 16;                        // k-steps per slab
   constexpr int kWUnits = kKs * MT * 64;                // 16-byte units of one (tap, slab)
-  __shared__ int sSrc[27][kTileCols];                   // source row of (tap, column), in 16-byte units of the copy
+  constexpr int kCols = kWaveCols * WAVES;              // columns of a workgroup
+  __shared__ int sSrc[27][kCols];                   // source row of (tap, column), in 16-byte units of the copy
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int tile = xcd_tile(blockIdx.x, n_tiles);
   if (tile >= n_tiles) return;
-  const int n0 = tile * kTileCols + wave * kWaveCols;
+  const int n0 = tile * kCols + wave * kWaveCols;
   const int r = lane & 31, kh = lane >> 5;
   const int nslab = (cpad + SLAB - 1) / SLAB;
   const int npass = (a.mtiles + MT - 1) / MT;
   const int cpad8 = in_pitch >> 3;
-  tile_sources(a, tile * kTileCols + (int)threadIdx.x,
+  tile_sources(a, tile * kCols + (int)threadIdx.x,
       [&](int k, int row) { sSrc[k][threadIdx.x] = (row < 0 ? a.Hin : row) * cpad8; });
   const int c0 = wave * kWaveCols + r;
   union Frag { u32x4 q; bf16x8 v; };
@@ -3739,21 +3759,34 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
     const int n_tiles = (a.N + kTileCols - 1) / kTileCols;
     const dim3 grid(((n_tiles + 7) / 8) * 8, pass_split(n_tiles, r.npass));
     const bool direct = a.K >= 3 && g_rows_direct.load() != 0;
+    // the barrier-free kernel in workgroups of four, two or one wavefront (direct_waves)
+    auto launch_direct = [&](auto mt, auto slab, auto wps) {
+      constexpr int MT_ = decltype(mt)::value, SLAB_ = decltype(slab)::value, WPS_ = decltype(wps)::value;
+      const int waves = direct_waves(a.N, r.npass);
+      const int tiles = (a.N + kWaveCols * waves - 1) / (kWaveCols * waves);
+      const dim3 g(((tiles + 7) / 8) * 8, pass_split(tiles, r.npass));
+      if (waves == 4)
+        conv_rows_bf16_direct_kernel<MT_, SLAB_, true, WPS_, 4><<<g, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
+            (const u32x4*)wpk, tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
+      else if (waves == 2)
+        conv_rows_bf16_direct_kernel<MT_, SLAB_, true, WPS_, 2><<<g, 128, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
+            (const u32x4*)wpk, tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
+      else
+        conv_rows_bf16_direct_kernel<MT_, SLAB_, true, WPS_, 1><<<g, 64, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
+            (const u32x4*)wpk, tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
+    };
+    using std::integral_constant;
     if (r.slab_ch == 32 && r.MT == 2 && direct && !r.staged)
-      conv_rows_bf16_direct_kernel<2, 32, true, 3><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
-          (const u32x4*)wpk, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
+      launch_direct(integral_constant<int, 2>(), integral_constant<int, 32>(), integral_constant<int, 3>());
     else if (r.slab_ch == 32 && r.MT == 2)
       conv_rows_bf16_deep_kernel<2, 32, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
           (const u32x4*)wpk, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
     else if (direct && r.MT == 4)
-      conv_rows_bf16_direct_kernel<4, 32, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
-          (const u32x4*)wpk, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
+      launch_direct(integral_constant<int, 4>(), integral_constant<int, 32>(), integral_constant<int, 2>());
     else if (direct && r.MT == 2)
-      conv_rows_bf16_direct_kernel<2, kRowSlab, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
-          (const u32x4*)wpk, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
+      launch_direct(integral_constant<int, 2>(), integral_constant<int, kRowSlab>(), integral_constant<int, 2>());
     else if (direct)
-      conv_rows_bf16_direct_kernel<1, kRowSlab, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
-          (const u32x4*)wpk, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
+      launch_direct(integral_constant<int, 1>(), integral_constant<int, kRowSlab>(), integral_constant<int, 2>());
     else if (r.MT == 4)
       conv_rows_bf16_deep_kernel<4, 32, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
           (const u32x4*)wpk, n_tiles, r.cpad, btm_pitch, top_pitch, r.out_cpad);
