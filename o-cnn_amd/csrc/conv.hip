@@ -2642,19 +2642,33 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     transpose_rows_bf16_kernel<<<tg, 256, 0, s>>>(xt, (const uint16_t*)btm, a.Cin, a.Hin, cpad);
     OCNN_LAUNCH_OK("transpose_rows");
     const dim3 rgrid(grid, pass_split(n_tiles, npass));
-    // (with whole blocks of 128 output channels and a channel-major store the staged kernel is ahead)
-    const bool direct = deep && !wide && g_rows_direct.load() != 0;
+    // (with whole blocks of 128 output channels and a channel-major store the staged kernel is ahead,
+    // unless the level is one that smaller workgroups spread better over the device: direct_waves)
+    const int waves = deep ? direct_waves(a.N, npass) : kConvWaves;
+    const bool direct = deep && (!wide || waves < kConvWaves) && g_rows_direct.load() != 0;
     const bool staged = dense_level && (int64_t)o->nnum_nempty[p.top_depth] * 5 >= (int64_t)o->nnum[p.top_depth] * 2;
+    auto launch_direct = [&](auto mt, auto slab, auto wps) {
+      constexpr int MT_ = decltype(mt)::value, SLAB_ = decltype(slab)::value, WPS_ = decltype(wps)::value;
+      const int tiles = (a.N + kWaveCols * waves - 1) / (kWaveCols * waves);
+      const dim3 g(((tiles + 7) / 8) * 8, pass_split(tiles, npass));
+      if (waves == 4)
+        conv_rows_bf16_direct_kernel<MT_, SLAB_, false, WPS_, 4><<<g, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, tiles, cpad, cpad, 0, 0);
+      else if (waves == 2)
+        conv_rows_bf16_direct_kernel<MT_, SLAB_, false, WPS_, 2><<<g, 128, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, tiles, cpad, cpad, 0, 0);
+      else
+        conv_rows_bf16_direct_kernel<MT_, SLAB_, false, WPS_, 1><<<g, 64, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, tiles, cpad, cpad, 0, 0);
+    };
+    using std::integral_constant;
     if (dense_level && direct && !staged)
-      conv_rows_bf16_direct_kernel<2, 32, false, 3><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad, cpad, 0, 0);
+      launch_direct(integral_constant<int, 2>(), integral_constant<int, 32>(), integral_constant<int, 3>());
     else if (dense_level)
       conv_rows_bf16_deep_kernel<2, 32, false><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad, cpad, 0, 0);
     else if (direct && wide)
-      conv_rows_bf16_direct_kernel<4, 32, false><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad, cpad, 0, 0);
+      launch_direct(integral_constant<int, 4>(), integral_constant<int, 32>(), integral_constant<int, 2>());
     else if (direct && MT == 1)
-      conv_rows_bf16_direct_kernel<1, kRowSlab, false><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad, cpad, 0, 0);
+      launch_direct(integral_constant<int, 1>(), integral_constant<int, kRowSlab>(), integral_constant<int, 2>());
     else if (direct)
-      conv_rows_bf16_direct_kernel<2, kRowSlab, false><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad, cpad, 0, 0);
+      launch_direct(integral_constant<int, 2>(), integral_constant<int, kRowSlab>(), integral_constant<int, 2>());
     else if (wide)
       conv_rows_bf16_deep_kernel<4, 32, false><<<rgrid, 256, 0, s>>>(a, (uint16_t*)top, (const u32x4*)xt, (const u32x4*)wsb, n_tiles, cpad, cpad, 0, 0);
     else if (deep && MT == 1)
