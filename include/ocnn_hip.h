@@ -581,11 +581,20 @@ int ocnn_octree_grow(void* out_dev, const void* out_info, const void* in_dev, co
     int target_depth, int full_octree, ocnn_stream_t stream);
 /* octree_update rewrites children[depth] of `octree_dev` IN PLACE from
  * `label` (the caller clones first, as pytorch/cpp/octree_grow.cpp:165 does),
- * copies the split count back (one device-to-host copy, waited for), patches
- * nnum_nempty[depth] in `info` (host) and in the device header. */
+ * waits for the split count (written by the device into pinned host memory that
+ * the call polls), patches nnum_nempty[depth] in `info` (host) and in the device
+ * header.
+ * ocnn_octree_update_copy is octree_update with the clone inside
+ * (pytorch/cpp/octree_grow.cpp:164-190 as a whole): `out_dev` (as large as the blob
+ * at `in_dev`, another buffer, both 16-byte aligned) gets the blob with the new
+ * children[depth] and count; the copy runs in the launch that writes the
+ * children, behind the one that counts, so the call returns with the count
+ * while the copy is still on its way and the caller can size the next level. */
 size_t ocnn_octree_update_scratch_bytes(int n_label);
 int ocnn_octree_update(void* octree_dev, void* info, const int* label, int n_label, int depth,
     int split, void* scratch_dev, size_t scratch_bytes, ocnn_stream_t stream);
+int ocnn_octree_update_copy(void* out_dev, const void* in_dev, void* info, const int* label, int n_label,
+    int depth, int split, void* scratch_dev, size_t scratch_bytes, ocnn_stream_t stream);
 
 #ifdef __cplusplus
 }

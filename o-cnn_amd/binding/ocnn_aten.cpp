@@ -426,15 +426,15 @@ Tensor octree_grow(Tensor octree_in, int target_depth, bool full_octree) {
 // children[depth] from the split labels, on a copy of the blob (octree_grow.cpp:164-190)
 Tensor octree_update(Tensor octree_in, Tensor label_in, int depth, int split) {
   Info in(octree_in);
-  Tensor out = octree_in.clone();
+  Tensor out = torch::empty_like(octree_in);   // the library copies the blob while it waits for the count
   unsigned char hdr[OCNN_HEADER_BYTES];
   std::memcpy(hdr, in.bytes, OCNN_HEADER_BYTES);
   Tensor label = label_in.contiguous().to(torch::kInt32);
   const int n = (int)label.numel();
   const size_t sb = ocnn_octree_update_scratch_bytes(n);
   Tensor ws = bytes_on(octree_in, sb);
-  check(ocnn_octree_update(out.data_ptr(), hdr, label.data_ptr<int>(), n, depth, split, ws.data_ptr(), sb,
-      current_stream()));
+  check(ocnn_octree_update_copy(out.data_ptr(), octree_in.data_ptr(), hdr, label.data_ptr<int>(), n, depth, split,
+      ws.data_ptr(), sb, current_stream()));
   headers().put(out, hdr);
   return out;
 }

@@ -8,11 +8,19 @@
 #include "scan.h"
 
 #include <algorithm>
+#include <atomic>
+#include <chrono>
 #include <mutex>
 #include <vector>
 
 namespace ocnn {
 namespace {
+
+struct SplitPred {   // label == split
+  const int* label;
+  int split;
+  __device__ bool operator()(int64_t i) const { return label[i] == split; }
+};
 
 struct HeaderArg { uint32_t w[OCNN_HEADER_BYTES / 4]; };
 __global__ void g_write_header_kernel(uint32_t* __restrict__ dst, HeaderArg h) {
@@ -75,13 +83,14 @@ __global__ void g_seq_key_child_kernel(uint64_t* __restrict__ key, int* __restri
 // that every wavefront stores one whole aligned line.
 constexpr int kGrowRanges = 20;
 constexpr int kGrowWordsPerBlock = kBlock * 16;
-enum { kGrowHeader = 0, kGrowCopy, kGrowZero, kGrowSequence, kGrowKeyChild };
+enum { kGrowHeader = 0, kGrowCopy, kGrowZero, kGrowSequence, kGrowKeyChild, kGrowNeigh };
 struct GrowPlan {
   int n;
   int kind[kGrowRanges];
   unsigned first_block[kGrowRanges + 1];
   int64_t dst[kGrowRanges], src[kGrowRanges], words[kGrowRanges];  // byte offsets; words or items
-  int64_t parent_key, parent_child;                                   // byte offsets in the old blob
+  int64_t parent_key, parent_child, parent_neigh;                     // byte offsets in the old blob
+  int parent_nodes, new_groups;                                       // nodes of the old deepest level, sibling groups of the new one
 };
 
 __global__ void __launch_bounds__(kBlock) g_grow_kernel(char* __restrict__ out,
@@ -90,6 +99,12 @@ __global__ void __launch_bounds__(kBlock) g_grow_kernel(char* __restrict__ out,
   while (r + 1 < p.n && blockIdx.x >= p.first_block[r + 1]) ++r;
   const int kind = p.kind[r];
   const int64_t begin = (int64_t)(blockIdx.x - p.first_block[r]) * kGrowWordsPerBlock;
+  if (kind == kGrowNeigh) {   // the new level's neighbour table from the old blob's, beside the copies (calc_neigh, octree_nn.cpp:357-380)
+    const int wave = (int)((blockIdx.x - p.first_block[r]) * (kBlock / 64) + (threadIdx.x >> 6));
+    neigh_sparse_wave<2>(reinterpret_cast<int*>(out + p.dst[r]), reinterpret_cast<const int*>(in + p.parent_neigh),
+        reinterpret_cast<const int*>(in + p.parent_child), p.parent_nodes, 1, p.new_groups, wave, 0);
+    return;
+  }
   if (kind == kGrowKeyChild) {  // generate_key, octree_nn.cpp:427-463, for the children of the old level
     const uint64_t* pkey = reinterpret_cast<const uint64_t*>(in + p.parent_key);
     const int* pchild = reinterpret_cast<const int*>(in + p.parent_child);
@@ -112,13 +127,26 @@ __global__ void __launch_bounds__(kBlock) g_grow_kernel(char* __restrict__ out,
   uint32_t* dst = reinterpret_cast<uint32_t*>(dst_addr) - lead;
   const uint32_t* src = reinterpret_cast<const uint32_t*>(in + p.src[r]) - lead;
   const int64_t stop = min(p.words[r] + lead, begin + kGrowWordsPerBlock);
-  for (int64_t v = begin + threadIdx.x; v < stop; v += kBlock) {
-    if (v < lead) continue;
-    uint32_t val = 0;
-    if (kind == kGrowCopy) val = src[v];
-    else if (kind == kGrowSequence) val = (uint32_t)(v - lead);
-    else if (kind == kGrowHeader) val = h.w[v - lead];
-    dst[v] = val;
+  // four words a thread and step (one 16-byte store; the source of a copy sits at another offset
+  // inside its lines, so it is read as 16 bytes only when it happens to be aligned)
+  const bool src16 = kind == kGrowCopy && (reinterpret_cast<uintptr_t>(src) & 15) == 0;
+  for (int64_t v = begin + 4 * (int64_t)threadIdx.x; v < stop; v += 4 * kBlock) {
+    if (v >= lead && v + 4 <= stop) {
+      uint4 q = make_uint4(0u, 0u, 0u, 0u);
+      if (src16) q = *reinterpret_cast<const uint4*>(src + v);
+      else if (kind == kGrowCopy) q = make_uint4(src[v], src[v + 1], src[v + 2], src[v + 3]);
+      else if (kind == kGrowSequence) q = make_uint4((uint32_t)(v - lead), (uint32_t)(v - lead + 1), (uint32_t)(v - lead + 2), (uint32_t)(v - lead + 3));
+      else if (kind == kGrowHeader) q = make_uint4(h.w[v - lead], h.w[v - lead + 1], h.w[v - lead + 2], h.w[v - lead + 3]);
+      *reinterpret_cast<uint4*>(dst + v) = q;
+      continue;
+    }
+    for (int64_t u = max(v, lead); u < min(v + 4, stop); ++u) {
+      uint32_t val = 0;
+      if (kind == kGrowCopy) val = src[u];
+      else if (kind == kGrowSequence) val = (uint32_t)(u - lead);
+      else if (kind == kGrowHeader) val = h.w[u - lead];
+      dst[u] = val;
+    }
   }
 }
 
@@ -137,7 +165,7 @@ struct GrowRanges {
     unsigned total = 0;
     for (int r = 0; r < plan.n; ++r) {
       plan.first_block[r] = total;
-      int64_t span = plan.words[r] + (plan.kind[r] == kGrowKeyChild ? 0 : 63);
+      int64_t span = plan.words[r] + (plan.kind[r] == kGrowKeyChild || plan.kind[r] == kGrowNeigh ? 0 : 63);
       total += (unsigned)((span + kGrowWordsPerBlock - 1) / kGrowWordsPerBlock);
     }
     plan.first_block[plan.n] = total;
@@ -535,6 +563,14 @@ int ocnn_octree_grow(void* out_dev, const void* out_info, const void* in_dev, co
   std::vector<Span> written;  // payload bytes that some rule or a later kernel writes
   GrowRanges g;
   memset(&g.plan, 0, sizeof(g.plan));
+  if (!full_octree && o.nnum[target_depth - 1] > 0) {   // first: its wavefronts wait longest
+    const int64_t groups = ((int64_t)o.nnum[target_depth - 1] + 7) / 8;
+    g.add(kGrowNeigh, neigh_new, 0, (int64_t)blocks_for((groups + 1) / 2, kBlock / 64) * kGrowWordsPerBlock);
+    g.plan.parent_neigh = oi.ptr_dis(OCNN_NEIGH, target_depth - 1);
+    g.plan.parent_child = oi.ptr_dis(OCNN_CHILD, target_depth - 1);
+    g.plan.parent_nodes = o.nnum[target_depth - 1];
+    g.plan.new_groups = node_num / 8;
+  }
   g.add(kGrowHeader, 0, 0, OCNN_HEADER_BYTES / 4);
   const int props[4] = {OCNN_KEY, OCNN_CHILD, OCNN_NEIGH, OCNN_FEATURE};
   const int elem[4] = {8, 4, 4, 4};
@@ -574,39 +610,144 @@ int ocnn_octree_grow(void* out_dev, const void* out_info, const void* in_dev, co
     if (e) return e;
     e = ocnn_generate_key_full(reinterpret_cast<uint64_t*>(blob + key_new), target_depth, o.batch_size, stream);
     if (e) return e;
-  } else {
-    if (o.nnum[target_depth - 1] > 0) {
-      launch_neigh_sparse(neigh, reinterpret_cast<const int*>(in + oi.ptr_dis(OCNN_NEIGH, target_depth - 1)),
-          reinterpret_cast<const int*>(in + oi.ptr_dis(OCNN_CHILD, target_depth - 1)), o.nnum[target_depth - 1], s,
-          node_num / 8);
-      OCNN_LAUNCH_OK("calc_neigh_sparse");
-    }
   }
   return OCNN_OK;
 }
 
 // pinned words for counts that a call waits for; kept for the life of the process
+struct UpdateSlot { int count; int seq; };
 static std::mutex g_pinned_mutex;
-static std::vector<int*> g_pinned_free;
-static int* take_pinned_int() {
+static std::vector<UpdateSlot*> g_pinned_free;
+static std::atomic<int> g_update_seq{1};
+static UpdateSlot* take_slot() {
   {
     std::lock_guard<std::mutex> lock(g_pinned_mutex);
-    if (!g_pinned_free.empty()) { int* p = g_pinned_free.back(); g_pinned_free.pop_back(); return p; }
+    if (!g_pinned_free.empty()) { UpdateSlot* p = g_pinned_free.back(); g_pinned_free.pop_back(); return p; }
   }
   void* p = nullptr;
-  if (hipHostMalloc(&p, 64, hipHostMallocDefault) != hipSuccess) return nullptr;
-  return static_cast<int*>(p);
+  if (hipHostMalloc(&p, 64, hipHostMallocCoherent) != hipSuccess) return nullptr;
+  memset(p, 0, 64);
+  return static_cast<UpdateSlot*>(p);
 }
-static void give_pinned_int(int* p) {
+static void give_slot(UpdateSlot* p) {
   std::lock_guard<std::mutex> lock(g_pinned_mutex);
   g_pinned_free.push_back(p);
 }
 
-__global__ void g_fix_empty_split_kernel(int* children, int* count) {
-  if (threadIdx.x == 0 && blockIdx.x == 0 && *count == 0) { children[0] = 0; *count = 1; }
+// Scan of the tile counts (one workgroup, as scan_tiles_kernel) that also settles the split count:
+// nothing splits -> one node is kept (octree_grow.cpp:180-185; result[1] says so).  The count goes
+// to the device words and, `seq` last, to the pinned host slot that the caller polls: the launches
+// behind this one (the ranks, the copy of the blob) then run while the host already sizes the next
+// level.
+__global__ void g_update_tiles_kernel(int* __restrict__ tile_count, int n_tiles, int* __restrict__ result,
+    UpdateSlot* __restrict__ host, int seq) {
+  __shared__ int carry;
+  if (threadIdx.x == 0) carry = 0;
+  __syncthreads();
+  for (int start = 0; start < n_tiles; start += kBlock) {
+    const int i = start + threadIdx.x;
+    const int v = i < n_tiles ? tile_count[i] : 0;
+    int total;
+    const int ex = block_exclusive_scan(v, &total);
+    const int c = carry;
+    if (i < n_tiles) tile_count[i] = c + ex;
+    __syncthreads();
+    if (threadIdx.x == 0) carry = c + total;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    const int none = carry == 0 ? 1 : 0;
+    const int count = none ? 1 : carry;
+    result[0] = count;
+    result[1] = none;
+    __hip_atomic_store(&host->count, count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    __threadfence_system();
+    __hip_atomic_store(&host->seq, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
 }
-__global__ void g_patch_nempty_kernel(int* header_nempty_d, const int* count) {
-  if (threadIdx.x == 0 && blockIdx.x == 0) *header_nempty_d = *count;
+
+// Workgroups 0 .. tiles-1: children[i] = rank among the labels equal to `split`, -1 for the others
+// (generate_label, octree_nn.h:176-177).  Workgroups from `tiles` on: the words of the source blob
+// outside the child array go to the result, the header word nnum_nempty[depth] replaced by the
+// count; in place (`src` null) the first workgroup patches that word.
+__global__ void __launch_bounds__(kBlock) g_update_apply_kernel(uint32_t* __restrict__ dst, const uint32_t* __restrict__ src,
+    const int* __restrict__ label, int split, int n, const int* __restrict__ tile_offset, const int* __restrict__ result,
+    int tiles, int64_t child_word, int64_t count_word, int64_t blob_words) {
+  if ((int)blockIdx.x < tiles) {
+    int* children = reinterpret_cast<int*>(dst + child_word);
+    const int64_t base = (int64_t)blockIdx.x * kScanTile + (int64_t)threadIdx.x * kScanItems;
+    bool f[kScanItems];
+    int c = 0;
+#pragma unroll
+    for (int j = 0; j < kScanItems; ++j) {
+      f[j] = base + j < n && label[base + j] == split;
+      c += f[j] ? 1 : 0;
+    }
+    int total;
+    int rank = tile_offset[blockIdx.x] + block_exclusive_scan(c, &total);
+    const bool none = result[1] != 0;
+#pragma unroll
+    for (int j = 0; j < kScanItems; ++j) {
+      if (base + j < n) children[base + j] = f[j] ? rank : ((none && base + j == 0) ? 0 : -1);
+      rank += f[j] ? 1 : 0;
+    }
+    if (!src && blockIdx.x == 0 && threadIdx.x == 0) dst[count_word] = (uint32_t)result[0];
+    return;
+  }
+  // four words a thread; a piece that touches the child array or lies at the end goes word by word
+  const int64_t w0 = ((int64_t)(blockIdx.x - tiles) * kBlock + threadIdx.x) * 4;
+  if (w0 >= blob_words) return;
+  const uint32_t count = (uint32_t)result[0];
+  if (w0 + 4 <= blob_words && (w0 + 4 <= child_word || w0 >= child_word + n)) {
+    uint4 v = *reinterpret_cast<const uint4*>(src + w0);
+    if (count_word >= w0 && count_word < w0 + 4) (&v.x)[count_word - w0] = count;
+    *reinterpret_cast<uint4*>(dst + w0) = v;
+    return;
+  }
+  for (int64_t w = w0; w < w0 + 4 && w < blob_words; ++w)
+    if (w < child_word || w >= child_word + n) dst[w] = w == count_word ? count : src[w];
+}
+
+// children[depth] from the labels into `out` (the rest of `in` copied along when `in` is given),
+// the split count to *split_num
+static int update_impl(char* out, const char* in, const Info& o, const int* label, int n_label, int depth, int split,
+    void* scratch_dev, size_t scratch_bytes, hipStream_t s, int* split_num) {
+  const size_t need = scan_scratch_bytes(n_label) + 256;
+  OCNN_REQUIRE(scratch_dev && scratch_bytes >= need, OCNN_E_WORKSPACE, "scratch %zu < %zu bytes", scratch_bytes, need);
+  OCNN_REQUIRE((reinterpret_cast<uintptr_t>(out) & 15) == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0, OCNN_E_BADARG,
+      "octree blobs must be 16-byte aligned");
+  int* result = reinterpret_cast<int*>(scratch_dev);
+  int* tile_count = reinterpret_cast<int*>(static_cast<char*>(scratch_dev) + 256);
+  int tiles = scan_tiles(n_label);
+  if (tiles == 0) tiles = 1;
+  UpdateSlot* slot = take_slot();
+  OCNN_REQUIRE(slot, OCNN_E_HIP, "no pinned host memory for the split count");
+  const int seq = g_update_seq.fetch_add(1) & 0x3fffffff;
+  SplitPred pred{label, split};
+  scan_count_kernel<SplitPred><<<tiles, kBlock, 0, s>>>(pred, n_label, tile_count);
+  g_update_tiles_kernel<<<1, kBlock, 0, s>>>(tile_count, tiles, result, slot, seq);
+  const int64_t blob_words = o.sizeof_octree() / 4;
+  const unsigned copy_blocks = in ? blocks_for(blob_words, kBlock * 4) : 0;
+  g_update_apply_kernel<<<tiles + copy_blocks, kBlock, 0, s>>>(reinterpret_cast<uint32_t*>(out),
+      reinterpret_cast<const uint32_t*>(in), label, split, n_label, tile_count, result, tiles,
+      o.ptr_dis(OCNN_CHILD, depth) / 4, (int64_t)(offsetof(Info, nnum_nempty) / 4) + depth, blob_words);
+  if (hipGetLastError() != hipSuccess) { give_slot(slot); return fail(OCNN_E_HIP, "launch of octree_update failed"); }
+  // the count is a few microseconds away; after 20 ms of polling the stream is asked (which also
+  // reports a launch that failed)
+  const auto t0 = std::chrono::steady_clock::now();
+  bool seen = false;
+  for (int spins = 0;; ++spins) {
+    if (__atomic_load_n(&slot->seq, __ATOMIC_ACQUIRE) == seq) { seen = true; break; }
+    if ((spins & 1023) == 1023 && std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(20)) break;
+  }
+  if (!seen) {
+    const hipError_t err = hipStreamSynchronize(s);
+    seen = err == hipSuccess && __atomic_load_n(&slot->seq, __ATOMIC_ACQUIRE) == seq;
+    if (!seen) { give_slot(slot); return fail(OCNN_E_HIP, "split count: %s", hipGetErrorString(err)); }
+  }
+  *split_num = slot->count;
+  give_slot(slot);
+  return OCNN_OK;
 }
 
 int ocnn_octree_update(void* octree_dev, void* info, const int* label, int n_label, int depth, int split,
@@ -616,27 +757,26 @@ int ocnn_octree_update(void* octree_dev, void* info, const int* label, int n_lab
   OCNN_REQUIRE(depth >= 0 && depth <= o->depth, OCNN_E_BADARG, "depth %d", depth);
   OCNN_REQUIRE(n_label == o->nnum[depth], OCNN_E_SHAPE, "label has %d entries, depth %d has %d nodes", n_label,
       depth, o->nnum[depth]);
-  size_t need = scan_scratch_bytes(n_label) + 256;
-  OCNN_REQUIRE(scratch_dev && scratch_bytes >= need, OCNN_E_WORKSPACE, "scratch %zu < %zu bytes", scratch_bytes, need);
-  hipStream_t s = as_stream(stream);
-  char* blob = static_cast<char*>(octree_dev);
-  int* children = reinterpret_cast<int*>(blob + o->ptr_dis(OCNN_CHILD, depth));
-  int* count_dev = reinterpret_cast<int*>(scratch_dev);
-  void* scan_scratch = static_cast<char*>(scratch_dev) + 256;
-  int e = ocnn_generate_label(children, count_dev, label, n_label, split, scan_scratch, scratch_bytes - 256, stream);
+  int split_num = 0;
+  const int e = update_impl(static_cast<char*>(octree_dev), nullptr, *o, label, n_label, depth, split, scratch_dev,
+      scratch_bytes, as_stream(stream), &split_num);
   if (e) return e;
-  // degenerate case: nothing splits -> keep one node (octree_grow.cpp:180-185)
-  g_fix_empty_split_kernel<<<1, 64, 0, s>>>(children, count_dev);
-  g_patch_nempty_kernel<<<1, 64, 0, s>>>(reinterpret_cast<int*>(blob + offsetof(Info, nnum_nempty)) + depth, count_dev);
-  OCNN_LAUNCH_OK("octree_update");
-  // the count comes back through pinned memory: a copy into pageable memory is staged
-  int* pinned = take_pinned_int();
-  OCNN_REQUIRE(pinned, OCNN_E_HIP, "no pinned host memory for the split count");
-  hipError_t err = hipMemcpyAsync(pinned, count_dev, sizeof(int), hipMemcpyDeviceToHost, s);
-  if (err == hipSuccess) err = hipStreamSynchronize(s);
-  int split_num = *pinned;
-  give_pinned_int(pinned);
-  OCNN_REQUIRE(err == hipSuccess, OCNN_E_HIP, "split count: %s", hipGetErrorString(err));
+  o->nnum_nempty[depth] = split_num;
+  return OCNN_OK;
+}
+
+int ocnn_octree_update_copy(void* out_dev, const void* in_dev, void* info, const int* label, int n_label, int depth,
+    int split, void* scratch_dev, size_t scratch_bytes, ocnn_stream_t stream) {
+  OCNN_REQUIRE(out_dev && in_dev && info && label, OCNN_E_BADARG, "null pointer");
+  OCNN_REQUIRE(out_dev != in_dev, OCNN_E_BADARG, "ocnn_octree_update_copy writes a second blob: use ocnn_octree_update in place");
+  Info* o = static_cast<Info*>(info);
+  OCNN_REQUIRE(depth >= 0 && depth <= o->depth, OCNN_E_BADARG, "depth %d", depth);
+  OCNN_REQUIRE(n_label == o->nnum[depth], OCNN_E_SHAPE, "label has %d entries, depth %d has %d nodes", n_label,
+      depth, o->nnum[depth]);
+  int split_num = 0;
+  const int e = update_impl(static_cast<char*>(out_dev), static_cast<const char*>(in_dev), *o, label, n_label, depth,
+      split, scratch_dev, scratch_bytes, as_stream(stream), &split_num);
+  if (e) return e;
   o->nnum_nempty[depth] = split_num;
   return OCNN_OK;
 }

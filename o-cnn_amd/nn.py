@@ -1342,14 +1342,14 @@ def octree_update(octree_in, label_in, depth, split):
   """pytorch/cpp/octree_grow.cpp:164-190: children[depth] from the split labels."""
   octree_in = _to_dev(octree_in)
   iin = octree_info(octree_in)
-  out = octree_in.clone()
+  out = torch.empty_like(octree_in)     # (the library copies the blob while the host waits for the count)
   info = _Info(iin.raw)
   label = _to_dev(label_in.contiguous().to(torch.int32))
   n = label.numel()
   sb = _lib.get().ocnn_octree_update_scratch_bytes(n)
   ws = _workspace(sb + 256, "update")
   base = (ws.data_ptr() + 255) & ~255
-  _lib.call("ocnn_octree_update", _ptr(out), info.p, _ptr(label), n, depth, split,
+  _lib.call("ocnn_octree_update_copy", _ptr(out), _ptr(octree_in), info.p, _ptr(label), n, depth, split,
             C.c_void_p(base), C.c_size_t(sb), _stream())
   out._ocnn_info = _Info(info.raw)
   return out
