@@ -1296,8 +1296,10 @@ int adaptive_finish(const AdaptiveInput& in, ocnn_alloc_fn alloc, void* alloc_ct
       }
     }
     int h[64];
-    OCNN_HIP_OK(hipMemcpyAsync(h, d_counts, sizeof(h), hipMemcpyDeviceToHost, s));
-    OCNN_HIP_OK(hipStreamSynchronize(s));
+    {
+      const int e = fetch_words(h, d_counts, 64, s);
+      if (e) return e;
+    }
     for (int d = A; d <= D; ++d) { o.nnum[d] = h[d]; o.nnum_nempty[d] = h[17 + d]; }
   }
   o.set_nnum_cum();

@@ -2,7 +2,11 @@
 // kernel-shape tables.  Layout rules follow octree/octree/octree_info.cpp:143-268.
 #include "ocnn_common.h"
 
+#include <atomic>
+#include <chrono>
 #include <cstdint>
+#include <mutex>
+#include <vector>
 
 #include <stdarg.h>
 #include <stdio.h>
@@ -17,6 +21,60 @@ int fail(int code, const char* fmt, ...) {
   vsnprintf(g_err, sizeof(g_err), fmt, ap);
   va_end(ap);
   return code;
+}
+
+// ---- small results back to the host -------------------------------------------------------------
+namespace {
+struct FetchSlot { uint32_t w[kFetchWords]; int seq; int pad[63]; };
+std::mutex g_fetch_mutex;
+std::vector<FetchSlot*> g_fetch_free;
+std::atomic<int> g_fetch_seq{1};
+
+__global__ void fetch_words_kernel(FetchSlot* __restrict__ host, const uint32_t* __restrict__ dev, int n, int seq) {
+  const int i = threadIdx.x;
+  if (i < n) __hip_atomic_store(&host->w[i], dev[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  __threadfence_system();
+  __syncthreads();
+  if (i == 0) __hip_atomic_store(&host->seq, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+}  // namespace
+
+int fetch_words(void* host_out, const void* dev_words, int n, hipStream_t s) {
+  OCNN_REQUIRE(host_out && dev_words && n >= 0 && n <= kFetchWords, OCNN_E_BADARG, "fetch of %d words", n);
+  FetchSlot* slot = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(g_fetch_mutex);
+    if (!g_fetch_free.empty()) { slot = g_fetch_free.back(); g_fetch_free.pop_back(); }
+  }
+  if (!slot) {
+    void* p = nullptr;
+    OCNN_REQUIRE(hipHostMalloc(&p, sizeof(FetchSlot), hipHostMallocCoherent) == hipSuccess, OCNN_E_HIP,
+        "no pinned host memory for a result of the device");
+    memset(p, 0, sizeof(FetchSlot));
+    slot = static_cast<FetchSlot*>(p);
+  }
+  const int seq = g_fetch_seq.fetch_add(1) & 0x3fffffff;
+  fetch_words_kernel<<<1, kFetchWords, 0, s>>>(slot, static_cast<const uint32_t*>(dev_words), n, seq);
+  hipError_t err = hipGetLastError();
+  bool seen = false;
+  if (err == hipSuccess) {
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int spins = 0;; ++spins) {
+      if (__atomic_load_n(&slot->seq, __ATOMIC_ACQUIRE) == seq) { seen = true; break; }
+      if ((spins & 1023) == 1023 && std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(20)) break;
+    }
+    if (!seen) {
+      err = hipStreamSynchronize(s);
+      seen = err == hipSuccess && __atomic_load_n(&slot->seq, __ATOMIC_ACQUIRE) == seq;
+    }
+  }
+  if (seen) memcpy(host_out, slot->w, sizeof(uint32_t) * (size_t)n);
+  {
+    std::lock_guard<std::mutex> lock(g_fetch_mutex);
+    g_fetch_free.push_back(slot);
+  }
+  OCNN_REQUIRE(seen, OCNN_E_HIP, "a result of the device did not arrive: %s", hipGetErrorString(err));
+  return OCNN_OK;
 }
 
 void Info::reset() {

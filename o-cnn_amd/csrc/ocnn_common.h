@@ -105,6 +105,14 @@ int prepare_builtin_scratch();
 
 inline hipStream_t as_stream(ocnn_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
+// `n` (at most kFetchWords) 32-bit words of device memory that work queued on `s` produces, to
+// host memory: a one-wavefront launch writes them into pinned memory and a sequence number
+// behind them, and the call polls that number (the answer is a few microseconds behind the
+// producing kernel; a copy into pageable memory plus a wait for the stream takes three to four
+// times as long).  After 20 ms of polling the stream is asked, which also reports a failed launch.
+constexpr int kFetchWords = 64;
+int fetch_words(void* host_out, const void* dev_words, int n, hipStream_t s);
+
 constexpr int kBlock = 256;
 inline unsigned blocks_for(int64_t n, int per_block = kBlock) {
   int64_t b = (n + per_block - 1) / per_block;

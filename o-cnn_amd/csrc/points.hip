@@ -308,9 +308,7 @@ int ocnn_bounding_sphere(const void* points_dev, const void* points_info, int me
   OCNN_LAUNCH_OK("extremes");
   sphere_kernel<<<1, kSphereThreads, 0, s>>>(out_dev, partial, blocks, pt, pi->pt_num, method_box ? 1 : 0);
   OCNN_LAUNCH_OK("sphere");
-  OCNN_HIP_OK(hipMemcpyAsync(out4, out_dev, 4 * sizeof(float), hipMemcpyDeviceToHost, s));
-  OCNN_HIP_OK(hipStreamSynchronize(s));
-  return OCNN_OK;
+  return fetch_words(out4, out_dev, 4, s);
 }
 
 int ocnn_normalize_points(void* out_dev, const void* in_dev, const void* points_info, float radius,
@@ -385,8 +383,10 @@ int ocnn_clip_points(void* out_dev, void* out_info, int* inbox_mask_dev, const v
   int* scratch = reinterpret_cast<int*>(static_cast<char*>(workspace_dev) + 256);
   OCNN_HIP_OK(flag_scan(pred, co, npt, scratch, total_dev, s));
   int inside = 0;
-  OCNN_HIP_OK(hipMemcpyAsync(&inside, total_dev, sizeof(int), hipMemcpyDeviceToHost, s));
-  OCNN_HIP_OK(hipStreamSynchronize(s));
+  {
+    const int e = fetch_words(&inside, total_dev, 1, s);
+    if (e) return e;
+  }
   PointsInfo hdr = *pi;
   const int none = inside == 0;
   hdr.pt_num = none ? 1 : inside;

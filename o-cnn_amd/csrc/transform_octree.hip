@@ -297,8 +297,10 @@ extern "C" int ocnn_octree_scan(const void* octree_dev, const void* info, const 
     OCNN_REQUIRE(e == hipSuccess, OCNN_E_HIP, "scan: %s", hipGetErrorString(e));
   }
   int h[32];
-  OCNN_HIP_OK(hipMemcpyAsync(h, d_counts, sizeof(h), hipMemcpyDeviceToHost, s));
-  OCNN_HIP_OK(hipStreamSynchronize(s));
+  {
+    const int e = fetch_words(h, d_counts, 32, s);
+    if (e) return e;
+  }
 
   Info o = oi;
   for (int d = 0; d <= D; ++d) o.nnum_nempty[d] = d < fl ? (1 << (3 * d)) : h[d];
@@ -417,8 +419,11 @@ extern "C" int ocnn_octree_dropout(const void* octree_dev, const void* info, con
     OCNN_REQUIRE(e == hipSuccess, OCNN_E_HIP, "scan: %s", hipGetErrorString(e));
   }
   int h[2 * kMaxD];
-  OCNN_HIP_OK(hipMemcpyAsync(h, d_counts, sizeof(h), hipMemcpyDeviceToHost, s));
-  OCNN_HIP_OK(hipStreamSynchronize(s));
+  {
+    static_assert(2 * kMaxD <= kFetchWords, "counts of both scans in one fetch");
+    const int e = fetch_words(h, d_counts, 2 * kMaxD, s);
+    if (e) return e;
+  }
 
   Info o = oi;
   for (int d = dd + 1; d <= D; ++d) o.nnum[d] = h[d];
