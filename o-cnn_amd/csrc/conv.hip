@@ -185,6 +185,69 @@ __device__ inline void store_tiles(const ConvArgs& a, OutT* __restrict__ out, fl
     }
 }
 
+// ---- one tap, stride 1 (1x1x1): no neighbours --------------------------------------------------
+// out[m][n] = sum over c of W(m, c) x[c][n]: the product of two matrices on the channel-major
+// tensor as it lies (lanes 0 .. 31 read 32 consecutive columns of channel c, lanes 32 .. 63 of
+// channel c + 1: the B operand of one k-step), bound by the bytes of x and out.  The weights of a
+// chunk of channels wait in LDS in A-fragment order.
+constexpr int kOneTapChunk = 128;   // channels per LDS stage
+template <int MT>
+__global__ __launch_bounds__(256) void conv_one_tap_f32_kernel(ConvArgs a, float* __restrict__ out,
+    const float* __restrict__ in, const float* __restrict__ W, int64_t sm, int64_t sc, int n_tiles) {
+  __shared__ float sW[(kOneTapChunk / 2) * MT * 64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = xcd_tile(blockIdx.x, n_tiles);
+  if (tile >= n_tiles) return;
+  const int n0 = tile * kTileCols + wave * kWaveCols;
+  const int r = lane & 31, kh = lane >> 5;
+  const int npass = (a.mtiles + MT - 1) / MT;
+  // columns past the end read the last column (their results are not stored)
+  const float* x0 = in + min(n0 + r, a.N - 1);
+  const float* x1 = in + min(n0 + 32 + r, a.N - 1);
+  for (int pass = blockIdx.y; pass < npass; pass += gridDim.y) {
+    floatx16 acc[MT][2];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
+    for (int c0 = 0; c0 < a.Cin; c0 += kOneTapChunk) {
+      const int nks = (min(kOneTapChunk, a.Cin - c0) + 1) >> 1;
+      __syncthreads();   // the previous chunk's fragments are no longer read
+      for (int e = threadIdx.x; e < nks * MT * 64; e += 256) {
+        const int l = e & 63, mt = (e >> 6) % MT, ks = (e >> 6) / MT;
+        const int m = (pass * MT + mt) * 32 + (l & 31), c = c0 + 2 * ks + (l >> 5);
+        sW[e] = (m < a.M && c < a.Cin) ? W[m * sm + c * sc] : 0.0f;
+      }
+      __syncthreads();
+      constexpr int kAhead = 8;   // k-steps whose operands are requested together
+      for (int k0 = 0; k0 < nks; k0 += kAhead) {
+        float b0[kAhead], b1[kAhead];
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+          const int c = c0 + 2 * (k0 + u) + kh;
+          const int64_t row = (int64_t)min(c, a.Cin - 1) * a.Hin;
+          b0[u] = x0[row];
+          b1[u] = x1[row];
+          if (c >= a.Cin || k0 + u >= nks) { b0[u] = 0.0f; b1[u] = 0.0f; }   // (an odd channel count: the weight there is zero too)
+        }
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+          if (k0 + u >= nks) break;   // uniform
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            const float av = sW[((k0 + u) * MT + mt) * 64 + lane];
+            acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b0[u], acc[mt][0], 0, 0, 0);
+            acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b1[u], acc[mt][1], 0, 0, 0);
+          }
+        }
+      }
+    }
+    if (n0 < a.N) store_tiles<float, MT>(a, out, acc, pass * MT, n0, lane);
+  }
+}
+
 // ---- general gather kernel over a row-major copy of the input -------------------------------
 // Every case without a dedicated kernel (non-empty-node convolutions, the small kernel shapes,
 // stride-2 cases other than 2x2x2 over all nodes) runs here.  The input is first copied
@@ -2491,9 +2554,13 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
   // which kernel runs, and how much of the workspace it touches: the weights in their packed
   // order always come first, the inverted child links of the non-empty mode second, the
   // row-major copy of the input (only some kernels read one) last
-  enum { kPathS2Conv, kPathS2Deconv, kPathS1LdsF32, kPathRowsF32, kPathS1LdsBf16, kPathRowsBf16 } path;
+  enum { kPathS2Conv, kPathS2Deconv, kPathS1LdsF32, kPathRowsF32, kPathS1LdsBf16, kPathRowsBf16, kPathOneTapF32 } path;
   bool copies_input = true;
-  if (a.mode == kModeS2Conv && !a.nempty && k222 && (a.Hin & 7) == 0 &&
+  if (dtype == OCNN_F32 && a.mode == kModeS1 && a.K == 1 && a.Hin == a.N && a.Hin > 0) {
+    // 1x1x1: every column reads its own row, over all nodes and over the non-empty ones alike
+    path = kPathOneTapF32;
+    copies_input = false;
+  } else if (a.mode == kModeS2Conv && !a.nempty && k222 && (a.Hin & 7) == 0 &&
       (reinterpret_cast<uintptr_t>(btm) & 15) == 0) {
     path = kPathS2Conv;
     copies_input = false;
@@ -2518,7 +2585,7 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
         "this call needs %zu bytes of scratch memory, the built-in array holds %zu: "
         "use ocnn_octree_conv_fused with a workspace of your own", used, ws_bytes);
   }
-  if (nempty) {
+  if (nempty && path != kPathOneTapF32) {
     int* ichild = reinterpret_cast<int*>(wsb + p.wt_bytes);
     ichild_kernel<<<blocks_for(p.child_h), kBlock, 0, s>>>(ichild, p.ichild_h, a.child, p.child_h);
     OCNN_LAUNCH_OK("ichild");
@@ -2567,6 +2634,13 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
       else
         deconv_s2_bf16_kernel<<<dim3(d_grid, pass_split(d_tiles, (d.M * 8 + 32 * kD2MT - 1) / (32 * kD2MT))), 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles, cpad / 8);
     }
+  } else if (path == kPathOneTapF32) {
+    const int MT = a.mtiles == 1 ? 1 : 2;
+    const int npass = (a.mtiles + MT - 1) / MT;
+    if (MT == 1)
+      conv_one_tap_f32_kernel<1><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)weights, sm, sc, n_tiles);
+    else
+      conv_one_tap_f32_kernel<2><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)weights, sm, sc, n_tiles);
   } else if (path == kPathS1LdsF32) {
     // Two row tiles a workgroup halve the gathers per product, one row tile doubles the number of
     // workgroups: the latter where a level is so small that the former leaves the CUs short of work
