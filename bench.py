@@ -459,9 +459,14 @@ def main():
       grown = F.octree_grow(F.octree_update(oct8, lab, 8, 1), 9, False)
     torch.cuda.synchronize()
     t = (time.perf_counter() - t0) / reps
+    # (GBs: the bytes of the new level and what they are made from; moved: both operators return a
+    # new blob as the reference's do, so the depth-8 blob is read twice and written once beside the
+    # grown one)
+    moved = 3 * oct8.numel() + grown.numel() + H8 * 4
     extra["octree_update_d8_plus_grow_d9"] = {
         "ms": t * 1e3, "new_nodes": F.octree_info(grown).nnum(9),
-        "GBs": (H9 * (8 + 4 + 32) + H8 * (4 + 4 + 32 + 8)) / t / 1e9}
+        "GBs": (H9 * (8 + 4 + 32) + H8 * (4 + 4 + 32 + 8)) / t / 1e9,
+        "GBs_moved": moved / t / 1e9, "frac_hbm_peak_moved": moved / t / 1e9 / PEAK_HBM_GBS}
     # merge of 16 separately built, serialized octrees (octree_batch on device blobs)
     singles = [F.points2octree(c, 7, 2) for c in cl]
     torch.cuda.synchronize()
