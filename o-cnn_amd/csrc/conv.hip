@@ -2028,8 +2028,13 @@ constexpr int kD2MT = 4;  // row tiles per pass: 128 rows = 16 output channels x
 constexpr int kD2fMT = 2;
 constexpr int kD2fChunk = 64;
 
+// HALF: a layer of 32 input channels or fewer fills the first half of its one chunk only, and the
+// k-steps of the other half (zero weights) are left out at compile time (a test inside the loop
+// costs the schedule of every k-step).
+template <bool HALF>
 __global__ __launch_bounds__(256, 3) void deconv_s2_f32_kernel(ConvArgs a, float* __restrict__ out,
     const float* __restrict__ in, const float* __restrict__ W, int n_tiles) {
+  constexpr int kSteps = HALF ? kD2fChunk / 4 : kD2fChunk / 2;   // k-steps (channel pairs) of a stage
   __shared__ __attribute__((aligned(16))) float sW[kD2fChunk * 32 * kD2fMT];
   constexpr int kWVec = kD2fChunk * 32 * kD2fMT / 4 / 256;  // float4 per thread and stage
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -2068,7 +2073,7 @@ __global__ __launch_bounds__(256, 3) void deconv_s2_f32_kernel(ConvArgs a, float
     }
   };
 #pragma unroll
-  for (int ks = 0; ks < kD2fChunk / 2; ++ks) load_x(0, ks);
+  for (int ks = 0; ks < kSteps; ++ks) load_x(0, ks);
   fetch_w(0);
   floatx16 acc[kD2fMT][2];
   for (int stage = 0; stage < nstage; ++stage) {
@@ -2089,7 +2094,7 @@ __global__ __launch_bounds__(256, 3) void deconv_s2_f32_kernel(ConvArgs a, float
     const int next_chunk = (chunk + 1) % nchunk;
     const bool refill = nchunk > 1 && stage + 1 < nstage;
 #pragma unroll
-    for (int ks = 0; ks < kD2fChunk / 2; ++ks) {
+    for (int ks = 0; ks < kSteps; ++ks) {
       const float b0 = xb[ks][0], b1 = xb[ks][1];
       if (refill) load_x(next_chunk, ks);
 #pragma unroll
@@ -2614,7 +2619,10 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     int d_tiles = (d.N + kTileCols - 1) / kTileCols;
     int d_grid = ((d_tiles + 7) / 8) * 8;
     if (dtype == OCNN_F32) {
-      deconv_s2_f32_kernel<<<d_grid, 256, 0, s>>>(d, (float*)top, (const float*)btm, (const float*)weights, d_tiles);
+      if (d.Cin <= kD2fChunk / 2)
+        deconv_s2_f32_kernel<true><<<d_grid, 256, 0, s>>>(d, (float*)top, (const float*)btm, (const float*)weights, d_tiles);
+      else
+        deconv_s2_f32_kernel<false><<<d_grid, 256, 0, s>>>(d, (float*)top, (const float*)btm, (const float*)weights, d_tiles);
     } else {
       const int cpad = (a.Cin + 15) / 16 * 16;
       const int rows = a.M * 8, npass = (rows + 32 * kD2MT - 1) / (32 * kD2MT), ksteps = cpad / 16;

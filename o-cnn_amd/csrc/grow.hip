@@ -639,7 +639,7 @@ static void give_slot(UpdateSlot* p) {
 // to the device words and, `seq` last, to the pinned host slot that the caller polls: the launches
 // behind this one (the ranks, the copy of the blob) then run while the host already sizes the next
 // level.
-__global__ void g_update_tiles_kernel(int* __restrict__ tile_count, int n_tiles, int* __restrict__ result,
+static __global__ void g_update_tiles_kernel(int* __restrict__ tile_count, int n_tiles, int* __restrict__ result,
     UpdateSlot* __restrict__ host, int seq) {
   __shared__ int carry;
   if (threadIdx.x == 0) carry = 0;
@@ -670,7 +670,7 @@ __global__ void g_update_tiles_kernel(int* __restrict__ tile_count, int n_tiles,
 // (generate_label, octree_nn.h:176-177).  Workgroups from `tiles` on: the words of the source blob
 // outside the child array go to the result, the header word nnum_nempty[depth] replaced by the
 // count; in place (`src` null) the first workgroup patches that word.
-__global__ void __launch_bounds__(kBlock) g_update_apply_kernel(uint32_t* __restrict__ dst, const uint32_t* __restrict__ src,
+static __global__ void __launch_bounds__(kBlock) g_update_apply_kernel(uint32_t* __restrict__ dst, const uint32_t* __restrict__ src,
     const int* __restrict__ label, int split, int n, const int* __restrict__ tile_offset, const int* __restrict__ result,
     int tiles, int64_t child_word, int64_t count_word, int64_t blob_words) {
   if ((int)blockIdx.x < tiles) {
