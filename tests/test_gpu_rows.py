@@ -386,3 +386,35 @@ def test_row_kernel_forms_and_source_tables_agree(oc, octree):
         assert torch.equal(r, results[0]), (depth, cin, cout, ks, stride, deconv)
   finally:
     L.ocnn_conv_rows_direct(1)
+
+
+def test_row_kernel_workgroup_sizes_at_scene_levels(oc, synthetic):
+  """The barrier-free row kernel runs in workgroups of four, two or one wavefront, picked by how the
+  level's tiles spread over the device (depth 6 of the scene: four; depth 7: two; depth 9: one).
+  Whatever the size, it forms the same products in the same order as the staged kernel (always 256
+  columns a workgroup), so at each of those levels the two forms, row-major and channel-major,
+  give the same bits."""
+  F = oc.nn
+  L = oc.lib.get()
+  p, n, f = synthetic.room_cloud(250000, 3)
+  octree = F.points2octree_batch([T(make_points_blob(p, n, f)).cuda()], 9, 2)
+  info = F.octree_info(octree)
+  g = torch.Generator().manual_seed(17)
+  try:
+    for depth, cin, cout in ((6, 256, 256), (7, 128, 128), (7, 64, 64), (9, 64, 64), (9, 32, 32)):
+      H = info.nnum_nempty(depth)
+      x = torch.randn(1, cin, H, 1, generator=g).bfloat16().cuda()
+      xr = F.to_rows(x)
+      w = (torch.randn(cout, cin * 27, generator=g) * 0.05).bfloat16().cuda()
+      b = (torch.randn(cout, generator=g) * 0.1).cuda()
+      results = []
+      for form in (1, 0):
+        L.ocnn_conv_rows_direct(form)
+        F.forget_cached(octree)
+        results.append(F.octree_conv_rows(xr, cin, w, octree, depth, cout, bias=b, relu=True, nempty=True))
+        results.append(F.to_rows(F.octree_conv_fused(x, w, b, True, octree, depth, cout, [3, 3, 3], 1, True)))
+      for r in results[1:]:
+        assert torch.equal(r, results[0]), (depth, cin, cout)
+      assert float(results[0].float().abs().max()) > 0
+  finally:
+    L.ocnn_conv_rows_direct(1)

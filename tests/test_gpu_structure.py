@@ -557,3 +557,35 @@ def test_octree_beyond_the_format_limit_is_refused(oc, synthetic):
   # the workspace is reusable after the refusal
   o = F.points2octree_batch(clouds[:2], 9, 2)
   assert F.octree_info(o).batch_size == 2
+
+
+@pytest.mark.parametrize("n_scenes,depth", [(1, 9), (3, 9), (2, 7)], ids=["three_levels", "two_levels", "small"])
+def test_neighbour_tables_of_fused_levels_at_full_size(oc, synthetic, n_scenes, depth):
+  """The build writes the neighbour tables of its last sparse levels in one launch (three levels up
+  to 2 M nodes on the finest, two up to 8 M, one above).  Whatever it fused, every sparse level's
+  table must be what calc_neigh makes of the level above (ocnn_calc_neigh_sparse, one level a
+  launch, checked against the oracle in test_gpu_ops.py): the identity that defines the table
+  (octree/octree/octree_nn.cpp:357-380), at the sizes that pick each form."""
+  import ctypes as C
+  F = oc.nn
+  p, n, f = synthetic.room_cloud(250000, 3)
+  clouds = [T(make_points_blob(p + np.float32(1e-4 * i), n, f)).cuda() for i in range(n_scenes)]
+  octree = F.points2octree_batch(clouds, depth, 2)
+  info = F.octree_info(octree)
+  finest = info.nnum(depth)
+  if n_scenes == 3:
+    assert 1 << 21 < finest <= 1 << 23      # the size class that fuses two levels
+  else:
+    assert finest <= 1 << 21                # ... three
+  P = lambda t: C.c_void_p(t.data_ptr())
+  checked = 0
+  for d in range(info.full_depth + 1, depth + 1):
+    above = F.octree_property(octree, "neigh", d - 1).contiguous()
+    child = F.octree_property(octree, "child", d - 1).contiguous()
+    got = F.octree_property(octree, "neigh", d)
+    exp = torch.empty_like(got)
+    oc.lib.call("ocnn_calc_neigh_sparse", P(exp), P(above), P(child), info.nnum(d - 1), None)
+    torch.cuda.synchronize()
+    assert torch.equal(got, exp), d
+    checked += 1
+  assert checked >= 3
