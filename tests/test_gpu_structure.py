@@ -540,6 +540,42 @@ def test_update_degenerate_and_errors(oc, orc):
     F.octree_grow(o, 3, False)
 
 
+def test_update_in_place_and_with_the_clone_inside(oc, orc, samples):
+  """ocnn_octree_update (in place, on the caller's clone) and ocnn_octree_update_copy (the clone of
+  pytorch/cpp/octree_grow.cpp:165 inside the call, beside the scan) give the same blob, the oracle's,
+  for blobs whose child array starts at an odd word and for the case where nothing splits; the source
+  blob stays untouched; writing onto the source is refused."""
+  import ctypes as C
+  F = oc.nn
+  L = oc.lib.get()
+  P = lambda t: C.c_void_p(t.data_ptr())
+  rng = np.random.default_rng(7)
+  for name in ("octree_1", "octree_2", "octree_3"):
+    host = orc.octree_batch([samples[name]])
+    src = T(host).cuda()
+    info = F.octree_info(src)
+    for depth in (info.depth, info.depth - 1):
+      n = info.nnum(depth)
+      for labels in (rng.integers(0, 2, n).astype(np.int32), np.zeros(n, np.int32)):
+        exp = orc.octree_update(host, labels, depth, 1)
+        lab = T(labels).cuda()
+        got = F.octree_update(src, lab, depth, 1)                       # the copy form
+        assert np.array_equal(got.cpu().numpy(), exp), (name, depth)
+        assert np.array_equal(src.cpu().numpy(), host)
+        assert F.octree_info(got).nnum_nempty(depth) == max(int(labels.sum()), 1)
+        mine = src.clone()                                              # in place
+        raw = np.array(info.raw, copy=True)
+        sb = L.ocnn_octree_update_scratch_bytes(n)
+        ws = torch.empty(sb + 256, dtype=torch.uint8, device="cuda")
+        oc.lib.call("ocnn_octree_update", P(mine), C.c_void_p(raw.ctypes.data), P(lab), n, depth, 1, P(ws), C.c_size_t(sb), None)
+        torch.cuda.synchronize()
+        assert torch.equal(mine, got) and np.array_equal(raw[:716], exp[:716])
+  raw = np.array(info.raw, copy=True)
+  with pytest.raises(oc.lib.OcnnError) as e:
+    oc.lib.call("ocnn_octree_update_copy", P(src), P(src), C.c_void_p(raw.ctypes.data), P(lab), n, depth, 1, P(ws), C.c_size_t(sb), None)
+  assert e.value.code == -1
+
+
 def test_octree_beyond_the_format_limit_is_refused(oc, synthetic):
   """The serialized format addresses its payload with 32-bit offsets (octree_info.h: ptr_dis_),
   so an octree above 2 GiB cannot be represented: an error code, never a wrapped size."""
