@@ -1698,20 +1698,26 @@ __global__ __launch_bounds__(256, 3) void conv_s2_f32_kernel(ConvArgs a, float* 
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) b[cc][nt] = *reinterpret_cast<const float4*>(xbase[nt] + (int64_t)c * a.Hin);
   };
-  const int nstage = npass * nslab;
+  // my passes: blockIdx.y, + gridDim.y, ... (a level of few tiles deals its passes out over workgroups);
+  // stages are counted over those
+  const int my_passes = ((int)blockIdx.y < npass) ? (npass - (int)blockIdx.y + (int)gridDim.y - 1) / (int)gridDim.y : 0;
+  const int nstage = my_passes * nslab;
   float4 wr[kWVec];
-  auto fetch_w = [&](int stage) {
-    const float4* wsrc = reinterpret_cast<const float4*>(Wt + (int64_t)stage * kWWords);
+  auto fetch_w = [&](int stage) {   // stage of my own count -> (pass, slab) of the packed weights
+    const int at = ((int)blockIdx.y + (stage / nslab) * (int)gridDim.y) * nslab + stage % nslab;
+    const float4* wsrc = reinterpret_cast<const float4*>(Wt + (int64_t)at * kWWords);
 #pragma unroll
     for (int v = 0; v < kWVec; ++v) {
       int idx = v * 256 + threadIdx.x;
       wr[v] = idx < kWWords / 4 ? wsrc[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
     }
   };
+  if (my_passes == 0) return;
   fetch_w(0);
 #pragma unroll
   for (int cc = 0; cc < kS2Slab; ++cc) load_x(0, cc);
-  for (int pass = 0; pass < npass; ++pass) {
+  for (int mine = 0; mine < my_passes; ++mine) {
+    const int pass = (int)blockIdx.y + mine * (int)gridDim.y;
     floatx16 acc[MT][2];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -1720,7 +1726,7 @@ __global__ __launch_bounds__(256, 3) void conv_s2_f32_kernel(ConvArgs a, float* 
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
     for (int slab = 0; slab < nslab; ++slab) {
-      const int stage = pass * nslab + slab;
+      const int stage = mine * nslab + slab;
       __syncthreads();
 #pragma unroll
       for (int v = 0; v < kWVec; ++v) {
@@ -2061,7 +2067,10 @@ __global__ __launch_bounds__(256, 3) void deconv_s2_f32_kernel(ConvArgs a, float
   const int rows = a.M * 8;
   const int npass = (rows + 32 * kD2fMT - 1) / (32 * kD2fMT);
   const int nchunk = (a.Cin + kD2fChunk - 1) / kD2fChunk;
-  const int nstage = npass * nchunk;
+  // my passes: blockIdx.y, + gridDim.y, ... (a level of few tiles deals its passes out over workgroups)
+  const int my_passes = ((int)blockIdx.y < npass) ? (npass - (int)blockIdx.y + (int)gridDim.y - 1) / (int)gridDim.y : 0;
+  if (my_passes == 0) return;
+  const int nstage = my_passes * nchunk;
   int ncol[2];
   const float* xcol[2];
 #pragma unroll
@@ -2078,7 +2087,7 @@ __global__ __launch_bounds__(256, 3) void deconv_s2_f32_kernel(ConvArgs a, float
   };
   float4 wr[kWVec];
   auto fetch_w = [&](int stage) {
-    const int pass = stage / nchunk, chunk = stage % nchunk;
+    const int pass = (int)blockIdx.y + (stage / nchunk) * (int)gridDim.y, chunk = stage % nchunk;
 #pragma unroll
     for (int v = 0; v < kWVec; ++v) {
       const int idx = v * 256 + threadIdx.x;              // [channel][16 row quads]
@@ -2093,7 +2102,7 @@ __global__ __launch_bounds__(256, 3) void deconv_s2_f32_kernel(ConvArgs a, float
   fetch_w(0);
   floatx16 acc[kD2fMT][2];
   for (int stage = 0; stage < nstage; ++stage) {
-    const int pass = stage / nchunk, chunk = stage % nchunk;
+    const int pass = (int)blockIdx.y + (stage / nchunk) * (int)gridDim.y, chunk = stage % nchunk;
     if (chunk == 0) {
 #pragma unroll
       for (int mt = 0; mt < kD2fMT; ++mt)
@@ -2619,8 +2628,9 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
       const int nslab = (a.Cin + kS2Slab - 1) / kS2Slab;
       int64_t total = (int64_t)npass * nslab * kS2Slab * 4 * MT * 64;
       pack_weights_s2_f32<<<blocks_for(total), kBlock, 0, s>>>((float*)wsb, (const float*)weights, a.M, a.Cin, MT, npass, nslab);
-      if (MT == 1) conv_s2_f32_kernel<1><<<grid, 256, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
-      else conv_s2_f32_kernel<2><<<grid, 256, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
+      const dim3 g2(grid, pass_split(n_tiles, npass));
+      if (MT == 1) conv_s2_f32_kernel<1><<<g2, 256, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
+      else conv_s2_f32_kernel<2><<<g2, 256, 0, s>>>(a, (float*)top, (const float*)btm, (const float*)wsb, n_tiles);
     } else {
       const int nslab = (a.Cin + 7) / 8;
       int64_t total = (int64_t)npass * nslab * 4 * MT * 64 * 8;
@@ -2635,10 +2645,11 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     int d_tiles = (d.N + kTileCols - 1) / kTileCols;
     int d_grid = ((d_tiles + 7) / 8) * 8;
     if (dtype == OCNN_F32) {
+      const dim3 g2(d_grid, pass_split(d_tiles, (d.M * 8 + 32 * kD2fMT - 1) / (32 * kD2fMT)));
       if (d.Cin <= kD2fChunk / 2)
-        deconv_s2_f32_kernel<true><<<d_grid, 256, 0, s>>>(d, (float*)top, (const float*)btm, (const float*)weights, d_tiles);
+        deconv_s2_f32_kernel<true><<<g2, 256, 0, s>>>(d, (float*)top, (const float*)btm, (const float*)weights, d_tiles);
       else
-        deconv_s2_f32_kernel<false><<<d_grid, 256, 0, s>>>(d, (float*)top, (const float*)btm, (const float*)weights, d_tiles);
+        deconv_s2_f32_kernel<false><<<g2, 256, 0, s>>>(d, (float*)top, (const float*)btm, (const float*)weights, d_tiles);
     } else {
       const int cpad = (a.Cin + 15) / 16 * 16;
       const int rows = a.M * 8, npass = (rows + 32 * kD2MT - 1) / (32 * kD2MT), ksteps = cpad / 16;
