@@ -1798,7 +1798,7 @@ __global__ __launch_bounds__(256, 3) void conv_s2_bf16_kernel(ConvArgs a, uint16
     int n = n0 + nt * 32 + r;
     xoff[nt] = n < a.N ? (int64_t)n * 8 : -1;
   }
-  for (int pass = 0; pass < npass; ++pass) {
+  for (int pass = blockIdx.y; pass < npass; pass += gridDim.y) {   // passes may be dealt out over workgroups
     floatx16 acc[MT][2];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -2211,14 +2211,18 @@ __global__ __launch_bounds__(256, 2) void deconv_s2_bf16_reg_kernel(ConvArgs a, 
   for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) b[ks][nt].v4 = xt[(int64_t)min(ncol[nt], a.Hin) * (2 * KS) + 2 * ks + kh];
+  // passes may be dealt out over workgroups (blockIdx.y) where the level has few column tiles
+  const int pass0 = blockIdx.y, pstep = gridDim.y;
+  if (pass0 >= npass) return;
 #pragma unroll
-  for (int v = 0; v < kVec; ++v) wr[v] = Wt[v * 256 + threadIdx.x];
+  for (int v = 0; v < kVec; ++v) wr[v] = Wt[(int64_t)pass0 * kUnits + v * 256 + threadIdx.x];
 #pragma unroll
   for (int v = 0; v < kVec; ++v) sW[0][v * 256 + threadIdx.x] = wr[v];
-  for (int pass = 0; pass < npass; ++pass) {
+  int buf = 0;
+  for (int pass = pass0; pass < npass; pass += pstep, buf ^= 1) {
     __syncthreads();   // this pass's weights are in LDS; the other buffer is free
-    const uint4* wcur = sW[pass & 1];
-    const int nxt = min(pass + 1, npass - 1);
+    const uint4* wcur = sW[buf];
+    const int nxt = pass + pstep < npass ? pass + pstep : pass;
 #pragma unroll
     for (int v = 0; v < kVec; ++v) wr[v] = Wt[(int64_t)nxt * kUnits + v * 256 + threadIdx.x];
     floatx16 acc[kD2MT][2];
@@ -2238,7 +2242,7 @@ __global__ __launch_bounds__(256, 2) void deconv_s2_bf16_reg_kernel(ConvArgs a, 
         acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av.v, b[ks][1].v, acc[mt][1], 0, 0, 0);
       }
 #pragma unroll
-    for (int v = 0; v < kVec; ++v) sW[(pass + 1) & 1][v * 256 + threadIdx.x] = wr[v];
+    for (int v = 0; v < kVec; ++v) sW[buf ^ 1][v * 256 + threadIdx.x] = wr[v];
     if (n0 < a.N) {
       const int row_base = pass * 32 * kD2MT;
 #pragma unroll
@@ -2635,8 +2639,9 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
       const int nslab = (a.Cin + 7) / 8;
       int64_t total = (int64_t)npass * nslab * 4 * MT * 64 * 8;
       pack_weights_s2_bf16<<<blocks_for(total), kBlock, 0, s>>>((uint16_t*)wsb, (const uint16_t*)weights, a.M, a.Cin, MT, npass, nslab);
-      if (MT == 1) conv_s2_bf16_kernel<1><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const uint16_t*)btm, (const uint4*)wsb, n_tiles);
-      else conv_s2_bf16_kernel<2><<<grid, 256, 0, s>>>(a, (uint16_t*)top, (const uint16_t*)btm, (const uint4*)wsb, n_tiles);
+      const dim3 g2(grid, pass_split(n_tiles, npass));
+      if (MT == 1) conv_s2_bf16_kernel<1><<<g2, 256, 0, s>>>(a, (uint16_t*)top, (const uint16_t*)btm, (const uint4*)wsb, n_tiles);
+      else conv_s2_bf16_kernel<2><<<g2, 256, 0, s>>>(a, (uint16_t*)top, (const uint16_t*)btm, (const uint4*)wsb, n_tiles);
     }
   } else if (path == kPathS2Deconv) {
     // columns are the parents here: one column tile writes the 8 children of 256 parents
@@ -2658,14 +2663,17 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
       uint16_t* xt = reinterpret_cast<uint16_t*>(wsb + p.wt_bytes + p.ichild_bytes);
       dim3 tgrid((a.Hin + 1 + 127) / 128, (cpad + 63) / 64);
       transpose_rows_bf16_kernel<<<tgrid, 256, 0, s>>>(xt, (const uint16_t*)btm, a.Cin, a.Hin, cpad);
+      // (this kernel keeps its columns in registers for all passes and is bound by its stores: its
+      // passes are dealt out only where the tiles alone leave compute units empty)
+      const dim3 g2(d_grid, d_tiles < 256 ? pass_split(d_tiles, npass) : 1);
       if (ksteps == 1)
-        deconv_s2_bf16_reg_kernel<1><<<d_grid, 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles);
+        deconv_s2_bf16_reg_kernel<1><<<g2, 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles);
       else if (ksteps == 2)
-        deconv_s2_bf16_reg_kernel<2><<<d_grid, 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles);
+        deconv_s2_bf16_reg_kernel<2><<<g2, 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles);
       else if (ksteps == 4)
-        deconv_s2_bf16_reg_kernel<4><<<d_grid, 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles);
+        deconv_s2_bf16_reg_kernel<4><<<g2, 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles);
       else if (ksteps == 8)
-        deconv_s2_bf16_reg_kernel<8><<<d_grid, 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles);
+        deconv_s2_bf16_reg_kernel<8><<<g2, 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles);
       else
         deconv_s2_bf16_kernel<<<dim3(d_grid, pass_split(d_tiles, (d.M * 8 + 32 * kD2MT - 1) / (32 * kD2MT))), 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles, cpad / 8);
     }
