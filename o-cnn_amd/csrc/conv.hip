@@ -132,6 +132,20 @@ inline int pass_split(int n_tiles, int npass) {
   return best;
 }
 
+// For a kernel that keeps its input columns in registers over all passes (every further workgroup of
+// a tile reads them again): more workgroups a tile only where that takes a tenth or more off the
+// most loaded unit's work.
+inline int pass_split_costly(int n_tiles, int npass) {
+  constexpr int kUnits = 256;
+  auto load = [&](int split) {
+    return (((int64_t)n_tiles * split + kUnits - 1) / kUnits) * ((npass + split - 1) / split);
+  };
+  int best = 1;
+  for (int split = 2; split <= npass; ++split)
+    if (load(split) * 10 <= load(best) * 9) best = split;
+  return best;
+}
+
 // Wavefronts per workgroup (64 columns each) of a kernel whose wavefronts share nothing but a table:
 // a level of a few hundred 256-column tiles leaves some compute units with two workgroups and others
 // with one (363 tiles on 256 units: the launch lasts as long as two), and smaller workgroups spread
@@ -2650,7 +2664,7 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     int d_tiles = (d.N + kTileCols - 1) / kTileCols;
     int d_grid = ((d_tiles + 7) / 8) * 8;
     if (dtype == OCNN_F32) {
-      const dim3 g2(d_grid, pass_split(d_tiles, (d.M * 8 + 32 * kD2fMT - 1) / (32 * kD2fMT)));
+      const dim3 g2(d_grid, pass_split_costly(d_tiles, (d.M * 8 + 32 * kD2fMT - 1) / (32 * kD2fMT)));
       if (d.Cin <= kD2fChunk / 2)
         deconv_s2_f32_kernel<true><<<g2, 256, 0, s>>>(d, (float*)top, (const float*)btm, (const float*)weights, d_tiles);
       else
@@ -2663,9 +2677,8 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
       uint16_t* xt = reinterpret_cast<uint16_t*>(wsb + p.wt_bytes + p.ichild_bytes);
       dim3 tgrid((a.Hin + 1 + 127) / 128, (cpad + 63) / 64);
       transpose_rows_bf16_kernel<<<tgrid, 256, 0, s>>>(xt, (const uint16_t*)btm, a.Cin, a.Hin, cpad);
-      // (this kernel keeps its columns in registers for all passes and is bound by its stores: its
-      // passes are dealt out only where the tiles alone leave compute units empty)
-      const dim3 g2(d_grid, d_tiles < 256 ? pass_split(d_tiles, npass) : 1);
+      // (bound by its stores: dealt out only where the tiles alone leave compute units empty)
+      const dim3 g2(d_grid, d_tiles < 256 ? pass_split_costly(d_tiles, npass) : 1);
       if (ksteps == 1)
         deconv_s2_bf16_reg_kernel<1><<<g2, 256, 0, s>>>(d, (uint16_t*)top, (const uint4*)xt, (const uint4*)wsb, d_tiles);
       else if (ksteps == 2)
