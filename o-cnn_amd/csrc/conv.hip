@@ -2054,6 +2054,24 @@ __device__ inline void store_children_bf16(const ConvArgs& a, uint16_t* __restri
   }
 }
 
+// Over the non-empty nodes the row of a child is its rank among the non-empty nodes of the finer
+// level (a.child: that level's child links); an empty child has no row and is not stored.
+__device__ inline void store_children_nempty_f32(const ConvArgs& a, float* __restrict__ out, const floatx16& acc,
+    int row0, int n, int kh) {
+  if (n >= a.N) return;
+  int link[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) link[j] = a.child[(int64_t)n * 8 + 4 * kh + j];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int co = (row0 >> 3) + q;
+    if (co >= a.M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (link[j] >= 0 && link[j] < a.Hout) out[(int64_t)co * a.Hout + link[j]] = finish(a, acc[4 * q + j], co);
+  }
+}
+
 constexpr int kD2MT = 4;  // row tiles per pass: 128 rows = 16 output channels x 8 children
 
 // fp32: a wavefront keeps its 64 columns x 64 input channels in registers (read once, coalesced,
@@ -2067,7 +2085,9 @@ constexpr int kD2fChunk = 64;
 // HALF: a layer of 32 input channels or fewer fills the first half of its one chunk only, and the
 // k-steps of the other half (zero weights) are left out at compile time (a test inside the loop
 // costs the schedule of every k-step).
-template <bool HALF>
+// NE: over the non-empty nodes (the columns are the non-empty parents either way; a child goes to
+// its rank among the non-empty nodes of the finer level or nowhere).
+template <bool HALF, bool NE = false>
 __global__ __launch_bounds__(256, 3) void deconv_s2_f32_kernel(ConvArgs a, float* __restrict__ out,
     const float* __restrict__ in, const float* __restrict__ W, int n_tiles) {
   constexpr int kSteps = HALF ? kD2fChunk / 4 : kD2fChunk / 2;   // k-steps (channel pairs) of a stage
@@ -2148,7 +2168,10 @@ __global__ __launch_bounds__(256, 3) void deconv_s2_f32_kernel(ConvArgs a, float
 #pragma unroll
       for (int mt = 0; mt < kD2fMT; ++mt)
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) store_children<float>(a, out, acc[mt][nt], row_base + mt * 32, ncol[nt], kh);
+        for (int nt = 0; nt < 2; ++nt) {
+          if constexpr (NE) store_children_nempty_f32(a, out, acc[mt][nt], row_base + mt * 32, ncol[nt], kh);
+          else store_children<float>(a, out, acc[mt][nt], row_base + mt * 32, ncol[nt], kh);
+        }
     }
   }
 }
@@ -2612,8 +2635,10 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
       (reinterpret_cast<uintptr_t>(btm) & 15) == 0) {
     path = kPathS2Conv;
     copies_input = false;
-  } else if (a.mode == kModeS2Deconv && !a.nempty && (reinterpret_cast<uintptr_t>(top) & 15) == 0 &&
-             (dtype != OCNN_F32 || (reinterpret_cast<uintptr_t>(weights) & 15) == 0)) {
+  } else if (a.mode == kModeS2Deconv && (!a.nempty || dtype == OCNN_F32) && (reinterpret_cast<uintptr_t>(top) & 15) == 0 &&
+             (dtype != OCNN_F32 || (reinterpret_cast<uintptr_t>(weights) & 15) == 0) &&
+             (!a.nempty || o->nnum[p.top_depth] == 8 * a.Hin)) {
+    // (fp32 also over the non-empty nodes: the same columns, the children stored by rank)
     path = kPathS2Deconv;
     copies_input = dtype != OCNN_F32;
   } else if (dtype == OCNN_F32 && a.mode == kModeS1 && !a.nempty && a.K == 27 &&
@@ -2633,7 +2658,7 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
         "this call needs %zu bytes of scratch memory, the built-in array holds %zu: "
         "use ocnn_octree_conv_fused with a workspace of your own", used, ws_bytes);
   }
-  if (nempty && path != kPathOneTapF32) {
+  if (nempty && path != kPathOneTapF32 && path != kPathS2Deconv) {
     int* ichild = reinterpret_cast<int*>(wsb + p.wt_bytes);
     ichild_kernel<<<blocks_for(p.child_h), kBlock, 0, s>>>(ichild, p.ichild_h, a.child, p.child_h);
     OCNN_LAUNCH_OK("ichild");
@@ -2665,7 +2690,11 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     int d_grid = ((d_tiles + 7) / 8) * 8;
     if (dtype == OCNN_F32) {
       const dim3 g2(d_grid, pass_split_costly(d_tiles, (d.M * 8 + 32 * kD2fMT - 1) / (32 * kD2fMT)));
-      if (d.Cin <= kD2fChunk / 2)
+      if (d.nempty && d.Cin <= kD2fChunk / 2)
+        deconv_s2_f32_kernel<true, true><<<g2, 256, 0, s>>>(d, (float*)top, (const float*)btm, (const float*)weights, d_tiles);
+      else if (d.nempty)
+        deconv_s2_f32_kernel<false, true><<<g2, 256, 0, s>>>(d, (float*)top, (const float*)btm, (const float*)weights, d_tiles);
+      else if (d.Cin <= kD2fChunk / 2)
         deconv_s2_f32_kernel<true><<<g2, 256, 0, s>>>(d, (float*)top, (const float*)btm, (const float*)weights, d_tiles);
       else
         deconv_s2_f32_kernel<false><<<g2, 256, 0, s>>>(d, (float*)top, (const float*)btm, (const float*)weights, d_tiles);
