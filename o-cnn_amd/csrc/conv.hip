@@ -1213,9 +1213,13 @@ __global__ __launch_bounds__(256) void transpose_channels_bf16_kernel(uint16_t* 
   }
 }
 
-template <int MT>
+// ROWS_OUT: the output is written row-major as well ([Hout + 1][out_pitch] bf16, row Hout zero); the
+// input rows may be a slice of a wider tensor (pitch8: 16-byte units a row).
+template <int MT, bool ROWS_OUT = false>
 __global__ __launch_bounds__(256, 2) void conv_s1_bf16_lds_kernel(ConvArgs a, uint16_t* __restrict__ out,
-    const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles, int cpad8) {
+    const u32x4* __restrict__ xt, const u32x4* __restrict__ Wt, int n_tiles, int cpad8, int pitch8 = 0,
+    int out_pitch = 0, int out_cpad = 0) {
+  if (pitch8 == 0) pitch8 = cpad8;
   constexpr int kWUnits = 9 * MT * 64;               // 16-byte units per weight chunk
   constexpr int kWVec = (kWUnits + 255) / 256;
   __shared__ u32x4 sX[2 * kB16Half];
@@ -1285,7 +1289,7 @@ __global__ __launch_bounds__(256, 2) void conv_s1_bf16_lds_kernel(ConvArgs a, ui
     do {                                                                                       \
       const int col = (SLAB) * 2 + s_kh;                                                       \
       _Pragma("unroll") for (int j = 0; j < 4; ++j)                                            \
-        xr[(L) & 1][j] = xt[(int64_t)nb[j][L] * cpad8 + col];                                  \
+        xr[(L) & 1][j] = xt[(int64_t)nb[j][L] * pitch8 + col];                                 \
     } while (0)
 #define OCNN_PHASE(SLAB, L)                                                                    \
     do {                                                                                       \
@@ -1333,7 +1337,13 @@ __global__ __launch_bounds__(256, 2) void conv_s1_bf16_lds_kernel(ConvArgs a, ui
 #undef OCNN_FETCH_W
 #undef OCNN_FETCH_X
 #undef OCNN_PHASE
-    if (n0 < a.N) store_tiles<uint16_t, MT>(a, out, acc, pass * MT, n0, lane);
+    if constexpr (ROWS_OUT) {
+      rows_out_tiles<MT>(a, out, out_pitch, out_cpad, acc, pass * MT * 32, n0, lane);
+      if (tile == 0 && wave == 0 && lane * 8 >= pass * MT * 32 && lane * 8 < min((pass + 1) * MT * 32, out_cpad))
+        *reinterpret_cast<uint4*>(out + (int64_t)a.Hout * out_pitch + lane * 8) = make_uint4(0, 0, 0, 0);
+    } else {
+      if (n0 < a.N) store_tiles<uint16_t, MT>(a, out, acc, pass * MT, n0, lane);
+    }
   }
 }
 
@@ -3989,6 +3999,22 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
     a.neigh = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_NEIGH, depth));
     a.child = reinterpret_cast<const int*>(blob + o->ptr_dis(OCNN_CHILD, depth));
     const int r_tiles = ((a.N >> 3) + kRegTileGroups - 1) / kRegTileGroups;
+    if (r_tiles * pass_split(r_tiles, r.npass) < 128 && g_bf16_reg_min_tiles.load(std::memory_order_relaxed) > 1) {
+      // a level that gives the 1024-column workgroups of the register-fed kernel fewer than 128
+      // (tiles x passes): the LDS kernel's 256-column workgroups, three a compute unit, fill the
+      // device better (same weights, same products in the same order).  Measured: 12 824 columns,
+      // 128 -> 256: 73 -> 48 us; 44 512 columns, 256 -> 256 (176 workgroups): 152 us against 163.
+      const int n_tiles = (a.N + kTileCols - 1) / kTileCols;
+      const dim3 lgrid(((n_tiles + 7) / 8) * 8, pass_split(n_tiles, r.npass));
+      if (r.MT == 1)
+        conv_s1_bf16_lds_kernel<1, true><<<lgrid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
+            (const u32x4*)wpk, n_tiles, r.cpad / 8, btm_pitch / 8, top_pitch, r.out_cpad);
+      else
+        conv_s1_bf16_lds_kernel<2, true><<<lgrid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
+            (const u32x4*)wpk, n_tiles, r.cpad / 8, btm_pitch / 8, top_pitch, r.out_cpad);
+      OCNN_LAUNCH_OK("octree_conv_rows");
+      return OCNN_OK;
+    }
     const dim3 grid(((r_tiles + 7) / 8) * 8, pass_split(r_tiles, r.npass));
     if (r.MT == 1)
       conv_s1_bf16_reg_kernel<1, true><<<grid, 256, 0, s>>>(a, (uint16_t*)top_rows, (const u32x4*)btm_rows,
