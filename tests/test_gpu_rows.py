@@ -418,3 +418,36 @@ def test_row_kernel_workgroup_sizes_at_scene_levels(oc, synthetic):
       assert float(results[0].float().abs().max()) > 0
   finally:
     L.ocnn_conv_rows_direct(1)
+
+
+def test_rows_small_levels_take_either_kernel(oc, octree):
+  """Row-major 3x3x3 over all nodes: a small level runs the LDS kernel with a row-major store, a
+  large one the register-fed kernel; forced onto the register-fed kernel (the test hook of the tile
+  threshold) the small level gives the same bits, with and without bias + ReLU, conv and deconv,
+  also into a channel slice of a wider tensor, and they are the channel-major operator's."""
+  F = oc.nn
+  L = oc.lib.get()
+  info = F.octree_info(octree)
+  g = torch.Generator().manual_seed(23)
+  try:
+    for depth, cin, cout, deconv in ((6, 32, 64, False), (5, 48, 130, False), (6, 16, 32, True), (4, 128, 256, False)):
+      H = info.nnum(depth)
+      x = torch.randn(1, cin, H, 1, generator=g).bfloat16().cuda()
+      xr = F.to_rows(x)
+      shape = (cin, cout * 27) if deconv else (cout, cin * 27)
+      w = (torch.randn(*shape, generator=g) * 0.05).bfloat16().cuda()
+      b = (torch.randn(cout, generator=g) * 0.1).cuda()
+      res = []
+      for thr in (0, -1):
+        L.ocnn_conv_bf16_tile_threshold(thr)
+        res.append(F.octree_conv_rows(xr, cin, w, octree, depth, cout, bias=b, relu=True, deconv=deconv))
+        res.append(F.octree_conv_rows(xr, cin, w, octree, depth, cout, deconv=deconv))
+        wide = torch.full((H + 1, F.rows_pitch(cout) + 32), 7.0, dtype=torch.bfloat16, device="cuda")
+        F.octree_conv_rows(xr, cin, w, octree, depth, cout, bias=b, relu=True, deconv=deconv, out=wide[:, 16:16 + F.rows_pitch(cout)])
+        assert torch.equal(wide[:, 16:16 + F.rows_pitch(cout)], res[-2]) and bool((wide[:, :16] == 7).all()) and bool((wide[:, 16 + F.rows_pitch(cout):] == 7).all())
+      assert torch.equal(res[0], res[2]) and torch.equal(res[1], res[3]), (depth, cin, cout, deconv)
+      ref = F.octree_conv_fused(x, w, b, True, octree, depth, cout, [3, 3, 3], 1, False, deconv=deconv)
+      assert torch.equal(F.from_rows(res[0], cout), ref), (depth, cin, cout, deconv)
+      assert bool((res[0][H] == 0).all()) and bool((res[0][:, cout:] == 0).all())
+  finally:
+    L.ocnn_conv_bf16_tile_threshold(0)
