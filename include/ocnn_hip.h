@@ -220,7 +220,7 @@ int ocnn_octree_conv_fused(void* top, const void* btm, int channel_in, int btm_h
  *       octree_pad that the reference's modules put behind the operator
  *       (pytorch/ocnn/octree_conv.py:102-127) is folded in, an empty node receives the bias alone;
  *     kernel 2x2x2 stride 2, deconv: rows of ALL nodes of `depth` in (the octree_depad of those
- *       modules is folded in), rows of depth+1 out; input channels padded to 16 .. 256;
+ *       modules is folded in), rows of depth+1 out; at most 256 input channels;
  *   with nempty 1 (rows = ranks of the non-empty nodes on both sides, the operator of the
  *   channel-major entry points, pytorch/cpp/octree_conv.cpp:131-216): kernel 3x3x3 stride 1 and
  *   kernel 2x2x2 stride 2, conv and deconv;

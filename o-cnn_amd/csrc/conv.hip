@@ -2333,8 +2333,9 @@ template <int KS, int MT2, bool NE = false>
 __global__ __launch_bounds__(256) void deconv_s2_rows_bf16_kernel(ConvArgs a, uint16_t* __restrict__ out,
     int out_pitch, int out_cpad, const u32x4* __restrict__ xt, int in_pitch, const u32x4* __restrict__ Wt, int n_tiles) {
   constexpr int kUnits = KS * MT2 * 64;
-  constexpr int kVec = kUnits / 256;
-  __shared__ u32x4 sW[2][kUnits];
+  constexpr int kVec = (kUnits + 255) / 256;          // (an odd KS above four leaves the last round half used)
+  constexpr bool kWhole = kUnits % 256 == 0;
+  __shared__ u32x4 sW[2][kVec * 256];
   __shared__ int sRow[NE ? kTileCols * 8 : 1];        // NE: byte offset of the output row of (column, child)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int tile = xcd_tile(blockIdx.x, n_tiles);
@@ -2372,7 +2373,8 @@ __global__ __launch_bounds__(256) void deconv_s2_rows_bf16_kernel(ConvArgs a, ui
   const int pass0 = blockIdx.y, pstep = gridDim.y;
   if (pass0 >= npass) return;
 #pragma unroll
-  for (int v = 0; v < kVec; ++v) wr[v] = Wt[(int64_t)pass0 * kUnits + v * 256 + threadIdx.x];
+  for (int v = 0; v < kVec; ++v)
+    wr[v] = Wt[(int64_t)pass0 * kUnits + (kWhole ? v * 256 + (int)threadIdx.x : min(v * 256 + (int)threadIdx.x, kUnits - 1))];
 #pragma unroll
   for (int v = 0; v < kVec; ++v) sW[0][v * 256 + threadIdx.x] = wr[v];
   const float floor = a.relu ? 0.0f : -__builtin_inff();
@@ -2382,7 +2384,8 @@ __global__ __launch_bounds__(256) void deconv_s2_rows_bf16_kernel(ConvArgs a, ui
     const u32x4* wcur = sW[buf];
     const int nxt = pass + pstep < npass ? pass + pstep : pass;
 #pragma unroll
-    for (int v = 0; v < kVec; ++v) wr[v] = Wt[(int64_t)nxt * kUnits + v * 256 + threadIdx.x];
+    for (int v = 0; v < kVec; ++v)
+      wr[v] = Wt[(int64_t)nxt * kUnits + (kWhole ? v * 256 + (int)threadIdx.x : min(v * 256 + (int)threadIdx.x, kUnits - 1))];
     floatx16 acc[MT2][2];
 #pragma unroll
     for (int mt = 0; mt < MT2; ++mt)
@@ -3738,8 +3741,7 @@ int make_rows_plan(const Info* o, int depth, int channel_in, int num_output, con
   r->slab_ch = kRowSlab;
   r->staged = false;
   const int mtiles = (num_output + 31) / 32;
-  if (nempty && stride == 2 && k222 && deconv && depth < o->depth &&
-      (r->ksteps == 1 || r->ksteps == 2 || r->ksteps == 4 || r->ksteps == 8 || r->ksteps == 16) &&
+  if (nempty && stride == 2 && k222 && deconv && depth < o->depth && r->ksteps >= 1 && r->ksteps <= 16 &&
       (int64_t)o->nnum_nempty[depth + 1] * 5 >= (int64_t)o->nnum[depth + 1] * 2) {
     // 2x2x2 stride-2 deconvolution over the non-empty nodes: the all-nodes kernel with the rows of
     // the input as its columns and the child links of the finer level as the map of its output rows.
@@ -3804,8 +3806,8 @@ int make_rows_plan(const Info* o, int depth, int channel_in, int num_output, con
     r->wt_bytes = align256((size_t)r->npass * 8 * r->ksteps * r->MT * 64 * 16);
   } else if (stride == 2 && k222 && deconv) {
     OCNN_REQUIRE(depth < o->depth, OCNN_E_BADARG, "output depth %d outside the octree", depth + 1);
-    OCNN_REQUIRE(r->ksteps == 1 || r->ksteps == 2 || r->ksteps == 4 || r->ksteps == 8 || r->ksteps == 16,
-        OCNN_E_UNSUPPORTED, "row-major stride-2 deconvolution: input channels padded to 16, 32, 64, 128 or 256");
+    OCNN_REQUIRE(r->ksteps >= 1 && r->ksteps <= 16, OCNN_E_UNSUPPORTED,
+        "row-major stride-2 deconvolution: at most 256 input channels");
     r->kind = 2;
     r->btm_h = o->nnum[depth];
     r->cols = o->nnum_nempty[depth];
@@ -4057,8 +4059,19 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
     switch (r.ksteps) {
       case 1: OCNN_D2_ROWS_NE(1, 4); break;
       case 2: OCNN_D2_ROWS_NE(2, 4); break;
+      case 3: OCNN_D2_ROWS_NE(3, 4); break;
       case 4: OCNN_D2_ROWS_NE(4, 4); break;
+      case 5: OCNN_D2_ROWS_NE(5, 2); break;
+      case 6: OCNN_D2_ROWS_NE(6, 2); break;
+      case 7: OCNN_D2_ROWS_NE(7, 2); break;
       case 8: OCNN_D2_ROWS_NE(8, 2); break;
+      case 9: OCNN_D2_ROWS_NE(9, 2); break;
+      case 10: OCNN_D2_ROWS_NE(10, 2); break;
+      case 11: OCNN_D2_ROWS_NE(11, 2); break;
+      case 12: OCNN_D2_ROWS_NE(12, 2); break;
+      case 13: OCNN_D2_ROWS_NE(13, 2); break;
+      case 14: OCNN_D2_ROWS_NE(14, 2); break;
+      case 15: OCNN_D2_ROWS_NE(15, 2); break;
       default: OCNN_D2_ROWS_NE(16, 2); break;
     }
 #undef OCNN_D2_ROWS_NE
@@ -4081,8 +4094,19 @@ int run_conv_rows(int deconv, void* top_rows, int top_pitch, const void* btm_row
     switch (r.ksteps) {
       case 1: OCNN_D2_ROWS(1, 4); break;
       case 2: OCNN_D2_ROWS(2, 4); break;
+      case 3: OCNN_D2_ROWS(3, 4); break;
       case 4: OCNN_D2_ROWS(4, 4); break;
+      case 5: OCNN_D2_ROWS(5, 2); break;
+      case 6: OCNN_D2_ROWS(6, 2); break;
+      case 7: OCNN_D2_ROWS(7, 2); break;
       case 8: OCNN_D2_ROWS(8, 2); break;
+      case 9: OCNN_D2_ROWS(9, 2); break;
+      case 10: OCNN_D2_ROWS(10, 2); break;
+      case 11: OCNN_D2_ROWS(11, 2); break;
+      case 12: OCNN_D2_ROWS(12, 2); break;
+      case 13: OCNN_D2_ROWS(13, 2); break;
+      case 14: OCNN_D2_ROWS(14, 2); break;
+      case 15: OCNN_D2_ROWS(15, 2); break;
       default: OCNN_D2_ROWS(16, 2); break;
     }
 #undef OCNN_D2_ROWS

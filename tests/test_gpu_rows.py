@@ -107,7 +107,7 @@ def small(oc, orc, synthetic):
   return host, T(host).cuda(), OctreeBlob(host)
 
 
-@pytest.mark.parametrize("cin,cout", [(16, 32), (32, 64), (24, 40), (128, 256), (64, 16)])
+@pytest.mark.parametrize("cin,cout", [(16, 32), (32, 64), (24, 40), (128, 256), (64, 16), (48, 64), (80, 32), (160, 24)])
 def test_stride2_rows_against_oracle(oc, orc, small, cin, cout):
   """2x2x2 stride 2 with the pad / depad of the reference's modules folded in
   (pytorch/ocnn/octree_conv.py:102-127), bias and ReLU fused: 2e-2 against the oracle in fp32 on
@@ -208,7 +208,7 @@ def test_rows_operators_full_size(oc, synthetic):
   close(F.from_rows(up, 32).float().cpu().numpy().reshape(32, -1), up_ref.float().cpu().numpy().reshape(32, -1), 2e-2, "up")
 
 
-@pytest.mark.parametrize("cin,cout", [(3, 32), (64, 64), (24, 40), (48, 128), (128, 256)])
+@pytest.mark.parametrize("cin,cout", [(3, 32), (64, 64), (24, 40), (48, 128), (128, 256), (80, 32), (176, 48)])
 def test_nonempty_rows_equal_channel_major(oc, octree, cin, cout):
   """over the non-empty nodes the row-major operators run the kernel of the channel-major entry
   points on the same operands in the same order: equal bits, for 3x3x3 stride 1 and for 2x2x2
