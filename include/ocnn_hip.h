@@ -206,6 +206,18 @@ int ocnn_octree_conv_fused(void* top, const void* btm, int channel_in, int btm_h
     int num_output, const int* kernel_size, int stride, int nempty, int dtype, void* workspace_dev,
     size_t workspace_bytes, ocnn_stream_t stream);
 
+/* Two 1x1x1 convolutions in one pass: hidden = W1 data + b1 (ReLU when relu1 != 0), out = W2 hidden
+ * + b2, label (may be NULL) = argmax over the channels of out (the first of equal maxima).  It is
+ * the prediction head of the reference's decoders, OctreeConv1x1BnRelu(C, 32) -> OctreeConv1x1(32, n)
+ * (pytorch/ocnn/ounet.py:46-49, modules.py:71-107; with `logit.argmax(1)`, ounet.py:82-88 and
+ * 114-119), with the BatchNorm folded into w1 / b1; the reference runs it as two torch Conv1d.
+ * fp32, channel-major: data [channel_in, height], w1 [hidden, channel_in], w2 [num_output, hidden],
+ * out [num_output, height], label int32 [height]; b1 / b2 may be NULL; hidden <= 32 and
+ * num_output <= 8, else OCNN_E_UNSUPPORTED (run two ocnn_octree_conv_fused then).  The hidden
+ * channels are not written anywhere. */
+int ocnn_conv1x1_pair(float* out, int* label, const float* data, int channel_in, int height, const float* w1,
+    const float* b1, int hidden, int relu1, const float* w2, const float* b2, int num_output, ocnn_stream_t stream);
+
 /* Row-major activations, no counterpart in the reference (whose tensors are channel-major
  * [1, C, H, 1]): rows [H + 1][pitch] bf16, row h = the channels of node h, pitch = channels
  * rounded up to a multiple of 16, padding channels zero, row H all zero (what a missing
@@ -360,6 +372,10 @@ int ocnn_octree_deconv_grad(void* grad_data, void* grad_weights, const void* dat
  * ignored and overwritten): idx is inverted there and every row of top is written once, its
  * source row or zero, instead of twice.  Where two rows of btm name one row of top (keys of an
  * octree never do) one of them wins, as in the scatter.
+ * ocnn_align_forward_add: top[c, idx[h]] += btm[c, h] for idx[h] != -1, the rows of top that
+ * nothing is moved to keep their values: `deconv + octree_align(skip, ...)` of the decoder loop
+ * (pytorch/ocnn/ounet.py:109-111) in one pass over the two tensors.  Two rows of btm must not
+ * name one row of top (keys of an octree never do).
  * ocnn_octree_interp: octree_nearest_pts (method 0) / octree_trilinear_pts (method 1) of
  * pytorch/ocnn/modules.py:209-275 in two kernels.  key[n_key]: the sorted Morton keys of the
  * searched depth (de-padded by the caller for nempty, as octree_search_key does,
@@ -367,6 +383,8 @@ int ocnn_octree_deconv_grad(void* grad_data, void* grad_weights, const void* dat
  * out [channel, n_pts].  idx / weight [n_pts * K] (K = 1 nearest, 8 linear) are filled for the
  * backward call, which zero-fills grad_data [channel, H] and scatters with fp32 atomics. */
 int ocnn_align_forward(float* top, int top_h, int channel, const float* btm, int btm_h, const int* idx,
+    ocnn_stream_t stream);
+int ocnn_align_forward_add(float* top, int top_h, int channel, const float* btm, int btm_h, const int* idx,
     ocnn_stream_t stream);
 int ocnn_align_forward_ws(float* top, int top_h, int channel, const float* btm, int btm_h, const int* idx,
     int* inverse_ws, ocnn_stream_t stream);

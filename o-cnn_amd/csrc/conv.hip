@@ -278,6 +278,95 @@ __global__ __launch_bounds__(256) void conv_one_tap_f32_kernel(ConvArgs a, float
   }
 }
 
+// ---- two 1x1x1 convolutions in a row (a prediction head) ----------------------------------------
+// hidden = relu(W1 x + b1) (at most 32 channels: one accumulator tile per 32 columns), out = W2 hidden
+// + b2 (at most kPairMaxOut channels), optionally label = argmax over the channels of out.  The
+// first product is the kernel above; the hidden channels never leave the registers: a lane holds
+// 16 of the 32 hidden values of its column, multiplies them with the matching 16 weights of every
+// output channel and adds the other half from its partner lane.  Bound by the bytes of x.
+constexpr int kPairMaxOut = 8;
+__global__ __launch_bounds__(256) void conv_one_tap_pair_f32_kernel(float* __restrict__ out, int* __restrict__ label,
+    const float* __restrict__ in, const float* __restrict__ W1, const float* __restrict__ b1,
+    const float* __restrict__ W2, const float* __restrict__ b2, int C, int H, int hidden, int relu1, int M2,
+    int n_tiles) {
+  __shared__ float sW[(kOneTapChunk / 2) * 64];
+  __shared__ float sW2[kPairMaxOut][32];
+  __shared__ float sB1[32];
+  __shared__ float sB2[kPairMaxOut];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = xcd_tile(blockIdx.x, n_tiles);
+  if (tile >= n_tiles) return;
+  const int n0 = tile * kTileCols + wave * kWaveCols;
+  const int r = lane & 31, kh = lane >> 5;
+  const float* x0 = in + min(n0 + r, H - 1);
+  const float* x1 = in + min(n0 + 32 + r, H - 1);
+  {  // (read behind the first barrier of the chunk loop)
+    const int j = threadIdx.x >> 5, m = threadIdx.x & 31;
+    sW2[j][m] = (j < M2 && m < hidden) ? W2[j * hidden + m] : 0.0f;
+    if (threadIdx.x < 32) sB1[threadIdx.x] = (b1 && (int)threadIdx.x < hidden) ? b1[threadIdx.x] : 0.0f;
+    if (threadIdx.x < kPairMaxOut) sB2[threadIdx.x] = (b2 && (int)threadIdx.x < M2) ? b2[threadIdx.x] : 0.0f;
+  }
+  floatx16 acc[2];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[nt][i] = 0.0f;
+  for (int c0 = 0; c0 < C; c0 += kOneTapChunk) {
+    const int nks = (min(kOneTapChunk, C - c0) + 1) >> 1;
+    __syncthreads();   // the previous chunk's fragments are no longer read
+    for (int e = threadIdx.x; e < nks * 64; e += 256) {
+      const int l = e & 63, ks = e >> 6;
+      const int m = l & 31, c = c0 + 2 * ks + (l >> 5);
+      sW[e] = (m < hidden && c < C) ? W1[(int64_t)m * C + c] : 0.0f;
+    }
+    __syncthreads();
+    constexpr int kAhead = 8;   // k-steps whose operands are requested together
+    for (int k0 = 0; k0 < nks; k0 += kAhead) {
+      float v0[kAhead], v1[kAhead];
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u) {
+        const int c = c0 + 2 * (k0 + u) + kh;
+        const int64_t row = (int64_t)min(c, C - 1) * H;
+        v0[u] = x0[row];
+        v1[u] = x1[row];
+        if (c >= C || k0 + u >= nks) { v0[u] = 0.0f; v1[u] = 0.0f; }
+      }
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u) {
+        if (k0 + u >= nks) break;   // uniform
+        const float av = sW[(k0 + u) * 64 + lane];
+        acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, v0[u], acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, v1[u], acc[1], 0, 0, 0);
+      }
+    }
+  }
+  const float floor = relu1 ? 0.0f : -__builtin_inff();
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+    const int col = n0 + nt * 32 + r;
+    float hval[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int m = 8 * (i / 4) + 4 * kh + (i % 4);   // the hidden channel of accumulator element i
+      hval[i] = fmaxf(acc[nt][i] + sB1[m], floor);
+    }
+    float best = 0.0f;
+    int arg = 0;
+#pragma unroll
+    for (int j = 0; j < kPairMaxOut; ++j) {
+      if (j >= M2) break;   // uniform
+      float p = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) p += sW2[j][8 * (i / 4) + 4 * kh + (i % 4)] * hval[i];
+      p += __shfl_xor(p, 32, 64);
+      p += sB2[j];
+      if (col < H && kh == (j & 1)) out[(int64_t)j * H + col] = p;
+      if (j == 0 || p > best) { best = p; arg = j; }   // the first of equal maxima, as torch.argmax
+    }
+    if (label && kh == 0 && col < H) label[col] = arg;
+  }
+}
+
 // ---- general gather kernel over a row-major copy of the input -------------------------------
 // Every case without a dedicated kernel (non-empty-node convolutions, the small kernel shapes,
 // stride-2 cases other than 2x2x2 over all nodes) runs here.  The input is first copied
@@ -4170,6 +4259,20 @@ int ocnn_octree_deconv(void* top, const void* btm, int channel_in, int btm_h, co
     int nempty, int dtype, void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream) {
   return run_conv(1, top, btm, channel_in, btm_h, weights, octree_dev, info, depth, num_output, kernel_size,
       stride, nempty, dtype, workspace_dev, workspace_bytes, as_stream(stream));
+}
+
+int ocnn_conv1x1_pair(float* out, int* label, const float* data, int channel_in, int height, const float* w1,
+    const float* b1, int hidden, int relu1, const float* w2, const float* b2, int num_output, ocnn_stream_t stream) {
+  OCNN_REQUIRE(out && data && w1 && w2, OCNN_E_BADARG, "null pointer");
+  OCNN_REQUIRE(channel_in > 0 && height >= 0 && hidden > 0 && num_output > 0, OCNN_E_BADARG, "bad argument");
+  OCNN_REQUIRE(hidden <= 32 && num_output <= kPairMaxOut, OCNN_E_UNSUPPORTED,
+      "two 1x1x1 convolutions in one pass: at most 32 hidden and %d output channels", kPairMaxOut);
+  if (height == 0) return OCNN_OK;
+  const int n_tiles = (height + kTileCols - 1) / kTileCols;
+  conv_one_tap_pair_f32_kernel<<<((n_tiles + 7) / 8) * 8, 256, 0, as_stream(stream)>>>(out, label, data, w1, b1, w2, b2,
+      channel_in, height, hidden, relu1, num_output, n_tiles);
+  OCNN_LAUNCH_OK("conv1x1_pair");
+  return OCNN_OK;
 }
 
 int ocnn_octree_conv_fused(void* top, const void* btm, int channel_in, int btm_h, const void* weights,

@@ -41,6 +41,27 @@ __global__ void align_backward_kernel(const float* __restrict__ top, int top_h, 
   for (int i = 0; i < kAlignChunk; ++i)
     if (c0 + i < channel) btm[(int64_t)(c0 + i) * btm_h + h] = ok ? v[i] : 0.0f;
 }
+// top[c][index[h]] += btm[c][h] where the index names a row: the transfer and the sum behind it
+// (a skip connection) in one pass.  The rows of top that nothing is moved to are not touched.
+__global__ void align_add_kernel(float* __restrict__ top, int top_h, const float* __restrict__ btm, int btm_h,
+    const int* __restrict__ index, int channel) {
+  const int h = blockIdx.x * kBlock + threadIdx.x;
+  if (h >= btm_h) return;
+  const int c0 = blockIdx.y * kAlignChunk;
+  const int j = index[h];
+  const bool ok = j >= 0 && j < top_h;
+  const int to = ok ? j : 0;
+  float v[kAlignChunk], t[kAlignChunk];
+#pragma unroll
+  for (int i = 0; i < kAlignChunk; ++i) {
+    const bool live = c0 + i < channel;
+    v[i] = live ? btm[(int64_t)(c0 + i) * btm_h + h] : 0.0f;
+    t[i] = live ? top[(int64_t)(c0 + i) * top_h + to] : 0.0f;
+  }
+#pragma unroll
+  for (int i = 0; i < kAlignChunk; ++i)
+    if (ok && c0 + i < channel) top[(int64_t)(c0 + i) * top_h + to] = t[i] + v[i];
+}
 __global__ void fill_i32_kernel(int* __restrict__ p, int n, int v) {
   const int i = blockIdx.x * kBlock + threadIdx.x;
   if (i < n) p[i] = v;
@@ -419,6 +440,16 @@ int ocnn_align_forward_ws(float* top, int top_h, int channel, const float* btm, 
   align_backward_kernel<<<dim3(blocks_for(top_h), (channel + kAlignChunk - 1) / kAlignChunk), kBlock, 0, s>>>(
       btm, btm_h, top, top_h, inverse_ws, channel);
   OCNN_LAUNCH_OK("align_forward_ws");
+  return OCNN_OK;
+}
+
+int ocnn_align_forward_add(float* top, int top_h, int channel, const float* btm, int btm_h, const int* idx,
+    ocnn_stream_t stream) {
+  OCNN_REQUIRE(top && btm && idx && top_h >= 0 && btm_h >= 0 && channel > 0, OCNN_E_BADARG, "bad argument");
+  if (top_h > 0 && btm_h > 0)
+    align_add_kernel<<<dim3(blocks_for(btm_h), (channel + kAlignChunk - 1) / kAlignChunk), kBlock, 0,
+        as_stream(stream)>>>(top, top_h, btm, btm_h, idx, channel);
+  OCNN_LAUNCH_OK("align_forward_add");
   return OCNN_OK;
 }
 

@@ -722,6 +722,29 @@ def octree_conv_fused(data_in, weights, bias, relu, octree, depth, num_output, k
                kernel_size, stride, nempty, bias=bias, relu=relu, out=out)
 
 
+def conv1x1_pair(data, w1, b1, w2, b2, relu=True, return_label=False):
+  """Two 1x1x1 convolutions in one pass over `data` [1, C, H, 1] fp32: relu(w1 data + b1) -> w2 . + b2,
+  the prediction head of pytorch/ocnn/ounet.py:46-49 with the BatchNorm folded into (w1, b1).
+  w1 [hidden <= 32, C], w2 [n_out <= 8, hidden]; the biases may be None.  Returns the logits
+  [1, n_out, H, 1], and with return_label their argmax over the channels (int32 [H], the labels of
+  ounet.py:117-118) from the same kernel."""
+  data = data.contiguous()
+  if data.dtype != torch.float32:
+    raise TypeError("conv1x1_pair is fp32")
+  c, h = data.size(1), data.size(2)
+  w1, w2 = w1.contiguous().float(), w2.contiguous().float()
+  hidden, n_out = w1.size(0), w2.size(0)
+  if w1.numel() != hidden * c or w2.numel() != n_out * hidden:
+    raise OcnnError(-3, "conv1x1_pair: weights [%d, %d] and [%d, %d] expected" % (hidden, c, n_out, hidden))
+  b1 = None if b1 is None else b1.contiguous().float()
+  b2 = None if b2 is None else b2.contiguous().float()
+  out = torch.empty(1, n_out, h, 1, dtype=torch.float32, device=data.device)
+  label = torch.empty(h, dtype=torch.int32, device=data.device) if return_label else None
+  _lib.call("ocnn_conv1x1_pair", _ptr(out), _ptr(label), _ptr(data), c, h, _ptr(w1), _ptr(b1), hidden, int(relu),
+            _ptr(w2), _ptr(b2), n_out, _stream())
+  return (out, label) if return_label else out
+
+
 def forget_cached(tensor):
   """Drops what this module keeps with a tensor between calls: the packed weights of
   octree_conv_rows(constant_weights=True), and for an octree blob the inverted child links, the
@@ -1189,9 +1212,12 @@ def octree_bilinear_xyz(xyz, depth_from, depth_to):
 
 
 # ---- feature transfer ---------------------------------------------------------------------------
-def octree_align(src_data, src_octree, des_octree, depth):
+def octree_align(src_data, src_octree, des_octree, depth, add_to=None):
   """pytorch/cpp/octree_align.cpp:9-61 -> [des_data [1,C,des_h,1], idx int32 [src_h]]: the
-  features of `src_octree`'s nodes moved to the nodes of `des_octree` with the same key."""
+  features of `src_octree`'s nodes moved to the nodes of `des_octree` with the same key.
+  add_to: a contiguous fp32 [1,C,des_h,1] tensor that the moved features are added to in place
+  (`x + octree_align(...)[0]` of the decoder loop, pytorch/ocnn/ounet.py:109-111, in one pass);
+  it is returned as des_data."""
   src_octree, des_octree = _to_dev(src_octree), _to_dev(des_octree)
   sinfo, dinfo = octree_info(src_octree), octree_info(des_octree)
   src_data = src_data.contiguous()
@@ -1205,6 +1231,12 @@ def octree_align(src_data, src_octree, des_octree, depth):
   des_key, des_h = _morton_keys(des_octree, dinfo, depth)
   idx = torch.empty(src_h, dtype=torch.int32, device=src_data.device)
   _search_key(idx, des_key, des_h, src_key, src_h, sorted_queries=True)
+  if add_to is not None:
+    if (add_to.dtype != torch.float32 or not add_to.is_contiguous() or add_to.device != src_data.device
+        or add_to.numel() != channel * des_h or add_to.dim() < 2 or add_to.size(1) != channel):
+      raise OcnnError(-3, "octree_align: add_to must be a contiguous fp32 [1, %d, %d, 1] tensor" % (channel, des_h))
+    _lib.call("ocnn_align_forward_add", _ptr(add_to), des_h, channel, _ptr(src_data), src_h, _ptr(idx), _stream())
+    return [add_to, idx]
   out = torch.empty(1, channel, des_h, 1, dtype=torch.float32, device=src_data.device)
   inverse = torch.empty(max(des_h, 1), dtype=torch.int32, device=src_data.device)
   _lib.call("ocnn_align_forward_ws", _ptr(out), des_h, channel, _ptr(src_data), src_h, _ptr(idx), _ptr(inverse),

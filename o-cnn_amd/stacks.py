@@ -182,13 +182,20 @@ def create_full_octree(depth, channel, batch_size=1, node_dis=True):
   return octree
 
 
-def predict_head(x, head, octree, depth):
+def predict_head(x, head, octree, depth, return_label=False):
   """The prediction module of pytorch/ocnn/ounet.py:46-49: a 1x1x1 conv -> BN -> ReLU to the hidden
   width and a 1x1x1 convolution with bias; head = ((w1, b1), (w2, b2)) with the BatchNorm folded
-  into (w1, b1).  Returns the logits [1, n_out, H, 1]."""
+  into (w1, b1).  Returns the logits [1, n_out, H, 1] (with return_label also their argmax over
+  the channels, int32 [H]).  fp32 heads of at most 32 hidden and 8 output channels run as one
+  kernel that keeps the hidden channels in registers."""
   (w1, b1), (w2, b2) = head
+  if x.dtype == torch.float32 and w1.shape[0] <= 32 and w2.shape[0] <= 8:
+    return F.conv1x1_pair(x, w1, b1, w2, b2, relu=True, return_label=return_label)
   hidden = conv_bn_relu(x, w1, b1, octree, depth, w1.shape[0], (1, 1, 1))
-  return conv_bn_relu(hidden, w2, b2, octree, depth, w2.shape[0], (1, 1, 1), relu=False)
+  logit = conv_bn_relu(hidden, w2, b2, octree, depth, w2.shape[0], (1, 1, 1), relu=False)
+  if return_label:
+    return logit, logit.view(logit.shape[1], -1).argmax(0).to(torch.int32)
+  return logit
 
 
 def completion_decoder(code, params, split_labels, depth, full_depth, batch_size=1, channel_out=4,
@@ -221,14 +228,15 @@ def completion_decoder(code, params, split_labels, depth, full_depth, batch_size
       w, b = params[("up", d)]
       x = conv_bn_relu(feats[d - 1], w, b, octree, d - 1, w.shape[1] // 8, (2, 2, 2), 2, deconv=True)
       if skips is not None and d in skips:
-        skip, _ = F.octree_align(skips[d], octree_in, octree, d)
-        x = x + skip
+        if x.dtype == torch.float32:
+          x, _ = F.octree_align(skips[d], octree_in, octree, d, add_to=x.contiguous())
+        else:
+          x = x + F.octree_align(skips[d], octree_in, octree, d)[0]
       w, b = params[("conv", d)]
       feats[d] = conv_bn_relu(x, w, b, octree, d, w.shape[0])
     predicted = None
     if ("predict", d) in params:
-      logit = predict_head(feats[d], params[("predict", d)], octree, d)
-      predicted = logit.view(logit.shape[1], -1).argmax(0).to(torch.int32)
+      logit, predicted = predict_head(feats[d], params[("predict", d)], octree, d, return_label=True)
       feats[("logit", d)], feats[("label", d)] = logit, predicted
     if split_labels is None:
       if predicted is None:

@@ -52,6 +52,12 @@ def test_align_between_different_octrees(oc, orc, synthetic):
     out, idx = oc.nn.octree_align(T(x).cuda().view(1, 7, -1, 1), T(ha).cuda(), T(hb).cuda(), d)
     assert np.array_equal(idx.cpu().numpy(), eidx) and 0 < (eidx >= 0).sum() < eidx.size
     assert np.array_equal(out.cpu().numpy().reshape(exp.shape), exp)
+    # the sum behind the transfer (`deconv + skip`, pytorch/ocnn/ounet.py:111) in the same pass
+    base = rng.standard_normal(exp.shape).astype(np.float32)
+    acc = T(base).cuda().view(1, 7, -1, 1)
+    got, idx2 = oc.nn.octree_align(T(x).cuda().view(1, 7, -1, 1), T(ha).cuda(), T(hb).cuda(), d, add_to=acc)
+    assert got.data_ptr() == acc.data_ptr() and torch.equal(idx2, idx)
+    assert np.array_equal(got.cpu().numpy().reshape(exp.shape), base + exp)
     g = rng.standard_normal(exp.shape).astype(np.float32)
     back = oc.nn.octree_align_grad(T(g).cuda().view(1, 7, -1, 1), idx)
     assert np.array_equal(back.cpu().numpy().reshape(x.shape), interp.octree_align_grad(g, eidx))

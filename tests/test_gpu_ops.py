@@ -677,3 +677,50 @@ def test_pad_with_a_value_per_channel(oc, orc, tree, dtype):
     exp = T(orc.pad(x.float().numpy(), child)).to(dtype)
     exp[:, child < 0] = fill.to(dtype)[:, None]
     assert got.dtype == dtype and torch.equal(got.cpu().view(Cc, -1), exp), (d, Cc)
+
+
+@pytest.mark.parametrize("cin,hidden,nout", [(3, 32, 2), (32, 32, 2), (64, 32, 4), (130, 20, 5), (256, 32, 8), (5, 1, 1)])
+def test_two_1x1x1_convolutions_in_one_pass(oc, orc, tree, cin, hidden, nout):
+  """The prediction head of pytorch/ocnn/ounet.py:46-49 (1x1x1 conv -> ReLU -> 1x1x1 conv with bias)
+  as one kernel against the oracle's two convolutions, 1e-4 of the largest magnitude; the labels
+  are the argmax of the kernel's own logits (ounet.py:117-118), and the operator-by-operator
+  path gives the same within the tolerance.  Levels of 64 to 5 000+ nodes (partial tiles); heights
+  of 1, 63 and 257 columns against the matrix product in float64, which is what a 1x1x1
+  convolution is."""
+  F = oc.nn
+  rng = np.random.default_rng(cin * 100 + hidden * 10 + nout)
+  host, dev, blob = tree["host"], tree["dev"], tree["blob"]
+  for d in (2, 5, 6):
+    H = int(blob.nnum[d])
+    x = rng.standard_normal((cin, H)).astype(np.float32)
+    w1 = (rng.standard_normal((hidden, cin)) / np.sqrt(cin)).astype(np.float32)
+    w2 = (rng.standard_normal((nout, hidden)) / np.sqrt(hidden)).astype(np.float32)
+    b1 = (rng.standard_normal(hidden) * 0.3).astype(np.float32)
+    b2 = (rng.standard_normal(nout) * 0.3).astype(np.float32)
+    hid = np.maximum(orc.octree_conv(x, w1, host, d, hidden, [1, 1, 1], 1, False) + b1[:, None], 0)
+    exp = orc.octree_conv(hid, w2, host, d, nout, [1, 1, 1], 1, False) + b2[:, None]
+    xd = T(x).cuda().view(1, cin, H, 1)
+    out, label = F.conv1x1_pair(xd, T(w1).cuda(), T(b1).cuda(), T(w2).cuda(), T(b2).cuda(), return_label=True)
+    got = out.cpu().numpy().reshape(nout, H)
+    assert np.abs(got - exp).max() <= 1e-4 * max(np.abs(exp).max(), 1.0), (d, cin, hidden, nout)
+    assert np.array_equal(label.cpu().numpy(), got.argmax(0).astype(np.int32)), (d, cin, hidden, nout)
+    # no biases, no ReLU, no labels
+    plain = F.conv1x1_pair(xd, T(w1).cuda(), None, T(w2).cuda(), None, relu=False)
+    e2 = orc.octree_conv(orc.octree_conv(x, w1, host, d, hidden, [1, 1, 1], 1, False), w2, host, d, nout, [1, 1, 1], 1, False)
+    assert np.abs(plain.cpu().numpy().reshape(nout, H) - e2).max() <= 1e-4 * max(np.abs(e2).max(), 1.0)
+    # the head of the decoder stack takes this kernel; operator by operator it is two convolutions
+    two = oc.stacks.conv_bn_relu(oc.stacks.conv_bn_relu(xd, T(w1).cuda(), T(b1).cuda(), dev, d, hidden, (1, 1, 1)),
+                                 T(w2).cuda(), T(b2).cuda(), dev, d, nout, (1, 1, 1), relu=False)
+    assert np.abs(two.cpu().numpy().reshape(nout, H) - exp).max() <= 1e-4 * max(np.abs(exp).max(), 1.0)
+  for H in (1, 63, 257):
+    x = rng.standard_normal((cin, H)).astype(np.float32)
+    exp = w2.astype(np.float64) @ np.maximum(w1.astype(np.float64) @ x + b1[:, None], 0) + b2[:, None]
+    out, label = F.conv1x1_pair(T(x).cuda().view(1, cin, H, 1), T(w1).cuda(), T(b1).cuda(), T(w2).cuda(), T(b2).cuda(),
+                                return_label=True)
+    got = out.cpu().numpy().reshape(nout, H)
+    assert np.abs(got - exp).max() <= 1e-4 * max(np.abs(exp).max(), 1.0), (H, cin, hidden, nout)
+    assert np.array_equal(label.cpu().numpy(), got.argmax(0).astype(np.int32))
+  with pytest.raises(oc.nn.OcnnError):
+    F.conv1x1_pair(xd, torch.zeros(33, cin).cuda(), None, torch.zeros(2, 33).cuda(), None)
+  with pytest.raises(oc.nn.OcnnError):
+    F.conv1x1_pair(xd, torch.zeros(8, cin).cuda(), None, torch.zeros(9, 8).cuda(), None)
