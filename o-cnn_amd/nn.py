@@ -1370,12 +1370,26 @@ def octree_grow(octree_in, target_depth, full_octree):
   return out
 
 
-def octree_update(octree_in, label_in, depth, split):
-  """pytorch/cpp/octree_grow.cpp:164-190: children[depth] from the split labels."""
+def octree_update(octree_in, label_in, depth, split, inplace=False):
+  """pytorch/cpp/octree_grow.cpp:164-190: children[depth] from the split labels.
+  inplace=True rewrites `octree_in` itself and returns it (for a caller that owns the tensor and
+  drops the old state anyway, as the decoder loop does with what octree_grow just returned): the
+  clone of the whole blob is saved.  What this module keeps with the tensor is dropped."""
   octree_in = _to_dev(octree_in)
   iin = octree_info(octree_in)
-  out = torch.empty_like(octree_in)     # (the library copies the blob while the host waits for the count)
   info = _Info(iin.raw)
+  if inplace:
+    label = _to_dev(label_in.contiguous().to(torch.int32))
+    n = label.numel()
+    sb = _lib.get().ocnn_octree_update_scratch_bytes(n)
+    ws = _workspace(sb + 256, "update")
+    base = (ws.data_ptr() + 255) & ~255
+    _lib.call("ocnn_octree_update", _ptr(octree_in), info.p, _ptr(label), n, depth, split, C.c_void_p(base),
+              C.c_size_t(sb), _stream())
+    forget_cached(octree_in)
+    octree_in._ocnn_info = _Info(info.raw)
+    return octree_in
+  out = torch.empty_like(octree_in)     # (the library copies the blob while the host waits for the count)
   label = _to_dev(label_in.contiguous().to(torch.int32))
   n = label.numel()
   sb = _lib.get().ocnn_octree_update_scratch_bytes(n)

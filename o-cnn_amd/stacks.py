@@ -244,7 +244,8 @@ def completion_decoder(code, params, split_labels, depth, full_depth, batch_size
       label = predicted
     else:
       label = split_labels(d, feats[d]) if callable(split_labels) else split_labels[d]
-    octree = F.octree_update(octree, label.to(torch.int32), d, 1)
+    # (the octree of this depth is the loop's own, fresh from octree_grow: updated in place)
+    octree = F.octree_update(octree, label.to(torch.int32), d, 1, inplace=True)
     if d < depth:
       octree = F.octree_grow(octree, d + 1, False)
     elif signal is not None:

@@ -570,6 +570,11 @@ def test_update_in_place_and_with_the_clone_inside(oc, orc, samples):
         oc.lib.call("ocnn_octree_update", P(mine), C.c_void_p(raw.ctypes.data), P(lab), n, depth, 1, P(ws), C.c_size_t(sb), None)
         torch.cuda.synchronize()
         assert torch.equal(mine, got) and np.array_equal(raw[:716], exp[:716])
+        own = src.clone()                                               # the same through the Python mirror
+        F.octree_info(own)
+        back = F.octree_update(own, lab, depth, 1, inplace=True)
+        assert back is own and torch.equal(own, got)
+        assert F.octree_info(own).nnum_nempty(depth) == max(int(labels.sum()), 1)
   raw = np.array(info.raw, copy=True)
   with pytest.raises(oc.lib.OcnnError) as e:
     oc.lib.call("ocnn_octree_update_copy", P(src), P(src), C.c_void_p(raw.ctypes.data), P(lab), n, depth, 1, P(ws), C.c_size_t(sb), None)
