@@ -461,16 +461,29 @@ int ocnn_octree_batch(void* out_dev, const void* out_info, const void* const* oc
   OCNN_LAUNCH_OK("merge");
   int e = OCNN_OK;
   OCNN_REQUIRE(o.has(OCNN_CHILD), OCNN_E_FORMAT, "octrees without child links cannot get neighbour tables");
-  for (int d = 1; d <= depth; ++d) {
+  for (int d = 1; d <= depth;) {
     int* neigh = reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_NEIGH, d));
     if (d <= fl) {
       e = ocnn_calc_neigh_full(neigh, d, B, stream);
       if (e) return e;
-    } else if (o.nnum[d - 1] > 0) {
-      launch_neigh_sparse(neigh, reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_NEIGH, d - 1)),
-          reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_CHILD, d - 1)), o.nnum[d - 1], s, o.nnum[d] / 8);
-      OCNN_LAUNCH_OK("calc_neigh_sparse");
+      ++d;
+      continue;
     }
+    if (o.nnum[d - 1] <= 0) { ++d; continue; }
+    // the last levels in one launch, their rows handed down in registers (levels of up to two
+    // million nodes: beyond that a launch per level is as fast)
+    int count = 1;
+    if (depth - d < kNeighLevels && o.nnum[depth] <= (1 << 21)) while (d + count <= depth && o.nnum[d + count - 1] > 0) ++count;
+    int* tables[kNeighLevels] = {nullptr, nullptr, nullptr};
+    const int* links[kNeighLevels] = {nullptr, nullptr, nullptr};
+    for (int i = 0; i < count; ++i) {
+      tables[i] = reinterpret_cast<int*>(blob + o.ptr_dis(OCNN_NEIGH, d + i));
+      links[i] = reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_CHILD, d + i - 1));
+    }
+    launch_neigh_sparse_levels(count, tables, reinterpret_cast<const int*>(blob + o.ptr_dis(OCNN_NEIGH, d - 1)), links,
+        o.nnum[d - 1], s);
+    OCNN_LAUNCH_OK("calc_neigh_sparse");
+    d += count;
   }
   return OCNN_OK;
 }
