@@ -157,3 +157,103 @@ def test_random_growth_and_adaptive_builds(oc, orc, block):
       continue   # a combination the reference's builder rejects
     got = F.points2octree(T(pb), dd, 2, **opts)
     assert np.array_equal(got.cpu().numpy(), exp), ("build", seed, dd, opts)
+
+
+CH = [3, 8, 16, 24, 32, 48, 64, 96, 128, 160, 256]
+SHAPES = [([3, 3, 3], 1), ([3, 3, 3], 1), ([2, 2, 2], 2), ([2, 2, 2], 2), ([1, 1, 1], 1), ([3, 1, 1], 1), ([3, 3, 1], 1)]
+
+
+def bf16_round(a):
+  return T(a).bfloat16().float().numpy()
+
+
+@pytest.mark.parametrize("block", range(4))
+def test_random_wide_channel_operators(oc, orc, synthetic, block):
+  """Seeded cases at the channel widths the networks use (3 .. 256, also 48, 96, 160) on levels of
+  hundreds to tens of thousands of nodes: convolution and deconvolution of a random shape, stride
+  and node set in fp32 (1e-4) and bf16 (2e-2, operands rounded to bf16 first) with both fp32
+  gradients, and for the shapes the row-major entry points serve (3x3x3 stride 1, 2x2x2 stride
+  2) the same operator on row-major tensors with bias and ReLU, with and without kept weights."""
+  F = oc.nn
+
+  def close(got, exp, tol, what):
+    if exp.size:
+      err = float(np.abs(got.reshape(exp.shape) - exp).max()) / (float(np.abs(exp).max()) + 1e-30)
+      assert err < tol, (what, err)
+
+  for seed in range(block * 6, block * 6 + 6):
+    rng = np.random.default_rng(7000 + seed)
+    depth = int(rng.integers(5, 8))
+    B = int(rng.integers(1, 4))
+    npts = int(rng.integers(2000, 30000))
+    pbs = []
+    for b in range(B):
+      p, n, _ = (synthetic.shape_cloud if rng.integers(0, 2) else synthetic.room_cloud)(npts, seed * 10 + b)
+      pbs.append(make_points_blob(p, n))
+    host = orc.octree_batch([orc.points2octree(pb, depth, 2) for pb in pbs])
+    dev = F.points2octree_batch([T(pb).cuda() for pb in pbs], depth, 2)
+    assert np.array_equal(dev.cpu().numpy(), host), seed
+    blob = OctreeBlob(host)
+    for rep in range(3):
+      d = int(rng.integers(3, depth + 1))
+      ks, stride = SHAPES[int(rng.integers(0, len(SHAPES)))]
+      nempty = bool(rng.integers(0, 2))
+      C, Co = CH[int(rng.integers(0, len(CH)))], CH[int(rng.integers(0, len(CH)))]
+      H, Hne = int(blob.nnum[d]), int(blob.nnum_nempty[d])
+      Hin = Hne if nempty else H
+      K = int(np.prod(ks))
+      if Hin == 0 or Hin * K * C * Co > 1e9:
+        continue
+      tag = "seed %d rep %d depth %d/%d H %d Hne %d %s stride %d nempty %d %d -> %d" % (seed, rep, d, depth, H, Hne, ks, stride, nempty, C, Co)
+      x = bf16_round(rng.standard_normal((C, Hin)).astype(np.float32))
+      w = bf16_round((rng.standard_normal((Co, C * K)) / np.sqrt(C * K)).astype(np.float32))
+      ye = orc.octree_conv(x, w, host, d, Co, ks, stride, nempty)
+      xd, wdv = T(x).cuda().view(1, C, Hin, 1), T(w).cuda()
+      close(F.octree_conv(xd, wdv, dev, d, Co, ks, stride, nempty).cpu().numpy(), ye, TOL, tag + " conv fp32")
+      close(F.octree_conv(xd.bfloat16(), wdv.bfloat16(), dev, d, Co, ks, stride, nempty).float().cpu().numpy(), ye, 2e-2, tag + " conv bf16")
+      if ye.size:
+        g = rng.standard_normal(ye.shape).astype(np.float32)
+        egd, egw = orc.octree_conv_grad(x, w, g, host, d, Co, ks, stride, nempty)
+        gd, gw = F.octree_conv_grad(xd, wdv, dev, T(g).cuda().view(1, Co, -1, 1), d, Co, ks, stride, nempty)
+        close(gw.cpu().numpy(), egw, TOL, tag + " weight gradient")
+        close(gd.cpu().numpy(), egd, TOL, tag + " data gradient")
+      rows_kind = (ks == [3, 3, 3] and stride == 1) or (ks == [2, 2, 2] and stride == 2)
+      if rows_kind and ye.size:
+        bias = (rng.standard_normal(Co) * 0.2).astype(np.float32)
+        exp = ye if (stride == 1 or nempty) else orc.pad(ye, blob.prop("child", d - 1))
+        exp = np.maximum(exp + bias[:, None], 0)
+        for const in (False, True):
+          r = F.octree_conv_rows(F.to_rows(xd.bfloat16()), C, wdv.bfloat16(), dev, d, Co, bias=T(bias).cuda(), relu=True,
+                                 kernel_size=tuple(ks), stride=stride, nempty=nempty, constant_weights=const)
+          assert not r[-1].any() and not r[:, Co:].any(), tag
+          close(F.from_rows(r, Co).float().cpu().numpy(), exp, 2e-2, tag + " conv on rows, kept weights %d" % const)
+      if stride == 1 or d < depth:
+        hin_d = Hin if stride == 1 else Hne
+        if hin_d == 0:
+          continue
+        xq = x if stride == 1 else bf16_round(rng.standard_normal((C, hin_d)).astype(np.float32))
+        wd = bf16_round((rng.standard_normal((C, Co * K)) / np.sqrt(C)).astype(np.float32))
+        ye = orc.octree_deconv(xq, wd, host, d, Co, ks, stride, nempty)
+        xqd = T(xq).cuda().view(1, C, hin_d, 1)
+        close(F.octree_deconv(xqd, T(wd).cuda(), dev, d, Co, ks, stride, nempty).cpu().numpy(), ye, TOL, tag + " deconv fp32")
+        close(F.octree_deconv(xqd.bfloat16(), T(wd).cuda().bfloat16(), dev, d, Co, ks, stride, nempty).float().cpu().numpy(), ye,
+              2e-2, tag + " deconv bf16")
+        if ye.size:
+          g = rng.standard_normal(ye.shape).astype(np.float32)
+          egd, egw = orc.octree_deconv_grad(xq, wd, g, host, d, Co, ks, stride, nempty)
+          gd, gw = F.octree_deconv_grad(xqd, T(wd).cuda(), dev, T(g).cuda().view(1, Co, -1, 1), d, Co, ks, stride, nempty)
+          close(gw.cpu().numpy(), egw, TOL, tag + " deconv weight gradient")
+          close(gd.cpu().numpy(), egd, TOL, tag + " deconv data gradient")
+        if rows_kind and ye.size:
+          for const in (False, True):
+            if stride == 1 or nempty:
+              rin = F.to_rows(xqd.bfloat16())
+            else:   # rows of ALL nodes of the depth in; what the empty ones hold must not be read
+              full = np.full((C, H), 3.0, np.float32)
+              child = blob.prop("child", d)
+              full[:, child >= 0] = xq[:, child[child >= 0]]
+              rin = F.to_rows(T(full).cuda().view(1, C, H, 1).bfloat16())
+            r = F.octree_conv_rows(rin, C, T(wd).cuda().bfloat16(), dev, d, Co, deconv=True, kernel_size=tuple(ks),
+                                   stride=stride, nempty=nempty, constant_weights=const)
+            assert not r[-1].any() and not r[:, Co:].any(), tag
+            close(F.from_rows(r, Co).float().cpu().numpy(), ye, 2e-2, tag + " deconv on rows, kept weights %d" % const)
