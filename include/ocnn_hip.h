@@ -315,8 +315,11 @@ int ocnn_conv_bf16_tile_threshold(int tiles);
  * kernels for tap sets of three taps or more exist in two forms that add the same products in the
  * same order -- weights staged in LDS for all taps of a tile, or read per live tap straight from
  * the packed weights (the default where it is faster: everywhere but the channel-major operators
- * with whole blocks of 128 output channels).  0 sends every call to the staged form, 1 restores
- * the default.  Returns the previous setting. */
+ * with whole blocks of 128 output channels).  The fp32 kernel for the non-empty nodes has the same
+ * two forms (the second one on levels where fewer than one node in five is non-empty) and follows
+ * the same switch.  0 sends every call to the staged form, 1 restores the default, 2 is 1 with the
+ * fp32 kernel's second form on every level (the tests run it on small octrees).  Returns the
+ * previous setting of the bf16 kernels (0 or 1). */
 int ocnn_conv_rows_direct(int on);
 
 /* Test hook, no counterpart in the reference (process-wide): the weight gradient of the shapes

@@ -579,16 +579,145 @@ __global__ __launch_bounds__(256) void conv_rows_f32_kernel(ConvArgs a, float* _
     if (n0 < a.N) store_tiles<float, MT>(a, out, acc, pass * MT, n0, lane);
   }
 }
+// The same operator without LDS for the weights and without barriers (the fp32 form of
+// conv_rows_bf16_direct_kernel below): a wavefront walks the (tap, 32-channel slab) stages of
+// the taps that are live for its own 64 columns, reads the A fragments of a stage straight from
+// the packed weights (16 bytes a lane: the four k-steps of an 8-channel group) and gathers the
+// rows of the column halves that have the neighbour, with the next stage's weights and rows in
+// flight (two register sets).  The staged kernel above takes every workgroup through all
+// K x slabs barriers and moves the weights of all taps through LDS whether a tap is live or not;
+// over the non-empty nodes of a surface about half of the (wavefront, tap) pairs are dead.
+// Stages in the same order as the staged kernel (tap, then slab), a dead half adds nothing:
+// the same sums.
+template <int MT, int WPS = 2, int WAVES = kConvWaves>
+__global__ __launch_bounds__(64 * WAVES, WPS) void conv_rows_f32_direct_kernel(ConvArgs a, float* __restrict__ out,
+    const float4* __restrict__ xt, const float4* __restrict__ Wt, int n_tiles, int cpad) {
+  constexpr int kG = kRowSlabF / 8;                    // 8-channel groups of a slab
+  constexpr int kWVecs = kG * MT * 64;                 // 16-byte units of one (tap, slab)
+  constexpr int kCols = kWaveCols * WAVES;             // columns of a workgroup
+  __shared__ int sSrc[27][kCols];                      // source row of (tap, column), in 16-byte units of the copy
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = xcd_tile(blockIdx.x, n_tiles);
+  if (tile >= n_tiles) return;
+  const int n0 = tile * kCols + wave * kWaveCols;
+  const int r = lane & 31, kh = lane >> 5;
+  const int nslab = (cpad + kRowSlabF - 1) / kRowSlabF;
+  const int npass = (a.mtiles + MT - 1) / MT;
+  const int cpad4 = cpad >> 2;
+  tile_sources(a, tile * kCols + (int)threadIdx.x,
+      [&](int k, int row) { sSrc[k][threadIdx.x] = (row < 0 ? a.Hin : row) * cpad4; });
+  const int c0 = wave * kWaveCols + r;
+  unsigned live[2] = {0, 0};
+  __syncthreads();                                     // source rows written
+  {
+    const int none = a.Hin * cpad4;
+#pragma unroll
+    for (int k = 0; k < 27; ++k) {
+      if (k >= a.K) break;
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+        if (__ballot(sSrc[k][c0 + 32 * nt] != none) != 0) live[nt] |= 1u << k;
+    }
+    live[0] = __builtin_amdgcn_readfirstlane(live[0]);
+    live[1] = __builtin_amdgcn_readfirstlane(live[1]);
+  }
+  const unsigned live_any = live[0] | live[1];
+  for (int pass = blockIdx.y; pass < npass; pass += gridDim.y) {
+    floatx16 acc[MT][2];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
+    float4 wa[2][kG][MT], x[2][kG][2];                 // two register sets: [set][group][row tile / column half]
+    auto fetch = [&](int tap, int slab, auto set) {
+      constexpr int S = decltype(set)::value;
+      if (tap < 0) return;                             // uniform
+      const int ngroup = min(kRowSlabF, cpad - slab * kRowSlabF) >> 3;
+      const float4* wsrc = Wt + (((int64_t)pass * a.K + tap) * nslab + slab) * kWVecs + lane;
+#pragma unroll
+      for (int c8 = 0; c8 < kG; ++c8)
+        if (c8 < ngroup) {
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) wa[S][c8][mt] = wsrc[(c8 * MT + mt) * 64];
+        }
+      const int s0 = sSrc[tap][c0], s1 = sSrc[tap][c0 + 32];
+      const int off = ((slab * kRowSlabF) >> 2) + kh;
+      if ((live[0] >> tap) & 1) {                      // uniform over the wavefront
+#pragma unroll
+        for (int c8 = 0; c8 < kG; ++c8)
+          if (c8 < ngroup) x[S][c8][0] = xt[(int64_t)s0 + off + 2 * c8];
+      }
+      if ((live[1] >> tap) & 1) {
+#pragma unroll
+        for (int c8 = 0; c8 < kG; ++c8)
+          if (c8 < ngroup) x[S][c8][1] = xt[(int64_t)s1 + off + 2 * c8];
+      }
+    };
+    auto part = [](const float4& v, int j) { return j == 0 ? v.x : j == 1 ? v.y : j == 2 ? v.z : v.w; };
+    auto compute = [&](int tap, int slab, auto set) {
+      constexpr int S = decltype(set)::value;
+      const bool l0 = (live[0] >> tap) & 1, l1 = (live[1] >> tap) & 1;   // uniform over the wavefront
+      const int ngroup = min(kRowSlabF, cpad - slab * kRowSlabF) >> 3;
+#pragma unroll
+      for (int c8 = 0; c8 < kG; ++c8) {
+        if (c8 >= ngroup) continue;                    // uniform
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            const float av = part(wa[S][c8][mt], j);
+            if (l0) acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, part(x[S][c8][0], j), acc[mt][0], 0, 0, 0);
+            if (l1) acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, part(x[S][c8][1], j), acc[mt][1], 0, 0, 0);
+          }
+        }
+      }
+    };
+    unsigned todo = live_any;                          // live taps not yet requested (uniform)
+    auto next_tap = [&]() {
+      if (todo == 0) return -1;
+      const int t = __builtin_ctz(todo);
+      todo &= todo - 1;
+      return t;
+    };
+    // the stages (live tap, slab) in order, two in flight
+    int t0 = next_tap(), s0 = 0;
+    fetch(t0, s0, std::integral_constant<int, 0>());
+    while (t0 >= 0) {
+      int t1 = t0, s1 = s0 + 1;
+      if (s1 == nslab) { s1 = 0; t1 = next_tap(); }
+      fetch(t1, s1, std::integral_constant<int, 1>());
+      compute(t0, s0, std::integral_constant<int, 0>());
+      if (t1 < 0) break;
+      t0 = t1; s0 = s1 + 1;
+      if (s0 == nslab) { s0 = 0; t0 = next_tap(); }
+      fetch(t0, s0, std::integral_constant<int, 0>());
+      compute(t1, s1, std::integral_constant<int, 1>());
+    }
+    if (n0 < a.N) store_tiles<float, MT>(a, out, acc, pass * MT, n0, lane);
+  }
+}
 // [pass][tap][slab][c8][j][mt][lane]: lane (m, kh) <- W'(m, slab*64 + c8*8 + 4kh + j, tap)
+// (direct: [pass][tap][slab][c8][mt][lane][j], the four k-steps of a group as one 16-byte unit a lane)
 __global__ void pack_weights_rows_f32(float* __restrict__ Wt, const float* __restrict__ W, int M, int Cin, int K,
-    int MT, int npass, int nslab, int64_t sm, int64_t sc) {
+    int MT, int npass, int nslab, int64_t sm, int64_t sc, int direct) {
   int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int64_t total = (int64_t)npass * K * nslab * (kRowSlabF / 8) * 4 * MT * 64;
   if (id >= total) return;
-  int l = (int)(id & 63);
-  int64_t f = id >> 6;
-  int mt = (int)(f % MT); f /= MT;
-  int j = (int)(f % 4); f /= 4;
+  int l, j, mt;
+  int64_t f;
+  if (direct) {
+    j = (int)(id & 3);
+    l = (int)((id >> 2) & 63);
+    f = id >> 8;
+    mt = (int)(f % MT); f /= MT;
+  } else {
+    l = (int)(id & 63);
+    f = id >> 6;
+    mt = (int)(f % MT); f /= MT;
+    j = (int)(f % 4); f /= 4;
+  }
   int c8 = (int)(f % (kRowSlabF / 8)); f /= (kRowSlabF / 8);
   int slab = (int)(f % nslab); f /= nslab;
   int k = (int)(f % K);
@@ -2574,6 +2703,7 @@ __global__ void ichild_kernel(int* __restrict__ ichild, int n_nempty, const int*
 // this many such tiles the LDS kernel (256 columns per workgroup, three workgroups per CU) fills
 // the device better.  Measured crossover on 256 CUs: between 110 and 215 tiles.
 std::atomic<int> g_bf16_reg_min_tiles{192};
+std::atomic<int> g_rows_direct_f32{1};   // fp32 row kernel over the non-empty nodes: the same choice
 std::atomic<int> g_rows_direct{1};   // bf16 row kernels with three taps or more: 1 = weights straight from memory per live tap
 
 struct ConvPlan {
@@ -2848,14 +2978,33 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
     const int cpad = (a.Cin + 7) / 8 * 8;
     const int npass = (a.mtiles + MT - 1) / MT, nslab = (cpad + kRowSlabF - 1) / kRowSlabF;
     int64_t total = (int64_t)npass * a.K * nslab * (kRowSlabF / 8) * 4 * MT * 64;
+    // Stride 1 over the non-empty nodes of a sparse level (fewer than one node in five non-empty: the
+    // finest levels of a surface), three taps or more: weights straight from memory per live tap.
+    // Depth 9 of the scene (one in six), 64 -> 64: 0.476 -> 0.383 ms, 64 -> 32: 0.358 -> 0.246 ms,
+    // 6 -> 32: 0.107 -> 0.074 ms.  On denser levels most taps are live and the staged kernel, which
+    // shares a stage's weights between its four wavefronts through LDS, is ahead (depth 7, one in
+    // two, 128 -> 128: 0.87 against 1.03 ms); stride 2 gains nothing either way.
+    const int direct_rule = g_rows_direct_f32.load();   // 2 (tests): whatever the level
+    const bool direct = nempty && a.mode == kModeS1 && a.K >= 3 && direct_rule != 0 &&
+        (direct_rule == 2 || (int64_t)o->nnum_nempty[p.top_depth] * 5 < o->nnum[p.top_depth]);
     pack_weights_rows_f32<<<blocks_for(total), kBlock, 0, s>>>((float*)wsb, (const float*)weights, a.M, a.Cin, a.K,
-        MT, npass, nslab, sm, sc);
+        MT, npass, nslab, sm, sc, direct ? 1 : 0);
     OCNN_LAUNCH_OK("pack_weights_rows");
     float* xt = (float*)(wsb + p.wt_bytes + p.ichild_bytes);
     dim3 tg((a.Hin + 64) / 64, (cpad + 63) / 64);
     transpose_rows_f32_kernel<<<tg, 256, 0, s>>>(xt, (const float*)btm, a.Cin, a.Hin, cpad);
     OCNN_LAUNCH_OK("transpose_rows");
-    if (MT == 1)
+    if (direct) {
+      const int waves = direct_waves(a.N, npass);
+      const int tiles = (a.N + kWaveCols * waves - 1) / (kWaveCols * waves);
+      const dim3 g(((tiles + 7) / 8) * 8, pass_split(tiles, npass));
+#define OCNN_ROWS_F32_DIRECT(MT_)                                                                                \
+      if (waves == 4) conv_rows_f32_direct_kernel<MT_, 2, 4><<<g, 256, 0, s>>>(a, (float*)top, (const float4*)xt, (const float4*)wsb, tiles, cpad); \
+      else if (waves == 2) conv_rows_f32_direct_kernel<MT_, 2, 2><<<g, 128, 0, s>>>(a, (float*)top, (const float4*)xt, (const float4*)wsb, tiles, cpad); \
+      else conv_rows_f32_direct_kernel<MT_, 2, 1><<<g, 64, 0, s>>>(a, (float*)top, (const float4*)xt, (const float4*)wsb, tiles, cpad)
+      if (MT == 1) { OCNN_ROWS_F32_DIRECT(1); } else { OCNN_ROWS_F32_DIRECT(2); }
+#undef OCNN_ROWS_F32_DIRECT
+    } else if (MT == 1)
       conv_rows_f32_kernel<1><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (float*)top, (const float4*)xt, (const float*)wsb, n_tiles, cpad);
     else
       conv_rows_f32_kernel<2><<<dim3(grid, pass_split(n_tiles, npass)), 256, 0, s>>>(a, (float*)top, (const float4*)xt, (const float*)wsb, n_tiles, cpad);
@@ -4226,7 +4375,10 @@ int ocnn_octree_conv_static(void* top, const void* btm, int channel_in, int btm_
       kernel_size, stride, nempty, dtype, ptr, kBuiltinScratchBytes, as_stream(stream), bias, relu, true);
 }
 
-int ocnn_conv_rows_direct(int on) { return g_rows_direct.exchange(on ? 1 : 0); }
+int ocnn_conv_rows_direct(int on) {
+  g_rows_direct_f32.store(on == 2 ? 2 : (on ? 1 : 0));
+  return g_rows_direct.exchange(on ? 1 : 0);
+}
 int ocnn_conv_wgrad_staged(int on) { return g_wgrad_lds.exchange(on ? 1 : 0); }
 
 int ocnn_conv_bf16_tile_threshold(int tiles) {

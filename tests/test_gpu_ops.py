@@ -724,3 +724,40 @@ def test_two_1x1x1_convolutions_in_one_pass(oc, orc, tree, cin, hidden, nout):
     F.conv1x1_pair(xd, torch.zeros(33, cin).cuda(), None, torch.zeros(2, 33).cuda(), None)
   with pytest.raises(oc.nn.OcnnError):
     F.conv1x1_pair(xd, torch.zeros(8, cin).cuda(), None, torch.zeros(9, 8).cuda(), None)
+
+
+def test_fp32_nonempty_kernel_forms(oc, orc, tree):
+  """The fp32 kernel over the non-empty nodes in its two forms (weights of every tap staged through
+  LDS; weights read per live tap by each wavefront, the choice on sparse levels): the same sums in
+  the same order, so equal bits, and the oracle's result within 1e-4; convolution, deconvolution
+  and both gradients; channel counts with partial stages and one or more passes; tap sets of 27, 9
+  and 3; levels from a few hundred to thousands of rows (workgroups of one to four wavefronts)."""
+  b, dev, host = tree["blob"], tree["dev"], tree["host"]
+  L = oc.lib.get()
+  rng = np.random.default_rng(16)
+  try:
+    for d, ci, co, ks in ((6, 3, 32, [3, 3, 3]), (6, 64, 64, [3, 3, 3]), (5, 20, 70, [3, 3, 3]), (5, 40, 32, [3, 3, 1]),
+                          (4, 72, 130, [3, 1, 1]), (3, 128, 64, [3, 3, 3]), (6, 33, 40, [1, 3, 3])):
+      K = ks[0] * ks[1] * ks[2]
+      hin = int(b.nnum_nempty[d])
+      x = rng.standard_normal((ci, hin)).astype(np.float32)
+      w = (rng.standard_normal((co, ci * K)) / np.sqrt(ci * K)).astype(np.float32)
+      wd = (rng.standard_normal((ci, co * K)) / np.sqrt(ci * K)).astype(np.float32)
+      g = rng.standard_normal((co, hin)).astype(np.float32)
+      xt, wt, wdt, gt = T(x).cuda().view(1, ci, hin, 1), T(w).cuda(), T(wd).cuda(), T(g).cuda().view(1, co, hin, 1)
+      got = {}
+      for form in (0, 2):
+        L.ocnn_conv_rows_direct(form)
+        got[form] = (oc.nn.octree_conv(xt, wt, dev, d, co, ks, 1, True), oc.nn.octree_deconv(xt, wdt, dev, d, co, ks, 1, True),
+                     *oc.nn.octree_conv_grad(xt, wt, dev, gt, d, co, ks, 1, True))
+      for i, name in enumerate(("conv", "deconv", "data gradient", "weight gradient")):
+        assert torch.equal(got[0][i], got[2][i]), (name, d, ci, co, ks)
+      exp = orc.octree_conv(x, w, host, d, co, ks, 1, True)
+      assert relerr(got[2][0].cpu().numpy().reshape(exp.shape), exp) < TOL_F32, (d, ci, co, ks)
+      exp = orc.octree_deconv(x, wd, host, d, co, ks, 1, True)
+      assert relerr(got[2][1].cpu().numpy().reshape(exp.shape), exp) < TOL_F32, (d, ci, co, ks)
+      egd, egw = orc.octree_conv_grad(x, w, g, host, d, co, ks, 1, True)
+      assert relerr(got[2][2].cpu().numpy().reshape(egd.shape), egd) < TOL_F32, (d, ci, co, ks)
+      assert relerr(got[2][3].cpu().numpy().reshape(egw.shape), egw) < TOL_F32, (d, ci, co, ks)
+  finally:
+    L.ocnn_conv_rows_direct(1)
