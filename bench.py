@@ -229,6 +229,16 @@ def main():
     xne = torch.randn(1, C, Hne9, 1, generator=g).to(dev)
     conv_case("conv333_s1_d9_f32_nempty", octree, 9, xne, w32, [3, 3, 3], 1, nempty=True)
     conv_case("conv333_s1_d9_bf16_nempty", octree, 9, xne.bfloat16(), w16, [3, 3, 3], 1, nempty=True)
+    # (over the non-empty nodes the table of source rows is kept with the octree, as a network's layers
+    # of one depth share it; what the first call on an octree pays for making it is stated beside)
+    def first_call(x, w):
+      octree.__dict__.pop("_ocnn_sources", None)
+      return F.octree_conv(x, w, octree, 9, C, [3, 3, 3], 1, True)
+    for name, xx, ww in (("conv333_s1_d9_f32_nempty", xne, w32), ("conv333_s1_d9_bf16_nempty", xne.bfloat16(), w16)):
+      t_first = timed(lambda: first_call(xx, ww), max(reps // 2, 3), 2)
+      extra[name]["sources"] = "table of source rows kept with the octree (one per depth, kernel shape and direction)"
+      extra[name]["ms_first_call_on_an_octree"] = t_first
+    F.octree_conv(xne, w32, octree, 9, C, [3, 3, 3], 1, True)
     rows_ne = F.to_rows(xne.bfloat16())
     rows_ne_out = torch.empty(Hne9 + 1, F.rows_pitch(C), dtype=torch.bfloat16, device=dev)
     t = timed(lambda: F.octree_conv_rows(rows_ne, C, w16, octree, 9, C, out=rows_ne_out, nempty=True), reps, wu)

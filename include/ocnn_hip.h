@@ -206,6 +206,19 @@ int ocnn_octree_conv_fused(void* top, const void* btm, int channel_in, int btm_h
     int num_output, const int* kernel_size, int stride, int nempty, int dtype, void* workspace_dev,
     size_t workspace_bytes, ocnn_stream_t stream);
 
+/* ocnn_octree_conv_fused with the caller's table of source rows for an operator over the non-empty
+ * nodes (`sources_dev` / `sources_bytes` as ocnn_conv_rows_sources_bytes / ocnn_conv_rows_sources
+ * make them for this octree, depth, kernel shape, stride and direction; NULL: the call is
+ * ocnn_octree_conv_fused).  The table depends on the octree level and the operator's geometry alone,
+ * so the layers of a depth share one; a call that brings it looks nothing up and makes no inverted
+ * child links.  The results are the same bits.  Ignored by the operators that look nothing up
+ * (nempty 0, 1x1x1, the fp32 2x2x2 stride-2 deconvolution).  No counterpart in the reference, which
+ * makes its gather indices inside every call (octree_nn.cu:179-253). */
+int ocnn_octree_conv_fused_sources(void* top, const void* btm, int channel_in, int btm_h, const void* weights,
+    const float* bias, int relu, int is_deconv, const int* sources_dev, size_t sources_bytes, const void* octree_dev,
+    const void* info, int depth, int num_output, const int* kernel_size, int stride, int nempty, int dtype,
+    void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream);
+
 /* Two 1x1x1 convolutions in one pass: hidden = W1 data + b1 (ReLU when relu1 != 0), out = W2 hidden
  * + b2, label (may be NULL) = argmax over the channels of out (the first of equal maxima).  It is
  * the prediction head of the reference's decoders, OctreeConv1x1BnRelu(C, 32) -> OctreeConv1x1(32, n)

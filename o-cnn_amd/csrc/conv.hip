@@ -2800,7 +2800,7 @@ int make_plan(const Info* o, int depth, int channel_in, int num_output, const in
 int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, const void* weights,
     const void* octree_dev, const void* info, int depth, int num_output, const int* ks, int stride,
     int nempty, int dtype, void* ws, size_t ws_bytes, hipStream_t s, const float* bias = nullptr,
-    int relu = 0, bool builtin_scratch = false) {
+    int relu = 0, bool builtin_scratch = false, const int* sources = nullptr, size_t sources_bytes = 0) {
   OCNN_REQUIRE(top && btm && weights && octree_dev && info, OCNN_E_BADARG, "null pointer");
   const Info* o = as_info(info);
   ConvPlan p;
@@ -2890,7 +2890,17 @@ int run_conv(int deconv, void* top, const void* btm, int channel_in, int btm_h, 
         "this call needs %zu bytes of scratch memory, the built-in array holds %zu: "
         "use ocnn_octree_conv_fused with a workspace of your own", used, ws_bytes);
   }
-  if (nempty && path != kPathOneTapF32 && path != kPathS2Deconv) {
+  a.src_table = nullptr;
+  a.src_pitch = 0;
+  if (nempty && sources && (path == kPathRowsF32 || path == kPathRowsBf16)) {
+    // the caller's table of source rows (ocnn_conv_rows_sources): no look-up in the kernel, and the
+    // inverted child links, which only the look-up reads, are not made
+    const int pitch = (a.N + kTileCols - 1) / kTileCols * kTileCols;
+    OCNN_REQUIRE(sources_bytes >= sizeof(int) * 27 * (size_t)pitch, OCNN_E_WORKSPACE,
+        "the table of source rows takes %zu bytes, the buffer holds %zu", sizeof(int) * 27 * (size_t)pitch, sources_bytes);
+    a.src_table = sources;
+    a.src_pitch = pitch;
+  } else if (nempty && path != kPathOneTapF32 && path != kPathS2Deconv) {
     int* ichild = reinterpret_cast<int*>(wsb + p.wt_bytes);
     ichild_kernel<<<blocks_for(p.child_h), kBlock, 0, s>>>(ichild, p.ichild_h, a.child, p.child_h);
     OCNN_LAUNCH_OK("ichild");
@@ -4433,6 +4443,15 @@ int ocnn_octree_conv_fused(void* top, const void* btm, int channel_in, int btm_h
     size_t workspace_bytes, ocnn_stream_t stream) {
   return run_conv(is_deconv ? 1 : 0, top, btm, channel_in, btm_h, weights, octree_dev, info, depth, num_output,
       kernel_size, stride, nempty, dtype, workspace_dev, workspace_bytes, as_stream(stream), bias, relu);
+}
+
+int ocnn_octree_conv_fused_sources(void* top, const void* btm, int channel_in, int btm_h, const void* weights,
+    const float* bias, int relu, int is_deconv, const int* sources_dev, size_t sources_bytes, const void* octree_dev,
+    const void* info, int depth, int num_output, const int* kernel_size, int stride, int nempty, int dtype,
+    void* workspace_dev, size_t workspace_bytes, ocnn_stream_t stream) {
+  return run_conv(is_deconv ? 1 : 0, top, btm, channel_in, btm_h, weights, octree_dev, info, depth, num_output,
+      kernel_size, stride, nempty, dtype, workspace_dev, workspace_bytes, as_stream(stream), bias, relu, false,
+      sources_dev, sources_bytes);
 }
 
 int ocnn_octree_conv_rows(void* top_rows, int top_pitch, const void* btm_rows, int btm_pitch, int channel_in,

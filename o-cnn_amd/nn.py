@@ -662,11 +662,37 @@ def col2octree(grad_in, octree, depth, kernel_size, stride, nempty):
 
 
 # ---- convolution -------------------------------------------------------------------------------
+def _conv_sources(octree, info, depth, kernel_size, ksc, stride, is_deconv, ws_base, ws_bytes):
+  """The source row of every (tap, column) of an operator over the non-empty nodes, made once per
+  octree version, depth, kernel shape and direction and kept with the octree tensor (every layer
+  of that depth reads the same table; the row-major entry points share it).  None for an
+  operator that looks nothing up."""
+  tables = octree.__dict__.setdefault("_ocnn_sources", {})
+  if tables.get("version") != octree._version:
+    tables.clear()
+    tables["version"] = octree._version
+  skey = (depth, tuple(int(k) for k in kernel_size), stride, bool(is_deconv))
+  sources = tables.get(skey, False)
+  if sources is False:
+    sources = None
+    nb = C.c_size_t()
+    try:
+      _lib.call("ocnn_conv_rows_sources_bytes", info.p, depth, ksc, stride, 1, int(is_deconv), C.byref(nb))
+    except OcnnError:       # a shape the row-major operators do not serve: the kernel looks its rows up itself
+      nb = C.c_size_t(0)
+    if nb.value:
+      sources = torch.empty(nb.value // 4, dtype=torch.int32, device=octree.device)
+      _lib.call("ocnn_conv_rows_sources", _ptr(sources), C.c_size_t(nb.value), None, _ptr(octree), info.p, depth, ksc,
+                stride, 1, int(is_deconv), C.c_void_p(ws_base), C.c_size_t(ws_bytes), _stream())
+    tables[skey] = sources
+  return sources
+
+
 def _conv(fn, is_deconv, data_in, weights, octree, depth, num_output, kernel_size, stride, nempty,
           bias=None, relu=False, out=None):
   octree = _to_dev(octree)
   info = octree_info(octree)
-  ksc, _ = _ks(kernel_size)
+  ksc, ks3 = _ks(kernel_size)
   data_in = data_in.contiguous()
   weights = weights.contiguous()
   dt = _dtype_code(data_in)
@@ -685,13 +711,19 @@ def _conv(fn, is_deconv, data_in, weights, octree, depth, num_output, kernel_siz
         or not out.is_contiguous()):
     # e.g. a channel slice of a larger [1, C, H, 1] tensor: the result lands there directly
     raise OcnnError(-3, "out must be a contiguous %s %s tensor on %s" % (shape, data_in.dtype, data_in.device))
-  if fn == "ocnn_octree_conv_fused":
+  sources = None
+  # (1x1x1 and the fp32 2x2x2 stride-2 deconvolution have kernels of their own that look nothing up)
+  own_kernel = ks3 == [1, 1, 1] or (dt == F32 and is_deconv and stride == 2 and ks3 == [2, 2, 2])
+  if nempty and top_h.value > 0 and btm_h > 0 and not own_kernel:
+    sources = _conv_sources(octree, info, depth, ks3, ksc, stride, is_deconv, base, ws_bytes.value)
+  if fn == "ocnn_octree_conv_fused" or sources is not None:
     if bias is not None:
       bias = bias.to(torch.float32).contiguous()
       if bias.numel() != num_output:
         raise OcnnError(-3, "bias needs num_output entries")
-    _lib.call(fn, _ptr(out), _ptr(data_in), channel_in, btm_h, _ptr(weights), _ptr(bias), int(relu),
-              int(is_deconv), _ptr(octree), info.p, depth, num_output, ksc, stride, int(nempty), dt,
+    _lib.call("ocnn_octree_conv_fused_sources", _ptr(out), _ptr(data_in), channel_in, btm_h, _ptr(weights), _ptr(bias),
+              int(relu), int(is_deconv), _ptr(sources), C.c_size_t(sources.numel() * 4 if sources is not None else 0),
+              _ptr(octree), info.p, depth, num_output, ksc, stride, int(nempty), dt,
               C.c_void_p(base), C.c_size_t(ws_bytes.value), _stream())
   else:
     _lib.call(fn, _ptr(out), _ptr(data_in), channel_in, btm_h, _ptr(weights), _ptr(octree), info.p,

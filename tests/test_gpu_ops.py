@@ -761,3 +761,57 @@ def test_fp32_nonempty_kernel_forms(oc, orc, tree):
       assert relerr(got[2][3].cpu().numpy().reshape(egw.shape), egw) < TOL_F32, (d, ci, co, ks)
   finally:
     L.ocnn_conv_rows_direct(1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_nonempty_convolutions_with_a_kept_table_of_sources(oc, orc, tree, dtype):
+  """Over the non-empty nodes the Python mirror keeps the table of source rows with the octree and
+  hands it to ocnn_octree_conv_fused_sources; the plain entry points look the rows up in the kernel.
+  Equal bits (conv and deconv, 3x3x3 / 3x1x1 stride 1 and 2x2x2 stride 2), the oracle's result within
+  the tolerance, one table per (depth, shape, direction) shared by the layers of a depth, and a new
+  one after the octree was written to."""
+  import ctypes as C
+  F = oc.nn
+  b, host = tree["blob"], tree["host"]
+  dev = T(host).cuda()
+  info = F.octree_info(dev)
+  P = lambda t: C.c_void_p(t.data_ptr())
+  rng = np.random.default_rng(23)
+  tol = TOL_F32 if dtype == torch.float32 else TOL_BF16
+  code = 0 if dtype == torch.float32 else 1
+  for d, ci, co, ks, stride in ((5, 24, 40, [3, 3, 3], 1), (6, 16, 16, [3, 1, 1], 1), (5, 32, 64, [2, 2, 2], 2)):
+    K = ks[0] * ks[1] * ks[2]
+    for deconv in (False, True):
+      hin = int(b.nnum_nempty[d])
+      x = T(rng.standard_normal((ci, hin)).astype(np.float32)).to(dtype).cuda().view(1, ci, hin, 1)
+      shape = (ci, co * K) if deconv else (co, ci * K)
+      w = T((rng.standard_normal(shape) / np.sqrt(ci * K)).astype(np.float32)).to(dtype).cuda()
+      got = (F.octree_deconv if deconv else F.octree_conv)(x, w, dev, d, co, ks, stride, True)
+      again = (F.octree_deconv if deconv else F.octree_conv)(x, w, dev, d, co, ks, stride, True)
+      assert torch.equal(got, again)
+      # the plain entry point, no table
+      ksc = (C.c_int * 3)(*ks)
+      top_h, need_h, wsb = C.c_int(), C.c_int(), C.c_size_t()
+      oc.lib.call("ocnn_conv_shape", info.p, d, ci, co, ksc, stride, 1, int(deconv), code, C.byref(top_h), C.byref(need_h), C.byref(wsb))
+      ws = torch.empty(wsb.value + 256, dtype=torch.uint8, device="cuda")
+      base = (ws.data_ptr() + 255) & ~255
+      plain = torch.empty_like(got)
+      oc.lib.call("ocnn_octree_deconv" if deconv else "ocnn_octree_conv", P(plain), P(x), ci, hin, P(w), P(dev), info.p, d, co,
+                  ksc, stride, 1, code, C.c_void_p(base), C.c_size_t(wsb.value), None)
+      torch.cuda.synchronize()
+      assert torch.equal(got, plain), (d, ks, stride, deconv)
+      fn = orc.octree_deconv if deconv else orc.octree_conv
+      exp = fn(x.float().cpu().numpy().reshape(ci, hin), w.float().cpu().numpy(), host, d, co, ks, stride, True)
+      assert relerr(got.float().cpu().numpy().reshape(exp.shape), exp) < tol, (d, ks, stride, deconv)
+  tables = dev.__dict__["_ocnn_sources"]
+  kept = [k for k in tables if k != "version"]
+  assert (5, (3, 3, 3), 1, False) in kept and (5, (3, 3, 3), 1, True) in kept
+  if dtype == torch.bfloat16:
+    assert tables[(5, (2, 2, 2), 2, False)] is not None
+  # a write through torch bumps the version: the tables are made again
+  first = tables[(5, (3, 3, 3), 1, False)]
+  dev[-1] = dev[-1]
+  x = T(rng.standard_normal((8, int(b.nnum_nempty[5]))).astype(np.float32)).to(dtype).cuda().view(1, 8, -1, 1)
+  w = T((rng.standard_normal((8, 8 * 27)) * 0.1).astype(np.float32)).to(dtype).cuda()
+  F.octree_conv(x, w, dev, 5, 8, [3, 3, 3], 1, True)
+  assert dev.__dict__["_ocnn_sources"][(5, (3, 3, 3), 1, False)] is not first
